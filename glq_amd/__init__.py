@@ -1,0 +1,18 @@
+"""glq_amd -- MI355X (gfx950) implementation of GLQ's quantized-linear forward.
+
+The compute path is hand-written HIP in ``libglq_hip.so`` (C ABI, see
+``include/glq_hip.h``); this package is the thin PyTorch-ROCm host side that mirrors
+the reference's operator surface:
+
+* ``glq_amd.ext``               the functions of the reference's pybind extension
+                                (``glq._C`` / ``glq_cuda``), same names and arguments
+* ``glq_amd.custom_ops``        the ``torch.ops.glq.*`` schemas of ``glq_vllm/custom_ops.py``
+* ``glq_amd.quantized_linear``  ``E8RHTLinear`` with the reference's buffer names
+
+There is no CPU fallback: importing ``glq_amd.ext`` without the built library, or
+calling an op without a GPU, raises.
+"""
+
+__version__ = "0.1.0"
+
+from .hadamard import block_decompose, pack_block_meta, pack_shard_meta  # noqa: F401

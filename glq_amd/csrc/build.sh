@@ -1,0 +1,11 @@
+#!/bin/bash
+# Builds glq_amd/libglq_hip.so for gfx950 (cross-compiles without a GPU).
+set -e
+here="$(cd "$(dirname "$0")" && pwd)"
+out="$here/../libglq_hip.so"
+/opt/rocm/bin/hipcc --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared \
+    -Xclang -target-feature -Xclang -packed-fp32-ops \
+    -Wall -Wno-unused-function \
+    "$here/capi.hip" "$here/fht.hip" "$here/trellis.hip" "$here/e8.hip" \
+    -o "$out" "$@"
+echo "built $out"

@@ -1,0 +1,389 @@
+// extern "C" entry points of libglq_hip.so: argument checks, dispatch, no allocation.
+#include "common.h"
+
+#include <mutex>
+#include <string.h>
+
+int glqh_rht_init(void);
+int glqh_e8_init(void);
+int glqh_launch_trellis_direct(const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
+                               int64_t k, float scale, float *out, int64_t out_stride, int accum,
+                               hipStream_t stream);
+int glqh_launch_trellis_decompress(const void *packed, int R, int64_t m, int64_t k, void *out,
+                                   hipStream_t stream);
+
+// ---- error plumbing -------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+int glqh_fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+int glqh_check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) return 0;
+    return glqh_fail("%s: %s", what, hipGetErrorString(e));
+}
+
+static int g_cus = 0;
+static int g_init_rc = -1;
+static std::once_flag g_once;
+
+int glqh_device_cus(void) { return g_cus > 0 ? g_cus : 256; }
+
+extern "C" const char *glqh_last_error(void) { return g_err; }
+extern "C" int glqh_version(void) { return 1; }
+
+extern "C" int glqh_init(void) {
+    std::call_once(g_once, [] {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (glqh_check_hip(hipGetDevice(&dev), "hipGetDevice") ||
+            glqh_check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties")) {
+            g_init_rc = 1;
+            return;
+        }
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+            g_init_rc = glqh_fail("libglq_hip is built for gfx950 only, device is %s", prop.gcnArchName);
+            return;
+        }
+        g_cus = prop.multiProcessorCount;
+        g_init_rc = glqh_rht_init() || glqh_e8_init();
+    });
+    if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
+    return g_init_rc;
+}
+
+#define GLQH_INIT()                      \
+    do {                                 \
+        if (glqh_init() != 0) return 1;  \
+    } while (0)
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// ---- trellis ---------------------------------------------------------------------
+extern "C" int glqh_trellis_kernel_supported(int64_t m, int64_t k) {
+    return m > 0 && k > 0 && m % 32 == 0 && k % 64 == 0;
+}
+
+static int tr_bits_from_packed(int64_t packed_cols, int allow_r1, int *R) {
+    int r = (int)(packed_cols / 16);
+    int lo = allow_r1 ? 1 : 2;
+    GLQH_REQUIRE(packed_cols % 16 == 0 && r >= lo && r <= 4,
+                 "trellis kernel supports R (bits/weight) %d-4, got packed width %lld", lo,
+                 (long long)packed_cols);
+    *R = r;
+    return 0;
+}
+
+static int tr_check_shape(int64_t m, int64_t k, int64_t packed_rows) {
+    GLQH_REQUIRE(m > 0 && m % 32 == 0, "trellis kernel needs m %% 32 == 0, got %lld", (long long)m);
+    GLQH_REQUIRE(k > 0 && k % 64 == 0, "trellis kernel needs k %% 64 == 0, got %lld", (long long)k);
+    GLQH_REQUIRE(packed_rows == (m / 16) * (k / 16), "trellis_packed rows %lld != (m/16)*(k/16)",
+                 (long long)packed_rows);
+    GLQH_REQUIRE(m / 32 <= 65535, "trellis kernel: m too large");
+    return 0;
+}
+
+extern "C" int glqh_decompress_trellis_3inst(const void *packed, int64_t packed_rows,
+                                             int64_t packed_cols, int64_t m, int64_t k, int allow_r1,
+                                             void *out_f16, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(packed && out_f16, "decompress: null pointer");
+    int R;
+    if (tr_bits_from_packed(packed_cols, allow_r1, &R) || tr_check_shape(m, k, packed_rows)) return 1;
+    return glqh_launch_trellis_decompress(packed, R, m, k, out_f16, (hipStream_t)stream);
+}
+
+extern "C" size_t glqh_trellis_gemv_workspace_bytes(int64_t m, int64_t k, int64_t B) {
+    if (!glqh_trellis_kernel_supported(m, k) || B < 1) return 0;
+    glqh_init();
+    int ks = glqh_trellis_pick_ksplit(m, k, B);
+    return ks > 1 ? align256((size_t)ks * B * m * sizeof(float)) : 0;
+}
+
+extern "C" int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B, const void *packed,
+                                                int64_t packed_rows, int64_t packed_cols, int64_t m,
+                                                int64_t k, double wscale, float *out,
+                                                int64_t out_stride, int accum, void *ws,
+                                                size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x_f16 && packed && out, "trellis matmul: null pointer");
+    GLQH_REQUIRE(B >= 1 && B <= 65535 * 8, "trellis matmul: B=%lld out of range", (long long)B);
+    GLQH_REQUIRE(out_stride >= m, "trellis matmul: out stride %lld < m", (long long)out_stride);
+    int R;
+    if (tr_bits_from_packed(packed_cols, accum, &R) || tr_check_shape(m, k, packed_rows)) return 1;
+    hipStream_t st = (hipStream_t)stream;
+    int ks = glqh_trellis_pick_ksplit(m, k, B);
+    if (ks == 1)
+        return glqh_launch_trellis_direct(x_f16, B, packed, R, m, k, (float)wscale, out, out_stride,
+                                          accum, st);
+    size_t need = (size_t)ks * B * m * sizeof(float);
+    GLQH_REQUIRE(ws && ws_bytes >= need, "trellis matmul: workspace of %zu bytes needed, got %zu", need,
+                 ws_bytes);
+    if (glqh_launch_trellis_partial(x_f16, B, packed, R, m, k, ks, (float *)ws, st)) return 1;
+    return glqh_launch_reduce_splits((const float *)ws, ks, B * m, B, m, (float)wscale, out, out_stride, accum, st);
+}
+
+// ---- RHT -------------------------------------------------------------------------
+extern "C" int glqh_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv_f16,
+                              void *out, int out_dtype, int64_t B, int64_t in_features,
+                              int64_t n_pad, const glqh_block_meta *meta_dev,
+                              const int64_t *blocks_host, int64_t n_blocks, double rsqrt_n,
+                              void *stream) {
+    GLQH_INIT();
+    return glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, out, out_dtype, B, in_features, n_pad,
+                                 meta_dev, blocks_host, n_blocks, (float)rsqrt_n, (hipStream_t)stream);
+}
+
+extern "C" int glqh_output_rht(const float *y_rht, int64_t y_rht_stride, const void *su_f16, void *y,
+                               int y_dtype, int64_t y_stride, int64_t B, int64_t out_features,
+                               int64_t m_pad, const glqh_block_meta *meta_dev,
+                               const int64_t *blocks_host, int64_t n_blocks, double rsqrt_m,
+                               void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(y_rht && y, "output_rht: null pointer");
+    GLQH_REQUIRE(y_rht_stride >= m_pad && y_stride >= out_features, "output_rht: bad strides");
+    glqh_ysrc src = {};
+    src.direct = y_rht;
+    src.stride = y_rht_stride;
+    return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, meta_dev,
+                                  blocks_host, n_blocks, 0, (float)rsqrt_m, (hipStream_t)stream);
+}
+
+extern "C" int glqh_output_rht_shards(const float *y_rht, const void *su_f16, void *y, int y_dtype,
+                                      int64_t B, int64_t out_features, int64_t total_m,
+                                      const glqh_block_meta *shard_meta_dev, int64_t n_rows,
+                                      int64_t max_bs, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(y_rht && y && shard_meta_dev, "output_rht_shards: null pointer");
+    GLQH_REQUIRE(n_rows >= 1 && n_rows <= 65535, "output_rht_shards: %lld meta rows", (long long)n_rows);
+    GLQH_REQUIRE(max_bs >= 1 && max_bs <= total_m, "output_rht_shards: max_bs %lld out of range",
+                 (long long)max_bs);
+    glqh_ysrc src = {};
+    src.direct = y_rht;
+    src.stride = total_m;
+    return glqh_launch_output_rht(src, su_f16, y, y_dtype, out_features, B, out_features, total_m,
+                                  shard_meta_dev, nullptr, n_rows, max_bs, 0.0f, (hipStream_t)stream);
+}
+
+// ---- fused trellis linear ----------------------------------------------------------
+// workspace layout: [x_rht f16 (B, n_pad)] [partials stage 1] [partials stage 2]
+static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
+    int ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
+    return align256((size_t)ks * B * m_pad * sizeof(float));
+}
+
+extern "C" size_t glqh_fused_linear_trellis_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
+    if (!glqh_trellis_kernel_supported(m_pad, n_pad) || B < 1) return 0;
+    glqh_init();
+    return align256((size_t)B * n_pad * sizeof(f16)) + 2 * tr_fused_part_bytes(B, n_pad, m_pad);
+}
+
+extern "C" int glqh_fused_linear_trellis_3inst(
+    const void *x, int x_dtype, int64_t x_stride, int64_t B, const void *sv_f16, const void *su_f16,
+    const void *packed, int64_t packed_rows, int64_t packed_cols, const void *packed2,
+    int64_t packed2_rows, int64_t packed2_cols, const int64_t *blocks_n, int64_t n_blocks_n,
+    const int64_t *blocks_m, int64_t n_blocks_m, const glqh_block_meta *bn_meta_dev,
+    const glqh_block_meta *bm_meta_dev, double wscale, double inv_resid_scale2, int64_t in_features,
+    int64_t out_features, int64_t n_pad, int64_t m_pad, void *y, int y_dtype, int64_t y_stride,
+    float *y_rht_out, int64_t y_rht_stride, void *ws, size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x && sv_f16 && packed, "fused trellis linear: null pointer");
+    GLQH_REQUIRE(y || y_rht_out, "fused trellis linear: no output buffer");
+    GLQH_REQUIRE(!y || su_f16, "fused trellis linear: null su");
+    GLQH_REQUIRE(B >= 1 && B <= 65535, "fused trellis linear: B=%lld out of range", (long long)B);
+    const bool has_s2 = packed2 != nullptr && packed2_rows > 0;
+    GLQH_REQUIRE(has_s2 == (inv_resid_scale2 != 0.0),
+                 "trellis RVQ stage 2 is half-configured: trellis_packed2 is %s but inv_resid_scale2 = %g. "
+                 "Refusing rather than silently decoding stage 1 only.",
+                 has_s2 ? "present" : "absent", inv_resid_scale2);
+    int R1, R2 = 0;
+    if (tr_bits_from_packed(packed_cols, 0, &R1) || tr_check_shape(m_pad, n_pad, packed_rows)) return 1;
+    if (has_s2 && (tr_bits_from_packed(packed2_cols, 1, &R2) || tr_check_shape(m_pad, n_pad, packed2_rows)))
+        return 1;
+    GLQH_REQUIRE(in_features <= n_pad && out_features <= m_pad, "fused trellis linear: features exceed padded dims");
+    GLQH_REQUIRE(!y_rht_out || y_rht_stride >= m_pad, "fused trellis linear: y_rht stride %lld < m_pad",
+                 (long long)y_rht_stride);
+    hipStream_t st = (hipStream_t)stream;
+
+    const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
+    const size_t pb = tr_fused_part_bytes(B, n_pad, m_pad);
+    GLQH_REQUIRE(ws && ws_bytes >= xb + 2 * pb, "fused trellis linear: workspace of %zu bytes needed, got %zu",
+                 xb + 2 * pb, ws_bytes);
+    f16 *x_rht = (f16 *)ws;
+    float *part1 = (float *)((char *)ws + xb);
+    float *part2 = (float *)((char *)ws + xb + pb);
+
+    if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
+                              bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
+        return 1;
+    const int ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
+    if (glqh_launch_trellis_partial(x_rht, B, packed, R1, m_pad, n_pad, ks, part1, st)) return 1;
+    if (has_s2 && glqh_launch_trellis_partial(x_rht, B, packed2, R2, m_pad, n_pad, ks, part2, st)) return 1;
+
+    const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);
+    if (!y) {
+        // stop at the RHT-domain product: combine the split-K partials into the caller's rows
+        if (glqh_launch_reduce_splits(part1, ks, B * m_pad, B, m_pad, s1, y_rht_out, y_rht_stride, 0, st)) return 1;
+        if (has_s2 && glqh_launch_reduce_splits(part2, ks, B * m_pad, B, m_pad, s2, y_rht_out, y_rht_stride, 1, st))
+            return 1;
+        return 0;
+    }
+    glqh_ysrc src = {};
+    src.nparts = has_s2 ? 2 : 1;
+    src.part[0] = part1;
+    src.part[1] = part2;
+    src.part_kstride = B * m_pad;
+    src.ksplit = ks;
+    src.scale[0] = s1;
+    src.scale[1] = s2;
+    src.copy_out = y_rht_out;
+    src.copy_stride = y_rht_stride;
+    return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,
+                                  blocks_m, n_blocks_m, 0, 0.0f, st);
+}
+
+// ---- E8 shell ------------------------------------------------------------------------
+extern "C" int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, uint32_t *packed_out,
+                                  int32_t *bad_dev, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(codebook_f16 && packed_out && bad_dev, "e8 pack table: null pointer");
+    GLQH_REQUIRE(n_entries >= 1 && n_entries <= 65536, "e8 pack table: %lld entries (1..65536)",
+                 (long long)n_entries);
+    return glqh_launch_e8_pack_table(codebook_f16, n_entries, packed_out, bad_dev, (hipStream_t)stream);
+}
+
+struct e8_stages {
+    const void *q[4];
+    float scale[4];
+    int n;
+};
+
+static int e8_resolve_stages(const void *q1, const void *q2, const void *q3, const void *q4,
+                             double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                             const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                             e8_stages *out) {
+    GLQH_REQUIRE(q1 && table1, "e8 matmul: null index or table pointer");
+    out->q[0] = q1; out->q[1] = q1; out->q[2] = q1; out->q[3] = q1;
+    out->scale[0] = (float)wscale;
+    out->n = 1;
+    if (q2 && inv_rs != 0.0) {
+        GLQH_REQUIRE(table2 && n_entries2 >= 1 && n_entries2 <= 65536,
+                     "e8 matmul: stage 2 needs its table (1..65536 entries)");
+        out->q[1] = q2;
+        out->scale[1] = (float)(wscale * inv_rs);
+        out->n = 2;
+        if (q3 && inv_rs2 != 0.0) {
+            out->q[2] = q3;
+            out->scale[2] = (float)(wscale * inv_rs2);
+            out->n = 3;
+            if (q4 && inv_rs3 != 0.0) {
+                out->q[3] = q4;
+                out->scale[3] = (float)(wscale * inv_rs3);
+                out->n = 4;
+            }
+        }
+    }
+    return 0;
+}
+
+static int e8_check_dims(int64_t m_pad, int64_t n_pad, int64_t B) {
+    GLQH_REQUIRE(m_pad >= 1 && n_pad >= 8 && n_pad % 8 == 0, "e8 matmul: n_pad %lld must be a multiple of 8",
+                 (long long)n_pad);
+    GLQH_REQUIRE(B >= 1 && B <= 65535 * 4, "e8 matmul: B=%lld out of range", (long long)B);
+    GLQH_REQUIRE((m_pad + 31) / 32 <= 2147483647ll, "e8 matmul: m_pad too large");
+    return 0;
+}
+
+static size_t e8_part_bytes(int64_t m_pad, int64_t n_pad, int64_t B) {
+    int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    return align256((size_t)ks * 4 * B * m_pad * sizeof(float));
+}
+
+extern "C" size_t glqh_e8_matmul_workspace_bytes(int64_t m_pad, int64_t n_pad, int64_t B) {
+    if (m_pad < 1 || n_pad < 8 || B < 1) return 0;
+    glqh_init();
+    return e8_part_bytes(m_pad, n_pad, B);
+}
+
+extern "C" int glqh_e8_dequant_matmul(const void *x_f16, int64_t B, const void *q1, const void *q2,
+                                      const void *q3, const void *q4, const uint32_t *table1,
+                                      const uint32_t *table2, int64_t n_entries2, double wscale,
+                                      double inv_rs, double inv_rs2, double inv_rs3, int64_t m_pad,
+                                      int64_t n_pad, float *out, void *ws, size_t ws_bytes,
+                                      void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x_f16 && out, "e8 matmul: null pointer");
+    e8_stages sg;
+    if (e8_check_dims(m_pad, n_pad, B) ||
+        e8_resolve_stages(q1, q2, q3, q4, wscale, inv_rs, inv_rs2, inv_rs3, table1, table2, n_entries2, &sg))
+        return 1;
+    const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    const size_t need = (size_t)ks * sg.n * B * m_pad * sizeof(float);
+    GLQH_REQUIRE(ws && ws_bytes >= need, "e8 matmul: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    float *part = (float *)ws;
+    if (glqh_launch_e8_partial(x_f16, B, sg.q, sg.n, table1, table2 ? table2 : table1,
+                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st))
+        return 1;
+    for (int s = 0; s < sg.n; ++s)
+        if (glqh_launch_reduce_splits(part + (int64_t)s * B * m_pad, ks, (int64_t)sg.n * B * m_pad, B, m_pad,
+                                      sg.scale[s], out, m_pad, s > 0, st))
+            return 1;
+    return 0;
+}
+
+extern "C" size_t glqh_fused_linear_e8_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
+    if (m_pad < 1 || n_pad < 8 || B < 1) return 0;
+    glqh_init();
+    return align256((size_t)B * n_pad * sizeof(f16)) + e8_part_bytes(m_pad, n_pad, B);
+}
+
+extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                    const void *sv_f16, const void *su_f16, const void *q1,
+                                    const void *q2, const void *q3, const void *q4,
+                                    const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                    double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                                    const int64_t *blocks_n, int64_t n_blocks_n, const int64_t *blocks_m,
+                                    int64_t n_blocks_m, const glqh_block_meta *bn_meta_dev,
+                                    const glqh_block_meta *bm_meta_dev, int64_t in_features,
+                                    int64_t out_features, int64_t n_pad, int64_t m_pad, void *y,
+                                    int y_dtype, int64_t y_stride, void *ws, size_t ws_bytes,
+                                    void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x && sv_f16 && su_f16 && y, "fused e8 linear: null pointer");
+    e8_stages sg;
+    if (e8_check_dims(m_pad, n_pad, B) ||
+        e8_resolve_stages(q1, q2, q3, q4, wscale, inv_rs, inv_rs2, inv_rs3, table1, table2, n_entries2, &sg))
+        return 1;
+    GLQH_REQUIRE(B <= 65535, "fused e8 linear: B=%lld out of range", (long long)B);
+    GLQH_REQUIRE(in_features <= n_pad && out_features <= m_pad, "fused e8 linear: features exceed padded dims");
+    const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
+    const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    const size_t need = xb + (size_t)ks * sg.n * B * m_pad * sizeof(float);
+    GLQH_REQUIRE(ws && ws_bytes >= need, "fused e8 linear: workspace of %zu bytes needed, got %zu", need,
+                 ws_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    f16 *x_rht = (f16 *)ws;
+    float *part = (float *)((char *)ws + xb);
+    if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
+                              bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
+        return 1;
+    if (glqh_launch_e8_partial(x_rht, B, sg.q, sg.n, table1, table2 ? table2 : table1,
+                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st))
+        return 1;
+    glqh_ysrc src = {};
+    src.nparts = sg.n;
+    for (int s = 0; s < sg.n; ++s) {
+        src.part[s] = part + (int64_t)s * B * m_pad;
+        src.scale[s] = sg.scale[s];
+    }
+    src.part_kstride = (int64_t)sg.n * B * m_pad;
+    src.ksplit = ks;
+    return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,
+                                  blocks_m, n_blocks_m, 0, 0.0f, st);
+}

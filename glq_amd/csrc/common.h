@@ -1,0 +1,102 @@
+// Shared host/device helpers for libglq_hip (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/glq_hip.h"
+
+typedef _Float16 f16;
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define GLQH_WAVE 64
+#define GLQH_MAX_LDS_BYTES (160 * 1024)
+
+// ---- error reporting (host) -------------------------------------------------
+int glqh_fail(const char *fmt, ...);             // sets the thread-local message, returns 1
+int glqh_check_hip(hipError_t e, const char *what);
+int glqh_device_cus(void);                       // cached compute-unit count
+
+#define GLQH_REQUIRE(cond, ...)            \
+    do {                                   \
+        if (!(cond)) return glqh_fail(__VA_ARGS__); \
+    } while (0)
+
+#define GLQH_LAUNCH_CHECK(what)                                   \
+    do {                                                          \
+        int rc_ = glqh_check_hip(hipGetLastError(), what);        \
+        if (rc_) return rc_;                                      \
+    } while (0)
+
+// ---- small device helpers -----------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) {
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {   // round-to-nearest-even
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);   // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_act(const void *p, int dtype, int64_t i) {
+    if (dtype == GLQH_F16) return (float)((const f16 *)p)[i];
+    if (dtype == GLQH_BF16) return bf16_bits_to_f32(((const uint16_t *)p)[i]);
+    return ((const float *)p)[i];
+}
+
+__device__ __forceinline__ void store_act(void *p, int dtype, int64_t i, float v) {
+    if (dtype == GLQH_F16) ((f16 *)p)[i] = (f16)v;
+    else if (dtype == GLQH_BF16) ((uint16_t *)p)[i] = f32_to_bf16_bits(v);
+    else ((float *)p)[i] = v;
+}
+
+// internal kernels' host launchers (defined in fht.hip / trellis.hip / e8.hip)
+struct glqh_ysrc {                 // where the output RHT reads its RHT-domain input
+    const float *direct;           // (B, stride) fp32, or NULL when partials are used
+    int64_t stride;                // row stride of `direct`
+    const float *part[4];          // split-K partial sums per stage: element (k, b, row) at
+                                   // part[st][k * part_kstride + b * m_pad + row]
+    int64_t part_kstride;
+    int ksplit;
+    float scale[4];                // wscale per stage (already multiplied by inv_rs)
+    int nparts;
+    float *copy_out;               // optional: also write the combined fp32 row here
+    int64_t copy_stride;
+};
+
+int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv,
+                          void *out, int out_dtype, int64_t B, int64_t in_features, int64_t n_pad,
+                          const glqh_block_meta *meta_dev, const int64_t *blocks_host,
+                          int64_t n_blocks, float rsqrt_n, hipStream_t stream);
+
+int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_dtype,
+                           int64_t y_stride, int64_t B, int64_t out_features, int64_t m_pad,
+                           const glqh_block_meta *meta_dev, const int64_t *blocks_host,
+                           int64_t n_blocks, int64_t max_bs_hint, float rsqrt_m,
+                           hipStream_t stream);
+
+// trellis GEMV/GEMM into split-K partials (or directly into `out` when ksplit == 1)
+int glqh_trellis_pick_ksplit(int64_t m, int64_t k, int64_t B);
+int glqh_launch_trellis_partial(const void *x_f16, int64_t B, const void *packed, int R,
+                                int64_t m, int64_t k, int ksplit, float *part,
+                                hipStream_t stream);
+// out[tok, row] = (accum ? out : 0) + scale * sum_s part[s * kstride + tok * m + row]
+int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, int64_t B, int64_t m,
+                              float scale, float *out, int64_t out_stride, int accum,
+                              hipStream_t stream);
+
+// E8 gather matmul into per-stage split-K partials:
+// part[((slot * nstages + stage) * B + tok) * m_pad + row]
+int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B);
+int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, int32_t *bad,
+                              hipStream_t stream);
+int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
+                           const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
+                           int64_t n_pad, int ksplit, float *part, hipStream_t stream);

@@ -1,0 +1,200 @@
+// E8 shell codebook: table packing and gather GEMV / small-batch GEMM (gfx950).
+//
+// Weight row i, columns 8j..8j+7 = table[u16(Qidxs[i,j])] (+ residual stages scaled by
+// cumulative 1/resid_scale), glq/codebook.py:280-282, glq/quantized_linear.py:1177-1194.
+// Every table coordinate is one of the 13 values -3, -2.5, ..., 3, so a row packs into
+// eight 4-bit codes n = 2v + 6 (glq/codebook.py:102-115).  The packed word used here
+// interleaves the codes so that one mask yields two adjacent columns:
+//     nibble p     = code of column 2p
+//     nibble p + 4 = code of column 2p + 1            (p = 0..3)
+// and (word >> 4p) & 0x000F000F | 0x60006000 is the fp16 pair (512 + n/2) of columns
+// (2p, 2p+1); subtracting 515 gives the exact coordinates.
+//
+// Work split: eight lanes share a row (one 16-byte run of 8 indices = 64 columns per
+// lane and step), a wave covers 8 rows, a workgroup 32.  K is split over gridDim.y; the
+// partial sums of each stage go to a scratch array and are combined in a fixed order by
+// the consumer, so outputs are bit-identical from run to run.
+#include "common.h"
+
+namespace {
+
+constexpr int E8_THREADS = 256;
+constexpr int E8_ROWS_PER_WG = 32;
+
+__global__ void __launch_bounds__(256)
+e8_pack_table_kernel(const f16 *__restrict__ cb, int n_entries, uint32_t *__restrict__ out,
+                     int32_t *__restrict__ bad) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_entries) return;
+    uint32_t word = 0;
+    bool ok = true;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        float v = (float)cb[(int64_t)i * 8 + c];
+        float n = 2.0f * v + 6.0f;
+        int code = (int)n;
+        ok = ok && (n == (float)code) && code >= 0 && code <= 12;
+        const int pos = (c >> 1) + 4 * (c & 1);
+        word |= (uint32_t)(code & 15) << (4 * pos);
+    }
+    out[i] = word;
+    if (!ok) atomicAdd(bad, 1);
+}
+
+__device__ __forceinline__ f16x2 e8_pair(uint32_t word, int p) {
+    uint32_t u = ((word >> (4 * p)) & 0x000F000Fu) | 0x60006000u;
+    f16x2 v = __builtin_bit_cast(f16x2, u);
+    const f16x2 off = {(f16)515.0f, (f16)515.0f};
+    return v - off;
+}
+
+// grid = (ceil(m_pad/32), ksplit, ceil(B/NB)).  part[((slot*NS + stage)*B + tok)*m_pad + row]
+template <int NS, int NB>
+__global__ void __launch_bounds__(E8_THREADS)
+e8_gemv_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
+               const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
+               const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n2,
+               const f16 *__restrict__ x, int B, int m_pad, int n_pad, float *__restrict__ part) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int c = lane & 7;
+    const int row = blockIdx.x * E8_ROWS_PER_WG + wave * 8 + (lane >> 3);
+    const bool row_ok = row < m_pad;
+    const int nblk = n_pad >> 3;                      // 8-column blocks per row
+    const int nchunks = (nblk + 7) >> 3;              // 64-column chunks (last may be ragged)
+    const int tok0 = blockIdx.z * NB;
+    const bool vec_ok = (nblk & 7) == 0;              // rows are 16-byte aligned runs
+
+    float acc[NB][NS];
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int s = 0; s < NS; ++s) acc[t][s] = 0.0f;
+
+    const uint16_t *qs[4] = {q1, q2, q3, q4};
+    const int64_t rbase = (int64_t)(row_ok ? row : 0) * nblk;
+
+    for (int ch = blockIdx.y * 8 + c; ch < nchunks; ch += gridDim.y * 8) {
+        uint32_t idxw[NS][4];                          // 8 indices per stage, two per word
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const uint16_t *qp = qs[s] + rbase + 8 * ch;
+            if (vec_ok) {
+                u32x4 v = __builtin_nontemporal_load((const u32x4 *)qp);
+                idxw[s][0] = v.x; idxw[s][1] = v.y; idxw[s][2] = v.z; idxw[s][3] = v.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int b0 = 8 * ch + 2 * e;
+                    uint32_t lo = b0 < nblk ? qp[2 * e] : 0u;
+                    uint32_t hi = b0 + 1 < nblk ? qp[2 * e + 1] : 0u;
+                    idxw[s][e] = lo | (hi << 16);
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int blk = 8 * ch + e;
+            const bool live_blk = blk < nblk;          // only the ragged tail can be false
+            uint32_t word[NS];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                uint32_t idx = (idxw[s][e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                if (s == 1) {
+                    idx = idx < n2 ? idx : n2 - 1;
+                    word[s] = t2[idx];
+                } else {
+                    word[s] = t1[idx];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NB; ++t) {
+                const int tok = tok0 + t;
+                u32x4 xv = {0u, 0u, 0u, 0u};
+                if (tok < B && live_blk) xv = *(const u32x4 *)(x + (int64_t)tok * n_pad + 8 * blk);
+                const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+#pragma unroll
+                    for (int p = 0; p < 4; ++p)
+                        acc[t][s] = __builtin_amdgcn_fdot2(e8_pair(word[s], p),
+                                                           __builtin_bit_cast(f16x2, xw[p]),
+                                                           acc[t][s], false);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            float v = acc[t][s];
+            v += __shfl_xor(v, 1, GLQH_WAVE);
+            v += __shfl_xor(v, 2, GLQH_WAVE);
+            v += __shfl_xor(v, 4, GLQH_WAVE);
+            const int tok = tok0 + t;
+            if (c == 0 && row_ok && tok < B)
+                part[(((int64_t)blockIdx.y * NS + s) * B + tok) * m_pad + row] = v;
+        }
+}
+
+template <int NS>
+int launch_e8_NS(const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
+                 const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, int ksplit,
+                 float *part, hipStream_t stream) {
+    const unsigned gx = (unsigned)((m_pad + E8_ROWS_PER_WG - 1) / E8_ROWS_PER_WG);
+    const uint16_t *q1 = (const uint16_t *)q[0], *q2 = (const uint16_t *)q[1];
+    const uint16_t *q3 = (const uint16_t *)q[2], *q4 = (const uint16_t *)q[3];
+    const f16 *xp = (const f16 *)x;
+    if (B == 1) {
+        hipLaunchKernelGGL((e8_gemv_kernel<NS, 1>), dim3(gx, ksplit, 1), dim3(E8_THREADS), 0, stream, q1,
+                           q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B, (int)m_pad, (int)n_pad, part);
+    } else if (B <= 2) {
+        hipLaunchKernelGGL((e8_gemv_kernel<NS, 2>), dim3(gx, ksplit, 1), dim3(E8_THREADS), 0, stream, q1,
+                           q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B, (int)m_pad, (int)n_pad, part);
+    } else {
+        hipLaunchKernelGGL((e8_gemv_kernel<NS, 4>), dim3(gx, ksplit, (unsigned)((B + 3) / 4)),
+                           dim3(E8_THREADS), 0, stream, q1, q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B,
+                           (int)m_pad, (int)n_pad, part);
+    }
+    GLQH_LAUNCH_CHECK("e8 gemv launch");
+    return 0;
+}
+
+}  // namespace
+
+int glqh_e8_init(void) { return 0; }
+
+// Shape-only K-split (independent of the token count): batched rows sum like the GEMV.
+int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B) {
+    (void)B;
+    const int64_t wgs = (m_pad + E8_ROWS_PER_WG - 1) / E8_ROWS_PER_WG;
+    const int64_t target = (int64_t)glqh_device_cus() * 4;
+    int64_t ks = (target + wgs - 1) / wgs;
+    int64_t cap = ((n_pad / 8 + 7) / 8) / 8;             // every lane gets at least one chunk
+    if (cap < 1) cap = 1;
+    if (ks > cap) ks = cap;
+    if (ks > 32) ks = 32;
+    if (ks < 1) ks = 1;
+    return (int)ks;
+}
+
+int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, int32_t *bad,
+                              hipStream_t stream) {
+    hipLaunchKernelGGL(e8_pack_table_kernel, dim3((unsigned)((n_entries + 255) / 256)), dim3(256), 0,
+                       stream, (const f16 *)cb, (int)n_entries, out, bad);
+    GLQH_LAUNCH_CHECK("e8 pack table launch");
+    return 0;
+}
+
+int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
+                           const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
+                           int64_t n_pad, int ksplit, float *part, hipStream_t stream) {
+    switch (nstages) {
+    case 1: return launch_e8_NS<1>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
+    case 2: return launch_e8_NS<2>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
+    case 3: return launch_e8_NS<3>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
+    case 4: return launch_e8_NS<4>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
+    }
+    return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
+}

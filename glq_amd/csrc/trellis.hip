@@ -1,0 +1,350 @@
+// Trellis-3INST decode, GEMV and small-batch GEMM for gfx950 (wave64).
+//
+// Storage (one layer (m,k), R bits per weight, R = packed width / 16):
+//   * 16x16 tiles; a tile is a cyclic stream of 256*R bits; trellis step t has the
+//     16-bit state = stream bits [R t, R t + 16) and the weight decode_3inst(state)
+//     (glq/trellis.py:122-134, 486-523).
+//   * step t = 8 l + j sits at row (l>>2) + 8*((j>>1)&1), col 2*(l&3) + 8*(j>>2) + (j&1)
+//     of its tile (glq/trellis.py:99-101).
+//   * tiles are stored in 2x2 blocks (m-pair mp, k-pair kp), blocks ordered mp-major.
+//     Inside a block, "stream lane" l in [0,32) owns one 4R-byte record holding its
+//     8R-bit chunk of the four tiles in the order (k0,m0),(k0,m1),(k1,m0),(k1,m1), each
+//     chunk little-endian with its most significant bit first in the stream
+//     (glq/trellis.py:580-602).  A lane needs 16 more bits: the top of lane l+1's chunk
+//     (R = 1: lanes l+1 and l+2), wrapping at 32.
+//
+// Mapping to the hardware: one wave64 step covers two adjacent blocks of the same
+// m-pair -- lanes 0..31 take block (mp, 2q), lanes 32..63 block (mp, 2q+1) -- so a wave
+// reads 256*R contiguous bytes with one load instruction per lane, rotates the
+// continuation bits inside each 32-lane half with one cross-lane permute per two
+// chunks, decodes 32 weights per lane in registers and multiplies them against the
+// activations with fp32 accumulation.  Every output row is owned by one workgroup per
+// K-split slot and summed in a fixed order, so results are bit-identical run to run.
+#include "common.h"
+
+namespace {
+
+constexpr int TR_WAVES = 4;
+constexpr int TR_THREADS = TR_WAVES * GLQH_WAVE;
+
+// (s * 89226354 + 64248484) mod 2^32, masked and xored: the two fp16 halves of 3INST.
+__device__ __forceinline__ uint32_t tr_hash(uint32_t s) {
+    uint32_t h = s * 89226354u + 64248484u;
+    return (h & 0x8FFF8FFFu) ^ 0x3B603B60u;
+}
+
+// Exact reference weight: the two halves added in fp16 with one rounding.
+__device__ __forceinline__ f16 tr_weight(uint32_t s) {
+    f16x2 r = __builtin_bit_cast(f16x2, tr_hash(s));
+    return r.y + r.x;
+}
+
+template <int R>
+struct tr_record {
+    uint32_t c[4];      // 8R-bit chunks of tiles (k0,m0),(k0,m1),(k1,m0),(k1,m1)
+    uint32_t raw;       // R == 1 only: the four 8-bit chunks as loaded
+};
+
+template <int R>
+__device__ __forceinline__ tr_record<R> tr_load_record(const uint8_t *__restrict__ p) {
+    tr_record<R> r;
+    r.raw = 0;
+    if constexpr (R == 4) {
+        u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
+        r.c[0] = v.x; r.c[1] = v.y; r.c[2] = v.z; r.c[3] = v.w;
+    } else if constexpr (R == 3) {
+        const uint32_t *q = (const uint32_t *)p;
+        uint32_t r0 = __builtin_nontemporal_load(q);
+        uint32_t r1 = __builtin_nontemporal_load(q + 1);
+        uint32_t r2 = __builtin_nontemporal_load(q + 2);
+        r.c[0] = r0 & 0xFFFFFFu;
+        r.c[1] = ((r0 >> 24) | (r1 << 8)) & 0xFFFFFFu;
+        r.c[2] = ((r1 >> 16) | (r2 << 16)) & 0xFFFFFFu;
+        r.c[3] = r2 >> 8;
+    } else if constexpr (R == 2) {
+        u32x2 v = __builtin_nontemporal_load((const u32x2 *)p);
+        r.c[0] = v.x & 0xFFFFu; r.c[1] = v.x >> 16;
+        r.c[2] = v.y & 0xFFFFu; r.c[3] = v.y >> 16;
+    } else {
+        uint32_t v = __builtin_nontemporal_load((const uint32_t *)p);
+        r.raw = v;
+        r.c[0] = v & 0xFFu; r.c[1] = (v >> 8) & 0xFFu;
+        r.c[2] = (v >> 16) & 0xFFu; r.c[3] = v >> 24;
+    }
+    return r;
+}
+
+// 16 continuation bits per chunk, fetched from the next stream lane(s) of the same
+// 32-lane half.
+template <int R>
+__device__ __forceinline__ void tr_continuation(const tr_record<R> &r, int lane, uint32_t cont[4]) {
+    const int half = lane & 32;
+    const int next1 = half | ((lane + 1) & 31);
+    if constexpr (R >= 2) {
+        constexpr int sh = 8 * R - 16;
+        uint32_t t01 = ((r.c[0] >> sh) & 0xFFFFu) | (((r.c[1] >> sh) & 0xFFFFu) << 16);
+        uint32_t t23 = ((r.c[2] >> sh) & 0xFFFFu) | (((r.c[3] >> sh) & 0xFFFFu) << 16);
+        uint32_t n01 = (uint32_t)__shfl((int)t01, next1, GLQH_WAVE);
+        uint32_t n23 = (uint32_t)__shfl((int)t23, next1, GLQH_WAVE);
+        cont[0] = n01 & 0xFFFFu; cont[1] = n01 >> 16;
+        cont[2] = n23 & 0xFFFFu; cont[3] = n23 >> 16;
+    } else {
+        const int next2 = half | ((lane + 2) & 31);
+        uint32_t a = (uint32_t)__shfl((int)r.raw, next1, GLQH_WAVE);
+        uint32_t b = (uint32_t)__shfl((int)r.raw, next2, GLQH_WAVE);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            cont[i] = (((a >> (8 * i)) & 0xFFu) << 8) | ((b >> (8 * i)) & 0xFFu);
+    }
+}
+
+template <int R>
+__device__ __forceinline__ uint32_t tr_state(uint32_t chunk, uint32_t cont, int j) {
+    uint64_t ext = ((uint64_t)chunk << 16) | cont;
+    return (uint32_t)(ext >> (8 * R - R * j)) & 0xFFFFu;
+}
+
+// ---------------------------------------------------------------------------------
+// decompress: packed -> dense fp16 (m,k), bit-exact with the reference dequantizer
+// ---------------------------------------------------------------------------------
+template <int R>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_decompress_kernel(const uint8_t *__restrict__ packed, f16 *__restrict__ W, int m, int k) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nsteps = k >> 6;
+    const int q = blockIdx.x * TR_WAVES + wave;
+    if (q >= nsteps) return;                               // whole wave exits together
+    const int mp = blockIdx.y;
+    const int l = lane & 31;
+    const int kp = 2 * q + (lane >> 5);
+    const int64_t rec = ((int64_t)mp * (k >> 5) + kp) * 32 + l;
+    tr_record<R> r = tr_load_record<R>(packed + rec * (4 * R));
+    uint32_t cont[4];
+    tr_continuation<R>(r, lane, cont);
+    const int a = l >> 2, b = l & 3;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) {
+            const int ci = ks * 2 + ms;
+            const int row0 = 32 * mp + 16 * ms + a;
+            const int col0 = 32 * kp + 16 * ks + 2 * b;
+#pragma unroll
+            for (int jp = 0; jp < 4; ++jp) {               // states 2jp, 2jp+1: adjacent columns
+                f16x2 w;
+                w.x = tr_weight(tr_state<R>(r.c[ci], cont[ci], 2 * jp));
+                w.y = tr_weight(tr_state<R>(r.c[ci], cont[ci], 2 * jp + 1));
+                const int row = row0 + 8 * (jp & 1);
+                const int col = col0 + 8 * (jp >> 1);
+                *(f16x2 *)(W + (int64_t)row * k + col) = w;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// GEMV / small-batch GEMM against the packed stream
+// ---------------------------------------------------------------------------------
+// grid = (m/32, ksplit, ceil(B/NB)); each workgroup owns one m-pair (32 rows) for NB
+// tokens and a round-robin share of the k/64 wave-steps.  Output: raw fp32 sums to
+// part[(slot*B + token)*m + row], or (direct) scaled into out.
+template <int R, int NB>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_gemv_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int B, int m, int k,
+               float *__restrict__ part, int direct, float scale, int accum, int64_t out_stride) {
+    __shared__ float red[TR_WAVES][NB][32];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int l = lane & 31;
+    const int hf = lane >> 5;
+    const int a = l >> 2, b = l & 3;
+    const int mp = blockIdx.x;
+    const int nsteps = k >> 6;
+    const int stride = gridDim.y * TR_WAVES;
+    const int tok0 = blockIdx.z * NB;
+
+    float acc[NB][4];
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i] = 0.0f;
+
+    const uint8_t *row_base = packed + (int64_t)mp * (k >> 5) * 32 * (4 * R);
+    for (int q = blockIdx.y * TR_WAVES + wave; q < nsteps; q += stride) {
+        const int kp = 2 * q + hf;
+        tr_record<R> r = tr_load_record<R>(row_base + ((int64_t)kp * 32 + l) * (4 * R));
+        // activations of this lane's four columns in each of the two k-tiles
+        uint32_t xa[NB][2], xb[NB][2];
+#pragma unroll
+        for (int t = 0; t < NB; ++t) {
+            const int tok = tok0 + t;
+            const bool live = tok < B;
+            const uint32_t *xp = (const uint32_t *)(x + (int64_t)(live ? tok : 0) * k + 32 * kp + 2 * b);
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                uint32_t va = xp[8 * ks], vb = xp[8 * ks + 4];
+                xa[t][ks] = live ? va : 0u;
+                xb[t][ks] = live ? vb : 0u;
+            }
+        }
+        uint32_t cont[4];
+        tr_continuation<R>(r, lane, cont);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int ms = 0; ms < 2; ++ms) {
+                const int ci = ks * 2 + ms;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    // both fp16 halves of the state multiply the same activation
+                    f16x2 w = __builtin_bit_cast(f16x2, tr_hash(tr_state<R>(r.c[ci], cont[ci], j)));
+                    const int rh = (j >> 1) & 1;
+#pragma unroll
+                    for (int t = 0; t < NB; ++t) {
+                        f16x2 xp2 = __builtin_bit_cast(f16x2, (j >> 2) ? xb[t][ks] : xa[t][ks]);
+                        f16 xe = (j & 1) ? xp2.y : xp2.x;
+                        f16x2 xx = {xe, xe};
+                        acc[t][ms * 2 + rh] = __builtin_amdgcn_fdot2(w, xx, acc[t][ms * 2 + rh], false);
+                    }
+                }
+            }
+        }
+    }
+
+    // sum over the four column groups (lane bits 0,1) and the two halves (bit 5)
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = acc[t][i];
+            v += __shfl_xor(v, 1, GLQH_WAVE);
+            v += __shfl_xor(v, 2, GLQH_WAVE);
+            v += __shfl_xor(v, 32, GLQH_WAVE);
+            acc[t][i] = v;
+        }
+    if (hf == 0 && b == 0) {
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][t][(i >> 1) * 16 + (i & 1) * 8 + a] = acc[t][i];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < NB * 32; idx += TR_THREADS) {
+        const int t = idx >> 5, row = idx & 31;
+        const int tok = tok0 + t;
+        if (tok >= B) continue;
+        float v = red[0][t][row];
+#pragma unroll
+        for (int w = 1; w < TR_WAVES; ++w) v += red[w][t][row];
+        if (direct) {
+            float *o = part + (int64_t)tok * out_stride + 32 * mp + row;
+            *o = accum ? (*o + scale * v) : scale * v;
+        } else {
+            part[((int64_t)blockIdx.y * B + tok) * m + 32 * mp + row] = v;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+reduce_splits_kernel(const float *__restrict__ part, int ksplit, int64_t kstride, int m, float scale,
+                     float *__restrict__ out, int64_t out_stride, int accum) {
+    const int row = blockIdx.x * 256 + threadIdx.x;
+    const int tok = blockIdx.y;
+    if (row >= m) return;
+    float v = 0.0f;
+    for (int s = 0; s < ksplit; ++s) v += part[(int64_t)s * kstride + (int64_t)tok * m + row];
+    float *o = out + (int64_t)tok * out_stride + row;
+    *o = accum ? (*o + scale * v) : scale * v;
+}
+
+template <int R>
+int launch_gemv_R(const void *x, int64_t B, const void *packed, int64_t m, int64_t k, int ksplit,
+                  float *part, int direct, float scale, int accum, int64_t out_stride,
+                  hipStream_t stream) {
+    const uint8_t *p = (const uint8_t *)packed;
+    const f16 *xp = (const f16 *)x;
+    if (B == 1) {
+        dim3 grid((unsigned)(m / 32), (unsigned)ksplit, 1);
+        hipLaunchKernelGGL((tr_gemv_kernel<R, 1>), grid, dim3(TR_THREADS), 0, stream, p, xp, (int)B,
+                           (int)m, (int)k, part, direct, scale, accum, out_stride);
+    } else if (B <= 4) {
+        dim3 grid((unsigned)(m / 32), (unsigned)ksplit, 1);
+        hipLaunchKernelGGL((tr_gemv_kernel<R, 4>), grid, dim3(TR_THREADS), 0, stream, p, xp, (int)B,
+                           (int)m, (int)k, part, direct, scale, accum, out_stride);
+    } else {
+        dim3 grid((unsigned)(m / 32), (unsigned)ksplit, (unsigned)((B + 7) / 8));
+        hipLaunchKernelGGL((tr_gemv_kernel<R, 8>), grid, dim3(TR_THREADS), 0, stream, p, xp, (int)B,
+                           (int)m, (int)k, part, direct, scale, accum, out_stride);
+    }
+    GLQH_LAUNCH_CHECK("trellis gemv launch");
+    return 0;
+}
+
+}  // namespace
+
+// The K-split depends on the layer shape only, never on the token count, so that row b of
+// a batched call sums in exactly the order of the GEMV on x[b].
+int glqh_trellis_pick_ksplit(int64_t m, int64_t k, int64_t B) {
+    (void)B;
+    const int64_t nsteps = k / 64;
+    const int64_t wgs = m / 32;
+    const int64_t target = (int64_t)glqh_device_cus() * 4;       // 16 waves per CU
+    int64_t ks = (target + wgs - 1) / wgs;
+    int64_t cap = nsteps / TR_WAVES;
+    if (cap < 1) cap = 1;
+    if (ks > cap) ks = cap;
+    if (ks > 32) ks = 32;
+    if (ks < 1) ks = 1;
+    return (int)ks;
+}
+
+int glqh_launch_trellis_partial(const void *x_f16, int64_t B, const void *packed, int R,
+                                int64_t m, int64_t k, int ksplit, float *part,
+                                hipStream_t stream) {
+    switch (R) {
+    case 1: return launch_gemv_R<1>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
+    case 2: return launch_gemv_R<2>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
+    case 3: return launch_gemv_R<3>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
+    case 4: return launch_gemv_R<4>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
+    }
+    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}
+
+int glqh_launch_trellis_direct(const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
+                               int64_t k, float scale, float *out, int64_t out_stride, int accum,
+                               hipStream_t stream) {
+    switch (R) {
+    case 1: return launch_gemv_R<1>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
+    case 2: return launch_gemv_R<2>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
+    case 3: return launch_gemv_R<3>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
+    case 4: return launch_gemv_R<4>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
+    }
+    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}
+
+int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, int64_t B, int64_t m,
+                              float scale, float *out, int64_t out_stride, int accum,
+                              hipStream_t stream) {
+    dim3 grid((unsigned)((m + 255) / 256), (unsigned)B);
+    hipLaunchKernelGGL(reduce_splits_kernel, grid, dim3(256), 0, stream, part, ksplit, kstride, (int)m,
+                       scale, out, out_stride, accum);
+    GLQH_LAUNCH_CHECK("reduce_splits launch");
+    return 0;
+}
+
+int glqh_launch_trellis_decompress(const void *packed, int R, int64_t m, int64_t k, void *out,
+                                   hipStream_t stream) {
+    const uint8_t *p = (const uint8_t *)packed;
+    f16 *W = (f16 *)out;
+    dim3 grid((unsigned)((k / 64 + TR_WAVES - 1) / TR_WAVES), (unsigned)(m / 32));
+    switch (R) {
+    case 1: hipLaunchKernelGGL(tr_decompress_kernel<1>, grid, dim3(TR_THREADS), 0, stream, p, W, (int)m, (int)k); break;
+    case 2: hipLaunchKernelGGL(tr_decompress_kernel<2>, grid, dim3(TR_THREADS), 0, stream, p, W, (int)m, (int)k); break;
+    case 3: hipLaunchKernelGGL(tr_decompress_kernel<3>, grid, dim3(TR_THREADS), 0, stream, p, W, (int)m, (int)k); break;
+    case 4: hipLaunchKernelGGL(tr_decompress_kernel<4>, grid, dim3(TR_THREADS), 0, stream, p, W, (int)m, (int)k); break;
+    default: return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+    }
+    GLQH_LAUNCH_CHECK("trellis decompress launch");
+    return 0;
+}

@@ -1,0 +1,417 @@
+"""The reference's native-extension surface, served by libglq_hip.so.
+
+Every function here has the name and positional signature of the matching pybind
+function of the reference extension (``glq._C`` / JIT ``glq_cuda``,
+glq/csrc/glq_bindings.cpp:334-550), so this module can stand where
+``glq.inference_kernel._glq_cuda`` stands; call sites probe capabilities with
+``hasattr(ext, "<name>")`` exactly as they do there.  Tensors are checked, outputs
+and scratch are allocated with torch (caching allocator, graph-capture friendly) and
+raw pointers go to the C ABI on the current stream.  Nothing is computed in Python.
+
+Two deliberate extensions beyond the reference: activations may be bf16 as well as
+fp16 (the reference casts to fp16 first), and the fused linears accept ``out_dtype``
+so the result can be written in the caller's dtype without a cast kernel.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib
+from ._lib import GLQH_BF16, GLQH_F16, GLQH_F32, check
+
+_DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F32}
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _chk(t, name, dtype=None, dev=True):
+    if dev and not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype not in (dtype if isinstance(dtype, tuple) else (dtype,)):
+        raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+def _ws(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _host_i64(t):
+    """CPU int64 block list -> (ctypes array, count)."""
+    if t is None:
+        return None, 0
+    vals = [int(v) for v in (t.tolist() if isinstance(t, torch.Tensor) else t)]
+    return (C.c_int64 * len(vals))(*vals), len(vals)
+
+
+def _meta_ptr(meta):
+    if meta is None or (isinstance(meta, torch.Tensor) and meta.numel() == 0):
+        return C.c_void_p(0)
+    _chk(meta, "block meta", torch.int32)
+    return _p(meta)
+
+
+# --------------------------------------------------------------------------- trellis
+def glq_trellis_kernel_supported(m, k):
+    return bool(_lib.load().glqh_trellis_kernel_supported(int(m), int(k)))
+
+
+def glq_decompress_trellis_3inst_cuda(trellis_packed, m, k, allow_r1=False):
+    lib = _lib.load()
+    _chk(trellis_packed, "trellis_packed", torch.int16)
+    if trellis_packed.dim() != 2:
+        raise RuntimeError("trellis_packed must be 2-D [(m/16)*(k/16), 16*R]")
+    out = torch.empty((int(m), int(k)), dtype=torch.float16, device=trellis_packed.device)
+    with torch.cuda.device(trellis_packed.device):
+        check(lib.glqh_decompress_trellis_3inst(_p(trellis_packed), trellis_packed.shape[0],
+                                                trellis_packed.shape[1], int(m), int(k),
+                                                int(bool(allow_r1)), _p(out), _stream()))
+    return out
+
+
+def _trellis_matmul(x2d, trellis_packed, m, k, wscale, out, accum):
+    lib = _lib.load()
+    _chk(x2d, "x", torch.float16)
+    _chk(trellis_packed, "trellis_packed", torch.int16)
+    if trellis_packed.dim() != 2:
+        raise RuntimeError("trellis_packed must be 2-D [(m/16)*(k/16), 16*R]")
+    B = x2d.shape[0]
+    if accum and out is None:
+        raise RuntimeError("accumulate mode needs the caller's `out` (stage 1 is the initializer)")
+    if out is None:
+        out = torch.empty((B, int(m)), dtype=torch.float32, device=x2d.device)
+    else:
+        if not (out.is_contiguous() and out.numel() == B * int(m) and out.dtype == torch.float32):
+            raise RuntimeError("out must be a contiguous fp32 tensor of B*m elements")
+    with torch.cuda.device(x2d.device):
+        nb = lib.glqh_trellis_gemv_workspace_bytes(int(m), int(k), B)
+        ws = _ws(nb, x2d.device)
+        check(lib.glqh_decode_matmul_trellis_3inst(
+            _p(x2d), B, _p(trellis_packed), trellis_packed.shape[0], trellis_packed.shape[1],
+            int(m), int(k), float(wscale), _p(out), int(m), int(bool(accum)),
+            _p(ws), ws.numel(), _stream()))
+    return out
+
+
+def glq_decode_matvec_trellis_3inst_cuda(x, trellis_packed, m, k, wscale=1.0, out=None, accum=False):
+    if x.numel() != int(k):
+        raise RuntimeError(f"x must have k elements, got {x.numel()}")
+    y = _trellis_matmul(x.reshape(1, -1), trellis_packed, m, k, wscale,
+                        None if out is None else out, accum)
+    return y.reshape(int(m)) if out is None else out
+
+
+def glq_decode_matmul_trellis_3inst_cuda(x, trellis_packed, m, k, wscale=1.0, out=None, accum=False):
+    if x.dim() != 2 or x.shape[1] != int(k):
+        raise RuntimeError(f"x must be (B, k), got {tuple(x.shape)}")
+    return _trellis_matmul(x, trellis_packed, m, k, wscale, out, accum)
+
+
+# --------------------------------------------------------------------------- RHT
+def glq_input_rht_cuda(x, sv, out, in_features, stride_x, rsqrt_n, n_pad, log_n):
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(sv, "sv", torch.float16)
+    _chk(out, "out", (torch.float32, torch.float16))
+    B = x.shape[0] if x.dim() == 2 else 1
+    if (1 << int(log_n)) != int(n_pad):
+        raise RuntimeError(f"n_pad={n_pad} is not 2**log_n")
+    with torch.cuda.device(x.device):
+        check(lib.glqh_input_rht(_p(x), _DT[x.dtype], int(stride_x), _p(sv), _p(out), _DT[out.dtype],
+                                 B, int(in_features), int(n_pad), None, None, 1, float(rsqrt_n),
+                                 _stream()))
+
+
+def glq_output_rht_cuda(y_rht, su, out, out_features, m_pad, log_m, rsqrt_m):
+    lib = _lib.load()
+    _chk(y_rht, "y_rht", torch.float32)
+    _chk(su, "su", torch.float16)
+    _chk(out, "out", (torch.float16, torch.bfloat16, torch.float32))
+    B = y_rht.shape[0] if y_rht.dim() == 2 else 1
+    if (1 << int(log_m)) != int(m_pad):
+        raise RuntimeError(f"m_pad={m_pad} is not 2**log_m")
+    with torch.cuda.device(y_rht.device):
+        check(lib.glqh_output_rht(_p(y_rht), int(m_pad), _p(su), _p(out), _DT[out.dtype],
+                                  int(out_features), B, int(out_features), int(m_pad), None, None, 1,
+                                  float(rsqrt_m), _stream()))
+
+
+def glq_input_rht_blockdiag_cuda(x, sv, x_rht, in_features, n_pad, blocks_n, blocks_n_meta):
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(sv, "sv", torch.float16)
+    _chk(x_rht, "x_rht", (torch.float32, torch.float16))
+    arr, nb = _host_i64(blocks_n)
+    B = x.shape[0]
+    with torch.cuda.device(x.device):
+        check(lib.glqh_input_rht(_p(x), _DT[x.dtype], x.shape[1], _p(sv), _p(x_rht), _DT[x_rht.dtype],
+                                 B, int(in_features), int(n_pad), _meta_ptr(blocks_n_meta) if nb > 1 else None,
+                                 arr, nb, 0.0, _stream()))
+
+
+def glq_output_rht_blockdiag_cuda(y_rht, su, y, out_features, m_pad, blocks_m, blocks_m_meta):
+    lib = _lib.load()
+    _chk(y_rht, "y_rht", torch.float32)
+    _chk(su, "su", torch.float16)
+    _chk(y, "y", (torch.float16, torch.bfloat16, torch.float32))
+    arr, nb = _host_i64(blocks_m)
+    B = y_rht.shape[0]
+    with torch.cuda.device(y_rht.device):
+        check(lib.glqh_output_rht(_p(y_rht), int(m_pad), _p(su), _p(y), _DT[y.dtype], y.shape[1], B,
+                                  int(out_features), int(m_pad),
+                                  _meta_ptr(blocks_m_meta) if nb > 1 else None, arr, nb, 0.0, _stream()))
+
+
+def glq_output_rht_shards_cuda(y_rht, su, y, out_features, shard_meta, max_bs):
+    lib = _lib.load()
+    _chk(y_rht, "y_rht", torch.float32)
+    _chk(su, "su", torch.float16)
+    _chk(y, "y", (torch.float16, torch.bfloat16, torch.float32))
+    _chk(shard_meta, "shard_meta", torch.int32)
+    B, total_m = y_rht.shape
+    if int(out_features) != total_m or y.shape[1] != int(out_features):
+        raise RuntimeError("output_rht_shards needs out_features == total_m == y.shape[1]")
+    with torch.cuda.device(y_rht.device):
+        check(lib.glqh_output_rht_shards(_p(y_rht), _p(su), _p(y), _DT[y.dtype], B, int(out_features),
+                                         total_m, _p(shard_meta), shard_meta.shape[0], int(max_bs),
+                                         _stream()))
+
+
+# --------------------------------------------------------------------------- fused trellis
+def _fused_trellis(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_meta, wscale,
+                   inv_rs2, in_features, out_features, n_pad, m_pad, y, y_rht_out, out_dtype):
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(sv, "sv", torch.float16)
+    _chk(packed, "trellis_packed", torch.int16)
+    if packed.dim() != 2:
+        raise RuntimeError("trellis_packed must be 2-D [(m/16)*(k/16), 16*R]")
+    has2 = packed2 is not None and packed2.numel() > 0
+    if has2:
+        _chk(packed2, "trellis_packed2", torch.int16)
+    B = x.shape[0]
+    bn, nbn = _host_i64(blocks_n)
+    bm, nbm = _host_i64(blocks_m)
+    if y is None and y_rht_out is None:
+        _chk(su, "su", torch.float16)
+        y = torch.empty((B, int(out_features)), dtype=out_dtype or torch.float16, device=x.device)
+    ystride = 0
+    yrp, yrs = C.c_void_p(0), 0
+    if y_rht_out is not None:
+        yrp, yrs = y_rht_out
+    with torch.cuda.device(x.device):
+        nb = lib.glqh_fused_linear_trellis_workspace_bytes(B, int(n_pad), int(m_pad))
+        ws = _ws(nb, x.device)
+        check(lib.glqh_fused_linear_trellis_3inst(
+            _p(x), _DT[x.dtype], x.shape[1], B, _p(sv), _p(su) if su is not None else None,
+            _p(packed), packed.shape[0], packed.shape[1],
+            _p(packed2) if has2 else None, packed2.shape[0] if has2 else 0,
+            packed2.shape[1] if has2 else 0,
+            bn, nbn, bm, nbm, _meta_ptr(bn_meta) if nbn > 1 else None,
+            _meta_ptr(bm_meta) if nbm > 1 else None,
+            float(wscale), float(inv_rs2), int(in_features), int(out_features), int(n_pad), int(m_pad),
+            _p(y) if y is not None else None, _DT[y.dtype] if y is not None else GLQH_F16,
+            y.shape[1] if y is not None else ystride, yrp, int(yrs), _p(ws), ws.numel(), _stream()))
+    return y
+
+
+def glq_fused_linear_trellis_3inst_cuda(x, sv, su, trellis_packed, blocks_n, blocks_m,
+                                        blocks_n_meta, blocks_m_meta, wscale, in_features,
+                                        out_features, n_pad, m_pad, out_dtype=None):
+    return _fused_trellis(x, sv, su, trellis_packed, None, blocks_n, blocks_m, blocks_n_meta,
+                          blocks_m_meta, wscale, 0.0, in_features, out_features, n_pad, m_pad,
+                          None, None, out_dtype)
+
+
+def glq_fused_linear_trellis_3inst_rvq2_cuda(x, sv, su, trellis_packed, trellis_packed2, blocks_n,
+                                             blocks_m, blocks_n_meta, blocks_m_meta, wscale,
+                                             inv_resid_scale2, in_features, out_features, n_pad,
+                                             m_pad, out_dtype=None):
+    if trellis_packed2 is None or trellis_packed2.numel() == 0:
+        raise RuntimeError("trellis RVQ stage 2 is half-configured: trellis_packed2 is absent "
+                           f"but inv_resid_scale2 = {inv_resid_scale2}")
+    return _fused_trellis(x, sv, su, trellis_packed, trellis_packed2, blocks_n, blocks_m,
+                          blocks_n_meta, blocks_m_meta, wscale, inv_resid_scale2, in_features,
+                          out_features, n_pad, m_pad, None, None, out_dtype)
+
+
+def _yrht_slice(y_rht_out, col, m_pad):
+    _chk(y_rht_out, "y_rht_out", torch.float32)
+    if y_rht_out.dim() != 2 or int(col) < 0 or int(col) + int(m_pad) > y_rht_out.shape[1]:
+        raise RuntimeError("y_rht_out must be (B, total_m) with col + m_pad <= total_m")
+    return C.c_void_p(y_rht_out.data_ptr() + 4 * int(col)), y_rht_out.shape[1]
+
+
+def glq_fused_linear_trellis_3inst_yrht_cuda(x, sv, trellis_packed, blocks_n, blocks_n_meta, wscale,
+                                             in_features, n_pad, m_pad, y_rht_out, col):
+    if y_rht_out.shape[0] != x.shape[0]:
+        raise RuntimeError("y_rht_out rows must equal the token count")
+    _fused_trellis(x, sv, None, trellis_packed, None, blocks_n, None, blocks_n_meta, None, wscale,
+                   0.0, in_features, m_pad, n_pad, m_pad, None, _yrht_slice(y_rht_out, col, m_pad),
+                   None)
+
+
+def glq_fused_linear_trellis_3inst_yrht_rvq2_cuda(x, sv, trellis_packed, trellis_packed2, blocks_n,
+                                                  blocks_n_meta, wscale, inv_resid_scale2,
+                                                  in_features, n_pad, m_pad, y_rht_out, col):
+    if y_rht_out.shape[0] != x.shape[0]:
+        raise RuntimeError("y_rht_out rows must equal the token count")
+    if trellis_packed2 is None or trellis_packed2.numel() == 0:
+        raise RuntimeError("trellis RVQ stage 2 is half-configured: trellis_packed2 is absent "
+                           f"but inv_resid_scale2 = {inv_resid_scale2}")
+    _fused_trellis(x, sv, None, trellis_packed, trellis_packed2, blocks_n, None, blocks_n_meta, None,
+                   wscale, inv_resid_scale2, in_features, m_pad, n_pad, m_pad, None,
+                   _yrht_slice(y_rht_out, col, m_pad), None)
+
+
+def glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, trellis_packed, m, k, in_features,
+                                                wscale=1.0, blocks_n_meta=None, num_blocks=1,
+                                                max_bs=0, out=None):
+    """B=1 GEMV on the raw activations: input RHT + decode + x wscale, (m,) fp32."""
+    x2 = x_raw.reshape(1, -1)
+    if num_blocks > 1:
+        if blocks_n_meta is None:
+            raise RuntimeError("block-diagonal fused-input GEMV needs blocks_n_meta")
+        blocks = [int(v) for v in blocks_n_meta[:, 1].tolist()]
+    else:
+        blocks = [int(k)]
+    if out is None:
+        out = torch.empty(int(m), dtype=torch.float32, device=x_raw.device)
+    _fused_trellis(x2.contiguous(), sv, None, trellis_packed, None, blocks, None, blocks_n_meta, None,
+                   wscale, 0.0, in_features, m, k, m, None, (C.c_void_p(out.data_ptr()), int(m)), None)
+    return out
+
+
+# --------------------------------------------------------------------------- E8 shell
+_TABLES = {}
+
+
+def _packed_table(codebook):
+    """Nibble-packed copy of an (N, 8) fp16 E8 table, built once per tensor."""
+    key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device))
+    hit = _TABLES.get(key)
+    if hit is not None:
+        return hit
+    lib = _lib.load()
+    _chk(codebook, "codebook", torch.float16)
+    if codebook.dim() != 2 or codebook.shape[1] != 8 or not 1 <= codebook.shape[0] <= 65536:
+        raise RuntimeError(f"codebook must be (N<=65536, 8) fp16, got {tuple(codebook.shape)}")
+    packed = torch.empty(codebook.shape[0], dtype=torch.int32, device=codebook.device)
+    bad = torch.zeros(1, dtype=torch.int32, device=codebook.device)
+    with torch.cuda.device(codebook.device):
+        check(lib.glqh_e8_pack_table(_p(codebook), codebook.shape[0], _p(packed), _p(bad), _stream()))
+    nbad = int(bad.item())
+    if nbad:
+        raise RuntimeError(f"codebook has {nbad} rows outside the E8 half-integer grid "
+                           "{-3, -2.5, ..., 3}; only E8 shell tables are supported")
+    _TABLES[key] = packed
+    return packed
+
+
+def _absent(t):
+    return t is None or t.numel() == 0
+
+
+def _e8_args(qidxs, codebook, qidxs2, codebook2, inv_rs, qidxs3, inv_rs2, qidxs4, inv_rs3):
+    _chk(qidxs, "qidxs", torch.int16)
+    t1 = _packed_table(codebook)
+    q2 = None if _absent(qidxs2) or float(inv_rs) == 0.0 else qidxs2
+    t2, n2 = None, 0
+    if q2 is not None:
+        _chk(q2, "qidxs2", torch.int16)
+        t2 = _packed_table(codebook if _absent(codebook2) else codebook2)
+        n2 = t2.shape[0]
+    q3 = None if q2 is None or _absent(qidxs3) or float(inv_rs2) == 0.0 else qidxs3
+    q4 = None if q3 is None or _absent(qidxs4) or float(inv_rs3) == 0.0 else qidxs4
+    for q, nme in ((q3, "qidxs3"), (q4, "qidxs4")):
+        if q is not None:
+            _chk(q, nme, torch.int16)
+    return t1, q2, t2, n2, q3, q4
+
+
+def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=None,
+                            inv_resid_scale=0.0, codebook_abs=None, qidxs3=None, codebook3=None,
+                            inv_resid_scale2=0.0, qidxs4=None, codebook4=None, inv_resid_scale3=0.0):
+    """(B, N) fp16 RHT-domain activations -> (B, M) fp32."""
+    lib = _lib.load()
+    _chk(x, "x", torch.float16)
+    t1, q2, t2, n2, q3, q4 = _e8_args(qidxs, codebook, qidxs2, codebook2, inv_resid_scale, qidxs3,
+                                      inv_resid_scale2, qidxs4, inv_resid_scale3)
+    B = x.shape[0]
+    M, nblk = qidxs.shape
+    if x.shape[1] != nblk * 8:
+        raise RuntimeError(f"x has {x.shape[1]} columns, qidxs implies {nblk * 8}")
+    out = torch.empty((B, M), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        nb = lib.glqh_e8_matmul_workspace_bytes(M, nblk * 8, B)
+        ws = _ws(nb, x.device)
+        check(lib.glqh_e8_dequant_matmul(
+            _p(x), B, _p(qidxs), _p(q2), _p(q3), _p(q4), _p(t1), _p(t2), n2, float(wscale),
+            float(inv_resid_scale), float(inv_resid_scale2), float(inv_resid_scale3), M, nblk * 8,
+            _p(out), _p(ws), ws.numel(), _stream()))
+    return out
+
+
+def glq_dequant_matvec_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=None,
+                            inv_resid_scale=0.0, codebook_abs=None):
+    """(N,) fp16 -> (M,) fp32."""
+    return glq_dequant_matmul_cuda(x.reshape(1, -1), qidxs, codebook, wscale, qidxs2, codebook2,
+                                   inv_resid_scale).reshape(-1)
+
+
+def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad, m_pad,
+              blocks_n, blocks_m, bn_meta, bm_meta, qidxs2, codebook2, inv_rs, qidxs3, inv_rs2,
+              qidxs4, inv_rs3, out_dtype):
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    _chk(sv, "sv", torch.float16)
+    _chk(su, "su", torch.float16)
+    t1, q2, t2, n2, q3, q4 = _e8_args(qidxs, codebook, qidxs2, codebook2, inv_rs, qidxs3, inv_rs2,
+                                      qidxs4, inv_rs3)
+    if tuple(qidxs.shape) != (int(m_pad), int(n_pad) // 8):
+        raise RuntimeError(f"qidxs shape {tuple(qidxs.shape)} != (m_pad, n_pad/8)")
+    B = x.shape[0]
+    bn, nbn = _host_i64(blocks_n)
+    bm, nbm = _host_i64(blocks_m)
+    y = torch.empty((B, int(out_features)), dtype=out_dtype or torch.float16, device=x.device)
+    with torch.cuda.device(x.device):
+        nb = lib.glqh_fused_linear_e8_workspace_bytes(B, int(n_pad), int(m_pad))
+        ws = _ws(nb, x.device)
+        check(lib.glqh_fused_linear_e8(
+            _p(x), _DT[x.dtype], x.shape[1], B, _p(sv), _p(su), _p(qidxs), _p(q2), _p(q3), _p(q4),
+            _p(t1), _p(t2), n2, float(wscale), float(inv_rs), float(inv_rs2), float(inv_rs3),
+            bn, nbn, bm, nbm, _meta_ptr(bn_meta) if nbn > 1 else None,
+            _meta_ptr(bm_meta) if nbm > 1 else None, int(in_features), int(out_features), int(n_pad),
+            int(m_pad), _p(y), _DT[y.dtype], y.shape[1], _p(ws), ws.numel(), _stream()))
+    return y
+
+
+def glq_fused_linear_cuda(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad,
+                          m_pad, log_n, log_m, qidxs2=None, codebook2=None, inv_resid_scale=0.0,
+                          qidxs3=None, codebook3=None, inv_resid_scale2=0.0, qidxs4=None,
+                          codebook4=None, inv_resid_scale3=0.0, out_dtype=None):
+    if (1 << int(log_n)) != int(n_pad) or (1 << int(log_m)) != int(m_pad):
+        raise RuntimeError("glq_fused_linear_cuda needs power-of-two n_pad and m_pad")
+    return _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad, m_pad,
+                     [int(n_pad)], [int(m_pad)], None, None, qidxs2, codebook2, inv_resid_scale,
+                     qidxs3, inv_resid_scale2, qidxs4, inv_resid_scale3, out_dtype)
+
+
+def glq_fused_linear_block_diag_cuda(x, sv, su, qidxs, codebook, wscale, in_features, out_features,
+                                     n_pad, m_pad, blocks_n, blocks_m, blocks_n_meta, blocks_m_meta,
+                                     qidxs2=None, codebook2=None, inv_resid_scale=0.0, qidxs3=None,
+                                     codebook3=None, inv_resid_scale2=0.0, qidxs4=None,
+                                     codebook4=None, inv_resid_scale3=0.0, out_dtype=None):
+    return _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad, m_pad,
+                     blocks_n, blocks_m, blocks_n_meta, blocks_m_meta, qidxs2, codebook2,
+                     inv_resid_scale, qidxs3, inv_resid_scale2, qidxs4, inv_resid_scale3, out_dtype)

@@ -1,0 +1,169 @@
+/* libglq_hip.so -- C ABI of the MI355X (gfx950) quantized-linear forward.
+ *
+ * Every entry point takes plain device pointers, sizes and a hipStream_t (passed
+ * as void*), launches on that stream, never synchronises and never allocates.
+ * Scratch memory is supplied by the caller (`ws`, sized by the matching
+ * *_workspace_bytes function).  Return value: 0 on success, non-zero on a refused
+ * call; glqh_last_error() then returns the reason (thread-local, valid until the
+ * next call on the same thread).
+ *
+ * Each declaration names the reference interface it stands in for; paths are
+ * relative to the reference checkout (cnygaard/glq v0.8.8).
+ */
+#ifndef GLQ_HIP_H
+#define GLQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of activation / output buffers */
+#define GLQH_F16  0
+#define GLQH_BF16 1
+#define GLQH_F32  2
+
+/* block meta row: {offset, bs, log2(bs), w}; w != 0 is the bit pattern of an fp32
+ * normalisation factor that overrides 1/sqrt(bs).
+ * glq/quantized_linear.py:36-76 (_pack_block_meta, _pack_shard_meta). */
+typedef struct { int32_t offset, bs, log_bs, w; } glqh_block_meta;
+
+int         glqh_version(void);
+const char *glqh_last_error(void);
+/* One-time per-process setup (kernel attributes, device limits); idempotent and
+ * called implicitly by every entry point.  glq/csrc/glq_trellis.cu:823-853. */
+int         glqh_init(void);
+
+/* ---- trellis 3INST ------------------------------------------------------ */
+
+/* m % 32 == 0 && k % 64 == 0.  glq/csrc/glq_trellis.cu:979-981. */
+int glqh_trellis_kernel_supported(int64_t m, int64_t k);
+
+/* packed ((m/16)(k/16), 16R) int16 -> dense (m,k) fp16, bit-exact with the
+ * reference dequantizer.  R = packed_cols/16 in 2..4 (1 only with allow_r1).
+ * glq_decompress_trellis_3inst_cuda, glq/csrc/glq_trellis.cu:1064-1085. */
+int glqh_decompress_trellis_3inst(const void *packed, int64_t packed_rows, int64_t packed_cols,
+                                  int64_t m, int64_t k, int allow_r1,
+                                  void *out_f16, void *stream);
+
+/* Scratch bytes needed by the matvec / matmul below for B tokens. */
+size_t glqh_trellis_gemv_workspace_bytes(int64_t m, int64_t k, int64_t B);
+
+/* out[b, :] (fp32, row stride out_stride) = (accum ? out : 0) + wscale * W @ x[b, :]
+ * with x (B,k) fp16 already in the RHT domain.  B == 1 is the GEMV
+ * (glq_decode_matvec_trellis_3inst_cuda, glq/csrc/glq_trellis.cu:1087-1126), B > 1 the
+ * batched form that keeps the weights compressed
+ * (glq_decode_matmul_trellis_3inst_cuda, glq/csrc/glq_trellis.cu:1192-1232).
+ * R == 1 is accepted only with accum (a residual stage). */
+int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B,
+                                     const void *packed, int64_t packed_rows, int64_t packed_cols,
+                                     int64_t m, int64_t k, double wscale,
+                                     float *out, int64_t out_stride, int accum,
+                                     void *ws, size_t ws_bytes, void *stream);
+
+/* ---- randomized Hadamard transforms ------------------------------------- */
+
+/* out[b, 0:n_pad] = blockFHT(pad(x[b, 0:in_features]) * sv), per block 1/sqrt(bs).
+ * x is f16 or bf16 with row stride x_stride; out is f32 or f16, contiguous rows of
+ * n_pad.  meta (device, n_blocks rows) may be NULL when n_blocks == 1 (one block of
+ * n_pad, normalised by rsqrt_n if non-zero).
+ * glq_input_rht_cuda / glq_input_rht_blockdiag_cuda, glq/csrc/glq_cuda.cu:2385-2441,
+ * 2774-2823. */
+int glqh_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv_f16,
+                   void *out, int out_dtype, int64_t B, int64_t in_features, int64_t n_pad,
+                   const glqh_block_meta *meta_dev, const int64_t *blocks_host, int64_t n_blocks,
+                   double rsqrt_n, void *stream);
+
+/* y[b, 0:out_features] = (blockFHT(y_rht[b, 0:m_pad]) * su)[0:out_features], cast to
+ * f16 / bf16 / f32.  y_rht has row stride y_rht_stride (a slice of a wider buffer is
+ * allowed), y has row stride y_stride.
+ * glq_output_rht_cuda / glq_output_rht_blockdiag_cuda, glq/csrc/glq_cuda.cu:2444-2499,
+ * 2825-2874. */
+int glqh_output_rht(const float *y_rht, int64_t y_rht_stride, const void *su_f16,
+                    void *y, int y_dtype, int64_t y_stride, int64_t B,
+                    int64_t out_features, int64_t m_pad,
+                    const glqh_block_meta *meta_dev, const int64_t *blocks_host, int64_t n_blocks,
+                    double rsqrt_m, void *stream);
+
+/* One launch over every sub-block of every output shard of a fused qkv / gate_up
+ * linear: shard_meta rows carry global offsets into y_rht (B, total_m); su and y are
+ * indexed with the same offsets (y is (B, out_features), out_features == total_m).
+ * glq_output_rht_shards_cuda, glq/csrc/glq_cuda.cu:2882-2916. */
+int glqh_output_rht_shards(const float *y_rht, const void *su_f16, void *y, int y_dtype,
+                           int64_t B, int64_t out_features, int64_t total_m,
+                           const glqh_block_meta *shard_meta_dev, int64_t n_rows, int64_t max_bs,
+                           void *stream);
+
+/* ---- fused trellis linear ------------------------------------------------ */
+
+size_t glqh_fused_linear_trellis_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad);
+
+/* y (B,out_features) = outRHT( wscale * W1 @ inRHT(x) [+ wscale*inv_rs2 * W2 @ inRHT(x)] ).
+ * packed2 == NULL with inv_resid_scale2 == 0 is the single-stage layer; any other
+ * mismatch of the two is refused ("half-configured").  x is f16 or bf16, y f16 or bf16.
+ * glq_fused_linear_trellis_3inst_cuda / ..._rvq2_cuda, glq/csrc/glq_trellis.cu:1339-1366,
+ * 1407-1440.  When y_rht_out != NULL the call stops at the RHT-domain product and
+ * writes fp32 into y_rht_out[b*y_rht_stride + 0 .. m_pad) (the caller passes the column
+ * offset folded into the pointer) and y may be NULL:
+ * glq_fused_linear_trellis_3inst_yrht_cuda / ..._yrht_rvq2_cuda, :1373-1397, 1443-1473. */
+int glqh_fused_linear_trellis_3inst(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                    const void *sv_f16, const void *su_f16,
+                                    const void *packed, int64_t packed_rows, int64_t packed_cols,
+                                    const void *packed2, int64_t packed2_rows, int64_t packed2_cols,
+                                    const int64_t *blocks_n, int64_t n_blocks_n,
+                                    const int64_t *blocks_m, int64_t n_blocks_m,
+                                    const glqh_block_meta *bn_meta_dev,
+                                    const glqh_block_meta *bm_meta_dev,
+                                    double wscale, double inv_resid_scale2,
+                                    int64_t in_features, int64_t out_features,
+                                    int64_t n_pad, int64_t m_pad,
+                                    void *y, int y_dtype, int64_t y_stride,
+                                    float *y_rht_out, int64_t y_rht_stride,
+                                    void *ws, size_t ws_bytes, void *stream);
+
+/* ---- E8 shell codebook ---------------------------------------------------- */
+
+/* (n_entries, 8) fp16 table -> n_entries uint32, nibble i = round(2 v_i) + 6
+ * (glq/codebook.py:102-115).  *ok_dev (device int32) is set to 0 if any coordinate is
+ * outside {-3, -2.5, ..., 3}; the packed table must then not be used. */
+int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, uint32_t *packed_out,
+                       int32_t *ok_dev, void *stream);
+
+size_t glqh_e8_matmul_workspace_bytes(int64_t m_pad, int64_t n_pad, int64_t B);
+
+/* out[b, :] (fp32, stride m_pad) = wscale * (cb[q1] + inv_rs*cb2[q2] + inv_rs2*cb3[q3]
+ * + inv_rs3*cb4[q4]) @ x[b, :], x (B, n_pad) fp16 in the RHT domain, q* (m_pad, n_pad/8)
+ * int16 read as unsigned.  A stage is absent when its index pointer is NULL or its scale
+ * is 0.  Tables are nibble-packed (glqh_e8_pack_table); table2 has n_entries2 rows
+ * (65536, or 256 for the 3-bit recipe), stages 3-4 use table 1.
+ * glq_dequant_matvec_cuda / glq_dequant_matmul_cuda, glq/csrc/glq_cuda.cu:1384-1637. */
+int glqh_e8_dequant_matmul(const void *x_f16, int64_t B,
+                           const void *q1, const void *q2, const void *q3, const void *q4,
+                           const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                           double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                           int64_t m_pad, int64_t n_pad,
+                           float *out, void *ws, size_t ws_bytes, void *stream);
+
+size_t glqh_fused_linear_e8_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad);
+
+/* Whole E8 linear: input RHT -> gather-matmul -> output RHT.
+ * glq_fused_linear_cuda (pow2, one block each side) and
+ * glq_fused_linear_block_diag_cuda, glq/csrc/glq_cuda.cu:2533-2742, 3038-3266. */
+int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                         const void *sv_f16, const void *su_f16,
+                         const void *q1, const void *q2, const void *q3, const void *q4,
+                         const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                         double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                         const int64_t *blocks_n, int64_t n_blocks_n,
+                         const int64_t *blocks_m, int64_t n_blocks_m,
+                         const glqh_block_meta *bn_meta_dev, const glqh_block_meta *bm_meta_dev,
+                         int64_t in_features, int64_t out_features, int64_t n_pad, int64_t m_pad,
+                         void *y, int y_dtype, int64_t y_stride,
+                         void *ws, size_t ws_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GLQ_HIP_H */

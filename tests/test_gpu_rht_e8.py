@@ -1,0 +1,180 @@
+"""RHT kernels and the E8 shell path against the oracle (needs an MI355X)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glq_oracle as O
+from tests.gpu_util import DEV, e8_table_f16, rel, say, t
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from glq_amd import ext as e
+    return e
+
+
+@pytest.mark.parametrize("n,inf", [(16, 16), (64, 50), (2048, 2048), (2048, 2000), (16384, 16384),
+                                   (32768, 30000)])
+def test_input_rht_pow2(ext, n, inf):
+    say("input_rht", n, inf)
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal((3, inf)).astype(np.float16)
+    sv = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    out = torch.empty(3, n, dtype=torch.float32, device=DEV)
+    ext.glq_input_rht_cuda(t(x), t(sv), out, inf, inf, 1.0 / np.sqrt(n), n, int(np.log2(n)))
+    xp = np.zeros((3, n), np.float32)
+    xp[:, :inf] = x
+    ref = O.fht(xp * sv.astype(np.float32)[None])
+    assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("n,inf,dtype", [(960, 960, torch.float16), (11008, 11008, torch.bfloat16),
+                                         (14336, 14000, torch.bfloat16), (160, 160, torch.float16)])
+def test_input_output_rht_blockdiag(ext, n, inf, dtype):
+    from glq_amd import hadamard as H
+    say("blockdiag rht", n, inf, dtype)
+    blocks = O.block_decompose(n)
+    x = torch.randn(2, inf).to(dtype)
+    rng = np.random.default_rng(n)
+    sv = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    out = torch.empty(2, n, dtype=torch.float32, device=DEV)
+    ext.glq_input_rht_blockdiag_cuda(x.to(DEV), t(sv), out, inf, n, torch.tensor(blocks),
+                                     H.pack_block_meta(blocks).to(DEV))
+    xp = np.zeros((2, n), np.float32)
+    xp[:, :inf] = x.float().numpy()
+    ref = O.block_diag_fht(xp * sv.astype(np.float32)[None], blocks)
+    assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=2e-5)
+    # output side: FHT * su, unpad, cast
+    y = torch.empty(2, inf, dtype=dtype, device=DEV)
+    ext.glq_output_rht_blockdiag_cuda(out, t(sv), y, inf, n, torch.tensor(blocks),
+                                      H.pack_block_meta(blocks).to(DEV))
+    yref = (O.block_diag_fht(ref, blocks) * sv.astype(np.float32)[None])[:, :inf]
+    assert rel(y, yref) < 5e-3
+    if inf == n:                                     # H(H(x sv)) sv == x
+        assert rel(y, x.float().numpy()) < 5e-3
+
+
+def test_rht_refusals(ext):
+    x = torch.zeros(1, 96, dtype=torch.float16, device=DEV)
+    sv = torch.ones(96, dtype=torch.float16, device=DEV)
+    out = torch.empty(1, 96, dtype=torch.float32, device=DEV)
+    with pytest.raises(RuntimeError, match="power of two"):
+        ext.glq_input_rht_blockdiag_cuda(x, sv, out, 96, 96, torch.tensor([96]), None)
+    with pytest.raises(RuntimeError, match="sum"):
+        from glq_amd import hadamard as H
+        ext.glq_input_rht_blockdiag_cuda(x, sv, out, 96, 96, torch.tensor([64, 16]),
+                                         H.pack_block_meta([64, 16]).to(DEV))
+
+
+# ------------------------------------------------------------------- E8 shell
+def _rand_idx(rng, m, nb):
+    return rng.integers(0, 65536, size=(m, nb)).astype(np.uint16).view(np.int16)
+
+
+@pytest.mark.parametrize("m,n", [(32, 64), (96, 160), (960, 960), (100, 72)])
+@pytest.mark.parametrize("stages", [1, 2, 4])
+def test_e8_dequant_matmul_matches_oracle(ext, m, n, stages):
+    say("e8 matmul", m, n, stages)
+    rng = np.random.default_rng(m + stages)
+    cb = e8_table_f16()
+    q = [_rand_idx(rng, m, n // 8) for _ in range(4)]
+    q[0][0, 0] = 0
+    q[0][0, 1] = -1                                   # index 65535
+    sc = [0.0, 0.0, 0.0]
+    for s in range(1, stages):
+        sc[s - 1] = [1 / 3.0, 1 / 9.0, 1 / 27.0][s - 1]
+    B = 3
+    x = (rng.standard_normal((B, n)) * 0.5).astype(np.float16)
+    W = O.e8_dequant(q[0], q[1], sc[0], q[2], sc[1], q[3], sc[2])
+    ref = x.astype(np.float32) @ W.T * np.float32(0.021)
+    out = ext.glq_dequant_matmul_cuda(t(x), t(q[0]), cb, 0.021, t(q[1]), cb, sc[0], None, t(q[2]), cb,
+                                      sc[1], t(q[3]), cb, sc[2])
+    assert out.shape == (B, m) and out.dtype == torch.float32
+    assert rel(out, ref) < 1e-3, rel(out, ref)
+    out2 = ext.glq_dequant_matmul_cuda(t(x), t(q[0]), cb, 0.021, t(q[1]), cb, sc[0], None, t(q[2]), cb,
+                                       sc[1], t(q[3]), cb, sc[2])
+    assert torch.equal(out, out2)
+    gv = ext.glq_dequant_matvec_cuda(t(x[1]), t(q[0]), cb, 0.021, t(q[1]), cb, sc[0])
+    if stages <= 2:
+        assert torch.equal(gv, out[1])
+
+
+def test_e8_small_secondary_table(ext):
+    """3 bpw recipe: the second stage indexes the first 256 rows."""
+    rng = np.random.default_rng(0)
+    m, n = 64, 128
+    cb = e8_table_f16()
+    cb2 = cb[:256].contiguous()
+    q1 = _rand_idx(rng, m, n // 8)
+    q2 = rng.integers(0, 256, size=(m, n // 8)).astype(np.int16)
+    x = rng.standard_normal((1, n)).astype(np.float16)
+    W = O.e8_dequant(q1, q2, 0.5)
+    out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
+    assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
+
+
+def test_e8_rejects_foreign_table(ext):
+    bad = torch.randn(256, 8, device=DEV).half()
+    q = torch.zeros(32, 8, dtype=torch.int16, device=DEV)
+    x = torch.zeros(1, 64, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="half-integer grid"):
+        ext.glq_dequant_matmul_cuda(x, q, bad, 1.0)
+
+
+@pytest.mark.parametrize("tag,bpw,bd", [("bd2", 2, True), ("bd4", 4, True), ("p2", 2, False),
+                                        ("p4", 4, False)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_e8_fused_linear_on_reference_layers(ext, golden, tag, bpw, bd, dtype):
+    from glq_amd import hadamard as H
+    g = golden("e8_layer")
+    say("e8 fused golden", tag, dtype)
+    m, n = g[f"{tag}_W"].shape
+    bm, bn = list(g[f"{tag}_blocks_m"]), list(g[f"{tag}_blocks_n"])
+    m_pad, n_pad = sum(bm), sum(bn)
+    art = {"Qidxs": g[f"{tag}_Qidxs"], "SU": g[f"{tag}_SU"], "SV": g[f"{tag}_SV"],
+           "Wscale": g[f"{tag}_Wscale"], "blocks_m": bm, "blocks_n": bn}
+    q2, irs = None, 0.0
+    if bpw == 4:
+        art["Qidxs2"], art["inv_resid_scale"] = g[f"{tag}_Qidxs2"], g[f"{tag}_inv_resid_scale"]
+        q2, irs = t(art["Qidxs2"]), float(art["inv_resid_scale"])
+    x = torch.from_numpy(g[f"{tag}_x"]).to(dtype)
+    ref = O.e8_linear_forward(x.float().numpy(), art, n, m)
+    cb = e8_table_f16()
+    common = (x.to(DEV), t(art["SV"]), t(art["SU"]), t(art["Qidxs"]), cb, float(art["Wscale"]), n, m,
+              n_pad, m_pad)
+    if bd:
+        y = ext.glq_fused_linear_block_diag_cuda(
+            *common, torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV),
+            H.pack_block_meta(bm).to(DEV), q2, cb if q2 is not None else None, irs, out_dtype=dtype)
+    else:
+        y = ext.glq_fused_linear_cuda(*common, int(np.log2(n_pad)), int(np.log2(m_pad)), q2,
+                                      cb if q2 is not None else None, irs, out_dtype=dtype)
+    assert y.shape == (x.shape[0], m) and y.dtype == dtype
+    assert rel(y, ref) < TOL, rel(y, ref)
+    assert rel(y, g[f"{tag}_y"]) < TOL
+
+
+@pytest.mark.parametrize("B", [1, 8])
+def test_e8_config1_layer(ext, B):
+    """960x960 at 2 bpw, weights N(0, 0.02) seed 0, quantised by RHT + nearest-E8,
+    fp16 activations N(0,1), batch 1 and 8."""
+    from glq_amd import hadamard as H
+    say("e8 config1", B)
+    torch.manual_seed(0)
+    Wt = (torch.randn(960, 960) * 0.02).numpy()
+    art, _ = O.e8_quantize_layer(Wt, bpw=2, seed=42)
+    assert art["blocks_n"] == [512, 256, 128, 64]
+    x = torch.randn(B, 960).to(torch.float16)
+    ref = O.e8_linear_forward(x.float().numpy(), art, 960, 960)
+    bn = bm = art["blocks_n"]
+    y = ext.glq_fused_linear_block_diag_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(art["Qidxs"]), e8_table_f16(), float(art["Wscale"]),
+        960, 960, 960, 960, torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV),
+        H.pack_block_meta(bm).to(DEV))
+    assert rel(y, ref) < TOL, rel(y, ref)
+    # and against the unquantised layer: 2 bpw E8 keeps ~9 dB
+    dense = x.float().numpy() @ Wt.T
+    assert rel(y, dense) < 0.5

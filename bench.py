@@ -1,0 +1,237 @@
+#!/usr/bin/env python3
+"""Headline benchmark: 4 bpw trellis-3INST batch-1 decode over SmolLM3-3B linear shapes.
+
+One "step" is the quantized-linear forward of the seven linears of one decoder layer
+(q, k, v, o, gate, up, down; input RHT -> fused decode GEMV -> output RHT each) at batch
+1 with bf16 activations.  The step's weights come from a pool of distinct layers that is
+walked round-robin, so every launch streams its packed weights from HBM rather than from
+the 256 MB Infinity Cache.  `value` is compressed-weight bytes per second over the timed
+steps (inputs resident in HBM, whole steps replayed from one HIP graph).
+
+Prints ONE JSON line on stdout; everything else goes to stderr.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+# (name, out_features, in_features) of one SmolLM3-3B decoder layer
+LINEARS = [("q", 2048, 2048), ("k", 512, 2048), ("v", 512, 2048), ("o", 2048, 2048),
+           ("gate", 11008, 2048), ("up", 11008, 2048), ("down", 2048, 11008)]
+K_BITS = 4
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_pool(torch, hadamard, n_layers, dev):
+    """Random code bits (every bit pattern is a valid tail-biting trellis stream), seeded
+    sign vectors, Wscale = 0.02 * opt_scale, i.e. weights of rms 0.02."""
+    g = torch.Generator(device=dev).manual_seed(0)
+    wscale = 0.02 * 0.8933837
+    shapes = {}
+    for name, m, n in LINEARS:
+        if (m, n) in shapes:
+            continue
+        bn, bm = hadamard.block_decompose(n), hadamard.block_decompose(m)
+        shapes[(m, n)] = dict(
+            bn=torch.tensor(bn, dtype=torch.int64), bm=torch.tensor(bm, dtype=torch.int64),
+            bn_meta=hadamard.pack_block_meta(bn).to(dev), bm_meta=hadamard.pack_block_meta(bm).to(dev))
+    pool = []
+    for _ in range(n_layers):
+        layer = []
+        for name, m, n in LINEARS:
+            packed = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 16 * K_BITS),
+                                   generator=g, device=dev, dtype=torch.int16)
+            su = (torch.randint(0, 2, (m,), generator=g, device=dev) * 2 - 1).to(torch.float16)
+            sv = (torch.randint(0, 2, (n,), generator=g, device=dev) * 2 - 1).to(torch.float16)
+            layer.append(dict(name=name, m=m, n=n, packed=packed, su=su, sv=sv, wscale=wscale,
+                              **shapes[(m, n)]))
+        pool.append(layer)
+    return pool
+
+
+def cpu_baseline(n_calls=10):
+    """The reference's CPU path for the same step (decode once and cache, then per call
+    FHT -> fp32 matmul -> FHT, glq/quantized_linear.py:986-1010), restated in the oracle,
+    on this host's cores.  Sample: one decoder layer (7 linears), weights decoded once
+    (timed separately), then n_calls forward steps."""
+    import numpy as np
+    from oracle import glq_oracle as O
+    rng = np.random.default_rng(0)
+    layers = []
+    t0 = time.perf_counter()
+    for i, (name, m, n) in enumerate(LINEARS):
+        packed = O.random_packed(m, n, K_BITS, seed=i)
+        su, sv = O.rht_signs(m, n, 42 + i)
+        W = O.decode_layer(packed, m, n, fast=True) * np.float32(0.02 * 0.8933837)
+        layers.append((m, n, W, su, sv, O.block_decompose(n), O.block_decompose(m)))
+    t_decode = time.perf_counter() - t0
+    xs = [rng.standard_normal((1, n)).astype(np.float32) for _, _, n in LINEARS]
+
+    def step():
+        for (m, n, W, su, sv, bn, bm), x in zip(layers, xs):
+            O.linear_forward_rht(x, W, su, sv, bn, bm, n, m)
+    step()
+    t0 = time.perf_counter()
+    for _ in range(n_calls):
+        step()
+    dt = (time.perf_counter() - t0) / n_calls
+    bytes_step = sum(m * n * K_BITS // 8 for _, m, n in LINEARS)
+    return {"value": round(bytes_step / dt / 1e9, 3), "unit": "GB/s", "cores": os.cpu_count(),
+            "kind": "port",
+            "sample": (f"one decoder layer (7 linears, 4 bpw, batch 1): weights decoded once in "
+                       f"{t_decode:.1f} s (not timed), then {n_calls} forward steps of fp32 FHT + "
+                       f"cached dense matmul + FHT, {dt * 1e3:.2f} ms/step; numpy with "
+                       f"multi-threaded BLAS for the matmul, single-threaded butterflies")}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=720)
+    ap.add_argument("--warmup", type=int, default=72)
+    ap.add_argument("--layers", type=int, default=36, help="distinct weight sets in the pool")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
+        sys.exit(2)
+
+    import torch
+    from glq_amd import _lib, ext, hadamard
+    _lib.load()                                       # fails loudly if the HIP library is absent
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU: the HIP path has no CPU fallback.")
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = max(1, args.layers)
+    pool = build_pool(torch, hadamard, L, dev)
+    xs = {n: torch.randn(1, n, generator=torch.Generator(device=dev).manual_seed(1), device=dev)
+          .to(torch.bfloat16) for _, _, n in LINEARS}
+    bytes_step = sum(m * n * K_BITS // 8 for _, m, n in LINEARS)
+    log(f"pool: {L} layers x {bytes_step / 1e6:.2f} MB packed = {L * bytes_step / 1e9:.2f} GB")
+
+    def run_step(layer):
+        out = None
+        for lin in layer:
+            out = ext.glq_fused_linear_trellis_3inst_cuda(
+                xs[lin["n"]], lin["sv"], lin["su"], lin["packed"], lin["bn"], lin["bm"],
+                lin["bn_meta"], lin["bm_meta"], lin["wscale"], lin["n"], lin["m"], lin["n"],
+                lin["m"], out_dtype=torch.bfloat16)
+        return out
+
+    # eager warm-up (also initialises the library outside of graph capture)
+    for i in range(min(L, 4)):
+        run_step(pool[i])
+    torch.cuda.synchronize()
+
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        def capture(n_steps):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                keep = [run_step(pool[i % L]) for i in range(n_steps)]
+            return g, keep
+        full, keep_full = capture(L)
+        K, W = args.steps, args.warmup
+        rem_graphs = {}
+
+        def replay_steps(n):
+            q, r = divmod(n, L)
+            for _ in range(q):
+                full.replay()
+            if r:
+                if r not in rem_graphs:
+                    rem_graphs[r] = capture(r)
+                rem_graphs[r][0].replay()
+        # capture any remainder graph before timing
+        for n in (W, K):
+            if n % L and (n % L) not in rem_graphs:
+                rem_graphs[n % L] = capture(n % L)
+        replay_steps(W)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        replay_steps(K)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    ms_per_step = dt / K * 1e3
+    value = bytes_step / (dt / K) / 1e9
+    log(f"timed {K} steps: {ms_per_step * 1e3:.1f} us/step, {value:.1f} GB/s packed weights")
+
+    # ---- roofline leg: the decode GEMV kernel alone, HIP events on its own stream -------
+    with torch.cuda.stream(stream):
+        xr = {n: torch.randn(1, n, device=dev).to(torch.float16) for _, _, n in LINEARS}
+        part = torch.empty(32 * 11008, dtype=torch.float32, device=dev)
+        for lin in pool[0]:
+            ext.trellis_gemv_partials(xr[lin["n"]], lin["packed"], lin["m"], lin["n"], part)
+        torch.cuda.synchronize()
+        gk = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gk, stream=stream):
+            for layer in pool:
+                for lin in layer:
+                    ext.trellis_gemv_partials(xr[lin["n"]], lin["packed"], lin["m"], lin["n"], part)
+        gk.replay()
+        torch.cuda.synchronize()
+        reps = 10
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            gk.replay()
+        e1.record(stream)
+        e1.synchronize()
+        n_launch = reps * L * len(LINEARS)
+        avg_us = e0.elapsed_time(e1) * 1e3 / n_launch
+    bytes_launch = bytes_step / len(LINEARS)
+    achieved = bytes_launch / (avg_us * 1e-6) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("tr_gemv_bytes_per_launch")
+        except Exception:
+            traffic = None
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "kernel": "tr_gemv_kernel<4,1>", "avg_launch_us": round(avg_us, 3),
+                "bytes_per_launch": int(bytes_launch),
+                "method": (f"{n_launch} back-to-back launches of the decode GEMV alone (the 7 layer "
+                           f"shapes x {L} distinct weight sets) replayed from a HIP graph between two "
+                           f"HIP events on the launch stream; bytes = packed weights m*n*4/8")}
+    log(f"decode GEMV alone: {avg_us:.2f} us/launch avg, {achieved:.0f} GB/s "
+        f"({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak)")
+
+    result = {
+        "metric": "4bpw GEMV effective HBM GB/s (% of peak); batch-1 decode tok/s, 3B shape",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic (random code bits, seeded signs, N(0,1) bf16 activations)",
+        "config": {"workload": "configs[1]: trellis-3INST 4 bpw linear set, SmolLM3-3B shapes "
+                               "(q/o 2048x2048, k/v 2048x512, gate/up 2048x11008, down 11008x2048), "
+                               "batch-1 fused linear (input RHT + GEMV + output RHT) per layer",
+                   "step": "7 linears of one decoder layer", "packed_bytes_per_step": bytes_step,
+                   "distinct_layers": L, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+                   "linear_only_tok_s_36_layers": round(1e3 / (ms_per_step * 36), 1)},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        log("timing the CPU baseline (oracle port of the reference CPU path) ...")
+        result["cpu_baseline"] = cpu_baseline()
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

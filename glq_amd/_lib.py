@@ -23,6 +23,8 @@ SIGNATURES = {
     "glqh_decode_matmul_trellis_3inst": (
         c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_i64, c_i64, c_dbl, c_vp, c_i64, c_int,
                 c_vp, c_sz, c_vp]),
+    "glqh_trellis_gemv_partials": (
+        c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_i64, c_i64, c_vp, c_sz, c_vp, c_vp]),
     "glqh_input_rht": (
         c_int, [c_vp, c_int, c_i64, c_vp, c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_vp, c_i64,
                 c_dbl, c_vp]),

@@ -128,6 +128,22 @@ extern "C" int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B, co
     return glqh_launch_reduce_splits((const float *)ws, ks, B * m, B, m, (float)wscale, out, out_stride, accum, st);
 }
 
+extern "C" int glqh_trellis_gemv_partials(const void *x_f16, int64_t B, const void *packed,
+                                          int64_t packed_rows, int64_t packed_cols, int64_t m,
+                                          int64_t k, float *part, size_t part_bytes, int *ksplit_out,
+                                          void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x_f16 && packed && part && ksplit_out, "trellis partials: null pointer");
+    GLQH_REQUIRE(B >= 1 && B <= 65535 * 8, "trellis partials: B=%lld out of range", (long long)B);
+    int R;
+    if (tr_bits_from_packed(packed_cols, 1, &R) || tr_check_shape(m, k, packed_rows)) return 1;
+    const int ks = glqh_trellis_pick_ksplit(m, k, B);
+    const size_t need = (size_t)ks * B * m * sizeof(float);
+    GLQH_REQUIRE(part_bytes >= need, "trellis partials: buffer of %zu bytes needed, got %zu", need, part_bytes);
+    *ksplit_out = ks;
+    return glqh_launch_trellis_partial(x_f16, B, packed, R, m, k, ks, part, (hipStream_t)stream);
+}
+
 // ---- RHT -------------------------------------------------------------------------
 extern "C" int glqh_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv_f16,
                               void *out, int out_dtype, int64_t B, int64_t in_features,

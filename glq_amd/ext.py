@@ -117,6 +117,22 @@ def glq_decode_matmul_trellis_3inst_cuda(x, trellis_packed, m, k, wscale=1.0, ou
     return _trellis_matmul(x, trellis_packed, m, k, wscale, out, accum)
 
 
+def trellis_gemv_partials(x2d, trellis_packed, m, k, part):
+    """Decode kernel alone: raw split-K partial sums into `part` (fp32, caller-owned);
+    returns the number of K slots written.  Not part of the reference surface."""
+    lib = _lib.load()
+    _chk(x2d, "x", torch.float16)
+    _chk(trellis_packed, "trellis_packed", torch.int16)
+    _chk(part, "part", torch.float32)
+    ks = C.c_int(0)
+    with torch.cuda.device(x2d.device):
+        check(lib.glqh_trellis_gemv_partials(
+            _p(x2d), x2d.shape[0], _p(trellis_packed), trellis_packed.shape[0],
+            trellis_packed.shape[1], int(m), int(k), _p(part), part.numel() * 4, C.byref(ks),
+            _stream()))
+    return ks.value
+
+
 # --------------------------------------------------------------------------- RHT
 def glq_input_rht_cuda(x, sv, out, in_features, stride_x, rsqrt_n, n_pad, log_n):
     lib = _lib.load()

@@ -63,6 +63,17 @@ int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B,
                                      float *out, int64_t out_stride, int accum,
                                      void *ws, size_t ws_bytes, void *stream);
 
+/* First of the two launches of glqh_decode_matmul_trellis_3inst, on its own: raw fp32
+ * split-K partial sums part[(slot*B + token)*m + row], slot < *ksplit_out, unscaled.
+ * For callers that fold the fixed-order reduction into their own consumer (as the fused
+ * linear does) and for timing the decode kernel in isolation.  The reference has no
+ * separate entry for this step (its GEMV reduces inside the block,
+ * glq/csrc/glq_trellis.cu:485-510). */
+int glqh_trellis_gemv_partials(const void *x_f16, int64_t B,
+                               const void *packed, int64_t packed_rows, int64_t packed_cols,
+                               int64_t m, int64_t k, float *part, size_t part_bytes,
+                               int *ksplit_out, void *stream);
+
 /* ---- randomized Hadamard transforms ------------------------------------- */
 
 /* out[b, 0:n_pad] = blockFHT(pad(x[b, 0:in_features]) * sv), per block 1/sqrt(bs).

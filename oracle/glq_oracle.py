@@ -316,6 +316,19 @@ def unpack_states(sb: np.ndarray, K: int) -> np.ndarray:
     return (bits[:, idx] * w).sum(-1).reshape(T, 256)
 
 
+def unpack_states_fast(sb: np.ndarray, K: int) -> np.ndarray:
+    """Same result as unpack_states, computed with 32-bit byte windows instead of a
+    bit array (an order of magnitude faster; used for full-size layers).  State t
+    starts at stream bit K t = 8 q + r: take bytes q..q+2 as a 24-bit big-endian
+    window and drop the 8 - r low bits."""
+    T, nbytes = sb.shape
+    ext = np.concatenate([sb, sb[:, :3]], axis=1).astype(np.uint32)
+    start = np.arange(256) * K
+    q, r = start >> 3, start & 7
+    win = (ext[:, q] << np.uint32(16)) | (ext[:, q + 1] << np.uint32(8)) | ext[:, q + 2]
+    return ((win >> (8 - r).astype(np.uint32)[None, :]) & np.uint32(0xFFFF)).astype(np.int64)
+
+
 def pack_states(states: np.ndarray, K: int) -> np.ndarray:
     """(T,256) states of a valid tail-biting path -> (T, 32K) stream bytes.
     Bit K t + i of the stream is bit (15-i) of state t; consecutive states must
@@ -343,18 +356,31 @@ def matrix_to_tiles(W: np.ndarray) -> np.ndarray:
     return nat[:, PERMUTE]
 
 
-def trellis_states(packed: np.ndarray, m: int, n: int) -> np.ndarray:
+def trellis_states(packed: np.ndarray, m: int, n: int, fast: bool = False) -> np.ndarray:
     K = trellis_bits_from_packed(packed)
     if packed.shape[0] != (m // 16) * (n // 16):
         raise ValueError("packed rows != (m/16)*(n/16)")
-    return unpack_states(kernel_to_stream_bytes(packed, m, n, K), K)
+    sb = kernel_to_stream_bytes(packed, m, n, K)
+    return unpack_states_fast(sb, K) if fast else unpack_states(sb, K)
 
 
-def decode_layer(packed: np.ndarray, m: int, n: int) -> np.ndarray:
+def decode_layer(packed: np.ndarray, m: int, n: int, fast: bool = False) -> np.ndarray:
     """Kernel-layout packed int16 -> normalised hatW (m,n) fp16-exact values in
-    fp32 (glq/trellis.py:629-643)."""
-    st = trellis_states(packed, m, n)
-    return tiles_to_matrix(lut_3inst()[st].astype(np.float32), m, n)
+    fp32 (glq/trellis.py:629-643).  fast=True uses unpack_states_fast and works in
+    strips of 32 rows to bound memory on full-size layers."""
+    if not fast:
+        st = trellis_states(packed, m, n)
+        return tiles_to_matrix(lut_3inst()[st].astype(np.float32), m, n)
+    lut = lut_3inst().astype(np.float32)
+    out = np.empty((m, n), dtype=np.float32)
+    per_strip = 2 * (n // 16)
+    rows = 256                                                   # strip height per pass
+    for r0 in range(0, m, rows):
+        h = min(rows, m - r0)
+        sub = packed[(r0 // 32) * per_strip:((r0 + h) // 32) * per_strip]
+        st = trellis_states(sub, h, n, fast=True)
+        out[r0:r0 + h] = tiles_to_matrix(lut[st], h, n)
+    return out
 
 
 def decode_layer_nstage(packed_list, cum_inv_rs, m, n) -> np.ndarray:

@@ -143,6 +143,15 @@ def test_viterbi_matches_reference(golden, K):
     assert np.array_equal(hat, g[f"K{K}_hat"])
 
 
+@pytest.mark.parametrize("K", [1, 2, 3, 4])
+def test_fast_unpack_equals_bit_array_unpack(K):
+    p = O.random_packed(64, 128, K, seed=40 + K)
+    sb = O.kernel_to_stream_bytes(p, 64, 128, K)
+    assert np.array_equal(O.unpack_states_fast(sb, K), O.unpack_states(sb, K))
+    big = O.random_packed(512, 192, K, seed=K)
+    assert np.array_equal(O.decode_layer(big, 512, 192, fast=True), O.decode_layer(big, 512, 192))
+
+
 def test_nstage_sum():
     p1 = O.random_packed(32, 64, 4, 1)
     p2 = O.random_packed(32, 64, 2, 2)

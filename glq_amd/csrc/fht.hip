@@ -1,10 +1,8 @@
 // Randomized Hadamard transforms around the quantized matmul.
 //
-// One workgroup transforms one power-of-two sub-block of one token.  The block is
-// staged in LDS as fp32 and the log2(bs) butterfly stages run in place in ascending
-// distance with (lo, hi) <- (a + b, a - b), the order the reference's CPU and CUDA
-// paths use (glq/hadamard.py:10-28, glq/csrc/glq_fht.cuh:14-21), followed by one
-// multiplication with 1/sqrt(bs).
+// One workgroup transforms one power-of-two sub-block of one token in fp32 and
+// multiplies once with 1/sqrt(bs) (glq/hadamard.py:10-28, glq/csrc/glq_fht.cuh:14-21,
+// glq/csrc/glq_cuda.cu:1756-1839, 2005-2079, 2092-2208).
 #include "common.h"
 
 namespace {
@@ -30,77 +28,179 @@ __device__ __forceinline__ rht_block rht_get_block(const glqh_block_meta *meta, 
     return b;
 }
 
-// In-place Walsh-Hadamard butterflies over s[0..bs) held in LDS.  All threads of the
-// workgroup must call it; ends with a barrier.
-__device__ __forceinline__ void fht_lds(float *s, int bs) {
-    const int tid = threadIdx.x;
-    const int nthr = blockDim.x;
-    for (int h = 1; h < bs; h <<= 1) {
-        __syncthreads();
-        for (int p = tid; p < (bs >> 1); p += nthr) {
-            int i = ((p & ~(h - 1)) << 1) | (p & (h - 1));
-            int j = i | h;
-            float a = s[i], b = s[j];
-            s[i] = a + b;
-            s[j] = a - b;
+// ---------------------------------------------------------------------------------
+// Block transform in a few register-radix passes.
+//
+// The log2(bs) index bits are split into fields of at most RMAX bits, taken from the top
+// bit down.  In one pass a thread owns groups of 2^r elements that differ only in the
+// field's bits, runs the field's r butterfly stages in registers and puts the group
+// back.  The first pass reads its elements through `load` (global memory: consecutive
+// lanes touch consecutive addresses), the last pass hands them to `store`; in between
+// the block lives in LDS with one pad word per 32 so that the strided accesses of the
+// low fields stay conflict-free.  A butterfly stage is (lo, hi) <- (a + b, a - b); the
+// stages of different bits commute, so the result is the Walsh-Hadamard transform of
+// the block (summation order differs from the ascending-distance order of
+// glq/hadamard.py:10-28 by fp32 rounding only).
+// ---------------------------------------------------------------------------------
+constexpr int RMAX = 5;
+
+__device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
+
+template <int R, bool FIRST, bool LAST, class Load, class Store>
+__device__ __forceinline__ void fht_pass(float *lds, int bs, int s, Load &load, Store &store) {
+    constexpr int N = 1 << R;
+    const int ngroups = bs >> R;
+    for (int g = threadIdx.x; g < ngroups; g += blockDim.x) {
+        const int lo = g & ((1 << s) - 1);
+        const int base = ((g >> s) << (s + R)) | lo;
+        float v[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) {                       // N independent loads in flight
+            const int idx = base + (j << s);
+            if constexpr (FIRST) v[j] = load(idx);
+            else v[j] = lds[lds_pad(idx)];
         }
-    }
-    __syncthreads();
-}
-
-__global__ void __launch_bounds__(RHT_THREADS)
-input_rht_kernel(const void *__restrict__ x, int x_dtype, int64_t x_stride,
-                 const f16 *__restrict__ sv, void *__restrict__ out, int out_dtype,
-                 int in_features, int n_pad, const glqh_block_meta *__restrict__ meta,
-                 glqh_block_meta single, float single_norm) {
-    extern __shared__ float s[];
-    const rht_block blk = rht_get_block(meta, single, single_norm);
-    const int64_t b = blockIdx.y;
-    for (int i = threadIdx.x; i < blk.bs; i += blockDim.x) {
-        int col = blk.off + i;
-        float v = 0.0f;
-        if (col < in_features) v = load_act(x, x_dtype, b * x_stride + col) * (float)sv[col];
-        s[i] = v;
-    }
-    fht_lds(s, blk.bs);
-    for (int i = threadIdx.x; i < blk.bs; i += blockDim.x)
-        store_act(out, out_dtype, b * (int64_t)n_pad + blk.off + i, s[i] * blk.norm);
-}
-
-__global__ void __launch_bounds__(RHT_THREADS)
-output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, void *__restrict__ y, int y_dtype,
-                  int64_t y_stride, int out_features, int m_pad,
-                  const glqh_block_meta *__restrict__ meta, glqh_block_meta single,
-                  float single_norm) {
-    extern __shared__ float s[];
-    const rht_block blk = rht_get_block(meta, single, single_norm);
-    const int64_t b = blockIdx.y;
-    for (int i = threadIdx.x; i < blk.bs; i += blockDim.x) {
-        int row = blk.off + i;
-        float v;
-        if (src.nparts == 0) {
-            v = src.direct[b * src.stride + row];
-        } else {
-            // fixed-order sum of the split-K partials of each stage: deterministic
-            v = 0.0f;
-            for (int st = 0; st < src.nparts; ++st) {
-                const float *p = src.part[st] + b * (int64_t)m_pad + row;
-                float acc = 0.0f;
-                for (int k = 0; k < src.ksplit; ++k) acc += p[(int64_t)k * src.part_kstride];
-                v += src.scale[st] * acc;
+#pragma unroll
+        for (int h = 1; h < N; h <<= 1) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                if ((j & h) == 0) {
+                    const float a = v[j], b = v[j | h];
+                    v[j] = a + b;
+                    v[j | h] = a - b;
+                }
             }
-            if (src.copy_out) src.copy_out[b * src.copy_stride + row] = v;
         }
-        s[i] = v;
-    }
-    if (y == nullptr) return;                 // caller only wanted the RHT-domain row
-    fht_lds(s, blk.bs);
-    for (int i = threadIdx.x; i < blk.bs; i += blockDim.x) {
-        int row = blk.off + i;
-        if (row < out_features)
-            store_act(y, y_dtype, b * y_stride + row, s[i] * blk.norm * (float)su[row]);
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = base + (j << s);
+            if constexpr (LAST) store(idx, v[j]);
+            else lds[lds_pad(idx)] = v[j];
+        }
     }
 }
+
+template <bool FIRST, bool LAST, class Load, class Store>
+__device__ __forceinline__ void fht_pass_r(int r, float *lds, int bs, int s, Load &load, Store &store) {
+    switch (r) {
+    case 1: fht_pass<1, FIRST, LAST>(lds, bs, s, load, store); break;
+    case 2: fht_pass<2, FIRST, LAST>(lds, bs, s, load, store); break;
+    case 3: fht_pass<3, FIRST, LAST>(lds, bs, s, load, store); break;
+    case 4: fht_pass<4, FIRST, LAST>(lds, bs, s, load, store); break;
+    default: fht_pass<5, FIRST, LAST>(lds, bs, s, load, store); break;
+    }
+}
+
+// All threads of the workgroup must call it.  lds needs bs + bs/32 floats.  With
+// STAGED the block is already in LDS (padded layout) and `load` is not used.
+template <bool STAGED, class Load, class Store>
+__device__ __forceinline__ void fht_block(float *lds, int log_bs, Load load, Store store) {
+    const int bs = 1 << log_bs;
+    if (log_bs == 0) {
+        if (threadIdx.x == 0) store(0, STAGED ? lds[0] : load(0));
+        return;
+    }
+    const int npass = (log_bs + RMAX - 1) / RMAX;
+    int s = log_bs;
+    for (int p = 0; p < npass; ++p) {
+        const int left = npass - p;
+        const int r = (s + left - 1) / left;              // balanced field widths
+        s -= r;
+        const bool first = p == 0 && !STAGED, last = p == npass - 1;
+        if (first && last) fht_pass_r<true, true>(r, lds, bs, s, load, store);
+        else if (first) fht_pass_r<true, false>(r, lds, bs, s, load, store);
+        else if (last) fht_pass_r<false, true>(r, lds, bs, s, load, store);
+        else fht_pass_r<false, false>(r, lds, bs, s, load, store);
+        if (!last) __syncthreads();
+    }
+}
+
+template <typename T> __device__ __forceinline__ float act_to_f32(T v);
+template <> __device__ __forceinline__ float act_to_f32<f16>(f16 v) { return (float)v; }
+template <> __device__ __forceinline__ float act_to_f32<uint16_t>(uint16_t v) { return bf16_bits_to_f32(v); }
+template <> __device__ __forceinline__ float act_to_f32<float>(float v) { return v; }
+template <typename T> __device__ __forceinline__ T f32_to_act(float v);
+template <> __device__ __forceinline__ f16 f32_to_act<f16>(float v) { return (f16)v; }
+template <> __device__ __forceinline__ uint16_t f32_to_act<uint16_t>(float v) { return f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ float f32_to_act<float>(float v) { return v; }
+
+// XT / OT: element types (bf16 travels as uint16_t)
+template <typename XT, typename OT>
+__global__ void __launch_bounds__(RHT_THREADS)
+input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
+                 OT *__restrict__ out, int in_features, int n_pad,
+                 const glqh_block_meta *__restrict__ meta, glqh_block_meta single,
+                 float single_norm) {
+    extern __shared__ float s[];
+    const rht_block blk = rht_get_block(meta, single, single_norm);
+    const XT *xr = x + (int64_t)blockIdx.y * x_stride;
+    OT *orow = out + (int64_t)blockIdx.y * n_pad + blk.off;
+    auto load = [&](int i) -> float {
+        const int col = blk.off + i;
+        return col < in_features ? act_to_f32<XT>(xr[col]) * (float)sv[col] : 0.0f;
+    };
+    auto store = [&](int i, float v) { orow[i] = f32_to_act<OT>(v * blk.norm); };
+    fht_block<false>(s, blk.log_bs, load, store);
+}
+
+template <typename YT, bool PARTS>
+__global__ void __launch_bounds__(RHT_THREADS)
+output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
+                  int out_features, int m_pad, const glqh_block_meta *__restrict__ meta,
+                  glqh_block_meta single, float single_norm) {
+    extern __shared__ float s[];
+    const rht_block blk = rht_get_block(meta, single, single_norm);
+    const int64_t b = blockIdx.y;
+    YT *yrow = y + b * y_stride;
+    auto store = [&](int i, float v) {
+        const int row = blk.off + i;
+        if (row < out_features) yrow[row] = f32_to_act<YT>(v * blk.norm * (float)su[row]);
+    };
+    if constexpr (!PARTS) {
+        const float *__restrict__ d = src.direct + b * src.stride + blk.off;
+        auto load = [&](int i) -> float { return d[i]; };
+        fht_block<false>(s, blk.log_bs, load, store);
+    } else {
+        // Stage the block into LDS while summing the split-K partials of each stage in a
+        // fixed order (deterministic).  Eight rows per thread are in flight at once.
+        constexpr int U = 8;
+        const int bs = blk.bs;
+        for (int i0 = threadIdx.x; i0 < bs; i0 += U * RHT_THREADS) {
+            float tot[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) tot[u] = 0.0f;
+            for (int st = 0; st < src.nparts; ++st) {
+                const float *__restrict__ p = src.part[st] + b * (int64_t)m_pad + blk.off;
+                float acc[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) acc[u] = 0.0f;
+#pragma unroll 4
+                for (int k = 0; k < src.ksplit; ++k) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int i = i0 + u * RHT_THREADS;
+                        acc[u] += i < bs ? p[(int64_t)k * src.part_kstride + i] : 0.0f;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) tot[u] += src.scale[st] * acc[u];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = i0 + u * RHT_THREADS;
+                if (i < bs) {
+                    s[lds_pad(i)] = tot[u];
+                    if (src.copy_out) src.copy_out[b * src.copy_stride + blk.off + i] = tot[u];
+                }
+            }
+        }
+        __syncthreads();
+        auto load = [&](int i) -> float { return 0.0f; };
+        fht_block<true>(s, blk.log_bs, load, store);
+    }
+}
+
+size_t rht_lds_bytes(int64_t max_bs) { return (size_t)(max_bs + max_bs / 32 + 32) * sizeof(float); }
 
 int check_blocks(const int64_t *blocks_host, int64_t n_blocks, int64_t total, int64_t *max_bs,
                  const char *what) {
@@ -149,11 +249,23 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
         meta_dev = nullptr;
         n_blocks = 1;
     }
-    GLQH_REQUIRE(max_bs * 4 <= GLQH_MAX_LDS_BYTES, "input_rht: block of %lld exceeds LDS", (long long)max_bs);
+    GLQH_REQUIRE(rht_lds_bytes(max_bs) <= GLQH_MAX_LDS_BYTES, "input_rht: block of %lld exceeds LDS", (long long)max_bs);
     dim3 grid((unsigned)n_blocks, (unsigned)B);
-    hipLaunchKernelGGL(input_rht_kernel, grid, dim3(RHT_THREADS), (size_t)max_bs * 4, stream, x, x_dtype,
-                       x_stride, (const f16 *)sv, out, out_dtype, (int)in_features, (int)n_pad,
-                       meta_dev, single, rsqrt_n);
+    const size_t lds = rht_lds_bytes(max_bs);
+#define GLQH_IN_LAUNCH(XT, OT)                                                                      \
+    hipLaunchKernelGGL((input_rht_kernel<XT, OT>), grid, dim3(RHT_THREADS), lds, stream,            \
+                       (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
+                       (int)n_pad, meta_dev, single, rsqrt_n)
+    if (out_dtype == GLQH_F32) {
+        if (x_dtype == GLQH_F16) GLQH_IN_LAUNCH(f16, float);
+        else if (x_dtype == GLQH_BF16) GLQH_IN_LAUNCH(uint16_t, float);
+        else GLQH_IN_LAUNCH(float, float);
+    } else {
+        if (x_dtype == GLQH_F16) GLQH_IN_LAUNCH(f16, f16);
+        else if (x_dtype == GLQH_BF16) GLQH_IN_LAUNCH(uint16_t, f16);
+        else GLQH_IN_LAUNCH(float, f16);
+    }
+#undef GLQH_IN_LAUNCH
     GLQH_LAUNCH_CHECK("input_rht launch");
     return 0;
 }
@@ -164,7 +276,7 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
                            int64_t n_blocks, int64_t max_bs_hint, float rsqrt_m,
                            hipStream_t stream) {
     GLQH_REQUIRE(B >= 1 && B <= 65535, "output_rht: B=%lld out of range", (long long)B);
-    GLQH_REQUIRE(y == nullptr || su != nullptr, "output_rht: null su");
+    GLQH_REQUIRE(y != nullptr && su != nullptr, "output_rht: null y or su");
     GLQH_REQUIRE(out_features >= 1 && out_features <= m_pad,
                  "output_rht: out_features %lld must be in 1..m_pad=%lld", (long long)out_features,
                  (long long)m_pad);
@@ -187,21 +299,45 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
         meta_dev = nullptr;
         n_blocks = 1;
     }
-    GLQH_REQUIRE(max_bs * 4 <= GLQH_MAX_LDS_BYTES, "output_rht: block of %lld exceeds LDS", (long long)max_bs);
+    GLQH_REQUIRE(rht_lds_bytes(max_bs) <= GLQH_MAX_LDS_BYTES, "output_rht: block of %lld exceeds LDS", (long long)max_bs);
     dim3 grid((unsigned)n_blocks, (unsigned)B);
-    hipLaunchKernelGGL(output_rht_kernel, grid, dim3(RHT_THREADS), (size_t)max_bs * 4, stream, src,
-                       (const f16 *)su, y, y_dtype, y_stride, (int)out_features, (int)m_pad,
-                       meta_dev, single, rsqrt_m);
+    const size_t lds = rht_lds_bytes(max_bs);
+#define GLQH_OUT_LAUNCH(YT, PARTS)                                                                  \
+    hipLaunchKernelGGL((output_rht_kernel<YT, PARTS>), grid, dim3(RHT_THREADS), lds, stream, src,   \
+                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, meta_dev, \
+                       single, rsqrt_m)
+    if (src.nparts == 0) {
+        if (y_dtype == GLQH_F16) GLQH_OUT_LAUNCH(f16, false);
+        else if (y_dtype == GLQH_BF16) GLQH_OUT_LAUNCH(uint16_t, false);
+        else GLQH_OUT_LAUNCH(float, false);
+    } else {
+        if (y_dtype == GLQH_F16) GLQH_OUT_LAUNCH(f16, true);
+        else if (y_dtype == GLQH_BF16) GLQH_OUT_LAUNCH(uint16_t, true);
+        else GLQH_OUT_LAUNCH(float, true);
+    }
+#undef GLQH_OUT_LAUNCH
     GLQH_LAUNCH_CHECK("output_rht launch");
     return 0;
 }
 
-int glqh_rht_init(void) {
-    int rc = glqh_check_hip(hipFuncSetAttribute((const void *)input_rht_kernel,
-                                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                GLQH_MAX_LDS_BYTES), "input_rht attribute");
-    if (rc) return rc;
-    return glqh_check_hip(hipFuncSetAttribute((const void *)output_rht_kernel,
+template <typename K>
+static int set_max_lds(K kernel, const char *what) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel,
                                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              GLQH_MAX_LDS_BYTES), "output_rht attribute");
+                                              GLQH_MAX_LDS_BYTES), what);
+}
+
+int glqh_rht_init(void) {
+    return set_max_lds(input_rht_kernel<f16, float>, "input_rht attribute") ||
+           set_max_lds(input_rht_kernel<uint16_t, float>, "input_rht attribute") ||
+           set_max_lds(input_rht_kernel<float, float>, "input_rht attribute") ||
+           set_max_lds(input_rht_kernel<f16, f16>, "input_rht attribute") ||
+           set_max_lds(input_rht_kernel<uint16_t, f16>, "input_rht attribute") ||
+           set_max_lds(input_rht_kernel<float, f16>, "input_rht attribute") ||
+           set_max_lds(output_rht_kernel<f16, false>, "output_rht attribute") ||
+           set_max_lds(output_rht_kernel<uint16_t, false>, "output_rht attribute") ||
+           set_max_lds(output_rht_kernel<float, false>, "output_rht attribute") ||
+           set_max_lds(output_rht_kernel<f16, true>, "output_rht attribute") ||
+           set_max_lds(output_rht_kernel<uint16_t, true>, "output_rht attribute") ||
+           set_max_lds(output_rht_kernel<float, true>, "output_rht attribute");
 }

@@ -286,6 +286,7 @@ static int e8_resolve_stages(const void *q1, const void *q2, const void *q3, con
     GLQH_REQUIRE(q1 && table1, "e8 matmul: null index or table pointer");
     out->q[0] = q1; out->q[1] = q1; out->q[2] = q1; out->q[3] = q1;
     out->scale[0] = (float)wscale;
+    out->scale[1] = out->scale[2] = out->scale[3] = 0.0f;
     out->n = 1;
     if (q2 && inv_rs != 0.0) {
         GLQH_REQUIRE(table2 && n_entries2 >= 1 && n_entries2 <= 65536,
@@ -351,6 +352,21 @@ extern "C" int glqh_e8_dequant_matmul(const void *x_f16, int64_t B, const void *
                                       sg.scale[s], out, m_pad, s > 0, st))
             return 1;
     return 0;
+}
+
+extern "C" int glqh_e8_decompress(const void *q1, const void *q2, const void *q3, const void *q4,
+                                  const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                  double inv_rs, double inv_rs2, double inv_rs3, int64_t m_pad,
+                                  int64_t n_pad, void *out_f16, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(out_f16, "e8 decompress: null pointer");
+    e8_stages sg;
+    if (e8_check_dims(m_pad, n_pad, 1) ||
+        e8_resolve_stages(q1, q2, q3, q4, 1.0, inv_rs, inv_rs2, inv_rs3, table1, table2, n_entries2, &sg))
+        return 1;
+    return glqh_launch_e8_decompress(sg.q, sg.n, table1, table2 ? table2 : table1,
+                                     table2 ? n_entries2 : 65536, sg.scale[1], sg.scale[2], sg.scale[3],
+                                     m_pad, n_pad, out_f16, (hipStream_t)stream);
 }
 
 extern "C" size_t glqh_fused_linear_e8_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {

@@ -100,3 +100,6 @@ int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, 
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream);
+int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,
+                              const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
+                              int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream);

@@ -138,6 +138,47 @@ e8_gemv_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
         }
 }
 
+// Dense fp16 weight (m_pad, n_pad) in the RHT domain, before Wscale: stages combined in
+// fp32 and rounded once (the reference's batched path rounds the combined weight to fp16
+// as well, glq/csrc/glq_cuda.cu:868-899).  One thread per 8-column block.
+__global__ void __launch_bounds__(256)
+e8_decompress_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
+                     const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
+                     const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n2,
+                     float s2, float s3, float s4, int nstages, int64_t total_blocks,
+                     f16 *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total_blocks) return;
+    float w[8];
+    {
+        const uint32_t word = t1[q1[i]];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            f16x2 v = e8_pair(word, p);
+            w[2 * p] = (float)v.x;
+            w[2 * p + 1] = (float)v.y;
+        }
+    }
+    const uint16_t *qs[3] = {q2, q3, q4};
+    const float sc[3] = {s2, s3, s4};
+    for (int st = 1; st < nstages; ++st) {
+        uint32_t idx = qs[st - 1][i];
+        uint32_t word;
+        if (st == 1) word = t2[idx < n2 ? idx : n2 - 1];
+        else word = t1[idx];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            f16x2 v = e8_pair(word, p);
+            w[2 * p] += sc[st - 1] * (float)v.x;
+            w[2 * p + 1] += sc[st - 1] * (float)v.y;
+        }
+    }
+    f16 o[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) o[c] = (f16)w[c];
+    *(u32x4 *)(out + i * 8) = *(const u32x4 *)o;
+}
+
 template <int NS>
 int launch_e8_NS(const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
                  const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, int ksplit,
@@ -197,4 +238,16 @@ int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int
     case 4: return launch_e8_NS<4>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
     }
     return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
+}
+
+int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,
+                              const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
+                              int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream) {
+    const int64_t total = m_pad * (n_pad / 8);
+    hipLaunchKernelGGL(e8_decompress_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
+                       (const uint16_t *)q[3], t1, t2, (uint32_t)n2, s2, s3, s4, nstages, total,
+                       (f16 *)out);
+    GLQH_LAUNCH_CHECK("e8 decompress launch");
+    return 0;
 }

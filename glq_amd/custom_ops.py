@@ -1,0 +1,181 @@
+"""``torch.ops.glq.*`` for the quantized-linear path, backed by libglq_hip.so.
+
+Same op names and schemas as the reference's registration
+(glq_vllm/custom_ops.py:56-131, 359-428), so the call sites that prefer
+``torch.ops.glq.<op>`` when it exists (glq/quantized_linear.py:863-896, 1079-1120,
+glq_vllm/linear_method.py:451, 664-710) run unchanged, and torch.compile / graph capture
+see one opaque node per linear.  Fake (meta) implementations give shapes and dtypes
+without touching data.  On ROCm the dispatch key of GPU tensors is "CUDA".
+
+One widening: the fused ops accept bf16 activations and then return bf16 (the reference
+only ever passes fp16 and gets fp16 back, which is unchanged).
+"""
+from __future__ import annotations
+
+import torch
+from torch.library import Library
+
+_lib = Library("glq", "FRAGMENT")
+_registered = False
+
+SCHEMAS = {
+    "dequant_matvec": "dequant_matvec(Tensor x, Tensor qidxs, Tensor codebook, float wscale, "
+                      "Tensor qidxs2, Tensor codebook2, float inv_resid_scale, "
+                      "Tensor codebook_abs) -> Tensor",
+    "dequant_matmul": "dequant_matmul(Tensor x, Tensor qidxs, Tensor codebook, float wscale, "
+                      "Tensor qidxs2, Tensor codebook2, float inv_resid_scale, "
+                      "Tensor codebook_abs, "
+                      "Tensor qidxs3, Tensor codebook3, float inv_resid_scale2, "
+                      "Tensor qidxs4, Tensor codebook4, float inv_resid_scale3) -> Tensor",
+    "input_rht": "input_rht(Tensor x, Tensor sv, Tensor(a!) out, int in_features, "
+                 "int stride_x, float rsqrt_n, int n_pad, int log_n) -> ()",
+    "output_rht": "output_rht(Tensor y_rht, Tensor su, Tensor(a!) out, int out_features, "
+                  "int m_pad, int log_m, float rsqrt_m) -> ()",
+    "fused_linear": "fused_linear(Tensor x, Tensor sv, Tensor su, "
+                    "Tensor qidxs, Tensor codebook, float wscale, "
+                    "int in_features, int out_features, "
+                    "int n_pad, int m_pad, int log_n, int log_m, "
+                    "Tensor qidxs2, Tensor codebook2, float inv_resid_scale, "
+                    "Tensor qidxs3, Tensor codebook3, float inv_resid_scale2, "
+                    "Tensor qidxs4, Tensor codebook4, float inv_resid_scale3) -> Tensor",
+    "fused_linear_block_diag": "fused_linear_block_diag(Tensor x, Tensor sv, Tensor su, "
+                               "Tensor qidxs, Tensor codebook, float wscale, "
+                               "int in_features, int out_features, int n_pad, int m_pad, "
+                               "Tensor blocks_n, Tensor blocks_m, "
+                               "Tensor blocks_n_meta, Tensor blocks_m_meta, "
+                               "Tensor qidxs2, Tensor codebook2, float inv_resid_scale, "
+                               "Tensor qidxs3, Tensor codebook3, float inv_resid_scale2, "
+                               "Tensor qidxs4, Tensor codebook4, float inv_resid_scale3) -> Tensor",
+    "fused_linear_trellis_3inst": "fused_linear_trellis_3inst(Tensor x, Tensor sv, Tensor su, "
+                                  "Tensor trellis_packed, "
+                                  "Tensor blocks_n, Tensor blocks_m, Tensor blocks_n_meta, "
+                                  "Tensor blocks_m_meta, "
+                                  "float wscale, int in_features, int out_features, "
+                                  "int n_pad, int m_pad) -> Tensor",
+    "fused_linear_trellis_3inst_yrht": "fused_linear_trellis_3inst_yrht(Tensor x, Tensor sv, "
+                                       "Tensor trellis_packed, "
+                                       "Tensor blocks_n, Tensor blocks_n_meta, float wscale, "
+                                       "int in_features, int n_pad, int m_pad, "
+                                       "Tensor(a!) y_rht_out, int col) -> ()",
+    "fused_linear_trellis_3inst_rvq2": "fused_linear_trellis_3inst_rvq2(Tensor x, Tensor sv, Tensor su, "
+                                       "Tensor trellis_packed, Tensor trellis_packed2, "
+                                       "Tensor blocks_n, Tensor blocks_m, Tensor blocks_n_meta, "
+                                       "Tensor blocks_m_meta, "
+                                       "float wscale, float inv_resid_scale2, int in_features, "
+                                       "int out_features, int n_pad, int m_pad) -> Tensor",
+    "fused_linear_trellis_3inst_yrht_rvq2": "fused_linear_trellis_3inst_yrht_rvq2(Tensor x, Tensor sv, "
+                                            "Tensor trellis_packed, Tensor trellis_packed2, "
+                                            "Tensor blocks_n, Tensor blocks_n_meta, float wscale, "
+                                            "float inv_resid_scale2, "
+                                            "int in_features, int n_pad, int m_pad, "
+                                            "Tensor(a!) y_rht_out, int col) -> ()",
+    "output_rht_shards": "output_rht_shards(Tensor y_rht, Tensor su, Tensor(a!) y, "
+                         "int out_features, Tensor shard_meta, int max_bs) -> ()",
+}
+
+
+def _act_dtype(x):
+    return x.dtype if x.dtype in (torch.float16, torch.bfloat16) else torch.float16
+
+
+# ---- fake implementations (shapes / dtypes only) ---------------------------------------
+def _dequant_matvec_fake(x, qidxs, codebook, wscale, qidxs2, codebook2, inv_resid_scale, codebook_abs):
+    return x.new_empty((qidxs.shape[0],), dtype=torch.float32)
+
+
+def _dequant_matmul_fake(x, qidxs, codebook, wscale, qidxs2, codebook2, inv_resid_scale, codebook_abs,
+                         qidxs3, codebook3, inv_resid_scale2, qidxs4, codebook4, inv_resid_scale3):
+    return x.new_empty((x.shape[0], qidxs.shape[0]), dtype=torch.float32)
+
+
+def _none_fake(*args):
+    return None
+
+
+def _fused_linear_fake(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad, m_pad,
+                       log_n, log_m, qidxs2, codebook2, inv_resid_scale, qidxs3, codebook3,
+                       inv_resid_scale2, qidxs4, codebook4, inv_resid_scale3):
+    return x.new_empty((x.shape[0], out_features), dtype=_act_dtype(x))
+
+
+def _fused_linear_block_diag_fake(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad,
+                                  m_pad, blocks_n, blocks_m, blocks_n_meta, blocks_m_meta, qidxs2,
+                                  codebook2, inv_resid_scale, qidxs3, codebook3, inv_resid_scale2,
+                                  qidxs4, codebook4, inv_resid_scale3):
+    return x.new_empty((x.shape[0], out_features), dtype=_act_dtype(x))
+
+
+def _fused_linear_trellis_3inst_fake(x, sv, su, trellis_packed, blocks_n, blocks_m, blocks_n_meta,
+                                     blocks_m_meta, wscale, in_features, out_features, n_pad, m_pad):
+    return x.new_empty((x.shape[0], out_features), dtype=_act_dtype(x))
+
+
+def _fused_linear_trellis_3inst_rvq2_fake(x, sv, su, trellis_packed, trellis_packed2, blocks_n,
+                                          blocks_m, blocks_n_meta, blocks_m_meta, wscale,
+                                          inv_resid_scale2, in_features, out_features, n_pad, m_pad):
+    return x.new_empty((x.shape[0], out_features), dtype=_act_dtype(x))
+
+
+FAKES = {
+    "dequant_matvec": _dequant_matvec_fake,
+    "dequant_matmul": _dequant_matmul_fake,
+    "input_rht": _none_fake,
+    "output_rht": _none_fake,
+    "fused_linear": _fused_linear_fake,
+    "fused_linear_block_diag": _fused_linear_block_diag_fake,
+    "fused_linear_trellis_3inst": _fused_linear_trellis_3inst_fake,
+    "fused_linear_trellis_3inst_yrht": _none_fake,
+    "fused_linear_trellis_3inst_rvq2": _fused_linear_trellis_3inst_rvq2_fake,
+    "fused_linear_trellis_3inst_yrht_rvq2": _none_fake,
+    "output_rht_shards": _none_fake,
+}
+
+
+def _impls():
+    from . import ext
+
+    def fused_linear(x, *a):
+        return ext.glq_fused_linear_cuda(x, *a, out_dtype=_act_dtype(x))
+
+    def fused_linear_block_diag(x, *a):
+        return ext.glq_fused_linear_block_diag_cuda(x, *a, out_dtype=_act_dtype(x))
+
+    def fused_linear_trellis_3inst(x, *a):
+        return ext.glq_fused_linear_trellis_3inst_cuda(x, *a, out_dtype=_act_dtype(x))
+
+    def fused_linear_trellis_3inst_rvq2(x, *a):
+        return ext.glq_fused_linear_trellis_3inst_rvq2_cuda(x, *a, out_dtype=_act_dtype(x))
+
+    return {
+        "dequant_matvec": ext.glq_dequant_matvec_cuda,
+        "dequant_matmul": ext.glq_dequant_matmul_cuda,
+        "input_rht": ext.glq_input_rht_cuda,
+        "output_rht": ext.glq_output_rht_cuda,
+        "fused_linear": fused_linear,
+        "fused_linear_block_diag": fused_linear_block_diag,
+        "fused_linear_trellis_3inst": fused_linear_trellis_3inst,
+        "fused_linear_trellis_3inst_yrht": ext.glq_fused_linear_trellis_3inst_yrht_cuda,
+        "fused_linear_trellis_3inst_rvq2": fused_linear_trellis_3inst_rvq2,
+        "fused_linear_trellis_3inst_yrht_rvq2": ext.glq_fused_linear_trellis_3inst_yrht_rvq2_cuda,
+        "output_rht_shards": ext.glq_output_rht_shards_cuda,
+    }
+
+
+def register():
+    """Define the ops and attach the HIP implementations.  Idempotent; raises if the
+    library cannot be loaded (there is nothing to fall back to)."""
+    global _registered
+    if _registered:
+        return
+    from . import _lib as loader
+    loader.load()
+    impls = _impls()
+    for name, schema in SCHEMAS.items():
+        _lib.define(schema)
+        _lib.impl(name, impls[name], "CUDA")
+        _lib._register_fake(name, FAKES[name])
+    _registered = True
+
+
+def is_registered() -> bool:
+    return _registered

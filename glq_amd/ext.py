@@ -15,7 +15,7 @@ so the result can be written in the caller's dtype without a cast kernel.
 from __future__ import annotations
 
 import ctypes as C
-import math
+import os
 
 import torch
 
@@ -23,6 +23,13 @@ from . import _lib
 from ._lib import GLQH_BF16, GLQH_F16, GLQH_F32, check
 
 _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F32}
+
+# Token counts above these take the dense route: dequantize the weight to fp16 once with
+# the HIP kernel, then one library GEMM (hipBLASLt through torch.matmul), as the reference
+# does above GLQ_TRELLIS_BATCH_MAX (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334).  Below
+# them the weights stay compressed and are re-read once per token group.
+TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "64")))
+E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "16")))
 
 
 def _p(t):
@@ -225,6 +232,13 @@ def _fused_trellis(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_m
     yrp, yrs = C.c_void_p(0), 0
     if y_rht_out is not None:
         yrp, yrs = y_rht_out
+    if B > TRELLIS_BATCH_MAX and y_rht_out is None:
+        if (packed2 is not None and packed2.numel() > 0) != (float(inv_rs2) != 0.0):
+            raise RuntimeError("trellis RVQ stage 2 is half-configured: trellis_packed2 is "
+                               f"{'present' if has2 else 'absent'} but inv_resid_scale2 = {inv_rs2}")
+        return _trellis_dense(x, sv, su, packed, packed2 if has2 else None, blocks_n, blocks_m,
+                              bn_meta, bm_meta, wscale, inv_rs2, in_features, out_features, n_pad,
+                              m_pad, y)
     with torch.cuda.device(x.device):
         nb = lib.glqh_fused_linear_trellis_workspace_bytes(B, int(n_pad), int(m_pad))
         ws = _ws(nb, x.device)
@@ -238,6 +252,22 @@ def _fused_trellis(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_m
             float(wscale), float(inv_rs2), int(in_features), int(out_features), int(n_pad), int(m_pad),
             _p(y) if y is not None else None, _DT[y.dtype] if y is not None else GLQH_F16,
             y.shape[1] if y is not None else ystride, yrp, int(yrs), _p(ws), ws.numel(), _stream()))
+    return y
+
+
+def _trellis_dense(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_meta, wscale,
+                   inv_rs2, in_features, out_features, n_pad, m_pad, y):
+    """Many tokens: input RHT (fp16) -> fp16 weight from the decompress kernel -> one GEMM
+    with fp32 accumulation -> x wscale -> output RHT."""
+    B = x.shape[0]
+    x_rht = torch.empty((B, int(n_pad)), dtype=torch.float16, device=x.device)
+    glq_input_rht_blockdiag_cuda(x, sv, x_rht, in_features, n_pad, blocks_n, bn_meta)
+    W = glq_decompress_trellis_3inst_cuda(packed, m_pad, n_pad)
+    if packed2 is not None:
+        W.add_(glq_decompress_trellis_3inst_cuda(packed2, m_pad, n_pad, allow_r1=True),
+               alpha=float(inv_rs2))
+    y_rht = torch.matmul(x_rht, W.t()).to(torch.float32).mul_(float(wscale))
+    glq_output_rht_blockdiag_cuda(y_rht, su, y, out_features, m_pad, blocks_m, bm_meta)
     return y
 
 
@@ -355,6 +385,17 @@ def _e8_args(qidxs, codebook, qidxs2, codebook2, inv_rs, qidxs3, inv_rs2, qidxs4
     return t1, q2, t2, n2, q3, q4
 
 
+def _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3):
+    lib = _lib.load()
+    M, nblk = qidxs.shape
+    W = torch.empty((M, nblk * 8), dtype=torch.float16, device=qidxs.device)
+    with torch.cuda.device(qidxs.device):
+        check(lib.glqh_e8_decompress(_p(qidxs), _p(q2), _p(q3), _p(q4), _p(t1), _p(t2), n2,
+                                     float(inv_rs), float(inv_rs2), float(inv_rs3), M, nblk * 8,
+                                     _p(W), _stream()))
+    return W
+
+
 def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=None,
                             inv_resid_scale=0.0, codebook_abs=None, qidxs3=None, codebook3=None,
                             inv_resid_scale2=0.0, qidxs4=None, codebook4=None, inv_resid_scale3=0.0):
@@ -367,6 +408,10 @@ def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=N
     M, nblk = qidxs.shape
     if x.shape[1] != nblk * 8:
         raise RuntimeError(f"x has {x.shape[1]} columns, qidxs implies {nblk * 8}")
+    if B > E8_BATCH_MAX:
+        W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_resid_scale, inv_resid_scale2,
+                             inv_resid_scale3)
+        return torch.matmul(x, W.t()).to(torch.float32).mul_(float(wscale))
     out = torch.empty((B, M), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         nb = lib.glqh_e8_matmul_workspace_bytes(M, nblk * 8, B)
@@ -400,6 +445,13 @@ def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_p
     bn, nbn = _host_i64(blocks_n)
     bm, nbm = _host_i64(blocks_m)
     y = torch.empty((B, int(out_features)), dtype=out_dtype or torch.float16, device=x.device)
+    if B > E8_BATCH_MAX:
+        x_rht = torch.empty((B, int(n_pad)), dtype=torch.float16, device=x.device)
+        glq_input_rht_blockdiag_cuda(x, sv, x_rht, in_features, n_pad, blocks_n, bn_meta)
+        W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
+        y_rht = torch.matmul(x_rht, W.t()).to(torch.float32).mul_(float(wscale))
+        glq_output_rht_blockdiag_cuda(y_rht, su, y, out_features, m_pad, blocks_m, bm_meta)
+        return y
     with torch.cuda.device(x.device):
         nb = lib.glqh_fused_linear_e8_workspace_bytes(B, int(n_pad), int(m_pad))
         ws = _ws(nb, x.device)

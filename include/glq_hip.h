@@ -157,6 +157,15 @@ int glqh_e8_dequant_matmul(const void *x_f16, int64_t B,
                            int64_t m_pad, int64_t n_pad,
                            float *out, void *ws, size_t ws_bytes, void *stream);
 
+/* Dense fp16 (m_pad, n_pad) RHT-domain weight before Wscale: cb[q1] + inv_rs*cb2[q2] + ...
+ * combined in fp32 and rounded once.  First half of the many-token path of
+ * glq_dequant_matmul_cuda (glq/csrc/glq_cuda.cu:1519-1637): dequantize once, then one
+ * library GEMM, as the reference's trellis prefill does (glq/csrc/glq_trellis.cu:1322-1334). */
+int glqh_e8_decompress(const void *q1, const void *q2, const void *q3, const void *q4,
+                       const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                       double inv_rs, double inv_rs2, double inv_rs3,
+                       int64_t m_pad, int64_t n_pad, void *out_f16, void *stream);
+
 size_t glqh_fused_linear_e8_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad);
 
 /* Whole E8 linear: input RHT -> gather-matmul -> output RHT.

@@ -1,0 +1,150 @@
+"""E8RHTLinear module, torch.ops.glq, dense many-token route and graph replay (MI355X)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glq_oracle as O
+from tests.gpu_util import DEV, e8_table_f16, rel, say, t
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.mark.parametrize("tag", ["k2", "k4", "k4k2"])
+def test_trellis_module_loads_reference_checkpoint(golden, tag):
+    from glq_amd.quantized_linear import E8RHTLinear
+    g = golden("trellis_layer")
+    say("module trellis", tag)
+    m, n = g[f"{tag}_W"].shape
+    keys = ["trellis_packed", "SU", "SV", "Wscale"] + (
+        ["trellis_packed2", "inv_resid_scale2"] if tag == "k4k2" else [])
+    sd = {k: torch.from_numpy(np.asarray(g[f"{tag}_{k}"])) for k in keys}
+    layer = E8RHTLinear(n, m, codebook_type="trellis")
+    layer.load_state_dict(sd)
+    layer.to(DEV)
+    x = torch.from_numpy(g[f"{tag}_x"])
+    for dtype in (torch.float16, torch.bfloat16):
+        y = layer(x.to(DEV, dtype))
+        assert y.dtype == dtype and y.shape == (x.shape[0], m)
+        assert rel(y, g[f"{tag}_y"]) < TOL
+    y3 = layer(x.to(DEV, torch.bfloat16).reshape(1, 5, n))
+    assert y3.shape == (1, 5, m)
+
+
+@pytest.mark.parametrize("tag,bpw,bd", [("bd2", 2, True), ("bd4", 4, True), ("p2", 2, False),
+                                        ("p4", 4, False)])
+def test_shell_module_loads_reference_checkpoint(golden, tag, bpw, bd):
+    from glq_amd.quantized_linear import E8RHTLinear
+    g = golden("e8_layer")
+    say("module shell", tag)
+    m, n = g[f"{tag}_W"].shape
+    keys = ["Qidxs", "SU", "SV", "Wscale"] + (["Qidxs2", "inv_resid_scale"] if bpw == 4 else [])
+    sd = {k: torch.from_numpy(np.asarray(g[f"{tag}_{k}"])) for k in keys}
+    layer = E8RHTLinear(n, m, block_diagonal=bd)
+    layer.load_state_dict(sd)
+    layer.to(DEV)
+    cb = e8_table_f16()
+    layer.set_codebook(cb, cb if bpw == 4 else None)
+    x = torch.from_numpy(g[f"{tag}_x"]).to(DEV, torch.bfloat16)
+    y = layer(x)
+    assert y.dtype == torch.bfloat16 and y.shape == (3, m)
+    assert rel(y, g[f"{tag}_y"]) < TOL
+    assert torch.equal(y, layer(x))
+
+
+def test_ops_namespace_runs_the_hip_path():
+    from glq_amd import custom_ops, hadamard as H
+    custom_ops.register()
+    m, n = 128, 256
+    p = t(O.random_packed(m, n, 4, 3))
+    su, sv = O.rht_signs(m, n, 7)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    x = torch.randn(2, n, device=DEV).half()
+    from glq_amd import ext
+    args = (x, t(sv.astype(np.float16)), t(su.astype(np.float16)), p, torch.tensor(bn), torch.tensor(bm),
+            H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), 0.02, n, m, n, m)
+    assert torch.equal(torch.ops.glq.fused_linear_trellis_3inst(*args),
+                       ext.glq_fused_linear_trellis_3inst_cuda(*args))
+
+
+@pytest.mark.parametrize("B", [65, 200])
+def test_trellis_dense_route_many_tokens(B):
+    from glq_amd import ext, hadamard as H
+    m, n = 256, 512
+    say("trellis dense", B)
+    p1, p2 = O.random_packed(m, n, 4, 1), O.random_packed(m, n, 2, 2)
+    su, sv = O.rht_signs(m, n, 42)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"trellis_packed": p1, "trellis_packed2": p2, "inv_resid_scale2": np.float32(0.3),
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
+           "blocks_m": bm, "blocks_n": bn}
+    x = torch.randn(B, n).to(torch.bfloat16)
+    ref = O.trellis_linear_forward(x.float().numpy(), art, n, m)
+    y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), t(p2), torch.tensor(bn), torch.tensor(bm),
+        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), 0.02, 0.3, n, m, n, m,
+        out_dtype=torch.bfloat16)
+    assert y.shape == (B, m) and rel(y, ref) < TOL
+    # rows agree with the compressed small-batch route
+    y8 = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+        x[:8].to(DEV), t(art["SV"]), t(art["SU"]), t(p1), t(p2), torch.tensor(bn), torch.tensor(bm),
+        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), 0.02, 0.3, n, m, n, m,
+        out_dtype=torch.bfloat16)
+    assert rel(y[:8], y8.float()) < 5e-3
+
+
+def test_e8_dense_route_many_tokens():
+    from glq_amd import ext, hadamard as H
+    m, n, B = 96, 160, 40
+    rng = np.random.default_rng(0)
+    q1 = rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16)
+    q2 = rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16)
+    su, sv = O.rht_signs(m, n, 42)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"Qidxs": q1, "Qidxs2": q2, "inv_resid_scale": np.float32(1 / 3.0), "SU": su.astype(np.float16),
+           "SV": sv.astype(np.float16), "Wscale": np.float32(0.02), "blocks_m": bm, "blocks_n": bn}
+    x = torch.randn(B, n).to(torch.float16)
+    ref = O.e8_linear_forward(x.float().numpy(), art, n, m)
+    cb = e8_table_f16()
+    y = ext.glq_fused_linear_block_diag_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(q1), cb, 0.02, n, m, n, m, torch.tensor(bn),
+        torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), t(q2), cb, 1 / 3.0)
+    assert rel(y, ref) < TOL
+    xr = torch.randn(B, n, device=DEV).half()
+    W = O.e8_dequant(q1, q2, 1 / 3.0)
+    out = ext.glq_dequant_matmul_cuda(xr, t(q1), cb, 0.5, t(q2), cb, 1 / 3.0)
+    assert rel(out, xr.float().cpu().numpy() @ W.T * 0.5) < 2e-3
+
+
+def test_graph_capture_and_replay_is_bit_exact():
+    """A decode step is replayed from a HIP graph: every replay, with eager work and
+    synchronisation in between, must equal the eager result bit for bit."""
+    from glq_amd.quantized_linear import E8RHTLinear
+    m, n = 512, 2048
+    layer = E8RHTLinear(n, m, codebook_type="trellis")
+    su, sv = O.rht_signs(m, n, 1)
+    layer.load_state_dict({"trellis_packed": torch.from_numpy(O.random_packed(m, n, 4, 9)),
+                           "SU": torch.from_numpy(su).half(), "SV": torch.from_numpy(sv).half(),
+                           "Wscale": torch.tensor(0.02)})
+    layer.to(DEV)
+    xs = torch.randn(1, n, device=DEV).to(torch.bfloat16)
+    eager = layer(xs).clone()
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            y = layer(xs)
+    torch.cuda.synchronize()
+    for i in range(4):
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), f"replay {i}"
+        other = layer(torch.randn(1, n, device=DEV).to(torch.bfloat16))      # eager work in between
+        torch.cuda.synchronize()
+        assert other.shape == (1, m)
+    xs.copy_(torch.randn(1, n, device=DEV).to(torch.bfloat16))               # new input, same graph
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, layer(xs))

@@ -1,0 +1,88 @@
+"""CPU-only: the torch.ops.glq schemas exist, their fakes agree with the schema arity and
+give the shapes/dtypes the call sites rely on (reference tests/test_glq_vllm.py:94-140)."""
+import inspect
+
+import pytest
+import torch
+
+from glq_amd import custom_ops
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _registered():
+    custom_ops.register()
+    custom_ops.register()            # idempotent
+
+
+def _n_schema_args(schema):
+    inside = schema[schema.index("(") + 1:schema.rindex(") ->")]
+    return len([a for a in inside.split(",") if a.strip()])
+
+
+def test_every_schema_has_fake_with_same_arity():
+    for name, schema in custom_ops.SCHEMAS.items():
+        assert hasattr(torch.ops.glq, name), name
+        fake = custom_ops.FAKES[name]
+        if fake is custom_ops._none_fake:
+            continue
+        assert len(inspect.signature(fake).parameters) == _n_schema_args(schema), name
+
+
+def test_fakes_on_meta_tensors():
+    m, n, B = 64, 128, 3
+    mt = lambda *s, dt=torch.float16: torch.empty(*s, dtype=dt, device="meta")  # noqa: E731
+    x = mt(B, n)
+    i64 = torch.empty(1, dtype=torch.int64, device="meta")
+    i32 = torch.empty(1, 4, dtype=torch.int32, device="meta")
+    packed = mt(32, 64, dt=torch.int16)
+    y = torch.ops.glq.fused_linear_trellis_3inst(x, mt(n), mt(m), packed, i64, i64, i32, i32, 0.02,
+                                                 n, m, n, m)
+    assert y.shape == (B, m) and y.dtype == torch.float16 and y.device.type == "meta"
+    y = torch.ops.glq.fused_linear_trellis_3inst_rvq2(mt(B, n, dt=torch.bfloat16), mt(n), mt(m), packed,
+                                                      packed, i64, i64, i32, i32, 0.02, 0.3, n, m, n, m)
+    assert y.shape == (B, m) and y.dtype == torch.bfloat16
+    q = mt(m, n // 8, dt=torch.int16)
+    cb = mt(65536, 8)
+    e = mt(0, dt=torch.int16)
+    ef = mt(0)
+    y = torch.ops.glq.fused_linear_block_diag(x, mt(n), mt(m), q, cb, 0.02, n, m, n, m, i64, i64, i32,
+                                              i32, e, ef, 0.0, e, ef, 0.0, e, ef, 0.0)
+    assert y.shape == (B, m) and y.dtype == torch.float16
+    y = torch.ops.glq.dequant_matmul(x, q, cb, 0.02, e, ef, 0.0, ef, e, ef, 0.0, e, ef, 0.0)
+    assert y.shape == (B, m) and y.dtype == torch.float32
+    yr = mt(B, 2 * m, dt=torch.float32)
+    assert torch.ops.glq.fused_linear_trellis_3inst_yrht(x, mt(n), packed, i64, i32, 0.02, n, n, m,
+                                                         yr, m) is None
+
+
+def test_module_buffers_match_the_checkpoint_contract():
+    from glq_amd.quantized_linear import E8RHTLinear
+    lin = E8RHTLinear(960, 960, block_diagonal=True)
+    sd = lin.state_dict()
+    assert sd["Qidxs"].shape == (960, 120) and sd["Qidxs"].dtype == torch.int16
+    assert sd["SU"].dtype == torch.float16 and sd["Wscale"].shape == ()
+    assert {"Qidxs2", "Qidxs3", "Qidxs4", "inv_resid_scale", "inv_resid_scale2",
+            "inv_resid_scale3", "SV"} <= set(sd)
+    assert lin.blocks_n == [512, 256, 128, 64]
+    legacy = E8RHTLinear(100, 48)
+    assert (legacy.m_pad, legacy.n_pad) == (64, 128) and not legacy.block_diagonal
+    tr = E8RHTLinear(2048, 11008, codebook_type="trellis")
+    assert tr.block_diagonal and tr.blocks_m == [8192, 2048, 512, 256]
+    assert tr.trellis_packed.numel() == 0 and tr.tlut.numel() == 0
+    # a single-stage trellis checkpoint loads without the optional keys
+    tr2 = E8RHTLinear(128, 64, codebook_type="trellis")
+    tr2.load_state_dict({"trellis_packed": torch.zeros(32, 64, dtype=torch.int16),
+                         "SU": torch.ones(64, dtype=torch.float16),
+                         "SV": torch.ones(128, dtype=torch.float16),
+                         "Wscale": torch.tensor(0.5)})
+    assert tr2.trellis_packed.shape == (32, 64) and tr2.trellis_packed2.numel() == 0
+    # a block-diagonal shell checkpoint re-shapes a module built with the legacy default
+    adapt = E8RHTLinear(160, 96)
+    adapt.load_state_dict({"Qidxs": torch.zeros(96, 20, dtype=torch.int16),
+                           "SU": torch.ones(96, dtype=torch.float16),
+                           "SV": torch.ones(160, dtype=torch.float16), "Wscale": torch.tensor(1.0)})
+    assert adapt.block_diagonal and adapt.blocks_n == [128, 32] and adapt.blocks_m == [64, 32]
+    with pytest.raises(RuntimeError, match="GPU only"):
+        tr2(torch.zeros(1, 128))
+    with pytest.raises(NotImplementedError):
+        E8RHTLinear(64, 64, codebook_type="e8p")

@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libglq_hip.so")
+# GLQ_HIP_LIB overrides the in-tree library (e.g. to try another build of the same ABI)
+LIB_PATH = os.environ.get("GLQ_HIP_LIB") or os.path.join(_HERE, "libglq_hip.so")
 
 _lib = None
 _load_error = None

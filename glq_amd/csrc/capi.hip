@@ -51,7 +51,7 @@ extern "C" int glqh_init(void) {
             return;
         }
         g_cus = prop.multiProcessorCount;
-        g_init_rc = glqh_rht_init() || glqh_e8_init();
+        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
     return g_init_rc;
@@ -190,6 +190,8 @@ extern "C" int glqh_output_rht_shards(const float *y_rht, const void *su_f16, vo
 // workspace layout: [x_rht f16 (B, n_pad)] [partials stage 1] [partials stage 2]
 static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
     int ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
+    int steps = 0, ks2 = 0;
+    if (glqh_trellis_fusein_plan(m_pad, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
     return align256((size_t)ks * B * m_pad * sizeof(float));
 }
 
@@ -234,12 +236,36 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     float *part1 = (float *)((char *)ws + xb);
     float *part2 = (float *)((char *)ws + xb + pb);
 
-    if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
-                              bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
-        return 1;
-    const int ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
-    if (glqh_launch_trellis_partial(x_rht, B, packed, R1, m_pad, n_pad, ks, part1, st)) return 1;
-    if (has_s2 && glqh_launch_trellis_partial(x_rht, B, packed2, R2, m_pad, n_pad, ks, part2, st)) return 1;
+    // Single-stage layers at up to four tokens fold the input transform into the GEMV;
+    // everything else transforms x once into scratch and reads it from every workgroup.
+    int ks = 0, fi_steps = 0;
+    const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
+    const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
+    if (!has_s2 && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
+        glqh_trellis_fusein_plan(m_pad, n_pad, B, &fi_steps, &ks)) {
+        if (n_blocks_n > 1) {
+            int64_t sum = 0;
+            for (int64_t i = 0; i < n_blocks_n; ++i) {
+                GLQH_REQUIRE(blocks_n[i] > 0 && (blocks_n[i] & (blocks_n[i] - 1)) == 0,
+                             "fused trellis linear: block size %lld is not a power of two",
+                             (long long)blocks_n[i]);
+                sum += blocks_n[i];
+            }
+            GLQH_REQUIRE(sum == n_pad, "fused trellis linear: block sizes sum to %lld, expected %lld",
+                         (long long)sum, (long long)n_pad);
+        }
+        GLQH_REQUIRE(in_features >= 1, "fused trellis linear: in_features must be positive");
+        if (glqh_launch_trellis_fusein(packed, R1, x, x_dtype, x_stride, sv_f16, B, m_pad, n_pad,
+                                       in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, part1, st))
+            return 1;
+    } else {
+        if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
+                                  bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
+            return 1;
+        ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
+        if (glqh_launch_trellis_partial(x_rht, B, packed, R1, m_pad, n_pad, ks, part1, st)) return 1;
+        if (has_s2 && glqh_launch_trellis_partial(x_rht, B, packed2, R2, m_pad, n_pad, ks, part2, st)) return 1;
+    }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);
     if (!y) {
@@ -251,8 +277,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     }
     glqh_ysrc src = {};
     src.nparts = has_s2 ? 2 : 1;
-    src.part[0] = part1;
-    src.part[1] = part2;
+    src.part = part1;
+    src.part_sstride = (int64_t)(pb / sizeof(float));
     src.part_kstride = B * m_pad;
     src.ksplit = ks;
     src.scale[0] = s1;
@@ -410,10 +436,9 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
         return 1;
     glqh_ysrc src = {};
     src.nparts = sg.n;
-    for (int s = 0; s < sg.n; ++s) {
-        src.part[s] = part + (int64_t)s * B * m_pad;
-        src.scale[s] = sg.scale[s];
-    }
+    for (int s = 0; s < sg.n; ++s) src.scale[s] = sg.scale[s];
+    src.part = part;
+    src.part_sstride = B * m_pad;
     src.part_kstride = (int64_t)sg.n * B * m_pad;
     src.ksplit = ks;
     return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,

@@ -57,12 +57,58 @@ __device__ __forceinline__ void store_act(void *p, int dtype, int64_t i, float v
     else ((float *)p)[i] = v;
 }
 
+// Block meta carried in the kernel arguments (no dependent global load at the start of a
+// latency-bound kernel).  When the block sizes are the descending power-of-two decomposition
+// of their total (what block_decompose yields), the total alone determines every row:
+// block j is the j-th set bit of `canon` from the top and its offset is the sum of the bits
+// above it.  canon == 0 means "read the device array".
+struct glqh_meta_args {
+    int canon;
+};
+
+__device__ __forceinline__ glqh_block_meta glqh_meta_row(const glqh_meta_args a,
+                                                         const glqh_block_meta *dev, int j) {
+    if (a.canon == 0) return dev[j];
+    uint32_t rem = (uint32_t)a.canon;
+    for (int i = 0; i < j; ++i) rem &= ~(0x80000000u >> __builtin_clz(rem));   // j is uniform
+    const int l = 31 - __builtin_clz(rem);
+    glqh_block_meta r;
+    r.offset = a.canon - (int)rem;
+    r.bs = 1 << l;
+    r.log_bs = l;
+    r.w = 0;
+    return r;
+}
+
+// canon from host block sizes; 0 when they are not the canonical decomposition
+inline int glqh_fill_meta_args(glqh_meta_args *out, const int64_t *blocks, int64_t n_blocks,
+                               int64_t single_size) {
+    out->canon = 0;
+    if (n_blocks <= 1) {
+        if (single_size <= 0 || single_size > 0x40000000ll || (single_size & (single_size - 1))) return 0;
+        out->canon = (int)single_size;
+        return 1;
+    }
+    if (!blocks) return 0;
+    int64_t sum = 0, prev = 0x7fffffffffffffffll;
+    for (int64_t i = 0; i < n_blocks; ++i) {
+        const int64_t b = blocks[i];
+        if (b <= 0 || (b & (b - 1)) || b >= prev) return 0;
+        prev = b;
+        sum += b;
+    }
+    if (sum > 0x7fffffffll) return 0;
+    out->canon = (int)sum;
+    return 1;
+}
+
 // internal kernels' host launchers (defined in fht.hip / trellis.hip / e8.hip)
 struct glqh_ysrc {                 // where the output RHT reads its RHT-domain input
     const float *direct;           // (B, stride) fp32, or NULL when partials are used
     int64_t stride;                // row stride of `direct`
-    const float *part[4];          // split-K partial sums per stage: element (k, b, row) at
-                                   // part[st][k * part_kstride + b * m_pad + row]
+    const float *part;             // split-K partial sums: element (stage, k, b, row) at
+                                   // part[stage * part_sstride + k * part_kstride + b * m_pad + row]
+    int64_t part_sstride;
     int64_t part_kstride;
     int ksplit;
     float scale[4];                // wscale per stage (already multiplied by inv_rs)
@@ -103,3 +149,13 @@ int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int
 int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,
                               const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
                               int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream);
+
+// fused-input trellis GEMV (B <= 4): plan returns 0 when the shape/batch is not eligible
+int glqh_trellis_fusein_plan(int64_t m, int64_t k, int64_t B, int *steps_out, int *ksplit_out);
+size_t glqh_trellis_fusein_lds(int steps, int NB);
+int glqh_launch_trellis_fusein(const void *packed, int R, const void *x, int x_dtype, int64_t x_stride,
+                               const void *sv, int64_t B, int64_t m, int64_t k, int64_t in_features,
+                               int steps, int ksplit, const glqh_block_meta *bn_meta,
+                               const int64_t *blocks_host, int n_blocks, float *part,
+                               hipStream_t stream);
+int glqh_trellis_init(void);

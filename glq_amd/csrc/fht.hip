@@ -4,203 +4,159 @@
 // multiplies once with 1/sqrt(bs) (glq/hadamard.py:10-28, glq/csrc/glq_fht.cuh:14-21,
 // glq/csrc/glq_cuda.cu:1756-1839, 2005-2079, 2092-2208).
 #include "common.h"
+#include "fht_device.h"
 
 namespace {
 
-constexpr int RHT_THREADS = 256;
+#ifndef GLQH_RHT_THREADS
+#define GLQH_RHT_THREADS 256
+#endif
+constexpr int RHT_THREADS = GLQH_RHT_THREADS;
 
-struct rht_block {
-    int off, bs, log_bs;
+struct rht_slice {
+    int off, bs, log_bs;     // the Hadamard block
+    int log_len, r, nsub;    // this workgroup's slice: len = 2^log_len, index r of nsub
     float norm;
+    bool live;
 };
 
-__device__ __forceinline__ rht_block rht_get_block(const glqh_block_meta *meta, glqh_block_meta single,
-                                                   float single_norm) {
-    glqh_block_meta mrow = meta ? meta[blockIdx.x] : single;
-    rht_block b;
+// blockIdx.x = block * spb + slice; workgroups past a block's slice count retire.
+__device__ __forceinline__ rht_slice rht_get_slice(const glqh_block_meta *meta, const glqh_meta_args margs,
+                                                   float single_norm, int spb) {
+    const int j = blockIdx.x / spb;
+    glqh_block_meta mrow = glqh_meta_row(margs, meta, j);
+    rht_slice b;
     b.off = mrow.offset;
     b.bs = mrow.bs;
     b.log_bs = mrow.log_bs;
+    b.log_len = min(mrow.log_bs, LOG_SLICE);
+    b.nsub = mrow.bs >> b.log_len;
+    b.r = blockIdx.x % spb;
+    b.live = b.r < b.nsub;
     if (mrow.w != 0) b.norm = __builtin_bit_cast(float, mrow.w);
-    else if (!meta && single_norm != 0.0f) b.norm = single_norm;
-    else  // 1/sqrt(2^L) exactly rounded: a power of two, times 1/sqrt(2) when L is odd
-        b.norm = ldexpf((mrow.log_bs & 1) ? 0.70710678118654752f : 1.0f, -(mrow.log_bs >> 1));
+    else if ((margs.canon & (margs.canon - 1)) == 0 && margs.canon != 0 && single_norm != 0.0f) b.norm = single_norm;
+    else b.norm = rsqrt_pow2(mrow.log_bs);
     return b;
 }
-
-// ---------------------------------------------------------------------------------
-// Block transform in a few register-radix passes.
-//
-// The log2(bs) index bits are split into fields of at most RMAX bits, taken from the top
-// bit down.  In one pass a thread owns groups of 2^r elements that differ only in the
-// field's bits, runs the field's r butterfly stages in registers and puts the group
-// back.  The first pass reads its elements through `load` (global memory: consecutive
-// lanes touch consecutive addresses), the last pass hands them to `store`; in between
-// the block lives in LDS with one pad word per 32 so that the strided accesses of the
-// low fields stay conflict-free.  A butterfly stage is (lo, hi) <- (a + b, a - b); the
-// stages of different bits commute, so the result is the Walsh-Hadamard transform of
-// the block (summation order differs from the ascending-distance order of
-// glq/hadamard.py:10-28 by fp32 rounding only).
-// ---------------------------------------------------------------------------------
-constexpr int RMAX = 5;
-
-__device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
-
-template <int R, bool FIRST, bool LAST, class Load, class Store>
-__device__ __forceinline__ void fht_pass(float *lds, int bs, int s, Load &load, Store &store) {
-    constexpr int N = 1 << R;
-    const int ngroups = bs >> R;
-    for (int g = threadIdx.x; g < ngroups; g += blockDim.x) {
-        const int lo = g & ((1 << s) - 1);
-        const int base = ((g >> s) << (s + R)) | lo;
-        float v[N];
-#pragma unroll
-        for (int j = 0; j < N; ++j) {                       // N independent loads in flight
-            const int idx = base + (j << s);
-            if constexpr (FIRST) v[j] = load(idx);
-            else v[j] = lds[lds_pad(idx)];
-        }
-#pragma unroll
-        for (int h = 1; h < N; h <<= 1) {
-#pragma unroll
-            for (int j = 0; j < N; ++j) {
-                if ((j & h) == 0) {
-                    const float a = v[j], b = v[j | h];
-                    v[j] = a + b;
-                    v[j | h] = a - b;
-                }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < N; ++j) {
-            const int idx = base + (j << s);
-            if constexpr (LAST) store(idx, v[j]);
-            else lds[lds_pad(idx)] = v[j];
-        }
-    }
-}
-
-template <bool FIRST, bool LAST, class Load, class Store>
-__device__ __forceinline__ void fht_pass_r(int r, float *lds, int bs, int s, Load &load, Store &store) {
-    switch (r) {
-    case 1: fht_pass<1, FIRST, LAST>(lds, bs, s, load, store); break;
-    case 2: fht_pass<2, FIRST, LAST>(lds, bs, s, load, store); break;
-    case 3: fht_pass<3, FIRST, LAST>(lds, bs, s, load, store); break;
-    case 4: fht_pass<4, FIRST, LAST>(lds, bs, s, load, store); break;
-    default: fht_pass<5, FIRST, LAST>(lds, bs, s, load, store); break;
-    }
-}
-
-// All threads of the workgroup must call it.  lds needs bs + bs/32 floats.  With
-// STAGED the block is already in LDS (padded layout) and `load` is not used.
-template <bool STAGED, class Load, class Store>
-__device__ __forceinline__ void fht_block(float *lds, int log_bs, Load load, Store store) {
-    const int bs = 1 << log_bs;
-    if (log_bs == 0) {
-        if (threadIdx.x == 0) store(0, STAGED ? lds[0] : load(0));
-        return;
-    }
-    const int npass = (log_bs + RMAX - 1) / RMAX;
-    int s = log_bs;
-    for (int p = 0; p < npass; ++p) {
-        const int left = npass - p;
-        const int r = (s + left - 1) / left;              // balanced field widths
-        s -= r;
-        const bool first = p == 0 && !STAGED, last = p == npass - 1;
-        if (first && last) fht_pass_r<true, true>(r, lds, bs, s, load, store);
-        else if (first) fht_pass_r<true, false>(r, lds, bs, s, load, store);
-        else if (last) fht_pass_r<false, true>(r, lds, bs, s, load, store);
-        else fht_pass_r<false, false>(r, lds, bs, s, load, store);
-        if (!last) __syncthreads();
-    }
-}
-
-template <typename T> __device__ __forceinline__ float act_to_f32(T v);
-template <> __device__ __forceinline__ float act_to_f32<f16>(f16 v) { return (float)v; }
-template <> __device__ __forceinline__ float act_to_f32<uint16_t>(uint16_t v) { return bf16_bits_to_f32(v); }
-template <> __device__ __forceinline__ float act_to_f32<float>(float v) { return v; }
-template <typename T> __device__ __forceinline__ T f32_to_act(float v);
-template <> __device__ __forceinline__ f16 f32_to_act<f16>(float v) { return (f16)v; }
-template <> __device__ __forceinline__ uint16_t f32_to_act<uint16_t>(float v) { return f32_to_bf16_bits(v); }
-template <> __device__ __forceinline__ float f32_to_act<float>(float v) { return v; }
 
 // XT / OT: element types (bf16 travels as uint16_t)
 template <typename XT, typename OT>
 __global__ void __launch_bounds__(RHT_THREADS)
 input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
                  OT *__restrict__ out, int in_features, int n_pad,
-                 const glqh_block_meta *__restrict__ meta, glqh_block_meta single,
-                 float single_norm) {
-    extern __shared__ float s[];
-    const rht_block blk = rht_get_block(meta, single, single_norm);
+                 const glqh_block_meta *__restrict__ meta, glqh_meta_args margs,
+                 float single_norm, int spb) {
+    __shared__ float s[SLICE_LDS_FLOATS];
+    const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb);
+    if (!blk.live) return;
     const XT *xr = x + (int64_t)blockIdx.y * x_stride;
-    OT *orow = out + (int64_t)blockIdx.y * n_pad + blk.off;
-    auto load = [&](int i) -> float {
-        const int col = blk.off + i;
-        return col < in_features ? act_to_f32<XT>(xr[col]) * (float)sv[col] : 0.0f;
-    };
-    auto store = [&](int i, float v) { orow[i] = f32_to_act<OT>(v * blk.norm); };
-    fht_block<false>(s, blk.log_bs, load, store);
+    stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, [&](int h, int i) -> float {
+        const int col = blk.off + (h << blk.log_len) + i;
+        const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
+        return col < in_features ? v : 0.0f;
+    });
+    struct {
+        OT *orow;
+        float norm;
+        __device__ float aux(int) const { return norm; }
+        __device__ void put(int i, float v, float f) const { orow[i] = f32_to_act<OT>(v * f); }
+    } store = {out + (int64_t)blockIdx.y * n_pad + blk.off + (blk.r << blk.log_len), blk.norm};
+    fht_staged(s, blk.log_len, store);
 }
 
 template <typename YT, bool PARTS>
 __global__ void __launch_bounds__(RHT_THREADS)
 output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
                   int out_features, int m_pad, const glqh_block_meta *__restrict__ meta,
-                  glqh_block_meta single, float single_norm) {
-    extern __shared__ float s[];
-    const rht_block blk = rht_get_block(meta, single, single_norm);
+                  glqh_meta_args margs, float single_norm, int spb) {
+    __shared__ float s[SLICE_LDS_FLOATS];
+    const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb);
+    if (!blk.live) return;
     const int64_t b = blockIdx.y;
-    YT *yrow = y + b * y_stride;
-    auto store = [&](int i, float v) {
-        const int row = blk.off + i;
-        if (row < out_features) yrow[row] = f32_to_act<YT>(v * blk.norm * (float)su[row]);
-    };
     if constexpr (!PARTS) {
         const float *__restrict__ d = src.direct + b * src.stride + blk.off;
-        auto load = [&](int i) -> float { return d[i]; };
-        fht_block<false>(s, blk.log_bs, load, store);
+        stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r,
+                                         [&](int h, int i) -> float { return d[(h << blk.log_len) + i]; });
     } else {
-        // Stage the block into LDS while summing the split-K partials of each stage in a
-        // fixed order (deterministic).  Eight rows per thread are in flight at once.
-        constexpr int U = 8;
-        const int bs = blk.bs;
-        for (int i0 = threadIdx.x; i0 < bs; i0 += U * RHT_THREADS) {
-            float tot[U];
+        // Element e of the block is v(e) = sum_stage scale * (sum_k partial), summed in this
+        // fixed order (the same order as the stand-alone reduction, so both give the same
+        // bits); slice r needs sum_h sign(r,h) v(h*len + i).  The (h, stage, k) terms are
+        // walked as one flat sequence so that 8 terms x 4 elements of loads are in flight.
+        constexpr int U = 4, C = 8;
+        const int len = 1 << blk.log_len;
+        const int ks = src.ksplit, nst = src.nparts;
+        const int total = blk.nsub * nst * ks;
+        const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
+        for (int i0 = threadIdx.x; i0 < len; i0 += U * RHT_THREADS) {
+            float z[U], v[U], acc[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) tot[u] = 0.0f;
-            for (int st = 0; st < src.nparts; ++st) {
-                const float *__restrict__ p = src.part[st] + b * (int64_t)m_pad + blk.off;
-                float acc[U];
+            for (int u = 0; u < U; ++u) z[u] = v[u] = acc[u] = 0.0f;
+            int h = 0, st = 0, k = 0;                       // position of term t0 (uniform)
+            for (int t0 = 0; t0 < total; t0 += C) {
+                float vals[C][U];
+                int hh = h, ss = st, kk = k;
 #pragma unroll
-                for (int u = 0; u < U; ++u) acc[u] = 0.0f;
-#pragma unroll 4
-                for (int k = 0; k < src.ksplit; ++k) {
+                for (int c = 0; c < C; ++c) {
+                    const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        const int i = i0 + u * RHT_THREADS;
-                        acc[u] += i < bs ? p[(int64_t)k * src.part_kstride + i] : 0.0f;
+                    for (int u = 0; u < U; ++u) vals[c][u] = p[min(i0 + u * RHT_THREADS, len - 1)];
+                    if (t0 + c + 1 < total) {               // advance, clamped at the last term
+                        if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
                     }
                 }
 #pragma unroll
-                for (int u = 0; u < U; ++u) tot[u] += src.scale[st] * acc[u];
-            }
+                for (int c = 0; c < C; ++c) {
+                    if (t0 + c < total) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int i = i0 + u * RHT_THREADS;
-                if (i < bs) {
-                    s[lds_pad(i)] = tot[u];
-                    if (src.copy_out) src.copy_out[b * src.copy_stride + blk.off + i] = tot[u];
+                        for (int u = 0; u < U; ++u) acc[u] += vals[c][u];
+                        if (++k == ks) {
+                            const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
+                                           : st == 2 ? src.scale[2] : src.scale[3];
+#pragma unroll
+                            for (int u = 0; u < U; ++u) { v[u] += sc * acc[u]; acc[u] = 0.0f; }
+                            k = 0;
+                            if (++st == nst) {
+#pragma unroll
+                                for (int u = 0; u < U; ++u) {
+                                    const int i = i0 + u * RHT_THREADS;
+                                    if (src.copy_out && blk.r == 0 && i < len)
+                                        src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i] = v[u];
+                                    z[u] += had_sign(blk.r, h, v[u]);
+                                    v[u] = 0.0f;
+                                }
+                                st = 0;
+                                ++h;
+                            }
+                        }
+                    }
                 }
             }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (i0 + u * RHT_THREADS < len) s[lds_pad(i0 + u * RHT_THREADS)] = z[u];
         }
         __syncthreads();
-        auto load = [&](int i) -> float { return 0.0f; };
-        fht_block<true>(s, blk.log_bs, load, store);
     }
+    const int base = blk.off + (blk.r << blk.log_len);
+    struct {
+        YT *yrow;
+        const f16 *su;
+        int base, out_features;
+        float norm;
+        // su has m_pad entries, so the load is always in bounds
+        __device__ float aux(int i) const { return norm * (float)su[base + i]; }
+        __device__ void put(int i, float v, float f) const {
+            const int row = base + i;
+            if (row < out_features) yrow[row] = f32_to_act<YT>(v * f);
+        }
+    } store = {y + b * y_stride, su, base, out_features, blk.norm};
+    fht_staged(s, blk.log_len, store);
 }
 
-size_t rht_lds_bytes(int64_t max_bs) { return (size_t)(max_bs + max_bs / 32 + 32) * sizeof(float); }
+int rht_slices_per_block(int64_t max_bs) {
+    int64_t spb = max_bs >> LOG_SLICE;
+    return spb < 1 ? 1 : (int)spb;
+}
 
 int check_blocks(const int64_t *blocks_host, int64_t n_blocks, int64_t total, int64_t *max_bs,
                  const char *what) {
@@ -239,7 +195,7 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
                  "input_rht: bad x dtype");
     GLQH_REQUIRE(out_dtype == GLQH_F32 || out_dtype == GLQH_F16, "input_rht: out must be f32 or f16");
     int64_t max_bs = n_pad;
-    glqh_block_meta single = {0, (int32_t)n_pad, ilog2(n_pad), 0};
+    glqh_meta_args margs;
     if (n_blocks > 1) {
         GLQH_REQUIRE(meta_dev && blocks_host, "input_rht: block-diagonal call needs meta and sizes");
         if (check_blocks(blocks_host, n_blocks, n_pad, &max_bs, "input_rht")) return 1;
@@ -249,13 +205,15 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
         meta_dev = nullptr;
         n_blocks = 1;
     }
-    GLQH_REQUIRE(rht_lds_bytes(max_bs) <= GLQH_MAX_LDS_BYTES, "input_rht: block of %lld exceeds LDS", (long long)max_bs);
-    dim3 grid((unsigned)n_blocks, (unsigned)B);
-    const size_t lds = rht_lds_bytes(max_bs);
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, n_pad))
+        margs.canon = 0;                               // not canonical: kernel reads meta_dev
+    const int spb = rht_slices_per_block(max_bs);
+    GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "input_rht: too many slices");
+    dim3 grid((unsigned)(n_blocks * spb), (unsigned)B);
 #define GLQH_IN_LAUNCH(XT, OT)                                                                      \
-    hipLaunchKernelGGL((input_rht_kernel<XT, OT>), grid, dim3(RHT_THREADS), lds, stream,            \
+    hipLaunchKernelGGL((input_rht_kernel<XT, OT>), grid, dim3(RHT_THREADS), 0, stream,              \
                        (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
-                       (int)n_pad, meta_dev, single, rsqrt_n)
+                       (int)n_pad, meta_dev, margs, rsqrt_n, spb)
     if (out_dtype == GLQH_F32) {
         if (x_dtype == GLQH_F16) GLQH_IN_LAUNCH(f16, float);
         else if (x_dtype == GLQH_BF16) GLQH_IN_LAUNCH(uint16_t, float);
@@ -283,7 +241,7 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
     GLQH_REQUIRE(y_dtype == GLQH_F16 || y_dtype == GLQH_BF16 || y_dtype == GLQH_F32,
                  "output_rht: bad y dtype");
     int64_t max_bs = m_pad;
-    glqh_block_meta single = {0, (int32_t)m_pad, ilog2(m_pad), 0};
+    glqh_meta_args margs;
     if (n_blocks > 1 || (meta_dev && !blocks_host)) {
         GLQH_REQUIRE(meta_dev, "output_rht: block-diagonal call needs meta");
         if (blocks_host) {
@@ -299,13 +257,15 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
         meta_dev = nullptr;
         n_blocks = 1;
     }
-    GLQH_REQUIRE(rht_lds_bytes(max_bs) <= GLQH_MAX_LDS_BYTES, "output_rht: block of %lld exceeds LDS", (long long)max_bs);
-    dim3 grid((unsigned)n_blocks, (unsigned)B);
-    const size_t lds = rht_lds_bytes(max_bs);
+    if (meta_dev && !blocks_host) margs.canon = 0;         // shard-batched call: device meta only
+    else if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, m_pad)) margs.canon = 0;
+    const int spb = rht_slices_per_block(max_bs);
+    GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "output_rht: too many slices");
+    dim3 grid((unsigned)(n_blocks * spb), (unsigned)B);
 #define GLQH_OUT_LAUNCH(YT, PARTS)                                                                  \
-    hipLaunchKernelGGL((output_rht_kernel<YT, PARTS>), grid, dim3(RHT_THREADS), lds, stream, src,   \
+    hipLaunchKernelGGL((output_rht_kernel<YT, PARTS>), grid, dim3(RHT_THREADS), 0, stream, src,     \
                        (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, meta_dev, \
-                       single, rsqrt_m)
+                       margs, rsqrt_m, spb)
     if (src.nparts == 0) {
         if (y_dtype == GLQH_F16) GLQH_OUT_LAUNCH(f16, false);
         else if (y_dtype == GLQH_BF16) GLQH_OUT_LAUNCH(uint16_t, false);
@@ -320,24 +280,4 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
     return 0;
 }
 
-template <typename K>
-static int set_max_lds(K kernel, const char *what) {
-    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel,
-                                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              GLQH_MAX_LDS_BYTES), what);
-}
-
-int glqh_rht_init(void) {
-    return set_max_lds(input_rht_kernel<f16, float>, "input_rht attribute") ||
-           set_max_lds(input_rht_kernel<uint16_t, float>, "input_rht attribute") ||
-           set_max_lds(input_rht_kernel<float, float>, "input_rht attribute") ||
-           set_max_lds(input_rht_kernel<f16, f16>, "input_rht attribute") ||
-           set_max_lds(input_rht_kernel<uint16_t, f16>, "input_rht attribute") ||
-           set_max_lds(input_rht_kernel<float, f16>, "input_rht attribute") ||
-           set_max_lds(output_rht_kernel<f16, false>, "output_rht attribute") ||
-           set_max_lds(output_rht_kernel<uint16_t, false>, "output_rht attribute") ||
-           set_max_lds(output_rht_kernel<float, false>, "output_rht attribute") ||
-           set_max_lds(output_rht_kernel<f16, true>, "output_rht attribute") ||
-           set_max_lds(output_rht_kernel<uint16_t, true>, "output_rht attribute") ||
-           set_max_lds(output_rht_kernel<float, true>, "output_rht attribute");
-}
+int glqh_rht_init(void) { return 0; }

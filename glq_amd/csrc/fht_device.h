@@ -1,0 +1,162 @@
+// Device-side Walsh-Hadamard transform of a block staged in LDS, shared by the RHT
+// kernels and by the fused input transform of the trellis GEMV.
+#pragma once
+
+#include "common.h"
+
+// ---------------------------------------------------------------------------------
+// The log2(n) index bits are split into fields of at most RMAX bits, taken from the top
+// bit down.  In one pass a thread owns groups of 2^r elements that differ only in the
+// field's bits, runs the field's r butterfly stages (lo, hi) <- (a + b, a - b) in
+// registers and puts the group back; the last pass hands the elements to `store`.  The
+// block lives in LDS with one pad word per 32 so that the strided accesses of the low
+// fields stay conflict-free.  The stages of different bits commute, so the result is the
+// Walsh-Hadamard transform of the block (summation order differs from the
+// ascending-distance order of glq/hadamard.py:10-28 by fp32 rounding only).
+//
+// Blocks larger than a slice (GLQH_LOG_SLICE) are never transformed whole: H_bs factors
+// as H_(bs/len) (x) H_len, so slice r of the output is
+//     H_len( sum_h (-1)^popcount(r & h) * in[h*len + i] ),
+// one pass over the block's inputs followed by a short transform -- which lets every slice
+// go to its own workgroup.
+//
+// `store` is an object with aux(i) -> float (a per-element factor that may come from
+// memory; all of a group's factors are requested before the butterflies) and
+// put(i, value, factor).  RMAX is kept small on purpose: a pass is straight-line code that
+// runs once per launch, and instruction fetch of a 32-point pass costs more than the extra
+// barrier of two 8-point passes.
+// ---------------------------------------------------------------------------------
+#ifndef GLQH_RMAX
+#define GLQH_RMAX 4
+#endif
+#ifndef GLQH_LOG_SLICE
+#define GLQH_LOG_SLICE 10
+#endif
+constexpr int RMAX = GLQH_RMAX;
+constexpr int LOG_SLICE = GLQH_LOG_SLICE;
+constexpr int SLICE_LDS_FLOATS = (1 << LOG_SLICE) + (1 << LOG_SLICE) / 32 + 32;
+
+__device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
+
+template <int R, bool LAST, class Store>
+__device__ __forceinline__ void fht_pass(float *lds, int n, int s, Store &store) {
+    constexpr int N = 1 << R;
+    const int ngroups = n >> R;
+    for (int g = threadIdx.x; g < ngroups; g += blockDim.x) {
+        const int lo = g & ((1 << s) - 1);
+        const int base = ((g >> s) << (s + R)) | lo;
+        float v[N], aux[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = base + (j << s);
+            v[j] = lds[lds_pad(idx)];
+            if constexpr (LAST) aux[j] = store.aux(idx);
+        }
+#pragma unroll
+        for (int h = 1; h < N; h <<= 1) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                if ((j & h) == 0) {
+                    const float a = v[j], b = v[j | h];
+                    v[j] = a + b;
+                    v[j | h] = a - b;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int idx = base + (j << s);
+            if constexpr (LAST) store.put(idx, v[j], aux[j]);
+            else lds[lds_pad(idx)] = v[j];
+        }
+    }
+}
+
+template <bool LAST, class Store>
+__device__ __forceinline__ void fht_pass_r(int r, float *lds, int n, int s, Store &store) {
+    switch (r) {
+    case 1: fht_pass<1, LAST>(lds, n, s, store); break;
+    case 2: fht_pass<2, LAST>(lds, n, s, store); break;
+    case 3: fht_pass<3, LAST>(lds, n, s, store); break;
+#if GLQH_RMAX >= 5
+    case 4: fht_pass<4, LAST>(lds, n, s, store); break;
+    default: fht_pass<5, LAST>(lds, n, s, store); break;
+#else
+    default: fht_pass<4, LAST>(lds, n, s, store); break;
+#endif
+    }
+}
+
+// Transform lds[0 .. 2^log_n) (padded layout, already staged and visible to the whole
+// workgroup) and pass the result to `store`.  All threads of the workgroup must call it.
+template <class Store>
+__device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store) {
+    const int n = 1 << log_n;
+    if (log_n == 0) {
+        if (threadIdx.x == 0) store.put(0, lds[0], store.aux(0));
+        return;
+    }
+    const int npass = (log_n + RMAX - 1) / RMAX;
+    int s = log_n;
+    for (int p = 0; p < npass; ++p) {
+        const int left = npass - p;
+        const int r = (s + left - 1) / left;              // balanced field widths
+        s -= r;
+        if (p == npass - 1) fht_pass_r<true>(r, lds, n, s, store);
+        else {
+            fht_pass_r<false>(r, lds, n, s, store);
+            __syncthreads();
+        }
+    }
+}
+
+// sign of element (r, h) of the Sylvester matrix
+__device__ __forceinline__ float had_sign(int r, int h, float v) {
+    return (__builtin_popcount(r & h) & 1) ? -v : v;
+}
+
+// lds[pad(i)] = sum_h sign(r, h) * val(h, i) for i < 2^log_len: slice r of the first
+// factor of H_(nsub*len).  Loads of 8 terms x 4 elements are issued before any of them is
+// used; indices are clamped instead of branched on so that the loads cluster.  Ends with
+// a barrier.
+template <int T, class Val>
+__device__ __forceinline__ void stage_signed_slices(float *lds, int log_len, int nsub, int r, Val val) {
+    constexpr int U = 4, C = 8;
+    const int len = 1 << log_len;
+    for (int i0 = threadIdx.x; i0 < len; i0 += U * T) {
+        float z[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) z[u] = 0.0f;
+        for (int h0 = 0; h0 < nsub; h0 += C) {
+            float vals[C][U];
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    vals[c][u] = val(min(h0 + c, nsub - 1), min(i0 + u * T, len - 1));
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    z[u] += (h0 + c < nsub) ? had_sign(r, h0 + c, vals[c][u]) : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (i0 + u * T < len) lds[lds_pad(i0 + u * T)] = z[u];
+    }
+    __syncthreads();
+}
+
+template <typename T> __device__ __forceinline__ float act_to_f32(T v);
+template <> __device__ __forceinline__ float act_to_f32<f16>(f16 v) { return (float)v; }
+template <> __device__ __forceinline__ float act_to_f32<uint16_t>(uint16_t v) { return bf16_bits_to_f32(v); }
+template <> __device__ __forceinline__ float act_to_f32<float>(float v) { return v; }
+template <typename T> __device__ __forceinline__ T f32_to_act(float v);
+template <> __device__ __forceinline__ f16 f32_to_act<f16>(float v) { return (f16)v; }
+template <> __device__ __forceinline__ uint16_t f32_to_act<uint16_t>(float v) { return f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ float f32_to_act<float>(float v) { return v; }
+
+// 1/sqrt(2^L) exactly rounded: a power of two, times 1/sqrt(2) when L is odd.
+__device__ __forceinline__ float rsqrt_pow2(int log_bs) {
+    return ldexpf((log_bs & 1) ? 0.70710678118654752f : 1.0f, -(log_bs >> 1));
+}

@@ -21,11 +21,13 @@
 // activations with fp32 accumulation.  Every output row is owned by one workgroup per
 // K-split slot and summed in a fixed order, so results are bit-identical run to run.
 #include "common.h"
+#include "fht_device.h"
 
 namespace {
 
 constexpr int TR_WAVES = 4;
 constexpr int TR_THREADS = TR_WAVES * GLQH_WAVE;
+constexpr int TR_PRE = 4;      // records a wave keeps in flight in the fused-input GEMV
 
 // (s * 89226354 + 64248484) mod 2^32, masked and xored: the two fp16 halves of 3INST.
 __device__ __forceinline__ uint32_t tr_hash(uint32_t s) {
@@ -143,6 +145,74 @@ tr_decompress_kernel(const uint8_t *__restrict__ packed, f16 *__restrict__ W, in
     }
 }
 
+// Decode the 32 weights of one record and accumulate them against the lane's activations.
+// xa[t][ks] = (x[2b], x[2b+1]) and xb[t][ks] = (x[2b+8], x[2b+9]) of k-tile ks, token t;
+// acc[t][ms*2 + rh] is the fp32 sum of row 16*ms + 8*rh + a.
+template <int NB>
+struct tr_xfrag {
+    uint32_t a[NB][2], b[NB][2];
+};
+
+template <int NB>
+struct tr_acc {
+    float v[NB][4];
+};
+
+template <int R, int NB>
+__device__ __forceinline__ tr_acc<NB> tr_accumulate(const tr_record<R> r, int lane, const tr_xfrag<NB> xf,
+                                                    tr_acc<NB> acc) {
+    uint32_t cont[4];
+    tr_continuation<R>(r, lane, cont);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) {
+            const int ci = ks * 2 + ms;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                // both fp16 halves of the state multiply the same activation
+                f16x2 w = __builtin_bit_cast(f16x2, tr_hash(tr_state<R>(r.c[ci], cont[ci], j)));
+                const int rh = (j >> 1) & 1;
+#pragma unroll
+                for (int t = 0; t < NB; ++t) {
+                    const uint32_t xw = (j >> 2) ? xf.b[t][ks] : xf.a[t][ks];
+                    // splat the selected half: (lo,lo) or (hi,hi)
+                    const uint32_t sp = (j & 1) ? __builtin_amdgcn_perm(xw, xw, 0x07060706u)
+                                                : __builtin_amdgcn_perm(xw, xw, 0x05040504u);
+                    acc.v[t][ms * 2 + rh] = __builtin_amdgcn_fdot2(w, __builtin_bit_cast(f16x2, sp),
+                                                                   acc.v[t][ms * 2 + rh], false);
+                }
+            }
+        }
+    }
+    return acc;
+}
+
+// Workgroup reduction shared by the GEMV kernels: lanes -> waves -> 32 rows per token.
+// Returns through `red` (LDS, [TR_WAVES][NB][32]); ends with a barrier.
+template <int NB>
+__device__ __forceinline__ void tr_reduce_to_lds(tr_acc<NB> acc, float (*red)[NB][32], int lane,
+                                                 int wave) {
+    const int l = lane & 31, a = l >> 2, b = l & 3, hf = lane >> 5;
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = acc.v[t][i];
+            v += __shfl_xor(v, 1, GLQH_WAVE);
+            v += __shfl_xor(v, 2, GLQH_WAVE);
+            v += __shfl_xor(v, 32, GLQH_WAVE);
+            acc.v[t][i] = v;
+        }
+    if (hf == 0 && b == 0) {
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][t][(i >> 1) * 16 + (i & 1) * 8 + a] = acc.v[t][i];
+    }
+    __syncthreads();
+}
+
 // ---------------------------------------------------------------------------------
 // GEMV / small-batch GEMM against the packed stream
 // ---------------------------------------------------------------------------------
@@ -158,24 +228,20 @@ tr_gemv_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, in
     const int wave = threadIdx.x >> 6;
     const int l = lane & 31;
     const int hf = lane >> 5;
-    const int a = l >> 2, b = l & 3;
+    const int b = l & 3;
     const int mp = blockIdx.x;
     const int nsteps = k >> 6;
     const int stride = gridDim.y * TR_WAVES;
     const int tok0 = blockIdx.z * NB;
 
-    float acc[NB][4];
-#pragma unroll
-    for (int t = 0; t < NB; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[t][i] = 0.0f;
+    tr_acc<NB> acc = {};
 
     const uint8_t *row_base = packed + (int64_t)mp * (k >> 5) * 32 * (4 * R);
     for (int q = blockIdx.y * TR_WAVES + wave; q < nsteps; q += stride) {
         const int kp = 2 * q + hf;
         tr_record<R> r = tr_load_record<R>(row_base + ((int64_t)kp * 32 + l) * (4 * R));
         // activations of this lane's four columns in each of the two k-tiles
-        uint32_t xa[NB][2], xb[NB][2];
+        tr_xfrag<NB> xf;
 #pragma unroll
         for (int t = 0; t < NB; ++t) {
             const int tok = tok0 + t;
@@ -184,52 +250,14 @@ tr_gemv_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, in
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 uint32_t va = xp[8 * ks], vb = xp[8 * ks + 4];
-                xa[t][ks] = live ? va : 0u;
-                xb[t][ks] = live ? vb : 0u;
+                xf.a[t][ks] = live ? va : 0u;
+                xf.b[t][ks] = live ? vb : 0u;
             }
         }
-        uint32_t cont[4];
-        tr_continuation<R>(r, lane, cont);
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int ms = 0; ms < 2; ++ms) {
-                const int ci = ks * 2 + ms;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    // both fp16 halves of the state multiply the same activation
-                    f16x2 w = __builtin_bit_cast(f16x2, tr_hash(tr_state<R>(r.c[ci], cont[ci], j)));
-                    const int rh = (j >> 1) & 1;
-#pragma unroll
-                    for (int t = 0; t < NB; ++t) {
-                        f16x2 xp2 = __builtin_bit_cast(f16x2, (j >> 2) ? xb[t][ks] : xa[t][ks]);
-                        f16 xe = (j & 1) ? xp2.y : xp2.x;
-                        f16x2 xx = {xe, xe};
-                        acc[t][ms * 2 + rh] = __builtin_amdgcn_fdot2(w, xx, acc[t][ms * 2 + rh], false);
-                    }
-                }
-            }
-        }
+        acc = tr_accumulate<R, NB>(r, lane, xf, acc);
     }
 
-    // sum over the four column groups (lane bits 0,1) and the two halves (bit 5)
-#pragma unroll
-    for (int t = 0; t < NB; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float v = acc[t][i];
-            v += __shfl_xor(v, 1, GLQH_WAVE);
-            v += __shfl_xor(v, 2, GLQH_WAVE);
-            v += __shfl_xor(v, 32, GLQH_WAVE);
-            acc[t][i] = v;
-        }
-    if (hf == 0 && b == 0) {
-#pragma unroll
-        for (int t = 0; t < NB; ++t)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) red[wave][t][(i >> 1) * 16 + (i & 1) * 8 + a] = acc[t][i];
-    }
-    __syncthreads();
+    tr_reduce_to_lds<NB>(acc, red, lane, wave);
     for (int idx = threadIdx.x; idx < NB * 32; idx += TR_THREADS) {
         const int t = idx >> 5, row = idx & 31;
         const int tok = tok0 + t;
@@ -243,6 +271,128 @@ tr_gemv_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, in
         } else {
             part[((int64_t)blockIdx.y * B + tok) * m + 32 * mp + row] = v;
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// GEMV with the input transform folded in (B <= NB tokens).
+//
+// grid = (m/32, ksplit).  K slot s owns the `steps` consecutive wave-steps starting at
+// s*steps, i.e. the Ls = 64*steps columns [s*Ls, (s+1)*Ls) of the transformed activations
+// (Ls a power of two).  A Hadamard block of size bs >= Ls that contains the slice factors as
+// H_bs = H_(bs/Ls) (x) H_Ls, so the slice r of its output is
+//     H_Ls( sum_h (-1)^popcount(r & h) * xs[h*Ls + j] ) / sqrt(bs),   xs = sv * x,
+// which costs one pass over the block's inputs (they sit in L2) and a short transform;
+// blocks smaller than the slice are transformed whole.  The slice is kept in LDS as fp16
+// and feeds the decode loop.  The first record of every wave is requested before the
+// prologue so that the HBM latency overlaps it.
+// ---------------------------------------------------------------------------------
+template <int R, typename XT, int NB>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_gemv_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
+                      const f16 *__restrict__ sv, int B, int m, int k, int in_features, int steps,
+                      const glqh_block_meta *__restrict__ bn_meta, int n_blocks,
+                      glqh_meta_args margs, float *__restrict__ part) {
+    extern __shared__ float smem[];
+    __shared__ float red[TR_WAVES][NB][32];
+    const int Ls = steps << 6;
+    float *fbuf = smem;                                         // Ls + Ls/32 floats
+    f16 *xh = (f16 *)(smem + Ls + (Ls >> 5) + 32);              // [NB][Ls] fp16
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int l = lane & 31;
+    const int hf = lane >> 5;
+    const int b = l & 3;
+    const int mp = blockIdx.x;
+    const int slot = blockIdx.y;
+    const int nsteps = k >> 6;
+    const int q0 = slot * steps;
+    const int q1 = min(q0 + steps, nsteps);
+    const int c0 = q0 << 6;
+
+    // Request this wave's first TR_PRE records now: the packed stream arrives from HBM while
+    // the prologue below runs.
+    const uint8_t *row_base = packed + (int64_t)mp * (k >> 5) * 32 * (4 * R);
+    const uint8_t *lane_base = row_base + ((int64_t)hf * 32 + l) * (4 * R);   // + q * 64 * 4R
+    constexpr int64_t STEP_BYTES = 64 * 4 * R;
+    int q = q0 + wave;
+    tr_record<R> cur[TR_PRE];
+#pragma unroll
+    for (int i = 0; i < TR_PRE; ++i) {
+        cur[i] = tr_record<R>{};
+        if (q + i * TR_WAVES < q1) cur[i] = tr_load_record<R>(lane_base + (q + i * TR_WAVES) * STEP_BYTES);
+    }
+
+    // ---- prologue: transformed activations of this slot's columns -> xh ----
+    for (int jb = 0; jb < n_blocks; ++jb) {
+        const glqh_block_meta bm = glqh_meta_row(margs, bn_meta, jb);
+        const int lo = max(bm.offset, c0), hi = min(bm.offset + bm.bs, c0 + Ls);
+        if (lo >= hi) continue;                                  // uniform over the workgroup
+        const int len = hi - lo;                                 // min(bs, Ls), a power of two
+        const int log_len = 31 - __builtin_clz(len);
+        const int nsub = bm.bs >> log_len;
+        const int r = (lo - bm.offset) >> log_len;
+        const float norm = bm.w != 0 ? __builtin_bit_cast(float, bm.w) : rsqrt_pow2(bm.log_bs);
+        for (int t = 0; t < NB; ++t) {
+            if (t >= B) break;
+            const XT *xr = x + (int64_t)t * x_stride;
+            __syncthreads();                                     // fbuf free again
+            stage_signed_slices<TR_THREADS>(fbuf, log_len, nsub, r, [&](int h, int j) -> float {
+                const int col = bm.offset + (h << log_len) + j;
+                const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
+                return col < in_features ? v : 0.0f;
+            });
+            f16 *xo = xh + t * Ls + (lo - c0);
+            struct {
+                f16 *xo;
+                float norm;
+                __device__ float aux(int) const { return norm; }
+                __device__ void put(int i, float v, float f) const { xo[i] = (f16)(v * f); }
+            } store = {xo, norm};
+            fht_staged(fbuf, log_len, store);
+        }
+    }
+    __syncthreads();
+
+    // ---- decode loop ----
+    tr_acc<NB> acc = {};
+    for (; q < q1; q += TR_PRE * TR_WAVES) {
+        tr_record<R> nxt[TR_PRE];
+#pragma unroll
+        for (int i = 0; i < TR_PRE; ++i) {
+            const int qn = q + (TR_PRE + i) * TR_WAVES;
+            nxt[i] = cur[i];
+            if (qn < q1) nxt[i] = tr_load_record<R>(lane_base + qn * STEP_BYTES);
+        }
+#pragma unroll
+        for (int i = 0; i < TR_PRE; ++i) {
+            const int qi = q + i * TR_WAVES;
+            if (qi < q1) {                                       // uniform over the wave
+                const int kp = 2 * qi + hf;
+                tr_xfrag<NB> xf;
+#pragma unroll
+                for (int t = 0; t < NB; ++t) {
+                    const uint32_t *xp = (const uint32_t *)(xh + t * Ls + (32 * kp - c0) + 2 * b);
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        xf.a[t][ks] = t < B ? xp[8 * ks] : 0u;
+                        xf.b[t][ks] = t < B ? xp[8 * ks + 4] : 0u;
+                    }
+                }
+                acc = tr_accumulate<R, NB>(cur[i], lane, xf, acc);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TR_PRE; ++i) cur[i] = nxt[i];
+    }
+    tr_reduce_to_lds<NB>(acc, red, lane, wave);
+    for (int idx = threadIdx.x; idx < NB * 32; idx += TR_THREADS) {
+        const int t = idx >> 5, row = idx & 31;
+        if (t >= B) continue;
+        float v = red[0][t][row];
+#pragma unroll
+        for (int w = 1; w < TR_WAVES; ++w) v += red[w][t][row];
+        part[((int64_t)slot * B + t) * m + 32 * mp + row] = v;
     }
 }
 
@@ -347,4 +497,90 @@ int glqh_launch_trellis_decompress(const void *packed, int R, int64_t m, int64_t
     }
     GLQH_LAUNCH_CHECK("trellis decompress launch");
     return 0;
+}
+
+// ---- fused-input GEMV: plan and launch ----------------------------------------------
+// steps per K slot: a power of two >= TR_WAVES chosen so that about four workgroups per CU
+// are in flight; the slice 64*steps is capped at 8192 columns (LDS).
+int glqh_trellis_fusein_plan(int64_t m, int64_t k, int64_t B, int *steps_out, int *ksplit_out) {
+    if (B < 1 || B > 4) return 0;
+    const int64_t nsteps = k / 64;
+    const int64_t wgs = m / 32;
+    const int64_t target = (int64_t)glqh_device_cus() * 4;
+    int64_t ks_target = (target + wgs - 1) / wgs;
+    if (ks_target < 1) ks_target = 1;
+    int64_t want = (nsteps + ks_target - 1) / ks_target;
+    int64_t steps = TR_WAVES;
+    while (steps < want) steps <<= 1;
+    if (steps > 128) steps = 128;
+    *steps_out = (int)steps;
+    *ksplit_out = (int)((nsteps + steps - 1) / steps);
+    return 1;
+}
+
+size_t glqh_trellis_fusein_lds(int steps, int NB) {
+    const size_t Ls = (size_t)steps * 64;
+    return (Ls + Ls / 32 + 32) * sizeof(float) + (size_t)NB * Ls * sizeof(f16);
+}
+
+template <int R, typename XT, int NB>
+static int launch_fusein(const void *packed, const void *x, int64_t x_stride, const void *sv, int64_t B,
+                         int64_t m, int64_t k, int64_t in_features, int steps, int ksplit,
+                         const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                         float *part, hipStream_t stream) {
+    glqh_meta_args margs;
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
+    dim3 grid((unsigned)(m / 32), (unsigned)ksplit, 1);
+    hipLaunchKernelGGL((tr_gemv_fusein_kernel<R, XT, NB>), grid, dim3(TR_THREADS),
+                       glqh_trellis_fusein_lds(steps, NB), stream, (const uint8_t *)packed, (const XT *)x,
+                       x_stride, (const f16 *)sv, (int)B, (int)m, (int)k, (int)in_features, steps,
+                       n_blocks > 1 ? bn_meta : nullptr, n_blocks > 1 ? n_blocks : 1, margs, part);
+    GLQH_LAUNCH_CHECK("trellis fused-input gemv launch");
+    return 0;
+}
+
+template <int R>
+static int launch_fusein_R(const void *packed, const void *x, int x_dtype, int64_t x_stride,
+                           const void *sv, int64_t B, int64_t m, int64_t k, int64_t in_features,
+                           int steps, int ksplit, const glqh_block_meta *bn_meta,
+                           const int64_t *blocks_host, int n_blocks, float *part, hipStream_t stream) {
+#define GLQH_FI(XT, NB) launch_fusein<R, XT, NB>(packed, x, x_stride, sv, B, m, k, in_features, steps, \
+                                                 ksplit, bn_meta, blocks_host, n_blocks, part, stream)
+    if (B == 1) return x_dtype == GLQH_F16 ? GLQH_FI(f16, 1) : GLQH_FI(uint16_t, 1);
+    return x_dtype == GLQH_F16 ? GLQH_FI(f16, 4) : GLQH_FI(uint16_t, 4);
+#undef GLQH_FI
+}
+
+int glqh_launch_trellis_fusein(const void *packed, int R, const void *x, int x_dtype, int64_t x_stride,
+                               const void *sv, int64_t B, int64_t m, int64_t k, int64_t in_features,
+                               int steps, int ksplit, const glqh_block_meta *bn_meta,
+                               const int64_t *blocks_host, int n_blocks, float *part,
+                               hipStream_t stream) {
+    switch (R) {
+    case 2: return launch_fusein_R<2>(packed, x, x_dtype, x_stride, sv, B, m, k, in_features, steps, ksplit, bn_meta, blocks_host, n_blocks, part, stream);
+    case 3: return launch_fusein_R<3>(packed, x, x_dtype, x_stride, sv, B, m, k, in_features, steps, ksplit, bn_meta, blocks_host, n_blocks, part, stream);
+    case 4: return launch_fusein_R<4>(packed, x, x_dtype, x_stride, sv, B, m, k, in_features, steps, ksplit, bn_meta, blocks_host, n_blocks, part, stream);
+    }
+    return glqh_fail("fused-input trellis kernel supports R (bits/weight) 2-4, got %d", R);
+}
+
+template <typename K>
+static int tr_set_max_lds(K kernel, int NB) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel,
+                                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)glqh_trellis_fusein_lds(128, NB)),
+                          "trellis fused-input attribute");
+}
+
+int glqh_trellis_init(void) {
+    int rc = 0;
+#define GLQH_ATTR(R) rc = rc || tr_set_max_lds(tr_gemv_fusein_kernel<R, f16, 1>, 1) ||         \
+                          tr_set_max_lds(tr_gemv_fusein_kernel<R, uint16_t, 1>, 1) ||          \
+                          tr_set_max_lds(tr_gemv_fusein_kernel<R, f16, 4>, 4) ||               \
+                          tr_set_max_lds(tr_gemv_fusein_kernel<R, uint16_t, 4>, 4)
+    GLQH_ATTR(2);
+    GLQH_ATTR(3);
+    GLQH_ATTR(4);
+#undef GLQH_ATTR
+    return rc;
 }

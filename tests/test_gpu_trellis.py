@@ -235,7 +235,7 @@ def test_yrht_shards_equal_sequential(ext):
     assert torch.equal(y, torch.cat(seq, dim=1))
 
 
-def test_fusein_gemv_equals_unfused_pipeline(ext):
+def test_fusein_gemv_matches_unfused_pipeline(ext):
     from glq_amd import hadamard as H
     m, n, inf = 64, 2048, 2000
     say("fusein")
@@ -246,4 +246,6 @@ def test_fusein_gemv_equals_unfused_pipeline(ext):
     ext.glq_input_rht_cuda(x_raw.unsqueeze(0), sv, x_rht, inf, inf, 1.0 / np.sqrt(n), n, 11)
     ref = ext.glq_decode_matvec_trellis_3inst_cuda(x_rht[0].half(), p, m, n, 0.01371)
     out = ext.glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, p, m, n, inf, 0.01371)
-    assert torch.equal(out, ref)
+    # the fused kernel builds its slice of the transform in a different summation order
+    assert rel(out, ref) < 1e-3, rel(out, ref)
+    assert torch.equal(out, ext.glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, p, m, n, inf, 0.01371))

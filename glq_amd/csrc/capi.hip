@@ -3,6 +3,7 @@
 
 #include <mutex>
 #include <string.h>
+#include <stdlib.h>
 
 int glqh_rht_init(void);
 int glqh_e8_init(void);
@@ -11,6 +12,33 @@ int glqh_launch_trellis_direct(const void *x_f16, int64_t B, const void *packed,
                                hipStream_t stream);
 int glqh_launch_trellis_decompress(const void *packed, int R, int64_t m, int64_t k, void *out,
                                    hipStream_t stream);
+int glqh_trellis_mma_plan(int64_t m, int64_t k, int *S_out, int *ksplit_out);
+int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, int R, int64_t m, int64_t k,
+                            int S, int ksplit, float *part, int direct, float scale, int accum,
+                            int64_t out_stride, hipStream_t stream);
+int glqh_trellis_mma_init(void);
+
+// GEMV / small-batch plan for activations already in the transformed domain
+static int g_use_mma = 1;
+struct tr_plan {
+    int ks, S;
+};
+static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
+    tr_plan p = {1, 0};
+    if (g_use_mma) glqh_trellis_mma_plan(m, k, &p.S, &p.ks);
+    else p.ks = glqh_trellis_pick_ksplit(m, k, B);
+    return p;
+}
+static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
+                            int64_t k, float *part, hipStream_t st) {
+    if (g_use_mma) return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
+    return glqh_launch_trellis_partial(x_f16, B, packed, R, m, k, p.ks, part, st);
+}
+static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
+                           int64_t k, float scale, float *out, int64_t out_stride, int accum, hipStream_t st) {
+    if (g_use_mma) return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
+    return glqh_launch_trellis_direct(x_f16, B, packed, R, m, k, scale, out, out_stride, accum, st);
+}
 
 // ---- error plumbing -------------------------------------------------------------
 static thread_local char g_err[512] = "";
@@ -51,7 +79,8 @@ extern "C" int glqh_init(void) {
             return;
         }
         g_cus = prop.multiProcessorCount;
-        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init();
+        if (const char *e = getenv("GLQ_TRELLIS_MMA")) g_use_mma = atoi(e);
+        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init() || glqh_trellis_mma_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
     return g_init_rc;
@@ -101,7 +130,7 @@ extern "C" int glqh_decompress_trellis_3inst(const void *packed, int64_t packed_
 extern "C" size_t glqh_trellis_gemv_workspace_bytes(int64_t m, int64_t k, int64_t B) {
     if (!glqh_trellis_kernel_supported(m, k) || B < 1) return 0;
     glqh_init();
-    int ks = glqh_trellis_pick_ksplit(m, k, B);
+    int ks = tr_plain_plan(m, k, B).ks;
     return ks > 1 ? align256((size_t)ks * B * m * sizeof(float)) : 0;
 }
 
@@ -117,14 +146,14 @@ extern "C" int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B, co
     int R;
     if (tr_bits_from_packed(packed_cols, accum, &R) || tr_check_shape(m, k, packed_rows)) return 1;
     hipStream_t st = (hipStream_t)stream;
-    int ks = glqh_trellis_pick_ksplit(m, k, B);
+    const tr_plan plan = tr_plain_plan(m, k, B);
+    const int ks = plan.ks;
     if (ks == 1)
-        return glqh_launch_trellis_direct(x_f16, B, packed, R, m, k, (float)wscale, out, out_stride,
-                                          accum, st);
+        return tr_plain_direct(plan, x_f16, B, packed, R, m, k, (float)wscale, out, out_stride, accum, st);
     size_t need = (size_t)ks * B * m * sizeof(float);
     GLQH_REQUIRE(ws && ws_bytes >= need, "trellis matmul: workspace of %zu bytes needed, got %zu", need,
                  ws_bytes);
-    if (glqh_launch_trellis_partial(x_f16, B, packed, R, m, k, ks, (float *)ws, st)) return 1;
+    if (tr_plain_partial(plan, x_f16, B, packed, R, m, k, (float *)ws, st)) return 1;
     return glqh_launch_reduce_splits((const float *)ws, ks, B * m, B, m, (float)wscale, out, out_stride, accum, st);
 }
 
@@ -137,11 +166,12 @@ extern "C" int glqh_trellis_gemv_partials(const void *x_f16, int64_t B, const vo
     GLQH_REQUIRE(B >= 1 && B <= 65535 * 8, "trellis partials: B=%lld out of range", (long long)B);
     int R;
     if (tr_bits_from_packed(packed_cols, 1, &R) || tr_check_shape(m, k, packed_rows)) return 1;
-    const int ks = glqh_trellis_pick_ksplit(m, k, B);
+    const tr_plan plan = tr_plain_plan(m, k, B);
+    const int ks = plan.ks;
     const size_t need = (size_t)ks * B * m * sizeof(float);
     GLQH_REQUIRE(part_bytes >= need, "trellis partials: buffer of %zu bytes needed, got %zu", need, part_bytes);
     *ksplit_out = ks;
-    return glqh_launch_trellis_partial(x_f16, B, packed, R, m, k, ks, part, (hipStream_t)stream);
+    return tr_plain_partial(plan, x_f16, B, packed, R, m, k, part, (hipStream_t)stream);
 }
 
 // ---- RHT -------------------------------------------------------------------------
@@ -189,7 +219,7 @@ extern "C" int glqh_output_rht_shards(const float *y_rht, const void *su_f16, vo
 // ---- fused trellis linear ----------------------------------------------------------
 // workspace layout: [x_rht f16 (B, n_pad)] [partials stage 1] [partials stage 2]
 static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
-    int ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
+    int ks = tr_plain_plan(m_pad, n_pad, B).ks;
     int steps = 0, ks2 = 0;
     if (glqh_trellis_fusein_plan(m_pad, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
     return align256((size_t)ks * B * m_pad * sizeof(float));
@@ -262,9 +292,10 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
                                   bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
             return 1;
-        ks = glqh_trellis_pick_ksplit(m_pad, n_pad, B);
-        if (glqh_launch_trellis_partial(x_rht, B, packed, R1, m_pad, n_pad, ks, part1, st)) return 1;
-        if (has_s2 && glqh_launch_trellis_partial(x_rht, B, packed2, R2, m_pad, n_pad, ks, part2, st)) return 1;
+        const tr_plan plan = tr_plain_plan(m_pad, n_pad, B);
+        ks = plan.ks;
+        if (tr_plain_partial(plan, x_rht, B, packed, R1, m_pad, n_pad, part1, st)) return 1;
+        if (has_s2 && tr_plain_partial(plan, x_rht, B, packed2, R2, m_pad, n_pad, part2, st)) return 1;
     }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);

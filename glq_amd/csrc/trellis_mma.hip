@@ -1,0 +1,334 @@
+// Trellis-3INST GEMV / small-batch GEMM on the matrix cores (gfx950, wave64).
+//
+// The decoded weights never leave registers: the lane that decodes a state already holds
+// it where v_mfma_f32_16x16x32_f16 expects its A operand.
+//
+//   * A wave step covers 64 rows x 32 columns: the block (m-pair, k-pair) = (2*bx + hm, kp)
+//     for hm = 0, 1.  Lane L = 16*q + i takes stream lane l = 4*(i & 7) + q of block
+//     hm = i >> 3.  That stream lane owns, in each of the four row groups s = 0..3
+//     (rows 32*hm + (i & 7) + 8*s) and each k-tile ks, the four weights of columns
+//     16*ks + 2*q + {0, 1, 8, 9} (glq/trellis.py:99-101).
+//   * 3INST yields a weight as the sum of two fp16 halves packed in one register
+//     (glq/trellis.py:122-134).  The halves are fed to the MFMA unadded, as two k-elements
+//     that meet the same activation, so the A operand of (row i, k-group q) is simply the
+//     four hash registers {w, w', w'', w'''} = 8 fp16 values, with no repacking.
+//   * The B operand of (k-group q, token t) is then the activation pairs
+//     (x[c], x[c]), (x[c+1], x[c+1]), (x[c+8], x[c+8]), (x[c+9], x[c+9]), c = 16*ks + 2*q:
+//     16 bytes, staged once per workgroup into LDS in exactly that form, one slot per
+//     (k-pair, token tile, ks, q, token).
+//   * D[i][t] accumulates in fp32 over k; lane L holds rows 4*(L >> 4) + {0..3} of token
+//     L & 15.
+//
+// One MFMA multiplies 16 rows x 32 fp16 against 16 tokens, so 1..16 tokens cost the same
+// vector-ALU work (the state decode), and the dot products are off the vector ALU.
+// K is split into contiguous slots (shape-only, so that row b of a batched call sums in
+// exactly the order of the GEMV on x[b]; glq/csrc/glq_trellis.cu:555-715); the four waves
+// of a workgroup take the slot's k-pairs round-robin and are summed in wave order.
+#include "common.h"
+#include "trellis_device.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int NT>
+struct mma_acc {
+    f32x4 v[4][NT];          // [row group s][token tile]
+};
+
+// 16-byte slots per (k-pair, token tile, ks, q) group: 17 for full tiles so that the
+// staging writes of one wave (q fastest) land in distinct banks.
+template <int TP>
+constexpr int mma_tps() { return TP == 16 ? 17 : TP; }
+
+__host__ __device__ constexpr int mma_slot_bytes(int TP, int NT) {
+    return NT * 8 * (TP == 16 ? 17 : TP) * 16;                  // LDS bytes per k-pair
+}
+
+// decode one record (32 weights per lane) and multiply it against NT token tiles
+template <int R, int TP, int NT>
+__device__ __forceinline__ mma_acc<NT> mma_record(const tr_record<R> r, int next1, int next2,
+                                                  const u32x4 *xs, mma_acc<NT> acc) {
+    constexpr int TPS = mma_tps<TP>();
+    uint32_t cont[4];
+    tr_continuation_from<R>(r, next1, next2, cont);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        f16x8 bf[NT];
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) {
+            bf[tt] = __builtin_bit_cast(f16x8, xs[((tt * 2 + ks) * 4) * TPS]);
+        }
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) {
+            const int ci = ks * 2 + ms;
+            uint32_t h[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) h[j] = tr_hash(tr_state<R>(r.c[ci], cont[ci], j));
+            const f16x8 a0 = __builtin_bit_cast(f16x8, u32x4{h[0], h[1], h[4], h[5]});
+            const f16x8 a1 = __builtin_bit_cast(f16x8, u32x4{h[2], h[3], h[6], h[7]});
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) {
+                acc.v[2 * ms][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, bf[tt], acc.v[2 * ms][tt], 0, 0, 0);
+                acc.v[2 * ms + 1][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, bf[tt], acc.v[2 * ms + 1][tt], 0, 0, 0);
+            }
+        }
+    }
+    return acc;
+}
+
+// (lo, lo) / (hi, hi) of a packed fp16 pair
+__device__ __forceinline__ uint32_t splat_lo(uint32_t v) { return __builtin_amdgcn_perm(v, v, 0x05040504u); }
+__device__ __forceinline__ uint32_t splat_hi(uint32_t v) { return __builtin_amdgcn_perm(v, v, 0x07060706u); }
+
+struct mma_lane {
+    int i, q, hm, l, next1, next2, tokl;
+    bool live;
+};
+
+template <int TP>
+__device__ __forceinline__ mma_lane mma_lane_of(int lane) {
+    mma_lane a;
+    a.i = lane & 15;
+    a.q = lane >> 4;
+    a.hm = a.i >> 3;
+    a.l = 4 * (a.i & 7) + a.q;
+    const int l1 = (a.l + 1) & 31, l2 = (a.l + 2) & 31;
+    a.next1 = 16 * (l1 & 3) + 8 * a.hm + (l1 >> 2);
+    a.next2 = 16 * (l2 & 3) + 8 * a.hm + (l2 >> 2);
+    a.tokl = lane & 15;
+    a.live = a.tokl < TP;
+    return a;
+}
+
+// Sum the four waves' accumulators through LDS in wave order and write them out, G row
+// groups per pass (all four when the buffer allows).  red: [TR_WAVES][G][NT][4][4*TP] floats.
+template <int NT>
+constexpr int mma_red_groups() { return NT <= 2 ? 4 : 2; }
+
+template <int TP, int NT>
+constexpr int mma_red_bytes() { return TR_WAVES * mma_red_groups<NT>() * NT * 4 * 4 * TP * 4; }
+
+template <int TP, int NT>
+__device__ __forceinline__ void mma_reduce_store(const mma_acc<NT> acc, float *red, const mma_lane a,
+                                                 int wave, int B, int m, int tok0, int row0, int slot,
+                                                 float *__restrict__ part, int direct, float scale,
+                                                 int accum, int64_t out_stride) {
+    constexpr int CL = 4 * TP;
+    constexpr int G = mma_red_groups<NT>();
+    constexpr int PER_WAVE = G * NT * 4 * CL;
+#pragma unroll
+    for (int s0 = 0; s0 < 4; s0 += G) {
+        __syncthreads();
+        if (a.live) {
+            const int cl = a.q * TP + a.tokl;
+#pragma unroll
+            for (int sg = 0; sg < G; ++sg)
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        red[wave * PER_WAVE + ((sg * NT + tt) * 4 + r) * CL + cl] = acc.v[s0 + sg][tt][r];
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < PER_WAVE; e += TR_THREADS) {
+            const int cl = e % CL;
+            int rest = e / CL;
+            const int r = rest & 3;
+            rest >>= 2;
+            const int tt = rest % NT, sg = rest / NT;
+            const int i = 4 * (cl / TP) + r;
+            const int row = row0 + 32 * (i >> 3) + (i & 7) + 8 * (s0 + sg);
+            const int tok = tok0 + 16 * tt + (cl % TP);
+            if (tok >= B || row >= m) continue;
+            float v = red[e];
+#pragma unroll
+            for (int w = 1; w < TR_WAVES; ++w) v += red[w * PER_WAVE + e];
+            if (direct) {
+                float *o = part + (int64_t)tok * out_stride + row;
+                *o = accum ? (*o + scale * v) : scale * v;
+            } else {
+                part[((int64_t)slot * B + tok) * m + row] = v;
+            }
+        }
+    }
+}
+
+// Stage the activations of k-pairs [c0, c0+n) and tokens [tok0, tok0 + 16*NT) into the LDS
+// slots.  One item = 16 bytes of one token (columns 8h..8h+7 of a k-pair), which feeds the
+// (2*hb, 2*hb+1) dwords of four slots; U items are requested before any is written.
+template <int TP, int NT>
+__device__ __forceinline__ void mma_stage(uint32_t *xs, const f16 *__restrict__ x, int B, int k, int tok0,
+                                          int c0, int n) {
+    constexpr int TPS = mma_tps<TP>();
+    constexpr int U = 4;
+    const int total = NT * TP * n * 4;
+    for (int base = 0; base < total; base += U * TR_THREADS) {
+        u32x4 v[U];
+        int dst[U];
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu) {
+            const int idx = min(base + uu * TR_THREADS + (int)threadIdx.x, total - 1);
+            const int h = idx & 3;
+            const int u = (idx >> 2) % n, tk = (idx >> 2) / n;
+            const int tt = tk / TP, tl = tk % TP;
+            const int tok = tok0 + 16 * tt + tl;
+            const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tok, B - 1) * k + 32 * (c0 + u) + 8 * h);
+            v[uu] = tok < B ? ld : u32x4{0u, 0u, 0u, 0u};
+            // dword index of (u, tt, ks = h>>1, q = 0, tl), plus 2*hb
+            dst[uu] = ((((u * NT + tt) * 2 + (h >> 1)) * 4) * TPS + tl) * 4 + 2 * (h & 1);
+        }
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu) {
+            if (base + uu * TR_THREADS + (int)threadIdx.x < total) {
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq)
+                    *(u32x2 *)(xs + dst[uu] + qq * TPS * 4) = u32x2{splat_lo(v[uu][qq]), splat_hi(v[uu][qq])};
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// x given as fp16 (B, k) in the transformed domain.
+// grid = (ceil(m/64), ksplit, ceil(B / (16*NT))); slot s owns k-pairs [s*S, (s+1)*S); the
+// slot's activations are staged through LDS in chunks of CH k-pairs (CH % 4 == 0).
+// ---------------------------------------------------------------------------------
+template <int R, int TP, int NT>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int B, int m, int k,
+              int S, int CH, float *__restrict__ part, int direct, float scale, int accum,
+              int64_t out_stride) {
+    extern __shared__ u32x4 xs_lds[];
+    constexpr int TPS = mma_tps<TP>();
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const mma_lane a = mma_lane_of<TP>(lane);
+    const int nkp = k >> 5;
+    const int mpairs = m >> 5;
+    const int slot = blockIdx.y;
+    const int kp0 = slot * S;
+    const int kp1 = min(kp0 + S, nkp);
+    const int tok0 = blockIdx.z * (16 * NT);
+    const int mp = min(2 * (int)blockIdx.x + a.hm, mpairs - 1);      // odd m/32: clamp, rows dropped later
+
+    constexpr int REC = 4 * R;
+    const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;   // + kp * 32 * REC
+    int kp = kp0 + wave;
+    tr_record<R> cur = {};
+    if (kp < kp1) cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
+
+    mma_acc<NT> acc;
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) acc.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // lanes past the token count read a zeroed block (one k-pair's worth, after the chunk)
+    u32x4 *zero_blk = xs_lds + CH * (NT * 8 * TPS);
+    if constexpr (TP < 16) {
+        for (int i = threadIdx.x; i < NT * 8 * TPS; i += TR_THREADS) zero_blk[i] = u32x4{0u, 0u, 0u, 0u};
+    }
+    for (int c0 = kp0; c0 < kp1; c0 += CH) {
+        const int c1 = min(c0 + CH, kp1);
+        __syncthreads();                                       // previous chunk consumed
+        mma_stage<TP, NT>((uint32_t *)xs_lds, x, B, k, tok0, c0, c1 - c0);
+        __syncthreads();
+        for (; kp < c1; kp += TR_WAVES) {
+            tr_record<R> nxt = cur;
+            if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
+            const u32x4 *xs = a.live ? xs_lds + ((kp - c0) * NT * 8 + a.q) * TPS + a.tokl : zero_blk;
+            acc = mma_record<R, TP, NT>(cur, a.next1, a.next2, xs, acc);
+            cur = nxt;
+        }
+    }
+    mma_reduce_store<TP, NT>(acc, (float *)xs_lds, a, wave, B, m, tok0, 64 * blockIdx.x, slot, part,
+                             direct, scale, accum, out_stride);
+}
+
+// LDS per workgroup: a chunk of CH k-pairs (CH % 4 == 0) plus, for partial token tiles, one
+// zeroed block; small enough that the register-limited number of workgroups fits a CU.
+constexpr int MMA_LDS_MAX = 64 * 1024;
+
+template <int TP, int NT>
+constexpr int mma_chunk_cap() {
+    return TP == 1 ? 448 : TP == 4 ? 64 : NT == 1 ? 8 : 4;
+}
+
+template <int R, int TP, int NT>
+int launch_mma(const void *x, int64_t B, const void *packed, int64_t m, int64_t k, int S, int ksplit,
+               float *part, int direct, float scale, int accum, int64_t out_stride, hipStream_t stream) {
+    const int per_kp = mma_slot_bytes(TP, NT);
+    int CH = mma_chunk_cap<TP, NT>();
+    if (CH > S) CH = (S + 3) & ~3;
+    size_t lds = (size_t)(CH + (TP < 16 ? 1 : 0)) * per_kp;
+    if (lds < (size_t)mma_red_bytes<TP, NT>()) lds = mma_red_bytes<TP, NT>();
+    dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, (unsigned)((B + 16 * NT - 1) / (16 * NT)));
+    hipLaunchKernelGGL((tr_mma_kernel<R, TP, NT>), grid, dim3(TR_THREADS), lds, stream,
+                       (const uint8_t *)packed, (const f16 *)x, (int)B, (int)m, (int)k, S, CH, part, direct,
+                       scale, accum, out_stride);
+    GLQH_LAUNCH_CHECK("trellis mma launch");
+    return 0;
+}
+
+template <int R>
+int launch_mma_R(const void *x, int64_t B, const void *packed, int64_t m, int64_t k, int S, int ksplit,
+                 float *part, int direct, float scale, int accum, int64_t out_stride, hipStream_t stream) {
+#define GLQH_MMA(TP, NT) launch_mma<R, TP, NT>(x, B, packed, m, k, S, ksplit, part, direct, scale, accum, \
+                                               out_stride, stream)
+    if (B == 1) return GLQH_MMA(1, 1);
+    if (B <= 4) return GLQH_MMA(4, 1);
+    if (B <= 16) return GLQH_MMA(16, 1);
+    if (B <= 32) return GLQH_MMA(16, 2);
+    return GLQH_MMA(16, 4);
+#undef GLQH_MMA
+}
+
+template <typename K>
+int mma_set_lds(K kernel) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              MMA_LDS_MAX),
+                          "trellis mma attribute");
+}
+
+template <int R>
+int mma_init_R() {
+    return mma_set_lds(tr_mma_kernel<R, 1, 1>) || mma_set_lds(tr_mma_kernel<R, 4, 1>) ||
+           mma_set_lds(tr_mma_kernel<R, 16, 1>) || mma_set_lds(tr_mma_kernel<R, 16, 2>) ||
+           mma_set_lds(tr_mma_kernel<R, 16, 4>);
+}
+
+}  // namespace
+
+// K slots: S k-pairs (32 columns) each, a multiple of the wave count, chosen from the
+// layer shape only; about four workgroups per CU.
+int glqh_trellis_mma_plan(int64_t m, int64_t k, int *S_out, int *ksplit_out) {
+    const int64_t nkp = k / 32;
+    const int64_t wgs = (m + 63) / 64;
+    const int64_t target = (int64_t)glqh_device_cus() * 4;
+    int64_t ks = (target + wgs - 1) / wgs;
+    if (ks > 64) ks = 64;
+    if (ks < 1) ks = 1;
+    int64_t S = (nkp + ks - 1) / ks;
+    S = (S + TR_WAVES - 1) / TR_WAVES * TR_WAVES;
+    *S_out = (int)S;
+    *ksplit_out = (int)((nkp + S - 1) / S);
+    return 1;
+}
+
+int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, int R, int64_t m, int64_t k,
+                            int S, int ksplit, float *part, int direct, float scale, int accum,
+                            int64_t out_stride, hipStream_t stream) {
+    switch (R) {
+    case 1: return launch_mma_R<1>(x_f16, B, packed, m, k, S, ksplit, part, direct, scale, accum, out_stride, stream);
+    case 2: return launch_mma_R<2>(x_f16, B, packed, m, k, S, ksplit, part, direct, scale, accum, out_stride, stream);
+    case 3: return launch_mma_R<3>(x_f16, B, packed, m, k, S, ksplit, part, direct, scale, accum, out_stride, stream);
+    case 4: return launch_mma_R<4>(x_f16, B, packed, m, k, S, ksplit, part, direct, scale, accum, out_stride, stream);
+    }
+    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}
+
+int glqh_trellis_mma_init(void) {
+    return mma_init_R<1>() || mma_init_R<2>() || mma_init_R<3>() || mma_init_R<4>();
+}

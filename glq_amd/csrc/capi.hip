@@ -7,9 +7,6 @@
 
 int glqh_rht_init(void);
 int glqh_e8_init(void);
-int glqh_launch_trellis_direct(const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                               int64_t k, float scale, float *out, int64_t out_stride, int accum,
-                               hipStream_t stream);
 int glqh_launch_trellis_decompress(const void *packed, int R, int64_t m, int64_t k, void *out,
                                    hipStream_t stream);
 int glqh_trellis_mma_plan(int64_t m, int64_t k, int *S_out, int *ksplit_out);
@@ -18,26 +15,32 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
                             int64_t out_stride, hipStream_t stream);
 int glqh_trellis_mma_init(void);
 
-// GEMV / small-batch plan for activations already in the transformed domain
-static int g_use_mma = 1;
+int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out);
+int glqh_launch_trellis_prefill(const void *x_f16, int64_t M, const void *packed, int R, int64_t m, int64_t k,
+                                int S, int ksplit, float *out, int direct, float scale, int accum,
+                                int64_t out_stride, hipStream_t stream);
+
+// Plan for activations already in the transformed domain: up to 64 tokens share one pass
+// over the packed stream with K split by shape only; larger batches use 128-token tiles.
+#define GLQH_TRELLIS_SMALL_BATCH 64
 struct tr_plan {
-    int ks, S;
+    int ks, S, prefill;
 };
 static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
-    tr_plan p = {1, 0};
-    if (g_use_mma) glqh_trellis_mma_plan(m, k, &p.S, &p.ks);
-    else p.ks = glqh_trellis_pick_ksplit(m, k, B);
+    tr_plan p = {1, 0, B > GLQH_TRELLIS_SMALL_BATCH};
+    if (p.prefill) glqh_trellis_prefill_plan(m, k, B, &p.S, &p.ks);
+    else glqh_trellis_mma_plan(m, k, &p.S, &p.ks);
     return p;
 }
 static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
                             int64_t k, float *part, hipStream_t st) {
-    if (g_use_mma) return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
-    return glqh_launch_trellis_partial(x_f16, B, packed, R, m, k, p.ks, part, st);
+    if (p.prefill) return glqh_launch_trellis_prefill(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
+    return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
 }
 static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
                            int64_t k, float scale, float *out, int64_t out_stride, int accum, hipStream_t st) {
-    if (g_use_mma) return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
-    return glqh_launch_trellis_direct(x_f16, B, packed, R, m, k, scale, out, out_stride, accum, st);
+    if (p.prefill) return glqh_launch_trellis_prefill(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
+    return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
 }
 
 // ---- error plumbing -------------------------------------------------------------
@@ -79,7 +82,6 @@ extern "C" int glqh_init(void) {
             return;
         }
         g_cus = prop.multiProcessorCount;
-        if (const char *e = getenv("GLQ_TRELLIS_MMA")) g_use_mma = atoi(e);
         g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init() || glqh_trellis_mma_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");

@@ -128,11 +128,6 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
                            int64_t n_blocks, int64_t max_bs_hint, float rsqrt_m,
                            hipStream_t stream);
 
-// trellis GEMV/GEMM into split-K partials (or directly into `out` when ksplit == 1)
-int glqh_trellis_pick_ksplit(int64_t m, int64_t k, int64_t B);
-int glqh_launch_trellis_partial(const void *x_f16, int64_t B, const void *packed, int R,
-                                int64_t m, int64_t k, int ksplit, float *part,
-                                hipStream_t stream);
 // out[tok, row] = (accum ? out : 0) + scale * sum_s part[s * kstride + tok * m + row]
 int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, int64_t B, int64_t m,
                               float scale, float *out, int64_t out_stride, int accum,

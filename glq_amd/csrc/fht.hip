@@ -22,14 +22,14 @@ struct rht_slice {
 
 // blockIdx.x = block * spb + slice; workgroups past a block's slice count retire.
 __device__ __forceinline__ rht_slice rht_get_slice(const glqh_block_meta *meta, const glqh_meta_args margs,
-                                                   float single_norm, int spb) {
+                                                   float single_norm, int spb, int log_slice) {
     const int j = blockIdx.x / spb;
     glqh_block_meta mrow = glqh_meta_row(margs, meta, j);
     rht_slice b;
     b.off = mrow.offset;
     b.bs = mrow.bs;
     b.log_bs = mrow.log_bs;
-    b.log_len = min(mrow.log_bs, LOG_SLICE);
+    b.log_len = min(mrow.log_bs, log_slice);
     b.nsub = mrow.bs >> b.log_len;
     b.r = blockIdx.x % spb;
     b.live = b.r < b.nsub;
@@ -45,9 +45,9 @@ __global__ void __launch_bounds__(RHT_THREADS)
 input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
                  OT *__restrict__ out, int in_features, int n_pad,
                  const glqh_block_meta *__restrict__ meta, glqh_meta_args margs,
-                 float single_norm, int spb) {
-    __shared__ float s[SLICE_LDS_FLOATS];
-    const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb);
+                 float single_norm, int spb, int log_slice) {
+    extern __shared__ float s[];
+    const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const XT *xr = x + (int64_t)blockIdx.y * x_stride;
     stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, [&](int h, int i) -> float {
@@ -68,9 +68,9 @@ template <typename YT, bool PARTS>
 __global__ void __launch_bounds__(RHT_THREADS)
 output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
                   int out_features, int m_pad, const glqh_block_meta *__restrict__ meta,
-                  glqh_meta_args margs, float single_norm, int spb) {
-    __shared__ float s[SLICE_LDS_FLOATS];
-    const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb);
+                  glqh_meta_args margs, float single_norm, int spb, int log_slice) {
+    extern __shared__ float s[];
+    const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const int64_t b = blockIdx.y;
     if constexpr (!PARTS) {
@@ -153,9 +153,18 @@ output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y,
     fht_staged(s, blk.log_len, store);
 }
 
-int rht_slices_per_block(int64_t max_bs) {
-    int64_t spb = max_bs >> LOG_SLICE;
+// Few tokens: 1024-point slices, one workgroup each, so that a single row still spreads
+// over the chip (each slice re-reads its whole block).  Many tokens fill the chip by
+// themselves: blocks up to 8192 points are then transformed whole, read once.
+int rht_log_slice(int64_t B) { return B > 64 ? 13 : LOG_SLICE; }
+
+int rht_slices_per_block(int64_t max_bs, int log_slice) {
+    int64_t spb = max_bs >> log_slice;
     return spb < 1 ? 1 : (int)spb;
+}
+
+size_t rht_lds_bytes(int log_slice) {
+    return (((size_t)1 << log_slice) + ((size_t)1 << log_slice) / 32 + 32) * sizeof(float);
 }
 
 int check_blocks(const int64_t *blocks_host, int64_t n_blocks, int64_t total, int64_t *max_bs,
@@ -207,13 +216,15 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
     }
     if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, n_pad))
         margs.canon = 0;                               // not canonical: kernel reads meta_dev
-    const int spb = rht_slices_per_block(max_bs);
+    const int log_slice = rht_log_slice(B);
+    const int spb = rht_slices_per_block(max_bs, log_slice);
     GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "input_rht: too many slices");
     dim3 grid((unsigned)(n_blocks * spb), (unsigned)B);
 #define GLQH_IN_LAUNCH(XT, OT)                                                                      \
-    hipLaunchKernelGGL((input_rht_kernel<XT, OT>), grid, dim3(RHT_THREADS), 0, stream,              \
-                       (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
-                       (int)n_pad, meta_dev, margs, rsqrt_n, spb)
+    hipLaunchKernelGGL((input_rht_kernel<XT, OT>), grid, dim3(RHT_THREADS),                         \
+                       rht_lds_bytes(log_slice), stream, (const XT *)x, x_stride, (const f16 *)sv,  \
+                       (OT *)out, (int)in_features, (int)n_pad, meta_dev, margs, rsqrt_n, spb,      \
+                       log_slice)
     if (out_dtype == GLQH_F32) {
         if (x_dtype == GLQH_F16) GLQH_IN_LAUNCH(f16, float);
         else if (x_dtype == GLQH_BF16) GLQH_IN_LAUNCH(uint16_t, float);
@@ -259,13 +270,14 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
     }
     if (meta_dev && !blocks_host) margs.canon = 0;         // shard-batched call: device meta only
     else if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, m_pad)) margs.canon = 0;
-    const int spb = rht_slices_per_block(max_bs);
+    const int log_slice = rht_log_slice(B);
+    const int spb = rht_slices_per_block(max_bs, log_slice);
     GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "output_rht: too many slices");
     dim3 grid((unsigned)(n_blocks * spb), (unsigned)B);
 #define GLQH_OUT_LAUNCH(YT, PARTS)                                                                  \
-    hipLaunchKernelGGL((output_rht_kernel<YT, PARTS>), grid, dim3(RHT_THREADS), 0, stream, src,     \
-                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, meta_dev, \
-                       margs, rsqrt_m, spb)
+    hipLaunchKernelGGL((output_rht_kernel<YT, PARTS>), grid, dim3(RHT_THREADS),                     \
+                       rht_lds_bytes(log_slice), stream, src, (const f16 *)su, (YT *)y, y_stride,   \
+                       (int)out_features, (int)m_pad, meta_dev, margs, rsqrt_m, spb, log_slice)
     if (src.nparts == 0) {
         if (y_dtype == GLQH_F16) GLQH_OUT_LAUNCH(f16, false);
         else if (y_dtype == GLQH_BF16) GLQH_OUT_LAUNCH(uint16_t, false);

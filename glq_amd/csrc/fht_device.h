@@ -14,8 +14,8 @@
 // Walsh-Hadamard transform of the block (summation order differs from the
 // ascending-distance order of glq/hadamard.py:10-28 by fp32 rounding only).
 //
-// Blocks larger than a slice (GLQH_LOG_SLICE) are never transformed whole: H_bs factors
-// as H_(bs/len) (x) H_len, so slice r of the output is
+// Blocks larger than a slice (a launch parameter) are not transformed whole: H_bs factors as
+// H_(bs/len) (x) H_len, so slice r of the output is
 //     H_len( sum_h (-1)^popcount(r & h) * in[h*len + i] ),
 // one pass over the block's inputs followed by a short transform -- which lets every slice
 // go to its own workgroup.
@@ -34,7 +34,6 @@
 #endif
 constexpr int RMAX = GLQH_RMAX;
 constexpr int LOG_SLICE = GLQH_LOG_SLICE;
-constexpr int SLICE_LDS_FLOATS = (1 << LOG_SLICE) + (1 << LOG_SLICE) / 32 + 32;
 
 __device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
 

@@ -134,67 +134,6 @@ __device__ __forceinline__ void tr_reduce_to_lds(tr_acc<NB> acc, float (*red)[NB
 }
 
 // ---------------------------------------------------------------------------------
-// GEMV / small-batch GEMM against the packed stream
-// ---------------------------------------------------------------------------------
-// grid = (m/32, ksplit, ceil(B/NB)); each workgroup owns one m-pair (32 rows) for NB
-// tokens and a round-robin share of the k/64 wave-steps.  Output: raw fp32 sums to
-// part[(slot*B + token)*m + row], or (direct) scaled into out.
-template <int R, int NB>
-__global__ void __launch_bounds__(TR_THREADS)
-tr_gemv_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int B, int m, int k,
-               float *__restrict__ part, int direct, float scale, int accum, int64_t out_stride) {
-    __shared__ float red[TR_WAVES][NB][32];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int l = lane & 31;
-    const int hf = lane >> 5;
-    const int b = l & 3;
-    const int mp = blockIdx.x;
-    const int nsteps = k >> 6;
-    const int stride = gridDim.y * TR_WAVES;
-    const int tok0 = blockIdx.z * NB;
-
-    tr_acc<NB> acc = {};
-
-    const uint8_t *row_base = packed + (int64_t)mp * (k >> 5) * 32 * (4 * R);
-    for (int q = blockIdx.y * TR_WAVES + wave; q < nsteps; q += stride) {
-        const int kp = 2 * q + hf;
-        tr_record<R> r = tr_load_record<R>(row_base + ((int64_t)kp * 32 + l) * (4 * R));
-        // activations of this lane's four columns in each of the two k-tiles
-        tr_xfrag<NB> xf;
-#pragma unroll
-        for (int t = 0; t < NB; ++t) {
-            const int tok = tok0 + t;
-            const bool live = tok < B;
-            const uint32_t *xp = (const uint32_t *)(x + (int64_t)(live ? tok : 0) * k + 32 * kp + 2 * b);
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                uint32_t va = xp[8 * ks], vb = xp[8 * ks + 4];
-                xf.a[t][ks] = live ? va : 0u;
-                xf.b[t][ks] = live ? vb : 0u;
-            }
-        }
-        acc = tr_accumulate<R, NB>(r, lane, xf, acc);
-    }
-
-    tr_reduce_to_lds<NB>(acc, red, lane, wave);
-    for (int idx = threadIdx.x; idx < NB * 32; idx += TR_THREADS) {
-        const int t = idx >> 5, row = idx & 31;
-        const int tok = tok0 + t;
-        if (tok >= B) continue;
-        float v = red[0][t][row];
-#pragma unroll
-        for (int w = 1; w < TR_WAVES; ++w) v += red[w][t][row];
-        if (direct) {
-            float *o = part + (int64_t)tok * out_stride + 32 * mp + row;
-            *o = accum ? (*o + scale * v) : scale * v;
-        } else {
-            part[((int64_t)blockIdx.y * B + tok) * m + 32 * mp + row] = v;
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------------
 // GEMV with the input transform folded in (B <= NB tokens).
 //
 // grid = (m/32, ksplit).  K slot s owns the `steps` consecutive wave-steps starting at
@@ -328,70 +267,7 @@ reduce_splits_kernel(const float *__restrict__ part, int ksplit, int64_t kstride
     *o = accum ? (*o + scale * v) : scale * v;
 }
 
-template <int R>
-int launch_gemv_R(const void *x, int64_t B, const void *packed, int64_t m, int64_t k, int ksplit,
-                  float *part, int direct, float scale, int accum, int64_t out_stride,
-                  hipStream_t stream) {
-    const uint8_t *p = (const uint8_t *)packed;
-    const f16 *xp = (const f16 *)x;
-    if (B == 1) {
-        dim3 grid((unsigned)(m / 32), (unsigned)ksplit, 1);
-        hipLaunchKernelGGL((tr_gemv_kernel<R, 1>), grid, dim3(TR_THREADS), 0, stream, p, xp, (int)B,
-                           (int)m, (int)k, part, direct, scale, accum, out_stride);
-    } else if (B <= 4) {
-        dim3 grid((unsigned)(m / 32), (unsigned)ksplit, 1);
-        hipLaunchKernelGGL((tr_gemv_kernel<R, 4>), grid, dim3(TR_THREADS), 0, stream, p, xp, (int)B,
-                           (int)m, (int)k, part, direct, scale, accum, out_stride);
-    } else {
-        dim3 grid((unsigned)(m / 32), (unsigned)ksplit, (unsigned)((B + 7) / 8));
-        hipLaunchKernelGGL((tr_gemv_kernel<R, 8>), grid, dim3(TR_THREADS), 0, stream, p, xp, (int)B,
-                           (int)m, (int)k, part, direct, scale, accum, out_stride);
-    }
-    GLQH_LAUNCH_CHECK("trellis gemv launch");
-    return 0;
-}
-
 }  // namespace
-
-// The K-split depends on the layer shape only, never on the token count, so that row b of
-// a batched call sums in exactly the order of the GEMV on x[b].
-int glqh_trellis_pick_ksplit(int64_t m, int64_t k, int64_t B) {
-    (void)B;
-    const int64_t nsteps = k / 64;
-    const int64_t wgs = m / 32;
-    const int64_t target = (int64_t)glqh_device_cus() * 4;       // 16 waves per CU
-    int64_t ks = (target + wgs - 1) / wgs;
-    int64_t cap = nsteps / TR_WAVES;
-    if (cap < 1) cap = 1;
-    if (ks > cap) ks = cap;
-    if (ks > 32) ks = 32;
-    if (ks < 1) ks = 1;
-    return (int)ks;
-}
-
-int glqh_launch_trellis_partial(const void *x_f16, int64_t B, const void *packed, int R,
-                                int64_t m, int64_t k, int ksplit, float *part,
-                                hipStream_t stream) {
-    switch (R) {
-    case 1: return launch_gemv_R<1>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
-    case 2: return launch_gemv_R<2>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
-    case 3: return launch_gemv_R<3>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
-    case 4: return launch_gemv_R<4>(x_f16, B, packed, m, k, ksplit, part, 0, 1.0f, 0, 0, stream);
-    }
-    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
-}
-
-int glqh_launch_trellis_direct(const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                               int64_t k, float scale, float *out, int64_t out_stride, int accum,
-                               hipStream_t stream) {
-    switch (R) {
-    case 1: return launch_gemv_R<1>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
-    case 2: return launch_gemv_R<2>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
-    case 3: return launch_gemv_R<3>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
-    case 4: return launch_gemv_R<4>(x_f16, B, packed, m, k, 1, out, 1, scale, accum, out_stride, stream);
-    }
-    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
-}
 
 int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, int64_t B, int64_t m,
                               float scale, float *out, int64_t out_stride, int accum,

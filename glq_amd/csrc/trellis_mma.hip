@@ -247,6 +247,173 @@ tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int
                              direct, scale, accum, out_stride);
 }
 
+// ---------------------------------------------------------------------------------
+// Prefill / large batch: 128 tokens x 256 rows per workgroup.
+// grid = (ceil(m/256), ceil(M/128), ksplit).  Each wave owns 64 rows and walks every k-pair
+// of the slot; the 128-token activation tile of PF_CH k-pairs at a time is staged in LDS and
+// shared by the four waves.  Here the matrix cores set the pace, so the two halves of a
+// weight are added first (one fp16 add with the rounding of the reference dequantizer,
+// glq/trellis.py:122-134) and a lane's eight weights of a row group -- columns
+// 2q + {0,1,8,9,16,17,24,25} of the k-pair -- form one A operand: 32 MFMAs per record
+// against eight token tiles.  The B operand of (q, token) is those eight activations, one
+// 16-byte LDS slot.
+// ---------------------------------------------------------------------------------
+constexpr int PF_NT = 8;
+constexpr int PF_CH = 8;
+constexpr int PF_KP_SLOTS = PF_NT * 4 * 17 + 4;                 // 16-byte slots per k-pair (+4: bank skew)
+
+// (a.lo + a.hi, b.lo + b.hi) in fp16
+__device__ __forceinline__ uint32_t pair_sum(uint32_t ha, uint32_t hb) {
+    uint32_t d;
+    asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %0, %2, %2 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1"
+        : "=&v"(d)
+        : "v"(ha), "v"(hb));
+    return d;
+}
+
+// stage tokens [tok0, tok0+128) x k-pairs [c0, c0+n): item = 16 bytes of one token
+// (columns 8h..8h+7), whose dword q goes to dword h of slot (q, token)
+__device__ __forceinline__ void pf_stage(uint32_t *xs, const f16 *__restrict__ x, int M, int k, int tok0,
+                                         int c0, int n) {
+    constexpr int U = 4;
+    const int total = 16 * PF_NT * n * 4;
+    for (int base = 0; base < total; base += U * TR_THREADS) {
+        u32x4 v[U];
+        int dst[U];
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu) {
+            const int idx = min(base + uu * TR_THREADS + (int)threadIdx.x, total - 1);
+            const int h = idx & 3;
+            const int u = (idx >> 2) % n, tk = (idx >> 2) / n;
+            const int tok = tok0 + tk;
+            const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tok, M - 1) * k + 32 * (c0 + u) + 8 * h);
+            v[uu] = tok < M ? ld : u32x4{0u, 0u, 0u, 0u};
+            dst[uu] = (u * PF_KP_SLOTS + (tk >> 4) * (4 * 17) + (tk & 15)) * 4 + h;
+        }
+#pragma unroll
+        for (int uu = 0; uu < U; ++uu) {
+            if (base + uu * TR_THREADS + (int)threadIdx.x < total) {
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) xs[dst[uu] + qq * 17 * 4] = v[uu][qq];
+            }
+        }
+    }
+}
+
+template <int R>
+__global__ void __launch_bounds__(TR_THREADS, 2)
+tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int M, int m, int k,
+                      int S, float *__restrict__ out, int direct, float scale, int accum,
+                      int64_t out_stride) {
+    extern __shared__ u32x4 xs_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const mma_lane a = mma_lane_of<16>(lane);
+    const int nkp = k >> 5;
+    const int mpairs = m >> 5;
+    const int slot = blockIdx.z;
+    const int kp0 = slot * S;
+    const int kp1 = min(kp0 + S, nkp);
+    const int tok0 = blockIdx.y * (16 * PF_NT);
+    const int rowblk = blockIdx.x * TR_WAVES + wave;                // 64-row unit of this wave
+    const bool active = rowblk * 2 < mpairs;                        // uniform over the wave
+    const int mp = min(2 * rowblk + a.hm, mpairs - 1);
+
+    constexpr int REC = 4 * R;
+    const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
+    tr_record<R> cur = {};
+    if (active) cur = tr_load_record<R>(lane_base + (int64_t)kp0 * 32 * REC);
+
+    mma_acc<PF_NT> acc;
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int tt = 0; tt < PF_NT; ++tt) acc.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int c0 = kp0; c0 < kp1; c0 += PF_CH) {
+        const int c1 = min(c0 + PF_CH, kp1);
+        __syncthreads();
+        pf_stage((uint32_t *)xs_lds, x, M, k, tok0, c0, c1 - c0);
+        __syncthreads();
+        if (active) {
+            for (int kp = c0; kp < c1; ++kp) {
+                tr_record<R> nxt = cur;
+                if (kp + 1 < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + 1) * 32 * REC);
+                const u32x4 *xs = xs_lds + (kp - c0) * PF_KP_SLOTS + a.q * 17 + a.tokl;
+                f16x8 bf[PF_NT];
+#pragma unroll
+                for (int tt = 0; tt < PF_NT; ++tt) bf[tt] = __builtin_bit_cast(f16x8, xs[tt * 4 * 17]);
+                uint32_t cont[4];
+                tr_continuation_from<R>(cur, a.next1, a.next2, cont);
+#pragma unroll
+                for (int ms = 0; ms < 2; ++ms) {
+                    uint32_t h0[8], h1[8];                          // k-tiles 0 and 1 of m-tile ms
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        h0[j] = tr_hash(tr_state<R>(cur.c[ms], cont[ms], j));
+                        h1[j] = tr_hash(tr_state<R>(cur.c[2 + ms], cont[2 + ms], j));
+                    }
+#pragma unroll
+                    for (int rh = 0; rh < 2; ++rh) {
+                        const int j0 = 2 * rh;
+                        const f16x8 af = __builtin_bit_cast(
+                            f16x8, u32x4{pair_sum(h0[j0], h0[j0 + 1]), pair_sum(h0[j0 + 4], h0[j0 + 5]),
+                                         pair_sum(h1[j0], h1[j0 + 1]), pair_sum(h1[j0 + 4], h1[j0 + 5])});
+#pragma unroll
+                        for (int tt = 0; tt < PF_NT; ++tt)
+                            acc.v[2 * ms + rh][tt] =
+                                __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf[tt], acc.v[2 * ms + rh][tt], 0, 0, 0);
+                    }
+                }
+                cur = nxt;
+            }
+        }
+    }
+    if (!active) return;
+    // lane holds rows i0 .. i0+3 (consecutive) of token tokl for every (s, tt)
+    const int i0 = 4 * a.q;
+    const int rbase = 64 * rowblk + 32 * (i0 >> 3) + (i0 & 7);
+    const bool vec = (out_stride & 3) == 0;
+#pragma unroll
+    for (int tt = 0; tt < PF_NT; ++tt) {
+        const int tok = tok0 + 16 * tt + a.tokl;
+        if (tok >= M) continue;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int row = rbase + 8 * s;
+            if (row >= m) continue;
+            f32x4 v = acc.v[s][tt];
+            float *o;
+            if (direct) {
+                o = out + (int64_t)tok * out_stride + row;
+                v *= scale;
+                if (accum) {
+                    if (vec) v += *(const f32x4 *)o;
+                    else { v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3]; }
+                }
+            } else {
+                o = out + ((int64_t)slot * M + tok) * m + row;
+            }
+            if (vec || !direct) *(f32x4 *)o = v;
+            else { o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3]; }
+        }
+    }
+}
+
+constexpr int PF_LDS = PF_CH * PF_KP_SLOTS * 16;                  // 70144 bytes
+
+template <int R>
+int launch_prefill(const void *x, int64_t M, const void *packed, int64_t m, int64_t k, int S, int ksplit,
+                   float *out, int direct, float scale, int accum, int64_t out_stride, hipStream_t stream) {
+    dim3 grid((unsigned)((m + 255) / 256), (unsigned)((M + 16 * PF_NT - 1) / (16 * PF_NT)), (unsigned)ksplit);
+    hipLaunchKernelGGL((tr_mma_prefill_kernel<R>), grid, dim3(TR_THREADS), PF_LDS, stream,
+                       (const uint8_t *)packed, (const f16 *)x, (int)M, (int)m, (int)k, S, out, direct, scale,
+                       accum, out_stride);
+    GLQH_LAUNCH_CHECK("trellis prefill launch");
+    return 0;
+}
+
 // LDS per workgroup: a chunk of CH k-pairs (CH % 4 == 0) plus, for partial token tiles, one
 // zeroed block; small enough that the register-limited number of workgroups fits a CU.
 constexpr int MMA_LDS_MAX = 64 * 1024;
@@ -329,6 +496,42 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
     return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
+// Prefill plan: split K only while the grid would leave most CUs idle.
+int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out) {
+    const int64_t nkp = k / 32;
+    const int64_t wgs = ((m + 255) / 256) * ((M + 127) / 128);
+    const int64_t target = (int64_t)glqh_device_cus() * 2;
+    int64_t ks = (target + wgs - 1) / wgs;
+    if (ks > 8) ks = 8;
+    if (ks < 1) ks = 1;
+    int64_t S = (nkp + ks - 1) / ks;
+    S = (S + PF_CH - 1) / PF_CH * PF_CH;
+    *S_out = (int)S;
+    *ksplit_out = (int)((nkp + S - 1) / S);
+    return 1;
+}
+
+int glqh_launch_trellis_prefill(const void *x_f16, int64_t M, const void *packed, int R, int64_t m, int64_t k,
+                                int S, int ksplit, float *out, int direct, float scale, int accum,
+                                int64_t out_stride, hipStream_t stream) {
+    switch (R) {
+    case 1: return launch_prefill<1>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
+    case 2: return launch_prefill<2>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
+    case 3: return launch_prefill<3>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
+    case 4: return launch_prefill<4>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
+    }
+    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}
+
+template <typename K>
+static int pf_set_lds(K kernel) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              PF_LDS),
+                          "trellis prefill attribute");
+}
+
 int glqh_trellis_mma_init(void) {
-    return mma_init_R<1>() || mma_init_R<2>() || mma_init_R<3>() || mma_init_R<4>();
+    return mma_init_R<1>() || mma_init_R<2>() || mma_init_R<3>() || mma_init_R<4>() ||
+           pf_set_lds(tr_mma_prefill_kernel<1>) || pf_set_lds(tr_mma_prefill_kernel<2>) ||
+           pf_set_lds(tr_mma_prefill_kernel<3>) || pf_set_lds(tr_mma_prefill_kernel<4>);
 }

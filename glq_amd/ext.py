@@ -27,8 +27,9 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 # Token counts above these take the dense route: dequantize the weight to fp16 once with
 # the HIP kernel, then one library GEMM (hipBLASLt through torch.matmul), as the reference
 # does above GLQ_TRELLIS_BATCH_MAX (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334).  Below
-# them the weights stay compressed and are re-read once per token group.
-TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "64")))
+# them the weights stay compressed: the trellis kernels decode straight into MFMA operands
+# for any token count, so the trellis threshold is off unless the variable is set.
+TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", str(1 << 30))))
 E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "16")))
 
 

@@ -67,11 +67,16 @@ def test_ops_namespace_runs_the_hip_path():
                        ext.glq_fused_linear_trellis_3inst_cuda(*args))
 
 
+@pytest.mark.parametrize("route", ["mfma", "dense"])
 @pytest.mark.parametrize("B", [65, 200])
-def test_trellis_dense_route_many_tokens(B):
+def test_trellis_many_tokens(B, route, monkeypatch):
+    """More than 64 tokens: the 128-token MFMA tiles over the compressed stream, and the
+    dequantize-then-GEMM route the reference takes (GLQ_TRELLIS_BATCH_MAX)."""
     from glq_amd import ext, hadamard as H
+    if route == "dense":
+        monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 64)
     m, n = 256, 512
-    say("trellis dense", B)
+    say("trellis many tokens", B, route)
     p1, p2 = O.random_packed(m, n, 4, 1), O.random_packed(m, n, 2, 2)
     su, sv = O.rht_signs(m, n, 42)
     bn, bm = O.block_decompose(n), O.block_decompose(m)

@@ -31,24 +31,26 @@ def test_input_rht_pow2(ext, n, inf):
     assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("B", [2, 70])       # few tokens: 1024-point slices; many: whole blocks
 @pytest.mark.parametrize("n,inf,dtype", [(960, 960, torch.float16), (11008, 11008, torch.bfloat16),
-                                         (14336, 14000, torch.bfloat16), (160, 160, torch.float16)])
-def test_input_output_rht_blockdiag(ext, n, inf, dtype):
+                                         (14336, 14000, torch.bfloat16), (160, 160, torch.float16),
+                                         (49152, 49152, torch.float16)])
+def test_input_output_rht_blockdiag(ext, n, inf, dtype, B):
     from glq_amd import hadamard as H
-    say("blockdiag rht", n, inf, dtype)
+    say("blockdiag rht", n, inf, dtype, B)
     blocks = O.block_decompose(n)
-    x = torch.randn(2, inf).to(dtype)
+    x = torch.randn(B, inf).to(dtype)
     rng = np.random.default_rng(n)
     sv = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
-    out = torch.empty(2, n, dtype=torch.float32, device=DEV)
+    out = torch.empty(B, n, dtype=torch.float32, device=DEV)
     ext.glq_input_rht_blockdiag_cuda(x.to(DEV), t(sv), out, inf, n, torch.tensor(blocks),
                                      H.pack_block_meta(blocks).to(DEV))
-    xp = np.zeros((2, n), np.float32)
+    xp = np.zeros((B, n), np.float32)
     xp[:, :inf] = x.float().numpy()
     ref = O.block_diag_fht(xp * sv.astype(np.float32)[None], blocks)
     assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=2e-5)
     # output side: FHT * su, unpad, cast
-    y = torch.empty(2, inf, dtype=dtype, device=DEV)
+    y = torch.empty(B, inf, dtype=dtype, device=DEV)
     ext.glq_output_rht_blockdiag_cuda(out, t(sv), y, inf, n, torch.tensor(blocks),
                                       H.pack_block_meta(blocks).to(DEV))
     yref = (O.block_diag_fht(ref, blocks) * sv.astype(np.float32)[None])[:, :inf]

@@ -115,6 +115,30 @@ def test_matmul_batched_rows_equal_gemv(ext, B):
     assert torch.equal(out, ext.glq_decode_matmul_trellis_3inst_cuda(xt, pt, m, n, 1.0))
 
 
+@pytest.mark.parametrize("m,n,B,K", [(96, 192, 65, 4), (320, 1024, 130, 2), (256, 512, 257, 3),
+                                     (64, 2048, 128, 4)])
+def test_matmul_large_batch_tiles(ext, m, n, B, K):
+    """B > 64 takes the 128-token tiles (one wave per 64 rows, K split only to fill the
+    chip): odd m/32, ragged token tiles, direct and accumulating outputs."""
+    say("matmul tiles", m, n, B, K)
+    p1, p2 = O.random_packed(m, n, K, seed=3), O.random_packed(m, n, 1, seed=4)
+    W1, W2 = O.decode_layer(p1, m, n), O.decode_layer(p2, m, n)
+    x = (np.random.default_rng(B).standard_normal((B, n)) * 0.5).astype(np.float16)
+    xt = t(x)
+    out = ext.glq_decode_matmul_trellis_3inst_cuda(xt, t(p1), m, n, 0.25)
+    ref1 = x.astype(np.float32) @ W1.T * np.float32(0.25)
+    assert out.shape == (B, m) and rel(out, ref1) < 2e-3, rel(out, ref1)
+    assert torch.equal(out, ext.glq_decode_matmul_trellis_3inst_cuda(xt, t(p1), m, n, 0.25))
+    ext.glq_decode_matmul_trellis_3inst_cuda(xt, t(p2), m, n, 0.125, out=out, accum=True)
+    ref = ref1 + x.astype(np.float32) @ W2.T * np.float32(0.125)
+    assert rel(out, ref) < 2e-3, rel(out, ref)
+    # rows agree with the small-batch kernel up to rounding: the tiles add a weight's two
+    # fp16 halves before the multiply (as the dequantizer does), the small-batch kernel after
+    rows = ext.glq_decode_matmul_trellis_3inst_cuda(xt[:3].contiguous(), t(p1), m, n, 0.25)
+    first = ext.glq_decode_matmul_trellis_3inst_cuda(xt, t(p1), m, n, 0.25)[:3]
+    assert rel(first, rows) < 1e-3
+
+
 def _layer_args(art, m, n, dtype):
     from glq_amd import hadamard as H
     bn, bm = art["blocks_n"], art["blocks_m"]

@@ -39,6 +39,68 @@ __device__ __forceinline__ rht_slice rht_get_slice(const glqh_block_meta *meta, 
     return b;
 }
 
+// Split-K partials -> LDS.  Element e of the block is v(e) = sum_stage scale * (sum_k
+// partial), summed in this fixed order (the same order as the stand-alone reduction, so
+// both give the same bits); slice r needs sum_h sign(r,h) v(h*len + i).  The (h, stage, k)
+// terms are walked as one flat sequence so that C terms x U elements of loads are in flight.
+template <int U, int C>
+__device__ __forceinline__ void stage_partials(float *s, const glqh_ysrc &src, const rht_slice &blk,
+                                           int64_t b, int m_pad) {
+    const int len = 1 << blk.log_len;
+    const int ks = src.ksplit, nst = src.nparts;
+    const int total = blk.nsub * nst * ks;
+    const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
+    for (int i0 = threadIdx.x; i0 < len; i0 += U * RHT_THREADS) {
+        float z[U], v[U], acc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) z[u] = v[u] = acc[u] = 0.0f;
+        int h = 0, st = 0, k = 0;                       // position of term t0 (uniform)
+        for (int t0 = 0; t0 < total; t0 += C) {
+            float vals[C][U];
+            int hh = h, ss = st, kk = k;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
+#pragma unroll
+                for (int u = 0; u < U; ++u) vals[c][u] = p[min(i0 + u * RHT_THREADS, len - 1)];
+                if (t0 + c + 1 < total) {               // advance, clamped at the last term
+                    if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                if (t0 + c < total) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) acc[u] += vals[c][u];
+                    if (++k == ks) {
+                        const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
+                                       : st == 2 ? src.scale[2] : src.scale[3];
+#pragma unroll
+                        for (int u = 0; u < U; ++u) { v[u] += sc * acc[u]; acc[u] = 0.0f; }
+                        k = 0;
+                        if (++st == nst) {
+#pragma unroll
+                            for (int u = 0; u < U; ++u) {
+                                const int i = i0 + u * RHT_THREADS;
+                                if (src.copy_out && blk.r == 0 && i < len)
+                                    src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i] = v[u];
+                                z[u] += had_sign(blk.r, h, v[u]);
+                                v[u] = 0.0f;
+                            }
+                            st = 0;
+                            ++h;
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (i0 + u * RHT_THREADS < len) s[lds_pad(i0 + u * RHT_THREADS)] = z[u];
+    }
+    __syncthreads();
+}
+
 // XT / OT: element types (bf16 travels as uint16_t)
 template <typename XT, typename OT>
 __global__ void __launch_bounds__(RHT_THREADS)
@@ -50,11 +112,13 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
     const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const XT *xr = x + (int64_t)blockIdx.y * x_stride;
-    stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, [&](int h, int i) -> float {
+    auto val = [&](int h, int i) -> float {
         const int col = blk.off + (h << blk.log_len) + i;
         const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
         return col < in_features ? v : 0.0f;
-    });
+    };
+    if (blk.nsub == 1 && blk.log_len >= 11) stage_signed_slices<RHT_THREADS, 8, 1>(s, blk.log_len, 1, 0, val);
+    else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
     struct {
         OT *orow;
         float norm;
@@ -75,67 +139,13 @@ output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y,
     const int64_t b = blockIdx.y;
     if constexpr (!PARTS) {
         const float *__restrict__ d = src.direct + b * src.stride + blk.off;
-        stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r,
-                                         [&](int h, int i) -> float { return d[(h << blk.log_len) + i]; });
+        auto val = [&](int h, int i) -> float { return d[(h << blk.log_len) + i]; };
+        if (blk.nsub == 1 && blk.log_len >= 11) stage_signed_slices<RHT_THREADS, 8, 1>(s, blk.log_len, 1, 0, val);
+        else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
     } else {
-        // Element e of the block is v(e) = sum_stage scale * (sum_k partial), summed in this
-        // fixed order (the same order as the stand-alone reduction, so both give the same
-        // bits); slice r needs sum_h sign(r,h) v(h*len + i).  The (h, stage, k) terms are
-        // walked as one flat sequence so that 8 terms x 4 elements of loads are in flight.
-        constexpr int U = 4, C = 8;
-        const int len = 1 << blk.log_len;
-        const int ks = src.ksplit, nst = src.nparts;
-        const int total = blk.nsub * nst * ks;
-        const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
-        for (int i0 = threadIdx.x; i0 < len; i0 += U * RHT_THREADS) {
-            float z[U], v[U], acc[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) z[u] = v[u] = acc[u] = 0.0f;
-            int h = 0, st = 0, k = 0;                       // position of term t0 (uniform)
-            for (int t0 = 0; t0 < total; t0 += C) {
-                float vals[C][U];
-                int hh = h, ss = st, kk = k;
-#pragma unroll
-                for (int c = 0; c < C; ++c) {
-                    const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
-#pragma unroll
-                    for (int u = 0; u < U; ++u) vals[c][u] = p[min(i0 + u * RHT_THREADS, len - 1)];
-                    if (t0 + c + 1 < total) {               // advance, clamped at the last term
-                        if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
-                    }
-                }
-#pragma unroll
-                for (int c = 0; c < C; ++c) {
-                    if (t0 + c < total) {
-#pragma unroll
-                        for (int u = 0; u < U; ++u) acc[u] += vals[c][u];
-                        if (++k == ks) {
-                            const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
-                                           : st == 2 ? src.scale[2] : src.scale[3];
-#pragma unroll
-                            for (int u = 0; u < U; ++u) { v[u] += sc * acc[u]; acc[u] = 0.0f; }
-                            k = 0;
-                            if (++st == nst) {
-#pragma unroll
-                                for (int u = 0; u < U; ++u) {
-                                    const int i = i0 + u * RHT_THREADS;
-                                    if (src.copy_out && blk.r == 0 && i < len)
-                                        src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i] = v[u];
-                                    z[u] += had_sign(blk.r, h, v[u]);
-                                    v[u] = 0.0f;
-                                }
-                                st = 0;
-                                ++h;
-                            }
-                        }
-                    }
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (i0 + u * RHT_THREADS < len) s[lds_pad(i0 + u * RHT_THREADS)] = z[u];
-        }
-        __syncthreads();
+        const int total = blk.nsub * src.nparts * src.ksplit;
+        if (total == 1 && blk.log_len >= 11) stage_partials<8, 1>(s, src, blk, b, m_pad);
+        else stage_partials<4, 8>(s, src, blk, b, m_pad);
     }
     const int base = blk.off + (blk.r << blk.log_len);
     struct {

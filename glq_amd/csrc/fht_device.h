@@ -115,12 +115,12 @@ __device__ __forceinline__ float had_sign(int r, int h, float v) {
 }
 
 // lds[pad(i)] = sum_h sign(r, h) * val(h, i) for i < 2^log_len: slice r of the first
-// factor of H_(nsub*len).  Loads of 8 terms x 4 elements are issued before any of them is
-// used; indices are clamped instead of branched on so that the loads cluster.  Ends with
-// a barrier.
-template <int T, class Val>
+// factor of H_(nsub*len).  Loads of C terms x U elements are issued before any of them is
+// used; indices are clamped instead of branched on so that the loads cluster (callers pick
+// U <= len / T and C <= nsub where they can, clamped loads are wasted issue slots).  Ends
+// with a barrier.
+template <int T, int U = 4, int C = 8, class Val>
 __device__ __forceinline__ void stage_signed_slices(float *lds, int log_len, int nsub, int r, Val val) {
-    constexpr int U = 4, C = 8;
     const int len = 1 << log_len;
     for (int i0 = threadIdx.x; i0 < len; i0 += U * T) {
         float z[U];

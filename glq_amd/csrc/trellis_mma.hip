@@ -259,7 +259,7 @@ tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int
 // 16-byte LDS slot.
 // ---------------------------------------------------------------------------------
 constexpr int PF_NT = 8;
-constexpr int PF_CH = 8;
+constexpr int PF_CH = 4;
 constexpr int PF_KP_SLOTS = PF_NT * 4 * 17 + 4;                 // 16-byte slots per k-pair (+4: bank skew)
 
 // (a.lo + a.hi, b.lo + b.hi) in fp16
@@ -272,33 +272,75 @@ __device__ __forceinline__ uint32_t pair_sum(uint32_t ha, uint32_t hb) {
     return d;
 }
 
-// stage tokens [tok0, tok0+128) x k-pairs [c0, c0+n): item = 16 bytes of one token
-// (columns 8h..8h+7), whose dword q goes to dword h of slot (q, token)
-__device__ __forceinline__ void pf_stage(uint32_t *xs, const f16 *__restrict__ x, int M, int k, int tok0,
-                                         int c0, int n) {
-    constexpr int U = 4;
-    const int total = 16 * PF_NT * n * 4;
-    for (int base = 0; base < total; base += U * TR_THREADS) {
-        u32x4 v[U];
-        int dst[U];
+// Staging of tokens [tok0, tok0+128) x k-pairs [c0, c0+PF_CH) in two halves, so that the
+// global loads of the next chunk are in flight while the current one is multiplied: item =
+// 16 bytes of one token (columns 8h..8h+7 of a k-pair), whose dword q goes to dword h of slot
+// (q, token).  The loads are unconditional (addresses clamped into the matrix); tokens past
+// M and k-pairs past the slot are zeroed or skipped when written.
+constexpr int PF_ITEMS = 16 * PF_NT * PF_CH * 4 / TR_THREADS;   // per thread
+
+struct pf_regs {
+    u32x4 v[PF_ITEMS];
+};
+
+__device__ __forceinline__ pf_regs pf_stage_load(const f16 *__restrict__ x, int M, int k, int tok0, int c0,
+                                                 int kp_last) {
+    pf_regs r;
 #pragma unroll
-        for (int uu = 0; uu < U; ++uu) {
-            const int idx = min(base + uu * TR_THREADS + (int)threadIdx.x, total - 1);
-            const int h = idx & 3;
-            const int u = (idx >> 2) % n, tk = (idx >> 2) / n;
-            const int tok = tok0 + tk;
-            const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tok, M - 1) * k + 32 * (c0 + u) + 8 * h);
-            v[uu] = tok < M ? ld : u32x4{0u, 0u, 0u, 0u};
-            dst[uu] = (u * PF_KP_SLOTS + (tk >> 4) * (4 * 17) + (tk & 15)) * 4 + h;
-        }
+    for (int i = 0; i < PF_ITEMS; ++i) {
+        const int idx = i * TR_THREADS + (int)threadIdx.x;
+        const int h = idx & 3;
+        const int u = (idx >> 2) % PF_CH, tk = (idx >> 2) / PF_CH;
+        r.v[i] = *(const u32x4 *)(x + (int64_t)min(tok0 + tk, M - 1) * k + 32 * min(c0 + u, kp_last) + 8 * h);
+    }
+    return r;
+}
+
+__device__ __forceinline__ void pf_stage_write(uint32_t *xs, const pf_regs r, int M, int tok0, int n) {
 #pragma unroll
-        for (int uu = 0; uu < U; ++uu) {
-            if (base + uu * TR_THREADS + (int)threadIdx.x < total) {
+    for (int i = 0; i < PF_ITEMS; ++i) {
+        const int idx = i * TR_THREADS + (int)threadIdx.x;
+        const int h = idx & 3;
+        const int u = (idx >> 2) % PF_CH, tk = (idx >> 2) / PF_CH;
+        if (u < n) {
+            const u32x4 v = tok0 + tk < M ? r.v[i] : u32x4{0u, 0u, 0u, 0u};
+            const int dst = (u * PF_KP_SLOTS + (tk >> 4) * (4 * 17) + (tk & 15)) * 4 + h;
 #pragma unroll
-                for (int qq = 0; qq < 4; ++qq) xs[dst[uu] + qq * 17 * 4] = v[uu][qq];
-            }
+            for (int qq = 0; qq < 4; ++qq) xs[dst + qq * 17 * 4] = v[qq];
         }
     }
+}
+
+// one record against the eight token tiles of k-pair slot `u` of the staged chunk
+template <int R>
+__device__ __forceinline__ mma_acc<PF_NT> pf_record(const tr_record<R> r, const mma_lane a,
+                                                     const u32x4 *xs, mma_acc<PF_NT> acc) {
+    f16x8 bf[PF_NT];
+#pragma unroll
+    for (int tt = 0; tt < PF_NT; ++tt) bf[tt] = __builtin_bit_cast(f16x8, xs[tt * 4 * 17]);
+    uint32_t cont[4];
+    tr_continuation_from<R>(r, a.next1, a.next2, cont);
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms) {
+        uint32_t h0[8], h1[8];                                      // k-tiles 0 and 1 of m-tile ms
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            h0[j] = tr_hash(tr_state<R>(r.c[ms], cont[ms], j));
+            h1[j] = tr_hash(tr_state<R>(r.c[2 + ms], cont[2 + ms], j));
+        }
+#pragma unroll
+        for (int rh = 0; rh < 2; ++rh) {
+            const int j0 = 2 * rh;
+            const f16x8 af = __builtin_bit_cast(
+                f16x8, u32x4{pair_sum(h0[j0], h0[j0 + 1]), pair_sum(h0[j0 + 4], h0[j0 + 5]),
+                             pair_sum(h1[j0], h1[j0 + 1]), pair_sum(h1[j0 + 4], h1[j0 + 5])});
+#pragma unroll
+            for (int tt = 0; tt < PF_NT; ++tt)
+                acc.v[2 * ms + rh][tt] =
+                    __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf[tt], acc.v[2 * ms + rh][tt], 0, 0, 0);
+        }
+    }
+    return acc;
 }
 
 template <int R>
@@ -315,15 +357,19 @@ tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict_
     const int slot = blockIdx.z;
     const int kp0 = slot * S;
     const int kp1 = min(kp0 + S, nkp);
+    const int last = kp1 - 1;
     const int tok0 = blockIdx.y * (16 * PF_NT);
     const int rowblk = blockIdx.x * TR_WAVES + wave;                // 64-row unit of this wave
     const bool active = rowblk * 2 < mpairs;                        // uniform over the wave
     const int mp = min(2 * rowblk + a.hm, mpairs - 1);
 
+    // The packed stream is requested two records ahead and the next activation chunk one
+    // chunk ahead; every load is unconditional with a clamped address, so the waits the
+    // compiler places count loads exactly.
     constexpr int REC = 4 * R;
     const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
-    tr_record<R> cur = {};
-    if (active) cur = tr_load_record<R>(lane_base + (int64_t)kp0 * 32 * REC);
+    tr_record<R> r0 = tr_load_record<R>(lane_base + (int64_t)kp0 * 32 * REC);
+    tr_record<R> r1 = tr_load_record<R>(lane_base + (int64_t)min(kp0 + 1, last) * 32 * REC);
 
     mma_acc<PF_NT> acc;
 #pragma unroll
@@ -331,77 +377,69 @@ tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict_
 #pragma unroll
         for (int tt = 0; tt < PF_NT; ++tt) acc.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    pf_stage_write((uint32_t *)xs_lds, pf_stage_load(x, M, k, tok0, kp0, last), M, tok0, kp1 - kp0);
+    __syncthreads();
     for (int c0 = kp0; c0 < kp1; c0 += PF_CH) {
-        const int c1 = min(c0 + PF_CH, kp1);
-        __syncthreads();
-        pf_stage((uint32_t *)xs_lds, x, M, k, tok0, c0, c1 - c0);
-        __syncthreads();
-        if (active) {
-            for (int kp = c0; kp < c1; ++kp) {
-                tr_record<R> nxt = cur;
-                if (kp + 1 < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + 1) * 32 * REC);
-                const u32x4 *xs = xs_lds + (kp - c0) * PF_KP_SLOTS + a.q * 17 + a.tokl;
-                f16x8 bf[PF_NT];
+        pf_regs next;
 #pragma unroll
-                for (int tt = 0; tt < PF_NT; ++tt) bf[tt] = __builtin_bit_cast(f16x8, xs[tt * 4 * 17]);
-                uint32_t cont[4];
-                tr_continuation_from<R>(cur, a.next1, a.next2, cont);
-#pragma unroll
-                for (int ms = 0; ms < 2; ++ms) {
-                    uint32_t h0[8], h1[8];                          // k-tiles 0 and 1 of m-tile ms
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        h0[j] = tr_hash(tr_state<R>(cur.c[ms], cont[ms], j));
-                        h1[j] = tr_hash(tr_state<R>(cur.c[2 + ms], cont[2 + ms], j));
-                    }
-#pragma unroll
-                    for (int rh = 0; rh < 2; ++rh) {
-                        const int j0 = 2 * rh;
-                        const f16x8 af = __builtin_bit_cast(
-                            f16x8, u32x4{pair_sum(h0[j0], h0[j0 + 1]), pair_sum(h0[j0 + 4], h0[j0 + 5]),
-                                         pair_sum(h1[j0], h1[j0 + 1]), pair_sum(h1[j0 + 4], h1[j0 + 5])});
-#pragma unroll
-                        for (int tt = 0; tt < PF_NT; ++tt)
-                            acc.v[2 * ms + rh][tt] =
-                                __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf[tt], acc.v[2 * ms + rh][tt], 0, 0, 0);
-                    }
-                }
-                cur = nxt;
-            }
+        for (int i = 0; i < PF_CH; ++i) {
+            const int kp = c0 + i;
+            const tr_record<R> r2 = tr_load_record<R>(lane_base + (int64_t)min(kp + 2, last) * 32 * REC);
+            if (i == 0) next = pf_stage_load(x, M, k, tok0, c0 + PF_CH, last);
+            if (active && kp < kp1)
+                acc = pf_record<R>(r0, a, xs_lds + i * PF_KP_SLOTS + a.q * 17 + a.tokl, acc);
+            r0 = r1;
+            r1 = r2;
         }
+        __syncthreads();                                         // chunk consumed by every wave
+        pf_stage_write((uint32_t *)xs_lds, next, M, tok0, kp1 - (c0 + PF_CH));
+        __syncthreads();
     }
     if (!active) return;
     // lane holds rows i0 .. i0+3 (consecutive) of token tokl for every (s, tt)
     const int i0 = 4 * a.q;
     const int rbase = 64 * rowblk + 32 * (i0 >> 3) + (i0 & 7);
     const bool vec = (out_stride & 3) == 0;
+    if (!direct) {
 #pragma unroll
-    for (int tt = 0; tt < PF_NT; ++tt) {
-        const int tok = tok0 + 16 * tt + a.tokl;
-        if (tok >= M) continue;
+        for (int tt = 0; tt < PF_NT; ++tt) {
+            const int tok = tok0 + 16 * tt + a.tokl;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const int row = rbase + 8 * s;
-            if (row >= m) continue;
-            f32x4 v = acc.v[s][tt];
-            float *o;
-            if (direct) {
-                o = out + (int64_t)tok * out_stride + row;
-                v *= scale;
-                if (accum) {
-                    if (vec) v += *(const f32x4 *)o;
-                    else { v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3]; }
+            for (int s = 0; s < 4; ++s)
+                if (tok < M && rbase + 8 * s < m)
+                    *(f32x4 *)(out + ((int64_t)slot * M + tok) * m + rbase + 8 * s) = acc.v[s][tt];
+        }
+    } else if (vec) {
+#pragma unroll
+        for (int tt = 0; tt < PF_NT; ++tt) {
+            const int tok = tok0 + 16 * tt + a.tokl;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                if (tok < M && rbase + 8 * s < m) {
+                    f32x4 *o = (f32x4 *)(out + (int64_t)tok * out_stride + rbase + 8 * s);
+                    f32x4 v = acc.v[s][tt] * scale;
+                    if (accum) v += *o;
+                    *o = v;
                 }
-            } else {
-                o = out + ((int64_t)slot * M + tok) * m + row;
             }
-            if (vec || !direct) *(f32x4 *)o = v;
-            else { o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3]; }
+        }
+    } else {
+#pragma unroll
+        for (int tt = 0; tt < PF_NT; ++tt) {
+            const int tok = tok0 + 16 * tt + a.tokl;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                if (tok < M && rbase + 8 * s < m) {
+                    float *o = out + (int64_t)tok * out_stride + rbase + 8 * s;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = accum ? o[e] + acc.v[s][tt][e] * scale : acc.v[s][tt][e] * scale;
+                }
+            }
         }
     }
 }
 
-constexpr int PF_LDS = PF_CH * PF_KP_SLOTS * 16;                  // 70144 bytes
+constexpr int PF_LDS = PF_CH * PF_KP_SLOTS * 16;                  // 35072 bytes
 
 template <int R>
 int launch_prefill(const void *x, int64_t M, const void *packed, int64_t m, int64_t k, int S, int ksplit,

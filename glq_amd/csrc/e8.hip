@@ -204,11 +204,19 @@ int launch_e8_NS(const void *x, int64_t B, const void *const q[4], const uint32_
 
 }  // namespace
 
-int glqh_e8_init(void) { return 0; }
+int glqh_e8_mma_init(void);
+int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1);
+int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
+                       int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
+                       hipStream_t stream);
 
-// Shape-only K-split (independent of the token count): batched rows sum like the GEMV.
+int glqh_e8_init(void) { return glqh_e8_mma_init(); }
+
+// K-split of the kernel that will serve the call.
 int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B) {
-    (void)B;
+    // large layers at up to 16 tokens go to the LDS-table kernel, which has its own slots
+    const int mma_ks = glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536);
+    if (mma_ks > 0) return mma_ks;
     const int64_t wgs = (m_pad + E8_ROWS_PER_WG - 1) / E8_ROWS_PER_WG;
     const int64_t target = (int64_t)glqh_device_cus() * 4;
     int64_t ks = (target + wgs - 1) / wgs;
@@ -231,6 +239,8 @@ int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, 
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream) {
+    if (glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536) > 0)
+        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream);
     switch (nstages) {
     case 1: return launch_e8_NS<1>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
     case 2: return launch_e8_NS<2>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);

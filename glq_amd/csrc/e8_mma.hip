@@ -1,0 +1,333 @@
+// E8 shell codebook GEMV / small-batch GEMM on the matrix cores with the table in LDS
+// (gfx950, wave64).
+//
+// One 16-bit index stands for 8 consecutive weights of one row (glq/codebook.py:280-282):
+// exactly the A operand a lane supplies to v_mfma_f32_16x16x32_f16 (row L & 15, k-group
+// L >> 4, eight consecutive k).  A lane reads a 16-byte run of 8 indices of its row, looks
+// each one up, expands the eight 4-bit codes to fp16 and issues one MFMA per index against
+// the 8 activations of the same columns (B operand, 16 bytes per token, from LDS).  Up to
+// 16 tokens share the decode.
+//
+// The lookup is what bounds this codebook: a random 4-byte gather from L2 sustains well
+// under one lane per clock and CU, an LDS gather about twenty times that.  The nibble-packed
+// table is 256 KiB and LDS 160 KiB, but the table is sorted by norm and both the first-stage
+// indices and, more so, the residual-stage indices concentrate on the low-norm shells, so
+// each workgroup keeps the first P entries (a launch parameter, ~120-144 KiB) in LDS and
+// sends only the tail to L2.  Lanes that hit LDS all point their L2 load at entry 0, so the
+// loads stay unconditional (exact wait counts) and coalesce.  Workgroups are persistent
+// (one per CU, 16 waves) so the table prefix is loaded once per CU and launch.
+//
+// Work split: tile = (16*WR rows) x (one K slot); the 16 waves of a workgroup form WR row
+// groups x WK k-parts (WK = 4 for up to 4 tokens, 1 above); k-parts are summed through LDS
+// in a fixed order; every stage keeps its own accumulator and partial sum, combined by the
+// consumer in stage order (glq/quantized_linear.py:1177-1194).
+#include "common.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int EM_WAVES = 16;
+constexpr int EM_THREADS = EM_WAVES * GLQH_WAVE;
+constexpr int EM_STEP_BLKS = 32;               // 8-column blocks a wave covers per step
+
+// eight 4-bit codes (interleaved: nibble p = column 2p, nibble p+4 = column 2p+1) -> 8 fp16.
+// A code c in mantissa bits 0..3 of an fp16 with exponent 2^9 reads 512 + c/2, in bits 4..7
+// it reads 512 + 8c; one fused multiply-add each gives c/2 - 3 exactly.  The upper byte of
+// each half needs one shift first.
+__device__ __forceinline__ uint32_t em_and_or(uint32_t a, uint32_t mask, uint32_t magic) {
+    uint32_t d;                                    // (a & mask) | magic in one VOP3 (magic in a VGPR:
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask), "v"(magic));   // one scalar operand only)
+    return d;
+}
+
+__device__ __forceinline__ f16x8 em_expand(uint32_t word) {
+    const f16x2 one = {(f16)1.0f, (f16)1.0f}, sixteenth = {(f16)0.0625f, (f16)0.0625f};
+    const f16x2 off0 = {(f16)-515.0f, (f16)-515.0f}, off1 = {(f16)-35.0f, (f16)-35.0f};
+    const uint32_t magic = 0x60006000u;
+    const uint32_t hi = word >> 8;
+    const f16x2 p0 = __builtin_bit_cast(f16x2, em_and_or(word, 0x000F000Fu, magic));
+    const f16x2 p1 = __builtin_bit_cast(f16x2, em_and_or(word, 0x00F000F0u, magic));
+    const f16x2 p2 = __builtin_bit_cast(f16x2, em_and_or(hi, 0x000F000Fu, magic));
+    const f16x2 p3 = __builtin_bit_cast(f16x2, em_and_or(hi, 0x00F000F0u, magic));
+    u32x4 r;
+    r[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(p0, one, off0));
+    r[1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(p1, sixteenth, off1));
+    r[2] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(p2, one, off0));
+    r[3] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(p3, sixteenth, off1));
+    return __builtin_bit_cast(f16x8, r);
+}
+
+template <int NS>
+struct em_idx {
+    u32x4 v[NS];                               // 8 indices per stage, two per dword
+};
+
+template <int NS>
+__device__ __forceinline__ em_idx<NS> em_load_idx(const uint16_t *const q[4], int64_t off) {
+    em_idx<NS> r;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) r.v[s] = __builtin_nontemporal_load((const u32x4 *)(q[s] + off));
+    return r;
+}
+
+template <int NS, int TP, int WK>
+__global__ void __launch_bounds__(EM_THREADS)
+e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
+              const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
+              const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n1, uint32_t n2,
+              int t2_is_t1, const f16 *__restrict__ x, int B, int m_pad, int n_pad, int P, int slot_blks,
+              int xs_slots, int ksplit, int ns_total, int s_off, float *__restrict__ part) {
+    constexpr int WR = EM_WAVES / WK;
+    constexpr int ROWS = 16 * WR;
+    extern __shared__ u32x4 lds[];
+    uint32_t *tab = (uint32_t *)lds;                           // P entries
+    u32x4 *xs = lds + P / 4;                                   // xs_slots slots, then 8*TP zero slots
+    const int nblk = n_pad >> 3;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wr = wave / WK, wk = wave % WK;
+    const int i = lane & 15, g = lane >> 4;
+    const bool live = i < TP;                                  // token column of this lane
+    u32x4 *zero_slots = xs + xs_slots;
+
+    const uint16_t *const qs[4] = {q1, q2, q3, q4};
+    const int RB = (m_pad + ROWS - 1) / ROWS;
+    const int ntiles = RB * ksplit;
+    const uint32_t P2 = t2_is_t1 ? (uint32_t)P : 0u;           // a separate stage-2 table stays in L2
+
+    // The wave's steps over all of its workgroup's tiles form one sequence; the index runs
+    // of steps n+1 and n+2 are requested while step n is looked up, across tile boundaries,
+    // and the first two before the table prefix is copied in.
+    const int spt = slot_blks / (WK * EM_STEP_BLKS);           // steps per tile
+    const int my_tiles = (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int nsteps = my_tiles * spt;
+    auto idx_offset = [&](int sidx) -> int64_t {
+        sidx = min(sidx, nsteps - 1);
+        const int tile = blockIdx.x + (sidx / spt) * gridDim.x;
+        const int slot = tile / RB, rb = tile % RB;
+        const int row = rb * ROWS + wr * 16 + i;
+        const int b0 = slot * slot_blks + ((sidx % spt) * WK + wk) * EM_STEP_BLKS;
+        return (int64_t)min(row, m_pad - 1) * nblk + min(b0 + 8 * g, nblk - 8);
+    };
+    em_idx<NS> cur = em_load_idx<NS>(qs, idx_offset(0));
+    em_idx<NS> nx1 = em_load_idx<NS>(qs, idx_offset(1));
+
+    // table prefix -> LDS with every load in flight before the first write
+    {
+        constexpr int U = 10;                                  // 10 * 1024 * 16 bytes = 160 KiB >= P * 4
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = ((const u32x4 *)t1)[min(u * EM_THREADS + (int)threadIdx.x, P / 4 - 1)];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u * EM_THREADS + (int)threadIdx.x < P / 4) lds[u * EM_THREADS + threadIdx.x] = v[u];
+    }
+    for (int j = threadIdx.x; j < 8 * TP; j += EM_THREADS) zero_slots[j] = u32x4{0u, 0u, 0u, 0u};
+
+    const int nblk_r = (nblk + EM_STEP_BLKS - 1) / EM_STEP_BLKS * EM_STEP_BLKS;
+    int sidx = 0;
+    for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int slot = tile / RB, rb = tile % RB;
+        const int sb0 = slot * slot_blks;
+        __syncthreads();                                       // previous tile is done with xs
+        // activations of the slot: one 16-byte slot per (block, token), zero past B and n_pad
+        for (int j0 = 0; j0 < slot_blks * TP; j0 += 4 * EM_THREADS) {
+            u32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = min(j0 + u * EM_THREADS + (int)threadIdx.x, slot_blks * TP - 1);
+                const int tl = j / slot_blks, blk = j % slot_blks;
+                const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tl, B - 1) * n_pad + 8 * min(sb0 + blk, nblk - 1));
+                v[u] = (tl < B && sb0 + blk < nblk) ? ld : u32x4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + u * EM_THREADS + (int)threadIdx.x;
+                if (j < slot_blks * TP) xs[(j % slot_blks) * TP + j / slot_blks] = v[u];
+            }
+        }
+        __syncthreads();
+
+        f32x4 acc[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        for (int st = 0; st < spt; ++st, ++sidx) {
+            const int b0 = sb0 + (st * WK + wk) * EM_STEP_BLKS;  // blocks [b0, b0+32), lane's run b0 + 8g
+            const u32x4 *xl = live ? xs + (b0 - sb0 + 8 * g) * TP + i : zero_slots;
+            // all lookups of the step first: LDS for the prefix, L2 for the tail
+            uint32_t wl[NS][8], wg[NS][8];
+            bool hit[NS][8];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    uint32_t idx = (cur.v[s][t >> 1] >> (16 * (t & 1))) & 0xFFFFu;
+                    const uint32_t *tg = s == 1 ? t2 : t1;
+                    const uint32_t pre = s == 1 ? P2 : (uint32_t)P;
+                    if (s == 1) idx = min(idx, n2 - 1);
+                    // hits read LDS and aim their L2 load at one shared entry; misses the reverse
+                    hit[s][t] = idx < pre;
+                    wg[s][t] = tg[max(idx, pre)];
+                    wl[s][t] = tab[min(idx, (uint32_t)P - 1)];
+                }
+            }
+            // requested after the lookups, so that waiting for those does not wait for this
+            const em_idx<NS> nx2 = em_load_idx<NS>(qs, idx_offset(sidx + 2));
+            if (b0 < nblk_r) {                                 // uniform; past the row the activations are zero
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const f16x8 bf = __builtin_bit_cast(f16x8, xl[t * TP]);
+#pragma unroll
+                    for (int s = 0; s < NS; ++s) {
+                        const f16x8 af = em_expand(hit[s][t] ? wl[s][t] : wg[s][t]);
+                        acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf, acc[s], 0, 0, 0);
+                    }
+                }
+            }
+            cur = nx1;
+            nx1 = nx2;
+        }
+
+        // lane holds rows 4g .. 4g+3 of token i (D layout of the 16x16 MFMA)
+        if constexpr (WK == 1) {
+            if (live && i < B) {
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int orow = rb * ROWS + wr * 16 + 4 * g + r;
+                        if (orow < m_pad) part[(((int64_t)slot * ns_total + s_off + s) * B + i) * m_pad + orow] = acc[s][r];
+                    }
+            }
+        } else {
+            __syncthreads();                                   // xs is free: reuse it for the k-part sums
+            float *red = (float *)xs;                          // [WK][NS][TP][ROWS]
+            if (live) {
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        red[((wk * NS + s) * TP + i) * ROWS + wr * 16 + 4 * g + r] = acc[s][r];
+            }
+            __syncthreads();
+            for (int e = threadIdx.x; e < NS * TP * ROWS; e += EM_THREADS) {
+                const int rl = e % ROWS, tl = (e / ROWS) % TP, s = e / (ROWS * TP);
+                const int orow = rb * ROWS + rl;
+                if (tl >= B || orow >= m_pad) continue;
+                float v = red[e];
+#pragma unroll
+                for (int w = 1; w < WK; ++w) v += red[w * NS * TP * ROWS + e];
+                part[(((int64_t)slot * ns_total + s_off + s) * B + tl) * m_pad + orow] = v;
+            }
+        }
+    }
+}
+
+struct em_plan {
+    int TP, WK, P, slot_blks, xs_slots, ksplit, grid;
+    size_t lds;
+};
+
+constexpr size_t EM_LDS_TOTAL = 160 * 1024;
+
+// 0 when the shape is better served by the plain gather kernel
+int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p) {
+    const int64_t nblk = n_pad / 8;
+    if (B < 1 || B > 16 || nblk < 8 || (nblk & 7) || n1 < 4096) return 0;
+    if (m_pad * n_pad < (int64_t)1 << 22) return 0;             // the table load would dominate
+    p->TP = B == 1 ? 1 : B <= 4 ? 4 : 16;
+    p->WK = p->TP == 16 ? 1 : 4;
+    const int rows = 16 * (EM_WAVES / p->WK);
+    const int64_t RB = (m_pad + rows - 1) / rows;
+    const int unit = p->WK * EM_STEP_BLKS;                      // blocks per workgroup step
+    const int64_t nunits = (nblk + unit - 1) / unit;
+    const int slot_cap_blks = p->TP == 16 ? 128 : 256;          // activations: at most 32 KB of LDS
+    const int cus = glqh_device_cus();
+    int64_t ks = RB >= cus ? 1 : cus / RB;                      // one tile per workgroup where possible
+    if (ks > nunits) ks = nunits;
+    if (ks < 1) ks = 1;
+    int64_t slot_units = (nunits + ks - 1) / ks;
+    if (slot_units * unit > slot_cap_blks) slot_units = slot_cap_blks / unit;
+    if (slot_units < 1) slot_units = 1;
+    p->slot_blks = (int)(slot_units * unit);
+    p->ksplit = (int)((nunits + slot_units - 1) / slot_units);
+    // LDS: activations (or the k-part sums that reuse their space) + 8*TP zero slots + table
+    size_t xbytes = (size_t)p->slot_blks * p->TP * 16;
+    const size_t red = (size_t)p->WK * 4 * p->TP * rows * sizeof(float);
+    if (p->WK > 1 && xbytes < red) xbytes = red;
+    p->xs_slots = (int)(xbytes / 16);
+    const size_t rest = xbytes + (size_t)8 * p->TP * 16;
+    int64_t P = (int64_t)((EM_LDS_TOTAL - rest) / 4) & ~(int64_t)1023;
+    if (P > n1) P = n1 & ~(int64_t)3;
+    p->P = (int)P;
+    p->lds = (size_t)P * 4 + rest;
+    const int64_t ntiles = RB * p->ksplit;
+    p->grid = (int)(ntiles < cus ? ntiles : cus);
+    return 1;
+}
+
+template <int NS, int TP, int WK>
+int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
+              const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad, int ns_total,
+              int s_off, float *part, hipStream_t stream) {
+    hipLaunchKernelGGL((e8_mma_kernel<NS, TP, WK>), dim3((unsigned)p.grid), dim3(EM_THREADS), p.lds, stream,
+                       (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
+                       (const uint16_t *)q[3], t1, t2, (uint32_t)n1, (uint32_t)n2, (int)(t1 == t2 && n1 == n2),
+                       (const f16 *)x, (int)B, (int)m_pad, (int)n_pad, p.P, p.slot_blks, p.xs_slots, p.ksplit,
+                       ns_total, s_off, part);
+    GLQH_LAUNCH_CHECK("e8 mma launch");
+    return 0;
+}
+
+template <int NS>
+int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
+                 const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad, int ns_total,
+                 int s_off, float *part, hipStream_t stream) {
+#define GLQH_EM(TP, WK) em_launch<NS, TP, WK>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, part, stream)
+    if (p.TP == 1) return GLQH_EM(1, 4);
+    if (p.TP == 4) return GLQH_EM(4, 4);
+    return GLQH_EM(16, 1);
+#undef GLQH_EM
+}
+
+template <typename K>
+int em_set_lds(K kernel) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)EM_LDS_TOTAL),
+                          "e8 mma attribute");
+}
+
+template <int NS>
+int em_init_NS() {
+    return em_set_lds(e8_mma_kernel<NS, 1, 4>) || em_set_lds(e8_mma_kernel<NS, 4, 4>) ||
+           em_set_lds(e8_mma_kernel<NS, 16, 1>);
+}
+
+}  // namespace
+
+int glqh_e8_mma_init(void) { return em_init_NS<1>() || em_init_NS<2>(); }
+
+// ksplit of the LDS-table kernel for this call, or 0 when the shape is not eligible
+int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1) {
+    em_plan p;
+    return em_make_plan(m_pad, n_pad, B, n1, &p) ? p.ksplit : 0;
+}
+
+// One launch covers two stages (the register budget of the three-deep pipeline); layers of
+// three and four stages take a second launch for stages 3-4, which index the primary table.
+int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
+                       int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
+                       hipStream_t stream) {
+    em_plan p;
+    if (!em_make_plan(m_pad, n_pad, B, n1, &p)) return glqh_fail("e8 mma: shape not eligible");
+    if (nstages < 1 || nstages > 4) return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
+    if (nstages == 1) return em_launch_NS<1>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, 1, 0, part, stream);
+    if (em_launch_NS<2>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, nstages, 0, part, stream)) return 1;
+    if (nstages == 2) return 0;
+    const void *const q34[4] = {q[2], q[3], q[2], q[3]};
+    if (nstages == 3) return em_launch_NS<1>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 3, 2, part, stream);
+    return em_launch_NS<2>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 4, 2, part, stream);
+}

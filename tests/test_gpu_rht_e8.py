@@ -104,6 +104,48 @@ def test_e8_dequant_matmul_matches_oracle(ext, m, n, stages):
         assert torch.equal(gv, out[1])
 
 
+@pytest.mark.parametrize("m,n,B,stages", [(2048, 2048, 1, 1), (2048, 2048, 3, 2), (2100, 2048, 16, 2),
+                                          (1024, 4160, 1, 4), (4096, 1024, 9, 3), (512, 8192, 4, 2)])
+def test_e8_large_layers_lds_table(ext, m, n, B, stages):
+    """Layers of 4M weights and more at up to 16 tokens: the table prefix sits in LDS, the
+    tail comes from L2, the products run on MFMA.  Half of the indices are drawn from the
+    low shells, half uniformly, and the extremes are planted."""
+    say("e8 large", m, n, B, stages)
+    rng = np.random.default_rng(m + n + B)
+    cb = e8_table_f16()
+    q = []
+    for s in range(4):
+        lo = rng.integers(0, 30000, size=(m, n // 8))
+        hi = rng.integers(0, 65536, size=(m, n // 8))
+        q.append(np.where(rng.random((m, n // 8)) < 0.5, lo, hi).astype(np.uint16).view(np.int16))
+    q[0][0, 0] = 0
+    q[0][0, 1] = -1
+    q[0][m - 1, n // 8 - 1] = -1
+    sc = [0.0, 0.0, 0.0]
+    for s in range(1, stages):
+        sc[s - 1] = [1 / 3.0, 1 / 9.0, 1 / 27.0][s - 1]
+    x = (rng.standard_normal((B, n)) * 0.5).astype(np.float16)
+    W = O.e8_dequant(q[0], q[1], sc[0], q[2], sc[1], q[3], sc[2])
+    ref = x.astype(np.float32) @ W.T * np.float32(0.021)
+    args = (t(q[0]), cb, 0.021, t(q[1]), cb, sc[0], None, t(q[2]), cb, sc[1], t(q[3]), cb, sc[2])
+    out = ext.glq_dequant_matmul_cuda(t(x), *args)
+    assert out.shape == (B, m) and rel(out, ref) < 1e-3, rel(out, ref)
+    assert torch.equal(out, ext.glq_dequant_matmul_cuda(t(x), *args))
+
+
+def test_e8_large_layer_small_secondary_table(ext):
+    rng = np.random.default_rng(5)
+    m, n = 2048, 2048
+    cb = e8_table_f16()
+    cb2 = cb[:256].contiguous()
+    q1 = _rand_idx(rng, m, n // 8)
+    q2 = rng.integers(0, 256, size=(m, n // 8)).astype(np.int16)
+    x = rng.standard_normal((2, n)).astype(np.float16)
+    W = O.e8_dequant(q1, q2, 0.5)
+    out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
+    assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
+
+
 def test_e8_small_secondary_table(ext):
     """3 bpw recipe: the second stage indexes the first 256 rows."""
     rng = np.random.default_rng(0)

@@ -55,6 +55,13 @@ SIGNATURES = {
                 c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_dbl,
                 c_vp, c_i64, c_vp, c_i64, c_vp, c_vp,
                 c_i64, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_sz, c_vp]),
+    # include/glq_decoder_ops.h
+    "glqh_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),
+    "glqh_add_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),
+    "glqh_rope_kv_store_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
+                                        c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
+    "glqh_attn_decode_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_vp]),
+    "glqh_silu_mul_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_vp]),
 }
 
 GLQH_F16, GLQH_BF16, GLQH_F32 = 0, 1, 2

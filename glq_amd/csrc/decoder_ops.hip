@@ -1,0 +1,265 @@
+// Glue kernels of the batch-1 decode loop around the quantized linears (RMSNorm, rotary
+// embedding + KV-cache append, single-query grouped-query attention, SiLU gate).  They keep
+// the end-to-end decode measurement from being dominated by dozens of tiny framework kernels
+// per layer; arithmetic follows the usual Llama-family definitions in fp32 with bf16 storage.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, GLQH_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, GLQH_WAVE));
+    return v;
+}
+
+// out[t] = bf16( bf16(x[t] * rsqrt(mean(x[t]^2) + eps)) * w ), one workgroup per token
+__global__ void __launch_bounds__(256)
+rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ w, uint16_t *__restrict__ out,
+               int H, float eps) {
+    __shared__ float red[4];
+    const uint16_t *xr = x + (int64_t)blockIdx.x * H;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+        const float v = bf16_bits_to_f32(xr[i]);
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float r = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += 256) {
+        const float n = bf16_bits_to_f32(f32_to_bf16_bits(bf16_bits_to_f32(xr[i]) * r));
+        out[(int64_t)blockIdx.x * H + i] = f32_to_bf16_bits(n * bf16_bits_to_f32(w[i]));
+    }
+}
+
+// Rotate q and k (pairs (i, i + D/2), angle row pos[t]) and append k, v to the caches.
+// grid = (T, heads + 2*kv_heads); block = D/2 threads.
+__global__ void rope_kv_store_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ k,
+                                     const uint16_t *__restrict__ v, const int64_t *__restrict__ pos,
+                                     const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t,
+                                     uint16_t *__restrict__ q_out, uint16_t *__restrict__ kc,
+                                     uint16_t *__restrict__ vc, int heads, int kv_heads, int D, int max_len,
+                                     int apply_rope) {
+    const int t = blockIdx.x, h = blockIdx.y, i = threadIdx.x, half = D >> 1;
+    const int64_t p = pos[t];
+    const uint16_t *src;
+    uint16_t *dst;
+    bool rot = apply_rope != 0;
+    if (h < heads) {
+        src = q + ((int64_t)t * heads + h) * D;
+        dst = q_out + ((int64_t)t * heads + h) * D;
+    } else if (h < heads + kv_heads) {
+        src = k + ((int64_t)t * kv_heads + (h - heads)) * D;
+        dst = kc + ((int64_t)(h - heads) * max_len + p) * D;
+    } else {
+        src = v + ((int64_t)t * kv_heads + (h - heads - kv_heads)) * D;
+        dst = vc + ((int64_t)(h - heads - kv_heads) * max_len + p) * D;
+        rot = false;
+    }
+    const float a = bf16_bits_to_f32(src[i]), b = bf16_bits_to_f32(src[i + half]);
+    if (!rot) {
+        dst[i] = src[i];
+        dst[i + half] = src[i + half];
+        return;
+    }
+    const float c0 = bf16_bits_to_f32(cos_t[p * D + i]), s0 = bf16_bits_to_f32(sin_t[p * D + i]);
+    const float c1 = bf16_bits_to_f32(cos_t[p * D + i + half]), s1 = bf16_bits_to_f32(sin_t[p * D + i + half]);
+    dst[i] = f32_to_bf16_bits(a * c0 - b * s0);
+    dst[i + half] = f32_to_bf16_bits(b * c1 + a * s1);
+}
+
+// One query token: out[h] = softmax(q[h] . K[g][0..pos] / sqrt(D)) V[g][0..pos], g = h / (heads/kv_heads).
+// One workgroup of 16 waves per head; D = 128; scores live in LDS (max_len floats).
+// Scores: 8 lanes per key with 16-byte loads (128 keys per pass).  Output: lane = column
+// pair, wave = key group, four rows of V in flight per thread; the 16 partial rows are summed
+// through LDS in wave order.
+constexpr int AT_THREADS = 1024;
+constexpr int AT_WAVES = AT_THREADS / 64;
+
+__global__ void __launch_bounds__(AT_THREADS)
+attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
+                   const uint16_t *__restrict__ vc, const int64_t *__restrict__ pos_ptr,
+                   uint16_t *__restrict__ out, int heads, int kv_heads, int max_len, float scale) {
+    constexpr int D = 128;
+    extern __shared__ float sc[];                  // max_len scores
+    __shared__ float qs[D];
+    __shared__ float red[AT_WAVES];
+    __shared__ float part[AT_WAVES][D];
+    const int h = blockIdx.x, g = h / (heads / kv_heads);
+    const int n = (int)pos_ptr[0] + 1;             // keys 0..pos (the current token is already cached)
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (threadIdx.x < D) qs[threadIdx.x] = bf16_bits_to_f32(q[(int64_t)h * D + threadIdx.x]) * scale;
+    __syncthreads();
+    const uint16_t *K = kc + (int64_t)g * max_len * D;
+    const uint16_t *V = vc + (int64_t)g * max_len * D;
+    const int sub = threadIdx.x & 7;
+    float mx = -3.0e38f;
+    for (int j0 = threadIdx.x >> 3; j0 < n; j0 += AT_THREADS / 8) {
+        const u32x4 k0 = *(const u32x4 *)(K + (int64_t)j0 * D + sub * 8);
+        const u32x4 k1 = *(const u32x4 *)(K + (int64_t)j0 * D + 64 + sub * 8);
+        float s = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            s += qs[sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k0[e] & 0xFFFFu));
+            s += qs[sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k0[e] >> 16));
+            s += qs[64 + sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k1[e] & 0xFFFFu));
+            s += qs[64 + sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k1[e] >> 16));
+        }
+        s += __shfl_xor(s, 1, GLQH_WAVE);
+        s += __shfl_xor(s, 2, GLQH_WAVE);
+        s += __shfl_xor(s, 4, GLQH_WAVE);
+        if (sub == 0) sc[j0] = s;
+        mx = fmaxf(mx, s);
+    }
+    mx = wave_max(mx);
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = red[0];
+#pragma unroll
+    for (int w = 1; w < AT_WAVES; ++w) mx = fmaxf(mx, red[w]);
+    __syncthreads();
+    float sum = 0.0f;
+    for (int j = threadIdx.x; j < n; j += AT_THREADS) {
+        const float e = __expf(sc[j] - mx);
+        sc[j] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int w = 0; w < AT_WAVES; ++w) tot += red[w];
+    // weighted rows of V: wave = key group, lane = columns (2 lane, 2 lane + 1)
+    float a0 = 0.0f, a1 = 0.0f;
+    for (int j0 = wave; j0 < n; j0 += 4 * AT_WAVES) {
+        uint32_t vv[4];
+        float pw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = j0 + u * AT_WAVES;
+            vv[u] = *(const uint32_t *)(V + (int64_t)min(j, n - 1) * D + 2 * lane);
+            pw[u] = j < n ? sc[j] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            a0 += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u] & 0xFFFFu));
+            a1 += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u] >> 16));
+        }
+    }
+    part[wave][2 * lane] = a0;
+    part[wave][2 * lane + 1] = a1;
+    __syncthreads();
+    if (threadIdx.x < D) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int w = 0; w < AT_WAVES; ++w) acc += part[w][threadIdx.x];
+        out[(int64_t)h * D + threadIdx.x] = f32_to_bf16_bits(acc / tot);
+    }
+}
+
+// x_out = bf16(x + delta); h_out = RMSNorm(x_out) * w as in rmsnorm_kernel (one pass, one launch)
+__global__ void __launch_bounds__(256)
+add_rmsnorm_kernel(const uint16_t *__restrict__ x, const uint16_t *__restrict__ delta,
+                   const uint16_t *__restrict__ w, uint16_t *__restrict__ x_out, uint16_t *__restrict__ h_out,
+                   int H, float eps) {
+    __shared__ float red[4];
+    extern __shared__ float row[];                 // H floats
+    const int64_t base = (int64_t)blockIdx.x * H;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+        const uint16_t sb = f32_to_bf16_bits(bf16_bits_to_f32(x[base + i]) + bf16_bits_to_f32(delta[base + i]));
+        x_out[base + i] = sb;
+        const float v = bf16_bits_to_f32(sb);
+        row[i] = v;
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float r = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += 256) {
+        const float nrm = bf16_bits_to_f32(f32_to_bf16_bits(row[i] * r));
+        h_out[base + i] = f32_to_bf16_bits(nrm * bf16_bits_to_f32(w[i]));
+    }
+}
+
+// out = bf16( bf16(silu(g)) * u )
+__global__ void __launch_bounds__(256)
+silu_mul_kernel(const uint16_t *__restrict__ g, const uint16_t *__restrict__ u, uint16_t *__restrict__ out,
+                int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float a = bf16_bits_to_f32(g[i]);
+    const float s = bf16_bits_to_f32(f32_to_bf16_bits(a / (1.0f + __expf(-a))));
+    out[i] = f32_to_bf16_bits(s * bf16_bits_to_f32(u[i]));
+}
+
+}  // namespace
+
+extern "C" int glqh_rmsnorm_bf16(const void *x, const void *w, void *out, int64_t T, int64_t H, double eps,
+                                 void *stream) {
+    GLQH_REQUIRE(x && w && out && T >= 1 && H >= 1, "rmsnorm: bad arguments");
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t *)x, (const uint16_t *)w, (uint16_t *)out, (int)H, (float)eps);
+    GLQH_LAUNCH_CHECK("rmsnorm launch");
+    return 0;
+}
+
+extern "C" int glqh_rope_kv_store_bf16(const void *q, const void *k, const void *v, const int64_t *pos,
+                                       const void *cos_t, const void *sin_t, void *q_out, void *k_cache,
+                                       void *v_cache, int64_t T, int64_t heads, int64_t kv_heads,
+                                       int64_t head_dim, int64_t max_len, int apply_rope, void *stream) {
+    GLQH_REQUIRE(q && k && v && pos && q_out && k_cache && v_cache, "rope: null pointer");
+    GLQH_REQUIRE(head_dim >= 2 && head_dim <= 1024 && (head_dim & 1) == 0, "rope: bad head_dim");
+    GLQH_REQUIRE(!apply_rope || (cos_t && sin_t), "rope: missing angle tables");
+    hipLaunchKernelGGL(rope_kv_store_kernel, dim3((unsigned)T, (unsigned)(heads + 2 * kv_heads)),
+                       dim3((unsigned)(head_dim / 2)), 0, (hipStream_t)stream, (const uint16_t *)q,
+                       (const uint16_t *)k, (const uint16_t *)v, pos, (const uint16_t *)cos_t,
+                       (const uint16_t *)sin_t, (uint16_t *)q_out, (uint16_t *)k_cache, (uint16_t *)v_cache,
+                       (int)heads, (int)kv_heads, (int)head_dim, (int)max_len, apply_rope);
+    GLQH_LAUNCH_CHECK("rope launch");
+    return 0;
+}
+
+extern "C" int glqh_attn_decode_bf16(const void *q, const void *k_cache, const void *v_cache,
+                                     const int64_t *pos, void *out, int64_t heads, int64_t kv_heads,
+                                     int64_t head_dim, int64_t max_len, void *stream) {
+    GLQH_REQUIRE(q && k_cache && v_cache && pos && out, "attention: null pointer");
+    GLQH_REQUIRE(head_dim == 128, "attention: head_dim must be 128, got %lld", (long long)head_dim);
+    GLQH_REQUIRE(kv_heads >= 1 && heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads");
+    const size_t lds = (size_t)max_len * sizeof(float);
+    GLQH_REQUIRE(lds <= 48 * 1024, "attention: cache of %lld positions does not fit the score buffer",
+                 (long long)max_len);
+    hipLaunchKernelGGL(attn_decode_kernel, dim3((unsigned)heads), dim3(AT_THREADS), lds, (hipStream_t)stream,
+                       (const uint16_t *)q, (const uint16_t *)k_cache, (const uint16_t *)v_cache, pos,
+                       (uint16_t *)out, (int)heads, (int)kv_heads, (int)max_len,
+                       1.0f / sqrtf((float)head_dim));
+    GLQH_LAUNCH_CHECK("attention launch");
+    return 0;
+}
+
+extern "C" int glqh_add_rmsnorm_bf16(const void *x, const void *delta, const void *w, void *x_out,
+                                     void *h_out, int64_t T, int64_t H, double eps, void *stream) {
+    GLQH_REQUIRE(x && delta && w && x_out && h_out && T >= 1 && H >= 1 && H <= 12288, "add_rmsnorm: bad arguments");
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)T), dim3(256), (size_t)H * sizeof(float),
+                       (hipStream_t)stream, (const uint16_t *)x, (const uint16_t *)delta, (const uint16_t *)w,
+                       (uint16_t *)x_out, (uint16_t *)h_out, (int)H, (float)eps);
+    GLQH_LAUNCH_CHECK("add_rmsnorm launch");
+    return 0;
+}
+
+extern "C" int glqh_silu_mul_bf16(const void *gate, const void *up, void *out, int64_t n, void *stream) {
+    GLQH_REQUIRE(gate && up && out && n >= 1, "silu_mul: bad arguments");
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint16_t *)gate, (const uint16_t *)up, (uint16_t *)out, n);
+    GLQH_LAUNCH_CHECK("silu_mul launch");
+    return 0;
+}

@@ -1,0 +1,222 @@
+"""A SmolLM3-shaped decoder whose seven linears per layer are trellis-3INST quantized, used
+to measure end-to-end batch-1 decode (the caller of the quantized-linear forward in the
+reference's HF path, glq/hf_integration.py and benchmarks/run_model.py:8).
+
+Random initialisation only: every bit pattern is a valid tail-biting trellis stream, so the
+packed weights are random bits with Wscale = 0.02 * opt_scale (weights of rms 0.02), the
+sign vectors are seeded, norms are ones and the tied bf16 embedding is N(0, 0.02).  The
+architecture follows transformers' SmolLM3Config defaults: grouped-query attention, RMSNorm,
+SiLU-gated MLP, rotary embeddings skipped on every fourth layer, tied lm_head.
+
+The whole decode step (embedding row -> 36 layers -> logits -> argmax -> position + 1) is
+captured once in a HIP graph and replayed per token; position and token live on the device.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+
+from . import _lib, ext, hadamard
+from ._lib import check
+
+
+@dataclass
+class DecoderConfig:
+    hidden: int = 2048
+    layers: int = 36
+    heads: int = 16
+    kv_heads: int = 4
+    head_dim: int = 128
+    ffn: int = 11008
+    vocab: int = 128256
+    rms_eps: float = 1e-6
+    rope_theta: float = 2e6
+    no_rope_interval: int = 4          # every 4th layer skips the rotary embedding
+    bits: int = 4
+
+
+class _Linear:
+    """One quantized linear: the buffers E8RHTLinear registers for a trellis layer."""
+
+    def __init__(self, out_f, in_f, bits, gen, dev):
+        self.m, self.n = out_f, in_f
+        self.packed = torch.randint(-32768, 32768, ((out_f // 16) * (in_f // 16), 16 * bits),
+                                    generator=gen, device=dev, dtype=torch.int16)
+        self.su = (torch.randint(0, 2, (out_f,), generator=gen, device=dev) * 2 - 1).to(torch.float16)
+        self.sv = (torch.randint(0, 2, (in_f,), generator=gen, device=dev) * 2 - 1).to(torch.float16)
+        self.wscale = 0.02 * 0.8933837
+        bn, bm = hadamard.block_decompose(in_f), hadamard.block_decompose(out_f)
+        self.bn, self.bm = torch.tensor(bn, dtype=torch.int64), torch.tensor(bm, dtype=torch.int64)
+        self.bn_meta = hadamard.pack_block_meta(bn).to(dev)
+        self.bm_meta = hadamard.pack_block_meta(bm).to(dev)
+
+    def __call__(self, x):                                   # (B, in) bf16 -> (B, out) bf16
+        return ext.glq_fused_linear_trellis_3inst_cuda(
+            x, self.sv, self.su, self.packed, self.bn, self.bm, self.bn_meta, self.bm_meta,
+            self.wscale, self.n, self.m, self.n, self.m, out_dtype=torch.bfloat16)
+
+    @property
+    def packed_bytes(self):
+        return self.packed.numel() * 2
+
+
+def _rms_norm(x, w, eps):
+    out = torch.empty_like(x)
+    check(_lib.load().glqh_rmsnorm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1],
+                                        float(eps), _stream()))
+    return out
+
+
+def _add_rms_norm(x, delta, w, eps):
+    x_out, h = torch.empty_like(x), torch.empty_like(x)
+    check(_lib.load().glqh_add_rmsnorm_bf16(x.data_ptr(), delta.data_ptr(), w.data_ptr(), x_out.data_ptr(),
+                                            h.data_ptr(), x.shape[0], x.shape[1], float(eps), _stream()))
+    return x_out, h
+
+
+def _rms_norm_torch(x, w, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * w
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _rope(x, cos, sin):                                      # x (T, H, D); cos/sin (T, D)
+    d = x.shape[-1] // 2
+    rot = torch.cat((-x[..., d:], x[..., :d]), dim=-1)
+    return x * cos[:, None, :] + rot * sin[:, None, :]
+
+
+class TrellisDecoder:
+    def __init__(self, cfg: DecoderConfig | None = None, device="cuda:0", seed=0, max_len=1024):
+        self.cfg = cfg = cfg or DecoderConfig()
+        self.dev = dev = torch.device(device)
+        self.max_len = max_len
+        g = torch.Generator(device=dev).manual_seed(seed)
+        H, D = cfg.hidden, cfg.head_dim
+        self.emb = (torch.randn(cfg.vocab, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        self.layers = []
+        for _ in range(cfg.layers):
+            self.layers.append(dict(
+                q=_Linear(cfg.heads * D, H, cfg.bits, g, dev), k=_Linear(cfg.kv_heads * D, H, cfg.bits, g, dev),
+                v=_Linear(cfg.kv_heads * D, H, cfg.bits, g, dev), o=_Linear(H, cfg.heads * D, cfg.bits, g, dev),
+                gate=_Linear(cfg.ffn, H, cfg.bits, g, dev), up=_Linear(cfg.ffn, H, cfg.bits, g, dev),
+                down=_Linear(H, cfg.ffn, cfg.bits, g, dev),
+                ln1=torch.ones(H, dtype=torch.bfloat16, device=dev),
+                ln2=torch.ones(H, dtype=torch.bfloat16, device=dev)))
+        self.ln_f = torch.ones(H, dtype=torch.bfloat16, device=dev)
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
+        ang = torch.arange(max_len, device=dev, dtype=torch.float32)[:, None] * inv[None]
+        ang = torch.cat((ang, ang), dim=-1)
+        self.cos, self.sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+        self.kc = torch.zeros(cfg.layers, cfg.kv_heads, max_len, D, dtype=torch.bfloat16, device=dev)
+        self.vc = torch.zeros_like(self.kc)
+        self.pos = torch.zeros(1, dtype=torch.int64, device=dev)     # next position to write
+        self.tok = torch.zeros(1, dtype=torch.int64, device=dev)     # token to feed next
+        self.arange = torch.arange(max_len, device=dev)
+        self.graph = None
+
+    @property
+    def packed_bytes_per_token(self):
+        return sum(l[k].packed_bytes for l in self.layers for k in ("q", "k", "v", "o", "gate", "up", "down"))
+
+    # ---- one block over T tokens at positions pos (T,) ----------------------------------
+    # The residual stream travels as (x, delta): the pending branch output is added by the
+    # kernel that also computes the next RMSNorm.
+    def _block(self, li, x, delta, pos, mask):
+        cfg, L = self.cfg, self.layers[li]
+        T, D = x.shape[0], cfg.head_dim
+        lib = _lib.load()
+        if delta is None:
+            h = _rms_norm(x, L["ln1"], cfg.rms_eps)
+        else:
+            x, h = _add_rms_norm(x, delta, L["ln1"], cfg.rms_eps)
+        q, k, v = L["q"](h), L["k"](h), L["v"](h)
+        qr = torch.empty_like(q)
+        check(lib.glqh_rope_kv_store_bf16(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), pos.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(),
+            qr.data_ptr(), self.kc[li].data_ptr(), self.vc[li].data_ptr(), T, cfg.heads, cfg.kv_heads, D,
+            self.max_len, int((li + 1) % cfg.no_rope_interval != 0), _stream()))
+        if T == 1 and D == 128:
+            a = torch.empty(1, cfg.heads * D, dtype=torch.bfloat16, device=x.device)
+            check(lib.glqh_attn_decode_bf16(qr.data_ptr(), self.kc[li].data_ptr(), self.vc[li].data_ptr(),
+                                            pos.data_ptr(), a.data_ptr(), cfg.heads, cfg.kv_heads, D,
+                                            self.max_len, _stream()))
+        else:
+            a = F.scaled_dot_product_attention(qr.view(T, cfg.heads, D).transpose(0, 1)[None], self.kc[li][None],
+                                               self.vc[li][None], attn_mask=mask, enable_gqa=True)
+            a = a[0].transpose(0, 1).reshape(T, cfg.heads * D)
+        x, h = _add_rms_norm(x, L["o"](a), L["ln2"], cfg.rms_eps)
+        gate, up = L["gate"](h), L["up"](h)
+        act = torch.empty_like(gate)
+        check(lib.glqh_silu_mul_bf16(gate.data_ptr(), up.data_ptr(), act.data_ptr(), gate.numel(), _stream()))
+        return x, L["down"](act)
+
+    def _forward(self, ids, pos):
+        """ids, pos: (T,) int64 on the device.  Returns the logits of the last token."""
+        T = ids.numel()
+        mask = None
+        if not (T == 1 and self.cfg.head_dim == 128):
+            mask = (self.arange[None, :] <= pos[:, None])[None, None]   # (1,1,T,max_len): causal over the cache
+        x, delta = self.emb.index_select(0, ids), None
+        for li in range(self.cfg.layers):
+            x, delta = self._block(li, x, delta, pos, mask)
+        _, h = _add_rms_norm(x[-1:], delta[-1:], self.ln_f, self.cfg.rms_eps)
+        return torch.matmul(h, self.emb.t()).float()
+
+    def prefill(self, prompt_ids):
+        T = prompt_ids.numel()
+        assert T < self.max_len
+        logits = self._forward(prompt_ids.to(self.dev), self.arange[:T])
+        self.tok.copy_(logits.argmax(-1))
+        self.pos.fill_(T)
+        return logits
+
+    def _step(self):
+        logits = self._forward(self.tok, self.pos)
+        self.tok.copy_(logits.argmax(-1))
+        self.pos.add_(1)
+        return logits
+
+    def capture(self):
+        """Capture the decode step.  State (pos, tok, caches) is restored afterwards."""
+        pos0, tok0 = self.pos.clone(), self.tok.clone()
+        self._step()                                              # eager warm-up outside capture
+        torch.cuda.synchronize()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, stream=s):
+                self._logits = self._step()
+        torch.cuda.current_stream().wait_stream(s)
+        self.pos.copy_(pos0)
+        self.tok.copy_(tok0)
+        torch.cuda.synchronize()
+
+    def generate(self, prompt_ids, n_new, use_graph=True):
+        """Greedy decode.  Returns (tokens (n_new,), prefill seconds, decode seconds)."""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        self.prefill(prompt_ids)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        if use_graph and self.graph is None:
+            self.capture()
+        out = torch.empty(n_new, dtype=torch.int64, device=self.dev)
+        assert int(self.pos.item()) + n_new <= self.max_len
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_new):
+            out[i:i + 1].copy_(self.tok)
+            if use_graph:
+                self.graph.replay()
+            else:
+                self._step()
+        torch.cuda.synchronize()
+        return out, t_prefill, time.perf_counter() - t0

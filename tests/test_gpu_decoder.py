@@ -1,0 +1,97 @@
+"""The SmolLM3-shaped decoder around the quantized linears: cache consistency and graph
+replay on a small configuration (needs an MI355X)."""
+import pytest
+import torch
+
+from tests.gpu_util import DEV, rel, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _small():
+    from glq_amd.decoder import DecoderConfig, TrellisDecoder
+    cfg = DecoderConfig(hidden=256, layers=3, heads=2, kv_heads=1, head_dim=128, ffn=512, vocab=1000,
+                        no_rope_interval=2, bits=4)
+    return TrellisDecoder(cfg, device=DEV, seed=3, max_len=64)
+
+
+def test_decode_step_matches_prefill_of_longer_prompt():
+    say("decoder cache")
+    dec = _small()
+    ids = torch.randint(0, 1000, (20,), generator=torch.Generator().manual_seed(0)).to(DEV)
+    full = dec.prefill(ids)                                   # logits after 20 tokens
+    dec.prefill(ids[:19])
+    dec.tok.copy_(ids[19:20])
+    step = dec._step()                                        # 19 cached + 1 decoded
+    assert rel(step, full.cpu().numpy()) < 3e-2
+    assert int(dec.pos.item()) == 20
+
+
+def test_graph_replay_equals_eager_decode():
+    say("decoder graph")
+    dec = _small()
+    ids = torch.randint(0, 1000, (12,), generator=torch.Generator().manual_seed(1)).to(DEV)
+    eager, _, _ = dec.generate(ids, 10, use_graph=False)
+    graph, _, _ = dec.generate(ids, 10, use_graph=True)
+    again, _, _ = dec.generate(ids, 10, use_graph=True)
+    assert torch.equal(eager, graph) and torch.equal(graph, again)
+
+
+def test_glue_ops_match_torch():
+    """RMSNorm, rotary + cache append, single-query GQA attention and the SiLU gate against
+    plain PyTorch fp32 references."""
+    import torch.nn.functional as F
+    from glq_amd import _lib, decoder as D
+    say("decoder glue ops")
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=DEV).manual_seed(0)
+    T, H, heads, kvh, hd, L = 5, 2048, 16, 4, 128, 96
+    x = torch.randn(T, H, generator=g, device=DEV).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(H, generator=g, device=DEV)).to(torch.bfloat16)
+    assert rel(D._rms_norm(x, w, 1e-6), D._rms_norm_torch(x, w, 1e-6).float().cpu().numpy()) < 4e-3
+
+    q = torch.randn(T, heads, hd, generator=g, device=DEV).to(torch.bfloat16)
+    k = torch.randn(T, kvh, hd, generator=g, device=DEV).to(torch.bfloat16)
+    v = torch.randn(T, kvh, hd, generator=g, device=DEV).to(torch.bfloat16)
+    pos = torch.tensor([7, 3, 11, 0, 90], device=DEV)
+    inv = 1.0 / (2e6 ** (torch.arange(0, hd, 2, device=DEV, dtype=torch.float32) / hd))
+    ang = torch.arange(L, device=DEV, dtype=torch.float32)[:, None] * inv[None]
+    ang = torch.cat((ang, ang), -1)
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+    kc = torch.zeros(kvh, L, hd, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    qo = torch.empty_like(q)
+    _lib.check(lib.glqh_rope_kv_store_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), pos.data_ptr(),
+                                           cos.data_ptr(), sin.data_ptr(), qo.data_ptr(), kc.data_ptr(),
+                                           vc.data_ptr(), T, heads, kvh, hd, L, 1, st))
+    c, s = cos.float()[pos], sin.float()[pos]
+    def rope(t):
+        tf = t.float()
+        rot = torch.cat((-tf[..., hd // 2:], tf[..., :hd // 2]), -1)
+        return tf * c[:, None] + rot * s[:, None]
+    assert rel(qo, rope(q).cpu().numpy()) < 4e-3
+    assert rel(kc[:, pos].transpose(0, 1), rope(k).cpu().numpy()) < 4e-3
+    assert torch.equal(vc[:, pos].transpose(0, 1), v)
+
+    kc = torch.randn(kvh, L, hd, generator=g, device=DEV).to(torch.bfloat16)
+    vc = torch.randn(kvh, L, hd, generator=g, device=DEV).to(torch.bfloat16)
+    q1 = torch.randn(heads, hd, generator=g, device=DEV).to(torch.bfloat16)
+    p1 = torch.tensor([40], device=DEV)
+    out = torch.empty(heads, hd, dtype=torch.bfloat16, device=DEV)
+    _lib.check(lib.glqh_attn_decode_bf16(q1.data_ptr(), kc.data_ptr(), vc.data_ptr(), p1.data_ptr(),
+                                         out.data_ptr(), heads, kvh, hd, L, st))
+    ref = F.scaled_dot_product_attention(q1.float()[None, :, None], kc.float()[None, :, :41],
+                                         vc.float()[None, :, :41], enable_gqa=True)[0, :, 0]
+    assert rel(out, ref.cpu().numpy()) < 5e-3
+
+    d = torch.randn(T, H, generator=g, device=DEV).to(torch.bfloat16)
+    xo, ho = D._add_rms_norm(x, d, w, 1e-6)
+    assert torch.equal(xo, x + d)
+    assert rel(ho, D._rms_norm_torch(x + d, w, 1e-6).float().cpu().numpy()) < 4e-3
+
+    a = torch.randn(3, 11008, generator=g, device=DEV).to(torch.bfloat16)
+    b = torch.randn(3, 11008, generator=g, device=DEV).to(torch.bfloat16)
+    o = torch.empty_like(a)
+    _lib.check(lib.glqh_silu_mul_bf16(a.data_ptr(), b.data_ptr(), o.data_ptr(), a.numel(), st))
+    assert rel(o, (F.silu(a.float()) * b.float()).cpu().numpy()) < 4e-3

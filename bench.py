@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=72)
     ap.add_argument("--layers", type=int, default=36, help="distinct weight sets in the pool")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ungrouped", action="store_true", help="seven separate fused linears per step")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
@@ -121,14 +122,26 @@ def main():
     bytes_step = sum(m * n * K_BITS // 8 for _, m, n in LINEARS)
     log(f"pool: {L} layers x {bytes_step / 1e6:.2f} MB packed = {L * bytes_step / 1e9:.2f} GB")
 
+    def one(lin):
+        return ext.glq_fused_linear_trellis_3inst_cuda(
+            xs[lin["n"]], lin["sv"], lin["su"], lin["packed"], lin["bn"], lin["bm"],
+            lin["bn_meta"], lin["bm_meta"], lin["wscale"], lin["n"], lin["m"], lin["n"],
+            lin["m"], out_dtype=torch.bfloat16)
+
+    def group(lins):
+        a = lins[0]
+        return ext.glq_fused_linear_trellis_3inst_group(
+            xs[a["n"]], [(l["sv"], l["su"], l["packed"], l["wscale"], l["m"], l["m"]) for l in lins],
+            a["bn"], a["bn_meta"], a["n"], a["n"], out_dtype=torch.bfloat16)
+
     def run_step(layer):
-        out = None
-        for lin in layer:
-            out = ext.glq_fused_linear_trellis_3inst_cuda(
-                xs[lin["n"]], lin["sv"], lin["su"], lin["packed"], lin["bn"], lin["bm"],
-                lin["bn_meta"], lin["bm_meta"], lin["wscale"], lin["n"], lin["m"], lin["n"],
-                lin["m"], out_dtype=torch.bfloat16)
-        return out
+        """q/k/v and gate/up read the same activations and go out as one grouped call each,
+        as a merged linear does (glq_vllm/linear_method.py:664-710); o and down on their own."""
+        by = {lin["name"]: lin for lin in layer}
+        if args.ungrouped:
+            return [one(lin) for lin in layer]
+        return [group([by["q"], by["k"], by["v"]]), one(by["o"]), group([by["gate"], by["up"]]),
+                one(by["down"])]
 
     # eager warm-up (also initialises the library outside of graph capture)
     for i in range(min(L, 4)):

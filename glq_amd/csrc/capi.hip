@@ -322,6 +322,85 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                                   blocks_m, n_blocks_m, 0, 0.0f, st);
 }
 
+// ---- grouped trellis linears -------------------------------------------------------
+static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {
+    int64_t total = 0;
+    for (int i = 0; i < n_shards; ++i) total += m_pads[i];
+    return glqh_trellis_fusein_plan(total, n_pad, B, steps, ks);
+}
+
+extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad, int64_t total_m_pad,
+                                                                  int n_shards) {
+    if (B < 1 || B > 4 || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64) return 0;
+    glqh_init();
+    int steps = 0, ks = 0;
+    if (!glqh_trellis_fusein_plan(total_m_pad, n_pad, B, &steps, &ks)) return 0;
+    return (size_t)n_shards * 256 + align256((size_t)ks * B * total_m_pad * sizeof(float));
+}
+
+extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                                     const glqh_trellis_shard *shards, int n_shards,
+                                                     const int64_t *blocks_n, int64_t n_blocks_n,
+                                                     const glqh_block_meta *bn_meta_dev, int64_t in_features,
+                                                     int64_t n_pad, int y_dtype, int64_t y_stride, void *ws,
+                                                     size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x && shards, "trellis group: null pointer");
+    GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis group: %d shards (1..%d)", n_shards,
+                 GLQH_MAX_SHARDS);
+    GLQH_REQUIRE(B >= 1 && B <= 4, "trellis group: B=%lld (the grouped launch serves 1..4 tokens)", (long long)B);
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis group: x must be f16 or bf16");
+    GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad, "trellis group: in_features exceeds n_pad");
+    const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
+    GLQH_REQUIRE(n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n,
+                 "trellis group: input block sizes missing");
+    if (n_blocks_n > 1) {
+        int64_t sum = 0;
+        for (int64_t i = 0; i < n_blocks_n; ++i) {
+            GLQH_REQUIRE(blocks_n[i] > 0 && (blocks_n[i] & (blocks_n[i] - 1)) == 0,
+                         "trellis group: block size %lld is not a power of two", (long long)blocks_n[i]);
+            sum += blocks_n[i];
+        }
+        GLQH_REQUIRE(sum == n_pad, "trellis group: block sizes sum to %lld, expected %lld", (long long)sum,
+                     (long long)n_pad);
+    }
+    int R = 0;
+    int64_t m_pads[GLQH_MAX_SHARDS], outs[GLQH_MAX_SHARDS];
+    const void *packed[GLQH_MAX_SHARDS], *sv[GLQH_MAX_SHARDS], *su[GLQH_MAX_SHARDS];
+    void *ys[GLQH_MAX_SHARDS];
+    float scale[GLQH_MAX_SHARDS];
+    int64_t total = 0;
+    for (int i = 0; i < n_shards; ++i) {
+        const glqh_trellis_shard &sh = shards[i];
+        GLQH_REQUIRE(sh.sv_f16 && sh.su_f16 && sh.packed && sh.y, "trellis group: null pointer in shard %d", i);
+        int Ri;
+        if (tr_bits_from_packed(sh.packed_cols, 0, &Ri) || tr_check_shape(sh.m_pad, n_pad, sh.packed_rows)) return 1;
+        GLQH_REQUIRE(i == 0 || Ri == R, "trellis group: shards of %d and %d bits/weight cannot share a launch", R, Ri);
+        GLQH_REQUIRE(Ri >= 2, "trellis group: the grouped launch serves 2-4 bits/weight");
+        R = Ri;
+        GLQH_REQUIRE(sh.out_features >= 1 && sh.out_features <= sh.m_pad, "trellis group: out_features exceeds m_pad");
+        m_pads[i] = sh.m_pad; outs[i] = sh.out_features;
+        packed[i] = sh.packed; sv[i] = sh.sv_f16; su[i] = sh.su_f16; ys[i] = sh.y;
+        scale[i] = (float)sh.wscale;
+        total += sh.m_pad;
+    }
+    int steps = 0, ks = 0;
+    GLQH_REQUIRE(tr_group_plan(m_pads, n_shards, n_pad, B, &steps, &ks), "trellis group: shape not eligible");
+    const size_t need = align256((size_t)ks * B * total * sizeof(float));
+    GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    float *parts[GLQH_MAX_SHARDS];
+    float *p = (float *)ws;
+    for (int i = 0; i < n_shards; ++i) {
+        parts[i] = p;
+        p += (size_t)ks * B * m_pads[i];
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (glqh_launch_trellis_fusein_group(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B, n_pad,
+                                         in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
+        return 1;
+    return glqh_launch_output_rht_group(parts, su, ys, scale, m_pads, outs, n_shards, y_dtype, y_stride, B, ks, st);
+}
+
 // ---- E8 shell ------------------------------------------------------------------------
 extern "C" int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, uint32_t *packed_out,
                                   int32_t *bad_dev, void *stream) {

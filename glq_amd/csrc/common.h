@@ -15,6 +15,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define GLQH_WAVE 64
+#define GLQH_MAX_GROUP GLQH_MAX_SHARDS      // layers per grouped launch
 #define GLQH_MAX_LDS_BYTES (160 * 1024)
 
 // ---- error reporting (host) -------------------------------------------------
@@ -153,4 +154,14 @@ int glqh_launch_trellis_fusein(const void *packed, int R, const void *x, int x_d
                                int steps, int ksplit, const glqh_block_meta *bn_meta,
                                const int64_t *blocks_host, int n_blocks, float *part,
                                hipStream_t stream);
+int glqh_launch_trellis_fusein_group(const void *const packed[], const void *const sv[], float *const part[],
+                                     const int64_t m[], int n_shards, int R, const void *x, int x_dtype,
+                                     int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int steps,
+                                     int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                                     int n_blocks, hipStream_t stream);
+// one output transform per shard from its split-K partials, all in one launch
+int glqh_launch_output_rht_group(const float *const part[], const void *const su[], void *const y[],
+                                 const float scale[], const int64_t m_pad[], const int64_t out_features[],
+                                 int n_shards, int y_dtype, int64_t y_stride, int64_t B, int ksplit,
+                                 hipStream_t stream);
 int glqh_trellis_init(void);

@@ -129,11 +129,10 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
 }
 
 template <typename YT, bool PARTS>
-__global__ void __launch_bounds__(RHT_THREADS)
-output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
-                  int out_features, int m_pad, const glqh_block_meta *__restrict__ meta,
-                  glqh_meta_args margs, float single_norm, int spb, int log_slice) {
-    extern __shared__ float s[];
+__device__ __forceinline__ void
+output_rht_body(const glqh_ysrc &src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
+                int out_features, int m_pad, const glqh_block_meta *__restrict__ meta,
+                glqh_meta_args margs, float single_norm, int spb, int log_slice, float *s) {
     const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const int64_t b = blockIdx.y;
@@ -161,6 +160,55 @@ output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y,
         }
     } store = {y + b * y_stride, su, base, out_features, blk.norm};
     fht_staged(s, blk.log_len, store);
+}
+
+template <typename YT, bool PARTS>
+__global__ void __launch_bounds__(RHT_THREADS)
+output_rht_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
+                  int out_features, int m_pad, const glqh_block_meta *__restrict__ meta,
+                  glqh_meta_args margs, float single_norm, int spb, int log_slice) {
+    extern __shared__ float s[];
+    output_rht_body<YT, PARTS>(src, su, y, y_stride, out_features, m_pad, meta, margs, single_norm, spb,
+                               log_slice, s);
+}
+
+// The output transforms of several layers in one launch (blockIdx.z = shard), each from its
+// own single-stage split-K partials; block sizes are the canonical decomposition of m_pad.
+struct rht_out_group {
+    const float *part[GLQH_MAX_GROUP];
+    const f16 *su[GLQH_MAX_GROUP];
+    void *y[GLQH_MAX_GROUP];
+    float scale[GLQH_MAX_GROUP];
+    int m_pad[GLQH_MAX_GROUP], out_features[GLQH_MAX_GROUP], nwg[GLQH_MAX_GROUP];
+};
+
+template <typename YT>
+__global__ void __launch_bounds__(RHT_THREADS)
+output_rht_group_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, int spb, int log_slice) {
+    extern __shared__ float s[];
+    const int z = blockIdx.z;
+    const float *part = g.part[0];
+    const f16 *su = g.su[0];
+    void *y = g.y[0];
+    float scale = g.scale[0];
+    int m_pad = g.m_pad[0], out_features = g.out_features[0], nwg = g.nwg[0];
+#pragma unroll
+    for (int i = 1; i < GLQH_MAX_GROUP; ++i)
+        if (i == z) {
+            part = g.part[i]; su = g.su[i]; y = g.y[i]; scale = g.scale[i];
+            m_pad = g.m_pad[i]; out_features = g.out_features[i]; nwg = g.nwg[i];
+        }
+    if ((int)blockIdx.x >= nwg) return;
+    glqh_ysrc src = {};
+    src.part = part;
+    src.part_kstride = (int64_t)B * m_pad;
+    src.ksplit = ksplit;
+    src.scale[0] = scale;
+    src.nparts = 1;
+    glqh_meta_args margs;
+    margs.canon = m_pad;
+    output_rht_body<YT, true>(src, su, (YT *)y, y_stride, out_features, m_pad, nullptr, margs, 0.0f, spb,
+                              log_slice, s);
 }
 
 // Few tokens: 1024-point slices, one workgroup each, so that a single row still spreads
@@ -303,3 +351,46 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
 }
 
 int glqh_rht_init(void) { return 0; }
+
+int glqh_launch_output_rht_group(const float *const part[], const void *const su[], void *const y[],
+                                 const float scale[], const int64_t m_pad[], const int64_t out_features[],
+                                 int n_shards, int y_dtype, int64_t y_stride, int64_t B, int ksplit,
+                                 hipStream_t stream) {
+    GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_GROUP, "output_rht group: 1..%d shards", GLQH_MAX_GROUP);
+    GLQH_REQUIRE(B >= 1 && B <= 65535, "output_rht group: B=%lld out of range", (long long)B);
+    GLQH_REQUIRE(y_dtype == GLQH_F16 || y_dtype == GLQH_BF16 || y_dtype == GLQH_F32, "output_rht group: bad y dtype");
+    const int log_slice = rht_log_slice(B);
+    rht_out_group g = {};
+    int64_t max_bs = 1;
+    int max_nwg = 0;
+    for (int i = 0; i < n_shards; ++i) {                       // largest block = top bit of m_pad
+        int64_t top = 1;
+        while (top * 2 <= m_pad[i]) top *= 2;
+        if (top > max_bs) max_bs = top;
+    }
+    const int spb = rht_slices_per_block(max_bs, log_slice);
+    for (int i = 0; i < GLQH_MAX_GROUP; ++i) {
+        const int j = i < n_shards ? i : 0;
+        GLQH_REQUIRE(part[j] && su[j] && y[j] && m_pad[j] >= 1 && m_pad[j] <= 0x40000000ll &&
+                         out_features[j] >= 1 && out_features[j] <= m_pad[j],
+                     "output_rht group: bad shard %d", j);
+        g.part[i] = part[j];
+        g.su[i] = (const f16 *)su[j];
+        g.y[i] = y[j];
+        g.scale[i] = scale[j];
+        g.m_pad[i] = (int)m_pad[j];
+        g.out_features[i] = (int)out_features[j];
+        g.nwg[i] = __builtin_popcountll((unsigned long long)m_pad[j]) * spb;
+        if (g.nwg[i] > max_nwg) max_nwg = g.nwg[i];
+    }
+    dim3 grid((unsigned)max_nwg, (unsigned)B, (unsigned)n_shards);
+    const size_t lds = rht_lds_bytes(log_slice);
+    if (y_dtype == GLQH_F16)
+        hipLaunchKernelGGL(output_rht_group_kernel<f16>, grid, dim3(RHT_THREADS), lds, stream, g, y_stride, (int)B, ksplit, spb, log_slice);
+    else if (y_dtype == GLQH_BF16)
+        hipLaunchKernelGGL(output_rht_group_kernel<uint16_t>, grid, dim3(RHT_THREADS), lds, stream, g, y_stride, (int)B, ksplit, spb, log_slice);
+    else
+        hipLaunchKernelGGL(output_rht_group_kernel<float>, grid, dim3(RHT_THREADS), lds, stream, g, y_stride, (int)B, ksplit, spb, log_slice);
+    GLQH_LAUNCH_CHECK("output_rht group launch");
+    return 0;
+}

@@ -147,13 +147,11 @@ __device__ __forceinline__ void tr_reduce_to_lds(tr_acc<NB> acc, float (*red)[NB
 // prologue so that the HBM latency overlaps it.
 // ---------------------------------------------------------------------------------
 template <int R, typename XT, int NB>
-__global__ void __launch_bounds__(TR_THREADS)
-tr_gemv_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
-                      const f16 *__restrict__ sv, int B, int m, int k, int in_features, int steps,
-                      const glqh_block_meta *__restrict__ bn_meta, int n_blocks,
-                      glqh_meta_args margs, float *__restrict__ part) {
-    extern __shared__ float smem[];
-    __shared__ float red[TR_WAVES][NB][32];
+__device__ __forceinline__ void
+tr_gemv_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
+                    const f16 *__restrict__ sv, int B, int m, int k, int in_features, int steps,
+                    const glqh_block_meta *__restrict__ bn_meta, int n_blocks,
+                    glqh_meta_args margs, float *__restrict__ part, float *smem, float (*red)[NB][32]) {
     const int Ls = steps << 6;
     float *fbuf = smem;                                         // Ls + Ls/32 floats
     f16 *xh = (f16 *)(smem + Ls + (Ls >> 5) + 32);              // [NB][Ls] fp16
@@ -253,6 +251,49 @@ tr_gemv_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__
         for (int w = 1; w < TR_WAVES; ++w) v += red[w][t][row];
         part[((int64_t)slot * B + t) * m + 32 * mp + row] = v;
     }
+}
+
+template <int R, typename XT, int NB>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_gemv_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
+                      const f16 *__restrict__ sv, int B, int m, int k, int in_features, int steps,
+                      const glqh_block_meta *__restrict__ bn_meta, int n_blocks,
+                      glqh_meta_args margs, float *__restrict__ part) {
+    extern __shared__ float smem[];
+    __shared__ float red[TR_WAVES][NB][32];
+    tr_gemv_fusein_body<R, XT, NB>(packed, x, x_stride, sv, B, m, k, in_features, steps, bn_meta, n_blocks,
+                                   margs, part, smem, red);
+}
+
+// Several layers that read the same activations (fused q/k/v, gate/up:
+// glq_vllm/linear_method.py:664-710) in one launch: blockIdx.z picks the shard, each with
+// its own packed stream, input signs and partial-sum buffer; workgroups past a shard's
+// rows retire.
+struct tr_fusein_group {
+    const uint8_t *packed[GLQH_MAX_GROUP];
+    const f16 *sv[GLQH_MAX_GROUP];
+    float *part[GLQH_MAX_GROUP];
+    int m[GLQH_MAX_GROUP];
+};
+
+template <int R, typename XT, int NB>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_gemv_fusein_group_kernel(tr_fusein_group g, const XT *__restrict__ x, int64_t x_stride, int B, int k,
+                            int in_features, int steps, const glqh_block_meta *__restrict__ bn_meta,
+                            int n_blocks, glqh_meta_args margs) {
+    extern __shared__ float smem[];
+    __shared__ float red[TR_WAVES][NB][32];
+    const int z = blockIdx.z;
+    const uint8_t *packed = g.packed[0];
+    const f16 *sv = g.sv[0];
+    float *part = g.part[0];
+    int m = g.m[0];
+#pragma unroll
+    for (int i = 1; i < GLQH_MAX_GROUP; ++i)
+        if (i == z) { packed = g.packed[i]; sv = g.sv[i]; part = g.part[i]; m = g.m[i]; }
+    if ((int)blockIdx.x * 32 >= m) return;
+    tr_gemv_fusein_body<R, XT, NB>(packed, x, x_stride, sv, B, m, k, in_features, steps, bn_meta, n_blocks,
+                                   margs, part, smem, red);
 }
 
 __global__ void __launch_bounds__(256)
@@ -360,6 +401,53 @@ int glqh_launch_trellis_fusein(const void *packed, int R, const void *x, int x_d
     return glqh_fail("fused-input trellis kernel supports R (bits/weight) 2-4, got %d", R);
 }
 
+template <int R, typename XT, int NB>
+static int launch_fusein_group(const tr_fusein_group &g, int64_t max_m, int n_shards, const void *x,
+                               int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int steps,
+                               int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                               int n_blocks, hipStream_t stream) {
+    glqh_meta_args margs;
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
+    dim3 grid((unsigned)(max_m / 32), (unsigned)ksplit, (unsigned)n_shards);
+    hipLaunchKernelGGL((tr_gemv_fusein_group_kernel<R, XT, NB>), grid, dim3(TR_THREADS),
+                       glqh_trellis_fusein_lds(steps, NB), stream, g, (const XT *)x, x_stride, (int)B, (int)k,
+                       (int)in_features, steps, n_blocks > 1 ? bn_meta : nullptr, n_blocks > 1 ? n_blocks : 1,
+                       margs);
+    GLQH_LAUNCH_CHECK("trellis fused-input group launch");
+    return 0;
+}
+
+int glqh_launch_trellis_fusein_group(const void *const packed[], const void *const sv[], float *const part[],
+                                     const int64_t m[], int n_shards, int R, const void *x, int x_dtype,
+                                     int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int steps,
+                                     int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                                     int n_blocks, hipStream_t stream) {
+    GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_GROUP, "trellis group: 1..%d shards", GLQH_MAX_GROUP);
+    tr_fusein_group g = {};
+    int64_t max_m = 0;
+    for (int i = 0; i < GLQH_MAX_GROUP; ++i) {
+        const int j = i < n_shards ? i : 0;
+        g.packed[i] = (const uint8_t *)packed[j];
+        g.sv[i] = (const f16 *)sv[j];
+        g.part[i] = part[j];
+        g.m[i] = (int)m[j];
+        if (m[j] > max_m) max_m = m[j];
+    }
+#define GLQH_FG(RR, XT, NB) launch_fusein_group<RR, XT, NB>(g, max_m, n_shards, x, x_stride, B, k, in_features, \
+                                                            steps, ksplit, bn_meta, blocks_host, n_blocks, stream)
+#define GLQH_FG_R(RR)                                                                   \
+    (B == 1 ? (x_dtype == GLQH_F16 ? GLQH_FG(RR, f16, 1) : GLQH_FG(RR, uint16_t, 1))     \
+            : (x_dtype == GLQH_F16 ? GLQH_FG(RR, f16, 4) : GLQH_FG(RR, uint16_t, 4)))
+    switch (R) {
+    case 2: return GLQH_FG_R(2);
+    case 3: return GLQH_FG_R(3);
+    case 4: return GLQH_FG_R(4);
+    }
+#undef GLQH_FG_R
+#undef GLQH_FG
+    return glqh_fail("fused-input trellis kernel supports R (bits/weight) 2-4, got %d", R);
+}
+
 template <typename K>
 static int tr_set_max_lds(K kernel, int NB) {
     return glqh_check_hip(hipFuncSetAttribute((const void *)kernel,
@@ -373,7 +461,11 @@ int glqh_trellis_init(void) {
 #define GLQH_ATTR(R) rc = rc || tr_set_max_lds(tr_gemv_fusein_kernel<R, f16, 1>, 1) ||         \
                           tr_set_max_lds(tr_gemv_fusein_kernel<R, uint16_t, 1>, 1) ||          \
                           tr_set_max_lds(tr_gemv_fusein_kernel<R, f16, 4>, 4) ||               \
-                          tr_set_max_lds(tr_gemv_fusein_kernel<R, uint16_t, 4>, 4)
+                          tr_set_max_lds(tr_gemv_fusein_kernel<R, uint16_t, 4>, 4) ||          \
+                          tr_set_max_lds(tr_gemv_fusein_group_kernel<R, f16, 1>, 1) ||         \
+                          tr_set_max_lds(tr_gemv_fusein_group_kernel<R, uint16_t, 1>, 1) ||    \
+                          tr_set_max_lds(tr_gemv_fusein_group_kernel<R, f16, 4>, 4) ||         \
+                          tr_set_max_lds(tr_gemv_fusein_group_kernel<R, uint16_t, 4>, 4)
     GLQH_ATTR(2);
     GLQH_ATTR(3);
     GLQH_ATTR(4);

@@ -63,6 +63,14 @@ class _Linear:
         return self.packed.numel() * 2
 
 
+def _group(x, lins):
+    """Layers that read the same activations, two launches for all of them."""
+    a = lins[0]
+    return ext.glq_fused_linear_trellis_3inst_group(
+        x, [(l.sv, l.su, l.packed, l.wscale, l.m, l.m) for l in lins], a.bn, a.bn_meta, a.n, a.n,
+        out_dtype=torch.bfloat16)
+
+
 def _rms_norm(x, w, eps):
     out = torch.empty_like(x)
     check(_lib.load().glqh_rmsnorm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1],
@@ -136,7 +144,14 @@ class TrellisDecoder:
             h = _rms_norm(x, L["ln1"], cfg.rms_eps)
         else:
             x, h = _add_rms_norm(x, delta, L["ln1"], cfg.rms_eps)
-        q, k, v = L["q"](h), L["k"](h), L["v"](h)
+        if T <= 4:
+            qkv = _group(h, (L["q"], L["k"], L["v"]))
+            nq, nk = L["q"].m, L["k"].m
+            q, k, v = qkv[:, :nq], qkv[:, nq:nq + nk], qkv[:, nq + nk:]
+            if T > 1:
+                q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        else:
+            q, k, v = L["q"](h), L["k"](h), L["v"](h)
         qr = torch.empty_like(q)
         check(lib.glqh_rope_kv_store_bf16(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), pos.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(),
@@ -152,9 +167,13 @@ class TrellisDecoder:
                                                self.vc[li][None], attn_mask=mask, enable_gqa=True)
             a = a[0].transpose(0, 1).reshape(T, cfg.heads * D)
         x, h = _add_rms_norm(x, L["o"](a), L["ln2"], cfg.rms_eps)
-        gate, up = L["gate"](h), L["up"](h)
-        act = torch.empty_like(gate)
-        check(lib.glqh_silu_mul_bf16(gate.data_ptr(), up.data_ptr(), act.data_ptr(), gate.numel(), _stream()))
+        if T == 1:
+            gu = _group(h, (L["gate"], L["up"]))
+            gate, up = gu[:, :cfg.ffn], gu[:, cfg.ffn:]               # one row: both halves contiguous
+        else:
+            gate, up = L["gate"](h), L["up"](h)
+        act = torch.empty(T, cfg.ffn, dtype=torch.bfloat16, device=x.device)
+        check(lib.glqh_silu_mul_bf16(gate.data_ptr(), up.data_ptr(), act.data_ptr(), act.numel(), _stream()))
         return x, L["down"](act)
 
     def _forward(self, ids, pos):

@@ -292,6 +292,52 @@ def glq_fused_linear_trellis_3inst_rvq2_cuda(x, sv, su, trellis_packed, trellis_
                           out_features, n_pad, m_pad, None, None, out_dtype)
 
 
+class _TrellisShard(C.Structure):
+    _fields_ = [("sv_f16", C.c_void_p), ("su_f16", C.c_void_p), ("packed", C.c_void_p),
+                ("packed_rows", C.c_int64), ("packed_cols", C.c_int64), ("wscale", C.c_double),
+                ("out_features", C.c_int64), ("m_pad", C.c_int64), ("y", C.c_void_p)]
+
+
+def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_features, n_pad,
+                                         out_dtype=None):
+    """Several separately quantized trellis layers on the same x (fused q/k/v, gate/up) with
+    one decode launch and one output-transform launch: the per-shard loop of the reference's
+    vLLM linear method (glq_vllm/linear_method.py:664-710) as a single call.
+
+    shards: sequence of (sv, su, trellis_packed, wscale, out_features, m_pad).  Returns one
+    (B, sum(out_features)) tensor, shard s in columns [off_s, off_s + out_features_s).
+    Needs 1..4 tokens, single-stage layers of one rate and block_decompose block sizes; raises
+    RuntimeError otherwise (callers then use the per-layer op)."""
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    B = x.shape[0]
+    dt = out_dtype or torch.float16
+    total_out = sum(int(s[4]) for s in shards)
+    total_m = sum(int(s[5]) for s in shards)
+    y = torch.empty((B, total_out), dtype=dt, device=x.device)
+    arr = (_TrellisShard * len(shards))()
+    off = 0
+    esz = y.element_size()
+    for i, (sv, su, packed, wscale, out_f, m_pad) in enumerate(shards):
+        _chk(sv, "sv", torch.float16)
+        _chk(su, "su", torch.float16)
+        _chk(packed, "trellis_packed", torch.int16)
+        if packed.dim() != 2:
+            raise RuntimeError("trellis_packed must be 2-D [(m/16)*(k/16), 16*R]")
+        arr[i] = _TrellisShard(_p(sv), _p(su), _p(packed), packed.shape[0], packed.shape[1], float(wscale),
+                               int(out_f), int(m_pad), y.data_ptr() + off * esz)
+        off += int(out_f)
+    bn, nbn = _host_i64(blocks_n)
+    with torch.cuda.device(x.device):
+        nb = lib.glqh_fused_linear_trellis_group_workspace_bytes(B, int(n_pad), total_m, len(shards))
+        ws = _ws(max(nb, 256), x.device)
+        check(lib.glqh_fused_linear_trellis_3inst_group(
+            _p(x), _DT[x.dtype], x.shape[1], B, C.addressof(arr), len(shards), bn, nbn,
+            _meta_ptr(blocks_n_meta) if nbn > 1 else None, int(in_features), int(n_pad), _DT[dt],
+            total_out, _p(ws), ws.numel(), _stream()))
+    return y
+
+
 def _yrht_slice(y_rht_out, col, m_pad):
     _chk(y_rht_out, "y_rht_out", torch.float32)
     if y_rht_out.dim() != 2 or int(col) < 0 or int(col) + int(m_pad) > y_rht_out.shape[1]:

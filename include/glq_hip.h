@@ -134,6 +134,40 @@ int glqh_fused_linear_trellis_3inst(const void *x, int x_dtype, int64_t x_stride
                                     float *y_rht_out, int64_t y_rht_stride,
                                     void *ws, size_t ws_bytes, void *stream);
 
+/* ---- several trellis layers on the same activations, two launches ------------- */
+
+#define GLQH_MAX_SHARDS 4
+
+typedef struct {
+    const void *sv_f16;          /* (n_pad) input signs of this layer */
+    const void *su_f16;          /* (m_pad) output signs */
+    const void *packed;          /* ((m_pad/16)(n_pad/16), 16R) int16 */
+    int64_t packed_rows, packed_cols;
+    double wscale;
+    int64_t out_features, m_pad; /* m_pad's block sizes are block_decompose(m_pad) */
+    void *y;                     /* this layer's first output element, row stride y_stride */
+} glqh_trellis_shard;
+
+size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad, int64_t total_m_pad,
+                                                       int n_shards);
+
+/* Separately quantized layers that consume the same x (fused q/k/v, gate/up of a merged
+ * linear): one decode launch and one output-transform launch for all of them instead of
+ * two or three per layer.  Replaces the per-shard loop of the vLLM linear method
+ * (glq_vllm/linear_method.py:664-710: fused_linear_trellis_3inst_yrht per shard, then
+ * output_rht_shards; glq/csrc/glq_trellis.cu:1373-1397, glq/csrc/glq_cuda.cu:2882-2916) and
+ * gives, per shard, the result of glqh_fused_linear_trellis_3inst on that shard up to the
+ * rounding of a different K split.  Single-stage layers of one rate R, at most 4 tokens,
+ * canonical (block_decompose) output block sizes; anything else is refused and the caller
+ * falls back to per-layer calls. */
+int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                          const glqh_trellis_shard *shards, int n_shards,
+                                          const int64_t *blocks_n, int64_t n_blocks_n,
+                                          const glqh_block_meta *bn_meta_dev,
+                                          int64_t in_features, int64_t n_pad,
+                                          int y_dtype, int64_t y_stride,
+                                          void *ws, size_t ws_bytes, void *stream);
+
 /* ---- E8 shell codebook ---------------------------------------------------- */
 
 /* (n_entries, 8) fp16 table -> n_entries uint32, nibble i = round(2 v_i) + 6

@@ -229,6 +229,40 @@ def test_fused_linear_smollm3_shapes(ext, m, n):
     assert rel(y2, y.float() * 2) < 1e-3
 
 
+@pytest.mark.parametrize("outs,n,B,dtype", [((2048, 512, 512), 2048, 1, torch.bfloat16),
+                                            ((11008, 11008), 2048, 1, torch.bfloat16),
+                                            ((96, 320, 64, 2048), 960, 3, torch.float16)])
+def test_grouped_layers_match_per_layer_calls(ext, outs, n, B, dtype):
+    """Fused q/k/v and gate/up: several separately quantized layers on one x in two launches
+    equal the per-layer fused linears up to the rounding of a different K split."""
+    from glq_amd import hadamard as H
+    say("group", outs, n, B)
+    bn = O.block_decompose(n)
+    bnt, bnm = torch.tensor(bn), H.pack_block_meta(bn).to(DEV)
+    rng = np.random.default_rng(len(outs))
+    x = torch.from_numpy(rng.standard_normal((B, n)).astype(np.float32)).to(dtype).to(DEV)
+    shards, singles = [], []
+    for i, m in enumerate(outs):
+        p = t(O.random_packed(m, n, 4, seed=10 + i))
+        su, sv = O.rht_signs(m, n, 100 + i)
+        su, sv = t(su.astype(np.float16)), t(sv.astype(np.float16))
+        wscale = 0.02 + 0.001 * i
+        bm = O.block_decompose(m)
+        shards.append((sv, su, p, wscale, m, m))
+        singles.append(ext.glq_fused_linear_trellis_3inst_cuda(
+            x, sv, su, p, bnt, torch.tensor(bm), bnm, H.pack_block_meta(bm).to(DEV), wscale, n, m, n, m,
+            out_dtype=dtype))
+    y = ext.glq_fused_linear_trellis_3inst_group(x, shards, bnt, bnm, n, n, out_dtype=dtype)
+    assert y.shape == (B, sum(outs)) and y.dtype == dtype
+    off = 0
+    for m, ref in zip(outs, singles):
+        assert rel(y[:, off:off + m], ref.float().cpu().numpy()) < 4e-3, (m, rel(y[:, off:off + m], ref.float().cpu().numpy()))
+        off += m
+    assert torch.equal(y, ext.glq_fused_linear_trellis_3inst_group(x, shards, bnt, bnm, n, n, out_dtype=dtype))
+    with pytest.raises(RuntimeError, match="1..4 tokens"):
+        ext.glq_fused_linear_trellis_3inst_group(x[:1].repeat(5, 1), shards, bnt, bnm, n, n, out_dtype=dtype)
+
+
 def test_yrht_shards_equal_sequential(ext):
     """Fused q/k/v: three shards write their RHT-domain rows into one buffer and one
     shard-batched output transform finishes them; equals the per-shard fused op."""

@@ -94,6 +94,73 @@ def cpu_baseline(n_calls=10):
                        f"multi-threaded BLAS for the matmul, single-threaded butterflies")}
 
 
+def _graph_time(torch, fn, n_inner, reps=10):
+    """us per inner call of fn(), replayed from a HIP graph between HIP events."""
+    fn()
+    torch.cuda.synchronize()
+    st = torch.cuda.Stream()
+    st.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(st):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            keep = fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(reps):
+            g.replay()
+        e1.record(st)
+        e1.synchronize()
+    del keep
+    return e0.elapsed_time(e1) * 1e3 / (reps * n_inner)
+
+
+def extras(torch, ext, dev):
+    """Side measurements of the other BASELINE configs (bounded, a few seconds): whole-model
+    batch-1 decode tok/s (config 5), large-layer GEMV rates where the kernels are not launch
+    bound, and the prefill tiles (config 4 shape)."""
+    out = {}
+    try:
+        from glq_amd.decoder import TrellisDecoder
+        dec = TrellisDecoder(max_len=1024)
+        ids = torch.randint(0, 128256, (512,), generator=torch.Generator().manual_seed(0))
+        dec.generate(ids, 8)                                  # warm-up + graph capture
+        _, t_prefill, t_decode = dec.generate(ids, 256)
+        out["decode_tok_s_3b_shape"] = round(256 / t_decode, 1)
+        out["decode_ms_per_token"] = round(t_decode / 256 * 1e3, 3)
+        out["prefill_512_ms"] = round(t_prefill * 1e3, 2)
+        out["decoder"] = ("36 layers, hidden 2048, 16/4 heads x 128, FFN 11008, vocab 128256, all 7 linears "
+                          "trellis 4 bpw (random bits), 512-token prompt then 256 greedy tokens, decode step "
+                          "replayed from one HIP graph")
+        del dec
+        torch.cuda.empty_cache()
+    except Exception as e:                                    # report, never hide
+        out["decoder_error"] = f"{type(e).__name__}: {e}"
+    try:
+        m = n = 16384
+        packs = [torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
+                 for _ in range(4)]
+        part = torch.empty(64 * m, dtype=torch.float32, device=dev)
+        for B in (1, 16):
+            xh = torch.randn(B, n, device=dev).to(torch.float16)
+            pb = torch.empty(64 * B * m, dtype=torch.float32, device=dev)
+            us = _graph_time(torch, lambda: [ext.trellis_gemv_partials(xh, p, m, n, pb) for p in packs], len(packs))
+            out[f"trellis_gemv_16384x16384_B{B}_GBs"] = round(m * n / 2 / us / 1e3, 1)
+        del packs, part
+        m, n, M = 14336, 4096, 4096
+        p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
+        xh = torch.randn(M, n, device=dev).to(torch.float16)
+        o = torch.empty(M, m, dtype=torch.float32, device=dev)
+        us = _graph_time(torch, lambda: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o), 1, reps=5)
+        out["trellis_prefill_14336x4096_M4096_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        del p, xh, o
+        torch.cuda.empty_cache()
+    except Exception as e:
+        out["large_layer_error"] = f"{type(e).__name__}: {e}"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,6 +169,10 @@ def main():
     ap.add_argument("--layers", type=int, default=36, help="distinct weight sets in the pool")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ungrouped", action="store_true", help="seven separate fused linears per step")
+    ap.add_argument("--no-extras", action="store_true", help="skip the decoder / large-layer side measurements")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch a plain 256 MiB read + 256 MiB write elementwise kernel three times "
+                         "(calibration of the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
@@ -128,20 +199,23 @@ def main():
             lin["bn_meta"], lin["bm_meta"], lin["wscale"], lin["n"], lin["m"], lin["n"],
             lin["m"], out_dtype=torch.bfloat16)
 
-    def group(lins):
-        a = lins[0]
-        return ext.glq_fused_linear_trellis_3inst_group(
-            xs[a["n"]], [(l["sv"], l["su"], l["packed"], l["wscale"], l["m"], l["m"]) for l in lins],
-            a["bn"], a["bn_meta"], a["n"], a["n"], out_dtype=torch.bfloat16)
+    GROUPS = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
 
-    def run_step(layer):
+    def run_step(layer, decode_only=False):
         """q/k/v and gate/up read the same activations and go out as one grouped call each,
-        as a merged linear does (glq_vllm/linear_method.py:664-710); o and down on their own."""
+        as a merged linear does (glq_vllm/linear_method.py:664-710); o and down are groups of
+        one.  Every call is one decode launch plus one output-transform launch."""
         by = {lin["name"]: lin for lin in layer}
-        if args.ungrouped:
+        if args.ungrouped and not decode_only:
             return [one(lin) for lin in layer]
-        return [group([by["q"], by["k"], by["v"]]), one(by["o"]), group([by["gate"], by["up"]]),
-                one(by["down"])]
+        outs = []
+        for names in GROUPS:
+            lins = [by[nm] for nm in names]
+            a = lins[0]
+            outs.append(ext.glq_fused_linear_trellis_3inst_group(
+                xs[a["n"]], [(l["sv"], l["su"], l["packed"], l["wscale"], l["m"], l["m"]) for l in lins],
+                a["bn"], a["bn_meta"], a["n"], a["n"], out_dtype=torch.bfloat16, decode_only=decode_only))
+        return outs
 
     # eager warm-up (also initialises the library outside of graph capture)
     for i in range(min(L, 4)):
@@ -182,18 +256,16 @@ def main():
     value = bytes_step / (dt / K) / 1e9
     log(f"timed {K} steps: {ms_per_step * 1e3:.1f} us/step, {value:.1f} GB/s packed weights")
 
-    # ---- roofline leg: the decode GEMV kernel alone, HIP events on its own stream -------
+    # ---- roofline leg: the decode launches alone, HIP events on their own stream ---------
+    # The same grouped calls as the timed steps, stopped after the decode kernel (input
+    # transform + packed-stream GEMV into split-K partials), over the whole pool.
     with torch.cuda.stream(stream):
-        xr = {n: torch.randn(1, n, device=dev).to(torch.float16) for _, _, n in LINEARS}
-        part = torch.empty(32 * 11008, dtype=torch.float32, device=dev)
-        for lin in pool[0]:
-            ext.trellis_gemv_partials(xr[lin["n"]], lin["packed"], lin["m"], lin["n"], part)
+        run_step(pool[0], decode_only=True)
         torch.cuda.synchronize()
         gk = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gk, stream=stream):
             for layer in pool:
-                for lin in layer:
-                    ext.trellis_gemv_partials(xr[lin["n"]], lin["packed"], lin["m"], lin["n"], part)
+                run_step(layer, decode_only=True)
         gk.replay()
         torch.cuda.synchronize()
         reps = 10
@@ -203,26 +275,39 @@ def main():
             gk.replay()
         e1.record(stream)
         e1.synchronize()
-        n_launch = reps * L * len(LINEARS)
+        n_launch = reps * L * len(GROUPS)
         avg_us = e0.elapsed_time(e1) * 1e3 / n_launch
-    bytes_launch = bytes_step / len(LINEARS)
+    bytes_launch = bytes_step / len(GROUPS)
     achieved = bytes_launch / (avg_us * 1e-6) / 1e9
+    # HBM bytes per launch from the committed counter summary (FETCH_SIZE / WRITE_SIZE runs)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_tr_gemv_fusein_group_smollm3_4bpw_batch1.txt")
     if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("tr_gemv_bytes_per_launch")
-        except Exception:
-            traffic = None
+        import re
+        mt = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(tpath).read(), re.M)
+        traffic = int(mt.group(1)) if mt else None
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "kernel": "tr_gemv_kernel<4,1>", "avg_launch_us": round(avg_us, 3),
+                "kernel": "tr_gemv_fusein_group_kernel<4,bf16,1>", "avg_launch_us": round(avg_us, 3),
                 "bytes_per_launch": int(bytes_launch),
-                "method": (f"{n_launch} back-to-back launches of the decode GEMV alone (the 7 layer "
-                           f"shapes x {L} distinct weight sets) replayed from a HIP graph between two "
-                           f"HIP events on the launch stream; bytes = packed weights m*n*4/8")}
-    log(f"decode GEMV alone: {avg_us:.2f} us/launch avg, {achieved:.0f} GB/s "
+                "method": (f"{n_launch} back-to-back decode launches (the 4 grouped calls of a step: q/k/v, o, "
+                           f"gate/up, down; x {L} distinct weight sets), stopped before the output "
+                           f"transform, replayed from a HIP graph between two HIP events on the launch "
+                           f"stream; bytes = packed weights of the step / 4 launches")}
+    log(f"decode launches alone: {avg_us:.2f} us/launch avg, {achieved:.0f} GB/s "
         f"({100 * achieved / HBM_PEAK_GBS:.1f}% of HBM peak)")
+
+    if args.copy_probe:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)                      # 268435456 B read, 268435456 B written
+        torch.cuda.synchronize()
+        del src, dst
+
+    extra = {}
+    if not args.no_extras:
+        extra = extras(torch, ext, dev)
 
     result = {
         "metric": "4bpw GEMV effective HBM GB/s (% of peak); batch-1 decode tok/s, 3B shape",
@@ -232,11 +317,13 @@ def main():
         "data": "synthetic (random code bits, seeded signs, N(0,1) bf16 activations)",
         "config": {"workload": "configs[1]: trellis-3INST 4 bpw linear set, SmolLM3-3B shapes "
                                "(q/o 2048x2048, k/v 2048x512, gate/up 2048x11008, down 11008x2048), "
-                               "batch-1 fused linear (input RHT + GEMV + output RHT) per layer",
+                               "batch-1 fused linear (input RHT + GEMV + output RHT) per layer; q/k/v and "
+                               "gate/up issued as grouped calls (2 launches per group)",
                    "step": "7 linears of one decoder layer", "packed_bytes_per_step": bytes_step,
                    "distinct_layers": L, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
                    "linear_only_tok_s_36_layers": round(1e3 / (ms_per_step * 36), 1)},
         "roofline": roofline,
+        "extra": extra,
     }
     if not args.no_cpu_baseline:
         log("timing the CPU baseline (oracle port of the reference CPU path) ...")

@@ -372,7 +372,9 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
     int64_t total = 0;
     for (int i = 0; i < n_shards; ++i) {
         const glqh_trellis_shard &sh = shards[i];
-        GLQH_REQUIRE(sh.sv_f16 && sh.su_f16 && sh.packed && sh.y, "trellis group: null pointer in shard %d", i);
+        GLQH_REQUIRE(sh.sv_f16 && sh.packed, "trellis group: null pointer in shard %d", i);
+        GLQH_REQUIRE((sh.y != nullptr) == (shards[0].y != nullptr) && (!sh.y || sh.su_f16),
+                     "trellis group: shard %d: outputs must be given for all shards or for none", i);
         int Ri;
         if (tr_bits_from_packed(sh.packed_cols, 0, &Ri) || tr_check_shape(sh.m_pad, n_pad, sh.packed_rows)) return 1;
         GLQH_REQUIRE(i == 0 || Ri == R, "trellis group: shards of %d and %d bits/weight cannot share a launch", R, Ri);
@@ -398,6 +400,7 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
     if (glqh_launch_trellis_fusein_group(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B, n_pad,
                                          in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
         return 1;
+    if (!shards[0].y) return 0;                                // decode launch only: partial sums stay in ws
     return glqh_launch_output_rht_group(parts, su, ys, scale, m_pads, outs, n_shards, y_dtype, y_stride, B, ks, st);
 }
 

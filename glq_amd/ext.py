@@ -299,7 +299,7 @@ class _TrellisShard(C.Structure):
 
 
 def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_features, n_pad,
-                                         out_dtype=None):
+                                         out_dtype=None, decode_only=False):
     """Several separately quantized trellis layers on the same x (fused q/k/v, gate/up) with
     one decode launch and one output-transform launch: the per-shard loop of the reference's
     vLLM linear method (glq_vllm/linear_method.py:664-710) as a single call.
@@ -307,17 +307,18 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
     shards: sequence of (sv, su, trellis_packed, wscale, out_features, m_pad).  Returns one
     (B, sum(out_features)) tensor, shard s in columns [off_s, off_s + out_features_s).
     Needs 1..4 tokens, single-stage layers of one rate and block_decompose block sizes; raises
-    RuntimeError otherwise (callers then use the per-layer op)."""
+    RuntimeError otherwise (callers then use the per-layer op).  decode_only=True stops
+    after the decode launch (no output transform, returns None): a measurement hook."""
     lib = _lib.load()
     _chk(x, "x", (torch.float16, torch.bfloat16))
     B = x.shape[0]
     dt = out_dtype or torch.float16
     total_out = sum(int(s[4]) for s in shards)
     total_m = sum(int(s[5]) for s in shards)
-    y = torch.empty((B, total_out), dtype=dt, device=x.device)
+    y = None if decode_only else torch.empty((B, total_out), dtype=dt, device=x.device)
     arr = (_TrellisShard * len(shards))()
     off = 0
-    esz = y.element_size()
+    esz = torch.empty((), dtype=dt).element_size()
     for i, (sv, su, packed, wscale, out_f, m_pad) in enumerate(shards):
         _chk(sv, "sv", torch.float16)
         _chk(su, "su", torch.float16)
@@ -325,7 +326,7 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
         if packed.dim() != 2:
             raise RuntimeError("trellis_packed must be 2-D [(m/16)*(k/16), 16*R]")
         arr[i] = _TrellisShard(_p(sv), _p(su), _p(packed), packed.shape[0], packed.shape[1], float(wscale),
-                               int(out_f), int(m_pad), y.data_ptr() + off * esz)
+                               int(out_f), int(m_pad), None if y is None else y.data_ptr() + off * esz)
         off += int(out_f)
     bn, nbn = _host_i64(blocks_n)
     with torch.cuda.device(x.device):

@@ -145,7 +145,9 @@ typedef struct {
     int64_t packed_rows, packed_cols;
     double wscale;
     int64_t out_features, m_pad; /* m_pad's block sizes are block_decompose(m_pad) */
-    void *y;                     /* this layer's first output element, row stride y_stride */
+    void *y;                     /* this layer's first output element, row stride y_stride;
+                                    NULL in every shard: stop after the decode launch (the
+                                    split-K partial sums stay in the workspace) */
 } glqh_trellis_shard;
 
 size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad, int64_t total_m_pad,

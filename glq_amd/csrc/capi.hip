@@ -15,6 +15,22 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
                             int64_t out_stride, hipStream_t stream);
 int glqh_trellis_mma_init(void);
 
+int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
+int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const sv[], float *const part[],
+                                   const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
+                                   int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
+                                   int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                                   int n_blocks, hipStream_t stream);
+// K plan of the fused-input GEMV for layers of the given padded heights sharing one input.
+// Returns 0 (not eligible), 1 (32-row workgroups, v_dot2 decode: more, shorter workgroups,
+// which is what the latency-bound attention shapes want) or 2 (64-row workgroups, MFMA decode:
+// fewer vector-ALU operations per weight, which pays once the rows alone fill the chip).
+static int tr_fusein_plan(const int64_t *m_pads, int n, int64_t n_pad, int64_t B, int *S, int *ks) {
+    int64_t total = 0, wgs = 0;
+    for (int i = 0; i < n; ++i) { total += m_pads[i]; wgs += (m_pads[i] + 63) / 64; }
+    if (wgs >= glqh_device_cus()) return glqh_trellis_mma_fusein_plan(wgs, n_pad, B, S, ks) ? 2 : 0;
+    return glqh_trellis_fusein_plan(total, n_pad, B, S, ks) ? 1 : 0;
+}
 int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out);
 int glqh_launch_trellis_prefill(const void *x_f16, int64_t M, const void *packed, int R, int64_t m, int64_t k,
                                 int S, int ksplit, float *out, int direct, float scale, int accum,
@@ -223,7 +239,7 @@ extern "C" int glqh_output_rht_shards(const float *y_rht, const void *su_f16, vo
 static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
     int ks = tr_plain_plan(m_pad, n_pad, B).ks;
     int steps = 0, ks2 = 0;
-    if (glqh_trellis_fusein_plan(m_pad, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
+    if (tr_fusein_plan(&m_pad, 1, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
     return align256((size_t)ks * B * m_pad * sizeof(float));
 }
 
@@ -270,11 +286,11 @@ extern "C" int glqh_fused_linear_trellis_3inst(
 
     // Single-stage layers at up to four tokens fold the input transform into the GEMV;
     // everything else transforms x once into scratch and reads it from every workgroup.
-    int ks = 0, fi_steps = 0;
+    int ks = 0, fi_steps = 0, fi_mode = 0;
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
     const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
     if (!has_s2 && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
-        glqh_trellis_fusein_plan(m_pad, n_pad, B, &fi_steps, &ks)) {
+        (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0) {
         if (n_blocks_n > 1) {
             int64_t sum = 0;
             for (int64_t i = 0; i < n_blocks_n; ++i) {
@@ -287,8 +303,14 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                          (long long)sum, (long long)n_pad);
         }
         GLQH_REQUIRE(in_features >= 1, "fused trellis linear: in_features must be positive");
-        if (glqh_launch_trellis_fusein(packed, R1, x, x_dtype, x_stride, sv_f16, B, m_pad, n_pad,
-                                       in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, part1, st))
+        if (fi_mode == 2) {
+            const void *pk[1] = {packed}, *svs[1] = {sv_f16};
+            float *pt[1] = {part1};
+            if (glqh_launch_trellis_mma_fusein(pk, svs, pt, &m_pad, 1, R1, x, x_dtype, x_stride, B, n_pad,
+                                               in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
+                return 1;
+        } else if (glqh_launch_trellis_fusein(packed, R1, x, x_dtype, x_stride, sv_f16, B, m_pad, n_pad,
+                                              in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, part1, st))
             return 1;
     } else {
         if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
@@ -326,7 +348,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
 static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {
     int64_t total = 0;
     for (int i = 0; i < n_shards; ++i) total += m_pads[i];
-    return glqh_trellis_fusein_plan(total, n_pad, B, steps, ks);
+    (void)total;
+    return tr_fusein_plan(m_pads, n_shards, n_pad, B, steps, ks);
 }
 
 extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad, int64_t total_m_pad,
@@ -334,7 +357,11 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
     if (B < 1 || B > 4 || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64) return 0;
     glqh_init();
     int steps = 0, ks = 0;
+    // upper bound over how the rows may be split among the layers: the most workgroups (and
+    // so the fewest K slots) arise from many short layers, the most slots from one tall layer
+    int ks2 = 0;
     if (!glqh_trellis_fusein_plan(total_m_pad, n_pad, B, &steps, &ks)) return 0;
+    if (glqh_trellis_mma_fusein_plan((total_m_pad + 63) / 64, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
     return (size_t)n_shards * 256 + align256((size_t)ks * B * total_m_pad * sizeof(float));
 }
 
@@ -387,7 +414,8 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
         total += sh.m_pad;
     }
     int steps = 0, ks = 0;
-    GLQH_REQUIRE(tr_group_plan(m_pads, n_shards, n_pad, B, &steps, &ks), "trellis group: shape not eligible");
+    const int fi_mode = tr_group_plan(m_pads, n_shards, n_pad, B, &steps, &ks);
+    GLQH_REQUIRE(fi_mode != 0, "trellis group: shape not eligible");
     const size_t need = align256((size_t)ks * B * total * sizeof(float));
     GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
     float *parts[GLQH_MAX_SHARDS];
@@ -397,8 +425,13 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
         p += (size_t)ks * B * m_pads[i];
     }
     hipStream_t st = (hipStream_t)stream;
-    if (glqh_launch_trellis_fusein_group(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B, n_pad,
-                                         in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
+    if (fi_mode == 2) {
+        if (glqh_launch_trellis_mma_fusein(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B, n_pad,
+                                           in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
+            return 1;
+    } else if (glqh_launch_trellis_fusein_group(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B,
+                                                n_pad, in_features, steps, ks, bn_meta_dev, blocks_n,
+                                                (int)n_blocks_n, st))
         return 1;
     if (!shards[0].y) return 0;                                // decode launch only: partial sums stay in ws
     return glqh_launch_output_rht_group(parts, su, ys, scale, m_pads, outs, n_shards, y_dtype, y_stride, B, ks, st);

@@ -25,6 +25,7 @@
 // exactly the order of the GEMV on x[b]; glq/csrc/glq_trellis.cu:555-715); the four waves
 // of a workgroup take the slot's k-pairs round-robin and are summed in wave order.
 #include "common.h"
+#include "fht_device.h"
 #include "trellis_device.h"
 
 namespace {
@@ -452,6 +453,165 @@ int launch_prefill(const void *x, int64_t M, const void *packed, int64_t m, int6
     return 0;
 }
 
+// ---------------------------------------------------------------------------------
+// GEMV with the input transform folded in (1..4 tokens), MFMA form.
+//
+// grid = (ceil(m/64), ksplit[, layers]).  K slot s owns the S = 2^j k-pairs starting at s*S,
+// i.e. the Ls = 32*S columns [s*Ls, (s+1)*Ls) of the transformed activations.  A Hadamard
+// block of size bs >= Ls that contains the slice factors as H_bs = H_(bs/Ls) (x) H_Ls, so the
+// slice r of its output is
+//     H_Ls( sum_h (-1)^popcount(r & h) * xs[h*Ls + j] ) / sqrt(bs),   xs = sv * x,
+// one pass over the block's inputs (they sit in L2) and a short transform in LDS; smaller
+// blocks are transformed whole (glq/hadamard.py:166-178, glq/csrc/glq_trellis.cu:315-370).
+// The last pass writes each value as the duplicated fp16 pair of its B-operand slot, and the
+// decode loop is mma_record.  The wave's first two records are requested before the prologue.
+// ---------------------------------------------------------------------------------
+template <int TP>
+__host__ __device__ constexpr int fi_xs_slots(int S) {
+    return S * 8 * mma_tps<TP>() + (TP < 16 ? 8 * mma_tps<TP>() : 0);          // slots + zero block
+}
+
+template <int R, typename XT, int TP>
+__device__ __forceinline__ void
+tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
+                   const f16 *__restrict__ sv, int B, int m, int k, int in_features, int S,
+                   const glqh_block_meta *__restrict__ bn_meta, int n_blocks, glqh_meta_args margs,
+                   float *__restrict__ part, u32x4 *lds) {
+    constexpr int TPS = mma_tps<TP>();
+    const int Ls = S << 5;
+    uint32_t *xs32 = (uint32_t *)lds;
+    u32x4 *zero_blk = lds + S * 8 * TPS;
+    float *fbuf = (float *)(lds + fi_xs_slots<TP>(S));          // Ls + Ls/32 floats
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const mma_lane a = mma_lane_of<TP>(lane);
+    const int nkp = k >> 5;
+    const int mpairs = m >> 5;
+    const int slot = blockIdx.y;
+    const int kp0 = slot * S;
+    const int kp1 = min(kp0 + S, nkp);
+    const int c0 = kp0 << 5;
+    const int mp = min(2 * (int)blockIdx.x + a.hm, mpairs - 1);
+
+    constexpr int REC = 4 * R;
+    const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
+    int kp = kp0 + wave;
+    tr_record<R> cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
+    tr_record<R> nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
+
+    if constexpr (TP < 16) {
+        for (int i = threadIdx.x; i < 8 * TPS; i += TR_THREADS) zero_blk[i] = u32x4{0u, 0u, 0u, 0u};
+    }
+    // ---- prologue: transformed activations of this slot's columns -> B-operand slots ----
+    for (int jb = 0; jb < n_blocks; ++jb) {
+        const glqh_block_meta bm = glqh_meta_row(margs, bn_meta, jb);
+        const int lo = max(bm.offset, c0), hi = min(bm.offset + bm.bs, c0 + Ls);
+        if (lo >= hi) continue;                                  // uniform over the workgroup
+        const int len = hi - lo;                                 // min(bs, Ls), a power of two
+        const int log_len = 31 - __builtin_clz(len);
+        const int nsub = bm.bs >> log_len;
+        const int r = (lo - bm.offset) >> log_len;
+        const float norm = bm.w != 0 ? __builtin_bit_cast(float, bm.w) : rsqrt_pow2(bm.log_bs);
+        for (int t = 0; t < TP; ++t) {
+            if (t >= B) break;
+            const XT *xr = x + (int64_t)t * x_stride;
+            __syncthreads();                                     // fbuf free again
+            stage_signed_slices<TR_THREADS>(fbuf, log_len, nsub, r, [&](int h, int j) -> float {
+                const int col = bm.offset + (h << log_len) + j;
+                const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
+                return col < in_features ? v : 0.0f;
+            });
+            struct {
+                uint32_t *xs32;
+                int c_rel, t;
+                float norm;
+                __device__ float aux(int) const { return norm; }
+                __device__ void put(int i, float v, float f) const {
+                    const int c = c_rel + i;                     // column inside the slot
+                    const int u = c >> 5, ks = (c >> 4) & 1, q = (c >> 1) & 3;
+                    const int p = 2 * ((c >> 3) & 1) + (c & 1);
+                    const f16 hv = (f16)(v * f);
+                    const f16x2 pair = {hv, hv};
+                    xs32[((((u * 2 + ks) * 4) + q) * mma_tps<TP>() + t) * 4 + p] = __builtin_bit_cast(uint32_t, pair);
+                }
+            } store = {xs32, lo - c0, t, norm};
+            fht_staged(fbuf, log_len, store);
+        }
+    }
+    if constexpr (TP > 1) {
+        // tokens past B read zeros: clear their slots once (every k-pair of the slot)
+        for (int idx = threadIdx.x; idx < S * 8 * (TP - 1); idx += TR_THREADS) {
+            const int t = 1 + idx % (TP - 1), g = idx / (TP - 1);
+            if (t >= B) lds[g * TPS + t] = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    __syncthreads();
+
+    mma_acc<1> acc;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) acc.v[s][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (; kp < kp1; kp += TR_WAVES) {
+        const tr_record<R> nx2 = tr_load_record<R>(lane_base + (int64_t)min(kp + 2 * TR_WAVES, kp1 - 1) * 32 * REC);
+        const u32x4 *xsl = a.live ? lds + ((kp - kp0) * 8 + a.q) * TPS + a.tokl : zero_blk;
+        acc = mma_record<R, TP, 1>(cur, a.next1, a.next2, xsl, acc);
+        cur = nx1;
+        nx1 = nx2;
+    }
+    mma_reduce_store<TP, 1>(acc, (float *)lds, a, wave, B, m, 0, 64 * blockIdx.x, slot, part, 0, 1.0f, 0, 0);
+}
+
+template <int R, typename XT, int TP>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
+                     const f16 *__restrict__ sv, int B, int m, int k, int in_features, int S,
+                     const glqh_block_meta *__restrict__ bn_meta, int n_blocks, glqh_meta_args margs,
+                     float *__restrict__ part) {
+    extern __shared__ u32x4 xs_lds[];
+    tr_mma_fusein_body<R, XT, TP>(packed, x, x_stride, sv, B, m, k, in_features, S, bn_meta, n_blocks, margs,
+                                  part, xs_lds);
+}
+
+// Several layers that read the same activations (fused q/k/v, gate/up:
+// glq_vllm/linear_method.py:664-710) in one launch: blockIdx.z picks the layer, each with
+// its own packed stream, input signs and partial-sum buffer; workgroups past a layer's rows
+// retire.
+struct tr_fusein_group {
+    const uint8_t *packed[GLQH_MAX_GROUP];
+    const f16 *sv[GLQH_MAX_GROUP];
+    float *part[GLQH_MAX_GROUP];
+    int m[GLQH_MAX_GROUP];
+};
+
+template <int R, typename XT, int TP>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_fusein_group_kernel(tr_fusein_group g, const XT *__restrict__ x, int64_t x_stride, int B, int k,
+                           int in_features, int S, const glqh_block_meta *__restrict__ bn_meta,
+                           int n_blocks, glqh_meta_args margs) {
+    extern __shared__ u32x4 xs_lds[];
+    const int z = blockIdx.z;
+    const uint8_t *packed = g.packed[0];
+    const f16 *sv = g.sv[0];
+    float *part = g.part[0];
+    int m = g.m[0];
+#pragma unroll
+    for (int i = 1; i < GLQH_MAX_GROUP; ++i)
+        if (i == z) { packed = g.packed[i]; sv = g.sv[i]; part = g.part[i]; m = g.m[i]; }
+    if ((int)blockIdx.x * 64 >= m) return;
+    tr_mma_fusein_body<R, XT, TP>(packed, x, x_stride, sv, B, m, k, in_features, S, bn_meta, n_blocks, margs,
+                                  part, xs_lds);
+}
+
+template <int TP>
+size_t fi_lds_bytes(int S) {
+    const size_t Ls = (size_t)S * 32;
+    size_t b = (size_t)fi_xs_slots<TP>(S) * 16 + (Ls + Ls / 32 + 32) * sizeof(float);
+    if (b < (size_t)mma_red_bytes<TP, 1>()) b = mma_red_bytes<TP, 1>();
+    return b;
+}
+
+constexpr int FI_MAX_S = 256;                                    // 8192 columns per slot
+constexpr int FI_MAX_S_TP4 = 128;
+
 // LDS per workgroup: a chunk of CH k-pairs (CH % 4 == 0) plus, for partial token tiles, one
 // zeroed block; small enough that the register-limited number of workgroups fits a CU.
 constexpr int MMA_LDS_MAX = 64 * 1024;
@@ -568,8 +728,103 @@ static int pf_set_lds(K kernel) {
                           "trellis prefill attribute");
 }
 
+// ---- fused-input GEMV (MFMA form): plan and launch -----------------------------------
+// S k-pairs per K slot: a power of two >= 4 chosen so that about four workgroups per CU are
+// in flight; the slice 32*S is capped by LDS (8192 columns at one token, 4096 at 2..4).
+int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out) {
+    if (B < 1 || B > 4 || wgs_rows < 1) return 0;
+    const int64_t nkp = k / 32;
+    const int64_t target = (int64_t)glqh_device_cus() * 4;
+    int64_t ks_target = (target + wgs_rows - 1) / wgs_rows;
+    if (ks_target < 1) ks_target = 1;
+    const int64_t want = (nkp + ks_target - 1) / ks_target;
+    int64_t S = 2 * TR_WAVES;                                   // at least 256 columns per slot
+    while (S < want) S <<= 1;
+    const int64_t cap = B == 1 ? FI_MAX_S : FI_MAX_S_TP4;
+    if (S > cap) S = cap;
+    *S_out = (int)S;
+    *ksplit_out = (int)((nkp + S - 1) / S);
+    return 1;
+}
+
+template <int R, typename XT, int TP>
+static int launch_mma_fusein(const tr_fusein_group &g, int n_layers, int64_t max_m, const void *x,
+                             int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S, int ksplit,
+                             const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                             hipStream_t stream) {
+    glqh_meta_args margs;
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
+    const glqh_block_meta *meta = n_blocks > 1 ? bn_meta : nullptr;
+    const int nb = n_blocks > 1 ? n_blocks : 1;
+    const size_t lds = fi_lds_bytes<TP>(S);
+    if (n_layers == 1) {
+        dim3 grid((unsigned)((max_m + 63) / 64), (unsigned)ksplit, 1);
+        hipLaunchKernelGGL((tr_mma_fusein_kernel<R, XT, TP>), grid, dim3(TR_THREADS), lds, stream, g.packed[0],
+                           (const XT *)x, x_stride, g.sv[0], (int)B, g.m[0], (int)k, (int)in_features, S, meta, nb,
+                           margs, g.part[0]);
+    } else {
+        dim3 grid((unsigned)((max_m + 63) / 64), (unsigned)ksplit, (unsigned)n_layers);
+        hipLaunchKernelGGL((tr_mma_fusein_group_kernel<R, XT, TP>), grid, dim3(TR_THREADS), lds, stream, g,
+                           (const XT *)x, x_stride, (int)B, (int)k, (int)in_features, S, meta, nb, margs);
+    }
+    GLQH_LAUNCH_CHECK("trellis fused-input gemv launch");
+    return 0;
+}
+
+// packed / sv / part / m: one entry per layer (1..GLQH_MAX_GROUP)
+int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const sv[], float *const part[],
+                                   const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
+                                   int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
+                                   int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                                   int n_blocks, hipStream_t stream) {
+    GLQH_REQUIRE(n_layers >= 1 && n_layers <= GLQH_MAX_GROUP, "trellis group: 1..%d layers", GLQH_MAX_GROUP);
+    GLQH_REQUIRE(B >= 1 && B <= 4, "fused-input trellis kernel serves 1..4 tokens");
+    tr_fusein_group g = {};
+    int64_t max_m = 0;
+    for (int i = 0; i < GLQH_MAX_GROUP; ++i) {
+        const int j = i < n_layers ? i : 0;
+        g.packed[i] = (const uint8_t *)packed[j];
+        g.sv[i] = (const f16 *)sv[j];
+        g.part[i] = part[j];
+        g.m[i] = (int)m[j];
+        if (m[j] > max_m) max_m = m[j];
+    }
+#define GLQH_FI(RR, XT, TP) launch_mma_fusein<RR, XT, TP>(g, n_layers, max_m, x, x_stride, B, k, in_features, S, \
+                                                          ksplit, bn_meta, blocks_host, n_blocks, stream)
+#define GLQH_FI_R(RR)                                                                   \
+    (B == 1 ? (x_dtype == GLQH_F16 ? GLQH_FI(RR, f16, 1) : GLQH_FI(RR, uint16_t, 1))     \
+            : (x_dtype == GLQH_F16 ? GLQH_FI(RR, f16, 4) : GLQH_FI(RR, uint16_t, 4)))
+    switch (R) {
+    case 2: return GLQH_FI_R(2);
+    case 3: return GLQH_FI_R(3);
+    case 4: return GLQH_FI_R(4);
+    }
+#undef GLQH_FI_R
+#undef GLQH_FI
+    return glqh_fail("fused-input trellis kernel supports R (bits/weight) 2-4, got %d", R);
+}
+
+template <typename K>
+static int fi_set_lds(K kernel, size_t bytes) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)bytes),
+                          "trellis fused-input attribute");
+}
+
+template <int R>
+static int fi_init_R() {
+    const size_t b1 = fi_lds_bytes<1>(FI_MAX_S), b4 = fi_lds_bytes<4>(FI_MAX_S_TP4);
+    return fi_set_lds(tr_mma_fusein_kernel<R, f16, 1>, b1) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 1>, b1) ||
+           fi_set_lds(tr_mma_fusein_kernel<R, f16, 4>, b4) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 4>, b4) ||
+           fi_set_lds(tr_mma_fusein_group_kernel<R, f16, 1>, b1) ||
+           fi_set_lds(tr_mma_fusein_group_kernel<R, uint16_t, 1>, b1) ||
+           fi_set_lds(tr_mma_fusein_group_kernel<R, f16, 4>, b4) ||
+           fi_set_lds(tr_mma_fusein_group_kernel<R, uint16_t, 4>, b4);
+}
+
 int glqh_trellis_mma_init(void) {
     return mma_init_R<1>() || mma_init_R<2>() || mma_init_R<3>() || mma_init_R<4>() ||
            pf_set_lds(tr_mma_prefill_kernel<1>) || pf_set_lds(tr_mma_prefill_kernel<2>) ||
-           pf_set_lds(tr_mma_prefill_kernel<3>) || pf_set_lds(tr_mma_prefill_kernel<4>);
+           pf_set_lds(tr_mma_prefill_kernel<3>) || pf_set_lds(tr_mma_prefill_kernel<4>) ||
+           fi_init_R<2>() || fi_init_R<3>() || fi_init_R<4>();
 }

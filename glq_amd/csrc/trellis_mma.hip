@@ -464,7 +464,7 @@ int launch_prefill(const void *x, int64_t M, const void *packed, int64_t m, int6
 // one pass over the block's inputs (they sit in L2) and a short transform in LDS; smaller
 // blocks are transformed whole (glq/hadamard.py:166-178, glq/csrc/glq_trellis.cu:315-370).
 // The last pass writes each value as the duplicated fp16 pair of its B-operand slot, and the
-// decode loop is mma_record.  The wave's first two records are requested before the prologue.
+// decode loop is mma_record.
 // ---------------------------------------------------------------------------------
 template <int TP>
 __host__ __device__ constexpr int fi_xs_slots(int S) {
@@ -496,8 +496,8 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
     constexpr int REC = 4 * R;
     const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
     int kp = kp0 + wave;
-    tr_record<R> cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
-    tr_record<R> nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
+    tr_record<R> cur, nx1;
+    bool requested = false;
 
     if constexpr (TP < 16) {
         for (int i = threadIdx.x; i < 8 * TPS; i += TR_THREADS) zero_blk[i] = u32x4{0u, 0u, 0u, 0u};
@@ -521,6 +521,14 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
                 const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
                 return col < in_features ? v : 0.0f;
             });
+            if (!requested) {
+                // The wave's first records are requested here, after the activations have
+                // arrived (loads complete in order, so an earlier request would hold the
+                // transform back by the HBM latency) and before the butterflies, which hide it.
+                requested = true;
+                cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
+                nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
+            }
             struct {
                 uint32_t *xs32;
                 int c_rel, t;
@@ -537,6 +545,10 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
             } store = {xs32, lo - c0, t, norm};
             fht_staged(fbuf, log_len, store);
         }
+    }
+    if (!requested) {
+        cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
+        nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
     }
     if constexpr (TP > 1) {
         // tokens past B read zeros: clear their slots once (every k-pair of the slot)

@@ -59,6 +59,7 @@ SIGNATURES = {
     "glqh_fused_linear_trellis_3inst_group": (
         c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_int, c_vp, c_i64, c_vp, c_i64, c_i64, c_int, c_i64,
                 c_vp, c_sz, c_vp]),
+    "glqh_e8_quantize": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp]),
     # include/glq_decoder_ops.h
     "glqh_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),
     "glqh_add_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),

@@ -592,3 +592,18 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
     return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,
                                   blocks_m, n_blocks_m, 0, 0.0f, st);
 }
+
+// ---- encode side -------------------------------------------------------------------
+int glqh_launch_e8_quantize(const float *x, const float *table, const float *norms, int64_t N, int K,
+                            int64_t *idx_out, float *dec_out, hipStream_t stream);
+
+extern "C" int glqh_e8_quantize(const float *x, const float *table_f32, const float *norms_f32, int64_t N,
+                                int64_t n_entries, int64_t *idx_out, float *decoded_out, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x && table_f32 && norms_f32 && idx_out, "e8 quantize: null pointer");
+    GLQH_REQUIRE(N >= 1, "e8 quantize: N=%lld", (long long)N);
+    GLQH_REQUIRE(n_entries >= 1 && n_entries <= 65536, "e8 quantize: %lld table rows (1..65536)",
+                 (long long)n_entries);
+    return glqh_launch_e8_quantize(x, table_f32, norms_f32, N, (int)n_entries, idx_out, decoded_out,
+                                   (hipStream_t)stream);
+}

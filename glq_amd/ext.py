@@ -531,3 +531,24 @@ def glq_fused_linear_block_diag_cuda(x, sv, su, qidxs, codebook, wscale, in_feat
     return _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad, m_pad,
                      blocks_n, blocks_m, blocks_n_meta, blocks_m_meta, qidxs2, codebook2,
                      inv_resid_scale, qidxs3, inv_resid_scale2, qidxs4, inv_resid_scale3, out_dtype)
+
+
+# ---- encode side ----------------------------------------------------------------------
+def e8_quantize(x, codebook, codebook_norms=None, return_decoded=True):
+    """E8ShellCodebook.quantize (glq/codebook.py:227-278) on the GPU: nearest row of
+    `codebook` (K, 8) for every row of x (N, 8), lowest index on ties.  fp32 arithmetic in
+    coordinate order, the reference's CPU branch.  Returns (decoded fp32 (N, 8), idx int64)."""
+    lib = _lib.load()
+    if x.dim() != 2 or x.shape[1] != 8:
+        raise RuntimeError(f"x must be (N, 8), got {tuple(x.shape)}")
+    xf = x.contiguous().to(torch.float32)
+    _chk(xf, "x", torch.float32)
+    cb = codebook.contiguous().to(torch.float32)
+    norms = (cb * cb).sum(-1) if codebook_norms is None else codebook_norms.contiguous().to(torch.float32)
+    N = xf.shape[0]
+    idx = torch.empty(N, dtype=torch.int64, device=x.device)
+    dec = torch.empty(N, 8, dtype=torch.float32, device=x.device) if return_decoded else None
+    if N:
+        with torch.cuda.device(x.device):
+            check(lib.glqh_e8_quantize(_p(xf), _p(cb), _p(norms), N, cb.shape[0], _p(idx), _p(dec), _stream()))
+    return dec, idx

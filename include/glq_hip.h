@@ -219,6 +219,16 @@ int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride, int64_t B
                          void *y, int y_dtype, int64_t y_stride,
                          void *ws, size_t ws_bytes, void *stream);
 
+/* ---- encode side --------------------------------------------------------------- */
+
+/* Nearest row of an (n_entries, 8) fp32 table for each of N fp32 vectors:
+ * argmin_k( norms[k] - 2 <x, table[k]> ) with the lowest index winning ties; idx_out (N) int64,
+ * decoded_out (N, 8) fp32 or NULL.  E8ShellCodebook.quantize / _quantize_pytorch
+ * (glq/codebook.py:227-278), triton_codebook_nn(_decode) (glq/codebook_kernel.py:169-256).
+ * norms = |table[k]|^2 (fp32), as the reference's codebook_norms buffer. */
+int glqh_e8_quantize(const float *x, const float *table_f32, const float *norms_f32, int64_t N,
+                     int64_t n_entries, int64_t *idx_out, float *decoded_out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

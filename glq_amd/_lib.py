@@ -60,6 +60,9 @@ SIGNATURES = {
         c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_int, c_vp, c_i64, c_vp, c_i64, c_i64, c_int, c_i64,
                 c_vp, c_sz, c_vp]),
     "glqh_e8_quantize": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp]),
+    "glqh_trellis_quantize_workspace_bytes": (c_sz, [c_int, c_i64]),
+    "glqh_trellis_quantize_tiles": (c_int, [c_vp, c_i64, c_int, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "glqh_trellis_pack_states": (c_int, [c_vp, c_i64, c_i64, c_int, c_vp, c_vp]),
     # include/glq_decoder_ops.h
     "glqh_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),
     "glqh_add_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),

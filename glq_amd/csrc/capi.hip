@@ -14,6 +14,7 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
                             int S, int ksplit, float *part, int direct, float scale, int accum,
                             int64_t out_stride, hipStream_t stream);
 int glqh_trellis_mma_init(void);
+int glqh_viterbi_init(void);
 
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
 int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const sv[], float *const part[],
@@ -98,7 +99,7 @@ extern "C" int glqh_init(void) {
             return;
         }
         g_cus = prop.multiProcessorCount;
-        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init() || glqh_trellis_mma_init();
+        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init() || glqh_trellis_mma_init() || glqh_viterbi_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
     return g_init_rc;
@@ -606,4 +607,38 @@ extern "C" int glqh_e8_quantize(const float *x, const float *table_f32, const fl
                  (long long)n_entries);
     return glqh_launch_e8_quantize(x, table_f32, norms_f32, N, (int)n_entries, idx_out, decoded_out,
                                    (hipStream_t)stream);
+}
+
+int glqh_viterbi_init(void);
+size_t glqh_viterbi_scratch_bytes(int K, int64_t n_tiles);
+int glqh_launch_viterbi(const float *tiles, int64_t n_tiles, int K, uint8_t *scratch, int32_t *states,
+                        float *hat, hipStream_t stream);
+
+extern "C" size_t glqh_trellis_quantize_workspace_bytes(int K, int64_t n_tiles) {
+    if (K < 2 || K > 4 || n_tiles < 1) return 0;
+    glqh_init();
+    return glqh_viterbi_scratch_bytes(K, n_tiles);
+}
+
+extern "C" int glqh_trellis_quantize_tiles(const float *tiles, int64_t n_tiles, int K, int32_t *states_out,
+                                           float *hat_out, void *ws, size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(tiles && states_out && hat_out, "trellis quantize: null pointer");
+    GLQH_REQUIRE(K >= 2 && K <= 4, "trellis encoder supports K (bits/weight) 2-4, got %d", K);
+    GLQH_REQUIRE(n_tiles >= 1, "trellis quantize: n_tiles=%lld", (long long)n_tiles);
+    const size_t need = glqh_viterbi_scratch_bytes(K, n_tiles);
+    GLQH_REQUIRE(ws && ws_bytes >= need, "trellis quantize: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    return glqh_launch_viterbi(tiles, n_tiles, K, (uint8_t *)ws, states_out, hat_out, (hipStream_t)stream);
+}
+
+int glqh_launch_pack_states(const int32_t *states, int64_t m, int64_t n, int K, void *packed, hipStream_t stream);
+
+extern "C" int glqh_trellis_pack_states(const int32_t *states, int64_t m, int64_t n, int K, void *packed_out,
+                                        void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(states && packed_out, "trellis pack: null pointer");
+    GLQH_REQUIRE(K >= 1 && K <= 4, "trellis kernel supports R (bits/weight) 1-4, got %d", K);
+    GLQH_REQUIRE(glqh_trellis_kernel_supported(m, n), "trellis pack: m %% 32 and n %% 64 must be 0 (m=%lld, n=%lld)",
+                 (long long)m, (long long)n);
+    return glqh_launch_pack_states(states, m, n, K, packed_out, (hipStream_t)stream);
 }

@@ -552,3 +552,69 @@ def e8_quantize(x, codebook, codebook_norms=None, return_decoded=True):
         with torch.cuda.device(x.device):
             check(lib.glqh_e8_quantize(_p(xf), _p(cb), _p(norms), N, cb.shape[0], _p(idx), _p(dec), _stream()))
     return dec, idx
+
+
+def trellis_quantize_tiles(tiles, K):
+    """bitshift_codebook.quantize (glq/trellis.py:467-484) on the GPU: (B, 256) tiles in step
+    order -> (hat (B, 256) fp32, states (B, 256) int32), tail-biting Viterbi, K = 2..4."""
+    lib = _lib.load()
+    if tiles.dim() != 2 or tiles.shape[1] != 256:
+        raise RuntimeError(f"tiles must be (B, 256), got {tuple(tiles.shape)}")
+    x = tiles.contiguous().to(torch.float32)
+    _chk(x, "tiles", torch.float32)
+    B = x.shape[0]
+    states = torch.empty(B, 256, dtype=torch.int32, device=x.device)
+    hat = torch.empty(B, 256, dtype=torch.float32, device=x.device)
+    if B:
+        with torch.cuda.device(x.device):
+            nb = lib.glqh_trellis_quantize_workspace_bytes(int(K), B)
+            ws = _ws(max(nb, 256), x.device)
+            check(lib.glqh_trellis_quantize_tiles(_p(x), B, int(K), _p(states), _p(hat), _p(ws), ws.numel(),
+                                                  _stream()))
+    return hat, states
+
+
+def _step_permutation(device):
+    """Position (row*16 + col) of trellis step t = 8l + j inside its 16x16 tile
+    (glq/trellis.py:99-101)."""
+    t = torch.arange(256, device=device)
+    l, j = t >> 3, t & 7
+    row = (l >> 2) + 8 * ((j >> 1) & 1)
+    col = 2 * (l & 3) + 8 * (j >> 2) + (j & 1)
+    return row * 16 + col
+
+
+def trellis_matrix_to_tiles(W):
+    """(m, n) -> (tiles, 256) in trellis-step order, tiles row-major (glq/trellis.py:679-681)."""
+    m, n = W.shape
+    nat = W.reshape(m // 16, 16, n // 16, 16).permute(0, 2, 1, 3).reshape(-1, 256)
+    return nat[:, _step_permutation(W.device)].contiguous()
+
+
+def trellis_tiles_to_matrix(tiles, m, n):
+    inv = torch.empty(256, dtype=torch.int64, device=tiles.device)
+    inv[_step_permutation(tiles.device)] = torch.arange(256, device=tiles.device)
+    nat = tiles[:, inv].reshape(m // 16, n // 16, 16, 16).permute(0, 2, 1, 3)
+    return nat.reshape(m, n).contiguous()
+
+
+def trellis_pack_states(states, m, n, K):
+    """(tiles, 256) int32 states -> trellis_packed ((m/16)(n/16), 16K) int16
+    (glq/trellis.py:486-510, 580-619)."""
+    lib = _lib.load()
+    _chk(states, "states", torch.int32)
+    if states.shape != ((int(m) // 16) * (int(n) // 16), 256):
+        raise RuntimeError(f"states must be ((m/16)(n/16), 256), got {tuple(states.shape)}")
+    packed = torch.empty((states.shape[0], 16 * int(K)), dtype=torch.int16, device=states.device)
+    with torch.cuda.device(states.device):
+        check(lib.glqh_trellis_pack_states(_p(states), int(m), int(n), int(K), _p(packed), _stream()))
+    return packed
+
+
+def trellis_quantize_matrix(W_rht, K):
+    """Normalised RHT-domain weight (m, n) -> (trellis_packed, reconstruction (m, n) fp32):
+    tiles -> tail-biting Viterbi -> pack (the identity-Hessian case of
+    quantize_layer_trellis_rht, glq/trellis.py:649-688)."""
+    m, n = W_rht.shape
+    hat, states = trellis_quantize_tiles(trellis_matrix_to_tiles(W_rht.to(torch.float32)), K)
+    return trellis_pack_states(states, m, n, K), trellis_tiles_to_matrix(hat, m, n)

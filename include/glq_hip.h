@@ -229,6 +229,23 @@ int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride, int64_t B
 int glqh_e8_quantize(const float *x, const float *table_f32, const float *norms_f32, int64_t N,
                      int64_t n_entries, int64_t *idx_out, float *decoded_out, void *stream);
 
+size_t glqh_trellis_quantize_workspace_bytes(int K, int64_t n_tiles);
+
+/* Tail-biting Viterbi search of the 3INST trellis for n_tiles sequences of 256 fp32 values
+ * (a 16x16 tile in step order): states_out (n_tiles, 256) int32, hat_out (n_tiles, 256) fp32 =
+ * decode_3inst(state).  Inputs are rounded to fp16 first, costs are fp32, ties go to the
+ * lowest predecessor / lowest final state; two passes tie the ends together.
+ * bitshift_codebook.quantize / viterbi (glq/trellis.py:253-296, 467-484) and the Triton
+ * add-compare-select step (glq/trellis_step_kernel.py:30-109).  K = 2, 3 or 4. */
+int glqh_trellis_quantize_tiles(const float *tiles, int64_t n_tiles, int K, int32_t *states_out,
+                                float *hat_out, void *ws, size_t ws_bytes, void *stream);
+
+/* Trellis states of an (m, n) layer (tiles in row-major tile order, 256 steps each, int32)
+ * -> packed ((m/16)(n/16), 16K) int16 in the kernel layout, K = 1..4.
+ * bitshift_codebook.pack_trellis + pack_layer (glq/trellis.py:486-510, 580-619). */
+int glqh_trellis_pack_states(const int32_t *states, int64_t m, int64_t n, int K, void *packed_out,
+                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -158,6 +158,29 @@ def extras(torch, ext, dev):
         torch.cuda.empty_cache()
     except Exception as e:
         out["large_layer_error"] = f"{type(e).__name__}: {e}"
+    try:
+        # config 3: E8 two-stage 4 bpw GEMV, 4096 x 14336, indices from quantizing N(0,1)
+        # vectors with the GPU encoder (the index distribution decides the LDS hit rate)
+        from glq_amd.checkpoint import load_shell_table
+        cb = load_shell_table(None).to(dev)
+        m, n = 4096, 14336
+        W = torch.randn(m * (n // 8), 8, device=dev)
+        d1, i1 = ext.e8_quantize(W, cb)
+        _, i2 = ext.e8_quantize((W - d1) * 3.0, cb)
+        del W, d1
+
+        def to16(i):
+            return (i.to(torch.int32) - ((i >= 32768).to(torch.int32) << 16)).to(torch.int16).reshape(m, n // 8)
+        qs = [(to16(i1.roll(r * 977)).contiguous(), to16(i2.roll(r * 977)).contiguous()) for r in range(4)]
+        for B in (1, 16):
+            xh = torch.randn(B, n, device=dev).to(torch.float16)
+            us = _graph_time(torch, lambda: [ext.glq_dequant_matmul_cuda(xh, a, cb, 0.02, b, cb, 1 / 3.0)
+                                             for a, b in qs], len(qs))
+            out[f"e8_2stage_gemv_4096x14336_B{B}_GBs"] = round(m * (n // 8) * 4 / us / 1e3, 1)
+        del qs, i1, i2
+        torch.cuda.empty_cache()
+    except Exception as e:
+        out["e8_error"] = f"{type(e).__name__}: {e}"
     return out
 
 
@@ -288,7 +311,10 @@ def main():
         traffic = int(mt.group(1)) if mt else None
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "kernel": "tr_gemv_fusein_group_kernel<4,bf16,1>", "avg_launch_us": round(avg_us, 3),
+                "kernel": ("tr_gemv_fusein_group_kernel<4,bf16,1> (q/k/v, o, down) and "
+                           "tr_mma_fusein_group_kernel<4,bf16,1> (gate/up): the fused-input decode "
+                           "launch, averaged over the four groups of a step"),
+                "avg_launch_us": round(avg_us, 3),
                 "bytes_per_launch": int(bytes_launch),
                 "method": (f"{n_launch} back-to-back decode launches (the 4 grouped calls of a step: q/k/v, o, "
                            f"gate/up, down; x {L} distinct weight sets), stopped before the output "

@@ -304,7 +304,7 @@ def main():
     achieved = bytes_launch / (avg_us * 1e-6) / 1e9
     # HBM bytes per launch from the committed counter summary (FETCH_SIZE / WRITE_SIZE runs)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_tr_gemv_fusein_group_smollm3_4bpw_batch1.txt")
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_tr_fusein_group_kernels_smollm3_4bpw_batch1.txt")
     if os.path.exists(tpath):
         import re
         mt = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(tpath).read(), re.M)

@@ -146,6 +146,59 @@ __device__ __forceinline__ void stage_signed_slices(float *lds, int log_len, int
     __syncthreads();
 }
 
+// The same staging for the input transform when the activations are 16-bit and the block lies
+// wholly inside the row: lds[pad(i)] = sum_h sign(r, h) * x[h*len + i] * sv[h*len + i], in the
+// same order and with the same roundings as the element-wise form above, but a thread owns
+// four consecutive elements and reads them with one 8-byte load per operand (the prologue of
+// the fused-input GEMV is bound by instruction issue, not by latency).  xb / svb point at the
+// block's first element and must be 8-byte aligned; len >= 4.  Ends with a barrier.
+template <typename XT> __device__ __forceinline__ void unpack_quad(uint2 w, float *f);
+template <> __device__ __forceinline__ void unpack_quad<f16>(uint2 w, float *f) {
+    const f16x2 a = __builtin_bit_cast(f16x2, w.x), b = __builtin_bit_cast(f16x2, w.y);
+    f[0] = (float)a[0]; f[1] = (float)a[1]; f[2] = (float)b[0]; f[3] = (float)b[1];
+}
+template <> __device__ __forceinline__ void unpack_quad<uint16_t>(uint2 w, float *f) {   // bf16
+    f[0] = __builtin_bit_cast(float, w.x << 16); f[1] = __builtin_bit_cast(float, w.x & 0xffff0000u);
+    f[2] = __builtin_bit_cast(float, w.y << 16); f[3] = __builtin_bit_cast(float, w.y & 0xffff0000u);
+}
+
+template <int T, typename XT, int C = 8>
+__device__ __forceinline__ void stage_signed_input_quads(float *lds, int log_len, int nsub, int r,
+                                                         const XT *__restrict__ xb,
+                                                         const f16 *__restrict__ svb) {
+    const unsigned len = 1u << log_len;
+    for (unsigned i0 = 4 * threadIdx.x; i0 < len; i0 += 4 * T) {
+        float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int h0 = 0; h0 < nsub; h0 += C) {
+            uint2 xv[C], sg[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                // uniform base + 32-bit lane offset: the load takes its base from scalar registers
+                const size_t hb = (size_t)min(h0 + c, nsub - 1) << log_len;
+                xv[c] = *(const uint2 *)(xb + hb + i0);
+                sg[c] = *(const uint2 *)(svb + hb + i0);
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                if (h0 + c < nsub) {                              // uniform
+                    float xf[4], sf[4];
+                    unpack_quad<XT>(xv[c], xf);
+                    unpack_quad<f16>(sg[c], sf);
+                    const float sgn = (__builtin_popcount(r & (h0 + c)) & 1) ? -1.0f : 1.0f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float v = xf[e] * sf[e];
+                        z[e] = __builtin_fmaf(v, sgn, z[e]);      // z +- v, rounded once like the add
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) lds[lds_pad(i0 + e)] = z[e];
+    }
+    __syncthreads();
+}
+
 template <typename T> __device__ __forceinline__ float act_to_f32(T v);
 template <> __device__ __forceinline__ float act_to_f32<f16>(f16 v) { return (float)v; }
 template <> __device__ __forceinline__ float act_to_f32<uint16_t>(uint16_t v) { return bf16_bits_to_f32(v); }

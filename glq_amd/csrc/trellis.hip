@@ -180,6 +180,8 @@ tr_gemv_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x
         if (q + i * TR_WAVES < q1) cur[i] = tr_load_record<R>(lane_base + (q + i * TR_WAVES) * STEP_BYTES);
     }
 
+    // 8-byte loads of four activations / signs are possible (uniform over the launch)
+    const bool quads = (((uintptr_t)x | (uintptr_t)sv) & 7) == 0 && (x_stride & 3) == 0;
     // ---- prologue: transformed activations of this slot's columns -> xh ----
     for (int jb = 0; jb < n_blocks; ++jb) {
         const glqh_block_meta bm = glqh_meta_row(margs, bn_meta, jb);
@@ -194,11 +196,14 @@ tr_gemv_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x
             if (t >= B) break;
             const XT *xr = x + (int64_t)t * x_stride;
             __syncthreads();                                     // fbuf free again
-            stage_signed_slices<TR_THREADS>(fbuf, log_len, nsub, r, [&](int h, int j) -> float {
-                const int col = bm.offset + (h << log_len) + j;
-                const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
-                return col < in_features ? v : 0.0f;
-            });
+            if (quads && (bm.offset & 3) == 0 && log_len >= 2 && bm.offset + bm.bs <= in_features)
+                stage_signed_input_quads<TR_THREADS, XT>(fbuf, log_len, nsub, r, xr + bm.offset, sv + bm.offset);
+            else
+                stage_signed_slices<TR_THREADS>(fbuf, log_len, nsub, r, [&](int h, int j) -> float {
+                    const int col = bm.offset + (h << log_len) + j;
+                    const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
+                    return col < in_features ? v : 0.0f;
+                });
             f16 *xo = xh + t * Ls + (lo - c0);
             struct {
                 f16 *xo;

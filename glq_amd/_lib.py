@@ -49,6 +49,9 @@ SIGNATURES = {
     "glqh_e8_decompress": (
         c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_i64, c_i64,
                 c_vp, c_vp]),
+    "glqh_e8_embedding_rows": (
+        c_int, [c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
+                c_dbl, c_vp, c_int, c_i64, c_vp]),
     "glqh_fused_linear_e8_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64]),
     "glqh_fused_linear_e8": (
         c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,

@@ -544,6 +544,21 @@ extern "C" int glqh_e8_decompress(const void *q1, const void *q2, const void *q3
                                      m_pad, n_pad, out_f16, (hipStream_t)stream);
 }
 
+extern "C" int glqh_e8_embedding_rows(const int64_t *ids, int64_t n_ids, const void *q1, const void *q2,
+                                      const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                      const float *wscale_rows, const float *inv_rs_rows, const void *sv_f16,
+                                      int64_t n_pad, int64_t embedding_dim, int64_t num_embeddings,
+                                      double embed_scale, void *out, int out_dtype, int64_t out_stride,
+                                      void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(num_embeddings >= 1, "e8 embedding: empty table");
+    GLQH_REQUIRE(!q2 || !table2 || (n_entries2 >= 1 && n_entries2 <= 65536), "e8 embedding: bad secondary table size");
+    return glqh_launch_e8_embedding(ids, n_ids, q1, q2, table1, q2 ? (table2 ? table2 : table1) : nullptr,
+                                    q2 ? (table2 ? n_entries2 : 65536) : 0, wscale_rows, inv_rs_rows, sv_f16,
+                                    n_pad, embedding_dim, num_embeddings, (float)embed_scale, out, out_dtype,
+                                    out_stride, (hipStream_t)stream);
+}
+
 extern "C" size_t glqh_fused_linear_e8_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
     if (m_pad < 1 || n_pad < 8 || B < 1) return 0;
     glqh_init();

@@ -146,6 +146,12 @@ int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_
                               const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
                               int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream);
 
+int glqh_launch_e8_embedding(const int64_t *ids, int64_t n_ids, const void *q1, const void *q2,
+                             const uint32_t *t1, const uint32_t *t2, int64_t n2, const float *wscale,
+                             const float *inv_rs, const void *sv, int64_t n_pad, int64_t embedding_dim,
+                             int64_t num_embeddings, float embed_scale, void *out, int out_dtype,
+                             int64_t out_stride, hipStream_t stream);
+
 // fused-input trellis GEMV (B <= 4): plan returns 0 when the shape/batch is not eligible
 int glqh_trellis_fusein_plan(int64_t m, int64_t k, int64_t B, int *steps_out, int *ksplit_out);
 size_t glqh_trellis_fusein_lds(int steps, int NB);

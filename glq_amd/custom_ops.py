@@ -71,6 +71,11 @@ SCHEMAS = {
                                             "Tensor(a!) y_rht_out, int col) -> ()",
     "output_rht_shards": "output_rht_shards(Tensor y_rht, Tensor su, Tensor(a!) y, "
                          "int out_features, Tensor shard_meta, int max_bs) -> ()",
+    # glq_vllm/custom_ops.py:301-308
+    "embedding_dequant": "embedding_dequant(Tensor input_ids, Tensor qidxs, Tensor sv, "
+                         "Tensor wscale, Tensor codebook, Tensor? qidxs2, "
+                         "Tensor? inv_resid_scale, Tensor? codebook2, int n_pad, "
+                         "int embedding_dim, float embed_scale, ScalarType? out_dtype) -> Tensor",
 }
 
 
@@ -116,6 +121,12 @@ def _fused_linear_trellis_3inst_rvq2_fake(x, sv, su, trellis_packed, trellis_pac
     return x.new_empty((x.shape[0], out_features), dtype=_act_dtype(x))
 
 
+def _embedding_dequant_fake(input_ids, qidxs, sv, wscale, codebook, qidxs2, inv_resid_scale, codebook2,
+                            n_pad, embedding_dim, embed_scale, out_dtype):
+    dt = out_dtype if out_dtype is not None else sv.dtype
+    return input_ids.new_empty((*input_ids.shape, embedding_dim), dtype=dt)
+
+
 FAKES = {
     "dequant_matvec": _dequant_matvec_fake,
     "dequant_matmul": _dequant_matmul_fake,
@@ -128,6 +139,7 @@ FAKES = {
     "fused_linear_trellis_3inst_rvq2": _fused_linear_trellis_3inst_rvq2_fake,
     "fused_linear_trellis_3inst_yrht_rvq2": _none_fake,
     "output_rht_shards": _none_fake,
+    "embedding_dequant": _embedding_dequant_fake,
 }
 
 
@@ -158,6 +170,7 @@ def _impls():
         "fused_linear_trellis_3inst_rvq2": fused_linear_trellis_3inst_rvq2,
         "fused_linear_trellis_3inst_yrht_rvq2": ext.glq_fused_linear_trellis_3inst_yrht_rvq2_cuda,
         "output_rht_shards": ext.glq_output_rht_shards_cuda,
+        "embedding_dequant": ext.glq_embedding_dequant,
     }
 
 

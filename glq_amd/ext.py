@@ -412,6 +412,77 @@ def _packed_table(codebook):
     return packed
 
 
+_HALF_TABLES = {}
+
+
+def _half_table(codebook):
+    """The table as fp16 (exact for E8 values); converted once per tensor."""
+    if codebook.dtype == torch.float16:
+        return codebook
+    key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device), codebook.dtype)
+    hit = _HALF_TABLES.get(key)
+    if hit is None:
+        hit = _HALF_TABLES[key] = codebook.to(torch.float16).contiguous()
+    return hit
+
+
+def _per_row(t, n, name):
+    """(n,) fp32 per-row scale; a one-element tensor is broadcast."""
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be float32, got {t.dtype}")
+    if t.numel() == 1:
+        return t.reshape(1).expand(n).contiguous()
+    if t.numel() != n:
+        raise RuntimeError(f"{name} has {t.numel()} entries, expected {n} (one per row)")
+    return t.reshape(n).contiguous()
+
+
+def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, inv_resid_scale=None,
+                          codebook2=None, n_pad=None, embedding_dim=None, embed_scale=1.0, out_dtype=None):
+    """Rows `input_ids` of a quantized embedding: gather + E8 decode + inverse transform + scale.
+
+    Argument order and semantics of `_dequant_embedding_rows`
+    (glq/quantized_linear.py:1277-1340; op schema glq_vllm/custom_ops.py:301-308): returns
+    `(*input_ids.shape, embedding_dim)` in `out_dtype` (default: `sv.dtype`).  The tables may
+    be fp32 or fp16 `(N, 8)`; `wscale` / `inv_resid_scale` hold one fp32 per row.
+    """
+    lib = _lib.load()
+    _chk(qidxs, "qidxs", torch.int16)
+    _chk(sv, "sv", torch.float16)
+    dev = qidxs.device
+    vocab, nblk = qidxs.shape
+    n_pad = int(nblk * 8 if n_pad is None else n_pad)
+    if n_pad != nblk * 8:
+        raise RuntimeError(f"n_pad={n_pad} but qidxs has {nblk} index columns (n_pad/8 expected)")
+    embedding_dim = int(n_pad if embedding_dim is None else embedding_dim)
+    if sv.numel() != n_pad:
+        raise RuntimeError(f"sv has {sv.numel()} entries, expected n_pad={n_pad}")
+    ids = input_ids.reshape(-1).to(device=dev, dtype=torch.int64).contiguous()
+    t1 = _packed_table(_half_table(codebook.to(dev) if codebook.device != dev else codebook))
+    two = qidxs2 is not None and codebook2 is not None and inv_resid_scale is not None
+    q2 = t2 = inv = None
+    n2 = 0
+    if two:
+        _chk(qidxs2, "qidxs2", torch.int16)
+        if tuple(qidxs2.shape) != (vocab, nblk):
+            raise RuntimeError(f"qidxs2 shape {tuple(qidxs2.shape)} != qidxs shape {(vocab, nblk)}")
+        q2 = qidxs2
+        t2 = _packed_table(_half_table(codebook2.to(dev) if codebook2.device != dev else codebook2))
+        n2 = t2.shape[0]
+        inv = _per_row(inv_resid_scale.to(dev), vocab, "inv_resid_scale")
+    ws = _per_row(wscale.to(dev), vocab, "wscale")
+    dt = sv.dtype if out_dtype is None else out_dtype
+    if dt not in _DT:
+        raise RuntimeError(f"unsupported output dtype {dt}")
+    out = torch.empty((ids.numel(), embedding_dim), dtype=dt, device=dev)
+    with torch.cuda.device(dev):
+        check(lib.glqh_e8_embedding_rows(_p(ids), ids.numel(), _p(qidxs), _p(q2) if two else None, _p(t1),
+                                         _p(t2) if two else None, n2, _p(ws), _p(inv) if two else None,
+                                         _p(sv), n_pad, embedding_dim, vocab, float(embed_scale), _p(out),
+                                         _DT[dt], embedding_dim, _stream()))
+    return out.reshape(*input_ids.shape, embedding_dim)
+
+
 def _absent(t):
     return t is None or t.numel() == 0
 

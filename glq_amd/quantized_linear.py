@@ -289,3 +289,69 @@ class E8RHTLinear(nn.Module):
         kind = "trellis" if self._is_trellis else "e8_shell"
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
                 f"bias={self.bias is not None}, m_pad={self.m_pad}, n_pad={self.n_pad}, {kind}")
+
+
+class E8RHTEmbedding(nn.Module):
+    """nn.Embedding equivalent over per-row E8-quantized weights with a right-side transform.
+
+    Mirrors the reference module (glq/quantized_linear.py:1343-1452): buffers ``Qidxs``
+    (vocab, n_pad/8) int16, ``SV`` (n_pad,) fp16, ``SU`` (1,) fp16 (never read), ``Wscale``
+    (vocab,) fp32, ``Qidxs2`` and ``inv_resid_scale`` (vocab,) fp32 for the residual stage;
+    ``n_pad`` is the next power of two of ``embedding_dim``; ``embed_scale`` multiplies the
+    looked-up rows.  ``forward`` is one kernel launch (gather, decode, transform, scale).
+    """
+
+    def __init__(self, num_embeddings: int, embedding_dim: int, embed_scale: float = 1.0):
+        super().__init__()
+        self.num_embeddings = num_embeddings
+        self.embedding_dim = embedding_dim
+        self.embed_scale = float(embed_scale)
+        self.n_pad = next_pow2(embedding_dim) if embedding_dim > 0 else 1
+        self.register_buffer("Qidxs", torch.zeros(num_embeddings, self.n_pad // 8, dtype=torch.int16))
+        self.register_buffer("SV", torch.ones(self.n_pad, dtype=torch.float16))
+        self.register_buffer("SU", torch.ones(1, dtype=torch.float16))
+        self.register_buffer("Wscale", torch.ones(num_embeddings, dtype=torch.float32))
+        self.register_buffer("Qidxs2", torch.zeros(num_embeddings, self.n_pad // 8, dtype=torch.int16))
+        self.register_buffer("inv_resid_scale", torch.zeros(num_embeddings, dtype=torch.float32))
+        self.codebook = None
+        self.codebook2 = None
+        self._n_stages = 1
+
+    def set_codebook(self, codebook, codebook2=None):
+        self.codebook, self.codebook2 = codebook, codebook2
+        if self.Wscale.device.type == "meta":
+            return
+        self._n_stages = 1
+        if codebook2 is not None and bool(self.inv_resid_scale.abs().any().item()):
+            self._n_stages = 2
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys,
+                              unexpected_keys, error_msgs):
+        # 2-bpw checkpoints omit the residual-stage keys
+        if prefix + "Qidxs" in state_dict:
+            if prefix + "Qidxs2" not in state_dict:
+                state_dict[prefix + "Qidxs2"] = torch.zeros(self.num_embeddings, self.n_pad // 8,
+                                                            dtype=torch.int16)
+            if prefix + "inv_resid_scale" not in state_dict:
+                state_dict[prefix + "inv_resid_scale"] = torch.zeros(self.num_embeddings, dtype=torch.float32)
+            elif state_dict[prefix + "inv_resid_scale"].dim() == 0:
+                state_dict[prefix + "inv_resid_scale"] = (
+                    state_dict[prefix + "inv_resid_scale"].reshape(1).expand(self.num_embeddings).clone())
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys,
+                                      unexpected_keys, error_msgs)
+
+    def forward(self, input_ids: torch.Tensor) -> torch.Tensor:
+        if self.codebook is None:
+            raise RuntimeError("E8RHTEmbedding.set_codebook() must be called first")
+        from . import ext
+        out_dtype = getattr(self, "_compute_dtype", self.SV.dtype)
+        two = self._n_stages >= 2 and self.codebook2 is not None
+        return ext.glq_embedding_dequant(
+            input_ids, self.Qidxs, self.SV, self.Wscale, _codebook_tensor(self.codebook),
+            self.Qidxs2 if two else None, self.inv_resid_scale if two else None,
+            _codebook_tensor(self.codebook2) if two else None, n_pad=self.n_pad,
+            embedding_dim=self.embedding_dim, embed_scale=self.embed_scale, out_dtype=out_dtype)
+
+    def extra_repr(self) -> str:
+        return (f"num_embeddings={self.num_embeddings}, embedding_dim={self.embedding_dim}, "
+                f"n_pad={self.n_pad}")

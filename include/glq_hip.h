@@ -202,6 +202,22 @@ int glqh_e8_decompress(const void *q1, const void *q2, const void *q3, const voi
                        double inv_rs, double inv_rs2, double inv_rs3,
                        int64_t m_pad, int64_t n_pad, void *out_f16, void *stream);
 
+/* Quantized embedding lookup: rows `ids` of a (num_embeddings, n_pad/8) index matrix are decoded,
+ * scaled per row, inverse-transformed (one power-of-two block of n_pad <= 8192 values) and
+ * written as (n_ids, embedding_dim) rows of `out`:
+ *   out[t] = embed_scale * sv * H(Wscale[id] * (cb[q1[id]] + inv_rs[id] * cb2[q2[id]])) / sqrt(n_pad).
+ * ids: int64 on the device; an id outside [0, num_embeddings) yields a zero row.  q2 / table2 /
+ * inv_rs may be NULL (single stage); wscale and inv_rs hold one fp32 per row.
+ * _dequant_embedding_rows / E8RHTEmbedding.forward, glq/quantized_linear.py:1277-1340, 1427-1446;
+ * op schema glq_vllm/custom_ops.py:301-308. */
+int glqh_e8_embedding_rows(const int64_t *ids, int64_t n_ids,
+                           const void *q1, const void *q2,
+                           const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                           const float *wscale_rows, const float *inv_rs_rows, const void *sv_f16,
+                           int64_t n_pad, int64_t embedding_dim, int64_t num_embeddings,
+                           double embed_scale, void *out, int out_dtype, int64_t out_stride,
+                           void *stream);
+
 size_t glqh_fused_linear_e8_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad);
 
 /* Whole E8 linear: input RHT -> gather-matmul -> output RHT.

@@ -22,6 +22,8 @@ Pinned by (see tests/test_oracle_*.py):
                          decode_layer (tests/golden/), plus a second, independent
                          lane-walk formulation in the tests
   viterbi / e8 nearest   golden state/index sequences from the reference encoders
+  e8_embedding_rows      closed form: brute-force Sylvester matrix product on small n, and
+                         equality with row-by-row (one-hot) use of e8_dequant + fht
   linear forwards        golden end-to-end outputs from E8RHTLinear.forward (CPU)
 """
 from __future__ import annotations
@@ -206,6 +208,28 @@ def e8_dequant_matmul(x_rht, Qidxs, wscale, Qidxs2=None, inv_rs=0.0, table=None,
     """y_rht = x_rht @ W^T * Wscale (glq/inference_kernel.py:1194-1216)."""
     W = e8_dequant(Qidxs, Qidxs2, inv_rs, table=table, table2=table2)
     return (np.asarray(x_rht, dtype=np.float32) @ W.T * np.float32(wscale)).astype(np.float32)
+
+
+def e8_embedding_rows(ids, Qidxs, sv, wscale_rows, Qidxs2=None, inv_rs_rows=None, embedding_dim=None,
+                      embed_scale=1.0, table=None, table2=None) -> np.ndarray:
+    """Quantized-embedding lookup, fp32 (glq/quantized_linear.py:1277-1340):
+    deq = cb[q1[id]] (+ cb2[q2[id]] * inv_rs[id]); deq *= Wscale[id]; FHT over the padded
+    row; * sv; * embed_scale; trimmed to embedding_dim."""
+    ids = np.asarray(ids, dtype=np.int64)
+    flat = ids.reshape(-1)
+    nb = Qidxs.shape[1]
+    n_pad = nb * 8
+    deq = e8_decode(Qidxs[flat].reshape(-1), table).reshape(flat.shape[0], n_pad).astype(np.float32)
+    if Qidxs2 is not None and inv_rs_rows is not None:
+        t2 = table if table2 is None else table2
+        deq2 = e8_decode(Qidxs2[flat].reshape(-1), t2).reshape(flat.shape[0], n_pad).astype(np.float32)
+        deq = deq + deq2 * np.asarray(inv_rs_rows, dtype=np.float32)[flat][:, None]
+    deq = deq * np.asarray(wscale_rows, dtype=np.float32)[flat][:, None]
+    deq = fht(deq) * np.asarray(sv, dtype=np.float32)
+    if embed_scale != 1.0:
+        deq = deq * np.float32(embed_scale)
+    d = n_pad if embedding_dim is None else embedding_dim
+    return deq[:, :d].reshape(*ids.shape, d).astype(np.float32)
 
 
 def e8_quantize_layer(W, bpw=2, seed=42, block_diagonal=True):

@@ -162,3 +162,29 @@ def test_e8_layer_quantize_and_forward_match_reference(golden, tag, bpw, bd):
     assert O.rel_fro(y, g[f"{tag}_y"]) < 1e-5
     # and equals x @ W_hat^T with the reference's own dequantised weight
     assert O.rel_fro(y, g[f"{tag}_x"] @ g[f"{tag}_W_hat"].T) < 1e-4
+
+
+def test_embedding_rows_closed_form():
+    """Embedding lookup against the Sylvester matrix written out (n = 32) and against the
+    linear-layer pieces used row by row."""
+    rng = np.random.default_rng(5)
+    vocab, n = 11, 32
+    tab = O.e8_table()
+    q1 = rng.integers(0, 65536, (vocab, n // 8)).astype(np.uint16).view(np.int16)
+    q2 = rng.integers(0, 65536, (vocab, n // 8)).astype(np.uint16).view(np.int16)
+    sv = rng.choice([-1.0, 1.0], n).astype(np.float32)
+    ws = rng.uniform(0.5, 2.0, vocab).astype(np.float32)
+    inv = rng.uniform(0.1, 0.5, vocab).astype(np.float32)
+    ids = np.array([[3, 0], [10, 3]])
+    got = O.e8_embedding_rows(ids, q1, sv, ws, q2, inv, embedding_dim=27, embed_scale=1.5)
+    assert got.shape == (2, 2, 27)
+    H = sylvester(n)
+    for (a, b), i in np.ndenumerate(ids):
+        row = np.concatenate([tab[int(c) & 0xFFFF] for c in q1[i].view(np.uint16)]).astype(np.float64)
+        row2 = np.concatenate([tab[int(c) & 0xFFFF] for c in q2[i].view(np.uint16)]).astype(np.float64)
+        want = (H @ ((row + row2 * inv[i]) * ws[i])) * sv * 1.5
+        assert np.allclose(got[a, b], want[:27], atol=1e-5)
+    # one stage == the dequantizer of the linear path on the same rows
+    one = O.e8_embedding_rows(np.arange(vocab), q1, sv, ws)
+    W = O.e8_dequant(q1) * ws[:, None]
+    assert np.allclose(one, O.fht(W) * sv, atol=1e-6)

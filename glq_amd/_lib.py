@@ -32,6 +32,8 @@ SIGNATURES = {
     "glqh_output_rht": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_vp, c_vp, c_i64,
                 c_dbl, c_vp]),
+    "glqh_output_rht_scaled": (
+        c_int, [c_vp, c_dbl, c_vp, c_vp, c_int, c_i64, c_i64, c_i64, c_i64, c_vp, c_vp, c_i64, c_vp]),
     "glqh_output_rht_shards": (
         c_int, [c_vp, c_vp, c_vp, c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_i64, c_vp]),
     "glqh_fused_linear_trellis_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64]),

@@ -219,6 +219,22 @@ extern "C" int glqh_output_rht(const float *y_rht, int64_t y_rht_stride, const v
                                   blocks_host, n_blocks, 0, (float)rsqrt_m, (hipStream_t)stream);
 }
 
+extern "C" int glqh_output_rht_scaled(const float *y_rht, double scale, const void *su_f16, void *y,
+                                      int y_dtype, int64_t y_stride, int64_t B, int64_t out_features,
+                                      int64_t m_pad, const glqh_block_meta *meta_dev,
+                                      const int64_t *blocks_host, int64_t n_blocks, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(y_rht && y, "output_rht: null pointer");
+    GLQH_REQUIRE(y_stride >= out_features, "output_rht: bad strides");
+    glqh_ysrc src = {};                                          // one "partial sum" per element, one stage
+    src.part = y_rht;
+    src.ksplit = 1;
+    src.nparts = 1;
+    src.scale[0] = (float)scale;
+    return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, meta_dev,
+                                  blocks_host, n_blocks, 0, 0.0f, (hipStream_t)stream);
+}
+
 extern "C" int glqh_output_rht_shards(const float *y_rht, const void *su_f16, void *y, int y_dtype,
                                       int64_t B, int64_t out_features, int64_t total_m,
                                       const glqh_block_meta *shard_meta_dev, int64_t n_rows,

@@ -13,6 +13,7 @@ typedef _Float16 f16;
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define GLQH_WAVE 64
 #define GLQH_MAX_GROUP GLQH_MAX_SHARDS      // layers per grouped launch

@@ -128,6 +128,194 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
     fht_staged(s, blk.log_len, store);
 }
 
+// ---- many tokens: whole blocks, 16-byte accesses ------------------------------------
+// With many tokens the transforms are bound by HBM, and what matters is how many bytes each
+// thread keeps in flight and how the stores coalesce.  A workgroup owns one whole block
+// (at most 8192 points) of one token, every thread moves eight consecutive elements per
+// access (16 bytes of 16-bit data), and the last butterfly pass puts its results back into
+// LDS so that the copy-out can write rows in the same 8-element runs.  Arithmetic and
+// rounding are the same as in the element-wise kernels above.
+constexpr int WIDE_LOG_MAX = 13;
+
+template <typename T> __device__ __forceinline__ void load8(const T *p, float *f);
+template <> __device__ __forceinline__ void load8<float>(const float *p, float *f) {
+    const f32x4 a = *(const f32x4 *)p, b = *(const f32x4 *)(p + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { f[e] = a[e]; f[4 + e] = b[e]; }
+}
+template <> __device__ __forceinline__ void load8<f16>(const f16 *p, float *f) {
+    const u32x4 w = *(const u32x4 *)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t we = w[e];                    // (bit_cast straight from a vector element reads element 0)
+        const f16x2 h = __builtin_bit_cast(f16x2, we);
+        f[2 * e] = (float)h[0];
+        f[2 * e + 1] = (float)h[1];
+    }
+}
+template <> __device__ __forceinline__ void load8<uint16_t>(const uint16_t *p, float *f) {   // bf16
+    const u32x4 w = *(const u32x4 *)p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        f[2 * e] = __builtin_bit_cast(float, w[e] << 16);
+        f[2 * e + 1] = __builtin_bit_cast(float, w[e] & 0xffff0000u);
+    }
+}
+template <typename T> __device__ __forceinline__ void store8(T *p, const float *f);
+template <> __device__ __forceinline__ void store8<float>(float *p, const float *f) {
+    *(f32x4 *)p = f32x4{f[0], f[1], f[2], f[3]};
+    *(f32x4 *)(p + 4) = f32x4{f[4], f[5], f[6], f[7]};
+}
+template <> __device__ __forceinline__ void store8<f16>(f16 *p, const float *f) {
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const f16x2 h = {(f16)f[2 * e], (f16)f[2 * e + 1]};
+        w[e] = __builtin_bit_cast(uint32_t, h);
+    }
+    *(u32x4 *)p = w;
+}
+template <> __device__ __forceinline__ void store8<uint16_t>(uint16_t *p, const float *f) {  // bf16
+    u32x4 w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        w[e] = (uint32_t)f32_to_bf16_bits(f[2 * e]) | ((uint32_t)f32_to_bf16_bits(f[2 * e + 1]) << 16);
+    *(u32x4 *)p = w;
+}
+
+struct lds_writeback {                                   // last pass: results stay in LDS
+    float *lds;
+    __device__ float aux(int) const { return 0.0f; }
+    __device__ void put(int i, float v, float) const { lds[lds_pad(i)] = v; }
+};
+
+// blockIdx.x = block, blockIdx.y = token.  Requires canonical blocks of 8..8192 points, 16-byte
+// aligned rows of x (x_stride % 8 == 0 elements for 16-bit types) and out.
+template <typename XT, typename OT>
+__global__ void __launch_bounds__(RHT_THREADS)
+input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
+                      OT *__restrict__ out, int in_features, int n_pad, glqh_meta_args margs,
+                      float single_norm) {
+    extern __shared__ float s[];
+    const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
+    const XT *xr = x + (int64_t)blockIdx.y * x_stride + blk.off;
+    const f16 *svb = sv + blk.off;
+    const int lim = in_features - blk.off;               // elements of the block inside the row
+    constexpr int U = 2;
+    for (int i0 = 8 * threadIdx.x; i0 < blk.bs; i0 += 8 * U * RHT_THREADS) {
+        float xf[U][8], sf[U][8];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + 8 * u * RHT_THREADS;
+            if (i < blk.bs) {
+                load8<f16>(svb + i, sf[u]);
+                if (i + 8 <= lim) load8<XT>(xr + i, xf[u]);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) xf[u][e] = i + e < lim ? act_to_f32<XT>(xr[i + e]) : 0.0f;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + 8 * u * RHT_THREADS;
+            if (i < blk.bs) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s[lds_pad(i + e)] = xf[u][e] * sf[u][e];
+            }
+        }
+    }
+    __syncthreads();
+    fht_staged(s, blk.log_len, lds_writeback{s});
+    __syncthreads();
+    OT *orow = out + (int64_t)blockIdx.y * n_pad + blk.off;
+    for (int i = 8 * threadIdx.x; i < blk.bs; i += 8 * RHT_THREADS) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = s[lds_pad(i + e)] * blk.norm;
+        store8<OT>(orow + i, v);
+    }
+}
+
+// src: direct rows (stride % 4 == 0) or split-K partials; y rows 16-byte aligned.
+template <typename YT>
+__global__ void __launch_bounds__(RHT_THREADS)
+output_rht_wide_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
+                       int out_features, int m_pad, glqh_meta_args margs, float single_norm) {
+    extern __shared__ float s[];
+    const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
+    const int64_t b = blockIdx.y;
+    if (src.nparts == 0) {
+        const float *__restrict__ d = src.direct + b * src.stride + blk.off;
+        constexpr int U = 2;
+        for (int i0 = 8 * threadIdx.x; i0 < blk.bs; i0 += 8 * U * RHT_THREADS) {
+            float v[U][8];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (i0 + 8 * u * RHT_THREADS < blk.bs) load8<float>(d + i0 + 8 * u * RHT_THREADS, v[u]);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (i0 + 8 * u * RHT_THREADS < blk.bs) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) s[lds_pad(i0 + 8 * u * RHT_THREADS + e)] = v[u][e];
+                }
+        }
+    } else {
+        // v = sum_stage scale * (sum_k partial), in this fixed order (as stage_partials)
+        const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
+        for (int i = 8 * threadIdx.x; i < blk.bs; i += 8 * RHT_THREADS) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+            for (int st = 0; st < src.nparts; ++st) {
+                float acc[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+                const float *p = pbase + st * src.part_sstride + i;
+                int k = 0;
+                for (; k + 2 <= src.ksplit; k += 2) {            // two terms in flight
+                    float t0[8], t1[8];
+                    load8<float>(p + k * src.part_kstride, t0);
+                    load8<float>(p + (k + 1) * src.part_kstride, t1);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = (acc[e] + t0[e]) + t1[e];
+                }
+                if (k < src.ksplit) {
+                    float t0[8];
+                    load8<float>(p + k * src.part_kstride, t0);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] += t0[e];
+                }
+                const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
+                               : st == 2 ? src.scale[2] : src.scale[3];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += sc * acc[e];
+            }
+            if (src.copy_out) store8<float>(src.copy_out + b * src.copy_stride + blk.off + i, v);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[lds_pad(i + e)] = v[e];
+        }
+    }
+    __syncthreads();
+    fht_staged(s, blk.log_len, lds_writeback{s});
+    __syncthreads();
+    YT *yrow = y + b * y_stride;
+    for (int i = 8 * threadIdx.x; i < blk.bs; i += 8 * RHT_THREADS) {
+        const int row = blk.off + i;
+        if (row >= out_features) continue;
+        float f[8], v[8];
+        load8<f16>(su + row, f);                                 // su has m_pad entries
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = s[lds_pad(i + e)] * (blk.norm * f[e]);
+        if (row + 8 <= out_features) store8<YT>(yrow + row, v);
+        else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (row + e < out_features) yrow[row + e] = f32_to_act<YT>(v[e]);
+        }
+    }
+}
+
 template <typename YT, bool PARTS>
 __device__ __forceinline__ void
 output_rht_body(const glqh_ysrc &src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
@@ -249,6 +437,15 @@ int ilog2(int64_t v) {
 
 }  // namespace
 
+namespace {
+// whole-block 16-byte kernels: many tokens, canonical blocks of 8..8192 points
+bool rht_wide_ok(int64_t B, const glqh_meta_args &margs, int64_t total, int64_t max_bs) {
+    if (B <= 64 || margs.canon == 0 || max_bs > (1 << WIDE_LOG_MAX)) return false;
+    return (total & 7) == 0;                                 // smallest block >= 8
+}
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+}  // namespace
+
 int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv,
                           void *out, int out_dtype, int64_t B, int64_t in_features, int64_t n_pad,
                           const glqh_block_meta *meta_dev, const int64_t *blocks_host,
@@ -274,6 +471,28 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
     }
     if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, n_pad))
         margs.canon = 0;                               // not canonical: kernel reads meta_dev
+    const int x_size = x_dtype == GLQH_F32 ? 4 : 2, o_size = out_dtype == GLQH_F32 ? 4 : 2;
+    if (rht_wide_ok(B, margs, n_pad, max_bs) && aligned16(x) && aligned16(out) && aligned16(sv) &&
+        (x_stride * x_size) % 16 == 0 && (n_pad * o_size) % 16 == 0) {
+        dim3 wgrid((unsigned)n_blocks, (unsigned)B);
+        const size_t lds = rht_lds_bytes(WIDE_LOG_MAX < 63 && max_bs < (1 << WIDE_LOG_MAX) ? ilog2(max_bs) : WIDE_LOG_MAX);
+#define GLQH_INW_LAUNCH(XT, OT)                                                                     \
+    hipLaunchKernelGGL((input_rht_wide_kernel<XT, OT>), wgrid, dim3(RHT_THREADS), lds, stream,      \
+                       (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
+                       (int)n_pad, margs, rsqrt_n)
+        if (out_dtype == GLQH_F32) {
+            if (x_dtype == GLQH_F16) GLQH_INW_LAUNCH(f16, float);
+            else if (x_dtype == GLQH_BF16) GLQH_INW_LAUNCH(uint16_t, float);
+            else GLQH_INW_LAUNCH(float, float);
+        } else {
+            if (x_dtype == GLQH_F16) GLQH_INW_LAUNCH(f16, f16);
+            else if (x_dtype == GLQH_BF16) GLQH_INW_LAUNCH(uint16_t, f16);
+            else GLQH_INW_LAUNCH(float, f16);
+        }
+#undef GLQH_INW_LAUNCH
+        GLQH_LAUNCH_CHECK("input_rht launch");
+        return 0;
+    }
     const int log_slice = rht_log_slice(B);
     const int spb = rht_slices_per_block(max_bs, log_slice);
     GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "input_rht: too many slices");
@@ -328,6 +547,27 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
     }
     if (meta_dev && !blocks_host) margs.canon = 0;         // shard-batched call: device meta only
     else if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, m_pad)) margs.canon = 0;
+    {
+        const int y_size = y_dtype == GLQH_F32 ? 4 : 2;
+        const bool src_ok = src.nparts == 0
+            ? (aligned16(src.direct) && src.stride % 4 == 0)
+            : (aligned16(src.part) && m_pad % 4 == 0 && src.part_kstride % 4 == 0 && src.part_sstride % 4 == 0 &&
+               (!src.copy_out || (aligned16(src.copy_out) && src.copy_stride % 4 == 0)));
+        if (rht_wide_ok(B, margs, m_pad, max_bs) && src_ok && aligned16(y) && aligned16(su) &&
+            (y_stride * y_size) % 16 == 0) {
+            dim3 wgrid((unsigned)n_blocks, (unsigned)B);
+            const size_t lds = rht_lds_bytes(max_bs < (1 << WIDE_LOG_MAX) ? ilog2(max_bs) : WIDE_LOG_MAX);
+#define GLQH_OUTW_LAUNCH(YT)                                                                        \
+    hipLaunchKernelGGL((output_rht_wide_kernel<YT>), wgrid, dim3(RHT_THREADS), lds, stream, src,    \
+                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, margs, rsqrt_m)
+            if (y_dtype == GLQH_F16) GLQH_OUTW_LAUNCH(f16);
+            else if (y_dtype == GLQH_BF16) GLQH_OUTW_LAUNCH(uint16_t);
+            else GLQH_OUTW_LAUNCH(float);
+#undef GLQH_OUTW_LAUNCH
+            GLQH_LAUNCH_CHECK("output_rht launch");
+            return 0;
+        }
+    }
     const int log_slice = rht_log_slice(B);
     const int spb = rht_slices_per_block(max_bs, log_slice);
     GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "output_rht: too many slices");

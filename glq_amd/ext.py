@@ -196,6 +196,19 @@ def glq_output_rht_blockdiag_cuda(y_rht, su, y, out_features, m_pad, blocks_m, b
                                   _meta_ptr(blocks_m_meta) if nb > 1 else None, arr, nb, 0.0, _stream()))
 
 
+def _dense_matmul_output(x_rht, W, wscale, su, y, out_features, m_pad, blocks_m, blocks_m_meta):
+    """Tail of the many-token route: one library GEMM with fp32 output, then the output
+    transform with Wscale applied on the way in (no separate pass over y_rht)."""
+    lib = _lib.load()
+    y_rht = torch.mm(x_rht, W.t(), out_dtype=torch.float32)
+    arr, nb = _host_i64(blocks_m)
+    with torch.cuda.device(y_rht.device):
+        check(lib.glqh_output_rht_scaled(_p(y_rht), float(wscale), _p(su), _p(y), _DT[y.dtype], y.shape[1],
+                                         y_rht.shape[0], int(out_features), int(m_pad),
+                                         _meta_ptr(blocks_m_meta) if nb > 1 else None, arr, nb, _stream()))
+    return y
+
+
 def glq_output_rht_shards_cuda(y_rht, su, y, out_features, shard_meta, max_bs):
     lib = _lib.load()
     _chk(y_rht, "y_rht", torch.float32)
@@ -267,9 +280,7 @@ def _trellis_dense(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_m
     if packed2 is not None:
         W.add_(glq_decompress_trellis_3inst_cuda(packed2, m_pad, n_pad, allow_r1=True),
                alpha=float(inv_rs2))
-    y_rht = torch.matmul(x_rht, W.t()).to(torch.float32).mul_(float(wscale))
-    glq_output_rht_blockdiag_cuda(y_rht, su, y, out_features, m_pad, blocks_m, bm_meta)
-    return y
+    return _dense_matmul_output(x_rht, W, wscale, su, y, out_features, m_pad, blocks_m, bm_meta)
 
 
 def glq_fused_linear_trellis_3inst_cuda(x, sv, su, trellis_packed, blocks_n, blocks_m,
@@ -530,7 +541,7 @@ def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=N
     if B > E8_BATCH_MAX:
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_resid_scale, inv_resid_scale2,
                              inv_resid_scale3)
-        return torch.matmul(x, W.t()).to(torch.float32).mul_(float(wscale))
+        return torch.mm(x, W.t(), out_dtype=torch.float32).mul_(float(wscale))
     out = torch.empty((B, M), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         nb = lib.glqh_e8_matmul_workspace_bytes(M, nblk * 8, B)
@@ -568,9 +579,7 @@ def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_p
         x_rht = torch.empty((B, int(n_pad)), dtype=torch.float16, device=x.device)
         glq_input_rht_blockdiag_cuda(x, sv, x_rht, in_features, n_pad, blocks_n, bn_meta)
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
-        y_rht = torch.matmul(x_rht, W.t()).to(torch.float32).mul_(float(wscale))
-        glq_output_rht_blockdiag_cuda(y_rht, su, y, out_features, m_pad, blocks_m, bm_meta)
-        return y
+        return _dense_matmul_output(x_rht, W, wscale, su, y, out_features, m_pad, blocks_m, bm_meta)
     with torch.cuda.device(x.device):
         nb = lib.glqh_fused_linear_e8_workspace_bytes(B, int(n_pad), int(m_pad))
         ws = _ws(nb, x.device)

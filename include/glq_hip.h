@@ -98,6 +98,16 @@ int glqh_output_rht(const float *y_rht, int64_t y_rht_stride, const void *su_f16
                     const glqh_block_meta *meta_dev, const int64_t *blocks_host, int64_t n_blocks,
                     double rsqrt_m, void *stream);
 
+/* The same transform of scale * y_rht, y_rht contiguous (B, m_pad) fp32.  No counterpart in
+ * the reference's binding list: it finishes the many-token route (dequantize once, one
+ * library GEMM with fp32 output, glq/csrc/glq_trellis.cu:1322-1334), where Wscale has not been
+ * applied yet, without a separate pass over y_rht. */
+int glqh_output_rht_scaled(const float *y_rht, double scale, const void *su_f16,
+                           void *y, int y_dtype, int64_t y_stride, int64_t B,
+                           int64_t out_features, int64_t m_pad,
+                           const glqh_block_meta *meta_dev, const int64_t *blocks_host, int64_t n_blocks,
+                           void *stream);
+
 /* One launch over every sub-block of every output shard of a fused qkv / gate_up
  * linear: shard_meta rows carry global offsets into y_rht (B, total_m); su and y are
  * indexed with the same offsets (y is (B, out_features), out_features == total_m).

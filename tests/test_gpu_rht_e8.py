@@ -222,3 +222,58 @@ def test_e8_config1_layer(ext, B):
     # and against the unquantised layer: 2 bpw E8 keeps ~9 dB
     dense = x.float().numpy() @ Wt.T
     assert rel(y, dense) < 0.5
+
+
+@pytest.mark.parametrize("xdt,odt", [(torch.bfloat16, torch.float16), (torch.float16, torch.float32),
+                                     (torch.float32, torch.float16)])
+def test_many_token_transforms_with_ragged_rows(ext, xdt, odt):
+    """Whole-block 16-byte kernels (more than 64 tokens): rows that end inside an 8-element
+    run on the input side, out_features that end inside one on the output side, fp32 /
+    16-bit inputs and outputs, and equality with the few-token kernels row by row."""
+    import ctypes as C
+    from glq_amd import _lib, hadamard as H
+    say("wide rht", xdt, odt)
+    lib = _lib.load()
+    B, n, inf, stride = 70, 2688, 2685, 2696                # blocks [2048, 512, 128]
+    blocks = O.block_decompose(n)
+    meta = H.pack_block_meta(blocks).to(DEV)
+    xw = torch.randn(B, stride).to(xdt).to(DEV)
+    rng = np.random.default_rng(7)
+    sv = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    out = torch.empty(B, n, dtype=odt, device=DEV)
+    arr = (C.c_int64 * len(blocks))(*blocks)
+    dt = {torch.float16: _lib.GLQH_F16, torch.bfloat16: _lib.GLQH_BF16, torch.float32: _lib.GLQH_F32}
+    svt = t(sv)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.glqh_input_rht(C.c_void_p(xw.data_ptr()), dt[xdt], stride, C.c_void_p(svt.data_ptr()),
+                                  C.c_void_p(out.data_ptr()), dt[odt], B, inf, n, C.c_void_p(meta.data_ptr()),
+                                  arr, len(blocks), 0.0, stream))
+    xp = np.zeros((B, n), np.float32)
+    xp[:, :inf] = xw[:, :inf].float().cpu().numpy()
+    ref = O.block_diag_fht(xp * sv.astype(np.float32)[None], blocks)
+    tol = 2e-5 if odt == torch.float32 else 2e-3
+    assert np.allclose(out.float().cpu().numpy(), ref, rtol=tol, atol=tol)
+    few = torch.empty(3, n, dtype=odt, device=DEV)
+    _lib.check(lib.glqh_input_rht(C.c_void_p(xw.data_ptr()), dt[xdt], stride, C.c_void_p(svt.data_ptr()),
+                                  C.c_void_p(few.data_ptr()), dt[odt], 3, inf, n, C.c_void_p(meta.data_ptr()),
+                                  arr, len(blocks), 0.0, stream))
+    assert torch.allclose(out[:3].float(), few.float(), rtol=tol, atol=tol)   # sliced vs whole 2048-point block
+    # output side: out_features ends inside a run; y rows padded to a 16-byte multiple
+    outf, ystride = 2683, 2688
+    yr = torch.randn(B, n, device=DEV)
+    su = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float16)
+    sut = t(su)
+    y = torch.zeros(B, ystride, dtype=xdt, device=DEV)
+    _lib.check(lib.glqh_output_rht(C.c_void_p(yr.data_ptr()), n, C.c_void_p(sut.data_ptr()), C.c_void_p(y.data_ptr()),
+                                   dt[xdt], ystride, B, outf, n, C.c_void_p(meta.data_ptr()), arr, len(blocks),
+                                   0.0, stream))
+    ref = (O.block_diag_fht(yr.cpu().numpy(), blocks) * su.astype(np.float32)[None])[:, :outf]
+    tol = 2e-5 if xdt == torch.float32 else 1e-2
+    assert np.allclose(y[:, :outf].float().cpu().numpy(), ref, rtol=tol, atol=tol)
+    assert torch.count_nonzero(y[:, outf:]) == 0
+    y3 = torch.zeros(3, ystride, dtype=xdt, device=DEV)
+    _lib.check(lib.glqh_output_rht(C.c_void_p(yr.data_ptr()), n, C.c_void_p(sut.data_ptr()), C.c_void_p(y3.data_ptr()),
+                                   dt[xdt], ystride, 3, outf, n, C.c_void_p(meta.data_ptr()), arr, len(blocks),
+                                   0.0, stream))
+    # the few-token kernels cut the 2048-point block into two slices: other summation order
+    assert torch.allclose(y[:3].float(), y3.float(), rtol=4e-3, atol=4e-3)

@@ -181,6 +181,34 @@ def extras(torch, ext, dev):
         torch.cuda.empty_cache()
     except Exception as e:
         out["e8_error"] = f"{type(e).__name__}: {e}"
+    try:
+        # config 4: whole fused linears (both transforms included) at 14336 x 4096, trellis 4 bpw
+        # and E8 two-stage 4 bpw (random code bits), in the route the library picks by itself
+        from glq_amd import hadamard as H
+        from glq_amd.checkpoint import load_shell_table
+        cbh = load_shell_table(None).to(dev).half()
+        m, n = 14336, 4096
+        bn, bm = H.block_decompose(n), H.block_decompose(m)
+        bnt, bmt = torch.tensor(bn), torch.tensor(bm)
+        bnm, bmm = H.pack_block_meta(bn).to(dev), H.pack_block_meta(bm).to(dev)
+        sv = torch.ones(n, dtype=torch.float16, device=dev)
+        su = torch.ones(m, dtype=torch.float16, device=dev)
+        p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
+        q1 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
+        q2 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
+        for M in (256, 4096):
+            xb = torch.randn(M, n, device=dev).to(torch.bfloat16)
+            us = _graph_time(torch, lambda: ext.glq_fused_linear_trellis_3inst_cuda(
+                xb, sv, su, p, bnt, bmt, bnm, bmm, 0.02, n, m, n, m, out_dtype=torch.bfloat16), 1, reps=5)
+            out[f"trellis_linear_14336x4096_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+            us = _graph_time(torch, lambda: ext.glq_fused_linear_block_diag_cuda(
+                xb, sv, su, q1, cbh, 0.02, n, m, n, m, bnt, bmt, bnm, bmm, q2, cbh, 1 / 3.0,
+                out_dtype=torch.bfloat16), 1, reps=5)
+            out[f"e8_2stage_linear_14336x4096_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        del p, q1, q2
+        torch.cuda.empty_cache()
+    except Exception as e:
+        out["prefill_linear_error"] = f"{type(e).__name__}: {e}"
     return out
 
 

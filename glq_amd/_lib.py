@@ -75,6 +75,10 @@ SIGNATURES = {
                                         c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
     "glqh_attn_decode_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "glqh_silu_mul_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_vp]),
+    "glqh_trellis_linear_add_rmsnorm_bf16": (
+        c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_dbl, c_vp, c_vp, c_vp, c_sz, c_vp]),
+    "glqh_trellis_gate_up_silu_bf16": (
+        c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_sz, c_vp]),
 }
 
 GLQH_F16, GLQH_BF16, GLQH_F32 = 0, 1, 2

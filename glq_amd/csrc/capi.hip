@@ -382,13 +382,21 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
     return (size_t)n_shards * 256 + align256((size_t)ks * B * total_m_pad * sizeof(float));
 }
 
-extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
-                                                     const glqh_trellis_shard *shards, int n_shards,
-                                                     const int64_t *blocks_n, int64_t n_blocks_n,
-                                                     const glqh_block_meta *bn_meta_dev, int64_t in_features,
-                                                     int64_t n_pad, int y_dtype, int64_t y_stride, void *ws,
-                                                     size_t ws_bytes, void *stream) {
-    GLQH_INIT();
+// Decode launch of a group: checks, K plan, partial-sum layout in ws.  On return parts[i] holds
+// layer i's [slot][token][row] fp32 partial sums and *ks_out the slot count.
+struct tr_group_ctx {
+    int R, ks, fi_mode;
+    int64_t m_pads[GLQH_MAX_SHARDS], outs[GLQH_MAX_SHARDS];
+    const void *su[GLQH_MAX_SHARDS];
+    void *ys[GLQH_MAX_SHARDS];
+    float scale[GLQH_MAX_SHARDS];
+    float *parts[GLQH_MAX_SHARDS];
+};
+
+static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                           const glqh_trellis_shard *shards, int n_shards, const int64_t *blocks_n,
+                           int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev, int64_t in_features,
+                           int64_t n_pad, void *ws, size_t ws_bytes, hipStream_t st, tr_group_ctx *c) {
     GLQH_REQUIRE(x && shards, "trellis group: null pointer");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis group: %d shards (1..%d)", n_shards,
                  GLQH_MAX_SHARDS);
@@ -409,10 +417,7 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
                      (long long)n_pad);
     }
     int R = 0;
-    int64_t m_pads[GLQH_MAX_SHARDS], outs[GLQH_MAX_SHARDS];
-    const void *packed[GLQH_MAX_SHARDS], *sv[GLQH_MAX_SHARDS], *su[GLQH_MAX_SHARDS];
-    void *ys[GLQH_MAX_SHARDS];
-    float scale[GLQH_MAX_SHARDS];
+    const void *packed[GLQH_MAX_SHARDS], *sv[GLQH_MAX_SHARDS];
     int64_t total = 0;
     for (int i = 0; i < n_shards; ++i) {
         const glqh_trellis_shard &sh = shards[i];
@@ -425,33 +430,87 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
         GLQH_REQUIRE(Ri >= 2, "trellis group: the grouped launch serves 2-4 bits/weight");
         R = Ri;
         GLQH_REQUIRE(sh.out_features >= 1 && sh.out_features <= sh.m_pad, "trellis group: out_features exceeds m_pad");
-        m_pads[i] = sh.m_pad; outs[i] = sh.out_features;
-        packed[i] = sh.packed; sv[i] = sh.sv_f16; su[i] = sh.su_f16; ys[i] = sh.y;
-        scale[i] = (float)sh.wscale;
+        c->m_pads[i] = sh.m_pad; c->outs[i] = sh.out_features;
+        packed[i] = sh.packed; sv[i] = sh.sv_f16; c->su[i] = sh.su_f16; c->ys[i] = sh.y;
+        c->scale[i] = (float)sh.wscale;
         total += sh.m_pad;
     }
     int steps = 0, ks = 0;
-    const int fi_mode = tr_group_plan(m_pads, n_shards, n_pad, B, &steps, &ks);
+    const int fi_mode = tr_group_plan(c->m_pads, n_shards, n_pad, B, &steps, &ks);
     GLQH_REQUIRE(fi_mode != 0, "trellis group: shape not eligible");
     const size_t need = align256((size_t)ks * B * total * sizeof(float));
     GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
-    float *parts[GLQH_MAX_SHARDS];
     float *p = (float *)ws;
     for (int i = 0; i < n_shards; ++i) {
-        parts[i] = p;
-        p += (size_t)ks * B * m_pads[i];
+        c->parts[i] = p;
+        p += (size_t)ks * B * c->m_pads[i];
     }
+    c->R = R; c->ks = ks; c->fi_mode = fi_mode;
+    if (fi_mode == 2)
+        return glqh_launch_trellis_mma_fusein(packed, sv, c->parts, c->m_pads, n_shards, R, x, x_dtype, x_stride, B,
+                                              n_pad, in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st);
+    return glqh_launch_trellis_fusein_group(packed, sv, c->parts, c->m_pads, n_shards, R, x, x_dtype, x_stride, B,
+                                            n_pad, in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st);
+}
+
+extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                                     const glqh_trellis_shard *shards, int n_shards,
+                                                     const int64_t *blocks_n, int64_t n_blocks_n,
+                                                     const glqh_block_meta *bn_meta_dev, int64_t in_features,
+                                                     int64_t n_pad, int y_dtype, int64_t y_stride, void *ws,
+                                                     size_t ws_bytes, void *stream) {
+    GLQH_INIT();
     hipStream_t st = (hipStream_t)stream;
-    if (fi_mode == 2) {
-        if (glqh_launch_trellis_mma_fusein(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B, n_pad,
-                                           in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
-            return 1;
-    } else if (glqh_launch_trellis_fusein_group(packed, sv, parts, m_pads, n_shards, R, x, x_dtype, x_stride, B,
-                                                n_pad, in_features, steps, ks, bn_meta_dev, blocks_n,
-                                                (int)n_blocks_n, st))
+    tr_group_ctx c;
+    if (tr_group_decode(x, x_dtype, x_stride, B, shards, n_shards, blocks_n, n_blocks_n, bn_meta_dev, in_features,
+                        n_pad, ws, ws_bytes, st, &c))
         return 1;
     if (!shards[0].y) return 0;                                // decode launch only: partial sums stay in ws
-    return glqh_launch_output_rht_group(parts, su, ys, scale, m_pads, outs, n_shards, y_dtype, y_stride, B, ks, st);
+    return glqh_launch_output_rht_group(c.parts, c.su, c.ys, c.scale, c.m_pads, c.outs, n_shards, y_dtype, y_stride,
+                                        B, c.ks, st);
+}
+
+// ---- batch-1 decode loop: output transform fused with what follows it (glq_decoder_ops.h) ----
+extern "C" int glqh_trellis_linear_add_rmsnorm_bf16(const void *x, int64_t in_features,
+                                                    const glqh_trellis_shard *shard, const int64_t *blocks_n,
+                                                    int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                                                    int64_t n_pad, const void *resid, const void *norm_w,
+                                                    double eps, void *x_out, void *h_out, void *ws,
+                                                    size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(shard && resid && norm_w && x_out && h_out, "linear+add+rmsnorm: null pointer");
+    GLQH_REQUIRE(shard->su_f16 && shard->out_features == shard->m_pad,
+                 "linear+add+rmsnorm: needs su and out_features == m_pad");
+    hipStream_t st = (hipStream_t)stream;
+    glqh_trellis_shard sh = *shard;
+    sh.y = nullptr;
+    tr_group_ctx c;
+    if (tr_group_decode(x, GLQH_BF16, in_features, 1, &sh, 1, blocks_n, n_blocks_n, bn_meta_dev, in_features, n_pad,
+                        ws, ws_bytes, st, &c))
+        return 1;
+    return glqh_launch_out_add_rmsnorm(c.parts[0], c.ks, c.scale[0], c.su[0], c.m_pads[0], resid, norm_w, (float)eps,
+                                       x_out, h_out, st);
+}
+
+extern "C" int glqh_trellis_gate_up_silu_bf16(const void *x, int64_t in_features,
+                                              const glqh_trellis_shard *gate_up, const int64_t *blocks_n,
+                                              int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                                              int64_t n_pad, void *act_out, void *ws, size_t ws_bytes,
+                                              void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(gate_up && act_out, "gate/up+silu: null pointer");
+    GLQH_REQUIRE(gate_up[0].m_pad == gate_up[1].m_pad && gate_up[0].out_features == gate_up[1].out_features &&
+                     gate_up[0].su_f16 && gate_up[1].su_f16,
+                 "gate/up+silu: the two layers must have the same shape and carry su");
+    hipStream_t st = (hipStream_t)stream;
+    glqh_trellis_shard sh[2] = {gate_up[0], gate_up[1]};
+    sh[0].y = sh[1].y = nullptr;
+    tr_group_ctx c;
+    if (tr_group_decode(x, GLQH_BF16, in_features, 1, sh, 2, blocks_n, n_blocks_n, bn_meta_dev, in_features, n_pad,
+                        ws, ws_bytes, st, &c))
+        return 1;
+    return glqh_launch_out_silu_mul(c.parts[0], c.parts[1], c.ks, c.scale[0], c.scale[1], c.su[0], c.su[1],
+                                    c.m_pads[0], c.outs[0], act_out, st);
 }
 
 // ---- E8 shell ------------------------------------------------------------------------

@@ -171,4 +171,11 @@ int glqh_launch_output_rht_group(const float *const part[], const void *const su
                                  const float scale[], const int64_t m_pad[], const int64_t out_features[],
                                  int n_shards, int y_dtype, int64_t y_stride, int64_t B, int ksplit,
                                  hipStream_t stream);
+// decode-loop epilogues (decoder_ops.hip): one token, split-K partials -> output transform -> ...
+int glqh_launch_out_add_rmsnorm(const float *part, int ksplit, float scale, const void *su, int64_t m,
+                                const void *resid, const void *norm_w, float eps, void *x_out, void *h_out,
+                                hipStream_t stream);
+int glqh_launch_out_silu_mul(const float *part_gate, const float *part_up, int ksplit, float scale_gate,
+                             float scale_up, const void *su_gate, const void *su_up, int64_t m_pad,
+                             int64_t out_features, void *act_out, hipStream_t stream);
 int glqh_trellis_init(void);

@@ -3,6 +3,7 @@
 // the end-to-end decode measurement from being dominated by dozens of tiny framework kernels
 // per layer; arithmetic follows the usual Llama-family definitions in fp32 with bf16 storage.
 #include "common.h"
+#include "fht_device.h"
 
 namespace {
 
@@ -202,6 +203,106 @@ silu_mul_kernel(const uint16_t *__restrict__ g, const uint16_t *__restrict__ u, 
     out[i] = f32_to_bf16_bits(s * bf16_bits_to_f32(u[i]));
 }
 
+// ---- output transform fused with what follows it in the decode loop (one token) --------
+// o_proj / down_proj: split-K partial sums -> output transform (whole Hadamard blocks, one
+// after the other) -> x_out = bf16(resid + bf16(y)) -> h_out = RMSNorm(x_out) * w, with the
+// roundings of output_rht + add_rmsnorm_kernel.  One workgroup: the row is 2-8 K values.
+constexpr int FN_THREADS = 1024;
+
+__global__ void __launch_bounds__(FN_THREADS)
+out_add_rmsnorm_kernel(const float *__restrict__ part, int ksplit, float scale, const f16 *__restrict__ su,
+                       int m, const uint16_t *__restrict__ resid, const uint16_t *__restrict__ w, float eps,
+                       uint16_t *__restrict__ x_out, uint16_t *__restrict__ h_out, int row_off) {
+    extern __shared__ float s[];                   // [0, row_off): transform buffer; then m floats: the row
+    __shared__ float red[FN_THREADS / 64];
+    float *row = s + row_off;
+    glqh_ysrc src = {};
+    src.part = part;
+    src.part_kstride = m;
+    src.ksplit = ksplit;
+    src.scale[0] = scale;
+    src.nparts = 1;
+    glqh_meta_args margs;
+    margs.canon = m;
+    const int nb = __builtin_popcount((unsigned)m);
+    float ss = 0.0f;
+    for (int j = 0; j < nb; ++j) {
+        const glqh_block_meta bm = glqh_meta_row(margs, nullptr, j);
+        rht_slice blk;
+        blk.off = bm.offset; blk.bs = bm.bs; blk.log_bs = blk.log_len = bm.log_bs;
+        blk.r = 0; blk.nsub = 1; blk.live = true;
+        blk.norm = rsqrt_pow2(bm.log_bs);
+        stage_partials<FN_THREADS, 2, 8>(s, src, blk, 0, m);
+        fht_staged(s, blk.log_len, lds_writeback{s});
+        __syncthreads();
+        for (int i = threadIdx.x; i < blk.bs; i += FN_THREADS) {
+            const int r = blk.off + i;
+            const float y = bf16_bits_to_f32(f32_to_bf16_bits(s[lds_pad(i)] * (blk.norm * (float)su[r])));
+            const uint16_t sb = f32_to_bf16_bits(bf16_bits_to_f32(resid[r]) + y);
+            x_out[r] = sb;
+            const float v = bf16_bits_to_f32(sb);
+            row[r] = v;
+            ss += v * v;
+        }
+        __syncthreads();                           // s is staged again for the next block
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < FN_THREADS / 64; ++i) tot += red[i];
+    const float r = rsqrtf(tot / (float)m + eps);
+    for (int i = threadIdx.x; i < m; i += FN_THREADS) {
+        const float nrm = bf16_bits_to_f32(f32_to_bf16_bits(row[i] * r));
+        h_out[i] = f32_to_bf16_bits(nrm * bf16_bits_to_f32(w[i]));
+    }
+}
+
+// gate_proj / up_proj: both layers' partial sums -> the two output transforms, slice by slice
+// as output_rht_group_kernel cuts them -> act = bf16(bf16(silu(bf16 gate)) * bf16 up), the
+// roundings of output_rht_group_kernel + silu_mul_kernel (bit-identical to the two launches).
+__global__ void __launch_bounds__(256)
+out_silu_mul_kernel(const float *__restrict__ part_g, const float *__restrict__ part_u, int ksplit, float sc_g,
+                    float sc_u, const f16 *__restrict__ su_g, const f16 *__restrict__ su_u, int m_pad,
+                    int out_features, uint16_t *__restrict__ act, int spb, int log_slice) {
+    extern __shared__ float s[];
+    glqh_meta_args margs;
+    margs.canon = m_pad;
+    const rht_slice blk = rht_get_slice(nullptr, margs, 0.0f, spb, log_slice);
+    if (!blk.live) return;
+    const int len = 1 << blk.log_len;
+    const int base = blk.off + (blk.r << blk.log_len);
+    float g[4];                                    // len <= 1024: at most 4 values per thread
+#pragma unroll
+    for (int layer = 0; layer < 2; ++layer) {
+        glqh_ysrc src = {};
+        src.part = layer ? part_u : part_g;
+        src.part_kstride = m_pad;
+        src.ksplit = ksplit;
+        src.scale[0] = layer ? sc_u : sc_g;
+        src.nparts = 1;
+        const f16 *su = layer ? su_u : su_g;
+        stage_partials<256, 4, 8>(s, src, blk, 0, m_pad);
+        fht_staged(s, blk.log_len, lds_writeback{s});
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < len) {
+                const float y = bf16_bits_to_f32(f32_to_bf16_bits(s[lds_pad(i)] * (blk.norm * (float)su[base + i])));
+                if (layer == 0) g[u] = y;
+                else if (base + i < out_features) {
+                    const float a = g[u];
+                    const float sl = bf16_bits_to_f32(f32_to_bf16_bits(a / (1.0f + __expf(-a))));
+                    act[base + i] = f32_to_bf16_bits(sl * y);
+                }
+            }
+        }
+        __syncthreads();                           // s is staged again for the second layer
+    }
+}
+
 }  // namespace
 
 extern "C" int glqh_rmsnorm_bf16(const void *x, const void *w, void *out, int64_t T, int64_t H, double eps,
@@ -261,5 +362,40 @@ extern "C" int glqh_silu_mul_bf16(const void *gate, const void *up, void *out, i
     hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                        (const uint16_t *)gate, (const uint16_t *)up, (uint16_t *)out, n);
     GLQH_LAUNCH_CHECK("silu_mul launch");
+    return 0;
+}
+
+int glqh_launch_out_add_rmsnorm(const float *part, int ksplit, float scale, const void *su, int64_t m,
+                                const void *resid, const void *norm_w, float eps, void *x_out, void *h_out,
+                                hipStream_t stream) {
+    GLQH_REQUIRE(part && su && resid && norm_w && x_out && h_out && ksplit >= 1, "out+add+rmsnorm: bad arguments");
+    GLQH_REQUIRE(m >= 32 && m <= 8192, "out+add+rmsnorm: %lld rows (32..8192)", (long long)m);
+    int64_t top = 1;
+    while (top * 2 <= m) top *= 2;
+    const int row_off = (int)(top + top / 32 + 32);
+    const size_t lds = (size_t)(row_off + m) * sizeof(float);
+    hipLaunchKernelGGL(out_add_rmsnorm_kernel, dim3(1), dim3(FN_THREADS), lds, stream, part, ksplit, scale,
+                       (const f16 *)su, (int)m, (const uint16_t *)resid, (const uint16_t *)norm_w, eps,
+                       (uint16_t *)x_out, (uint16_t *)h_out, row_off);
+    GLQH_LAUNCH_CHECK("out+add+rmsnorm launch");
+    return 0;
+}
+
+int glqh_launch_out_silu_mul(const float *part_gate, const float *part_up, int ksplit, float scale_gate,
+                             float scale_up, const void *su_gate, const void *su_up, int64_t m_pad,
+                             int64_t out_features, void *act_out, hipStream_t stream) {
+    GLQH_REQUIRE(part_gate && part_up && su_gate && su_up && act_out && ksplit >= 1, "out+silu: bad arguments");
+    GLQH_REQUIRE(m_pad >= 32 && m_pad <= 0x40000000ll && out_features >= 1 && out_features <= m_pad,
+                 "out+silu: bad shape");
+    int64_t top = 1;
+    while (top * 2 <= m_pad) top *= 2;
+    const int log_slice = 10;                      // the slices of the few-token output transform
+    const int spb = top >> log_slice < 1 ? 1 : (int)(top >> log_slice);
+    const int nwg = __builtin_popcountll((unsigned long long)m_pad) * spb;
+    const size_t lds = (size_t)((1 << log_slice) + (1 << log_slice) / 32 + 32) * sizeof(float);
+    hipLaunchKernelGGL(out_silu_mul_kernel, dim3((unsigned)nwg), dim3(256), lds, stream, part_gate, part_up, ksplit,
+                       scale_gate, scale_up, (const f16 *)su_gate, (const f16 *)su_up, (int)m_pad, (int)out_features,
+                       (uint16_t *)act_out, spb, log_slice);
+    GLQH_LAUNCH_CHECK("out+silu launch");
     return 0;
 }

@@ -13,94 +13,6 @@ namespace {
 #endif
 constexpr int RHT_THREADS = GLQH_RHT_THREADS;
 
-struct rht_slice {
-    int off, bs, log_bs;     // the Hadamard block
-    int log_len, r, nsub;    // this workgroup's slice: len = 2^log_len, index r of nsub
-    float norm;
-    bool live;
-};
-
-// blockIdx.x = block * spb + slice; workgroups past a block's slice count retire.
-__device__ __forceinline__ rht_slice rht_get_slice(const glqh_block_meta *meta, const glqh_meta_args margs,
-                                                   float single_norm, int spb, int log_slice) {
-    const int j = blockIdx.x / spb;
-    glqh_block_meta mrow = glqh_meta_row(margs, meta, j);
-    rht_slice b;
-    b.off = mrow.offset;
-    b.bs = mrow.bs;
-    b.log_bs = mrow.log_bs;
-    b.log_len = min(mrow.log_bs, log_slice);
-    b.nsub = mrow.bs >> b.log_len;
-    b.r = blockIdx.x % spb;
-    b.live = b.r < b.nsub;
-    if (mrow.w != 0) b.norm = __builtin_bit_cast(float, mrow.w);
-    else if ((margs.canon & (margs.canon - 1)) == 0 && margs.canon != 0 && single_norm != 0.0f) b.norm = single_norm;
-    else b.norm = rsqrt_pow2(mrow.log_bs);
-    return b;
-}
-
-// Split-K partials -> LDS.  Element e of the block is v(e) = sum_stage scale * (sum_k
-// partial), summed in this fixed order (the same order as the stand-alone reduction, so
-// both give the same bits); slice r needs sum_h sign(r,h) v(h*len + i).  The (h, stage, k)
-// terms are walked as one flat sequence so that C terms x U elements of loads are in flight.
-template <int U, int C>
-__device__ __forceinline__ void stage_partials(float *s, const glqh_ysrc &src, const rht_slice &blk,
-                                           int64_t b, int m_pad) {
-    const int len = 1 << blk.log_len;
-    const int ks = src.ksplit, nst = src.nparts;
-    const int total = blk.nsub * nst * ks;
-    const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
-    for (int i0 = threadIdx.x; i0 < len; i0 += U * RHT_THREADS) {
-        float z[U], v[U], acc[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) z[u] = v[u] = acc[u] = 0.0f;
-        int h = 0, st = 0, k = 0;                       // position of term t0 (uniform)
-        for (int t0 = 0; t0 < total; t0 += C) {
-            float vals[C][U];
-            int hh = h, ss = st, kk = k;
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
-#pragma unroll
-                for (int u = 0; u < U; ++u) vals[c][u] = p[min(i0 + u * RHT_THREADS, len - 1)];
-                if (t0 + c + 1 < total) {               // advance, clamped at the last term
-                    if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                if (t0 + c < total) {
-#pragma unroll
-                    for (int u = 0; u < U; ++u) acc[u] += vals[c][u];
-                    if (++k == ks) {
-                        const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
-                                       : st == 2 ? src.scale[2] : src.scale[3];
-#pragma unroll
-                        for (int u = 0; u < U; ++u) { v[u] += sc * acc[u]; acc[u] = 0.0f; }
-                        k = 0;
-                        if (++st == nst) {
-#pragma unroll
-                            for (int u = 0; u < U; ++u) {
-                                const int i = i0 + u * RHT_THREADS;
-                                if (src.copy_out && blk.r == 0 && i < len)
-                                    src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i] = v[u];
-                                z[u] += had_sign(blk.r, h, v[u]);
-                                v[u] = 0.0f;
-                            }
-                            st = 0;
-                            ++h;
-                        }
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (i0 + u * RHT_THREADS < len) s[lds_pad(i0 + u * RHT_THREADS)] = z[u];
-    }
-    __syncthreads();
-}
-
 // XT / OT: element types (bf16 travels as uint16_t)
 template <typename XT, typename OT>
 __global__ void __launch_bounds__(RHT_THREADS)
@@ -182,12 +94,6 @@ template <> __device__ __forceinline__ void store8<uint16_t>(uint16_t *p, const 
         w[e] = (uint32_t)f32_to_bf16_bits(f[2 * e]) | ((uint32_t)f32_to_bf16_bits(f[2 * e + 1]) << 16);
     *(u32x4 *)p = w;
 }
-
-struct lds_writeback {                                   // last pass: results stay in LDS
-    float *lds;
-    __device__ float aux(int) const { return 0.0f; }
-    __device__ void put(int i, float v, float) const { lds[lds_pad(i)] = v; }
-};
 
 // blockIdx.x = block, blockIdx.y = token.  Requires canonical blocks of 8..8192 points, 16-byte
 // aligned rows of x (x_stride % 8 == 0 elements for 16-bit types) and out.
@@ -331,8 +237,8 @@ output_rht_body(const glqh_ysrc &src, const f16 *__restrict__ su, YT *__restrict
         else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
     } else {
         const int total = blk.nsub * src.nparts * src.ksplit;
-        if (total == 1 && blk.log_len >= 11) stage_partials<8, 1>(s, src, blk, b, m_pad);
-        else stage_partials<4, 8>(s, src, blk, b, m_pad);
+        if (total == 1 && blk.log_len >= 11) stage_partials<RHT_THREADS, 8, 1>(s, src, blk, b, m_pad);
+        else stage_partials<RHT_THREADS, 4, 8>(s, src, blk, b, m_pad);
     }
     const int base = blk.off + (blk.r << blk.log_len);
     struct {

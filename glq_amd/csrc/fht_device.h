@@ -109,6 +109,12 @@ __device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store) {
     }
 }
 
+struct lds_writeback {                                   // last pass: results stay in LDS
+    float *lds;
+    __device__ float aux(int) const { return 0.0f; }
+    __device__ void put(int i, float v, float) const { lds[lds_pad(i)] = v; }
+};
+
 // sign of element (r, h) of the Sylvester matrix
 __device__ __forceinline__ float had_sign(int r, int h, float v) {
     return (__builtin_popcount(r & h) & 1) ? -v : v;
@@ -199,6 +205,76 @@ __device__ __forceinline__ void stage_signed_input_quads(float *lds, int log_len
     __syncthreads();
 }
 
+// One workgroup's share of an output transform: the Hadamard block and the slice of it.
+struct rht_slice {
+    int off, bs, log_bs;     // the Hadamard block
+    int log_len, r, nsub;    // this workgroup's slice: len = 2^log_len, index r of nsub
+    float norm;
+    bool live;
+};
+
+// Split-K partials -> LDS.  Element e of the block is v(e) = sum_stage scale * (sum_k
+// partial), summed in this fixed order (the same order as the stand-alone reduction, so
+// both give the same bits); slice r needs sum_h sign(r,h) v(h*len + i).  The (h, stage, k)
+// terms are walked as one flat sequence so that C terms x U elements of loads are in flight.
+template <int T, int U, int C>
+__device__ __forceinline__ void stage_partials(float *s, const glqh_ysrc &src, const rht_slice &blk,
+                                           int64_t b, int m_pad) {
+    const int len = 1 << blk.log_len;
+    const int ks = src.ksplit, nst = src.nparts;
+    const int total = blk.nsub * nst * ks;
+    const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
+    for (int i0 = threadIdx.x; i0 < len; i0 += U * T) {
+        float z[U], v[U], acc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) z[u] = v[u] = acc[u] = 0.0f;
+        int h = 0, st = 0, k = 0;                       // position of term t0 (uniform)
+        for (int t0 = 0; t0 < total; t0 += C) {
+            float vals[C][U];
+            int hh = h, ss = st, kk = k;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
+#pragma unroll
+                for (int u = 0; u < U; ++u) vals[c][u] = p[min(i0 + u * T, len - 1)];
+                if (t0 + c + 1 < total) {               // advance, clamped at the last term
+                    if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                if (t0 + c < total) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) acc[u] += vals[c][u];
+                    if (++k == ks) {
+                        const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
+                                       : st == 2 ? src.scale[2] : src.scale[3];
+#pragma unroll
+                        for (int u = 0; u < U; ++u) { v[u] += sc * acc[u]; acc[u] = 0.0f; }
+                        k = 0;
+                        if (++st == nst) {
+#pragma unroll
+                            for (int u = 0; u < U; ++u) {
+                                const int i = i0 + u * T;
+                                if (src.copy_out && blk.r == 0 && i < len)
+                                    src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i] = v[u];
+                                z[u] += had_sign(blk.r, h, v[u]);
+                                v[u] = 0.0f;
+                            }
+                            st = 0;
+                            ++h;
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (i0 + u * T < len) s[lds_pad(i0 + u * T)] = z[u];
+    }
+    __syncthreads();
+}
+
 template <typename T> __device__ __forceinline__ float act_to_f32(T v);
 template <> __device__ __forceinline__ float act_to_f32<f16>(f16 v) { return (float)v; }
 template <> __device__ __forceinline__ float act_to_f32<uint16_t>(uint16_t v) { return bf16_bits_to_f32(v); }
@@ -212,3 +288,23 @@ template <> __device__ __forceinline__ float f32_to_act<float>(float v) { return
 __device__ __forceinline__ float rsqrt_pow2(int log_bs) {
     return ldexpf((log_bs & 1) ? 0.70710678118654752f : 1.0f, -(log_bs >> 1));
 }
+
+// blockIdx.x = block * spb + slice; workgroups past a block's slice count retire.
+__device__ __forceinline__ rht_slice rht_get_slice(const glqh_block_meta *meta, const glqh_meta_args margs,
+                                                   float single_norm, int spb, int log_slice) {
+    const int j = blockIdx.x / spb;
+    glqh_block_meta mrow = glqh_meta_row(margs, meta, j);
+    rht_slice b;
+    b.off = mrow.offset;
+    b.bs = mrow.bs;
+    b.log_bs = mrow.log_bs;
+    b.log_len = min(mrow.log_bs, log_slice);
+    b.nsub = mrow.bs >> b.log_len;
+    b.r = blockIdx.x % spb;
+    b.live = b.r < b.nsub;
+    if (mrow.w != 0) b.norm = __builtin_bit_cast(float, mrow.w);
+    else if ((margs.canon & (margs.canon - 1)) == 0 && margs.canon != 0 && single_norm != 0.0f) b.norm = single_norm;
+    else b.norm = rsqrt_pow2(mrow.log_bs);
+    return b;
+}
+

@@ -13,6 +13,7 @@ captured once in a HIP graph and replayed per token; position and token live on 
 """
 from __future__ import annotations
 
+import ctypes as C
 import time
 from dataclasses import dataclass
 
@@ -71,6 +72,46 @@ def _group(x, lins):
         out_dtype=torch.bfloat16)
 
 
+def _shard_array(lins):
+    arr = (ext._TrellisShard * len(lins))()
+    for i, l in enumerate(lins):
+        arr[i] = ext._TrellisShard(l.sv.data_ptr(), l.su.data_ptr(), l.packed.data_ptr(), l.packed.shape[0],
+                                   l.packed.shape[1], float(l.wscale), l.m, l.m, None)
+    return arr
+
+
+def _group_ws(lins, dev):
+    lib = _lib.load()
+    nb = lib.glqh_fused_linear_trellis_group_workspace_bytes(1, lins[0].n, sum(l.m for l in lins), len(lins))
+    return torch.empty(max(int(nb), 256), dtype=torch.uint8, device=dev)
+
+
+def _linear_add_rms_norm(lin, a, x, w, eps):
+    """x_out = x + lin(a); h = RMSNorm(x_out) * w: decode launch + one finishing launch."""
+    x_out, h = torch.empty_like(x), torch.empty_like(x)
+    ws = _group_ws((lin,), x.device)
+    bn, nbn = ext._host_i64(lin.bn)
+    arr = _shard_array((lin,))                                   # kept alive across the call
+    check(_lib.load().glqh_trellis_linear_add_rmsnorm_bf16(
+        a.data_ptr(), lin.n, C.addressof(arr), bn, nbn,
+        lin.bn_meta.data_ptr() if nbn > 1 else None, lin.n, x.data_ptr(), w.data_ptr(), float(eps),
+        x_out.data_ptr(), h.data_ptr(), ws.data_ptr(), ws.numel(), _stream()))
+    return x_out, h
+
+
+def _gate_up_silu(gate, up, h):
+    """act = silu(gate(h)) * up(h): decode launch + one finishing launch."""
+    act = torch.empty(1, gate.m, dtype=torch.bfloat16, device=h.device)
+    ws = _group_ws((gate, up), h.device)
+    bn, nbn = ext._host_i64(gate.bn)
+    arr = _shard_array((gate, up))                               # kept alive across the call
+    check(_lib.load().glqh_trellis_gate_up_silu_bf16(
+        h.data_ptr(), gate.n, C.addressof(arr), bn, nbn,
+        gate.bn_meta.data_ptr() if nbn > 1 else None, gate.n, act.data_ptr(), ws.data_ptr(), ws.numel(),
+        _stream()))
+    return act
+
+
 def _rms_norm(x, w, eps):
     out = torch.empty_like(x)
     check(_lib.load().glqh_rmsnorm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1],
@@ -101,8 +142,11 @@ def _rope(x, cos, sin):                                      # x (T, H, D); cos/
 
 
 class TrellisDecoder:
-    def __init__(self, cfg: DecoderConfig | None = None, device="cuda:0", seed=0, max_len=1024):
+    def __init__(self, cfg: DecoderConfig | None = None, device="cuda:0", seed=0, max_len=1024,
+                 fuse_epilogues=True):
         self.cfg = cfg = cfg or DecoderConfig()
+        # one-token steps finish o / gate+up / down inside the launch that transforms their output
+        self.fuse_epilogues = fuse_epilogues and cfg.hidden <= 6144
         self.dev = dev = torch.device(device)
         self.max_len = max_len
         g = torch.Generator(device=dev).manual_seed(seed)
@@ -142,6 +186,8 @@ class TrellisDecoder:
         lib = _lib.load()
         if delta is None:
             h = _rms_norm(x, L["ln1"], cfg.rms_eps)
+        elif isinstance(delta, tuple):                           # (layer, its input): not applied yet
+            x, h = _linear_add_rms_norm(delta[0], delta[1], x, L["ln1"], cfg.rms_eps)
         else:
             x, h = _add_rms_norm(x, delta, L["ln1"], cfg.rms_eps)
         if T <= 4:
@@ -166,6 +212,10 @@ class TrellisDecoder:
             a = F.scaled_dot_product_attention(qr.view(T, cfg.heads, D).transpose(0, 1)[None], self.kc[li][None],
                                                self.vc[li][None], attn_mask=mask, enable_gqa=True)
             a = a[0].transpose(0, 1).reshape(T, cfg.heads * D)
+        if T == 1 and self.fuse_epilogues:
+            # the output transforms of o / gate+up / down run in the launch that consumes them
+            x, h = _linear_add_rms_norm(L["o"], a, x, L["ln2"], cfg.rms_eps)
+            return x, (L["down"], _gate_up_silu(L["gate"], L["up"], h))
         x, h = _add_rms_norm(x, L["o"](a), L["ln2"], cfg.rms_eps)
         if T == 1:
             gu = _group(h, (L["gate"], L["up"]))
@@ -185,7 +235,10 @@ class TrellisDecoder:
         x, delta = self.emb.index_select(0, ids), None
         for li in range(self.cfg.layers):
             x, delta = self._block(li, x, delta, pos, mask)
-        _, h = _add_rms_norm(x[-1:], delta[-1:], self.ln_f, self.cfg.rms_eps)
+        if isinstance(delta, tuple):
+            _, h = _linear_add_rms_norm(delta[0], delta[1], x, self.ln_f, self.cfg.rms_eps)
+        else:
+            _, h = _add_rms_norm(x[-1:], delta[-1:], self.ln_f, self.cfg.rms_eps)
         return torch.matmul(h, self.emb.t()).float()
 
     def prefill(self, prompt_ids):

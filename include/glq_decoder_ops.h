@@ -11,7 +11,10 @@
 #ifndef GLQ_DECODER_OPS_H
 #define GLQ_DECODER_OPS_H
 
+#include <stddef.h>
 #include <stdint.h>
+
+#include "glq_hip.h"
 
 #ifdef __cplusplus
 extern "C" {
@@ -42,6 +45,30 @@ int glqh_attn_decode_bf16(const void *q, const void *k_cache, const void *v_cach
 
 /* out = bf16(bf16(silu(gate)) * up), n elements. */
 int glqh_silu_mul_bf16(const void *gate, const void *up, void *out, int64_t n, void *stream);
+
+/* One token through a trellis linear whose output is a residual branch (o_proj, down_proj),
+ * finished in the launch that transforms the output:
+ *   y = linear(x);  x_out = bf16(resid + bf16(y));  h_out = RMSNorm(x_out) * norm_w
+ * (the results of glqh_fused_linear_trellis_3inst_group + glqh_add_rmsnorm_bf16 up to fp32
+ * summation order, in two launches instead of three).  x (in_features) bf16; shard as in
+ * glqh_fused_linear_trellis_3inst_group with out_features == m_pad <= ~7000 (its y is
+ * ignored); ws: glqh_fused_linear_trellis_group_workspace_bytes(1, n_pad, m_pad, 1) bytes. */
+int glqh_trellis_linear_add_rmsnorm_bf16(const void *x, int64_t in_features,
+                                         const glqh_trellis_shard *shard, const int64_t *blocks_n,
+                                         int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                                         int64_t n_pad, const void *resid, const void *norm_w,
+                                         double eps, void *x_out, void *h_out, void *ws,
+                                         size_t ws_bytes, void *stream);
+
+/* One token through gate_proj and up_proj (gate_up[0], gate_up[1], same shape) and the gate:
+ *   act = bf16(bf16(silu(bf16 gate(x))) * bf16 up(x)),  act (out_features) bf16
+ * bit-identical to glqh_fused_linear_trellis_3inst_group + glqh_silu_mul_bf16, in two launches
+ * instead of three.  ws: ...group_workspace_bytes(1, n_pad, 2 * m_pad, 2) bytes. */
+int glqh_trellis_gate_up_silu_bf16(const void *x, int64_t in_features,
+                                   const glqh_trellis_shard *gate_up, const int64_t *blocks_n,
+                                   int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                                   int64_t n_pad, void *act_out, void *ws, size_t ws_bytes,
+                                   void *stream);
 
 #ifdef __cplusplus
 }

@@ -95,3 +95,46 @@ def test_glue_ops_match_torch():
     o = torch.empty_like(a)
     _lib.check(lib.glqh_silu_mul_bf16(a.data_ptr(), b.data_ptr(), o.data_ptr(), a.numel(), st))
     assert rel(o, (F.silu(a.float()) * b.float()).cpu().numpy()) < 4e-3
+
+
+@pytest.mark.parametrize("hidden,ffn", [(2048, 11008), (256, 512), (2560, 768)])
+def test_fused_output_epilogues_match_separate_launches(hidden, ffn):
+    """o/down + residual add + RMSNorm and gate/up + SiLU gate finished inside the launch that
+    transforms the linear's output, against the separate launches (same kernels before the
+    output transform).  The gate is bit-identical; the norm path transforms whole blocks
+    where the separate launch uses 1024-point slices, so it agrees to bf16 rounding."""
+    from glq_amd import decoder as D
+    say("fused epilogues", hidden, ffn)
+    g = torch.Generator(device=DEV).manual_seed(hidden)
+    down = D._Linear(hidden, ffn, 4, g, DEV)
+    gate, up = D._Linear(ffn, hidden, 4, g, DEV), D._Linear(ffn, hidden, 4, g, DEV)
+    a = torch.randn(1, ffn, generator=g, device=DEV).to(torch.bfloat16)
+    x = torch.randn(1, hidden, generator=g, device=DEV).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g, device=DEV)).to(torch.bfloat16)
+    x_ref, h_ref = D._add_rms_norm(x, down(a), w, 1e-6)
+    x_out, h = D._linear_add_rms_norm(down, a, x, w, 1e-6)
+    assert rel(x_out, x_ref.float().cpu().numpy()) < 4e-3 and rel(h, h_ref.float().cpu().numpy()) < 6e-3
+    x2, h2 = D._linear_add_rms_norm(down, a, x, w, 1e-6)
+    assert torch.equal(x_out, x2) and torch.equal(h, h2)
+
+    hin = torch.randn(1, hidden, generator=g, device=DEV).to(torch.bfloat16)
+    gu = D._group(hin, (gate, up))
+    act_ref = torch.empty(1, ffn, dtype=torch.bfloat16, device=DEV)
+    D.check(D._lib.load().glqh_silu_mul_bf16(gu[:, :ffn].data_ptr(), gu[:, ffn:].data_ptr(), act_ref.data_ptr(),
+                                             ffn, D._stream()))
+    act = D._gate_up_silu(gate, up, hin)
+    assert torch.equal(act, act_ref)
+
+
+def test_decoder_with_and_without_fused_epilogues():
+    say("decoder fused vs separate")
+    from glq_amd.decoder import DecoderConfig, TrellisDecoder
+    cfg = DecoderConfig(hidden=256, layers=3, heads=2, kv_heads=1, head_dim=128, ffn=512, vocab=1000,
+                        no_rope_interval=2, bits=4)
+    ids = torch.randint(0, 1000, (12,), generator=torch.Generator().manual_seed(1)).to(DEV)
+    outs = []
+    for fuse in (True, False):
+        dec = TrellisDecoder(cfg, device=DEV, seed=3, max_len=64, fuse_epilogues=fuse)
+        dec.prefill(ids)
+        outs.append(dec._step().float())
+    assert rel(outs[0], outs[1].cpu().numpy()) < 2e-2

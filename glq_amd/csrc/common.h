@@ -178,4 +178,8 @@ int glqh_launch_out_add_rmsnorm(const float *part, int ksplit, float scale, cons
 int glqh_launch_out_silu_mul(const float *part_gate, const float *part_up, int ksplit, float scale_gate,
                              float scale_up, const void *su_gate, const void *su_up, int64_t m_pad,
                              int64_t out_features, void *act_out, hipStream_t stream);
+int glqh_launch_out_rope_store(const float *const part[3], const void *const su[3], const float scale[3],
+                               const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
+                               const void *sin_t, void *q_out, void *k_cache, void *v_cache, int64_t head_dim,
+                               int64_t max_len, int apply_rope, hipStream_t stream);
 int glqh_trellis_init(void);

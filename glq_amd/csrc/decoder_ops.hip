@@ -262,44 +262,110 @@ out_add_rmsnorm_kernel(const float *__restrict__ part, int ksplit, float scale, 
 // gate_proj / up_proj: both layers' partial sums -> the two output transforms, slice by slice
 // as output_rht_group_kernel cuts them -> act = bf16(bf16(silu(bf16 gate)) * bf16 up), the
 // roundings of output_rht_group_kernel + silu_mul_kernel (bit-identical to the two launches).
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 out_silu_mul_kernel(const float *__restrict__ part_g, const float *__restrict__ part_u, int ksplit, float sc_g,
                     float sc_u, const f16 *__restrict__ su_g, const f16 *__restrict__ su_u, int m_pad,
-                    int out_features, uint16_t *__restrict__ act, int spb, int log_slice) {
-    extern __shared__ float s[];
+                    int out_features, uint16_t *__restrict__ act, int spb, int log_slice, int buf_floats) {
+    extern __shared__ float s[];                   // two transform buffers, then the gate values
     glqh_meta_args margs;
     margs.canon = m_pad;
     const rht_slice blk = rht_get_slice(nullptr, margs, 0.0f, spb, log_slice);
     if (!blk.live) return;
     const int len = 1 << blk.log_len;
     const int base = blk.off + (blk.r << blk.log_len);
-    float g[4];                                    // len <= 1024: at most 4 values per thread
+    // threads 0..255 transform the gate slice, 256..511 the up slice, side by side
+    const int layer = threadIdx.x >> 8, tid = threadIdx.x & 255;
+    float *buf = s + layer * buf_floats;
+    float *gv = s + 2 * buf_floats;
+    glqh_ysrc src = {};
+    src.part = layer ? part_u : part_g;
+    src.part_kstride = m_pad;
+    src.ksplit = ksplit;
+    src.scale[0] = layer ? sc_u : sc_g;
+    src.nparts = 1;
+    const f16 *su = layer ? su_u : su_g;
+    stage_partials<256, 4, 8>(buf, src, blk, 0, m_pad, tid);
+    fht_staged(buf, blk.log_len, lds_writeback{buf}, tid, 256);
+    __syncthreads();
+    float y[4];
 #pragma unroll
-    for (int layer = 0; layer < 2; ++layer) {
-        glqh_ysrc src = {};
-        src.part = layer ? part_u : part_g;
-        src.part_kstride = m_pad;
-        src.ksplit = ksplit;
-        src.scale[0] = layer ? sc_u : sc_g;
-        src.nparts = 1;
-        const f16 *su = layer ? su_u : su_g;
-        stage_partials<256, 4, 8>(s, src, blk, 0, m_pad);
-        fht_staged(s, blk.log_len, lds_writeback{s});
-        __syncthreads();
+    for (int u = 0; u < 4; ++u) {
+        const int i = tid + 256 * u;
+        y[u] = 0.0f;
+        if (i < len) {
+            y[u] = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(i)] * (blk.norm * (float)su[base + i])));
+            if (layer == 0) gv[i] = y[u];
+        }
+    }
+    __syncthreads();
+    if (layer == 1) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int i = threadIdx.x + 256 * u;
-            if (i < len) {
-                const float y = bf16_bits_to_f32(f32_to_bf16_bits(s[lds_pad(i)] * (blk.norm * (float)su[base + i])));
-                if (layer == 0) g[u] = y;
-                else if (base + i < out_features) {
-                    const float a = g[u];
-                    const float sl = bf16_bits_to_f32(f32_to_bf16_bits(a / (1.0f + __expf(-a))));
-                    act[base + i] = f32_to_bf16_bits(sl * y);
-                }
+            const int i = tid + 256 * u;
+            if (i < len && base + i < out_features) {
+                const float a = gv[i];
+                const float sl = bf16_bits_to_f32(f32_to_bf16_bits(a / (1.0f + __expf(-a))));
+                act[base + i] = f32_to_bf16_bits(sl * y[u]);
             }
         }
-        __syncthreads();                           // s is staged again for the second layer
+    }
+}
+
+// q_proj / k_proj / v_proj (blockIdx.y = layer): output transform slice by slice as
+// output_rht_group_kernel cuts it, then what rope_kv_store_kernel does with the bf16 result:
+// rotate q and k by the angle row of position *pos, q -> q_out, k and v -> cache row *pos.
+// Slices are whole heads (len % D == 0).  Bit-identical to the two separate launches.
+struct qkv_fin {
+    const float *part[3];
+    const f16 *su[3];
+    float scale[3];
+    int m[3];
+};
+
+__global__ void __launch_bounds__(256)
+out_rope_store_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos, const uint16_t *__restrict__ cos_t,
+                      const uint16_t *__restrict__ sin_t, uint16_t *__restrict__ q_out, uint16_t *__restrict__ kc,
+                      uint16_t *__restrict__ vc, int D, int max_len, int apply_rope, int spb, int log_slice) {
+    extern __shared__ float s[];
+    const int z = blockIdx.y;
+    const float *part = z == 0 ? a.part[0] : z == 1 ? a.part[1] : a.part[2];
+    const f16 *su = z == 0 ? a.su[0] : z == 1 ? a.su[1] : a.su[2];
+    const float scale = z == 0 ? a.scale[0] : z == 1 ? a.scale[1] : a.scale[2];
+    const int m = z == 0 ? a.m[0] : z == 1 ? a.m[1] : a.m[2];
+    if ((int)blockIdx.x >= __builtin_popcount((unsigned)m) * spb) return;
+    glqh_meta_args margs;
+    margs.canon = m;
+    const rht_slice blk = rht_get_slice(nullptr, margs, 0.0f, spb, log_slice);
+    if (!blk.live) return;
+    glqh_ysrc src = {};
+    src.part = part;
+    src.part_kstride = m;
+    src.ksplit = ksplit;
+    src.scale[0] = scale;
+    src.nparts = 1;
+    stage_partials<256, 4, 8>(s, src, blk, 0, m);
+    fht_staged(s, blk.log_len, lds_writeback{s});
+    __syncthreads();
+    const int len = 1 << blk.log_len, base = blk.off + (blk.r << blk.log_len), half = D >> 1;
+    const int64_t p = *pos;
+    // y rounded to bf16, as the separate output transform stores it
+    auto yv = [&](int i) { return bf16_bits_to_f32(f32_to_bf16_bits(s[lds_pad(i)] * (blk.norm * (float)su[base + i]))); };
+    for (int e = threadIdx.x; e < len / 2; e += 256) {
+        const int hl = e / half, d = e - hl * half;            // head inside the slice, column pair (d, d + half)
+        const int i0 = hl * D + d, i1 = i0 + half;
+        const int head = (base + i0) / D;
+        const float va = yv(i0), vb = yv(i1);
+        uint16_t *dst = z == 0 ? q_out + (int64_t)head * D
+                      : (z == 1 ? kc : vc) + ((int64_t)head * max_len + p) * D;
+        if (z == 2 || !apply_rope) {
+            dst[d] = f32_to_bf16_bits(va);
+            dst[d + half] = f32_to_bf16_bits(vb);
+        } else {
+            const float c0 = bf16_bits_to_f32(cos_t[p * D + d]), s0 = bf16_bits_to_f32(sin_t[p * D + d]);
+            const float c1 = bf16_bits_to_f32(cos_t[p * D + d + half]), s1 = bf16_bits_to_f32(sin_t[p * D + d + half]);
+            dst[d] = f32_to_bf16_bits(va * c0 - vb * s0);
+            dst[d + half] = f32_to_bf16_bits(vb * c1 + va * s1);
+        }
     }
 }
 
@@ -392,10 +458,44 @@ int glqh_launch_out_silu_mul(const float *part_gate, const float *part_up, int k
     const int log_slice = 10;                      // the slices of the few-token output transform
     const int spb = top >> log_slice < 1 ? 1 : (int)(top >> log_slice);
     const int nwg = __builtin_popcountll((unsigned long long)m_pad) * spb;
-    const size_t lds = (size_t)((1 << log_slice) + (1 << log_slice) / 32 + 32) * sizeof(float);
-    hipLaunchKernelGGL(out_silu_mul_kernel, dim3((unsigned)nwg), dim3(256), lds, stream, part_gate, part_up, ksplit,
+    const int buf_floats = (1 << log_slice) + (1 << log_slice) / 32 + 32;
+    const size_t lds = (size_t)(2 * buf_floats + (1 << log_slice)) * sizeof(float);
+    hipLaunchKernelGGL(out_silu_mul_kernel, dim3((unsigned)nwg), dim3(512), lds, stream, part_gate, part_up, ksplit,
                        scale_gate, scale_up, (const f16 *)su_gate, (const f16 *)su_up, (int)m_pad, (int)out_features,
-                       (uint16_t *)act_out, spb, log_slice);
+                       (uint16_t *)act_out, spb, log_slice, buf_floats);
     GLQH_LAUNCH_CHECK("out+silu launch");
+    return 0;
+}
+
+int glqh_launch_out_rope_store(const float *const part[3], const void *const su[3], const float scale[3],
+                               const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
+                               const void *sin_t, void *q_out, void *k_cache, void *v_cache, int64_t head_dim,
+                               int64_t max_len, int apply_rope, hipStream_t stream) {
+    GLQH_REQUIRE(pos && q_out && k_cache && v_cache && ksplit >= 1, "out+rope: bad arguments");
+    GLQH_REQUIRE(!apply_rope || (cos_t && sin_t), "out+rope: missing angle tables");
+    GLQH_REQUIRE(head_dim >= 2 && (head_dim & (head_dim - 1)) == 0 && head_dim <= 1024, "out+rope: bad head_dim");
+    const int log_slice = 10;
+    qkv_fin a = {};
+    int64_t top_max = 1;
+    int max_nwg = 0;
+    for (int i = 0; i < 3; ++i) {
+        GLQH_REQUIRE(part[i] && su[i] && m[i] >= head_dim && m[i] <= 0x40000000ll && m[i] % head_dim == 0,
+                     "out+rope: layer %d: rows must be whole heads", i);
+        GLQH_REQUIRE((m[i] & (head_dim - 1)) == 0, "out+rope: every output block must hold whole heads");
+        a.part[i] = part[i]; a.su[i] = (const f16 *)su[i]; a.scale[i] = scale[i]; a.m[i] = (int)m[i];
+        int64_t top = 1;
+        while (top * 2 <= m[i]) top *= 2;
+        if (top > top_max) top_max = top;
+    }
+    const int spb = top_max >> log_slice < 1 ? 1 : (int)(top_max >> log_slice);
+    for (int i = 0; i < 3; ++i) {
+        const int nwg = __builtin_popcountll((unsigned long long)m[i]) * spb;
+        if (nwg > max_nwg) max_nwg = nwg;
+    }
+    const size_t lds = (size_t)((1 << log_slice) + (1 << log_slice) / 32 + 32) * sizeof(float);
+    hipLaunchKernelGGL(out_rope_store_kernel, dim3((unsigned)max_nwg, 3), dim3(256), lds, stream, a, ksplit, pos,
+                       (const uint16_t *)cos_t, (const uint16_t *)sin_t, (uint16_t *)q_out, (uint16_t *)k_cache,
+                       (uint16_t *)v_cache, (int)head_dim, (int)max_len, apply_rope, spb, log_slice);
+    GLQH_LAUNCH_CHECK("out+rope launch");
     return 0;
 }

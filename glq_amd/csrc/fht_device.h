@@ -38,10 +38,10 @@ constexpr int LOG_SLICE = GLQH_LOG_SLICE;
 __device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
 
 template <int R, bool LAST, class Store>
-__device__ __forceinline__ void fht_pass(float *lds, int n, int s, Store &store) {
+__device__ __forceinline__ void fht_pass(float *lds, int n, int s, Store &store, int tid, int nthr) {
     constexpr int N = 1 << R;
     const int ngroups = n >> R;
-    for (int g = threadIdx.x; g < ngroups; g += blockDim.x) {
+    for (int g = tid; g < ngroups; g += nthr) {
         const int lo = g & ((1 << s) - 1);
         const int base = ((g >> s) << (s + R)) | lo;
         float v[N], aux[N];
@@ -72,27 +72,30 @@ __device__ __forceinline__ void fht_pass(float *lds, int n, int s, Store &store)
 }
 
 template <bool LAST, class Store>
-__device__ __forceinline__ void fht_pass_r(int r, float *lds, int n, int s, Store &store) {
+__device__ __forceinline__ void fht_pass_r(int r, float *lds, int n, int s, Store &store, int tid, int nthr) {
     switch (r) {
-    case 1: fht_pass<1, LAST>(lds, n, s, store); break;
-    case 2: fht_pass<2, LAST>(lds, n, s, store); break;
-    case 3: fht_pass<3, LAST>(lds, n, s, store); break;
+    case 1: fht_pass<1, LAST>(lds, n, s, store, tid, nthr); break;
+    case 2: fht_pass<2, LAST>(lds, n, s, store, tid, nthr); break;
+    case 3: fht_pass<3, LAST>(lds, n, s, store, tid, nthr); break;
 #if GLQH_RMAX >= 5
-    case 4: fht_pass<4, LAST>(lds, n, s, store); break;
-    default: fht_pass<5, LAST>(lds, n, s, store); break;
+    case 4: fht_pass<4, LAST>(lds, n, s, store, tid, nthr); break;
+    default: fht_pass<5, LAST>(lds, n, s, store, tid, nthr); break;
 #else
-    default: fht_pass<4, LAST>(lds, n, s, store); break;
+    default: fht_pass<4, LAST>(lds, n, s, store, tid, nthr); break;
 #endif
     }
 }
 
 // Transform lds[0 .. 2^log_n) (padded layout, already staged and visible to the whole
 // workgroup) and pass the result to `store`.  All threads of the workgroup must call it.
+// A workgroup may run several transforms of the same size side by side: each group of nthr
+// threads (numbered tid = 0..nthr-1) passes its own buffer; the barriers are shared.
 template <class Store>
-__device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store) {
+__device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store, int tid = threadIdx.x,
+                                           int nthr = blockDim.x) {
     const int n = 1 << log_n;
     if (log_n == 0) {
-        if (threadIdx.x == 0) store.put(0, lds[0], store.aux(0));
+        if (tid == 0) store.put(0, lds[0], store.aux(0));
         return;
     }
     const int npass = (log_n + RMAX - 1) / RMAX;
@@ -101,9 +104,9 @@ __device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store) {
         const int left = npass - p;
         const int r = (s + left - 1) / left;              // balanced field widths
         s -= r;
-        if (p == npass - 1) fht_pass_r<true>(r, lds, n, s, store);
+        if (p == npass - 1) fht_pass_r<true>(r, lds, n, s, store, tid, nthr);
         else {
-            fht_pass_r<false>(r, lds, n, s, store);
+            fht_pass_r<false>(r, lds, n, s, store, tid, nthr);
             __syncthreads();
         }
     }
@@ -219,12 +222,12 @@ struct rht_slice {
 // terms are walked as one flat sequence so that C terms x U elements of loads are in flight.
 template <int T, int U, int C>
 __device__ __forceinline__ void stage_partials(float *s, const glqh_ysrc &src, const rht_slice &blk,
-                                           int64_t b, int m_pad) {
+                                           int64_t b, int m_pad, int tid = threadIdx.x) {
     const int len = 1 << blk.log_len;
     const int ks = src.ksplit, nst = src.nparts;
     const int total = blk.nsub * nst * ks;
     const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
-    for (int i0 = threadIdx.x; i0 < len; i0 += U * T) {
+    for (int i0 = tid; i0 < len; i0 += U * T) {
         float z[U], v[U], acc[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) z[u] = v[u] = acc[u] = 0.0f;

@@ -70,6 +70,19 @@ int glqh_trellis_gate_up_silu_bf16(const void *x, int64_t in_features,
                                    int64_t n_pad, void *act_out, void *ws, size_t ws_bytes,
                                    void *stream);
 
+/* One token through q_proj, k_proj, v_proj (qkv[0..2], out_features == m_pad, rows = whole heads of
+ * head_dim, every Hadamard block of m_pad at least one head) and glqh_rope_kv_store_bf16 in the
+ * launch that transforms their outputs: q rotated -> q_out (heads, D); k rotated and v -> cache
+ * row *pos.  Bit-identical to glqh_fused_linear_trellis_3inst_group + glqh_rope_kv_store_bf16.
+ * ws: ...group_workspace_bytes(1, n_pad, sum of m_pad, 3) bytes. */
+int glqh_trellis_qkv_rope_store_bf16(const void *x, int64_t in_features, const glqh_trellis_shard *qkv,
+                                     const int64_t *blocks_n, int64_t n_blocks_n,
+                                     const glqh_block_meta *bn_meta_dev, int64_t n_pad,
+                                     const int64_t *pos, const void *cos_t, const void *sin_t,
+                                     void *q_out, void *k_cache, void *v_cache, int64_t head_dim,
+                                     int64_t max_len, int apply_rope, void *ws, size_t ws_bytes,
+                                     void *stream);
+
 #ifdef __cplusplus
 }
 #endif

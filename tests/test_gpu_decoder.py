@@ -138,3 +138,32 @@ def test_decoder_with_and_without_fused_epilogues():
         dec.prefill(ids)
         outs.append(dec._step().float())
     assert rel(outs[0], outs[1].cpu().numpy()) < 2e-2
+
+
+@pytest.mark.parametrize("rope", [1, 0])
+def test_fused_qkv_rope_store_is_bit_identical(rope):
+    from glq_amd import decoder as D
+    say("fused qkv rope", rope)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    hidden, heads, kvh, hd, L = 2048, 16, 4, 128, 64
+    q, k, v = (D._Linear(heads * hd, hidden, 4, g, DEV), D._Linear(kvh * hd, hidden, 4, g, DEV),
+               D._Linear(kvh * hd, hidden, 4, g, DEV))
+    h = torch.randn(1, hidden, generator=g, device=DEV).to(torch.bfloat16)
+    pos = torch.tensor([37], device=DEV)
+    inv = 1.0 / (2e6 ** (torch.arange(0, hd, 2, device=DEV, dtype=torch.float32) / hd))
+    ang = torch.arange(L, device=DEV, dtype=torch.float32)[:, None] * inv[None]
+    ang = torch.cat((ang, ang), -1)
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+    lib = D._lib.load()
+    qkv = D._group(h, (q, k, v))
+    nq, nk = q.m, k.m
+    qr0 = torch.zeros(1, nq, dtype=torch.bfloat16, device=DEV)
+    kc0 = torch.zeros(kvh, L, hd, dtype=torch.bfloat16, device=DEV)
+    vc0 = torch.zeros_like(kc0)
+    D.check(lib.glqh_rope_kv_store_bf16(qkv[:, :nq].data_ptr(), qkv[:, nq:nq + nk].data_ptr(), qkv[:, nq + nk:].data_ptr(),
+                                        pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), qr0.data_ptr(), kc0.data_ptr(),
+                                        vc0.data_ptr(), 1, heads, kvh, hd, L, rope, D._stream()))
+    qr1, kc1, vc1 = torch.zeros_like(qr0), torch.zeros_like(kc0), torch.zeros_like(vc0)
+    D._qkv_rope_store(q, k, v, h, pos, cos, sin, qr1, kc1, vc1, hd, L, rope)
+    assert torch.count_nonzero(qr0) > 0 and torch.count_nonzero(kc0[:, 37]) > 0
+    assert torch.equal(qr0, qr1) and torch.equal(kc0, kc1) and torch.equal(vc0, vc1)

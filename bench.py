@@ -212,6 +212,67 @@ def extras(torch, ext, dev):
     return out
 
 
+CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "e8_gemv_2stage", "decoder")
+
+
+def run_case(torch, ext, dev, name, steps):
+    """One side measurement alone, `steps` launches back to back (eager, so that a profiler
+    sees plain kernel dispatches): the command behind the per-kernel summaries in profiles/."""
+    import time
+    res = {"case": name, "steps": steps}
+    if name == "trellis_gemv_16384":
+        m = n = 16384
+        packs = [torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
+                 for _ in range(4)]
+        xh = torch.randn(1, n, device=dev).to(torch.float16)
+        pb = torch.empty(64 * m, dtype=torch.float32, device=dev)
+        fn = lambda i: ext.trellis_gemv_partials(xh, packs[i % 4], m, n, pb)
+        res["bytes_per_launch"] = m * n // 2
+    elif name == "trellis_prefill_4096":
+        m, n, M = 14336, 4096, 4096
+        p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
+        xh = torch.randn(M, n, device=dev).to(torch.float16)
+        o = torch.empty(M, m, dtype=torch.float32, device=dev)
+        fn = lambda i: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o)
+        res["flop_per_launch"] = 2.0 * M * m * n
+    elif name == "e8_gemv_2stage":
+        from glq_amd.checkpoint import load_shell_table
+        cb = load_shell_table(None).to(dev)
+        m, n = 4096, 14336
+        W = torch.randn(m * (n // 8), 8, device=dev)
+        d1, i1 = ext.e8_quantize(W, cb)
+        _, i2 = ext.e8_quantize((W - d1) * 3.0, cb)
+        del W, d1
+
+        def to16(i):
+            return (i.to(torch.int32) - ((i >= 32768).to(torch.int32) << 16)).to(torch.int16).reshape(m, n // 8)
+        qs = [(to16(i1.roll(r * 977)).contiguous(), to16(i2.roll(r * 977)).contiguous()) for r in range(4)]
+        xh = torch.randn(1, n, device=dev).to(torch.float16)
+        fn = lambda i: ext.glq_dequant_matmul_cuda(xh, qs[i % 4][0], cb, 0.02, qs[i % 4][1], cb, 1 / 3.0)
+        res["bytes_per_launch"] = m * (n // 8) * 4
+    elif name == "decoder":
+        from glq_amd.decoder import TrellisDecoder
+        dec = TrellisDecoder(max_len=1024)
+        ids = torch.randint(0, 128256, (512,), generator=torch.Generator().manual_seed(0))
+        dec.generate(ids, 4)
+        _, _, t_decode = dec.generate(ids, steps)
+        res["decode_tok_s"] = round(steps / t_decode, 1)
+        print(json.dumps(res), flush=True)
+        return
+    else:
+        raise SystemExit(f"unknown case {name}; one of {CASES}")
+    for i in range(8):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i)
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / steps
+    res["us_per_launch_eager"] = round(us, 2)
+    print(json.dumps(res), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -224,6 +285,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain 256 MiB read + 256 MiB write elementwise kernel three times "
                          "(calibration of the FETCH_SIZE / WRITE_SIZE counters under rocprofv3 --pmc)")
+    ap.add_argument("--case", choices=CASES, default=None,
+                    help="run one side measurement alone (for profiling) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1).")
@@ -237,6 +300,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.case:
+        run_case(torch, ext, dev, args.case, max(1, args.steps if args.steps != 720 else 40))
+        return
     L = max(1, args.layers)
     pool = build_pool(torch, hadamard, L, dev)
     xs = {n: torch.randn(1, n, generator=torch.Generator(device=dev).manual_seed(1), device=dev)

@@ -78,9 +78,9 @@ __global__ void rope_kv_store_kernel(const uint16_t *__restrict__ q, const uint1
 
 // One query token: out[h] = softmax(q[h] . K[g][0..pos] / sqrt(D)) V[g][0..pos], g = h / (heads/kv_heads).
 // One workgroup of 16 waves per head; D = 128; scores live in LDS (max_len floats).
-// Scores: 8 lanes per key with 16-byte loads (128 keys per pass).  Output: lane = column
-// pair, wave = key group, four rows of V in flight per thread; the 16 partial rows are summed
-// through LDS in wave order.
+// Scores: 8 lanes per key with 16-byte loads, four keys per thread in flight.  Output: 16
+// lanes per row of V with 16-byte loads, four rows in flight per thread; the waves' partial rows
+// are summed through LDS in wave order.
 constexpr int AT_THREADS = 1024;
 constexpr int AT_WAVES = AT_THREADS / 64;
 
@@ -102,22 +102,34 @@ attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ 
     const uint16_t *V = vc + (int64_t)g * max_len * D;
     const int sub = threadIdx.x & 7;
     float mx = -3.0e38f;
-    for (int j0 = threadIdx.x >> 3; j0 < n; j0 += AT_THREADS / 8) {
-        const u32x4 k0 = *(const u32x4 *)(K + (int64_t)j0 * D + sub * 8);
-        const u32x4 k1 = *(const u32x4 *)(K + (int64_t)j0 * D + 64 + sub * 8);
-        float s = 0.0f;
+    // four keys per thread in flight (512 keys per round of the workgroup)
+    for (int j0 = threadIdx.x >> 3; j0 < n; j0 += 4 * (AT_THREADS / 8)) {
+        u32x4 k0[4], k1[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            s += qs[sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k0[e] & 0xFFFFu));
-            s += qs[sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k0[e] >> 16));
-            s += qs[64 + sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k1[e] & 0xFFFFu));
-            s += qs[64 + sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k1[e] >> 16));
+        for (int u = 0; u < 4; ++u) {
+            const int j = min(j0 + u * (AT_THREADS / 8), n - 1);
+            k0[u] = *(const u32x4 *)(K + (int64_t)j * D + sub * 8);
+            k1[u] = *(const u32x4 *)(K + (int64_t)j * D + 64 + sub * 8);
         }
-        s += __shfl_xor(s, 1, GLQH_WAVE);
-        s += __shfl_xor(s, 2, GLQH_WAVE);
-        s += __shfl_xor(s, 4, GLQH_WAVE);
-        if (sub == 0) sc[j0] = s;
-        mx = fmaxf(mx, s);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = j0 + u * (AT_THREADS / 8);
+            float s = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                s += qs[sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k0[u][e] & 0xFFFFu));
+                s += qs[sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k0[u][e] >> 16));
+                s += qs[64 + sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k1[u][e] & 0xFFFFu));
+                s += qs[64 + sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k1[u][e] >> 16));
+            }
+            s += __shfl_xor(s, 1, GLQH_WAVE);
+            s += __shfl_xor(s, 2, GLQH_WAVE);
+            s += __shfl_xor(s, 4, GLQH_WAVE);
+            if (j < n) {
+                if (sub == 0) sc[j] = s;
+                mx = fmaxf(mx, s);
+            }
+        }
     }
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
@@ -138,25 +150,38 @@ attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ 
     float tot = 0.0f;
 #pragma unroll
     for (int w = 0; w < AT_WAVES; ++w) tot += red[w];
-    // weighted rows of V: wave = key group, lane = columns (2 lane, 2 lane + 1)
-    float a0 = 0.0f, a1 = 0.0f;
-    for (int j0 = wave; j0 < n; j0 += 4 * AT_WAVES) {
-        uint32_t vv[4];
+    // weighted rows of V: 16 lanes per row (8 columns, one 16-byte load each), 4 rows per wave
+    // per load and four loads in flight: 256 keys per round of the workgroup
+    const int vr = lane >> 4, vcol = lane & 15;
+    float a[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[e] = 0.0f;
+    for (int j0 = wave * 4 + vr; j0 < n; j0 += 4 * 4 * AT_WAVES) {
+        u32x4 vv[4];
         float pw[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int j = j0 + u * AT_WAVES;
-            vv[u] = *(const uint32_t *)(V + (int64_t)min(j, n - 1) * D + 2 * lane);
+            const int j = j0 + u * 4 * AT_WAVES;
+            vv[u] = *(const u32x4 *)(V + (int64_t)min(j, n - 1) * D + 8 * vcol);
             pw[u] = j < n ? sc[j] : 0.0f;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            a0 += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u] & 0xFFFFu));
-            a1 += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u] >> 16));
-        }
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a[2 * e] += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u][e] & 0xFFFFu));
+                a[2 * e + 1] += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u][e] >> 16));
+            }
     }
-    part[wave][2 * lane] = a0;
-    part[wave][2 * lane + 1] = a1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {                               // the wave's four row lanes
+        a[e] += __shfl_xor(a[e], 16, GLQH_WAVE);
+        a[e] += __shfl_xor(a[e], 32, GLQH_WAVE);
+    }
+    if (vr == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part[wave][8 * vcol + e] = a[e];
+    }
     __syncthreads();
     if (threadIdx.x < D) {
         float acc = 0.0f;

@@ -179,6 +179,61 @@ e8_decompress_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict
     *(u32x4 *)(out + i * 8) = *(const u32x4 *)o;
 }
 
+// The same for large layers: the table's first P entries (the low-norm shells that Gaussian
+// weights mostly hit) live in LDS, one persistent 1024-thread workgroup per CU; only the
+// tail goes to L2 (random 4-byte L2 gathers run at 0.5 per clock per CU, LDS ones at ~10).
+// Every lookup issues both loads, the unused one aimed at a shared entry, so that all loads
+// stay unconditional.  Values and rounding are those of e8_decompress_kernel.
+constexpr int E8D_THREADS = 1024;
+constexpr int E8D_LDS_ENTRIES = 39936;                         // 156 KB of the 160 KB LDS
+
+__global__ void __launch_bounds__(E8D_THREADS)
+e8_decompress_lds_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
+                         const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
+                         const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n2,
+                         int t2_is_t1, float s2, float s3, float s4, int nstages, int64_t total_blocks,
+                         int P, f16 *__restrict__ out) {
+    extern __shared__ uint32_t tab[];
+    for (int j = threadIdx.x; j < P / 4; j += E8D_THREADS) ((u32x4 *)tab)[j] = ((const u32x4 *)t1)[j];
+    __syncthreads();
+    const uint32_t pre = (uint32_t)P, pre2 = t2_is_t1 ? (uint32_t)P : 0u;
+    const uint16_t *qs[3] = {q2, q3, q4};
+    const float sc[3] = {s2, s3, s4};
+    for (int64_t i = (int64_t)blockIdx.x * E8D_THREADS + threadIdx.x; i < total_blocks;
+         i += (int64_t)gridDim.x * E8D_THREADS) {
+        float w[8];
+        {
+            const uint32_t idx = q1[i];
+            const uint32_t wl = tab[min(idx, pre - 1)], wg = t1[max(idx, pre)];
+            const uint32_t word = idx < pre ? wl : wg;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                f16x2 v = e8_pair(word, p);
+                w[2 * p] = (float)v.x;
+                w[2 * p + 1] = (float)v.y;
+            }
+        }
+        for (int st = 1; st < nstages; ++st) {
+            uint32_t idx = qs[st - 1][i];
+            const uint32_t *tg = st == 1 ? t2 : t1;
+            const uint32_t pp = st == 1 ? pre2 : pre;
+            if (st == 1) idx = idx < n2 ? idx : n2 - 1;
+            const uint32_t wl = tab[min(idx, pre - 1)], wg = tg[max(idx, pp)];
+            const uint32_t word = idx < pp ? wl : wg;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                f16x2 v = e8_pair(word, p);
+                w[2 * p] += sc[st - 1] * (float)v.x;
+                w[2 * p + 1] += sc[st - 1] * (float)v.y;
+            }
+        }
+        f16 o[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o[c] = (f16)w[c];
+        *(u32x4 *)(out + i * 8) = *(const u32x4 *)o;
+    }
+}
+
 template <int NS>
 int launch_e8_NS(const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
                  const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, int ksplit,
@@ -210,7 +265,13 @@ int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nst
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
                        hipStream_t stream);
 
-int glqh_e8_init(void) { return glqh_e8_mma_init(); }
+int glqh_e8_init(void) {
+    if (glqh_check_hip(hipFuncSetAttribute((const void *)e8_decompress_lds_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, E8D_LDS_ENTRIES * 4),
+                       "e8 decompress attribute"))
+        return 1;
+    return glqh_e8_mma_init();
+}
 
 // K-split of the kernel that will serve the call.
 int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B) {
@@ -254,6 +315,15 @@ int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_
                               const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
                               int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream) {
     const int64_t total = m_pad * (n_pad / 8);
+    if (total >= ((int64_t)1 << 19)) {                           // the table load pays from 4 M weights up
+        const int P = E8D_LDS_ENTRIES;
+        hipLaunchKernelGGL(e8_decompress_lds_kernel, dim3((unsigned)glqh_device_cus()), dim3(E8D_THREADS),
+                           (size_t)P * 4, stream, (const uint16_t *)q[0], (const uint16_t *)q[1],
+                           (const uint16_t *)q[2], (const uint16_t *)q[3], t1, t2, (uint32_t)n2,
+                           (int)(t1 == t2 && n2 == 65536), s2, s3, s4, nstages, total, P, (f16 *)out);
+        GLQH_LAUNCH_CHECK("e8 decompress launch");
+        return 0;
+    }
     hipLaunchKernelGGL(e8_decompress_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                        (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
                        (const uint16_t *)q[3], t1, t2, (uint32_t)n2, s2, s3, s4, nstages, total,

@@ -105,11 +105,13 @@ def test_e8_dequant_matmul_matches_oracle(ext, m, n, stages):
 
 
 @pytest.mark.parametrize("m,n,B,stages", [(2048, 2048, 1, 1), (2048, 2048, 3, 2), (2100, 2048, 16, 2),
-                                          (1024, 4160, 1, 4), (4096, 1024, 9, 3), (512, 8192, 4, 2)])
+                                          (1024, 4160, 1, 4), (4096, 1024, 9, 3), (512, 8192, 4, 2),
+                                          (2048, 2048, 40, 2), (1024, 4160, 33, 4), (2100, 2048, 17, 1)])
 def test_e8_large_layers_lds_table(ext, m, n, B, stages):
-    """Layers of 4M weights and more at up to 16 tokens: the table prefix sits in LDS, the
-    tail comes from L2, the products run on MFMA.  Half of the indices are drawn from the
-    low shells, half uniformly, and the extremes are planted."""
+    """Layers of 4M weights and more: the table prefix sits in LDS, the tail comes from L2.
+    Up to 16 tokens the products run on MFMA straight from the indices; above, the weight is
+    dequantized once (same LDS table) for a library GEMM.  Half of the indices are drawn from
+    the low shells, half uniformly, and the extremes are planted."""
     say("e8 large", m, n, B, stages)
     rng = np.random.default_rng(m + n + B)
     cb = e8_table_f16()
@@ -142,6 +144,9 @@ def test_e8_large_layer_small_secondary_table(ext):
     q2 = rng.integers(0, 256, size=(m, n // 8)).astype(np.int16)
     x = rng.standard_normal((2, n)).astype(np.float16)
     W = O.e8_dequant(q1, q2, 0.5)
+    out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
+    assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
+    x = rng.standard_normal((24, n)).astype(np.float16)          # many tokens: dequantize + GEMM
     out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
     assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
 

@@ -728,7 +728,7 @@ int glqh_launch_viterbi(const float *tiles, int64_t n_tiles, int K, uint8_t *scr
                         float *hat, hipStream_t stream);
 
 extern "C" size_t glqh_trellis_quantize_workspace_bytes(int K, int64_t n_tiles) {
-    if (K < 2 || K > 4 || n_tiles < 1) return 0;
+    if (K < 1 || K > 4 || n_tiles < 1) return 0;
     glqh_init();
     return glqh_viterbi_scratch_bytes(K, n_tiles);
 }
@@ -737,7 +737,7 @@ extern "C" int glqh_trellis_quantize_tiles(const float *tiles, int64_t n_tiles, 
                                            float *hat_out, void *ws, size_t ws_bytes, void *stream) {
     GLQH_INIT();
     GLQH_REQUIRE(tiles && states_out && hat_out, "trellis quantize: null pointer");
-    GLQH_REQUIRE(K >= 2 && K <= 4, "trellis encoder supports K (bits/weight) 2-4, got %d", K);
+    GLQH_REQUIRE(K >= 1 && K <= 4, "trellis encoder supports K (bits/weight) 1-4, got %d", K);
     GLQH_REQUIRE(n_tiles >= 1, "trellis quantize: n_tiles=%lld", (long long)n_tiles);
     const size_t need = glqh_viterbi_scratch_bytes(K, n_tiles);
     GLQH_REQUIRE(ws && ws_bytes >= need, "trellis quantize: workspace of %zu bytes needed, got %zu", need, ws_bytes);

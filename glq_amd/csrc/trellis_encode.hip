@@ -14,7 +14,10 @@
 // input is rounded to fp16 first (glq/trellis.py:468), lut = decode_3inst computed on the fly.
 //
 // One workgroup (16 waves) per tile at a time; workgroups are persistent and walk the tiles
-// with a fixed stride, each owning one scratch slab.
+// with a fixed stride, each owning one scratch slab.  At K = 1 the two buffers of G = 32768
+// floats do not fit the LDS together: the new costs of a step go through a slab of global
+// scratch (each thread reads back what it wrote itself) into the one LDS buffer once every
+// thread has finished reading the old ones.
 #include "common.h"
 #include "trellis_device.h"
 
@@ -34,12 +37,14 @@ struct vt_best {
 // overlap < 0: unconstrained.  Returns, in `states` (LDS, T ints), the best state sequence.
 template <int K>
 __device__ __forceinline__ void viterbi_pass(const float *x, float *best, uint8_t *__restrict__ from_k,
-                                             int overlap, int *states, vt_best *red) {
+                                             float *__restrict__ spill, int overlap, int *states,
+                                             vt_best *red) {
     constexpr int G = 1 << (16 - K);
     constexpr int NK = 1 << K;
     constexpr int PER = G / VT_THREADS;                       // groups per thread
     const float inf = __builtin_inff();
-    float *cur = best, *nxt = best + G;
+    constexpr bool ONE_BUF = K == 1;
+    float *cur = best, *nxt = ONE_BUF ? spill : best + G;
     for (int g = threadIdx.x; g < G; g += VT_THREADS) cur[g] = (overlap < 0 || g == overlap) ? 0.0f : inf;
     __syncthreads();
     for (int i = 1; i < VT_T; ++i) {
@@ -61,7 +66,13 @@ __device__ __forceinline__ void viterbi_pass(const float *x, float *best, uint8_
             from_k[(int64_t)i * G + g] = (uint8_t)bk;
         }
         __syncthreads();
-        float *t = cur; cur = nxt; nxt = t;
+        if constexpr (ONE_BUF) {
+#pragma unroll 4
+            for (int u = 0; u < PER; ++u) cur[threadIdx.x + u * VT_THREADS] = nxt[threadIdx.x + u * VT_THREADS];
+            __syncthreads();
+        } else {
+            float *t = cur; cur = nxt; nxt = t;
+        }
     }
     // final costs, with the tail-biting mask on the low 16-K bits; lowest state on ties
     {
@@ -115,11 +126,13 @@ __global__ void __launch_bounds__(VT_THREADS)
 viterbi_kernel(const float *__restrict__ tiles, int64_t n_tiles, uint8_t *__restrict__ scratch,
                int32_t *__restrict__ states_out, float *__restrict__ hat_out) {
     constexpr int G = 1 << (16 - K);
-    extern __shared__ float best[];                            // 2 * G floats
+    extern __shared__ float best[];                            // 2 * G floats (G at K = 1)
     __shared__ float x[VT_T], xr[VT_T];
     __shared__ int states[VT_T];
     __shared__ vt_best red[VT_THREADS / 64];
     uint8_t *from_k = scratch + (int64_t)blockIdx.x * VT_T * G;
+    // K = 1: the spill slabs follow the back-pointer slabs of all workgroups
+    float *spill = K == 1 ? (float *)(scratch + (int64_t)gridDim.x * VT_T * G) + (int64_t)blockIdx.x * G : nullptr;
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
         if (threadIdx.x < VT_T) {
             const float v = (float)(f16)tiles[tile * VT_T + threadIdx.x];
@@ -127,10 +140,10 @@ viterbi_kernel(const float *__restrict__ tiles, int64_t n_tiles, uint8_t *__rest
             xr[(threadIdx.x + VT_T / 2) & (VT_T - 1)] = v;    // np.roll(x, T/2)
         }
         __syncthreads();
-        viterbi_pass<K>(xr, best, from_k, -1, states, red);
+        viterbi_pass<K>(xr, best, from_k, spill, -1, states, red);
         const int overlap = states[VT_T / 2] >> K;
         __syncthreads();
-        viterbi_pass<K>(x, best, from_k, overlap, states, red);
+        viterbi_pass<K>(x, best, from_k, spill, overlap, states, red);
         if (threadIdx.x < VT_T) {
             const int s = states[threadIdx.x];
             states_out[tile * VT_T + threadIdx.x] = s;
@@ -163,7 +176,7 @@ pack_states_kernel(const int32_t *__restrict__ states, int m, int n, int K, uint
 template <int K>
 int vt_launch(const float *tiles, int64_t n_tiles, uint8_t *scratch, int grid, int32_t *states, float *hat,
               hipStream_t stream) {
-    constexpr size_t lds = 2 * sizeof(float) * ((size_t)1 << (16 - K));
+    constexpr size_t lds = (K == 1 ? 1 : 2) * sizeof(float) * ((size_t)1 << (16 - K));
     hipLaunchKernelGGL(viterbi_kernel<K>, dim3((unsigned)grid), dim3(VT_THREADS), lds, stream, tiles, n_tiles,
                        scratch, states, hat);
     GLQH_LAUNCH_CHECK("viterbi launch");
@@ -180,7 +193,7 @@ int vt_set_lds(Kn kernel, size_t bytes) {
 }  // namespace
 
 int glqh_viterbi_init(void) {
-    return vt_set_lds(viterbi_kernel<2>, 2 * 4 * 16384) || vt_set_lds(viterbi_kernel<3>, 2 * 4 * 8192) ||
+    return vt_set_lds(viterbi_kernel<1>, 4 * 32768) || vt_set_lds(viterbi_kernel<2>, 2 * 4 * 16384) || vt_set_lds(viterbi_kernel<3>, 2 * 4 * 8192) ||
            vt_set_lds(viterbi_kernel<4>, 2 * 4 * 4096);
 }
 
@@ -191,18 +204,20 @@ int glqh_viterbi_grid(int K, int64_t n_tiles) {
 }
 
 size_t glqh_viterbi_scratch_bytes(int K, int64_t n_tiles) {
-    return (size_t)glqh_viterbi_grid(K, n_tiles) * VT_T * ((size_t)1 << (16 - K));
+    const size_t G = (size_t)1 << (16 - K);
+    return (size_t)glqh_viterbi_grid(K, n_tiles) * (VT_T * G + (K == 1 ? G * sizeof(float) : 0));
 }
 
 int glqh_launch_viterbi(const float *tiles, int64_t n_tiles, int K, uint8_t *scratch, int32_t *states,
                         float *hat, hipStream_t stream) {
     const int grid = glqh_viterbi_grid(K, n_tiles);
     switch (K) {
+    case 1: return vt_launch<1>(tiles, n_tiles, scratch, grid, states, hat, stream);
     case 2: return vt_launch<2>(tiles, n_tiles, scratch, grid, states, hat, stream);
     case 3: return vt_launch<3>(tiles, n_tiles, scratch, grid, states, hat, stream);
     case 4: return vt_launch<4>(tiles, n_tiles, scratch, grid, states, hat, stream);
     }
-    return glqh_fail("trellis encoder supports K (bits/weight) 2-4, got %d", K);
+    return glqh_fail("trellis encoder supports K (bits/weight) 1-4, got %d", K);
 }
 
 int glqh_launch_pack_states(const int32_t *states, int64_t m, int64_t n, int K, void *packed, hipStream_t stream) {

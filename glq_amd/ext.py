@@ -638,7 +638,7 @@ def e8_quantize(x, codebook, codebook_norms=None, return_decoded=True):
 
 def trellis_quantize_tiles(tiles, K):
     """bitshift_codebook.quantize (glq/trellis.py:467-484) on the GPU: (B, 256) tiles in step
-    order -> (hat (B, 256) fp32, states (B, 256) int32), tail-biting Viterbi, K = 2..4."""
+    order -> (hat (B, 256) fp32, states (B, 256) int32), tail-biting Viterbi, K = 1..4."""
     lib = _lib.load()
     if tiles.dim() != 2 or tiles.shape[1] != 256:
         raise RuntimeError(f"tiles must be (B, 256), got {tuple(tiles.shape)}")

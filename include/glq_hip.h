@@ -262,7 +262,7 @@ size_t glqh_trellis_quantize_workspace_bytes(int K, int64_t n_tiles);
  * decode_3inst(state).  Inputs are rounded to fp16 first, costs are fp32, ties go to the
  * lowest predecessor / lowest final state; two passes tie the ends together.
  * bitshift_codebook.quantize / viterbi (glq/trellis.py:253-296, 467-484) and the Triton
- * add-compare-select step (glq/trellis_step_kernel.py:30-109).  K = 2, 3 or 4. */
+ * add-compare-select step (glq/trellis_step_kernel.py:30-109).  K = 1..4. */
 int glqh_trellis_quantize_tiles(const float *tiles, int64_t n_tiles, int K, int32_t *states_out,
                                 float *hat_out, void *ws, size_t ws_bytes, void *stream);
 

@@ -53,7 +53,7 @@ def test_e8_quantize_residual_stage_and_size():
     assert torch.equal(i1, again)
 
 
-@pytest.mark.parametrize("K", [2, 3, 4])
+@pytest.mark.parametrize("K", [1, 2, 3, 4])
 def test_viterbi_matches_oracle_states(K, golden):
     """Tail-biting Viterbi: the reference's own tiles (golden vectors) and random tiles, state
     sequences and reconstructions bit-equal to the oracle (which is pinned on the reference)."""

@@ -23,13 +23,16 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
                                    int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
                                    int n_blocks, hipStream_t stream);
 // K plan of the fused-input GEMV for layers of the given padded heights sharing one input.
-// Returns 0 (not eligible), 1 (32-row workgroups, v_dot2 decode: more, shorter workgroups,
-// which is what the latency-bound attention shapes want) or 2 (64-row workgroups, MFMA decode:
-// fewer vector-ALU operations per weight, which pays once the rows alone fill the chip).
+// Returns 0 (not eligible), 1 (32-row workgroups, v_dot2 decode) or 2 (64-row workgroups, MFMA
+// decode: fewer vector-ALU operations per weight and half as many redundant input transforms).
+// The MFMA form wins from 32 strips of 64 rows on (measured on the 2048-row attention / down
+// shapes: 9.8 vs 10.7 us per launch on average); below that the launch is pure latency and the
+// smaller workgroups of the v_dot2 form spread it over more CUs.
+#define GLQH_FUSEIN_MMA_MIN_STRIPS 32
 static int tr_fusein_plan(const int64_t *m_pads, int n, int64_t n_pad, int64_t B, int *S, int *ks) {
     int64_t total = 0, wgs = 0;
     for (int i = 0; i < n; ++i) { total += m_pads[i]; wgs += (m_pads[i] + 63) / 64; }
-    if (wgs >= glqh_device_cus()) return glqh_trellis_mma_fusein_plan(wgs, n_pad, B, S, ks) ? 2 : 0;
+    if (wgs >= GLQH_FUSEIN_MMA_MIN_STRIPS) return glqh_trellis_mma_fusein_plan(wgs, n_pad, B, S, ks) ? 2 : 0;
     return glqh_trellis_fusein_plan(total, n_pad, B, S, ks) ? 1 : 0;
 }
 int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out);

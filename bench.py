@@ -398,16 +398,16 @@ def main():
     achieved = bytes_launch / (avg_us * 1e-6) / 1e9
     # HBM bytes per launch from the committed counter summary (FETCH_SIZE / WRITE_SIZE runs)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_tr_fusein_group_kernels_smollm3_4bpw_batch1.txt")
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_tr_mma_fusein_kernels_smollm3_4bpw_batch1.txt")
     if os.path.exists(tpath):
         import re
         mt = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(tpath).read(), re.M)
         traffic = int(mt.group(1)) if mt else None
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "kernel": ("tr_gemv_fusein_group_kernel<4,bf16,1> (q/k/v, o, down) and "
-                           "tr_mma_fusein_group_kernel<4,bf16,1> (gate/up): the fused-input decode "
-                           "launch, averaged over the four groups of a step"),
+                "kernel": ("tr_mma_fusein_kernel<4,bf16,1> (o, down) and tr_mma_fusein_group_kernel<4,bf16,1> "
+                           "(q/k/v, gate/up): the fused-input decode launch, averaged over the four "
+                           "groups of a step"),
                 "avg_launch_us": round(avg_us, 3),
                 "bytes_per_launch": int(bytes_launch),
                 "method": (f"{n_launch} back-to-back decode launches (the 4 grouped calls of a step: q/k/v, o, "

@@ -465,6 +465,7 @@ int glqh_launch_out_add_rmsnorm(const float *part, int ksplit, float scale, cons
     while (top * 2 <= m) top *= 2;
     const int row_off = (int)(top + top / 32 + 32);
     const size_t lds = (size_t)(row_off + m) * sizeof(float);
+    GLQH_REQUIRE(lds <= 64 * 1024, "out+add+rmsnorm: %lld rows need %zu bytes of LDS (64 KB at most)", (long long)m, lds);
     hipLaunchKernelGGL(out_add_rmsnorm_kernel, dim3(1), dim3(FN_THREADS), lds, stream, part, ksplit, scale,
                        (const f16 *)su, (int)m, (const uint16_t *)resid, (const uint16_t *)norm_w, eps,
                        (uint16_t *)x_out, (uint16_t *)h_out, row_off);

@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+import weakref
 
 import torch
 
@@ -407,8 +408,8 @@ def _packed_table(codebook):
     """Nibble-packed copy of an (N, 8) fp16 E8 table, built once per tensor."""
     key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device))
     hit = _TABLES.get(key)
-    if hit is not None:
-        return hit
+    if hit is not None and hit[0]() is codebook:            # same live tensor, not a reused address
+        return hit[1]
     lib = _lib.load()
     _chk(codebook, "codebook", torch.float16)
     if codebook.dim() != 2 or codebook.shape[1] != 8 or not 1 <= codebook.shape[0] <= 65536:
@@ -421,7 +422,10 @@ def _packed_table(codebook):
     if nbad:
         raise RuntimeError(f"codebook has {nbad} rows outside the E8 half-integer grid "
                            "{-3, -2.5, ..., 3}; only E8 shell tables are supported")
-    _TABLES[key] = packed
+    if len(_TABLES) > 64:                                   # drop entries whose tensor is gone
+        for k in [k for k, v in _TABLES.items() if v[0]() is None]:
+            del _TABLES[k]
+    _TABLES[key] = (weakref.ref(codebook), packed)
     return packed
 
 
@@ -434,9 +438,9 @@ def _half_table(codebook):
         return codebook
     key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device), codebook.dtype)
     hit = _HALF_TABLES.get(key)
-    if hit is None:
-        hit = _HALF_TABLES[key] = codebook.to(torch.float16).contiguous()
-    return hit
+    if hit is None or hit[0]() is not codebook:
+        hit = _HALF_TABLES[key] = (weakref.ref(codebook), codebook.to(torch.float16).contiguous())
+    return hit[1]
 
 
 def _per_row(t, n, name):
@@ -471,7 +475,7 @@ def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, i
     if sv.numel() != n_pad:
         raise RuntimeError(f"sv has {sv.numel()} entries, expected n_pad={n_pad}")
     ids = input_ids.reshape(-1).to(device=dev, dtype=torch.int64).contiguous()
-    t1 = _packed_table(_half_table(codebook.to(dev) if codebook.device != dev else codebook))
+    t1 = _primary_table(_half_table(codebook.to(dev) if codebook.device != dev else codebook))
     two = qidxs2 is not None and codebook2 is not None and inv_resid_scale is not None
     q2 = t2 = inv = None
     n2 = 0
@@ -496,13 +500,22 @@ def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, i
     return out.reshape(*input_ids.shape, embedding_dim)
 
 
+def _primary_table(codebook):
+    """Packed first-stage table: the kernels index it with the full 16-bit pattern and keep
+    its low-norm prefix in LDS, so it must be the whole 65536-entry table (the reference's
+    first-stage codebook always is, glq/codebook.py:169-192)."""
+    if codebook.dim() != 2 or codebook.shape[0] != 65536:
+        raise RuntimeError(f"the first-stage E8 table must have 65536 entries, got {tuple(codebook.shape)}")
+    return _packed_table(codebook)
+
+
 def _absent(t):
     return t is None or t.numel() == 0
 
 
 def _e8_args(qidxs, codebook, qidxs2, codebook2, inv_rs, qidxs3, inv_rs2, qidxs4, inv_rs3):
     _chk(qidxs, "qidxs", torch.int16)
-    t1 = _packed_table(codebook)
+    t1 = _primary_table(codebook)
     q2 = None if _absent(qidxs2) or float(inv_rs) == 0.0 else qidxs2
     t2, n2 = None, 0
     if q2 is not None:

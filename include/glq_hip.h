@@ -193,8 +193,9 @@ size_t glqh_e8_matmul_workspace_bytes(int64_t m_pad, int64_t n_pad, int64_t B);
 /* out[b, :] (fp32, stride m_pad) = wscale * (cb[q1] + inv_rs*cb2[q2] + inv_rs2*cb3[q3]
  * + inv_rs3*cb4[q4]) @ x[b, :], x (B, n_pad) fp16 in the RHT domain, q* (m_pad, n_pad/8)
  * int16 read as unsigned.  A stage is absent when its index pointer is NULL or its scale
- * is 0.  Tables are nibble-packed (glqh_e8_pack_table); table2 has n_entries2 rows
- * (65536, or 256 for the 3-bit recipe), stages 3-4 use table 1.
+ * is 0.  Tables are nibble-packed (glqh_e8_pack_table); table1 must hold all 65536 rows
+ * (it is indexed with the full 16-bit pattern and its low-norm prefix is copied to LDS),
+ * table2 has n_entries2 rows (65536, or 256 for the 3-bit recipe), stages 3-4 use table 1.
  * glq_dequant_matvec_cuda / glq_dequant_matmul_cuda, glq/csrc/glq_cuda.cu:1384-1637. */
 int glqh_e8_dequant_matmul(const void *x_f16, int64_t B,
                            const void *q1, const void *q2, const void *q3, const void *q4,

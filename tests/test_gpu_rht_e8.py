@@ -166,11 +166,13 @@ def test_e8_small_secondary_table(ext):
 
 
 def test_e8_rejects_foreign_table(ext):
-    bad = torch.randn(256, 8, device=DEV).half()
+    bad = torch.randn(65536, 8, device=DEV).half()
     q = torch.zeros(32, 8, dtype=torch.int16, device=DEV)
     x = torch.zeros(1, 64, dtype=torch.float16, device=DEV)
     with pytest.raises(RuntimeError, match="half-integer grid"):
         ext.glq_dequant_matmul_cuda(x, q, bad, 1.0)
+    with pytest.raises(RuntimeError, match="65536 entries"):   # a first-stage table must be whole
+        ext.glq_dequant_matmul_cuda(x, q, e8_table_f16()[:256].contiguous(), 1.0)
 
 
 @pytest.mark.parametrize("tag,bpw,bd", [("bd2", 2, True), ("bd4", 4, True), ("p2", 2, False),

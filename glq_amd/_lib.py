@@ -80,6 +80,9 @@ SIGNATURES = {
     "glqh_trellis_qkv_rope_store_bf16": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
                 c_int, c_vp, c_sz, c_vp]),
+    "glqh_trellis_qkv_rope_attn_bf16": (
+        c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
+                c_i64, c_i64, c_int, c_vp, c_sz, c_vp]),
     "glqh_trellis_gate_up_silu_bf16": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_sz, c_vp]),
 }

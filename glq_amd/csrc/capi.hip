@@ -539,6 +539,30 @@ extern "C" int glqh_trellis_qkv_rope_store_bf16(const void *x, int64_t in_featur
                                       v_cache, head_dim, max_len, apply_rope, st);
 }
 
+extern "C" int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_features, const glqh_trellis_shard *qkv,
+                                               const int64_t *blocks_n, int64_t n_blocks_n,
+                                               const glqh_block_meta *bn_meta_dev, int64_t n_pad,
+                                               const int64_t *pos, const void *cos_t, const void *sin_t,
+                                               void *k_cache, void *v_cache, void *out, int64_t heads,
+                                               int64_t kv_heads, int64_t head_dim, int64_t max_len,
+                                               int apply_rope, void *ws, size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(qkv, "qkv+rope+attention: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    glqh_trellis_shard sh[3] = {qkv[0], qkv[1], qkv[2]};
+    for (int i = 0; i < 3; ++i) {
+        GLQH_REQUIRE(sh[i].su_f16 && sh[i].out_features == sh[i].m_pad,
+                     "qkv+rope+attention: needs su and out_features == m_pad");
+        sh[i].y = nullptr;
+    }
+    tr_group_ctx c;
+    if (tr_group_decode(x, GLQH_BF16, in_features, 1, sh, 3, blocks_n, n_blocks_n, bn_meta_dev, in_features, n_pad,
+                        ws, ws_bytes, st, &c))
+        return 1;
+    return glqh_launch_out_rope_attn(c.parts, c.su, c.scale, c.m_pads, c.ks, pos, cos_t, sin_t, k_cache, v_cache,
+                                     out, heads, kv_heads, head_dim, max_len, apply_rope, st);
+}
+
 // ---- E8 shell ------------------------------------------------------------------------
 extern "C" int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, uint32_t *packed_out,
                                   int32_t *bad_dev, void *stream) {

@@ -182,4 +182,9 @@ int glqh_launch_out_rope_store(const float *const part[3], const void *const su[
                                const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
                                const void *sin_t, void *q_out, void *k_cache, void *v_cache, int64_t head_dim,
                                int64_t max_len, int apply_rope, hipStream_t stream);
+int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3], const float scale[3],
+                              const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
+                              const void *sin_t, void *k_cache, void *v_cache, void *out, int64_t heads,
+                              int64_t kv_heads, int64_t head_dim, int64_t max_len, int apply_rope,
+                              hipStream_t stream);
 int glqh_trellis_init(void);

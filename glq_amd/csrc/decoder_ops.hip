@@ -84,22 +84,18 @@ __global__ void rope_kv_store_kernel(const uint16_t *__restrict__ q, const uint1
 constexpr int AT_THREADS = 1024;
 constexpr int AT_WAVES = AT_THREADS / 64;
 
-__global__ void __launch_bounds__(AT_THREADS)
-attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
-                   const uint16_t *__restrict__ vc, const int64_t *__restrict__ pos_ptr,
-                   uint16_t *__restrict__ out, int heads, int kv_heads, int max_len, float scale) {
+// The attention of one head once its scaled query sits in qs (LDS, D floats): scores over
+// keys 0..n-1, softmax, weighted rows of V, result to out (D bf16).  NEWROW: row n-1 of K and V
+// is not read from the cache but from knew / vnew (LDS, D bf16 each) -- the caller has just
+// produced it and another workgroup is writing it to the cache at the same time.
+template <bool NEWROW>
+__device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__restrict__ K,
+                                          const uint16_t *__restrict__ V, int n, const uint16_t *knew,
+                                          const uint16_t *vnew, float *sc, float *red,
+                                          float (*part)[128], uint16_t *__restrict__ out) {
     constexpr int D = 128;
-    extern __shared__ float sc[];                  // max_len scores
-    __shared__ float qs[D];
-    __shared__ float red[AT_WAVES];
-    __shared__ float part[AT_WAVES][D];
-    const int h = blockIdx.x, g = h / (heads / kv_heads);
-    const int n = (int)pos_ptr[0] + 1;             // keys 0..pos (the current token is already cached)
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    if (threadIdx.x < D) qs[threadIdx.x] = bf16_bits_to_f32(q[(int64_t)h * D + threadIdx.x]) * scale;
-    __syncthreads();
-    const uint16_t *K = kc + (int64_t)g * max_len * D;
-    const uint16_t *V = vc + (int64_t)g * max_len * D;
+    const int last = NEWROW ? max(n - 2, 0) : n - 1;          // last row that is read from the cache
     const int sub = threadIdx.x & 7;
     float mx = -3.0e38f;
     // four keys per thread in flight (512 keys per round of the workgroup)
@@ -107,13 +103,17 @@ attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ 
         u32x4 k0[4], k1[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int j = min(j0 + u * (AT_THREADS / 8), n - 1);
+            const int j = min(j0 + u * (AT_THREADS / 8), last);
             k0[u] = *(const u32x4 *)(K + (int64_t)j * D + sub * 8);
             k1[u] = *(const u32x4 *)(K + (int64_t)j * D + 64 + sub * 8);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int j = j0 + u * (AT_THREADS / 8);
+            if (NEWROW && j == n - 1) {
+                k0[u] = *(const u32x4 *)(knew + sub * 8);
+                k1[u] = *(const u32x4 *)(knew + 64 + sub * 8);
+            }
             float s = 0.0f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -162,7 +162,8 @@ attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ 
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int j = j0 + u * 4 * AT_WAVES;
-            vv[u] = *(const u32x4 *)(V + (int64_t)min(j, n - 1) * D + 8 * vcol);
+            vv[u] = *(const u32x4 *)(V + (int64_t)min(j, last) * D + 8 * vcol);
+            if (NEWROW && j == n - 1) vv[u] = *(const u32x4 *)(vnew + 8 * vcol);
             pw[u] = j < n ? sc[j] : 0.0f;
         }
 #pragma unroll
@@ -187,8 +188,25 @@ attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ 
         float acc = 0.0f;
 #pragma unroll
         for (int w = 0; w < AT_WAVES; ++w) acc += part[w][threadIdx.x];
-        out[(int64_t)h * D + threadIdx.x] = f32_to_bf16_bits(acc / tot);
+        out[threadIdx.x] = f32_to_bf16_bits(acc / tot);
     }
+}
+
+__global__ void __launch_bounds__(AT_THREADS)
+attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kc,
+                   const uint16_t *__restrict__ vc, const int64_t *__restrict__ pos_ptr,
+                   uint16_t *__restrict__ out, int heads, int kv_heads, int max_len, float scale) {
+    constexpr int D = 128;
+    extern __shared__ float sc[];                  // max_len scores
+    __shared__ float qs[D];
+    __shared__ float red[AT_WAVES];
+    __shared__ float part[AT_WAVES][D];
+    const int h = blockIdx.x, g = h / (heads / kv_heads);
+    const int n = (int)pos_ptr[0] + 1;             // keys 0..pos (the current token is already cached)
+    if (threadIdx.x < D) qs[threadIdx.x] = bf16_bits_to_f32(q[(int64_t)h * D + threadIdx.x]) * scale;
+    __syncthreads();
+    attn_core<false>(qs, kc + (int64_t)g * max_len * D, vc + (int64_t)g * max_len * D, n, nullptr, nullptr, sc, red,
+                     part, out + (int64_t)h * D);
 }
 
 // x_out = bf16(x + delta); h_out = RMSNorm(x_out) * w as in rmsnorm_kernel (one pass, one launch)
@@ -394,6 +412,114 @@ out_rope_store_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos, co
     }
 }
 
+// q_proj / k_proj / v_proj finished inside the attention launch: workgroup h (one per query
+// head) transforms the 1024-point slice of q that holds its head and the slices of k and v that
+// hold its key/value head -- three transforms side by side on thread groups of 512 / 256 / 256
+// with shared barriers -- rotates q and k, and attends over cache rows 0..pos-1 plus the new
+// row, which it keeps in LDS; the first query head of each group also appends the row to the
+// caches.  Same slices, term order and roundings as out_rope_store_kernel + attn_decode_kernel:
+// bit-identical to the two launches.
+__device__ __forceinline__ rht_slice slice_of_row(int m, int row, int log_slice) {
+    glqh_meta_args margs;
+    margs.canon = m;
+    const int nb = __builtin_popcount((unsigned)m);
+    rht_slice blk = {};
+    for (int j = 0; j < nb; ++j) {
+        const glqh_block_meta bm = glqh_meta_row(margs, nullptr, j);
+        if (row < bm.offset + bm.bs || j == nb - 1) {
+            blk.off = bm.offset;
+            blk.bs = bm.bs;
+            blk.log_bs = bm.log_bs;
+            blk.log_len = min(bm.log_bs, log_slice);
+            blk.nsub = bm.bs >> blk.log_len;
+            blk.r = (row - bm.offset) >> blk.log_len;
+            blk.norm = rsqrt_pow2(bm.log_bs);
+            blk.live = true;
+            break;
+        }
+    }
+    return blk;
+}
+
+__device__ __forceinline__ int fht_barriers(int log_n) {       // barriers inside fht_staged
+    return log_n == 0 ? 0 : (log_n + RMAX - 1) / RMAX - 1;
+}
+
+__global__ void __launch_bounds__(AT_THREADS)
+out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
+                     const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t,
+                     uint16_t *__restrict__ kc, uint16_t *__restrict__ vc, uint16_t *__restrict__ out, int heads,
+                     int kv_heads, int max_len, int apply_rope, float scale, int log_slice, int sc_floats,
+                     int buf_floats) {
+    constexpr int D = 128, half = D / 2;
+    extern __shared__ float lds[];                 // scores, then the three transform buffers
+    __shared__ float qs[D];
+    __shared__ float red[AT_WAVES];
+    __shared__ float part[AT_WAVES][D];
+    __shared__ __align__(16) uint16_t knew[D], vnew[D];
+    float *sc = lds;
+    const int h = blockIdx.x, per = heads / kv_heads, g = h / per;
+    const int64_t p = pos_ptr[0];
+    const int n = (int)p + 1;
+    const int tid = threadIdx.x;
+    const int grp = tid < 512 ? 0 : tid < 768 ? 1 : 2;         // q | k | v, whole waves each
+    const int gt = grp == 0 ? tid : grp == 1 ? tid - 512 : tid - 768;
+    const int m = grp == 0 ? a.m[0] : grp == 1 ? a.m[1] : a.m[2];
+    const int row0 = (grp == 0 ? h : g) * D;
+    const rht_slice blk = slice_of_row(m, row0, log_slice);
+    const int bq = fht_barriers(slice_of_row(a.m[0], h * D, log_slice).log_len);
+    const int bk = fht_barriers(slice_of_row(a.m[1], g * D, log_slice).log_len);
+    const int bv = fht_barriers(slice_of_row(a.m[2], g * D, log_slice).log_len);
+    float *buf = lds + sc_floats + grp * buf_floats;
+    glqh_ysrc src = {};
+    src.part = grp == 0 ? a.part[0] : grp == 1 ? a.part[1] : a.part[2];
+    src.part_kstride = m;
+    src.ksplit = ksplit;
+    src.scale[0] = grp == 0 ? a.scale[0] : grp == 1 ? a.scale[1] : a.scale[2];
+    src.nparts = 1;
+    const f16 *su = grp == 0 ? a.su[0] : grp == 1 ? a.su[1] : a.su[2];
+    if (grp == 0) {
+        stage_partials<512, 2, 8>(buf, src, blk, 0, m, gt);
+        fht_staged(buf, blk.log_len, lds_writeback{buf}, gt, 512);
+    } else {
+        stage_partials<256, 2, 8>(buf, src, blk, 0, m, gt);
+        fht_staged(buf, blk.log_len, lds_writeback{buf}, gt, 256);
+    }
+    // every thread passes the same number of barriers whatever its group's transform size
+    for (int i = grp == 0 ? bq : grp == 1 ? bk : bv; i < max(bq, max(bk, bv)); ++i) __syncthreads();
+    __syncthreads();
+    if (gt < half) {
+        const int li = row0 - (blk.off + (blk.r << blk.log_len));  // the head inside the slice
+        const int d = gt;
+        const float va = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(li + d)] * (blk.norm * (float)su[row0 + d])));
+        const float vb = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(li + d + half)] *
+                                                           (blk.norm * (float)su[row0 + d + half])));
+        uint16_t o0 = f32_to_bf16_bits(va), o1 = f32_to_bf16_bits(vb);
+        if (grp != 2 && apply_rope) {
+            const float c0 = bf16_bits_to_f32(cos_t[p * D + d]), s0 = bf16_bits_to_f32(sin_t[p * D + d]);
+            const float c1 = bf16_bits_to_f32(cos_t[p * D + d + half]), s1 = bf16_bits_to_f32(sin_t[p * D + d + half]);
+            o0 = f32_to_bf16_bits(va * c0 - vb * s0);
+            o1 = f32_to_bf16_bits(vb * c1 + va * s1);
+        }
+        if (grp == 0) {
+            qs[d] = bf16_bits_to_f32(o0) * scale;
+            qs[d + half] = bf16_bits_to_f32(o1) * scale;
+        } else {
+            uint16_t *nw = grp == 1 ? knew : vnew;
+            nw[d] = o0;
+            nw[d + half] = o1;
+            if (h % per == 0) {                                  // one writer per key/value head
+                uint16_t *dst = (grp == 1 ? kc : vc) + ((int64_t)g * max_len + p) * D;
+                dst[d] = o0;
+                dst[d + half] = o1;
+            }
+        }
+    }
+    __syncthreads();
+    attn_core<true>(qs, kc + (int64_t)g * max_len * D, vc + (int64_t)g * max_len * D, n, knew, vnew, sc, red, part,
+                    out + (int64_t)h * D);
+}
+
 }  // namespace
 
 extern "C" int glqh_rmsnorm_bf16(const void *x, const void *w, void *out, int64_t T, int64_t H, double eps,
@@ -523,5 +649,36 @@ int glqh_launch_out_rope_store(const float *const part[3], const void *const su[
                        (const uint16_t *)cos_t, (const uint16_t *)sin_t, (uint16_t *)q_out, (uint16_t *)k_cache,
                        (uint16_t *)v_cache, (int)head_dim, (int)max_len, apply_rope, spb, log_slice);
     GLQH_LAUNCH_CHECK("out+rope launch");
+    return 0;
+}
+
+int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3], const float scale[3],
+                              const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
+                              const void *sin_t, void *k_cache, void *v_cache, void *out, int64_t heads,
+                              int64_t kv_heads, int64_t head_dim, int64_t max_len, int apply_rope,
+                              hipStream_t stream) {
+    GLQH_REQUIRE(pos && k_cache && v_cache && out && ksplit >= 1, "out+rope+attention: bad arguments");
+    GLQH_REQUIRE(!apply_rope || (cos_t && sin_t), "out+rope+attention: missing angle tables");
+    GLQH_REQUIRE(head_dim == 128, "out+rope+attention: head_dim must be 128, got %lld", (long long)head_dim);
+    GLQH_REQUIRE(kv_heads >= 1 && heads % kv_heads == 0, "out+rope+attention: heads must be a multiple of kv_heads");
+    GLQH_REQUIRE(m[0] == heads * head_dim && m[1] == kv_heads * head_dim && m[2] == m[1],
+                 "out+rope+attention: layer heights do not match the head counts");
+    qkv_fin a = {};
+    for (int i = 0; i < 3; ++i) {
+        GLQH_REQUIRE(part[i] && su[i] && m[i] <= 0x40000000ll && (m[i] & (head_dim - 1)) == 0,
+                     "out+rope+attention: layer %d: every output block must hold whole heads", i);
+        a.part[i] = part[i]; a.su[i] = (const f16 *)su[i]; a.scale[i] = scale[i]; a.m[i] = (int)m[i];
+    }
+    const int log_slice = 10;
+    const int buf_floats = (1 << log_slice) + (1 << log_slice) / 32 + 32;
+    const int sc_floats = (int)((max_len + 31) / 32 * 32);
+    const size_t lds = (size_t)(sc_floats + 3 * buf_floats) * sizeof(float);
+    GLQH_REQUIRE(lds <= 60 * 1024, "out+rope+attention: cache of %lld positions does not fit the score buffer",
+                 (long long)max_len);
+    hipLaunchKernelGGL(out_rope_attn_kernel, dim3((unsigned)heads), dim3(AT_THREADS), lds, stream, a, ksplit, pos,
+                       (const uint16_t *)cos_t, (const uint16_t *)sin_t, (uint16_t *)k_cache, (uint16_t *)v_cache,
+                       (uint16_t *)out, (int)heads, (int)kv_heads, (int)max_len, apply_rope,
+                       1.0f / sqrtf((float)head_dim), log_slice, sc_floats, buf_floats);
+    GLQH_LAUNCH_CHECK("out+rope+attention launch");
     return 0;
 }

@@ -123,6 +123,18 @@ def _qkv_rope_store(q, k, v, h, pos, cos, sin, qr, kc, vc, head_dim, max_len, ap
         max_len, int(apply_rope), ws.data_ptr(), ws.numel(), _stream()))
 
 
+def _qkv_rope_attn(q, k, v, h, pos, cos, sin, kc, vc, out, heads, kv_heads, head_dim, max_len, apply_rope):
+    """q/k/v projections of one token, rotated, appended to the cache and attended over:
+    decode launch + one finishing launch."""
+    ws = _group_ws((q, k, v), h.device)
+    bn, nbn = ext._host_i64(q.bn)
+    arr = _shard_array((q, k, v))                                # kept alive across the call
+    check(_lib.load().glqh_trellis_qkv_rope_attn_bf16(
+        h.data_ptr(), q.n, C.addressof(arr), bn, nbn, q.bn_meta.data_ptr() if nbn > 1 else None, q.n,
+        pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(), heads,
+        kv_heads, head_dim, max_len, int(apply_rope), ws.data_ptr(), ws.numel(), _stream()))
+
+
 def _rms_norm(x, w, eps):
     out = torch.empty_like(x)
     check(_lib.load().glqh_rmsnorm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1],
@@ -203,13 +215,9 @@ class TrellisDecoder:
             x, h = _add_rms_norm(x, delta, L["ln1"], cfg.rms_eps)
         apply_rope = int((li + 1) % cfg.no_rope_interval != 0)
         if T == 1 and self.fuse_epilogues and D == 128:
-            qr = torch.empty(1, cfg.heads * D, dtype=torch.bfloat16, device=x.device)
-            _qkv_rope_store(L["q"], L["k"], L["v"], h, pos, self.cos, self.sin, qr, self.kc[li], self.vc[li], D,
-                            self.max_len, apply_rope)
             a = torch.empty(1, cfg.heads * D, dtype=torch.bfloat16, device=x.device)
-            check(lib.glqh_attn_decode_bf16(qr.data_ptr(), self.kc[li].data_ptr(), self.vc[li].data_ptr(),
-                                            pos.data_ptr(), a.data_ptr(), cfg.heads, cfg.kv_heads, D,
-                                            self.max_len, _stream()))
+            _qkv_rope_attn(L["q"], L["k"], L["v"], h, pos, self.cos, self.sin, self.kc[li], self.vc[li], a,
+                           cfg.heads, cfg.kv_heads, D, self.max_len, apply_rope)
             x, h = _linear_add_rms_norm(L["o"], a, x, L["ln2"], cfg.rms_eps)
             return x, (L["down"], _gate_up_silu(L["gate"], L["up"], h))
         if T <= 4:

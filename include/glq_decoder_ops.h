@@ -83,6 +83,18 @@ int glqh_trellis_qkv_rope_store_bf16(const void *x, int64_t in_features, const g
                                      int64_t max_len, int apply_rope, void *ws, size_t ws_bytes,
                                      void *stream);
 
+/* The same with the attention of the token in that launch as well: q / k / v projections,
+ * rotary, cache append at *pos and single-query attention over positions 0..*pos ->
+ * out (heads, D) bf16.  Bit-identical to glqh_trellis_qkv_rope_store_bf16 +
+ * glqh_attn_decode_bf16; head_dim = 128, max_len <= ~11000. */
+int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_features, const glqh_trellis_shard *qkv,
+                                    const int64_t *blocks_n, int64_t n_blocks_n,
+                                    const glqh_block_meta *bn_meta_dev, int64_t n_pad,
+                                    const int64_t *pos, const void *cos_t, const void *sin_t,
+                                    void *k_cache, void *v_cache, void *out, int64_t heads,
+                                    int64_t kv_heads, int64_t head_dim, int64_t max_len,
+                                    int apply_rope, void *ws, size_t ws_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -167,3 +167,20 @@ def test_fused_qkv_rope_store_is_bit_identical(rope):
     D._qkv_rope_store(q, k, v, h, pos, cos, sin, qr1, kc1, vc1, hd, L, rope)
     assert torch.count_nonzero(qr0) > 0 and torch.count_nonzero(kc0[:, 37]) > 0
     assert torch.equal(qr0, qr1) and torch.equal(kc0, kc1) and torch.equal(vc0, vc1)
+    # and with the attention in the same launch: earlier cache rows are random, row 37 is new
+    kc0[:, :37] = torch.randn(kvh, 37, hd, generator=g, device=DEV).to(torch.bfloat16)
+    vc0[:, :37] = torch.randn(kvh, 37, hd, generator=g, device=DEV).to(torch.bfloat16)
+    a0 = torch.zeros(1, nq, dtype=torch.bfloat16, device=DEV)
+    D.check(lib.glqh_attn_decode_bf16(qr0.data_ptr(), kc0.data_ptr(), vc0.data_ptr(), pos.data_ptr(), a0.data_ptr(),
+                                      heads, kvh, hd, L, D._stream()))
+    kc2, vc2 = kc0.clone(), vc0.clone()
+    kc2[:, 37] = 0
+    vc2[:, 37] = 0
+    a2 = torch.zeros_like(a0)
+    D._qkv_rope_attn(q, k, v, h, pos, cos, sin, kc2, vc2, a2, heads, kvh, hd, L, rope)
+    assert torch.count_nonzero(a0) > 0
+    assert torch.equal(a0, a2) and torch.equal(kc0, kc2) and torch.equal(vc0, vc2)
+    pos0 = torch.tensor([0], device=DEV)                        # first position: only the new row
+    kc3, vc3, a3 = torch.zeros_like(kc0), torch.zeros_like(vc0), torch.zeros_like(a0)
+    D._qkv_rope_attn(q, k, v, h, pos0, cos, sin, kc3, vc3, a3, heads, kvh, hd, L, rope)
+    assert torch.equal(a3.view(heads, hd), vc3[:, 0].repeat_interleave(heads // kvh, 0))

@@ -2,6 +2,8 @@
 // embedding + KV-cache append, single-query grouped-query attention, SiLU gate).  They keep
 // the end-to-end decode measurement from being dominated by dozens of tiny framework kernels
 // per layer; arithmetic follows the usual Llama-family definitions in fp32 with bf16 storage.
+#include <type_traits>
+
 #include "common.h"
 #include "fht_device.h"
 
@@ -275,7 +277,39 @@ out_add_rmsnorm_kernel(const float *__restrict__ part, int ksplit, float scale, 
         blk.off = bm.offset; blk.bs = bm.bs; blk.log_bs = blk.log_len = bm.log_bs;
         blk.r = 0; blk.nsub = 1; blk.live = true;
         blk.norm = rsqrt_pow2(bm.log_bs);
-        stage_partials<FN_THREADS, 2, 8>(s, src, blk, 0, m);
+        // whole block, one stage: element i is scale * (p_0[i] + p_1[i] + ...) in slot order, every
+        // term's load in flight before the first add (the partial sums come from other XCDs'
+        // writes, a round trip to memory each time)
+        {
+            const float *__restrict__ pb = part + blk.off;
+            auto sum_terms = [&](auto cnt) {
+                constexpr int C = decltype(cnt)::value;
+                for (int i0 = threadIdx.x; i0 < blk.bs; i0 += 2 * FN_THREADS) {
+                    float t[2][C];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int c = 0; c < C; ++c)
+                            t[u][c] = pb[(int64_t)min(c, ksplit - 1) * m + min(i0 + u * FN_THREADS, blk.bs - 1)];
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        float acc = 0.0f;
+#pragma unroll
+                        for (int c = 0; c < C; ++c) acc += c < ksplit ? t[u][c] : 0.0f;
+                        if (i0 + u * FN_THREADS < blk.bs) s[lds_pad(i0 + u * FN_THREADS)] = 0.0f + scale * acc;
+                    }
+                }
+            };
+            if (ksplit <= 8) sum_terms(std::integral_constant<int, 8>{});
+            else if (ksplit <= 12) sum_terms(std::integral_constant<int, 12>{});
+            else if (ksplit <= 24) sum_terms(std::integral_constant<int, 24>{});
+            else {
+                stage_partials<FN_THREADS, 2, 8>(s, src, blk, 0, m);
+                goto staged;
+            }
+            __syncthreads();
+        }
+    staged:
         fht_staged(s, blk.log_len, lds_writeback{s});
         __syncthreads();
         for (int i = threadIdx.x; i < blk.bs; i += FN_THREADS) {

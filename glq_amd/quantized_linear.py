@@ -36,6 +36,8 @@ def _codebook_tensor(cb):
     raise TypeError(f"cannot take an E8 table from {type(cb).__name__}")
 
 
+_MAX_TOKENS_PER_CALL = 32768
+
 class E8RHTLinear(nn.Module):
     def __init__(self, in_features: int, out_features: int, bias: bool = False,
                  block_diagonal: bool = False, codebook_type: str = "e8_shell"):
@@ -234,6 +236,11 @@ class E8RHTLinear(nn.Module):
         sc = self._resolve(x.device)
         shape = x.shape
         x2d = x.reshape(-1, self.in_features)
+        if x2d.shape[0] == 0:                      # no tokens: nothing to launch
+            return x.new_empty(*shape[:-1], self.out_features)
+        if x2d.shape[0] > _MAX_TOKENS_PER_CALL:    # the kernels' grids carry the token index in 16 bits
+            parts = [self.forward(c) for c in x2d.split(_MAX_TOKENS_PER_CALL)]
+            return torch.cat(parts).reshape(*shape[:-1], self.out_features)
         if self._is_trellis:
             if not self._trellis_has_kernel:
                 raise RuntimeError("natural-layout trellis checkpoints cannot be decoded by the "

@@ -52,6 +52,38 @@ def test_shell_module_loads_reference_checkpoint(golden, tag, bpw, bd):
     assert torch.equal(y, layer(x))
 
 
+@pytest.mark.parametrize("kind", ["trellis", "shell"])
+def test_module_with_no_tokens_and_with_more_than_one_call_holds(golden, kind):
+    """An empty batch gives an empty result (as the reference's torch path does), and a batch
+    beyond what one launch grid indexes is served in pieces with the same rows as a short call."""
+    from glq_amd.quantized_linear import E8RHTLinear
+    say("module empty / long batch", kind)
+    if kind == "trellis":
+        g, tag = golden("trellis_layer"), "k4"
+        keys = ["trellis_packed", "SU", "SV", "Wscale"]
+        m, n = g[f"{tag}_W"].shape
+        layer = E8RHTLinear(n, m, codebook_type="trellis")
+    else:
+        g, tag = golden("e8_layer"), "bd2"
+        keys = ["Qidxs", "SU", "SV", "Wscale"]
+        m, n = g[f"{tag}_W"].shape
+        layer = E8RHTLinear(n, m, block_diagonal=True)
+    layer.load_state_dict({k: torch.from_numpy(np.asarray(g[f"{tag}_{k}"])) for k in keys})
+    layer.to(DEV)
+    if kind == "shell":
+        layer.set_codebook(e8_table_f16())
+    y0 = layer(torch.empty(0, n, dtype=torch.bfloat16, device=DEV))
+    assert y0.shape == (0, m) and y0.dtype == torch.bfloat16
+    assert layer(torch.empty(2, 0, n, dtype=torch.float16, device=DEV)).shape == (2, 0, m)
+    B = 32768 + 700
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(3)).to(DEV, torch.bfloat16)
+    y = layer(x)
+    assert y.shape == (B, m)
+    for lo in (0, 32768 - 300, B - 600):                   # rows either side of the split
+        assert rel(y[lo:lo + 600], layer(x[lo:lo + 600]).float()) < 5e-3
+    assert rel(y[-3:], x[-3:].float().cpu().numpy() @ g[f"{tag}_W_hat"].T) < TOL
+
+
 def test_ops_namespace_runs_the_hip_path():
     from glq_amd import custom_ops, hadamard as H
     custom_ops.register()

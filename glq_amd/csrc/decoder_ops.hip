@@ -249,18 +249,28 @@ silu_mul_kernel(const uint16_t *__restrict__ g, const uint16_t *__restrict__ u, 
 }
 
 // ---- output transform fused with what follows it in the decode loop (one token) --------
-// o_proj / down_proj: split-K partial sums -> output transform (whole Hadamard blocks, one
-// after the other) -> x_out = bf16(resid + bf16(y)) -> h_out = RMSNorm(x_out) * w, with the
-// roundings of output_rht + add_rmsnorm_kernel.  One workgroup: the row is 2-8 K values.
+// o_proj / down_proj: split-K partial sums -> output transform -> x_out = bf16(resid + bf16(y))
+// -> h_out = RMSNorm(x_out) * w, with the terms, order and roundings of
+// output_rht_group_kernel + add_rmsnorm_kernel.  One workgroup, the row is 2-8 K values: a
+// Hadamard block is cut into the same 1024-point slices, one per group of 256 threads, but
+// every group sums the split-K terms of its own 1024 rows only and the groups then combine
+// each other's sums through LDS (the separate launch re-reads the whole block per slice).
 constexpr int FN_THREADS = 1024;
+constexpr int FN_GROUPS = FN_THREADS / 256;
+constexpr int FN_LOG_SLICE = 10;
+constexpr int FN_MAX_ROWS = 8192;
 
 __global__ void __launch_bounds__(FN_THREADS)
 out_add_rmsnorm_kernel(const float *__restrict__ part, int ksplit, float scale, const f16 *__restrict__ su,
                        int m, const uint16_t *__restrict__ resid, const uint16_t *__restrict__ w, float eps,
-                       uint16_t *__restrict__ x_out, uint16_t *__restrict__ h_out, int row_off) {
-    extern __shared__ float s[];                   // [0, row_off): transform buffer; then m floats: the row
+                       uint16_t *__restrict__ x_out, uint16_t *__restrict__ h_out) {
+    // FN_GROUPS exchange buffers and FN_GROUPS sum buffers of one slice each, then m floats: the row
+    extern __shared__ float s[];
     __shared__ float red[FN_THREADS / 64];
-    float *row = s + row_off;
+    const int grp = threadIdx.x >> 8, gt = threadIdx.x & 255;
+    float *xchg = s + (grp << FN_LOG_SLICE);
+    float *sums = s + (FN_GROUPS << FN_LOG_SLICE);
+    float *row = s + (2 * FN_GROUPS << FN_LOG_SLICE);
     glqh_ysrc src = {};
     src.part = part;
     src.part_kstride = m;
@@ -270,58 +280,66 @@ out_add_rmsnorm_kernel(const float *__restrict__ part, int ksplit, float scale, 
     glqh_meta_args margs;
     margs.canon = m;
     const int nb = __builtin_popcount((unsigned)m);
+    uint16_t w_raw[FN_MAX_ROWS / FN_THREADS];                // the norm weights of the last loop, requested first
+#pragma unroll
+    for (int u = 0; u < FN_MAX_ROWS / FN_THREADS; ++u) w_raw[u] = w[min((int)threadIdx.x + u * FN_THREADS, m - 1)];
+    for (int j = 0; j < nb; ++j) {
+        const glqh_block_meta bm = glqh_meta_row(margs, nullptr, j);
+        const int log_len = min(bm.log_bs, FN_LOG_SLICE);
+        const int nsub = bm.bs >> log_len;                   // <= FN_GROUPS (checked by the launcher)
+        const bool mine = grp < nsub, live = mine && 4 * gt < (1 << log_len);
+        const int base = bm.offset + (grp << log_len);       // this group's rows: slice grp of the block
+        const float norm = rsqrt_pow2(bm.log_bs);
+        float z[4];
+        f16 su_raw[4];                                       // requested before the partial sums and
+        uint16_t rs_raw[4];                                  // not touched until those have arrived
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int r = base + fht_wave_index<4>(log_len, live ? gt : 0, q);
+            su_raw[q] = su[mine ? r : 0];
+            rs_raw[q] = resid[mine ? r : 0];
+        }
+        if (mine) {
+            // v_h for h = grp: the split-K terms of rows base .. base + len - 1, in slot order
+            rht_slice own = {};
+            own.off = base; own.bs = 1 << log_len; own.log_bs = own.log_len = log_len;
+            own.nsub = 1; own.r = 0; own.live = true;
+            float v[4];
+            if (ksplit <= 8) stage_partials_quad<8>(v, src, own, 0, m, gt);
+            else stage_partials_quad<12>(v, src, own, 0, m, gt);   // 24 terms in flight would spill registers
+            if (live) *(f32x4 *)(sums + (grp << FN_LOG_SLICE) + 4 * gt) = f32x4{v[0], v[1], v[2], v[3]};
+        }
+        __syncthreads();
+        // slice r = grp of the block: z = sum_h sign(r, h) v_h, h ascending
+#pragma unroll
+        for (int e = 0; e < 4; ++e) z[e] = 0.0f;
+        if (live) {
+            for (int h = 0; h < nsub; ++h) {
+                const f32x4 vh = *(const f32x4 *)(sums + (h << FN_LOG_SLICE) + 4 * gt);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) z[e] += had_sign(grp, h, vh[e]);
+            }
+        }
+        fht_wave<4, true>(z, log_len, xchg, gt);
+        if (live) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int r = base + fht_wave_index<4>(log_len, gt, q);
+                const float y = bf16_bits_to_f32(f32_to_bf16_bits(z[q] * (norm * (float)su_raw[q])));
+                const uint16_t sb = f32_to_bf16_bits(bf16_bits_to_f32(rs_raw[q]) + y);
+                x_out[r] = sb;
+                row[r] = bf16_bits_to_f32(sb);
+            }
+        }
+        __syncthreads();                                     // row written, buffers free for the next block
+    }
     float ss = 0.0f;
     for (int j = 0; j < nb; ++j) {
         const glqh_block_meta bm = glqh_meta_row(margs, nullptr, j);
-        rht_slice blk;
-        blk.off = bm.offset; blk.bs = bm.bs; blk.log_bs = blk.log_len = bm.log_bs;
-        blk.r = 0; blk.nsub = 1; blk.live = true;
-        blk.norm = rsqrt_pow2(bm.log_bs);
-        // whole block, one stage: element i is scale * (p_0[i] + p_1[i] + ...) in slot order, every
-        // term's load in flight before the first add (the partial sums come from other XCDs'
-        // writes, a round trip to memory each time)
-        {
-            const float *__restrict__ pb = part + blk.off;
-            auto sum_terms = [&](auto cnt) {
-                constexpr int C = decltype(cnt)::value;
-                for (int i0 = threadIdx.x; i0 < blk.bs; i0 += 2 * FN_THREADS) {
-                    float t[2][C];
-#pragma unroll
-                    for (int u = 0; u < 2; ++u)
-#pragma unroll
-                        for (int c = 0; c < C; ++c)
-                            t[u][c] = pb[(int64_t)min(c, ksplit - 1) * m + min(i0 + u * FN_THREADS, blk.bs - 1)];
-#pragma unroll
-                    for (int u = 0; u < 2; ++u) {
-                        float acc = 0.0f;
-#pragma unroll
-                        for (int c = 0; c < C; ++c) acc += c < ksplit ? t[u][c] : 0.0f;
-                        if (i0 + u * FN_THREADS < blk.bs) s[lds_pad(i0 + u * FN_THREADS)] = 0.0f + scale * acc;
-                    }
-                }
-            };
-            if (ksplit <= 8) sum_terms(std::integral_constant<int, 8>{});
-            else if (ksplit <= 12) sum_terms(std::integral_constant<int, 12>{});
-            else if (ksplit <= 24) sum_terms(std::integral_constant<int, 24>{});
-            else {
-                stage_partials<FN_THREADS, 2, 8>(s, src, blk, 0, m);
-                goto staged;
-            }
-            __syncthreads();
-        }
-    staged:
-        fht_staged(s, blk.log_len, lds_writeback{s});
-        __syncthreads();
-        for (int i = threadIdx.x; i < blk.bs; i += FN_THREADS) {
-            const int r = blk.off + i;
-            const float y = bf16_bits_to_f32(f32_to_bf16_bits(s[lds_pad(i)] * (blk.norm * (float)su[r])));
-            const uint16_t sb = f32_to_bf16_bits(bf16_bits_to_f32(resid[r]) + y);
-            x_out[r] = sb;
-            const float v = bf16_bits_to_f32(sb);
-            row[r] = v;
+        for (int i = threadIdx.x; i < bm.bs; i += FN_THREADS) {
+            const float v = row[bm.offset + i];
             ss += v * v;
         }
-        __syncthreads();                           // s is staged again for the next block
     }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
@@ -330,9 +348,13 @@ out_add_rmsnorm_kernel(const float *__restrict__ part, int ksplit, float scale, 
 #pragma unroll
     for (int i = 0; i < FN_THREADS / 64; ++i) tot += red[i];
     const float r = rsqrtf(tot / (float)m + eps);
-    for (int i = threadIdx.x; i < m; i += FN_THREADS) {
-        const float nrm = bf16_bits_to_f32(f32_to_bf16_bits(row[i] * r));
-        h_out[i] = f32_to_bf16_bits(nrm * bf16_bits_to_f32(w[i]));
+#pragma unroll
+    for (int u = 0; u < FN_MAX_ROWS / FN_THREADS; ++u) {
+        const int i = threadIdx.x + u * FN_THREADS;
+        if (i < m) {
+            const float nrm = bf16_bits_to_f32(f32_to_bf16_bits(row[i] * r));
+            h_out[i] = f32_to_bf16_bits(nrm * bf16_bits_to_f32(w_raw[u]));
+        }
     }
 }
 
@@ -361,28 +383,28 @@ out_silu_mul_kernel(const float *__restrict__ part_g, const float *__restrict__ 
     src.scale[0] = layer ? sc_u : sc_g;
     src.nparts = 1;
     const f16 *su = layer ? su_u : su_g;
-    stage_partials<256, 4, 8>(buf, src, blk, 0, m_pad, tid);
-    fht_staged(buf, blk.log_len, lds_writeback{buf}, tid, 256);
-    __syncthreads();
+    const bool live = 4 * tid < len;
+    float z[4];
+    f16 su_raw[4];                                 // requested before the partial sums, used after
+    int idx[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) su_raw[q] = su[base + fht_wave_index<4>(blk.log_len, live ? tid : 0, q)];
+    partials_fht_quad(z, idx, src, blk, 0, m_pad, buf, tid);
     float y[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int i = tid + 256 * u;
-        y[u] = 0.0f;
-        if (i < len) {
-            y[u] = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(i)] * (blk.norm * (float)su[base + i])));
-            if (layer == 0) gv[i] = y[u];
-        }
+    for (int q = 0; q < 4; ++q) {
+        y[q] = bf16_bits_to_f32(f32_to_bf16_bits(z[q] * (blk.norm * (float)su_raw[q])));
+        if (layer == 0 && live) gv[idx[q]] = y[q];
     }
     __syncthreads();
-    if (layer == 1) {
+    if (layer == 1 && live) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int i = tid + 256 * u;
-            if (i < len && base + i < out_features) {
+        for (int q = 0; q < 4; ++q) {
+            const int i = idx[q];
+            if (base + i < out_features) {
                 const float a = gv[i];
                 const float sl = bf16_bits_to_f32(f32_to_bf16_bits(a / (1.0f + __expf(-a))));
-                act[base + i] = f32_to_bf16_bits(sl * y[u]);
+                act[base + i] = f32_to_bf16_bits(sl * y[q]);
             }
         }
     }
@@ -420,13 +442,27 @@ out_rope_store_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos, co
     src.ksplit = ksplit;
     src.scale[0] = scale;
     src.nparts = 1;
-    stage_partials<256, 4, 8>(s, src, blk, 0, m);
-    fht_staged(s, blk.log_len, lds_writeback{s});
-    __syncthreads();
     const int len = 1 << blk.log_len, base = blk.off + (blk.r << blk.log_len), half = D >> 1;
     const int64_t p = *pos;
-    // y rounded to bf16, as the separate output transform stores it
-    auto yv = [&](int i) { return bf16_bits_to_f32(f32_to_bf16_bits(s[lds_pad(i)] * (blk.norm * (float)su[base + i]))); };
+    {
+        const int tid = threadIdx.x;
+        const bool live = 4 * tid < len;
+        float zq[4];
+        f16 su_raw[4];                             // requested before the partial sums, used after
+        int idx[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) su_raw[q] = su[base + fht_wave_index<4>(blk.log_len, live ? tid : 0, q)];
+        partials_fht_quad(zq, idx, src, blk, 0, m, s, tid);
+        __syncthreads();                           // the exchange has been read: s takes the result
+        // y rounded to bf16, as the separate output transform stores it
+        if (live) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                s[lds_pad(idx[q])] = bf16_bits_to_f32(f32_to_bf16_bits(zq[q] * (blk.norm * (float)su_raw[q])));
+        }
+        __syncthreads();
+    }
+    auto yv = [&](int i) { return s[lds_pad(i)]; };
     for (int e = threadIdx.x; e < len / 2; e += 256) {
         const int hl = e / half, d = e - hl * half;            // head inside the slice, column pair (d, d + half)
         const int i0 = hl * D + d, i1 = i0 + half;
@@ -475,10 +511,6 @@ __device__ __forceinline__ rht_slice slice_of_row(int m, int row, int log_slice)
     return blk;
 }
 
-__device__ __forceinline__ int fht_barriers(int log_n) {       // barriers inside fht_staged
-    return log_n == 0 ? 0 : (log_n + RMAX - 1) / RMAX - 1;
-}
-
 __global__ void __launch_bounds__(AT_THREADS)
 out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
                      const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t,
@@ -501,9 +533,6 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
     const int m = grp == 0 ? a.m[0] : grp == 1 ? a.m[1] : a.m[2];
     const int row0 = (grp == 0 ? h : g) * D;
     const rht_slice blk = slice_of_row(m, row0, log_slice);
-    const int bq = fht_barriers(slice_of_row(a.m[0], h * D, log_slice).log_len);
-    const int bk = fht_barriers(slice_of_row(a.m[1], g * D, log_slice).log_len);
-    const int bv = fht_barriers(slice_of_row(a.m[2], g * D, log_slice).log_len);
     float *buf = lds + sc_floats + grp * buf_floats;
     glqh_ysrc src = {};
     src.part = grp == 0 ? a.part[0] : grp == 1 ? a.part[1] : a.part[2];
@@ -512,15 +541,17 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
     src.scale[0] = grp == 0 ? a.scale[0] : grp == 1 ? a.scale[1] : a.scale[2];
     src.nparts = 1;
     const f16 *su = grp == 0 ? a.su[0] : grp == 1 ? a.su[1] : a.su[2];
-    if (grp == 0) {
-        stage_partials<512, 2, 8>(buf, src, blk, 0, m, gt);
-        fht_staged(buf, blk.log_len, lds_writeback{buf}, gt, 512);
-    } else {
-        stage_partials<256, 2, 8>(buf, src, blk, 0, m, gt);
-        fht_staged(buf, blk.log_len, lds_writeback{buf}, gt, 256);
+    {
+        // three transforms of possibly different sizes side by side: one shared barrier each
+        float zq[4];
+        int idx[4];
+        const bool live = partials_fht_quad<true>(zq, idx, src, blk, 0, m, buf, gt);
+        __syncthreads();                           // the exchanges have been read: buf takes the result
+        if (live) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) buf[lds_pad(idx[q])] = zq[q];
+        }
     }
-    // every thread passes the same number of barriers whatever its group's transform size
-    for (int i = grp == 0 ? bq : grp == 1 ? bk : bv; i < max(bq, max(bk, bv)); ++i) __syncthreads();
     __syncthreads();
     if (gt < half) {
         const int li = row0 - (blk.off + (blk.r << blk.log_len));  // the head inside the slice
@@ -620,15 +651,18 @@ int glqh_launch_out_add_rmsnorm(const float *part, int ksplit, float scale, cons
                                 const void *resid, const void *norm_w, float eps, void *x_out, void *h_out,
                                 hipStream_t stream) {
     GLQH_REQUIRE(part && su && resid && norm_w && x_out && h_out && ksplit >= 1, "out+add+rmsnorm: bad arguments");
-    GLQH_REQUIRE(m >= 32 && m <= 8192, "out+add+rmsnorm: %lld rows (32..8192)", (long long)m);
+    GLQH_REQUIRE(m >= 32 && m <= FN_MAX_ROWS, "out+add+rmsnorm: %lld rows (32..%d)", (long long)m, FN_MAX_ROWS);
     int64_t top = 1;
     while (top * 2 <= m) top *= 2;
-    const int row_off = (int)(top + top / 32 + 32);
-    const size_t lds = (size_t)(row_off + m) * sizeof(float);
+    const size_t lds = (size_t)((2 * FN_GROUPS << FN_LOG_SLICE) + m) * sizeof(float);
+    GLQH_REQUIRE(top <= (int64_t)FN_GROUPS << FN_LOG_SLICE, "out+add+rmsnorm: %lld rows: blocks of more than %d rows",
+                 (long long)m, FN_GROUPS << FN_LOG_SLICE);
     GLQH_REQUIRE(lds <= 64 * 1024, "out+add+rmsnorm: %lld rows need %zu bytes of LDS (64 KB at most)", (long long)m, lds);
+    GLQH_REQUIRE((m & 3) == 0 && ((uintptr_t)part & 15) == 0,
+                 "out+add+rmsnorm: rows must be a multiple of 4 and the partial sums 16-byte aligned");
     hipLaunchKernelGGL(out_add_rmsnorm_kernel, dim3(1), dim3(FN_THREADS), lds, stream, part, ksplit, scale,
                        (const f16 *)su, (int)m, (const uint16_t *)resid, (const uint16_t *)norm_w, eps,
-                       (uint16_t *)x_out, (uint16_t *)h_out, row_off);
+                       (uint16_t *)x_out, (uint16_t *)h_out);
     GLQH_LAUNCH_CHECK("out+add+rmsnorm launch");
     return 0;
 }
@@ -639,6 +673,8 @@ int glqh_launch_out_silu_mul(const float *part_gate, const float *part_up, int k
     GLQH_REQUIRE(part_gate && part_up && su_gate && su_up && act_out && ksplit >= 1, "out+silu: bad arguments");
     GLQH_REQUIRE(m_pad >= 32 && m_pad <= 0x40000000ll && out_features >= 1 && out_features <= m_pad,
                  "out+silu: bad shape");
+    GLQH_REQUIRE((m_pad & 3) == 0 && (((uintptr_t)part_gate | (uintptr_t)part_up) & 15) == 0,
+                 "out+silu: rows must be a multiple of 4 and the partial sums 16-byte aligned");
     int64_t top = 1;
     while (top * 2 <= m_pad) top *= 2;
     const int log_slice = 10;                      // the slices of the few-token output transform
@@ -668,6 +704,7 @@ int glqh_launch_out_rope_store(const float *const part[3], const void *const su[
         GLQH_REQUIRE(part[i] && su[i] && m[i] >= head_dim && m[i] <= 0x40000000ll && m[i] % head_dim == 0,
                      "out+rope: layer %d: rows must be whole heads", i);
         GLQH_REQUIRE((m[i] & (head_dim - 1)) == 0, "out+rope: every output block must hold whole heads");
+        GLQH_REQUIRE(head_dim >= 4 && ((uintptr_t)part[i] & 15) == 0, "out+rope: layer %d: partial sums must be 16-byte aligned", i);
         a.part[i] = part[i]; a.su[i] = (const f16 *)su[i]; a.scale[i] = scale[i]; a.m[i] = (int)m[i];
         int64_t top = 1;
         while (top * 2 <= m[i]) top *= 2;
@@ -701,6 +738,7 @@ int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3
     for (int i = 0; i < 3; ++i) {
         GLQH_REQUIRE(part[i] && su[i] && m[i] <= 0x40000000ll && (m[i] & (head_dim - 1)) == 0,
                      "out+rope+attention: layer %d: every output block must hold whole heads", i);
+        GLQH_REQUIRE(((uintptr_t)part[i] & 15) == 0, "out+rope+attention: layer %d: partial sums must be 16-byte aligned", i);
         a.part[i] = part[i]; a.su[i] = (const f16 *)su[i]; a.scale[i] = scale[i]; a.m[i] = (int)m[i];
     }
     const int log_slice = 10;

@@ -230,16 +230,6 @@ output_rht_body(const glqh_ysrc &src, const f16 *__restrict__ su, YT *__restrict
     const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const int64_t b = blockIdx.y;
-    if constexpr (!PARTS) {
-        const float *__restrict__ d = src.direct + b * src.stride + blk.off;
-        auto val = [&](int h, int i) -> float { return d[(h << blk.log_len) + i]; };
-        if (blk.nsub == 1 && blk.log_len >= 11) stage_signed_slices<RHT_THREADS, 8, 1>(s, blk.log_len, 1, 0, val);
-        else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
-    } else {
-        const int total = blk.nsub * src.nparts * src.ksplit;
-        if (total == 1 && blk.log_len >= 11) stage_partials<RHT_THREADS, 8, 1>(s, src, blk, b, m_pad);
-        else stage_partials<RHT_THREADS, 4, 8>(s, src, blk, b, m_pad);
-    }
     const int base = blk.off + (blk.r << blk.log_len);
     struct {
         YT *yrow;
@@ -253,6 +243,42 @@ output_rht_body(const glqh_ysrc &src, const f16 *__restrict__ su, YT *__restrict
             if (row < out_features) yrow[row] = f32_to_act<YT>(v * f);
         }
     } store = {y + b * y_stride, su, base, out_features, blk.norm};
+    // slices of 4 .. 1024 points with 16-byte aligned rows are transformed in registers
+    bool in_regs;                                              // uniform over the workgroup
+    if constexpr (PARTS) in_regs = stage_partials_quad_ok(src, blk, b, m_pad);
+    else
+        in_regs = blk.log_len >= 2 && blk.log_len <= fht_wave_max_log<4>() &&
+                  ((uintptr_t)(src.direct + b * src.stride + blk.off) & 15) == 0;
+    if (in_regs) {
+        const int tid = threadIdx.x;
+        const bool active = 4 * tid < (1 << blk.log_len);
+        int idx[4];
+        float z[4];
+        f16 su_raw[4];                                         // in flight beside the row, used after it
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            idx[q] = fht_wave_index<4>(blk.log_len, active ? tid : 0, q);
+            su_raw[q] = su[base + idx[q]];
+        }
+        if constexpr (PARTS) stage_partials_quad<16>(z, src, blk, b, m_pad, tid);
+        else stage_signed_row_quad<8>(z, src.direct + b * src.stride + blk.off, blk.log_len, blk.nsub, blk.r, tid);
+        fht_wave<4>(z, blk.log_len, s, tid);
+        if (active) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) store.put(idx[q], z[q], blk.norm * (float)su_raw[q]);
+        }
+        return;
+    }
+    if constexpr (!PARTS) {
+        const float *__restrict__ d = src.direct + b * src.stride + blk.off;
+        auto val = [&](int h, int i) -> float { return d[(h << blk.log_len) + i]; };
+        if (blk.nsub == 1 && blk.log_len >= 11) stage_signed_slices<RHT_THREADS, 8, 1>(s, blk.log_len, 1, 0, val);
+        else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
+    } else {
+        const int total = blk.nsub * src.nparts * src.ksplit;
+        if (total == 1 && blk.log_len >= 11) stage_partials<RHT_THREADS, 8, 1>(s, src, blk, b, m_pad);
+        else stage_partials<RHT_THREADS, 4, 8>(s, src, blk, b, m_pad);
+    }
     fht_staged(s, blk.log_len, store);
 }
 

@@ -118,6 +118,113 @@ struct lds_writeback {                                   // last pass: results s
     __device__ void put(int i, float v, float) const { lds[lds_pad(i)] = v; }
 };
 
+// ---------------------------------------------------------------------------------
+// Register form of short transforms.  The LDS passes above cost a few hundred instructions
+// per thread, and in the one-token kernels a wave has its SIMD to itself, so every one of
+// them is paid in full (4+ cycles each, nothing to overlap with).  Here thread tid holds E
+// consecutive elements, E*tid .. E*tid+E-1, of a 2^log_n-point vector in registers:
+// log2(E) butterfly levels stay inside the thread, up to six run across the lanes of the
+// wave (DPP quad permutes, ds_swizzle, ds_bpermute: no LDS storage, no barrier), and up to
+// log2(E) more, across waves, take one exchange through LDS.  log2(E) <= log_n <=
+// 6 + 2*log2(E); threads tid >= n/E carry don't-care values but must make the call.
+//
+// After the call the thread holds elements fht_wave_index<E>(log_n, tid, q), q = 0..E-1.
+// The exchange contains the call's only __syncthreads(); with ALWAYS_SYNC the shorter
+// transforms pass one too, so that thread groups of one workgroup may run transforms of
+// different sizes side by side (each with its own tid numbering and exchange buffer).
+// ---------------------------------------------------------------------------------
+template <int E> struct fht_wave_log { };
+template <> struct fht_wave_log<4> { static constexpr int v = 2; };
+template <> struct fht_wave_log<8> { static constexpr int v = 3; };
+
+template <int E>
+__device__ __forceinline__ constexpr int fht_wave_max_log() { return 6 + 2 * fht_wave_log<E>::v; }
+
+template <int E>
+__device__ __forceinline__ int fht_wave_index(int log_n, int tid, int q) {
+    constexpr int LE = fht_wave_log<E>::v;
+    return log_n > LE + 6 ? tid + (q << (log_n - LE)) : tid * E + q;
+}
+
+// value of the lane whose number differs in bit K
+template <int K>
+__device__ __forceinline__ float fht_lane_partner(float v, int swap32_addr) {
+    const int b = __builtin_bit_cast(int, v);
+    int o;
+    if constexpr (K == 0) o = __builtin_amdgcn_mov_dpp(b, 0xB1, 0xF, 0xF, true);        // quad_perm [1,0,3,2]
+    else if constexpr (K == 1) o = __builtin_amdgcn_mov_dpp(b, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    else if constexpr (K < 5) o = __builtin_amdgcn_ds_swizzle(b, ((1 << K) << 10) | 0x1F);  // xor mask, 32-lane groups
+    else o = __builtin_amdgcn_ds_bpermute(swap32_addr, b);
+    return __builtin_bit_cast(float, o);
+}
+
+template <int K, int E>
+__device__ __forceinline__ void fht_lane_level(float (&v)[E], int lane, int swap32_addr) {
+    const float sgn = ((lane >> K) & 1) ? -1.0f : 1.0f;      // upper element of the pair: partner - own
+    float o[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j) o[j] = fht_lane_partner<K>(v[j], swap32_addr);
+#pragma unroll
+    for (int j = 0; j < E; ++j) v[j] = __builtin_fmaf(v[j], sgn, o[j]);   // exact: one rounding, like the add
+}
+
+template <int E, bool ALWAYS_SYNC = false>
+__device__ __forceinline__ void fht_wave(float (&v)[E], int log_n, float *xchg, int tid) {
+    constexpr int LE = fht_wave_log<E>::v;
+#pragma unroll
+    for (int h = 1; h < E; h <<= 1) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) {
+            if ((j & h) == 0) {
+                const float a = v[j], b = v[j | h];
+                v[j] = a + b;
+                v[j | h] = a - b;
+            }
+        }
+    }
+    const int lane = tid & 63;
+    const int lane_bits = min(log_n - LE, 6);                // uniform
+    const int swap32_addr = (lane ^ 32) << 2;
+    if (lane_bits > 0) fht_lane_level<0>(v, lane, swap32_addr);
+    if (lane_bits > 1) fht_lane_level<1>(v, lane, swap32_addr);
+    if (lane_bits > 2) fht_lane_level<2>(v, lane, swap32_addr);
+    if (lane_bits > 3) fht_lane_level<3>(v, lane, swap32_addr);
+    if (lane_bits > 4) fht_lane_level<4>(v, lane, swap32_addr);
+    if (lane_bits > 5) fht_lane_level<5>(v, lane, swap32_addr);
+    if (log_n <= LE + 6) {
+        if constexpr (ALWAYS_SYNC) __syncthreads();           // the barrier the longer transforms take
+        return;
+    }
+    // levels LE+6 .. log_n-1 pair elements held by different waves: through LDS once, after
+    // which thread u holds elements u + q * (n / E) and the open levels are the top bits of q
+    const int wave_bits = log_n - LE - 6;                     // 1 .. LE
+    const int nthr = 1 << (log_n - LE);
+    if (tid < nthr) {
+#pragma unroll
+        for (int j = 0; j < E; j += 4)
+            *(f32x4 *)(xchg + E * tid + j) = f32x4{v[j], v[j + 1], v[j + 2], v[j + 3]};
+    }
+    __syncthreads();
+    if (tid < nthr) {
+#pragma unroll
+        for (int q = 0; q < E; ++q) v[q] = xchg[tid + q * nthr];
+    }
+#pragma unroll
+    for (int c = 0; c < LE; ++c) {
+        if (c >= LE - wave_bits) {                            // uniform
+            const int h = 1 << c;
+#pragma unroll
+            for (int j = 0; j < E; ++j) {
+                if ((j & h) == 0) {
+                    const float a = v[j], b = v[j | h];
+                    v[j] = a + b;
+                    v[j | h] = a - b;
+                }
+            }
+        }
+    }
+}
+
 // sign of element (r, h) of the Sylvester matrix
 __device__ __forceinline__ float had_sign(int r, int h, float v) {
     return (__builtin_popcount(r & h) & 1) ? -v : v;
@@ -276,6 +383,106 @@ __device__ __forceinline__ void stage_partials(float *s, const glqh_ysrc &src, c
             if (i0 + u * T < len) s[lds_pad(i0 + u * T)] = z[u];
     }
     __syncthreads();
+}
+
+// stage_partials for the register transform: the same sums in the same order, but thread tid
+// takes elements 4*tid .. 4*tid+3 of the slice with one 16-byte load per term and keeps them in
+// registers.  The caller has checked 2 <= log_len and that every term's row is 16-byte aligned.
+template <int C>
+__device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ysrc &src, const rht_slice &blk,
+                                                    int64_t b, int m_pad, int tid) {
+    const int len = 1 << blk.log_len;
+    const int ks = src.ksplit, nst = src.nparts;
+    const int total = blk.nsub * nst * ks;
+    const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
+    const bool active = 4 * tid < len;
+    const int i0 = active ? 4 * tid : len - 4;             // idle threads repeat the last quad
+    float v[4], acc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) z[e] = v[e] = acc[e] = 0.0f;
+    int h = 0, st = 0, k = 0;                               // position of term t0 (uniform)
+    for (int t0 = 0; t0 < total; t0 += C) {
+        f32x4 vals[C];
+        int hh = h, ss = st, kk = k;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
+            vals[c] = *(const f32x4 *)(p + i0);
+            if (t0 + c + 1 < total) {                       // advance, clamped at the last term
+                if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (t0 + c < total) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += vals[c][e];
+                if (++k == ks) {
+                    const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
+                                   : st == 2 ? src.scale[2] : src.scale[3];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { v[e] += sc * acc[e]; acc[e] = 0.0f; }
+                    k = 0;
+                    if (++st == nst) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (src.copy_out && blk.r == 0 && active)
+                                src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i0 + e] = v[e];
+                            z[e] += had_sign(blk.r, h, v[e]);
+                            v[e] = 0.0f;
+                        }
+                        st = 0;
+                        ++h;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// The same for a plain fp32 row: z[e] = sum_h sign(r, h) * d[h * len + 4*tid + e], h ascending
+// as in stage_signed_slices.  d must be 16-byte aligned, 2 <= log_len.
+template <int C>
+__device__ __forceinline__ void stage_signed_row_quad(float (&z)[4], const float *__restrict__ d, int log_len,
+                                                      int nsub, int r, int tid) {
+    const int len = 1 << log_len;
+    const int i0 = 4 * tid < len ? 4 * tid : len - 4;        // idle threads repeat the last quad
+#pragma unroll
+    for (int e = 0; e < 4; ++e) z[e] = 0.0f;
+    for (int h0 = 0; h0 < nsub; h0 += C) {
+        f32x4 vals[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) vals[c] = *(const f32x4 *)(d + ((size_t)min(h0 + c, nsub - 1) << log_len) + i0);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (h0 + c < nsub) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) z[e] += had_sign(r, h0 + c, vals[c][e]);
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ bool stage_partials_quad_ok(const glqh_ysrc &src, const rht_slice &blk, int64_t b,
+                                                       int m_pad) {
+    const uintptr_t base = (uintptr_t)(src.part + b * (int64_t)m_pad + blk.off);
+    return blk.log_len >= 2 && blk.log_len <= fht_wave_max_log<4>() &&
+           ((base | (uintptr_t)(src.part_sstride * 4) | (uintptr_t)(src.part_kstride * 4)) & 15) == 0;
+}
+
+// One slice of an output transform, from split-K partial sums to transform values in
+// registers: thread tid (active when it returns true) ends up with value z[q] of slice
+// element idx[q].  Requires stage_partials_quad_ok().
+template <bool ALWAYS_SYNC = false>
+__device__ __forceinline__ bool partials_fht_quad(float (&z)[4], int (&idx)[4], const glqh_ysrc &src,
+                                                  const rht_slice &blk, int64_t b, int m_pad, float *xchg,
+                                                  int tid) {
+    const bool active = 4 * tid < (1 << blk.log_len);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) idx[q] = fht_wave_index<4>(blk.log_len, active ? tid : 0, q);
+    stage_partials_quad<16>(z, src, blk, b, m_pad, tid);
+    fht_wave<4, ALWAYS_SYNC>(z, blk.log_len, xchg, tid);
+    return active;
 }
 
 template <typename T> __device__ __forceinline__ float act_to_f32(T v);

@@ -24,6 +24,28 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
     const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const XT *xr = x + (int64_t)blockIdx.y * x_stride;
+    struct {
+        OT *orow;
+        float norm;
+        __device__ float aux(int) const { return norm; }
+        __device__ void put(int i, float v, float f) const { orow[i] = f32_to_act<OT>(v * f); }
+    } store = {out + (int64_t)blockIdx.y * n_pad + blk.off + (blk.r << blk.log_len), blk.norm};
+    if constexpr (sizeof(XT) == 2) {
+        // 16-bit activations, block wholly inside the row, 8-byte aligned: the slice in registers
+        if (blk.log_len >= 2 && blk.log_len <= fht_wave_max_log<4>() && blk.off + blk.bs <= in_features &&
+            (((uintptr_t)(xr + blk.off) | (uintptr_t)(sv + blk.off)) & 7) == 0) {   // uniform
+            const int tid = threadIdx.x;
+            const bool live = 4 * tid < (1 << blk.log_len);
+            float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (live) signed_input_quad<XT>(z, 4u * tid, blk.log_len, blk.nsub, blk.r, xr + blk.off, sv + blk.off);
+            fht_wave<4>(z, blk.log_len, s, tid);
+            if (live) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) store.put(fht_wave_index<4>(blk.log_len, tid, q), z[q], blk.norm);
+            }
+            return;
+        }
+    }
     auto val = [&](int h, int i) -> float {
         const int col = blk.off + (h << blk.log_len) + i;
         const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
@@ -31,12 +53,6 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
     };
     if (blk.nsub == 1 && blk.log_len >= 11) stage_signed_slices<RHT_THREADS, 8, 1>(s, blk.log_len, 1, 0, val);
     else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
-    struct {
-        OT *orow;
-        float norm;
-        __device__ float aux(int) const { return norm; }
-        __device__ void put(int i, float v, float f) const { orow[i] = f32_to_act<OT>(v * f); }
-    } store = {out + (int64_t)blockIdx.y * n_pad + blk.off + (blk.r << blk.log_len), blk.norm};
     fht_staged(s, blk.log_len, store);
 }
 

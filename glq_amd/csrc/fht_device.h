@@ -278,37 +278,46 @@ template <> __device__ __forceinline__ void unpack_quad<uint16_t>(uint2 w, float
     f[2] = __builtin_bit_cast(float, w.y << 16); f[3] = __builtin_bit_cast(float, w.y & 0xffff0000u);
 }
 
+// elements i0 .. i0+3 of that vector into registers (i0 a multiple of 4, i0 + 3 < len)
+template <typename XT, int C = 8>
+__device__ __forceinline__ void signed_input_quad(float (&z)[4], unsigned i0, int log_len, int nsub, int r,
+                                                  const XT *__restrict__ xb, const f16 *__restrict__ svb) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) z[e] = 0.0f;
+    for (int h0 = 0; h0 < nsub; h0 += C) {
+        uint2 xv[C], sg[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            // uniform base + 32-bit lane offset: the load takes its base from scalar registers
+            const size_t hb = (size_t)min(h0 + c, nsub - 1) << log_len;
+            xv[c] = *(const uint2 *)(xb + hb + i0);
+            sg[c] = *(const uint2 *)(svb + hb + i0);
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (h0 + c < nsub) {                              // uniform
+                float xf[4], sf[4];
+                unpack_quad<XT>(xv[c], xf);
+                unpack_quad<f16>(sg[c], sf);
+                const float sgn = (__builtin_popcount(r & (h0 + c)) & 1) ? -1.0f : 1.0f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = xf[e] * sf[e];
+                    z[e] = __builtin_fmaf(v, sgn, z[e]);      // z +- v, rounded once like the add
+                }
+            }
+        }
+    }
+}
+
 template <int T, typename XT, int C = 8>
 __device__ __forceinline__ void stage_signed_input_quads(float *lds, int log_len, int nsub, int r,
                                                          const XT *__restrict__ xb,
                                                          const f16 *__restrict__ svb) {
     const unsigned len = 1u << log_len;
     for (unsigned i0 = 4 * threadIdx.x; i0 < len; i0 += 4 * T) {
-        float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int h0 = 0; h0 < nsub; h0 += C) {
-            uint2 xv[C], sg[C];
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                // uniform base + 32-bit lane offset: the load takes its base from scalar registers
-                const size_t hb = (size_t)min(h0 + c, nsub - 1) << log_len;
-                xv[c] = *(const uint2 *)(xb + hb + i0);
-                sg[c] = *(const uint2 *)(svb + hb + i0);
-            }
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                if (h0 + c < nsub) {                              // uniform
-                    float xf[4], sf[4];
-                    unpack_quad<XT>(xv[c], xf);
-                    unpack_quad<f16>(sg[c], sf);
-                    const float sgn = (__builtin_popcount(r & (h0 + c)) & 1) ? -1.0f : 1.0f;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float v = xf[e] * sf[e];
-                        z[e] = __builtin_fmaf(v, sgn, z[e]);      // z +- v, rounded once like the add
-                    }
-                }
-            }
-        }
+        float z[4];
+        signed_input_quad<XT, C>(z, i0, log_len, nsub, r, xb, svb);
 #pragma unroll
         for (int e = 0; e < 4; ++e) lds[lds_pad(i0 + e)] = z[e];
     }

@@ -347,6 +347,79 @@ output_rht_group_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, in
                               log_slice, s);
 }
 
+// The same for layers whose Hadamard blocks have at most G slices: one workgroup per block,
+// one group of 256 threads per slice.  Every group sums the split-K terms of its own rows
+// only and the groups combine each other's sums through LDS, where the kernel above has every
+// slice re-read the whole block: same terms, same order, same bits, 1/nsub of the loads.
+// Rows are multiples of 4 and the partial sums 16-byte aligned (checked by the launcher).
+template <typename YT, int G>
+__global__ void __launch_bounds__(256 * G)
+output_rht_block_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, int log_slice) {
+    extern __shared__ float s[];                   // G exchange buffers, then G sum buffers, one slice each
+    const int z = blockIdx.z;
+    const float *part = g.part[0];
+    const f16 *su = g.su[0];
+    void *y = g.y[0];
+    float scale = g.scale[0];
+    int m_pad = g.m_pad[0], out_features = g.out_features[0];
+#pragma unroll
+    for (int i = 1; i < GLQH_MAX_GROUP; ++i)
+        if (i == z) {
+            part = g.part[i]; su = g.su[i]; y = g.y[i]; scale = g.scale[i];
+            m_pad = g.m_pad[i]; out_features = g.out_features[i];
+        }
+    if ((int)blockIdx.x >= __builtin_popcount((unsigned)m_pad)) return;
+    glqh_meta_args margs;
+    margs.canon = m_pad;
+    const glqh_block_meta bm = glqh_meta_row(margs, nullptr, blockIdx.x);
+    const int log_len = min(bm.log_bs, log_slice);
+    const int nsub = bm.bs >> log_len;                         // <= G
+    const int grp = threadIdx.x >> 8, gt = threadIdx.x & 255;
+    const bool mine = grp < nsub, live = mine && 4 * gt < (1 << log_len);
+    const int base = bm.offset + (grp << log_len);             // this group's rows: slice grp of the block
+    const float norm = rsqrt_pow2(bm.log_bs);
+    const int64_t b = blockIdx.y;
+    float *xchg = s + (grp << log_slice);
+    float *sums = s + (G << log_slice);
+    f16 su_raw[4];                                             // in flight beside the partial sums, used after them
+#pragma unroll
+    for (int q = 0; q < 4; ++q) su_raw[q] = su[mine ? base + fht_wave_index<4>(log_len, live ? gt : 0, q) : 0];
+    if (mine) {
+        glqh_ysrc src = {};
+        src.part = part;
+        src.part_kstride = (int64_t)B * m_pad;
+        src.ksplit = ksplit;
+        src.scale[0] = scale;
+        src.nparts = 1;
+        rht_slice own = {};                                    // v_h for h = grp: rows base .. base + len - 1
+        own.off = base; own.bs = 1 << log_len; own.log_bs = own.log_len = log_len;
+        own.nsub = 1; own.r = 0; own.live = true;
+        float v[4];
+        if (ksplit <= 8) stage_partials_quad<8>(v, src, own, b, m_pad, gt);
+        else if (ksplit <= 12 || G > 2) stage_partials_quad<12>(v, src, own, b, m_pad, gt);
+        else stage_partials_quad<24>(v, src, own, b, m_pad, gt);
+        if (live) *(f32x4 *)(sums + (grp << log_slice) + 4 * gt) = f32x4{v[0], v[1], v[2], v[3]};
+    }
+    __syncthreads();
+    float zv[4] = {0.0f, 0.0f, 0.0f, 0.0f};                    // slice r = grp: sum_h sign(r, h) v_h, h ascending
+    if (live) {
+        for (int h = 0; h < nsub; ++h) {
+            const f32x4 vh = *(const f32x4 *)(sums + (h << log_slice) + 4 * gt);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) zv[e] += had_sign(grp, h, vh[e]);
+        }
+    }
+    fht_wave<4, true>(zv, log_len, xchg, gt);
+    if (live) {
+        YT *yrow = (YT *)y + b * y_stride;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int row = base + fht_wave_index<4>(log_len, gt, q);
+            if (row < out_features) yrow[row] = f32_to_act<YT>(zv[q] * (norm * (float)su_raw[q]));
+        }
+    }
+}
+
 // Few tokens: 1024-point slices, one workgroup each, so that a single row still spreads
 // over the chip (each slice re-reads its whole block).  Many tokens fill the chip by
 // themselves: blocks up to 8192 points are then transformed whole, read once.
@@ -570,6 +643,34 @@ int glqh_launch_output_rht_group(const float *const part[], const void *const su
         g.out_features[i] = (int)out_features[j];
         g.nwg[i] = __builtin_popcountll((unsigned long long)m_pad[j]) * spb;
         if (g.nwg[i] > max_nwg) max_nwg = g.nwg[i];
+    }
+    // blocks of at most four slices: one workgroup per block (see output_rht_block_kernel)
+    bool aligned = spb <= 4 && log_slice == LOG_SLICE;
+    int max_blocks = 0;
+    for (int i = 0; i < n_shards && aligned; ++i) {
+        aligned = (m_pad[i] & 3) == 0 && ((uintptr_t)part[i] & 15) == 0;
+        const int nb = __builtin_popcountll((unsigned long long)m_pad[i]);
+        if (nb > max_blocks) max_blocks = nb;
+    }
+    if (aligned) {
+        const int G = spb <= 1 ? 1 : spb <= 2 ? 2 : 4;
+        dim3 bgrid((unsigned)max_blocks, (unsigned)B, (unsigned)n_shards);
+        const size_t blds = ((size_t)2 * G << log_slice) * sizeof(float);
+#define GLQH_BLK(YT)                                                                                          \
+    do {                                                                                                      \
+        if (G == 1) hipLaunchKernelGGL((output_rht_block_kernel<YT, 1>), bgrid, dim3(256), blds, stream, g,   \
+                                       y_stride, (int)B, ksplit, log_slice);                                  \
+        else if (G == 2) hipLaunchKernelGGL((output_rht_block_kernel<YT, 2>), bgrid, dim3(512), blds, stream, \
+                                            g, y_stride, (int)B, ksplit, log_slice);                          \
+        else hipLaunchKernelGGL((output_rht_block_kernel<YT, 4>), bgrid, dim3(1024), blds, stream, g,         \
+                                y_stride, (int)B, ksplit, log_slice);                                         \
+    } while (0)
+        if (y_dtype == GLQH_F16) GLQH_BLK(f16);
+        else if (y_dtype == GLQH_BF16) GLQH_BLK(uint16_t);
+        else GLQH_BLK(float);
+#undef GLQH_BLK
+        GLQH_LAUNCH_CHECK("output_rht block launch");
+        return 0;
     }
     dim3 grid((unsigned)max_nwg, (unsigned)B, (unsigned)n_shards);
     const size_t lds = rht_lds_bytes(log_slice);

@@ -350,6 +350,17 @@ extern "C" int glqh_fused_linear_trellis_3inst(
             return 1;
         return 0;
     }
+    glqh_meta_args canon_m;
+    if (!has_s2 && !y_rht_out && B <= 4 && glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
+                                                              n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
+        canon_m.canon == m_pad) {
+        // one stage, canonical blocks, a few tokens: the grouped launcher's kernels (a group of one)
+        const float *pt[1] = {part1};
+        const void *sus[1] = {su_f16};
+        void *ys[1] = {y};
+        const float sc[1] = {s1};
+        return glqh_launch_output_rht_group(pt, sus, ys, sc, &m_pad, &out_features, 1, y_dtype, y_stride, B, ks, st);
+    }
     glqh_ysrc src = {};
     src.nparts = has_s2 ? 2 : 1;
     src.part = part1;

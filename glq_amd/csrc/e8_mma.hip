@@ -114,12 +114,28 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
     em_idx<NS> cur = em_load_idx<NS>(qs, idx_offset(0));
     em_idx<NS> nx1 = em_load_idx<NS>(qs, idx_offset(1));
 
-    // table prefix -> LDS with every load in flight before the first write
+    // activations of a slot: one 16-byte LDS slot per (block, token), zero past B and n_pad
+    auto x_load = [&](int sb0, int j) -> u32x4 {
+        j = min(j, slot_blks * TP - 1);
+        const int tl = j / slot_blks, blk = j % slot_blks;
+        const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tl, B - 1) * n_pad + 8 * min(sb0 + blk, nblk - 1));
+        return (tl < B && sb0 + blk < nblk) ? ld : u32x4{0u, 0u, 0u, 0u};
+    };
+    auto x_store = [&](int j, u32x4 v) {
+        if (j < slot_blks * TP) xs[(j % slot_blks) * TP + j / slot_blks] = v;
+    };
+    // table prefix -> LDS with every load in flight before the first write; the first
+    // round of the first tile's activations travels with it
     {
         constexpr int U = 10;                                  // 10 * 1024 * 16 bytes = 160 KiB >= P * 4
-        u32x4 v[U];
+        u32x4 v[U], xv[4];
+        const int sb0 = ((int)blockIdx.x / RB) * slot_blks;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) xv[u] = x_load(sb0, u * EM_THREADS + (int)threadIdx.x);
 #pragma unroll
         for (int u = 0; u < U; ++u) v[u] = ((const u32x4 *)t1)[min(u * EM_THREADS + (int)threadIdx.x, P / 4 - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x_store(u * EM_THREADS + (int)threadIdx.x, xv[u]);
 #pragma unroll
         for (int u = 0; u < U; ++u)
             if (u * EM_THREADS + (int)threadIdx.x < P / 4) lds[u * EM_THREADS + threadIdx.x] = v[u];
@@ -131,22 +147,14 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
     for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const int slot = tile / RB, rb = tile % RB;
         const int sb0 = slot * slot_blks;
-        __syncthreads();                                       // previous tile is done with xs
-        // activations of the slot: one 16-byte slot per (block, token), zero past B and n_pad
-        for (int j0 = 0; j0 < slot_blks * TP; j0 += 4 * EM_THREADS) {
+        const bool first = tile == (int)blockIdx.x;
+        if (!first) __syncthreads();                           // previous tile is done with xs
+        for (int j0 = first ? 4 * EM_THREADS : 0; j0 < slot_blks * TP; j0 += 4 * EM_THREADS) {
             u32x4 v[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int j = min(j0 + u * EM_THREADS + (int)threadIdx.x, slot_blks * TP - 1);
-                const int tl = j / slot_blks, blk = j % slot_blks;
-                const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tl, B - 1) * n_pad + 8 * min(sb0 + blk, nblk - 1));
-                v[u] = (tl < B && sb0 + blk < nblk) ? ld : u32x4{0u, 0u, 0u, 0u};
-            }
+            for (int u = 0; u < 4; ++u) v[u] = x_load(sb0, j0 + u * EM_THREADS + (int)threadIdx.x);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int j = j0 + u * EM_THREADS + (int)threadIdx.x;
-                if (j < slot_blks * TP) xs[(j % slot_blks) * TP + j / slot_blks] = v[u];
-            }
+            for (int u = 0; u < 4; ++u) x_store(j0 + u * EM_THREADS + (int)threadIdx.x, v[u]);
         }
         __syncthreads();
 
@@ -175,7 +183,8 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                 }
             }
             // requested after the lookups, so that waiting for those does not wait for this
-            const em_idx<NS> nx2 = em_load_idx<NS>(qs, idx_offset(sidx + 2));
+            em_idx<NS> nx2 = nx1;
+            if (sidx + 2 < nsteps) nx2 = em_load_idx<NS>(qs, idx_offset(sidx + 2));   // uniform
             if (b0 < nblk_r) {                                 // uniform; past the row the activations are zero
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
@@ -244,7 +253,8 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
     const int64_t RB = (m_pad + rows - 1) / rows;
     const int unit = p->WK * EM_STEP_BLKS;                      // blocks per workgroup step
     const int64_t nunits = (nblk + unit - 1) / unit;
-    const int slot_cap_blks = p->TP == 16 ? 128 : 256;          // activations: at most 32 KB of LDS
+    // activations: at most 32 KB of LDS; one token can afford slots long enough for one tile per workgroup
+    const int slot_cap_blks = p->TP == 16 ? 128 : p->TP == 4 ? 256 : 512;
     const int cus = glqh_device_cus();
     int64_t ks = RB >= cus ? 1 : cus / RB;                      // one tile per workgroup where possible
     if (ks > nunits) ks = nunits;

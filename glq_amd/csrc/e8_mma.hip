@@ -253,8 +253,9 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
     const int64_t RB = (m_pad + rows - 1) / rows;
     const int unit = p->WK * EM_STEP_BLKS;                      // blocks per workgroup step
     const int64_t nunits = (nblk + unit - 1) / unit;
-    // activations: at most 32 KB of LDS; one token can afford slots long enough for one tile per workgroup
-    const int slot_cap_blks = p->TP == 16 ? 128 : p->TP == 4 ? 256 : 512;
+    // activations: at most 32 KB of LDS; slots as long as that allows, so that a workgroup has one
+    // tile (and one table fill per tile) where the shape permits
+    const int slot_cap_blks = p->TP == 16 ? 128 : 512;
     const int cus = glqh_device_cus();
     int64_t ks = RB >= cus ? 1 : cus / RB;                      // one tile per workgroup where possible
     if (ks > nunits) ks = nunits;

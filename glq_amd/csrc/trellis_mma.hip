@@ -568,7 +568,8 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
 #pragma unroll
     for (int s = 0; s < 4; ++s) acc.v[s][0] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (; kp < kp1; kp += TR_WAVES) {
-        const tr_record<R> nx2 = tr_load_record<R>(lane_base + (int64_t)min(kp + 2 * TR_WAVES, kp1 - 1) * 32 * REC);
+        tr_record<R> nx2 = nx1;                                  // nothing is requested past the wave's last record
+        if (kp + 2 * TR_WAVES < kp1) nx2 = tr_load_record<R>(lane_base + (int64_t)(kp + 2 * TR_WAVES) * 32 * REC);
         const u32x4 *xsl = a.live ? lds + ((kp - kp0) * 8 + a.q) * TPS + a.tokl : zero_blk;
         acc = mma_record<R, TP, 1>(cur, a.next1, a.next2, xsl, acc);
         cur = nx1;

@@ -37,6 +37,15 @@ constexpr int LOG_SLICE = GLQH_LOG_SLICE;
 
 __device__ __forceinline__ int lds_pad(int i) { return i + (i >> 5); }
 
+// Workgroup barrier for exchanges through LDS: waits for this wave's LDS operations only.
+// __syncthreads() also drains the wave's global loads, which stalls a transform that runs
+// while a long-latency request of its caller is in flight.
+template <bool LDS_ONLY>
+__device__ __forceinline__ void fht_barrier() {
+    if constexpr (LDS_ONLY) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else __syncthreads();
+}
+
 template <int R, bool LAST, class Store>
 __device__ __forceinline__ void fht_pass(float *lds, int n, int s, Store &store, int tid, int nthr) {
     constexpr int N = 1 << R;
@@ -90,7 +99,7 @@ __device__ __forceinline__ void fht_pass_r(int r, float *lds, int n, int s, Stor
 // workgroup) and pass the result to `store`.  All threads of the workgroup must call it.
 // A workgroup may run several transforms of the same size side by side: each group of nthr
 // threads (numbered tid = 0..nthr-1) passes its own buffer; the barriers are shared.
-template <class Store>
+template <bool LDS_ONLY = false, class Store>
 __device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store, int tid = threadIdx.x,
                                            int nthr = blockDim.x) {
     const int n = 1 << log_n;
@@ -107,7 +116,7 @@ __device__ __forceinline__ void fht_staged(float *lds, int log_n, Store store, i
         if (p == npass - 1) fht_pass_r<true>(r, lds, n, s, store, tid, nthr);
         else {
             fht_pass_r<false>(r, lds, n, s, store, tid, nthr);
-            __syncthreads();
+            fht_barrier<LDS_ONLY>();
         }
     }
 }
@@ -168,7 +177,7 @@ __device__ __forceinline__ void fht_lane_level(float (&v)[E], int lane, int swap
     for (int j = 0; j < E; ++j) v[j] = __builtin_fmaf(v[j], sgn, o[j]);   // exact: one rounding, like the add
 }
 
-template <int E, bool ALWAYS_SYNC = false>
+template <int E, bool ALWAYS_SYNC = false, bool LDS_ONLY = false>
 __device__ __forceinline__ void fht_wave(float (&v)[E], int log_n, float *xchg, int tid) {
     constexpr int LE = fht_wave_log<E>::v;
 #pragma unroll
@@ -192,7 +201,7 @@ __device__ __forceinline__ void fht_wave(float (&v)[E], int log_n, float *xchg, 
     if (lane_bits > 4) fht_lane_level<4>(v, lane, swap32_addr);
     if (lane_bits > 5) fht_lane_level<5>(v, lane, swap32_addr);
     if (log_n <= LE + 6) {
-        if constexpr (ALWAYS_SYNC) __syncthreads();           // the barrier the longer transforms take
+        if constexpr (ALWAYS_SYNC) fht_barrier<LDS_ONLY>();   // the barrier the longer transforms take
         return;
     }
     // levels LE+6 .. log_n-1 pair elements held by different waves: through LDS once, after
@@ -204,7 +213,7 @@ __device__ __forceinline__ void fht_wave(float (&v)[E], int log_n, float *xchg, 
         for (int j = 0; j < E; j += 4)
             *(f32x4 *)(xchg + E * tid + j) = f32x4{v[j], v[j + 1], v[j + 2], v[j + 3]};
     }
-    __syncthreads();
+    fht_barrier<LDS_ONLY>();
     if (tid < nthr) {
 #pragma unroll
         for (int q = 0; q < E; ++q) v[q] = xchg[tid + q * nthr];
@@ -278,10 +287,17 @@ template <> __device__ __forceinline__ void unpack_quad<uint16_t>(uint2 w, float
     f[2] = __builtin_bit_cast(float, w.y << 16); f[3] = __builtin_bit_cast(float, w.y & 0xffff0000u);
 }
 
-// elements i0 .. i0+3 of that vector into registers (i0 a multiple of 4, i0 + 3 < len)
-template <typename XT, int C = 8>
+// elements i0 .. i0+3 of that vector into registers (i0 a multiple of 4, i0 + 3 < len);
+// `issued` runs once, right after the first round of loads has been issued and before any of
+// them is waited for (a place for the caller's own, longer-latency requests)
+struct fht_nothing {
+    __device__ void operator()() const {}
+};
+
+template <typename XT, int C = 8, class Issued = fht_nothing>
 __device__ __forceinline__ void signed_input_quad(float (&z)[4], unsigned i0, int log_len, int nsub, int r,
-                                                  const XT *__restrict__ xb, const f16 *__restrict__ svb) {
+                                                  const XT *__restrict__ xb, const f16 *__restrict__ svb,
+                                                  Issued issued = Issued()) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) z[e] = 0.0f;
     for (int h0 = 0; h0 < nsub; h0 += C) {
@@ -293,6 +309,7 @@ __device__ __forceinline__ void signed_input_quad(float (&z)[4], unsigned i0, in
             xv[c] = *(const uint2 *)(xb + hb + i0);
             sg[c] = *(const uint2 *)(svb + hb + i0);
         }
+        if (h0 == 0) issued();
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             if (h0 + c < nsub) {                              // uniform
@@ -310,18 +327,22 @@ __device__ __forceinline__ void signed_input_quad(float (&z)[4], unsigned i0, in
     }
 }
 
-template <int T, typename XT, int C = 8>
+template <int T, typename XT, int C = 8, bool LDS_ONLY = false, class Issued = fht_nothing>
 __device__ __forceinline__ void stage_signed_input_quads(float *lds, int log_len, int nsub, int r,
                                                          const XT *__restrict__ xb,
-                                                         const f16 *__restrict__ svb) {
+                                                         const f16 *__restrict__ svb, Issued issued = Issued()) {
     const unsigned len = 1u << log_len;
+    bool pending = true;                                       // waves without elements still run `issued`
     for (unsigned i0 = 4 * threadIdx.x; i0 < len; i0 += 4 * T) {
         float z[4];
-        signed_input_quad<XT, C>(z, i0, log_len, nsub, r, xb, svb);
+        if (pending) signed_input_quad<XT, C>(z, i0, log_len, nsub, r, xb, svb, issued);
+        else signed_input_quad<XT, C>(z, i0, log_len, nsub, r, xb, svb);
+        pending = false;
 #pragma unroll
         for (int e = 0; e < 4; ++e) lds[lds_pad(i0 + e)] = z[e];
     }
-    __syncthreads();
+    if (pending) issued();
+    fht_barrier<LDS_ONLY>();
 }
 
 // One workgroup's share of an output transform: the Hadamard block and the slice of it.

@@ -517,23 +517,49 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
         for (int t = 0; t < TP; ++t) {
             if (t >= B) break;
             const XT *xr = x + (int64_t)t * x_stride;
-            __syncthreads();                                     // fbuf free again
-            if (quads && (bm.offset & 3) == 0 && log_len >= 2 && bm.offset + bm.bs <= in_features)
-                stage_signed_input_quads<TR_THREADS, XT>(fbuf, log_len, nsub, r, xr + bm.offset, sv + bm.offset);
+            fht_barrier<true>();                                 // fbuf free again (record loads stay in flight)
+            // The wave's first records are requested as soon as the activations have been: loads
+            // complete in order, so the transform waits for the activations only and the packed
+            // stream's first bytes are on their way while it runs.
+            auto request = [&]() {
+                if (!requested) {
+                    requested = true;
+                    cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
+                    nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
+                }
+            };
+            const bool quad_rows = quads && (bm.offset & 3) == 0 && log_len >= 2 && bm.offset + bm.bs <= in_features;
+            if (quad_rows && log_len <= fht_wave_max_log<4>()) {  // the slice in registers
+                const unsigned tid = threadIdx.x;
+                float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                const bool live = 4 * tid < (1u << log_len);
+                if (live) signed_input_quad<XT>(z, 4 * tid, log_len, nsub, r, xr + bm.offset, sv + bm.offset, request);
+                else request();                                  // waves without elements load nothing
+                fht_wave<4, false, true>(z, log_len, fbuf, tid);
+                if (live) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int i = fht_wave_index<4>(log_len, tid, q);
+                        const int c = lo - c0 + i;               // column inside the slot
+                        const int u = c >> 5, ks = (c >> 4) & 1, qq = (c >> 1) & 3;
+                        const int p = 2 * ((c >> 3) & 1) + (c & 1);
+                        const f16 hv = (f16)(z[q] * norm);
+                        const f16x2 pair = {hv, hv};
+                        xs32[((((u * 2 + ks) * 4) + qq) * mma_tps<TP>() + t) * 4 + p] = __builtin_bit_cast(uint32_t, pair);
+                    }
+                }
+                continue;
+            }
+            if (quad_rows)
+                stage_signed_input_quads<TR_THREADS, XT, 8, true>(fbuf, log_len, nsub, r, xr + bm.offset, sv + bm.offset,
+                                                                  request);
             else
                 stage_signed_slices<TR_THREADS>(fbuf, log_len, nsub, r, [&](int h, int j) -> float {
                     const int col = bm.offset + (h << log_len) + j;
                     const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
                     return col < in_features ? v : 0.0f;
                 });
-            if (!requested) {
-                // The wave's first records are requested here, after the activations have
-                // arrived (loads complete in order, so an earlier request would hold the
-                // transform back by the HBM latency) and before the butterflies, which hide it.
-                requested = true;
-                cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
-                nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
-            }
+            request();
             struct {
                 uint32_t *xs32;
                 int c_rel, t;
@@ -548,7 +574,7 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
                     xs32[((((u * 2 + ks) * 4) + q) * mma_tps<TP>() + t) * 4 + p] = __builtin_bit_cast(uint32_t, pair);
                 }
             } store = {xs32, lo - c0, t, norm};
-            fht_staged(fbuf, log_len, store);
+            fht_staged<true>(fbuf, log_len, store);             // barriers that leave the record loads in flight
         }
     }
     if (!requested) {

@@ -167,18 +167,24 @@ tr_gemv_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x
     const int q1 = min(q0 + steps, nsteps);
     const int c0 = q0 << 6;
 
-    // Request this wave's first TR_PRE records now: the packed stream arrives from HBM while
-    // the prologue below runs.
+    // This wave's first TR_PRE records are requested right behind its first activation loads
+    // (loads complete in order: the transform then waits for the activations only, and the
+    // packed stream arrives from HBM while it runs).
     const uint8_t *row_base = packed + (int64_t)mp * (k >> 5) * 32 * (4 * R);
     const uint8_t *lane_base = row_base + ((int64_t)hf * 32 + l) * (4 * R);   // + q * 64 * 4R
     constexpr int64_t STEP_BYTES = 64 * 4 * R;
     int q = q0 + wave;
     tr_record<R> cur[TR_PRE];
+    bool requested = false;
+    auto request = [&]() {
+        if (requested) return;
+        requested = true;
 #pragma unroll
-    for (int i = 0; i < TR_PRE; ++i) {
-        cur[i] = tr_record<R>{};
-        if (q + i * TR_WAVES < q1) cur[i] = tr_load_record<R>(lane_base + (q + i * TR_WAVES) * STEP_BYTES);
-    }
+        for (int i = 0; i < TR_PRE; ++i) {
+            cur[i] = tr_record<R>{};
+            if (q + i * TR_WAVES < q1) cur[i] = tr_load_record<R>(lane_base + (q + i * TR_WAVES) * STEP_BYTES);
+        }
+    };
 
     // 8-byte loads of four activations / signs are possible (uniform over the launch)
     const bool quads = (((uintptr_t)x | (uintptr_t)sv) & 7) == 0 && (x_stride & 3) == 0;
@@ -195,25 +201,42 @@ tr_gemv_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x
         for (int t = 0; t < NB; ++t) {
             if (t >= B) break;
             const XT *xr = x + (int64_t)t * x_stride;
-            __syncthreads();                                     // fbuf free again
-            if (quads && (bm.offset & 3) == 0 && log_len >= 2 && bm.offset + bm.bs <= in_features)
-                stage_signed_input_quads<TR_THREADS, XT>(fbuf, log_len, nsub, r, xr + bm.offset, sv + bm.offset);
+            fht_barrier<true>();                                 // fbuf free again (record loads stay in flight)
+            f16 *xo = xh + t * Ls + (lo - c0);
+            const bool quad_rows = quads && (bm.offset & 3) == 0 && log_len >= 2 && bm.offset + bm.bs <= in_features;
+            if (quad_rows && log_len <= fht_wave_max_log<4>()) {  // the slice in registers
+                const unsigned tid = threadIdx.x;
+                float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                const bool live = 4 * tid < (1u << log_len);
+                if (live) signed_input_quad<XT>(z, 4 * tid, log_len, nsub, r, xr + bm.offset, sv + bm.offset, request);
+                else request();                                  // waves without elements load nothing
+                fht_wave<4, false, true>(z, log_len, fbuf, tid);
+                if (live) {
+#pragma unroll
+                    for (int qq = 0; qq < 4; ++qq) xo[fht_wave_index<4>(log_len, tid, qq)] = (f16)(z[qq] * norm);
+                }
+                continue;
+            }
+            if (quad_rows)
+                stage_signed_input_quads<TR_THREADS, XT, 8, true>(fbuf, log_len, nsub, r, xr + bm.offset, sv + bm.offset,
+                                                                  request);
             else
                 stage_signed_slices<TR_THREADS>(fbuf, log_len, nsub, r, [&](int h, int j) -> float {
                     const int col = bm.offset + (h << log_len) + j;
                     const float v = act_to_f32<XT>(xr[min(col, in_features - 1)]) * (float)sv[col];
                     return col < in_features ? v : 0.0f;
                 });
-            f16 *xo = xh + t * Ls + (lo - c0);
+            request();
             struct {
                 f16 *xo;
                 float norm;
                 __device__ float aux(int) const { return norm; }
                 __device__ void put(int i, float v, float f) const { xo[i] = (f16)(v * f); }
             } store = {xo, norm};
-            fht_staged(fbuf, log_len, store);
+            fht_staged<true>(fbuf, log_len, store);             // barriers that leave the record loads in flight
         }
     }
+    request();                                                   // a slot without columns of its own
     __syncthreads();
 
     // ---- decode loop ----

@@ -233,9 +233,10 @@ tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int
     }
     for (int c0 = kp0; c0 < kp1; c0 += CH) {
         const int c1 = min(c0 + CH, kp1);
-        __syncthreads();                                       // previous chunk consumed
+        // LDS-only barriers: the record requested ahead stays in flight across them
+        fht_barrier<true>();                                   // previous chunk consumed
         mma_stage<TP, NT>((uint32_t *)xs_lds, x, B, k, tok0, c0, c1 - c0);
-        __syncthreads();
+        fht_barrier<true>();
         for (; kp < c1; kp += TR_WAVES) {
             tr_record<R> nxt = cur;
             if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
@@ -392,9 +393,10 @@ tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict_
             r0 = r1;
             r1 = r2;
         }
-        __syncthreads();                                         // chunk consumed by every wave
+        // LDS-only barriers: the records requested two ahead stay in flight across them
+        fht_barrier<true>();                                     // chunk consumed by every wave
         pf_stage_write((uint32_t *)xs_lds, next, M, tok0, kp1 - (c0 + PF_CH));
-        __syncthreads();
+        fht_barrier<true>();
     }
     if (!active) return;
     // lane holds rows i0 .. i0+3 (consecutive) of token tokl for every (s, tt)

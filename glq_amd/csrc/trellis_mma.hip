@@ -664,7 +664,7 @@ constexpr int MMA_LDS_MAX = 64 * 1024;
 
 template <int TP, int NT>
 constexpr int mma_chunk_cap() {
-    return TP == 1 ? 448 : TP == 4 ? 64 : NT == 1 ? 8 : 4;
+    return TP == 1 ? 448 : TP == 4 ? 64 : NT == 1 ? 16 : 4;
 }
 
 template <int R, int TP, int NT>

@@ -90,11 +90,46 @@ constexpr int AT_WAVES = AT_THREADS / 64;
 // keys 0..n-1, softmax, weighted rows of V, result to out (D bf16).  NEWROW: row n-1 of K and V
 // is not read from the cache but from knew / vnew (LDS, D bf16 each) -- the caller has just
 // produced it and another workgroup is writing it to the cache at the same time.
+// four keys of a thread's round (keys j0 + u * AT_THREADS / 8; 8 lanes per key, 16 + 16 bytes each)
+struct attn_kregs {
+    u32x4 k0[4], k1[4];
+};
+
+__device__ __forceinline__ attn_kregs attn_load_k(const uint16_t *__restrict__ K, int j0, int last) {
+    constexpr int D = 128;
+    const int sub = threadIdx.x & 7;
+    attn_kregs r;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int j = min(j0 + u * (AT_THREADS / 8), last);
+        r.k0[u] = *(const u32x4 *)(K + (int64_t)j * D + sub * 8);
+        r.k1[u] = *(const u32x4 *)(K + (int64_t)j * D + 64 + sub * 8);
+    }
+    return r;
+}
+
+// four rows of V of a thread's round (rows j0 + u * 4 * AT_WAVES; 16 lanes per row, 16 bytes each)
+struct attn_vregs {
+    u32x4 v[4];
+};
+
+__device__ __forceinline__ attn_vregs attn_load_v(const uint16_t *__restrict__ V, int j0, int last) {
+    constexpr int D = 128;
+    const int vcol = threadIdx.x & 15;
+    attn_vregs r;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) r.v[u] = *(const u32x4 *)(V + (int64_t)min(j0 + u * 4 * AT_WAVES, last) * D + 8 * vcol);
+    return r;
+}
+
+// `first_k`: the thread's first round of keys when the caller has requested it already
+// (attn_load_k(K, threadIdx.x >> 3, last) with last as computed here), else nullptr.
 template <bool NEWROW>
 __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__restrict__ K,
                                           const uint16_t *__restrict__ V, int n, const uint16_t *knew,
                                           const uint16_t *vnew, float *sc, float *red,
-                                          float (*part)[128], uint16_t *__restrict__ out) {
+                                          float (*part)[128], uint16_t *__restrict__ out,
+                                          const attn_kregs *first_k = nullptr) {
     constexpr int D = 128;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int last = NEWROW ? max(n - 2, 0) : n - 1;          // last row that is read from the cache
@@ -102,27 +137,25 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
     float mx = -3.0e38f;
     // four keys per thread in flight (512 keys per round of the workgroup)
     for (int j0 = threadIdx.x >> 3; j0 < n; j0 += 4 * (AT_THREADS / 8)) {
-        u32x4 k0[4], k1[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int j = min(j0 + u * (AT_THREADS / 8), last);
-            k0[u] = *(const u32x4 *)(K + (int64_t)j * D + sub * 8);
-            k1[u] = *(const u32x4 *)(K + (int64_t)j * D + 64 + sub * 8);
-        }
+        attn_kregs kr;
+        if (first_k && j0 == (int)(threadIdx.x >> 3)) kr = *first_k;
+        else kr = attn_load_k(K, j0, last);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int j = j0 + u * (AT_THREADS / 8);
+            u32x4 k0 = kr.k0[u], k1 = kr.k1[u];
             if (NEWROW && j == n - 1) {
-                k0[u] = *(const u32x4 *)(knew + sub * 8);
-                k1[u] = *(const u32x4 *)(knew + 64 + sub * 8);
+                k0 = *(const u32x4 *)(knew + sub * 8);
+                k1 = *(const u32x4 *)(knew + 64 + sub * 8);
             }
             float s = 0.0f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                s += qs[sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k0[u][e] & 0xFFFFu));
-                s += qs[sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k0[u][e] >> 16));
-                s += qs[64 + sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(k1[u][e] & 0xFFFFu));
-                s += qs[64 + sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(k1[u][e] >> 16));
+                const uint32_t w0 = k0[e], w1 = k1[e];
+                s += qs[sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(w0 & 0xFFFFu));
+                s += qs[sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(w0 >> 16));
+                s += qs[64 + sub * 8 + 2 * e] * bf16_bits_to_f32((uint16_t)(w1 & 0xFFFFu));
+                s += qs[64 + sub * 8 + 2 * e + 1] * bf16_bits_to_f32((uint16_t)(w1 >> 16));
             }
             s += __shfl_xor(s, 1, GLQH_WAVE);
             s += __shfl_xor(s, 2, GLQH_WAVE);
@@ -133,6 +166,12 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
             }
         }
     }
+    // weighted rows of V: 16 lanes per row (8 columns, one 16-byte load each), 4 rows per wave
+    // per load and four loads in flight: 256 keys per round of the workgroup.  The first round
+    // is requested here, ahead of the softmax, every later one a round ahead of its use.
+    const int vr = lane >> 4, vcol = lane & 15;
+    const int vj0 = wave * 4 + vr;
+    attn_vregs vcur = attn_load_v(V, vj0, last);
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
     __syncthreads();
@@ -152,29 +191,28 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
     float tot = 0.0f;
 #pragma unroll
     for (int w = 0; w < AT_WAVES; ++w) tot += red[w];
-    // weighted rows of V: 16 lanes per row (8 columns, one 16-byte load each), 4 rows per wave
-    // per load and four loads in flight: 256 keys per round of the workgroup
-    const int vr = lane >> 4, vcol = lane & 15;
     float a[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) a[e] = 0.0f;
-    for (int j0 = wave * 4 + vr; j0 < n; j0 += 4 * 4 * AT_WAVES) {
-        u32x4 vv[4];
+    for (int j0 = vj0; j0 < n; j0 += 4 * 4 * AT_WAVES) {
+        attn_vregs vnext = vcur;
+        if (j0 + 4 * 4 * AT_WAVES < n) vnext = attn_load_v(V, j0 + 4 * 4 * AT_WAVES, last);
         float pw[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int j = j0 + u * 4 * AT_WAVES;
-            vv[u] = *(const u32x4 *)(V + (int64_t)min(j, last) * D + 8 * vcol);
-            if (NEWROW && j == n - 1) vv[u] = *(const u32x4 *)(vnew + 8 * vcol);
+            if (NEWROW && j == n - 1) vcur.v[u] = *(const u32x4 *)(vnew + 8 * vcol);
             pw[u] = j < n ? sc[j] : 0.0f;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                a[2 * e] += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u][e] & 0xFFFFu));
-                a[2 * e + 1] += pw[u] * bf16_bits_to_f32((uint16_t)(vv[u][e] >> 16));
+                const uint32_t w = vcur.v[u][e];
+                a[2 * e] += pw[u] * bf16_bits_to_f32((uint16_t)(w & 0xFFFFu));
+                a[2 * e + 1] += pw[u] * bf16_bits_to_f32((uint16_t)(w >> 16));
             }
+        vcur = vnext;
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {                               // the wave's four row lanes
@@ -541,28 +579,43 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
     src.scale[0] = grp == 0 ? a.scale[0] : grp == 1 ? a.scale[1] : a.scale[2];
     src.nparts = 1;
     const f16 *su = grp == 0 ? a.su[0] : grp == 1 ? a.su[1] : a.su[2];
+    // sign, cosine and sine values of the rotation step: requested now, used after the transform
+    const int d = min(gt, half - 1);
+    const f16 su_a = su[row0 + d], su_b = su[row0 + d + half];
+    uint16_t cs[4] = {0, 0, 0, 0};
+    if (grp != 2 && apply_rope) {
+        cs[0] = cos_t[p * D + d]; cs[1] = sin_t[p * D + d];
+        cs[2] = cos_t[p * D + d + half]; cs[3] = sin_t[p * D + d + half];
+    }
+    const uint16_t *Kh = kc + (int64_t)g * max_len * D, *Vh = vc + (int64_t)g * max_len * D;
+    attn_kregs first_k;
     {
         // three transforms of possibly different sizes side by side: one shared barrier each
         float zq[4];
         int idx[4];
-        const bool live = partials_fht_quad<true>(zq, idx, src, blk, 0, m, buf, gt);
-        __syncthreads();                           // the exchanges have been read: buf takes the result
+        const bool live = 4 * gt < (1 << blk.log_len);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) idx[q] = fht_wave_index<4>(blk.log_len, live ? gt : 0, q);
+        stage_partials_quad<16>(zq, src, blk, 0, m, gt);
+        // the first round of cached keys travels while the transform and the rotation run
+        first_k = attn_load_k(Kh, tid >> 3, max(n - 2, 0));
+        // barriers that wait for LDS only: the key loads stay in flight across them
+        fht_wave<4, true, true>(zq, blk.log_len, buf, gt);
+        fht_barrier<true>();                       // the exchanges have been read: buf takes the result
         if (live) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) buf[lds_pad(idx[q])] = zq[q];
         }
     }
-    __syncthreads();
+    fht_barrier<true>();
     if (gt < half) {
         const int li = row0 - (blk.off + (blk.r << blk.log_len));  // the head inside the slice
-        const int d = gt;
-        const float va = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(li + d)] * (blk.norm * (float)su[row0 + d])));
-        const float vb = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(li + d + half)] *
-                                                           (blk.norm * (float)su[row0 + d + half])));
+        const float va = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(li + d)] * (blk.norm * (float)su_a)));
+        const float vb = bf16_bits_to_f32(f32_to_bf16_bits(buf[lds_pad(li + d + half)] * (blk.norm * (float)su_b)));
         uint16_t o0 = f32_to_bf16_bits(va), o1 = f32_to_bf16_bits(vb);
         if (grp != 2 && apply_rope) {
-            const float c0 = bf16_bits_to_f32(cos_t[p * D + d]), s0 = bf16_bits_to_f32(sin_t[p * D + d]);
-            const float c1 = bf16_bits_to_f32(cos_t[p * D + d + half]), s1 = bf16_bits_to_f32(sin_t[p * D + d + half]);
+            const float c0 = bf16_bits_to_f32(cs[0]), s0 = bf16_bits_to_f32(cs[1]);
+            const float c1 = bf16_bits_to_f32(cs[2]), s1 = bf16_bits_to_f32(cs[3]);
             o0 = f32_to_bf16_bits(va * c0 - vb * s0);
             o1 = f32_to_bf16_bits(vb * c1 + va * s1);
         }
@@ -580,9 +633,8 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
             }
         }
     }
-    __syncthreads();
-    attn_core<true>(qs, kc + (int64_t)g * max_len * D, vc + (int64_t)g * max_len * D, n, knew, vnew, sc, red, part,
-                    out + (int64_t)h * D);
+    fht_barrier<true>();                           // qs, knew, vnew are in LDS
+    attn_core<true>(qs, Kh, Vh, n, knew, vnew, sc, red, part, out + (int64_t)h * D, &first_k);
 }
 
 }  // namespace

@@ -426,10 +426,11 @@ __device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ys
     const int total = blk.nsub * nst * ks;
     const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
     const bool active = 4 * tid < len;
-    const int i0 = active ? 4 * tid : len - 4;             // idle threads repeat the last quad
+    const int i0 = 4 * tid;
     float v[4], acc[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) z[e] = v[e] = acc[e] = 0.0f;
+    if (!active) return;                                    // threads without elements issue nothing
     int h = 0, st = 0, k = 0;                               // position of term t0 (uniform)
     for (int t0 = 0; t0 < total; t0 += C) {
         f32x4 vals[C];
@@ -476,9 +477,10 @@ template <int C>
 __device__ __forceinline__ void stage_signed_row_quad(float (&z)[4], const float *__restrict__ d, int log_len,
                                                       int nsub, int r, int tid) {
     const int len = 1 << log_len;
-    const int i0 = 4 * tid < len ? 4 * tid : len - 4;        // idle threads repeat the last quad
+    const int i0 = 4 * tid;
 #pragma unroll
     for (int e = 0; e < 4; ++e) z[e] = 0.0f;
+    if (i0 >= len) return;                                   // threads without elements issue nothing
     for (int h0 = 0; h0 < nsub; h0 += C) {
         f32x4 vals[C];
 #pragma unroll

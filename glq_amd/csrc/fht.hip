@@ -348,13 +348,14 @@ output_rht_group_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, in
 }
 
 // The same for layers whose Hadamard blocks have at most G slices: one workgroup per block,
-// one group of 256 threads per slice.  Every group sums the split-K terms of its own rows
-// only and the groups combine each other's sums through LDS, where the kernel above has every
-// slice re-read the whole block: same terms, same order, same bits, 1/nsub of the loads.
-// Rows are multiples of 4 and the partial sums 16-byte aligned (checked by the launcher).
-template <typename YT, int G>
-__global__ void __launch_bounds__(256 * G)
+// one group of 1024 / E threads per slice (E elements per thread).  Every group sums the split-K terms of its own rows only and the groups
+// combine each other's sums through LDS, where the kernel above has every slice re-read the
+// whole block: same terms, same order, same bits, 1/nsub of the loads.  Rows are multiples
+// of E and the partial sums 16-byte aligned (checked by the launcher).
+template <typename YT, int G, int E>
+__global__ void __launch_bounds__((1024 / E) * G)
 output_rht_block_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, int log_slice) {
+    constexpr int GS = 1024 / E;                   // threads per slice
     extern __shared__ float s[];                   // G exchange buffers, then G sum buffers, one slice each
     const int z = blockIdx.z;
     const float *part = g.part[0];
@@ -374,16 +375,16 @@ output_rht_block_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, in
     const glqh_block_meta bm = glqh_meta_row(margs, nullptr, blockIdx.x);
     const int log_len = min(bm.log_bs, log_slice);
     const int nsub = bm.bs >> log_len;                         // <= G
-    const int grp = threadIdx.x >> 8, gt = threadIdx.x & 255;
-    const bool mine = grp < nsub, live = mine && 4 * gt < (1 << log_len);
+    const int grp = threadIdx.x / GS, gt = threadIdx.x % GS;
+    const bool mine = grp < nsub, live = mine && E * gt < (1 << log_len);
     const int base = bm.offset + (grp << log_len);             // this group's rows: slice grp of the block
     const float norm = rsqrt_pow2(bm.log_bs);
     const int64_t b = blockIdx.y;
     float *xchg = s + (grp << log_slice);
     float *sums = s + (G << log_slice);
-    f16 su_raw[4];                                             // in flight beside the partial sums, used after them
+    f16 su_raw[E];                                             // in flight beside the partial sums, used after them
 #pragma unroll
-    for (int q = 0; q < 4; ++q) su_raw[q] = su[mine ? base + fht_wave_index<4>(log_len, live ? gt : 0, q) : 0];
+    for (int q = 0; q < E; ++q) su_raw[q] = su[mine ? base + fht_wave_index<E>(log_len, live ? gt : 0, q) : 0];
     if (mine) {
         glqh_ysrc src = {};
         src.part = part;
@@ -394,27 +395,39 @@ output_rht_block_kernel(rht_out_group g, int64_t y_stride, int B, int ksplit, in
         rht_slice own = {};                                    // v_h for h = grp: rows base .. base + len - 1
         own.off = base; own.bs = 1 << log_len; own.log_bs = own.log_len = log_len;
         own.nsub = 1; own.r = 0; own.live = true;
-        float v[4];
-        if (ksplit <= 8) stage_partials_quad<8>(v, src, own, b, m_pad, gt);
-        else if (ksplit <= 12 || G > 2) stage_partials_quad<12>(v, src, own, b, m_pad, gt);
-        else stage_partials_quad<24>(v, src, own, b, m_pad, gt);
-        if (live) *(f32x4 *)(sums + (grp << log_slice) + 4 * gt) = f32x4{v[0], v[1], v[2], v[3]};
-    }
-    __syncthreads();
-    float zv[4] = {0.0f, 0.0f, 0.0f, 0.0f};                    // slice r = grp: sum_h sign(r, h) v_h, h ascending
-    if (live) {
-        for (int h = 0; h < nsub; ++h) {
-            const f32x4 vh = *(const f32x4 *)(sums + (h << log_slice) + 4 * gt);
+        float v[E];
+        // terms in flight: as many as there are (clamped repeats still cost their issue slots)
+        if (ksplit <= 2) stage_partials_vec<E, 2>(v, src, own, b, m_pad, gt);
+        else if (ksplit <= 4) stage_partials_vec<E, 4>(v, src, own, b, m_pad, gt);
+        else if (ksplit <= 8) stage_partials_vec<E, 8>(v, src, own, b, m_pad, gt);
+        else if (ksplit <= 12 || G > 2) stage_partials_vec<E, 12>(v, src, own, b, m_pad, gt);
+        else stage_partials_vec<E, 24>(v, src, own, b, m_pad, gt);
+        if (live) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) zv[e] += had_sign(grp, h, vh[e]);
+            for (int w = 0; w < E; w += 4)
+                *(f32x4 *)(sums + (grp << log_slice) + E * gt + w) = f32x4{v[w], v[w + 1], v[w + 2], v[w + 3]};
         }
     }
-    fht_wave<4, true>(zv, log_len, xchg, gt);
+    __syncthreads();
+    float zv[E];                                               // slice r = grp: sum_h sign(r, h) v_h, h ascending
+#pragma unroll
+    for (int e = 0; e < E; ++e) zv[e] = 0.0f;
+    if (live) {
+        for (int h = 0; h < nsub; ++h) {
+#pragma unroll
+            for (int w = 0; w < E; w += 4) {
+                const f32x4 vh = *(const f32x4 *)(sums + (h << log_slice) + E * gt + w);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) zv[w + e] += had_sign(grp, h, vh[e]);
+            }
+        }
+    }
+    fht_wave<E, true>(zv, log_len, xchg, gt);
     if (live) {
         YT *yrow = (YT *)y + b * y_stride;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int row = base + fht_wave_index<4>(log_len, gt, q);
+        for (int q = 0; q < E; ++q) {
+            const int row = base + fht_wave_index<E>(log_len, gt, q);
             if (row < out_features) yrow[row] = f32_to_act<YT>(zv[q] * (norm * (float)su_raw[q]));
         }
     }
@@ -644,7 +657,8 @@ int glqh_launch_output_rht_group(const float *const part[], const void *const su
         g.nwg[i] = __builtin_popcountll((unsigned long long)m_pad[j]) * spb;
         if (g.nwg[i] > max_nwg) max_nwg = g.nwg[i];
     }
-    // blocks of at most four slices: one workgroup per block (see output_rht_block_kernel)
+    // blocks of at most four slices: one workgroup per block (see output_rht_block_kernel); larger
+    // blocks are faster as one workgroup per slice (measured with eight slices on 1024 threads)
     bool aligned = spb <= 4 && log_slice == LOG_SLICE;
     int max_blocks = 0;
     for (int i = 0; i < n_shards && aligned; ++i) {
@@ -658,11 +672,11 @@ int glqh_launch_output_rht_group(const float *const part[], const void *const su
         const size_t blds = ((size_t)2 * G << log_slice) * sizeof(float);
 #define GLQH_BLK(YT)                                                                                          \
     do {                                                                                                      \
-        if (G == 1) hipLaunchKernelGGL((output_rht_block_kernel<YT, 1>), bgrid, dim3(256), blds, stream, g,   \
-                                       y_stride, (int)B, ksplit, log_slice);                                  \
-        else if (G == 2) hipLaunchKernelGGL((output_rht_block_kernel<YT, 2>), bgrid, dim3(512), blds, stream, \
-                                            g, y_stride, (int)B, ksplit, log_slice);                          \
-        else hipLaunchKernelGGL((output_rht_block_kernel<YT, 4>), bgrid, dim3(1024), blds, stream, g,         \
+        if (G == 1) hipLaunchKernelGGL((output_rht_block_kernel<YT, 1, 4>), bgrid, dim3(256), blds, stream,   \
+                                       g, y_stride, (int)B, ksplit, log_slice);                               \
+        else if (G == 2) hipLaunchKernelGGL((output_rht_block_kernel<YT, 2, 4>), bgrid, dim3(512), blds,      \
+                                            stream, g, y_stride, (int)B, ksplit, log_slice);                  \
+        else hipLaunchKernelGGL((output_rht_block_kernel<YT, 4, 4>), bgrid, dim3(1024), blds, stream, g,      \
                                 y_stride, (int)B, ksplit, log_slice);                                         \
     } while (0)
         if (y_dtype == GLQH_F16) GLQH_BLK(f16);

@@ -416,29 +416,32 @@ __device__ __forceinline__ void stage_partials(float *s, const glqh_ysrc &src, c
 }
 
 // stage_partials for the register transform: the same sums in the same order, but thread tid
-// takes elements 4*tid .. 4*tid+3 of the slice with one 16-byte load per term and keeps them in
-// registers.  The caller has checked 2 <= log_len and that every term's row is 16-byte aligned.
-template <int C>
-__device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ysrc &src, const rht_slice &blk,
-                                                    int64_t b, int m_pad, int tid) {
+// takes elements E*tid .. E*tid+E-1 of the slice (E = 4 or 8) with E/4 16-byte loads per term
+// and keeps them in registers.  The caller has checked log2(E) <= log_len and that every term's
+// row is 16-byte aligned.
+template <int E, int C>
+__device__ __forceinline__ void stage_partials_vec(float (&z)[E], const glqh_ysrc &src, const rht_slice &blk,
+                                                   int64_t b, int m_pad, int tid) {
+    constexpr int NV = E / 4;
     const int len = 1 << blk.log_len;
     const int ks = src.ksplit, nst = src.nparts;
     const int total = blk.nsub * nst * ks;
     const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
-    const bool active = 4 * tid < len;
-    const int i0 = 4 * tid;
-    float v[4], acc[4];
+    const bool active = E * tid < len;
+    const int i0 = E * tid;
+    float v[E], acc[E];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) z[e] = v[e] = acc[e] = 0.0f;
+    for (int e = 0; e < E; ++e) z[e] = v[e] = acc[e] = 0.0f;
     if (!active) return;                                    // threads without elements issue nothing
     int h = 0, st = 0, k = 0;                               // position of term t0 (uniform)
     for (int t0 = 0; t0 < total; t0 += C) {
-        f32x4 vals[C];
+        f32x4 vals[C][NV];
         int hh = h, ss = st, kk = k;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const float *p = pbase + ss * src.part_sstride + kk * src.part_kstride + (hh << blk.log_len);
-            vals[c] = *(const f32x4 *)(p + i0);
+#pragma unroll
+            for (int w = 0; w < NV; ++w) vals[c][w] = *(const f32x4 *)(p + i0 + 4 * w);
             if (t0 + c + 1 < total) {                       // advance, clamped at the last term
                 if (++kk == ks) { kk = 0; if (++ss == nst) { ss = 0; ++hh; } }
             }
@@ -447,17 +450,17 @@ __device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ys
         for (int c = 0; c < C; ++c) {
             if (t0 + c < total) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] += vals[c][e];
+                for (int e = 0; e < E; ++e) acc[e] += vals[c][e >> 2][e & 3];
                 if (++k == ks) {
                     const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
                                    : st == 2 ? src.scale[2] : src.scale[3];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) { v[e] += sc * acc[e]; acc[e] = 0.0f; }
+                    for (int e = 0; e < E; ++e) { v[e] += sc * acc[e]; acc[e] = 0.0f; }
                     k = 0;
                     if (++st == nst) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if (src.copy_out && blk.r == 0 && active)
+                        for (int e = 0; e < E; ++e) {
+                            if (src.copy_out && blk.r == 0)
                                 src.copy_out[b * src.copy_stride + blk.off + (h << blk.log_len) + i0 + e] = v[e];
                             z[e] += had_sign(blk.r, h, v[e]);
                             v[e] = 0.0f;
@@ -469,6 +472,12 @@ __device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ys
             }
         }
     }
+}
+
+template <int C>
+__device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ysrc &src, const rht_slice &blk,
+                                                    int64_t b, int m_pad, int tid) {
+    stage_partials_vec<4, C>(z, src, blk, b, m_pad, tid);
 }
 
 // The same for a plain fp32 row: z[e] = sum_h sign(r, h) * d[h * len + 4*tid + e], h ascending

@@ -37,7 +37,7 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
             const int tid = threadIdx.x;
             const bool live = 4 * tid < (1 << blk.log_len);
             float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (live) signed_input_quad<XT>(z, 4u * tid, blk.log_len, blk.nsub, blk.r, xr + blk.off, sv + blk.off);
+            if (live) signed_input_quad_n<XT>(z, 4u * tid, blk.log_len, blk.nsub, blk.r, xr + blk.off, sv + blk.off);
             fht_wave<4>(z, blk.log_len, s, tid);
             if (live) {
 #pragma unroll

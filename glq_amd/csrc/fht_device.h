@@ -327,6 +327,18 @@ __device__ __forceinline__ void signed_input_quad(float (&z)[4], unsigned i0, in
     }
 }
 
+// signed_input_quad with as many terms in flight as the block has sub-slices, up to eight
+// (a clamped repeat of the last term still costs its issue slots)
+template <typename XT, class Issued = fht_nothing>
+__device__ __forceinline__ void signed_input_quad_n(float (&z)[4], unsigned i0, int log_len, int nsub, int r,
+                                                    const XT *__restrict__ xb, const f16 *__restrict__ svb,
+                                                    Issued issued = Issued()) {
+    if (nsub <= 1) signed_input_quad<XT, 1>(z, i0, log_len, nsub, r, xb, svb, issued);
+    else if (nsub <= 2) signed_input_quad<XT, 2>(z, i0, log_len, nsub, r, xb, svb, issued);
+    else if (nsub <= 4) signed_input_quad<XT, 4>(z, i0, log_len, nsub, r, xb, svb, issued);
+    else signed_input_quad<XT, 8>(z, i0, log_len, nsub, r, xb, svb, issued);
+}
+
 template <int T, typename XT, int C = 8, bool LDS_ONLY = false, class Issued = fht_nothing>
 __device__ __forceinline__ void stage_signed_input_quads(float *lds, int log_len, int nsub, int r,
                                                          const XT *__restrict__ xb,

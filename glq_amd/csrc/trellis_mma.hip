@@ -535,7 +535,7 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
                 const unsigned tid = threadIdx.x;
                 float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
                 const bool live = 4 * tid < (1u << log_len);
-                if (live) signed_input_quad<XT>(z, 4 * tid, log_len, nsub, r, xr + bm.offset, sv + bm.offset, request);
+                if (live) signed_input_quad_n<XT>(z, 4 * tid, log_len, nsub, r, xr + bm.offset, sv + bm.offset, request);
                 else request();                                  // waves without elements load nothing
                 fht_wave<4, false, true>(z, log_len, fbuf, tid);
                 if (live) {

@@ -596,7 +596,7 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
         const bool live = 4 * gt < (1 << blk.log_len);
 #pragma unroll
         for (int q = 0; q < 4; ++q) idx[q] = fht_wave_index<4>(blk.log_len, live ? gt : 0, q);
-        stage_partials_quad<16>(zq, src, blk, 0, m, gt);
+        stage_partials_quad_n(zq, src, blk, 0, m, gt);
         // the first round of cached keys travels while the transform and the rotation run
         first_k = attn_load_k(Kh, tid >> 3, max(n - 2, 0));
         // barriers that wait for LDS only: the key loads stay in flight across them

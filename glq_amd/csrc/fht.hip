@@ -276,7 +276,7 @@ output_rht_body(const glqh_ysrc &src, const f16 *__restrict__ su, YT *__restrict
             idx[q] = fht_wave_index<4>(blk.log_len, active ? tid : 0, q);
             su_raw[q] = su[base + idx[q]];
         }
-        if constexpr (PARTS) stage_partials_quad<16>(z, src, blk, b, m_pad, tid);
+        if constexpr (PARTS) stage_partials_quad_n(z, src, blk, b, m_pad, tid);
         else stage_signed_row_quad<8>(z, src.direct + b * src.stride + blk.off, blk.log_len, blk.nsub, blk.r, tid);
         fht_wave<4>(z, blk.log_len, s, tid);
         if (active) {

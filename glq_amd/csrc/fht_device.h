@@ -492,6 +492,17 @@ __device__ __forceinline__ void stage_partials_quad(float (&z)[4], const glqh_ys
     stage_partials_vec<4, C>(z, src, blk, b, m_pad, tid);
 }
 
+// with as many terms in flight as the slice has, up to sixteen (a clamped repeat of the last
+// term still costs its issue slots)
+__device__ __forceinline__ void stage_partials_quad_n(float (&z)[4], const glqh_ysrc &src, const rht_slice &blk,
+                                                      int64_t b, int m_pad, int tid) {
+    const int total = blk.nsub * src.nparts * src.ksplit;
+    if (total <= 2) stage_partials_vec<4, 2>(z, src, blk, b, m_pad, tid);
+    else if (total <= 4) stage_partials_vec<4, 4>(z, src, blk, b, m_pad, tid);
+    else if (total <= 8) stage_partials_vec<4, 8>(z, src, blk, b, m_pad, tid);
+    else stage_partials_vec<4, 16>(z, src, blk, b, m_pad, tid);
+}
+
 // The same for a plain fp32 row: z[e] = sum_h sign(r, h) * d[h * len + 4*tid + e], h ascending
 // as in stage_signed_slices.  d must be 16-byte aligned, 2 <= log_len.
 template <int C>
@@ -533,7 +544,7 @@ __device__ __forceinline__ bool partials_fht_quad(float (&z)[4], int (&idx)[4], 
     const bool active = 4 * tid < (1 << blk.log_len);
 #pragma unroll
     for (int q = 0; q < 4; ++q) idx[q] = fht_wave_index<4>(blk.log_len, active ? tid : 0, q);
-    stage_partials_quad<16>(z, src, blk, b, m_pad, tid);
+    stage_partials_quad_n(z, src, blk, b, m_pad, tid);
     fht_wave<4, ALWAYS_SYNC>(z, blk.log_len, xchg, tid);
     return active;
 }

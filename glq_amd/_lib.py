@@ -44,6 +44,7 @@ SIGNATURES = {
                 c_dbl, c_dbl, c_i64, c_i64, c_i64, c_i64,
                 c_vp, c_int, c_i64, c_vp, c_i64, c_vp, c_sz, c_vp]),
     "glqh_e8_pack_table": (c_int, [c_vp, c_i64, c_vp, c_vp, c_vp]),
+    "glqh_e8_repack_table": (c_int, [c_vp, c_i64, c_vp, c_vp, c_vp]),
     "glqh_e8_matmul_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64]),
     "glqh_e8_dequant_matmul": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
@@ -68,6 +69,7 @@ SIGNATURES = {
     "glqh_trellis_quantize_workspace_bytes": (c_sz, [c_int, c_i64]),
     "glqh_trellis_quantize_tiles": (c_int, [c_vp, c_i64, c_int, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "glqh_trellis_pack_states": (c_int, [c_vp, c_i64, c_i64, c_int, c_vp, c_vp]),
+    "glqh_viterbi_acs_step": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_int, c_vp]),
     # include/glq_decoder_ops.h
     "glqh_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),
     "glqh_add_rmsnorm_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_dbl, c_vp]),

@@ -584,6 +584,15 @@ extern "C" int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, u
     return glqh_launch_e8_pack_table(codebook_f16, n_entries, packed_out, bad_dev, (hipStream_t)stream);
 }
 
+extern "C" int glqh_e8_repack_table(const uint32_t *codebook_packed, int64_t n_entries,
+                                    uint32_t *packed_out, int32_t *bad_dev, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(codebook_packed && packed_out && bad_dev, "e8 repack table: null pointer");
+    GLQH_REQUIRE(n_entries >= 1 && n_entries <= 65536, "e8 repack table: %lld entries (1..65536)",
+                 (long long)n_entries);
+    return glqh_launch_e8_repack_table(codebook_packed, n_entries, packed_out, bad_dev, (hipStream_t)stream);
+}
+
 struct e8_stages {
     const void *q[4];
     float scale[4];
@@ -792,4 +801,18 @@ extern "C" int glqh_trellis_pack_states(const int32_t *states, int64_t m, int64_
     GLQH_REQUIRE(glqh_trellis_kernel_supported(m, n), "trellis pack: m %% 32 and n %% 64 must be 0 (m=%lld, n=%lld)",
                  (long long)m, (long long)n);
     return glqh_launch_pack_states(states, m, n, K, packed_out, (hipStream_t)stream);
+}
+
+int glqh_launch_viterbi_acs_step(const float *cost, const void *x_f16, const float *lut, float *cost_out,
+                                 int32_t *prev, int64_t B, int K, hipStream_t stream);
+
+extern "C" int glqh_viterbi_acs_step(const float *cost, const void *x_f16, const float *lut_f32, float *cost_out,
+                                     int32_t *prev_out, int64_t B, int K, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(cost && x_f16 && lut_f32 && cost_out && prev_out, "viterbi step: null pointer");
+    GLQH_REQUIRE(cost != cost_out, "viterbi step: cost_out must not alias cost");
+    GLQH_REQUIRE(K >= 1 && K <= 4, "viterbi step supports K (bits/weight) 1-4, got %d", K);
+    GLQH_REQUIRE(B >= 0 && B <= 65535, "viterbi step: %lld sequences (0..65535 per call)", (long long)B);
+    if (B == 0) return 0;
+    return glqh_launch_viterbi_acs_step(cost, x_f16, lut_f32, cost_out, prev_out, B, K, (hipStream_t)stream);
 }

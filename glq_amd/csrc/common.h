@@ -14,6 +14,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 #define GLQH_WAVE 64
 #define GLQH_MAX_GROUP GLQH_MAX_SHARDS      // layers per grouped launch
@@ -140,6 +141,8 @@ int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, in
 int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B);
 int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, int32_t *bad,
                               hipStream_t stream);
+int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t *out, int32_t *bad,
+                                hipStream_t stream);
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream);

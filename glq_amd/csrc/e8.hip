@@ -41,6 +41,26 @@ e8_pack_table_kernel(const f16 *__restrict__ cb, int n_entries, uint32_t *__rest
     if (!ok) atomicAdd(bad, 1);
 }
 
+// Words in the reference's own packing (nibble c = code of column c,
+// glq/codebook.py:102-115, the `codebook_packed` buffer) -> the interleaved order above.
+__global__ void __launch_bounds__(256)
+e8_repack_table_kernel(const uint32_t *__restrict__ in, int n_entries, uint32_t *__restrict__ out,
+                       int32_t *__restrict__ bad) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_entries) return;
+    const uint32_t w = in[i];
+    uint32_t word = 0;
+    bool ok = true;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const uint32_t code = (w >> (4 * c)) & 15u;
+        ok = ok && code <= 12u;
+        word |= code << (4 * ((c >> 1) + 4 * (c & 1)));
+    }
+    out[i] = word;
+    if (!ok) atomicAdd(bad, 1);
+}
+
 __device__ __forceinline__ f16x2 e8_pair(uint32_t word, int p) {
     uint32_t u = ((word >> (4 * p)) & 0x000F000Fu) | 0x60006000u;
     f16x2 v = __builtin_bit_cast(f16x2, u);
@@ -294,6 +314,14 @@ int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, 
     hipLaunchKernelGGL(e8_pack_table_kernel, dim3((unsigned)((n_entries + 255) / 256)), dim3(256), 0,
                        stream, (const f16 *)cb, (int)n_entries, out, bad);
     GLQH_LAUNCH_CHECK("e8 pack table launch");
+    return 0;
+}
+
+int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t *out, int32_t *bad,
+                                hipStream_t stream) {
+    hipLaunchKernelGGL(e8_repack_table_kernel, dim3((unsigned)((n_entries + 255) / 256)), dim3(256), 0,
+                       stream, in, (int)n_entries, out, bad);
+    GLQH_LAUNCH_CHECK("e8 repack table launch");
     return 0;
 }
 

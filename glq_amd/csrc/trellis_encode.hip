@@ -173,6 +173,71 @@ pack_states_kernel(const int32_t *__restrict__ states, int m, int n, int K, uint
     for (int b = 0; b < K; ++b) dst[b] = (uint8_t)(chunk >> (8 * b));
 }
 
+// One add-compare-select step over cost rows that live in memory, for callers that drive the
+// search step by step (bitshift_codebook.update, glq/trellis.py:230-251; its one-kernel form
+// _viterbi_acs_step, glq/trellis_step_kernel.py:30-84).  V = 1, 2^16 states, NK = 2^K
+// candidates: group j takes the minimum of cost[b, k*G + j] over ascending k (strict <, a NaN
+// displaces a number and is never displaced), stores the predecessor j + (k << (16-K)) and
+// the NK new costs (lut[s] - x[b])^2 + best of states s = j*NK .. j*NK + NK-1.  One thread per
+// group: its loads are coalesced across the wave for every k, its stores are NK consecutive
+// floats.  Streams 2 * B * 2^16 floats; bound by HBM.
+template <int K>
+__global__ void __launch_bounds__(256)
+viterbi_acs_step_kernel(const float *__restrict__ cost, const f16 *__restrict__ x,
+                        const float *__restrict__ lut, float *__restrict__ cost_out,
+                        int32_t *__restrict__ prev) {
+    constexpr int G = 1 << (16 - K);
+    constexpr int NK = 1 << K;
+    const int j = blockIdx.x * 256 + threadIdx.x;             // G is a multiple of 256
+    const int b = blockIdx.y;
+    const float *row = cost + (int64_t)b * 65536;
+    float v[NK];
+#pragma unroll
+    for (int k = 0; k < NK; ++k) v[k] = row[k * G + j];
+    float best = __builtin_inff();
+    int bestk = 0;
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+        const bool take = (v[k] < best) || ((v[k] != v[k]) && (best == best));
+        best = take ? v[k] : best;
+        bestk = take ? k : bestk;
+    }
+    prev[(int64_t)b * G + j] = j + (bestk << (16 - K));
+    const float xb = (float)x[b];
+    float *o = cost_out + (int64_t)b * 65536 + (int64_t)j * NK;
+    const float *l = lut + (int64_t)j * NK;
+    if constexpr (NK >= 4) {
+#pragma unroll
+        for (int r = 0; r < NK; r += 4) {
+            const f32x4 lv = *(const f32x4 *)(l + r);
+            f32x4 e;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float d = lv[c] - xb;
+                e[c] = d * d + best;                          // contraction is off in this file
+            }
+            *(f32x4 *)(o + r) = e;
+        }
+    } else {
+        const f32x2 lv = *(const f32x2 *)l;
+        f32x2 e;
+        for (int c = 0; c < 2; ++c) {
+            const float d = lv[c] - xb;
+            e[c] = d * d + best;
+        }
+        *(f32x2 *)o = e;
+    }
+}
+
+template <int K>
+int acs_launch(const float *cost, const void *x, const float *lut, float *cost_out, int32_t *prev, int64_t B,
+               hipStream_t stream) {
+    hipLaunchKernelGGL(viterbi_acs_step_kernel<K>, dim3((1u << (16 - K)) / 256, (unsigned)B), dim3(256), 0, stream,
+                       cost, (const f16 *)x, lut, cost_out, prev);
+    GLQH_LAUNCH_CHECK("viterbi step launch");
+    return 0;
+}
+
 template <int K>
 int vt_launch(const float *tiles, int64_t n_tiles, uint8_t *scratch, int grid, int32_t *states, float *hat,
               hipStream_t stream) {
@@ -226,4 +291,15 @@ int glqh_launch_pack_states(const int32_t *states, int64_t m, int64_t n, int K, 
                        (int)m, (int)n, K, (uint8_t *)packed);
     GLQH_LAUNCH_CHECK("pack states launch");
     return 0;
+}
+
+int glqh_launch_viterbi_acs_step(const float *cost, const void *x_f16, const float *lut, float *cost_out,
+                                 int32_t *prev, int64_t B, int K, hipStream_t stream) {
+    switch (K) {
+    case 1: return acs_launch<1>(cost, x_f16, lut, cost_out, prev, B, stream);
+    case 2: return acs_launch<2>(cost, x_f16, lut, cost_out, prev, B, stream);
+    case 3: return acs_launch<3>(cost, x_f16, lut, cost_out, prev, B, stream);
+    case 4: return acs_launch<4>(cost, x_f16, lut, cost_out, prev, B, stream);
+    }
+    return glqh_fail("viterbi step supports K (bits/weight) 1-4, got %d", K);
 }

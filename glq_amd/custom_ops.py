@@ -27,10 +27,21 @@ SCHEMAS = {
                       "Tensor codebook_abs, "
                       "Tensor qidxs3, Tensor codebook3, float inv_resid_scale2, "
                       "Tensor qidxs4, Tensor codebook4, float inv_resid_scale3) -> Tensor",
+    "dequant_matvec_packed": "dequant_matvec_packed(Tensor x, Tensor qidxs, Tensor codebook_packed, "
+                             "float wscale) -> Tensor",
+    "dequant_matmul_packed": "dequant_matmul_packed(Tensor x, Tensor qidxs, Tensor codebook_packed, "
+                             "float wscale) -> Tensor",
     "input_rht": "input_rht(Tensor x, Tensor sv, Tensor(a!) out, int in_features, "
                  "int stride_x, float rsqrt_n, int n_pad, int log_n) -> ()",
     "output_rht": "output_rht(Tensor y_rht, Tensor su, Tensor(a!) out, int out_features, "
                   "int m_pad, int log_m, float rsqrt_m) -> ()",
+    # Same schemas under the names the reference gives its transforms of more than 16384
+    # points (glq_vllm/custom_ops.py:132-148, callers glq_vllm/linear_method.py:473, 518);
+    # here one set of kernels serves every size.
+    "input_rht_triton": "input_rht_triton(Tensor x, Tensor sv, Tensor(a!) out, int in_features, "
+                        "int stride_x, float rsqrt_n, int n_pad, int log_n) -> ()",
+    "output_rht_triton": "output_rht_triton(Tensor y_rht, Tensor su, Tensor(a!) out, "
+                         "int out_features, int m_pad, int log_m, float rsqrt_m) -> ()",
     "fused_linear": "fused_linear(Tensor x, Tensor sv, Tensor su, "
                     "Tensor qidxs, Tensor codebook, float wscale, "
                     "int in_features, int out_features, "
@@ -93,6 +104,14 @@ def _dequant_matmul_fake(x, qidxs, codebook, wscale, qidxs2, codebook2, inv_resi
     return x.new_empty((x.shape[0], qidxs.shape[0]), dtype=torch.float32)
 
 
+def _dequant_matvec_packed_fake(x, qidxs, codebook_packed, wscale):
+    return x.new_empty((qidxs.shape[0],), dtype=torch.float32)
+
+
+def _dequant_matmul_packed_fake(x, qidxs, codebook_packed, wscale):
+    return x.new_empty((x.shape[0], qidxs.shape[0]), dtype=torch.float32)
+
+
 def _none_fake(*args):
     return None
 
@@ -130,7 +149,11 @@ def _embedding_dequant_fake(input_ids, qidxs, sv, wscale, codebook, qidxs2, inv_
 FAKES = {
     "dequant_matvec": _dequant_matvec_fake,
     "dequant_matmul": _dequant_matmul_fake,
+    "dequant_matvec_packed": _dequant_matvec_packed_fake,
+    "dequant_matmul_packed": _dequant_matmul_packed_fake,
     "input_rht": _none_fake,
+    "input_rht_triton": _none_fake,
+    "output_rht_triton": _none_fake,
     "output_rht": _none_fake,
     "fused_linear": _fused_linear_fake,
     "fused_linear_block_diag": _fused_linear_block_diag_fake,
@@ -161,7 +184,11 @@ def _impls():
     return {
         "dequant_matvec": ext.glq_dequant_matvec_cuda,
         "dequant_matmul": ext.glq_dequant_matmul_cuda,
+        "dequant_matvec_packed": ext.glq_dequant_matvec_packed_cuda,
+        "dequant_matmul_packed": ext.glq_dequant_matmul_packed_cuda,
         "input_rht": ext.glq_input_rht_cuda,
+        "input_rht_triton": ext.glq_input_rht_cuda,
+        "output_rht_triton": ext.glq_output_rht_cuda,
         "output_rht": ext.glq_output_rht_cuda,
         "fused_linear": fused_linear,
         "fused_linear_block_diag": fused_linear_block_diag,

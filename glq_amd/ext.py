@@ -541,21 +541,16 @@ def _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3):
     return W
 
 
-def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=None,
-                            inv_resid_scale=0.0, codebook_abs=None, qidxs3=None, codebook3=None,
-                            inv_resid_scale2=0.0, qidxs4=None, codebook4=None, inv_resid_scale3=0.0):
-    """(B, N) fp16 RHT-domain activations -> (B, M) fp32."""
+def _e8_matmul_tables(x, qidxs, t1, q2, t2, n2, q3, q4, wscale, inv_rs, inv_rs2, inv_rs3):
+    """(B, N) fp16 x against packed tables -> (B, M) fp32."""
     lib = _lib.load()
     _chk(x, "x", torch.float16)
-    t1, q2, t2, n2, q3, q4 = _e8_args(qidxs, codebook, qidxs2, codebook2, inv_resid_scale, qidxs3,
-                                      inv_resid_scale2, qidxs4, inv_resid_scale3)
     B = x.shape[0]
     M, nblk = qidxs.shape
     if x.shape[1] != nblk * 8:
         raise RuntimeError(f"x has {x.shape[1]} columns, qidxs implies {nblk * 8}")
     if B > E8_BATCH_MAX:
-        W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_resid_scale, inv_resid_scale2,
-                             inv_resid_scale3)
+        W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
         return torch.mm(x, W.t(), out_dtype=torch.float32).mul_(float(wscale))
     out = torch.empty((B, M), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
@@ -563,9 +558,19 @@ def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=N
         ws = _ws(nb, x.device)
         check(lib.glqh_e8_dequant_matmul(
             _p(x), B, _p(qidxs), _p(q2), _p(q3), _p(q4), _p(t1), _p(t2), n2, float(wscale),
-            float(inv_resid_scale), float(inv_resid_scale2), float(inv_resid_scale3), M, nblk * 8,
+            float(inv_rs), float(inv_rs2), float(inv_rs3), M, nblk * 8,
             _p(out), _p(ws), ws.numel(), _stream()))
     return out
+
+
+def glq_dequant_matmul_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=None,
+                            inv_resid_scale=0.0, codebook_abs=None, qidxs3=None, codebook3=None,
+                            inv_resid_scale2=0.0, qidxs4=None, codebook4=None, inv_resid_scale3=0.0):
+    """(B, N) fp16 RHT-domain activations -> (B, M) fp32."""
+    t1, q2, t2, n2, q3, q4 = _e8_args(qidxs, codebook, qidxs2, codebook2, inv_resid_scale, qidxs3,
+                                      inv_resid_scale2, qidxs4, inv_resid_scale3)
+    return _e8_matmul_tables(x, qidxs, t1, q2, t2, n2, q3, q4, wscale, inv_resid_scale,
+                             inv_resid_scale2, inv_resid_scale3)
 
 
 def glq_dequant_matvec_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=None,
@@ -573,6 +578,49 @@ def glq_dequant_matvec_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=N
     """(N,) fp16 -> (M,) fp32."""
     return glq_dequant_matmul_cuda(x.reshape(1, -1), qidxs, codebook, wscale, qidxs2, codebook2,
                                    inv_resid_scale).reshape(-1)
+
+
+_REPACKED = {}
+
+
+def _repacked_table(codebook_packed):
+    """The reference's `codebook_packed` (65536 int32, nibble c = column c,
+    glq/codebook.py:102-115) in the kernels' nibble order, converted once per tensor."""
+    _chk(codebook_packed, "codebook_packed", torch.int32)
+    if codebook_packed.dim() != 1 or codebook_packed.shape[0] != 65536:
+        raise RuntimeError("codebook_packed must hold 65536 int32 words, got "
+                           f"{tuple(codebook_packed.shape)}")
+    key = (codebook_packed.data_ptr(), codebook_packed._version, str(codebook_packed.device))
+    hit = _REPACKED.get(key)
+    if hit is not None and hit[0]() is codebook_packed:
+        return hit[1]
+    lib = _lib.load()
+    out = torch.empty_like(codebook_packed)
+    bad = torch.zeros(1, dtype=torch.int32, device=codebook_packed.device)
+    with torch.cuda.device(codebook_packed.device):
+        check(lib.glqh_e8_repack_table(_p(codebook_packed), 65536, _p(out), _p(bad), _stream()))
+    nbad = int(bad.item())
+    if nbad:
+        raise RuntimeError(f"codebook_packed has {nbad} words with a code above 12; only E8 shell "
+                           "tables are supported")
+    if len(_REPACKED) > 64:
+        for k in [k for k, v in _REPACKED.items() if v[0]() is None]:
+            del _REPACKED[k]
+    _REPACKED[key] = (weakref.ref(codebook_packed), out)
+    return out
+
+
+def glq_dequant_matmul_packed_cuda(x, qidxs, codebook_packed, wscale):
+    """Single-stage (B, N) fp16 -> (B, M) fp32 against the 4-bit packed table
+    (glq/csrc/glq_bindings.cpp:45-50; caller glq/inference_kernel.py:1047-1054)."""
+    _chk(qidxs, "qidxs", torch.int16)
+    t1 = _repacked_table(codebook_packed)
+    return _e8_matmul_tables(x, qidxs, t1, None, None, 0, None, None, wscale, 0.0, 0.0, 0.0)
+
+
+def glq_dequant_matvec_packed_cuda(x, qidxs, codebook_packed, wscale):
+    """Single-stage (N,) fp16 -> (M,) fp32 (glq/csrc/glq_bindings.cpp:38-43)."""
+    return glq_dequant_matmul_packed_cuda(x.reshape(1, -1), qidxs, codebook_packed, wscale).reshape(-1)
 
 
 def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_pad, m_pad,
@@ -667,6 +715,31 @@ def trellis_quantize_tiles(tiles, K):
             check(lib.glqh_trellis_quantize_tiles(_p(x), B, int(K), _p(states), _p(hat), _p(ws), ws.numel(),
                                                   _stream()))
     return hat, states
+
+
+def viterbi_acs_step(cost, x, lut, K, prev_out, cost_out=None):
+    """One add-compare-select step (bitshift_codebook.update, glq/trellis.py:230-251): cost
+    (B, 65536) fp32, x (B) fp16 (the step's inputs), lut (65536) fp32 -> new cost; the int32
+    predecessors go to prev_out (B, 2^(16-K))."""
+    lib = _lib.load()
+    _chk(cost, "cost", torch.float32)
+    _chk(x, "x", torch.float16)
+    _chk(lut, "lut", torch.float32)
+    _chk(prev_out, "prev_out", torch.int32)
+    B = cost.shape[0]
+    if cost.dim() != 2 or cost.shape[1] != 65536 or x.numel() != B or lut.numel() != 65536:
+        raise RuntimeError(f"viterbi step: cost {tuple(cost.shape)}, x {tuple(x.shape)}, lut "
+                           f"{tuple(lut.shape)} do not describe B sequences over 65536 states")
+    if tuple(prev_out.shape) != (B, 1 << (16 - int(K))):
+        raise RuntimeError(f"viterbi step: prev_out {tuple(prev_out.shape)} != (B, 2^(16-K))")
+    if cost_out is None:
+        cost_out = torch.empty_like(cost)
+    else:
+        _chk(cost_out, "cost_out", torch.float32)
+    with torch.cuda.device(cost.device):
+        check(lib.glqh_viterbi_acs_step(_p(cost), _p(x), _p(lut), _p(cost_out), _p(prev_out), B, int(K),
+                                        _stream()))
+    return cost_out
 
 
 def _step_permutation(device):

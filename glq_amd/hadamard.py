@@ -54,3 +54,48 @@ def pack_shard_meta(shard_blocks) -> torch.Tensor:
             rows.append([off, bs, int(math.log2(bs)), w])
             off += bs
     return torch.tensor(rows, dtype=torch.int32, device="cpu").reshape(-1, 4)
+
+
+# ---- transforms under the reference's names (glq/hadamard.py:77-131, 166-178) ----------
+_block_decompose = block_decompose
+_ONES = {}
+
+
+def _ones(n, device):
+    key = (n, str(device))
+    t = _ONES.get(key)
+    if t is None:
+        t = _ONES[key] = torch.ones(n, dtype=torch.float16, device=device)
+    return t
+
+
+def _fht_rows(x: torch.Tensor, block_sizes) -> torch.Tensor:
+    """Normalised Walsh-Hadamard transform of every block of the last dim, computed in fp32
+    by the output-transform kernel with unit signs; the result has x's dtype and shape."""
+    if not x.is_cuda:
+        raise RuntimeError("the Hadamard transforms are GPU only here; there is no CPU fallback")
+    from . import ext
+    n = x.shape[-1]
+    rows = x.reshape(-1, n).to(torch.float32).contiguous()
+    out = torch.empty_like(rows)
+    blocks = [int(b) for b in block_sizes]
+    if rows.shape[0]:
+        meta = pack_block_meta(blocks).to(x.device) if len(blocks) > 1 else None
+        ext.glq_output_rht_blockdiag_cuda(rows, _ones(n, x.device), out, n, n,
+                                          torch.tensor(blocks, dtype=torch.int64), meta)
+    return out.to(x.dtype).reshape(x.shape)
+
+
+def fast_hadamard_transform(x: torch.Tensor) -> torch.Tensor:
+    """H_n x / sqrt(n) along the last dim, n a power of two (glq/hadamard.py:77-131)."""
+    n = x.shape[-1]
+    assert n > 0 and (n & (n - 1)) == 0, f"Last dim {n} must be power of 2"
+    return _fht_rows(x, [n])
+
+
+def block_diagonal_fht(x: torch.Tensor, block_sizes) -> torch.Tensor:
+    """Independent transforms of consecutive power-of-two blocks of the last dim, written
+    back into x, which is also returned (glq/hadamard.py:166-178)."""
+    assert sum(int(b) for b in block_sizes) == x.shape[-1], (list(block_sizes), x.shape[-1])
+    x.copy_(_fht_rows(x, block_sizes))
+    return x

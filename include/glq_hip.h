@@ -182,11 +182,20 @@ int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_
 
 /* ---- E8 shell codebook ---------------------------------------------------- */
 
-/* (n_entries, 8) fp16 table -> n_entries uint32, nibble i = round(2 v_i) + 6
- * (glq/codebook.py:102-115).  *ok_dev (device int32) is set to 0 if any coordinate is
- * outside {-3, -2.5, ..., 3}; the packed table must then not be used. */
+/* (n_entries, 8) fp16 table -> n_entries uint32 of eight 4-bit codes round(2 v) + 6, the
+ * codes of glq/codebook.py:102-115 in the kernels' own nibble order (nibble p = column 2p,
+ * nibble p + 4 = column 2p + 1).  *bad_dev (device int32, zeroed by the caller) counts the
+ * rows with a coordinate outside {-3, -2.5, ..., 3}; if it is nonzero afterwards the packed
+ * table must not be used. */
 int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, uint32_t *packed_out,
-                       int32_t *ok_dev, void *stream);
+                       int32_t *bad_dev, void *stream);
+
+/* The reference's `codebook_packed` buffer (n_entries int32, nibble c = code of column c,
+ * glq/codebook.py:102-115, consumed by glq_dequant_matvec_packed_cuda /
+ * glq_dequant_matmul_packed_cuda, glq/csrc/glq_bindings.cpp:38-50) -> the kernels' nibble
+ * order.  *bad_dev counts words holding a code above 12. */
+int glqh_e8_repack_table(const uint32_t *codebook_packed, int64_t n_entries, uint32_t *packed_out,
+                         int32_t *bad_dev, void *stream);
 
 size_t glqh_e8_matmul_workspace_bytes(int64_t m_pad, int64_t n_pad, int64_t B);
 
@@ -266,6 +275,17 @@ size_t glqh_trellis_quantize_workspace_bytes(int K, int64_t n_tiles);
  * add-compare-select step (glq/trellis_step_kernel.py:30-109).  K = 1..4. */
 int glqh_trellis_quantize_tiles(const float *tiles, int64_t n_tiles, int K, int32_t *states_out,
                                 float *hat_out, void *ws, size_t ws_bytes, void *stream);
+
+/* One add-compare-select step of that search on cost rows in memory, for callers that
+ * drive the search step by step: cost (B, 65536) fp32 -> cost_out (B, 65536) fp32 and
+ * prev_out (B, 2^(16-K)) int32, with x (B) fp16 the step's inputs and lut (65536) fp32 the
+ * state values.  prev_out[b, j] = j + (k* << (16-K)), k* = first minimum over ascending k of
+ * cost[b, k*2^(16-K) + j] (a NaN displaces a number); cost_out[b, j*2^K + r] =
+ * (lut[j*2^K + r] - x[b])^2 + that minimum, separate subtract, multiply and add.
+ * bitshift_codebook.update (glq/trellis.py:230-251) = fused_update
+ * (glq/trellis_step_kernel.py:30-109) at V = 1, L = 16.  cost_out must not alias cost. */
+int glqh_viterbi_acs_step(const float *cost, const void *x_f16, const float *lut_f32, float *cost_out,
+                          int32_t *prev_out, int64_t B, int K, void *stream);
 
 /* Trellis states of an (m, n) layer (tiles in row-major tile order, 256 steps each, int32)
  * -> packed ((m/16)(n/16), 16K) int16 in the kernel layout, K = 1..4.

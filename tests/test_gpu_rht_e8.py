@@ -104,6 +104,65 @@ def test_e8_dequant_matmul_matches_oracle(ext, m, n, stages):
         assert torch.equal(gv, out[1])
 
 
+@pytest.mark.parametrize("m,n,B", [(96, 160, 1), (960, 960, 8), (2048, 2048, 5), (2048, 2048, 40)])
+def test_e8_packed_table_variants(ext, m, n, B):
+    """The single-stage entries that take the reference's 4-bit `codebook_packed` buffer
+    (glq/inference_kernel.py:1047-1054) give what the fp16-table entries give, bit for bit,
+    and match the oracle; a word with a code above 12 is refused."""
+    say("e8 packed table", m, n, B)
+    rng = np.random.default_rng(m + B)
+    q = _rand_idx(rng, m, n // 8)
+    q[0, 0], q[0, 1] = 0, -1
+    x = (rng.standard_normal((B, n)) * 0.5).astype(np.float16)
+    cbp = t(O.e8_nibbles().view(np.int32))             # == the reference's codebook_packed
+    out = ext.glq_dequant_matmul_packed_cuda(t(x), t(q), cbp, 0.021)
+    ref = x.astype(np.float32) @ O.e8_dequant(q).T * np.float32(0.021)
+    assert out.shape == (B, m) and out.dtype == torch.float32
+    assert rel(out, ref) < 1e-3, rel(out, ref)
+    assert torch.equal(out, ext.glq_dequant_matmul_cuda(t(x), t(q), e8_table_f16(), 0.021))
+    gv = ext.glq_dequant_matvec_packed_cuda(t(x[0]), t(q), cbp, 0.021)
+    assert gv.shape == (m,) and torch.equal(gv, ext.glq_dequant_matvec_cuda(t(x[0]), t(q), e8_table_f16(), 0.021))
+    from glq_amd import custom_ops
+    custom_ops.register()
+    assert torch.equal(torch.ops.glq.dequant_matmul_packed(t(x), t(q), cbp, 0.021), out)
+    assert torch.equal(torch.ops.glq.dequant_matvec_packed(t(x[0]), t(q), cbp, 0.021), gv)
+    bad = cbp.clone()
+    bad[7] = 0x0000000D
+    with pytest.raises(RuntimeError, match="code above 12"):
+        ext.glq_dequant_matmul_packed_cuda(t(x), t(q), bad, 0.021)
+    with pytest.raises(RuntimeError, match="65536"):
+        ext.glq_dequant_matmul_packed_cuda(t(x), t(q), cbp[:256].contiguous(), 0.021)
+
+
+def test_large_transform_op_names(ext):
+    """`input_rht_triton` / `output_rht_triton` are the names the vLLM call sites use above
+    16384 points (glq_vllm/linear_method.py:470-473, 506-518); same kernels, same results."""
+    from glq_amd import custom_ops
+    custom_ops.register()
+    n, feat, B = 32768, 30000, 2
+    say("large transform op names", n)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((B, feat)).astype(np.float16)
+    sgn = (rng.integers(0, 2, n) * 2 - 1).astype(np.float16)
+    a = torch.empty(B, n, dtype=torch.float32, device=DEV)
+    b = torch.empty_like(a)
+    r = float(1.0 / np.sqrt(n))
+    torch.ops.glq.input_rht(t(x), t(sgn), a, feat, feat, r, n, 15)
+    torch.ops.glq.input_rht_triton(t(x), t(sgn), b, feat, feat, r, n, 15)
+    assert torch.equal(a, b)
+    xp = np.zeros((B, n), np.float32)
+    xp[:, :feat] = x.astype(np.float32)
+    ref = O.fht(xp * sgn.astype(np.float32)[None, :])
+    assert rel(a, ref) < 1e-5, rel(a, ref)
+    ya = torch.empty(B, feat, dtype=torch.float16, device=DEV)
+    yb = torch.empty_like(ya)
+    torch.ops.glq.output_rht(a, t(sgn), ya, feat, n, 15, r)
+    torch.ops.glq.output_rht_triton(a, t(sgn), yb, feat, n, 15, r)
+    assert torch.equal(ya, yb)
+    back = (O.fht(ref) * sgn.astype(np.float32)[None, :])[:, :feat]
+    assert rel(ya, back) < 2e-3, rel(ya, back)
+
+
 @pytest.mark.parametrize("m,n,B,stages", [(2048, 2048, 1, 1), (2048, 2048, 3, 2), (2100, 2048, 16, 2),
                                           (1024, 4160, 1, 4), (4096, 1024, 9, 3), (512, 8192, 4, 2),
                                           (2048, 2048, 40, 2), (1024, 4160, 33, 4), (2100, 2048, 17, 1)])

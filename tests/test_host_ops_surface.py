@@ -50,6 +50,13 @@ def test_fakes_on_meta_tensors():
     assert y.shape == (B, m) and y.dtype == torch.float16
     y = torch.ops.glq.dequant_matmul(x, q, cb, 0.02, e, ef, 0.0, ef, e, ef, 0.0, e, ef, 0.0)
     assert y.shape == (B, m) and y.dtype == torch.float32
+    cbp = mt(65536, dt=torch.int32)
+    y = torch.ops.glq.dequant_matmul_packed(x, q, cbp, 0.02)
+    assert y.shape == (B, m) and y.dtype == torch.float32
+    y = torch.ops.glq.dequant_matvec_packed(mt(n), q, cbp, 0.02)
+    assert y.shape == (m,) and y.dtype == torch.float32
+    assert torch.ops.glq.input_rht_triton(x, mt(n), mt(B, n, dt=torch.float32), n, n, 0.1, n, 7) is None
+    assert torch.ops.glq.output_rht_triton(mt(B, m, dt=torch.float32), mt(m), mt(B, m), m, m, 6, 0.1) is None
     yr = mt(B, 2 * m, dt=torch.float32)
     assert torch.ops.glq.fused_linear_trellis_3inst_yrht(x, mt(n), packed, i64, i32, 0.02, n, n, m,
                                                          yr, m) is None

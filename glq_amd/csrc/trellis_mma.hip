@@ -740,18 +740,35 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
     return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
-// Prefill plan: split K only while the grid would leave most CUs idle.
+// Prefill plan: K is split over the grid when the 256-row x 128-token tiles alone leave CUs idle.
+// The split is chosen by a small cost model fitted to this kernel on the 4096 <-> 14336 shapes:
+// a workgroup takes 6 us + 1.0 us per k-pair when it has its CU to itself and 9 us + 1.53 us per
+// k-pair when two share one; a launch runs in rounds of two workgroups per CU, and a last round
+// of at most one workgroup per CU runs at the faster rate; every partial-sum slot costs its
+// write and the consumer's read, about 0.35 us per MB.  (A split that spills a few workgroups into a second
+// round, or one more slot than the grid needs, costs more than it gains.)
 int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out) {
     const int64_t nkp = k / 32;
-    const int64_t wgs = ((m + 255) / 256) * ((M + 127) / 128);
-    const int64_t target = (int64_t)glqh_device_cus() * 2;
-    int64_t ks = (target + wgs - 1) / wgs;
-    if (ks > 8) ks = 8;
-    if (ks < 1) ks = 1;
-    int64_t S = (nkp + ks - 1) / ks;
-    S = (S + PF_CH - 1) / PF_CH * PF_CH;
-    *S_out = (int)S;
-    *ksplit_out = (int)((nkp + S - 1) / S);
+    const int64_t tiles = ((m + 255) / 256) * ((M + 127) / 128);
+    const int64_t cus = glqh_device_cus(), slots = 2 * cus;
+    double best = 0.0;
+    int64_t best_S = (nkp + PF_CH - 1) / PF_CH * PF_CH, best_ks = 1;
+    for (int64_t ks = 1; ks <= 16; ++ks) {
+        int64_t S = (nkp + ks - 1) / ks;
+        S = (S + PF_CH - 1) / PF_CH * PF_CH;
+        const int64_t ksp = (nkp + S - 1) / S;
+        if (ksp != ks && ks > 1) continue;                      // same split as a smaller ks
+        const int64_t W = tiles * ksp, full = W / slots, rem = W % slots;
+        double t = (double)full * (S * 1.53 + 9.0) + (rem == 0 ? 0.0 : rem <= cus ? S * 1.0 + 6.0 : S * 1.53 + 9.0);
+        if (ksp > 1) t += 0.35e-6 * 4.0 * (double)ksp * (double)M * (double)m;
+        if (ks == 1 || t < best) {
+            best = t;
+            best_S = S;
+            best_ks = ksp;
+        }
+    }
+    *S_out = (int)best_S;
+    *ksplit_out = (int)best_ks;
     return 1;
 }
 

@@ -117,7 +117,7 @@ def _graph_time(torch, fn, n_inner, reps=10):
 
 
 def extras(torch, ext, dev):
-    """Side measurements of the other BASELINE configs (bounded, a few seconds): whole-model
+    """Side measurements of the other benchmark configurations (bounded, a few seconds): whole-model
     batch-1 decode tok/s (config 5), large-layer GEMV rates where the kernels are not launch
     bound, and the prefill tiles (config 4 shape)."""
     out = {}

@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full shapes (needs an MI355X): configs[2] (E8 two-stage
+"""The large benchmark configurations at their full shapes (needs an MI355X): configs[2] (E8 two-stage
 4 bpw, 4096 <-> 14336, M = 1, 4, 16) and configs[3] (the same shapes, trellis and E8, M = 256 and
 1024) against the oracle's fp32 CPU path, plus properties that do not need an oracle at these
 sizes: linearity in x, rows of a batch equal to single-token calls, repeated runs bit-identical."""

@@ -21,7 +21,7 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
                                    const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
                                    int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
                                    int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
-                                   int n_blocks, hipStream_t stream);
+                                   int n_blocks, float pscale, hipStream_t stream);
 // K plan of the fused-input GEMV for layers of the given padded heights sharing one input.
 // Returns 0 (not eligible), 1 (32-row workgroups, v_dot2 decode) or 2 (64-row workgroups, MFMA
 // decode: fewer vector-ALU operations per weight and half as many redundant input transforms).
@@ -52,10 +52,12 @@ static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
     else glqh_trellis_mma_plan(m, k, &p.S, &p.ks);
     return p;
 }
+// pscale multiplies the partial sums as they are written (small-batch kernel only): a second
+// stage stored pre-scaled is just more K slots to whoever sums them.
 static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                            int64_t k, float *part, hipStream_t st) {
+                            int64_t k, float *part, hipStream_t st, float pscale = 1.0f) {
     if (p.prefill) return glqh_launch_trellis_prefill(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
-    return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
+    return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, pscale, 0, 0, st);
 }
 static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
                            int64_t k, float scale, float *out, int64_t out_stride, int accum, hipStream_t st) {
@@ -304,13 +306,29 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     float *part1 = (float *)((char *)ws + xb);
     float *part2 = (float *)((char *)ws + xb + pb);
 
-    // Single-stage layers at up to four tokens fold the input transform into the GEMV;
-    // everything else transforms x once into scratch and reads it from every workgroup.
+    // Two stages at up to four tokens with canonical output blocks: the second stage's partial
+    // sums are written already multiplied by inv_resid_scale2, right behind the first stage's
+    // slots, and the finishing kernels of the single-stage path sum all 2*ks slots (the generic
+    // two-part transform takes twice as long: 14.3 against 6.8 us at 4096 x 4096).
+    glqh_meta_args canon_m;
+    const bool canon_out = B <= 4 && glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
+                                                         n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
+                           canon_m.canon == m_pad;
+    const bool merge2 = has_s2 && canon_out && !(y && y_rht_out);
+    const float ps2 = merge2 ? (float)inv_resid_scale2 : 1.0f;
+
+    // Up to four tokens the input transform is folded into the GEMV launch.  A two-stage layer
+    // repeats it in both launches at one token, where that is cheaper than a launch of its own
+    // (2048 x 2048: 14.5 against 17.4 us; at four tokens 23.9 against 18.0, so two to four
+    // tokens transform x once); only the MFMA form takes a pre-scaled second stage, and a 1-bit
+    // second stage has no such kernel.  Everything else transforms x once into scratch and
+    // reads it from every workgroup.
     int ks = 0, fi_steps = 0, fi_mode = 0;
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
     const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
-    if (!has_s2 && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
-        (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0) {
+    if (fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
+        (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0 &&
+        (!has_s2 || (B == 1 && R2 >= 2 && fi_mode == 2 && merge2))) {
         if (n_blocks_n > 1) {
             int64_t sum = 0;
             for (int64_t i = 0; i < n_blocks_n; ++i) {
@@ -323,43 +341,48 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                          (long long)sum, (long long)n_pad);
         }
         GLQH_REQUIRE(in_features >= 1, "fused trellis linear: in_features must be positive");
-        if (fi_mode == 2) {
-            const void *pk[1] = {packed}, *svs[1] = {sv_f16};
-            float *pt[1] = {part1};
-            if (glqh_launch_trellis_mma_fusein(pk, svs, pt, &m_pad, 1, R1, x, x_dtype, x_stride, B, n_pad,
-                                               in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
+        if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
+        for (int stage = 0; stage < (has_s2 ? 2 : 1); ++stage) {
+            const void *pk[1] = {stage ? packed2 : packed}, *svs[1] = {sv_f16};
+            float *pt[1] = {stage ? part2 : part1};
+            const int R = stage ? R2 : R1;
+            if (fi_mode == 2) {
+                if (glqh_launch_trellis_mma_fusein(pk, svs, pt, &m_pad, 1, R, x, x_dtype, x_stride, B, n_pad,
+                                                   in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n,
+                                                   stage ? ps2 : 1.0f, st))
+                    return 1;
+            } else if (glqh_launch_trellis_fusein(pk[0], R, x, x_dtype, x_stride, sv_f16, B, m_pad, n_pad,
+                                                  in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, pt[0], st))
                 return 1;
-        } else if (glqh_launch_trellis_fusein(packed, R1, x, x_dtype, x_stride, sv_f16, B, m_pad, n_pad,
-                                              in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, part1, st))
-            return 1;
+        }
     } else {
         if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
                                   bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
             return 1;
         const tr_plan plan = tr_plain_plan(m_pad, n_pad, B);
         ks = plan.ks;
+        if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
         if (tr_plain_partial(plan, x_rht, B, packed, R1, m_pad, n_pad, part1, st)) return 1;
-        if (has_s2 && tr_plain_partial(plan, x_rht, B, packed2, R2, m_pad, n_pad, part2, st)) return 1;
+        if (has_s2 && tr_plain_partial(plan, x_rht, B, packed2, R2, m_pad, n_pad, part2, st, ps2)) return 1;
     }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);
+    const int ks_all = merge2 ? 2 * ks : ks;
     if (!y) {
         // stop at the RHT-domain product: combine the split-K partials into the caller's rows
-        if (glqh_launch_reduce_splits(part1, ks, B * m_pad, B, m_pad, s1, y_rht_out, y_rht_stride, 0, st)) return 1;
-        if (has_s2 && glqh_launch_reduce_splits(part2, ks, B * m_pad, B, m_pad, s2, y_rht_out, y_rht_stride, 1, st))
+        if (glqh_launch_reduce_splits(part1, ks_all, B * m_pad, B, m_pad, s1, y_rht_out, y_rht_stride, 0, st)) return 1;
+        if (has_s2 && !merge2 &&
+            glqh_launch_reduce_splits(part2, ks, B * m_pad, B, m_pad, s2, y_rht_out, y_rht_stride, 1, st))
             return 1;
         return 0;
     }
-    glqh_meta_args canon_m;
-    if (!has_s2 && !y_rht_out && B <= 4 && glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
-                                                              n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
-        canon_m.canon == m_pad) {
-        // one stage, canonical blocks, a few tokens: the grouped launcher's kernels (a group of one)
+    if ((!has_s2 || merge2) && !y_rht_out && canon_out) {
+        // canonical blocks, a few tokens: the grouped launcher's kernels (a group of one)
         const float *pt[1] = {part1};
         const void *sus[1] = {su_f16};
         void *ys[1] = {y};
         const float sc[1] = {s1};
-        return glqh_launch_output_rht_group(pt, sus, ys, sc, &m_pad, &out_features, 1, y_dtype, y_stride, B, ks, st);
+        return glqh_launch_output_rht_group(pt, sus, ys, sc, &m_pad, &out_features, 1, y_dtype, y_stride, B, ks_all, st);
     }
     glqh_ysrc src = {};
     src.nparts = has_s2 ? 2 : 1;
@@ -462,7 +485,7 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
     c->R = R; c->ks = ks; c->fi_mode = fi_mode;
     if (fi_mode == 2)
         return glqh_launch_trellis_mma_fusein(packed, sv, c->parts, c->m_pads, n_shards, R, x, x_dtype, x_stride, B,
-                                              n_pad, in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st);
+                                              n_pad, in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, 1.0f, st);
     return glqh_launch_trellis_fusein_group(packed, sv, c->parts, c->m_pads, n_shards, R, x, x_dtype, x_stride, B,
                                             n_pad, in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st);
 }

@@ -150,7 +150,7 @@ __device__ __forceinline__ void mma_reduce_store(const mma_acc<NT> acc, float *r
                 float *o = part + (int64_t)tok * out_stride + row;
                 *o = accum ? (*o + scale * v) : scale * v;
             } else {
-                part[((int64_t)slot * B + tok) * m + row] = v;
+                part[((int64_t)slot * B + tok) * m + row] = scale * v;   // 1.0f unless a stage is pre-scaled
             }
         }
     }
@@ -478,7 +478,7 @@ __device__ __forceinline__ void
 tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
                    const f16 *__restrict__ sv, int B, int m, int k, int in_features, int S,
                    const glqh_block_meta *__restrict__ bn_meta, int n_blocks, glqh_meta_args margs,
-                   float *__restrict__ part, u32x4 *lds) {
+                   float *__restrict__ part, float pscale, u32x4 *lds) {
     constexpr int TPS = mma_tps<TP>();
     const int Ls = S << 5;
     uint32_t *xs32 = (uint32_t *)lds;
@@ -603,7 +603,7 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
         cur = nx1;
         nx1 = nx2;
     }
-    mma_reduce_store<TP, 1>(acc, (float *)lds, a, wave, B, m, 0, 64 * blockIdx.x, slot, part, 0, 1.0f, 0, 0);
+    mma_reduce_store<TP, 1>(acc, (float *)lds, a, wave, B, m, 0, 64 * blockIdx.x, slot, part, 0, pscale, 0, 0);
 }
 
 template <int R, typename XT, int TP>
@@ -611,10 +611,10 @@ __global__ void __launch_bounds__(TR_THREADS)
 tr_mma_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
                      const f16 *__restrict__ sv, int B, int m, int k, int in_features, int S,
                      const glqh_block_meta *__restrict__ bn_meta, int n_blocks, glqh_meta_args margs,
-                     float *__restrict__ part) {
+                     float *__restrict__ part, float pscale) {
     extern __shared__ u32x4 xs_lds[];
     tr_mma_fusein_body<R, XT, TP>(packed, x, x_stride, sv, B, m, k, in_features, S, bn_meta, n_blocks, margs,
-                                  part, xs_lds);
+                                  part, pscale, xs_lds);
 }
 
 // Several layers that read the same activations (fused q/k/v, gate/up:
@@ -644,7 +644,7 @@ tr_mma_fusein_group_kernel(tr_fusein_group g, const XT *__restrict__ x, int64_t 
         if (i == z) { packed = g.packed[i]; sv = g.sv[i]; part = g.part[i]; m = g.m[i]; }
     if ((int)blockIdx.x * 64 >= m) return;
     tr_mma_fusein_body<R, XT, TP>(packed, x, x_stride, sv, B, m, k, in_features, S, bn_meta, n_blocks, margs,
-                                  part, xs_lds);
+                                  part, 1.0f, xs_lds);
 }
 
 template <int TP>
@@ -792,7 +792,7 @@ static int pf_set_lds(K kernel) {
 }
 
 // ---- fused-input GEMV (MFMA form): plan and launch -----------------------------------
-// S k-pairs per K slot: a power of two >= 4 chosen so that about four workgroups per CU are
+// S k-pairs per K slot: a power of two >= 8 chosen so that about four workgroups per CU are
 // in flight; the slice 32*S is capped by LDS (8192 columns at one token, 4096 at 2..4).
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out) {
     if (B < 1 || B > 4 || wgs_rows < 1) return 0;
@@ -802,6 +802,11 @@ int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_
     if (ks_target < 1) ks_target = 1;
     const int64_t want = (nkp + ks_target - 1) / ks_target;
     int64_t S = 2 * TR_WAVES;                                   // at least 256 columns per slot
+    // Every workgroup sums the (block / slice) sub-slices of its Hadamard block before it
+    // decodes anything: 256-column slices of a block of 4096 points or more are 16+ terms in
+    // front of two records per wave (4096 x 4096: 17.6 us per linear with them, 11.9 us with
+    // 512-column slices).
+    if (k >= 4096) S = 4 * TR_WAVES;
     while (S < want) S <<= 1;
     const int64_t cap = B == 1 ? FI_MAX_S : FI_MAX_S_TP4;
     if (S > cap) S = cap;
@@ -814,7 +819,7 @@ template <int R, typename XT, int TP>
 static int launch_mma_fusein(const tr_fusein_group &g, int n_layers, int64_t max_m, const void *x,
                              int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S, int ksplit,
                              const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
-                             hipStream_t stream) {
+                             float pscale, hipStream_t stream) {
     glqh_meta_args margs;
     if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
     const glqh_block_meta *meta = n_blocks > 1 ? bn_meta : nullptr;
@@ -824,7 +829,7 @@ static int launch_mma_fusein(const tr_fusein_group &g, int n_layers, int64_t max
         dim3 grid((unsigned)((max_m + 63) / 64), (unsigned)ksplit, 1);
         hipLaunchKernelGGL((tr_mma_fusein_kernel<R, XT, TP>), grid, dim3(TR_THREADS), lds, stream, g.packed[0],
                            (const XT *)x, x_stride, g.sv[0], (int)B, g.m[0], (int)k, (int)in_features, S, meta, nb,
-                           margs, g.part[0]);
+                           margs, g.part[0], pscale);
     } else {
         dim3 grid((unsigned)((max_m + 63) / 64), (unsigned)ksplit, (unsigned)n_layers);
         hipLaunchKernelGGL((tr_mma_fusein_group_kernel<R, XT, TP>), grid, dim3(TR_THREADS), lds, stream, g,
@@ -839,8 +844,9 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
                                    const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
                                    int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
                                    int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
-                                   int n_blocks, hipStream_t stream) {
+                                   int n_blocks, float pscale, hipStream_t stream) {
     GLQH_REQUIRE(n_layers >= 1 && n_layers <= GLQH_MAX_GROUP, "trellis group: 1..%d layers", GLQH_MAX_GROUP);
+    GLQH_REQUIRE(n_layers == 1 || pscale == 1.0f, "trellis group: pre-scaled partial sums are a single-layer option");
     GLQH_REQUIRE(B >= 1 && B <= 4, "fused-input trellis kernel serves 1..4 tokens");
     tr_fusein_group g = {};
     int64_t max_m = 0;
@@ -853,7 +859,7 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
         if (m[j] > max_m) max_m = m[j];
     }
 #define GLQH_FI(RR, XT, TP) launch_mma_fusein<RR, XT, TP>(g, n_layers, max_m, x, x_stride, B, k, in_features, S, \
-                                                          ksplit, bn_meta, blocks_host, n_blocks, stream)
+                                                          ksplit, bn_meta, blocks_host, n_blocks, pscale, stream)
 #define GLQH_FI_R(RR)                                                                   \
     (B == 1 ? (x_dtype == GLQH_F16 ? GLQH_FI(RR, f16, 1) : GLQH_FI(RR, uint16_t, 1))     \
             : (x_dtype == GLQH_F16 ? GLQH_FI(RR, f16, 4) : GLQH_FI(RR, uint16_t, 4)))

@@ -130,6 +130,48 @@ def test_trellis_many_tokens(B, route, monkeypatch):
     assert rel(y[:8], y8.float()) < 5e-3
 
 
+@pytest.mark.parametrize("m,n", [(256, 512), (2048, 2048), (2080, 1152)])
+@pytest.mark.parametrize("K2", [1, 2, 3, 4])
+@pytest.mark.parametrize("B", [1, 3, 6])
+def test_trellis_two_stage_few_tokens(m, n, K2, B):
+    """Two-stage layers at a few tokens: up to four tokens both stages fold the input transform
+    into their launch (small and large layers take the two decode forms; a 1-bit second stage
+    and more tokens take the separate transform).  Against the oracle, against the stages
+    computed one at a time, and through the y_rht entry."""
+    from glq_amd import ext, hadamard as H
+    say("trellis two stages", m, n, K2, B)
+    p1, p2 = O.random_packed(m, n, 4, 1), O.random_packed(m, n, K2, 2)
+    su, sv = O.rht_signs(m, n, 42)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"trellis_packed": p1, "trellis_packed2": p2, "inv_resid_scale2": np.float32(0.3),
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
+           "blocks_m": bm, "blocks_n": bn}
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).to(torch.bfloat16)
+    args = (torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV))
+    y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), t(p2), *args, 0.02, 0.3, n, m, n, m,
+        out_dtype=torch.bfloat16)
+    if m * n <= 1 << 20:
+        ref = O.trellis_linear_forward(x.float().numpy(), art, n, m)
+        assert y.shape == (B, m) and rel(y, ref) < TOL, rel(y, ref)
+    assert torch.equal(y, ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), t(p2), *args, 0.02, 0.3, n, m, n, m,
+        out_dtype=torch.bfloat16))
+    # the same sum from single-stage calls (fp32 out): y1 + 0.3 * y2, linear in the weights
+    y1 = ext.glq_fused_linear_trellis_3inst_cuda(x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), *args, 0.02,
+                                                 n, m, n, m, out_dtype=torch.bfloat16).float()
+    yr = torch.zeros(B, m, dtype=torch.float32, device=DEV)
+    ext.glq_fused_linear_trellis_3inst_yrht_rvq2_cuda(x.to(DEV), t(art["SV"]), t(p1), t(p2), args[0], args[2],
+                                                      0.02, 0.3, n, n, m, yr, 0)
+    yo = torch.empty(B, m, dtype=torch.bfloat16, device=DEV)
+    ext.glq_output_rht_blockdiag_cuda(yr, t(art["SU"]), yo, m, m, args[1], args[3])
+    assert rel(yo, y.float()) < 5e-3, rel(yo, y.float())
+    if K2 >= 2:
+        y2 = ext.glq_fused_linear_trellis_3inst_cuda(x.to(DEV), t(art["SV"]), t(art["SU"]), t(p2), *args, 0.02 * 0.3,
+                                                     n, m, n, m, out_dtype=torch.bfloat16).float()
+        assert rel(y1 + y2, y.float()) < 1e-2, rel(y1 + y2, y.float())
+
+
 def test_e8_dense_route_many_tokens():
     from glq_amd import ext, hadamard as H
     m, n, B = 96, 160, 40

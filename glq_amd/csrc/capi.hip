@@ -326,7 +326,14 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     int ks = 0, fi_steps = 0, fi_mode = 0;
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
     const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
-    if (fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
+    // Where folding pays (whole linear, us, folded vs separate transform): one token 8.6 vs 11.1
+    // at 2048 x 2048, 12.0 vs 15.6 at 4096 x 4096, 13.9 vs 17.0 at 2048 x 11008, but 21.8 vs 21.0 at
+    // 14336 x 4096 and 63 vs 49 at 28672 x 8192 (every workgroup repeats the prologue); the
+    // folded form grows by a quarter per extra token and the separate one hardly at all, so two
+    // tokens fold only single power-of-two blocks (10.8 vs 11.3, 14.7 vs 15.8; 960 x 960: 12.7 vs
+    // 9.4) and three or four tokens never do (2048 x 2048: 13.6 vs 11.5; 8192 x 8192: 38 vs 26).
+    const bool fi_pays = m_pad * n_pad <= ((int64_t)32 << 20) && (B == 1 || (B == 2 && pow2_n));
+    if (fi_pays && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
         (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0 &&
         (!has_s2 || (B == 1 && R2 >= 2 && fi_mode == 2 && merge2))) {
         if (n_blocks_n > 1) {

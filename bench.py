@@ -148,6 +148,31 @@ def extras(torch, ext, dev):
             us = _graph_time(torch, lambda: [ext.trellis_gemv_partials(xh, p, m, n, pb) for p in packs], len(packs))
             out[f"trellis_gemv_16384x16384_B{B}_GBs"] = round(m * n / 2 / us / 1e3, 1)
         del packs, part
+        # 4096 x 4096, one token: the shape of the reference's own GEMV table
+        # (benchmarks/_trellis_rvq_decode.md:41-52), single stage and 4+2 bits, rotating over 36
+        # weight sets (302 MB of 4-bit streams, more than the 256 MB Infinity Cache)
+        from glq_amd import hadamard as H
+        m = n = 4096
+        bn = H.block_decompose(n)
+        bnt, bnm = torch.tensor(bn), H.pack_block_meta(bn).to(dev)
+        sv = torch.ones(n, dtype=torch.float16, device=dev)
+        p4 = [torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
+              for _ in range(36)]
+        p2 = [torch.randint(-32768, 32768, ((m // 16) * (n // 16), 32), device=dev, dtype=torch.int16)
+              for _ in range(36)]
+        xh = torch.randn(1, n, device=dev).to(torch.float16)
+        pb = torch.empty(64 * m, dtype=torch.float32, device=dev)
+        out["trellis_gemv_4096x4096_B1_us"] = round(_graph_time(
+            torch, lambda: [ext.trellis_gemv_partials(xh, p, m, n, pb) for p in p4], len(p4)), 2)
+        xb = xh.to(torch.bfloat16)
+        out["trellis_linear_4096x4096_B1_us"] = round(_graph_time(
+            torch, lambda: [ext.glq_fused_linear_trellis_3inst_cuda(xb, sv, sv, p, bnt, bnt, bnm, bnm, 0.02, n, m, n, m,
+                                                                    out_dtype=torch.bfloat16) for p in p4], len(p4)), 2)
+        out["trellis_linear_4096x4096_6bpw_B1_us"] = round(_graph_time(
+            torch, lambda: [ext.glq_fused_linear_trellis_3inst_rvq2_cuda(xb, sv, sv, a, b, bnt, bnt, bnm, bnm, 0.02, 0.3,
+                                                                         n, m, n, m, out_dtype=torch.bfloat16)
+                            for a, b in zip(p4, p2)], len(p4)), 2)
+        del p4, p2
         m, n, M = 14336, 4096, 4096
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
         xh = torch.randn(M, n, device=dev).to(torch.float16)

@@ -237,7 +237,7 @@ def extras(torch, ext, dev):
     return out
 
 
-CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "e8_gemv_2stage", "decoder")
+CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "decoder")
 
 
 def run_case(torch, ext, dev, name, steps):
@@ -253,8 +253,8 @@ def run_case(torch, ext, dev, name, steps):
         pb = torch.empty(64 * m, dtype=torch.float32, device=dev)
         fn = lambda i: ext.trellis_gemv_partials(xh, packs[i % 4], m, n, pb)
         res["bytes_per_launch"] = m * n // 2
-    elif name == "trellis_prefill_4096":
-        m, n, M = 14336, 4096, 4096
+    elif name in ("trellis_prefill_4096", "trellis_prefill_256"):
+        m, n, M = 14336, 4096, int(name.rsplit("_", 1)[1])
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
         xh = torch.randn(M, n, device=dev).to(torch.float16)
         o = torch.empty(M, m, dtype=torch.float32, device=dev)

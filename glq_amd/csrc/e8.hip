@@ -301,7 +301,7 @@ int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B) {
     const int64_t wgs = (m_pad + E8_ROWS_PER_WG - 1) / E8_ROWS_PER_WG;
     const int64_t target = (int64_t)glqh_device_cus() * 4;
     int64_t ks = (target + wgs - 1) / wgs;
-    int64_t cap = ((n_pad / 8 + 7) / 8) / 8;             // every lane gets at least one chunk
+    int64_t cap = (((n_pad / 8 + 7) / 8) + 7) / 8;       // one chunk per lane at the most slots (a last slot may be ragged)
     if (cap < 1) cap = 1;
     if (ks > cap) ks = cap;
     if (ks > 32) ks = 32;

@@ -77,6 +77,8 @@ SIGNATURES = {
                                         c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_vp]),
     "glqh_attn_decode_bf16": (c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "glqh_silu_mul_bf16": (c_int, [c_vp, c_vp, c_vp, c_i64, c_vp]),
+    "glqh_lm_head_workspace_bytes": (c_sz, []),
+    "glqh_lm_head_argmax_bf16": (c_int, [c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "glqh_trellis_linear_add_rmsnorm_bf16": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_dbl, c_vp, c_vp, c_vp, c_sz, c_vp]),
     "glqh_trellis_qkv_rope_store_bf16": (

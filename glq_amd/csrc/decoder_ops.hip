@@ -637,6 +637,99 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
     attn_core<true>(qs, Kh, Vh, n, knew, vnew, sc, red, part, out + (int64_t)h * D, &first_k);
 }
 
+// Output head of the decode step: logits[r] = <h, E[r, :]> (bf16 x bf16, fp32 sums) over a
+// (vocab, hidden) bf16 table, and the arg-max of the row.  A wave takes rows r, r + W, ...;
+// every lane keeps its 8*HC activations in registers and reads HC 16-byte runs of each row, two
+// rows at a time (2*HC loads in flight per lane).  Streams the table once: bound by HBM.
+// Ties go to the lowest row.  best: [waves] (value, row) pairs for lm_head_argmax_kernel.
+template <int HC>
+__global__ void __launch_bounds__(256)
+lm_head_kernel(const uint16_t *__restrict__ h, const uint16_t *__restrict__ E, float *__restrict__ logits,
+               float *__restrict__ best_val, int *__restrict__ best_row, int vocab) {
+    constexpr int hidden = 512 * HC;
+    const int lane = threadIdx.x & 63;
+    const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int nw = gridDim.x * 4;
+    float x[HC][8];
+#pragma unroll
+    for (int c = 0; c < HC; ++c) {
+        const u32x4 v = *(const u32x4 *)(h + 8 * (lane + 64 * c));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x[c][2 * e] = __builtin_bit_cast(float, v[e] << 16);
+            x[c][2 * e + 1] = __builtin_bit_cast(float, v[e] & 0xFFFF0000u);
+        }
+    }
+    float bv = -__builtin_inff();
+    int br = 0x7FFFFFFF;
+    for (int r0 = wid; r0 < vocab; r0 += 2 * nw) {
+        const int r1 = r0 + nw;
+        const int r1c = r1 < vocab ? r1 : r0;                    // clamped: the loads stay unconditional
+        u32x4 a[HC], b[HC];
+#pragma unroll
+        for (int c = 0; c < HC; ++c) {
+            a[c] = __builtin_nontemporal_load((const u32x4 *)(E + (int64_t)r0 * hidden + 8 * (lane + 64 * c)));
+            b[c] = __builtin_nontemporal_load((const u32x4 *)(E + (int64_t)r1c * hidden + 8 * (lane + 64 * c)));
+        }
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+        for (int c = 0; c < HC; ++c)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                s0 += x[c][2 * e] * __builtin_bit_cast(float, a[c][e] << 16);
+                s0 += x[c][2 * e + 1] * __builtin_bit_cast(float, a[c][e] & 0xFFFF0000u);
+                s1 += x[c][2 * e] * __builtin_bit_cast(float, b[c][e] << 16);
+                s1 += x[c][2 * e + 1] * __builtin_bit_cast(float, b[c][e] & 0xFFFF0000u);
+            }
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            s0 += __shfl_xor(s0, d, GLQH_WAVE);
+            s1 += __shfl_xor(s1, d, GLQH_WAVE);
+        }
+        if (lane == 0) {
+            if (logits) {
+                logits[r0] = s0;
+                if (r1 < vocab) logits[r1] = s1;
+            }
+        }
+        if (s0 > bv) { bv = s0; br = r0; }                       // rows ascend within a wave
+        if (r1 < vocab && s1 > bv) { bv = s1; br = r1; }
+    }
+    if (lane == 0) {
+        best_val[wid] = bv;
+        best_row[wid] = br;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+lm_head_argmax_kernel(const float *__restrict__ best_val, const int *__restrict__ best_row, int n,
+                      int64_t *__restrict__ token) {
+    __shared__ float sv[256];
+    __shared__ int sr[256];
+    float bv = -__builtin_inff();
+    int br = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const float v = best_val[i];
+        const int r = best_row[i];
+        if (v > bv || (v == bv && r < br)) { bv = v; br = r; }
+    }
+    sv[threadIdx.x] = bv;
+    sr[threadIdx.x] = br;
+    __syncthreads();
+    for (int d = 128; d >= 1; d >>= 1) {
+        if ((int)threadIdx.x < d) {
+            const float v = sv[threadIdx.x + d];
+            const int r = sr[threadIdx.x + d];
+            if (v > sv[threadIdx.x] || (v == sv[threadIdx.x] && r < sr[threadIdx.x])) {
+                sv[threadIdx.x] = v;
+                sr[threadIdx.x] = r;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *token = sr[0];
+}
+
 }  // namespace
 
 extern "C" int glqh_rmsnorm_bf16(const void *x, const void *w, void *out, int64_t T, int64_t H, double eps,
@@ -804,5 +897,33 @@ int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3
                        (uint16_t *)out, (int)heads, (int)kv_heads, (int)max_len, apply_rope,
                        1.0f / sqrtf((float)head_dim), log_slice, sc_floats, buf_floats);
     GLQH_LAUNCH_CHECK("out+rope+attention launch");
+    return 0;
+}
+
+static int lm_head_wgs(void) { return glqh_device_cus() * 4; }
+
+extern "C" size_t glqh_lm_head_workspace_bytes(void) { return (size_t)lm_head_wgs() * 4 * 8; }
+
+extern "C" int glqh_lm_head_argmax_bf16(const void *h, const void *table, int64_t vocab, int64_t hidden,
+                                        float *logits_out, int64_t *token_out, void *ws, size_t ws_bytes,
+                                        void *stream) {
+    GLQH_REQUIRE(h && table && token_out && ws, "lm_head: null pointer");
+    GLQH_REQUIRE(vocab >= 1 && vocab < ((int64_t)1 << 31), "lm_head: vocab %lld out of range", (long long)vocab);
+    GLQH_REQUIRE(hidden == 2048 || hidden == 4096, "lm_head: hidden size %lld (2048 or 4096)", (long long)hidden);
+    GLQH_REQUIRE((((uintptr_t)h | (uintptr_t)table) & 15) == 0, "lm_head: pointers must be 16-byte aligned");
+    const int wgs = lm_head_wgs(), nw = wgs * 4;
+    GLQH_REQUIRE(ws_bytes >= (size_t)nw * 8, "lm_head: workspace of %zu bytes needed, got %zu", (size_t)nw * 8, ws_bytes);
+    float *bv = (float *)ws;
+    int *br = (int *)ws + nw;
+    hipStream_t st = (hipStream_t)stream;
+    if (hidden == 2048)
+        hipLaunchKernelGGL(lm_head_kernel<4>, dim3((unsigned)wgs), dim3(256), 0, st, (const uint16_t *)h,
+                           (const uint16_t *)table, logits_out, bv, br, (int)vocab);
+    else
+        hipLaunchKernelGGL(lm_head_kernel<8>, dim3((unsigned)wgs), dim3(256), 0, st, (const uint16_t *)h,
+                           (const uint16_t *)table, logits_out, bv, br, (int)vocab);
+    GLQH_LAUNCH_CHECK("lm_head launch");
+    hipLaunchKernelGGL(lm_head_argmax_kernel, dim3(1), dim3(256), 0, st, bv, br, nw, token_out);
+    GLQH_LAUNCH_CHECK("lm_head argmax launch");
     return 0;
 }

@@ -195,6 +195,12 @@ class TrellisDecoder:
         self.tok = torch.zeros(1, dtype=torch.int64, device=dev)     # token to feed next
         self.arange = torch.arange(max_len, device=dev)
         self.graph = None
+        # one-token steps: output head and arg-max in the library (table streamed once)
+        self.fast_head = H in (2048, 4096)
+        if self.fast_head:
+            self.logits = torch.empty(1, cfg.vocab, dtype=torch.float32, device=dev)
+            self.head_ws = torch.empty(max(int(_lib.load().glqh_lm_head_workspace_bytes()), 256), dtype=torch.uint8,
+                                       device=dev)
 
     @property
     def packed_bytes_per_token(self):
@@ -256,8 +262,9 @@ class TrellisDecoder:
         check(lib.glqh_silu_mul_bf16(gate.data_ptr(), up.data_ptr(), act.data_ptr(), act.numel(), _stream()))
         return x, L["down"](act)
 
-    def _forward(self, ids, pos):
-        """ids, pos: (T,) int64 on the device.  Returns the logits of the last token."""
+    def _forward(self, ids, pos, tok_out=None):
+        """ids, pos: (T,) int64 on the device.  Returns the logits of the last token; with
+        tok_out (one-token steps) their arg-max is written there as well."""
         T = ids.numel()
         mask = None
         if not (T == 1 and self.cfg.head_dim == 128):
@@ -269,7 +276,15 @@ class TrellisDecoder:
             _, h = _linear_add_rms_norm(delta[0], delta[1], x, self.ln_f, self.cfg.rms_eps)
         else:
             _, h = _add_rms_norm(x[-1:], delta[-1:], self.ln_f, self.cfg.rms_eps)
-        return torch.matmul(h, self.emb.t()).float()
+        if tok_out is not None and T == 1 and self.fast_head:
+            check(_lib.load().glqh_lm_head_argmax_bf16(
+                h.data_ptr(), self.emb.data_ptr(), self.cfg.vocab, self.cfg.hidden, self.logits.data_ptr(),
+                tok_out.data_ptr(), self.head_ws.data_ptr(), self.head_ws.numel(), _stream()))
+            return self.logits
+        logits = torch.matmul(h, self.emb.t()).float()
+        if tok_out is not None:
+            tok_out.copy_(logits.argmax(-1))
+        return logits
 
     def prefill(self, prompt_ids):
         T = prompt_ids.numel()
@@ -280,8 +295,7 @@ class TrellisDecoder:
         return logits
 
     def _step(self):
-        logits = self._forward(self.tok, self.pos)
-        self.tok.copy_(logits.argmax(-1))
+        logits = self._forward(self.tok, self.pos, tok_out=self.tok)
         self.pos.add_(1)
         return logits
 

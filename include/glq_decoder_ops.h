@@ -95,6 +95,16 @@ int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_features, const gl
                                     int64_t kv_heads, int64_t head_dim, int64_t max_len,
                                     int apply_rope, void *ws, size_t ws_bytes, void *stream);
 
+size_t glqh_lm_head_workspace_bytes(void);
+
+/* Output head of a decode step: logits[r] = <h, table[r, :]> for a (vocab, hidden) bf16 table and
+ * one bf16 activation row (fp32 sums), *token_out = the row of the largest logit (lowest row on
+ * ties).  logits_out (vocab fp32) may be NULL.  hidden = 2048 or 4096; ws:
+ * glqh_lm_head_workspace_bytes() bytes.  Two launches; the table is streamed once. */
+int glqh_lm_head_argmax_bf16(const void *h, const void *table, int64_t vocab, int64_t hidden,
+                             float *logits_out, int64_t *token_out, void *ws, size_t ws_bytes,
+                             void *stream);
+
 #ifdef __cplusplus
 }
 #endif

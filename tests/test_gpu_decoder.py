@@ -184,3 +184,39 @@ def test_fused_qkv_rope_store_is_bit_identical(rope):
     kc3, vc3, a3 = torch.zeros_like(kc0), torch.zeros_like(vc0), torch.zeros_like(a0)
     D._qkv_rope_attn(q, k, v, h, pos0, cos, sin, kc3, vc3, a3, heads, kvh, hd, L, rope)
     assert torch.equal(a3.view(heads, hd), vc3[:, 0].repeat_interleave(heads // kvh, 0))
+
+
+@pytest.mark.parametrize("hidden,vocab", [(2048, 128256), (4096, 1000), (2048, 7)])
+def test_output_head_and_argmax(hidden, vocab):
+    """Logits of the library's output head against a float64 product, its arg-max against the
+    arg-max of its own logits, ties to the lowest row; with and without the logits buffer."""
+    from glq_amd import _lib
+    from glq_amd._lib import check
+    say("lm head", hidden, vocab)
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(vocab)
+    E = (torch.randn(vocab, hidden, generator=g) * 0.02).to(torch.bfloat16)
+    h = torch.randn(1, hidden, generator=g).to(torch.bfloat16)
+    E[vocab - 1] = E[3]                                        # an exact tie between rows 3 and vocab-1
+    h = (E[3:4].float() * 40).to(torch.bfloat16) if vocab <= 1000 else h   # make that pair the maximum
+    Ed, hd = E.to(DEV), h.to(DEV)
+    logits = torch.empty(1, vocab, dtype=torch.float32, device=DEV)
+    tok = torch.full((1,), -1, dtype=torch.int64, device=DEV)
+    ws = torch.empty(int(lib.glqh_lm_head_workspace_bytes()), dtype=torch.uint8, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    check(lib.glqh_lm_head_argmax_bf16(hd.data_ptr(), Ed.data_ptr(), vocab, hidden, logits.data_ptr(),
+                                       tok.data_ptr(), ws.data_ptr(), ws.numel(), st))
+    ref = (h.double() @ E.double().t()).numpy()
+    assert rel(logits, ref) < 1e-5, rel(logits, ref)
+    lg = logits[0].cpu()
+    top = int(tok.item())
+    assert lg[top] == lg.max() and top == int((lg == lg.max()).nonzero()[0])
+    if vocab <= 1000:
+        assert top == 3 and lg[3] == lg[vocab - 1]
+    tok2 = torch.full((1,), -1, dtype=torch.int64, device=DEV)
+    check(lib.glqh_lm_head_argmax_bf16(hd.data_ptr(), Ed.data_ptr(), vocab, hidden, None, tok2.data_ptr(),
+                                       ws.data_ptr(), ws.numel(), st))
+    assert int(tok2.item()) == top
+    with pytest.raises(RuntimeError, match="hidden size"):
+        check(lib.glqh_lm_head_argmax_bf16(hd.data_ptr(), Ed.data_ptr(), vocab, 1024, None, tok2.data_ptr(),
+                                           ws.data_ptr(), ws.numel(), st))

@@ -406,6 +406,12 @@ extern "C" int glqh_fused_linear_trellis_3inst(
 }
 
 // ---- grouped trellis linears -------------------------------------------------------
+// Two to four tokens on a large group: every workgroup of the fused-input launch repeats the
+// transform of all tokens, and one transform launch + one plain GEMV per layer is faster
+// (gate/up 4096 -> 2 x 14336 at four tokens: 63 us folded, 46 us as separate per-layer calls).
+static bool tr_group_plain(int64_t total_m_pad, int64_t n_pad, int64_t B) {
+    return B >= 2 && total_m_pad * n_pad > ((int64_t)48 << 20);
+}
 static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {
     int64_t total = 0;
     for (int i = 0; i < n_shards; ++i) total += m_pads[i];
@@ -423,7 +429,12 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
     int ks2 = 0;
     if (!glqh_trellis_fusein_plan(total_m_pad, n_pad, B, &steps, &ks)) return 0;
     if (glqh_trellis_mma_fusein_plan((total_m_pad + 63) / 64, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
-    return (size_t)n_shards * 256 + align256((size_t)ks * B * total_m_pad * sizeof(float));
+    // the separate-transform route of large groups: slots of the plain plan (at most 64) and x_rht
+    size_t plain = 0;
+    if (tr_group_plain(total_m_pad, n_pad, B))
+        plain = align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)64 * B * total_m_pad * sizeof(float));
+    const size_t fused = align256((size_t)ks * B * total_m_pad * sizeof(float));
+    return (size_t)n_shards * 256 + (plain > fused ? plain : fused);
 }
 
 // Decode launch of a group: checks, K plan, partial-sum layout in ws.  On return parts[i] holds
@@ -480,6 +491,32 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
         total += sh.m_pad;
     }
     int steps = 0, ks = 0;
+    if (tr_group_plain(total, n_pad, B)) {
+        // one K plan for all layers (that of the tallest), so that the finishing launch sees one slot count
+        int64_t mmax = 0;
+        for (int i = 0; i < n_shards; ++i) mmax = c->m_pads[i] > mmax ? c->m_pads[i] : mmax;
+        int S = 0;
+        glqh_trellis_mma_plan(mmax, n_pad, &S, &ks);
+        const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
+        const size_t need = xb + align256((size_t)ks * B * total * sizeof(float));
+        GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+        f16 *x_rht = (f16 *)ws;
+        float *p = (float *)((char *)ws + xb);
+        c->R = R; c->ks = ks; c->fi_mode = 0;
+        for (int i = 0; i < n_shards; ++i) {
+            // layers quantized with the same sign vector share one transform of x; launches on
+            // one stream run in order, so x_rht can be rewritten between layers
+            if ((i == 0 || sv[i] != sv[i - 1]) &&
+                glqh_launch_input_rht(x, x_dtype, x_stride, sv[i], x_rht, GLQH_F16, B, in_features, n_pad, bn_meta_dev,
+                                      blocks_n, n_blocks_n, 0.0f, st))
+                return 1;
+            c->parts[i] = p;
+            p += (size_t)ks * B * c->m_pads[i];
+            if (glqh_launch_trellis_mma(x_rht, B, packed[i], R, c->m_pads[i], n_pad, S, ks, c->parts[i], 0, 1.0f, 0, 0, st))
+                return 1;
+        }
+        return 0;
+    }
     const int fi_mode = tr_group_plan(c->m_pads, n_shards, n_pad, B, &steps, &ks);
     GLQH_REQUIRE(fi_mode != 0, "trellis group: shape not eligible");
     const size_t need = align256((size_t)ks * B * total * sizeof(float));

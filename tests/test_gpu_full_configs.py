@@ -50,7 +50,7 @@ def test_e8_two_stage_full_shapes(ext, m, n):
     ref = O.e8_linear_forward(x[:272].float().numpy(), art, n, m)
     xd = x.to(DEV)
     ys = {}
-    for M in (1, 4, 16, 256, 1024):                        # indices -> MFMA up to 16 tokens, dense route above
+    for M in (1, 4, 16, 40, 256, 1024):                    # indices -> MFMA up to 16 tokens, dense route above
         y = _e8_forward(ext, xd[:M], q1, q2, su, sv, m, n, torch.bfloat16)
         assert y.shape == (M, m)
         assert rel(y[:min(M, 272)], ref[:min(M, 272)]) < TOL
@@ -86,7 +86,7 @@ def test_trellis_full_shapes_many_tokens(ext, m, n):
             H.pack_block_meta(bm).to(DEV), 0.018, n, m, n, m)
     xd = x.to(DEV)
     ys = {}
-    for M in (1, 16, 256, 1024):                           # fused-input GEMV, MFMA GEMV, 128-token tiles, dense
+    for M in (1, 3, 16, 40, 64, 256, 1024):                # GEMV forms, 32+ tokens: whole-block finishing on tall layers, 128-token tiles, dense
         y = ext.glq_fused_linear_trellis_3inst_cuda(xd[:M], *args, out_dtype=torch.bfloat16)
         assert rel(y[:min(M, 272)], ref[:min(M, 272)]) < TOL
         assert torch.equal(y, ext.glq_fused_linear_trellis_3inst_cuda(xd[:M], *args, out_dtype=torch.bfloat16))

@@ -264,51 +264,69 @@ constexpr int PF_NT = 8;
 constexpr int PF_CH = 4;
 constexpr int PF_KP_SLOTS = PF_NT * 4 * 17 + 4;                 // 16-byte slots per k-pair (+4: bank skew)
 
-// (a.lo + a.hi, b.lo + b.hi) in fp16
-__device__ __forceinline__ uint32_t pair_sum(uint32_t ha, uint32_t hb) {
-    uint32_t d;
-    asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %0, %2, %2 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1"
-        : "=&v"(d)
-        : "v"(ha), "v"(hb));
-    return d;
+// One A operand: four words (a.lo + a.hi, b.lo + b.hi) in fp16 from eight hash results, as
+// eight SDWA adds.  gfx950 needs one wait state between an instruction that writes part of a
+// register (dst_sel) and the next one that reads that register, and the compiler cannot see
+// into an asm block: the four low-half writes come first and the four high-half writes (which
+// read their destination to preserve it) after them, and a trailing s_nop covers whoever reads
+// the last word next.  (Adjacent pairs, as this was first written, gave wrong rows once the
+// scheduler moved an MFMA right behind them.)
+__device__ __forceinline__ u32x4 pair_sum4(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1, uint32_t a2,
+                                           uint32_t b2, uint32_t a3, uint32_t b3) {
+    uint32_t d0, d1, d2, d3;
+    asm("v_add_f16_sdwa %0, %4, %4 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %1, %6, %6 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %2, %8, %8 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %3, %10, %10 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %0, %5, %5 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %1, %7, %7 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %2, %9, %9 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %3, %11, %11 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "s_nop 0"
+        : "=&v"(d0), "=&v"(d1), "=&v"(d2), "=&v"(d3)
+        : "v"(a0), "v"(b0), "v"(a1), "v"(b1), "v"(a2), "v"(b2), "v"(a3), "v"(b3));
+    return u32x4{d0, d1, d2, d3};
 }
 
-// Staging of tokens [tok0, tok0+128) x k-pairs [c0, c0+PF_CH) in two halves, so that the
-// global loads of the next chunk are in flight while the current one is multiplied: item =
-// 16 bytes of one token (columns 8h..8h+7 of a k-pair), whose dword q goes to dword h of slot
-// (q, token).  The loads are unconditional (addresses clamped into the matrix); tokens past
-// M and k-pairs past the slot are zeroed or skipped when written.
-constexpr int PF_ITEMS = 16 * PF_NT * PF_CH * 4 / TR_THREADS;   // per thread
+// Staging of tokens [tok0, tok0+128) x k-pairs [c0, c0+PF_CH), loaded one chunk ahead so that
+// the global loads are in flight while the current chunk is multiplied: a group = the 64 bytes
+// of one token in one k-pair (four 16-byte items, columns 8h..8h+7), whose dwords q of the four
+// items make up slot (q, token) -- one 16-byte LDS write per q.  Consecutive lanes take the
+// k-pairs of a token first (256 contiguous bytes of its row).  The loads are unconditional
+// (addresses clamped into the matrix); tokens past M and k-pairs past the slot are written as
+// zeros or skipped.
+constexpr int PF_GROUPS = 16 * PF_NT * PF_CH / TR_THREADS;      // per thread
 
 struct pf_regs {
-    u32x4 v[PF_ITEMS];
+    u32x4 v[PF_GROUPS][4];
 };
 
 __device__ __forceinline__ pf_regs pf_stage_load(const f16 *__restrict__ x, int M, int k, int tok0, int c0,
                                                  int kp_last) {
     pf_regs r;
 #pragma unroll
-    for (int i = 0; i < PF_ITEMS; ++i) {
+    for (int i = 0; i < PF_GROUPS; ++i) {
         const int idx = i * TR_THREADS + (int)threadIdx.x;
-        const int h = idx & 3;
-        const int u = (idx >> 2) % PF_CH, tk = (idx >> 2) / PF_CH;
-        r.v[i] = *(const u32x4 *)(x + (int64_t)min(tok0 + tk, M - 1) * k + 32 * min(c0 + u, kp_last) + 8 * h);
+        const int u = idx % PF_CH, tk = idx / PF_CH;
+        const f16 *p = x + (int64_t)min(tok0 + tk, M - 1) * k + 32 * min(c0 + u, kp_last);
+#pragma unroll
+        for (int h = 0; h < 4; ++h) r.v[i][h] = *(const u32x4 *)(p + 8 * h);
     }
     return r;
 }
 
-__device__ __forceinline__ void pf_stage_write(uint32_t *xs, const pf_regs r, int M, int tok0, int n) {
+__device__ __forceinline__ void pf_stage_write(u32x4 *xs, const pf_regs r, int M, int tok0, int n) {
 #pragma unroll
-    for (int i = 0; i < PF_ITEMS; ++i) {
+    for (int i = 0; i < PF_GROUPS; ++i) {
         const int idx = i * TR_THREADS + (int)threadIdx.x;
-        const int h = idx & 3;
-        const int u = (idx >> 2) % PF_CH, tk = (idx >> 2) / PF_CH;
+        const int u = idx % PF_CH, tk = idx / PF_CH;
         if (u < n) {
-            const u32x4 v = tok0 + tk < M ? r.v[i] : u32x4{0u, 0u, 0u, 0u};
-            const int dst = (u * PF_KP_SLOTS + (tk >> 4) * (4 * 17) + (tk & 15)) * 4 + h;
+            const bool ok = tok0 + tk < M;
+            const int dst = u * PF_KP_SLOTS + (tk >> 4) * (4 * 17) + (tk & 15);
 #pragma unroll
-            for (int qq = 0; qq < 4; ++qq) xs[dst + qq * 17 * 4] = v[qq];
+            for (int qq = 0; qq < 4; ++qq)
+                xs[dst + qq * 17] = ok ? u32x4{r.v[i][0][qq], r.v[i][1][qq], r.v[i][2][qq], r.v[i][3][qq]}
+                                       : u32x4{0u, 0u, 0u, 0u};
         }
     }
 }
@@ -333,9 +351,8 @@ __device__ __forceinline__ mma_acc<PF_NT> pf_record(const tr_record<R> r, const 
 #pragma unroll
         for (int rh = 0; rh < 2; ++rh) {
             const int j0 = 2 * rh;
-            const f16x8 af = __builtin_bit_cast(
-                f16x8, u32x4{pair_sum(h0[j0], h0[j0 + 1]), pair_sum(h0[j0 + 4], h0[j0 + 5]),
-                             pair_sum(h1[j0], h1[j0 + 1]), pair_sum(h1[j0 + 4], h1[j0 + 5])});
+            const f16x8 af = __builtin_bit_cast(f16x8, pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5],
+                                                                 h1[j0], h1[j0 + 1], h1[j0 + 4], h1[j0 + 5]));
 #pragma unroll
             for (int tt = 0; tt < PF_NT; ++tt)
                 acc.v[2 * ms + rh][tt] =
@@ -379,7 +396,7 @@ tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict_
 #pragma unroll
         for (int tt = 0; tt < PF_NT; ++tt) acc.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    pf_stage_write((uint32_t *)xs_lds, pf_stage_load(x, M, k, tok0, kp0, last), M, tok0, kp1 - kp0);
+    pf_stage_write(xs_lds, pf_stage_load(x, M, k, tok0, kp0, last), M, tok0, kp1 - kp0);
     __syncthreads();
     for (int c0 = kp0; c0 < kp1; c0 += PF_CH) {
         pf_regs next;
@@ -395,7 +412,7 @@ tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict_
         }
         // LDS-only barriers: the records requested two ahead stay in flight across them
         fht_barrier<true>();                                     // chunk consumed by every wave
-        pf_stage_write((uint32_t *)xs_lds, next, M, tok0, kp1 - (c0 + PF_CH));
+        pf_stage_write(xs_lds, next, M, tok0, kp1 - (c0 + PF_CH));
         fht_barrier<true>();
     }
     if (!active) return;

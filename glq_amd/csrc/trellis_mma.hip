@@ -157,35 +157,39 @@ __device__ __forceinline__ void mma_reduce_store(const mma_acc<NT> acc, float *r
 }
 
 // Stage the activations of k-pairs [c0, c0+n) and tokens [tok0, tok0 + 16*NT) into the LDS
-// slots.  One item = 16 bytes of one token (columns 8h..8h+7 of a k-pair), which feeds the
-// (2*hb, 2*hb+1) dwords of four slots; U items are requested before any is written.
+// slots.  One item = 32 bytes of one token (columns 16ks..16ks+15 of a k-pair): its dword q
+// and dword 4+q, each splat into a duplicated pair, are the whole 16-byte slot (ks, q, token)
+// -- one LDS write per q.  U items (2U loads) are requested before any is written.
 template <int TP, int NT>
 __device__ __forceinline__ void mma_stage(uint32_t *xs, const f16 *__restrict__ x, int B, int k, int tok0,
                                           int c0, int n) {
     constexpr int TPS = mma_tps<TP>();
-    constexpr int U = 4;
-    const int total = NT * TP * n * 4;
+    constexpr int U = 2;
+    const int total = NT * TP * n * 2;
     for (int base = 0; base < total; base += U * TR_THREADS) {
-        u32x4 v[U];
+        u32x4 v[U][2];
         int dst[U];
 #pragma unroll
         for (int uu = 0; uu < U; ++uu) {
             const int idx = min(base + uu * TR_THREADS + (int)threadIdx.x, total - 1);
-            const int h = idx & 3;
-            const int u = (idx >> 2) % n, tk = (idx >> 2) / n;
+            const int ks = idx & 1;
+            const int u = (idx >> 1) % n, tk = (idx >> 1) / n;
             const int tt = tk / TP, tl = tk % TP;
             const int tok = tok0 + 16 * tt + tl;
-            const u32x4 ld = *(const u32x4 *)(x + (int64_t)min(tok, B - 1) * k + 32 * (c0 + u) + 8 * h);
-            v[uu] = tok < B ? ld : u32x4{0u, 0u, 0u, 0u};
-            // dword index of (u, tt, ks = h>>1, q = 0, tl), plus 2*hb
-            dst[uu] = ((((u * NT + tt) * 2 + (h >> 1)) * 4) * TPS + tl) * 4 + 2 * (h & 1);
+            const f16 *p = x + (int64_t)min(tok, B - 1) * k + 32 * (c0 + u) + 16 * ks;
+            const u32x4 l0 = *(const u32x4 *)p, l1 = *(const u32x4 *)(p + 8);
+            v[uu][0] = tok < B ? l0 : u32x4{0u, 0u, 0u, 0u};
+            v[uu][1] = tok < B ? l1 : u32x4{0u, 0u, 0u, 0u};
+            // dword index of slot (u, tt, ks, q = 0, tl)
+            dst[uu] = ((((u * NT + tt) * 2 + ks) * 4) * TPS + tl) * 4;
         }
 #pragma unroll
         for (int uu = 0; uu < U; ++uu) {
             if (base + uu * TR_THREADS + (int)threadIdx.x < total) {
 #pragma unroll
                 for (int qq = 0; qq < 4; ++qq)
-                    *(u32x2 *)(xs + dst[uu] + qq * TPS * 4) = u32x2{splat_lo(v[uu][qq]), splat_hi(v[uu][qq])};
+                    *(u32x4 *)(xs + dst[uu] + qq * TPS * 4) =
+                        u32x4{splat_lo(v[uu][0][qq]), splat_hi(v[uu][0][qq]), splat_lo(v[uu][1][qq]), splat_hi(v[uu][1][qq])};
             }
         }
     }

@@ -172,6 +172,29 @@ def test_trellis_two_stage_few_tokens(m, n, K2, B):
         assert rel(y1 + y2, y.float()) < 1e-2, rel(y1 + y2, y.float())
 
 
+@pytest.mark.parametrize("K1,K2", [(2, 2), (3, 1), (3, 3), (2, 4)])
+@pytest.mark.parametrize("B", [1, 2, 4])
+def test_trellis_two_stage_other_rates(K1, K2, B):
+    """First stages of 2 and 3 bits per weight through the same routes (one layer large enough
+    for the MFMA form of the folded transform), against the oracle."""
+    from glq_amd import ext, hadamard as H
+    m, n = 2048, 512
+    say("trellis two stages, rates", K1, K2, B)
+    p1, p2 = O.random_packed(m, n, K1, 5), O.random_packed(m, n, K2, 6)
+    su, sv = O.rht_signs(m, n, 7)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"trellis_packed": p1, "trellis_packed2": p2, "inv_resid_scale2": np.float32(0.25),
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.03),
+           "blocks_m": bm, "blocks_n": bn}
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(K1 * 10 + K2)).to(torch.bfloat16)
+    ref = O.trellis_linear_forward(x.float().numpy(), art, n, m)
+    y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), t(p2), torch.tensor(bn), torch.tensor(bm),
+        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), 0.03, 0.25, n, m, n, m,
+        out_dtype=torch.bfloat16)
+    assert y.shape == (B, m) and rel(y, ref) < TOL, rel(y, ref)
+
+
 def test_e8_dense_route_many_tokens():
     from glq_amd import ext, hadamard as H
     m, n, B = 96, 160, 40

@@ -320,9 +320,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     // Up to four tokens the input transform is folded into the GEMV launch.  A two-stage layer
     // repeats it in both launches at one token, where that is cheaper than a launch of its own
     // (2048 x 2048: 14.5 against 17.4 us; at four tokens 23.9 against 18.0, so two to four
-    // tokens transform x once); only the MFMA form takes a pre-scaled second stage, and a 1-bit
-    // second stage has no such kernel.  Everything else transforms x once into scratch and
-    // reads it from every workgroup.
+    // tokens transform x once); only the MFMA form takes a pre-scaled second stage.  Everything
+    // else transforms x once into scratch and reads it from every workgroup.
     int ks = 0, fi_steps = 0, fi_mode = 0;
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
     const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
@@ -335,7 +334,7 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     const bool fi_pays = m_pad * n_pad <= ((int64_t)32 << 20) && (B == 1 || (B == 2 && pow2_n));
     if (fi_pays && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
         (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0 &&
-        (!has_s2 || (B == 1 && R2 >= 2 && fi_mode == 2 && merge2))) {
+        (!has_s2 || (B == 1 && fi_mode == 2 && merge2))) {
         if (n_blocks_n > 1) {
             int64_t sum = 0;
             for (int64_t i = 0; i < n_blocks_n; ++i) {

@@ -885,13 +885,14 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
     (B == 1 ? (x_dtype == GLQH_F16 ? GLQH_FI(RR, f16, 1) : GLQH_FI(RR, uint16_t, 1))     \
             : (x_dtype == GLQH_F16 ? GLQH_FI(RR, f16, 4) : GLQH_FI(RR, uint16_t, 4)))
     switch (R) {
+    case 1: return GLQH_FI_R(1);                               // second stage of the 5 bpw recipe
     case 2: return GLQH_FI_R(2);
     case 3: return GLQH_FI_R(3);
     case 4: return GLQH_FI_R(4);
     }
 #undef GLQH_FI_R
 #undef GLQH_FI
-    return glqh_fail("fused-input trellis kernel supports R (bits/weight) 2-4, got %d", R);
+    return glqh_fail("fused-input trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
 template <typename K>
@@ -916,5 +917,5 @@ int glqh_trellis_mma_init(void) {
     return mma_init_R<1>() || mma_init_R<2>() || mma_init_R<3>() || mma_init_R<4>() ||
            pf_set_lds(tr_mma_prefill_kernel<1>) || pf_set_lds(tr_mma_prefill_kernel<2>) ||
            pf_set_lds(tr_mma_prefill_kernel<3>) || pf_set_lds(tr_mma_prefill_kernel<4>) ||
-           fi_init_R<2>() || fi_init_R<3>() || fi_init_R<4>();
+           fi_init_R<1>() || fi_init_R<2>() || fi_init_R<3>() || fi_init_R<4>();
 }

@@ -409,7 +409,10 @@ extern "C" int glqh_fused_linear_trellis_3inst(
 // transform of all tokens, and one transform launch + one plain GEMV per layer is faster
 // (gate/up 4096 -> 2 x 14336 at four tokens: 63 us folded, 46 us as separate per-layer calls).
 static bool tr_group_plain(int64_t total_m_pad, int64_t n_pad, int64_t B) {
-    return B >= 2 && total_m_pad * n_pad > ((int64_t)48 << 20);
+    const int64_t w = total_m_pad * n_pad;
+    // q/k/v of a 4096-wide model (25M weights): 22.1 / 25.6 / 28.5 us folded at 2 / 3 / 4 tokens,
+    // 24.5 / 24.5 / 25.1 us separate; gate/up 2048 -> 2 x 11008 (45M): 19-22 us folded, 25-26 separate
+    return B >= 2 && (w > ((int64_t)48 << 20) || (B >= 3 && n_pad >= 4096 && w > ((int64_t)16 << 20)));
 }
 static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {
     int64_t total = 0;

@@ -306,13 +306,17 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     float *part1 = (float *)((char *)ws + xb);
     float *part2 = (float *)((char *)ws + xb + pb);
 
-    // Two stages at up to four tokens with canonical output blocks: the second stage's partial
+    // Two stages at a small batch with canonical output blocks: the second stage's partial
     // sums are written already multiplied by inv_resid_scale2, right behind the first stage's
     // slots, and the finishing kernels of the single-stage path sum all 2*ks slots (the generic
     // two-part transform takes twice as long: 14.3 against 6.8 us at 4096 x 4096).
     glqh_meta_args canon_m;
-    const bool canon_out = B <= 4 && glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
-                                                         n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
+    // The slice kernels of the grouped launcher finish canonical layers faster than the generic
+    // transform at every small batch (4096 x 4096 whole linear: 20.7 -> 17.5 us at 8 tokens, 27.5 ->
+    // 23.5 at 24, 41.3 -> 36.5 at 64); tall layers from 32 tokens on take whole blocks instead.
+    const bool canon_out = (B <= 31 || (B <= 64 && m_pad < 8192)) &&
+                           glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
+                                               n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
                            canon_m.canon == m_pad;
     const bool merge2 = has_s2 && canon_out && !(y && y_rht_out);
     const float ps2 = merge2 ? (float)inv_resid_scale2 : 1.0f;
@@ -383,7 +387,7 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         return 0;
     }
     if ((!has_s2 || merge2) && !y_rht_out && canon_out) {
-        // canonical blocks, a few tokens: the grouped launcher's kernels (a group of one)
+        // canonical blocks, small batch: the grouped launcher's kernels (a group of one)
         const float *pt[1] = {part1};
         const void *sus[1] = {su_f16};
         void *ys[1] = {y};

@@ -813,9 +813,24 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
     if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
                               bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
         return 1;
+    // Canonical output blocks at up to 16 tokens: every stage's partial sums are written already
+    // multiplied by that stage's scale, which makes them ks * stages plain slots for the slice
+    // kernels of the grouped launcher (faster than the generic multi-part transform).
+    glqh_meta_args canon_m;
+    const bool canon_out = B <= 16 && glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
+                                                          n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
+                           canon_m.canon == m_pad;
     if (glqh_launch_e8_partial(x_rht, B, sg.q, sg.n, table1, table2 ? table2 : table1,
-                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st))
+                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st, canon_out ? sg.scale : nullptr))
         return 1;
+    if (canon_out) {
+        const float *pt[1] = {part};
+        const void *sus[1] = {su_f16};
+        void *ys[1] = {y};
+        const float sc[1] = {1.0f};
+        return glqh_launch_output_rht_group(pt, sus, ys, sc, &m_pad, &out_features, 1, y_dtype, y_stride, B,
+                                            ks * sg.n, st);
+    }
     glqh_ysrc src = {};
     src.nparts = sg.n;
     for (int s = 0; s < sg.n; ++s) src.scale[s] = sg.scale[s];

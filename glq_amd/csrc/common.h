@@ -143,9 +143,14 @@ int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, 
                               hipStream_t stream);
 int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t *out, int32_t *bad,
                                 hipStream_t stream);
+// pscale: per-stage factors applied to the partial sums as they are written (NULL: ones)
+struct glqh_e8_pscale {
+    float v[4];
+};
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
-                           int64_t n_pad, int ksplit, float *part, hipStream_t stream);
+                           int64_t n_pad, int ksplit, float *part, hipStream_t stream,
+                           const float *pscale = nullptr);
 int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,
                               const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
                               int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream);

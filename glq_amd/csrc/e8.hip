@@ -74,7 +74,8 @@ __global__ void __launch_bounds__(E8_THREADS)
 e8_gemv_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
                const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n2,
-               const f16 *__restrict__ x, int B, int m_pad, int n_pad, float *__restrict__ part) {
+               const f16 *__restrict__ x, int B, int m_pad, int n_pad, float *__restrict__ part,
+               glqh_e8_pscale ps) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int c = lane & 7;
@@ -154,7 +155,7 @@ e8_gemv_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
             v += __shfl_xor(v, 4, GLQH_WAVE);
             const int tok = tok0 + t;
             if (c == 0 && row_ok && tok < B)
-                part[(((int64_t)blockIdx.y * NS + s) * B + tok) * m_pad + row] = v;
+                part[(((int64_t)blockIdx.y * NS + s) * B + tok) * m_pad + row] = ps.v[s] * v;
         }
 }
 
@@ -257,21 +258,21 @@ e8_decompress_lds_kernel(const uint16_t *__restrict__ q1, const uint16_t *__rest
 template <int NS>
 int launch_e8_NS(const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
                  const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, int ksplit,
-                 float *part, hipStream_t stream) {
+                 float *part, hipStream_t stream, glqh_e8_pscale ps) {
     const unsigned gx = (unsigned)((m_pad + E8_ROWS_PER_WG - 1) / E8_ROWS_PER_WG);
     const uint16_t *q1 = (const uint16_t *)q[0], *q2 = (const uint16_t *)q[1];
     const uint16_t *q3 = (const uint16_t *)q[2], *q4 = (const uint16_t *)q[3];
     const f16 *xp = (const f16 *)x;
     if (B == 1) {
         hipLaunchKernelGGL((e8_gemv_kernel<NS, 1>), dim3(gx, ksplit, 1), dim3(E8_THREADS), 0, stream, q1,
-                           q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B, (int)m_pad, (int)n_pad, part);
+                           q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B, (int)m_pad, (int)n_pad, part, ps);
     } else if (B <= 2) {
         hipLaunchKernelGGL((e8_gemv_kernel<NS, 2>), dim3(gx, ksplit, 1), dim3(E8_THREADS), 0, stream, q1,
-                           q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B, (int)m_pad, (int)n_pad, part);
+                           q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B, (int)m_pad, (int)n_pad, part, ps);
     } else {
         hipLaunchKernelGGL((e8_gemv_kernel<NS, 4>), dim3(gx, ksplit, (unsigned)((B + 3) / 4)),
                            dim3(E8_THREADS), 0, stream, q1, q2, q3, q4, t1, t2, (uint32_t)n2, xp, (int)B,
-                           (int)m_pad, (int)n_pad, part);
+                           (int)m_pad, (int)n_pad, part, ps);
     }
     GLQH_LAUNCH_CHECK("e8 gemv launch");
     return 0;
@@ -283,7 +284,7 @@ int glqh_e8_mma_init(void);
 int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1);
 int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
-                       hipStream_t stream);
+                       hipStream_t stream, const float *pscale);
 
 int glqh_e8_init(void) {
     if (glqh_check_hip(hipFuncSetAttribute((const void *)e8_decompress_lds_kernel,
@@ -327,14 +328,17 @@ int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t 
 
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
-                           int64_t n_pad, int ksplit, float *part, hipStream_t stream) {
+                           int64_t n_pad, int ksplit, float *part, hipStream_t stream, const float *pscale) {
+    glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
+    if (pscale)
+        for (int i = 0; i < 4; ++i) ps.v[i] = pscale[i];
     if (glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536) > 0)
-        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream);
+        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream, pscale);
     switch (nstages) {
-    case 1: return launch_e8_NS<1>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
-    case 2: return launch_e8_NS<2>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
-    case 3: return launch_e8_NS<3>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
-    case 4: return launch_e8_NS<4>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream);
+    case 1: return launch_e8_NS<1>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);
+    case 2: return launch_e8_NS<2>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);
+    case 3: return launch_e8_NS<3>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);
+    case 4: return launch_e8_NS<4>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);
     }
     return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
 }

@@ -78,7 +78,8 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
               const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
               const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n1, uint32_t n2,
               int t2_is_t1, const f16 *__restrict__ x, int B, int m_pad, int n_pad, int P, int slot_blks,
-              int xs_slots, int ksplit, int ns_total, int s_off, float *__restrict__ part) {
+              int xs_slots, int ksplit, int ns_total, int s_off, float *__restrict__ part,
+              glqh_e8_pscale ps) {                              // ps.v[s]: factor of stage s_off + s
     constexpr int WR = EM_WAVES / WK;
     constexpr int ROWS = 16 * WR;
     extern __shared__ u32x4 lds[];
@@ -208,7 +209,7 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int orow = rb * ROWS + wr * 16 + 4 * g + r;
-                        if (orow < m_pad) part[(((int64_t)slot * ns_total + s_off + s) * B + i) * m_pad + orow] = acc[s][r];
+                        if (orow < m_pad) part[(((int64_t)slot * ns_total + s_off + s) * B + i) * m_pad + orow] = ps.v[s] * acc[s][r];
                     }
             }
         } else {
@@ -229,7 +230,7 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                 float v = red[e];
 #pragma unroll
                 for (int w = 1; w < WK; ++w) v += red[w * NS * TP * ROWS + e];
-                part[(((int64_t)slot * ns_total + s_off + s) * B + tl) * m_pad + orow] = v;
+                part[(((int64_t)slot * ns_total + s_off + s) * B + tl) * m_pad + orow] = ps.v[s] * v;
             }
         }
     }
@@ -285,12 +286,12 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
 template <int NS, int TP, int WK>
 int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
               const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad, int ns_total,
-              int s_off, float *part, hipStream_t stream) {
+              int s_off, float *part, hipStream_t stream, glqh_e8_pscale ps) {
     hipLaunchKernelGGL((e8_mma_kernel<NS, TP, WK>), dim3((unsigned)p.grid), dim3(EM_THREADS), p.lds, stream,
                        (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
                        (const uint16_t *)q[3], t1, t2, (uint32_t)n1, (uint32_t)n2, (int)(t1 == t2 && n1 == n2),
                        (const f16 *)x, (int)B, (int)m_pad, (int)n_pad, p.P, p.slot_blks, p.xs_slots, p.ksplit,
-                       ns_total, s_off, part);
+                       ns_total, s_off, part, ps);
     GLQH_LAUNCH_CHECK("e8 mma launch");
     return 0;
 }
@@ -298,8 +299,11 @@ int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4]
 template <int NS>
 int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
                  const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad, int ns_total,
-                 int s_off, float *part, hipStream_t stream) {
-#define GLQH_EM(TP, WK) em_launch<NS, TP, WK>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, part, stream)
+                 int s_off, float *part, hipStream_t stream, const float *pscale) {
+    glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
+    if (pscale)
+        for (int i = 0; i + s_off < 4; ++i) ps.v[i] = pscale[s_off + i];
+#define GLQH_EM(TP, WK) em_launch<NS, TP, WK>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, part, stream, ps)
     if (p.TP == 1) return GLQH_EM(1, 4);
     if (p.TP == 4) return GLQH_EM(4, 4);
     return GLQH_EM(16, 1);
@@ -333,14 +337,14 @@ int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1) {
 // three and four stages take a second launch for stages 3-4, which index the primary table.
 int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
-                       hipStream_t stream) {
+                       hipStream_t stream, const float *pscale) {
     em_plan p;
     if (!em_make_plan(m_pad, n_pad, B, n1, &p)) return glqh_fail("e8 mma: shape not eligible");
     if (nstages < 1 || nstages > 4) return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
-    if (nstages == 1) return em_launch_NS<1>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, 1, 0, part, stream);
-    if (em_launch_NS<2>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, nstages, 0, part, stream)) return 1;
+    if (nstages == 1) return em_launch_NS<1>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, 1, 0, part, stream, pscale);
+    if (em_launch_NS<2>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, nstages, 0, part, stream, pscale)) return 1;
     if (nstages == 2) return 0;
     const void *const q34[4] = {q[2], q[3], q[2], q[3]};
-    if (nstages == 3) return em_launch_NS<1>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 3, 2, part, stream);
-    return em_launch_NS<2>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 4, 2, part, stream);
+    if (nstages == 3) return em_launch_NS<1>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 3, 2, part, stream, pscale);
+    return em_launch_NS<2>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 4, 2, part, stream, pscale);
 }

@@ -43,6 +43,13 @@ SIGNATURES = {
                 c_vp, c_i64, c_vp, c_i64, c_vp, c_vp,
                 c_dbl, c_dbl, c_i64, c_i64, c_i64, c_i64,
                 c_vp, c_int, c_i64, c_vp, c_i64, c_vp, c_sz, c_vp]),
+    "glqh_noalloc_scratch_bytes": (c_sz, []),
+    "glqh_fused_linear_trellis_3inst_noalloc": (
+        c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_vp,
+                c_vp, c_i64, c_i64, c_vp, c_i64, c_i64,
+                c_vp, c_i64, c_vp, c_i64, c_vp, c_vp,
+                c_dbl, c_dbl, c_i64, c_i64, c_i64, c_i64,
+                c_vp, c_int, c_i64, c_vp, c_i64, c_vp]),
     "glqh_e8_pack_table": (c_int, [c_vp, c_i64, c_vp, c_vp, c_vp]),
     "glqh_e8_repack_table": (c_int, [c_vp, c_i64, c_vp, c_vp, c_vp]),
     "glqh_e8_matmul_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64]),

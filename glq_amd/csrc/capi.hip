@@ -408,6 +408,60 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                                   blocks_m, n_blocks_m, 0, 0.0f, st);
 }
 
+// ---- the same linear for callers that cannot allocate -----------------------------------
+// Scratch of the fused trellis linear (x_rht + split-K partial sums) in a file-scope device
+// array instead of a caller-provided workspace.  Every GPU holds its own copy of the array at
+// its own address, resolved once per device; host code uses that address only, never the
+// array's name.  Nothing in it has to start at zero: the decode launch writes every
+// [slot][token][row] partial sum before the finishing launch reads it.
+#define GLQH_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
+#define GLQH_NOALLOC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[GLQH_NOALLOC_SCRATCH_BYTES];
+static void *g_scratch_ptr[GLQH_NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mu;
+
+static int noalloc_scratch_for_current_device(void **out) {
+    int dev = -1;
+    if (glqh_check_hip(hipGetDevice(&dev), "hipGetDevice")) return 1;
+    GLQH_REQUIRE(dev >= 0 && dev < GLQH_NOALLOC_MAX_DEVICES, "no-alloc entry: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        if (glqh_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return 1;
+        GLQH_REQUIRE(p != nullptr, "no-alloc entry: scratch array has no device address");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" size_t glqh_noalloc_scratch_bytes(void) { return GLQH_NOALLOC_SCRATCH_BYTES; }
+
+extern "C" int glqh_fused_linear_trellis_3inst_noalloc(
+    const void *x, int x_dtype, int64_t x_stride, int64_t B, const void *sv_f16, const void *su_f16,
+    const void *packed, int64_t packed_rows, int64_t packed_cols, const void *packed2,
+    int64_t packed2_rows, int64_t packed2_cols, const int64_t *blocks_n, int64_t n_blocks_n,
+    const int64_t *blocks_m, int64_t n_blocks_m, const glqh_block_meta *bn_meta_dev,
+    const glqh_block_meta *bm_meta_dev, double wscale, double inv_resid_scale2, int64_t in_features,
+    int64_t out_features, int64_t n_pad, int64_t m_pad, void *y, int y_dtype, int64_t y_stride,
+    float *y_rht_out, int64_t y_rht_stride, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(glqh_trellis_kernel_supported(m_pad, n_pad) && B >= 1,
+                 "fused trellis linear (no-alloc): needs m %% 32 == 0, k %% 64 == 0 and B >= 1");
+    const size_t need = glqh_fused_linear_trellis_workspace_bytes(B, n_pad, m_pad);
+    GLQH_REQUIRE(need <= GLQH_NOALLOC_SCRATCH_BYTES,
+                 "fused trellis linear (no-alloc): %lld tokens of a %lld x %lld layer need %zu bytes of scratch, "
+                 "the built-in buffer holds %zu; use glqh_fused_linear_trellis_3inst with a workspace",
+                 (long long)B, (long long)m_pad, (long long)n_pad, need, (size_t)GLQH_NOALLOC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (noalloc_scratch_for_current_device(&ws)) return 1;
+    return glqh_fused_linear_trellis_3inst(x, x_dtype, x_stride, B, sv_f16, su_f16, packed, packed_rows, packed_cols,
+                                           packed2, packed2_rows, packed2_cols, blocks_n, n_blocks_n, blocks_m,
+                                           n_blocks_m, bn_meta_dev, bm_meta_dev, wscale, inv_resid_scale2,
+                                           in_features, out_features, n_pad, m_pad, y, y_dtype, y_stride, y_rht_out,
+                                           y_rht_stride, ws, GLQH_NOALLOC_SCRATCH_BYTES, stream);
+}
+
 // ---- grouped trellis linears -------------------------------------------------------
 // Two to four tokens on a large group: every workgroup of the fused-input launch repeats the
 // transform of all tokens, and one transform launch + one plain GEMV per layer is faster

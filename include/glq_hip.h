@@ -144,6 +144,31 @@ int glqh_fused_linear_trellis_3inst(const void *x, int x_dtype, int64_t x_stride
                                     float *y_rht_out, int64_t y_rht_stride,
                                     void *ws, size_t ws_bytes, void *stream);
 
+/* glqh_fused_linear_trellis_3inst without the workspace argument, for callers that cannot
+ * allocate device memory (code under HIP-graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  The scratch (x_rht and the split-K
+ * partial sums) lives in a device array built into the library, glqh_noalloc_scratch_bytes()
+ * = 8 MiB per GPU, resolved once per device on the first call with that device current; the
+ * call allocates nothing and is refused with a message when
+ * glqh_fused_linear_trellis_workspace_bytes(B, n_pad, m_pad) exceeds that size.  Results are
+ * bit-identical to glqh_fused_linear_trellis_3inst.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (different streams, different threads) race; calls on one
+ * stream are ordered and safe. */
+size_t glqh_noalloc_scratch_bytes(void);
+int glqh_fused_linear_trellis_3inst_noalloc(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                            const void *sv_f16, const void *su_f16,
+                                            const void *packed, int64_t packed_rows, int64_t packed_cols,
+                                            const void *packed2, int64_t packed2_rows, int64_t packed2_cols,
+                                            const int64_t *blocks_n, int64_t n_blocks_n,
+                                            const int64_t *blocks_m, int64_t n_blocks_m,
+                                            const glqh_block_meta *bn_meta_dev,
+                                            const glqh_block_meta *bm_meta_dev,
+                                            double wscale, double inv_resid_scale2,
+                                            int64_t in_features, int64_t out_features,
+                                            int64_t n_pad, int64_t m_pad,
+                                            void *y, int y_dtype, int64_t y_stride,
+                                            float *y_rht_out, int64_t y_rht_stride, void *stream);
+
 /* ---- several trellis layers on the same activations, two launches ------------- */
 
 #define GLQH_MAX_SHARDS 4

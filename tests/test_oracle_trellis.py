@@ -143,6 +143,23 @@ def test_viterbi_matches_reference(golden, K):
     assert np.array_equal(hat, g[f"K{K}_hat"])
 
 
+@pytest.mark.parametrize("K", [1, 3])
+def test_viterbi_matches_reference_layer_states(golden, K):
+    """The rates the tile vectors above do not cover, on the states the reference's trellis_ldlq
+    (identity Hessian: no feedback, glq/trellis.py:649-688) wrote for a 64 x 128 layer: tile (i, k)
+    is rows 16i.., columns 16k.. of W / Wscale in step order, its states the same window of Qidxs."""
+    g = golden("trellis_storage")
+    W = g[f"K{K}_W"]
+    m, n = W.shape
+    tiles = O.matrix_to_tiles((W / np.float32(g[f"K{K}_Wscale"])).astype(np.float32))
+    want = g[f"K{K}_Qidxs"].reshape(m // 16, 16, n // 16, 16).transpose(0, 2, 1, 3).reshape(-1, 256)
+    sel = [0, 7, 13, 31] if K == 1 else [0, 5, 9, 14, 22, 31]
+    hat, st = O.trellis_quantize_tiles(tiles[sel], K)
+    assert np.array_equal(st.astype(np.uint16), want[sel])
+    dec = O.matrix_to_tiles(g[f"K{K}_decoded"].astype(np.float32))
+    assert np.array_equal(hat, dec[sel])
+
+
 @pytest.mark.parametrize("K", [1, 2, 3, 4])
 def test_fast_unpack_equals_bit_array_unpack(K):
     p = O.random_packed(64, 128, K, seed=40 + K)

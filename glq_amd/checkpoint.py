@@ -16,7 +16,7 @@ import os
 import numpy as np
 import torch
 
-from .quantized_linear import E8RHTLinear
+from .quantized_linear import E8RHTEmbedding, E8RHTLinear
 
 LAYER_BUFFERS = ("Qidxs", "Qidxs2", "Qidxs3", "Qidxs4", "trellis_packed", "trellis_packed2", "tlut",
                  "SU", "SV", "Wscale", "inv_resid_scale", "inv_resid_scale2", "inv_resid_scale3", "bias")
@@ -71,7 +71,8 @@ def _layer_groups(model_dir):
 
 
 def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None = None) -> dict:
-    """{layer name: E8RHTLinear on `device`} for every quantized linear of the checkpoint.
+    """{layer name: E8RHTLinear on `device`} for every quantized linear of the checkpoint; a
+    quantized embedding (per-row `Wscale`, one-element `SU`) becomes an `E8RHTEmbedding`.
 
     Block-diagonal checkpoints store unpadded dims, so (out, in) = (len(SU), len(SV)); legacy
     power-of-two padded shell checkpoints need the true shapes in `shapes[name] = (out, in)`
@@ -89,6 +90,21 @@ def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None 
                 if path not in handles:
                     handles[path] = safe_open(path, framework="pt", device="cpu")
                 sd[leaf] = handles[path].get_tensor(key)
+            if "Qidxs" in sd and sd["Wscale"].dim() == 1 and sd["SU"].numel() == 1:
+                # a quantized embedding (per-row scales, unit SU, glq/quantized_linear.py:1343-1452)
+                vocab, n_pad = sd["Qidxs"].shape[0], sd["SV"].numel()
+                dim = (shapes or {}).get(name, (vocab, n_pad))[1]
+                emb = E8RHTEmbedding(vocab, dim)
+                if emb.n_pad != n_pad:
+                    raise RuntimeError(f"{name}: embedding of width {dim} pads to {emb.n_pad}, the checkpoint "
+                                       f"stores {n_pad} columns; pass its true width in shapes[name]")
+                missing, unexpected = emb.load_state_dict(sd, strict=False)
+                if unexpected:
+                    raise RuntimeError(f"{name}: unexpected buffers {unexpected}")
+                emb = emb.to(device)
+                emb.set_codebook(table, table)
+                out[name] = emb
+                continue
             m_pad, n_pad = sd["SU"].numel(), sd["SV"].numel()
             o, i = (shapes or {}).get(name, (m_pad, n_pad))
             # legacy power-of-two padding is recognised by the module from the buffer shapes
@@ -100,6 +116,9 @@ def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None 
                 raise RuntimeError(f"{name}: unexpected buffers {unexpected}")
             lin = lin.to(device)
             if not trellis:
+                # one table serves both stages, also at 3 bpw: the 256-entry secondary table of that
+                # recipe is the first 256 rows of the full one (glq/codebook.py:348-368), and its
+                # indices never exceed 255
                 lin.set_codebook(table, table)
             out[name] = lin
     finally:

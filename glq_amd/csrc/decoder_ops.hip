@@ -52,6 +52,7 @@ __global__ void rope_kv_store_kernel(const uint16_t *__restrict__ q, const uint1
                                      int apply_rope) {
     const int t = blockIdx.x, h = blockIdx.y, i = threadIdx.x, half = D >> 1;
     const int64_t p = pos[t];
+    if (p < 0 || p >= max_len) return;             // position outside the cache: this token writes nothing
     const uint16_t *src;
     uint16_t *dst;
     bool rot = apply_rope != 0;
@@ -242,7 +243,9 @@ attn_decode_kernel(const uint16_t *__restrict__ q, const uint16_t *__restrict__ 
     __shared__ float red[AT_WAVES];
     __shared__ float part[AT_WAVES][D];
     const int h = blockIdx.x, g = h / (heads / kv_heads);
-    const int n = (int)pos_ptr[0] + 1;             // keys 0..pos (the current token is already cached)
+    const int64_t p = pos_ptr[0];
+    if (p < 0 || p >= max_len) return;             // position outside the cache (sc holds max_len scores)
+    const int n = (int)p + 1;                      // keys 0..pos (the current token is already cached)
     if (threadIdx.x < D) qs[threadIdx.x] = bf16_bits_to_f32(q[(int64_t)h * D + threadIdx.x]) * scale;
     __syncthreads();
     attn_core<false>(qs, kc + (int64_t)g * max_len * D, vc + (int64_t)g * max_len * D, n, nullptr, nullptr, sc, red,
@@ -482,6 +485,7 @@ out_rope_store_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos, co
     src.nparts = 1;
     const int len = 1 << blk.log_len, base = blk.off + (blk.r << blk.log_len), half = D >> 1;
     const int64_t p = *pos;
+    if (p < 0 || p >= max_len) return;             // position outside the cache: nothing is written
     {
         const int tid = threadIdx.x;
         const bool live = 4 * tid < len;
@@ -564,6 +568,7 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
     float *sc = lds;
     const int h = blockIdx.x, per = heads / kv_heads, g = h / per;
     const int64_t p = pos_ptr[0];
+    if (p < 0 || p >= max_len) return;             // position outside the cache and the score buffer
     const int n = (int)p + 1;
     const int tid = threadIdx.x;
     const int grp = tid < 512 ? 0 : tid < 768 ? 1 : 2;         // q | k | v, whole waves each

@@ -288,7 +288,8 @@ class TrellisDecoder:
 
     def prefill(self, prompt_ids):
         T = prompt_ids.numel()
-        assert T < self.max_len
+        if not 0 < T < self.max_len:
+            raise RuntimeError(f"prefill: prompt of {T} tokens does not fit max_len = {self.max_len}")
         logits = self._forward(prompt_ids.to(self.dev), self.arange[:T])
         self.tok.copy_(logits.argmax(-1))
         self.pos.fill_(T)
@@ -325,7 +326,9 @@ class TrellisDecoder:
         if use_graph and self.graph is None:
             self.capture()
         out = torch.empty(n_new, dtype=torch.int64, device=self.dev)
-        assert int(self.pos.item()) + n_new <= self.max_len
+        if int(self.pos.item()) + n_new > self.max_len:
+            raise RuntimeError(f"generate: {int(self.pos.item())} cached + {n_new} new tokens exceed "
+                               f"max_len = {self.max_len}")
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(n_new):

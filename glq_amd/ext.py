@@ -382,6 +382,21 @@ def glq_fused_linear_trellis_3inst_yrht_rvq2_cuda(x, sv, trellis_packed, trellis
                    _yrht_slice(y_rht_out, col, m_pad), None)
 
 
+_META_BLOCKS = {}
+
+
+def _meta_blocks(meta, num_blocks):
+    """Block sizes of a device meta tensor, read back once per tensor (a device-to-host copy on
+    every call would stall the batch-1 path and cannot run under graph capture)."""
+    key = (meta.data_ptr(), meta._version, tuple(meta.shape), str(meta.device))
+    hit = _META_BLOCKS.get(key)
+    if hit is None or hit[0]() is not meta:
+        for k in [k for k, v in _META_BLOCKS.items() if v[0]() is None]:
+            del _META_BLOCKS[k]
+        hit = _META_BLOCKS[key] = (weakref.ref(meta), [int(v) for v in meta[:num_blocks, 1].tolist()])
+    return hit[1]
+
+
 def glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, trellis_packed, m, k, in_features,
                                                 wscale=1.0, blocks_n_meta=None, num_blocks=1,
                                                 max_bs=0, out=None):
@@ -390,7 +405,7 @@ def glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, trellis_packed, m, k,
     if num_blocks > 1:
         if blocks_n_meta is None:
             raise RuntimeError("block-diagonal fused-input GEMV needs blocks_n_meta")
-        blocks = [int(v) for v in blocks_n_meta[:, 1].tolist()]
+        blocks = _meta_blocks(blocks_n_meta, int(num_blocks))
     else:
         blocks = [int(k)]
     if out is None:
@@ -439,7 +454,27 @@ def _half_table(codebook):
     key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device), codebook.dtype)
     hit = _HALF_TABLES.get(key)
     if hit is None or hit[0]() is not codebook:
+        for k in [k for k, v in _HALF_TABLES.items() if v[0]() is None]:   # tensors that are gone
+            del _HALF_TABLES[k]
         hit = _HALF_TABLES[key] = (weakref.ref(codebook), codebook.to(torch.float16).contiguous())
+    return hit[1]
+
+
+_DEV_TABLES = {}
+
+
+def _on_device(codebook, dev):
+    """`codebook` on `dev`; a table kept on another device (the reference keeps its codebooks on
+    the CPU until first use) is copied once per tensor, so the packed table built from the copy
+    is found again on the next call."""
+    if codebook.device == dev:
+        return codebook
+    key = (id(codebook), codebook._version, tuple(codebook.shape), str(codebook.device), str(dev))
+    hit = _DEV_TABLES.get(key)
+    if hit is None or hit[0]() is not codebook:
+        for k in [k for k, v in _DEV_TABLES.items() if v[0]() is None]:
+            del _DEV_TABLES[k]
+        hit = _DEV_TABLES[key] = (weakref.ref(codebook), codebook.to(dev))
     return hit[1]
 
 
@@ -475,7 +510,7 @@ def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, i
     if sv.numel() != n_pad:
         raise RuntimeError(f"sv has {sv.numel()} entries, expected n_pad={n_pad}")
     ids = input_ids.reshape(-1).to(device=dev, dtype=torch.int64).contiguous()
-    t1 = _primary_table(_half_table(codebook.to(dev) if codebook.device != dev else codebook))
+    t1 = _primary_table(_half_table(_on_device(codebook, dev)))
     two = qidxs2 is not None and codebook2 is not None and inv_resid_scale is not None
     q2 = t2 = inv = None
     n2 = 0
@@ -484,7 +519,7 @@ def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, i
         if tuple(qidxs2.shape) != (vocab, nblk):
             raise RuntimeError(f"qidxs2 shape {tuple(qidxs2.shape)} != qidxs shape {(vocab, nblk)}")
         q2 = qidxs2
-        t2 = _packed_table(_half_table(codebook2.to(dev) if codebook2.device != dev else codebook2))
+        t2 = _packed_table(_half_table(_on_device(codebook2, dev)))
         n2 = t2.shape[0]
         inv = _per_row(inv_resid_scale.to(dev), vocab, "inv_resid_scale")
     ws = _per_row(wscale.to(dev), vocab, "wscale")

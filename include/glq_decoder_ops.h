@@ -29,6 +29,13 @@ int glqh_rmsnorm_bf16(const void *x, const void *w, void *out, int64_t T, int64_
 int glqh_add_rmsnorm_bf16(const void *x, const void *delta, const void *w, void *x_out, void *h_out,
                           int64_t T, int64_t H, double eps, void *stream);
 
+/* Positions live on the device (`pos`), so the host cannot check them: every kernel below that
+ * takes `pos` compares it with max_len itself.  Precondition: 0 <= pos[t] < max_len, and cos_t /
+ * sin_t hold at least max_len rows.  A position outside [0, max_len) makes the kernels skip that
+ * token entirely -- no cache row, no q_out / out row is written and nothing is read through the
+ * position -- instead of overrunning the caches or the score buffer; the caller's output rows
+ * then keep what they held before the call. */
+
 /* Rotate q (T, heads, D) and k (T, kv_heads, D) by the angle rows pos[t] of cos_t / sin_t
  * (max_len, D; halves (i, i + D/2) paired) when apply_rope != 0, write q to q_out and append
  * k, v to the caches (kv_heads, max_len, D) at positions pos[t]. */

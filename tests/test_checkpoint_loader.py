@@ -93,3 +93,33 @@ def test_loaded_layers_forward_like_the_reference(tmp_path, golden):
         x = torch.from_numpy(g[f"{tag}_x"]).half().to(DEV)
         y = lins[name](x)
         assert rel(y, g[f"{tag}_y"]) < 1e-2, (tag, rel(y, g[f"{tag}_y"]))
+
+
+def test_quantized_embedding_group_becomes_an_embedding_module(tmp_path, golden):
+    """A checkpoint with a quantized embedding beside its linears (Qidxs (vocab, n/8), per-row
+    Wscale, one-element SU) loads as E8RHTEmbedding instead of failing as a one-row linear; and
+    the 3-bpw secondary table is the first 256 rows of the full table, which is why one table
+    serves both stages."""
+    from glq_amd.quantized_linear import E8RHTEmbedding
+    from oracle import glq_oracle as O
+    g = golden("e8_layer")
+    rng = np.random.default_rng(0)
+    vocab, dim = 50, 64
+    tensors = {f"a.b.{leaf}": torch.from_numpy(np.asarray(g[f"bd4_{leaf}"]))
+               for leaf in ("Qidxs", "Qidxs2", "SU", "SV", "Wscale", "inv_resid_scale")}
+    tensors.update({
+        "model.embed_tokens.Qidxs": torch.from_numpy(rng.integers(-32768, 32768, (vocab, dim // 8)).astype(np.int16)),
+        "model.embed_tokens.SV": torch.ones(dim, dtype=torch.float16),
+        "model.embed_tokens.SU": torch.ones(1, dtype=torch.float16),
+        "model.embed_tokens.Wscale": torch.rand(vocab) + 0.5})
+    _write(str(tmp_path), tensors, {"quant_method": "glq", "codebook": "e8_shell", "block_diagonal": True,
+                                    "codesz": 8, "bpw": 4})
+    mods = C.load_quantized_linears(str(tmp_path), device="cpu")
+    emb = mods["model.embed_tokens"]
+    assert isinstance(emb, E8RHTEmbedding) and (emb.num_embeddings, emb.embedding_dim, emb.n_pad) == (vocab, dim, dim)
+    assert torch.equal(emb.Qidxs, tensors["model.embed_tokens.Qidxs"]) and emb.codebook is not None
+    assert float(emb.inv_resid_scale.abs().sum()) == 0.0           # single stage: residual keys absent
+    assert mods["a.b"].out_features == 96
+    table = O.e8_table()
+    norms = (table[:256] ** 2).sum(-1)
+    assert np.all(norms[1:] >= norms[:-1]) and norms[255] <= 4.0    # the low-norm prefix, in table order

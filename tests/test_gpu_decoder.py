@@ -220,3 +220,48 @@ def test_output_head_and_argmax(hidden, vocab):
     with pytest.raises(RuntimeError, match="hidden size"):
         check(lib.glqh_lm_head_argmax_bf16(hd.data_ptr(), Ed.data_ptr(), vocab, 1024, None, tok2.data_ptr(),
                                            ws.data_ptr(), ws.numel(), st))
+
+
+def test_positions_outside_the_cache_are_skipped_not_written():
+    """Device-side positions are compared with max_len inside the kernels: a position outside
+    [0, max_len) writes no cache row and no output row (the kernels return before any access
+    that depends on it), and generate() refuses a run that would pass the end of the cache."""
+    from glq_amd import _lib
+    say("decoder position guard")
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=DEV).manual_seed(4)
+    T, heads, kvh, hd, L = 3, 4, 2, 128, 16
+    q = torch.randn(T, heads, hd, generator=g, device=DEV).to(torch.bfloat16)
+    k = torch.randn(T, kvh, hd, generator=g, device=DEV).to(torch.bfloat16)
+    v = torch.randn(T, kvh, hd, generator=g, device=DEV).to(torch.bfloat16)
+    cos = torch.ones(L, hd, dtype=torch.bfloat16, device=DEV)
+    sin = torch.zeros(L, hd, dtype=torch.bfloat16, device=DEV)
+    kc = torch.full((kvh, L, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((kvh, L, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    qo = torch.full((T, heads, hd), 5.0, dtype=torch.bfloat16, device=DEV)
+    pos = torch.tensor([L, 2, -1], device=DEV)                 # first and last token out of range
+    _lib.check(lib.glqh_rope_kv_store_bf16(q.data_ptr(), k.data_ptr(), v.data_ptr(), pos.data_ptr(),
+                                           cos.data_ptr(), sin.data_ptr(), qo.data_ptr(), kc.data_ptr(),
+                                           vc.data_ptr(), T, heads, kvh, hd, L, 1, st))
+    assert torch.equal(qo[1], q[1]) and torch.all(qo[0] == 5.0) and torch.all(qo[2] == 5.0)
+    assert torch.equal(kc[:, 2], k[1]) and torch.equal(vc[:, 2], v[1])
+    keep = [i for i in range(L) if i != 2]
+    assert torch.all(kc[:, keep] == 7.0) and torch.all(vc[:, keep] == 7.0)
+    out = torch.full((heads, hd), 3.0, dtype=torch.bfloat16, device=DEV)
+    for bad in (L, L + 5, -1):
+        p1 = torch.tensor([bad], device=DEV)
+        _lib.check(lib.glqh_attn_decode_bf16(q[0].contiguous().data_ptr(), kc.data_ptr(), vc.data_ptr(),
+                                             p1.data_ptr(), out.data_ptr(), heads, kvh, hd, L, st))
+        assert torch.all(out == 3.0)
+    # the fused finishing launches: a decode step at pos == max_len leaves the caches untouched
+    dec = _small()
+    ids = torch.randint(0, 1000, (10,), generator=torch.Generator().manual_seed(2)).to(DEV)
+    dec.prefill(ids)
+    dec.pos.fill_(dec.max_len)
+    kc0, vc0 = dec.kc.clone(), dec.vc.clone()
+    dec._step()
+    torch.cuda.synchronize()
+    assert torch.equal(dec.kc, kc0) and torch.equal(dec.vc, vc0)
+    with pytest.raises(RuntimeError, match="exceed max_len"):
+        dec.generate(ids, dec.max_len, use_graph=False)

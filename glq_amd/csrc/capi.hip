@@ -16,6 +16,19 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
 int glqh_trellis_mma_init(void);
 int glqh_viterbi_init(void);
 
+// many-token E8 kernel on the compressed indices (e8_tile.hip)
+int glqh_e8_tile_init(void);
+int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages);
+size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M);
+int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
+                        const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
+                        int64_t n_pad, float *part, hipStream_t stream);
+// Above 16 tokens the weights are decoded once per 128 x 512 tile instead of once per 16 tokens.
+#define GLQH_E8_SMALL_BATCH 16
+static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages) {
+    return B > GLQH_E8_SMALL_BATCH ? glqh_e8_tile_ksplit(m_pad, n_pad, B, nstages) : 0;
+}
+
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
 int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const sv[], float *const part[],
                                    const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
@@ -104,7 +117,7 @@ extern "C" int glqh_init(void) {
             return;
         }
         g_cus = prop.multiProcessorCount;
-        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_trellis_init() || glqh_trellis_mma_init() || glqh_viterbi_init();
+        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_e8_tile_init() || glqh_trellis_init() || glqh_trellis_mma_init() || glqh_viterbi_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
     return g_init_rc;
@@ -764,6 +777,10 @@ static int e8_check_dims(int64_t m_pad, int64_t n_pad, int64_t B) {
 }
 
 static size_t e8_part_bytes(int64_t m_pad, int64_t n_pad, int64_t B) {
+    const int tks = e8_tile_ks(m_pad, n_pad, B, 1);              // stages are combined before the product; one or two
+                                                                 // stages get the most K slots
+    if (tks > 0)                                                 // + the repacked activations
+        return align256((size_t)tks * B * m_pad * sizeof(float)) + align256(glqh_e8_tile_xb_bytes(n_pad, B));
     int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
     return align256((size_t)ks * 4 * B * m_pad * sizeof(float));
 }
@@ -786,11 +803,22 @@ extern "C" int glqh_e8_dequant_matmul(const void *x_f16, int64_t B, const void *
     if (e8_check_dims(m_pad, n_pad, B) ||
         e8_resolve_stages(q1, q2, q3, q4, wscale, inv_rs, inv_rs2, inv_rs3, table1, table2, n_entries2, &sg))
         return 1;
+    hipStream_t st = (hipStream_t)stream;
+    float *part = (float *)ws;
+    const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n);
+    if (tks > 0) {
+        const size_t pbytes = align256((size_t)tks * B * m_pad * sizeof(float));
+        const size_t need = pbytes + glqh_e8_tile_xb_bytes(n_pad, B);
+        GLQH_REQUIRE(ws && ws_bytes >= need, "e8 matmul: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+        const float rel[3] = {(float)inv_rs, (float)inv_rs2, (float)inv_rs3};
+        if (glqh_launch_e8_tile(x_f16, (char *)ws + pbytes, B, sg.q, sg.n, table1, table2 ? table2 : table1, table2 ? n_entries2 : 65536,
+                                rel, m_pad, n_pad, part, st))
+            return 1;
+        return glqh_launch_reduce_splits(part, tks, B * m_pad, B, m_pad, (float)wscale, out, m_pad, 0, st);
+    }
     const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
     const size_t need = (size_t)ks * sg.n * B * m_pad * sizeof(float);
     GLQH_REQUIRE(ws && ws_bytes >= need, "e8 matmul: workspace of %zu bytes needed, got %zu", need, ws_bytes);
-    hipStream_t st = (hipStream_t)stream;
-    float *part = (float *)ws;
     if (glqh_launch_e8_partial(x_f16, B, sg.q, sg.n, table1, table2 ? table2 : table1,
                                table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st))
         return 1;
@@ -857,8 +885,11 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
     GLQH_REQUIRE(B <= 65535, "fused e8 linear: B=%lld out of range", (long long)B);
     GLQH_REQUIRE(in_features <= n_pad && out_features <= m_pad, "fused e8 linear: features exceed padded dims");
     const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
-    const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
-    const size_t need = xb + (size_t)ks * sg.n * B * m_pad * sizeof(float);
+    const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n);
+    const int ks = tks > 0 ? tks : glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    const size_t tile_part = align256((size_t)ks * B * m_pad * sizeof(float));
+    const size_t need = tks > 0 ? xb + tile_part + glqh_e8_tile_xb_bytes(n_pad, B)
+                                : xb + (size_t)ks * sg.n * B * m_pad * sizeof(float);
     GLQH_REQUIRE(ws && ws_bytes >= need, "fused e8 linear: workspace of %zu bytes needed, got %zu", need,
                  ws_bytes);
     hipStream_t st = (hipStream_t)stream;
@@ -867,6 +898,22 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
     if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
                               bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
         return 1;
+    if (tks > 0) {
+        // many tokens: one combined product on the compressed indices, summed over its K slots and
+        // scaled by the output transform
+        const float rel[3] = {(float)inv_rs, (float)inv_rs2, (float)inv_rs3};
+        if (glqh_launch_e8_tile(x_rht, (char *)ws + xb + tile_part, B, sg.q, sg.n, table1, table2 ? table2 : table1, table2 ? n_entries2 : 65536,
+                                rel, m_pad, n_pad, part, st))
+            return 1;
+        glqh_ysrc src = {};
+        src.nparts = 1;
+        src.scale[0] = (float)wscale;
+        src.part = part;
+        src.part_kstride = B * m_pad;
+        src.ksplit = tks;
+        return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,
+                                      blocks_m, n_blocks_m, 0, 0.0f, st);
+    }
     // Canonical output blocks at up to 16 tokens: every stage's partial sums are written already
     // multiplied by that stage's scale, which makes them ks * stages plain slots for the slice
     // kernels of the grouped launcher (faster than the generic multi-part transform).

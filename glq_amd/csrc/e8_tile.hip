@@ -1,0 +1,453 @@
+// E8 shell codebook GEMM for many tokens on the compressed indices (gfx950, wave64).
+//
+// Y_rht[token, row] = sum_k X_rht[token, k] * W[row, k] with W[row, 8j..8j+7] = cb[q1[row, j]]
+// + r2 * cb2[q2[row, j]] + ... (glq/codebook.py:280-282, glq/quantized_linear.py:1177-1194;
+// the reference's tensor-core kernel for B >= 2 is glq/csrc/glq_cuda.cu:791-955).  Looking an
+// index up and expanding its eight 4-bit codes costs far more than the eight multiply-adds of
+// one token, so a decoded weight has to meet as many tokens as possible:
+//
+//   workgroup tile = 128 rows x (128 * NTW) tokens, 8 waves (two per SIMD);
+//   wave w DECODES row fragment w (16 rows) of every 64-column step into LDS, in the operand
+//   layout of v_mfma_f32_16x16x32_f16 (lane L's 16 bytes at slot L: conflict-free both ways),
+//   and MULTIPLIES all 8 row fragments, read back from LDS, with ITS OWN 16 * NTW tokens, whose
+//   activations it holds in registers, straight from global memory.
+//
+// The B operand of the MFMA puts consecutive tokens in consecutive lanes, so row-major activations
+// would be read as 64 scattered 16-byte pieces per instruction (one lane per clock in the memory
+// pipeline: measured 2.7 us per 64-column step and CU, three times the multiplications).  They are
+// repacked once per call into 8-column blocks with the token as the fast index,
+// xb[k / 8][token][k % 8], which turns every operand load into four runs of 256 contiguous bytes.
+//
+// Every weight is therefore looked up once per 128 * NTW tokens (once per 512 at NTW = 4), the
+// B operands never pass through LDS, and LDS carries 16 KB of A operands per step and CU.  The
+// table's low-norm prefix (32768 entries, 128 KB) lives in LDS as in the small-batch kernel
+// (e8_mma.hip); the tail is read from L2.  Stages are combined into one fp16 operand per stage
+// in sequence, a = fma(c_s, r_s, a) in fp16 (the reference rounds to fp16 after every stage as
+// well, glq/csrc/glq_cuda.cu:868-899).  Workgroups are persistent (one per CU) and walk tiles in
+// an order that gives the CUs of one XCD the same tokens at the same time, so the activations
+// are served by that XCD's L2.  K is split into slots only while the tiles alone would leave CUs
+// idle; partial sums [slot][token][row] are combined in slot order by the consumer.
+#include "e8_device.h"
+
+namespace {
+
+constexpr int ET_WAVES = 8;
+constexpr int ET_THREADS = ET_WAVES * GLQH_WAVE;
+constexpr int ET_FRAGS = 8;                        // 16-row fragments per tile, one per wave
+constexpr int ET_ROWS = 16 * ET_FRAGS;
+constexpr int ET_P = 32767;                        // table entries kept in LDS; word ET_P is a sentinel
+constexpr uint32_t ET_MISS = 0xFFFFFFFFu;          // no table word has a code above 12
+constexpr int ET_BUF = 2 * ET_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer: 2 sub-steps x 8 fragments
+constexpr size_t ET_LDS = (size_t)(ET_P + 1) * 4 + (size_t)2 * ET_BUF * 16;   // 128 KB + 32 KB
+
+struct et_args {
+    const uint16_t *q[4];
+    const uint32_t *t1, *t2;
+    uint32_t n2;
+    int t2_is_t1;
+    float r[3];                                    // factors of stages 2..4 relative to stage 1
+    const f16 *xb;                                 // transformed activations, (n_pad / 8, Mp, 8) fp16
+    int Mp;                                        // M rounded up to whole token tiles
+    int M, m_pad, n_pad;
+    int RT, TT, KS, slot_ds;                       // row tiles, token tiles, K slots, 64-column steps per slot
+    float *part;                                   // [slot][token][row]
+};
+
+__device__ __forceinline__ void et_barrier() {     // waits for LDS only: global prefetches stay in flight
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int NS, int NTW>
+__global__ void __launch_bounds__(ET_THREADS)
+e8_tile_kernel(const et_args a) {
+    extern __shared__ u32x4 lds[];
+    const uint32_t *tab = (const uint32_t *)lds;
+    u32x4 *abuf = lds + (ET_P + 1) / 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int nblk = a.n_pad >> 3, nds = a.n_pad >> 6;
+
+    // table prefix -> LDS, all loads of a round in flight before its first write
+    {
+        constexpr int PER = (ET_P + 1) / 4 / ET_THREADS;       // 16 x 16 bytes per thread
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            u32x4 v[PER / 2];
+#pragma unroll
+            for (int u = 0; u < PER / 2; ++u) v[u] = ((const u32x4 *)a.t1)[(h * (PER / 2) + u) * ET_THREADS + threadIdx.x];
+#pragma unroll
+            for (int u = 0; u < PER / 2; ++u) lds[(h * (PER / 2) + u) * ET_THREADS + threadIdx.x] = v[u];
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) ((uint32_t *)lds)[ET_P] = ET_MISS;   // what a lookup past the prefix reads
+    __syncthreads();
+
+    // a separate stage-2 table stays in L2: its LDS lookups are all sent to the sentinel
+    const uint32_t P2 = a.t2_is_t1 ? (uint32_t)ET_P : 0u, force2 = a.t2_is_t1 ? 0u : 0xFFFFu;
+    f16x2 rs[3];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) rs[s] = f16x2{(f16)a.r[s], (f16)a.r[s]};
+
+    // Workgroups with equal blockIdx % 8 run on one XCD and share its L2: each XCD takes a
+    // contiguous range of the item list, whose fastest index is the row tile, so its CUs read
+    // the same activations at the same time.
+    const int nitems = a.TT * a.KS * a.RT;
+    const int per_xcd = (nitems + 7) >> 3;
+    const int xcd = blockIdx.x & 7, bx = blockIdx.x >> 3;
+    const int nbx = ((int)gridDim.x - xcd + 7) >> 3;
+    for (int w = bx; w < per_xcd; w += nbx) {
+        const int item = xcd * per_xcd + w;
+        if (item >= nitems) break;                              // uniform
+        const int rt = item % a.RT, slot = (item / a.RT) % a.KS, tt0 = item / (a.RT * a.KS);
+        const int r0 = rt * ET_ROWS, tok0 = tt0 * (ET_WAVES * 16 * NTW) + wave * 16 * NTW;
+        const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
+
+        // decode role: row fragment `wave`; lane (i, g) owns blocks 8d + 2g, 8d + 2g + 1 of step d
+        const int drow = min(r0 + 16 * wave + i, a.m_pad - 1);
+        const u32x4 *qrow[NS];                                  // 8 indices = the 64 columns of step 4q + g
+#pragma unroll
+        for (int s = 0; s < NS; ++s) qrow[s] = (const u32x4 *)(a.q[s] + (int64_t)drow * nblk) + (ds0 >> 2) * 4 + g;
+        // multiply role: token 16 * tt + i of the wave's tokens, blocks 8d + 2g and 8d + 2g + 1
+        // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
+        const int64_t bstep = (int64_t)a.Mp * 8;                // elements from one block to the next
+        const f16 *xrow = a.xb + (int64_t)(tok0 + i) * 8 + 2 * g * bstep;
+
+        // Every load below is unconditional with a clamped step index, so the wait counts the
+        // compiler derives are exact and nothing waits for a request younger than the one it needs.
+        // The L2 words of a step are requested LA steps before its operands are expanded (hits aim
+        // their load at one shared entry); the LDS words are read at expansion time from the index
+        // pairs, which travel with the L2 words (misses read the sentinel).
+        struct looked {
+            uint32_t wg[NS][2], pair[NS];
+        };
+        auto index_of = [&](uint32_t pair, int s, int u) {
+            uint32_t idx = (pair >> (16 * u)) & 0xFFFFu;
+            if (s == 1) idx = min(idx, a.n2 - 1);
+            return idx;
+        };
+        auto lookups = [&](const uint32_t (&T)[NS][4], int dd) {
+            looked r;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                r.pair[s] = T[s][dd];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t *tg = s == 1 ? a.t2 : a.t1;
+                    const uint32_t pre = s == 1 ? P2 : (uint32_t)ET_P;
+                    r.wg[s][u] = tg[max(index_of(r.pair[s], s, u), pre)];
+                }
+            }
+            return r;
+        };
+        struct lds_words {
+            uint32_t w[NS][2];
+        };
+        auto lds_lookups = [&](const looked &r) {
+            lds_words wl;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t idx = index_of(r.pair[s], s, u);
+                    wl.w[s][u] = tab[min(s == 1 ? idx | force2 : idx, (uint32_t)ET_P)];
+                }
+            return wl;
+        };
+        auto expand_half = [&](const looked &r, const lds_words &wlw, int u, u32x4 *dst) {   // one A fragment
+            const auto &wl = wlw.w;
+            {
+                f16x8 af = em_expand(wl[0][u] != ET_MISS ? wl[0][u] : r.wg[0][u]);
+#pragma unroll
+                for (int s = 1; s < NS; ++s) {
+                    const f16x8 e = em_expand(wl[s][u] != ET_MISS ? wl[s][u] : r.wg[s][u]);
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const f16x2 ev = {e[2 * p], e[2 * p + 1]}, av = {af[2 * p], af[2 * p + 1]};
+                        const f16x2 rv = __builtin_elementwise_fma(ev, rs[s - 1], av);
+                        af[2 * p] = rv[0];
+                        af[2 * p + 1] = rv[1];
+                    }
+                }
+                dst[(u * ET_FRAGS + wave) * GLQH_WAVE + lane] = __builtin_bit_cast(u32x4, af);
+            }
+        };
+        auto emit = [&](const looked &r, u32x4 *dst) {          // two A fragments of this wave's rows
+            const lds_words wl = lds_lookups(r);
+            expand_half(r, wl, 0, dst);
+            expand_half(r, wl, 1, dst);
+        };
+        // Index runs are requested 16 bytes per lane, a whole group of four steps ahead of their
+        // use.  Lane (i, g) receives the 8 indices of step 4q + g of its row, but in step 4q + dd
+        // it decodes index pair g of that step: a 4 x 4 transpose of dwords over the four lanes
+        // that share row i (lane distance 16), done with two pairs of lane-swap instructions.
+        const int nquads = (ds1 - ds0) >> 2;
+        auto load_quad = [&](u32x4 (&run)[NS], int q) {
+            q = min(q, nquads - 1);
+#pragma unroll
+            for (int s = 0; s < NS; ++s) run[s] = __builtin_nontemporal_load(qrow[s] + 4 * q);
+        };
+        auto transpose = [&](const u32x4 (&run)[NS], uint32_t (&T)[NS][4]) {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const auto p02 = __builtin_amdgcn_permlane32_swap(run[s][0], run[s][2], false, false);
+                const auto p13 = __builtin_amdgcn_permlane32_swap(run[s][1], run[s][3], false, false);
+                const auto lo = __builtin_amdgcn_permlane16_swap(p02[0], p13[0], false, false);
+                const auto hi = __builtin_amdgcn_permlane16_swap(p02[1], p13[1], false, false);
+                T[s][0] = lo[0];
+                T[s][1] = lo[1];
+                T[s][2] = hi[0];
+                T[s][3] = hi[1];
+            }
+        };
+        auto load_b = [&](u32x4 (&b)[NTW][2], int d) {
+            d = min(d, ds1 - 1);
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) {
+                b[tt][0] = *(const u32x4 *)(xrow + 8 * d * bstep + tt * 128);
+                b[tt][1] = *(const u32x4 *)(xrow + (8 * d + 1) * bstep + tt * 128);
+            }
+        };
+
+        f32x4 acc[ET_FRAGS][NTW];
+#pragma unroll
+        for (int f = 0; f < ET_FRAGS; ++f)
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) acc[f][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        // Software pipeline over the 64-column steps.  At step d: the operands of d + 1 are expanded
+        // into the other LDS buffer from table entries requested LA steps earlier, the entries of
+        // d + 1 + LA are requested, and the activations of d + 1 are requested -- a whole step ahead
+        // into a second register set where registers allow (NTW <= 2), otherwise half a step ahead
+        // into the registers the half-step just multiplied has freed.  Index runs arrive a group of
+        // four steps ahead.
+        constexpr int LA = NTW <= 2 ? 2 : 1;
+        constexpr bool BDB = NTW <= 2;
+        u32x4 run[NS];
+        uint32_t T[NS][4];
+        u32x4 b[BDB ? 2 : 1][NTW][2];
+        looked lk[LA];
+        load_quad(run, 0);
+        load_b(b[0], ds0);
+        transpose(run, T);
+        load_quad(run, 1);
+        {
+            const looked first = lookups(T, 0);
+            emit(first, abuf);
+        }
+        static_assert(LA <= 3, "the prologue requests entries from the first index group only");
+#pragma unroll
+        for (int j = 1; j <= LA; ++j) lk[j % LA] = lookups(T, j & 3);
+        et_barrier();
+
+        for (int q = 0; q < nquads; ++q) {
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                const int d = ds0 + 4 * q + dd;
+                const int cur = BDB ? (dd & 1) : 0, nxt = BDB ? (cur ^ 1) : 0;
+                const u32x4 *rd = abuf + (dd & 1) * ET_BUF;
+                u32x4 *wr = abuf + ((dd & 1) ^ 1) * ET_BUF;
+                const int dn = min(d + 1, ds1 - 1);
+                if constexpr (BDB) load_b(b[nxt], d + 1);
+                const looked &lke = lk[(dd + 1) % LA];          // entries of d + 1: expanded during this step
+                const lds_words wle = lds_lookups(lke);
+                const looked lkn = [&] {
+                    const int sl = dd + 1 + LA;                 // step looked up now, relative to 4q
+                    if ((sl & 3) == 0) {                        // its group's indices take over
+                        transpose(run, T);
+                        load_quad(run, q + (sl >> 2) + 1);
+                    }
+                    return lookups(T, sl & 3);
+                }();
+                // 16 operand fragments (2 half-steps x 8 row fragments), each read from LDS one
+                // fragment ahead of the multiplications that use it; the expansion of the next
+                // step's operands is spread between them
+                f16x8 afn = __builtin_bit_cast(f16x8, rd[lane]);
+                __builtin_amdgcn_sched_barrier(0);              // requests stay ahead of the multiplications
+#pragma unroll
+                for (int k = 0; k < 2 * ET_FRAGS; ++k) {
+                    const int u = k / ET_FRAGS, f = k % ET_FRAGS;
+                    const f16x8 af = afn;
+                    if (k + 1 < 2 * ET_FRAGS) afn = __builtin_bit_cast(f16x8, rd[(k + 1) * GLQH_WAVE + lane]);
+#pragma unroll
+                    for (int tt = 0; tt < NTW; ++tt)
+                        acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            af, __builtin_bit_cast(f16x8, b[cur][tt][u]), acc[f][tt], 0, 0, 0);
+                    if (k == 1) expand_half(lke, wle, 0, wr);   // operands of d + 1 (unused after the last step)
+                    if (k == 9) expand_half(lke, wle, 1, wr);
+                    if constexpr (!BDB) {
+                        if (f == ET_FRAGS - 1) {                // this half's activations are free: request the next
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + (8 * dn + u) * bstep + tt * 128);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+                lk[(dd + 1) % LA] = lkn;
+                et_barrier();                                   // rd has been read, wr is written
+            }
+        }
+
+        // lane holds rows 4g .. 4g+3 of token i of every (fragment, token tile)
+        const bool vec = (a.m_pad & 3) == 0;
+#pragma unroll
+        for (int tt = 0; tt < NTW; ++tt) {
+            const int tok = tok0 + 16 * tt + i;
+            if (tok >= a.M) continue;
+            float *orow = a.part + ((int64_t)slot * a.M + tok) * a.m_pad;
+#pragma unroll
+            for (int f = 0; f < ET_FRAGS; ++f) {
+                const int row = r0 + 16 * f + 4 * g;
+                if (vec && row + 3 < a.m_pad) {
+                    *(f32x4 *)(orow + row) = acc[f][tt];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (row + e < a.m_pad) orow[row + e] = acc[f][tt][e];
+                }
+            }
+        }
+    }
+}
+
+// (M, n_pad) row-major fp16 -> (n_pad / 8, M, 8): 64 tokens x 16 blocks per workgroup through LDS,
+// both sides in runs of 256 bytes and more.
+__global__ void __launch_bounds__(256)
+e8_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, int Mp, int n_pad) {
+    __shared__ u32x4 tile[16][65];
+    const int tok0 = blockIdx.x * 64, kb0 = blockIdx.y * 16, nblk = n_pad >> 3;
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int tl = r * 16 + (t >> 4), kb = t & 15;
+        const int tok = min(tok0 + tl, M - 1), b = min(kb0 + kb, nblk - 1);
+        tile[kb][tl] = *(const u32x4 *)(x + (int64_t)tok * n_pad + 8 * b);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int kb = r * 4 + (t >> 6), tl = t & 63;
+        if (tok0 + tl < M && kb0 + kb < nblk) *(u32x4 *)(xb + ((int64_t)(kb0 + kb) * Mp + tok0 + tl) * 8) = tile[kb][tl];
+    }
+}
+
+// token tiles per wave: 512-token workgroup tiles from 257 tokens on; layers of three and four stages
+// stay at 256 (the registers of their longer lookup pipeline)
+static int et_ntw(int64_t M, int nstages) { return M <= 128 ? 1 : (M <= 256 || nstages > 2) ? 2 : 4; }
+
+static int64_t et_padded_tokens(int64_t M, int nstages) {
+    const int64_t tile = ET_WAVES * 16 * et_ntw(M, nstages);
+    return (M + tile - 1) / tile * tile;
+}
+
+struct et_plan {
+    int NTW, RT, TT, KS, slot_ds, grid;
+};
+
+int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *p) {
+    if (M < 1 || m_pad < 1 || n_pad < 256 || (n_pad & 255) || M > ((int64_t)1 << 22) || m_pad > ((int64_t)1 << 24))
+        return 0;
+    p->NTW = et_ntw(M, nstages);
+    const int tile_tok = ET_WAVES * 16 * p->NTW;
+    p->RT = (int)((m_pad + ET_ROWS - 1) / ET_ROWS);
+    p->TT = (int)((M + tile_tok - 1) / tile_tok);
+    const int nds = (int)(n_pad / 64);
+    const int cus = glqh_device_cus();
+    const int64_t base = (int64_t)p->RT * p->TT;
+    int64_t ks = 1;
+    if (base < cus) {
+        ks = cus / base;
+        const int64_t cap_len = nds / 8 > 0 ? nds / 8 : 1;      // slots of at least 512 columns
+        if (ks > cap_len) ks = cap_len;
+        // partial sums stay under 128 MB
+        const int64_t cap_bytes = ((int64_t)128 << 20) / (M * m_pad * 4);
+        if (ks > cap_bytes) ks = cap_bytes;
+        if (ks < 1) ks = 1;
+    }
+    p->slot_ds = (int)((nds / 4 + ks - 1) / ks) * 4;            // whole groups of four steps
+    p->KS = (nds + p->slot_ds - 1) / p->slot_ds;
+    const int64_t items = base * p->KS;
+    p->grid = (int)(items < cus ? items : cus);
+    return 1;
+}
+
+template <int NS, int NTW>
+int et_launch(const et_plan &p, const et_args &a, hipStream_t stream) {
+    hipLaunchKernelGGL((e8_tile_kernel<NS, NTW>), dim3((unsigned)p.grid), dim3(ET_THREADS), ET_LDS, stream, a);
+    GLQH_LAUNCH_CHECK("e8 tile launch");
+    return 0;
+}
+
+template <int NS>
+int et_launch_NS(const et_plan &p, const et_args &a, hipStream_t stream) {
+    if (p.NTW == 1) return et_launch<NS, 1>(p, a, stream);
+    if (p.NTW == 2) return et_launch<NS, 2>(p, a, stream);
+    if constexpr (NS <= 2) return et_launch<NS, 4>(p, a, stream);
+    return glqh_fail("e8 tile kernel: no 512-token tiles for %d stages", NS);
+}
+
+template <typename K>
+int et_set_lds(K kernel) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)ET_LDS),
+                          "e8 tile attribute");
+}
+
+template <int NS>
+int et_init_NS() {
+    if (et_set_lds(e8_tile_kernel<NS, 1>) || et_set_lds(e8_tile_kernel<NS, 2>)) return 1;
+    if constexpr (NS <= 2) return et_set_lds(e8_tile_kernel<NS, 4>);
+    return 0;
+}
+
+}  // namespace
+
+int glqh_e8_tile_init(void) { return et_init_NS<1>() || et_init_NS<2>() || et_init_NS<3>() || et_init_NS<4>(); }
+
+// bytes of the repacked activations (the larger tile size bounds the padding)
+size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M) { return (size_t)et_padded_tokens(M, 1) * n_pad * sizeof(f16); }
+
+// K slots of the many-token kernel for this call, or 0 when the shape is not eligible
+// (n_pad must be a multiple of 256)
+int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages) {
+    et_plan p;
+    return et_make_plan(m_pad, n_pad, M, nstages, &p) ? p.KS : 0;
+}
+
+// part[(slot * M + token) * m_pad + row] = sum over the slot's columns of x[token, k] * W[row, k],
+// W = cb[q0] + rel[0] * cb2[q1] + rel[1] * cb[q2] + rel[2] * cb[q3] (nstages terms), unscaled.
+// x_f16 is (M, n_pad) row-major; xb_scratch takes its repacked copy (glqh_e8_tile_xb_bytes).
+int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
+                        const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
+                        int64_t n_pad, float *part, hipStream_t stream) {
+    et_plan p;
+    if (!et_make_plan(m_pad, n_pad, M, nstages, &p)) return glqh_fail("e8 tile kernel: shape not eligible (n_pad %% 256)");
+    hipLaunchKernelGGL(e8_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((n_pad / 8 + 15) / 16)),
+                       dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, (int)et_padded_tokens(M, nstages), (int)n_pad);
+    GLQH_LAUNCH_CHECK("e8 pack launch");
+    et_args a;
+    for (int s = 0; s < 4; ++s) a.q[s] = (const uint16_t *)q[s];
+    a.t1 = t1;
+    a.t2 = t2;
+    a.n2 = (uint32_t)n2;
+    a.t2_is_t1 = (t1 == t2 && n2 == 65536);
+    for (int s = 0; s < 3; ++s) a.r[s] = rel[s];
+    a.xb = (const f16 *)xb_scratch;
+    a.M = (int)M;
+    a.Mp = (int)et_padded_tokens(M, nstages);
+    a.m_pad = (int)m_pad;
+    a.n_pad = (int)n_pad;
+    a.RT = p.RT;
+    a.TT = p.TT;
+    a.KS = p.KS;
+    a.slot_ds = p.slot_ds;
+    a.part = part;
+    switch (nstages) {
+    case 1: return et_launch_NS<1>(p, a, stream);
+    case 2: return et_launch_NS<2>(p, a, stream);
+    case 3: return et_launch_NS<3>(p, a, stream);
+    case 4: return et_launch_NS<4>(p, a, stream);
+    }
+    return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
+}

@@ -33,7 +33,16 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 # 4096 <-> 14336: 66 vs 95 us at 128 tokens, 96 vs 113 us at 256, 241 vs 197 us at 1024), so
 # the default trellis threshold is 512.
 TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "512")))
-E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "16")))
+# E8 layers stay on their compressed indices at every token count (above 16 tokens: one lookup per
+# weight and 128 x 512 tile, csrc/e8_tile.hip); GLQ_E8_BATCH_MAX=<n> sends calls above n tokens to
+# the dense route instead.
+E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", str(1 << 30))))
+
+
+def _e8_dense_route(B, n_pad):
+    """Dequantize + library GEMM: on request, and for the widths the tile kernel does not take
+    (n_pad not a multiple of 256) above 16 tokens."""
+    return B > E8_BATCH_MAX or (B > 16 and int(n_pad) % 256 != 0)
 
 
 def _p(t):
@@ -584,7 +593,7 @@ def _e8_matmul_tables(x, qidxs, t1, q2, t2, n2, q3, q4, wscale, inv_rs, inv_rs2,
     M, nblk = qidxs.shape
     if x.shape[1] != nblk * 8:
         raise RuntimeError(f"x has {x.shape[1]} columns, qidxs implies {nblk * 8}")
-    if B > E8_BATCH_MAX:
+    if _e8_dense_route(B, nblk * 8):
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
         return torch.mm(x, W.t(), out_dtype=torch.float32).mul_(float(wscale))
     out = torch.empty((B, M), dtype=torch.float32, device=x.device)
@@ -673,7 +682,7 @@ def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_p
     bn, nbn = _host_i64(blocks_n)
     bm, nbm = _host_i64(blocks_m)
     y = torch.empty((B, int(out_features)), dtype=out_dtype or torch.float16, device=x.device)
-    if B > E8_BATCH_MAX:
+    if _e8_dense_route(B, n_pad):
         x_rht = torch.empty((B, int(n_pad)), dtype=torch.float16, device=x.device)
         glq_input_rht_blockdiag_cuda(x, sv, x_rht, in_features, n_pad, blocks_n, bn_meta)
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)

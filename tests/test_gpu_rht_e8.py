@@ -168,8 +168,9 @@ def test_large_transform_op_names(ext):
                                           (2048, 2048, 40, 2), (1024, 4160, 33, 4), (2100, 2048, 17, 1)])
 def test_e8_large_layers_lds_table(ext, m, n, B, stages):
     """Layers of 4M weights and more: the table prefix sits in LDS, the tail comes from L2.
-    Up to 16 tokens the products run on MFMA straight from the indices; above, the weight is
-    dequantized once (same LDS table) for a library GEMM.  Half of the indices are drawn from
+    Up to 16 tokens the products run on MFMA straight from the indices; above, the tile kernel
+    decodes them once per 128-row x 512-token tile (widths that are multiples of 256; others are
+    dequantized once for a library GEMM).  Half of the indices are drawn from
     the low shells, half uniformly, and the extremes are planted."""
     say("e8 large", m, n, B, stages)
     rng = np.random.default_rng(m + n + B)
@@ -205,9 +206,38 @@ def test_e8_large_layer_small_secondary_table(ext):
     W = O.e8_dequant(q1, q2, 0.5)
     out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
     assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
-    x = rng.standard_normal((24, n)).astype(np.float16)          # many tokens: dequantize + GEMM
+    x = rng.standard_normal((24, n)).astype(np.float16)          # many tokens: tile kernel, second table from L2
     out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
     assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
+
+
+@pytest.mark.parametrize("m,n,stages", [(100, 512, 1), (300, 768, 2), (128, 1024, 3), (200, 256, 4)])
+def test_e8_many_token_tile_kernel_edges(ext, m, n, stages):
+    """The kernel that keeps E8 layers compressed above 16 tokens: token counts on both sides of
+    its 128 / 256 / 512-token tiles, row counts that end inside a 16-row fragment, 1-4 stages,
+    against the oracle; rows of a larger call equal the rows of a smaller one up to the K split."""
+    say("e8 tile edges", m, n, stages)
+    rng = np.random.default_rng(m + stages)
+    cb = e8_table_f16()
+    q = [_rand_idx(rng, m, n // 8) for _ in range(4)]
+    q[0][0, 0], q[0][0, 1], q[0][m - 1, n // 8 - 1] = 0, -1, -1
+    sc = [0.0, 0.0, 0.0]
+    for s in range(1, stages):
+        sc[s - 1] = [1 / 3.0, 1 / 9.0, 1 / 27.0][s - 1]
+    W = O.e8_dequant(q[0], q[1], sc[0], q[2], sc[1], q[3], sc[2])
+    args = (t(q[0]), cb, 0.021, t(q[1]), cb, sc[0], None, t(q[2]), cb, sc[1], t(q[3]), cb, sc[2])
+    xs = (rng.standard_normal((600, n)) * 0.5).astype(np.float16)
+    ref = xs.astype(np.float32) @ W.T * np.float32(0.021)
+    outs = {}
+    for B in (17, 128, 129, 256, 257, 513, 600):
+        out = ext.glq_dequant_matmul_cuda(t(xs[:B]), *args)
+        assert out.shape == (B, m)
+        # fp16 operands combined stage by stage: each stage adds one fp16 rounding of the weight
+        assert rel(out, ref[:B]) < 1.5e-3, (B, rel(out, ref[:B]))
+        assert torch.equal(out, ext.glq_dequant_matmul_cuda(t(xs[:B]), *args))
+        outs[B] = out
+    assert rel(outs[600][:129], outs[129].cpu().numpy()) < 1e-5
+    assert rel(outs[257][:17], outs[17].cpu().numpy()) < 1e-5
 
 
 def test_e8_small_secondary_table(ext):

@@ -48,33 +48,43 @@ static int tr_fusein_plan(const int64_t *m_pads, int n, int64_t n_pad, int64_t B
     if (wgs >= GLQH_FUSEIN_MMA_MIN_STRIPS) return glqh_trellis_mma_fusein_plan(wgs, n_pad, B, S, ks) ? 2 : 0;
     return glqh_trellis_fusein_plan(total, n_pad, B, S, ks) ? 1 : 0;
 }
-int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out);
-int glqh_launch_trellis_prefill(const void *x_f16, int64_t M, const void *packed, int R, int64_t m, int64_t k,
-                                int S, int ksplit, float *out, int direct, float scale, int accum,
-                                int64_t out_stride, hipStream_t stream);
+// many-token kernel (trellis_tile.hip): weights decoded once per 128-row x 512-token tile
+size_t glqh_trellis_tile_xb_bytes(int64_t k, int64_t M);
+int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M);
+int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
+                             int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
+                             hipStream_t stream);
 
 // Plan for activations already in the transformed domain: up to 64 tokens share one pass
-// over the packed stream with K split by shape only; larger batches use 128-token tiles.
+// over the packed stream with K split by shape only; larger batches use the tile kernel, which
+// needs scratch for its repacked activations (xb_bytes).
 #define GLQH_TRELLIS_SMALL_BATCH 64
 struct tr_plan {
-    int ks, S, prefill;
+    int ks, S, tile;
+    size_t xb_bytes;
 };
 static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
-    tr_plan p = {1, 0, B > GLQH_TRELLIS_SMALL_BATCH};
-    if (p.prefill) glqh_trellis_prefill_plan(m, k, B, &p.S, &p.ks);
-    else glqh_trellis_mma_plan(m, k, &p.S, &p.ks);
+    tr_plan p = {1, 0, B > GLQH_TRELLIS_SMALL_BATCH, 0};
+    if (p.tile) {
+        p.ks = glqh_trellis_tile_ksplit(m, k, B);
+        p.xb_bytes = (glqh_trellis_tile_xb_bytes(k, B) + 255) & ~(size_t)255;
+    } else {
+        glqh_trellis_mma_plan(m, k, &p.S, &p.ks);
+    }
     return p;
 }
 // pscale multiplies the partial sums as they are written (small-batch kernel only): a second
-// stage stored pre-scaled is just more K slots to whoever sums them.
+// stage stored pre-scaled is just more K slots to whoever sums them.  xb: scratch of
+// plan.xb_bytes for the tile kernel (unused otherwise).
 static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                            int64_t k, float *part, hipStream_t st, float pscale = 1.0f) {
-    if (p.prefill) return glqh_launch_trellis_prefill(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, 1.0f, 0, 0, st);
+                            int64_t k, float *part, void *xb, hipStream_t st, float pscale = 1.0f) {
+    if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, part, 0, 1.0f, 0, 0, st);
     return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, pscale, 0, 0, st);
 }
 static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                           int64_t k, float scale, float *out, int64_t out_stride, int accum, hipStream_t st) {
-    if (p.prefill) return glqh_launch_trellis_prefill(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
+                           int64_t k, float scale, float *out, int64_t out_stride, int accum, void *xb,
+                           hipStream_t st) {
+    if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, out, 1, scale, accum, out_stride, st);
     return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
 }
 
@@ -167,8 +177,9 @@ extern "C" int glqh_decompress_trellis_3inst(const void *packed, int64_t packed_
 extern "C" size_t glqh_trellis_gemv_workspace_bytes(int64_t m, int64_t k, int64_t B) {
     if (!glqh_trellis_kernel_supported(m, k) || B < 1) return 0;
     glqh_init();
-    int ks = tr_plain_plan(m, k, B).ks;
-    return ks > 1 ? align256((size_t)ks * B * m * sizeof(float)) : 0;
+    const tr_plan p = tr_plain_plan(m, k, B);
+    // (the many-token kernel's figure also serves glqh_trellis_gemv_partials, which always stores the sums)
+    return (p.ks > 1 || p.tile ? align256((size_t)p.ks * B * m * sizeof(float)) : 0) + p.xb_bytes;
 }
 
 extern "C" int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B, const void *packed,
@@ -185,12 +196,14 @@ extern "C" int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B, co
     hipStream_t st = (hipStream_t)stream;
     const tr_plan plan = tr_plain_plan(m, k, B);
     const int ks = plan.ks;
+    const size_t pbytes = ks > 1 ? align256((size_t)ks * B * m * sizeof(float)) : 0;
+    const size_t need = pbytes + plan.xb_bytes;
+    GLQH_REQUIRE(need == 0 || (ws && ws_bytes >= need), "trellis matmul: workspace of %zu bytes needed, got %zu",
+                 need, ws_bytes);
+    void *xb = (char *)ws + pbytes;
     if (ks == 1)
-        return tr_plain_direct(plan, x_f16, B, packed, R, m, k, (float)wscale, out, out_stride, accum, st);
-    size_t need = (size_t)ks * B * m * sizeof(float);
-    GLQH_REQUIRE(ws && ws_bytes >= need, "trellis matmul: workspace of %zu bytes needed, got %zu", need,
-                 ws_bytes);
-    if (tr_plain_partial(plan, x_f16, B, packed, R, m, k, (float *)ws, st)) return 1;
+        return tr_plain_direct(plan, x_f16, B, packed, R, m, k, (float)wscale, out, out_stride, accum, xb, st);
+    if (tr_plain_partial(plan, x_f16, B, packed, R, m, k, (float *)ws, xb, st)) return 1;
     return glqh_launch_reduce_splits((const float *)ws, ks, B * m, B, m, (float)wscale, out, out_stride, accum, st);
 }
 
@@ -205,10 +218,12 @@ extern "C" int glqh_trellis_gemv_partials(const void *x_f16, int64_t B, const vo
     if (tr_bits_from_packed(packed_cols, 1, &R) || tr_check_shape(m, k, packed_rows)) return 1;
     const tr_plan plan = tr_plain_plan(m, k, B);
     const int ks = plan.ks;
-    const size_t need = (size_t)ks * B * m * sizeof(float);
+    // above 64 tokens the repacked activations of the tile kernel follow the partial sums
+    const size_t pbytes = align256((size_t)ks * B * m * sizeof(float));
+    const size_t need = plan.tile ? pbytes + plan.xb_bytes : (size_t)ks * B * m * sizeof(float);
     GLQH_REQUIRE(part_bytes >= need, "trellis partials: buffer of %zu bytes needed, got %zu", need, part_bytes);
     *ksplit_out = ks;
-    return tr_plain_partial(plan, x_f16, B, packed, R, m, k, part, (hipStream_t)stream);
+    return tr_plain_partial(plan, x_f16, B, packed, R, m, k, part, (char *)part + pbytes, (hipStream_t)stream);
 }
 
 // ---- RHT -------------------------------------------------------------------------
@@ -281,7 +296,8 @@ static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
 extern "C" size_t glqh_fused_linear_trellis_workspace_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
     if (!glqh_trellis_kernel_supported(m_pad, n_pad) || B < 1) return 0;
     glqh_init();
-    return align256((size_t)B * n_pad * sizeof(f16)) + 2 * tr_fused_part_bytes(B, n_pad, m_pad);
+    return align256((size_t)B * n_pad * sizeof(f16)) + 2 * tr_fused_part_bytes(B, n_pad, m_pad) +
+           tr_plain_plan(m_pad, n_pad, B).xb_bytes;
 }
 
 extern "C" int glqh_fused_linear_trellis_3inst(
@@ -313,8 +329,10 @@ extern "C" int glqh_fused_linear_trellis_3inst(
 
     const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
     const size_t pb = tr_fused_part_bytes(B, n_pad, m_pad);
-    GLQH_REQUIRE(ws && ws_bytes >= xb + 2 * pb, "fused trellis linear: workspace of %zu bytes needed, got %zu",
-                 xb + 2 * pb, ws_bytes);
+    const size_t tile_xb = tr_plain_plan(m_pad, n_pad, B).xb_bytes;
+    GLQH_REQUIRE(ws && ws_bytes >= xb + 2 * pb + tile_xb, "fused trellis linear: workspace of %zu bytes needed, got %zu",
+                 xb + 2 * pb + tile_xb, ws_bytes);
+    void *xb_tile = (char *)ws + xb + 2 * pb;                  // repacked activations of the many-token kernel
     f16 *x_rht = (f16 *)ws;
     float *part1 = (float *)((char *)ws + xb);
     float *part2 = (float *)((char *)ws + xb + pb);
@@ -385,8 +403,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         const tr_plan plan = tr_plain_plan(m_pad, n_pad, B);
         ks = plan.ks;
         if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
-        if (tr_plain_partial(plan, x_rht, B, packed, R1, m_pad, n_pad, part1, st)) return 1;
-        if (has_s2 && tr_plain_partial(plan, x_rht, B, packed2, R2, m_pad, n_pad, part2, st, ps2)) return 1;
+        if (tr_plain_partial(plan, x_rht, B, packed, R1, m_pad, n_pad, part1, xb_tile, st)) return 1;
+        if (has_s2 && tr_plain_partial(plan, x_rht, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2)) return 1;
     }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);

@@ -103,4 +103,28 @@ __device__ __forceinline__ uint32_t tr_state(uint32_t chunk, uint32_t cont, int 
     return (uint32_t)(ext >> (8 * R - R * j)) & 0xFFFFu;
 }
 
+// One A operand: four words (a.lo + a.hi, b.lo + b.hi) in fp16 from eight hash results, as
+// eight SDWA adds.  gfx950 needs one wait state between an instruction that writes part of a
+// register (dst_sel) and the next one that reads that register, and the compiler cannot see
+// into an asm block: the four low-half writes come first and the four high-half writes (which
+// read their destination to preserve it) after them, and a trailing s_nop covers whoever reads
+// the last word next.  (Adjacent pairs, as this was first written, gave wrong rows once the
+// scheduler moved an MFMA right behind them.)
+__device__ __forceinline__ u32x4 pair_sum4(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1, uint32_t a2,
+                                           uint32_t b2, uint32_t a3, uint32_t b3) {
+    uint32_t d0, d1, d2, d3;
+    asm("v_add_f16_sdwa %0, %4, %4 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %1, %6, %6 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %2, %8, %8 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %3, %10, %10 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %0, %5, %5 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %1, %7, %7 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %2, %9, %9 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "v_add_f16_sdwa %3, %11, %11 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+        "s_nop 0"
+        : "=&v"(d0), "=&v"(d1), "=&v"(d2), "=&v"(d3)
+        : "v"(a0), "v"(b0), "v"(a1), "v"(b1), "v"(a2), "v"(b2), "v"(a3), "v"(b3));
+    return u32x4{d0, d1, d2, d3};
+}
+
 }  // namespace

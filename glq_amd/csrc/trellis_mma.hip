@@ -254,229 +254,6 @@ tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int
 }
 
 // ---------------------------------------------------------------------------------
-// Prefill / large batch: 128 tokens x 256 rows per workgroup.
-// grid = (ceil(m/256), ceil(M/128), ksplit).  Each wave owns 64 rows and walks every k-pair
-// of the slot; the 128-token activation tile of PF_CH k-pairs at a time is staged in LDS and
-// shared by the four waves.  Here the matrix cores set the pace, so the two halves of a
-// weight are added first (one fp16 add with the rounding of the reference dequantizer,
-// glq/trellis.py:122-134) and a lane's eight weights of a row group -- columns
-// 2q + {0,1,8,9,16,17,24,25} of the k-pair -- form one A operand: 32 MFMAs per record
-// against eight token tiles.  The B operand of (q, token) is those eight activations, one
-// 16-byte LDS slot.
-// ---------------------------------------------------------------------------------
-constexpr int PF_NT = 8;
-constexpr int PF_CH = 4;
-constexpr int PF_KP_SLOTS = PF_NT * 4 * 17 + 4;                 // 16-byte slots per k-pair (+4: bank skew)
-
-// One A operand: four words (a.lo + a.hi, b.lo + b.hi) in fp16 from eight hash results, as
-// eight SDWA adds.  gfx950 needs one wait state between an instruction that writes part of a
-// register (dst_sel) and the next one that reads that register, and the compiler cannot see
-// into an asm block: the four low-half writes come first and the four high-half writes (which
-// read their destination to preserve it) after them, and a trailing s_nop covers whoever reads
-// the last word next.  (Adjacent pairs, as this was first written, gave wrong rows once the
-// scheduler moved an MFMA right behind them.)
-__device__ __forceinline__ u32x4 pair_sum4(uint32_t a0, uint32_t b0, uint32_t a1, uint32_t b1, uint32_t a2,
-                                           uint32_t b2, uint32_t a3, uint32_t b3) {
-    uint32_t d0, d1, d2, d3;
-    asm("v_add_f16_sdwa %0, %4, %4 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %1, %6, %6 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %2, %8, %8 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %3, %10, %10 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %0, %5, %5 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %1, %7, %7 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %2, %9, %9 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "v_add_f16_sdwa %3, %11, %11 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-        "s_nop 0"
-        : "=&v"(d0), "=&v"(d1), "=&v"(d2), "=&v"(d3)
-        : "v"(a0), "v"(b0), "v"(a1), "v"(b1), "v"(a2), "v"(b2), "v"(a3), "v"(b3));
-    return u32x4{d0, d1, d2, d3};
-}
-
-// Staging of tokens [tok0, tok0+128) x k-pairs [c0, c0+PF_CH), loaded one chunk ahead so that
-// the global loads are in flight while the current chunk is multiplied: a group = the 64 bytes
-// of one token in one k-pair (four 16-byte items, columns 8h..8h+7), whose dwords q of the four
-// items make up slot (q, token) -- one 16-byte LDS write per q.  Consecutive lanes take the
-// k-pairs of a token first (256 contiguous bytes of its row).  The loads are unconditional
-// (addresses clamped into the matrix); tokens past M and k-pairs past the slot are written as
-// zeros or skipped.
-constexpr int PF_GROUPS = 16 * PF_NT * PF_CH / TR_THREADS;      // per thread
-
-struct pf_regs {
-    u32x4 v[PF_GROUPS][4];
-};
-
-__device__ __forceinline__ pf_regs pf_stage_load(const f16 *__restrict__ x, int M, int k, int tok0, int c0,
-                                                 int kp_last) {
-    pf_regs r;
-#pragma unroll
-    for (int i = 0; i < PF_GROUPS; ++i) {
-        const int idx = i * TR_THREADS + (int)threadIdx.x;
-        const int u = idx % PF_CH, tk = idx / PF_CH;
-        const f16 *p = x + (int64_t)min(tok0 + tk, M - 1) * k + 32 * min(c0 + u, kp_last);
-#pragma unroll
-        for (int h = 0; h < 4; ++h) r.v[i][h] = *(const u32x4 *)(p + 8 * h);
-    }
-    return r;
-}
-
-__device__ __forceinline__ void pf_stage_write(u32x4 *xs, const pf_regs r, int M, int tok0, int n) {
-#pragma unroll
-    for (int i = 0; i < PF_GROUPS; ++i) {
-        const int idx = i * TR_THREADS + (int)threadIdx.x;
-        const int u = idx % PF_CH, tk = idx / PF_CH;
-        if (u < n) {
-            const bool ok = tok0 + tk < M;
-            const int dst = u * PF_KP_SLOTS + (tk >> 4) * (4 * 17) + (tk & 15);
-#pragma unroll
-            for (int qq = 0; qq < 4; ++qq)
-                xs[dst + qq * 17] = ok ? u32x4{r.v[i][0][qq], r.v[i][1][qq], r.v[i][2][qq], r.v[i][3][qq]}
-                                       : u32x4{0u, 0u, 0u, 0u};
-        }
-    }
-}
-
-// one record against the eight token tiles of k-pair slot `u` of the staged chunk
-template <int R>
-__device__ __forceinline__ mma_acc<PF_NT> pf_record(const tr_record<R> r, const mma_lane a,
-                                                     const u32x4 *xs, mma_acc<PF_NT> acc) {
-    f16x8 bf[PF_NT];
-#pragma unroll
-    for (int tt = 0; tt < PF_NT; ++tt) bf[tt] = __builtin_bit_cast(f16x8, xs[tt * 4 * 17]);
-    uint32_t cont[4];
-    tr_continuation_from<R>(r, a.next1, a.next2, cont);
-#pragma unroll
-    for (int ms = 0; ms < 2; ++ms) {
-        uint32_t h0[8], h1[8];                                      // k-tiles 0 and 1 of m-tile ms
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            h0[j] = tr_hash(tr_state<R>(r.c[ms], cont[ms], j));
-            h1[j] = tr_hash(tr_state<R>(r.c[2 + ms], cont[2 + ms], j));
-        }
-#pragma unroll
-        for (int rh = 0; rh < 2; ++rh) {
-            const int j0 = 2 * rh;
-            const f16x8 af = __builtin_bit_cast(f16x8, pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5],
-                                                                 h1[j0], h1[j0 + 1], h1[j0 + 4], h1[j0 + 5]));
-#pragma unroll
-            for (int tt = 0; tt < PF_NT; ++tt)
-                acc.v[2 * ms + rh][tt] =
-                    __builtin_amdgcn_mfma_f32_16x16x32_f16(af, bf[tt], acc.v[2 * ms + rh][tt], 0, 0, 0);
-        }
-    }
-    return acc;
-}
-
-template <int R>
-__global__ void __launch_bounds__(TR_THREADS, 2)
-tr_mma_prefill_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int M, int m, int k,
-                      int S, float *__restrict__ out, int direct, float scale, int accum,
-                      int64_t out_stride) {
-    extern __shared__ u32x4 xs_lds[];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const mma_lane a = mma_lane_of<16>(lane);
-    const int nkp = k >> 5;
-    const int mpairs = m >> 5;
-    const int slot = blockIdx.z;
-    const int kp0 = slot * S;
-    const int kp1 = min(kp0 + S, nkp);
-    const int last = kp1 - 1;
-    const int tok0 = blockIdx.y * (16 * PF_NT);
-    const int rowblk = blockIdx.x * TR_WAVES + wave;                // 64-row unit of this wave
-    const bool active = rowblk * 2 < mpairs;                        // uniform over the wave
-    const int mp = min(2 * rowblk + a.hm, mpairs - 1);
-
-    // The packed stream is requested two records ahead and the next activation chunk one
-    // chunk ahead; every load is unconditional with a clamped address, so the waits the
-    // compiler places count loads exactly.
-    constexpr int REC = 4 * R;
-    const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
-    tr_record<R> r0 = tr_load_record<R>(lane_base + (int64_t)kp0 * 32 * REC);
-    tr_record<R> r1 = tr_load_record<R>(lane_base + (int64_t)min(kp0 + 1, last) * 32 * REC);
-
-    mma_acc<PF_NT> acc;
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-#pragma unroll
-        for (int tt = 0; tt < PF_NT; ++tt) acc.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    pf_stage_write(xs_lds, pf_stage_load(x, M, k, tok0, kp0, last), M, tok0, kp1 - kp0);
-    __syncthreads();
-    for (int c0 = kp0; c0 < kp1; c0 += PF_CH) {
-        pf_regs next;
-#pragma unroll
-        for (int i = 0; i < PF_CH; ++i) {
-            const int kp = c0 + i;
-            const tr_record<R> r2 = tr_load_record<R>(lane_base + (int64_t)min(kp + 2, last) * 32 * REC);
-            if (i == 0) next = pf_stage_load(x, M, k, tok0, c0 + PF_CH, last);
-            if (active && kp < kp1)
-                acc = pf_record<R>(r0, a, xs_lds + i * PF_KP_SLOTS + a.q * 17 + a.tokl, acc);
-            r0 = r1;
-            r1 = r2;
-        }
-        // LDS-only barriers: the records requested two ahead stay in flight across them
-        fht_barrier<true>();                                     // chunk consumed by every wave
-        pf_stage_write(xs_lds, next, M, tok0, kp1 - (c0 + PF_CH));
-        fht_barrier<true>();
-    }
-    if (!active) return;
-    // lane holds rows i0 .. i0+3 (consecutive) of token tokl for every (s, tt)
-    const int i0 = 4 * a.q;
-    const int rbase = 64 * rowblk + 32 * (i0 >> 3) + (i0 & 7);
-    const bool vec = (out_stride & 3) == 0;
-    if (!direct) {
-#pragma unroll
-        for (int tt = 0; tt < PF_NT; ++tt) {
-            const int tok = tok0 + 16 * tt + a.tokl;
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                if (tok < M && rbase + 8 * s < m)
-                    *(f32x4 *)(out + ((int64_t)slot * M + tok) * m + rbase + 8 * s) = acc.v[s][tt];
-        }
-    } else if (vec) {
-#pragma unroll
-        for (int tt = 0; tt < PF_NT; ++tt) {
-            const int tok = tok0 + 16 * tt + a.tokl;
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                if (tok < M && rbase + 8 * s < m) {
-                    f32x4 *o = (f32x4 *)(out + (int64_t)tok * out_stride + rbase + 8 * s);
-                    f32x4 v = acc.v[s][tt] * scale;
-                    if (accum) v += *o;
-                    *o = v;
-                }
-            }
-        }
-    } else {
-#pragma unroll
-        for (int tt = 0; tt < PF_NT; ++tt) {
-            const int tok = tok0 + 16 * tt + a.tokl;
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                if (tok < M && rbase + 8 * s < m) {
-                    float *o = out + (int64_t)tok * out_stride + rbase + 8 * s;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = accum ? o[e] + acc.v[s][tt][e] * scale : acc.v[s][tt][e] * scale;
-                }
-            }
-        }
-    }
-}
-
-constexpr int PF_LDS = PF_CH * PF_KP_SLOTS * 16;                  // 35072 bytes
-
-template <int R>
-int launch_prefill(const void *x, int64_t M, const void *packed, int64_t m, int64_t k, int S, int ksplit,
-                   float *out, int direct, float scale, int accum, int64_t out_stride, hipStream_t stream) {
-    dim3 grid((unsigned)((m + 255) / 256), (unsigned)((M + 16 * PF_NT - 1) / (16 * PF_NT)), (unsigned)ksplit);
-    hipLaunchKernelGGL((tr_mma_prefill_kernel<R>), grid, dim3(TR_THREADS), PF_LDS, stream,
-                       (const uint8_t *)packed, (const f16 *)x, (int)M, (int)m, (int)k, S, out, direct, scale,
-                       accum, out_stride);
-    GLQH_LAUNCH_CHECK("trellis prefill launch");
-    return 0;
-}
-
-// ---------------------------------------------------------------------------------
 // GEMV with the input transform folded in (1..4 tokens), MFMA form.
 //
 // grid = (ceil(m/64), ksplit[, layers]).  K slot s owns the S = 2^j k-pairs starting at s*S,
@@ -761,57 +538,6 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
     return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
-// Prefill plan: K is split over the grid when the 256-row x 128-token tiles alone leave CUs idle.
-// The split is chosen by a small cost model fitted to this kernel on the 4096 <-> 14336 shapes:
-// a workgroup takes 6 us + 1.0 us per k-pair when it has its CU to itself and 9 us + 1.53 us per
-// k-pair when two share one; a launch runs in rounds of two workgroups per CU, and a last round
-// of at most one workgroup per CU runs at the faster rate; every partial-sum slot costs its
-// write and the consumer's read, about 0.35 us per MB.  (A split that spills a few workgroups into a second
-// round, or one more slot than the grid needs, costs more than it gains.)
-int glqh_trellis_prefill_plan(int64_t m, int64_t k, int64_t M, int *S_out, int *ksplit_out) {
-    const int64_t nkp = k / 32;
-    const int64_t tiles = ((m + 255) / 256) * ((M + 127) / 128);
-    const int64_t cus = glqh_device_cus(), slots = 2 * cus;
-    double best = 0.0;
-    int64_t best_S = (nkp + PF_CH - 1) / PF_CH * PF_CH, best_ks = 1;
-    for (int64_t ks = 1; ks <= 16; ++ks) {
-        int64_t S = (nkp + ks - 1) / ks;
-        S = (S + PF_CH - 1) / PF_CH * PF_CH;
-        const int64_t ksp = (nkp + S - 1) / S;
-        if (ksp != ks && ks > 1) continue;                      // same split as a smaller ks
-        const int64_t W = tiles * ksp, full = W / slots, rem = W % slots;
-        double t = (double)full * (S * 1.53 + 9.0) + (rem == 0 ? 0.0 : rem <= cus ? S * 1.0 + 6.0 : S * 1.53 + 9.0);
-        if (ksp > 1) t += 0.35e-6 * 4.0 * (double)ksp * (double)M * (double)m;
-        if (ks == 1 || t < best) {
-            best = t;
-            best_S = S;
-            best_ks = ksp;
-        }
-    }
-    *S_out = (int)best_S;
-    *ksplit_out = (int)best_ks;
-    return 1;
-}
-
-int glqh_launch_trellis_prefill(const void *x_f16, int64_t M, const void *packed, int R, int64_t m, int64_t k,
-                                int S, int ksplit, float *out, int direct, float scale, int accum,
-                                int64_t out_stride, hipStream_t stream) {
-    switch (R) {
-    case 1: return launch_prefill<1>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
-    case 2: return launch_prefill<2>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
-    case 3: return launch_prefill<3>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
-    case 4: return launch_prefill<4>(x_f16, M, packed, m, k, S, ksplit, out, direct, scale, accum, out_stride, stream);
-    }
-    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
-}
-
-template <typename K>
-static int pf_set_lds(K kernel) {
-    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              PF_LDS),
-                          "trellis prefill attribute");
-}
-
 // ---- fused-input GEMV (MFMA form): plan and launch -----------------------------------
 // S k-pairs per K slot: a power of two >= 8 chosen so that about four workgroups per CU are
 // in flight; the slice 32*S is capped by LDS (8192 columns at one token, 4096 at 2..4).
@@ -915,7 +641,5 @@ static int fi_init_R() {
 
 int glqh_trellis_mma_init(void) {
     return mma_init_R<1>() || mma_init_R<2>() || mma_init_R<3>() || mma_init_R<4>() ||
-           pf_set_lds(tr_mma_prefill_kernel<1>) || pf_set_lds(tr_mma_prefill_kernel<2>) ||
-           pf_set_lds(tr_mma_prefill_kernel<3>) || pf_set_lds(tr_mma_prefill_kernel<4>) ||
            fi_init_R<1>() || fi_init_R<2>() || fi_init_R<3>() || fi_init_R<4>();
 }

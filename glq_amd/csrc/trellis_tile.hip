@@ -1,0 +1,337 @@
+// Trellis-3INST GEMM for many tokens on the packed stream (gfx950, wave64).
+//
+// Y_rht[token, row] = sum_k X_rht[token, k] * W[row, k], W the exact fp16 dequantizer values
+// (glq/trellis.py:122-134, 629-643; the reference's batched kernel is
+// glq/csrc/glq_trellis.cu:555-715 and above 64 tokens it dequantizes to a dense weight for a
+// library GEMM, :1322-1334).  Decoding a state costs about four vector instructions, as much as
+// the multiply-adds of a dozen tokens on the matrix cores, so a decoded weight has to meet as many
+// tokens as possible:
+//
+//   workgroup tile = 128 rows x (128 * NTW) tokens, 8 waves (two per SIMD);
+//   a step is 64 columns = two k-pairs of the four 32-row blocks of the tile.  Wave w DECODES half
+//   a record per lane -- block pair w >> 2, k-pair (w >> 1) & 1, m-tile w & 1: 16 states, two A
+//   operands of v_mfma_f32_16x16x32_f16 with the two fp16 halves of every weight added first (the
+//   dequantizer's rounding) -- and writes them to LDS in operand layout (lane L's 16 bytes at slot
+//   L: conflict-free both ways).  Every wave then MULTIPLIES all 16 operands of the step, read
+//   back from LDS one ahead of their use, with ITS OWN 16 * NTW tokens, whose activations it
+//   holds in registers, straight from global memory.
+//
+// A lane's eight weights of an operand are columns 2q + {0,1,8,9,16,17,24,25} of the k-pair
+// (glq/trellis.py:99-101), and the B operand puts consecutive tokens in consecutive lanes, so the
+// activations are repacked once per call into xb[k-pair][q][token][those 8 columns]: every operand
+// load is then four runs of 256 contiguous bytes.  Workgroups are persistent and walk tiles in an
+// order that gives the CUs of one XCD the same tokens at the same time.  K is split into slots only
+// while the tiles alone would leave CUs idle; partial sums [slot][token][row] are combined in slot
+// order by the consumer, or, with one slot, the scaled result is written (or added) in place.
+#include "common.h"
+#include "trellis_device.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int TT_WAVES = 8;
+constexpr int TT_THREADS = TT_WAVES * GLQH_WAVE;
+constexpr int TT_FRAGS = 8;                        // 16-row operands per 64-column half-step: 128 rows
+constexpr int TT_ROWS = 128;
+constexpr int TT_BUF = 2 * TT_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer
+constexpr size_t TT_LDS = (size_t)2 * TT_BUF * 16; // 32 KB
+
+struct tt_args {
+    const uint8_t *packed;
+    const f16 *xb;                                 // (k / 32, 4, Mp, 8) fp16
+    int M, Mp, m, k;
+    int RT, TT, KS, slot_ds;                       // row tiles, token tiles, K slots, 64-column steps per slot
+    float *out;                                    // partial sums [slot][token][row], or the result rows
+    int direct, accum;
+    float scale;
+    int64_t out_stride;
+};
+
+__device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global prefetches stay in flight
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_kernel(const tt_args a) {
+    extern __shared__ u32x4 abuf[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, q = lane >> 4;
+    const int nkp = a.k >> 5, nds = a.k >> 6, mpairs = a.m >> 5;
+    constexpr int REC = 4 * R;
+
+    // decode role
+    const int unit = wave >> 2, kpi = (wave >> 1) & 1, ms = wave & 1;
+    const int hm = i >> 3, l = 4 * (i & 7) + q;
+    const int l1 = (l + 1) & 31, l2 = (l + 2) & 31;
+    const int next1 = 16 * (l1 & 3) + 8 * hm + (l1 >> 2), next2 = 16 * (l2 & 3) + 8 * hm + (l2 >> 2);
+
+    const int nitems = a.TT * a.KS * a.RT;
+    const int per_xcd = (nitems + 7) >> 3;
+    const int xcd = blockIdx.x & 7, bx = blockIdx.x >> 3;
+    const int nbx = ((int)gridDim.x - xcd + 7) >> 3;
+    for (int w = bx; w < per_xcd; w += nbx) {
+        const int item = xcd * per_xcd + w;
+        if (item >= nitems) break;                              // uniform
+        const int rt = item % a.RT, slot = (item / a.RT) % a.KS, tt0 = item / (a.RT * a.KS);
+        const int r0 = rt * TT_ROWS, tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW;
+        const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
+
+        const int mp = min(2 * (2 * rt + unit) + hm, mpairs - 1);
+        const uint8_t *rec_base = a.packed + ((int64_t)mp * nkp * 32 + l) * REC + (int64_t)kpi * 32 * REC;
+        auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
+            return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
+        };
+        // two operands (row groups 2 ms, 2 ms + 1 of the 64-row unit) from half a record
+        auto emit = [&](const tr_record<R> &r, u32x4 *dst) {
+            uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
+            uint32_t n0, n1;
+            if constexpr (R >= 2) {
+                constexpr int sh = 8 * R - 16;
+                const uint32_t t = ((c0 >> sh) & 0xFFFFu) | (((c1 >> sh) & 0xFFFFu) << 16);
+                const uint32_t n = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
+                n0 = n & 0xFFFFu;
+                n1 = n >> 16;
+            } else {
+                const uint32_t t = c0 | (c1 << 8);
+                const uint32_t x1 = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
+                const uint32_t x2 = (uint32_t)__shfl((int)t, next2, GLQH_WAVE);
+                n0 = ((x1 & 0xFFu) << 8) | (x2 & 0xFFu);
+                n1 = (x1 & 0xFF00u) | ((x2 >> 8) & 0xFFu);
+            }
+            uint32_t h0[8], h1[8];                              // k-tiles 0 and 1 of m-tile ms
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                h0[j] = tr_hash(tr_state<R>(c0, n0, j));
+                h1[j] = tr_hash(tr_state<R>(c1, n1, j));
+            }
+#pragma unroll
+            for (int rh = 0; rh < 2; ++rh) {
+                const int j0 = 2 * rh;
+                const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1],
+                                           h1[j0 + 4], h1[j0 + 5]);
+                dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
+            }
+        };
+        // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(4 kp + q) * Mp + token]
+        // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
+        const int64_t bstep = (int64_t)a.Mp * 32;               // elements from one k-pair to the next
+        const f16 *xrow = a.xb + ((int64_t)q * a.Mp + tok0 + i) * 8;
+
+        f32x4 acc[TT_FRAGS][NTW];
+#pragma unroll
+        for (int f = 0; f < TT_FRAGS; ++f)
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) acc[f][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        // Software pipeline over the 64-column steps: records arrive two steps ahead, the operands
+        // of step d + 1 are written to the other LDS buffer during step d, and the activations of
+        // the next step arrive a whole step ahead in a second register set where registers allow
+        // (NTW <= 2), otherwise half a step ahead in the registers the half just multiplied freed.
+        constexpr bool BDB = NTW <= 2;
+        u32x4 b[BDB ? 2 : 1][NTW][2];
+        auto load_b = [&](u32x4 (&bb)[NTW][2], int d) {
+            d = min(d, ds1 - 1);
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) {
+                bb[tt][0] = *(const u32x4 *)(xrow + 2 * d * bstep + tt * 128);
+                bb[tt][1] = *(const u32x4 *)(xrow + (2 * d + 1) * bstep + tt * 128);
+            }
+        };
+        tr_record<R> rc = load_rec(ds0);
+        load_b(b[0], ds0);
+        tr_record<R> r1 = load_rec(ds0 + 1), r2 = load_rec(ds0 + 2);
+        emit(rc, abuf);
+        tt_barrier();
+
+        for (int d0 = ds0; d0 < ds1; d0 += 2) {
+#pragma unroll
+          for (int par = 0; par < 2; ++par) {                   // static buffer parity
+            const int d = d0 + par;
+            if (d >= ds1) break;                                // uniform
+            const int cur = BDB ? par : 0;
+            const u32x4 *rd = abuf + par * TT_BUF;
+            u32x4 *wr = abuf + (par ^ 1) * TT_BUF;
+            const int dn = min(d + 1, ds1 - 1);
+            if constexpr (BDB) load_b(b[par ^ 1], d + 1);
+            const tr_record<R> r3 = load_rec(d + 3);
+            f16x8 afn = __builtin_bit_cast(f16x8, rd[lane]);
+            __builtin_amdgcn_sched_barrier(0);                  // requests stay ahead of the multiplications
+#pragma unroll
+            for (int kk = 0; kk < 2 * TT_FRAGS; ++kk) {
+                const int u = kk / TT_FRAGS, f = kk % TT_FRAGS;
+                const f16x8 af = afn;
+                if (kk + 1 < 2 * TT_FRAGS) afn = __builtin_bit_cast(f16x8, rd[(kk + 1) * GLQH_WAVE + lane]);
+#pragma unroll
+                for (int tt = 0; tt < NTW; ++tt)
+                    acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        af, __builtin_bit_cast(f16x8, b[cur][tt][u]), acc[f][tt], 0, 0, 0);
+                if (kk == 1) emit(r1, wr);                      // operands of d + 1 (unused after the last step)
+                if constexpr (!BDB) {
+                    if (f == TT_FRAGS - 1) {                    // this half's activations are free: request the next
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + (2 * dn + u) * bstep + tt * 128);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            tt_barrier();                                       // rd has been read, wr is written
+            r1 = r2;
+            r2 = r3;
+          }
+        }
+
+        // lane holds four consecutive rows of token i for every (operand, token tile): operand
+        // f = 4 unit' + s covers rows 64 unit' + 32 h + 8 s + (0..7), h = 0, 1
+        const int rlane = 32 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int tt = 0; tt < NTW; ++tt) {
+            const int tok = tok0 + 16 * tt + i;
+            if (tok >= a.M) continue;
+#pragma unroll
+            for (int f = 0; f < TT_FRAGS; ++f) {
+                const int row = r0 + 64 * (f >> 2) + 8 * (f & 3) + rlane;
+                if (row >= a.m) continue;                       // m is a multiple of 32: whole groups of four
+                if (!a.direct) {
+                    *(f32x4 *)(a.out + ((int64_t)slot * a.M + tok) * a.m + row) = acc[f][tt];
+                } else {
+                    float *o = a.out + (int64_t)tok * a.out_stride + row;
+                    if ((a.out_stride & 3) == 0) {
+                        f32x4 v = acc[f][tt] * a.scale;
+                        if (a.accum) v += *(f32x4 *)o;
+                        *(f32x4 *)o = v;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = a.accum ? o[e] + acc[f][tt][e] * a.scale : acc[f][tt][e] * a.scale;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// (M, k) row-major fp16 -> xb[k-pair][q][token][8]: slot q of a k-pair takes columns
+// 2q + {0,1,8,9,16,17,24,25}, i.e. dword q of each of its four 16-byte items.  64 tokens x 4
+// k-pairs per workgroup through LDS; reads in runs of 256 bytes, writes in runs of 1 KB.
+__global__ void __launch_bounds__(256)
+tr_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, int Mp, int k) {
+    __shared__ u32x4 tile[16][65];                              // [k-pair * 4 + q][token]
+    const int tok0 = blockIdx.x * 64, kp0 = blockIdx.y * 4, nkp = k >> 5;
+    const int t = threadIdx.x;
+    {
+        const int kpi = t & 3, tl = t >> 2;
+        const int tok = min(tok0 + tl, M - 1), kp = min(kp0 + kpi, nkp - 1);
+        const u32x4 *src = (const u32x4 *)(x + (int64_t)tok * k + 32 * kp);
+        const u32x4 v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq) tile[kpi * 4 + qq][tl] = u32x4{v0[qq], v1[qq], v2[qq], v3[qq]};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int sl = r * 4 + (t >> 6), tl = t & 63;          // slot = k-pair * 4 + q
+        const int kp = kp0 + (sl >> 2);
+        if (tok0 + tl < M && kp < nkp)
+            *(u32x4 *)(xb + (((int64_t)kp * 4 + (sl & 3)) * Mp + tok0 + tl) * 8) = tile[sl][tl];
+    }
+}
+
+int tt_ntw(int64_t M) { return M <= 128 ? 1 : M <= 256 ? 2 : 4; }
+
+int64_t tt_padded_tokens(int64_t M) {
+    const int64_t tile = TT_WAVES * 16 * tt_ntw(M);
+    return (M + tile - 1) / tile * tile;
+}
+
+struct tt_plan {
+    int NTW, RT, TT, KS, slot_ds, grid;
+};
+
+void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p) {
+    p->NTW = tt_ntw(M);
+    const int tile_tok = TT_WAVES * 16 * p->NTW;
+    p->RT = (int)((m + TT_ROWS - 1) / TT_ROWS);
+    p->TT = (int)((M + tile_tok - 1) / tile_tok);
+    const int nds = (int)(k / 64);
+    const int cus = glqh_device_cus();
+    const int64_t base = (int64_t)p->RT * p->TT;
+    int64_t ks = 1;
+    if (base < cus) {
+        ks = cus / base;
+        const int64_t cap_len = nds / 8 > 0 ? nds / 8 : 1;      // slots of at least 512 columns
+        if (ks > cap_len) ks = cap_len;
+        const int64_t cap_bytes = ((int64_t)128 << 20) / (M * m * 4);   // partial sums stay under 128 MB
+        if (ks > cap_bytes) ks = cap_bytes;
+        if (ks < 1) ks = 1;
+    }
+    p->slot_ds = (int)((nds + ks - 1) / ks);
+    p->KS = (nds + p->slot_ds - 1) / p->slot_ds;
+    const int64_t items = base * p->KS;
+    p->grid = (int)(items < cus ? items : cus);
+}
+
+template <int R, int NTW>
+int tt_launch(const tt_plan &p, const tt_args &a, hipStream_t stream) {
+    hipLaunchKernelGGL((tr_tile_kernel<R, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a);
+    GLQH_LAUNCH_CHECK("trellis tile launch");
+    return 0;
+}
+
+template <int R>
+int tt_launch_R(const tt_plan &p, const tt_args &a, hipStream_t stream) {
+    if (p.NTW == 1) return tt_launch<R, 1>(p, a, stream);
+    if (p.NTW == 2) return tt_launch<R, 2>(p, a, stream);
+    return tt_launch<R, 4>(p, a, stream);
+}
+
+}  // namespace
+
+// bytes of the repacked activations of a many-token call
+size_t glqh_trellis_tile_xb_bytes(int64_t k, int64_t M) { return (size_t)tt_padded_tokens(M) * k * sizeof(f16); }
+
+// K slots the many-token kernel uses for this call (1: it can write the result in place)
+int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M) {
+    tt_plan p;
+    tt_make_plan(m, k, M, &p);
+    return p.KS;
+}
+
+// direct == 0: out[(slot * M + token) * m + row] = the slot's partial sum, unscaled;
+// direct == 1 (one slot only): out[token * out_stride + row] = (accum ? out : 0) + scale * sum.
+// x_f16 is (M, k) row-major; xb_scratch takes its repacked copy (glqh_trellis_tile_xb_bytes).
+int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
+                             int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
+                             hipStream_t stream) {
+    tt_plan p;
+    tt_make_plan(m, k, M, &p);
+    if (direct && p.KS != 1) return glqh_fail("trellis tile kernel: in-place output needs a single K slot");
+    const int Mp = (int)tt_padded_tokens(M);
+    hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)), dim3(256),
+                       0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, Mp, (int)k);
+    GLQH_LAUNCH_CHECK("trellis pack launch");
+    tt_args a;
+    a.packed = (const uint8_t *)packed;
+    a.xb = (const f16 *)xb_scratch;
+    a.M = (int)M;
+    a.Mp = Mp;
+    a.m = (int)m;
+    a.k = (int)k;
+    a.RT = p.RT;
+    a.TT = p.TT;
+    a.KS = p.KS;
+    a.slot_ds = p.slot_ds;
+    a.out = out;
+    a.direct = direct;
+    a.accum = accum;
+    a.scale = scale;
+    a.out_stride = out_stride;
+    switch (R) {
+    case 1: return tt_launch_R<1>(p, a, stream);
+    case 2: return tt_launch_R<2>(p, a, stream);
+    case 3: return tt_launch_R<3>(p, a, stream);
+    case 4: return tt_launch_R<4>(p, a, stream);
+    }
+    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}

@@ -25,14 +25,13 @@ from ._lib import GLQH_BF16, GLQH_F16, GLQH_F32, check
 
 _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F32}
 
-# Token counts above these take the dense route: dequantize the weight to fp16 once with
-# the HIP kernel, then one library GEMM (hipBLASLt through torch.mm), as the reference
-# does above GLQ_TRELLIS_BATCH_MAX (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334).  Below
-# them the weights stay compressed.  The trellis kernels decode straight into MFMA operands
-# for any token count and beat the dense route up to a few hundred tokens (measured on
-# 4096 <-> 14336: 66 vs 95 us at 128 tokens, 96 vs 113 us at 256, 241 vs 197 us at 1024), so
-# the default trellis threshold is 512.
-TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "512")))
+# Every token count is served on the compressed weights: 1-64 tokens by the GEMV / small-batch
+# kernels, above by the tile kernels that decode each weight once per 128-row x 512-token tile
+# (csrc/trellis_tile.hip, csrc/e8_tile.hip).  The reference's own many-token route -- dequantize
+# the weight to fp16 once with the HIP kernel, then one library GEMM (glq/csrc/glq_trellis.cu:
+# 1265-1268, 1322-1334) -- is kept behind its tunable: GLQ_TRELLIS_BATCH_MAX=<n> sends calls above
+# n tokens there.
+TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", str(1 << 30))))
 # E8 layers stay on their compressed indices at every token count (above 16 tokens: one lookup per
 # weight and 128 x 512 tile, csrc/e8_tile.hip); GLQ_E8_BATCH_MAX=<n> sends calls above n tokens to
 # the dense route instead.

@@ -68,7 +68,9 @@ int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B,
  * For callers that fold the fixed-order reduction into their own consumer (as the fused
  * linear does) and for timing the decode kernel in isolation.  The reference has no
  * separate entry for this step (its GEMV reduces inside the block,
- * glq/csrc/glq_trellis.cu:485-510). */
+ * glq/csrc/glq_trellis.cu:485-510).  Above 64 tokens the many-token kernel keeps its repacked
+ * activations behind the partial sums: part_bytes must then cover
+ * glqh_trellis_gemv_workspace_bytes(m, k, B) (the sums rounded up to 256 bytes + that copy). */
 int glqh_trellis_gemv_partials(const void *x_f16, int64_t B,
                                const void *packed, int64_t packed_rows, int64_t packed_cols,
                                int64_t m, int64_t k, float *part, size_t part_bytes,

@@ -196,12 +196,19 @@ def extras(torch, ext, dev):
 
         def to16(i):
             return (i.to(torch.int32) - ((i >= 32768).to(torch.int32) << 16)).to(torch.int16).reshape(m, n // 8)
-        qs = [(to16(i1.roll(r * 977)).contiguous(), to16(i2.roll(r * 977)).contiguous()) for r in range(4)]
+        # 10 rotated index sets x 29.4 MB = 294 MB > the 256 MB Infinity Cache: every launch streams from HBM
+        qs = [(to16(i1.roll(r * 977)).contiguous(), to16(i2.roll(r * 977)).contiguous()) for r in range(E8_SETS)]
         for B in (1, 16):
             xh = torch.randn(B, n, device=dev).to(torch.float16)
             us = _graph_time(torch, lambda: [ext.glq_dequant_matmul_cuda(xh, a, cb, 0.02, b, cb, 1 / 3.0)
                                              for a, b in qs], len(qs))
             out[f"e8_2stage_gemv_4096x14336_B{B}_GBs"] = round(m * (n // 8) * 4 / us / 1e3, 1)
+        # config 4, E8 half: the many-token kernel on the same quantized indices (kernel + K-slot sum)
+        for M in (256, 4096):
+            xh = torch.randn(M, n, device=dev).to(torch.float16)
+            us = _graph_time(torch, lambda: ext.glq_dequant_matmul_cuda(xh, qs[0][0], cb, 0.02, qs[0][1], cb, 1 / 3.0),
+                             1, reps=5)
+            out[f"e8_2stage_matmul_4096x14336_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
         del qs, i1, i2
         torch.cuda.empty_cache()
     except Exception as e:
@@ -237,7 +244,9 @@ def extras(torch, ext, dev):
     return out
 
 
-CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "decoder")
+CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
+         "e8_prefill_256", "decoder")
+E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 
 def run_case(torch, ext, dev, name, steps):
@@ -260,7 +269,7 @@ def run_case(torch, ext, dev, name, steps):
         o = torch.empty(M, m, dtype=torch.float32, device=dev)
         fn = lambda i: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o)
         res["flop_per_launch"] = 2.0 * M * m * n
-    elif name == "e8_gemv_2stage":
+    elif name in ("e8_gemv_2stage", "e8_prefill_4096", "e8_prefill_256"):
         from glq_amd.checkpoint import load_shell_table
         cb = load_shell_table(None).to(dev)
         m, n = 4096, 14336
@@ -271,10 +280,12 @@ def run_case(torch, ext, dev, name, steps):
 
         def to16(i):
             return (i.to(torch.int32) - ((i >= 32768).to(torch.int32) << 16)).to(torch.int16).reshape(m, n // 8)
-        qs = [(to16(i1.roll(r * 977)).contiguous(), to16(i2.roll(r * 977)).contiguous()) for r in range(4)]
-        xh = torch.randn(1, n, device=dev).to(torch.float16)
-        fn = lambda i: ext.glq_dequant_matmul_cuda(xh, qs[i % 4][0], cb, 0.02, qs[i % 4][1], cb, 1 / 3.0)
+        qs = [(to16(i1.roll(r * 977)).contiguous(), to16(i2.roll(r * 977)).contiguous()) for r in range(E8_SETS)]
+        M = 1 if name == "e8_gemv_2stage" else int(name.rsplit("_", 1)[1])
+        xh = torch.randn(M, n, device=dev).to(torch.float16)
+        fn = lambda i: ext.glq_dequant_matmul_cuda(xh, qs[i % E8_SETS][0], cb, 0.02, qs[i % E8_SETS][1], cb, 1 / 3.0)
         res["bytes_per_launch"] = m * (n // 8) * 4
+        res["flop_per_launch"] = 2.0 * M * m * n
     elif name == "decoder":
         from glq_amd.decoder import TrellisDecoder
         dec = TrellisDecoder(max_len=1024)
@@ -390,13 +401,36 @@ def main():
                 rem_graphs[n % L] = capture(n % L)
         replay_steps(W)
         torch.cuda.synchronize()
+        # exactly K steps between two HIP events on the replay stream (device time: a host clock
+        # around a millisecond of work mostly measures the submission), host clock kept beside it
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        ev0.record(stream)
         replay_steps(K)
+        ev1.record(stream)
         torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
+        dt_host = time.perf_counter() - t0
+        dt = ev0.elapsed_time(ev1) * 1e-3
+        # distribution: the whole pool (L steps) replayed 200 times, one event pair per replay
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(200)]
+        for a, b in evs:
+            a.record(stream)
+            full.replay()
+            b.record(stream)
+        torch.cuda.synchronize()
+        per_step = sorted(a.elapsed_time(b) * 1e3 / L for a, b in evs)
     ms_per_step = dt / K * 1e3
     value = bytes_step / (dt / K) / 1e9
-    log(f"timed {K} steps: {ms_per_step * 1e3:.1f} us/step, {value:.1f} GB/s packed weights")
+    stats = {"us_per_step_median": round(per_step[len(per_step) // 2], 2),
+             "us_per_step_p10": round(per_step[len(per_step) // 10], 2),
+             "us_per_step_p90": round(per_step[(len(per_step) * 9) // 10], 2),
+             "replays": len(per_step), "steps_per_replay": L,
+             "us_per_step_host_clock": round(dt_host / K * 1e6, 2),
+             "method": "HIP events on the replay stream; value is from the K timed steps, the "
+                       "distribution from 200 further replays of the whole weight pool"}
+    log(f"timed {K} steps: {ms_per_step * 1e3:.1f} us/step (host clock {dt_host / K * 1e6:.1f}), "
+        f"{value:.1f} GB/s packed weights; median {stats['us_per_step_median']} us "
+        f"(p10 {stats['us_per_step_p10']}, p90 {stats['us_per_step_p90']})")
 
     # ---- roofline leg: the decode launches alone, HIP events on their own stream ---------
     # The same grouped calls as the timed steps, stopped after the decode kernel (input
@@ -423,13 +457,17 @@ def main():
     achieved = bytes_launch / (avg_us * 1e-6) / 1e9
     # HBM bytes per launch from the committed counter summary (FETCH_SIZE / WRITE_SIZE runs)
     traffic = None
+    traffic_source = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic_tr_mma_fusein_kernels_smollm3_4bpw_batch1.txt")
     if os.path.exists(tpath):
         import re
         mt = re.search(r"^traffic_bytes_per_launch\s*=\s*(\d+)", open(tpath).read(), re.M)
         traffic = int(mt.group(1)) if mt else None
+        if traffic is not None:
+            traffic_source = ("not measured by this run: FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this "
+                              "command, recorded in profiles/" + os.path.basename(tpath))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                 "kernel": ("tr_mma_fusein_kernel<4,bf16,1> (o, down) and tr_mma_fusein_group_kernel<4,bf16,1> "
                            "(q/k/v, gate/up): the fused-input decode launch, averaged over the four "
                            "groups of a step"),
@@ -468,6 +506,7 @@ def main():
                    "distinct_layers": L, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
                    "linear_only_tok_s_36_layers": round(1e3 / (ms_per_step * 36), 1)},
         "roofline": roofline,
+        "timing": stats,
         "extra": extra,
     }
     if not args.no_cpu_baseline:

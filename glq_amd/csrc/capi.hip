@@ -837,14 +837,12 @@ extern "C" int glqh_e8_dequant_matmul(const void *x_f16, int64_t B, const void *
     const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
     const size_t need = (size_t)ks * sg.n * B * m_pad * sizeof(float);
     GLQH_REQUIRE(ws && ws_bytes >= need, "e8 matmul: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    // every stage's partial sums are written already multiplied by that stage's scale: one
+    // reduction over ks * stages plain slots instead of one launch per stage
     if (glqh_launch_e8_partial(x_f16, B, sg.q, sg.n, table1, table2 ? table2 : table1,
-                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st))
+                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st, sg.scale))
         return 1;
-    for (int s = 0; s < sg.n; ++s)
-        if (glqh_launch_reduce_splits(part + (int64_t)s * B * m_pad, ks, (int64_t)sg.n * B * m_pad, B, m_pad,
-                                      sg.scale[s], out, m_pad, s > 0, st))
-            return 1;
-    return 0;
+    return glqh_launch_reduce_splits(part, ks * sg.n, B * m_pad, B, m_pad, 1.0f, out, m_pad, 0, st);
 }
 
 extern "C" int glqh_e8_decompress(const void *q1, const void *q2, const void *q3, const void *q4,

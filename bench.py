@@ -245,7 +245,7 @@ def extras(torch, ext, dev):
 
 
 CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
-         "e8_prefill_256", "decoder")
+         "e8_prefill_256", "decoder", "batch1_step")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 
@@ -286,6 +286,23 @@ def run_case(torch, ext, dev, name, steps):
         fn = lambda i: ext.glq_dequant_matmul_cuda(xh, qs[i % E8_SETS][0], cb, 0.02, qs[i % E8_SETS][1], cb, 1 / 3.0)
         res["bytes_per_launch"] = m * (n // 8) * 4
         res["flop_per_launch"] = 2.0 * M * m * n
+    elif name == "batch1_step":
+        # the step of the headline measurement, eager: the four grouped calls of one decoder layer
+        # (decode launch + output-transform launch each), rotating over four weight sets
+        from glq_amd import hadamard
+        pool = build_pool(torch, hadamard, 4, dev)
+        xs = {n: torch.randn(1, n, generator=torch.Generator(device=dev).manual_seed(1), device=dev)
+              .to(torch.bfloat16) for _, _, n in LINEARS}
+
+        def fn(i):
+            by = {lin["name"]: lin for lin in pool[i % 4]}
+            for names in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",)):
+                lins = [by[nm] for nm in names]
+                a = lins[0]
+                ext.glq_fused_linear_trellis_3inst_group(
+                    xs[a["n"]], [(l["sv"], l["su"], l["packed"], l["wscale"], l["m"], l["m"]) for l in lins],
+                    a["bn"], a["bn_meta"], a["n"], a["n"], out_dtype=torch.bfloat16)
+        res["bytes_per_launch"] = sum(m * n * K_BITS // 8 for _, m, n in LINEARS)
     elif name == "decoder":
         from glq_amd.decoder import TrellisDecoder
         dec = TrellisDecoder(max_len=1024)

@@ -78,12 +78,14 @@ static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
 // plan.xb_bytes for the tile kernel (unused otherwise).
 static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
                             int64_t k, float *part, void *xb, hipStream_t st, float pscale = 1.0f) {
+    glqh_range range("dequant_matmul");
     if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, part, 0, 1.0f, 0, 0, st);
     return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, pscale, 0, 0, st);
 }
 static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
                            int64_t k, float scale, float *out, int64_t out_stride, int accum, void *xb,
                            hipStream_t st) {
+    glqh_range range("dequant_matmul");
     if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, out, 1, scale, accum, out_stride, st);
     return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, 1, out, 1, scale, accum, out_stride, st);
 }
@@ -102,6 +104,41 @@ int glqh_fail(const char *fmt, ...) {
 int glqh_check_hip(hipError_t e, const char *what) {
     if (e == hipSuccess) return 0;
     return glqh_fail("%s: %s", what, hipGetErrorString(e));
+}
+
+// ---- profiling ranges ---------------------------------------------------------------
+#include <dlfcn.h>
+static struct {
+    std::once_flag once;
+    int (*push)(const char *);
+    int (*pop)(void);
+} g_roctx;
+
+static void roctx_resolve() {
+    const char *e = getenv("GLQ_ROCTX");
+    if (e && e[0] == '0') return;
+    const int mode = (e && e[0] == '1') ? RTLD_NOW | RTLD_GLOBAL : RTLD_NOW | RTLD_NOLOAD;
+    const char *names[] = {"librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4",
+                           "libroctx64.so"};
+    for (const char *n : names) {
+        void *h = dlopen(n, mode);
+        if (!h) continue;
+        void *pu = dlsym(h, "roctxRangePushA"), *po = dlsym(h, "roctxRangePop");
+        if (pu && po) {
+            g_roctx.push = (int (*)(const char *))pu;
+            g_roctx.pop = (int (*)(void))po;
+            return;
+        }
+    }
+}
+
+glqh_range::glqh_range(const char *name) {
+    std::call_once(g_roctx.once, roctx_resolve);
+    on = g_roctx.push != nullptr;
+    if (on) g_roctx.push(name);
+}
+glqh_range::~glqh_range() {
+    if (on) g_roctx.pop();
 }
 
 static int g_cus = 0;
@@ -139,6 +176,16 @@ extern "C" int glqh_init(void) {
     } while (0)
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// GLQ_TRELLIS_FUSE_INPUT=0 keeps the input transform a launch of its own at every token count,
+// the reference's switch of the same name (glq/csrc/glq_trellis.cu:1270-1274).  Read once.
+static bool tr_fuse_input_enabled() {
+    static const bool on = [] {
+        const char *e = getenv("GLQ_TRELLIS_FUSE_INPUT");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
 
 // ---- trellis ---------------------------------------------------------------------
 extern "C" int glqh_trellis_kernel_supported(int64_t m, int64_t k) {
@@ -366,7 +413,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     // folded form grows by a quarter per extra token and the separate one hardly at all, so two
     // tokens fold only single power-of-two blocks (10.8 vs 11.3, 14.7 vs 15.8; 960 x 960: 12.7 vs
     // 9.4) and three or four tokens never do (2048 x 2048: 13.6 vs 11.5; 8192 x 8192: 38 vs 26).
-    const bool fi_pays = m_pad * n_pad <= ((int64_t)32 << 20) && (B == 1 || (B == 2 && pow2_n));
+    const bool fi_pays = tr_fuse_input_enabled() && m_pad * n_pad <= ((int64_t)32 << 20) &&
+                         (B == 1 || (B == 2 && pow2_n));
     if (fi_pays && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
         (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0 &&
         (!has_s2 || (B == 1 && fi_mode == 2 && merge2))) {
@@ -501,6 +549,7 @@ static bool tr_group_plain(int64_t total_m_pad, int64_t n_pad, int64_t B) {
     const int64_t w = total_m_pad * n_pad;
     // q/k/v of a 4096-wide model (25M weights): 22.1 / 25.6 / 28.5 us folded at 2 / 3 / 4 tokens,
     // 24.5 / 24.5 / 25.1 us separate; gate/up 2048 -> 2 x 11008 (45M): 19-22 us folded, 25-26 separate
+    if (!tr_fuse_input_enabled()) return true;
     return B >= 2 && (w > ((int64_t)48 << 20) || (B >= 3 && n_pad >= 4096 && w > ((int64_t)16 << 20)));
 }
 static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {

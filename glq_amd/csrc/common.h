@@ -25,6 +25,18 @@ int glqh_fail(const char *fmt, ...);             // sets the thread-local messag
 int glqh_check_hip(hipError_t e, const char *what);
 int glqh_device_cus(void);                       // cached compute-unit count
 
+// Named host-side range around the launches of one phase of a linear, under the reference's
+// three names (glq/quantized_linear.py:1132-1233: "input_rht", "dequant_matmul", "output_rht"),
+// for rocprofv3 --marker-trace.  Uses the roctx library when the process already has one loaded
+// (torch does) or GLQ_ROCTX=1 asks to load it; GLQ_ROCTX=0 switches the ranges off.
+struct glqh_range {
+    bool on;
+    explicit glqh_range(const char *name);
+    ~glqh_range();
+    glqh_range(const glqh_range &) = delete;
+    glqh_range &operator=(const glqh_range &) = delete;
+};
+
 #define GLQH_REQUIRE(cond, ...)            \
     do {                                   \
         if (!(cond)) return glqh_fail(__VA_ARGS__); \

@@ -329,6 +329,7 @@ int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t 
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream, const float *pscale) {
+    glqh_range range("dequant_matmul");
     glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
     if (pscale)
         for (int i = 0; i < 4; ++i) ps.v[i] = pscale[i];

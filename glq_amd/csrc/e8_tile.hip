@@ -421,6 +421,7 @@ int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages) {
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
                         int64_t n_pad, float *part, hipStream_t stream) {
+    glqh_range range("dequant_matmul");
     et_plan p;
     if (!et_make_plan(m_pad, n_pad, M, nstages, &p)) return glqh_fail("e8 tile kernel: shape not eligible (n_pad %% 256)");
     hipLaunchKernelGGL(e8_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((n_pad / 8 + 15) / 16)),

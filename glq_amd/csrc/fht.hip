@@ -484,6 +484,7 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
                           void *out, int out_dtype, int64_t B, int64_t in_features, int64_t n_pad,
                           const glqh_block_meta *meta_dev, const int64_t *blocks_host,
                           int64_t n_blocks, float rsqrt_n, hipStream_t stream) {
+    glqh_range range("input_rht");
     GLQH_REQUIRE(x && sv && out, "input_rht: null pointer");
     GLQH_REQUIRE(B >= 1 && B <= 65535, "input_rht: B=%lld out of range", (long long)B);
     GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad,
@@ -555,6 +556,7 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
                            const glqh_block_meta *meta_dev, const int64_t *blocks_host,
                            int64_t n_blocks, int64_t max_bs_hint, float rsqrt_m,
                            hipStream_t stream) {
+    glqh_range range("output_rht");
     GLQH_REQUIRE(B >= 1 && B <= 65535, "output_rht: B=%lld out of range", (long long)B);
     GLQH_REQUIRE(y != nullptr && su != nullptr, "output_rht: null y or su");
     GLQH_REQUIRE(out_features >= 1 && out_features <= m_pad,
@@ -633,6 +635,7 @@ int glqh_launch_output_rht_group(const float *const part[], const void *const su
                                  const float scale[], const int64_t m_pad[], const int64_t out_features[],
                                  int n_shards, int y_dtype, int64_t y_stride, int64_t B, int ksplit,
                                  hipStream_t stream) {
+    glqh_range range("output_rht");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_GROUP, "output_rht group: 1..%d shards", GLQH_MAX_GROUP);
     GLQH_REQUIRE(B >= 1 && B <= 65535, "output_rht group: B=%lld out of range", (long long)B);
     GLQH_REQUIRE(y_dtype == GLQH_F16 || y_dtype == GLQH_BF16 || y_dtype == GLQH_F32, "output_rht group: bad y dtype");

@@ -427,6 +427,7 @@ int glqh_launch_trellis_fusein(const void *packed, int R, const void *x, int x_d
                                int steps, int ksplit, const glqh_block_meta *bn_meta,
                                const int64_t *blocks_host, int n_blocks, float *part,
                                hipStream_t stream) {
+    glqh_range range("dequant_matmul");
     switch (R) {
     case 2: return launch_fusein_R<2>(packed, x, x_dtype, x_stride, sv, B, m, k, in_features, steps, ksplit, bn_meta, blocks_host, n_blocks, part, stream);
     case 3: return launch_fusein_R<3>(packed, x, x_dtype, x_stride, sv, B, m, k, in_features, steps, ksplit, bn_meta, blocks_host, n_blocks, part, stream);
@@ -456,6 +457,7 @@ int glqh_launch_trellis_fusein_group(const void *const packed[], const void *con
                                      int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int steps,
                                      int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
                                      int n_blocks, hipStream_t stream) {
+    glqh_range range("dequant_matmul");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_GROUP, "trellis group: 1..%d shards", GLQH_MAX_GROUP);
     tr_fusein_group g = {};
     int64_t max_m = 0;

@@ -592,6 +592,7 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
                                    int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
                                    int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
                                    int n_blocks, float pscale, hipStream_t stream) {
+    glqh_range range("dequant_matmul");
     GLQH_REQUIRE(n_layers >= 1 && n_layers <= GLQH_MAX_GROUP, "trellis group: 1..%d layers", GLQH_MAX_GROUP);
     GLQH_REQUIRE(n_layers == 1 || pscale == 1.0f, "trellis group: pre-scaled partial sums are a single-layer option");
     GLQH_REQUIRE(B >= 1 && B <= 4, "fused-input trellis kernel serves 1..4 tokens");

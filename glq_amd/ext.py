@@ -32,6 +32,9 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 # 1265-1268, 1322-1334) -- is kept behind its tunable: GLQ_TRELLIS_BATCH_MAX=<n> sends calls above
 # n tokens there.
 TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", str(1 << 30))))
+# GLQ_TRELLIS_DENSE (set to anything) sends every fused trellis call to that dense route, the
+# reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
+TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ
 # E8 layers stay on their compressed indices at every token count (above 16 tokens: one lookup per
 # weight and 128 x 512 tile, csrc/e8_tile.hip); GLQ_E8_BATCH_MAX=<n> sends calls above n tokens to
 # the dense route instead.
@@ -257,7 +260,7 @@ def _fused_trellis(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_m
     yrp, yrs = C.c_void_p(0), 0
     if y_rht_out is not None:
         yrp, yrs = y_rht_out
-    if B > TRELLIS_BATCH_MAX and y_rht_out is None:
+    if (TRELLIS_DENSE or B > TRELLIS_BATCH_MAX) and y_rht_out is None:
         if (packed2 is not None and packed2.numel() > 0) != (float(inv_rs2) != 0.0):
             raise RuntimeError("trellis RVQ stage 2 is half-configured: trellis_packed2 is "
                                f"{'present' if has2 else 'absent'} but inv_resid_scale2 = {inv_rs2}")

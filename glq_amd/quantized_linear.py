@@ -16,6 +16,7 @@ Buffers
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 import torch.nn as nn
@@ -37,6 +38,12 @@ def _codebook_tensor(cb):
 
 
 _MAX_TOKENS_PER_CALL = 32768
+
+# GLQ_FUSED_TRELLIS=0 replaces the single fused trellis call by its three parts, each an op of
+# its own (input transform, one decode matmul per stage, output transform): the reference's
+# kill-switch of the same name (glq/quantized_linear.py:23-30), there for A/B runs.  The parts
+# are still HIP kernels; there is no torch decode in this build.
+_GLQ_FUSED_TRELLIS_ENABLED = os.environ.get("GLQ_FUSED_TRELLIS", "1") != "0"
 
 class E8RHTLinear(nn.Module):
     def __init__(self, in_features: int, out_features: int, bias: bool = False,
@@ -210,7 +217,17 @@ class E8RHTLinear(nn.Module):
         x = x.contiguous()
         has_s2 = trellis_packed2 is not None and trellis_packed2.numel() > 0
         ops = torch.ops.glq if hasattr(torch.ops, "glq") else None
-        if has_s2:
+        if not _GLQ_FUSED_TRELLIS_ENABLED:
+            x_rht = torch.empty((x.shape[0], n_pad), dtype=torch.float16, device=x.device)
+            ext.glq_input_rht_blockdiag_cuda(x, SV, x_rht, in_features, n_pad, blocks_n, blocks_n_meta)
+            y_rht = ext.glq_decode_matmul_trellis_3inst_cuda(x_rht, trellis_packed, m_pad, n_pad, float(wscale))
+            if has_s2:
+                ext.glq_decode_matmul_trellis_3inst_cuda(
+                    x_rht, trellis_packed2, m_pad, n_pad, float(wscale) * float(inv_resid_scale2),
+                    out=y_rht, accum=True)
+            y = torch.empty((x.shape[0], out_features), dtype=x.dtype, device=x.device)
+            ext.glq_output_rht_blockdiag_cuda(y_rht, SU, y, out_features, m_pad, blocks_m, blocks_m_meta)
+        elif has_s2:
             fn = getattr(ops, "fused_linear_trellis_3inst_rvq2", None) if ops is not None else None
             args = (x, SV, SU, trellis_packed, trellis_packed2, blocks_n, blocks_m, blocks_n_meta,
                     blocks_m_meta, float(wscale), float(inv_resid_scale2), in_features, out_features,

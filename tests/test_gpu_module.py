@@ -250,3 +250,89 @@ def test_graph_capture_and_replay_is_bit_exact():
     g.replay()
     torch.cuda.synchronize()
     assert torch.equal(y, layer(xs))
+
+
+def _two_stage_module(m, n, seed):
+    from glq_amd.quantized_linear import E8RHTLinear
+    p1, p2 = O.random_packed(m, n, 4, seed), O.random_packed(m, n, 2, seed + 1)
+    su, sv = O.rht_signs(m, n, 42)
+    art = {"trellis_packed": p1, "trellis_packed2": p2, "inv_resid_scale2": np.float32(0.3),
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
+           "blocks_m": O.block_decompose(m), "blocks_n": O.block_decompose(n)}
+    lin = E8RHTLinear(n, m, codebook_type="trellis")
+    lin.load_state_dict({"trellis_packed": torch.from_numpy(p1), "trellis_packed2": torch.from_numpy(p2),
+                         "SU": torch.from_numpy(art["SU"]), "SV": torch.from_numpy(art["SV"]),
+                         "Wscale": torch.tensor(0.02), "inv_resid_scale2": torch.tensor(0.3)}, strict=False)
+    return lin.to(DEV), art
+
+
+@pytest.mark.parametrize("B", [1, 5, 70])
+def test_reference_switches_fused_trellis_and_trellis_dense(B, monkeypatch):
+    """GLQ_FUSED_TRELLIS=0 (three separate ops) and GLQ_TRELLIS_DENSE (dequantize + library GEMM),
+    the reference's A/B switches (glq/quantized_linear.py:23-30, glq/csrc/glq_trellis.cu:1023-1029):
+    both against the oracle, tolerance 1e-2 relative Frobenius."""
+    from glq_amd import ext, quantized_linear as QL
+    m, n = 512, 1024
+    say("trellis switches", B)
+    lin, art = _two_stage_module(m, n, 11)
+    x = torch.randn(B, n).to(torch.bfloat16)
+    ref = O.trellis_linear_forward(x.float().numpy(), art, n, m)
+    y0 = lin(x.to(DEV))
+    assert rel(y0, ref) < TOL
+    monkeypatch.setattr(QL, "_GLQ_FUSED_TRELLIS_ENABLED", False)
+    y1 = lin(x.to(DEV))
+    assert y1.shape == y0.shape and y1.dtype == y0.dtype and rel(y1, ref) < TOL
+    monkeypatch.setattr(QL, "_GLQ_FUSED_TRELLIS_ENABLED", True)
+    monkeypatch.setattr(ext, "TRELLIS_DENSE", True)
+    y2 = lin(x.to(DEV))
+    assert rel(y2, ref) < TOL
+
+
+def test_reference_switch_fuse_input_off_in_a_fresh_process(tmp_path):
+    """GLQ_TRELLIS_FUSE_INPUT=0 (glq/csrc/glq_trellis.cu:1270-1274) is read once by the library, so
+    the run with it set is a process of its own: same layer, same input, one token and three,
+    single call and grouped call; its outputs agree with this process's within 1e-2."""
+    import os
+    import subprocess
+    import sys
+    from glq_amd import ext, hadamard as H
+    m, n = 2048, 2048
+    say("fuse-input switch, child process")
+    script = r'''
+import sys, numpy as np, torch
+sys.path.insert(0, %r)
+from oracle import glq_oracle as O
+from glq_amd import ext, hadamard as H
+m, n = 2048, 2048
+dev = "cuda"
+p = torch.from_numpy(O.random_packed(m, n, 4, 3)).to(dev)
+su, sv = O.rht_signs(m, n, 42)
+su, sv = torch.from_numpy(su.astype(np.float16)).to(dev), torch.from_numpy(sv.astype(np.float16)).to(dev)
+bn = O.block_decompose(n)
+outs = {}
+for B in (1, 3):
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).to(torch.bfloat16).to(dev)
+    outs["single%%d" %% B] = ext.glq_fused_linear_trellis_3inst_cuda(
+        x, sv, su, p, torch.tensor(bn), torch.tensor(bn), H.pack_block_meta(bn).to(dev),
+        H.pack_block_meta(bn).to(dev), 0.02, n, m, n, m, out_dtype=torch.float32).cpu().numpy()
+    outs["group%%d" %% B] = ext.glq_fused_linear_trellis_3inst_group(
+        x, [(sv, su, p, 0.02, m, m)] * 2, torch.tensor(bn), H.pack_block_meta(bn).to(dev), n, n,
+        out_dtype=torch.float32)[:, m:].cpu().numpy()
+np.savez(sys.argv[1], **outs)
+''' % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    files = {}
+    for tag, env in (("on", {}), ("off", {"GLQ_TRELLIS_FUSE_INPUT": "0"})):
+        files[tag] = str(tmp_path / f"{tag}.npz")
+        r = subprocess.run([sys.executable, "-c", script, files[tag]], env={**os.environ, **env},
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+    a, b = np.load(files["on"]), np.load(files["off"])
+    for k in a.files:
+        assert np.isfinite(b[k]).all() and rel(a[k], b[k]) < TOL, k
+    # and both are the oracle's result
+    x = torch.randn(1, n, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    su, sv = O.rht_signs(m, n, 42)
+    W = O.decode_layer(O.random_packed(m, n, 4, 3), m, n, fast=True) * np.float32(0.02)
+    bn = O.block_decompose(n)
+    ref = O.linear_forward_rht(x.float().numpy(), W, su.astype(np.float32), sv.astype(np.float32), bn, bn, n, m)
+    assert rel(b["single1"], ref) < TOL and rel(a["single1"], ref) < TOL

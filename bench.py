@@ -122,6 +122,14 @@ def extras(torch, ext, dev):
     bound, and the prefill tiles (config 4 shape)."""
     out = {}
     try:
+        # what one more kernel node costs in a captured stream: 2000 dependent one-workgroup fill
+        # kernels (the floor under each of the step's eight launches)
+        tiny = torch.empty(1, device=dev)
+        out["graph_node_floor_us"] = round(_graph_time(
+            torch, lambda: [tiny.zero_() for _ in range(2000)], 2000), 2)
+    except Exception as e:
+        out["graph_node_floor_error"] = f"{type(e).__name__}: {e}"
+    try:
         from glq_amd.decoder import TrellisDecoder
         dec = TrellisDecoder(max_len=1024)
         ids = torch.randint(0, 128256, (512,), generator=torch.Generator().manual_seed(0))

@@ -121,6 +121,7 @@ def extras(torch, ext, dev):
     batch-1 decode tok/s (config 5), large-layer GEMV rates where the kernels are not launch
     bound, and the prefill tiles (config 4 shape)."""
     out = {}
+    tr_default, e8_default = ext.TRELLIS_BATCH_MAX, ext.E8_BATCH_MAX
     try:
         # what one more kernel node costs in a captured stream: 2000 dependent one-workgroup fill
         # kernels (the floor under each of the step's eight launches)
@@ -211,12 +212,15 @@ def extras(torch, ext, dev):
             us = _graph_time(torch, lambda: [ext.glq_dequant_matmul_cuda(xh, a, cb, 0.02, b, cb, 1 / 3.0)
                                              for a, b in qs], len(qs))
             out[f"e8_2stage_gemv_4096x14336_B{B}_GBs"] = round(m * (n // 8) * 4 / us / 1e3, 1)
-        # config 4, E8 half: the many-token kernel on the same quantized indices (kernel + K-slot sum)
+        # config 4, E8 half: the many-token kernel on the same quantized indices (kernel + K-slot sum),
+        # also at 4096 tokens, where the library route is the default
+        ext.E8_BATCH_MAX = 1 << 30
         for M in (256, 4096):
             xh = torch.randn(M, n, device=dev).to(torch.float16)
             us = _graph_time(torch, lambda: ext.glq_dequant_matmul_cuda(xh, qs[0][0], cb, 0.02, qs[0][1], cb, 1 / 3.0),
                              1, reps=5)
             out[f"e8_2stage_matmul_4096x14336_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        ext.E8_BATCH_MAX = e8_default
         del qs, i1, i2
         torch.cuda.empty_cache()
     except Exception as e:
@@ -236,15 +240,20 @@ def extras(torch, ext, dev):
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
         q1 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
         q2 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
-        for M in (256, 4096):
+        for M, route in ((256, ""), (4096, ""), (4096, "_compressed")):
+            # "" = the route the library picks (compressed up to 2048 tokens, dequantize + library
+            # GEMM above); "_compressed" = the tile kernels forced at 4096 tokens as well
+            ext.TRELLIS_BATCH_MAX = (1 << 30) if route else tr_default
+            ext.E8_BATCH_MAX = (1 << 30) if route else e8_default
             xb = torch.randn(M, n, device=dev).to(torch.bfloat16)
             us = _graph_time(torch, lambda: ext.glq_fused_linear_trellis_3inst_cuda(
                 xb, sv, su, p, bnt, bmt, bnm, bmm, 0.02, n, m, n, m, out_dtype=torch.bfloat16), 1, reps=5)
-            out[f"trellis_linear_14336x4096_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+            out[f"trellis_linear_14336x4096_M{M}{route}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
             us = _graph_time(torch, lambda: ext.glq_fused_linear_block_diag_cuda(
                 xb, sv, su, q1, cbh, 0.02, n, m, n, m, bnt, bmt, bnm, bmm, q2, cbh, 1 / 3.0,
                 out_dtype=torch.bfloat16), 1, reps=5)
-            out[f"e8_2stage_linear_14336x4096_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+            out[f"e8_2stage_linear_14336x4096_M{M}{route}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        ext.TRELLIS_BATCH_MAX, ext.E8_BATCH_MAX = tr_default, e8_default
         del p, q1, q2
         torch.cuda.empty_cache()
     except Exception as e:

@@ -25,20 +25,21 @@ from ._lib import GLQH_BF16, GLQH_F16, GLQH_F32, check
 
 _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F32}
 
-# Every token count is served on the compressed weights: 1-64 tokens by the GEMV / small-batch
-# kernels, above by the tile kernels that decode each weight once per 128-row x 512-token tile
-# (csrc/trellis_tile.hip, csrc/e8_tile.hip).  The reference's own many-token route -- dequantize
-# the weight to fp16 once with the HIP kernel, then one library GEMM (glq/csrc/glq_trellis.cu:
-# 1265-1268, 1322-1334) -- is kept behind its tunable: GLQ_TRELLIS_BATCH_MAX=<n> sends calls above
-# n tokens there.
-TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", str(1 << 30))))
+# Up to 2048 tokens every call is served on the compressed weights: 1-64 tokens by the GEMV /
+# small-batch kernels, above by the tile kernels that decode each weight once per 128-row x
+# 512-token tile (csrc/trellis_tile.hip, csrc/e8_tile.hip).  Above that the reference's own
+# many-token route -- dequantize the weight to fp16 once with the HIP kernel, then one library
+# GEMM (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334) -- is the faster one on this chip (measured on
+# 14336 x 4096 and 4096 x 14336, whole fused linear, compressed vs library: trellis 180 / 202 us
+# at 1024 tokens, 321 / 321 at 2048, 610 / 564 at 4096; E8 two-stage 198 / 202, 341 / 346,
+# 664 / 584) at the price of a transient fp16 copy of the weight.  The thresholds are the
+# reference's tunable and its E8 counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send
+# calls above n tokens to the library route (a large n keeps every call compressed).
+TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "2048")))
 # GLQ_TRELLIS_DENSE (set to anything) sends every fused trellis call to that dense route, the
 # reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
 TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ
-# E8 layers stay on their compressed indices at every token count (above 16 tokens: one lookup per
-# weight and 128 x 512 tile, csrc/e8_tile.hip); GLQ_E8_BATCH_MAX=<n> sends calls above n tokens to
-# the dense route instead.
-E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", str(1 << 30))))
+E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "2048")))
 
 
 def _e8_dense_route(B, n_pad):

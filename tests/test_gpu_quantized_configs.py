@@ -226,8 +226,9 @@ def _sample_rows(M):
 
 
 @pytest.mark.parametrize("m,n", [(14336, 4096), (4096, 14336)])
-def test_trellis_prefill_quantized_layer_up_to_4096_tokens(ext, m, n):
+def test_trellis_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatch):
     say("quantized trellis prefill", m, n)
+    monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 1 << 30)     # every size on the packed stream
     _, art, W_dec = trellis_layer(ext, m, n)
     su, sv = art["SU"].astype(np.float32), art["SV"].astype(np.float32)
     args = trellis_args(art, m, n)
@@ -251,11 +252,17 @@ def test_trellis_prefill_quantized_layer_up_to_4096_tokens(ext, m, n):
     rows = _sample_rows(4096)
     r = x[rows].float().numpy() @ W_hat.T
     assert sqnr(r, ys[4096][torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0
+    # the route the library takes by itself above 2048 tokens (dequantize + library GEMM): same result
+    monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 2048)
+    yl = ext.glq_fused_linear_trellis_3inst_cuda(xd, *args, out_dtype=torch.bfloat16)
+    assert rel(yl, ys[4096].float().cpu().numpy()) < 6e-3
+    assert sqnr(r, yl[torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0
 
 
 @pytest.mark.parametrize("m,n", [(14336, 4096), (4096, 14336)])
-def test_e8_prefill_quantized_layer_up_to_4096_tokens(ext, m, n):
+def test_e8_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatch):
     say("quantized e8 prefill", m, n)
+    monkeypatch.setattr(ext, "E8_BATCH_MAX", 1 << 30)          # every size on the compressed indices
     _, art, W_dec = e8_layer(ext, m, n)
     su, sv = art["SU"].astype(np.float32), art["SV"].astype(np.float32)
     x = torch.randn(4096, n, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
@@ -276,3 +283,7 @@ def test_e8_prefill_quantized_layer_up_to_4096_tokens(ext, m, n):
     rows = _sample_rows(4096)
     r = x[rows].float().numpy() @ W_hat.T
     assert sqnr(r, ys[4096][torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0
+    monkeypatch.setattr(ext, "E8_BATCH_MAX", 2048)             # the library route above 2048 tokens
+    yl = e8_forward(ext, xd, art, m, n, torch.bfloat16)
+    assert rel(yl, ys[4096].float().cpu().numpy()) < 6e-3
+    assert sqnr(r, yl[torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0

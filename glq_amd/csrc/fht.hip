@@ -59,10 +59,8 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
 // ---- many tokens: whole blocks, 16-byte accesses ------------------------------------
 // With many tokens the transforms are bound by HBM, and what matters is how many bytes each
 // thread keeps in flight and how the stores coalesce.  A workgroup owns one whole block
-// (at most 8192 points) of one token, every thread moves eight consecutive elements per
-// access (16 bytes of 16-bit data), and the last butterfly pass puts its results back into
-// LDS so that the copy-out can write rows in the same 8-element runs.  Arithmetic and
-// rounding are the same as in the element-wise kernels above.
+// (at most 8192 points) of one token and every thread moves runs of eight consecutive elements
+// (16 bytes of 16-bit data) in and out.
 constexpr int WIDE_LOG_MAX = 13;
 
 template <typename T> __device__ __forceinline__ void load8(const T *p, float *f);
@@ -112,130 +110,164 @@ template <> __device__ __forceinline__ void store8<uint16_t>(uint16_t *p, const 
 }
 
 // blockIdx.x = block, blockIdx.y = token.  Requires canonical blocks of 8..8192 points, 16-byte
-// aligned rows of x (x_stride % 8 == 0 elements for 16-bit types) and out.
-template <typename XT, typename OT>
-__global__ void __launch_bounds__(RHT_THREADS)
-input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
-                      OT *__restrict__ out, int in_features, int n_pad, glqh_meta_args margs,
-                      float single_norm) {
-    extern __shared__ float s[];
-    const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
-    const XT *xr = x + (int64_t)blockIdx.y * x_stride + blk.off;
-    const f16 *svb = sv + blk.off;
-    const int lim = in_features - blk.off;               // elements of the block inside the row
-    constexpr int U = 2;
-    for (int i0 = 8 * threadIdx.x; i0 < blk.bs; i0 += 8 * U * RHT_THREADS) {
-        float xf[U][8], sf[U][8];
+// aligned rows of x (x_stride % 8 == 0 elements for 16-bit types) and out.  The transform runs
+// in registers (fht_wave<E>): thread t of 512 holds elements E*t .. E*t+E-1 of the block (E = 16
+// for 8192 points, 8 below), log2(E) butterfly levels stay in the thread, six run across the
+// lanes, up to log2(E) across the waves through one LDS exchange; the results, which the exchange
+// leaves strided over the threads, pass through LDS once more so that every thread writes a run
+// of E consecutive elements.  84 LDS-pipe instructions per thread for an 8192-point block where
+// passes through LDS (fht_staged) take 320, and three barriers instead of ten: 4096 tokens x
+// 14336 points 117 -> 71 us in, 139 -> 87 us out.
+constexpr int REG_THREADS = 512;
+__device__ __forceinline__ int reg_pad(int p) { return p + ((p >> 5) << 2); }   // 16-byte groups stay whole
+size_t rht_reg_lds_bytes(int log_bs) {
+    const size_t n = (size_t)1 << log_bs;
+    return (n + n / 8 + 16) * sizeof(float);
+}
+
+// v (element tid + q * nthr when the transform went through the exchange, E * tid + q otherwise)
+// -> E consecutive elements E * tid + q, through s.  Every thread of the workgroup calls.
+template <int E>
+__device__ __forceinline__ void reg_gather_runs(float (&v)[E], int log_len, float *s, int tid, bool active) {
+    constexpr int LE = fht_wave_log<E>::v;
+    if (log_len <= 6 + LE) return;                           // uniform: already consecutive
+    const int nthr = 1 << (log_len - LE);
+    __syncthreads();                                         // the exchange buffer has been read
+    if (active) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int i = i0 + 8 * u * RHT_THREADS;
-            if (i < blk.bs) {
-                load8<f16>(svb + i, sf[u]);
-                if (i + 8 <= lim) load8<XT>(xr + i, xf[u]);
-                else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) xf[u][e] = i + e < lim ? act_to_f32<XT>(xr[i + e]) : 0.0f;
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int i = i0 + 8 * u * RHT_THREADS;
-            if (i < blk.bs) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) s[lds_pad(i + e)] = xf[u][e] * sf[u][e];
-            }
-        }
+        for (int q = 0; q < E; ++q) s[reg_pad(tid + q * nthr)] = v[q];
     }
     __syncthreads();
-    fht_staged(s, blk.log_len, lds_writeback{s});
-    __syncthreads();
-    OT *orow = out + (int64_t)blockIdx.y * n_pad + blk.off;
-    for (int i = 8 * threadIdx.x; i < blk.bs; i += 8 * RHT_THREADS) {
-        float v[8];
+    if (active) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = s[lds_pad(i + e)] * blk.norm;
-        store8<OT>(orow + i, v);
+        for (int q = 0; q < E; q += 4) {
+            const f32x4 w = *(const f32x4 *)(s + reg_pad(E * tid + q));
+            v[q] = w[0]; v[q + 1] = w[1]; v[q + 2] = w[2]; v[q + 3] = w[3];
+        }
     }
 }
 
-// src: direct rows (stride % 4 == 0) or split-K partials; y rows 16-byte aligned.
-template <typename YT>
-__global__ void __launch_bounds__(RHT_THREADS)
-output_rht_wide_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
-                       int out_features, int m_pad, glqh_meta_args margs, float single_norm) {
+template <int E, typename XT, typename OT>
+__device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, int64_t x_stride,
+                                                   const f16 *__restrict__ sv, OT *__restrict__ out,
+                                                   int in_features, int n_pad, const rht_slice &blk, float *s) {
+    const int tid = threadIdx.x;
+    const bool active = E * tid < blk.bs;
+    const int i = E * tid;
+    float v[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = 0.0f;
+    if (active) {
+        const XT *xr = x + (int64_t)blockIdx.y * x_stride + blk.off;
+        const int lim = in_features - blk.off;               // elements of the block inside the row
+        float sf[E];
+#pragma unroll
+        for (int e = 0; e < E; e += 8) load8<f16>(sv + blk.off + i + e, sf + e);
+        if (i + E <= lim) {
+#pragma unroll
+            for (int e = 0; e < E; e += 8) load8<XT>(xr + i + e, v + e);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) v[e] = i + e < lim ? act_to_f32<XT>(xr[i + e]) : 0.0f;
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] *= sf[e];
+    }
+    fht_wave<E>(v, blk.log_len, s, tid);
+    reg_gather_runs<E>(v, blk.log_len, s, tid, active);
+    if (active) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] *= blk.norm;
+        OT *orow = out + (int64_t)blockIdx.y * n_pad + blk.off + i;
+#pragma unroll
+        for (int e = 0; e < E; e += 8) store8<OT>(orow + e, v + e);
+    }
+}
+
+// blocks of 8192 points take 16 elements per thread, smaller ones 8 (all 512 threads busy on 4096)
+template <typename XT, typename OT>
+__global__ void __launch_bounds__(REG_THREADS)
+input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
+                     OT *__restrict__ out, int in_features, int n_pad, glqh_meta_args margs,
+                     float single_norm) {
     extern __shared__ float s[];
     const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
+    if (blk.log_bs > 12) input_rht_wide_body<16, XT, OT>(x, x_stride, sv, out, in_features, n_pad, blk, s);
+    else input_rht_wide_body<8, XT, OT>(x, x_stride, sv, out, in_features, n_pad, blk, s);
+}
+
+template <int E, typename YT>
+__device__ __forceinline__ void output_rht_wide_body(const glqh_ysrc &src, const f16 *__restrict__ su,
+                                                    YT *__restrict__ y, int64_t y_stride, int out_features,
+                                                    int m_pad, const rht_slice &blk, float *s) {
     const int64_t b = blockIdx.y;
-    if (src.nparts == 0) {
-        const float *__restrict__ d = src.direct + b * src.stride + blk.off;
-        constexpr int U = 2;
-        for (int i0 = 8 * threadIdx.x; i0 < blk.bs; i0 += 8 * U * RHT_THREADS) {
-            float v[U][8];
+    const int tid = threadIdx.x;
+    const bool active = E * tid < blk.bs;
+    const int i = E * tid;
+    float v[E];
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (i0 + 8 * u * RHT_THREADS < blk.bs) load8<float>(d + i0 + 8 * u * RHT_THREADS, v[u]);
+    for (int e = 0; e < E; ++e) v[e] = 0.0f;
+    if (active) {
+        if (src.nparts == 0) {
+            const float *d = src.direct + b * src.stride + blk.off + i;
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (i0 + 8 * u * RHT_THREADS < blk.bs) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) s[lds_pad(i0 + 8 * u * RHT_THREADS + e)] = v[u][e];
-                }
-        }
-    } else {
-        // v = sum_stage scale * (sum_k partial), in this fixed order (as stage_partials)
-        const float *__restrict__ pbase = src.part + b * (int64_t)m_pad + blk.off;
-        for (int i = 8 * threadIdx.x; i < blk.bs; i += 8 * RHT_THREADS) {
-            float v[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+            for (int e = 0; e < E; e += 8) load8<float>(d + e, v + e);
+        } else {
+            // v = sum_stage scale * (sum_k partial), in this fixed order (as stage_partials)
+            const float *pbase = src.part + b * (int64_t)m_pad + blk.off + i;
             for (int st = 0; st < src.nparts; ++st) {
-                float acc[8];
+                float acc[E];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
-                const float *p = pbase + st * src.part_sstride + i;
-                int k = 0;
-                for (; k + 2 <= src.ksplit; k += 2) {            // two terms in flight
-                    float t0[8], t1[8];
-                    load8<float>(p + k * src.part_kstride, t0);
-                    load8<float>(p + (k + 1) * src.part_kstride, t1);
+                for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+                const float *p = pbase + st * src.part_sstride;
+                for (int k = 0; k < src.ksplit; ++k) {
+                    float t0[E];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[e] = (acc[e] + t0[e]) + t1[e];
-                }
-                if (k < src.ksplit) {
-                    float t0[8];
-                    load8<float>(p + k * src.part_kstride, t0);
+                    for (int e = 0; e < E; e += 8) load8<float>(p + k * src.part_kstride + e, t0 + e);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[e] += t0[e];
+                    for (int e = 0; e < E; ++e) acc[e] += t0[e];
                 }
                 const float sc = st == 0 ? src.scale[0] : st == 1 ? src.scale[1]
                                : st == 2 ? src.scale[2] : src.scale[3];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] += sc * acc[e];
+                for (int e = 0; e < E; ++e) v[e] += sc * acc[e];
             }
-            if (src.copy_out) store8<float>(src.copy_out + b * src.copy_stride + blk.off + i, v);
+            if (src.copy_out) {
+                float *c = src.copy_out + b * src.copy_stride + blk.off + i;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s[lds_pad(i + e)] = v[e];
+                for (int e = 0; e < E; e += 8) store8<float>(c + e, v + e);
+            }
         }
     }
-    __syncthreads();
-    fht_staged(s, blk.log_len, lds_writeback{s});
-    __syncthreads();
-    YT *yrow = y + b * y_stride;
-    for (int i = 8 * threadIdx.x; i < blk.bs; i += 8 * RHT_THREADS) {
-        const int row = blk.off + i;
-        if (row >= out_features) continue;
-        float f[8], v[8];
-        load8<f16>(su + row, f);                                 // su has m_pad entries
+    fht_wave<E>(v, blk.log_len, s, tid);
+    reg_gather_runs<E>(v, blk.log_len, s, tid, active);
+    const int row = blk.off + i;
+    if (active && row < out_features) {
+        float f[E];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = s[lds_pad(i + e)] * (blk.norm * f[e]);
-        if (row + 8 <= out_features) store8<YT>(yrow + row, v);
-        else {
+        for (int e = 0; e < E; e += 8) load8<f16>(su + row + e, f + e);   // su has m_pad entries
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
+        for (int e = 0; e < E; ++e) v[e] *= blk.norm * f[e];
+        YT *yrow = y + b * y_stride;
+        if (row + E <= out_features) {
+#pragma unroll
+            for (int e = 0; e < E; e += 8) store8<YT>(yrow + row + e, v + e);
+        } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
                 if (row + e < out_features) yrow[row + e] = f32_to_act<YT>(v[e]);
         }
     }
+}
+
+template <typename YT>
+__global__ void __launch_bounds__(REG_THREADS)
+output_rht_wide_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
+                      int out_features, int m_pad, glqh_meta_args margs, float single_norm) {
+    extern __shared__ float s[];
+    const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
+    if (blk.log_bs > 12) output_rht_wide_body<16, YT>(src, su, y, y_stride, out_features, m_pad, blk, s);
+    else output_rht_wide_body<8, YT>(src, su, y, y_stride, out_features, m_pad, blk, s);
 }
 
 template <typename YT, bool PARTS>
@@ -510,9 +542,9 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
     if (rht_wide_ok(B, margs, n_pad, max_bs) && aligned16(x) && aligned16(out) && aligned16(sv) &&
         (x_stride * x_size) % 16 == 0 && (n_pad * o_size) % 16 == 0) {
         dim3 wgrid((unsigned)n_blocks, (unsigned)B);
-        const size_t lds = rht_lds_bytes(WIDE_LOG_MAX < 63 && max_bs < (1 << WIDE_LOG_MAX) ? ilog2(max_bs) : WIDE_LOG_MAX);
+        const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
 #define GLQH_INW_LAUNCH(XT, OT)                                                                     \
-    hipLaunchKernelGGL((input_rht_wide_kernel<XT, OT>), wgrid, dim3(RHT_THREADS), lds, stream,      \
+    hipLaunchKernelGGL((input_rht_wide_kernel<XT, OT>), wgrid, dim3(REG_THREADS), lds, stream,      \
                        (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
                        (int)n_pad, margs, rsqrt_n)
         if (out_dtype == GLQH_F32) {
@@ -595,9 +627,9 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
         if (rht_wide_ok(Bw, margs, m_pad, max_bs) && src_ok && aligned16(y) && aligned16(su) &&
             (y_stride * y_size) % 16 == 0) {
             dim3 wgrid((unsigned)n_blocks, (unsigned)B);
-            const size_t lds = rht_lds_bytes(max_bs < (1 << WIDE_LOG_MAX) ? ilog2(max_bs) : WIDE_LOG_MAX);
+            const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
 #define GLQH_OUTW_LAUNCH(YT)                                                                        \
-    hipLaunchKernelGGL((output_rht_wide_kernel<YT>), wgrid, dim3(RHT_THREADS), lds, stream, src,    \
+    hipLaunchKernelGGL((output_rht_wide_kernel<YT>), wgrid, dim3(REG_THREADS), lds, stream, src,    \
                        (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, margs, rsqrt_m)
             if (y_dtype == GLQH_F16) GLQH_OUTW_LAUNCH(f16);
             else if (y_dtype == GLQH_BF16) GLQH_OUTW_LAUNCH(uint16_t);

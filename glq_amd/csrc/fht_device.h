@@ -145,6 +145,7 @@ struct lds_writeback {                                   // last pass: results s
 template <int E> struct fht_wave_log { };
 template <> struct fht_wave_log<4> { static constexpr int v = 2; };
 template <> struct fht_wave_log<8> { static constexpr int v = 3; };
+template <> struct fht_wave_log<16> { static constexpr int v = 4; };
 
 template <int E>
 __device__ __forceinline__ constexpr int fht_wave_max_log() { return 6 + 2 * fht_wave_log<E>::v; }

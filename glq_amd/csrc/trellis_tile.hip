@@ -84,7 +84,8 @@ tr_tile_kernel(const tt_args a) {
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
         // two operands (row groups 2 ms, 2 ms + 1 of the 64-row unit) from half a record
-        auto emit = [&](const tr_record<R> &r, u32x4 *dst) {
+        // half = -1: both operands; 0 / 1: operand rh = half only (the step's two halves each decode one)
+        auto emit = [&](const tr_record<R> &r, u32x4 *dst, int half = -1) {
             uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
             uint32_t n0, n1;
             if constexpr (R >= 2) {
@@ -103,11 +104,13 @@ tr_tile_kernel(const tt_args a) {
             uint32_t h0[8], h1[8];                              // k-tiles 0 and 1 of m-tile ms
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
+                if (half >= 0 && ((j >> 1) & 1) != half) continue;   // operand rh takes states 2rh, 2rh+1, 2rh+4, 2rh+5
                 h0[j] = tr_hash(tr_state<R>(c0, n0, j));
                 h1[j] = tr_hash(tr_state<R>(c1, n1, j));
             }
 #pragma unroll
             for (int rh = 0; rh < 2; ++rh) {
+                if (half >= 0 && rh != half) continue;
                 const int j0 = 2 * rh;
                 const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1],
                                            h1[j0 + 4], h1[j0 + 5]);
@@ -156,18 +159,25 @@ tr_tile_kernel(const tt_args a) {
             const int dn = min(d + 1, ds1 - 1);
             if constexpr (BDB) load_b(b[par ^ 1], d + 1);
             const tr_record<R> r3 = load_rec(d + 3);
+            // operands two multiplications ahead: an LDS read takes longer than the NTW MFMAs of one operand
             f16x8 afn = __builtin_bit_cast(f16x8, rd[lane]);
+            f16x8 afn2 = __builtin_bit_cast(f16x8, rd[GLQH_WAVE + lane]);
             __builtin_amdgcn_sched_barrier(0);                  // requests stay ahead of the multiplications
 #pragma unroll
             for (int kk = 0; kk < 2 * TT_FRAGS; ++kk) {
                 const int u = kk / TT_FRAGS, f = kk % TT_FRAGS;
                 const f16x8 af = afn;
-                if (kk + 1 < 2 * TT_FRAGS) afn = __builtin_bit_cast(f16x8, rd[(kk + 1) * GLQH_WAVE + lane]);
+                afn = afn2;
+                if (kk + 2 < 2 * TT_FRAGS) afn2 = __builtin_bit_cast(f16x8, rd[(kk + 2) * GLQH_WAVE + lane]);
 #pragma unroll
                 for (int tt = 0; tt < NTW; ++tt)
                     acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                         af, __builtin_bit_cast(f16x8, b[cur][tt][u]), acc[f][tt], 0, 0, 0);
-                if (kk == 1) emit(r1, wr);                      // operands of d + 1 (unused after the last step)
+                // operands of d + 1 (unused after the last step), one per half of the step: spread over
+                // the step the decode fits under the MFMAs, bunched into one half it out-issues them
+                if (kk == 1) emit(r1, wr, 0);
+                if (kk == TT_FRAGS) __builtin_amdgcn_sched_barrier(0);
+                if (kk == TT_FRAGS + 1) emit(r1, wr, 1);
                 if constexpr (!BDB) {
                     if (f == TT_FRAGS - 1) {                    // this half's activations are free: request the next
                         __builtin_amdgcn_sched_barrier(0);

@@ -54,6 +54,12 @@ int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M);
 int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
                              hipStream_t stream);
+int64_t glqh_trellis_tile_padded_tokens(int64_t M);
+int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages);
+// input transform straight into a tile kernel's operand layout (fht.hip); -1 = not eligible, nothing launched
+int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, const void *sv, void *xb,
+                                  int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
+                                  const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
 
 // Plan for activations already in the transformed domain: up to 64 tokens share one pass
 // over the packed stream with K split by shape only; larger batches use the tile kernel, which
@@ -445,14 +451,23 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                 return 1;
         }
     } else {
-        if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
-                                  bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
-            return 1;
         const tr_plan plan = tr_plain_plan(m_pad, n_pad, B);
+        // tile kernel: the transform writes the kernel's blocked operand layout itself where it can
+        // (one pass over the activations less, and one repack instead of one per stage)
+        const void *x_in = x_rht;
+        int rc = -1;
+        if (plan.tile)
+            rc = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, sv_f16, xb_tile, 2, glqh_trellis_tile_padded_tokens(B),
+                                               B, in_features, n_pad, blocks_n, n_blocks_n, st);
+        if (rc > 0) return 1;
+        if (rc == 0) x_in = nullptr;
+        else if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
+                                       bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
+            return 1;
         ks = plan.ks;
         if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
-        if (tr_plain_partial(plan, x_rht, B, packed, R1, m_pad, n_pad, part1, xb_tile, st)) return 1;
-        if (has_s2 && tr_plain_partial(plan, x_rht, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2)) return 1;
+        if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st)) return 1;
+        if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2)) return 1;
     }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);
@@ -960,15 +975,23 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
     hipStream_t st = (hipStream_t)stream;
     f16 *x_rht = (f16 *)ws;
     float *part = (float *)((char *)ws + xb);
-    if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
+    // tile kernel: the transform writes the kernel's blocked operand layout itself where it can
+    int blocked = -1;
+    if (tks > 0)
+        blocked = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, sv_f16, (char *)ws + xb + tile_part, 1,
+                                                glqh_e8_tile_padded_tokens(B, sg.n), B, in_features, n_pad,
+                                                blocks_n, n_blocks_n, st);
+    if (blocked > 0) return 1;
+    if (blocked != 0 &&
+        glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
                               bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
         return 1;
     if (tks > 0) {
         // many tokens: one combined product on the compressed indices, summed over its K slots and
         // scaled by the output transform
         const float rel[3] = {(float)inv_rs, (float)inv_rs2, (float)inv_rs3};
-        if (glqh_launch_e8_tile(x_rht, (char *)ws + xb + tile_part, B, sg.q, sg.n, table1, table2 ? table2 : table1, table2 ? n_entries2 : 65536,
-                                rel, m_pad, n_pad, part, st))
+        if (glqh_launch_e8_tile(blocked == 0 ? nullptr : x_rht, (char *)ws + xb + tile_part, B, sg.q, sg.n, table1,
+                                table2 ? table2 : table1, table2 ? n_entries2 : 65536, rel, m_pad, n_pad, part, st))
             return 1;
         glqh_ysrc src = {};
         src.nparts = 1;

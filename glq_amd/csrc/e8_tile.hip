@@ -15,8 +15,10 @@
 // The B operand of the MFMA puts consecutive tokens in consecutive lanes, so row-major activations
 // would be read as 64 scattered 16-byte pieces per instruction (one lane per clock in the memory
 // pipeline: measured 2.7 us per 64-column step and CU, three times the multiplications).  They are
-// repacked once per call into 8-column blocks with the token as the fast index,
-// xb[k / 8][token][k % 8], which turns every operand load into four runs of 256 contiguous bytes.
+// repacked once per call (or written that way by the input transform) into groups of four
+// 8-column blocks with the token as the next index, xb[k / 32][token][(k / 8) % 4][k % 8], which
+// turns every operand load of a wave into two runs of 512 contiguous bytes and keeps the 32
+// columns of one token together (64 bytes) for whoever writes them.
 //
 // Every weight is therefore looked up once per 128 * NTW tokens (once per 512 at NTW = 4), the
 // B operands never pass through LDS, and LDS carries 16 KB of A operands per step and CU.  The
@@ -46,7 +48,7 @@ struct et_args {
     uint32_t n2;
     int t2_is_t1;
     float r[3];                                    // factors of stages 2..4 relative to stage 1
-    const f16 *xb;                                 // transformed activations, (n_pad / 8, Mp, 8) fp16
+    const f16 *xb;                                 // transformed activations, (n_pad / 32, Mp, 4, 8) fp16
     int Mp;                                        // M rounded up to whole token tiles
     int M, m_pad, n_pad;
     int RT, TT, KS, slot_ds;                       // row tiles, token tiles, K slots, 64-column steps per slot
@@ -110,8 +112,9 @@ e8_tile_kernel(const et_args a) {
         for (int s = 0; s < NS; ++s) qrow[s] = (const u32x4 *)(a.q[s] + (int64_t)drow * nblk) + (ds0 >> 2) * 4 + g;
         // multiply role: token 16 * tt + i of the wave's tokens, blocks 8d + 2g and 8d + 2g + 1
         // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
-        const int64_t bstep = (int64_t)a.Mp * 8;                // elements from one block to the next
-        const f16 *xrow = a.xb + (int64_t)(tok0 + i) * 8 + 2 * g * bstep;
+        // block 8 d + 2 g + u of step d: group of four blocks 2 d + (g >> 1), position 2 (g & 1) + u
+        const int64_t kstep = (int64_t)a.Mp * 64;               // elements from one 64-column step to the next
+        const f16 *xrow = a.xb + (int64_t)(g >> 1) * a.Mp * 32 + (int64_t)(tok0 + i) * 32 + (g & 1) * 16;
 
         // Every load below is unconditional with a clamped step index, so the wait counts the
         // compiler derives are exact and nothing waits for a request younger than the one it needs.
@@ -204,8 +207,8 @@ e8_tile_kernel(const et_args a) {
             d = min(d, ds1 - 1);
 #pragma unroll
             for (int tt = 0; tt < NTW; ++tt) {
-                b[tt][0] = *(const u32x4 *)(xrow + 8 * d * bstep + tt * 128);
-                b[tt][1] = *(const u32x4 *)(xrow + (8 * d + 1) * bstep + tt * 128);
+                b[tt][0] = *(const u32x4 *)(xrow + d * kstep + tt * 512);
+                b[tt][1] = *(const u32x4 *)(xrow + d * kstep + 8 + tt * 512);
             }
         };
 
@@ -279,7 +282,7 @@ e8_tile_kernel(const et_args a) {
                         if (f == ET_FRAGS - 1) {                // this half's activations are free: request the next
                             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                            for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + (8 * dn + u) * bstep + tt * 128);
+                            for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + dn * kstep + u * 8 + tt * 512);
                             __builtin_amdgcn_sched_barrier(0);
                         }
                     }
@@ -311,8 +314,8 @@ e8_tile_kernel(const et_args a) {
     }
 }
 
-// (M, n_pad) row-major fp16 -> (n_pad / 8, M, 8): 64 tokens x 16 blocks per workgroup through LDS,
-// both sides in runs of 256 bytes and more.
+// (M, n_pad) row-major fp16 -> (n_pad / 32, Mp, 4, 8): 64 tokens x 16 blocks per workgroup through
+// LDS, reads in runs of 256 bytes, writes in runs of 4 KB.
 __global__ void __launch_bounds__(256)
 e8_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, int Mp, int n_pad) {
     __shared__ u32x4 tile[16][65];
@@ -326,9 +329,10 @@ e8_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, i
     }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int kb = r * 4 + (t >> 6), tl = t & 63;
-        if (tok0 + tl < M && kb0 + kb < nblk) *(u32x4 *)(xb + ((int64_t)(kb0 + kb) * Mp + tok0 + tl) * 8) = tile[kb][tl];
+    for (int r = 0; r < 4; ++r) {                               // group of four blocks r: 64 tokens x 64 bytes contiguous
+        const int tl = t >> 2, pos = t & 3, kb = 4 * r + pos;
+        if (tok0 + tl < M && kb0 + kb < nblk)
+            *(u32x4 *)(xb + ((((int64_t)(kb0 + kb) >> 2) * Mp + tok0 + tl) * 4 + pos) * 8) = tile[kb][tl];
     }
 }
 
@@ -418,15 +422,21 @@ int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages) {
 // part[(slot * M + token) * m_pad + row] = sum over the slot's columns of x[token, k] * W[row, k],
 // W = cb[q0] + rel[0] * cb2[q1] + rel[1] * cb[q2] + rel[2] * cb[q3] (nstages terms), unscaled.
 // x_f16 is (M, n_pad) row-major; xb_scratch takes its repacked copy (glqh_e8_tile_xb_bytes).
+// tokens of the blocked activation layout: M padded to whole workgroup tiles
+int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages) { return et_padded_tokens(M, nstages); }
+
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
                         int64_t n_pad, float *part, hipStream_t stream) {
     glqh_range range("dequant_matmul");
     et_plan p;
     if (!et_make_plan(m_pad, n_pad, M, nstages, &p)) return glqh_fail("e8 tile kernel: shape not eligible (n_pad %% 256)");
-    hipLaunchKernelGGL(e8_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((n_pad / 8 + 15) / 16)),
-                       dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, (int)et_padded_tokens(M, nstages), (int)n_pad);
-    GLQH_LAUNCH_CHECK("e8 pack launch");
+    if (x_f16) {                                               // NULL: xb_scratch already holds the blocked layout
+        hipLaunchKernelGGL(e8_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((n_pad / 8 + 15) / 16)),
+                           dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M,
+                           (int)et_padded_tokens(M, nstages), (int)n_pad);
+        GLQH_LAUNCH_CHECK("e8 pack launch");
+    }
     et_args a;
     for (int s = 0; s < 4; ++s) a.q[s] = (const uint16_t *)q[s];
     a.t1 = t1;

@@ -147,10 +147,15 @@ __device__ __forceinline__ void reg_gather_runs(float (&v)[E], int log_len, floa
     }
 }
 
-template <int E, typename XT, typename OT>
+// LAYOUT of the transformed row: 0 = row-major (out + token * n_pad); 1 and 2 = the tile kernels'
+// operand layouts out[col / 32][token][4][8]: 32 columns of one token are 64 contiguous bytes, as
+// four 8-column blocks in order (1, E8) or as the four slots q = 0..3 holding columns
+// 2q + {0,1,8,9,16,17,24,25} of the k-pair (2, trellis).  Both save the tile kernels' repacking pass.
+template <int E, typename XT, typename OT, int LAYOUT>
 __device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, int64_t x_stride,
                                                    const f16 *__restrict__ sv, OT *__restrict__ out,
-                                                   int in_features, int n_pad, const rht_slice &blk, float *s) {
+                                                   int in_features, int n_pad, int Mp, int token,
+                                                   const rht_slice &blk, float *s) {
     const int tid = threadIdx.x;
     const bool active = E * tid < blk.bs;
     const int i = E * tid;
@@ -158,7 +163,7 @@ __device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, in
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = 0.0f;
     if (active) {
-        const XT *xr = x + (int64_t)blockIdx.y * x_stride + blk.off;
+        const XT *xr = x + (int64_t)token * x_stride + blk.off;
         const int lim = in_features - blk.off;               // elements of the block inside the row
         float sf[E];
 #pragma unroll
@@ -174,26 +179,68 @@ __device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, in
         for (int e = 0; e < E; ++e) v[e] *= sf[e];
     }
     fht_wave<E>(v, blk.log_len, s, tid);
+    if constexpr (LAYOUT == 2) {
+        // every element through LDS, then one 16-byte slot (k-pair, q) per thread and round
+        constexpr int LE = fht_wave_log<E>::v;
+        const bool strided = blk.log_len > 6 + LE;           // uniform
+        const int nthr = 1 << (blk.log_len - LE);
+        __syncthreads();                                      // the exchange buffer has been read
+        if (active) {
+#pragma unroll
+            for (int q = 0; q < E; ++q) s[reg_pad(strided ? tid + q * nthr : E * tid + q)] = v[q] * blk.norm;
+        }
+        __syncthreads();
+        for (int p = tid; p < (blk.bs >> 3); p += REG_THREADS) {   // blocks are multiples of 32 columns
+            const int kp = p >> 2, q = p & 3;
+            float w[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x2 t = *(const f32x2 *)(s + reg_pad(32 * kp + 2 * q + 8 * j));
+                w[2 * j] = t[0];
+                w[2 * j + 1] = t[1];
+            }
+            store8<OT>(out + ((((int64_t)(blk.off >> 5) + kp) * Mp + token) * 4 + q) * 8, w);
+        }
+        return;
+    }
     reg_gather_runs<E>(v, blk.log_len, s, tid, active);
     if (active) {
 #pragma unroll
         for (int e = 0; e < E; ++e) v[e] *= blk.norm;
-        OT *orow = out + (int64_t)blockIdx.y * n_pad + blk.off + i;
+        if constexpr (LAYOUT == 1) {
 #pragma unroll
-        for (int e = 0; e < E; e += 8) store8<OT>(orow + e, v + e);
+            for (int e = 0; e < E; e += 8) {
+                const int kb = (blk.off + i + e) >> 3;
+                store8<OT>(out + (((int64_t)(kb >> 2) * Mp + token) * 4 + (kb & 3)) * 8, v + e);
+            }
+        } else {
+            OT *orow = out + (int64_t)token * n_pad + blk.off + i;
+#pragma unroll
+            for (int e = 0; e < E; e += 8) store8<OT>(orow + e, v + e);
+        }
     }
 }
 
-// blocks of 8192 points take 16 elements per thread, smaller ones 8 (all 512 threads busy on 4096)
-template <typename XT, typename OT>
+// blocks of 8192 points take 16 elements per thread, smaller ones 8 (all 512 threads busy on 4096).
+// One-dimensional grid of 8 * ceil(B / 8) * n_blocks workgroups: workgroup L runs on XCD L % 8, and
+// the tokens are dealt out so that XCD r owns tokens r * ceil(B / 8) ..., consecutive ones
+// back to back: in the token-fast layouts the 16-byte pieces of eight consecutive tokens share a
+// 128-byte line, which is then completed inside one L2 instead of written back in eight parts.
+template <typename XT, typename OT, int LAYOUT>
 __global__ void __launch_bounds__(REG_THREADS)
 input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
-                     OT *__restrict__ out, int in_features, int n_pad, glqh_meta_args margs,
-                     float single_norm) {
+                     OT *__restrict__ out, int in_features, int n_pad, int Mp, int B, int n_blocks,
+                     glqh_meta_args margs, float single_norm) {
     extern __shared__ float s[];
-    const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
-    if (blk.log_bs > 12) input_rht_wide_body<16, XT, OT>(x, x_stride, sv, out, in_features, n_pad, blk, s);
-    else input_rht_wide_body<8, XT, OT>(x, x_stride, sv, out, in_features, n_pad, blk, s);
+    const int L = blockIdx.x, per_xcd = (B + 7) >> 3;
+    const int j = L >> 3;
+    const int token = (L & 7) * per_xcd + j / n_blocks;
+    if (token >= B || j / n_blocks >= per_xcd) return;        // uniform over the workgroup
+    const rht_slice blk = rht_slice_of(margs, single_norm, j % n_blocks);
+    if (blk.log_bs > 12)
+        input_rht_wide_body<16, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s);
+    else
+        input_rht_wide_body<8, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s);
 }
 
 template <int E, typename YT>
@@ -512,6 +559,64 @@ bool rht_wide_ok(int64_t B, const glqh_meta_args &margs, int64_t total, int64_t 
 bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 }  // namespace
 
+namespace {
+// layout 0: rows of n_pad; 1 / 2: the tile kernels' token-fast blocks with Mp padded tokens (fp16 only)
+int launch_input_rht_wide(const void *x, int x_dtype, int64_t x_stride, const void *sv, void *out, int out_dtype,
+                          int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
+                          const glqh_meta_args &margs, int n_blocks, int64_t max_bs, float rsqrt_n,
+                          hipStream_t stream) {
+    const int64_t wgs = 8 * ((B + 7) / 8) * n_blocks;
+    GLQH_REQUIRE(wgs <= 2147483647ll, "input_rht: too many blocks");
+    const dim3 wgrid((unsigned)wgs);
+    const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
+#define GLQH_INW_LAUNCH(XT, OT, LAYOUT)                                                             \
+    hipLaunchKernelGGL((input_rht_wide_kernel<XT, OT, LAYOUT>), wgrid, dim3(REG_THREADS), lds, stream, \
+                       (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
+                       (int)n_pad, (int)Mp, (int)B, n_blocks, margs, rsqrt_n)
+#define GLQH_INW_X(OT, LAYOUT)                                                                      \
+    do {                                                                                            \
+        if (x_dtype == GLQH_F16) GLQH_INW_LAUNCH(f16, OT, LAYOUT);                                  \
+        else if (x_dtype == GLQH_BF16) GLQH_INW_LAUNCH(uint16_t, OT, LAYOUT);                       \
+        else GLQH_INW_LAUNCH(float, OT, LAYOUT);                                                    \
+    } while (0)
+    if (layout == 1) GLQH_INW_X(f16, 1);
+    else if (layout == 2) GLQH_INW_X(f16, 2);
+    else if (out_dtype == GLQH_F32) GLQH_INW_X(float, 0);
+    else GLQH_INW_X(f16, 0);
+#undef GLQH_INW_X
+#undef GLQH_INW_LAUNCH
+    GLQH_LAUNCH_CHECK("input_rht launch");
+    return 0;
+}
+}  // namespace
+
+// The input transform written straight into a tile kernel's operand layout (layout 1: E8, 2:
+// trellis; Mp padded tokens).  Returns -1 without launching when the call does not qualify
+// (non-canonical blocks, blocks over 8192 points, unaligned rows): the caller then transforms into
+// rows and lets the tile launcher repack.
+int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, const void *sv, void *xb,
+                                  int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
+                                  const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream) {
+    glqh_range range("input_rht");
+    if (!x || !sv || !xb || B < 1 || in_features < 1 || in_features > n_pad) return -1;
+    if (x_dtype != GLQH_F16 && x_dtype != GLQH_BF16 && x_dtype != GLQH_F32) return -1;
+    glqh_meta_args margs;
+    int64_t max_bs = n_pad;
+    if (n_blocks > 1) {
+        if (!blocks_host) return -1;
+        max_bs = 0;
+        for (int64_t i = 0; i < n_blocks; ++i) max_bs = blocks_host[i] > max_bs ? blocks_host[i] : max_bs;
+    } else {
+        n_blocks = 1;
+    }
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, n_pad) || margs.canon != n_pad) return -1;
+    const int x_size = x_dtype == GLQH_F32 ? 4 : 2;
+    if (max_bs > (1 << WIDE_LOG_MAX) || (n_pad & 31) != 0) return -1;
+    if (!aligned16(x) || !aligned16(xb) || !aligned16(sv) || (x_stride * x_size) % 16 != 0) return -1;
+    return launch_input_rht_wide(x, x_dtype, x_stride, sv, xb, GLQH_F16, layout, Mp, B, in_features, n_pad, margs,
+                                 (int)n_blocks, max_bs, 0.0f, stream);
+}
+
 int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv,
                           void *out, int out_dtype, int64_t B, int64_t in_features, int64_t n_pad,
                           const glqh_block_meta *meta_dev, const int64_t *blocks_host,
@@ -540,26 +645,9 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
         margs.canon = 0;                               // not canonical: kernel reads meta_dev
     const int x_size = x_dtype == GLQH_F32 ? 4 : 2, o_size = out_dtype == GLQH_F32 ? 4 : 2;
     if (rht_wide_ok(B, margs, n_pad, max_bs) && aligned16(x) && aligned16(out) && aligned16(sv) &&
-        (x_stride * x_size) % 16 == 0 && (n_pad * o_size) % 16 == 0) {
-        dim3 wgrid((unsigned)n_blocks, (unsigned)B);
-        const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
-#define GLQH_INW_LAUNCH(XT, OT)                                                                     \
-    hipLaunchKernelGGL((input_rht_wide_kernel<XT, OT>), wgrid, dim3(REG_THREADS), lds, stream,      \
-                       (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
-                       (int)n_pad, margs, rsqrt_n)
-        if (out_dtype == GLQH_F32) {
-            if (x_dtype == GLQH_F16) GLQH_INW_LAUNCH(f16, float);
-            else if (x_dtype == GLQH_BF16) GLQH_INW_LAUNCH(uint16_t, float);
-            else GLQH_INW_LAUNCH(float, float);
-        } else {
-            if (x_dtype == GLQH_F16) GLQH_INW_LAUNCH(f16, f16);
-            else if (x_dtype == GLQH_BF16) GLQH_INW_LAUNCH(uint16_t, f16);
-            else GLQH_INW_LAUNCH(float, f16);
-        }
-#undef GLQH_INW_LAUNCH
-        GLQH_LAUNCH_CHECK("input_rht launch");
-        return 0;
-    }
+        (x_stride * x_size) % 16 == 0 && (n_pad * o_size) % 16 == 0)
+        return launch_input_rht_wide(x, x_dtype, x_stride, sv, out, out_dtype, 0, 0, B, in_features, n_pad, margs,
+                                     (int)n_blocks, max_bs, rsqrt_n, stream);
     const int log_slice = rht_log_slice(B);
     const int spb = rht_slices_per_block(max_bs, log_slice);
     GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "input_rht: too many slices");

@@ -565,6 +565,21 @@ __device__ __forceinline__ float rsqrt_pow2(int log_bs) {
 }
 
 // blockIdx.x = block * spb + slice; workgroups past a block's slice count retire.
+// whole canonical block j as one slice
+__device__ __forceinline__ rht_slice rht_slice_of(const glqh_meta_args margs, float single_norm, int j) {
+    const glqh_block_meta mrow = glqh_meta_row(margs, nullptr, j);
+    rht_slice b;
+    b.off = mrow.offset;
+    b.bs = mrow.bs;
+    b.log_bs = b.log_len = mrow.log_bs;
+    b.nsub = 1;
+    b.r = 0;
+    b.live = true;
+    if ((margs.canon & (margs.canon - 1)) == 0 && margs.canon != 0 && single_norm != 0.0f) b.norm = single_norm;
+    else b.norm = rsqrt_pow2(mrow.log_bs);
+    return b;
+}
+
 __device__ __forceinline__ rht_slice rht_get_slice(const glqh_block_meta *meta, const glqh_meta_args margs,
                                                    float single_norm, int spb, int log_slice) {
     const int j = blockIdx.x / spb;

@@ -18,8 +18,9 @@
 //
 // A lane's eight weights of an operand are columns 2q + {0,1,8,9,16,17,24,25} of the k-pair
 // (glq/trellis.py:99-101), and the B operand puts consecutive tokens in consecutive lanes, so the
-// activations are repacked once per call into xb[k-pair][q][token][those 8 columns]: every operand
-// load is then four runs of 256 contiguous bytes.  Workgroups are persistent and walk tiles in an
+// activations are repacked once per call (or written that way by the input transform) into
+// xb[k-pair][token][q][those 8 columns]: every operand load of a wave is then one run of 1 KB, and
+// the 32 columns of one token are 64 contiguous bytes for whoever writes them.  Workgroups are persistent and walk tiles in an
 // order that gives the CUs of one XCD the same tokens at the same time.  K is split into slots only
 // while the tiles alone would leave CUs idle; partial sums [slot][token][row] are combined in slot
 // order by the consumer, or, with one slot, the scaled result is written (or added) in place.
@@ -117,10 +118,10 @@ tr_tile_kernel(const tt_args a) {
                 dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
             }
         };
-        // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(4 kp + q) * Mp + token]
+        // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(kp * Mp + token) * 4 + q]
         // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
         const int64_t bstep = (int64_t)a.Mp * 32;               // elements from one k-pair to the next
-        const f16 *xrow = a.xb + ((int64_t)q * a.Mp + tok0 + i) * 8;
+        const f16 *xrow = a.xb + (int64_t)(tok0 + i) * 32 + q * 8;
 
         f32x4 acc[TT_FRAGS][NTW];
 #pragma unroll
@@ -138,8 +139,8 @@ tr_tile_kernel(const tt_args a) {
             d = min(d, ds1 - 1);
 #pragma unroll
             for (int tt = 0; tt < NTW; ++tt) {
-                bb[tt][0] = *(const u32x4 *)(xrow + 2 * d * bstep + tt * 128);
-                bb[tt][1] = *(const u32x4 *)(xrow + (2 * d + 1) * bstep + tt * 128);
+                bb[tt][0] = *(const u32x4 *)(xrow + 2 * d * bstep + tt * 512);
+                bb[tt][1] = *(const u32x4 *)(xrow + (2 * d + 1) * bstep + tt * 512);
             }
         };
         tr_record<R> rc = load_rec(ds0);
@@ -182,7 +183,7 @@ tr_tile_kernel(const tt_args a) {
                     if (f == TT_FRAGS - 1) {                    // this half's activations are free: request the next
                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                        for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + (2 * dn + u) * bstep + tt * 128);
+                        for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + (2 * dn + u) * bstep + tt * 512);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -222,9 +223,9 @@ tr_tile_kernel(const tt_args a) {
     }
 }
 
-// (M, k) row-major fp16 -> xb[k-pair][q][token][8]: slot q of a k-pair takes columns
+// (M, k) row-major fp16 -> xb[k-pair][token][q][8]: slot q of a k-pair takes columns
 // 2q + {0,1,8,9,16,17,24,25}, i.e. dword q of each of its four 16-byte items.  64 tokens x 4
-// k-pairs per workgroup through LDS; reads in runs of 256 bytes, writes in runs of 1 KB.
+// k-pairs per workgroup through LDS; reads in runs of 256 bytes, writes in runs of 4 KB.
 __global__ void __launch_bounds__(256)
 tr_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, int Mp, int k) {
     __shared__ u32x4 tile[16][65];                              // [k-pair * 4 + q][token]
@@ -240,11 +241,11 @@ tr_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, i
     }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int sl = r * 4 + (t >> 6), tl = t & 63;          // slot = k-pair * 4 + q
-        const int kp = kp0 + (sl >> 2);
+    for (int r = 0; r < 4; ++r) {                               // k-pair r: 64 tokens x 4 slots = 4 KB contiguous
+        const int tl = t >> 2, qq = t & 3;
+        const int kp = kp0 + r;
         if (tok0 + tl < M && kp < nkp)
-            *(u32x4 *)(xb + (((int64_t)kp * 4 + (sl & 3)) * Mp + tok0 + tl) * 8) = tile[sl][tl];
+            *(u32x4 *)(xb + (((int64_t)kp * Mp + tok0 + tl) * 4 + qq) * 8) = tile[r * 4 + qq][tl];
     }
 }
 
@@ -311,6 +312,9 @@ int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M) {
 // direct == 0: out[(slot * M + token) * m + row] = the slot's partial sum, unscaled;
 // direct == 1 (one slot only): out[token * out_stride + row] = (accum ? out : 0) + scale * sum.
 // x_f16 is (M, k) row-major; xb_scratch takes its repacked copy (glqh_trellis_tile_xb_bytes).
+// tokens of the blocked activation layout: M padded to whole workgroup tiles
+int64_t glqh_trellis_tile_padded_tokens(int64_t M) { return tt_padded_tokens(M); }
+
 int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
                              hipStream_t stream) {
@@ -318,9 +322,11 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     tt_make_plan(m, k, M, &p);
     if (direct && p.KS != 1) return glqh_fail("trellis tile kernel: in-place output needs a single K slot");
     const int Mp = (int)tt_padded_tokens(M);
-    hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)), dim3(256),
-                       0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, Mp, (int)k);
-    GLQH_LAUNCH_CHECK("trellis pack launch");
+    if (x_f16) {                                               // NULL: xb_scratch already holds the blocked layout
+        hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)),
+                           dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, Mp, (int)k);
+        GLQH_LAUNCH_CHECK("trellis pack launch");
+    }
     tt_args a;
     a.packed = (const uint8_t *)packed;
     a.xb = (const f16 *)xb_scratch;

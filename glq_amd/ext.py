@@ -25,21 +25,23 @@ from ._lib import GLQH_BF16, GLQH_F16, GLQH_F32, check
 
 _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F32}
 
-# Up to 2048 tokens every call is served on the compressed weights: 1-64 tokens by the GEMV /
+# Small and medium token counts are served on the compressed weights: 1-64 tokens by the GEMV /
 # small-batch kernels, above by the tile kernels that decode each weight once per 128-row x
-# 512-token tile (csrc/trellis_tile.hip, csrc/e8_tile.hip).  Above that the reference's own
-# many-token route -- dequantize the weight to fp16 once with the HIP kernel, then one library
-# GEMM (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334) -- is the faster one on this chip (measured on
-# 14336 x 4096 and 4096 x 14336, whole fused linear, compressed vs library: trellis 180 / 202 us
-# at 1024 tokens, 321 / 321 at 2048, 610 / 564 at 4096; E8 two-stage 198 / 202, 341 / 346,
-# 664 / 584) at the price of a transient fp16 copy of the weight.  The thresholds are the
-# reference's tunable and its E8 counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send
-# calls above n tokens to the library route (a large n keeps every call compressed).
+# 512-token tile (csrc/trellis_tile.hip, csrc/e8_tile.hip).  From a few thousand tokens on the
+# reference's own many-token route -- dequantize the weight to fp16 once with the HIP kernel, then
+# one library GEMM (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334) -- is the faster one on this chip,
+# at the price of a transient fp16 copy of the weight.  Whole fused linear, compressed / library,
+# us, on 14336 x 4096 and 4096 x 14336: trellis 172 / 201 and 157 / 204 at 1024 tokens, 353 / 334
+# and 268 / 301 at 2048, 564 / 531 and 488 / 487 at 4096; E8 two-stage 201 / 211 and 196 / 209 at
+# 1024, 400 / 335 and 312 / 327 at 2048, 639 / 552 and 553 / 511 at 4096 (the 14336-row shape pays
+# for 448 and 896 tiles on 256 CUs).  The thresholds are the reference's tunable and its E8
+# counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send calls above n tokens to the
+# library route (a large n keeps every call compressed).
 TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "2048")))
 # GLQ_TRELLIS_DENSE (set to anything) sends every fused trellis call to that dense route, the
 # reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
 TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ
-E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "2048")))
+E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "1024")))
 
 
 def _e8_dense_route(B, n_pad):

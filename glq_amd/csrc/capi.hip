@@ -706,6 +706,127 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
                                         B, c.ks, st);
 }
 
+// ---- routed experts of a mixture-of-experts layer ------------------------------------------------
+int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes, int R, const int64_t *topk_ids,
+                                       int n_slots, int n_experts, int x_div, const float *pscale_dev,
+                                       const void *x, int x_dtype, int64_t x_stride, const void *sv, int64_t m,
+                                       int64_t k, int64_t in_features, int S, int ksplit, float *part,
+                                       const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                                       hipStream_t stream);
+int glqh_launch_moe_output_rht(const float *part, int ks, int n_slots, int n_experts, const int64_t *topk_ids,
+                               const void *su_base, const float *wscale_dev, int64_t out_features, int64_t m_pad,
+                               const int64_t *blocks_m, int64_t n_blocks_m, void *h_f16, int64_t h_stride,
+                               hipStream_t stream);
+int glqh_launch_moe_gated_act(const void *h_f16, int64_t h_stride, void *out_f16, int n_slots, int64_t intermediate,
+                              int act, hipStream_t stream);
+int glqh_launch_moe_weighted_sum(const void *y_f16, int64_t y_stride, int num_tokens, int top_k, int n_experts,
+                                 const int64_t *topk_ids, const float *topk_w, int64_t out_features, void *out,
+                                 int out_dtype, int64_t out_stride, hipStream_t stream);
+
+struct moe_plan {
+    int R1, R2, S, ks, ks_all;
+    size_t part_bytes;
+};
+
+static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, const char *what, moe_plan *p) {
+    GLQH_REQUIRE(w && w->packed && w->su_f16 && w->sv_f16 && w->wscale_dev, "routed experts %s: null pointer", what);
+    if (tr_bits_from_packed(w->packed_cols, 0, &p->R1) || tr_check_shape(w->m_pad, w->n_pad, w->packed_rows)) return 1;
+    p->R2 = 0;
+    if (w->packed2) {
+        GLQH_REQUIRE(w->inv_rs2_dev, "routed experts %s: stage 2 is half-configured: packed2 present, inv_resid_scale2 absent",
+                     what);
+        if (tr_bits_from_packed(w->packed2_cols, 1, &p->R2)) return 1;
+    }
+    GLQH_REQUIRE(w->in_features >= 1 && w->in_features <= w->n_pad && w->out_features >= 1 &&
+                     w->out_features <= w->m_pad && w->out_features % 8 == 0,
+                 "routed experts %s: features %lld -> %lld do not fit %lld x %lld (out_features %% 8)", what,
+                 (long long)w->in_features, (long long)w->out_features, (long long)w->m_pad, (long long)w->n_pad);
+    const bool pow2_n = (w->n_pad & (w->n_pad - 1)) == 0;
+    GLQH_REQUIRE(w->n_blocks_n > 1 ? (w->bn_meta_dev != nullptr && w->blocks_n != nullptr) : pow2_n,
+                 "routed experts %s: input block sizes missing", what);
+    GLQH_REQUIRE(glqh_trellis_mma_fusein_plan((w->m_pad / 64) * n_slots, w->n_pad, 1, &p->S, &p->ks),
+                 "routed experts %s: no plan", what);
+    p->ks_all = p->R2 ? 2 * p->ks : p->ks;
+    p->part_bytes = align256((size_t)p->ks_all * n_slots * w->m_pad * sizeof(float));
+    return 0;
+}
+
+extern "C" size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int64_t top_k, const glqh_moe_proj *w13,
+                                                         const glqh_moe_proj *w2) {
+    if (glqh_init() != 0 || num_tokens < 1 || top_k < 1 || !w13 || !w2) return 0;
+    const int64_t n_slots = num_tokens * top_k;
+    moe_plan p13, p2;
+    if (moe_proj_plan(w13, n_slots, "w13", &p13) || moe_proj_plan(w2, n_slots, "w2", &p2)) return 0;
+    return p13.part_bytes + align256((size_t)n_slots * w13->out_features * sizeof(f16)) +
+           align256((size_t)n_slots * w2->in_features * sizeof(f16)) + p2.part_bytes +
+           align256((size_t)n_slots * w2->out_features * sizeof(f16));
+}
+
+// one projection: decode launch per stage into part[K slot][slot][row]
+static int moe_decode(const glqh_moe_proj *w, const moe_plan &p, const int64_t *topk_ids, int n_slots, int n_experts,
+                      int x_div, const void *x, int x_dtype, int64_t x_stride, float *part, hipStream_t st) {
+    if (glqh_launch_trellis_mma_fusein_moe(w->packed, w->packed_rows * w->packed_cols * 2, p.R1, topk_ids, n_slots,
+                                           n_experts, x_div, nullptr, x, x_dtype, x_stride, w->sv_f16, w->m_pad,
+                                           w->n_pad, w->in_features, p.S, p.ks, part, w->bn_meta_dev, w->blocks_n,
+                                           (int)w->n_blocks_n, st))
+        return 1;
+    if (p.R2 &&
+        glqh_launch_trellis_mma_fusein_moe(w->packed2, w->packed_rows * w->packed2_cols * 2, p.R2, topk_ids, n_slots,
+                                           n_experts, x_div, w->inv_rs2_dev, x, x_dtype, x_stride, w->sv_f16,
+                                           w->m_pad, w->n_pad, w->in_features, p.S, p.ks,
+                                           part + (int64_t)p.ks * n_slots * w->m_pad, w->bn_meta_dev, w->blocks_n,
+                                           (int)w->n_blocks_n, st))
+        return 1;
+    return 0;
+}
+
+extern "C" int glqh_fused_moe_trellis_3inst(const void *x, int x_dtype, int64_t x_stride, int64_t num_tokens,
+                                            const int64_t *topk_ids, const float *topk_weights, int64_t top_k,
+                                            int64_t num_experts, const glqh_moe_proj *w13, const glqh_moe_proj *w2,
+                                            int64_t intermediate_size, int activation_type, void *out, int out_dtype,
+                                            int64_t out_stride, void *ws, size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(x && topk_ids && topk_weights && out && w13 && w2, "routed experts: null pointer");
+    GLQH_REQUIRE(num_tokens >= 1 && top_k >= 1 && num_tokens * top_k <= 65535 && num_experts >= 1,
+                 "routed experts: %lld tokens x %lld choices (at most 65535 slots)", (long long)num_tokens,
+                 (long long)top_k);
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "routed experts: x must be f16 or bf16");
+    GLQH_REQUIRE(activation_type >= 0 && activation_type <= 2,
+                 "routed experts: gated activations 0 (silu), 1 (gelu-tanh), 2 (relu2) only, got %d", activation_type);
+    const int n_slots = (int)(num_tokens * top_k);
+    moe_plan p13, p2;
+    if (moe_proj_plan(w13, n_slots, "w13", &p13) || moe_proj_plan(w2, n_slots, "w2", &p2)) return 1;
+    GLQH_REQUIRE(w13->out_features == 2 * intermediate_size && w2->in_features == intermediate_size,
+                 "routed experts: w13 yields %lld values, w2 takes %lld, intermediate size %lld (gate | up)",
+                 (long long)w13->out_features, (long long)w2->in_features, (long long)intermediate_size);
+    const size_t hb = align256((size_t)n_slots * w13->out_features * sizeof(f16));
+    const size_t ab = align256((size_t)n_slots * intermediate_size * sizeof(f16));
+    const size_t yb = align256((size_t)n_slots * w2->out_features * sizeof(f16));
+    const size_t need = p13.part_bytes + hb + ab + p2.part_bytes + yb;
+    GLQH_REQUIRE(ws && ws_bytes >= need, "routed experts: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    float *part13 = (float *)ws;
+    f16 *h = (f16 *)((char *)ws + p13.part_bytes);
+    f16 *hact = (f16 *)((char *)ws + p13.part_bytes + hb);
+    float *part2 = (float *)((char *)ws + p13.part_bytes + hb + ab);
+    f16 *yslot = (f16 *)((char *)ws + p13.part_bytes + hb + ab + p2.part_bytes);
+    // gate | up of every slot: decode on the token's row, output transform with the expert's signs
+    if (moe_decode(w13, p13, topk_ids, n_slots, (int)num_experts, (int)top_k, x, x_dtype, x_stride, part13, st)) return 1;
+    if (glqh_launch_moe_output_rht(part13, p13.ks_all, n_slots, (int)num_experts, topk_ids, w13->su_f16,
+                                   w13->wscale_dev, w13->out_features, w13->m_pad, w13->blocks_m, w13->n_blocks_m, h,
+                                   w13->out_features, st))
+        return 1;
+    if (glqh_launch_moe_gated_act(h, w13->out_features, hact, n_slots, intermediate_size, activation_type, st)) return 1;
+    // down projection of every slot, then the weighted sum over each token's choices, in their order
+    if (moe_decode(w2, p2, topk_ids, n_slots, (int)num_experts, 1, hact, GLQH_F16, intermediate_size, part2, st)) return 1;
+    if (glqh_launch_moe_output_rht(part2, p2.ks_all, n_slots, (int)num_experts, topk_ids, w2->su_f16, w2->wscale_dev,
+                                   w2->out_features, w2->m_pad, w2->blocks_m, w2->n_blocks_m, yslot, w2->out_features,
+                                   st))
+        return 1;
+    return glqh_launch_moe_weighted_sum(yslot, w2->out_features, (int)num_tokens, (int)top_k, (int)num_experts,
+                                        topk_ids, topk_weights, w2->out_features, out, out_dtype, out_stride, st);
+}
+
 // ---- batch-1 decode loop: output transform fused with what follows it (glq_decoder_ops.h) ----
 extern "C" int glqh_trellis_linear_add_rmsnorm_bf16(const void *x, int64_t in_features,
                                                     const glqh_trellis_shard *shard, const int64_t *blocks_n,

@@ -243,15 +243,13 @@ input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__r
         input_rht_wide_body<8, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s);
 }
 
-template <int E, typename YT>
-__device__ __forceinline__ void output_rht_wide_body(const glqh_ysrc &src, const f16 *__restrict__ su,
-                                                    YT *__restrict__ y, int64_t y_stride, int out_features,
-                                                    int m_pad, const rht_slice &blk, float *s) {
-    const int64_t b = blockIdx.y;
-    const int tid = threadIdx.x;
-    const bool active = E * tid < blk.bs;
+// v = the transformed sums of elements E * tid .. E * tid + E - 1 of block `blk`, row b (before the
+// signs and the 1/sqrt(bs)): direct rows or split-K partial sums in, register transform, runs restored.
+// Every thread of the workgroup calls.
+template <int E>
+__device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysrc &src, int64_t b, int m_pad,
+                                                   const rht_slice &blk, float *s, int tid, bool active) {
     const int i = E * tid;
-    float v[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = 0.0f;
     if (active) {
@@ -288,7 +286,18 @@ __device__ __forceinline__ void output_rht_wide_body(const glqh_ysrc &src, const
     }
     fht_wave<E>(v, blk.log_len, s, tid);
     reg_gather_runs<E>(v, blk.log_len, s, tid, active);
-    const int row = blk.off + i;
+}
+
+template <int E, typename YT>
+__device__ __forceinline__ void output_rht_wide_body(const glqh_ysrc &src, const f16 *__restrict__ su,
+                                                    YT *__restrict__ y, int64_t y_stride, int out_features,
+                                                    int m_pad, const rht_slice &blk, float *s) {
+    const int64_t b = blockIdx.y;
+    const int tid = threadIdx.x;
+    const bool active = E * tid < blk.bs;
+    float v[E];
+    output_wide_values<E>(v, src, b, m_pad, blk, s, tid, active);
+    const int row = blk.off + E * tid;
     if (active && row < out_features) {
         float f[E];
 #pragma unroll
@@ -750,6 +759,149 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
 }
 
 int glqh_rht_init(void) { return 0; }
+
+// ---- routed experts (glq/csrc/glq_cuda.cu:5030-5250) ------------------------------------------
+// The finishing launches of the two projections of a mixture-of-experts layer.  Rows are slots
+// (token, choice); the slot's expert, read from topk_ids on the device, selects the output signs
+// (su_base + expert * m_pad) and the scale.  Partial sums: [K slot][slot][row].
+namespace {
+struct moe_out_args {
+    const float *part;
+    int ks, n_slots, n_experts;
+    const int64_t *topk_ids;
+    const f16 *su_base;
+    const float *wscale_dev;
+    int out_features, m_pad;
+};
+
+__device__ __forceinline__ glqh_ysrc moe_src(const moe_out_args &a, float scale) {
+    glqh_ysrc src = {};
+    src.part = a.part;
+    src.part_kstride = (int64_t)a.n_slots * a.m_pad;
+    src.ksplit = a.ks;
+    src.scale[0] = scale;
+    src.nparts = 1;
+    return src;
+}
+
+// first projection: h[slot][row] = su * H(sum) * Wscale, fp16 (slots of an invalid expert: zeros)
+__global__ void __launch_bounds__(REG_THREADS)
+moe_output_rht_kernel(moe_out_args a, f16 *__restrict__ h, int64_t h_stride, glqh_meta_args margs) {
+    extern __shared__ float s[];
+    const rht_slice blk = rht_slice_of(margs, 0.0f, blockIdx.x);
+    const int slot = blockIdx.y;
+    const int64_t e = a.topk_ids[slot];
+    if (e < 0 || e >= a.n_experts) {                            // uniform over the workgroup
+        for (int i = threadIdx.x; i < blk.bs; i += REG_THREADS)
+            if (blk.off + i < a.out_features) h[slot * h_stride + blk.off + i] = (f16)0.0f;
+        return;
+    }
+    const glqh_ysrc src = moe_src(a, a.wscale_dev[e]);
+    const f16 *su = a.su_base + e * a.m_pad;
+    if (blk.log_bs > 12) output_rht_wide_body<16, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s);
+    else output_rht_wide_body<8, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s);
+}
+
+// out[slot][i] = act(h[slot][i]) * h[slot][intermediate + i]: 0 SiLU, 1 GELU (tanh form), 2 squared ReLU
+// (glq/csrc/glq_cuda.cu:4540-4559)
+__global__ void __launch_bounds__(256)
+moe_gated_act_kernel(const f16 *__restrict__ h, int64_t h_stride, f16 *__restrict__ out, int n_slots,
+                     int intermediate, int act) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)n_slots * intermediate) return;
+    const int slot = (int)(idx / intermediate), i = (int)(idx % intermediate);
+    const float g = (float)h[slot * h_stride + i], up = (float)h[slot * h_stride + intermediate + i];
+    float v;
+    if (act == 0) v = g / (1.0f + expf(-g));
+    else if (act == 1) v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    else { const float r = fmaxf(g, 0.0f); v = r * r; }
+    out[idx] = (f16)(v * up);
+}
+
+// out[token][row] = sum_j w[token][j] * y[token * top_k + j][row], j in order, fp32 accumulation of the fp16
+// per-slot results (glq_moe_weighted_scatter_reduce_kernel, glq/csrc/glq_cuda.cu:4520-4537); slots of an
+// invalid expert are skipped.  One thread per 8 rows.
+template <typename YT>
+__global__ void __launch_bounds__(256)
+moe_weighted_sum_kernel(const f16 *__restrict__ y, int64_t y_stride, const int64_t *__restrict__ topk_ids,
+                        const float *__restrict__ topk_w, int top_k, int n_experts, int out_features,
+                        YT *__restrict__ out, int64_t out_stride) {
+    const int token = blockIdx.y;
+    const int row = 8 * (blockIdx.x * 256 + threadIdx.x);
+    if (row >= out_features) return;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < top_k; ++j) {
+        const int slot = token * top_k + j;
+        const int64_t ex = topk_ids[slot];
+        if (ex < 0 || ex >= n_experts) continue;
+        float v[8];
+        load8<f16>(y + slot * y_stride + row, v);
+        const float w = topk_w[slot];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += w * v[e];
+    }
+    store8<YT>(out + (int64_t)token * out_stride + row, acc);
+}
+
+int moe_check_blocks(const int64_t *blocks_m, int64_t n_blocks_m, int64_t m_pad, glqh_meta_args *margs,
+                     int64_t *max_bs) {
+    GLQH_REQUIRE(glqh_fill_meta_args(margs, n_blocks_m > 1 ? blocks_m : nullptr, n_blocks_m > 1 ? n_blocks_m : 1,
+                                     m_pad) && margs->canon == m_pad,
+                 "routed experts: output block sizes must be the descending power-of-two decomposition of m_pad");
+    *max_bs = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)m_pad));
+    GLQH_REQUIRE(*max_bs <= (1 << WIDE_LOG_MAX) && (m_pad & 7) == 0,
+                 "routed experts: output blocks of 8..8192 rows, got m_pad %lld", (long long)m_pad);
+    return 0;
+}
+}  // namespace
+
+int glqh_launch_moe_output_rht(const float *part, int ks, int n_slots, int n_experts, const int64_t *topk_ids,
+                               const void *su_base, const float *wscale_dev, int64_t out_features, int64_t m_pad,
+                               const int64_t *blocks_m, int64_t n_blocks_m, void *h_f16, int64_t h_stride,
+                               hipStream_t stream) {
+    glqh_range range("output_rht");
+    glqh_meta_args margs;
+    int64_t max_bs;
+    if (moe_check_blocks(blocks_m, n_blocks_m, m_pad, &margs, &max_bs)) return 1;
+    GLQH_REQUIRE(aligned16(part) && aligned16(su_base) && aligned16(h_f16) && (h_stride & 7) == 0,
+                 "routed experts: unaligned rows");
+    const moe_out_args a = {part, ks, n_slots, n_experts, topk_ids, (const f16 *)su_base, wscale_dev,
+                            (int)out_features, (int)m_pad};
+    const int nb = __builtin_popcountll((unsigned long long)m_pad);
+    hipLaunchKernelGGL(moe_output_rht_kernel, dim3((unsigned)nb, (unsigned)n_slots), dim3(REG_THREADS),
+                       rht_reg_lds_bytes(ilog2(max_bs)), stream, a, (f16 *)h_f16, h_stride, margs);
+    GLQH_LAUNCH_CHECK("routed-expert output_rht launch");
+    return 0;
+}
+
+int glqh_launch_moe_gated_act(const void *h_f16, int64_t h_stride, void *out_f16, int n_slots, int64_t intermediate,
+                              int act, hipStream_t stream) {
+    GLQH_REQUIRE(act >= 0 && act <= 2, "routed experts: gated activations 0 (silu), 1 (gelu-tanh), 2 (relu2), got %d", act);
+    const int64_t total = (int64_t)n_slots * intermediate;
+    hipLaunchKernelGGL(moe_gated_act_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       (const f16 *)h_f16, h_stride, (f16 *)out_f16, n_slots, (int)intermediate, act);
+    GLQH_LAUNCH_CHECK("routed-expert activation launch");
+    return 0;
+}
+
+int glqh_launch_moe_weighted_sum(const void *y_f16, int64_t y_stride, int num_tokens, int top_k, int n_experts,
+                                 const int64_t *topk_ids, const float *topk_w, int64_t out_features, void *out,
+                                 int out_dtype, int64_t out_stride, hipStream_t stream) {
+    GLQH_REQUIRE(out_dtype == GLQH_F16 || out_dtype == GLQH_BF16, "routed experts: output must be f16 or bf16");
+    GLQH_REQUIRE(aligned16(y_f16) && aligned16(out) && (out_stride & 7) == 0 && (y_stride & 7) == 0 &&
+                     (out_features & 7) == 0,
+                 "routed experts: unaligned rows");
+    const dim3 grid((unsigned)((out_features / 8 + 255) / 256), (unsigned)num_tokens);
+    if (out_dtype == GLQH_F16)
+        hipLaunchKernelGGL((moe_weighted_sum_kernel<f16>), grid, dim3(256), 0, stream, (const f16 *)y_f16, y_stride,
+                           topk_ids, topk_w, top_k, n_experts, (int)out_features, (f16 *)out, out_stride);
+    else
+        hipLaunchKernelGGL((moe_weighted_sum_kernel<uint16_t>), grid, dim3(256), 0, stream, (const f16 *)y_f16,
+                           y_stride, topk_ids, topk_w, top_k, n_experts, (int)out_features, (uint16_t *)out,
+                           out_stride);
+    GLQH_LAUNCH_CHECK("routed-expert weighted sum launch");
+    return 0;
+}
 
 int glqh_launch_output_rht_group(const float *const part[], const void *const su[], void *const y[],
                                  const float scale[], const int64_t m_pad[], const int64_t out_features[],

@@ -276,7 +276,7 @@ __device__ __forceinline__ void
 tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
                    const f16 *__restrict__ sv, int B, int m, int k, int in_features, int S,
                    const glqh_block_meta *__restrict__ bn_meta, int n_blocks, glqh_meta_args margs,
-                   float *__restrict__ part, float pscale, u32x4 *lds) {
+                   float *__restrict__ part, float pscale, u32x4 *lds, int part_B = 0) {
     constexpr int TPS = mma_tps<TP>();
     const int Ls = S << 5;
     uint32_t *xs32 = (uint32_t *)lds;
@@ -401,7 +401,10 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
         cur = nx1;
         nx1 = nx2;
     }
-    mma_reduce_store<TP, 1>(acc, (float *)lds, a, wave, B, m, 0, 64 * blockIdx.x, slot, part, 0, pscale, 0, 0);
+    // part_B: rows per K slot of the partial-sum array when it holds more rows than this call's
+    // tokens (the routed-expert launch: one row per (token, expert) slot, `part` offset to this one)
+    mma_reduce_store<TP, 1>(acc, (float *)lds, a, wave, part_B > 0 ? part_B : B, m, 0, 64 * blockIdx.x, slot, part,
+                            0, pscale, 0, 0);
 }
 
 template <int R, typename XT, int TP>
@@ -443,6 +446,37 @@ tr_mma_fusein_group_kernel(tr_fusein_group g, const XT *__restrict__ x, int64_t 
     if ((int)blockIdx.x * 64 >= m) return;
     tr_mma_fusein_body<R, XT, TP>(packed, x, x_stride, sv, B, m, k, in_features, S, bn_meta, n_blocks, margs,
                                   part, 1.0f, xs_lds);
+}
+
+// Routed experts of a mixture-of-experts layer, one token each (glq/csrc/glq_cuda.cu:5030-5250,
+// glq/csrc/glq_trellis.cu:539-588): blockIdx.z = slot = (token, choice); the slot's expert comes
+// from topk_ids on the device, so nothing about the routing is known to the host and the launch
+// can be captured.  Every expert has its own packed stream (stride_bytes apart) and scale; the
+// input signs are shared.  x row of slot s is s / x_div (the token for the first projection, the
+// slot itself for the second).  Partial sums: [K slot][slot][row].  Slots whose expert id is out
+// of range write nothing and are skipped by the finishing kernels as well.
+struct tr_moe_args {
+    const uint8_t *packed;                       // expert 0
+    int64_t stride_bytes;                        // from one expert's stream to the next
+    const int64_t *topk_ids;                     // (n_slots,)
+    const float *pscale_dev;                     // per-expert factor of the partial sums (a residual stage), or NULL
+    float *part;
+    int n_slots, n_experts, x_div;
+};
+
+template <int R, typename XT>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_fusein_moe_kernel(tr_moe_args g, const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
+                         int m, int k, int in_features, int S, const glqh_block_meta *__restrict__ bn_meta,
+                         int n_blocks, glqh_meta_args margs) {
+    extern __shared__ u32x4 xs_lds[];
+    const int slot = blockIdx.z;
+    const int64_t e = g.topk_ids[slot];
+    if (e < 0 || e >= g.n_experts) return;                      // uniform over the workgroup
+    tr_mma_fusein_body<R, XT, 1>(g.packed + e * g.stride_bytes, x + (int64_t)(slot / g.x_div) * x_stride, x_stride,
+                                 sv, 1, m, k, in_features, S, bn_meta, n_blocks, margs,
+                                 g.part + (int64_t)slot * m, g.pscale_dev ? g.pscale_dev[e] : 1.0f, xs_lds,
+                                 g.n_slots);
 }
 
 template <int TP>
@@ -622,6 +656,56 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
     return glqh_fail("fused-input trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
+template <int R, typename XT>
+static int launch_mma_fusein_moe(const tr_moe_args &g, const void *x, int64_t x_stride, const void *sv, int64_t m,
+                                 int64_t k, int64_t in_features, int S, int ksplit, const glqh_block_meta *bn_meta,
+                                 const int64_t *blocks_host, int n_blocks, hipStream_t stream) {
+    glqh_meta_args margs;
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
+    const glqh_block_meta *meta = n_blocks > 1 ? bn_meta : nullptr;
+    const int nb = n_blocks > 1 ? n_blocks : 1;
+    dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, (unsigned)g.n_slots);
+    hipLaunchKernelGGL((tr_mma_fusein_moe_kernel<R, XT>), grid, dim3(TR_THREADS), fi_lds_bytes<1>(S), stream, g,
+                       (const XT *)x, x_stride, (const f16 *)sv, (int)m, (int)k, (int)in_features, S, meta, nb, margs);
+    GLQH_LAUNCH_CHECK("trellis routed-expert gemv launch");
+    return 0;
+}
+
+// One projection of all routed experts: part[K slot][slot][row], one token per slot.
+int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes, int R, const int64_t *topk_ids,
+                                       int n_slots, int n_experts, int x_div, const float *pscale_dev,
+                                       const void *x, int x_dtype, int64_t x_stride, const void *sv, int64_t m,
+                                       int64_t k, int64_t in_features, int S, int ksplit, float *part,
+                                       const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                                       hipStream_t stream) {
+    glqh_range range("dequant_matmul");
+    GLQH_REQUIRE(n_slots >= 1 && n_slots <= 65535, "routed experts: %d slots (1..65535)", n_slots);
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "routed experts: x must be f16 or bf16");
+    tr_moe_args g;
+    g.packed = (const uint8_t *)packed;
+    g.stride_bytes = stride_bytes;
+    g.topk_ids = topk_ids;
+    g.pscale_dev = pscale_dev;
+    g.part = part;
+    g.n_slots = n_slots;
+    g.n_experts = n_experts;
+    g.x_div = x_div;
+#define GLQH_MOE(RR)                                                                                      \
+    (x_dtype == GLQH_F16                                                                                  \
+         ? launch_mma_fusein_moe<RR, f16>(g, x, x_stride, sv, m, k, in_features, S, ksplit, bn_meta,      \
+                                          blocks_host, n_blocks, stream)                                  \
+         : launch_mma_fusein_moe<RR, uint16_t>(g, x, x_stride, sv, m, k, in_features, S, ksplit, bn_meta, \
+                                               blocks_host, n_blocks, stream))
+    switch (R) {
+    case 1: return GLQH_MOE(1);
+    case 2: return GLQH_MOE(2);
+    case 3: return GLQH_MOE(3);
+    case 4: return GLQH_MOE(4);
+    }
+#undef GLQH_MOE
+    return glqh_fail("routed experts: R (bits/weight) 1-4, got %d", R);
+}
+
 template <typename K>
 static int fi_set_lds(K kernel, size_t bytes) {
     return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -632,6 +716,7 @@ static int fi_set_lds(K kernel, size_t bytes) {
 template <int R>
 static int fi_init_R() {
     const size_t b1 = fi_lds_bytes<1>(FI_MAX_S), b4 = fi_lds_bytes<4>(FI_MAX_S_TP4);
+    if (fi_set_lds(tr_mma_fusein_moe_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_moe_kernel<R, uint16_t>, b1)) return 1;
     return fi_set_lds(tr_mma_fusein_kernel<R, f16, 1>, b1) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 1>, b1) ||
            fi_set_lds(tr_mma_fusein_kernel<R, f16, 4>, b4) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 4>, b4) ||
            fi_set_lds(tr_mma_fusein_group_kernel<R, f16, 1>, b1) ||

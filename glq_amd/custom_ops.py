@@ -82,6 +82,21 @@ SCHEMAS = {
                                             "Tensor(a!) y_rht_out, int col) -> ()",
     "output_rht_shards": "output_rht_shards(Tensor y_rht, Tensor su, Tensor(a!) y, "
                          "int out_features, Tensor shard_meta, int max_bs) -> ()",
+    # glq_vllm/custom_ops.py:22-36: the routed-expert step of a mixture-of-experts layer
+    "fused_moe_trellis_3inst": "fused_moe_trellis_3inst(Tensor x, Tensor topk_ids, Tensor topk_weights, "
+                               "Tensor w13_trellis_packed, Tensor w13_trellis_packed2, "
+                               "Tensor w13_SU, Tensor w13_SV, Tensor w13_Wscale, "
+                               "Tensor w13_inv_resid_scale2, "
+                               "Tensor w2_trellis_packed, Tensor w2_trellis_packed2, "
+                               "Tensor w2_SU, Tensor w2_SV, Tensor w2_Wscale, "
+                               "Tensor w2_inv_resid_scale2, "
+                               "int hidden_size, int intermediate_size, int w13_out_features, "
+                               "int n_pad_w13, int m_pad_w13, int n_pad_w2, int m_pad_w2, "
+                               "Tensor blocks_n_w13, Tensor blocks_m_w13, "
+                               "Tensor blocks_n_w13_meta, Tensor blocks_m_w13_meta, "
+                               "Tensor blocks_n_w2, Tensor blocks_m_w2, "
+                               "Tensor blocks_n_w2_meta, Tensor blocks_m_w2_meta, "
+                               "int activation_type) -> Tensor",
     # glq_vllm/custom_ops.py:301-308
     "embedding_dequant": "embedding_dequant(Tensor input_ids, Tensor qidxs, Tensor sv, "
                          "Tensor wscale, Tensor codebook, Tensor? qidxs2, "
@@ -140,6 +155,20 @@ def _fused_linear_trellis_3inst_rvq2_fake(x, sv, su, trellis_packed, trellis_pac
     return x.new_empty((x.shape[0], out_features), dtype=_act_dtype(x))
 
 
+def _fused_moe_trellis_3inst_fake(x, topk_ids, topk_weights,
+                                  w13_trellis_packed, w13_trellis_packed2,
+                                  w13_SU, w13_SV, w13_Wscale, w13_inv_resid_scale2,
+                                  w2_trellis_packed, w2_trellis_packed2,
+                                  w2_SU, w2_SV, w2_Wscale, w2_inv_resid_scale2,
+                                  hidden_size, intermediate_size, w13_out_features,
+                                  n_pad_w13, m_pad_w13, n_pad_w2, m_pad_w2,
+                                  blocks_n_w13, blocks_m_w13, blocks_n_w13_meta, blocks_m_w13_meta,
+                                  blocks_n_w2, blocks_m_w2, blocks_n_w2_meta, blocks_m_w2_meta,
+                                  activation_type):
+    # (num_tokens, hidden) in the activation dtype (glq_vllm/custom_ops.py:701-718 returns fp16)
+    return x.new_empty((*x.shape[:-1], hidden_size), dtype=_act_dtype(x))
+
+
 def _embedding_dequant_fake(input_ids, qidxs, sv, wscale, codebook, qidxs2, inv_resid_scale, codebook2,
                             n_pad, embedding_dim, embed_scale, out_dtype):
     dt = out_dtype if out_dtype is not None else sv.dtype
@@ -163,6 +192,7 @@ FAKES = {
     "fused_linear_trellis_3inst_yrht_rvq2": _none_fake,
     "output_rht_shards": _none_fake,
     "embedding_dequant": _embedding_dequant_fake,
+    "fused_moe_trellis_3inst": _fused_moe_trellis_3inst_fake,
 }
 
 
@@ -198,6 +228,7 @@ def _impls():
         "fused_linear_trellis_3inst_yrht_rvq2": ext.glq_fused_linear_trellis_3inst_yrht_rvq2_cuda,
         "output_rht_shards": ext.glq_output_rht_shards_cuda,
         "embedding_dequant": ext.glq_embedding_dequant,
+        "fused_moe_trellis_3inst": ext.glq_fused_moe_trellis_3inst_cuda,
     }
 
 

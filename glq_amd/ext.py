@@ -367,6 +367,99 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
     return y
 
 
+class _MoeProj(C.Structure):
+    _fields_ = [("packed", C.c_void_p), ("packed_rows", C.c_int64), ("packed_cols", C.c_int64),
+                ("packed2", C.c_void_p), ("packed2_cols", C.c_int64), ("su", C.c_void_p), ("sv", C.c_void_p),
+                ("wscale", C.c_void_p), ("inv_rs2", C.c_void_p), ("blocks_n", C.c_void_p),
+                ("n_blocks_n", C.c_int64), ("bn_meta", C.c_void_p), ("blocks_m", C.c_void_p),
+                ("n_blocks_m", C.c_int64), ("in_features", C.c_int64), ("out_features", C.c_int64),
+                ("n_pad", C.c_int64), ("m_pad", C.c_int64)]
+
+
+def _moe_proj(what, packed, packed2, su, sv, wscale, inv_rs2, blocks_n, blocks_m, bn_meta, in_f, out_f, n_pad,
+              m_pad, keep):
+    _chk(packed, f"{what}_trellis_packed", torch.int16)
+    if packed.dim() != 3:
+        raise RuntimeError(f"{what}_trellis_packed must be (E, tiles, 16*R)")
+    E = packed.shape[0]
+    _chk(su, f"{what}_SU", torch.float16)
+    _chk(sv, f"{what}_SV", torch.float16)
+    if su.shape != (E, int(m_pad)) or sv.numel() != int(n_pad):
+        raise RuntimeError(f"{what}: SU must be (E, m_pad) and SV (n_pad,), got {tuple(su.shape)} and {tuple(sv.shape)}")
+    ws32 = wscale.to(device=packed.device, dtype=torch.float32).contiguous()
+    if ws32.numel() != E:
+        raise RuntimeError(f"{what}_Wscale must hold one scale per expert")
+    keep.append(ws32)
+    # a second stage registered as the (E, 1, 1) placeholder is "absent" (glq/csrc/glq_cuda.cu:5083-5088)
+    has2 = packed2 is not None and packed2.numel() > E
+    p2 = irs = None
+    if has2:
+        _chk(packed2, f"{what}_trellis_packed2", torch.int16)
+        if packed2.dim() != 3 or packed2.shape[0] != E or packed2.shape[1] != packed.shape[1]:
+            raise RuntimeError(f"trellis MoE {what} stage-2 tile count {tuple(packed2.shape)} != stage-1 "
+                               f"{tuple(packed.shape)}")
+        p2 = packed2
+        irs = inv_rs2.to(device=packed.device, dtype=torch.float32).contiguous()
+        if irs.numel() != E:
+            raise RuntimeError(f"{what}_inv_resid_scale2 must hold one value per expert")
+        keep.append(irs)
+    bn, nbn = _host_i64(blocks_n)
+    bm, nbm = _host_i64(blocks_m)
+    keep += [bn, bm]
+    return _MoeProj(_p(packed).value, packed.shape[1], packed.shape[2], _p(p2).value if has2 else None,
+                    p2.shape[2] if has2 else 0, _p(su).value, _p(sv).value, _p(ws32).value,
+                    _p(irs).value if has2 else None, C.cast(bn, C.c_void_p).value, nbn,
+                    _meta_ptr(bn_meta).value if nbn > 1 else None, C.cast(bm, C.c_void_p).value, nbm,
+                    int(in_f), int(out_f), int(n_pad), int(m_pad))
+
+
+def glq_fused_moe_trellis_3inst_cuda(x, topk_ids, topk_weights,
+                                     w13_trellis_packed, w13_trellis_packed2, w13_SU, w13_SV, w13_Wscale,
+                                     w13_inv_resid_scale2,
+                                     w2_trellis_packed, w2_trellis_packed2, w2_SU, w2_SV, w2_Wscale,
+                                     w2_inv_resid_scale2,
+                                     hidden_size, intermediate_size, w13_out_features,
+                                     n_pad_w13, m_pad_w13, n_pad_w2, m_pad_w2,
+                                     blocks_n_w13, blocks_m_w13, blocks_n_w13_meta, blocks_m_w13_meta,
+                                     blocks_n_w2, blocks_m_w2, blocks_n_w2_meta, blocks_m_w2_meta,
+                                     activation_type, out_dtype=None):
+    """The routed-expert step of a mixture-of-experts layer on stacked trellis-3INST experts, one
+    host call with the routing read on the device (argument order of the reference's binding,
+    glq/csrc/glq_bindings.cpp:509-525; glq/csrc/glq_cuda.cu:5030-5250).  Returns (num_tokens,
+    hidden) in the input's 16-bit dtype (the reference returns fp16)."""
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    if x.dim() != 2 or x.shape[1] != int(hidden_size):
+        raise RuntimeError(f"x must be (num_tokens, hidden), got {tuple(x.shape)}")
+    if topk_ids.dim() != 2 or topk_ids.shape != topk_weights.shape or topk_ids.shape[0] != x.shape[0]:
+        raise RuntimeError("topk_ids and topk_weights must be (num_tokens, top_k)")
+    if int(activation_type) not in (0, 1, 2):
+        raise RuntimeError(f"trellis MoE path supports gated activations (0/1/2) only, got {activation_type}")
+    T, K = topk_ids.shape
+    ids = topk_ids.to(device=x.device, dtype=torch.int64).contiguous()
+    tw = topk_weights.to(device=x.device, dtype=torch.float32).contiguous()
+    keep = []
+    w13 = _moe_proj("w13", w13_trellis_packed, w13_trellis_packed2, w13_SU, w13_SV, w13_Wscale,
+                    w13_inv_resid_scale2, blocks_n_w13, blocks_m_w13, blocks_n_w13_meta, hidden_size,
+                    w13_out_features, n_pad_w13, m_pad_w13, keep)
+    w2 = _moe_proj("w2", w2_trellis_packed, w2_trellis_packed2, w2_SU, w2_SV, w2_Wscale, w2_inv_resid_scale2,
+                   blocks_n_w2, blocks_m_w2, blocks_n_w2_meta, intermediate_size, hidden_size, n_pad_w2,
+                   m_pad_w2, keep)
+    dt = out_dtype or x.dtype
+    out = torch.empty((T, int(hidden_size)), dtype=dt, device=x.device)
+    with torch.cuda.device(x.device):
+        nb = lib.glqh_fused_moe_trellis_workspace_bytes(T, K, C.addressof(w13), C.addressof(w2))
+        if nb == 0:
+            # the entry itself reports what is wrong with the shapes
+            nb = 256
+        ws = _ws(nb, x.device)
+        check(lib.glqh_fused_moe_trellis_3inst(
+            _p(x), _DT[x.dtype], x.shape[1], T, _p(ids), _p(tw), K, w13_trellis_packed.shape[0],
+            C.addressof(w13), C.addressof(w2), int(intermediate_size), int(activation_type), _p(out), _DT[dt],
+            out.shape[1], _p(ws), ws.numel(), _stream()))
+    return out
+
+
 def _yrht_slice(y_rht_out, col, m_pad):
     _chk(y_rht_out, "y_rht_out", torch.float32)
     if y_rht_out.dim() != 2 or int(col) < 0 or int(col) + int(m_pad) > y_rht_out.shape[1]:

@@ -207,6 +207,46 @@ int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_
                                           int y_dtype, int64_t y_stride,
                                           void *ws, size_t ws_bytes, void *stream);
 
+/* One projection (gate/up "w13" or down "w2") of the routed experts of a mixture-of-experts
+ * layer, the experts stacked along the first dimension (glq/csrc/glq_cuda.cu:5043-5064). */
+typedef struct {
+    const void *packed;          /* (E, (m/16)(k/16), 16 R1) int16, stage 1, R1 = 2..4 */
+    int64_t packed_rows;         /* per expert: (m_pad/16)(n_pad/16) */
+    int64_t packed_cols;         /* 16 R1 */
+    const void *packed2;         /* (E, same rows, 16 R2) int16, R2 = 1..4, or NULL */
+    int64_t packed2_cols;
+    const void *su_f16;          /* (E, m_pad) */
+    const void *sv_f16;          /* (n_pad,) shared by the experts */
+    const float *wscale_dev;     /* (E,) fp32, device */
+    const float *inv_rs2_dev;    /* (E,) fp32, device; read only with a second stage */
+    const int64_t *blocks_n;     /* host */
+    int64_t n_blocks_n;
+    const glqh_block_meta *bn_meta_dev;
+    const int64_t *blocks_m;     /* host; must be the block_decompose sizes of m_pad */
+    int64_t n_blocks_m;
+    int64_t in_features, out_features, n_pad, m_pad;
+} glqh_moe_proj;
+
+size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int64_t top_k, const glqh_moe_proj *w13,
+                                              const glqh_moe_proj *w2);
+
+/* The routed-expert step of a mixture-of-experts layer on trellis-3INST weights,
+ * out[t] = sum_j topk_weights[t][j] * w2_e( act(gate) * up ),  (gate | up) = w13_e(x[t]),
+ * e = topk_ids[t][j], as one host call with the routing read on the device (no host
+ * synchronisation, no allocation: capturable).  Replaces glq_fused_moe_trellis_3inst_cuda
+ * (glq/csrc/glq_cuda.cu:5030-5250; grouped matmul glq/csrc/glq_trellis.cu:1475-1540) behind
+ * torch.ops.glq.fused_moe_trellis_3inst (glq_vllm/custom_ops.py:22-36).  Every (token, choice)
+ * slot is one fused-input GEMV on that expert's stream; intermediate results are rounded to
+ * fp16 where the reference rounds them (after each output transform and after the
+ * activation), the weighted sum runs over the choices in order in fp32.  activation_type:
+ * 0 SiLU, 1 GELU (tanh form), 2 squared ReLU, each times the up half.  Expert ids outside
+ * [0, num_experts) contribute nothing.  x f16 or bf16, out f16 or bf16. */
+int glqh_fused_moe_trellis_3inst(const void *x, int x_dtype, int64_t x_stride, int64_t num_tokens,
+                                 const int64_t *topk_ids, const float *topk_weights, int64_t top_k,
+                                 int64_t num_experts, const glqh_moe_proj *w13, const glqh_moe_proj *w2,
+                                 int64_t intermediate_size, int activation_type, void *out, int out_dtype,
+                                 int64_t out_stride, void *ws, size_t ws_bytes, void *stream);
+
 /* ---- E8 shell codebook ---------------------------------------------------- */
 
 /* (n_entries, 8) fp16 table -> n_entries uint32 of eight 4-bit codes round(2 v) + 6, the

@@ -25,6 +25,13 @@ Pinned by (see tests/test_oracle_*.py):
   e8_embedding_rows      closed form: brute-force Sylvester matrix product on small n, and
                          equality with row-by-row (one-hot) use of e8_dequant + fht
   linear forwards        golden end-to-end outputs from E8RHTLinear.forward (CPU)
+  moe_trellis_forward    no golden vector exists (the reference tests only the op's schema,
+                         tests/test_glq_vllm.py:595-640): pinned as a composition -- one expert
+                         with weight 1 equals down(act(gate) * up) built from the pinned
+                         trellis_linear_forward and activation values computed with math.exp /
+                         math.tanh in the test, linearity in the routing weights, invariance
+                         under reordering a token's choices, out-of-range expert ids
+                         contributing nothing, known activation values (silu(1), gelu(1), relu2)
 """
 from __future__ import annotations
 
@@ -564,6 +571,78 @@ def e8_linear_forward(x, art, in_features, out_features, table=None):
     y_rht = (x_rht @ W.T * np.float32(art["Wscale"])).astype(np.float32)
     y = block_diag_fht(y_rht, bm) * art["SU"].astype(np.float32)[None, :]
     return y[:, :out_features].astype(np.float32)
+
+
+# --------------------------------------------------------------------------- #
+# Routed experts of a mixture-of-experts layer                                 #
+# --------------------------------------------------------------------------- #
+def gated_activation(h, intermediate, act):
+    """act(gate) * up with gate = h[:, :intermediate], up = h[:, intermediate:2*intermediate]:
+    0 SiLU, 1 GELU (tanh form), 2 squared ReLU (glq/csrc/glq_cuda.cu:4540-4559)."""
+    h = np.asarray(h, np.float32)
+    g, up = h[:, :intermediate], h[:, intermediate:2 * intermediate]
+    if act == 0:
+        a = g / (np.float32(1.0) + np.exp(-g))
+    elif act == 1:
+        a = np.float32(0.5) * g * (np.float32(1.0) + np.tanh(np.float32(0.7978845608028654)
+                                                           * (g + np.float32(0.044715) * g * g * g)))
+    elif act == 2:
+        r = np.maximum(g, np.float32(0.0))
+        a = r * r
+    else:
+        raise ValueError(act)
+    return (a * up).astype(np.float32)
+
+
+def moe_dense_experts(arts, out_features, in_features):
+    """RHT-domain fp32 weight (with Wscale) of every expert of one projection, decoded once."""
+    out = []
+    for art in arts:
+        if "trellis_packed2" in art:
+            Wn = decode_layer_nstage([art["trellis_packed"], art["trellis_packed2"]],
+                                     [1.0, float(art["inv_resid_scale2"])], out_features, in_features)
+        else:
+            Wn = decode_layer(art["trellis_packed"], out_features, in_features, fast=True)
+        out.append((Wn.astype(np.float32) * np.float32(art["Wscale"])).astype(np.float32))
+    return out
+
+
+def moe_trellis_forward(x, topk_ids, topk_weights, w13_arts, w2_arts, hidden, intermediate, act,
+                        w13_dense=None, w2_dense=None):
+    """glq_fused_moe_trellis_3inst_cuda restated token by token (glq/csrc/glq_cuda.cu:5030-5250):
+    out[t] = sum_j w[t, j] * w2_e(act(gate) * up), (gate | up) = w13_e(x[t]), e = ids[t, j]; the
+    per-slot results are rounded to fp16 after each output transform and after the activation
+    (h_w13, h_act, expert_out are fp16 tensors there), the weighted sum runs over j in order
+    in fp32 (glq_moe_weighted_scatter_reduce_kernel, :4520-4537) and is rounded to fp16.
+    Expert ids outside [0, E) contribute nothing (pad slots, m_indices = -1).  *_arts: one
+    artifact dict per expert, as for trellis_linear_forward."""
+    x = np.asarray(x, np.float32).reshape(-1, hidden)
+    ids = np.asarray(topk_ids).reshape(x.shape[0], -1)
+    w = np.asarray(topk_weights, np.float32).reshape(ids.shape)
+    E = len(w13_arts)
+    if w13_dense is None:
+        w13_dense = moe_dense_experts(w13_arts, 2 * intermediate, hidden)
+    if w2_dense is None:
+        w2_dense = moe_dense_experts(w2_arts, hidden, intermediate)
+    f16 = lambda a: a.astype(np.float16).astype(np.float32)
+    out = np.zeros((x.shape[0], hidden), np.float32)
+    for t in range(x.shape[0]):
+        acc = np.zeros(hidden, np.float32)
+        for j in range(ids.shape[1]):
+            e = int(ids[t, j])
+            if e < 0 or e >= E:
+                continue
+            a13, a2 = w13_arts[e], w2_arts[e]
+            h = f16(linear_forward_rht(x[t:t + 1], w13_dense[e], a13["SU"].astype(np.float32),
+                                       a13["SV"].astype(np.float32), a13["blocks_n"], a13["blocks_m"],
+                                       hidden, 2 * intermediate))
+            a = f16(gated_activation(h, intermediate, act))
+            y = f16(linear_forward_rht(a, w2_dense[e], a2["SU"].astype(np.float32),
+                                       a2["SV"].astype(np.float32), a2["blocks_n"], a2["blocks_m"],
+                                       intermediate, hidden))
+            acc = acc + w[t, j] * y[0]
+        out[t] = acc
+    return f16(out)
 
 
 def rel_fro(a, b) -> float:

@@ -258,6 +258,40 @@ def extras(torch, ext, dev):
         torch.cuda.empty_cache()
     except Exception as e:
         out["prefill_linear_error"] = f"{type(e).__name__}: {e}"
+    try:
+        # routed experts of one mixture-of-experts layer, Qwen3-30B-A3B expert shapes (128 experts of
+        # 2048 -> 2 x 768 -> 2048, top-8, 4 bpw, random code bits: 302 MB of streams, more than the
+        # 256 MB Infinity Cache), eight routing tables used in turn; up to 95 slots every slot reads its
+        # expert's stream, from 96 on the rows are grouped by expert
+        from glq_amd import hadamard as H
+        E, hid, inter, K = 128, 2048, 768, 8
+        gen = torch.Generator().manual_seed(0)
+
+        def proj(m, n):
+            return [torch.randint(-32768, 32768, (E, (m // 16) * (n // 16), 64), device=dev, dtype=torch.int16),
+                    torch.zeros(E, 1, 1, dtype=torch.int16, device=dev),
+                    torch.ones(E, m, dtype=torch.float16, device=dev), torch.ones(n, dtype=torch.float16, device=dev),
+                    torch.full((E,), 0.02, device=dev), torch.zeros(E, device=dev)]
+
+        def meta(n):
+            b = H.block_decompose(n)
+            return torch.tensor(b), H.pack_block_meta(b).to(dev)
+        (bn13, bn13m), (bm13, bm13m), (bn2, bn2m), (bm2, bm2m) = meta(hid), meta(2 * inter), meta(inter), meta(hid)
+        args = proj(2 * inter, hid) + proj(hid, inter) + [hid, inter, 2 * inter, hid, 2 * inter, inter, hid,
+                                                          bn13, bm13, bn13m, bm13m, bn2, bm2, bn2m, bm2m, 0]
+        for T in (1, 16, 128):                                # 8 / 128 slots per expert stream, 1024 grouped by expert
+            xb = torch.randn(T, hid, device=dev).to(torch.bfloat16)
+            routes = [(torch.stack([torch.randperm(E, generator=gen)[:K] for _ in range(T)]).to(dev),
+                       torch.rand(T, K, generator=gen).to(dev)) for _ in range(8)]
+            us = _graph_time(torch, lambda: [ext.glq_fused_moe_trellis_3inst_cuda(xb, i, w, *args) for i, w in routes],
+                             len(routes))
+            out[f"moe_experts_qwen3_30b_shape_T{T}_us"] = round(us, 2)
+            if T == 1:                                        # eight expert streams read once each
+                out["moe_experts_qwen3_30b_shape_T1_GBs"] = round(K * 3 * inter * hid / 2 / us / 1e3, 1)
+        del args
+        torch.cuda.empty_cache()
+    except Exception as e:
+        out["moe_error"] = f"{type(e).__name__}: {e}"
     return out
 
 

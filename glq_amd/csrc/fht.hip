@@ -843,6 +843,30 @@ moe_weighted_sum_kernel(const f16 *__restrict__ y, int64_t y_stride, const int64
     store8<YT>(out + (int64_t)token * out_stride + row, acc);
 }
 
+// Slots grouped by expert, without a sort: wave e counts the valid slots of experts below e
+// (offs[e]; wave n_experts: the total, offs[n_experts]) and then writes its own slots, in ascending
+// slot order, from that position on.  Fixed by the routing alone: the same table on every call.
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const int64_t *__restrict__ topk_ids, int n_slots, int n_experts, int *__restrict__ perm,
+                 int *__restrict__ offs) {
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (e > n_experts) return;                                   // uniform over the wave
+    int below = 0;
+    for (int base = 0; base < n_slots; base += 64) {
+        const int64_t id = base + lane < n_slots ? topk_ids[base + lane] : -1;
+        below += __builtin_popcountll(__ballot(id >= 0 && id < e));
+    }
+    if (lane == 0) offs[e] = below;
+    if (e == n_experts) return;
+    int mine = 0;
+    for (int base = 0; base < n_slots; base += 64) {
+        const int64_t id = base + lane < n_slots ? topk_ids[base + lane] : -1;
+        const unsigned long long hit = __ballot(id == e);
+        if (id == e) perm[below + mine + __builtin_popcountll(hit & ((1ull << lane) - 1ull))] = base + lane;
+        mine += __builtin_popcountll(hit);
+    }
+}
+
 int moe_check_blocks(const int64_t *blocks_m, int64_t n_blocks_m, int64_t m_pad, glqh_meta_args *margs,
                      int64_t *max_bs) {
     GLQH_REQUIRE(glqh_fill_meta_args(margs, n_blocks_m > 1 ? blocks_m : nullptr, n_blocks_m > 1 ? n_blocks_m : 1,
@@ -881,6 +905,14 @@ int glqh_launch_moe_gated_act(const void *h_f16, int64_t h_stride, void *out_f16
     hipLaunchKernelGGL(moe_gated_act_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                        (const f16 *)h_f16, h_stride, (f16 *)out_f16, n_slots, (int)intermediate, act);
     GLQH_LAUNCH_CHECK("routed-expert activation launch");
+    return 0;
+}
+
+int glqh_launch_moe_route(const int64_t *topk_ids, int n_slots, int n_experts, int *perm, int *offs,
+                          hipStream_t stream) {
+    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((n_experts + 1 + 3) / 4)), dim3(256), 0, stream, topk_ids,
+                       n_slots, n_experts, perm, offs);
+    GLQH_LAUNCH_CHECK("routed-expert routing launch");
     return 0;
 }
 

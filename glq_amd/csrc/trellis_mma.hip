@@ -479,6 +479,102 @@ tr_mma_fusein_moe_kernel(tr_moe_args g, const XT *__restrict__ x, int64_t x_stri
                                  g.n_slots);
 }
 
+// The same step for many slots: the slots are grouped by expert (perm: slot numbers sorted by
+// expert, offs: first position of every expert, both made on the device by the routing launch), and
+// workgroup (row block, K slot, expert) reads its expert's stream once per 16 of the expert's rows
+// (glq/csrc/glq_trellis.cu:1475-1540 pads every expert to tiles of 16 rows in the same way).  x: fp16
+// rows in the transformed domain, row of slot s = s / x_div.  Experts without rows retire.
+struct tr_moe_group_args {
+    const uint8_t *packed;
+    int64_t stride_bytes;
+    const int *perm, *offs;
+    const float *pscale_dev;
+    float *part;                                 // [K slot][slot][row]
+    int n_slots, x_div;
+};
+
+template <int R>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_moe_grouped_kernel(tr_moe_group_args g, const f16 *__restrict__ x, int m, int k, int S, int CH) {
+    extern __shared__ u32x4 xs_lds[];
+    __shared__ int slotmap[16];
+    constexpr int TPS = mma_tps<16>();
+    const int e = blockIdx.z;
+    const int o0 = g.offs[e], cnt = g.offs[e + 1] - o0;
+    if (cnt <= 0) return;                                        // uniform over the workgroup
+    const uint8_t *packed = g.packed + (int64_t)e * g.stride_bytes;
+    const float pscale = g.pscale_dev ? g.pscale_dev[e] : 1.0f;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const mma_lane a = mma_lane_of<16>(lane);
+    const int nkp = k >> 5;
+    const int mpairs = m >> 5;
+    const int kslot = blockIdx.y;
+    const int kp0 = kslot * S;
+    const int kp1 = min(kp0 + S, nkp);
+    const int mp = min(2 * (int)blockIdx.x + a.hm, mpairs - 1);
+    constexpr int REC = 4 * R;
+    const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
+    uint32_t *xs = (uint32_t *)xs_lds;
+    float *red = (float *)xs_lds;                                // [TR_WAVES][4 row groups][4][64]
+
+    for (int t0 = 0; t0 < cnt; t0 += 16) {
+        __syncthreads();                                         // the previous tile is done with slotmap and red
+        if (threadIdx.x < 16) slotmap[threadIdx.x] = t0 + (int)threadIdx.x < cnt ? g.perm[o0 + t0 + threadIdx.x] : -1;
+        int kp = kp0 + wave;
+        tr_record<R> cur = {};
+        if (kp < kp1) cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
+        mma_acc<1> acc;
+#pragma unroll
+        for (int sg = 0; sg < 4; ++sg) acc.v[sg][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int c0 = kp0; c0 < kp1; c0 += CH) {
+            const int c1 = min(c0 + CH, kp1), n = c1 - c0;
+            fht_barrier<true>();                                 // slotmap written / previous chunk consumed
+            // one item = 32 bytes of one row: columns 16 ks .. 16 ks + 15 of k-pair c0 + u
+            for (int idx = threadIdx.x; idx < 32 * n; idx += TR_THREADS) {
+                const int ks = idx & 1, u = (idx >> 1) % n, tl = (idx >> 1) / n;
+                const int sl = slotmap[tl];
+                const f16 *p = x + (int64_t)(sl < 0 ? 0 : sl / g.x_div) * k + 32 * (c0 + u) + 16 * ks;
+                u32x4 l0 = *(const u32x4 *)p, l1 = *(const u32x4 *)(p + 8);
+                if (sl < 0) l0 = l1 = u32x4{0u, 0u, 0u, 0u};
+                uint32_t *dst = xs + ((((u * 2 + ks) * 4) * TPS) + tl) * 4;
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq)
+                    *(u32x4 *)(dst + qq * TPS * 4) =
+                        u32x4{splat_lo(l0[qq]), splat_hi(l0[qq]), splat_lo(l1[qq]), splat_hi(l1[qq])};
+            }
+            fht_barrier<true>();
+            for (; kp < c1; kp += TR_WAVES) {
+                tr_record<R> nxt = cur;
+                if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
+                acc = mma_record<R, 16, 1>(cur, a.next1, a.next2, xs_lds + ((kp - c0) * 8 + a.q) * TPS + a.tokl, acc);
+                cur = nxt;
+            }
+        }
+        // the four waves' sums in wave order, then one row of part per (K slot, slot)
+        __syncthreads();
+        {
+            const int cl = a.q * 16 + a.tokl;
+#pragma unroll
+            for (int sg = 0; sg < 4; ++sg)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) red[wave * 1024 + (sg * 4 + r) * 64 + cl] = acc.v[sg][0][r];
+        }
+        __syncthreads();
+        for (int i2 = threadIdx.x; i2 < 1024; i2 += TR_THREADS) {
+            const int cl = i2 & 63, r = (i2 >> 6) & 3, sg = i2 >> 8;
+            const int i = 4 * (cl >> 4) + r;
+            const int row = 64 * blockIdx.x + 32 * (i >> 3) + (i & 7) + 8 * sg;
+            const int sl = slotmap[cl & 15];
+            if (sl < 0 || row >= m) continue;
+            float v = red[i2];
+#pragma unroll
+            for (int w = 1; w < TR_WAVES; ++w) v += red[w * 1024 + i2];
+            g.part[((int64_t)kslot * g.n_slots + sl) * m + row] = pscale * v;
+        }
+    }
+}
+
 template <int TP>
 size_t fi_lds_bytes(int S) {
     const size_t Ls = (size_t)S * 32;
@@ -539,7 +635,7 @@ template <int R>
 int mma_init_R() {
     return mma_set_lds(tr_mma_kernel<R, 1, 1>) || mma_set_lds(tr_mma_kernel<R, 4, 1>) ||
            mma_set_lds(tr_mma_kernel<R, 16, 1>) || mma_set_lds(tr_mma_kernel<R, 16, 2>) ||
-           mma_set_lds(tr_mma_kernel<R, 16, 4>);
+           mma_set_lds(tr_mma_kernel<R, 16, 4>) || mma_set_lds(tr_mma_moe_grouped_kernel<R>);
 }
 
 }  // namespace
@@ -704,6 +800,36 @@ int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes,
     }
 #undef GLQH_MOE
     return glqh_fail("routed experts: R (bits/weight) 1-4, got %d", R);
+}
+
+// One projection of all routed experts, rows grouped by expert: part[K slot][slot][row].
+int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes, int R, const int *perm,
+                                        const int *offs, int n_slots, int n_experts, int x_div,
+                                        const float *pscale_dev, const void *x_f16, int64_t m, int64_t k, int S,
+                                        int ksplit, float *part, hipStream_t stream) {
+    glqh_range range("dequant_matmul");
+    GLQH_REQUIRE(n_experts >= 1 && n_experts <= 65535 && n_slots >= 1 && x_div >= 1,
+                 "routed experts: %d experts (1..65535), %d slots", n_experts, n_slots);
+    GLQH_REQUIRE(S >= 1 && ksplit >= 1 && (int64_t)S * ksplit >= k / 32, "routed experts: K plan does not cover the row");
+    int CH = mma_chunk_cap<16, 1>();
+    if (CH > S) CH = (S + 3) & ~3;
+    size_t lds = (size_t)CH * mma_slot_bytes(16, 1);
+    if (lds < (size_t)TR_WAVES * 1024 * sizeof(float)) lds = (size_t)TR_WAVES * 1024 * sizeof(float);
+    tr_moe_group_args g = {(const uint8_t *)packed, stride_bytes, perm, offs, pscale_dev, part, n_slots, x_div};
+    const dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, (unsigned)n_experts);
+#define GLQH_MOEG(RR)                                                                                        \
+    hipLaunchKernelGGL((tr_mma_moe_grouped_kernel<RR>), grid, dim3(TR_THREADS), lds, stream, g, (const f16 *)x_f16, \
+                       (int)m, (int)k, S, CH)
+    switch (R) {
+    case 1: GLQH_MOEG(1); break;
+    case 2: GLQH_MOEG(2); break;
+    case 3: GLQH_MOEG(3); break;
+    case 4: GLQH_MOEG(4); break;
+    default: return glqh_fail("routed experts: R (bits/weight) 1-4, got %d", R);
+    }
+#undef GLQH_MOEG
+    GLQH_LAUNCH_CHECK("trellis grouped routed-expert launch");
+    return 0;
 }
 
 template <typename K>

@@ -448,7 +448,8 @@ def glq_fused_moe_trellis_3inst_cuda(x, topk_ids, topk_weights,
     dt = out_dtype or x.dtype
     out = torch.empty((T, int(hidden_size)), dtype=dt, device=x.device)
     with torch.cuda.device(x.device):
-        nb = lib.glqh_fused_moe_trellis_workspace_bytes(T, K, C.addressof(w13), C.addressof(w2))
+        nb = lib.glqh_fused_moe_trellis_workspace_bytes(T, K, w13_trellis_packed.shape[0], C.addressof(w13),
+                                                        C.addressof(w2))
         if nb == 0:
             # the entry itself reports what is wrong with the shapes
             nb = 256

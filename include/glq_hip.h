@@ -227,16 +227,19 @@ typedef struct {
     int64_t in_features, out_features, n_pad, m_pad;
 } glqh_moe_proj;
 
-size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int64_t top_k, const glqh_moe_proj *w13,
-                                              const glqh_moe_proj *w2);
+size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int64_t top_k, int64_t num_experts,
+                                              const glqh_moe_proj *w13, const glqh_moe_proj *w2);
 
 /* The routed-expert step of a mixture-of-experts layer on trellis-3INST weights,
  * out[t] = sum_j topk_weights[t][j] * w2_e( act(gate) * up ),  (gate | up) = w13_e(x[t]),
  * e = topk_ids[t][j], as one host call with the routing read on the device (no host
  * synchronisation, no allocation: capturable).  Replaces glq_fused_moe_trellis_3inst_cuda
  * (glq/csrc/glq_cuda.cu:5030-5250; grouped matmul glq/csrc/glq_trellis.cu:1475-1540) behind
- * torch.ops.glq.fused_moe_trellis_3inst (glq_vllm/custom_ops.py:22-36).  Every (token, choice)
- * slot is one fused-input GEMV on that expert's stream; intermediate results are rounded to
+ * torch.ops.glq.fused_moe_trellis_3inst (glq_vllm/custom_ops.py:22-36).  With few (token,
+ * choice) slots every slot is one fused-input GEMV on its expert's stream; from
+ * max(16, 3/4 num_experts) slots on a routing launch groups the slots by expert and every
+ * expert's stream is read once per 16 of its rows (GLQ_MOE_GROUP_MIN sets that count).
+ * Intermediate results are rounded to
  * fp16 where the reference rounds them (after each output transform and after the
  * activation), the weighted sum runs over the choices in order in fp32.  activation_type:
  * 0 SiLU, 1 GELU (tanh form), 2 squared ReLU, each times the up half.  Expert ids outside

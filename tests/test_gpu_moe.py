@@ -197,6 +197,44 @@ def test_refusals(ext):
         ext.glq_fused_moe_trellis_3inst_cuda(x, ids, w, *b)
 
 
+@pytest.mark.parametrize("hidden,inter,T,K,K2", [(256, 128, 16, 4, 0), (320, 192, 40, 2, 0), (320, 192, 33, 3, 2)])
+def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
+    """From max(16, 3/4 of the experts) slots on the rows are grouped by expert.  Skewed routing: every token's first choice is
+    expert 2 (more than two tiles of 16 rows for it), expert 5 gets nothing, some ids are out of range."""
+    say("moe grouped", hidden, inter, T, K, K2)
+    ex = experts(6, hidden, inter, 4, K2, seed=2)
+    rng = np.random.default_rng(T)
+    ids = np.stack([np.concatenate([[2], rng.permutation([0, 1, 3, 4])[:K - 1]]) for _ in range(T)]).astype(np.int64)
+    ids[3, K - 1] = -1
+    ids[T - 1, 0] = 6
+    w = rng.random((T, K)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((T, hidden)).astype(np.float32)).bfloat16()
+    a = ex.device_args(1)
+    y = ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a)
+    ref = ex.oracle(x.float().numpy(), ids, w, 1)
+    assert rel(y, ref) < TOL, rel(y, ref)
+    worst = max(rel(y[i], ref[i]) for i in range(T))
+    assert worst < 3 * TOL, worst                            # no single token is off
+    assert torch.equal(y, ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a))
+
+
+@pytest.mark.parametrize("group_min", ["1", "1000000"])
+def test_both_forms_on_every_case_in_a_fresh_process(group_min):
+    """GLQ_MOE_GROUP_MIN (read once by the library) moves the slot count from which rows are grouped by
+    expert: with 1 every case of this file runs in the grouped form, with 1000000 in the per-slot form,
+    each against the oracle, in a process of its own."""
+    import os
+    import subprocess
+    import sys
+    say("moe forms, child process", group_min)
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu",
+                        "-k", "not fresh_process", "--timeout", "300", "--timeout-method", "thread",
+                        "-p", "no:cacheprovider"],
+                       env={**os.environ, "GLQ_MOE_GROUP_MIN": group_min}, capture_output=True, text=True, timeout=900,
+                       cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
+
+
 @pytest.mark.parametrize("T", [1, 4])
 def test_qwen3_moe_expert_shapes(ext, T):
     """Expert shapes of a Qwen3-MoE layer (hidden 2048, intermediate 768, top-8), 16 of the experts,

@@ -116,6 +116,36 @@ def _graph_time(torch, fn, n_inner, reps=10):
     return e0.elapsed_time(e1) * 1e3 / (reps * n_inner)
 
 
+def moe_setup(torch, dev):
+    """Routed experts of one mixture-of-experts layer, Qwen3-30B-A3B expert shapes (128 experts of
+    2048 -> 2 x 768 -> 2048, top-8, 4 bpw, random code bits: 302 MB of streams, more than the 256 MB
+    Infinity Cache).  Returns the op's weight arguments, a maker of (x, eight routing tables) for a
+    token count, and the packed bytes of one expert.  Up to 95 slots every slot reads its expert's
+    stream; from 96 on the rows are grouped by expert."""
+    from glq_amd import hadamard as H
+    E, hid, inter, K = 128, 2048, 768, 8
+    gen = torch.Generator().manual_seed(0)
+
+    def proj(m, n):
+        return [torch.randint(-32768, 32768, (E, (m // 16) * (n // 16), 64), device=dev, dtype=torch.int16),
+                torch.zeros(E, 1, 1, dtype=torch.int16, device=dev),
+                torch.ones(E, m, dtype=torch.float16, device=dev), torch.ones(n, dtype=torch.float16, device=dev),
+                torch.full((E,), 0.02, device=dev), torch.zeros(E, device=dev)]
+
+    def meta(n):
+        b = H.block_decompose(n)
+        return torch.tensor(b), H.pack_block_meta(b).to(dev)
+    (bn13, bn13m), (bm13, bm13m), (bn2, bn2m), (bm2, bm2m) = meta(hid), meta(2 * inter), meta(inter), meta(hid)
+    args = proj(2 * inter, hid) + proj(hid, inter) + [hid, inter, 2 * inter, hid, 2 * inter, inter, hid,
+                                                      bn13, bm13, bn13m, bm13m, bn2, bm2, bn2m, bm2m, 0]
+
+    def routes_for(T):
+        xb = torch.randn(T, hid, device=dev).to(torch.bfloat16)
+        return xb, [(torch.stack([torch.randperm(E, generator=gen)[:K] for _ in range(T)]).to(dev),
+                     torch.rand(T, K, generator=gen).to(dev)) for _ in range(8)]
+    return args, routes_for, 3 * inter * hid // 2
+
+
 def extras(torch, ext, dev):
     """Side measurements of the other benchmark configurations (bounded, a few seconds): whole-model
     batch-1 decode tok/s (config 5), large-layer GEMV rates where the kernels are not launch
@@ -259,35 +289,14 @@ def extras(torch, ext, dev):
     except Exception as e:
         out["prefill_linear_error"] = f"{type(e).__name__}: {e}"
     try:
-        # routed experts of one mixture-of-experts layer, Qwen3-30B-A3B expert shapes (128 experts of
-        # 2048 -> 2 x 768 -> 2048, top-8, 4 bpw, random code bits: 302 MB of streams, more than the
-        # 256 MB Infinity Cache), eight routing tables used in turn; up to 95 slots every slot reads its
-        # expert's stream, from 96 on the rows are grouped by expert
-        from glq_amd import hadamard as H
-        E, hid, inter, K = 128, 2048, 768, 8
-        gen = torch.Generator().manual_seed(0)
-
-        def proj(m, n):
-            return [torch.randint(-32768, 32768, (E, (m // 16) * (n // 16), 64), device=dev, dtype=torch.int16),
-                    torch.zeros(E, 1, 1, dtype=torch.int16, device=dev),
-                    torch.ones(E, m, dtype=torch.float16, device=dev), torch.ones(n, dtype=torch.float16, device=dev),
-                    torch.full((E,), 0.02, device=dev), torch.zeros(E, device=dev)]
-
-        def meta(n):
-            b = H.block_decompose(n)
-            return torch.tensor(b), H.pack_block_meta(b).to(dev)
-        (bn13, bn13m), (bm13, bm13m), (bn2, bn2m), (bm2, bm2m) = meta(hid), meta(2 * inter), meta(inter), meta(hid)
-        args = proj(2 * inter, hid) + proj(hid, inter) + [hid, inter, 2 * inter, hid, 2 * inter, inter, hid,
-                                                          bn13, bm13, bn13m, bm13m, bn2, bm2, bn2m, bm2m, 0]
+        args, routes_for, per_slot_bytes = moe_setup(torch, dev)
         for T in (1, 16, 128):                                # 8 / 128 slots per expert stream, 1024 grouped by expert
-            xb = torch.randn(T, hid, device=dev).to(torch.bfloat16)
-            routes = [(torch.stack([torch.randperm(E, generator=gen)[:K] for _ in range(T)]).to(dev),
-                       torch.rand(T, K, generator=gen).to(dev)) for _ in range(8)]
+            xb, routes = routes_for(T)
             us = _graph_time(torch, lambda: [ext.glq_fused_moe_trellis_3inst_cuda(xb, i, w, *args) for i, w in routes],
                              len(routes))
             out[f"moe_experts_qwen3_30b_shape_T{T}_us"] = round(us, 2)
             if T == 1:                                        # eight expert streams read once each
-                out["moe_experts_qwen3_30b_shape_T1_GBs"] = round(K * 3 * inter * hid / 2 / us / 1e3, 1)
+                out["moe_experts_qwen3_30b_shape_T1_GBs"] = round(per_slot_bytes * 8 / us / 1e3, 1)
         del args
         torch.cuda.empty_cache()
     except Exception as e:
@@ -296,7 +305,7 @@ def extras(torch, ext, dev):
 
 
 CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
-         "e8_prefill_256", "decoder", "batch1_step")
+         "e8_prefill_256", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 
@@ -354,6 +363,13 @@ def run_case(torch, ext, dev, name, steps):
                     xs[a["n"]], [(l["sv"], l["su"], l["packed"], l["wscale"], l["m"], l["m"]) for l in lins],
                     a["bn"], a["bn_meta"], a["n"], a["n"], out_dtype=torch.bfloat16)
         res["bytes_per_launch"] = sum(m * n * K_BITS // 8 for _, m, n in LINEARS)
+    elif name.startswith("moe_experts_"):
+        T = int(name.rsplit("_", 1)[1])
+        args, routes_for, per_slot_bytes = moe_setup(torch, dev)
+        xb, routes = routes_for(T)
+        fn = lambda i: ext.glq_fused_moe_trellis_3inst_cuda(xb, *routes[i % 8], *args)
+        res["slots"] = T * 8
+        res["bytes_per_slot"] = per_slot_bytes
     elif name == "decoder":
         from glq_amd.decoder import TrellisDecoder
         dec = TrellisDecoder(max_len=1024)

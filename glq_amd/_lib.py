@@ -56,6 +56,13 @@ SIGNATURES = {
     "glqh_e8_dequant_matmul": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
                 c_dbl, c_dbl, c_dbl, c_dbl, c_i64, c_i64, c_vp, c_vp, c_sz, c_vp]),
+    "glqh_e8_dequant_matmul_folded": (
+        c_int, [c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
+                c_dbl, c_dbl, c_dbl, c_dbl, c_i64, c_i64, c_vp, c_vp, c_sz, c_vp, c_vp]),
+    "glqh_e8_fold_table": (c_int, [c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp]),
+    "glqh_e8_fold_indices": (c_int, [c_vp, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp]),
+    "glqh_e8_folded_count": (c_i64, [c_i64, c_i64]),
+    "glqh_e8_fold_eligible": (c_int, [c_i64, c_i64, c_i64]),
     "glqh_e8_decompress": (
         c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_i64, c_i64,
                 c_vp, c_vp]),
@@ -68,6 +75,11 @@ SIGNATURES = {
                 c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_dbl,
                 c_vp, c_i64, c_vp, c_i64, c_vp, c_vp,
                 c_i64, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_sz, c_vp]),
+    "glqh_fused_linear_e8_folded": (
+        c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
+                c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_dbl,
+                c_vp, c_i64, c_vp, c_i64, c_vp, c_vp,
+                c_i64, c_i64, c_i64, c_i64, c_vp, c_int, c_i64, c_vp, c_sz, c_vp, c_vp]),
     "glqh_fused_linear_trellis_group_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64, c_int]),
     "glqh_fused_linear_trellis_3inst_group": (
         c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_int, c_vp, c_i64, c_vp, c_i64, c_i64, c_int, c_i64,

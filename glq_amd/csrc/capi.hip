@@ -1,4 +1,7 @@
 // extern "C" entry points of libglq_hip.so: argument checks, dispatch, no allocation.
+#include <unordered_map>
+#include <vector>
+
 #include "common.h"
 
 #include <mutex>
@@ -1020,6 +1023,78 @@ extern "C" int glqh_e8_repack_table(const uint32_t *codebook_packed, int64_t n_e
     return glqh_launch_e8_repack_table(codebook_packed, n_entries, packed_out, bad_dev, (hipStream_t)stream);
 }
 
+extern "C" int glqh_e8_fold_table(const uint32_t *table, int64_t n_entries, void *halves_out, int64_t capacity,
+                                  uint32_t *map_out, int64_t *n_halves_out, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(table && halves_out && map_out && n_halves_out, "e8 fold table: null pointer");
+    GLQH_REQUIRE(n_entries >= 1 && n_entries <= 65536 && capacity >= 1, "e8 fold table: %lld entries (1..65536)",
+                 (long long)n_entries);
+    hipStream_t st = (hipStream_t)stream;
+    std::vector<uint32_t> words((size_t)n_entries), map((size_t)n_entries);
+    std::vector<uint16_t> halves;                                  // 4 fp16 bit patterns per entry
+    if (glqh_check_hip(hipMemcpyAsync(words.data(), table, (size_t)n_entries * 4, hipMemcpyDeviceToHost, st),
+                       "e8 fold table: copy to host") ||
+        glqh_check_hip(hipStreamSynchronize(st), "e8 fold table: synchronize"))
+        return 1;
+    std::unordered_map<uint32_t, uint32_t> number;                 // four codes of a half -> its number
+    for (int64_t k = 0; k < n_entries; ++k) {
+        uint32_t ids[2];
+        for (int h = 0; h < 2; ++h) {
+            uint32_t key = 0;
+            uint16_t bits[4];
+            for (int c = 0; c < 4; ++c) {
+                const int col = 4 * h + c;                         // nibble p = column 2p, nibble p + 4 = column 2p + 1
+                const int code = (int)((words[(size_t)k] >> (4 * ((col >> 1) + 4 * (col & 1)))) & 15u);
+                GLQH_REQUIRE(code <= 12, "e8 fold table: entry %lld holds a code above 12", (long long)k);
+                key |= (uint32_t)code << (4 * c);
+                // fp16 bits of (code - 6) / 2: sign, then magnitude m / 2 for m = 1..6
+                static const uint16_t mag[7] = {0x0000, 0x3800, 0x3C00, 0x3E00, 0x4000, 0x4100, 0x4200};
+                bits[c] = (uint16_t)(mag[code < 6 ? 6 - code : code - 6] | (code < 6 ? 0x8000 : 0));
+            }
+            auto it = number.find(key);
+            if (it == number.end()) {
+                it = number.emplace(key, (uint32_t)(halves.size() / 4)).first;
+                halves.insert(halves.end(), bits, bits + 4);
+            }
+            ids[h] = it->second;
+        }
+        map[(size_t)k] = ids[0] | ids[1] << 16;
+    }
+    const size_t n = halves.size() / 4;
+    *n_halves_out = (int64_t)n;
+    GLQH_REQUIRE((int64_t)n <= capacity && n <= 2048, "e8 fold table: %zu half codewords, room for %lld (at most 2048)", n,
+                 (long long)capacity);
+    if (glqh_check_hip(hipMemcpyAsync(halves_out, halves.data(), n * 8, hipMemcpyHostToDevice, st),
+                       "e8 fold table: half codewords to device") ||
+        glqh_check_hip(hipMemcpyAsync(map_out, map.data(), (size_t)n_entries * 4, hipMemcpyHostToDevice, st),
+                       "e8 fold table: map to device") ||
+        glqh_check_hip(hipStreamSynchronize(st), "e8 fold table: synchronize"))
+        return 1;
+    return 0;
+}
+
+int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1);
+
+extern "C" int glqh_e8_fold_eligible(int64_t m_pad, int64_t n_pad, int64_t B) {
+    if (glqh_init() != 0 || m_pad < 1 || n_pad < 8 || (n_pad & 7) || B < 1) return 0;
+    return glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536) > 0 ? 1 : 0;
+}
+
+extern "C" int64_t glqh_e8_folded_count(int64_t rows, int64_t cols) {
+    if (rows < 1 || cols < 1) return 0;
+    return ((rows + 15) / 16) * ((cols + 31) / 32) * 512;
+}
+
+extern "C" int glqh_e8_fold_indices(const void *q, int64_t rows, int64_t cols, const uint32_t *map, int64_t n_entries,
+                                    uint16_t *lo16_out, uint8_t *hi8_out, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(q && map && lo16_out && hi8_out, "e8 fold indices: null pointer");
+    GLQH_REQUIRE(rows >= 1 && cols >= 1 && n_entries >= 1 && n_entries <= 65536,
+                 "e8 fold indices: %lld x %lld indices, %lld entries", (long long)rows, (long long)cols,
+                 (long long)n_entries);
+    return glqh_launch_e8_fold_indices(q, rows, cols, map, n_entries, lo16_out, hi8_out, (hipStream_t)stream);
+}
+
 struct e8_stages {
     const void *q[4];
     float scale[4];
@@ -1084,6 +1159,16 @@ extern "C" int glqh_e8_dequant_matmul(const void *x_f16, int64_t B, const void *
                                       double inv_rs, double inv_rs2, double inv_rs3, int64_t m_pad,
                                       int64_t n_pad, float *out, void *ws, size_t ws_bytes,
                                       void *stream) {
+    return glqh_e8_dequant_matmul_folded(x_f16, B, q1, q2, q3, q4, table1, table2, n_entries2, wscale, inv_rs, inv_rs2,
+                                         inv_rs3, m_pad, n_pad, out, ws, ws_bytes, stream, nullptr);
+}
+
+extern "C" int glqh_e8_dequant_matmul_folded(const void *x_f16, int64_t B, const void *q1, const void *q2,
+                                             const void *q3, const void *q4, const uint32_t *table1,
+                                             const uint32_t *table2, int64_t n_entries2, double wscale,
+                                             double inv_rs, double inv_rs2, double inv_rs3, int64_t m_pad,
+                                             int64_t n_pad, float *out, void *ws, size_t ws_bytes, void *stream,
+                                             const glqh_e8_folded *folded) {
     GLQH_INIT();
     GLQH_REQUIRE(x_f16 && out, "e8 matmul: null pointer");
     e8_stages sg;
@@ -1109,7 +1194,7 @@ extern "C" int glqh_e8_dequant_matmul(const void *x_f16, int64_t B, const void *
     // every stage's partial sums are written already multiplied by that stage's scale: one
     // reduction over ks * stages plain slots instead of one launch per stage
     if (glqh_launch_e8_partial(x_f16, B, sg.q, sg.n, table1, table2 ? table2 : table1,
-                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st, sg.scale))
+                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st, sg.scale, folded))
         return 1;
     return glqh_launch_reduce_splits(part, ks * sg.n, B * m_pad, B, m_pad, 1.0f, out, m_pad, 0, st);
 }
@@ -1161,6 +1246,23 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
                                     int64_t out_features, int64_t n_pad, int64_t m_pad, void *y,
                                     int y_dtype, int64_t y_stride, void *ws, size_t ws_bytes,
                                     void *stream) {
+    return glqh_fused_linear_e8_folded(x, x_dtype, x_stride, B, sv_f16, su_f16, q1, q2, q3, q4, table1, table2,
+                                       n_entries2, wscale, inv_rs, inv_rs2, inv_rs3, blocks_n, n_blocks_n, blocks_m,
+                                       n_blocks_m, bn_meta_dev, bm_meta_dev, in_features, out_features, n_pad, m_pad,
+                                       y, y_dtype, y_stride, ws, ws_bytes, stream, nullptr);
+}
+
+extern "C" int glqh_fused_linear_e8_folded(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                           const void *sv_f16, const void *su_f16, const void *q1,
+                                           const void *q2, const void *q3, const void *q4,
+                                           const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                           double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                                           const int64_t *blocks_n, int64_t n_blocks_n, const int64_t *blocks_m,
+                                           int64_t n_blocks_m, const glqh_block_meta *bn_meta_dev,
+                                           const glqh_block_meta *bm_meta_dev, int64_t in_features,
+                                           int64_t out_features, int64_t n_pad, int64_t m_pad, void *y,
+                                           int y_dtype, int64_t y_stride, void *ws, size_t ws_bytes,
+                                           void *stream, const glqh_e8_folded *folded) {
     GLQH_INIT();
     GLQH_REQUIRE(x && sv_f16 && su_f16 && y, "fused e8 linear: null pointer");
     e8_stages sg;
@@ -1215,7 +1317,8 @@ extern "C" int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride
                                                           n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
                            canon_m.canon == m_pad;
     if (glqh_launch_e8_partial(x_rht, B, sg.q, sg.n, table1, table2 ? table2 : table1,
-                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st, canon_out ? sg.scale : nullptr))
+                               table2 ? n_entries2 : 65536, m_pad, n_pad, ks, part, st, canon_out ? sg.scale : nullptr,
+                               folded))
         return 1;
     if (canon_out) {
         const float *pt[1] = {part};

@@ -162,7 +162,9 @@ struct glqh_e8_pscale {
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream,
-                           const float *pscale = nullptr);
+                           const float *pscale = nullptr, const glqh_e8_folded *fold = nullptr);
+int glqh_launch_e8_fold_indices(const void *q, int64_t rows, int64_t cols, const uint32_t *map, int64_t n_entries,
+                                uint16_t *lo16_out, uint8_t *hi8_out, hipStream_t stream);
 int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,
                               const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
                               int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream);

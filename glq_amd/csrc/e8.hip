@@ -284,7 +284,7 @@ int glqh_e8_mma_init(void);
 int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1);
 int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
-                       hipStream_t stream, const float *pscale);
+                       hipStream_t stream, const float *pscale, const glqh_e8_folded *fold);
 
 int glqh_e8_init(void) {
     if (glqh_check_hip(hipFuncSetAttribute((const void *)e8_decompress_lds_kernel,
@@ -310,6 +310,44 @@ int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B) {
     return (int)ks;
 }
 
+namespace {
+// index -> (16-bit word, byte) of its two half numbers through the map of glqh_e8_fold_table, written
+// in the order the small-batch kernel reads: tiles of 16 rows x 32 indices, inside a tile the 8
+// consecutive indices of lane 16 g + i (row i of the tile, indices 8 g .. 8 g + 7) at entry 8 * lane,
+// so that a wave's load of a step is one contiguous kilobyte.  Rows and columns are padded to whole
+// tiles with half number 0; indices past the table are clamped as the kernels clamp them.
+__global__ void __launch_bounds__(256)
+e8_fold_indices_kernel(const uint16_t *__restrict__ q, int rows, int cols, const uint32_t *__restrict__ map,
+                       uint32_t n_entries, uint16_t *__restrict__ lo16, uint8_t *__restrict__ hi8, int64_t count) {
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= count) return;
+    const int col_tiles = (cols + 31) >> 5;
+    const int64_t tile = o >> 9;
+    const int lane = (int)(o >> 3) & 63, e = (int)o & 7;
+    const int row = (int)(tile / col_tiles) * 16 + (lane & 15);
+    const int col = (int)(tile % col_tiles) * 32 + 8 * (lane >> 4) + e;
+    uint32_t first = 0, second = 0;
+    if (row < rows && col < cols) {
+        const uint32_t m = map[min((uint32_t)q[(int64_t)row * cols + col], n_entries - 1u)];
+        first = m & 0xFFFFu;
+        second = m >> 16;
+    }
+    lo16[o] = (uint16_t)(first | (second & 31u) << 11);
+    hi8[o] = (uint8_t)(second >> 5);
+}
+}  // namespace
+
+int glqh_launch_e8_fold_indices(const void *q, int64_t rows, int64_t cols, const uint32_t *map, int64_t n_entries,
+                                uint16_t *lo16_out, uint8_t *hi8_out, hipStream_t stream) {
+    const int64_t count = ((rows + 15) / 16) * ((cols + 31) / 32) * 512;
+    GLQH_REQUIRE(rows <= 2147483647ll && cols <= 2147483647ll && (count + 255) / 256 <= 2147483647ll,
+                 "e8 fold: too many indices");
+    hipLaunchKernelGGL(e8_fold_indices_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream,
+                       (const uint16_t *)q, (int)rows, (int)cols, map, (uint32_t)n_entries, lo16_out, hi8_out, count);
+    GLQH_LAUNCH_CHECK("e8 fold indices launch");
+    return 0;
+}
+
 int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, int32_t *bad,
                               hipStream_t stream) {
     hipLaunchKernelGGL(e8_pack_table_kernel, dim3((unsigned)((n_entries + 255) / 256)), dim3(256), 0,
@@ -328,13 +366,15 @@ int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t 
 
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
-                           int64_t n_pad, int ksplit, float *part, hipStream_t stream, const float *pscale) {
+                           int64_t n_pad, int ksplit, float *part, hipStream_t stream, const float *pscale,
+                           const glqh_e8_folded *fold) {
     glqh_range range("dequant_matmul");
     glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
     if (pscale)
         for (int i = 0; i < 4; ++i) ps.v[i] = pscale[i];
+    // the folded streams serve the LDS-table kernel only; every other route reads the indices themselves
     if (glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536) > 0)
-        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream, pscale);
+        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream, pscale, fold);
     switch (nstages) {
     case 1: return launch_e8_NS<1>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);
     case 2: return launch_e8_NS<2>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);

@@ -30,23 +30,38 @@ constexpr int EM_WAVES = 16;
 constexpr int EM_THREADS = EM_WAVES * GLQH_WAVE;
 constexpr int EM_STEP_BLKS = 32;               // 8-column blocks a wave covers per step
 
-template <int NS>
+// FOLD: the folded form of the streams (glqh_e8_fold_table / glqh_e8_fold_indices).  The 65536
+// codewords of the shell table are built from only 1286 distinct half codewords (columns 0..3 or
+// 4..7 with their signs), so a table of those as finished fp16 values (8 bytes each, 10 KB) fits
+// LDS whole: a lookup is two 8-byte LDS reads that are the MFMA operand as they arrive, no lookup
+// leaves the CU and nothing is expanded.  An index becomes two 11-bit half numbers, stored as a
+// 16-bit word (first half | low 5 bits of the second << 11) and a byte (its high 6 bits): 3 bytes
+// instead of 2.
+template <int NS, bool FOLD>
 struct em_idx {
     u32x4 v[NS];                               // 8 indices per stage, two per dword
+    u32x2 sg[FOLD ? NS : 1];                   // FOLD: their 8 high bytes
 };
 
-template <int NS>
-__device__ __forceinline__ em_idx<NS> em_load_idx(const uint16_t *const q[4], int64_t off) {
-    em_idx<NS> r;
+struct em_signs {
+    const uint8_t *p[4];                       // byte planes of the folded form, (m_pad, n_pad / 8) bytes per stage
+};
+
+template <int NS, bool FOLD>
+__device__ __forceinline__ em_idx<NS, FOLD> em_load_idx(const uint16_t *const q[4], const em_signs &sp, int64_t off) {
+    em_idx<NS, FOLD> r;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) r.v[s] = __builtin_nontemporal_load((const u32x4 *)(q[s] + off));
+    for (int s = 0; s < NS; ++s) {
+        r.v[s] = __builtin_nontemporal_load((const u32x4 *)(q[s] + off));
+        if constexpr (FOLD) r.sg[s] = __builtin_nontemporal_load((const u32x2 *)(sp.p[s] + off));
+    }
     return r;
 }
 
-template <int NS, int TP, int WK>
+template <int NS, int TP, int WK, bool FOLD>
 __global__ void __launch_bounds__(EM_THREADS)
 e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
-              const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
+              const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4, em_signs sp,
               const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n1, uint32_t n2,
               int t2_is_t1, const f16 *__restrict__ x, int B, int m_pad, int n_pad, int P, int slot_blks,
               int xs_slots, int ksplit, int ns_total, int s_off, float *__restrict__ part,
@@ -54,7 +69,8 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
     constexpr int WR = EM_WAVES / WK;
     constexpr int ROWS = 16 * WR;
     extern __shared__ u32x4 lds[];
-    uint32_t *tab = (uint32_t *)lds;                           // P entries
+    uint32_t *tab = (uint32_t *)lds;                           // P words (FOLD: the stage-1 half codewords, two
+                                                               // words each, then stage 2's if they differ)
     u32x4 *xs = lds + P / 4;                                   // xs_slots slots, then 8*TP zero slots
     const int nblk = n_pad >> 3;
     const int lane = threadIdx.x & 63;
@@ -81,10 +97,18 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
         const int slot = tile / RB, rb = tile % RB;
         const int row = rb * ROWS + wr * 16 + i;
         const int b0 = slot * slot_blks + ((sidx % spt) * WK + wk) * EM_STEP_BLKS;
+        if constexpr (FOLD) {                                  // tile (16 rows, 32 indices), 8 entries per lane
+            const int col_tiles = (nblk + 31) >> 5, row_tiles = (m_pad + 15) >> 4;
+            const int rt = min(rb * WR + wr, row_tiles - 1), ct = min(b0 >> 5, col_tiles - 1);
+            return (((int64_t)rt * col_tiles + ct) * 64 + lane) * 8;
+        }
         return (int64_t)min(row, m_pad - 1) * nblk + min(b0 + 8 * g, nblk - 8);
     };
-    em_idx<NS> cur = em_load_idx<NS>(qs, idx_offset(0));
-    em_idx<NS> nx1 = em_load_idx<NS>(qs, idx_offset(1));
+    em_idx<NS, FOLD> cur = em_load_idx<NS, FOLD>(qs, sp, idx_offset(0));
+    em_idx<NS, FOLD> nx1 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(1));
+    // FOLD: byte offset of stage 2's half codewords inside tab
+    const uint32_t n1r = (n1 + 1u) & ~1u;
+    const uint32_t tab2_off = t2_is_t1 ? 0u : 8u * n1r;
 
     // activations of a slot: one 16-byte LDS slot per (block, token), zero past B and n_pad
     auto x_load = [&](int sb0, int j) -> u32x4 {
@@ -107,11 +131,17 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
         const int sb0 = ((int)blockIdx.x / RB) * slot_blks;
 #pragma unroll
         for (int u = 0; u < 4; ++u) xv[u] = x_load(sb0, u * EM_THREADS + (int)threadIdx.x);
+        if constexpr (FOLD) {
+            for (uint32_t j = threadIdx.x; j < 2u * n1; j += EM_THREADS) tab[j] = t1[j];
+            if (!t2_is_t1)
+                for (uint32_t j = threadIdx.x; j < 2u * n2; j += EM_THREADS) tab[2u * n1r + j] = t2[j];
+        } else {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if ((u * EM_WAVES + wave) * GLQH_WAVE < P / 4)     // uniform over the wave
-                __builtin_amdgcn_global_load_lds((const u32x4 *)t1 + u * EM_THREADS + threadIdx.x,
-                                                 lds + (u * EM_WAVES + wave) * GLQH_WAVE, 16, 0, 0);
+            for (int u = 0; u < U; ++u) {
+                if ((u * EM_WAVES + wave) * GLQH_WAVE < P / 4)     // uniform over the wave
+                    __builtin_amdgcn_global_load_lds((const u32x4 *)t1 + u * EM_THREADS + threadIdx.x,
+                                                     lds + (u * EM_WAVES + wave) * GLQH_WAVE, 16, 0, 0);
+            }
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) x_store(u * EM_THREADS + (int)threadIdx.x, xv[u]);
@@ -141,6 +171,42 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
         for (int st = 0; st < spt; ++st, ++sidx) {
             const int b0 = sb0 + (st * WK + wk) * EM_STEP_BLKS;  // blocks [b0, b0+32), lane's run b0 + 8g
             const u32x4 *xl = live ? xs + (b0 - sb0 + 8 * g) * TP + i : zero_slots;
+            if constexpr (FOLD) {
+                em_idx<NS, FOLD> nx2 = nx1;
+                if (sidx + 2 < nsteps) nx2 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(sidx + 2));   // uniform
+                const char *tb = (const char *)tab;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {                  // four lookups per stage at a time: 32 registers of operands
+                    u32x4 af[NS][4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int t = 4 * h + u;
+#pragma unroll
+                        for (int s = 0; s < NS; ++s) {
+                            const uint32_t w = cur.v[s][t >> 1], sw = cur.sg[s][t >> 2];
+                            // byte offsets 8 * half number: first half from bits 0..10 of the index's 16-bit
+                            // word, second from its bits 11..15 and the index's byte
+                            const uint32_t lo = t & 1 ? (w >> 13) & 0x3FF8u : (w << 3) & 0x3FF8u;
+                            const uint32_t h5 = t & 1 ? (w >> 24) & 0xF8u : (w >> 8) & 0xF8u;
+                            const uint32_t b6 = u == 0 ? (sw << 8) & 0x3F00u : u == 1 ? sw & 0x3F00u
+                                              : u == 2 ? (sw >> 8) & 0x3F00u : (sw >> 16) & 0x3F00u;
+                            const char *tbs = tb + (s == 1 ? tab2_off : 0u);
+                            const u32x2 c03 = *(const u32x2 *)(tbs + lo), c47 = *(const u32x2 *)(tbs + (h5 | b6));
+                            af[s][u] = u32x4{c03[0], c03[1], c47[0], c47[1]};
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const f16x8 bf = __builtin_bit_cast(f16x8, xl[(4 * h + u) * TP]);
+#pragma unroll
+                        for (int s = 0; s < NS; ++s)
+                            acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[s][u]), bf, acc[s], 0, 0, 0);
+                    }
+                }
+                cur = nx1;
+                nx1 = nx2;
+                continue;
+            }
             // all lookups of the step first: LDS for the prefix, L2 for the tail
             uint32_t wl[NS][8], wg[NS][8];
             bool hit[NS][8];
@@ -159,8 +225,8 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                 }
             }
             // requested after the lookups, so that waiting for those does not wait for this
-            em_idx<NS> nx2 = nx1;
-            if (sidx + 2 < nsteps) nx2 = em_load_idx<NS>(qs, idx_offset(sidx + 2));   // uniform
+            em_idx<NS, FOLD> nx2 = nx1;
+            if (sidx + 2 < nsteps) nx2 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(sidx + 2));   // uniform
             if (b0 < nblk_r) {                                 // uniform; past the row the activations are zero
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
@@ -258,27 +324,28 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
     return 1;
 }
 
-template <int NS, int TP, int WK>
-int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
-              const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad, int ns_total,
-              int s_off, float *part, hipStream_t stream, glqh_e8_pscale ps) {
-    hipLaunchKernelGGL((e8_mma_kernel<NS, TP, WK>), dim3((unsigned)p.grid), dim3(EM_THREADS), p.lds, stream,
+template <int NS, int TP, int WK, bool FOLD>
+int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4], const em_signs &sp,
+              const uint32_t *t1, const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad,
+              int ns_total, int s_off, float *part, hipStream_t stream, glqh_e8_pscale ps) {
+    hipLaunchKernelGGL((e8_mma_kernel<NS, TP, WK, FOLD>), dim3((unsigned)p.grid), dim3(EM_THREADS), p.lds, stream,
                        (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
-                       (const uint16_t *)q[3], t1, t2, (uint32_t)n1, (uint32_t)n2, (int)(t1 == t2 && n1 == n2),
+                       (const uint16_t *)q[3], sp, t1, t2, (uint32_t)n1, (uint32_t)n2, (int)(t1 == t2 && n1 == n2),
                        (const f16 *)x, (int)B, (int)m_pad, (int)n_pad, p.P, p.slot_blks, p.xs_slots, p.ksplit,
                        ns_total, s_off, part, ps);
     GLQH_LAUNCH_CHECK("e8 mma launch");
     return 0;
 }
 
-template <int NS>
-int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q[4], const uint32_t *t1,
-                 const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad, int ns_total,
-                 int s_off, float *part, hipStream_t stream, const float *pscale) {
+template <int NS, bool FOLD>
+int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q[4], const em_signs &sp,
+                 const uint32_t *t1, const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad,
+                 int ns_total, int s_off, float *part, hipStream_t stream, const float *pscale) {
     glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
     if (pscale)
         for (int i = 0; i + s_off < 4; ++i) ps.v[i] = pscale[s_off + i];
-#define GLQH_EM(TP, WK) em_launch<NS, TP, WK>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, part, stream, ps)
+#define GLQH_EM(TP, WK) em_launch<NS, TP, WK, FOLD>(p, x, B, q, sp, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, \
+                                                    part, stream, ps)
     if (p.TP == 1) return GLQH_EM(1, 4);
     if (p.TP == 4) return GLQH_EM(4, 4);
     return GLQH_EM(16, 1);
@@ -294,8 +361,9 @@ int em_set_lds(K kernel) {
 
 template <int NS>
 int em_init_NS() {
-    return em_set_lds(e8_mma_kernel<NS, 1, 4>) || em_set_lds(e8_mma_kernel<NS, 4, 4>) ||
-           em_set_lds(e8_mma_kernel<NS, 16, 1>);
+    return em_set_lds(e8_mma_kernel<NS, 1, 4, false>) || em_set_lds(e8_mma_kernel<NS, 4, 4, false>) ||
+           em_set_lds(e8_mma_kernel<NS, 16, 1, false>) || em_set_lds(e8_mma_kernel<NS, 1, 4, true>) ||
+           em_set_lds(e8_mma_kernel<NS, 4, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 1, true>);
 }
 
 }  // namespace
@@ -310,16 +378,42 @@ int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1) {
 
 // One launch covers two stages (the register budget of the three-deep pipeline); layers of
 // three and four stages take a second launch for stages 3-4, which index the primary table.
+// fold: the folded streams of the same layer (then q and the tables are not read).
 int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
-                       hipStream_t stream, const float *pscale) {
+                       hipStream_t stream, const float *pscale, const glqh_e8_folded *fold) {
     em_plan p;
     if (!em_make_plan(m_pad, n_pad, B, n1, &p)) return glqh_fail("e8 mma: shape not eligible");
     if (nstages < 1 || nstages > 4) return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
-    if (nstages == 1) return em_launch_NS<1>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, 1, 0, part, stream, pscale);
-    if (em_launch_NS<2>(p, x, B, q, t1, t2, n1, n2, m_pad, n_pad, nstages, 0, part, stream, pscale)) return 1;
+    if (fold) {
+        const bool own2 = nstages >= 2 && fold->halves2 && fold->halves2 != fold->halves1;
+        const uint32_t *a1 = (const uint32_t *)fold->halves1, *a2 = own2 ? (const uint32_t *)fold->halves2 : a1;
+        const int64_t na1 = fold->n_halves1, na2 = own2 ? fold->n_halves2 : fold->n_halves1;
+        GLQH_REQUIRE(a1 && na1 >= 1 && na1 <= 2048 && na2 >= 1 && na2 <= 2048, "e8 folded: 1..2048 half codewords per table");
+        for (int s = 0; s < nstages; ++s)
+            GLQH_REQUIRE(fold->lo16[s] && fold->hi8[s], "e8 folded: stage %d has no folded stream", s + 1);
+        // LDS: stage-1 half codewords (two words each), stage 2's if they are a table of their own
+        const size_t rest = p.lds - (size_t)p.P * 4;
+        em_plan p12 = p, p34 = p;
+        p12.P = (int)(2 * ((na1 + 1) & ~(int64_t)1) + (own2 ? 2 * ((na2 + 1) & ~(int64_t)1) : 0));
+        p12.lds = (size_t)p12.P * 4 + rest;
+        p34.P = (int)(2 * ((na1 + 1) & ~(int64_t)1));
+        p34.lds = (size_t)p34.P * 4 + rest;
+        const void *const i12[4] = {fold->lo16[0], fold->lo16[nstages >= 2 ? 1 : 0], fold->lo16[0], fold->lo16[0]};
+        const em_signs s12 = {{fold->hi8[0], fold->hi8[nstages >= 2 ? 1 : 0], fold->hi8[0], fold->hi8[0]}};
+        if (nstages == 1) return em_launch_NS<1, true>(p12, x, B, i12, s12, a1, a1, na1, na1, m_pad, n_pad, 1, 0, part, stream, pscale);
+        if (em_launch_NS<2, true>(p12, x, B, i12, s12, a1, a2, na1, na2, m_pad, n_pad, nstages, 0, part, stream, pscale)) return 1;
+        if (nstages == 2) return 0;
+        const void *const i34[4] = {fold->lo16[2], fold->lo16[nstages == 4 ? 3 : 2], fold->lo16[2], fold->lo16[2]};
+        const em_signs s34 = {{fold->hi8[2], fold->hi8[nstages == 4 ? 3 : 2], fold->hi8[2], fold->hi8[2]}};
+        if (nstages == 3) return em_launch_NS<1, true>(p34, x, B, i34, s34, a1, a1, na1, na1, m_pad, n_pad, 3, 2, part, stream, pscale);
+        return em_launch_NS<2, true>(p34, x, B, i34, s34, a1, a1, na1, na1, m_pad, n_pad, 4, 2, part, stream, pscale);
+    }
+    const em_signs none = {{nullptr, nullptr, nullptr, nullptr}};
+    if (nstages == 1) return em_launch_NS<1, false>(p, x, B, q, none, t1, t2, n1, n2, m_pad, n_pad, 1, 0, part, stream, pscale);
+    if (em_launch_NS<2, false>(p, x, B, q, none, t1, t2, n1, n2, m_pad, n_pad, nstages, 0, part, stream, pscale)) return 1;
     if (nstages == 2) return 0;
     const void *const q34[4] = {q[2], q[3], q[2], q[3]};
-    if (nstages == 3) return em_launch_NS<1>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 3, 2, part, stream, pscale);
-    return em_launch_NS<2>(p, x, B, q34, t1, t1, n1, n1, m_pad, n_pad, 4, 2, part, stream, pscale);
+    if (nstages == 3) return em_launch_NS<1, false>(p, x, B, q34, none, t1, t1, n1, n1, m_pad, n_pad, 3, 2, part, stream, pscale);
+    return em_launch_NS<2, false>(p, x, B, q34, none, t1, t1, n1, n1, m_pad, n_pad, 4, 2, part, stream, pscale);
 }

@@ -643,6 +643,101 @@ def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, i
     return out.reshape(*input_ids.shape, embedding_dim)
 
 
+# Folded copies of the index streams for the small-batch kernel (include/glq_hip.h,
+# glqh_e8_fold_table): made on the first call that can use them and kept while the index tensor
+# lives, 1.5 times the bytes of the indices they copy.  GLQ_E8_FOLD=0 keeps the kernels on the
+# indices themselves.
+E8_FOLD = os.environ.get("GLQ_E8_FOLD", "1") != "0"
+_FOLD_TABLES = {}
+_FOLD_STREAMS = {}
+
+
+class _E8Folded(C.Structure):
+    _fields_ = [("lo16", C.c_void_p * 4), ("hi8", C.c_void_p * 4), ("halves1", C.c_void_p),
+                ("n_halves1", C.c_int64), ("halves2", C.c_void_p), ("n_halves2", C.c_int64)]
+
+
+def _fold_table(packed):
+    """(half codewords (n, 4) fp16, map) of a nibble-packed table tensor, once per tensor; (None, None)
+    for a table with more than 2048 distinct half codewords (no E8 shell table has: the full one has
+    1286), which the kernels then read through its indices."""
+    key = (packed.data_ptr(), packed._version, packed.shape[0], str(packed.device))
+    hit = _FOLD_TABLES.get(key)
+    if hit is not None and hit[0]() is packed:
+        return hit[1], hit[2]
+    lib = _lib.load()
+    halves = torch.empty((2048, 4), dtype=torch.float16, device=packed.device)
+    fmap = torch.empty(packed.shape[0], dtype=torch.int32, device=packed.device)
+    n = C.c_int64(0)
+    with torch.cuda.device(packed.device):
+        rc = lib.glqh_e8_fold_table(_p(packed), packed.shape[0], _p(halves), 2048, _p(fmap), C.addressof(n), _stream())
+    if rc != 0 and n.value <= 2048:
+        check(rc)
+    halves, fmap = (halves[:n.value].clone(), fmap) if rc == 0 else (None, None)
+    for k in [k for k, v in _FOLD_TABLES.items() if v[0]() is None]:
+        del _FOLD_TABLES[k]
+    _FOLD_TABLES[key] = (weakref.ref(packed), halves, fmap)
+    return halves, fmap
+
+
+def _fold_stream(q, packed):
+    """(16-bit words, bytes) of one stage's index tensor against its packed table."""
+    key = (q.data_ptr(), q._version, tuple(q.shape), str(q.device), packed.data_ptr())
+    hit = _FOLD_STREAMS.get(key)
+    if hit is not None and hit[0]() is q and hit[1]() is packed:
+        return hit[2], hit[3]
+    lib = _lib.load()
+    _, fmap = _fold_table(packed)
+    count = lib.glqh_e8_folded_count(q.shape[0], q.shape[1])
+    lo16 = torch.empty(count, dtype=torch.int16, device=q.device)
+    hi8 = torch.empty(count, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        check(lib.glqh_e8_fold_indices(_p(q), q.shape[0], q.shape[1], _p(fmap), packed.shape[0], _p(lo16), _p(hi8),
+                                       _stream()))
+    if len(_FOLD_STREAMS) % 64 == 63:                        # drop entries whose tensors are gone
+        for k in [k for k, v in _FOLD_STREAMS.items() if v[0]() is None or v[1]() is None]:
+            del _FOLD_STREAMS[k]
+    _FOLD_STREAMS[key] = (weakref.ref(q), weakref.ref(packed), lo16, hi8)
+    return lo16, hi8
+
+
+def _e8_folded(B, qidxs, t1, q2, t2, q3, q4):
+    """The folded streams of a layer as the C struct (and what must stay alive during the call), or
+    (None, None) when the call would not read them.  Not made under stream capture: the table fold
+    synchronizes; a layer first seen there runs on its indices."""
+    M, nblk = qidxs.shape
+    if not E8_FOLD or not qidxs.is_contiguous():
+        return None, None
+    lib = _lib.load()
+    if not lib.glqh_e8_fold_eligible(M, nblk * 8, B):
+        return None, None
+    stages = [(qidxs, t1)] + ([(q2, t2)] if q2 is not None else []) + [(q, t1) for q in (q3, q4) if q is not None]
+    capturing = torch.cuda.is_current_stream_capturing()
+    tables = [t1] + ([t2] if q2 is not None and t2 is not t1 else [])
+    if capturing and any(_FOLD_TABLES.get((t.data_ptr(), t._version, t.shape[0], str(t.device))) is None for t in tables):
+        return None, None
+    if any(_fold_table(t)[0] is None for t in tables):
+        return None, None
+    keep, f = [], _E8Folded()
+    for s, (q, t) in enumerate(stages):
+        if capturing:
+            key = (q.data_ptr(), q._version, tuple(q.shape), str(q.device), t.data_ptr())
+            hit = _FOLD_STREAMS.get(key)
+            if hit is None or hit[0]() is not q or hit[1]() is not t:
+                return None, None
+        lo16, hi8 = _fold_stream(q, t)
+        keep += [lo16, hi8]
+        f.lo16[s], f.hi8[s] = lo16.data_ptr(), hi8.data_ptr()
+    h1, _ = _fold_table(t1)
+    keep.append(h1)
+    f.halves1, f.n_halves1 = h1.data_ptr(), h1.shape[0]
+    if len(tables) == 2:
+        h2, _ = _fold_table(t2)
+        keep.append(h2)
+        f.halves2, f.n_halves2 = h2.data_ptr(), h2.shape[0]
+    return f, keep
+
+
 def _primary_table(codebook):
     """Packed first-stage table: the kernels index it with the full 16-bit pattern and keep
     its low-norm prefix in LDS, so it must be the whole 65536-entry table (the reference's
@@ -697,12 +792,14 @@ def _e8_matmul_tables(x, qidxs, t1, q2, t2, n2, q3, q4, wscale, inv_rs, inv_rs2,
         return torch.mm(x, W.t(), out_dtype=torch.float32).mul_(float(wscale))
     out = torch.empty((B, M), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
+        folded, keep = _e8_folded(B, qidxs, t1, q2, t2, q3, q4)
         nb = lib.glqh_e8_matmul_workspace_bytes(M, nblk * 8, B)
         ws = _ws(nb, x.device)
-        check(lib.glqh_e8_dequant_matmul(
+        check(lib.glqh_e8_dequant_matmul_folded(
             _p(x), B, _p(qidxs), _p(q2), _p(q3), _p(q4), _p(t1), _p(t2), n2, float(wscale),
             float(inv_rs), float(inv_rs2), float(inv_rs3), M, nblk * 8,
-            _p(out), _p(ws), ws.numel(), _stream()))
+            _p(out), _p(ws), ws.numel(), _stream(), C.addressof(folded) if folded is not None else None))
+    del keep
     return out
 
 
@@ -787,14 +884,17 @@ def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_p
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
         return _dense_matmul_output(x_rht, W, wscale, su, y, out_features, m_pad, blocks_m, bm_meta)
     with torch.cuda.device(x.device):
+        folded, keep = _e8_folded(B, qidxs, t1, q2, t2, q3, q4)
         nb = lib.glqh_fused_linear_e8_workspace_bytes(B, int(n_pad), int(m_pad))
         ws = _ws(nb, x.device)
-        check(lib.glqh_fused_linear_e8(
+        check(lib.glqh_fused_linear_e8_folded(
             _p(x), _DT[x.dtype], x.shape[1], B, _p(sv), _p(su), _p(qidxs), _p(q2), _p(q3), _p(q4),
             _p(t1), _p(t2), n2, float(wscale), float(inv_rs), float(inv_rs2), float(inv_rs3),
             bn, nbn, bm, nbm, _meta_ptr(bn_meta) if nbn > 1 else None,
             _meta_ptr(bm_meta) if nbm > 1 else None, int(in_features), int(out_features), int(n_pad),
-            int(m_pad), _p(y), _DT[y.dtype], y.shape[1], _p(ws), ws.numel(), _stream()))
+            int(m_pad), _p(y), _DT[y.dtype], y.shape[1], _p(ws), ws.numel(), _stream(),
+            C.addressof(folded) if folded is not None else None))
+    del keep
     return y
 
 

@@ -267,6 +267,48 @@ int glqh_e8_pack_table(const void *codebook_f16, int64_t n_entries, uint32_t *pa
 int glqh_e8_repack_table(const uint32_t *codebook_packed, int64_t n_entries, uint32_t *packed_out,
                          int32_t *bad_dev, void *stream);
 
+/* ---- folded form of the E8 streams (no counterpart in the reference) ---------------------
+ * The 65536 codewords of the shell table are built from only 1286 distinct half codewords
+ * (columns 0..3 or 4..7, signs included).  A table of those as finished fp16 values (8 bytes
+ * each) fits LDS whole, so the small-batch kernel (1..16 tokens) looks every index up without
+ * leaving the CU and without expanding anything -- at the price of a second, on-device copy
+ * of the index streams: per index two 11-bit half numbers, stored as a 16-bit word plus a
+ * byte (3 bytes instead of 2).  Made once per table and per layer at load time; the original
+ * indices stay in use for every other route (many tokens, small or ragged layers, decompress). */
+typedef struct {
+    const uint16_t *lo16[4];     /* per stage, tile order: first half number | (second & 31) << 11 */
+    const uint8_t *hi8[4];       /* per stage, tile order: second half number >> 5 */
+    const void *halves1;         /* half-codeword table of stage 1 (and of stages 3, 4): 4 fp16 per entry */
+    int64_t n_halves1;
+    const void *halves2;         /* the same for stage 2 when it has a table of its own, else NULL */
+    int64_t n_halves2;
+} glqh_e8_folded;
+
+/* table: n_entries nibble-packed words (glqh_e8_pack_table / glqh_e8_repack_table), device.
+ * halves_out (device, room for `capacity` entries of 8 bytes; the kernels take up to 2048): the
+ * distinct half codewords in order of first appearance (first half of an entry before its
+ * second), as 4 fp16 values; map_out (device, n_entries words): entry k = number of its first
+ * half | number of its second half << 16.  *n_halves_out (host) = the count; fails if it
+ * exceeds `capacity`.  Copies the table to the host and the results back: synchronizes the
+ * stream, not capturable. */
+int glqh_e8_fold_table(const uint32_t *table, int64_t n_entries, void *halves_out, int64_t capacity,
+                       uint32_t *map_out, int64_t *n_halves_out, void *stream);
+
+/* 1 when a product of this shape and token count reads the folded streams (the LDS-table
+ * kernel serves it), 0 when they would go unused. */
+int glqh_e8_fold_eligible(int64_t m_pad, int64_t n_pad, int64_t B);
+
+/* Entries of a folded stream of a (rows, cols) index matrix: rows padded to 16, cols to 32. */
+int64_t glqh_e8_folded_count(int64_t rows, int64_t cols);
+
+/* q: (rows, cols) int16 indices read as unsigned (clamped to n_entries - 1) -> lo16_out and
+ * hi8_out, glqh_e8_folded_count(rows, cols) entries each, through `map` of glqh_e8_fold_table,
+ * in the tile order the kernel reads (16 rows x 32 indices per tile, the 8 consecutive indices
+ * of row i, group g at entry 8 * (16 g + i) of the tile; padding holds half number 0).
+ * Asynchronous. */
+int glqh_e8_fold_indices(const void *q, int64_t rows, int64_t cols, const uint32_t *map, int64_t n_entries,
+                         uint16_t *lo16_out, uint8_t *hi8_out, void *stream);
+
 size_t glqh_e8_matmul_workspace_bytes(int64_t m_pad, int64_t n_pad, int64_t B);
 
 /* out[b, :] (fp32, stride m_pad) = wscale * (cb[q1] + inv_rs*cb2[q2] + inv_rs2*cb3[q3]
@@ -282,6 +324,18 @@ int glqh_e8_dequant_matmul(const void *x_f16, int64_t B,
                            double wscale, double inv_rs, double inv_rs2, double inv_rs3,
                            int64_t m_pad, int64_t n_pad,
                            float *out, void *ws, size_t ws_bytes, void *stream);
+
+/* The same with the layer's folded streams beside the indices: up to 16 tokens on shapes
+ * the LDS-table kernel serves, the product reads `folded` instead of q1..q4 / the tables
+ * (same workspace, same K slots, same order of summation); every other case ignores it.
+ * folded == NULL is glqh_e8_dequant_matmul. */
+int glqh_e8_dequant_matmul_folded(const void *x_f16, int64_t B,
+                                  const void *q1, const void *q2, const void *q3, const void *q4,
+                                  const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                  double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                                  int64_t m_pad, int64_t n_pad,
+                                  float *out, void *ws, size_t ws_bytes, void *stream,
+                                  const glqh_e8_folded *folded);
 
 /* Dense fp16 (m_pad, n_pad) RHT-domain weight before Wscale: cb[q1] + inv_rs*cb2[q2] + ...
  * combined in fp32 and rounded once.  First half of the many-token path of
@@ -324,6 +378,20 @@ int glqh_fused_linear_e8(const void *x, int x_dtype, int64_t x_stride, int64_t B
                          int64_t in_features, int64_t out_features, int64_t n_pad, int64_t m_pad,
                          void *y, int y_dtype, int64_t y_stride,
                          void *ws, size_t ws_bytes, void *stream);
+
+/* glqh_fused_linear_e8 with the layer's folded streams (see glqh_e8_dequant_matmul_folded). */
+int glqh_fused_linear_e8_folded(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                const void *sv_f16, const void *su_f16,
+                                const void *q1, const void *q2, const void *q3, const void *q4,
+                                const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                double wscale, double inv_rs, double inv_rs2, double inv_rs3,
+                                const int64_t *blocks_n, int64_t n_blocks_n,
+                                const int64_t *blocks_m, int64_t n_blocks_m,
+                                const glqh_block_meta *bn_meta_dev, const glqh_block_meta *bm_meta_dev,
+                                int64_t in_features, int64_t out_features, int64_t n_pad, int64_t m_pad,
+                                void *y, int y_dtype, int64_t y_stride,
+                                void *ws, size_t ws_bytes, void *stream,
+                                const glqh_e8_folded *folded);
 
 /* ---- encode side --------------------------------------------------------------- */
 

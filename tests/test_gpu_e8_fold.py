@@ -1,0 +1,166 @@
+"""Folded form of the E8 index streams (glqh_e8_fold_table / glqh_e8_fold_indices and the
+small-batch kernel that reads it): the fold is checked against a numpy restatement of its
+definition on the real table, and a product on the folded streams must give the same bits as the
+product on the indices themselves (same K slots, same order of summation, same decoded values);
+against the oracle the usual bound holds (relative Frobenius error <= 1e-2)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import DEV, e8_table_f16, rel, say, t
+from oracle import glq_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ext():
+    from glq_amd import ext as e
+    return e
+
+
+def _unfold(halves, fmap):
+    """(n, 8) values from the half-codeword table and the map (first | second << 16)"""
+    return np.concatenate([halves[fmap & 0xFFFF], halves[fmap >> 16]], axis=1).astype(np.float32)
+
+
+def test_fold_of_the_shell_table(ext):
+    say("e8 fold table")
+    packed = ext._packed_table(e8_table_f16())
+    halves, fmap = ext._fold_table(packed)
+    hv, fm = halves.cpu().numpy(), fmap.cpu().numpy().view(np.uint32)
+    table = O.e8_table()
+    # the 65536 codewords are built from 1286 distinct halves (a property of the table itself: the
+    # same count from the oracle's fp32 table)
+    n_half = len(np.unique(np.concatenate([table[:, :4], table[:, 4:]]), axis=0))
+    assert n_half == 1286 and hv.shape == (n_half, 4)
+    assert ((fm & 0xFFFF) < n_half).all() and ((fm >> 16) < n_half).all()
+    assert np.array_equal(_unfold(hv, fm), table)
+    # numbered in order of first appearance, the first half of an entry before its second
+    order = np.stack([fm & 0xFFFF, fm >> 16], axis=1).reshape(-1)
+    _, first = np.unique(order, return_index=True)
+    assert np.array_equal(order[np.sort(first)], np.arange(n_half))
+
+
+def test_fold_of_an_index_stream_and_a_short_table(ext):
+    say("e8 fold indices")
+    small = e8_table_f16()[:256].contiguous()                 # the 3 bpw recipe's secondary table
+    packed = ext._packed_table(small)
+    rng = np.random.default_rng(0)
+    q = rng.integers(0, 65536, size=(64, 40)).astype(np.uint16)          # indices past the table clamp to its last row
+    qd = t(q.view(np.int16))
+    lo16, hi8 = ext._fold_stream(qd, packed)
+    hv, fm = ext._fold_table(packed)
+    hv, fm = hv.cpu().numpy(), fm.cpu().numpy().view(np.uint32)
+    assert np.array_equal(_unfold(hv, fm), O.e8_table()[:256])
+    # tile order: 16 rows x 32 indices per tile, entry 8 * (16 g + i) + e = row i, index 8 g + e of the tile;
+    # 40 columns are padded to 64 with half number 0
+    want = np.zeros((64, 64), np.uint32)
+    want[:, :40] = fm[np.minimum(q, 255)]
+    tiles = want.reshape(4, 16, 2, 4, 8).transpose(0, 2, 3, 1, 4).reshape(-1)       # [row tile][col tile][g][i][e]
+    first, second = tiles & 0xFFFF, tiles >> 16
+    assert lo16.numel() == 4 * 2 * 512 == ext._lib.load().glqh_e8_folded_count(64, 40)
+    assert np.array_equal(lo16.cpu().numpy().view(np.uint16), (first | (second & 31) << 11).astype(np.uint16))
+    assert np.array_equal(hi8.cpu().numpy(), (second >> 5).astype(np.uint8))
+    # the same tensors again come from the cache; a changed index tensor is folded again
+    assert ext._fold_stream(qd, packed)[0] is lo16
+    qd[0, 0] = 5
+    lo2, _ = ext._fold_stream(qd, packed)
+    assert lo2 is not lo16 and int(lo2.view(torch.int16)[0]) & 0x7FF == int(fm[5] & 0xFFFF)
+
+
+def _indices(m, n, stages, seed):
+    rng = np.random.default_rng(seed)
+    lo = rng.integers(0, 30000, size=(stages, m, n // 8))
+    hi = rng.integers(0, 65536, size=(stages, m, n // 8))
+    return np.where(rng.random((stages, m, n // 8)) < 0.6, lo, hi).astype(np.uint16).view(np.int16)
+
+
+@pytest.mark.parametrize("m,n,B", [(4096, 2048, 1), (2048, 4096, 3), (1024, 8192, 16), (4096, 14336, 1)])
+@pytest.mark.parametrize("stages", [1, 2, 3, 4])
+def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stages):
+    say("e8 folded matmul", m, n, B, stages)
+    lib = ext._lib.load()
+    assert lib.glqh_e8_fold_eligible(m, n, B) == 1
+    q = [t(a) for a in _indices(m, n, stages, m + stages)]
+    cb = e8_table_f16()
+    cb2 = cb[:256].contiguous() if stages == 2 else cb        # two stages: the short secondary table
+    if stages == 2:
+        q[1] = t((_indices(m, n, 1, 7)[0].view(np.uint16) & 255).view(np.int16))
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).half().to(DEV)
+    args = dict(qidxs2=q[1] if stages > 1 else None, codebook2=cb2, inv_resid_scale=1 / 3.0 if stages > 1 else 0.0,
+                qidxs3=q[2] if stages > 2 else None, inv_resid_scale2=1 / 9.0 if stages > 2 else 0.0,
+                qidxs4=q[3] if stages > 3 else None, inv_resid_scale3=1 / 27.0 if stages > 3 else 0.0)
+    ext.E8_FOLD = True
+    try:
+        y_fold = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
+        assert any(k[0] == q[0].data_ptr() for k in ext._FOLD_STREAMS), "the folded streams were not made"
+        ext.E8_FOLD = False
+        y_idx = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
+    finally:
+        ext.E8_FOLD = True
+    assert torch.equal(y_fold, y_idx)
+    if m * n <= 1 << 23:                                       # and both are the oracle's product
+        tabs = [O.e8_table(), O.e8_table()[:256] if stages == 2 else O.e8_table(), O.e8_table(), O.e8_table()]
+        W = sum(tabs[s][q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)
+                for s in range(stages)).astype(np.float32) * np.float32(0.02)
+        assert rel(y_fold, x.float().cpu().numpy() @ W.T) < TOL
+
+
+def test_fused_linear_on_folded_streams_and_under_capture(ext):
+    say("e8 folded fused linear + graph")
+    from glq_amd import hadamard as H
+    m, n = 4096, 3072                                          # block-diagonal input side
+    q = [t(a) for a in _indices(m, n, 2, 3)]
+    su, sv = O.rht_signs(m, n, 42)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    cb = e8_table_f16()
+    args = (t(sv.astype(np.float16)), t(su.astype(np.float16)), q[0], cb, 0.02, n, m, n, m, torch.tensor(bn),
+            torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), q[1], cb, 1 / 3.0)
+    x = torch.randn(2, n, generator=torch.Generator().manual_seed(5)).bfloat16().to(DEV)
+    # first seen under capture: the fold (which synchronizes) is not made there, the call runs on the indices
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        warm = ext.glq_fused_linear_block_diag_cuda(x, *args[:2], q[0].clone(), *args[3:], out_dtype=torch.bfloat16)
+    torch.cuda.current_stream().wait_stream(s)
+    n_before = len(ext._FOLD_STREAMS)
+    q_new = [a.clone() for a in q]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        y_cap = ext.glq_fused_linear_block_diag_cuda(x, *args[:2], q_new[0], *args[3:13], q_new[1], *args[14:],
+                                                     out_dtype=torch.bfloat16)
+    assert len(ext._FOLD_STREAMS) == n_before
+    g.replay()
+    torch.cuda.synchronize()
+    y_fold = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
+    assert any(k[0] == q[0].data_ptr() for k in ext._FOLD_STREAMS)
+    assert torch.equal(y_cap, y_fold) and torch.equal(warm, y_fold)
+    # captured after the streams exist: the graph reads them
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        y2 = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
+    for _ in range(2):
+        g2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y2, y_fold)
+    art = {"Qidxs": q[0].cpu().numpy(), "Qidxs2": q[1].cpu().numpy(), "inv_resid_scale": np.float32(1 / 3.0),
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
+           "blocks_m": bm, "blocks_n": bn}
+    assert rel(y_fold, O.e8_linear_forward(x.float().cpu().numpy(), art, n, m)) < TOL
+
+
+def test_c_abi_refusals(ext):
+    say("e8 fold refusals")
+    lib = ext._lib.load()
+    packed = ext._packed_table(e8_table_f16())
+    fmap = torch.empty(65536, dtype=torch.int32, device=DEV)
+    n = C.c_int64(0)
+    small = torch.empty((16, 4), dtype=torch.float16, device=DEV)
+    rc = lib.glqh_e8_fold_table(packed.data_ptr(), 65536, small.data_ptr(), 16, fmap.data_ptr(), C.addressof(n), None)
+    assert rc != 0 and b"room for 16" in lib.glqh_last_error() and n.value == 1286
+    assert lib.glqh_e8_fold_eligible(960, 960, 1) == 0       # a small layer: the gather kernel serves it
+    assert lib.glqh_e8_fold_eligible(4096, 14336, 17) == 0   # the tile kernel's range

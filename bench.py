@@ -224,7 +224,9 @@ def extras(torch, ext, dev):
         out["large_layer_error"] = f"{type(e).__name__}: {e}"
     try:
         # config 3: E8 two-stage 4 bpw GEMV, 4096 x 14336, indices from quantizing N(0,1)
-        # vectors with the GPU encoder (the index distribution decides the LDS hit rate)
+        # vectors with the GPU encoder.  GB/s = algorithmic bytes (2 bytes per 8 weights and stage) per
+        # second; the kernel itself streams the folded copy of the indices, 3 bytes per index
+        # (made on the first call, outside the timed region; GLQ_E8_FOLD=0 for the indices themselves)
         from glq_amd.checkpoint import load_shell_table
         cb = load_shell_table(None).to(dev)
         m, n = 4096, 14336

@@ -289,7 +289,9 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
     const int64_t nblk = n_pad / 8;
     if (B < 1 || B > 16 || nblk < 8 || (nblk & 7) || n1 < 4096) return 0;
     // the table load would dominate (2048 x 2048, two stages, whole linear: 15.7 us here against
-    // 13.3 us with L2 gathers at one token, 16.5 against 16.6 at four; 3072 x 3072: 18.6 against 21.3)
+    // 13.3 us with L2 gathers at one token, 16.5 against 16.6 at four; 3072 x 3072: 18.6 against 21.3;
+    // on folded streams, whose table is small, the two kernels tie below these sizes: 960 x 960 11.9
+    // against 10.1 us, 2048 x 2048 12.8 against 12.4, 1024 x 4096 13.2 against 13.4)
     if (m_pad * n_pad < (B == 1 ? (int64_t)6 << 20 : (int64_t)1 << 22)) return 0;
     p->TP = B == 1 ? 1 : B <= 4 ? 4 : 16;
     p->WK = p->TP == 16 ? 1 : 4;

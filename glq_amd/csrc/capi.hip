@@ -1073,11 +1073,11 @@ extern "C" int glqh_e8_fold_table(const uint32_t *table, int64_t n_entries, void
     return 0;
 }
 
-int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1);
+int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, int fold);
 
 extern "C" int glqh_e8_fold_eligible(int64_t m_pad, int64_t n_pad, int64_t B) {
     if (glqh_init() != 0 || m_pad < 1 || n_pad < 8 || (n_pad & 7) || B < 1) return 0;
-    return glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536) > 0 ? 1 : 0;
+    return glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536, 1) > 0 ? 1 : 0;
 }
 
 extern "C" int64_t glqh_e8_folded_count(int64_t rows, int64_t cols) {
@@ -1143,7 +1143,9 @@ static size_t e8_part_bytes(int64_t m_pad, int64_t n_pad, int64_t B) {
                                                                  // stages get the most K slots
     if (tks > 0)                                                 // + the repacked activations
         return align256((size_t)tks * B * m_pad * sizeof(float)) + align256(glqh_e8_tile_xb_bytes(n_pad, B));
-    int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B, 0);
+    const int ksf = glqh_e8_pick_ksplit(m_pad, n_pad, B, 1);       // on folded streams
+    if (ksf > ks) ks = ksf;
     return align256((size_t)ks * 4 * B * m_pad * sizeof(float));
 }
 
@@ -1188,7 +1190,11 @@ extern "C" int glqh_e8_dequant_matmul_folded(const void *x_f16, int64_t B, const
             return 1;
         return glqh_launch_reduce_splits(part, tks, B * m_pad, B, m_pad, (float)wscale, out, m_pad, 0, st);
     }
-    const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    // folded streams with K inside the workgroups: the kernel writes the finished sums itself
+    if (folded && glqh_e8_mma_direct_ok(m_pad, n_pad, B, sg.n))
+        return glqh_launch_e8_partial(x_f16, B, sg.q, sg.n, table1, table2 ? table2 : table1, table2 ? n_entries2 : 65536,
+                                      m_pad, n_pad, 1, out, st, sg.scale, folded, 1);
+    const int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B, folded != nullptr);
     const size_t need = (size_t)ks * sg.n * B * m_pad * sizeof(float);
     GLQH_REQUIRE(ws && ws_bytes >= need, "e8 matmul: workspace of %zu bytes needed, got %zu", need, ws_bytes);
     // every stage's partial sums are written already multiplied by that stage's scale: one
@@ -1273,7 +1279,7 @@ extern "C" int glqh_fused_linear_e8_folded(const void *x, int x_dtype, int64_t x
     GLQH_REQUIRE(in_features <= n_pad && out_features <= m_pad, "fused e8 linear: features exceed padded dims");
     const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
     const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n);
-    const int ks = tks > 0 ? tks : glqh_e8_pick_ksplit(m_pad, n_pad, B);
+    const int ks = tks > 0 ? tks : glqh_e8_pick_ksplit(m_pad, n_pad, B, folded != nullptr);
     const size_t tile_part = align256((size_t)ks * B * m_pad * sizeof(float));
     const size_t need = tks > 0 ? xb + tile_part + glqh_e8_tile_xb_bytes(n_pad, B)
                                 : xb + (size_t)ks * sg.n * B * m_pad * sizeof(float);

@@ -150,7 +150,8 @@ int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, in
 
 // E8 gather matmul into per-stage split-K partials:
 // part[((slot * nstages + stage) * B + tok) * m_pad + row]
-int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B);
+int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int fold = 0);
+int glqh_e8_mma_direct_ok(int64_t m_pad, int64_t n_pad, int64_t B, int nstages);
 int glqh_launch_e8_pack_table(const void *cb, int64_t n_entries, uint32_t *out, int32_t *bad,
                               hipStream_t stream);
 int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t *out, int32_t *bad,
@@ -162,7 +163,7 @@ struct glqh_e8_pscale {
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream,
-                           const float *pscale = nullptr, const glqh_e8_folded *fold = nullptr);
+                           const float *pscale = nullptr, const glqh_e8_folded *fold = nullptr, int direct = 0);
 int glqh_launch_e8_fold_indices(const void *q, int64_t rows, int64_t cols, const uint32_t *map, int64_t n_entries,
                                 uint16_t *lo16_out, uint8_t *hi8_out, hipStream_t stream);
 int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,

@@ -281,10 +281,10 @@ int launch_e8_NS(const void *x, int64_t B, const void *const q[4], const uint32_
 }  // namespace
 
 int glqh_e8_mma_init(void);
-int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1);
+int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, int fold);
 int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
-                       hipStream_t stream, const float *pscale, const glqh_e8_folded *fold);
+                       hipStream_t stream, const float *pscale, const glqh_e8_folded *fold, int direct);
 
 int glqh_e8_init(void) {
     if (glqh_check_hip(hipFuncSetAttribute((const void *)e8_decompress_lds_kernel,
@@ -295,9 +295,9 @@ int glqh_e8_init(void) {
 }
 
 // K-split of the kernel that will serve the call.
-int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B) {
+int glqh_e8_pick_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int fold) {
     // large layers at up to 16 tokens go to the LDS-table kernel, which has its own slots
-    const int mma_ks = glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536);
+    const int mma_ks = glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536, fold);
     if (mma_ks > 0) return mma_ks;
     const int64_t wgs = (m_pad + E8_ROWS_PER_WG - 1) / E8_ROWS_PER_WG;
     const int64_t target = (int64_t)glqh_device_cus() * 4;
@@ -367,14 +367,15 @@ int glqh_launch_e8_repack_table(const uint32_t *in, int64_t n_entries, uint32_t 
 int glqh_launch_e8_partial(const void *x, int64_t B, const void *const q[4], int nstages,
                            const uint32_t *t1, const uint32_t *t2, int64_t n2, int64_t m_pad,
                            int64_t n_pad, int ksplit, float *part, hipStream_t stream, const float *pscale,
-                           const glqh_e8_folded *fold) {
+                           const glqh_e8_folded *fold, int direct) {
     glqh_range range("dequant_matmul");
     glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
     if (pscale)
         for (int i = 0; i < 4; ++i) ps.v[i] = pscale[i];
     // the folded streams serve the LDS-table kernel only; every other route reads the indices themselves
-    if (glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536) > 0)
-        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream, pscale, fold);
+    if (glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536, fold != nullptr) > 0)
+        return glqh_launch_e8_mma(x, B, q, nstages, t1, 65536, t2, n2, m_pad, n_pad, part, stream, pscale, fold, direct);
+    GLQH_REQUIRE(!direct, "e8 matmul: finished sums are an option of the LDS-table kernel");
     switch (nstages) {
     case 1: return launch_e8_NS<1>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);
     case 2: return launch_e8_NS<2>(x, B, q, t1, t2, n2, m_pad, n_pad, ksplit, part, stream, ps);

@@ -65,7 +65,9 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
               const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n1, uint32_t n2,
               int t2_is_t1, const f16 *__restrict__ x, int B, int m_pad, int n_pad, int P, int slot_blks,
               int xs_slots, int ksplit, int ns_total, int s_off, float *__restrict__ part,
-              glqh_e8_pscale ps) {                              // ps.v[s]: factor of stage s_off + s
+              glqh_e8_pscale ps, int direct) {                  // ps.v[s]: factor of stage s_off + s
+                                                                // direct (one K slot, WK > 1): part is the (B, m_pad)
+                                                                // result, the scaled stage sums added in stage order
     constexpr int WR = EM_WAVES / WK;
     constexpr int ROWS = 16 * WR;
     extern __shared__ u32x4 lds[];
@@ -271,7 +273,20 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                 float v = red[e];
 #pragma unroll
                 for (int w = 1; w < WK; ++w) v += red[w * NS * TP * ROWS + e];
-                part[(((int64_t)slot * ns_total + s_off + s) * B + tl) * m_pad + orow] = ps.v[s] * v;
+                if (!direct) part[(((int64_t)slot * ns_total + s_off + s) * B + tl) * m_pad + orow] = ps.v[s] * v;
+                else red[e] = ps.v[s] * v;                     // own element: nobody else reads or writes it
+            }
+            if (direct) {                                      // uniform
+                __syncthreads();
+                for (int e = threadIdx.x; e < TP * ROWS; e += EM_THREADS) {
+                    const int rl = e % ROWS, tl = e / ROWS;
+                    const int orow = rb * ROWS + rl;
+                    if (tl >= B || orow >= m_pad) continue;
+                    float v = red[e];
+#pragma unroll
+                    for (int s = 1; s < NS; ++s) v += red[s * TP * ROWS + e];
+                    part[(int64_t)tl * m_pad + orow] = v;
+                }
             }
         }
     }
@@ -285,7 +300,7 @@ struct em_plan {
 constexpr size_t EM_LDS_TOTAL = 160 * 1024;
 
 // 0 when the shape is better served by the plain gather kernel
-int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p) {
+int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, bool fold, em_plan *p) {
     const int64_t nblk = n_pad / 8;
     if (B < 1 || B > 16 || nblk < 8 || (nblk & 7) || n1 < 4096) return 0;
     // the table load would dominate (2048 x 2048, two stages, whole linear: 15.7 us here against
@@ -295,13 +310,18 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
     if (m_pad * n_pad < (B == 1 ? (int64_t)6 << 20 : (int64_t)1 << 22)) return 0;
     p->TP = B == 1 ? 1 : B <= 4 ? 4 : 16;
     p->WK = p->TP == 16 ? 1 : 4;
+    // One token on folded streams (no table to speak of in LDS, room for the whole row of activations):
+    // all sixteen waves of a workgroup split K among themselves when 16-row tiles fill the chip exactly once,
+    // so no K slot leaves the workgroup and the sums can be written finished (4096 x 14336, whole unfused
+    // call: 19.1 -> 17.7 us with the reduction launch kept; 14336 x 4096, 896 such tiles: 17.6 -> 21.7, not taken)
+    if (fold && p->TP == 1 && (m_pad + 15) / 16 <= glqh_device_cus() && nblk >= 16 * EM_STEP_BLKS) p->WK = 16;
     const int rows = 16 * (EM_WAVES / p->WK);
     const int64_t RB = (m_pad + rows - 1) / rows;
     const int unit = p->WK * EM_STEP_BLKS;                      // blocks per workgroup step
     const int64_t nunits = (nblk + unit - 1) / unit;
     // activations: at most 32 KB of LDS; slots as long as that allows, so that a workgroup has one
     // tile (and one table fill per tile) where the shape permits
-    const int slot_cap_blks = p->TP == 16 ? 128 : 512;
+    const int slot_cap_blks = p->TP == 16 ? 128 : p->WK == 16 ? 2048 : 512;
     const int cus = glqh_device_cus();
     int64_t ks = RB >= cus ? 1 : cus / RB;                      // one tile per workgroup where possible
     if (ks > nunits) ks = nunits;
@@ -329,12 +349,12 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, em_plan *p
 template <int NS, int TP, int WK, bool FOLD>
 int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4], const em_signs &sp,
               const uint32_t *t1, const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad,
-              int ns_total, int s_off, float *part, hipStream_t stream, glqh_e8_pscale ps) {
+              int ns_total, int s_off, float *part, hipStream_t stream, glqh_e8_pscale ps, int direct = 0) {
     hipLaunchKernelGGL((e8_mma_kernel<NS, TP, WK, FOLD>), dim3((unsigned)p.grid), dim3(EM_THREADS), p.lds, stream,
                        (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
                        (const uint16_t *)q[3], sp, t1, t2, (uint32_t)n1, (uint32_t)n2, (int)(t1 == t2 && n1 == n2),
                        (const f16 *)x, (int)B, (int)m_pad, (int)n_pad, p.P, p.slot_blks, p.xs_slots, p.ksplit,
-                       ns_total, s_off, part, ps);
+                       ns_total, s_off, part, ps, direct);
     GLQH_LAUNCH_CHECK("e8 mma launch");
     return 0;
 }
@@ -342,12 +362,13 @@ int em_launch(const em_plan &p, const void *x, int64_t B, const void *const q[4]
 template <int NS, bool FOLD>
 int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q[4], const em_signs &sp,
                  const uint32_t *t1, const uint32_t *t2, int64_t n1, int64_t n2, int64_t m_pad, int64_t n_pad,
-                 int ns_total, int s_off, float *part, hipStream_t stream, const float *pscale) {
+                 int ns_total, int s_off, float *part, hipStream_t stream, const float *pscale, int direct = 0) {
     glqh_e8_pscale ps = {{1.0f, 1.0f, 1.0f, 1.0f}};
     if (pscale)
         for (int i = 0; i + s_off < 4; ++i) ps.v[i] = pscale[s_off + i];
 #define GLQH_EM(TP, WK) em_launch<NS, TP, WK, FOLD>(p, x, B, q, sp, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, \
-                                                    part, stream, ps)
+                                                    part, stream, ps, direct)
+    if (p.TP == 1 && p.WK == 16) return GLQH_EM(1, 16);
     if (p.TP == 1) return GLQH_EM(1, 4);
     if (p.TP == 4) return GLQH_EM(4, 4);
     return GLQH_EM(16, 1);
@@ -365,7 +386,8 @@ template <int NS>
 int em_init_NS() {
     return em_set_lds(e8_mma_kernel<NS, 1, 4, false>) || em_set_lds(e8_mma_kernel<NS, 4, 4, false>) ||
            em_set_lds(e8_mma_kernel<NS, 16, 1, false>) || em_set_lds(e8_mma_kernel<NS, 1, 4, true>) ||
-           em_set_lds(e8_mma_kernel<NS, 4, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 1, true>);
+           em_set_lds(e8_mma_kernel<NS, 4, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 1, true>) ||
+           em_set_lds(e8_mma_kernel<NS, 1, 16, true>) || em_set_lds(e8_mma_kernel<NS, 1, 16, false>);
 }
 
 }  // namespace
@@ -373,9 +395,9 @@ int em_init_NS() {
 int glqh_e8_mma_init(void) { return em_init_NS<1>() || em_init_NS<2>(); }
 
 // ksplit of the LDS-table kernel for this call, or 0 when the shape is not eligible
-int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1) {
+int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, int fold) {
     em_plan p;
-    return em_make_plan(m_pad, n_pad, B, n1, &p) ? p.ksplit : 0;
+    return em_make_plan(m_pad, n_pad, B, n1, fold != 0, &p) ? p.ksplit : 0;
 }
 
 // One launch covers two stages (the register budget of the three-deep pipeline); layers of
@@ -383,9 +405,9 @@ int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1) {
 // fold: the folded streams of the same layer (then q and the tables are not read).
 int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nstages, const uint32_t *t1,
                        int64_t n1, const uint32_t *t2, int64_t n2, int64_t m_pad, int64_t n_pad, float *part,
-                       hipStream_t stream, const float *pscale, const glqh_e8_folded *fold) {
+                       hipStream_t stream, const float *pscale, const glqh_e8_folded *fold, int direct) {
     em_plan p;
-    if (!em_make_plan(m_pad, n_pad, B, n1, &p)) return glqh_fail("e8 mma: shape not eligible");
+    if (!em_make_plan(m_pad, n_pad, B, n1, fold != nullptr, &p)) return glqh_fail("e8 mma: shape not eligible");
     if (nstages < 1 || nstages > 4) return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
     if (fold) {
         const bool own2 = nstages >= 2 && fold->halves2 && fold->halves2 != fold->halves1;
@@ -403,14 +425,18 @@ int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nst
         p34.lds = (size_t)p34.P * 4 + rest;
         const void *const i12[4] = {fold->lo16[0], fold->lo16[nstages >= 2 ? 1 : 0], fold->lo16[0], fold->lo16[0]};
         const em_signs s12 = {{fold->hi8[0], fold->hi8[nstages >= 2 ? 1 : 0], fold->hi8[0], fold->hi8[0]}};
-        if (nstages == 1) return em_launch_NS<1, true>(p12, x, B, i12, s12, a1, a1, na1, na1, m_pad, n_pad, 1, 0, part, stream, pscale);
-        if (em_launch_NS<2, true>(p12, x, B, i12, s12, a1, a2, na1, na2, m_pad, n_pad, nstages, 0, part, stream, pscale)) return 1;
+        GLQH_REQUIRE(!direct || (p.WK > 1 && p.ksplit == 1 && nstages <= 2), "e8 folded: finished sums need one K slot");
+        if (nstages == 1)
+            return em_launch_NS<1, true>(p12, x, B, i12, s12, a1, a1, na1, na1, m_pad, n_pad, 1, 0, part, stream, pscale, direct);
+        if (em_launch_NS<2, true>(p12, x, B, i12, s12, a1, a2, na1, na2, m_pad, n_pad, nstages, 0, part, stream, pscale, direct))
+            return 1;
         if (nstages == 2) return 0;
         const void *const i34[4] = {fold->lo16[2], fold->lo16[nstages == 4 ? 3 : 2], fold->lo16[2], fold->lo16[2]};
         const em_signs s34 = {{fold->hi8[2], fold->hi8[nstages == 4 ? 3 : 2], fold->hi8[2], fold->hi8[2]}};
         if (nstages == 3) return em_launch_NS<1, true>(p34, x, B, i34, s34, a1, a1, na1, na1, m_pad, n_pad, 3, 2, part, stream, pscale);
         return em_launch_NS<2, true>(p34, x, B, i34, s34, a1, a1, na1, na1, m_pad, n_pad, 4, 2, part, stream, pscale);
     }
+    GLQH_REQUIRE(!direct, "e8 mma: finished sums are an option of the folded form");
     const em_signs none = {{nullptr, nullptr, nullptr, nullptr}};
     if (nstages == 1) return em_launch_NS<1, false>(p, x, B, q, none, t1, t2, n1, n2, m_pad, n_pad, 1, 0, part, stream, pscale);
     if (em_launch_NS<2, false>(p, x, B, q, none, t1, t2, n1, n2, m_pad, n_pad, nstages, 0, part, stream, pscale)) return 1;
@@ -418,4 +444,11 @@ int glqh_launch_e8_mma(const void *x, int64_t B, const void *const q[4], int nst
     const void *const q34[4] = {q[2], q[3], q[2], q[3]};
     if (nstages == 3) return em_launch_NS<1, false>(p, x, B, q34, none, t1, t1, n1, n1, m_pad, n_pad, 3, 2, part, stream, pscale);
     return em_launch_NS<2, false>(p, x, B, q34, none, t1, t1, n1, n1, m_pad, n_pad, 4, 2, part, stream, pscale);
+}
+
+// 1 when a call of this shape on folded streams keeps K inside the workgroups (one K slot, K parts summed
+// in LDS), so that up to two stages can be written as finished sums without a reduction launch
+int glqh_e8_mma_direct_ok(int64_t m_pad, int64_t n_pad, int64_t B, int nstages) {
+    em_plan p;
+    return em_make_plan(m_pad, n_pad, B, 65536, true, &p) && p.WK > 1 && p.ksplit == 1 && nstages <= 2;
 }

@@ -1,8 +1,9 @@
 """Folded form of the E8 index streams (glqh_e8_fold_table / glqh_e8_fold_indices and the
 small-batch kernel that reads it): the fold is checked against a numpy restatement of its
 definition on the real table, and a product on the folded streams must give the same bits as the
-product on the indices themselves (same K slots, same order of summation, same decoded values);
-against the oracle the usual bound holds (relative Frobenius error <= 1e-2)."""
+product on the indices themselves wherever both run the same K plan (same K slots, same order of
+summation, same decoded values) and agree to 1e-5 where the folded form sums K inside the
+workgroup; against the oracle the usual bound holds (relative Frobenius error <= 1e-2)."""
 import ctypes as C
 
 import numpy as np
@@ -102,7 +103,14 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
         y_idx = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
     finally:
         ext.E8_FOLD = True
-    assert torch.equal(y_fold, y_idx)
+    # same K slots and order of summation, same decoded values: the same bits -- except at one token when
+    # 16-row tiles fill the chip once: there the folded form keeps all of K inside a workgroup (sixteen K
+    # parts summed in LDS, finished sums written by the kernel, no reduction launch): another order
+    props = torch.cuda.get_device_properties(0)
+    if B == 1 and (m + 15) // 16 <= props.multi_processor_count and n // 8 >= 512:
+        assert rel(y_fold, y_idx) < 1e-5
+    else:
+        assert torch.equal(y_fold, y_idx)
     if m * n <= 1 << 23:                                       # and both are the oracle's product
         tabs = [O.e8_table(), O.e8_table()[:256] if stages == 2 else O.e8_table(), O.e8_table(), O.e8_table()]
         W = sum(tabs[s][q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)

@@ -310,11 +310,12 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, bool fold,
     if (m_pad * n_pad < (B == 1 ? (int64_t)6 << 20 : (int64_t)1 << 22)) return 0;
     p->TP = B == 1 ? 1 : B <= 4 ? 4 : 16;
     p->WK = p->TP == 16 ? 1 : 4;
-    // One token on folded streams (no table to speak of in LDS, room for the whole row of activations):
-    // all sixteen waves of a workgroup split K among themselves when 16-row tiles fill the chip exactly once,
+    // Up to four tokens on folded streams (no table to speak of in LDS, room for whole rows of activations):
+    // all sixteen waves of a workgroup split K among themselves when 16-row tiles fill the chip at most once,
     // so no K slot leaves the workgroup and the sums can be written finished (4096 x 14336, whole unfused
-    // call: 19.1 -> 17.7 us with the reduction launch kept; 14336 x 4096, 896 such tiles: 17.6 -> 21.7, not taken)
-    if (fold && p->TP == 1 && (m_pad + 15) / 16 <= glqh_device_cus() && nblk >= 16 * EM_STEP_BLKS) p->WK = 16;
+    // call at one token: 19.1 -> 17.7 us with the reduction launch kept, 15.8 without; at four tokens
+    // 20.1 -> 18.8; 14336 x 4096, 896 such tiles: 17.6 -> 21.7, not taken)
+    if (fold && p->TP <= 4 && (m_pad + 15) / 16 <= glqh_device_cus() && nblk >= 16 * EM_STEP_BLKS) p->WK = 16;
     const int rows = 16 * (EM_WAVES / p->WK);
     const int64_t RB = (m_pad + rows - 1) / rows;
     const int unit = p->WK * EM_STEP_BLKS;                      // blocks per workgroup step
@@ -369,6 +370,7 @@ int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q
 #define GLQH_EM(TP, WK) em_launch<NS, TP, WK, FOLD>(p, x, B, q, sp, t1, t2, n1, n2, m_pad, n_pad, ns_total, s_off, \
                                                     part, stream, ps, direct)
     if (p.TP == 1 && p.WK == 16) return GLQH_EM(1, 16);
+    if (p.TP == 4 && p.WK == 16) return GLQH_EM(4, 16);
     if (p.TP == 1) return GLQH_EM(1, 4);
     if (p.TP == 4) return GLQH_EM(4, 4);
     return GLQH_EM(16, 1);
@@ -387,7 +389,8 @@ int em_init_NS() {
     return em_set_lds(e8_mma_kernel<NS, 1, 4, false>) || em_set_lds(e8_mma_kernel<NS, 4, 4, false>) ||
            em_set_lds(e8_mma_kernel<NS, 16, 1, false>) || em_set_lds(e8_mma_kernel<NS, 1, 4, true>) ||
            em_set_lds(e8_mma_kernel<NS, 4, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 1, true>) ||
-           em_set_lds(e8_mma_kernel<NS, 1, 16, true>) || em_set_lds(e8_mma_kernel<NS, 1, 16, false>);
+           em_set_lds(e8_mma_kernel<NS, 1, 16, true>) || em_set_lds(e8_mma_kernel<NS, 1, 16, false>) ||
+           em_set_lds(e8_mma_kernel<NS, 4, 16, true>) || em_set_lds(e8_mma_kernel<NS, 4, 16, false>);
 }
 
 }  // namespace

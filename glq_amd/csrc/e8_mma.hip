@@ -310,19 +310,21 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, bool fold,
     if (m_pad * n_pad < (B == 1 ? (int64_t)6 << 20 : (int64_t)1 << 22)) return 0;
     p->TP = B == 1 ? 1 : B <= 4 ? 4 : 16;
     p->WK = p->TP == 16 ? 1 : 4;
-    // Up to four tokens on folded streams (no table to speak of in LDS, room for whole rows of activations):
-    // all sixteen waves of a workgroup split K among themselves when 16-row tiles fill the chip at most once,
-    // so no K slot leaves the workgroup and the sums can be written finished (4096 x 14336, whole unfused
-    // call at one token: 19.1 -> 17.7 us with the reduction launch kept, 15.8 without; at four tokens
-    // 20.1 -> 18.8; 14336 x 4096, 896 such tiles: 17.6 -> 21.7, not taken)
-    if (fold && p->TP <= 4 && (m_pad + 15) / 16 <= glqh_device_cus() && nblk >= 16 * EM_STEP_BLKS) p->WK = 16;
+    // On folded streams (no table to speak of in LDS, room for whole rows of activations) all sixteen waves
+    // of a workgroup split K among themselves when 16-row tiles fill the chip at most once and the row fits:
+    // no K slot leaves the workgroup and the sums can be written finished (4096 x 14336, whole unfused call
+    // at one token: 19.1 -> 17.7 us with the reduction launch kept, 15.8 without; at four tokens 20.1 -> 18.8;
+    // whole linear 4096 x 4096 at sixteen tokens 25.8 -> 19.6.  Not taken: 14336 x 4096, 896 such tiles,
+    // 17.6 -> 21.7 us; 4096 x 14336 at sixteen tokens, a row of 448 KB in four slots, 21.1 -> 39.3)
+    if (fold && (m_pad + 15) / 16 <= glqh_device_cus() && nblk >= 16 * EM_STEP_BLKS && nblk <= (p->TP == 16 ? 512 : 2048))
+        p->WK = 16;                                              // the whole row of activations in 128 KB / 32 KB of LDS
     const int rows = 16 * (EM_WAVES / p->WK);
     const int64_t RB = (m_pad + rows - 1) / rows;
     const int unit = p->WK * EM_STEP_BLKS;                      // blocks per workgroup step
     const int64_t nunits = (nblk + unit - 1) / unit;
     // activations: at most 32 KB of LDS; slots as long as that allows, so that a workgroup has one
     // tile (and one table fill per tile) where the shape permits
-    const int slot_cap_blks = p->TP == 16 ? 128 : p->WK == 16 ? 2048 : 512;
+    const int slot_cap_blks = p->WK == 16 ? (p->TP == 16 ? 512 : 2048) : p->TP == 16 ? 128 : 512;   // 128 KB / 32 KB of activations
     const int cus = glqh_device_cus();
     int64_t ks = RB >= cus ? 1 : cus / RB;                      // one tile per workgroup where possible
     if (ks > nunits) ks = nunits;
@@ -371,6 +373,7 @@ int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q
                                                     part, stream, ps, direct)
     if (p.TP == 1 && p.WK == 16) return GLQH_EM(1, 16);
     if (p.TP == 4 && p.WK == 16) return GLQH_EM(4, 16);
+    if (p.TP == 16 && p.WK == 16) return GLQH_EM(16, 16);
     if (p.TP == 1) return GLQH_EM(1, 4);
     if (p.TP == 4) return GLQH_EM(4, 4);
     return GLQH_EM(16, 1);
@@ -390,7 +393,8 @@ int em_init_NS() {
            em_set_lds(e8_mma_kernel<NS, 16, 1, false>) || em_set_lds(e8_mma_kernel<NS, 1, 4, true>) ||
            em_set_lds(e8_mma_kernel<NS, 4, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 1, true>) ||
            em_set_lds(e8_mma_kernel<NS, 1, 16, true>) || em_set_lds(e8_mma_kernel<NS, 1, 16, false>) ||
-           em_set_lds(e8_mma_kernel<NS, 4, 16, true>) || em_set_lds(e8_mma_kernel<NS, 4, 16, false>);
+           em_set_lds(e8_mma_kernel<NS, 4, 16, true>) || em_set_lds(e8_mma_kernel<NS, 4, 16, false>) ||
+           em_set_lds(e8_mma_kernel<NS, 16, 16, true>) || em_set_lds(e8_mma_kernel<NS, 16, 16, false>);
 }
 
 }  // namespace

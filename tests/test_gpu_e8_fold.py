@@ -103,11 +103,11 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
         y_idx = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
     finally:
         ext.E8_FOLD = True
-    # same K slots and order of summation, same decoded values: the same bits -- except at up to four tokens when
+    # same K slots and order of summation, same decoded values: the same bits -- except when
     # 16-row tiles fill the chip once: there the folded form keeps all of K inside a workgroup (sixteen K
     # parts summed in LDS, finished sums written by the kernel, no reduction launch): another order
     props = torch.cuda.get_device_properties(0)
-    if B <= 4 and (m + 15) // 16 <= props.multi_processor_count and n // 8 >= 512:
+    if (m + 15) // 16 <= props.multi_processor_count and 512 <= n // 8 <= (512 if B > 4 else 2048):
         assert rel(y_fold, y_idx) < 1e-5
     else:
         assert torch.equal(y_fold, y_idx)

@@ -694,10 +694,11 @@ def _fold_stream(q, packed):
     with torch.cuda.device(q.device):
         check(lib.glqh_e8_fold_indices(_p(q), q.shape[0], q.shape[1], _p(fmap), packed.shape[0], _p(lo16), _p(hi8),
                                        _stream()))
-    if len(_FOLD_STREAMS) % 64 == 63:                        # drop entries whose tensors are gone
-        for k in [k for k, v in _FOLD_STREAMS.items() if v[0]() is None or v[1]() is None]:
-            del _FOLD_STREAMS[k]
-    _FOLD_STREAMS[key] = (weakref.ref(q), weakref.ref(packed), lo16, hi8)
+    for k in [k for k, v in _FOLD_STREAMS.items()          # an older version of the same tensor
+              if k[0] == key[0] and k != key and v[0]() is q]:
+        del _FOLD_STREAMS[k]
+    drop = lambda _ref, key=key: _FOLD_STREAMS.pop(key, None)   # the copies go when the index tensor goes
+    _FOLD_STREAMS[key] = (weakref.ref(q, drop), weakref.ref(packed, drop), lo16, hi8)
     return lo16, hi8
 
 

@@ -73,6 +73,19 @@ def test_fold_of_an_index_stream_and_a_short_table(ext):
     assert lo2 is not lo16 and int(lo2.view(torch.int16)[0]) & 0x7FF == int(fm[5] & 0xFFFF)
 
 
+def test_folded_copies_go_with_their_index_tensor(ext):
+    say("e8 fold cache lifetime")
+    import gc
+    packed = ext._packed_table(e8_table_f16())
+    qd = t(np.zeros((32, 64), np.int16))
+    ext._fold_stream(qd, packed)
+    ptr = qd.data_ptr()
+    assert any(k[0] == ptr for k in ext._FOLD_STREAMS)
+    del qd
+    gc.collect()
+    assert not any(k[0] == ptr for k in ext._FOLD_STREAMS)
+
+
 def _indices(m, n, stages, seed):
     rng = np.random.default_rng(seed)
     lo = rng.integers(0, 30000, size=(stages, m, n // 8))

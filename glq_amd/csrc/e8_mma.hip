@@ -309,7 +309,12 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, bool fold,
     // against 10.1 us, 2048 x 2048 12.8 against 12.4, 1024 x 4096 13.2 against 13.4)
     if (m_pad * n_pad < (B == 1 ? (int64_t)6 << 20 : (int64_t)1 << 22)) return 0;
     p->TP = B == 1 ? 1 : B <= 4 ? 4 : 16;
-    p->WK = p->TP == 16 ? 1 : 4;
+    // 5..16 tokens on folded streams: LDS has room for 512-block slots of sixteen tokens (128 KB), so four
+    // K parts x 64-row tiles instead of 256-row tiles with up to sixteen K slots for the finishing kernel
+    // (whole two-stage linear at 16 tokens: 2048 x 2048 17.8 -> 15.0 us, 3072 x 3072 19.8 -> 15.6,
+    // 2048 x 11008 25.6 -> 21.7; unfused 14336 x 4096 20.2 -> 19.0; not for rows of more than 1536 blocks:
+    // 4096 x 14336 21.1 -> 24.3, every workgroup then stages 128 KB of activations for four steps)
+    p->WK = p->TP == 16 ? (fold && nblk <= 1536 ? 4 : 1) : 4;
     // On folded streams (no table to speak of in LDS, room for whole rows of activations) all sixteen waves
     // of a workgroup split K among themselves when 16-row tiles fill the chip at most once and the row fits:
     // no K slot leaves the workgroup and the sums can be written finished (4096 x 14336, whole unfused call
@@ -324,7 +329,7 @@ int em_make_plan(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, bool fold,
     const int64_t nunits = (nblk + unit - 1) / unit;
     // activations: at most 32 KB of LDS; slots as long as that allows, so that a workgroup has one
     // tile (and one table fill per tile) where the shape permits
-    const int slot_cap_blks = p->WK == 16 ? (p->TP == 16 ? 512 : 2048) : p->TP == 16 ? 128 : 512;   // 128 KB / 32 KB of activations
+    const int slot_cap_blks = p->WK == 16 ? (p->TP == 16 ? 512 : 2048) : p->TP == 16 ? (p->WK == 4 ? 512 : 128) : 512;   // 128 KB / 32 KB of activations
     const int cus = glqh_device_cus();
     int64_t ks = RB >= cus ? 1 : cus / RB;                      // one tile per workgroup where possible
     if (ks > nunits) ks = nunits;
@@ -376,6 +381,7 @@ int em_launch_NS(const em_plan &p, const void *x, int64_t B, const void *const q
     if (p.TP == 16 && p.WK == 16) return GLQH_EM(16, 16);
     if (p.TP == 1) return GLQH_EM(1, 4);
     if (p.TP == 4) return GLQH_EM(4, 4);
+    if (p.TP == 16 && p.WK == 4) return GLQH_EM(16, 4);
     return GLQH_EM(16, 1);
 #undef GLQH_EM
 }
@@ -394,7 +400,8 @@ int em_init_NS() {
            em_set_lds(e8_mma_kernel<NS, 4, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 1, true>) ||
            em_set_lds(e8_mma_kernel<NS, 1, 16, true>) || em_set_lds(e8_mma_kernel<NS, 1, 16, false>) ||
            em_set_lds(e8_mma_kernel<NS, 4, 16, true>) || em_set_lds(e8_mma_kernel<NS, 4, 16, false>) ||
-           em_set_lds(e8_mma_kernel<NS, 16, 16, true>) || em_set_lds(e8_mma_kernel<NS, 16, 16, false>);
+           em_set_lds(e8_mma_kernel<NS, 16, 16, true>) || em_set_lds(e8_mma_kernel<NS, 16, 16, false>) ||
+           em_set_lds(e8_mma_kernel<NS, 16, 4, true>) || em_set_lds(e8_mma_kernel<NS, 16, 4, false>);
 }
 
 }  // namespace

@@ -326,9 +326,12 @@ int glqh_e8_dequant_matmul(const void *x_f16, int64_t B,
                            float *out, void *ws, size_t ws_bytes, void *stream);
 
 /* The same with the layer's folded streams beside the indices: up to 16 tokens on shapes
- * the LDS-table kernel serves, the product reads `folded` instead of q1..q4 / the tables
- * (same workspace, same K slots, same order of summation); every other case ignores it.
- * folded == NULL is glqh_e8_dequant_matmul. */
+ * the LDS-table kernel serves, the product reads `folded` instead of q1..q4 / the tables;
+ * every other case ignores it.  Same workspace.  The decoded values are the same; the K plan
+ * may differ (on folded streams K can stay inside a workgroup, and one- and two-stage
+ * products are then written finished, without a reduction launch), so results agree with
+ * glqh_e8_dequant_matmul to fp32 summation order (1e-5 relative), bit for bit where the plans
+ * coincide.  folded == NULL is glqh_e8_dequant_matmul. */
 int glqh_e8_dequant_matmul_folded(const void *x_f16, int64_t B,
                                   const void *q1, const void *q2, const void *q3, const void *q4,
                                   const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,

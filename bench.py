@@ -254,6 +254,22 @@ def extras(torch, ext, dev):
             out[f"e8_2stage_matmul_4096x14336_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
         ext.E8_BATCH_MAX = e8_default
         del qs, i1, i2
+        # whole two-stage E8 linear (both transforms), 4096 x 4096, one token, rotating over 36 index sets
+        # (302 MB): the E8 counterpart of trellis_linear_4096x4096_B1_us
+        from glq_amd import hadamard as H
+        m = n = 4096
+        bn = H.block_decompose(n)
+        bnt, bnm = torch.tensor(bn), H.pack_block_meta(bn).to(dev)
+        sv = torch.ones(n, dtype=torch.float16, device=dev)
+        cbh = cb.half()
+        q4 = [(torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16),
+               torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)) for _ in range(36)]
+        xb = torch.randn(1, n, device=dev).to(torch.bfloat16)
+        out["e8_2stage_linear_4096x4096_B1_us"] = round(_graph_time(
+            torch, lambda: [ext.glq_fused_linear_block_diag_cuda(xb, sv, sv, a, cbh, 0.02, n, m, n, m, bnt, bnt, bnm, bnm,
+                                                                 b, cbh, 1 / 3.0, out_dtype=torch.bfloat16)
+                            for a, b in q4], len(q4)), 2)
+        del q4
         torch.cuda.empty_cache()
     except Exception as e:
         out["e8_error"] = f"{type(e).__name__}: {e}"

@@ -851,19 +851,28 @@ moe_route_kernel(const int64_t *__restrict__ topk_ids, int n_slots, int n_expert
                  int *__restrict__ offs) {
     const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (e > n_experts) return;                                   // uniform over the wave
+    constexpr int U = 8;                                         // 512 slots requested before the first is looked at
     int below = 0;
-    for (int base = 0; base < n_slots; base += 64) {
-        const int64_t id = base + lane < n_slots ? topk_ids[base + lane] : -1;
-        below += __builtin_popcountll(__ballot(id >= 0 && id < e));
+    for (int base = 0; base < n_slots; base += 64 * U) {
+        int64_t id[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) id[u] = base + 64 * u + lane < n_slots ? topk_ids[base + 64 * u + lane] : -1;
+#pragma unroll
+        for (int u = 0; u < U; ++u) below += __builtin_popcountll(__ballot(id[u] >= 0 && id[u] < e));
     }
     if (lane == 0) offs[e] = below;
     if (e == n_experts) return;
     int mine = 0;
-    for (int base = 0; base < n_slots; base += 64) {
-        const int64_t id = base + lane < n_slots ? topk_ids[base + lane] : -1;
-        const unsigned long long hit = __ballot(id == e);
-        if (id == e) perm[below + mine + __builtin_popcountll(hit & ((1ull << lane) - 1ull))] = base + lane;
-        mine += __builtin_popcountll(hit);
+    for (int base = 0; base < n_slots; base += 64 * U) {
+        int64_t id[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) id[u] = base + 64 * u + lane < n_slots ? topk_ids[base + 64 * u + lane] : -1;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned long long hit = __ballot(id[u] == e);
+            if (id[u] == e) perm[below + mine + __builtin_popcountll(hit & ((1ull << lane) - 1ull))] = base + 64 * u + lane;
+            mine += __builtin_popcountll(hit);
+        }
     }
 }
 

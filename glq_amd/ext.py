@@ -436,6 +436,8 @@ def glq_fused_moe_trellis_3inst_cuda(x, topk_ids, topk_weights,
     if int(activation_type) not in (0, 1, 2):
         raise RuntimeError(f"trellis MoE path supports gated activations (0/1/2) only, got {activation_type}")
     T, K = topk_ids.shape
+    if T == 0 or K == 0:                                      # an empty batch (or no choices): nothing to launch
+        return torch.zeros((T, int(hidden_size)), dtype=out_dtype or x.dtype, device=x.device)
     ids = topk_ids.to(device=x.device, dtype=torch.int64).contiguous()
     tw = topk_weights.to(device=x.device, dtype=torch.float32).contiguous()
     keep = []

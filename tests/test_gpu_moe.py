@@ -179,6 +179,15 @@ def test_registered_op_and_graph_replay(ext):
         assert rel(out, ex.oracle(x.float().cpu().numpy(), ids2, w2, 0)) < TOL
 
 
+def test_empty_batch(ext):
+    say("moe empty batch")
+    ex = experts(6, 256, 128)
+    x = torch.zeros(0, 256, dtype=torch.float16, device=DEV)
+    y = ext.glq_fused_moe_trellis_3inst_cuda(x, torch.zeros(0, 2, dtype=torch.int64, device=DEV),
+                                             torch.zeros(0, 2, device=DEV), *ex.device_args(0))
+    assert y.shape == (0, 256) and y.dtype == torch.float16
+
+
 def test_refusals(ext):
     say("moe refusals")
     ex = experts(6, 256, 128)

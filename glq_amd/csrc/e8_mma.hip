@@ -106,8 +106,16 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
         }
         return (int64_t)min(row, m_pad - 1) * nblk + min(b0 + 8 * g, nblk - 8);
     };
+    // a step whose 32 blocks all lie past the row (the last slot of a row that is not a multiple of the
+    // step round) is skipped: no index run is requested for it, nothing is looked up (uniform over the wave)
+    auto step_live = [&](int sidx) -> bool {
+        if (sidx >= nsteps) return false;
+        const int tile = blockIdx.x + (sidx / spt) * gridDim.x;
+        return (tile / RB) * slot_blks + ((sidx % spt) * WK + wk) * EM_STEP_BLKS < nblk;
+    };
     em_idx<NS, FOLD> cur = em_load_idx<NS, FOLD>(qs, sp, idx_offset(0));
-    em_idx<NS, FOLD> nx1 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(1));
+    em_idx<NS, FOLD> nx1 = cur;
+    if (step_live(1)) nx1 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(1));
     // FOLD: byte offset of stage 2's half codewords inside tab
     const uint32_t n1r = (n1 + 1u) & ~1u;
     const uint32_t tab2_off = t2_is_t1 ? 0u : 8u * n1r;
@@ -175,8 +183,9 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
             const u32x4 *xl = live ? xs + (b0 - sb0 + 8 * g) * TP + i : zero_slots;
             if constexpr (FOLD) {
                 em_idx<NS, FOLD> nx2 = nx1;
-                if (sidx + 2 < nsteps) nx2 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(sidx + 2));   // uniform
+                if (step_live(sidx + 2)) nx2 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(sidx + 2));   // uniform
                 const char *tb = (const char *)tab;
+                if (b0 < nblk) {                               // uniform
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {                  // four lookups per stage at a time: 32 registers of operands
                     u32x4 af[NS][4];
@@ -205,6 +214,7 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                             acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[s][u]), bf, acc[s], 0, 0, 0);
                     }
                 }
+                }
                 cur = nx1;
                 nx1 = nx2;
                 continue;
@@ -228,7 +238,7 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
             }
             // requested after the lookups, so that waiting for those does not wait for this
             em_idx<NS, FOLD> nx2 = nx1;
-            if (sidx + 2 < nsteps) nx2 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(sidx + 2));   // uniform
+            if (step_live(sidx + 2)) nx2 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(sidx + 2));   // uniform
             if (b0 < nblk_r) {                                 // uniform; past the row the activations are zero
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {

@@ -116,7 +116,7 @@ e8_mma_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
     em_idx<NS, FOLD> cur = em_load_idx<NS, FOLD>(qs, sp, idx_offset(0));
     // On the indices the runs of steps n + 1 and n + 2 are in flight while step n is looked up.  The folded
     // form requests one step ahead only: with more in flight the waves' requests queue up behind each other
-    // in the memory system (4096 x 14336, one token, whole call: three steps ahead 16.7 us, two 15.0, one 13.6).
+    // in the memory system (4096 x 14336, one token, whole call: three steps ahead 16.7 us, two 15.0, one 13.7).
     em_idx<NS, FOLD> nx1 = cur;
     if (!FOLD && step_live(1)) nx1 = em_load_idx<NS, FOLD>(qs, sp, idx_offset(1));
     // FOLD: byte offset of stage 2's half codewords inside tab

@@ -289,8 +289,8 @@ def extras(torch, ext, dev):
         q1 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
         q2 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
         for M, route in ((256, ""), (4096, ""), (4096, "_compressed")):
-            # "" = the route the library picks (compressed up to 2048 tokens for trellis and 1024 for
-            # E8, dequantize + library GEMM above); "_compressed" = the tile kernels forced at 4096 tokens
+            # "" = the route the library picks (compressed up to 2048 tokens for trellis and, on the folded
+            # streams, 4096 for E8; dequantize + library GEMM above); "_compressed" = the tile kernels forced
             ext.TRELLIS_BATCH_MAX = (1 << 30) if route else tr_default
             ext.E8_BATCH_MAX = (1 << 30) if route else e8_default
             xb = torch.randn(M, n, device=dev).to(torch.bfloat16)

@@ -25,7 +25,7 @@ int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages);
 size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M);
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
-                        int64_t n_pad, float *part, hipStream_t stream);
+                        int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold);
 // Above 16 tokens the weights are decoded once per 128 x 512 tile instead of once per 16 tokens.
 #define GLQH_E8_SMALL_BATCH 16
 static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages) {
@@ -1077,6 +1077,7 @@ int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, int 
 
 extern "C" int glqh_e8_fold_eligible(int64_t m_pad, int64_t n_pad, int64_t B) {
     if (glqh_init() != 0 || m_pad < 1 || n_pad < 8 || (n_pad & 7) || B < 1) return 0;
+    if (B > GLQH_E8_SMALL_BATCH) return glqh_e8_tile_ksplit(m_pad, n_pad, B, 1) > 0 ? 1 : 0;   // the many-token kernel
     return glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536, 1) > 0 ? 1 : 0;
 }
 
@@ -1186,7 +1187,7 @@ extern "C" int glqh_e8_dequant_matmul_folded(const void *x_f16, int64_t B, const
         GLQH_REQUIRE(ws && ws_bytes >= need, "e8 matmul: workspace of %zu bytes needed, got %zu", need, ws_bytes);
         const float rel[3] = {(float)inv_rs, (float)inv_rs2, (float)inv_rs3};
         if (glqh_launch_e8_tile(x_f16, (char *)ws + pbytes, B, sg.q, sg.n, table1, table2 ? table2 : table1, table2 ? n_entries2 : 65536,
-                                rel, m_pad, n_pad, part, st))
+                                rel, m_pad, n_pad, part, st, folded))
             return 1;
         return glqh_launch_reduce_splits(part, tks, B * m_pad, B, m_pad, (float)wscale, out, m_pad, 0, st);
     }
@@ -1304,7 +1305,7 @@ extern "C" int glqh_fused_linear_e8_folded(const void *x, int x_dtype, int64_t x
         // scaled by the output transform
         const float rel[3] = {(float)inv_rs, (float)inv_rs2, (float)inv_rs3};
         if (glqh_launch_e8_tile(blocked == 0 ? nullptr : x_rht, (char *)ws + xb + tile_part, B, sg.q, sg.n, table1,
-                                table2 ? table2 : table1, table2 ? n_entries2 : 65536, rel, m_pad, n_pad, part, st))
+                                table2 ? table2 : table1, table2 ? n_entries2 : 65536, rel, m_pad, n_pad, part, st, folded))
             return 1;
         glqh_ysrc src = {};
         src.nparts = 1;

@@ -29,6 +29,12 @@
 // an order that gives the CUs of one XCD the same tokens at the same time, so the activations
 // are served by that XCD's L2.  K is split into slots only while the tiles alone would leave CUs
 // idle; partial sums [slot][token][row] are combined in slot order by the consumer.
+//
+// FOLD: the same kernel on the folded streams (glqh_e8_fold_table / glqh_e8_fold_indices, e8_mma.hip):
+// an index is two 11-bit half-codeword numbers, the table of half codewords as finished fp16 values
+// (at most 16 KB per table) sits in LDS whole, and a lookup is two 8-byte LDS reads whose result is
+// the operand: no table word comes from L2, nothing is expanded, 128 KB of table fill per workgroup
+// fall away.  The fp16 values and the stage arithmetic are the same, so the results are bit-identical.
 #include "e8_device.h"
 
 namespace {
@@ -43,9 +49,11 @@ constexpr int ET_BUF = 2 * ET_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer
 constexpr size_t ET_LDS = (size_t)(ET_P + 1) * 4 + (size_t)2 * ET_BUF * 16;   // 128 KB + 32 KB
 
 struct et_args {
-    const uint16_t *q[4];
-    const uint32_t *t1, *t2;
+    const uint16_t *q[4];                          // FOLD: the 16-bit words of the folded streams
+    const uint8_t *hi8[4];                         // FOLD: their byte planes
+    const uint32_t *t1, *t2;                       // FOLD: half-codeword tables, two words per entry
     uint32_t n2;
+    uint32_t nh1, nh2;                             // FOLD: entries of the half-codeword tables
     int t2_is_t1;
     float r[3];                                    // factors of stages 2..4 relative to stage 1
     const f16 *xb;                                 // transformed activations, (n_pad / 32, Mp, 4, 8) fp16
@@ -59,18 +67,27 @@ __device__ __forceinline__ void et_barrier() {     // waits for LDS only: global
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <int NS, int NTW>
+template <int NS, int NTW, bool FOLD>
 __global__ void __launch_bounds__(ET_THREADS)
 e8_tile_kernel(const et_args a) {
     extern __shared__ u32x4 lds[];
     const uint32_t *tab = (const uint32_t *)lds;
-    u32x4 *abuf = lds + (ET_P + 1) / 4;
+    // FOLD: stage 1's half codewords (an even number of 8-byte entries), then stage 2's if they differ
+    const uint32_t nh1r = (a.nh1 + 1u) & ~1u, nh2r = (a.nh2 + 1u) & ~1u;
+    const uint32_t tab2_off = a.t2_is_t1 ? 0u : 8u * nh1r;     // bytes
+    u32x4 *abuf = lds + (FOLD ? (nh1r + (a.t2_is_t1 ? 0u : nh2r)) / 2 : (uint32_t)(ET_P + 1) / 4);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, g = lane >> 4;
     const int nblk = a.n_pad >> 3, nds = a.n_pad >> 6;
+    constexpr int NFB = FOLD ? NS : 1;                         // stages with a byte run
 
-    // table prefix -> LDS, all loads of a round in flight before its first write
-    {
+    if constexpr (FOLD) {
+        uint32_t *tw = (uint32_t *)lds;
+        for (uint32_t j = threadIdx.x; j < 2u * a.nh1; j += ET_THREADS) tw[j] = a.t1[j];
+        if (!a.t2_is_t1)
+            for (uint32_t j = threadIdx.x; j < 2u * a.nh2; j += ET_THREADS) tw[2u * nh1r + j] = a.t2[j];
+    } else {
+        // table prefix -> LDS, all loads of a round in flight before its first write
         constexpr int PER = (ET_P + 1) / 4 / ET_THREADS;       // 16 x 16 bytes per thread
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -82,7 +99,7 @@ e8_tile_kernel(const et_args a) {
         }
     }
     __syncthreads();
-    if (threadIdx.x == 0) ((uint32_t *)lds)[ET_P] = ET_MISS;   // what a lookup past the prefix reads
+    if (!FOLD && threadIdx.x == 0) ((uint32_t *)lds)[ET_P] = ET_MISS;   // what a lookup past the prefix reads
     __syncthreads();
 
     // a separate stage-2 table stays in L2: its LDS lookups are all sent to the sentinel
@@ -110,6 +127,9 @@ e8_tile_kernel(const et_args a) {
         const u32x4 *qrow[NS];                                  // 8 indices = the 64 columns of step 4q + g
 #pragma unroll
         for (int s = 0; s < NS; ++s) qrow[s] = (const u32x4 *)(a.q[s] + (int64_t)drow * nblk) + (ds0 >> 2) * 4 + g;
+        // FOLD: a stream tile is 16 rows x 32 indices = this wave's rows x one group of four steps; lane
+        // (i, g) holds indices 8g .. 8g+7 of row i at entry 8 * lane
+        const int64_t fbase = (((int64_t)min((r0 >> 4) + wave, ((a.m_pad + 15) >> 4) - 1) * (nblk >> 5) + (ds0 >> 2)) * 64 + lane) * 8;
         // multiply role: token 16 * tt + i of the wave's tokens, blocks 8d + 2g and 8d + 2g + 1
         // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
         // block 8 d + 2 g + u of step d: group of four blocks 2 d + (g >> 1), position 2 (g & 1) + u
@@ -185,23 +205,75 @@ e8_tile_kernel(const et_args a) {
         // it decodes index pair g of that step: a 4 x 4 transpose of dwords over the four lanes
         // that share row i (lane distance 16), done with two pairs of lane-swap instructions.
         const int nquads = (ds1 - ds0) >> 2;
-        auto load_quad = [&](u32x4 (&run)[NS], int q) {
+        auto load_quad = [&](u32x4 (&run)[NS], u32x2 (&runb)[NFB], int q) {
             q = min(q, nquads - 1);
 #pragma unroll
-            for (int s = 0; s < NS; ++s) run[s] = __builtin_nontemporal_load(qrow[s] + 4 * q);
+            for (int s = 0; s < NS; ++s) {
+                if constexpr (FOLD) {
+                    run[s] = __builtin_nontemporal_load((const u32x4 *)(a.q[s] + fbase + (int64_t)q * 512));
+                    runb[FOLD ? s : 0] = __builtin_nontemporal_load((const u32x2 *)(a.hi8[s] + fbase + (int64_t)q * 512));
+                } else {
+                    run[s] = __builtin_nontemporal_load(qrow[s] + 4 * q);
+                }
+            }
         };
-        auto transpose = [&](const u32x4 (&run)[NS], uint32_t (&T)[NS][4]) {
+        auto transpose4 = [&](uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3, uint32_t (&T)[4]) {
+            const auto p02 = __builtin_amdgcn_permlane32_swap(d0, d2, false, false);
+            const auto p13 = __builtin_amdgcn_permlane32_swap(d1, d3, false, false);
+            const auto lo = __builtin_amdgcn_permlane16_swap(p02[0], p13[0], false, false);
+            const auto hi = __builtin_amdgcn_permlane16_swap(p02[1], p13[1], false, false);
+            T[0] = lo[0];
+            T[1] = lo[1];
+            T[2] = hi[0];
+            T[3] = hi[1];
+        };
+        // T[s][dd] = the index pair this lane decodes in step dd; FOLD: TB[s][dd] = the pair's two bytes
+        // in bits 0..15 (the 16-bit pieces of the byte run take the same way as the dwords of the word run)
+        auto transpose = [&](const u32x4 (&run)[NS], const u32x2 (&runb)[NFB], uint32_t (&T)[NS][4], uint32_t (&TB)[NFB][4]) {
 #pragma unroll
             for (int s = 0; s < NS; ++s) {
-                const auto p02 = __builtin_amdgcn_permlane32_swap(run[s][0], run[s][2], false, false);
-                const auto p13 = __builtin_amdgcn_permlane32_swap(run[s][1], run[s][3], false, false);
-                const auto lo = __builtin_amdgcn_permlane16_swap(p02[0], p13[0], false, false);
-                const auto hi = __builtin_amdgcn_permlane16_swap(p02[1], p13[1], false, false);
-                T[s][0] = lo[0];
-                T[s][1] = lo[1];
-                T[s][2] = hi[0];
-                T[s][3] = hi[1];
+                transpose4(run[s][0], run[s][1], run[s][2], run[s][3], T[s]);
+                if constexpr (FOLD) transpose4(runb[s][0], runb[s][0] >> 16, runb[s][1], runb[s][1] >> 16, TB[s]);   // s < NFB
             }
+        };
+        // FOLD: the half codewords of a step's two index pairs, as they come out of LDS
+        struct halves {
+            u32x2 c[NS][2][2];                                  // [stage][pair member][half]
+        };
+        auto fold_lookups = [&](const uint32_t (&T)[NS][4], const uint32_t (&TB)[NFB][4], int dd) {
+            halves h;
+            const char *tb = (const char *)tab;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const uint32_t w = T[s][dd], by = TB[FOLD ? s : 0][dd];
+                const char *tbs = tb + (s == 1 ? tab2_off : 0u);
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    // byte offsets 8 * half number: first half from bits 0..10 of the index's 16-bit word,
+                    // second from its bits 11..15 and the index's byte
+                    const uint32_t lo = u ? (w >> 13) & 0x3FF8u : (w << 3) & 0x3FF8u;
+                    const uint32_t h5 = u ? (w >> 24) & 0xF8u : (w >> 8) & 0xF8u;
+                    const uint32_t b6 = u ? by & 0x3F00u : (by << 8) & 0x3F00u;
+                    h.c[s][u][0] = *(const u32x2 *)(tbs + lo);
+                    h.c[s][u][1] = *(const u32x2 *)(tbs + (h5 | b6));
+                }
+            }
+            return h;
+        };
+        auto fold_emit_half = [&](const halves &h, int u, u32x4 *dst) {   // one A fragment
+            f16x8 af = __builtin_bit_cast(f16x8, u32x4{h.c[0][u][0][0], h.c[0][u][0][1], h.c[0][u][1][0], h.c[0][u][1][1]});
+#pragma unroll
+            for (int s = 1; s < NS; ++s) {
+                const f16x8 e = __builtin_bit_cast(f16x8, u32x4{h.c[s][u][0][0], h.c[s][u][0][1], h.c[s][u][1][0], h.c[s][u][1][1]});
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const f16x2 ev = {e[2 * p], e[2 * p + 1]}, av = {af[2 * p], af[2 * p + 1]};
+                    const f16x2 rv = __builtin_elementwise_fma(ev, rs[s - 1], av);
+                    af[2 * p] = rv[0];
+                    af[2 * p + 1] = rv[1];
+                }
+            }
+            dst[(u * ET_FRAGS + wave) * GLQH_WAVE + lane] = __builtin_bit_cast(u32x4, af);
         };
         auto load_b = [&](u32x4 (&b)[NTW][2], int d) {
             d = min(d, ds1 - 1);
@@ -227,20 +299,25 @@ e8_tile_kernel(const et_args a) {
         constexpr int LA = NTW <= 2 ? 2 : 1;
         constexpr bool BDB = NTW <= 2;
         u32x4 run[NS];
-        uint32_t T[NS][4];
+        u32x2 runb[NFB];
+        uint32_t T[NS][4], TB[NFB][4];
         u32x4 b[BDB ? 2 : 1][NTW][2];
         looked lk[LA];
-        load_quad(run, 0);
+        load_quad(run, runb, 0);
         load_b(b[0], ds0);
-        transpose(run, T);
-        load_quad(run, 1);
-        {
+        transpose(run, runb, T, TB);
+        load_quad(run, runb, 1);
+        if constexpr (FOLD) {
+            const halves first = fold_lookups(T, TB, 0);
+            fold_emit_half(first, 0, abuf);
+            fold_emit_half(first, 1, abuf);
+        } else {
             const looked first = lookups(T, 0);
             emit(first, abuf);
-        }
-        static_assert(LA <= 3, "the prologue requests entries from the first index group only");
+            static_assert(LA <= 3, "the prologue requests entries from the first index group only");
 #pragma unroll
-        for (int j = 1; j <= LA; ++j) lk[j % LA] = lookups(T, j & 3);
+            for (int j = 1; j <= LA; ++j) lk[j % LA] = lookups(T, j & 3);
+        }
         et_barrier();
 
         for (int q = 0; q < nquads; ++q) {
@@ -252,16 +329,25 @@ e8_tile_kernel(const et_args a) {
                 u32x4 *wr = abuf + ((dd & 1) ^ 1) * ET_BUF;
                 const int dn = min(d + 1, ds1 - 1);
                 if constexpr (BDB) load_b(b[nxt], d + 1);
-                const looked &lke = lk[(dd + 1) % LA];          // entries of d + 1: expanded during this step
-                const lds_words wle = lds_lookups(lke);
-                const looked lkn = [&] {
+                looked lke, lkn;
+                lds_words wle;
+                halves hv;
+                if constexpr (FOLD) {                           // the half codewords of d + 1
+                    if (dd == 3) {                              // the next group's indices take over
+                        transpose(run, runb, T, TB);
+                        load_quad(run, runb, q + 2);
+                    }
+                    hv = fold_lookups(T, TB, (dd + 1) & 3);
+                } else {
+                    lke = lk[(dd + 1) % LA];                    // entries of d + 1: expanded during this step
+                    wle = lds_lookups(lke);
                     const int sl = dd + 1 + LA;                 // step looked up now, relative to 4q
                     if ((sl & 3) == 0) {                        // its group's indices take over
-                        transpose(run, T);
-                        load_quad(run, q + (sl >> 2) + 1);
+                        transpose(run, runb, T, TB);
+                        load_quad(run, runb, q + (sl >> 2) + 1);
                     }
-                    return lookups(T, sl & 3);
-                }();
+                    lkn = lookups(T, sl & 3);
+                }
                 // 16 operand fragments (2 half-steps x 8 row fragments), each read from LDS one
                 // fragment ahead of the multiplications that use it; the expansion of the next
                 // step's operands is spread between them
@@ -276,8 +362,13 @@ e8_tile_kernel(const et_args a) {
                     for (int tt = 0; tt < NTW; ++tt)
                         acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                             af, __builtin_bit_cast(f16x8, b[cur][tt][u]), acc[f][tt], 0, 0, 0);
-                    if (k == 1) expand_half(lke, wle, 0, wr);   // operands of d + 1 (unused after the last step)
-                    if (k == 9) expand_half(lke, wle, 1, wr);
+                    if constexpr (FOLD) {
+                        if (k == 1) fold_emit_half(hv, 0, wr);  // operands of d + 1 (unused after the last step)
+                        if (k == 9) fold_emit_half(hv, 1, wr);
+                    } else {
+                        if (k == 1) expand_half(lke, wle, 0, wr);
+                        if (k == 9) expand_half(lke, wle, 1, wr);
+                    }
                     if constexpr (!BDB) {
                         if (f == ET_FRAGS - 1) {                // this half's activations are free: request the next
                             __builtin_amdgcn_sched_barrier(0);
@@ -287,7 +378,7 @@ e8_tile_kernel(const et_args a) {
                         }
                     }
                 }
-                lk[(dd + 1) % LA] = lkn;
+                if constexpr (!FOLD) lk[(dd + 1) % LA] = lkn;
                 et_barrier();                                   // rd has been read, wr is written
             }
         }
@@ -376,32 +467,40 @@ int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *
     return 1;
 }
 
-template <int NS, int NTW>
+// FOLD: two tables of at most 2048 half codewords of 8 bytes, and the A buffers
+constexpr size_t ET_LDS_FOLD = (size_t)2 * 2048 * 8 + (size_t)2 * ET_BUF * 16;
+
+template <int NS, int NTW, bool FOLD>
 int et_launch(const et_plan &p, const et_args &a, hipStream_t stream) {
-    hipLaunchKernelGGL((e8_tile_kernel<NS, NTW>), dim3((unsigned)p.grid), dim3(ET_THREADS), ET_LDS, stream, a);
+    size_t lds = ET_LDS;
+    if (FOLD) lds = (size_t)(((a.nh1 + 1u) & ~1u) + (a.t2_is_t1 ? 0u : (a.nh2 + 1u) & ~1u)) * 8 + (size_t)2 * ET_BUF * 16;
+    hipLaunchKernelGGL((e8_tile_kernel<NS, NTW, FOLD>), dim3((unsigned)p.grid), dim3(ET_THREADS), lds, stream, a);
     GLQH_LAUNCH_CHECK("e8 tile launch");
     return 0;
 }
 
-template <int NS>
+template <int NS, bool FOLD>
 int et_launch_NS(const et_plan &p, const et_args &a, hipStream_t stream) {
-    if (p.NTW == 1) return et_launch<NS, 1>(p, a, stream);
-    if (p.NTW == 2) return et_launch<NS, 2>(p, a, stream);
-    if constexpr (NS <= 2) return et_launch<NS, 4>(p, a, stream);
+    if (p.NTW == 1) return et_launch<NS, 1, FOLD>(p, a, stream);
+    if (p.NTW == 2) return et_launch<NS, 2, FOLD>(p, a, stream);
+    if constexpr (NS <= 2) return et_launch<NS, 4, FOLD>(p, a, stream);
     return glqh_fail("e8 tile kernel: no 512-token tiles for %d stages", NS);
 }
 
 template <typename K>
-int et_set_lds(K kernel) {
+int et_set_lds(K kernel, size_t bytes) {
     return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              (int)ET_LDS),
+                                              (int)bytes),
                           "e8 tile attribute");
 }
 
 template <int NS>
 int et_init_NS() {
-    if (et_set_lds(e8_tile_kernel<NS, 1>) || et_set_lds(e8_tile_kernel<NS, 2>)) return 1;
-    if constexpr (NS <= 2) return et_set_lds(e8_tile_kernel<NS, 4>);
+    if (et_set_lds(e8_tile_kernel<NS, 1, false>, ET_LDS) || et_set_lds(e8_tile_kernel<NS, 2, false>, ET_LDS) ||
+        et_set_lds(e8_tile_kernel<NS, 1, true>, ET_LDS_FOLD) || et_set_lds(e8_tile_kernel<NS, 2, true>, ET_LDS_FOLD))
+        return 1;
+    if constexpr (NS <= 2)
+        return et_set_lds(e8_tile_kernel<NS, 4, false>, ET_LDS) || et_set_lds(e8_tile_kernel<NS, 4, true>, ET_LDS_FOLD);
     return 0;
 }
 
@@ -427,7 +526,7 @@ int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages) { return et_padded_to
 
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
-                        int64_t n_pad, float *part, hipStream_t stream) {
+                        int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold) {
     glqh_range range("dequant_matmul");
     et_plan p;
     if (!et_make_plan(m_pad, n_pad, M, nstages, &p)) return glqh_fail("e8 tile kernel: shape not eligible (n_pad %% 256)");
@@ -439,10 +538,28 @@ int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const vo
     }
     et_args a;
     for (int s = 0; s < 4; ++s) a.q[s] = (const uint16_t *)q[s];
+    for (int s = 0; s < 4; ++s) a.hi8[s] = nullptr;
     a.t1 = t1;
     a.t2 = t2;
     a.n2 = (uint32_t)n2;
+    a.nh1 = a.nh2 = 0;
     a.t2_is_t1 = (t1 == t2 && n2 == 65536);
+    if (fold) {                                                // the folded streams take the indices' place
+        const bool own2 = nstages >= 2 && !a.t2_is_t1;
+        GLQH_REQUIRE(!own2 || fold->halves2, "e8 folded: stage 2 has a table of its own but no folded table");
+        a.t1 = (const uint32_t *)fold->halves1;
+        a.t2 = own2 ? (const uint32_t *)fold->halves2 : a.t1;
+        a.nh1 = (uint32_t)fold->n_halves1;
+        a.nh2 = (uint32_t)(own2 ? fold->n_halves2 : fold->n_halves1);
+        a.t2_is_t1 = !own2;
+        GLQH_REQUIRE(a.t1 && fold->n_halves1 >= 1 && fold->n_halves1 <= 2048 && a.nh2 >= 1 && a.nh2 <= 2048,
+                     "e8 folded: 1..2048 half codewords per table");
+        for (int s = 0; s < nstages; ++s) {
+            GLQH_REQUIRE(fold->lo16[s] && fold->hi8[s], "e8 folded: stage %d has no folded stream", s + 1);
+            a.q[s] = fold->lo16[s];
+            a.hi8[s] = fold->hi8[s];
+        }
+    }
     for (int s = 0; s < 3; ++s) a.r[s] = rel[s];
     a.xb = (const f16 *)xb_scratch;
     a.M = (int)M;
@@ -454,11 +571,15 @@ int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const vo
     a.KS = p.KS;
     a.slot_ds = p.slot_ds;
     a.part = part;
-    switch (nstages) {
-    case 1: return et_launch_NS<1>(p, a, stream);
-    case 2: return et_launch_NS<2>(p, a, stream);
-    case 3: return et_launch_NS<3>(p, a, stream);
-    case 4: return et_launch_NS<4>(p, a, stream);
+    switch (nstages * 2 + (fold ? 1 : 0)) {
+    case 2: return et_launch_NS<1, false>(p, a, stream);
+    case 3: return et_launch_NS<1, true>(p, a, stream);
+    case 4: return et_launch_NS<2, false>(p, a, stream);
+    case 5: return et_launch_NS<2, true>(p, a, stream);
+    case 6: return et_launch_NS<3, false>(p, a, stream);
+    case 7: return et_launch_NS<3, true>(p, a, stream);
+    case 8: return et_launch_NS<4, false>(p, a, stream);
+    case 9: return et_launch_NS<4, true>(p, a, stream);
     }
     return glqh_fail("e8 matmul: %d stages unsupported (1-4)", nstages);
 }

@@ -42,12 +42,18 @@ TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "2048")))
 # reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
 TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ
 E8_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "1024")))
+# On the folded streams (see E8_FOLD below) the E8 tile kernel looks nothing up outside LDS and expands
+# nothing, and the compressed route wins or ties up to 4096 tokens (whole two-stage linear, compressed /
+# library, us: 268 / 322 and 300 / 321 at 2048 tokens on 4096 x 14336 and 14336 x 4096, 519 / 516 and
+# 585 / 595 at 4096, 1087 / 984 and 1146 / 1047 at 8192).  The larger of the two limits applies there.
+E8_FOLD_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "4096")))
 
 
-def _e8_dense_route(B, n_pad):
+def _e8_dense_route(B, n_pad, folded=False):
     """Dequantize + library GEMM: on request, and for the widths the tile kernel does not take
     (n_pad not a multiple of 256) above 16 tokens."""
-    return B > E8_BATCH_MAX or (B > 16 and int(n_pad) % 256 != 0)
+    limit = max(E8_BATCH_MAX, E8_FOLD_BATCH_MAX) if folded else E8_BATCH_MAX
+    return B > limit or (B > 16 and int(n_pad) % 256 != 0)
 
 
 def _p(t):
@@ -790,12 +796,15 @@ def _e8_matmul_tables(x, qidxs, t1, q2, t2, n2, q3, q4, wscale, inv_rs, inv_rs2,
     M, nblk = qidxs.shape
     if x.shape[1] != nblk * 8:
         raise RuntimeError(f"x has {x.shape[1]} columns, qidxs implies {nblk * 8}")
-    if _e8_dense_route(B, nblk * 8):
+    folded, keep = None, None
+    if not _e8_dense_route(B, nblk * 8, True):
+        with torch.cuda.device(x.device):
+            folded, keep = _e8_folded(B, qidxs, t1, q2, t2, q3, q4)
+    if _e8_dense_route(B, nblk * 8, folded is not None):
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
         return torch.mm(x, W.t(), out_dtype=torch.float32).mul_(float(wscale))
     out = torch.empty((B, M), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        folded, keep = _e8_folded(B, qidxs, t1, q2, t2, q3, q4)
         nb = lib.glqh_e8_matmul_workspace_bytes(M, nblk * 8, B)
         ws = _ws(nb, x.device)
         check(lib.glqh_e8_dequant_matmul_folded(
@@ -881,13 +890,16 @@ def _fused_e8(x, sv, su, qidxs, codebook, wscale, in_features, out_features, n_p
     bn, nbn = _host_i64(blocks_n)
     bm, nbm = _host_i64(blocks_m)
     y = torch.empty((B, int(out_features)), dtype=out_dtype or torch.float16, device=x.device)
-    if _e8_dense_route(B, n_pad):
+    folded, keep = None, None
+    if not _e8_dense_route(B, n_pad, True):
+        with torch.cuda.device(x.device):
+            folded, keep = _e8_folded(B, qidxs, t1, q2, t2, q3, q4)
+    if _e8_dense_route(B, n_pad, folded is not None):
         x_rht = torch.empty((B, int(n_pad)), dtype=torch.float16, device=x.device)
         glq_input_rht_blockdiag_cuda(x, sv, x_rht, in_features, n_pad, blocks_n, bn_meta)
         W = _e8_dense_weight(qidxs, t1, q2, t2, n2, q3, q4, inv_rs, inv_rs2, inv_rs3)
         return _dense_matmul_output(x_rht, W, wscale, su, y, out_features, m_pad, blocks_m, bm_meta)
     with torch.cuda.device(x.device):
-        folded, keep = _e8_folded(B, qidxs, t1, q2, t2, q3, q4)
         nb = lib.glqh_fused_linear_e8_workspace_bytes(B, int(n_pad), int(m_pad))
         ws = _ws(nb, x.device)
         check(lib.glqh_fused_linear_e8_folded(

@@ -133,6 +133,39 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
         assert rel(y_fold, x.float().cpu().numpy() @ W.T) < TOL
 
 
+@pytest.mark.parametrize("m,n,B", [(1000, 2048, 17), (4096, 1024, 130), (2048, 4096, 300), (1536, 2560, 520)])
+@pytest.mark.parametrize("stages", [1, 2, 3, 4])
+def test_many_token_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stages):
+    """Above 16 tokens the tile kernel reads the folded streams too: same tiles, same K slots, same fp16
+    operands (half codewords out of LDS instead of expanded table words), hence the same bits."""
+    say("e8 folded tile matmul", m, n, B, stages)
+    lib = ext._lib.load()
+    assert lib.glqh_e8_fold_eligible(m, n, B) == 1
+    q = [t(a) for a in _indices(m, n, stages, m + stages + B)]
+    cb = e8_table_f16()
+    cb2 = cb[:256].contiguous() if stages == 2 else cb        # two stages: the short secondary table
+    if stages == 2:
+        q[1] = t((_indices(m, n, 1, 7)[0].view(np.uint16) & 255).view(np.int16))
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).half().to(DEV)
+    args = dict(qidxs2=q[1] if stages > 1 else None, codebook2=cb2, inv_resid_scale=1 / 3.0 if stages > 1 else 0.0,
+                qidxs3=q[2] if stages > 2 else None, inv_resid_scale2=1 / 9.0 if stages > 2 else 0.0,
+                qidxs4=q[3] if stages > 3 else None, inv_resid_scale3=1 / 27.0 if stages > 3 else 0.0)
+    ext.E8_FOLD = True
+    try:
+        y_fold = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
+        assert any(k[0] == q[0].data_ptr() for k in ext._FOLD_STREAMS), "the folded streams were not made"
+        ext.E8_FOLD = False
+        y_idx = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
+    finally:
+        ext.E8_FOLD = True
+    assert torch.equal(y_fold, y_idx)
+    if m * n <= 1 << 23:
+        tabs = [O.e8_table(), O.e8_table()[:256] if stages == 2 else O.e8_table(), O.e8_table(), O.e8_table()]
+        W = sum(tabs[s][q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)
+                for s in range(stages)).astype(np.float32) * np.float32(0.02)
+        assert rel(y_fold, x.float().cpu().numpy() @ W.T) < TOL
+
+
 def test_fused_linear_on_folded_streams_and_under_capture(ext):
     say("e8 folded fused linear + graph")
     from glq_amd import hadamard as H
@@ -186,4 +219,5 @@ def test_c_abi_refusals(ext):
     rc = lib.glqh_e8_fold_table(packed.data_ptr(), 65536, small.data_ptr(), 16, fmap.data_ptr(), C.addressof(n), None)
     assert rc != 0 and b"room for 16" in lib.glqh_last_error() and n.value == 1286
     assert lib.glqh_e8_fold_eligible(960, 960, 1) == 0       # a small layer: the gather kernel serves it
-    assert lib.glqh_e8_fold_eligible(4096, 14336, 17) == 0   # the tile kernel's range
+    assert lib.glqh_e8_fold_eligible(4096, 14336, 17) == 1   # the tile kernel reads them too ...
+    assert lib.glqh_e8_fold_eligible(4096, 14336 + 8, 17) == 0   # ... on rows of whole 256-column groups

@@ -283,7 +283,13 @@ def test_e8_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatch):
     rows = _sample_rows(4096)
     r = x[rows].float().numpy() @ W_hat.T
     assert sqnr(r, ys[4096][torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0
-    monkeypatch.setattr(ext, "E8_BATCH_MAX", 1024)             # the library route, the default above 1024 tokens
+    # the tile kernel on the indices themselves (no folded streams): the same operands, the same bits
+    monkeypatch.setattr(ext, "E8_FOLD", False)
+    assert torch.equal(e8_forward(ext, xd, art, m, n, torch.bfloat16), ys[4096])
+    monkeypatch.setattr(ext, "E8_FOLD", True)
+    # the library route, the default above 4096 tokens (above 1024 without folded streams)
+    monkeypatch.setattr(ext, "E8_BATCH_MAX", 1024)
+    monkeypatch.setattr(ext, "E8_FOLD_BATCH_MAX", 1024)
     yl = e8_forward(ext, xd, art, m, n, torch.bfloat16)
     assert rel(yl, ys[4096].float().cpu().numpy()) < 6e-3
     assert sqnr(r, yl[torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0

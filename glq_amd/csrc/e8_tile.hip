@@ -297,6 +297,9 @@ e8_tile_kernel(const et_args a) {
         // into the registers the half-step just multiplied has freed.  Index runs arrive a group of
         // four steps ahead.
         constexpr int LA = NTW <= 2 ? 2 : 1;
+        // operand fragments read ahead of their multiplications: with one or two token tiles per wave a
+        // fragment is multiplied in 16-32 matrix-pipe cycles, less than an LDS read takes (1-3 % per call)
+        constexpr int PF = NTW <= 2 ? 2 : 1;
         constexpr bool BDB = NTW <= 2;
         u32x4 run[NS];
         u32x2 runb[NFB];
@@ -351,13 +354,15 @@ e8_tile_kernel(const et_args a) {
                 // 16 operand fragments (2 half-steps x 8 row fragments), each read from LDS one
                 // fragment ahead of the multiplications that use it; the expansion of the next
                 // step's operands is spread between them
-                f16x8 afn = __builtin_bit_cast(f16x8, rd[lane]);
+                f16x8 ring[PF];
+#pragma unroll
+                for (int j = 0; j < PF; ++j) ring[j] = __builtin_bit_cast(f16x8, rd[j * GLQH_WAVE + lane]);
                 __builtin_amdgcn_sched_barrier(0);              // requests stay ahead of the multiplications
 #pragma unroll
                 for (int k = 0; k < 2 * ET_FRAGS; ++k) {
                     const int u = k / ET_FRAGS, f = k % ET_FRAGS;
-                    const f16x8 af = afn;
-                    if (k + 1 < 2 * ET_FRAGS) afn = __builtin_bit_cast(f16x8, rd[(k + 1) * GLQH_WAVE + lane]);
+                    const f16x8 af = ring[k % PF];
+                    if (k + PF < 2 * ET_FRAGS) ring[k % PF] = __builtin_bit_cast(f16x8, rd[(k + PF) * GLQH_WAVE + lane]);
 #pragma unroll
                     for (int tt = 0; tt < NTW; ++tt)
                         acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(

@@ -32,9 +32,9 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 # one library GEMM (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334) -- is the faster one on this chip,
 # at the price of a transient fp16 copy of the weight.  Whole fused linear, compressed / library,
 # us, on 14336 x 4096 and 4096 x 14336: trellis 172 / 201 and 157 / 204 at 1024 tokens, 353 / 334
-# and 268 / 301 at 2048, 564 / 531 and 488 / 487 at 4096; E8 two-stage 201 / 211 and 196 / 209 at
-# 1024, 400 / 335 and 312 / 327 at 2048, 639 / 552 and 553 / 511 at 4096 (the 14336-row shape pays
-# for 448 and 896 tiles on 256 CUs).  The thresholds are the reference's tunable and its E8
+# and 268 / 301 at 2048, 564 / 531 and 488 / 487 at 4096; E8 two-stage on the indices 201 / 211 and
+# 196 / 209 at 1024, 400 / 335 and 312 / 327 at 2048, 639 / 552 and 553 / 511 at 4096 (the 14336-row
+# shape pays for 448 and 896 tiles on 256 CUs).  The thresholds are the reference's tunable and its E8
 # counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send calls above n tokens to the
 # library route (a large n keeps every call compressed).
 TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "2048")))

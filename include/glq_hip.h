@@ -270,11 +270,12 @@ int glqh_e8_repack_table(const uint32_t *codebook_packed, int64_t n_entries, uin
 /* ---- folded form of the E8 streams (no counterpart in the reference) ---------------------
  * The 65536 codewords of the shell table are built from only 1286 distinct half codewords
  * (columns 0..3 or 4..7, signs included).  A table of those as finished fp16 values (8 bytes
- * each) fits LDS whole, so the small-batch kernel (1..16 tokens) looks every index up without
- * leaving the CU and without expanding anything -- at the price of a second, on-device copy
- * of the index streams: per index two 11-bit half numbers, stored as a 16-bit word plus a
- * byte (3 bytes instead of 2).  Made once per table and per layer at load time; the original
- * indices stay in use for every other route (many tokens, small or ragged layers, decompress). */
+ * each) fits LDS whole, so the small-batch kernel (1..16 tokens) and the many-token tile kernel
+ * (17 tokens and more, n_pad a multiple of 256) look every index up without leaving the CU and
+ * without expanding anything -- at the price of a second, on-device copy of the index streams:
+ * per index two 11-bit half numbers, stored as a 16-bit word plus a byte (3 bytes instead of
+ * 2).  Made once per table and per layer at load time; the original indices stay in use for
+ * every other route (small or ragged layers, decompress + library GEMM, the embedding). */
 typedef struct {
     const uint16_t *lo16[4];     /* per stage, tile order: first half number | (second & 31) << 11 */
     const uint8_t *hi8[4];       /* per stage, tile order: second half number >> 5 */
@@ -295,7 +296,7 @@ int glqh_e8_fold_table(const uint32_t *table, int64_t n_entries, void *halves_ou
                        uint32_t *map_out, int64_t *n_halves_out, void *stream);
 
 /* 1 when a product of this shape and token count reads the folded streams (the LDS-table
- * kernel serves it), 0 when they would go unused. */
+ * kernel or, above 16 tokens, the tile kernel serves it), 0 when they would go unused. */
 int glqh_e8_fold_eligible(int64_t m_pad, int64_t n_pad, int64_t B);
 
 /* Entries of a folded stream of a (rows, cols) index matrix: rows padded to 16, cols to 32. */

@@ -44,6 +44,7 @@ constexpr int ET_THREADS = ET_WAVES * GLQH_WAVE;
 constexpr int ET_FRAGS = 8;                        // 16-row fragments per tile, one per wave
 constexpr int ET_ROWS = 16 * ET_FRAGS;
 constexpr int ET_P = 32767;                        // table entries kept in LDS; word ET_P is a sentinel
+constexpr int ET_SMALL_TOKENS = 64;                // up to here the folded form runs e8_tile_small_kernel
 constexpr uint32_t ET_MISS = 0xFFFFFFFFu;          // no table word has a code above 12
 constexpr int ET_BUF = 2 * ET_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer: 2 sub-steps x 8 fragments
 constexpr size_t ET_LDS = (size_t)(ET_P + 1) * 4 + (size_t)2 * ET_BUF * 16;   // 128 KB + 32 KB
@@ -410,6 +411,178 @@ e8_tile_kernel(const et_args a) {
     }
 }
 
+// 17..64 tokens on the folded streams.  With one token tile per wave every wave of the kernel above reads the
+// whole 16 KB operand buffer of a step from LDS (128 KB per step and workgroup: 1024 LDS cycles for 256-512
+// cycles of multiplications), and at 17..64 tokens most waves multiply padding.  Here the 8 waves split the
+// multiplications of a step by token group AND row fragment: TG = 2 or 4 token groups of 16, wave w takes
+// token group w % TG and the row fragments w / TG + (8 / TG) j, j < TG -- 2 TG operand reads and 2 TG MFMAs per
+// wave and step, every product computed once.  Decoding is as above (wave w decodes row fragment w).
+template <int NS, int TG>
+__global__ void __launch_bounds__(ET_THREADS)
+e8_tile_small_kernel(const et_args a) {
+    constexpr int RG = ET_FRAGS / TG;                          // row-fragment groups
+    extern __shared__ u32x4 lds[];
+    const uint32_t nh1r = (a.nh1 + 1u) & ~1u, nh2r = (a.nh2 + 1u) & ~1u;
+    const uint32_t tab2_off = a.t2_is_t1 ? 0u : 8u * nh1r;     // bytes
+    u32x4 *abuf = lds + (nh1r + (a.t2_is_t1 ? 0u : nh2r)) / 2;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, g = lane >> 4;
+    const int nblk = a.n_pad >> 3, nds = a.n_pad >> 6;
+    const int tg = wave % TG, rg = wave / TG;
+    {
+        uint32_t *tw = (uint32_t *)lds;
+        for (uint32_t j = threadIdx.x; j < 2u * a.nh1; j += ET_THREADS) tw[j] = a.t1[j];
+        if (!a.t2_is_t1)
+            for (uint32_t j = threadIdx.x; j < 2u * a.nh2; j += ET_THREADS) tw[2u * nh1r + j] = a.t2[j];
+    }
+    __syncthreads();
+    f16x2 rs[3];
+#pragma unroll
+    for (int s = 0; s < 3; ++s) rs[s] = f16x2{(f16)a.r[s], (f16)a.r[s]};
+    const char *tb = (const char *)lds;
+
+    const int nitems = a.KS * a.RT;                            // one token tile
+    for (int item = blockIdx.x; item < nitems; item += gridDim.x) {
+        const int rt = item % a.RT, slot = item / a.RT;
+        const int r0 = rt * ET_ROWS;
+        const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
+        const int nquads = (ds1 - ds0) >> 2;
+        const int64_t fbase = (((int64_t)min((r0 >> 4) + wave, ((a.m_pad + 15) >> 4) - 1) * (nblk >> 5) + (ds0 >> 2)) * 64 + lane) * 8;
+        const int64_t kstep = (int64_t)a.Mp * 64;
+        const f16 *xrow = a.xb + (int64_t)(g >> 1) * a.Mp * 32 + (int64_t)(16 * tg + i) * 32 + (g & 1) * 16;
+
+        u32x4 run[NS];
+        u32x2 runb[NS];
+        uint32_t T[NS][4], TB[NS][4];
+        auto load_quad = [&](int q) {
+            q = min(q, nquads - 1);
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                run[s] = __builtin_nontemporal_load((const u32x4 *)(a.q[s] + fbase + (int64_t)q * 512));
+                runb[s] = __builtin_nontemporal_load((const u32x2 *)(a.hi8[s] + fbase + (int64_t)q * 512));
+            }
+        };
+        auto transpose4 = [&](uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3, uint32_t (&O)[4]) {
+            const auto p02 = __builtin_amdgcn_permlane32_swap(d0, d2, false, false);
+            const auto p13 = __builtin_amdgcn_permlane32_swap(d1, d3, false, false);
+            const auto lo = __builtin_amdgcn_permlane16_swap(p02[0], p13[0], false, false);
+            const auto hi = __builtin_amdgcn_permlane16_swap(p02[1], p13[1], false, false);
+            O[0] = lo[0];
+            O[1] = lo[1];
+            O[2] = hi[0];
+            O[3] = hi[1];
+        };
+        auto transpose = [&]() {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                transpose4(run[s][0], run[s][1], run[s][2], run[s][3], T[s]);
+                transpose4(runb[s][0], runb[s][0] >> 16, runb[s][1], runb[s][1] >> 16, TB[s]);
+            }
+        };
+        // the two operand fragments (sub-steps u = 0, 1) of this wave's rows for the step whose index pair is
+        // (T, TB)[.][dd]: looked up, stages combined, written in operand layout
+        auto decode = [&](int dd, u32x4 *dst) {
+            u32x2 c[NS][2][2];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const uint32_t w = T[s][dd], by = TB[s][dd];
+                const char *tbs = tb + (s == 1 ? tab2_off : 0u);
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const uint32_t lo = u ? (w >> 13) & 0x3FF8u : (w << 3) & 0x3FF8u;
+                    const uint32_t h5 = u ? (w >> 24) & 0xF8u : (w >> 8) & 0xF8u;
+                    const uint32_t b6 = u ? by & 0x3F00u : (by << 8) & 0x3F00u;
+                    c[s][u][0] = *(const u32x2 *)(tbs + lo);
+                    c[s][u][1] = *(const u32x2 *)(tbs + (h5 | b6));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                f16x8 af = __builtin_bit_cast(f16x8, u32x4{c[0][u][0][0], c[0][u][0][1], c[0][u][1][0], c[0][u][1][1]});
+#pragma unroll
+                for (int s = 1; s < NS; ++s) {
+                    const f16x8 e = __builtin_bit_cast(f16x8, u32x4{c[s][u][0][0], c[s][u][0][1], c[s][u][1][0], c[s][u][1][1]});
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const f16x2 ev = {e[2 * p], e[2 * p + 1]}, av = {af[2 * p], af[2 * p + 1]};
+                        const f16x2 rv = __builtin_elementwise_fma(ev, rs[s - 1], av);
+                        af[2 * p] = rv[0];
+                        af[2 * p + 1] = rv[1];
+                    }
+                }
+                dst[(u * ET_FRAGS + wave) * GLQH_WAVE + lane] = __builtin_bit_cast(u32x4, af);
+            }
+        };
+        auto load_b = [&](u32x4 (&b)[2], int d) {
+            d = min(d, ds1 - 1);
+            b[0] = *(const u32x4 *)(xrow + d * kstep);
+            b[1] = *(const u32x4 *)(xrow + d * kstep + 8);
+        };
+
+        f32x4 acc[TG];
+#pragma unroll
+        for (int j = 0; j < TG; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // One barrier per group of four steps (256 columns): the operands of a whole group are decoded into one
+        // of two 64 KB buffers while the previous group is multiplied out of the other.  Activations of a group
+        // are requested a group ahead, index runs two groups ahead.
+        u32x4 b[2][4][2];
+        auto load_b4 = [&](u32x4 (&bb)[4][2], int q) {
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) load_b(bb[dd], ds0 + 4 * q + dd);
+        };
+        load_quad(0);
+        load_b4(b[0], 0);
+        transpose();
+        load_quad(1);
+        if (item != (int)blockIdx.x) et_barrier();              // the previous item's last buffer has been read
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) decode(dd, abuf + dd * ET_BUF);
+        et_barrier();
+        for (int q = 0; q < nquads; q += 2) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {                       // group q + h: buffers and registers h
+                if (q + h < nquads) {                           // uniform
+                    const u32x4 *rd = abuf + h * 4 * ET_BUF + rg * GLQH_WAVE + lane;
+                    u32x4 *wr = abuf + (h ^ 1) * 4 * ET_BUF;
+                    load_b4(b[h ^ 1], q + h + 1);
+                    transpose();                                // the next group's indices take over
+                    load_quad(q + h + 2);
+#pragma unroll
+                    for (int dd = 0; dd < 4; ++dd) {
+                        f16x8 af[2 * TG];
+#pragma unroll
+                        for (int k = 0; k < 2 * TG; ++k)        // sub-step k / TG, fragment rg + RG (k % TG)
+                            af[k] = __builtin_bit_cast(f16x8, rd[dd * ET_BUF + ((k / TG) * ET_FRAGS + RG * (k % TG)) * GLQH_WAVE]);
+                        decode(dd, wr + dd * ET_BUF);           // operands of the next group (unused after the last)
+#pragma unroll
+                        for (int k = 0; k < 2 * TG; ++k)
+                            acc[k % TG] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                af[k], __builtin_bit_cast(f16x8, b[h][dd][k / TG]), acc[k % TG], 0, 0, 0);
+                    }
+                    et_barrier();                               // rd has been read, wr is written
+                }
+            }
+        }
+        // lane holds rows 4g .. 4g+3 of token i of every fragment
+        const int tok = 16 * tg + i;
+        if (tok < a.M) {
+            float *orow = a.part + ((int64_t)slot * a.M + tok) * a.m_pad;
+            const bool vec = (a.m_pad & 3) == 0;
+#pragma unroll
+            for (int j = 0; j < TG; ++j) {
+                const int row = r0 + 16 * (rg + RG * j) + 4 * g;
+                if (vec && row + 3 < a.m_pad) {
+                    *(f32x4 *)(orow + row) = acc[j];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (row + e < a.m_pad) orow[row + e] = acc[j][e];
+                }
+            }
+        }
+    }
+}
+
 // (M, n_pad) row-major fp16 -> (n_pad / 32, Mp, 4, 8): 64 tokens x 16 blocks per workgroup through
 // LDS, reads in runs of 256 bytes, writes in runs of 4 KB.
 __global__ void __launch_bounds__(256)
@@ -499,8 +672,23 @@ int et_set_lds(K kernel, size_t bytes) {
                           "e8 tile attribute");
 }
 
+template <int NS, int TG>
+int et_launch_small(const et_plan &p, const et_args &a, hipStream_t stream) {
+    const size_t lds = (size_t)(((a.nh1 + 1u) & ~1u) + (a.t2_is_t1 ? 0u : (a.nh2 + 1u) & ~1u)) * 8 + (size_t)8 * ET_BUF * 16;
+    hipLaunchKernelGGL((e8_tile_small_kernel<NS, TG>), dim3((unsigned)p.grid), dim3(ET_THREADS), lds, stream, a);
+    GLQH_LAUNCH_CHECK("e8 small tile launch");
+    return 0;
+}
+
+template <int NS>
+int et_launch_small_NS(const et_plan &p, const et_args &a, hipStream_t stream) {
+    return a.M <= 32 ? et_launch_small<NS, 2>(p, a, stream) : et_launch_small<NS, 4>(p, a, stream);
+}
+
 template <int NS>
 int et_init_NS() {
+    constexpr size_t small_lds = (size_t)2 * 2048 * 8 + (size_t)8 * ET_BUF * 16;    // 32 KB + 128 KB
+    if (et_set_lds(e8_tile_small_kernel<NS, 2>, small_lds) || et_set_lds(e8_tile_small_kernel<NS, 4>, small_lds)) return 1;
     if (et_set_lds(e8_tile_kernel<NS, 1, false>, ET_LDS) || et_set_lds(e8_tile_kernel<NS, 2, false>, ET_LDS) ||
         et_set_lds(e8_tile_kernel<NS, 1, true>, ET_LDS_FOLD) || et_set_lds(e8_tile_kernel<NS, 2, true>, ET_LDS_FOLD))
         return 1;
@@ -576,6 +764,14 @@ int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const vo
     a.KS = p.KS;
     a.slot_ds = p.slot_ds;
     a.part = part;
+    if (fold && M <= ET_SMALL_TOKENS) {                        // one token tile: TT = 1
+        switch (nstages) {
+        case 1: return et_launch_small_NS<1>(p, a, stream);
+        case 2: return et_launch_small_NS<2>(p, a, stream);
+        case 3: return et_launch_small_NS<3>(p, a, stream);
+        case 4: return et_launch_small_NS<4>(p, a, stream);
+        }
+    }
     switch (nstages * 2 + (fold ? 1 : 0)) {
     case 2: return et_launch_NS<1, false>(p, a, stream);
     case 3: return et_launch_NS<1, true>(p, a, stream);

@@ -44,7 +44,7 @@ constexpr int ET_THREADS = ET_WAVES * GLQH_WAVE;
 constexpr int ET_FRAGS = 8;                        // 16-row fragments per tile, one per wave
 constexpr int ET_ROWS = 16 * ET_FRAGS;
 constexpr int ET_P = 32767;                        // table entries kept in LDS; word ET_P is a sentinel
-constexpr int ET_SMALL_TOKENS = 64;                // up to here the folded form runs e8_tile_small_kernel
+constexpr int ET_SMALL_TOKENS = 256;               // up to here the folded form runs e8_tile_small_kernel
 constexpr uint32_t ET_MISS = 0xFFFFFFFFu;          // no table word has a code above 12
 constexpr int ET_BUF = 2 * ET_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer: 2 sub-steps x 8 fragments
 constexpr size_t ET_LDS = (size_t)(ET_P + 1) * 4 + (size_t)2 * ET_BUF * 16;   // 128 KB + 32 KB
@@ -411,13 +411,14 @@ e8_tile_kernel(const et_args a) {
     }
 }
 
-// 17..64 tokens on the folded streams.  With one token tile per wave every wave of the kernel above reads the
-// whole 16 KB operand buffer of a step from LDS (128 KB per step and workgroup: 1024 LDS cycles for 256-512
-// cycles of multiplications), and at 17..64 tokens most waves multiply padding.  Here the 8 waves split the
-// multiplications of a step by token group AND row fragment: TG = 2 or 4 token groups of 16, wave w takes
-// token group w % TG and the row fragments w / TG + (8 / TG) j, j < TG -- 2 TG operand reads and 2 TG MFMAs per
-// wave and step, every product computed once.  Decoding is as above (wave w decodes row fragment w).
-template <int NS, int TG>
+// 17..256 tokens on the folded streams: one token tile, one barrier per group of four steps.  With one token
+// tile per wave every wave of the kernel above reads the whole 16 KB operand buffer of a step from LDS (128 KB
+// per step and workgroup: 1024 LDS cycles for 256-512 cycles of multiplications), and at 17..64 tokens most
+// waves multiply padding.  Here the 8 waves split the multiplications of a step by token group AND row
+// fragment: TG = 2, 4 or 8 token groups of 16 NTW tokens, wave w takes token group w % TG and the row
+// fragments w / TG + (8 / TG) j, j < TG -- 2 TG operand reads and 2 TG NTW MFMAs per wave and step, every
+// product computed once.  Decoding is as above (wave w decodes row fragment w).
+template <int NS, int TG, int NTW>
 __global__ void __launch_bounds__(ET_THREADS)
 e8_tile_small_kernel(const et_args a) {
     constexpr int RG = ET_FRAGS / TG;                          // row-fragment groups
@@ -449,7 +450,7 @@ e8_tile_small_kernel(const et_args a) {
         const int nquads = (ds1 - ds0) >> 2;
         const int64_t fbase = (((int64_t)min((r0 >> 4) + wave, ((a.m_pad + 15) >> 4) - 1) * (nblk >> 5) + (ds0 >> 2)) * 64 + lane) * 8;
         const int64_t kstep = (int64_t)a.Mp * 64;
-        const f16 *xrow = a.xb + (int64_t)(g >> 1) * a.Mp * 32 + (int64_t)(16 * tg + i) * 32 + (g & 1) * 16;
+        const f16 *xrow = a.xb + (int64_t)(g >> 1) * a.Mp * 32 + (int64_t)(16 * NTW * tg + i) * 32 + (g & 1) * 16;
 
         u32x4 run[NS];
         u32x2 runb[NS];
@@ -513,25 +514,28 @@ e8_tile_small_kernel(const et_args a) {
                 dst[(u * ET_FRAGS + wave) * GLQH_WAVE + lane] = __builtin_bit_cast(u32x4, af);
             }
         };
-        auto load_b = [&](u32x4 (&b)[2], int d) {
+        auto load_b = [&](u32x4 (&b)[NTW][2], int d) {
             d = min(d, ds1 - 1);
-            b[0] = *(const u32x4 *)(xrow + d * kstep);
-            b[1] = *(const u32x4 *)(xrow + d * kstep + 8);
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) {
+                b[tt][0] = *(const u32x4 *)(xrow + d * kstep + tt * 512);
+                b[tt][1] = *(const u32x4 *)(xrow + d * kstep + 8 + tt * 512);
+            }
         };
 
-        f32x4 acc[TG];
+        f32x4 acc[TG][NTW];
 #pragma unroll
-        for (int j = 0; j < TG; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < TG; ++j)
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) acc[j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
         // One barrier per group of four steps (256 columns): the operands of a whole group are decoded into one
-        // of two 64 KB buffers while the previous group is multiplied out of the other.  Activations of a group
-        // are requested a group ahead, index runs two groups ahead.
-        u32x4 b[2][4][2];
-        auto load_b4 = [&](u32x4 (&bb)[4][2], int q) {
-#pragma unroll
-            for (int dd = 0; dd < 4; ++dd) load_b(bb[dd], ds0 + 4 * q + dd);
-        };
+        // of two 64 KB buffers while the previous group is multiplied out of the other.  Activations are
+        // requested three steps ahead (a step is a few hundred cycles, less than an L2 round trip), index runs
+        // two groups ahead.
+        u32x4 b[4][NTW][2];
         load_quad(0);
-        load_b4(b[0], 0);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) load_b(b[j], ds0 + j);
         transpose();
         load_quad(1);
         if (item != (int)blockIdx.x) et_barrier();              // the previous item's last buffer has been read
@@ -544,39 +548,50 @@ e8_tile_small_kernel(const et_args a) {
                 if (q + h < nquads) {                           // uniform
                     const u32x4 *rd = abuf + h * 4 * ET_BUF + rg * GLQH_WAVE + lane;
                     u32x4 *wr = abuf + (h ^ 1) * 4 * ET_BUF;
-                    load_b4(b[h ^ 1], q + h + 1);
                     transpose();                                // the next group's indices take over
                     load_quad(q + h + 2);
 #pragma unroll
                     for (int dd = 0; dd < 4; ++dd) {
-                        f16x8 af[2 * TG];
+                        // operand k of the step: sub-step k / TG, fragment rg + RG (k % TG); read PF ahead
+                        constexpr int NK = 2 * TG, PF = NK < 4 ? NK : 4;
+                        auto frag = [&](int k) {
+                            return __builtin_bit_cast(f16x8, rd[dd * ET_BUF + ((k / TG) * ET_FRAGS + RG * (k % TG)) * GLQH_WAVE]);
+                        };
+                        f16x8 ring[PF];
 #pragma unroll
-                        for (int k = 0; k < 2 * TG; ++k)        // sub-step k / TG, fragment rg + RG (k % TG)
-                            af[k] = __builtin_bit_cast(f16x8, rd[dd * ET_BUF + ((k / TG) * ET_FRAGS + RG * (k % TG)) * GLQH_WAVE]);
+                        for (int k = 0; k < PF; ++k) ring[k] = frag(k);
+                        load_b(b[(dd + 3) & 3], ds0 + 4 * (q + h) + dd + 3);
                         decode(dd, wr + dd * ET_BUF);           // operands of the next group (unused after the last)
 #pragma unroll
-                        for (int k = 0; k < 2 * TG; ++k)
-                            acc[k % TG] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                af[k], __builtin_bit_cast(f16x8, b[h][dd][k / TG]), acc[k % TG], 0, 0, 0);
+                        for (int k = 0; k < NK; ++k) {
+                            const f16x8 af = ring[k % PF];
+                            if (k + PF < NK) ring[k % PF] = frag(k + PF);
+#pragma unroll
+                            for (int tt = 0; tt < NTW; ++tt)
+                                acc[k % TG][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                    af, __builtin_bit_cast(f16x8, b[dd][tt][k / TG]), acc[k % TG][tt], 0, 0, 0);
+                        }
                     }
                     et_barrier();                               // rd has been read, wr is written
                 }
             }
         }
-        // lane holds rows 4g .. 4g+3 of token i of every fragment
-        const int tok = 16 * tg + i;
-        if (tok < a.M) {
+        // lane holds rows 4g .. 4g+3 of token i of every (fragment, token tile)
+        const bool vec = (a.m_pad & 3) == 0;
+#pragma unroll
+        for (int tt = 0; tt < NTW; ++tt) {
+            const int tok = 16 * NTW * tg + 16 * tt + i;
+            if (tok >= a.M) continue;
             float *orow = a.part + ((int64_t)slot * a.M + tok) * a.m_pad;
-            const bool vec = (a.m_pad & 3) == 0;
 #pragma unroll
             for (int j = 0; j < TG; ++j) {
                 const int row = r0 + 16 * (rg + RG * j) + 4 * g;
                 if (vec && row + 3 < a.m_pad) {
-                    *(f32x4 *)(orow + row) = acc[j];
+                    *(f32x4 *)(orow + row) = acc[j][tt];
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        if (row + e < a.m_pad) orow[row + e] = acc[j][e];
+                        if (row + e < a.m_pad) orow[row + e] = acc[j][tt][e];
                 }
             }
         }
@@ -672,23 +687,28 @@ int et_set_lds(K kernel, size_t bytes) {
                           "e8 tile attribute");
 }
 
-template <int NS, int TG>
+template <int NS, int TG, int NTW>
 int et_launch_small(const et_plan &p, const et_args &a, hipStream_t stream) {
     const size_t lds = (size_t)(((a.nh1 + 1u) & ~1u) + (a.t2_is_t1 ? 0u : (a.nh2 + 1u) & ~1u)) * 8 + (size_t)8 * ET_BUF * 16;
-    hipLaunchKernelGGL((e8_tile_small_kernel<NS, TG>), dim3((unsigned)p.grid), dim3(ET_THREADS), lds, stream, a);
+    hipLaunchKernelGGL((e8_tile_small_kernel<NS, TG, NTW>), dim3((unsigned)p.grid), dim3(ET_THREADS), lds, stream, a);
     GLQH_LAUNCH_CHECK("e8 small tile launch");
     return 0;
 }
 
 template <int NS>
 int et_launch_small_NS(const et_plan &p, const et_args &a, hipStream_t stream) {
-    return a.M <= 32 ? et_launch_small<NS, 2>(p, a, stream) : et_launch_small<NS, 4>(p, a, stream);
+    if (a.M <= 32) return et_launch_small<NS, 2, 1>(p, a, stream);
+    if (a.M <= 64) return et_launch_small<NS, 4, 1>(p, a, stream);
+    if (a.M <= 128) return et_launch_small<NS, 8, 1>(p, a, stream);
+    return et_launch_small<NS, 8, 2>(p, a, stream);
 }
 
 template <int NS>
 int et_init_NS() {
     constexpr size_t small_lds = (size_t)2 * 2048 * 8 + (size_t)8 * ET_BUF * 16;    // 32 KB + 128 KB
-    if (et_set_lds(e8_tile_small_kernel<NS, 2>, small_lds) || et_set_lds(e8_tile_small_kernel<NS, 4>, small_lds)) return 1;
+    if (et_set_lds(e8_tile_small_kernel<NS, 2, 1>, small_lds) || et_set_lds(e8_tile_small_kernel<NS, 4, 1>, small_lds) ||
+        et_set_lds(e8_tile_small_kernel<NS, 8, 1>, small_lds) || et_set_lds(e8_tile_small_kernel<NS, 8, 2>, small_lds))
+        return 1;
     if (et_set_lds(e8_tile_kernel<NS, 1, false>, ET_LDS) || et_set_lds(e8_tile_kernel<NS, 2, false>, ET_LDS) ||
         et_set_lds(e8_tile_kernel<NS, 1, true>, ET_LDS_FOLD) || et_set_lds(e8_tile_kernel<NS, 2, true>, ET_LDS_FOLD))
         return 1;

@@ -64,10 +64,22 @@ int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, 
                                   int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
                                   const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
 
-// Plan for activations already in the transformed domain: up to 64 tokens share one pass
+// Plan for activations already in the transformed domain: up to 32 tokens share one pass
 // over the packed stream with K split by shape only; larger batches use the tile kernel, which
-// needs scratch for its repacked activations (xb_bytes).
-#define GLQH_TRELLIS_SMALL_BATCH 64
+// needs scratch for its repacked activations (xb_bytes).  (The small-batch kernel decodes the
+// stream once per 16 tokens; whole linear, us, at 32 / 48 / 64 tokens against the tile kernel at
+// 65: 4096 x 4096 27.2 / 34.7 / 38.3 vs 26.2, 14336 x 4096 42.2 / 55.2 / 57.1 vs 44.5.)
+#define GLQH_TRELLIS_SMALL_BATCH_DEFAULT 32
+// GLQ_TRELLIS_TILE_MIN=<n> (17..65, read once): the tile kernel takes calls of n tokens and more
+static int tr_small_batch() {
+    static const int v = [] {
+        const char *e = getenv("GLQ_TRELLIS_TILE_MIN");
+        const int n = e ? atoi(e) : 0;
+        return n >= 17 && n <= 65 ? n - 1 : GLQH_TRELLIS_SMALL_BATCH_DEFAULT;
+    }();
+    return v;
+}
+#define GLQH_TRELLIS_SMALL_BATCH tr_small_batch()
 struct tr_plan {
     int ks, S, tile;
     size_t xb_bytes;
@@ -274,7 +286,7 @@ extern "C" int glqh_trellis_gemv_partials(const void *x_f16, int64_t B, const vo
     if (tr_bits_from_packed(packed_cols, 1, &R) || tr_check_shape(m, k, packed_rows)) return 1;
     const tr_plan plan = tr_plain_plan(m, k, B);
     const int ks = plan.ks;
-    // above 64 tokens the repacked activations of the tile kernel follow the partial sums
+    // in the tile kernel's range its repacked activations follow the partial sums
     const size_t pbytes = align256((size_t)ks * B * m * sizeof(float));
     const size_t need = plan.tile ? pbytes + plan.xb_bytes : (size_t)ks * B * m * sizeof(float);
     GLQH_REQUIRE(part_bytes >= need, "trellis partials: buffer of %zu bytes needed, got %zu", need, part_bytes);
@@ -400,8 +412,9 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     glqh_meta_args canon_m;
     // The slice kernels of the grouped launcher finish canonical layers faster than the generic
     // transform at every small batch (4096 x 4096 whole linear: 20.7 -> 17.5 us at 8 tokens, 27.5 ->
-    // 23.5 at 24, 41.3 -> 36.5 at 64); tall layers from 32 tokens on take whole blocks instead.
-    const bool canon_out = (B <= 31 || (B <= 64 && m_pad < 8192)) &&
+    // 23.5 at 24); tall layers at 32 tokens, and every layer in the tile kernel's range, take whole
+    // blocks instead (the tile kernel does not pre-scale a second stage's sums).
+    const bool canon_out = (B <= 31 || (B <= GLQH_TRELLIS_SMALL_BATCH && m_pad < 8192)) &&
                            glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
                                                n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
                            canon_m.canon == m_pad;

@@ -720,7 +720,7 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
                (!src.copy_out || (aligned16(src.copy_out) && src.copy_stride % 4 == 0)));
         // whole blocks per workgroup also from 32 tokens on when the rows are many (whole linear,
         // 64 tokens: 11008 x 2048 56.9 -> 45.3 us, 14336 x 4096 70.4 -> 61.6; 2048 x 11008 41.5 -> 43.7)
-        const int64_t Bw = (B >= 32 && m_pad >= 8192) ? 65 : B;
+        const int64_t Bw = ((B >= 32 && m_pad >= 8192) || B > 32) ? 65 : B;
         if (rht_wide_ok(Bw, margs, m_pad, max_bs) && src_ok && aligned16(y) && aligned16(su) &&
             (y_stride * y_size) % 16 == 0) {
             dim3 wgrid((unsigned)n_blocks, (unsigned)B);

@@ -100,13 +100,13 @@ def test_ops_namespace_runs_the_hip_path():
 
 
 @pytest.mark.parametrize("route", ["mfma", "dense"])
-@pytest.mark.parametrize("B", [65, 200, 600])
+@pytest.mark.parametrize("B", [33, 64, 65, 200, 600])
 def test_trellis_many_tokens(B, route, monkeypatch):
-    """More than 64 tokens: the tile kernel over the compressed stream, and the
+    """More than 32 tokens: the tile kernel over the compressed stream, and the
     dequantize-then-GEMM route the reference takes (GLQ_TRELLIS_BATCH_MAX; by default above
     2048 tokens)."""
     from glq_amd import ext, hadamard as H
-    monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 64 if route == "dense" else 1 << 30)
+    monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 32 if route == "dense" else 1 << 30)
     m, n = 256, 512
     say("trellis many tokens", B, route)
     p1, p2 = O.random_packed(m, n, 4, 1), O.random_packed(m, n, 2, 2)

@@ -64,28 +64,30 @@ int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, 
                                   int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
                                   const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
 
-// Plan for activations already in the transformed domain: up to 32 tokens share one pass
-// over the packed stream with K split by shape only; larger batches use the tile kernel, which
-// needs scratch for its repacked activations (xb_bytes).  (The small-batch kernel decodes the
-// stream once per 16 tokens; whole linear, us, at 32 / 48 / 64 tokens against the tile kernel at
-// 65: 4096 x 4096 27.2 / 34.7 / 38.3 vs 26.2, 14336 x 4096 42.2 / 55.2 / 57.1 vs 44.5.)
-#define GLQH_TRELLIS_SMALL_BATCH_DEFAULT 32
+// Plan for activations already in the transformed domain: a small batch shares one pass over
+// the packed stream with K split by shape only; larger batches use the tile kernel, which
+// needs scratch for its repacked activations (xb_bytes).  The small-batch kernel decodes the
+// stream once per 16 tokens, the tile kernel once, at the price of a fixed K step of 64 columns
+// per barrier: it wins from 17 tokens on rows of 4096 columns and more, from 49 tokens on shorter rows
+// (whole linear, us, small-batch / tile kernel: 4096 x 4096 23.5 / 21.3 at 17 tokens, 26.9 / 24.1 at 32,
+// 35.6 / 24.5 at 48, 39.3 / 25.8 at 64; 2048 x 11008 27.3 / 24.9, 30.9 / 27.2, 41.0 / 29.0, 44.5 / 30.6;
+// 2048 x 2048 15.3 / 17.7, 17.1 / 18.0, 19.8 / 19.1, 21.9 / 19.4; 11008 x 2048 31.9 / 40.6, 30.3 / 40.9,
+// 39.1 / 42.7, 42.8 / 43.5).
 // GLQ_TRELLIS_TILE_MIN=<n> (17..65, read once): the tile kernel takes calls of n tokens and more
-static int tr_small_batch() {
+static int tr_small_batch(int64_t k) {
     static const int v = [] {
         const char *e = getenv("GLQ_TRELLIS_TILE_MIN");
         const int n = e ? atoi(e) : 0;
-        return n >= 17 && n <= 65 ? n - 1 : GLQH_TRELLIS_SMALL_BATCH_DEFAULT;
+        return n >= 17 && n <= 65 ? n - 1 : 0;
     }();
-    return v;
+    return v ? v : k >= 4096 ? 16 : 48;
 }
-#define GLQH_TRELLIS_SMALL_BATCH tr_small_batch()
 struct tr_plan {
     int ks, S, tile;
     size_t xb_bytes;
 };
 static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
-    tr_plan p = {1, 0, B > GLQH_TRELLIS_SMALL_BATCH, 0};
+    tr_plan p = {1, 0, B > tr_small_batch(k), 0};
     if (p.tile) {
         p.ks = glqh_trellis_tile_ksplit(m, k, B);
         p.xb_bytes = (glqh_trellis_tile_xb_bytes(k, B) + 255) & ~(size_t)255;
@@ -414,11 +416,11 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     // transform at every small batch (4096 x 4096 whole linear: 20.7 -> 17.5 us at 8 tokens, 27.5 ->
     // 23.5 at 24); tall layers at 32 tokens, and every layer in the tile kernel's range, take whole
     // blocks instead (the tile kernel does not pre-scale a second stage's sums).
-    const bool canon_out = (B <= 31 || (B <= GLQH_TRELLIS_SMALL_BATCH && m_pad < 8192)) &&
+    const bool canon_out = (B <= 31 || (B == 32 && m_pad < 8192)) &&
                            glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
                                                n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
                            canon_m.canon == m_pad;
-    const bool merge2 = has_s2 && canon_out && !(y && y_rht_out);
+    const bool merge2 = has_s2 && canon_out && !(y && y_rht_out) && !tr_plain_plan(m_pad, n_pad, B).tile;
     const float ps2 = merge2 ? (float)inv_resid_scale2 : 1.0f;
 
     // Up to four tokens the input transform is folded into the GEMV launch.  A two-stage layer

@@ -130,6 +130,35 @@ def test_trellis_many_tokens(B, route, monkeypatch):
     assert rel(y[:8], y8.float()) < 5e-3
 
 
+@pytest.mark.parametrize("B", [17, 24, 32, 40])
+def test_trellis_two_stage_tile_kernel_at_few_tokens(B):
+    """Rows of 4096 columns take the tile kernel from 17 tokens on; it does not pre-scale the second
+    stage's sums, so a two-stage layer with canonical output blocks must not be finished as plain K slots."""
+    from glq_amd import ext, hadamard as H
+    m, n = 256, 4096
+    say("trellis two-stage tile route", B)
+    p1, p2 = O.random_packed(m, n, 4, 1), O.random_packed(m, n, 2, 2)
+    su, sv = O.rht_signs(m, n, 42)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"trellis_packed": p1, "trellis_packed2": p2, "inv_resid_scale2": np.float32(0.3),
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
+           "blocks_m": bm, "blocks_n": bn}
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).to(torch.bfloat16)
+    ref = O.trellis_linear_forward(x.float().numpy(), art, n, m)
+    y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), t(p2), torch.tensor(bn), torch.tensor(bm),
+        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), 0.02, 0.3, n, m, n, m,
+        out_dtype=torch.bfloat16)
+    assert y.shape == (B, m) and rel(y, ref) < TOL
+    # single stage through the same route
+    art1 = {k: v for k, v in art.items() if k not in ("trellis_packed2", "inv_resid_scale2")}
+    ref1 = O.trellis_linear_forward(x.float().numpy(), art1, n, m)
+    y1 = ext.glq_fused_linear_trellis_3inst_cuda(
+        x.to(DEV), t(art["SV"]), t(art["SU"]), t(p1), torch.tensor(bn), torch.tensor(bm),
+        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), 0.02, n, m, n, m, out_dtype=torch.bfloat16)
+    assert rel(y1, ref1) < TOL
+
+
 @pytest.mark.parametrize("m,n", [(256, 512), (2048, 2048), (2080, 1152)])
 @pytest.mark.parametrize("K2", [1, 2, 3, 4])
 @pytest.mark.parametrize("B", [1, 3, 6])

@@ -323,7 +323,7 @@ def extras(torch, ext, dev):
 
 
 CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
-         "e8_prefill_256", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
+         "e8_prefill_256", "e8_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 
@@ -347,7 +347,7 @@ def run_case(torch, ext, dev, name, steps):
         o = torch.empty(M, m, dtype=torch.float32, device=dev)
         fn = lambda i: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o)
         res["flop_per_launch"] = 2.0 * M * m * n
-    elif name in ("e8_gemv_2stage", "e8_prefill_4096", "e8_prefill_256"):
+    elif name in ("e8_gemv_2stage", "e8_prefill_4096", "e8_prefill_256", "e8_prefill_32"):
         from glq_amd.checkpoint import load_shell_table
         cb = load_shell_table(None).to(dev)
         m, n = 4096, 14336

@@ -21,6 +21,7 @@ int glqh_viterbi_init(void);
 
 // many-token E8 kernel on the compressed indices (e8_tile.hip)
 int glqh_e8_tile_init(void);
+int glqh_trellis_tile_init(void);
 int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages);
 size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M);
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
@@ -64,30 +65,28 @@ int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, 
                                   int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
                                   const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
 
-// Plan for activations already in the transformed domain: a small batch shares one pass over
-// the packed stream with K split by shape only; larger batches use the tile kernel, which
-// needs scratch for its repacked activations (xb_bytes).  The small-batch kernel decodes the
-// stream once per 16 tokens, the tile kernel once, at the price of a fixed K step of 64 columns
-// per barrier: it wins from 17 tokens on rows of 4096 columns and more, from 49 tokens on shorter rows
-// (whole linear, us, small-batch / tile kernel: 4096 x 4096 23.5 / 21.3 at 17 tokens, 26.9 / 24.1 at 32,
-// 35.6 / 24.5 at 48, 39.3 / 25.8 at 64; 2048 x 11008 27.3 / 24.9, 30.9 / 27.2, 41.0 / 29.0, 44.5 / 30.6;
-// 2048 x 2048 15.3 / 17.7, 17.1 / 18.0, 19.8 / 19.1, 21.9 / 19.4; 11008 x 2048 31.9 / 40.6, 30.3 / 40.9,
-// 39.1 / 42.7, 42.8 / 43.5).
-// GLQ_TRELLIS_TILE_MIN=<n> (17..65, read once): the tile kernel takes calls of n tokens and more
-static int tr_small_batch(int64_t k) {
+// Plan for activations already in the transformed domain: up to 16 tokens share one pass over
+// the packed stream with K split by shape only; larger batches use the tile kernels, which
+// need scratch for their repacked activations (xb_bytes).  The small-batch kernel decodes the
+// stream once per 16 tokens, the tile kernels once (whole linear, us, small-batch / tile kernel:
+// 4096 x 4096 23.5 / 19.8 at 17 tokens, 26.9 / 21.2 at 32, 35.6 / 24.1 at 48, 39.3 / 25.4 at 64;
+// 2048 x 11008 27.3 / 23.2, 30.9 / 25.1, 41.0 / 30.6, 44.5 / 31.8; 11008 x 2048 32.0 / 24.0, 30.2 / 24.5,
+// 38.6 / 27.2, 42.8 / 28.0; 2048 x 2048 15.3 / 16.6, 16.9 / 16.3, 22.2 / 18.3, 21.9 / 18.9).
+// GLQ_TRELLIS_TILE_MIN=<n> (17..65, read once): the tile kernels take calls of n tokens and more
+static int tr_small_batch() {
     static const int v = [] {
         const char *e = getenv("GLQ_TRELLIS_TILE_MIN");
         const int n = e ? atoi(e) : 0;
-        return n >= 17 && n <= 65 ? n - 1 : 0;
+        return n >= 17 && n <= 65 ? n - 1 : 16;
     }();
-    return v ? v : k >= 4096 ? 16 : 48;
+    return v;
 }
 struct tr_plan {
     int ks, S, tile;
     size_t xb_bytes;
 };
 static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
-    tr_plan p = {1, 0, B > tr_small_batch(k), 0};
+    tr_plan p = {1, 0, B > tr_small_batch(), 0};
     if (p.tile) {
         p.ks = glqh_trellis_tile_ksplit(m, k, B);
         p.xb_bytes = (glqh_trellis_tile_xb_bytes(k, B) + 255) & ~(size_t)255;
@@ -187,7 +186,7 @@ extern "C" int glqh_init(void) {
             return;
         }
         g_cus = prop.multiProcessorCount;
-        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_e8_tile_init() || glqh_trellis_init() || glqh_trellis_mma_init() || glqh_viterbi_init();
+        g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_e8_tile_init() || glqh_trellis_init() || glqh_trellis_tile_init() || glqh_trellis_mma_init() || glqh_viterbi_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
     return g_init_rc;

@@ -223,6 +223,180 @@ tr_tile_kernel(const tt_args a) {
     }
 }
 
+// Up to 64 tokens: one barrier per group of four steps instead of one per step, and the eight waves split a
+// step's products by token group AND row fragment.  With one token tile per wave
+// every wave of the kernel above reads the whole 16 KB operand buffer of a step (128 KB per step and workgroup:
+// 1024 LDS cycles for 256-512 cycles of multiplications) and below 128 tokens most waves multiply padding.
+// Here: TG = 2 or 4 token groups of 16 NTW tokens; wave w takes token group w % TG and the operands
+// w / TG + (8 / TG) j, j < TG, of each half-step -- 2 TG operand reads and 2 TG NTW MFMAs per wave and step,
+// every product computed once.  The operands of a whole group of four steps (256 columns) are decoded into one
+// of two 64 KB buffers while the previous group is multiplied out of the other; decoding is as above (wave w:
+// block pair w >> 2, k-pair (w >> 1) & 1, m-tile w & 1).  Same K slots and order of summation as above.
+constexpr size_t TT_SMALL_LDS = (size_t)8 * TT_BUF * 16;       // 128 KB
+
+template <int R, int TG, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_small_kernel(const tt_args a) {
+    constexpr int RG = TT_FRAGS / TG;                          // operand groups
+    extern __shared__ u32x4 abuf[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, q = lane >> 4;
+    const int nkp = a.k >> 5, nds = a.k >> 6, mpairs = a.m >> 5;
+    constexpr int REC = 4 * R;
+    const int tg = wave % TG, rg = wave / TG;
+
+    // decode role
+    const int unit = wave >> 2, kpi = (wave >> 1) & 1, ms = wave & 1;
+    const int hm = i >> 3, l = 4 * (i & 7) + q;
+    const int l1 = (l + 1) & 31, l2 = (l + 2) & 31;
+    const int next1 = 16 * (l1 & 3) + 8 * hm + (l1 >> 2), next2 = 16 * (l2 & 3) + 8 * hm + (l2 >> 2);
+
+    const int nitems = a.KS * a.RT;                            // one token tile
+    for (int item = blockIdx.x; item < nitems; item += gridDim.x) {
+        const int rt = item % a.RT, slot = item / a.RT;
+        const int r0 = rt * TT_ROWS;
+        const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
+        const int nquads = (ds1 - ds0 + 3) >> 2;
+
+        const int mp = min(2 * (2 * rt + unit) + hm, mpairs - 1);
+        const uint8_t *rec_base = a.packed + ((int64_t)mp * nkp * 32 + l) * REC + (int64_t)kpi * 32 * REC;
+        auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
+            return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
+        };
+        // two operands (row groups 2 ms, 2 ms + 1 of the 64-row unit) from half a record
+        auto emit = [&](const tr_record<R> r, u32x4 *dst) {
+            uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
+            uint32_t n0, n1;
+            if constexpr (R >= 2) {
+                constexpr int sh = 8 * R - 16;
+                const uint32_t t = ((c0 >> sh) & 0xFFFFu) | (((c1 >> sh) & 0xFFFFu) << 16);
+                const uint32_t n = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
+                n0 = n & 0xFFFFu;
+                n1 = n >> 16;
+            } else {
+                const uint32_t t = c0 | (c1 << 8);
+                const uint32_t x1 = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
+                const uint32_t x2 = (uint32_t)__shfl((int)t, next2, GLQH_WAVE);
+                n0 = ((x1 & 0xFFu) << 8) | (x2 & 0xFFu);
+                n1 = (x1 & 0xFF00u) | ((x2 >> 8) & 0xFFu);
+            }
+            uint32_t h0[8], h1[8];                              // k-tiles 0 and 1 of m-tile ms
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                h0[j] = tr_hash(tr_state<R>(c0, n0, j));
+                h1[j] = tr_hash(tr_state<R>(c1, n1, j));
+            }
+#pragma unroll
+            for (int rh = 0; rh < 2; ++rh) {
+                const int j0 = 2 * rh;
+                const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1],
+                                           h1[j0 + 4], h1[j0 + 5]);
+                dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
+            }
+        };
+        // multiply role: token 16 * tt + i of the wave's token group
+        const int64_t bstep = (int64_t)a.Mp * 32;               // elements from one k-pair to the next
+        const f16 *xrow = a.xb + (int64_t)(16 * NTW * tg + i) * 32 + q * 8;
+        auto load_b = [&](u32x4 (&bb)[NTW][2], int d) {
+            d = min(d, ds1 - 1);
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) {
+                bb[tt][0] = *(const u32x4 *)(xrow + 2 * d * bstep + tt * 512);
+                bb[tt][1] = *(const u32x4 *)(xrow + (2 * d + 1) * bstep + tt * 512);
+            }
+        };
+
+        f32x4 acc[TG][NTW];
+#pragma unroll
+        for (int j = 0; j < TG; ++j)
+#pragma unroll
+            for (int tt = 0; tt < NTW; ++tt) acc[j][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        // records of a group arrive a group ahead, activations three steps ahead (a step is a few hundred
+        // cycles, less than an L2 round trip)
+        tr_record<R> rc[4], rn[4];
+        u32x4 b[4][NTW][2];
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) rc[dd] = load_rec(ds0 + dd);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) load_b(b[j], ds0 + j);
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) rn[dd] = load_rec(ds0 + 4 + dd);
+        if (item != (int)blockIdx.x) tt_barrier();              // the previous item's last buffer has been read
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) emit(rc[dd], abuf + dd * TT_BUF);
+        tt_barrier();
+        for (int qd = 0; qd < nquads; qd += 2) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {                       // group qd + h: buffer h
+                if (qd + h < nquads) {                          // uniform
+                    const int d0 = ds0 + 4 * (qd + h);
+                    const u32x4 *rd = abuf + h * 4 * TT_BUF + rg * GLQH_WAVE + lane;
+                    u32x4 *wr = abuf + (h ^ 1) * 4 * TT_BUF;
+#pragma unroll
+                    for (int dd = 0; dd < 4; ++dd) {
+                        rc[dd] = rn[dd];
+                        rn[dd] = load_rec(d0 + 8 + dd);
+                    }
+#pragma unroll
+                    for (int dd = 0; dd < 4; ++dd) {
+                        // operand kk of the step: half-step kk / TG, operand rg + RG (kk % TG); read PF ahead
+                        constexpr int NK = 2 * TG, PF = NK < 4 ? NK : 4;
+                        auto frag = [&](int kk) {
+                            return __builtin_bit_cast(f16x8, rd[dd * TT_BUF + ((kk / TG) * TT_FRAGS + RG * (kk % TG)) * GLQH_WAVE]);
+                        };
+                        f16x8 ring[PF];
+#pragma unroll
+                        for (int kk = 0; kk < PF; ++kk) ring[kk] = frag(kk);
+                        load_b(b[(dd + 3) & 3], d0 + dd + 3);
+                        emit(rc[dd], wr + dd * TT_BUF);         // operands of the next group (unused after the last)
+                        if (d0 + dd < ds1) {                    // uniform: a slot need not be whole groups
+#pragma unroll
+                            for (int kk = 0; kk < NK; ++kk) {
+                                const f16x8 af = ring[kk % PF];
+                                if (kk + PF < NK) ring[kk % PF] = frag(kk + PF);
+#pragma unroll
+                                for (int tt = 0; tt < NTW; ++tt)
+                                    acc[kk % TG][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                        af, __builtin_bit_cast(f16x8, b[dd][tt][kk / TG]), acc[kk % TG][tt], 0, 0, 0);
+                            }
+                        }
+                    }
+                    tt_barrier();                               // rd has been read, wr is written
+                }
+            }
+        }
+
+        // lane holds four consecutive rows of token i for every (operand, token tile): operand
+        // f = 4 unit' + s covers rows 64 unit' + 32 h + 8 s + (0..7), h = 0, 1
+        const int rlane = 32 * (q >> 1) + 4 * (q & 1);
+#pragma unroll
+        for (int tt = 0; tt < NTW; ++tt) {
+            const int tok = 16 * NTW * tg + 16 * tt + i;
+            if (tok >= a.M) continue;
+#pragma unroll
+            for (int j = 0; j < TG; ++j) {
+                const int f = rg + RG * j;
+                const int row = r0 + 64 * (f >> 2) + 8 * (f & 3) + rlane;
+                if (row >= a.m) continue;                       // m is a multiple of 32: whole groups of four
+                if (!a.direct) {
+                    *(f32x4 *)(a.out + ((int64_t)slot * a.M + tok) * a.m + row) = acc[j][tt];
+                } else {
+                    float *o = a.out + (int64_t)tok * a.out_stride + row;
+                    if ((a.out_stride & 3) == 0) {
+                        f32x4 v = acc[j][tt] * a.scale;
+                        if (a.accum) v += *(f32x4 *)o;
+                        *(f32x4 *)o = v;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = a.accum ? o[e] + acc[j][tt][e] * a.scale : acc[j][tt][e] * a.scale;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // (M, k) row-major fp16 -> xb[k-pair][token][q][8]: slot q of a k-pair takes columns
 // 2q + {0,1,8,9,16,17,24,25}, i.e. dword q of each of its four 16-byte items.  64 tokens x 4
 // k-pairs per workgroup through LDS; reads in runs of 256 bytes, writes in runs of 4 KB.
@@ -290,14 +464,39 @@ int tt_launch(const tt_plan &p, const tt_args &a, hipStream_t stream) {
     return 0;
 }
 
+template <int R, int TG, int NTW>
+int tt_launch_small(const tt_plan &p, const tt_args &a, hipStream_t stream) {
+    hipLaunchKernelGGL((tr_tile_small_kernel<R, TG, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_SMALL_LDS, stream, a);
+    GLQH_LAUNCH_CHECK("trellis small tile launch");
+    return 0;
+}
+
 template <int R>
 int tt_launch_R(const tt_plan &p, const tt_args &a, hipStream_t stream) {
+    // (with eight token groups, 65..256 tokens, the kernel above is as fast or faster: whole linear 4096 x 4096
+    // 30.8 against 33.1 us at 128 tokens, 4096 x 14336 57.2 against 62.6 at 256)
+    if (a.M <= 32) return tt_launch_small<R, 2, 1>(p, a, stream);
+    if (a.M <= 64) return tt_launch_small<R, 4, 1>(p, a, stream);
     if (p.NTW == 1) return tt_launch<R, 1>(p, a, stream);
     if (p.NTW == 2) return tt_launch<R, 2>(p, a, stream);
     return tt_launch<R, 4>(p, a, stream);
 }
 
+template <typename K>
+int tt_set_lds(K kernel) {
+    return glqh_check_hip(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              (int)TT_SMALL_LDS),
+                          "trellis tile attribute");
+}
+
+template <int R>
+int tt_init_R() {
+    return tt_set_lds(tr_tile_small_kernel<R, 2, 1>) || tt_set_lds(tr_tile_small_kernel<R, 4, 1>);
+}
+
 }  // namespace
+
+int glqh_trellis_tile_init(void) { return tt_init_R<1>() || tt_init_R<2>() || tt_init_R<3>() || tt_init_R<4>(); }
 
 // bytes of the repacked activations of a many-token call
 size_t glqh_trellis_tile_xb_bytes(int64_t k, int64_t M) { return (size_t)tt_padded_tokens(M) * k * sizeof(f16); }

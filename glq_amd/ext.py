@@ -25,7 +25,7 @@ from ._lib import GLQH_BF16, GLQH_F16, GLQH_F32, check
 
 _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F32}
 
-# Small and medium token counts are served on the compressed weights: 1-16 tokens (trellis on short rows: 1-48) by the GEMV /
+# Small and medium token counts are served on the compressed weights: 1-16 tokens by the GEMV /
 # small-batch kernels, above by the tile kernels that decode each weight once per 128-row x
 # 512-token tile (csrc/trellis_tile.hip, csrc/e8_tile.hip).  From a few thousand tokens on the
 # reference's own many-token route -- dequantize the weight to fp16 once with the HIP kernel, then

@@ -68,8 +68,7 @@ int glqh_decode_matmul_trellis_3inst(const void *x_f16, int64_t B,
  * For callers that fold the fixed-order reduction into their own consumer (as the fused
  * linear does) and for timing the decode kernel in isolation.  The reference has no
  * separate entry for this step (its GEMV reduces inside the block,
- * glq/csrc/glq_trellis.cu:485-510).  From 17 tokens on (49 on rows shorter than 4096 columns; or
- * GLQ_TRELLIS_TILE_MIN) the many-token kernel keeps its repacked
+ * glq/csrc/glq_trellis.cu:485-510).  From 17 tokens on (GLQ_TRELLIS_TILE_MIN) the many-token kernels keep their repacked
  * activations behind the partial sums: part_bytes must then cover
  * glqh_trellis_gemv_workspace_bytes(m, k, B) (the sums rounded up to 256 bytes + that copy). */
 int glqh_trellis_gemv_partials(const void *x_f16, int64_t B,

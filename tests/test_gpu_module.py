@@ -100,13 +100,13 @@ def test_ops_namespace_runs_the_hip_path():
 
 
 @pytest.mark.parametrize("route", ["mfma", "dense"])
-@pytest.mark.parametrize("B", [33, 64, 65, 200, 600])
+@pytest.mark.parametrize("B", [17, 33, 64, 65, 200, 600])
 def test_trellis_many_tokens(B, route, monkeypatch):
-    """More than 32 tokens: the tile kernel over the compressed stream, and the
+    """More than 16 tokens: the tile kernels over the compressed stream, and the
     dequantize-then-GEMM route the reference takes (GLQ_TRELLIS_BATCH_MAX; by default above
     2048 tokens)."""
     from glq_amd import ext, hadamard as H
-    monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 32 if route == "dense" else 1 << 30)
+    monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 16 if route == "dense" else 1 << 30)
     m, n = 256, 512
     say("trellis many tokens", B, route)
     p1, p2 = O.random_packed(m, n, 4, 1), O.random_packed(m, n, 2, 2)
@@ -132,7 +132,7 @@ def test_trellis_many_tokens(B, route, monkeypatch):
 
 @pytest.mark.parametrize("B", [17, 24, 32, 40])
 def test_trellis_two_stage_tile_kernel_at_few_tokens(B):
-    """Rows of 4096 columns take the tile kernel from 17 tokens on; it does not pre-scale the second
+    """From 17 tokens on the tile kernels run; they do not pre-scale the second
     stage's sums, so a two-stage layer with canonical output blocks must not be finished as plain K slots."""
     from glq_amd import ext, hadamard as H
     m, n = 256, 4096

@@ -302,6 +302,13 @@ def extras(torch, ext, dev):
                 out_dtype=torch.bfloat16), 1, reps=5)
             out[f"e8_2stage_linear_14336x4096_M{M}{route}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
         ext.TRELLIS_BATCH_MAX, ext.E8_BATCH_MAX = tr_default, e8_default
+        # the same two linears at 32 tokens (a batched decode step): the small-tile kernels
+        xb = torch.randn(32, n, device=dev).to(torch.bfloat16)
+        out["trellis_linear_14336x4096_M32_us"] = round(_graph_time(torch, lambda: ext.glq_fused_linear_trellis_3inst_cuda(
+            xb, sv, su, p, bnt, bmt, bnm, bmm, 0.02, n, m, n, m, out_dtype=torch.bfloat16), 1, reps=10), 1)
+        out["e8_2stage_linear_14336x4096_M32_us"] = round(_graph_time(torch, lambda: ext.glq_fused_linear_block_diag_cuda(
+            xb, sv, su, q1, cbh, 0.02, n, m, n, m, bnt, bmt, bnm, bmm, q2, cbh, 1 / 3.0,
+            out_dtype=torch.bfloat16), 1, reps=10), 1)
         del p, q1, q2
         torch.cuda.empty_cache()
     except Exception as e:

@@ -134,7 +134,7 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
 
 
 @pytest.mark.parametrize("m,n,B", [(1000, 2048, 17), (2048, 1024, 40), (520, 4096, 64), (1024, 2048, 100), (4096, 1024, 130),
-                                   (2048, 4096, 300), (1536, 2560, 520)])
+                                   (2048, 4096, 300), (1000, 1024, 300), (1536, 2560, 520)])
 @pytest.mark.parametrize("stages", [1, 2, 3, 4])
 def test_many_token_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stages):
     """Above 16 tokens the tile kernel reads the folded streams too: same tiles, same K slots, same fp16

@@ -330,7 +330,7 @@ def extras(torch, ext, dev):
 
 
 CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
-         "e8_prefill_256", "e8_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
+         "e8_prefill_256", "e8_prefill_32", "trellis_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 
@@ -347,7 +347,7 @@ def run_case(torch, ext, dev, name, steps):
         pb = torch.empty(64 * m, dtype=torch.float32, device=dev)
         fn = lambda i: ext.trellis_gemv_partials(xh, packs[i % 4], m, n, pb)
         res["bytes_per_launch"] = m * n // 2
-    elif name in ("trellis_prefill_4096", "trellis_prefill_256"):
+    elif name in ("trellis_prefill_4096", "trellis_prefill_256", "trellis_prefill_32"):
         m, n, M = 14336, 4096, int(name.rsplit("_", 1)[1])
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
         xh = torch.randn(M, n, device=dev).to(torch.float16)

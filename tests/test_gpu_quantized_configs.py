@@ -236,7 +236,7 @@ def test_trellis_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatc
     xd = x.to(DEV)
     Ws = (W_dec * art["Wscale"]).astype(np.float32)
     ys = {}
-    for M in (256, 1024, 4096):
+    for M in (24, 64, 256, 1024, 4096):                       # 24, 64: the small-tile kernel
         rows = _sample_rows(M)
         ref = O.linear_forward_rht(x[rows].float().numpy(), Ws, su, sv, art["blocks_n"], art["blocks_m"], n, m)
         y = ext.glq_fused_linear_trellis_3inst_cuda(xd[:M], *args, out_dtype=torch.bfloat16)
@@ -247,6 +247,8 @@ def test_trellis_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatc
     # every row of the 4096-token call against the 1024-token call (other route or other K split)
     assert rel(ys[4096][:1024], ys[1024].float().cpu().numpy()) < 6e-3
     assert rel(ys[1024][:256], ys[256].float().cpu().numpy()) < 6e-3
+    assert rel(ys[256][:64], ys[64].float().cpu().numpy()) < 6e-3
+    assert rel(ys[64][:24], ys[24].float().cpu().numpy()) < 6e-3
     # the reference's quality gate at the full prefill size
     W_hat = to_weight_domain(Ws, su, sv, art["blocks_m"], art["blocks_n"])
     rows = _sample_rows(4096)
@@ -269,7 +271,7 @@ def test_e8_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatch):
     xd = x.to(DEV)
     Ws = (W_dec * art["Wscale"]).astype(np.float32)
     ys = {}
-    for M in (64, 256, 1024, 4096):
+    for M in (24, 64, 256, 1024, 4096):                       # up to 256: the small-tile kernel
         rows = _sample_rows(M)
         ref = O.linear_forward_rht(x[rows].float().numpy(), Ws, su, sv, art["blocks_n"], art["blocks_m"], n, m)
         y = e8_forward(ext, xd[:M], art, m, n, torch.bfloat16)

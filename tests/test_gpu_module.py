@@ -281,6 +281,48 @@ def test_graph_capture_and_replay_is_bit_exact():
     assert torch.equal(y, layer(xs))
 
 
+@pytest.mark.parametrize("B", [24, 48, 200])
+def test_graph_capture_of_a_batched_step_on_the_tile_kernels(B):
+    """17 tokens and more run the tile kernels (small-tile kernels up to 64 tokens, E8 on its folded streams):
+    captured after a warm-up call, every replay equals the eager result bit for bit."""
+    from glq_amd import ext, hadamard as H
+    m, n = 512, 2048
+    p = t(O.random_packed(m, n, 4, 11))
+    su, sv = O.rht_signs(m, n, 3)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    meta = (torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV))
+    svt, sut = t(sv.astype(np.float16)), t(su.astype(np.float16))
+    rng = np.random.default_rng(B)
+    q1, q2 = (t(rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16)) for _ in range(2))
+    cb = e8_table_f16()
+    xs = torch.randn(B, n, device=DEV).to(torch.bfloat16)
+
+    def step():
+        return (ext.glq_fused_linear_trellis_3inst_cuda(xs, svt, sut, p, *meta, 0.02, n, m, n, m, out_dtype=torch.bfloat16),
+                ext.glq_fused_linear_block_diag_cuda(xs, svt, sut, q1, cb, 0.02, n, m, n, m, *meta, q2, cb, 1 / 3.0,
+                                                     out_dtype=torch.bfloat16))
+    eager = [y.clone() for y in step()]                       # also makes the folded streams
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            ys = step()
+    torch.cuda.synchronize()
+    for i in range(3):
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ys[0], eager[0]) and torch.equal(ys[1], eager[1]), f"replay {i}"
+        step()                                                # eager work in between
+        torch.cuda.synchronize()
+    xs.copy_(torch.randn(B, n, device=DEV).to(torch.bfloat16))  # new input, same graph
+    g.replay()
+    torch.cuda.synchronize()
+    again = step()
+    assert torch.equal(ys[0], again[0]) and torch.equal(ys[1], again[1])
+
+
 def _two_stage_module(m, n, seed):
     from glq_amd.quantized_linear import E8RHTLinear
     p1, p2 = O.random_packed(m, n, 4, seed), O.random_packed(m, n, 2, seed + 1)

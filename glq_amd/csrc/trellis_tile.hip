@@ -53,6 +53,45 @@ __device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Decode role of a wave in both tile kernels: from half a record (block pair `unit` of the tile, k-pair `kpi` of the
+// step, m-tile `ms`) the two A operands of row groups 2 ms and 2 ms + 1, the two fp16 halves of every weight added
+// first (the dequantizer's rounding), written in operand layout (lane L's 16 bytes at slot L of operand
+// kpi * 8 + unit * 4 + 2 ms + rh).  half = -1: both operands; 0 / 1: operand rh = half only.
+template <int R>
+__device__ __forceinline__ void tt_emit(const tr_record<R> &r, int unit, int kpi, int ms, int next1, int next2, int lane,
+                                        u32x4 *dst, int half = -1) {
+    uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
+    uint32_t n0, n1;
+    if constexpr (R >= 2) {
+        constexpr int sh = 8 * R - 16;
+        const uint32_t t = ((c0 >> sh) & 0xFFFFu) | (((c1 >> sh) & 0xFFFFu) << 16);
+        const uint32_t n = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
+        n0 = n & 0xFFFFu;
+        n1 = n >> 16;
+    } else {
+        const uint32_t t = c0 | (c1 << 8);
+        const uint32_t x1 = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
+        const uint32_t x2 = (uint32_t)__shfl((int)t, next2, GLQH_WAVE);
+        n0 = ((x1 & 0xFFu) << 8) | (x2 & 0xFFu);
+        n1 = (x1 & 0xFF00u) | ((x2 >> 8) & 0xFFu);
+    }
+    uint32_t h0[8], h1[8];                                      // k-tiles 0 and 1 of m-tile ms
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if (half >= 0 && ((j >> 1) & 1) != half) continue;      // operand rh takes states 2rh, 2rh+1, 2rh+4, 2rh+5
+        h0[j] = tr_hash(tr_state<R>(c0, n0, j));
+        h1[j] = tr_hash(tr_state<R>(c1, n1, j));
+    }
+#pragma unroll
+    for (int rh = 0; rh < 2; ++rh) {
+        if (half >= 0 && rh != half) continue;
+        const int j0 = 2 * rh;
+        const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1], h1[j0 + 4],
+                                   h1[j0 + 5]);
+        dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
+    }
+}
+
 template <int R, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_kernel(const tt_args a) {
@@ -84,39 +123,8 @@ tr_tile_kernel(const tt_args a) {
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
-        // two operands (row groups 2 ms, 2 ms + 1 of the 64-row unit) from half a record
-        // half = -1: both operands; 0 / 1: operand rh = half only (the step's two halves each decode one)
         auto emit = [&](const tr_record<R> &r, u32x4 *dst, int half = -1) {
-            uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
-            uint32_t n0, n1;
-            if constexpr (R >= 2) {
-                constexpr int sh = 8 * R - 16;
-                const uint32_t t = ((c0 >> sh) & 0xFFFFu) | (((c1 >> sh) & 0xFFFFu) << 16);
-                const uint32_t n = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
-                n0 = n & 0xFFFFu;
-                n1 = n >> 16;
-            } else {
-                const uint32_t t = c0 | (c1 << 8);
-                const uint32_t x1 = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
-                const uint32_t x2 = (uint32_t)__shfl((int)t, next2, GLQH_WAVE);
-                n0 = ((x1 & 0xFFu) << 8) | (x2 & 0xFFu);
-                n1 = (x1 & 0xFF00u) | ((x2 >> 8) & 0xFFu);
-            }
-            uint32_t h0[8], h1[8];                              // k-tiles 0 and 1 of m-tile ms
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                if (half >= 0 && ((j >> 1) & 1) != half) continue;   // operand rh takes states 2rh, 2rh+1, 2rh+4, 2rh+5
-                h0[j] = tr_hash(tr_state<R>(c0, n0, j));
-                h1[j] = tr_hash(tr_state<R>(c1, n1, j));
-            }
-#pragma unroll
-            for (int rh = 0; rh < 2; ++rh) {
-                if (half >= 0 && rh != half) continue;
-                const int j0 = 2 * rh;
-                const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1],
-                                           h1[j0 + 4], h1[j0 + 5]);
-                dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
-            }
+            tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst, half);
         };
         // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(kp * Mp + token) * 4 + q]
         // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
@@ -263,37 +271,7 @@ tr_tile_small_kernel(const tt_args a) {
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
-        // two operands (row groups 2 ms, 2 ms + 1 of the 64-row unit) from half a record
-        auto emit = [&](const tr_record<R> r, u32x4 *dst) {
-            uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
-            uint32_t n0, n1;
-            if constexpr (R >= 2) {
-                constexpr int sh = 8 * R - 16;
-                const uint32_t t = ((c0 >> sh) & 0xFFFFu) | (((c1 >> sh) & 0xFFFFu) << 16);
-                const uint32_t n = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
-                n0 = n & 0xFFFFu;
-                n1 = n >> 16;
-            } else {
-                const uint32_t t = c0 | (c1 << 8);
-                const uint32_t x1 = (uint32_t)__shfl((int)t, next1, GLQH_WAVE);
-                const uint32_t x2 = (uint32_t)__shfl((int)t, next2, GLQH_WAVE);
-                n0 = ((x1 & 0xFFu) << 8) | (x2 & 0xFFu);
-                n1 = (x1 & 0xFF00u) | ((x2 >> 8) & 0xFFu);
-            }
-            uint32_t h0[8], h1[8];                              // k-tiles 0 and 1 of m-tile ms
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                h0[j] = tr_hash(tr_state<R>(c0, n0, j));
-                h1[j] = tr_hash(tr_state<R>(c1, n1, j));
-            }
-#pragma unroll
-            for (int rh = 0; rh < 2; ++rh) {
-                const int j0 = 2 * rh;
-                const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1],
-                                           h1[j0 + 4], h1[j0 + 5]);
-                dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
-            }
-        };
+        auto emit = [&](const tr_record<R> r, u32x4 *dst) { tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst); };
         // multiply role: token 16 * tt + i of the wave's token group
         const int64_t bstep = (int64_t)a.Mp * 32;               // elements from one k-pair to the next
         const f16 *xrow = a.xb + (int64_t)(16 * NTW * tg + i) * 32 + q * 8;

@@ -299,9 +299,9 @@ e8_tile_kernel(const et_args a) {
         // four steps ahead.
         constexpr int LA = NTW <= 2 ? 2 : 1;
         // operand fragments read ahead of their multiplications: with one or two token tiles per wave a
-        // fragment is multiplied in 16-32 matrix-pipe cycles, less than an LDS read takes (1-3 % per call);
-        // two ahead also with four token tiles where the registers allow it (folded form: 3-4 % at 4096 tokens)
-        constexpr int PF = (NTW <= 2 || FOLD) ? 2 : 1;
+        // fragment is multiplied in 16-32 matrix-pipe cycles, less than an LDS read takes; with four token
+        // tiles two ahead changes nothing (527 against 525 us at 4096 tokens, one run) and costs registers
+        constexpr int PF = NTW <= 2 ? 2 : 1;
         constexpr bool BDB = NTW <= 2;
         u32x4 run[NS];
         u32x2 runb[NFB];

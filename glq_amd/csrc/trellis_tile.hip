@@ -452,7 +452,7 @@ int tt_launch_small(const tt_plan &p, const tt_args &a, hipStream_t stream) {
 template <int R>
 int tt_launch_R(const tt_plan &p, const tt_args &a, hipStream_t stream) {
     // (with eight token groups, 65..256 tokens, the kernel above is as fast or faster: whole linear 4096 x 4096
-    // 30.8 against 33.1 us at 128 tokens, 4096 x 14336 57.2 against 62.6 at 256)
+    // 31.4 against 33.3 us at 128 tokens, 4096 x 14336 59.7 against 64.4 at 256, both in one run)
     if (a.M <= 32) return tt_launch_small<R, 2, 1>(p, a, stream);
     if (a.M <= 64) return tt_launch_small<R, 4, 1>(p, a, stream);
     if (p.NTW == 1) return tt_launch<R, 1>(p, a, stream);

@@ -101,8 +101,8 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
     assert lib.glqh_e8_fold_eligible(m, n, B) == 1
     q = [t(a) for a in _indices(m, n, stages, m + stages)]
     cb = e8_table_f16()
-    cb2 = cb[:256].contiguous() if stages == 2 else cb        # two stages: the short secondary table
-    if stages == 2:
+    cb2 = cb[:256].contiguous() if stages in (2, 3) else cb   # two, three stages: the short secondary table
+    if stages in (2, 3):
         q[1] = t((_indices(m, n, 1, 7)[0].view(np.uint16) & 255).view(np.int16))
     x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).half().to(DEV)
     args = dict(qidxs2=q[1] if stages > 1 else None, codebook2=cb2, inv_resid_scale=1 / 3.0 if stages > 1 else 0.0,
@@ -127,7 +127,7 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
     else:
         assert torch.equal(y_fold, y_idx)
     if m * n <= 1 << 23:                                       # and both are the oracle's product
-        tabs = [O.e8_table(), O.e8_table()[:256] if stages == 2 else O.e8_table(), O.e8_table(), O.e8_table()]
+        tabs = [O.e8_table(), O.e8_table()[:256] if stages in (2, 3) else O.e8_table(), O.e8_table(), O.e8_table()]
         W = sum(tabs[s][q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)
                 for s in range(stages)).astype(np.float32) * np.float32(0.02)
         assert rel(y_fold, x.float().cpu().numpy() @ W.T) < TOL
@@ -144,8 +144,8 @@ def test_many_token_products_on_folded_streams_equal_products_on_indices(ext, m,
     assert lib.glqh_e8_fold_eligible(m, n, B) == 1
     q = [t(a) for a in _indices(m, n, stages, m + stages + B)]
     cb = e8_table_f16()
-    cb2 = cb[:256].contiguous() if stages == 2 else cb        # two stages: the short secondary table
-    if stages == 2:
+    cb2 = cb[:256].contiguous() if stages in (2, 3) else cb   # two, three stages: the short secondary table
+    if stages in (2, 3):
         q[1] = t((_indices(m, n, 1, 7)[0].view(np.uint16) & 255).view(np.int16))
     x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).half().to(DEV)
     args = dict(qidxs2=q[1] if stages > 1 else None, codebook2=cb2, inv_resid_scale=1 / 3.0 if stages > 1 else 0.0,
@@ -161,7 +161,7 @@ def test_many_token_products_on_folded_streams_equal_products_on_indices(ext, m,
         ext.E8_FOLD = True
     assert torch.equal(y_fold, y_idx)
     if m * n <= 1 << 23:
-        tabs = [O.e8_table(), O.e8_table()[:256] if stages == 2 else O.e8_table(), O.e8_table(), O.e8_table()]
+        tabs = [O.e8_table(), O.e8_table()[:256] if stages in (2, 3) else O.e8_table(), O.e8_table(), O.e8_table()]
         W = sum(tabs[s][q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)
                 for s in range(stages)).astype(np.float32) * np.float32(0.02)
         assert rel(y_fold, x.float().cpu().numpy() @ W.T) < TOL

@@ -66,6 +66,9 @@ SIGNATURES = {
     "glqh_e8_decompress": (
         c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_i64, c_i64,
                 c_vp, c_vp]),
+    "glqh_e8_decompress_f32": (
+        c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_dbl, c_dbl, c_dbl, c_i64, c_i64,
+                c_vp, c_vp]),
     "glqh_e8_embedding_rows": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64,
                 c_dbl, c_vp, c_int, c_i64, c_vp]),

@@ -70,13 +70,22 @@ def _layer_groups(model_dir):
     return {p: g for p, g in groups.items() if "Qidxs" in g or "trellis_packed" in g}
 
 
-def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None = None) -> dict:
+def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None = None, prepare: bool = True,
+                           embed_scales: dict | float | None = None) -> dict:
     """{layer name: E8RHTLinear on `device`} for every quantized linear of the checkpoint; a
     quantized embedding (per-row `Wscale`, one-element `SU`) becomes an `E8RHTEmbedding`.
 
     Block-diagonal checkpoints store unpadded dims, so (out, in) = (len(SU), len(SV)); legacy
     power-of-two padded shell checkpoints need the true shapes in `shapes[name] = (out, in)`
-    (the host model's layer shapes), otherwise the padded dims are used as they are."""
+    (the host model's layer shapes), otherwise the padded dims are used as they are.
+
+    `prepare` runs every layer's load-time step (`E8RHTLinear.prepare()`: host copies of the
+    scalars, packed tables, folded index streams) so that the first forward call, captured or
+    not, finds everything in place.  `embed_scales` gives the factor a scaled embedding multiplies
+    its rows by (sqrt(hidden) in Gemma-style models, glq/quantized_linear.py:1364-1370): one value
+    for every embedding or `{layer name: value}`.  The factor is a property of the host model, not
+    of the checkpoint -- it is not stored in the state dict -- so leaving it out loads such an
+    embedding with outputs too small by that factor."""
     from safetensors import safe_open
     cfg = read_quantization_config(model_dir)
     trellis = cfg.get("codebook") == "trellis"
@@ -94,7 +103,11 @@ def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None 
                 # a quantized embedding (per-row scales, unit SU, glq/quantized_linear.py:1343-1452)
                 vocab, n_pad = sd["Qidxs"].shape[0], sd["SV"].numel()
                 dim = (shapes or {}).get(name, (vocab, n_pad))[1]
-                emb = E8RHTEmbedding(vocab, dim)
+                if isinstance(embed_scales, dict):
+                    scale = float(embed_scales.get(name, 1.0))
+                else:
+                    scale = 1.0 if embed_scales is None else float(embed_scales)
+                emb = E8RHTEmbedding(vocab, dim, embed_scale=scale)
                 if emb.n_pad != n_pad:
                     raise RuntimeError(f"{name}: embedding of width {dim} pads to {emb.n_pad}, the checkpoint "
                                        f"stores {n_pad} columns; pass its true width in shapes[name]")
@@ -120,6 +133,8 @@ def load_quantized_linears(model_dir: str, device="cuda:0", shapes: dict | None 
                 # recipe is the first 256 rows of the full one (glq/codebook.py:348-368), and its
                 # indices never exceed 255
                 lin.set_codebook(table, table)
+            if prepare and torch.device(device).type == "cuda":
+                lin.prepare()
             out[name] = lin
     finally:
         handles.clear()

@@ -4,6 +4,7 @@
 
 #include "common.h"
 
+#include <atomic>
 #include <mutex>
 #include <string.h>
 #include <stdlib.h>
@@ -172,6 +173,34 @@ int glqh_device_cus(void) { return g_cus > 0 ? g_cus : 256; }
 extern "C" const char *glqh_last_error(void) { return g_err; }
 extern "C" int glqh_version(void) { return 1; }
 
+// Scratch of the entry point that allocates nothing (glqh_fused_linear_trellis_3inst_noalloc, below):
+// a file-scope device array.  Every GPU holds its own copy at its own address; the address is
+// resolved once per device -- by glqh_init() for whichever device is current when any entry of the
+// library is first called there -- and host code uses that address only, never the array's name.
+#define GLQH_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
+#define GLQH_NOALLOC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[GLQH_NOALLOC_SCRATCH_BYTES];
+static std::atomic<void *> g_scratch_ptr[GLQH_NOALLOC_MAX_DEVICES];
+static std::mutex g_scratch_mu;
+
+static int noalloc_scratch_for_current_device(void **out) {
+    int dev = -1;
+    if (glqh_check_hip(hipGetDevice(&dev), "hipGetDevice")) return 1;
+    GLQH_REQUIRE(dev >= 0 && dev < GLQH_NOALLOC_MAX_DEVICES, "no-alloc entry: device index %d out of range", dev);
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            if (glqh_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return 1;
+            GLQH_REQUIRE(p != nullptr, "no-alloc entry: scratch array has no device address");
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    if (out) *out = p;
+    return 0;
+}
+
 extern "C" int glqh_init(void) {
     std::call_once(g_once, [] {
         int dev = 0;
@@ -189,7 +218,9 @@ extern "C" int glqh_init(void) {
         g_init_rc = glqh_rht_init() || glqh_e8_init() || glqh_e8_tile_init() || glqh_trellis_init() || glqh_trellis_tile_init() || glqh_trellis_mma_init() || glqh_viterbi_init();
     });
     if (g_init_rc != 0 && g_err[0] == 0) glqh_fail("libglq_hip initialisation failed earlier");
-    return g_init_rc;
+    if (g_init_rc != 0) return g_init_rc;
+    // per device, so that the no-alloc entry has nothing left to set up when it runs under capture
+    return noalloc_scratch_for_current_device(nullptr);
 }
 
 #define GLQH_INIT()                      \
@@ -520,32 +551,10 @@ extern "C" int glqh_fused_linear_trellis_3inst(
 }
 
 // ---- the same linear for callers that cannot allocate -----------------------------------
-// Scratch of the fused trellis linear (x_rht + split-K partial sums) in a file-scope device
-// array instead of a caller-provided workspace.  Every GPU holds its own copy of the array at
-// its own address, resolved once per device; host code uses that address only, never the
-// array's name.  Nothing in it has to start at zero: the decode launch writes every
-// [slot][token][row] partial sum before the finishing launch reads it.
-#define GLQH_NOALLOC_SCRATCH_BYTES ((size_t)8 << 20)
-#define GLQH_NOALLOC_MAX_DEVICES 64
-static __device__ __align__(256) unsigned char scratch[GLQH_NOALLOC_SCRATCH_BYTES];
-static void *g_scratch_ptr[GLQH_NOALLOC_MAX_DEVICES];
-static std::mutex g_scratch_mu;
-
-static int noalloc_scratch_for_current_device(void **out) {
-    int dev = -1;
-    if (glqh_check_hip(hipGetDevice(&dev), "hipGetDevice")) return 1;
-    GLQH_REQUIRE(dev >= 0 && dev < GLQH_NOALLOC_MAX_DEVICES, "no-alloc entry: device index %d out of range", dev);
-    std::lock_guard<std::mutex> lk(g_scratch_mu);
-    if (!g_scratch_ptr[dev]) {
-        void *p = nullptr;
-        if (glqh_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return 1;
-        GLQH_REQUIRE(p != nullptr, "no-alloc entry: scratch array has no device address");
-        g_scratch_ptr[dev] = p;
-    }
-    *out = g_scratch_ptr[dev];
-    return 0;
-}
-
+// Scratch of the fused trellis linear (x_rht + split-K partial sums) in the file-scope device
+// array defined above glqh_init() instead of a caller-provided workspace.  Nothing in it has to
+// start at zero: the decode launch writes every [slot][token][row] partial sum before the
+// finishing launch reads it.
 extern "C" size_t glqh_noalloc_scratch_bytes(void) { return GLQH_NOALLOC_SCRATCH_BYTES; }
 
 extern "C" int glqh_fused_linear_trellis_3inst_noalloc(
@@ -1233,6 +1242,21 @@ extern "C" int glqh_e8_decompress(const void *q1, const void *q2, const void *q3
     return glqh_launch_e8_decompress(sg.q, sg.n, table1, table2 ? table2 : table1,
                                      table2 ? n_entries2 : 65536, sg.scale[1], sg.scale[2], sg.scale[3],
                                      m_pad, n_pad, out_f16, (hipStream_t)stream);
+}
+
+extern "C" int glqh_e8_decompress_f32(const void *q1, const void *q2, const void *q3, const void *q4,
+                                      const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                                      double inv_rs, double inv_rs2, double inv_rs3, int64_t m_pad,
+                                      int64_t n_pad, float *out_f32, void *stream) {
+    GLQH_INIT();
+    GLQH_REQUIRE(out_f32, "e8 decompress: null pointer");
+    e8_stages sg;
+    if (e8_check_dims(m_pad, n_pad, 1) ||
+        e8_resolve_stages(q1, q2, q3, q4, 1.0, inv_rs, inv_rs2, inv_rs3, table1, table2, n_entries2, &sg))
+        return 1;
+    return glqh_launch_e8_decompress_f32(sg.q, sg.n, table1, table2 ? table2 : table1,
+                                         table2 ? n_entries2 : 65536, sg.scale[1], sg.scale[2], sg.scale[3],
+                                         m_pad, n_pad, out_f32, (hipStream_t)stream);
 }
 
 extern "C" int glqh_e8_embedding_rows(const int64_t *ids, int64_t n_ids, const void *q1, const void *q2,

@@ -169,6 +169,9 @@ int glqh_launch_e8_fold_indices(const void *q, int64_t rows, int64_t cols, const
 int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_t *t1,
                               const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
                               int64_t m_pad, int64_t n_pad, void *out, hipStream_t stream);
+int glqh_launch_e8_decompress_f32(const void *const q[4], int nstages, const uint32_t *t1,
+                                  const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
+                                  int64_t m_pad, int64_t n_pad, float *out, hipStream_t stream);
 
 int glqh_launch_e8_embedding(const int64_t *ids, int64_t n_ids, const void *q1, const void *q2,
                              const uint32_t *t1, const uint32_t *t2, int64_t n2, const float *wscale,

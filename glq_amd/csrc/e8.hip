@@ -162,12 +162,13 @@ e8_gemv_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
 // Dense fp16 weight (m_pad, n_pad) in the RHT domain, before Wscale: stages combined in
 // fp32 and rounded once (the reference's batched path rounds the combined weight to fp16
 // as well, glq/csrc/glq_cuda.cu:868-899).  One thread per 8-column block.
+template <typename OT>
 __global__ void __launch_bounds__(256)
 e8_decompress_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict__ q2,
                      const uint16_t *__restrict__ q3, const uint16_t *__restrict__ q4,
                      const uint32_t *__restrict__ t1, const uint32_t *__restrict__ t2, uint32_t n2,
                      float s2, float s3, float s4, int nstages, int64_t total_blocks,
-                     f16 *__restrict__ out) {
+                     OT *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= total_blocks) return;
     float w[8];
@@ -194,10 +195,18 @@ e8_decompress_kernel(const uint16_t *__restrict__ q1, const uint16_t *__restrict
             w[2 * p + 1] += sc[st - 1] * (float)v.y;
         }
     }
-    f16 o[8];
+    if constexpr (sizeof(OT) == 4) {                            // the unrounded fp32 sums (dequantize)
 #pragma unroll
-    for (int c = 0; c < 8; ++c) o[c] = (f16)w[c];
-    *(u32x4 *)(out + i * 8) = *(const u32x4 *)o;
+        for (int h = 0; h < 2; ++h) {
+            const float4 o = {w[4 * h], w[4 * h + 1], w[4 * h + 2], w[4 * h + 3]};
+            *(float4 *)(out + i * 8 + 4 * h) = o;
+        }
+    } else {
+        f16 o[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o[c] = (f16)w[c];
+        *(u32x4 *)(out + i * 8) = *(const u32x4 *)o;
+    }
 }
 
 // The same for large layers: the table's first P entries (the low-norm shells that Gaussian
@@ -398,10 +407,21 @@ int glqh_launch_e8_decompress(const void *const q[4], int nstages, const uint32_
         GLQH_LAUNCH_CHECK("e8 decompress launch");
         return 0;
     }
-    hipLaunchKernelGGL(e8_decompress_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(e8_decompress_kernel<f16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                        (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
                        (const uint16_t *)q[3], t1, t2, (uint32_t)n2, s2, s3, s4, nstages, total,
                        (f16 *)out);
     GLQH_LAUNCH_CHECK("e8 decompress launch");
+    return 0;
+}
+
+int glqh_launch_e8_decompress_f32(const void *const q[4], int nstages, const uint32_t *t1,
+                                  const uint32_t *t2, int64_t n2, float s2, float s3, float s4,
+                                  int64_t m_pad, int64_t n_pad, float *out, hipStream_t stream) {
+    const int64_t total = m_pad * (n_pad / 8);
+    hipLaunchKernelGGL(e8_decompress_kernel<float>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       (const uint16_t *)q[0], (const uint16_t *)q[1], (const uint16_t *)q[2],
+                       (const uint16_t *)q[3], t1, t2, (uint32_t)n2, s2, s3, s4, nstages, total, out);
+    GLQH_LAUNCH_CHECK("e8 decompress (fp32) launch");
     return 0;
 }

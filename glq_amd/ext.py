@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+import warnings
 import weakref
 
 import torch
@@ -90,6 +91,50 @@ def _meta_ptr(meta):
         return C.c_void_p(0)
     _chk(meta, "block meta", torch.int32)
     return _p(meta)
+
+def _skey(t):
+    return (t.data_ptr(), t._version, tuple(t.shape), t.dtype, str(t.device))
+
+
+class _DerivedCache:
+    """Device data derived once from a source tensor (a packed table, a folded index stream, block
+    sizes read back to the host).  An entry is keyed by the source's bytes -- address, version
+    counter, shape, dtype, device -- and guarded by a weak reference to its storage: a fresh view
+    of the same memory hits, a new tensor at a reused address does not, an in-place write misses,
+    and the entry goes when the storage is freed."""
+
+    def __init__(self):
+        self._d = {}
+
+    def get(self, t, extra=()):
+        hit = self._d.get(_skey(t) + extra)
+        if hit is not None and hit[0]() is t.untyped_storage():
+            return hit[1]
+        return None
+
+    def put(self, t, value, extra=()):
+        key = _skey(t) + extra
+        store = t.untyped_storage()
+        d = self._d
+        for k in [k for k, v in d.items() if v[0]() is None or (v[0]() is store and k[0] == key[0] and k[1] != key[1]
+                                                                and k[2:] == key[2:])]:
+            del d[k]                                           # dead sources, older versions of this one
+
+        def drop(ref, key=key):
+            if d.get(key, (None,))[0] is ref:
+                del d[key]
+        d[key] = (weakref.ref(store, drop), value)
+        return value
+
+    def values(self):
+        return [v[1] for v in self._d.values() if v[0]() is not None]
+
+    def __len__(self):
+        return len(self._d)
+
+    def holds(self, t):
+        """True when some entry was derived from `t`'s bytes (any version, any table)."""
+        return any(k[0] == t.data_ptr() and v[0]() is t.untyped_storage() for k, v in self._d.items())
 
 
 # --------------------------------------------------------------------------- trellis
@@ -498,19 +543,16 @@ def glq_fused_linear_trellis_3inst_yrht_rvq2_cuda(x, sv, trellis_packed, trellis
                    _yrht_slice(y_rht_out, col, m_pad), None)
 
 
-_META_BLOCKS = {}
+_META_BLOCKS = _DerivedCache()
 
 
 def _meta_blocks(meta, num_blocks):
     """Block sizes of a device meta tensor, read back once per tensor (a device-to-host copy on
     every call would stall the batch-1 path and cannot run under graph capture)."""
-    key = (meta.data_ptr(), meta._version, tuple(meta.shape), str(meta.device))
-    hit = _META_BLOCKS.get(key)
-    if hit is None or hit[0]() is not meta:
-        for k in [k for k, v in _META_BLOCKS.items() if v[0]() is None]:
-            del _META_BLOCKS[k]
-        hit = _META_BLOCKS[key] = (weakref.ref(meta), [int(v) for v in meta[:num_blocks, 1].tolist()])
-    return hit[1]
+    hit = _META_BLOCKS.get(meta, (int(num_blocks),))
+    if hit is None:
+        hit = _META_BLOCKS.put(meta, [int(v) for v in meta[:num_blocks, 1].tolist()], (int(num_blocks),))
+    return hit
 
 
 def glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, trellis_packed, m, k, in_features,
@@ -532,15 +574,16 @@ def glq_decode_matvec_trellis_3inst_fusein_cuda(x_raw, sv, trellis_packed, m, k,
 
 
 # --------------------------------------------------------------------------- E8 shell
-_TABLES = {}
+_TABLES = _DerivedCache()
 
 
 def _packed_table(codebook):
-    """Nibble-packed copy of an (N, 8) fp16 E8 table, built once per tensor."""
-    key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device))
-    hit = _TABLES.get(key)
-    if hit is not None and hit[0]() is codebook:            # same live tensor, not a reused address
-        return hit[1]
+    """Nibble-packed copy of an (N, 8) fp16 E8 table, built once per table (the check of the
+    table's values reads one word back: made ahead of time by `e8_prepare`, it never runs under
+    stream capture)."""
+    hit = _TABLES.get(codebook)
+    if hit is not None:
+        return hit
     lib = _lib.load()
     _chk(codebook, "codebook", torch.float16)
     if codebook.dim() != 2 or codebook.shape[1] != 8 or not 1 <= codebook.shape[0] <= 65536:
@@ -553,45 +596,35 @@ def _packed_table(codebook):
     if nbad:
         raise RuntimeError(f"codebook has {nbad} rows outside the E8 half-integer grid "
                            "{-3, -2.5, ..., 3}; only E8 shell tables are supported")
-    if len(_TABLES) > 64:                                   # drop entries whose tensor is gone
-        for k in [k for k, v in _TABLES.items() if v[0]() is None]:
-            del _TABLES[k]
-    _TABLES[key] = (weakref.ref(codebook), packed)
-    return packed
+    return _TABLES.put(codebook, packed)
 
 
-_HALF_TABLES = {}
+_HALF_TABLES = _DerivedCache()
 
 
 def _half_table(codebook):
-    """The table as fp16 (exact for E8 values); converted once per tensor."""
+    """The table as fp16 (exact for E8 values); converted once per table."""
     if codebook.dtype == torch.float16:
         return codebook
-    key = (codebook.data_ptr(), codebook._version, tuple(codebook.shape), str(codebook.device), codebook.dtype)
-    hit = _HALF_TABLES.get(key)
-    if hit is None or hit[0]() is not codebook:
-        for k in [k for k, v in _HALF_TABLES.items() if v[0]() is None]:   # tensors that are gone
-            del _HALF_TABLES[k]
-        hit = _HALF_TABLES[key] = (weakref.ref(codebook), codebook.to(torch.float16).contiguous())
-    return hit[1]
+    hit = _HALF_TABLES.get(codebook)
+    if hit is None:
+        hit = _HALF_TABLES.put(codebook, codebook.to(torch.float16).contiguous())
+    return hit
 
 
-_DEV_TABLES = {}
+_DEV_TABLES = _DerivedCache()
 
 
 def _on_device(codebook, dev):
     """`codebook` on `dev`; a table kept on another device (the reference keeps its codebooks on
-    the CPU until first use) is copied once per tensor, so the packed table built from the copy
+    the CPU until first use) is copied once per table, so the packed table built from the copy
     is found again on the next call."""
     if codebook.device == dev:
         return codebook
-    key = (id(codebook), codebook._version, tuple(codebook.shape), str(codebook.device), str(dev))
-    hit = _DEV_TABLES.get(key)
-    if hit is None or hit[0]() is not codebook:
-        for k in [k for k, v in _DEV_TABLES.items() if v[0]() is None]:
-            del _DEV_TABLES[k]
-        hit = _DEV_TABLES[key] = (weakref.ref(codebook), codebook.to(dev))
-    return hit[1]
+    hit = _DEV_TABLES.get(codebook, (str(dev),))
+    if hit is None:
+        hit = _DEV_TABLES.put(codebook, codebook.to(dev), (str(dev),))
+    return hit
 
 
 def _per_row(t, n, name):
@@ -651,13 +684,18 @@ def glq_embedding_dequant(input_ids, qidxs, sv, wscale, codebook, qidxs2=None, i
     return out.reshape(*input_ids.shape, embedding_dim)
 
 
-# Folded copies of the index streams for the small-batch kernel (include/glq_hip.h,
-# glqh_e8_fold_table): made on the first call that can use them and kept while the index tensor
-# lives, 1.5 times the bytes of the indices they copy.  GLQ_E8_FOLD=0 keeps the kernels on the
-# indices themselves.
+# Folded copies of the index streams (include/glq_hip.h, glqh_e8_fold_table): made by `e8_prepare`
+# at load time -- the place the reference prepares its layers is process_weights_after_loading,
+# glq_vllm/linear_method.py:1031 -- and kept while the index tensor's storage lives, 1.5 times the
+# bytes of the indices they copy.  The forward path only looks them up: a layer that was never
+# prepared runs on its indices.  GLQ_E8_FOLD=0 keeps every layer on the indices;
+# GLQ_E8_FOLD_MAX_BYTES=<n> bounds the total of the copies (layers prepared after the bound is
+# reached stay on their indices).
 E8_FOLD = os.environ.get("GLQ_E8_FOLD", "1") != "0"
-_FOLD_TABLES = {}
-_FOLD_STREAMS = {}
+E8_FOLD_MAX_BYTES = int(os.environ.get("GLQ_E8_FOLD_MAX_BYTES", "0"))       # 0 = no bound
+_FOLD_TABLES = _DerivedCache()
+_FOLD_STREAMS = _DerivedCache()
+_fold_warned = set()
 
 
 class _E8Folded(C.Structure):
@@ -666,13 +704,13 @@ class _E8Folded(C.Structure):
 
 
 def _fold_table(packed):
-    """(half codewords (n, 4) fp16, map) of a nibble-packed table tensor, once per tensor; (None, None)
+    """(half codewords (n, 4) fp16, map) of a nibble-packed table tensor, once per table; (None, None)
     for a table with more than 2048 distinct half codewords (no E8 shell table has: the full one has
-    1286), which the kernels then read through its indices."""
-    key = (packed.data_ptr(), packed._version, packed.shape[0], str(packed.device))
-    hit = _FOLD_TABLES.get(key)
-    if hit is not None and hit[0]() is packed:
-        return hit[1], hit[2]
+    1286), which the kernels then read through its indices.  Copies the table to the host and
+    synchronizes: load time only."""
+    hit = _FOLD_TABLES.get(packed)
+    if hit is not None:
+        return hit
     lib = _lib.load()
     halves = torch.empty((2048, 4), dtype=torch.float16, device=packed.device)
     fmap = torch.empty(packed.shape[0], dtype=torch.int32, device=packed.device)
@@ -681,19 +719,16 @@ def _fold_table(packed):
         rc = lib.glqh_e8_fold_table(_p(packed), packed.shape[0], _p(halves), 2048, _p(fmap), C.addressof(n), _stream())
     if rc != 0 and n.value <= 2048:
         check(rc)
-    halves, fmap = (halves[:n.value].clone(), fmap) if rc == 0 else (None, None)
-    for k in [k for k, v in _FOLD_TABLES.items() if v[0]() is None]:
-        del _FOLD_TABLES[k]
-    _FOLD_TABLES[key] = (weakref.ref(packed), halves, fmap)
-    return halves, fmap
+    return _FOLD_TABLES.put(packed, (halves[:n.value].clone(), fmap) if rc == 0 else (None, None))
 
 
 def _fold_stream(q, packed):
-    """(16-bit words, bytes) of one stage's index tensor against its packed table."""
-    key = (q.data_ptr(), q._version, tuple(q.shape), str(q.device), packed.data_ptr())
-    hit = _FOLD_STREAMS.get(key)
-    if hit is not None and hit[0]() is q and hit[1]() is packed:
-        return hit[2], hit[3]
+    """(16-bit words, bytes) of one stage's index tensor against its packed table; made once per
+    index tensor and table."""
+    extra = (packed.data_ptr(),)
+    hit = _FOLD_STREAMS.get(q, extra)
+    if hit is not None and hit[0]() is packed:
+        return hit[1], hit[2]
     lib = _lib.load()
     _, fmap = _fold_table(packed)
     count = lib.glqh_e8_folded_count(q.shape[0], q.shape[1])
@@ -702,18 +737,63 @@ def _fold_stream(q, packed):
     with torch.cuda.device(q.device):
         check(lib.glqh_e8_fold_indices(_p(q), q.shape[0], q.shape[1], _p(fmap), packed.shape[0], _p(lo16), _p(hi8),
                                        _stream()))
-    for k in [k for k, v in _FOLD_STREAMS.items()          # an older version of the same tensor
-              if k[0] == key[0] and k != key and v[0]() is q]:
-        del _FOLD_STREAMS[k]
-    drop = lambda _ref, key=key: _FOLD_STREAMS.pop(key, None)   # the copies go when the index tensor goes
-    _FOLD_STREAMS[key] = (weakref.ref(q, drop), weakref.ref(packed, drop), lo16, hi8)
+    _FOLD_STREAMS.put(q, (weakref.ref(packed), lo16, hi8), extra)
     return lo16, hi8
+
+
+def e8_fold_bytes():
+    """Device bytes held by folded index streams right now."""
+    return sum(v[1].numel() * 2 + v[2].numel() for v in _FOLD_STREAMS.values())
+
+
+def e8_prepare(qidxs, codebook, qidxs2=None, codebook2=None, qidxs3=None, qidxs4=None):
+    """Load-time preparation of an E8 layer: the packed table(s) and, for a layer the folded kernels
+    serve, the folded copy of every stage's indices.  Call once per layer after its buffers are on
+    the GPU and before any stream capture (it allocates, launches and synchronizes); calling it again
+    is cheap.  Returns the number of bytes of folded streams the layer holds (0: the layer runs on
+    its indices -- too small, `GLQ_E8_FOLD=0`, or the `GLQ_E8_FOLD_MAX_BYTES` bound is reached).
+
+    The reference's counterpart is `GLQLinearMethod.process_weights_after_loading`
+    (glq_vllm/linear_method.py:1031-1110), which moves buffers, caches scalars and loads tables."""
+    _chk(qidxs, "qidxs", torch.int16)
+    dev = qidxs.device
+    t1 = _primary_table(_half_table(_on_device(codebook, dev)))
+    stages = [(qidxs, t1)]
+    if not _absent(qidxs2):
+        cb2 = codebook if _absent(codebook2) else codebook2
+        stages.append((qidxs2, _packed_table(_half_table(_on_device(cb2, dev)))))
+    stages += [(q, t1) for q in (qidxs3, qidxs4) if not _absent(q)]
+    M, nblk = qidxs.shape
+    lib = _lib.load()
+    if not E8_FOLD or not any(lib.glqh_e8_fold_eligible(M, nblk * 8, B) for B in (1, 4, 16, 17, 64)):
+        return 0
+    need = sum(3 * lib.glqh_e8_folded_count(q.shape[0], q.shape[1]) for q, t in stages
+               if _FOLD_STREAMS.get(q, (t.data_ptr(),)) is None)
+    if E8_FOLD_MAX_BYTES and e8_fold_bytes() + need > E8_FOLD_MAX_BYTES:
+        return 0
+    if any(_fold_table(t)[0] is None for _, t in stages):
+        return 0
+    total = 0
+    for q, t in stages:
+        _chk(q, "qidxs", torch.int16)
+        lo16, hi8 = _fold_stream(q, t)
+        total += lo16.numel() * 2 + hi8.numel()
+    return total
+
+
+def e8_release(*qidxs):
+    """Drop the folded copies of the given index tensors now (they also go with their storage)."""
+    for q in qidxs:
+        if q is None:
+            continue
+        for k in [k for k in _FOLD_STREAMS._d if k[0] == q.data_ptr()]:
+            del _FOLD_STREAMS._d[k]
 
 
 def _e8_folded(B, qidxs, t1, q2, t2, q3, q4):
     """The folded streams of a layer as the C struct (and what must stay alive during the call), or
-    (None, None) when the call would not read them.  Not made under stream capture: the table fold
-    synchronizes; a layer first seen there runs on its indices."""
+    (None, None) when the call would not read them or `e8_prepare` has not made them.  Looks up
+    only: nothing is allocated, launched or synchronized here, so it is safe under stream capture."""
     M, nblk = qidxs.shape
     if not E8_FOLD or not qidxs.is_contiguous():
         return None, None
@@ -721,29 +801,29 @@ def _e8_folded(B, qidxs, t1, q2, t2, q3, q4):
     if not lib.glqh_e8_fold_eligible(M, nblk * 8, B):
         return None, None
     stages = [(qidxs, t1)] + ([(q2, t2)] if q2 is not None else []) + [(q, t1) for q in (q3, q4) if q is not None]
-    capturing = torch.cuda.is_current_stream_capturing()
-    tables = [t1] + ([t2] if q2 is not None and t2 is not t1 else [])
-    if capturing and any(_FOLD_TABLES.get((t.data_ptr(), t._version, t.shape[0], str(t.device))) is None for t in tables):
-        return None, None
-    if any(_fold_table(t)[0] is None for t in tables):
-        return None, None
     keep, f = [], _E8Folded()
     for s, (q, t) in enumerate(stages):
-        if capturing:
-            key = (q.data_ptr(), q._version, tuple(q.shape), str(q.device), t.data_ptr())
-            hit = _FOLD_STREAMS.get(key)
-            if hit is None or hit[0]() is not q or hit[1]() is not t:
-                return None, None
-        lo16, hi8 = _fold_stream(q, t)
-        keep += [lo16, hi8]
-        f.lo16[s], f.hi8[s] = lo16.data_ptr(), hi8.data_ptr()
-    h1, _ = _fold_table(t1)
-    keep.append(h1)
-    f.halves1, f.n_halves1 = h1.data_ptr(), h1.shape[0]
+        hit = _FOLD_STREAMS.get(q, (t.data_ptr(),))
+        if hit is None or hit[0]() is not t:
+            key = (qidxs.data_ptr(), tuple(qidxs.shape))
+            if key not in _fold_warned and len(_fold_warned) < 4096:
+                _fold_warned.add(key)
+                warnings.warn(f"E8 layer {M}x{nblk * 8} was not prepared (glq_amd.ext.e8_prepare / "
+                              "E8RHTLinear.prepare): it runs on its indices, which is slower at 1-4096 "
+                              "tokens" + (" -- first seen under stream capture, the graph keeps that form"
+                                          if torch.cuda.is_current_stream_capturing() else ""),
+                              RuntimeWarning, stacklevel=4)
+            return None, None
+        keep += [hit[1], hit[2]]
+        f.lo16[s], f.hi8[s] = hit[1].data_ptr(), hit[2].data_ptr()
+    tables = [t1] + ([t2] if q2 is not None and t2 is not t1 else [])
+    halves = [_FOLD_TABLES.get(t) for t in tables]
+    if any(h is None or h[0] is None for h in halves):
+        return None, None
+    keep += [h[0] for h in halves]
+    f.halves1, f.n_halves1 = halves[0][0].data_ptr(), halves[0][0].shape[0]
     if len(tables) == 2:
-        h2, _ = _fold_table(t2)
-        keep.append(h2)
-        f.halves2, f.n_halves2 = h2.data_ptr(), h2.shape[0]
+        f.halves2, f.n_halves2 = halves[1][0].data_ptr(), halves[1][0].shape[0]
     return f, keep
 
 
@@ -832,20 +912,19 @@ def glq_dequant_matvec_cuda(x, qidxs, codebook, wscale, qidxs2=None, codebook2=N
                                    inv_resid_scale).reshape(-1)
 
 
-_REPACKED = {}
+_REPACKED = _DerivedCache()
 
 
 def _repacked_table(codebook_packed):
     """The reference's `codebook_packed` (65536 int32, nibble c = column c,
-    glq/codebook.py:102-115) in the kernels' nibble order, converted once per tensor."""
+    glq/codebook.py:102-115) in the kernels' nibble order, converted once per table."""
     _chk(codebook_packed, "codebook_packed", torch.int32)
     if codebook_packed.dim() != 1 or codebook_packed.shape[0] != 65536:
         raise RuntimeError("codebook_packed must hold 65536 int32 words, got "
                            f"{tuple(codebook_packed.shape)}")
-    key = (codebook_packed.data_ptr(), codebook_packed._version, str(codebook_packed.device))
-    hit = _REPACKED.get(key)
-    if hit is not None and hit[0]() is codebook_packed:
-        return hit[1]
+    hit = _REPACKED.get(codebook_packed)
+    if hit is not None:
+        return hit
     lib = _lib.load()
     out = torch.empty_like(codebook_packed)
     bad = torch.zeros(1, dtype=torch.int32, device=codebook_packed.device)
@@ -855,11 +934,7 @@ def _repacked_table(codebook_packed):
     if nbad:
         raise RuntimeError(f"codebook_packed has {nbad} words with a code above 12; only E8 shell "
                            "tables are supported")
-    if len(_REPACKED) > 64:
-        for k in [k for k, v in _REPACKED.items() if v[0]() is None]:
-            del _REPACKED[k]
-    _REPACKED[key] = (weakref.ref(codebook_packed), out)
-    return out
+    return _REPACKED.put(codebook_packed, out)
 
 
 def glq_dequant_matmul_packed_cuda(x, qidxs, codebook_packed, wscale):

@@ -89,6 +89,7 @@ class E8RHTLinear(nn.Module):
         self.codebook = None
         self.codebook2 = None
         self._scalars = None                 # host copies of Wscale / residual scales
+        self._prepared_for = None            # identity of the buffers the load-time step last saw
         self._trellis_has_kernel = True
         self._rebuild_meta()
 
@@ -113,6 +114,7 @@ class E8RHTLinear(nn.Module):
         if self._is_trellis:
             self._trellis_has_kernel = getattr(codebook, "has_kernel", True)
         self._scalars = None
+        self._prepared_for = None
 
     def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys,
                               unexpected_keys, error_msgs):
@@ -176,8 +178,84 @@ class E8RHTLinear(nn.Module):
         self.m_pad, self.n_pad = m_pad, n_pad
         self._rebuild_meta()
 
-    def _resolve(self, device):
-        """One-time host reads (scalars) and device copies (block meta) per device."""
+    def prepare(self):
+        """Load-time step, to be called once the buffers are on the GPU and the table is attached,
+        before any stream capture: host copies of the scalars, block meta on the device and, for an
+        E8 layer, the packed table(s) and the folded index streams the small-batch and tile kernels
+        read (1.5 x the index bytes; `GLQ_E8_FOLD=0` / `GLQ_E8_FOLD_MAX_BYTES` bound them).  The
+        reference's place for this work is `GLQLinearMethod.process_weights_after_loading`
+        (glq_vllm/linear_method.py:1031-1110).  A forward call outside capture runs it if the
+        caller did not; a layer first seen under capture is served on its indices and warns.
+        Returns the bytes of folded streams the layer holds."""
+        from . import ext
+        dev = self.SV.device
+        if dev.type != "cuda":
+            raise RuntimeError("E8RHTLinear.prepare() needs the buffers on the GPU")
+        self._scalars = None
+        sc = self._resolve(dev, prepare=False)
+        held = 0
+        if not self._is_trellis:
+            if self.codebook is None:
+                raise RuntimeError("set_codebook() must be called before prepare()")
+            n = sc["n_stages"]
+            cb, cb2 = self._tables(dev, n)
+            held = ext.e8_prepare(self.Qidxs, cb, self.Qidxs2 if n >= 2 else None, cb2,
+                                  self.Qidxs3 if n >= 3 else None, self.Qidxs4 if n >= 4 else None)
+        self._prepared_for = self._buffer_identity()
+        return held
+
+    def _buffer_identity(self):
+        names = ("trellis_packed", "trellis_packed2") if self._is_trellis else ("Qidxs", "Qidxs2", "Qidxs3", "Qidxs4")
+        return tuple((getattr(self, n).data_ptr(), getattr(self, n)._version) for n in names) + (str(self.SV.device),)
+
+    def _tables(self, device, n_stages):
+        """The attached table(s) as fp16 tensors on `device`, converted once."""
+        cb = _codebook_tensor(self.codebook)
+        if cb.device != device or cb.dtype != torch.float16:
+            cb = cb.to(device=device, dtype=torch.float16)
+            self.codebook = cb
+        cb2 = None
+        if n_stages >= 2:
+            cb2 = _codebook_tensor(self.codebook2)
+            if cb2.device != device or cb2.dtype != torch.float16:
+                cb2 = cb2.to(device=device, dtype=torch.float16)
+                self.codebook2 = cb2
+        return cb, cb2
+
+    def dequantize(self) -> torch.Tensor:
+        """The dense (out_features, in_features) fp32 weight, for validation
+        (glq/quantized_linear.py:1237-1265): every stage decoded and combined in fp32, scaled, both
+        transforms undone.  `forward(x)` equals `x @ dequantize().T` up to the fp16 rounding of the
+        forward path."""
+        from . import dequant
+        dev = self.SV.device
+        if dev.type != "cuda":
+            raise RuntimeError("E8RHTLinear.dequantize() (glq_amd) runs on the GPU only")
+        sc = self._resolve(dev, prepare=False)
+        if self._is_trellis:
+            W_rht = dequant.trellis_rht_domain_weight(self.trellis_packed, self.m_pad, self.n_pad,
+                                                      self.trellis_packed2 if sc["has2"] else None, sc["inv2"])
+        else:
+            if self.codebook is None:
+                raise RuntimeError("set_codebook() must be called before dequantize()")
+            n, inv = sc["n_stages"], sc["inv"]
+            cb, cb2 = self._tables(dev, n)
+            W_rht = dequant.e8_rht_domain_weight(self.Qidxs, cb, self.Qidxs2 if n >= 2 else None, cb2, inv[0],
+                                                 self.Qidxs3 if n >= 3 else None, inv[1],
+                                                 self.Qidxs4 if n >= 4 else None, inv[2])
+        return dequant.weight_from_rht_domain(W_rht, self.SU, self.SV, sc["wscale"], self.out_features,
+                                              self.in_features, self.blocks_m, self.blocks_n)
+
+    def _resolve(self, device, prepare=True):
+        """One-time host reads (scalars) and device copies (block meta) per device; outside stream
+        capture also the load-time step of `prepare()` if the caller has not run it."""
+        if prepare and not self._is_trellis and self._prepared_for != self._buffer_identity():
+            if torch.cuda.is_current_stream_capturing():
+                if self._scalars is None:
+                    raise RuntimeError("E8RHTLinear: first forward under stream capture; call prepare() "
+                                       "(or run one forward) before capturing")
+            else:
+                self.prepare()
         if self._scalars is None:
             if self._is_trellis:
                 has2 = self.trellis_packed2.numel() > 0
@@ -250,6 +328,8 @@ class E8RHTLinear(nn.Module):
         if not x.is_cuda:
             raise RuntimeError("E8RHTLinear (glq_amd) runs on the GPU only: there is no CPU path")
         from . import ext
+        if not self._is_trellis and self.codebook is None:
+            raise RuntimeError("set_codebook() must be called before forward")
         sc = self._resolve(x.device)
         shape = x.shape
         x2d = x.reshape(-1, self.in_features)
@@ -273,19 +353,8 @@ class E8RHTLinear(nn.Module):
                 inv_resid_scale2=sc["inv2"])
             return y.reshape(*shape[:-1], self.out_features)
 
-        if self.codebook is None:
-            raise RuntimeError("set_codebook() must be called before forward")
-        cb = _codebook_tensor(self.codebook)
-        if cb.device != x.device or cb.dtype != torch.float16:
-            cb = cb.to(device=x.device, dtype=torch.float16)
-            self.codebook = cb
         n = sc["n_stages"]
-        cb2 = None
-        if n >= 2:
-            cb2 = _codebook_tensor(self.codebook2)
-            if cb2.device != x.device or cb2.dtype != torch.float16:
-                cb2 = cb2.to(device=x.device, dtype=torch.float16)
-                self.codebook2 = cb2
+        cb, cb2 = self._tables(x.device, n)
         xin = x2d if x2d.dtype in (torch.float16, torch.bfloat16) else x2d.half()
         xin = xin.contiguous()
         inv = sc["inv"]

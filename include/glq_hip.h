@@ -150,7 +150,9 @@ int glqh_fused_linear_trellis_3inst(const void *x, int x_dtype, int64_t x_stride
  * allocate device memory (code under HIP-graph capture, tight serving loops, harnesses that
  * forbid hipMalloc).  No counterpart in the reference.  The scratch (x_rht and the split-K
  * partial sums) lives in a device array built into the library, glqh_noalloc_scratch_bytes()
- * = 8 MiB per GPU, resolved once per device on the first call with that device current; the
+ * = 8 MiB per GPU.  Its address is resolved once per device by glqh_init() -- which every entry
+ * of the library runs -- with that device current: call glqh_init() (or any entry) once on each
+ * device before capturing, and the captured call has nothing left to set up.  The
  * call allocates nothing and is refused with a message when
  * glqh_fused_linear_trellis_workspace_bytes(B, n_pad, m_pad) exceeds that size.  Results are
  * bit-identical to glqh_fused_linear_trellis_3inst.  All calls on one GPU share the array:
@@ -349,6 +351,14 @@ int glqh_e8_decompress(const void *q1, const void *q2, const void *q3, const voi
                        const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
                        double inv_rs, double inv_rs2, double inv_rs3,
                        int64_t m_pad, int64_t n_pad, void *out_f16, void *stream);
+
+/* The same weight as unrounded fp32 sums: the RHT-domain half of E8RHTLinear.dequantize
+ * (glq/quantized_linear.py:1237-1249) and dequantize_glq_weight (glq_vllm/dequant.py:31-44),
+ * which decode every stage and combine them in fp32. */
+int glqh_e8_decompress_f32(const void *q1, const void *q2, const void *q3, const void *q4,
+                           const uint32_t *table1, const uint32_t *table2, int64_t n_entries2,
+                           double inv_rs, double inv_rs2, double inv_rs3,
+                           int64_t m_pad, int64_t n_pad, float *out_f32, void *stream);
 
 /* Quantized embedding lookup: rows `ids` of a (num_embeddings, n_pad/8) index matrix are decoded,
  * scaled per row, inverse-transformed (one power-of-two block of n_pad <= 8192 values) and

@@ -543,6 +543,17 @@ def linear_forward_rht(x, W_rht, su, sv, blocks_n, blocks_m, in_features, out_fe
     return y.astype(np.float32)
 
 
+def dense_weight(W_rht, su, sv, blocks_m, blocks_n, out_features, in_features):
+    """Weight-domain matrix of an RHT-domain weight that already carries Wscale:
+    `su * H_m( (H_n(rows) * sv) columns )`, cut to (out, in)  (E8RHTLinear.dequantize,
+    glq/quantized_linear.py:1250-1265; dequantize_glq_weight, glq_vllm/dequant.py:46-55;
+    the reference has it for whole power-of-two transforms only, block-diagonal follows
+    glq/hadamard.py:166-178)."""
+    A = block_diag_fht(np.asarray(W_rht, np.float32), blocks_n) * np.asarray(sv, np.float32)[None, :]
+    B = block_diag_fht(np.ascontiguousarray(A.T), blocks_m).T * np.asarray(su, np.float32)[:, None]
+    return np.ascontiguousarray(B[:out_features, :in_features]).astype(np.float32)
+
+
 def trellis_linear_forward(x, art, in_features, out_features):
     """E8RHTLinear._forward_trellis CPU fallback (glq/quantized_linear.py:986-1010)."""
     m, n = out_features, in_features

@@ -123,3 +123,16 @@ def test_quantized_embedding_group_becomes_an_embedding_module(tmp_path, golden)
     table = O.e8_table()
     norms = (table[:256] ** 2).sum(-1)
     assert np.all(norms[1:] >= norms[:-1]) and norms[255] <= 4.0    # the low-norm prefix, in table order
+    # the embedding's scale factor is the host model's, not the checkpoint's: it is passed in
+    assert emb.embed_scale == 1.0
+    for arg, want in (({"model.embed_tokens": 8.0}, 8.0), (4.0, 4.0), ({"other": 3.0}, 1.0)):
+        scaled = C.load_quantized_linears(str(tmp_path), device="cpu", embed_scales=arg)["model.embed_tokens"]
+        assert scaled.embed_scale == want
+
+
+def test_prepare_needs_the_gpu(tmp_path, golden):
+    """The load-time step runs kernels: on CPU buffers it refuses instead of falling back."""
+    _trellis_dir(str(tmp_path), golden)
+    lins = C.load_quantized_linears(str(tmp_path), device="cpu")      # prepare is skipped for a CPU load
+    with pytest.raises(RuntimeError, match="GPU"):
+        next(iter(lins.values())).prepare()

@@ -80,10 +80,14 @@ def test_folded_copies_go_with_their_index_tensor(ext):
     qd = t(np.zeros((32, 64), np.int16))
     ext._fold_stream(qd, packed)
     ptr = qd.data_ptr()
-    assert any(k[0] == ptr for k in ext._FOLD_STREAMS)
+    assert ext._FOLD_STREAMS.holds(qd)
+    view = qd.view(64, 32)                                     # the storage lives on in a view
     del qd
     gc.collect()
-    assert not any(k[0] == ptr for k in ext._FOLD_STREAMS)
+    assert any(k[0] == ptr for k in ext._FOLD_STREAMS._d)
+    del view
+    gc.collect()
+    assert not any(k[0] == ptr for k in ext._FOLD_STREAMS._d)
 
 
 def _indices(m, n, stages, seed):
@@ -110,8 +114,9 @@ def test_products_on_folded_streams_equal_products_on_indices(ext, m, n, B, stag
                 qidxs4=q[3] if stages > 3 else None, inv_resid_scale3=1 / 27.0 if stages > 3 else 0.0)
     ext.E8_FOLD = True
     try:
+        held = ext.e8_prepare(q[0], cb, args["qidxs2"], cb2, args["qidxs3"], args["qidxs4"])
+        assert held == 3 * stages * lib.glqh_e8_folded_count(m, n // 8) and ext._FOLD_STREAMS.holds(q[0])
         y_fold = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
-        assert any(k[0] == q[0].data_ptr() for k in ext._FOLD_STREAMS), "the folded streams were not made"
         ext.E8_FOLD = False
         y_idx = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
     finally:
@@ -153,8 +158,9 @@ def test_many_token_products_on_folded_streams_equal_products_on_indices(ext, m,
                 qidxs4=q[3] if stages > 3 else None, inv_resid_scale3=1 / 27.0 if stages > 3 else 0.0)
     ext.E8_FOLD = True
     try:
+        held = ext.e8_prepare(q[0], cb, args["qidxs2"], cb2, args["qidxs3"], args["qidxs4"])
+        assert held == 3 * stages * lib.glqh_e8_folded_count(m, n // 8) and ext._FOLD_STREAMS.holds(q[0])
         y_fold = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
-        assert any(k[0] == q[0].data_ptr() for k in ext._FOLD_STREAMS), "the folded streams were not made"
         ext.E8_FOLD = False
         y_idx = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
     finally:
@@ -168,46 +174,87 @@ def test_many_token_products_on_folded_streams_equal_products_on_indices(ext, m,
 
 
 def test_fused_linear_on_folded_streams_and_under_capture(ext):
+    """The forward path only looks the folded streams up.  A layer that was never prepared runs on its
+    indices -- also under capture, with a warning -- and makes nothing; after `e8_prepare` a captured
+    first call reads the folded streams and equals the eager folded result bit for bit."""
     say("e8 folded fused linear + graph")
+    import warnings
     from glq_amd import hadamard as H
     m, n = 4096, 3072                                          # block-diagonal input side
     q = [t(a) for a in _indices(m, n, 2, 3)]
     su, sv = O.rht_signs(m, n, 42)
     bn, bm = O.block_decompose(n), O.block_decompose(m)
     cb = e8_table_f16()
+    ext._packed_table(cb)                                      # the table itself is known (another layer used it)
     args = (t(sv.astype(np.float16)), t(su.astype(np.float16)), q[0], cb, 0.02, n, m, n, m, torch.tensor(bn),
             torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), q[1], cb, 1 / 3.0)
     x = torch.randn(2, n, generator=torch.Generator().manual_seed(5)).bfloat16().to(DEV)
-    # first seen under capture: the fold (which synchronizes) is not made there, the call runs on the indices
-    s = torch.cuda.Stream()
-    s.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(s):
-        warm = ext.glq_fused_linear_block_diag_cuda(x, *args[:2], q[0].clone(), *args[3:], out_dtype=torch.bfloat16)
-    torch.cuda.current_stream().wait_stream(s)
     n_before = len(ext._FOLD_STREAMS)
-    q_new = [a.clone() for a in q]
+    with pytest.warns(RuntimeWarning, match="was not prepared"):
+        y_idx = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
+    q_new = [a.clone() for a in q]                             # first seen under capture
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        y_cap = ext.glq_fused_linear_block_diag_cuda(x, *args[:2], q_new[0], *args[3:13], q_new[1], *args[14:],
-                                                     out_dtype=torch.bfloat16)
-    assert len(ext._FOLD_STREAMS) == n_before
+    with pytest.warns(RuntimeWarning, match="under stream capture"):
+        with torch.cuda.graph(g):
+            y_cap = ext.glq_fused_linear_block_diag_cuda(x, *args[:2], q_new[0], *args[3:13], q_new[1], *args[14:],
+                                                         out_dtype=torch.bfloat16)
+    assert len(ext._FOLD_STREAMS) == n_before                  # nothing was made on the way
     g.replay()
     torch.cuda.synchronize()
-    y_fold = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
-    assert any(k[0] == q[0].data_ptr() for k in ext._FOLD_STREAMS)
-    assert torch.equal(y_cap, y_fold) and torch.equal(warm, y_fold)
-    # captured after the streams exist: the graph reads them
+    assert torch.equal(y_cap, y_idx)
+    # load-time step, then a captured FIRST call: it runs the folded kernel
+    bytes_before = ext.e8_fold_bytes()
+    held = ext.e8_prepare(q[0], cb, q[1], cb)
+    assert held == 2 * 3 * ext._lib.load().glqh_e8_folded_count(m, n // 8) == ext.e8_fold_bytes() - bytes_before
     g2 = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g2):
-        y2 = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")                         # no "not prepared" warning any more
+        with torch.cuda.graph(g2):
+            y2 = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
+        y_fold = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
     for _ in range(2):
         g2.replay()
         torch.cuda.synchronize()
         assert torch.equal(y2, y_fold)
+    assert torch.equal(y_fold, y_idx)                          # this shape keeps the K plan: the same bits as on the indices
     art = {"Qidxs": q[0].cpu().numpy(), "Qidxs2": q[1].cpu().numpy(), "inv_resid_scale": np.float32(1 / 3.0),
            "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
            "blocks_m": bm, "blocks_n": bn}
     assert rel(y_fold, O.e8_linear_forward(x.float().cpu().numpy(), art, n, m)) < TOL
+
+
+def test_fresh_views_of_the_indices_hit_the_one_fold(ext):
+    """A caller that passes a new view object of the same index memory on every call (a shard of a
+    stacked tensor, `.view()`) finds the one folded copy: nothing is folded again, nothing dropped."""
+    say("e8 fold: fresh views")
+    m, n = 2048, 4096
+    stacked = t(_indices(2 * m, n, 1, 12)[0])                  # two layers stacked row-wise
+    cb = e8_table_f16()
+    shard = lambda: stacked[m:]                                # noqa: E731  (a new tensor object per call)
+    assert ext.e8_prepare(shard(), cb) > 0
+    n_entries = len(ext._FOLD_STREAMS)
+    x = torch.randn(1, n, generator=torch.Generator().manual_seed(1)).half().to(DEV)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        y1 = ext.glq_dequant_matmul_cuda(x, shard(), cb, 0.02)
+        y2 = ext.glq_dequant_matmul_cuda(x, stacked.view(2, m, n // 8)[1], cb, 0.02)
+    assert len(ext._FOLD_STREAMS) == n_entries and torch.equal(y1, y2)
+    ext.E8_FOLD = False
+    try:
+        assert rel(y1, ext.glq_dequant_matmul_cuda(x, shard(), cb, 0.02)) < 1e-5
+    finally:
+        ext.E8_FOLD = True
+    assert ext.e8_prepare(shard(), cb) > 0 and len(ext._FOLD_STREAMS) == n_entries    # again: a lookup
+    # the bound on the copies: a layer prepared beyond it stays on its indices
+    other = t(_indices(m, n, 1, 13)[0])
+    ext.E8_FOLD_MAX_BYTES = ext.e8_fold_bytes() + 1024
+    try:
+        assert ext.e8_prepare(other, cb) == 0 and not ext._FOLD_STREAMS.holds(other)
+    finally:
+        ext.E8_FOLD_MAX_BYTES = 0
+    ext.e8_release(stacked[m:])
+    assert not ext._FOLD_STREAMS.holds(stacked[m:])
 
 
 def test_c_abi_refusals(ext):

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import glq_oracle as O
-from tests.gpu_util import DEV, e8_table_f16, rel, say, t
+from tests.gpu_util import DEV, e8_table_f16, rel, say, t, e8_prepared
 
 pytestmark = pytest.mark.gpu
 
@@ -34,9 +34,11 @@ def _e8_layer(m, n, seed):
 def _e8_forward(ext, x, q1, q2, su, sv, m, n, dtype):
     from glq_amd import hadamard as H
     bn, bm = O.block_decompose(n), O.block_decompose(m)
+    cb = e8_table_f16()
+    d1, d2, _, _ = e8_prepared(ext, cb, q1, q2)                   # folded once per layer, then looked up
     return ext.glq_fused_linear_block_diag_cuda(
-        x, t(sv), t(su), t(q1), e8_table_f16(), 0.02, n, m, n, m, torch.tensor(bn), torch.tensor(bm),
-        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), t(q2), e8_table_f16(), 1 / 3.0,
+        x, t(sv), t(su), d1, cb, 0.02, n, m, n, m, torch.tensor(bn), torch.tensor(bm),
+        H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), d2, cb, 1 / 3.0,
         out_dtype=dtype)
 
 

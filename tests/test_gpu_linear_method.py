@@ -1,0 +1,184 @@
+"""The serving-side call sequence of a merged trellis linear (glq_vllm/linear_method.py:643-741)
+through the registered `torch.ops.glq.*` ops: every shard against the oracle, the shard-batched
+output transform against the per-shard route, and the whole sequence captured in a HIP graph and
+replayed on new activations (needs an MI355X)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glq_oracle as O
+from tests.gpu_util import DEV, rel, say, t
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module", autouse=True)
+def ops():
+    from glq_amd import custom_ops
+    custom_ops.register()
+    return torch.ops.glq
+
+
+def _shard_art(m, n, K, K2, seed):
+    su, sv = O.rht_signs(m, n, 200 + seed)
+    art = {"trellis_packed": O.random_packed(m, n, K, seed), "SU": su.astype(np.float16),
+           "SV": sv.astype(np.float16), "Wscale": np.float32(0.02 + 0.003 * seed),
+           "blocks_m": O.block_decompose(m), "blocks_n": O.block_decompose(n)}
+    if K2:
+        art["trellis_packed2"] = O.random_packed(m, n, K2, 50 + seed)
+        art["inv_resid_scale2"] = np.float32(0.21 + 0.01 * seed)
+    return art
+
+
+def _merged(n, shards, bpw):
+    """shards: [(m, K, K2)] -> (MergedTrellisLinear after its load-time step, per-shard artifacts)."""
+    from glq_amd.linear_method import GLQShards, MergedTrellisLinear
+    arts = [_shard_art(m, n, K, K2, i) for i, (m, K, K2) in enumerate(shards)]
+    layer = MergedTrellisLinear(n, [m for m, _, _ in shards], bpw=bpw)
+    layer.trellis_packed = GLQShards(torch.from_numpy(a["trellis_packed"]) for a in arts)
+    layer.trellis_packed2 = GLQShards(torch.from_numpy(a["trellis_packed2"]) if "trellis_packed2" in a
+                                      else torch.zeros(0, dtype=torch.int16) for a in arts)
+    layer.SU = GLQShards(torch.from_numpy(a["SU"]) for a in arts)
+    layer.SV = GLQShards(torch.from_numpy(a["SV"]) for a in arts)
+    layer.Wscale = GLQShards(torch.tensor(float(a["Wscale"])) for a in arts)
+    layer.inv_resid_scale2 = GLQShards(torch.tensor(float(a.get("inv_resid_scale2", 0.0))) for a in arts)
+    layer.process_weights_after_loading(DEV)
+    return layer, arts
+
+
+def _oracle(x16, arts, n):
+    xs = x16.float().cpu().numpy()
+    return np.concatenate([O.trellis_linear_forward(xs, a, n, a["SU"].shape[0]) for a in arts], axis=1)
+
+
+@pytest.mark.parametrize("bpw,shards", [(4, [(256, 4, 0), (64, 4, 0), (64, 4, 0)]),       # fused q/k/v
+                                        (6, [(352, 4, 2), (352, 4, 2)]),                  # gate/up, 4+2 bits
+                                        (5, [(2048, 4, 1), (512, 4, 1), (512, 4, 1)])])   # SmolLM3 q/k/v rows, 4+1
+@pytest.mark.parametrize("B", [1, 3, 40])
+def test_s4b_sequence_through_registered_ops_matches_oracle(ops, bpw, shards, B):
+    """`fused_linear_trellis_3inst_yrht[_rvq2]` per shard into one (B, total_m) buffer + one
+    `output_rht_shards`, each called as `torch.ops.glq.<op>`: every shard's columns within 1e-2 of
+    the oracle's fp32 CPU forward of that shard; equal to the per-shard fused op's result up to the
+    fp16 rounding of its output; bit-identical when repeated."""
+    n = 512 if shards[0][0] < 2048 else 2048
+    say("s4b ops", bpw, shards, B)
+    layer, arts = _merged(n, shards, bpw)
+    assert layer._glq_s4b is not None and layer._glq_s4b["has_s2"] == (bpw > 4)
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).to(DEV, torch.float16)
+    ref = _oracle(x, arts, n)
+    # the sequence written out with the registered ops, as the reference's apply does
+    total = sum(m for m, _, _ in shards)
+    y_rht = torch.empty(B, total, dtype=torch.float32, device=DEV)
+    col = 0
+    for i, meta in enumerate(layer._glq_trellis_meta):
+        if meta["has_s2"]:
+            ops.fused_linear_trellis_3inst_yrht_rvq2(
+                x, layer.SV.get_shard(i), layer.trellis_packed.get_shard(i), layer.trellis_packed2.get_shard(i),
+                meta["_bn"], meta["_bnm"], meta["wscale"], meta["inv_rs2"], n, n, meta["m_pad"], y_rht, col)
+        else:
+            ops.fused_linear_trellis_3inst_yrht(
+                x, layer.SV.get_shard(i), layer.trellis_packed.get_shard(i), meta["_bn"], meta["_bnm"],
+                meta["wscale"], n, n, meta["m_pad"], y_rht, col)
+        col += meta["m_pad"]
+    y = torch.empty(B, total, dtype=torch.float16, device=DEV)
+    ops.output_rht_shards(y_rht, layer._glq_s4b["su_cat"], y, total, layer._glq_s4b["shard_meta"],
+                          layer._glq_s4b["max_bs"])
+    col = 0
+    for (m, _, _), a in zip(shards, arts):
+        e = rel(y[:, col:col + m], ref[:, col:col + m])
+        assert e < TOL, (m, e)
+        col += m
+    # the layer object's apply() is that sequence
+    ya = layer.apply(x)
+    assert ya.dtype == x.dtype and torch.equal(ya, y)
+    assert torch.equal(layer.apply(x), ya)
+    # and the transform-domain rows of a shard are what the oracle's transform-domain product gives
+    a0 = arts[0]
+    m0 = shards[0][0]
+    Wn = O.decode_layer_nstage([a0["trellis_packed"]] + ([a0["trellis_packed2"]] if "trellis_packed2" in a0 else []),
+                               [1.0] + ([float(a0["inv_resid_scale2"])] if "trellis_packed2" in a0 else []), m0, n)
+    xr = O.block_diag_fht(x.float().cpu().numpy() * a0["SV"].astype(np.float32)[None], a0["blocks_n"])
+    assert rel(y_rht[:, :m0], (xr @ Wn.T) * np.float32(a0["Wscale"])) < TOL
+
+
+def test_batched_output_transform_switch_and_unloaded_shard(ops, monkeypatch):
+    """GLQ_TRELLIS_BATCH_OUT_RHT=0: one fused op per shard, concatenated -- against the oracle and
+    against the shard-batched route (same decode, another launch for the output transform: equal to
+    fp16 rounding).  A shard that was never loaded gives exact-zero columns on both routes."""
+    from glq_amd import linear_method as LM
+    say("s4b switch")
+    n, shards = 512, [(256, 4, 0), (64, 4, 0), (64, 4, 0)]
+    layer, arts = _merged(n, shards, 4)
+    x = torch.randn(4, n, generator=torch.Generator().manual_seed(3)).to(DEV, torch.bfloat16)
+    ref = _oracle(x, arts, n)
+    y_batched = layer.apply(x)
+    monkeypatch.setattr(LM, "_GLQ_BATCH_OUT_RHT", False)
+    y_per_shard = layer.apply(x)
+    assert y_per_shard.dtype == torch.bfloat16
+    assert rel(y_per_shard, ref) < TOL and rel(y_batched, ref) < TOL
+    assert rel(y_per_shard, y_batched.float().cpu().numpy()) < 4e-3
+    # an unloaded k shard (KV-shared layers): zeros, the other columns unchanged
+    layer.trellis_packed._shard_data[1] = torch.zeros(0, dtype=torch.int16, device=DEV)
+    layer.process_weights_after_loading(DEV)
+    for flag in (True, False):
+        monkeypatch.setattr(LM, "_GLQ_BATCH_OUT_RHT", flag)
+        y0 = layer.apply(x)
+        assert float(y0[:, 256:320].abs().max()) == 0.0
+        want = y_batched if flag else y_per_shard
+        assert torch.equal(y0[:, :256], want[:, :256]) and torch.equal(y0[:, 320:], want[:, 320:])
+
+
+def test_load_time_invariants(ops):
+    """What the checkpoint carries must match the recipe (glq_vllm/linear_method.py:1372-1396)."""
+    from glq_amd.linear_method import MergedTrellisLinear, trellis_rvq_recipe
+    say("s4b invariants")
+    assert [trellis_rvq_recipe(b) for b in (2, 4, 5, 6, 8)] == [[2], [4], [4, 1], [4, 2], [4, 4]]
+    with pytest.raises(ValueError):
+        trellis_rvq_recipe(9)
+    n, shards = 512, [(64, 4, 2), (64, 4, 2)]
+    layer, _ = _merged(n, shards, 6)
+    layer.glq_bpw = 4
+    with pytest.raises(RuntimeError, match="no stage for"):
+        layer.process_weights_after_loading(DEV)
+    layer.glq_bpw = 6
+    layer.inv_resid_scale2._shard_data[1] = torch.tensor(0.0)
+    with pytest.raises(RuntimeError, match="half-written"):
+        layer.process_weights_after_loading(DEV)
+    layer.trellis_packed2._shard_data[1] = torch.zeros(0, dtype=torch.int16)
+    with pytest.raises(RuntimeError, match="trellis_packed2 is missing"):
+        layer.process_weights_after_loading(DEV)
+    fresh = MergedTrellisLinear(n, [64])
+    with pytest.raises(RuntimeError, match="process_weights_after_loading"):
+        fresh.apply(torch.zeros(1, n, device=DEV, dtype=torch.float16))
+
+
+@pytest.mark.parametrize("bpw,shards", [(4, [(2048, 4, 0), (512, 4, 0), (512, 4, 0)]), (6, [(352, 4, 2), (352, 4, 2)])])
+def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, shards):
+    """The whole apply() -- yrht ops, the shared buffer, output_rht_shards, the cast -- captured once;
+    replays with new contents in the static input equal the eager result bit for bit, replay after
+    replay, with eager work in between."""
+    n = 2048 if shards[0][0] == 2048 else 512
+    say("s4b graph", bpw)
+    layer, arts = _merged(n, shards, bpw)
+    gen = torch.Generator().manual_seed(11)
+    xs = [torch.randn(2, n, generator=gen).to(DEV, torch.bfloat16) for _ in range(4)]
+    static_x = xs[0].clone()
+    layer.apply(static_x)                                    # warm-up outside capture
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            static_y = layer.apply(static_x)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    for x in xs[1:] + xs[:1]:
+        eager = layer.apply(x)
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, eager)
+        assert rel(static_y, _oracle(x, arts, n)) < TOL

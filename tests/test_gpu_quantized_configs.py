@@ -22,7 +22,7 @@ import pytest
 import torch
 
 from oracle import glq_oracle as O
-from tests.gpu_util import DEV, e8_table_f16, rel, say, t
+from tests.gpu_util import DEV, e8_table_f16, rel, say, t, e8_prepared
 
 pytestmark = pytest.mark.gpu
 
@@ -180,9 +180,10 @@ def e8_forward(ext, x, art, m, n, dtype):
     from glq_amd import hadamard as H
     bn, bm = art["blocks_n"], art["blocks_m"]
     cb = e8_table_f16()
+    q1, q2, _, _ = e8_prepared(ext, cb, art["Qidxs"], art["Qidxs2"])     # load-time step once, then looked up
     return ext.glq_fused_linear_block_diag_cuda(
-        x, t(art["SV"]), t(art["SU"]), t(art["Qidxs"]), cb, float(art["Wscale"]), n, m, n, m, torch.tensor(bn),
-        torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), t(art["Qidxs2"]), cb,
+        x, t(art["SV"]), t(art["SU"]), q1, cb, float(art["Wscale"]), n, m, n, m, torch.tensor(bn),
+        torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), q2, cb,
         1 / 3.0, out_dtype=dtype)
 
 
@@ -204,8 +205,8 @@ def test_e8_two_stage_llama_mlp_whole_layer_oracle_and_quality_gates(ext, m, n):
     pref = xr.float().numpy() @ W_dec.T * art["Wscale"]
     cb = e8_table_f16()
     for M in (1, 4, 16):
-        out = ext.glq_dequant_matmul_cuda(xr[:M].to(DEV), t(art["Qidxs"]), cb, float(art["Wscale"]),
-                                          t(art["Qidxs2"]), cb, 1 / 3.0)
+        q1, q2, _, _ = e8_prepared(ext, cb, art["Qidxs"], art["Qidxs2"])
+        out = ext.glq_dequant_matmul_cuda(xr[:M].to(DEV), q1, cb, float(art["Wscale"]), q2, cb, 1 / 3.0)
         assert sqnr(pref[:M], out.float().cpu().numpy()) > 40.0, (M, sqnr(pref[:M], out.float().cpu().numpy()))
     W_hat = to_weight_domain(W_dec * art["Wscale"], su, sv, bm, bn)
     xh = x.to(torch.float16)

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import glq_oracle as O
-from tests.gpu_util import DEV, e8_table_f16, rel, say, t
+from tests.gpu_util import DEV, e8_table_f16, rel, say, t, e8_prepared
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -189,7 +189,9 @@ def test_e8_large_layers_lds_table(ext, m, n, B, stages):
     x = (rng.standard_normal((B, n)) * 0.5).astype(np.float16)
     W = O.e8_dequant(q[0], q[1], sc[0], q[2], sc[1], q[3], sc[2])
     ref = x.astype(np.float32) @ W.T * np.float32(0.021)
-    args = (t(q[0]), cb, 0.021, t(q[1]), cb, sc[0], None, t(q[2]), cb, sc[1], t(q[3]), cb, sc[2])
+    d = e8_prepared(ext, cb, *q[:stages])                         # the load-time step: folded streams where they serve
+    d += [t(q[s]) for s in range(stages, 4)]                      # absent stages (scale 0) are never read
+    args = (d[0], cb, 0.021, d[1], cb, sc[0], None, d[2], cb, sc[1], d[3], cb, sc[2])
     out = ext.glq_dequant_matmul_cuda(t(x), *args)
     assert out.shape == (B, m) and rel(out, ref) < 1e-3, rel(out, ref)
     assert torch.equal(out, ext.glq_dequant_matmul_cuda(t(x), *args))
@@ -204,10 +206,11 @@ def test_e8_large_layer_small_secondary_table(ext):
     q2 = rng.integers(0, 256, size=(m, n // 8)).astype(np.int16)
     x = rng.standard_normal((2, n)).astype(np.float16)
     W = O.e8_dequant(q1, q2, 0.5)
-    out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
+    d1, d2, _, _ = e8_prepared(ext, cb, q1, q2, cb2)
+    out = ext.glq_dequant_matmul_cuda(t(x), d1, cb, 1.0, d2, cb2, 0.5)
     assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
     x = rng.standard_normal((24, n)).astype(np.float16)          # many tokens: tile kernel, second table from L2
-    out = ext.glq_dequant_matmul_cuda(t(x), t(q1), cb, 1.0, t(q2), cb2, 0.5)
+    out = ext.glq_dequant_matmul_cuda(t(x), d1, cb, 1.0, d2, cb2, 0.5)
     assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
 
 

@@ -188,3 +188,24 @@ def test_embedding_rows_closed_form():
     one = O.e8_embedding_rows(np.arange(vocab), q1, sv, ws)
     W = O.e8_dequant(q1) * ws[:, None]
     assert np.allclose(one, O.fht(W) * sv, atol=1e-6)
+
+
+@pytest.mark.parametrize("tag,bpw", [("bd2", 2), ("bd4", 4), ("p2", 2), ("p4", 4)])
+def test_dense_weight_matches_reference_dequantize(golden, tag, bpw):
+    """The weight-domain matrix against the reference's own `dequantize()` output (stored for the
+    power-of-two layers, the only ones its method takes) and against the weight its quantizer
+    returned for every layer; a transposed transform, a swapped sign vector or a missing scale
+    fails both."""
+    g = golden("e8_layer")
+    inv = float(g[f"{tag}_inv_resid_scale"]) if bpw == 4 else 0.0
+    W_rht = O.e8_dequant(g[f"{tag}_Qidxs"], g[f"{tag}_Qidxs2"] if bpw == 4 else None, inv) \
+        * np.float32(g[f"{tag}_Wscale"])
+    m, n = g[f"{tag}_W"].shape
+    W = O.dense_weight(W_rht, g[f"{tag}_SU"], g[f"{tag}_SV"], list(g[f"{tag}_blocks_m"]),
+                       list(g[f"{tag}_blocks_n"]), m, n)
+    assert W.shape == (m, n)
+    assert O.rel_fro(W, g[f"{tag}_W_hat"]) < 1e-5
+    if f"{tag}_dequantize" in g.files:
+        assert O.rel_fro(W, g[f"{tag}_dequantize"]) < 1e-6
+    # forward(x) == x @ dequantize().T  (tests/test_quantized_linear.py:120-131)
+    assert O.rel_fro(g[f"{tag}_x"] @ W.T, g[f"{tag}_y"]) < 1e-5

@@ -84,6 +84,55 @@ def test_noalloc_entry_equals_workspace_entry_twice_in_a_row():
     assert torch.equal(y_ws, y_na)
 
 
+def test_noalloc_entry_under_capture_allocates_nothing():
+    """Captured after glqh_init() alone (no earlier call of the entry): replays on new activations
+    equal the workspace entry bit for bit, and the device's free memory is the same before and
+    after the calls (hipMemGetInfo through torch; the outputs are allocated beforehand)."""
+    from glq_amd import _lib
+    lib = _lib.load()
+    assert lib.glqh_init() == 0
+    m, n, B = 2048, 2048, 2
+    art, _ = _layer(m, n, 21, True)
+    xs = [torch.randn(B, n).to(torch.bfloat16).to(DEV) for _ in range(3)]
+    static_x, y_na = xs[0].clone(), torch.zeros(B, m, dtype=torch.bfloat16, device=DEV)
+    y_ws = torch.zeros(B, m, dtype=torch.bfloat16, device=DEV)
+    from glq_amd import hadamard as H
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    abn, abm = (C.c_int64 * len(bn))(*bn), (C.c_int64 * len(bm))(*bm)
+    mn, mm = H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV)
+    p1, p2 = art["p1"], art["p2"]
+
+    def launch():
+        _lib.check(lib.glqh_fused_linear_trellis_3inst_noalloc(
+            _vp(static_x), _lib.GLQH_BF16, n, B, _vp(art["sv"]), _vp(art["su"]), _vp(p1), p1.shape[0], p1.shape[1],
+            _vp(p2), p2.shape[0], p2.shape[1], abn, len(bn), abm, len(bm), _vp(mn), _vp(mm), art["wscale"],
+            art["inv_rs2"], n, m, n, m, _vp(y_na), _lib.GLQH_BF16, m, C.c_void_p(0), 0,
+            C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+    say("noalloc under capture")
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            launch()
+    torch.cuda.current_stream().wait_stream(s)
+    for x in xs[1:] + xs[:1]:
+        _call(lib, False, x, art, n, m, y_ws)                  # eager work between the replays
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_na, y_ws)
+    # an eager call between two readings of the device's free memory, nothing else in between
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    launch()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert torch.equal(y_na, y_ws)
+
+
 def test_noalloc_entry_refuses_what_does_not_fit():
     from glq_amd import _lib
     lib = _lib.load()

@@ -28,7 +28,7 @@ def td(a):
     return hit[1]
 
 
-def e8_prepared(ext, cb, q1, q2=None, cb2=None, q3=None, q4=None):
+def e8_prepared(ext, cb, q1, q2=None, q3=None, q4=None, cb2=None):
     """The index arrays on the device, through the library's load-time step (ext.e8_prepare)."""
     qs = [None if q is None else td(q) for q in (q1, q2, q3, q4)]
     ext.e8_prepare(qs[0], cb, qs[1], cb2 if cb2 is not None else cb, qs[2], qs[3])

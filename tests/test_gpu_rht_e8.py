@@ -206,7 +206,7 @@ def test_e8_large_layer_small_secondary_table(ext):
     q2 = rng.integers(0, 256, size=(m, n // 8)).astype(np.int16)
     x = rng.standard_normal((2, n)).astype(np.float16)
     W = O.e8_dequant(q1, q2, 0.5)
-    d1, d2, _, _ = e8_prepared(ext, cb, q1, q2, cb2)
+    d1, d2, _, _ = e8_prepared(ext, cb, q1, q2, cb2=cb2)
     out = ext.glq_dequant_matmul_cuda(t(x), d1, cb, 1.0, d2, cb2, 0.5)
     assert rel(out, x.astype(np.float32) @ W.T) < 1e-3
     x = rng.standard_normal((24, n)).astype(np.float16)          # many tokens: tile kernel, second table from L2

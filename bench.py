@@ -22,6 +22,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0          # dense fp16 / bf16
 # (name, out_features, in_features) of one SmolLM3-3B decoder layer
 LINEARS = [("q", 2048, 2048), ("k", 512, 2048), ("v", 512, 2048), ("o", 2048, 2048),
            ("gate", 11008, 2048), ("up", 11008, 2048), ("down", 2048, 11008)]
@@ -94,6 +95,68 @@ def cpu_baseline(n_calls=10):
                        f"multi-threaded BLAS for the matmul, single-threaded butterflies")}
 
 
+def cpu_baseline_more():
+    """The other CPU legs, on bounded samples (a few seconds each), each with its core count:
+    E8 two-stage 4096 x 14336 at one token "cold" (the weight re-decoded by table gather on every
+    call, as the reference's E8 CPU path does, glq/quantized_linear.py:1175-1195) and "warm" (decoded
+    weight cached, as its trellis path does), and three tokens of the 36-layer decoder of configs[4]
+    through cached transform-domain weights (four distinct decoded layers walked round-robin -- 1.25 GB
+    of fp32 weights, beyond any cache -- instead of 36, which would take minutes to decode)."""
+    import numpy as np
+    from oracle import cpu_decoder as CD
+    from oracle import glq_oracle as O
+    legs = []
+    cores = os.cpu_count()
+    # E8 two stages, 4096 x 14336, one token
+    m, n = 4096, 14336
+    rng = np.random.default_rng(1)
+    q1 = rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16)
+    q2 = rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16)
+    su, sv = O.rht_signs(m, n, 42)
+    art = {"Qidxs": q1, "Qidxs2": q2, "inv_resid_scale": np.float32(1 / 3.0), "SU": su.astype(np.float16),
+           "SV": sv.astype(np.float16), "Wscale": np.float32(0.02), "blocks_m": O.block_decompose(m),
+           "blocks_n": O.block_decompose(n)}
+    x = rng.standard_normal((1, n)).astype(np.float32)
+    O.e8_linear_forward(x, art, n, m)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        O.e8_linear_forward(x, art, n, m)
+    cold = (time.perf_counter() - t0) / 3
+    W = (O.e8_dequant(q1, q2, 1 / 3.0) * np.float32(0.02)).astype(np.float32)
+    suf, svf = su.astype(np.float32), sv.astype(np.float32)
+    O.linear_forward_rht(x, W, suf, svf, art["blocks_n"], art["blocks_m"], n, m)
+    t0 = time.perf_counter()
+    for _ in range(10):
+        O.linear_forward_rht(x, W, suf, svf, art["blocks_n"], art["blocks_m"], n, m)
+    warm = (time.perf_counter() - t0) / 10
+    eb = m * (n // 8) * 4
+    legs.append({"config": "configs[2]: E8 two-stage 4 bpw 4096x14336, one token, cold (weight decoded every call)",
+                 "value": round(eb / cold / 1e9, 3), "unit": "GB/s", "ms_per_call": round(cold * 1e3, 2), "cores": cores,
+                 "kind": "port", "sample": "3 calls after one warm-up"})
+    legs.append({"config": "configs[2]: E8 two-stage 4 bpw 4096x14336, one token, warm (decoded weight cached)",
+                 "value": round(eb / warm / 1e9, 3), "unit": "GB/s", "ms_per_call": round(warm * 1e3, 2), "cores": cores,
+                 "kind": "port", "sample": "10 calls after one warm-up"})
+    del W, q1, q2
+    # configs[4]: the 36-layer decoder, 3 tokens
+    hidden, heads, kv, hd, ffn, vocab, L = 2048, 16, 4, 128, 11008, 128256, 36
+    shapes = CD.linear_shapes(hidden, heads, kv, hd, ffn)
+    distinct = [CD.make_layer(shapes, K_BITS, s) for s in range(4)]
+    emb = (rng.standard_normal((vocab, hidden)) * 0.02).astype(np.float32)
+    dec = CD.CpuDecoder([distinct[i % 4] for i in range(L)], emb, hidden, heads, kv, hd, max_len=16)
+    tok = 1
+    tok = int(dec.step(tok).argmax())                          # warm-up token
+    t0 = time.perf_counter()
+    for _ in range(3):
+        tok = int(dec.step(tok).argmax())
+    per_tok = (time.perf_counter() - t0) / 3
+    legs.append({"config": "configs[4]: 36-layer SmolLM3-3B-shape decoder, trellis 4 bpw, greedy batch-1 decode",
+                 "value": round(1.0 / per_tok, 3), "unit": "tok/s", "ms_per_token": round(per_tok * 1e3, 1),
+                 "cores": cores, "kind": "port",
+                 "sample": "3 tokens after one warm-up token at context 1-4; 36 layers walking 4 distinct decoded "
+                           "weight sets (1.25 GB fp32), fp32 tied output head"})
+    return legs
+
+
 def _graph_time(torch, fn, n_inner, reps=10):
     """us per inner call of fn(), replayed from a HIP graph between HIP events."""
     fn()
@@ -151,6 +214,17 @@ def extras(torch, ext, dev):
     batch-1 decode tok/s (config 5), large-layer GEMV rates where the kernels are not launch
     bound, and the prefill tiles (config 4 shape)."""
     out = {}
+    roof = out["_roofline_extra"] = []
+
+    def hbm(kernel, config, nbytes, us):
+        gbs = nbytes / us / 1e3
+        roof.append({"kernel": kernel, "config": config, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "us": round(us, 2)})
+
+    def mfma(kernel, config, flop, us):
+        tf = flop / us / 1e6
+        roof.append({"kernel": kernel, "config": config, "bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS, 4), "us": round(us, 2)})
     tr_default, e8_default = ext.TRELLIS_BATCH_MAX, ext.E8_BATCH_MAX
     try:
         # what one more kernel node costs in a captured stream: 2000 dependent one-workgroup fill
@@ -186,6 +260,8 @@ def extras(torch, ext, dev):
             pb = torch.empty(64 * B * m, dtype=torch.float32, device=dev)
             us = _graph_time(torch, lambda: [ext.trellis_gemv_partials(xh, p, m, n, pb) for p in packs], len(packs))
             out[f"trellis_gemv_16384x16384_B{B}_GBs"] = round(m * n / 2 / us / 1e3, 1)
+            hbm("tr_mma_kernel<4> (decode launch alone, partial sums)", f"trellis 4 bpw 16384x16384, {B} token(s), "
+                "4 weight sets of 134 MB in rotation", m * n // 2, us)
         del packs, part
         # 4096 x 4096, one token: the shape of the reference's own GEMV table
         # (benchmarks/_trellis_rvq_decode.md:41-52), single stage and 4+2 bits, rotating over 36
@@ -218,6 +294,14 @@ def extras(torch, ext, dev):
         o = torch.empty(M, m, dtype=torch.float32, device=dev)
         us = _graph_time(torch, lambda: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o), 1, reps=5)
         out["trellis_prefill_14336x4096_M4096_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        mfma("tr_tile_kernel<4,4> + activation repack (matmul entry on transformed rows)",
+             "configs[3]: trellis 4 bpw 14336x4096, 4096 tokens", 2.0 * M * m * n, us)
+        xh = torch.randn(256, n, device=dev).to(torch.float16)
+        o = torch.empty(256, m, dtype=torch.float32, device=dev)
+        us = _graph_time(torch, lambda: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o), 1, reps=10)
+        out["trellis_prefill_14336x4096_M256_TFLOPs"] = round(2.0 * 256 * m * n / us / 1e6, 1)
+        mfma("tr_tile_kernel<4,2> + activation repack + K-slot sum", "configs[3]: trellis 4 bpw 14336x4096, 256 tokens",
+             2.0 * 256 * m * n, us)
         del p, xh, o
         torch.cuda.empty_cache()
     except Exception as e:
@@ -247,6 +331,9 @@ def extras(torch, ext, dev):
             us = _graph_time(torch, lambda: [ext.glq_dequant_matmul_cuda(xh, a, cb, 0.02, b, cb, 1 / 3.0)
                                              for a, b in qs], len(qs))
             out[f"e8_2stage_gemv_4096x14336_B{B}_GBs"] = round(m * (n // 8) * 4 / us / 1e3, 1)
+            hbm("e8_mma_kernel<2,FOLD> (whole unfused call; algorithmic bytes = 2 B per index and stage)",
+                f"configs[2]: E8 two-stage 4 bpw 4096x14336, {B} token(s), 10 index sets in rotation",
+                m * (n // 8) * 4, us)
         # config 4, E8 half: the many-token kernel on the same quantized indices (kernel + K-slot sum),
         # also at 4096 tokens, where the library route is the default
         ext.E8_BATCH_MAX = 1 << 30
@@ -255,6 +342,8 @@ def extras(torch, ext, dev):
             us = _graph_time(torch, lambda: ext.glq_dequant_matmul_cuda(xh, qs[0][0], cb, 0.02, qs[0][1], cb, 1 / 3.0),
                              1, reps=5)
             out[f"e8_2stage_matmul_4096x14336_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+            mfma("e8_tile_kernel<2,FOLD> + activation repack + K-slot sum (matmul entry on transformed rows)",
+                 f"configs[3]: E8 two-stage 4 bpw 4096x14336, {M} tokens", 2.0 * M * m * n, us)
         ext.E8_BATCH_MAX = e8_default
         del qs, i1, i2
         # whole two-stage E8 linear (both transforms), 4096 x 4096, one token, rotating over 36 index sets
@@ -605,9 +694,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    extra = {}
+    extra, roofline_extra = {}, []
     if not args.no_extras:
         extra = extras(torch, ext, dev)
+        roofline_extra = extra.pop("_roofline_extra", [])
 
     result = {
         "metric": "4bpw GEMV effective HBM GB/s (% of peak); batch-1 decode tok/s, 3B shape",
@@ -623,12 +713,17 @@ def main():
                    "distinct_layers": L, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
                    "linear_only_tok_s_36_layers": round(1e3 / (ms_per_step * 36), 1)},
         "roofline": roofline,
+        "roofline_extra": roofline_extra,
         "timing": stats,
         "extra": extra,
     }
     if not args.no_cpu_baseline:
         log("timing the CPU baseline (oracle port of the reference CPU path) ...")
         result["cpu_baseline"] = cpu_baseline()
+        try:
+            result["cpu_baseline"]["more"] = cpu_baseline_more()
+        except Exception as e:                                # report, never hide
+            result["cpu_baseline"]["more_error"] = f"{type(e).__name__}: {e}"
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result), flush=True)

@@ -58,7 +58,7 @@ size_t glqh_trellis_tile_xb_bytes(int64_t k, int64_t M);
 int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M);
 int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
-                             hipStream_t stream);
+                             hipStream_t stream, int out_f16 = 0);
 int64_t glqh_trellis_tile_padded_tokens(int64_t M);
 int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages);
 // input transform straight into a tile kernel's operand layout (fht.hip); -1 = not eligible, nothing launched
@@ -100,9 +100,9 @@ static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
 // stage stored pre-scaled is just more K slots to whoever sums them.  xb: scratch of
 // plan.xb_bytes for the tile kernel (unused otherwise).
 static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                            int64_t k, float *part, void *xb, hipStream_t st, float pscale = 1.0f) {
+                            int64_t k, float *part, void *xb, hipStream_t st, float pscale = 1.0f, int f16_sums = 0) {
     glqh_range range("dequant_matmul");
-    if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, part, 0, 1.0f, 0, 0, st);
+    if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, part, 0, 1.0f, 0, 0, st, f16_sums);
     return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, pscale, 0, 0, st);
 }
 static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
@@ -235,6 +235,14 @@ static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 static bool tr_fuse_input_enabled() {
     static const bool on = [] {
         const char *e = getenv("GLQ_TRELLIS_FUSE_INPUT");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+static bool tr_f16_sums_enabled() {
+    static const bool on = [] {
+        const char *e = getenv("GLQ_TRELLIS_F16_SUMS");
         return !(e && e[0] == '0');
     }();
     return on;
@@ -458,7 +466,7 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     // (2048 x 2048: 14.5 against 17.4 us; at four tokens 23.9 against 18.0, so two to four
     // tokens transform x once); only the MFMA form takes a pre-scaled second stage.  Everything
     // else transforms x once into scratch and reads it from every workgroup.
-    int ks = 0, fi_steps = 0, fi_mode = 0;
+    int ks = 0, fi_steps = 0, fi_mode = 0, f16_sums = 0;
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
     const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
     // Where folding pays (whole linear, us, folded vs separate transform): one token 8.6 vs 11.1
@@ -514,8 +522,14 @@ extern "C" int glqh_fused_linear_trellis_3inst(
             return 1;
         ks = plan.ks;
         if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
-        if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st)) return 1;
-        if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2)) return 1;
+        // Many tokens, one K slot: the tile kernel rounds its sums to fp16 on the way out, as the
+        // reference's many-token route does (its library GEMM of two fp16 matrices returns fp16,
+        // glq/csrc/glq_trellis.cu:1322-1334) -- half the bytes between the product and the output
+        // transform.  GLQ_TRELLIS_F16_SUMS=0 keeps them fp32.
+        f16_sums = plan.tile && ks == 1 && B > 64 && !y_rht_out && y && tr_f16_sums_enabled() &&
+                   glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad);
+        if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st, 1.0f, f16_sums)) return 1;
+        if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2, f16_sums)) return 1;
     }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);
@@ -539,9 +553,10 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     glqh_ysrc src = {};
     src.nparts = has_s2 ? 2 : 1;
     src.part = part1;
-    src.part_sstride = (int64_t)(pb / sizeof(float));
+    src.part_sstride = (int64_t)(pb / (f16_sums ? sizeof(f16) : sizeof(float)));
     src.part_kstride = B * m_pad;
     src.ksplit = ks;
+    src.part_f16 = f16_sums;
     src.scale[0] = s1;
     src.scale[1] = s2;
     src.copy_out = y_rht_out;

@@ -130,7 +130,13 @@ struct glqh_ysrc {                 // where the output RHT reads its RHT-domain 
     int nparts;
     float *copy_out;               // optional: also write the combined fp32 row here
     int64_t copy_stride;
+    int part_f16;                  // the partial sums are fp16 (same strides, in elements); served by the
+                                   // whole-block kernels only (glqh_output_rht_wide_eligible)
 };
+
+// 1 when glqh_launch_output_rht serves this call with the whole-block kernels (many tokens,
+// canonical blocks of 8..8192 rows), the only ones that read fp16 partial sums.
+int glqh_output_rht_wide_eligible(int64_t B, const int64_t *blocks_host, int64_t n_blocks, int64_t m_pad);
 
 int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const void *sv,
                           void *out, int out_dtype, int64_t B, int64_t in_features, int64_t n_pad,

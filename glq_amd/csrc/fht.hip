@@ -259,16 +259,21 @@ __device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysr
             for (int e = 0; e < E; e += 8) load8<float>(d + e, v + e);
         } else {
             // v = sum_stage scale * (sum_k partial), in this fixed order (as stage_partials)
-            const float *pbase = src.part + b * (int64_t)m_pad + blk.off + i;
+            const int64_t ebase = b * (int64_t)m_pad + blk.off + i;
             for (int st = 0; st < src.nparts; ++st) {
                 float acc[E];
 #pragma unroll
                 for (int e = 0; e < E; ++e) acc[e] = 0.0f;
-                const float *p = pbase + st * src.part_sstride;
+                const int64_t eoff = ebase + st * src.part_sstride;
                 for (int k = 0; k < src.ksplit; ++k) {
                     float t0[E];
+                    if (src.part_f16) {                         // uniform over the launch
 #pragma unroll
-                    for (int e = 0; e < E; e += 8) load8<float>(p + k * src.part_kstride + e, t0 + e);
+                        for (int e = 0; e < E; e += 8) load8<f16>((const f16 *)src.part + eoff + k * src.part_kstride + e, t0 + e);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < E; e += 8) load8<float>(src.part + eoff + k * src.part_kstride + e, t0 + e);
+                    }
 #pragma unroll
                     for (int e = 0; e < E; ++e) acc[e] += t0[e];
                 }
@@ -714,9 +719,10 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
     else if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, m_pad)) margs.canon = 0;
     {
         const int y_size = y_dtype == GLQH_F32 ? 4 : 2;
+        const int pq = src.part_f16 ? 8 : 4;                     // elements per 16 bytes of partial sums
         const bool src_ok = src.nparts == 0
             ? (aligned16(src.direct) && src.stride % 4 == 0)
-            : (aligned16(src.part) && m_pad % 4 == 0 && src.part_kstride % 4 == 0 && src.part_sstride % 4 == 0 &&
+            : (aligned16(src.part) && m_pad % pq == 0 && src.part_kstride % pq == 0 && src.part_sstride % pq == 0 &&
                (!src.copy_out || (aligned16(src.copy_out) && src.copy_stride % 4 == 0)));
         // whole blocks per workgroup also from 32 tokens on when the rows are many (whole linear,
         // 64 tokens: 11008 x 2048 56.9 -> 45.3 us, 14336 x 4096 70.4 -> 61.6; 2048 x 11008 41.5 -> 43.7)
@@ -736,6 +742,8 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
             return 0;
         }
     }
+    GLQH_REQUIRE(!src.part_f16, "output_rht: fp16 partial sums need the whole-block kernels (more than 32 tokens, "
+                                "canonical blocks of at most 8192 rows)");
     const int log_slice = rht_log_slice(B);
     const int spb = rht_slices_per_block(max_bs, log_slice);
     GLQH_REQUIRE(n_blocks * spb <= 2147483647ll, "output_rht: too many slices");
@@ -756,6 +764,19 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
 #undef GLQH_OUT_LAUNCH
     GLQH_LAUNCH_CHECK("output_rht launch");
     return 0;
+}
+
+int glqh_output_rht_wide_eligible(int64_t B, const int64_t *blocks_host, int64_t n_blocks, int64_t m_pad) {
+    glqh_meta_args margs;
+    int64_t max_bs = m_pad;
+    if (n_blocks > 1) {
+        if (!blocks_host || check_blocks(blocks_host, n_blocks, m_pad, &max_bs, "output_rht")) return 0;
+    } else if (m_pad & (m_pad - 1)) {
+        return 0;
+    }
+    if (!glqh_fill_meta_args(&margs, n_blocks > 1 ? blocks_host : nullptr, n_blocks > 1 ? n_blocks : 1, m_pad)) return 0;
+    const int64_t Bw = ((B >= 32 && m_pad >= 8192) || B > 32) ? 65 : B;
+    return rht_wide_ok(Bw, margs, m_pad, max_bs) ? 1 : 0;
 }
 
 int glqh_rht_init(void) { return 0; }

@@ -47,6 +47,7 @@ struct tt_args {
     int direct, accum;
     float scale;
     int64_t out_stride;
+    int out_f16;                                   // partial sums as fp16 (not with direct)
 };
 
 __device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global prefetches stay in flight
@@ -137,71 +138,56 @@ tr_tile_kernel(const tt_args a) {
 #pragma unroll
             for (int tt = 0; tt < NTW; ++tt) acc[f][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        // Software pipeline over the 64-column steps: records arrive two steps ahead, the operands
-        // of step d + 1 are written to the other LDS buffer during step d, and the activations of
-        // the next step arrive a whole step ahead in a second register set where registers allow
-        // (NTW <= 2), otherwise half a step ahead in the registers the half just multiplied freed.
-        constexpr bool BDB = NTW <= 2;
-        u32x4 b[BDB ? 2 : 1][NTW][2];
-        auto load_b = [&](u32x4 (&bb)[NTW][2], int d) {
-            d = min(d, ds1 - 1);
+        // Software pipeline over the 64-column steps: records arrive two steps ahead and the operands
+        // of step d + 1 are written to the other LDS buffer during step d.
+        // Activations in three register sets of one k-half each, rotating: the set a half has just
+        // finished with takes the half two ahead, so every request has a whole step to arrive.
+        u32x4 bs[3][NTW];
+        auto load_half = [&](u32x4 (&dst)[NTW], int hidx) {     // half hidx of the slot: step ds0 + hidx / 2, k-half hidx & 1
+            const int d = min(ds0 + (hidx >> 1), ds1 - 1);
 #pragma unroll
-            for (int tt = 0; tt < NTW; ++tt) {
-                bb[tt][0] = *(const u32x4 *)(xrow + 2 * d * bstep + tt * 512);
-                bb[tt][1] = *(const u32x4 *)(xrow + (2 * d + 1) * bstep + tt * 512);
-            }
+            for (int tt = 0; tt < NTW; ++tt) dst[tt] = *(const u32x4 *)(xrow + (2 * d + (hidx & 1)) * bstep + tt * 512);
         };
         tr_record<R> rc = load_rec(ds0);
-        load_b(b[0], ds0);
+        load_half(bs[0], 0);
+        load_half(bs[1], 1);
         tr_record<R> r1 = load_rec(ds0 + 1), r2 = load_rec(ds0 + 2);
         emit(rc, abuf);
         tt_barrier();
-
-        for (int d0 = ds0; d0 < ds1; d0 += 2) {
+        for (int d0 = ds0; d0 < ds1; d0 += 3) {
 #pragma unroll
-          for (int par = 0; par < 2; ++par) {                   // static buffer parity
-            const int d = d0 + par;
+          for (int j = 0; j < 3; ++j) {                         // static register sets: six halves = 0 mod 3
+            const int d = d0 + j;
             if (d >= ds1) break;                                // uniform
-            const int cur = BDB ? par : 0;
+            const int par = (d - ds0) & 1;
             const u32x4 *rd = abuf + par * TT_BUF;
             u32x4 *wr = abuf + (par ^ 1) * TT_BUF;
-            const int dn = min(d + 1, ds1 - 1);
-            if constexpr (BDB) load_b(b[par ^ 1], d + 1);
             const tr_record<R> r3 = load_rec(d + 3);
-            // operands two multiplications ahead: an LDS read takes longer than the NTW MFMAs of one operand
-            f16x8 afn = __builtin_bit_cast(f16x8, rd[lane]);
-            f16x8 afn2 = __builtin_bit_cast(f16x8, rd[GLQH_WAVE + lane]);
-            __builtin_amdgcn_sched_barrier(0);                  // requests stay ahead of the multiplications
+            f16x8 ring[2];
+            ring[0] = __builtin_bit_cast(f16x8, rd[lane]);
+            ring[1] = __builtin_bit_cast(f16x8, rd[GLQH_WAVE + lane]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kk = 0; kk < 2 * TT_FRAGS; ++kk) {
                 const int u = kk / TT_FRAGS, f = kk % TT_FRAGS;
-                const f16x8 af = afn;
-                afn = afn2;
-                if (kk + 2 < 2 * TT_FRAGS) afn2 = __builtin_bit_cast(f16x8, rd[(kk + 2) * GLQH_WAVE + lane]);
+                if (f == 0) {
+                    load_half(bs[(2 * j + u + 2) % 3], 2 * (d - ds0) + u + 2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                const f16x8 af = ring[kk & 1];
+                if (kk + 2 < 2 * TT_FRAGS) ring[kk & 1] = __builtin_bit_cast(f16x8, rd[(kk + 2) * GLQH_WAVE + lane]);
 #pragma unroll
                 for (int tt = 0; tt < NTW; ++tt)
                     acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                        af, __builtin_bit_cast(f16x8, b[cur][tt][u]), acc[f][tt], 0, 0, 0);
-                // operands of d + 1 (unused after the last step), one per half of the step: spread over
-                // the step the decode fits under the MFMAs, bunched into one half it out-issues them
+                        af, __builtin_bit_cast(f16x8, bs[(2 * j + u) % 3][tt]), acc[f][tt], 0, 0, 0);
                 if (kk == 1) emit(r1, wr, 0);
-                if (kk == TT_FRAGS) __builtin_amdgcn_sched_barrier(0);
                 if (kk == TT_FRAGS + 1) emit(r1, wr, 1);
-                if constexpr (!BDB) {
-                    if (f == TT_FRAGS - 1) {                    // this half's activations are free: request the next
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int tt = 0; tt < NTW; ++tt) b[0][tt][u] = *(const u32x4 *)(xrow + (2 * dn + u) * bstep + tt * 512);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
             }
             tt_barrier();                                       // rd has been read, wr is written
             r1 = r2;
             r2 = r3;
           }
         }
-
         // lane holds four consecutive rows of token i for every (operand, token tile): operand
         // f = 4 unit' + s covers rows 64 unit' + 32 h + 8 s + (0..7), h = 0, 1
         const int rlane = 32 * (q >> 1) + 4 * (q & 1);
@@ -214,7 +200,14 @@ tr_tile_kernel(const tt_args a) {
                 const int row = r0 + 64 * (f >> 2) + 8 * (f & 3) + rlane;
                 if (row >= a.m) continue;                       // m is a multiple of 32: whole groups of four
                 if (!a.direct) {
-                    *(f32x4 *)(a.out + ((int64_t)slot * a.M + tok) * a.m + row) = acc[f][tt];
+                    const int64_t e = ((int64_t)slot * a.M + tok) * a.m + row;
+                    if (a.out_f16) {
+                        typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+                        const f32x4 v = acc[f][tt];
+                        *(f16x4 *)((f16 *)a.out + e) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+                    } else {
+                        *(f32x4 *)(a.out + e) = acc[f][tt];
+                    }
                 } else {
                     float *o = a.out + (int64_t)tok * a.out_stride + row;
                     if ((a.out_stride & 3) == 0) {
@@ -494,10 +487,11 @@ int64_t glqh_trellis_tile_padded_tokens(int64_t M) { return tt_padded_tokens(M);
 
 int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
-                             hipStream_t stream) {
+                             hipStream_t stream, int out_f16) {
     tt_plan p;
     tt_make_plan(m, k, M, &p);
     if (direct && p.KS != 1) return glqh_fail("trellis tile kernel: in-place output needs a single K slot");
+    if (out_f16 && (direct || M <= 64)) return glqh_fail("trellis tile kernel: fp16 sums are partial sums of the large tiles");
     const int Mp = (int)tt_padded_tokens(M);
     if (x_f16) {                                               // NULL: xb_scratch already holds the blocked layout
         hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)),
@@ -520,6 +514,7 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     a.accum = accum;
     a.scale = scale;
     a.out_stride = out_stride;
+    a.out_f16 = out_f16;
     switch (R) {
     case 1: return tt_launch_R<1>(p, a, stream);
     case 2: return tt_launch_R<2>(p, a, stream);

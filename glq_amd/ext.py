@@ -28,17 +28,17 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 
 # Small and medium token counts are served on the compressed weights: 1-16 tokens by the GEMV /
 # small-batch kernels, above by the tile kernels that decode each weight once per 128-row x
-# 512-token tile (csrc/trellis_tile.hip, csrc/e8_tile.hip).  From a few thousand tokens on the
+# 512-token tile (csrc/trellis_tile.hip, csrc/e8_tile.hip).  Beyond a few thousand tokens the
 # reference's own many-token route -- dequantize the weight to fp16 once with the HIP kernel, then
-# one library GEMM (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334) -- is the faster one on this chip,
-# at the price of a transient fp16 copy of the weight.  Whole fused linear, compressed / library,
-# us, on 14336 x 4096 and 4096 x 14336: trellis 172 / 201 and 157 / 204 at 1024 tokens, 353 / 334
-# and 268 / 301 at 2048, 564 / 531 and 488 / 487 at 4096; E8 two-stage on the indices 201 / 211 and
-# 196 / 209 at 1024, 400 / 335 and 312 / 327 at 2048, 639 / 552 and 553 / 511 at 4096 (the 14336-row
-# shape pays for 448 and 896 tiles on 256 CUs).  The thresholds are the reference's tunable and its E8
-# counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send calls above n tokens to the
-# library route (a large n keeps every call compressed).
-TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "2048")))
+# one library GEMM (glq/csrc/glq_trellis.cu:1265-1268, 1322-1334) -- is a few per cent faster on this
+# chip, at the price of a transient fp16 copy of the weight.  Whole fused linear, compressed / library,
+# us, on 14336 x 4096 and 4096 x 14336: trellis 175 / 206 and 160 / 205 at 1024 tokens, 340 / 335 and
+# 267 / 300 at 2048, 565 / 545 and 481 / 487 at 4096, 1034 / 980 and 976 / 895 at 8192; E8 two-stage on
+# the indices 201 / 211 and 196 / 209 at 1024, 400 / 335 and 312 / 327 at 2048, 639 / 552 and 553 / 511 at
+# 4096 (the 14336-row shape pays for 448 and 896 tiles on 256 CUs).  The thresholds are the reference's
+# tunable and its E8 counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send calls above n
+# tokens to the library route (a large n keeps every call compressed).
+TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "4096")))
 # GLQ_TRELLIS_DENSE (set to anything) sends every fused trellis call to that dense route, the
 # reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
 TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ

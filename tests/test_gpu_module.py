@@ -295,13 +295,14 @@ def test_graph_capture_of_a_batched_step_on_the_tile_kernels(B):
     rng = np.random.default_rng(B)
     q1, q2 = (t(rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16)) for _ in range(2))
     cb = e8_table_f16()
+    assert ext.e8_prepare(q1, cb, q2, cb) > 0                  # the load-time step: folded streams exist before capture
     xs = torch.randn(B, n, device=DEV).to(torch.bfloat16)
 
     def step():
         return (ext.glq_fused_linear_trellis_3inst_cuda(xs, svt, sut, p, *meta, 0.02, n, m, n, m, out_dtype=torch.bfloat16),
                 ext.glq_fused_linear_block_diag_cuda(xs, svt, sut, q1, cb, 0.02, n, m, n, m, *meta, q2, cb, 1 / 3.0,
                                                      out_dtype=torch.bfloat16))
-    eager = [y.clone() for y in step()]                       # also makes the folded streams
+    eager = [y.clone() for y in step()]
     torch.cuda.synchronize()
     s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())

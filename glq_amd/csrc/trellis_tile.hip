@@ -48,6 +48,7 @@ struct tt_args {
     float scale;
     int64_t out_stride;
     int out_f16;                                   // partial sums as fp16 (not with direct)
+    int rt0;                                       // first row tile of this launch (RT counts from there)
 };
 
 __device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global prefetches stay in flight
@@ -116,10 +117,10 @@ tr_tile_kernel(const tt_args a) {
         const int item = xcd * per_xcd + w;
         if (item >= nitems) break;                              // uniform
         const int rt = item % a.RT, slot = (item / a.RT) % a.KS, tt0 = item / (a.RT * a.KS);
-        const int r0 = rt * TT_ROWS, tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW;
+        const int r0 = (a.rt0 + rt) * TT_ROWS, tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW;
         const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
 
-        const int mp = min(2 * (2 * rt + unit) + hm, mpairs - 1);
+        const int mp = min(2 * (2 * (a.rt0 + rt) + unit) + hm, mpairs - 1);
         const uint8_t *rec_base = a.packed + ((int64_t)mp * nkp * 32 + l) * REC + (int64_t)kpi * 32 * REC;
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
@@ -515,11 +516,48 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     a.scale = scale;
     a.out_stride = out_stride;
     a.out_f16 = out_f16;
-    switch (R) {
-    case 1: return tt_launch_R<1>(p, a, stream);
-    case 2: return tt_launch_R<2>(p, a, stream);
-    case 3: return tt_launch_R<3>(p, a, stream);
-    case 4: return tt_launch_R<4>(p, a, stream);
+    a.rt0 = 0;
+    // The last round of tiles: when the 512-token tiles fill at most half of the CUs in their last round,
+    // the row tiles of that remainder go to a second launch as 256-token tiles, twice as many, each a good
+    // half of the time (14336 rows at 4096 tokens: 896 tiles on 256 CUs = 3.5 rounds -> 3 rounds of 96 row
+    // tiles + one of 16 row tiles x 16 half token tiles; both forms replayed from a graph in one run:
+    // 577-586 -> 548 us).
+    tt_plan tail = p;
+    tail.RT = 0;
+    const int cus = glqh_device_cus();
+    if (p.NTW == 4 && p.KS == 1) {
+        const int64_t T = (int64_t)p.RT * p.TT, rounds = T / cus, rem = T - rounds * cus;
+        if (rounds >= 1 && rem > 0 && 2 * rem <= cus) {
+            const int rt_tail = (int)((rem + p.TT - 1) / p.TT);
+            const int tt2 = (int)((M + 255) / 256);
+            if (rt_tail < p.RT && (int64_t)rt_tail * tt2 <= cus) {
+                tail.RT = rt_tail;
+                tail.TT = tt2;
+                tail.NTW = 2;
+                tail.grid = rt_tail * tt2;
+                p.RT -= rt_tail;
+                const int64_t items = (int64_t)p.RT * p.TT;
+                p.grid = (int)(items < cus ? items : cus);
+                a.RT = p.RT;
+            }
+        }
     }
-    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+    int rc = 1;
+    switch (R) {
+    case 1: rc = tt_launch_R<1>(p, a, stream); break;
+    case 2: rc = tt_launch_R<2>(p, a, stream); break;
+    case 3: rc = tt_launch_R<3>(p, a, stream); break;
+    case 4: rc = tt_launch_R<4>(p, a, stream); break;
+    default: return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+    }
+    if (rc || tail.RT == 0) return rc;
+    a.rt0 = p.RT;
+    a.RT = tail.RT;
+    a.TT = tail.TT;
+    switch (R) {
+    case 1: return tt_launch<1, 2>(tail, a, stream);
+    case 2: return tt_launch<2, 2>(tail, a, stream);
+    case 3: return tt_launch<3, 2>(tail, a, stream);
+    default: return tt_launch<4, 2>(tail, a, stream);
+    }
 }

@@ -334,6 +334,26 @@ def extras(torch, ext, dev):
             hbm("e8_mma_kernel<2,FOLD> (whole unfused call; algorithmic bytes = 2 B per index and stage)",
                 f"configs[2]: E8 two-stage 4 bpw 4096x14336, {B} token(s), 10 index sets in rotation",
                 m * (n // 8) * 4, us)
+        # the same kernel where the launch's fixed costs amortise: 16384 x 16384, two stages, uniformly random
+        # indices, three index sets in rotation
+        try:
+            mm = nn = 16384
+            big = [tuple(torch.randint(-32768, 32768, (mm, nn // 8), device=dev, dtype=torch.int16) for _ in range(2))
+                   for _ in range(3)]
+            for a, b in big:
+                ext.e8_prepare(a, cb, b, cb)
+            xh = torch.randn(1, nn, device=dev).to(torch.float16)
+            us = _graph_time(torch, lambda: [ext.glq_dequant_matmul_cuda(xh, a, cb, 0.02, b, cb, 1 / 3.0) for a, b in big],
+                             len(big))
+            out["e8_2stage_gemv_16384x16384_B1_GBs"] = round(mm * (nn // 8) * 4 / us / 1e3, 1)
+            hbm("e8_mma_kernel<2,FOLD> (+ K-slot sum where the plan splits K across workgroups)",
+                "E8 two-stage 4 bpw 16384x16384, 1 token, 3 index sets of 134 MB in rotation", mm * (nn // 8) * 4, us)
+            for a, b in big:
+                ext.e8_release(a, b)
+            del big
+            torch.cuda.empty_cache()
+        except Exception as e:
+            out["e8_large_error"] = f"{type(e).__name__}: {e}"
         # config 4, E8 half: the many-token kernel on the same quantized indices (kernel + K-slot sum),
         # also at 4096 tokens, where the library route is the default
         ext.E8_BATCH_MAX = 1 << 30
@@ -424,7 +444,7 @@ def extras(torch, ext, dev):
     return out
 
 
-CASES = ("trellis_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
+CASES = ("trellis_gemv_16384", "e8_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
          "e8_prefill_256", "e8_prefill_32", "trellis_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
@@ -442,6 +462,19 @@ def run_case(torch, ext, dev, name, steps):
         pb = torch.empty(64 * m, dtype=torch.float32, device=dev)
         fn = lambda i: ext.trellis_gemv_partials(xh, packs[i % 4], m, n, pb)
         res["bytes_per_launch"] = m * n // 2
+    elif name == "e8_gemv_16384":
+        # the E8 counterpart of trellis_gemv_16384: two stages, uniformly random indices, three index sets of
+        # 134 MB (402 MB of indices, 604 MB of folded streams) in rotation
+        from glq_amd.checkpoint import load_shell_table
+        cb = load_shell_table(None).to(dev)
+        m = n = 16384
+        qs = [tuple(torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16) for _ in range(2))
+              for _ in range(3)]
+        for a, b in qs:
+            ext.e8_prepare(a, cb, b, cb)
+        xh = torch.randn(1, n, device=dev).to(torch.float16)
+        fn = lambda i: ext.glq_dequant_matmul_cuda(xh, qs[i % 3][0], cb, 0.02, qs[i % 3][1], cb, 1 / 3.0)
+        res["bytes_per_launch"] = m * (n // 8) * 4
     elif name in ("trellis_prefill_4096", "trellis_prefill_256", "trellis_prefill_32"):
         m, n, M = 14336, 4096, int(name.rsplit("_", 1)[1])
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)

@@ -23,15 +23,15 @@ int glqh_viterbi_init(void);
 // many-token E8 kernel on the compressed indices (e8_tile.hip)
 int glqh_e8_tile_init(void);
 int glqh_trellis_tile_init(void);
-int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages);
+int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, int fold);
 size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M);
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
                         int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold);
 // Above 16 tokens the weights are decoded once per 128 x 512 tile instead of once per 16 tokens.
 #define GLQH_E8_SMALL_BATCH 16
-static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages) {
-    return B > GLQH_E8_SMALL_BATCH ? glqh_e8_tile_ksplit(m_pad, n_pad, B, nstages) : 0;
+static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages, bool fold) {
+    return B > GLQH_E8_SMALL_BATCH ? glqh_e8_tile_ksplit(m_pad, n_pad, B, nstages, fold) : 0;
 }
 
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
@@ -1115,7 +1115,7 @@ int glqh_e8_mma_ksplit(int64_t m_pad, int64_t n_pad, int64_t B, int64_t n1, int 
 
 extern "C" int glqh_e8_fold_eligible(int64_t m_pad, int64_t n_pad, int64_t B) {
     if (glqh_init() != 0 || m_pad < 1 || n_pad < 8 || (n_pad & 7) || B < 1) return 0;
-    if (B > GLQH_E8_SMALL_BATCH) return glqh_e8_tile_ksplit(m_pad, n_pad, B, 1) > 0 ? 1 : 0;   // the many-token kernel
+    if (B > GLQH_E8_SMALL_BATCH) return glqh_e8_tile_ksplit(m_pad, n_pad, B, 1, 1) > 0 ? 1 : 0;   // the many-token kernel
     return glqh_e8_mma_ksplit(m_pad, n_pad, B, 65536, 1) > 0 ? 1 : 0;
 }
 
@@ -1178,14 +1178,18 @@ static int e8_check_dims(int64_t m_pad, int64_t n_pad, int64_t B) {
 }
 
 static size_t e8_part_bytes(int64_t m_pad, int64_t n_pad, int64_t B) {
-    const int tks = e8_tile_ks(m_pad, n_pad, B, 1);              // stages are combined before the product; one or two
-                                                                 // stages get the most K slots
+    // the many-token kernel: stages are combined before the product (one or two stages get the most K
+    // slots); folded streams take every width the indices take and more, so they bound the size
+    const int tks = e8_tile_ks(m_pad, n_pad, B, 1, true);
+    size_t tile = 0;
     if (tks > 0)                                                 // + the repacked activations
-        return align256((size_t)tks * B * m_pad * sizeof(float)) + align256(glqh_e8_tile_xb_bytes(n_pad, B));
+        tile = align256((size_t)tks * B * m_pad * sizeof(float)) + align256(glqh_e8_tile_xb_bytes(n_pad, B));
+    if (tks > 0 && e8_tile_ks(m_pad, n_pad, B, 1, false) > 0) return tile;
     int ks = glqh_e8_pick_ksplit(m_pad, n_pad, B, 0);
     const int ksf = glqh_e8_pick_ksplit(m_pad, n_pad, B, 1);       // on folded streams
     if (ksf > ks) ks = ksf;
-    return align256((size_t)ks * 4 * B * m_pad * sizeof(float));
+    const size_t plain = align256((size_t)ks * 4 * B * m_pad * sizeof(float));
+    return plain > tile ? plain : tile;
 }
 
 extern "C" size_t glqh_e8_matmul_workspace_bytes(int64_t m_pad, int64_t n_pad, int64_t B) {
@@ -1218,7 +1222,7 @@ extern "C" int glqh_e8_dequant_matmul_folded(const void *x_f16, int64_t B, const
         return 1;
     hipStream_t st = (hipStream_t)stream;
     float *part = (float *)ws;
-    const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n);
+    const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n, folded != nullptr);
     if (tks > 0) {
         const size_t pbytes = align256((size_t)tks * B * m_pad * sizeof(float));
         const size_t need = pbytes + glqh_e8_tile_xb_bytes(n_pad, B);
@@ -1332,7 +1336,7 @@ extern "C" int glqh_fused_linear_e8_folded(const void *x, int x_dtype, int64_t x
     GLQH_REQUIRE(B <= 65535, "fused e8 linear: B=%lld out of range", (long long)B);
     GLQH_REQUIRE(in_features <= n_pad && out_features <= m_pad, "fused e8 linear: features exceed padded dims");
     const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
-    const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n);
+    const int tks = e8_tile_ks(m_pad, n_pad, B, sg.n, folded != nullptr);
     const int ks = tks > 0 ? tks : glqh_e8_pick_ksplit(m_pad, n_pad, B, folded != nullptr);
     const size_t tile_part = align256((size_t)ks * B * m_pad * sizeof(float));
     const size_t need = tks > 0 ? xb + tile_part + glqh_e8_tile_xb_bytes(n_pad, B)

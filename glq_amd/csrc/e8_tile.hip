@@ -634,6 +634,11 @@ struct et_plan {
     int NTW, RT, TT, KS, slot_ds, grid;
 };
 
+// Widths the kernels walk: whole groups of four 64-column steps.  On folded streams a row of any multiple
+// of 32 columns is served: the folded tiles are padded to 32 indices with the zero codeword and the blocked
+// activations to the same width with zeros (the kernel's n_pad is then the padded width).
+static int64_t et_width(int64_t n_pad) { return (n_pad + 255) / 256 * 256; }
+
 int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *p) {
     if (M < 1 || m_pad < 1 || n_pad < 256 || (n_pad & 255) || M > ((int64_t)1 << 22) || m_pad > ((int64_t)1 << 24))
         return 0;
@@ -722,15 +727,23 @@ int et_init_NS() {
 
 int glqh_e8_tile_init(void) { return et_init_NS<1>() || et_init_NS<2>() || et_init_NS<3>() || et_init_NS<4>(); }
 
-// bytes of the repacked activations (the larger tile size bounds the padding)
-size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M) { return (size_t)et_padded_tokens(M, 1) * n_pad * sizeof(f16); }
+// bytes of the repacked activations (the larger tile size bounds the padding; width padded as on folded streams)
+size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M) { return (size_t)et_padded_tokens(M, 1) * et_width(n_pad) * sizeof(f16); }
 
-// K slots of the many-token kernel for this call, or 0 when the shape is not eligible
-// (n_pad must be a multiple of 256)
-int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages) {
+// K slots of the many-token kernel for this call, or 0 when the shape is not eligible: n_pad must be a
+// multiple of 256 on the indices themselves, of 32 on folded streams
+int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, int fold) {
     et_plan p;
+    if (fold && n_pad >= 32 && (n_pad & 31) == 0) n_pad = et_width(n_pad);
     return et_make_plan(m_pad, n_pad, M, nstages, &p) ? p.KS : 0;
 }
+
+namespace {
+__global__ void __launch_bounds__(256) et_zero_kernel(u32x4 *__restrict__ p, int64_t n16) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256)
+        p[i] = u32x4{0u, 0u, 0u, 0u};
+}
+}  // namespace
 
 // part[(slot * M + token) * m_pad + row] = sum over the slot's columns of x[token, k] * W[row, k],
 // W = cb[q0] + rel[0] * cb2[q1] + rel[1] * cb[q2] + rel[2] * cb[q3] (nstages terms), unscaled.
@@ -743,11 +756,21 @@ int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const vo
                         int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold) {
     glqh_range range("dequant_matmul");
     et_plan p;
-    if (!et_make_plan(m_pad, n_pad, M, nstages, &p)) return glqh_fail("e8 tile kernel: shape not eligible (n_pad %% 256)");
+    const int64_t n_cols = n_pad;                              // columns the caller's rows and activations have
+    if (fold && n_pad >= 32 && (n_pad & 31) == 0) n_pad = et_width(n_pad);
+    if (!et_make_plan(m_pad, n_pad, M, nstages, &p))
+        return glqh_fail("e8 tile kernel: shape not eligible (n_pad %% 256, or %% 32 on folded streams)");
+    if (n_pad != n_cols) {                                     // zero activations for the padding columns
+        const int64_t Mp = et_padded_tokens(M, nstages);
+        const int64_t n16 = (n_pad - n_cols) / 32 * Mp * 4;    // 16-byte slots of the k-pairs past the row
+        hipLaunchKernelGGL(et_zero_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0,
+                           stream, (u32x4 *)((f16 *)xb_scratch + n_cols / 32 * Mp * 32), n16);
+        GLQH_LAUNCH_CHECK("e8 tile padding launch");
+    }
     if (x_f16) {                                               // NULL: xb_scratch already holds the blocked layout
-        hipLaunchKernelGGL(e8_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((n_pad / 8 + 15) / 16)),
+        hipLaunchKernelGGL(e8_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((n_cols / 8 + 15) / 16)),
                            dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M,
-                           (int)et_padded_tokens(M, nstages), (int)n_pad);
+                           (int)et_padded_tokens(M, nstages), (int)n_cols);
         GLQH_LAUNCH_CHECK("e8 pack launch");
     }
     et_args a;

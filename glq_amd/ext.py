@@ -51,10 +51,10 @@ E8_FOLD_BATCH_MAX = max(1, int(os.environ.get("GLQ_E8_BATCH_MAX", "4096")))
 
 
 def _e8_dense_route(B, n_pad, folded=False):
-    """Dequantize + library GEMM: on request, and for the widths the tile kernel does not take
-    (n_pad not a multiple of 256) above 16 tokens."""
+    """Dequantize + library GEMM: on request, and above 16 tokens for the widths the tile kernel does
+    not take (n_pad must be a multiple of 32 on folded streams, of 256 on the indices themselves)."""
     limit = max(E8_BATCH_MAX, E8_FOLD_BATCH_MAX) if folded else E8_BATCH_MAX
-    return B > limit or (B > 16 and int(n_pad) % 256 != 0)
+    return B > limit or (B > 16 and int(n_pad) % (32 if folded else 256) != 0)
 
 
 def _p(t):

@@ -257,6 +257,47 @@ def test_fresh_views_of_the_indices_hit_the_one_fold(ext):
     assert not ext._FOLD_STREAMS.holds(stacked[m:])
 
 
+@pytest.mark.parametrize("m,n,B", [(960, 960, 24), (1024, 2080, 70), (520, 4128, 300), (2048, 1056, 17)])
+@pytest.mark.parametrize("stages", [1, 2, 4])
+def test_many_token_products_on_widths_that_are_not_whole_tile_groups(ext, m, n, B, stages):
+    """Rows of any multiple of 32 columns run the tile kernel on folded streams (the folded tiles end in the
+    zero codeword, the blocked activations in zero columns); on the indices themselves such widths go to the
+    dequantize + library route.  Against the oracle's product and against that route."""
+    say("e8 folded tile matmul, ragged width", m, n, B, stages)
+    lib = ext._lib.load()
+    assert n % 256 != 0 and lib.glqh_e8_fold_eligible(m, n, B) == 1
+    q = [t(a) for a in _indices(m, n, stages, m + n + stages)]
+    cb = e8_table_f16()
+    x = torch.randn(B, n, generator=torch.Generator().manual_seed(B)).half().to(DEV)
+    args = dict(qidxs2=q[1] if stages > 1 else None, codebook2=cb, inv_resid_scale=1 / 3.0 if stages > 1 else 0.0,
+                qidxs3=q[2] if stages > 2 else None, inv_resid_scale2=1 / 9.0 if stages > 2 else 0.0,
+                qidxs4=q[3] if stages > 3 else None, inv_resid_scale3=1 / 27.0 if stages > 3 else 0.0)
+    assert ext.e8_prepare(q[0], cb, args["qidxs2"], cb, args["qidxs3"], args["qidxs4"]) > 0
+    y_fold = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)
+    assert torch.equal(y_fold, ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args))
+    ext.E8_FOLD = False
+    try:
+        y_lib = ext.glq_dequant_matmul_cuda(x, q[0], cb, 0.02, **args)      # dequantize + library GEMM
+    finally:
+        ext.E8_FOLD = True
+    assert rel(y_fold, y_lib) < 2e-3
+    W = sum(O.e8_table()[q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)
+            for s in range(stages)).astype(np.float32) * np.float32(0.02)
+    assert rel(y_fold, x.float().cpu().numpy() @ W.T) < TOL
+    # the fused linear (transform writes the blocked layout, zero columns appended) on the same layer
+    from glq_amd import hadamard as H
+    su, sv = O.rht_signs(m, n, 7)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    xb = torch.randn(B, n, generator=torch.Generator().manual_seed(1)).bfloat16().to(DEV)
+    y = ext.glq_fused_linear_block_diag_cuda(
+        xb, t(sv.astype(np.float16)), t(su.astype(np.float16)), q[0], cb, 0.02, n, m, n, m, torch.tensor(bn),
+        torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), args["qidxs2"], cb,
+        args["inv_resid_scale"], args["qidxs3"], cb, args["inv_resid_scale2"], args["qidxs4"], cb,
+        args["inv_resid_scale3"], out_dtype=torch.bfloat16)
+    ref = O.linear_forward_rht(xb.float().cpu().numpy(), W, su.astype(np.float32), sv.astype(np.float32), bn, bm, n, m)
+    assert rel(y, ref) < TOL, rel(y, ref)
+
+
 def test_c_abi_refusals(ext):
     say("e8 fold refusals")
     lib = ext._lib.load()
@@ -268,4 +309,5 @@ def test_c_abi_refusals(ext):
     assert rc != 0 and b"room for 16" in lib.glqh_last_error() and n.value == 1286
     assert lib.glqh_e8_fold_eligible(960, 960, 1) == 0       # a small layer: the gather kernel serves it
     assert lib.glqh_e8_fold_eligible(4096, 14336, 17) == 1   # the tile kernel reads them too ...
-    assert lib.glqh_e8_fold_eligible(4096, 14336 + 8, 17) == 0   # ... on rows of whole 256-column groups
+    assert lib.glqh_e8_fold_eligible(4096, 14336 + 32, 17) == 1  # ... on rows of any multiple of 32 columns
+    assert lib.glqh_e8_fold_eligible(4096, 14336 + 8, 17) == 0

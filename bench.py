@@ -403,11 +403,15 @@ def extras(torch, ext, dev):
         q1 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
         q2 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
         ext.e8_prepare(q1, cbh, q2, cbh)
-        for M, route in ((256, ""), (4096, ""), (4096, "_compressed")):
-            # "" = the route the library picks (compressed up to 2048 tokens for trellis and, on the folded
-            # streams, 4096 for E8; dequantize + library GEMM above); "_compressed" = the tile kernels forced
-            ext.TRELLIS_BATCH_MAX = (1 << 30) if route else tr_default
-            ext.E8_BATCH_MAX = (1 << 30) if route else e8_default
+        e8_fold_default = ext.E8_FOLD_BATCH_MAX
+        for M, route in ((256, ""), (4096, ""), (4096, "_library"), (8192, ""), (8192, "_compressed")):
+            # "" = the route the library picks (compressed up to 4096 tokens: the tile kernels on the packed
+            # stream / the folded streams; dequantize + library GEMM above); "_library" / "_compressed" = the
+            # other route forced, for the comparison at the threshold and beyond it
+            lim = {"": None, "_library": 64, "_compressed": 1 << 30}[route]
+            ext.TRELLIS_BATCH_MAX = tr_default if lim is None else lim
+            ext.E8_BATCH_MAX = e8_default if lim is None else lim
+            ext.E8_FOLD_BATCH_MAX = e8_fold_default if lim is None else lim
             xb = torch.randn(M, n, device=dev).to(torch.bfloat16)
             us = _graph_time(torch, lambda: ext.glq_fused_linear_trellis_3inst_cuda(
                 xb, sv, su, p, bnt, bmt, bnm, bmm, 0.02, n, m, n, m, out_dtype=torch.bfloat16), 1, reps=5)
@@ -416,6 +420,7 @@ def extras(torch, ext, dev):
                 xb, sv, su, q1, cbh, 0.02, n, m, n, m, bnt, bmt, bnm, bmm, q2, cbh, 1 / 3.0,
                 out_dtype=torch.bfloat16), 1, reps=5)
             out[f"e8_2stage_linear_14336x4096_M{M}{route}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        ext.E8_FOLD_BATCH_MAX = e8_fold_default
         ext.TRELLIS_BATCH_MAX, ext.E8_BATCH_MAX = tr_default, e8_default
         # the same two linears at 32 tokens (a batched decode step): the small-tile kernels
         xb = torch.randn(32, n, device=dev).to(torch.bfloat16)

@@ -8,6 +8,9 @@ the reference's operator surface:
                                 (``glq._C`` / ``glq_cuda``), same names and arguments
 * ``glq_amd.custom_ops``        the ``torch.ops.glq.*`` schemas of ``glq_vllm/custom_ops.py``
 * ``glq_amd.quantized_linear``  ``E8RHTLinear`` with the reference's buffer names
+* ``glq_amd.linear_method``     the serving layer's call sequence for merged trellis linears
+                                (``glq_vllm/linear_method.py``) and the load-time step
+* ``glq_amd.dequant``           dense weights from quantized layers (``glq_vllm/dequant.py``)
 * ``glq_amd.inference_kernel``, ``glq_amd.hadamard``, ``glq_amd.codebook_kernel``,
   ``glq_amd.trellis_step_kernel``  the public functions of the reference's same-named
                                 modules (``glq_dequant_matmul``, ``fast_hadamard_transform``,

@@ -93,3 +93,55 @@ def test_module_buffers_match_the_checkpoint_contract():
         tr2(torch.zeros(1, 128))
     with pytest.raises(NotImplementedError):
         E8RHTLinear(64, 64, codebook_type="e8p")
+
+
+def test_derived_cache_is_keyed_by_memory_not_by_object():
+    """The cache behind the packed tables and the folded index streams (ext._DerivedCache): a fresh view
+    of the same memory hits, an in-place write or another tensor misses, and an entry goes with the
+    storage it was derived from.  (Plain CPU tensors: the cache itself touches no device.)"""
+    import gc
+    from glq_amd import ext
+    c = ext._DerivedCache()
+    base = torch.arange(64, dtype=torch.int16).reshape(8, 8)
+    c.put(base, "folded")
+    assert c.get(base) == "folded" and c.get(base.view(8, 8)) == "folded" and c.get(base[:]) == "folded"
+    assert c.get(base.view(64)) is None                       # another shape: another layer
+    assert c.get(base[2:]) is None and c.get(base.clone()) is None
+    assert c.get(base, ("table-2",)) is None                  # the same indices against another table
+    stacked = torch.zeros(2, 8, 8, dtype=torch.int16)
+    c.put(stacked[1], "shard")
+    assert c.get(stacked[1]) == "shard" and c.get(stacked.view(16, 8)[8:]) == "shard" and c.get(stacked[0]) is None
+    base.add_(1)                                              # written in place: the derived data is stale
+    assert c.get(base) is None
+    c.put(base, "again")
+    assert c.get(base) == "again" and len(c) == 2             # the older version of the same tensor is gone
+    assert c.holds(base) and c.holds(stacked[1]) and not c.holds(stacked[0].clone())
+    del base
+    gc.collect()
+    assert len(c) == 1                                        # dropped with its storage
+    keep = stacked[1]
+    del stacked
+    gc.collect()
+    assert c.get(keep) == "shard"                             # a view keeps the storage, and the entry, alive
+    del keep
+    gc.collect()
+    assert len(c) == 0
+
+
+def test_merged_trellis_linear_host_side():
+    """Shard bookkeeping and refusals of the merged-linear holder that need no GPU."""
+    from glq_amd.linear_method import GLQShards, MergedTrellisLinear, trellis_rvq_recipe
+    assert [trellis_rvq_recipe(b) for b in range(2, 9)] == [[2], [3], [4], [4, 1], [4, 2], [4, 3], [4, 4]]
+    layer = MergedTrellisLinear(2048, [2048, 512, 512], bpw=4)
+    assert layer.glq_is_fused and layer.glq_num_shards == 3 and layer.glq_n_pad == 2048
+    assert len(layer.SU) == 3 and layer.SU.get_shard(1).shape == (512,) and layer.SV.get_shard(2).shape == (2048,)
+    assert layer.trellis_packed.get_shard(0).numel() == 0     # nothing loaded yet
+    single = MergedTrellisLinear(512, [256])
+    assert not single.glq_is_fused
+    import pytest
+    with pytest.raises(RuntimeError, match="process_weights_after_loading"):
+        layer.apply(torch.zeros(1, 2048))
+    with pytest.raises(RuntimeError, match="trellis layers"):
+        MergedTrellisLinear.from_linears([])
+    sh = GLQShards([torch.zeros(1), torch.ones(2)])
+    assert len(sh) == 2 and sh.get_shard(1).numel() == 2

@@ -1,0 +1,139 @@
+"""Seeded sweeps over layer shapes, rates and token counts that straddle every route switch of the fused
+linears (fused-input GEMV, small-batch MFMA kernel, small and large tile kernels, K slots, block-diagonal
+transforms of odd sizes), each against the oracle's fp32 CPU forward within the 1e-2 bound, plus the
+many-token paths that only large layers reach (fp16 sums, the tail-round launch) through their properties
+(needs an MI355X)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import glq_oracle as O
+from tests.gpu_util import DEV, e8_table_f16, rel, say, t
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+TOKENS = [1, 2, 3, 4, 5, 8, 16, 17, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 257, 300]
+
+
+def _trellis_cases():
+    rng = np.random.default_rng(2024)
+    cases = []
+    for i in range(36):
+        m = int(rng.integers(1, 40)) * 32
+        n = int(rng.integers(1, 48)) * 64
+        K = int(rng.integers(2, 5))
+        K2 = int(rng.choice([0, 0, 1, 2, 3, 4]))
+        B = TOKENS[(i * 7) % len(TOKENS)]
+        cases.append((m, n, K, K2, B, i))
+    return cases
+
+
+@pytest.mark.parametrize("m,n,K,K2,B,seed", _trellis_cases())
+def test_trellis_fused_linear_random_shapes(m, n, K, K2, B, seed):
+    from glq_amd import ext, hadamard as H
+    say("random trellis", m, n, K, K2, B)
+    su, sv = O.rht_signs(m, n, 300 + seed)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"trellis_packed": O.random_packed(m, n, K, seed), "SU": su.astype(np.float16), "SV": sv.astype(np.float16),
+           "Wscale": np.float32(0.02), "blocks_m": bm, "blocks_n": bn}
+    if K2:
+        art["trellis_packed2"] = O.random_packed(m, n, K2, 1000 + seed)
+        art["inv_resid_scale2"] = np.float32(0.25)
+    dtype = torch.bfloat16 if seed % 2 else torch.float16
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(seed)) * 0.7).to(dtype)
+    ref = O.trellis_linear_forward(x.float().numpy(), art, n, m)
+    meta = (torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV))
+    if K2:
+        y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+            x.to(DEV), t(art["SV"]), t(art["SU"]), t(art["trellis_packed"]), t(art["trellis_packed2"]), *meta, 0.02, 0.25,
+            n, m, n, m, out_dtype=dtype)
+    else:
+        y = ext.glq_fused_linear_trellis_3inst_cuda(x.to(DEV), t(art["SV"]), t(art["SU"]), t(art["trellis_packed"]), *meta,
+                                                    0.02, n, m, n, m, out_dtype=dtype)
+    assert y.shape == (B, m) and y.dtype == dtype
+    e = rel(y, ref)
+    assert e < TOL, e
+
+
+def _e8_cases():
+    rng = np.random.default_rng(77)
+    cases = []
+    for i in range(30):
+        m = int(rng.integers(1, 300)) * (8 if i % 3 else 1)
+        n = int(rng.integers(1, 300)) * 8 if i % 4 else int(rng.integers(1, 12)) * 256
+        stages = int(rng.integers(1, 5))
+        B = TOKENS[(i * 11) % len(TOKENS)]
+        cases.append((m, n, stages, B, i))
+    return cases
+
+
+@pytest.mark.parametrize("m,n,stages,B,seed", _e8_cases())
+def test_e8_fused_linear_random_shapes(m, n, stages, B, seed):
+    """Rows and widths that are not multiples of anything but 8 columns, 1-4 stages, prepared (folded where
+    the kernels take it) and not."""
+    from glq_amd import ext, hadamard as H
+    say("random e8", m, n, stages, B)
+    rng = np.random.default_rng(seed)
+    q = [rng.integers(0, 65536, size=(m, n // 8)).astype(np.uint16).view(np.int16) for _ in range(stages)]
+    inv = [1 / 3.0, 1 / 9.0, 1 / 27.0]
+    su, sv = O.rht_signs(m, n, 500 + seed)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    art = {"Qidxs": q[0], "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.015),
+           "blocks_m": bm, "blocks_n": bn}
+    W = O.e8_dequant(q[0], q[1] if stages > 1 else None, inv[0] if stages > 1 else 0.0, q[2] if stages > 2 else None,
+                     inv[1] if stages > 2 else 0.0, q[3] if stages > 3 else None, inv[2] if stages > 3 else 0.0)
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(seed)) * 0.7).to(torch.bfloat16)
+    ref = O.linear_forward_rht(x.float().numpy(), W * np.float32(0.015), su.astype(np.float32), sv.astype(np.float32),
+                               bn, bm, n, m)
+    cb = e8_table_f16()
+    d = [t(a) for a in q] + [None] * (4 - stages)
+    if seed % 2 == 0:
+        ext.e8_prepare(d[0], cb, d[1], cb, d[2], d[3])
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)       # the unprepared half runs on its indices, by design
+        y = ext.glq_fused_linear_block_diag_cuda(
+            x.to(DEV), t(art["SV"]), t(art["SU"]), d[0], cb, 0.015, n, m, n, m, torch.tensor(bn), torch.tensor(bm),
+            H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), d[1], cb, inv[0] if stages > 1 else 0.0,
+            d[2], cb, inv[1] if stages > 2 else 0.0, d[3], cb, inv[2] if stages > 3 else 0.0, out_dtype=torch.bfloat16)
+    assert y.shape == (B, m)
+    e = rel(y, ref)
+    assert e < TOL, e
+
+
+@pytest.mark.parametrize("m,n,M,K", [(14336, 512, 4096, 4), (14336, 256, 4096, 2), (11008, 512, 8192, 3)])
+def test_many_token_trellis_paths_of_large_layers(m, n, M, K):
+    """Tile counts that trigger the tail-round launch (896 = 3.5 rounds, 1376 = 5.4 rounds of 256 CUs) on
+    narrow layers, so that the oracle stays cheap: sampled rows of every token tile and of both launches' row
+    ranges against the oracle; the fused linear (fp16 sums between tile kernel and output transform) against
+    the unfused pipeline (fp32 sums) on all rows; repeated runs bit-identical."""
+    from glq_amd import ext, hadamard as H
+    say("many-token trellis", m, n, M, K)
+    packed = O.random_packed(m, n, K, 5)
+    su, sv = O.rht_signs(m, n, 9)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    meta = (torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV))
+    x = (torch.randn(M, n, generator=torch.Generator().manual_seed(3)) * 0.7).to(torch.bfloat16)
+    xd, pd, sud, svd = x.to(DEV), t(packed), t(su.astype(np.float16)), t(sv.astype(np.float16))
+    old = ext.TRELLIS_BATCH_MAX
+    ext.TRELLIS_BATCH_MAX = 1 << 30
+    try:
+        y = ext.glq_fused_linear_trellis_3inst_cuda(xd, svd, sud, pd, *meta, 0.02, n, m, n, m, out_dtype=torch.bfloat16)
+        assert torch.equal(y, ext.glq_fused_linear_trellis_3inst_cuda(xd, svd, sud, pd, *meta, 0.02, n, m, n, m,
+                                                                      out_dtype=torch.bfloat16))
+    finally:
+        ext.TRELLIS_BATCH_MAX = old
+    rows = np.unique(np.concatenate([np.arange(0, M, 509), [M - 1, 255, 256, 511, 512]]))
+    art = {"trellis_packed": packed, "SU": su.astype(np.float16), "SV": sv.astype(np.float16), "Wscale": np.float32(0.02),
+           "blocks_m": bm, "blocks_n": bn}
+    ref = O.trellis_linear_forward(x[rows].float().numpy(), art, n, m)
+    assert rel(y[torch.from_numpy(rows).to(DEV)], ref) < TOL
+    # the unfused pipeline keeps fp32 sums: input transform, matmul entry, output transform
+    x_rht = torch.empty(M, n, dtype=torch.float16, device=DEV)
+    ext.glq_input_rht_blockdiag_cuda(xd, svd, x_rht, n, n, meta[0], meta[2])
+    y_rht = ext.glq_decode_matmul_trellis_3inst_cuda(x_rht, pd, m, n, 0.02)
+    y2 = torch.empty(M, m, dtype=torch.bfloat16, device=DEV)
+    ext.glq_output_rht_blockdiag_cuda(y_rht, sud, y2, m, m, meta[1], meta[3])
+    assert rel(y, y2.float().cpu().numpy()) < 4e-3
+    # every row range of the two launches is written: no row of the output is left at its initial value
+    assert bool(torch.isfinite(y.float()).all()) and float(y.float().abs().sum(0).min()) > 0.0

@@ -475,8 +475,12 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     // folded form grows by a quarter per extra token and the separate one hardly at all, so two
     // tokens fold only single power-of-two blocks (10.8 vs 11.3, 14.7 vs 15.8; 960 x 960: 12.7 vs
     // 9.4) and three or four tokens never do (2048 x 2048: 13.6 vs 11.5; 8192 x 8192: 38 vs 26).
+    // Checked on other model widths (one token, folded / separate, us: 3072 x 3072 10.4 / 11.3, 4096 x 4096
+    // 12.1 / 15.5, 8192 x 3072 15.2 / 17.3, 2048 x 6144 10.9 / 12.9, 6144 x 2048 11.5 / 12.6, 1536 x 1536 8.1 / 9.3,
+    // 5120 x 5120 17.0 / 15.8 -- the one loss; two tokens: 4096 x 4096 15.0 / 16.1, but 3072 x 8192 19.3 / 16.2 and
+    // 6144 x 2048 14.7 / 13.2, hence the size bound on two tokens).
     const bool fi_pays = tr_fuse_input_enabled() && m_pad * n_pad <= ((int64_t)32 << 20) &&
-                         (B == 1 || (B == 2 && pow2_n));
+                         (B == 1 || (B == 2 && pow2_n && n_pad <= 4096 && m_pad <= 4096));
     if (fi_pays && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
         (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0 &&
         (!has_s2 || (B == 1 && fi_mode == 2 && merge2))) {

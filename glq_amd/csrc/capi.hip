@@ -609,8 +609,14 @@ static bool tr_group_plain(int64_t total_m_pad, int64_t n_pad, int64_t B) {
     const int64_t w = total_m_pad * n_pad;
     // q/k/v of a 4096-wide model (25M weights): 22.1 / 25.6 / 28.5 us folded at 2 / 3 / 4 tokens,
     // 24.5 / 24.5 / 25.1 us separate; gate/up 2048 -> 2 x 11008 (45M): 19-22 us folded, 25-26 separate
+    // Checked on nine other groups (q/k/v and gate/up of 2048- to 8192-wide models, 1-4 tokens, folded /
+    // separate, us): one token folds with a gain of 5-8 us up to 50M weights (gate/up 3072 -> 2 x 8192: 18.1 /
+    // 24.4) and loses above 96M (4096 -> 2 x 14336: 37.4 / 33.9; 8192 -> 2 x 28672: 103.9 / 92.3; 5120 -> 2 x 13824
+    // ties); three and four tokens on q/k/v of a 3072-wide model lose 1-4 us folded (21.7 / 20.5, 24.4 / 20.2),
+    // which the rule below does not catch.
     if (!tr_fuse_input_enabled()) return true;
-    return B >= 2 && (w > ((int64_t)48 << 20) || (B >= 3 && n_pad >= 4096 && w > ((int64_t)16 << 20)));
+    if (B == 1) return w > ((int64_t)96 << 20);
+    return w > ((int64_t)48 << 20) || (B >= 3 && n_pad >= 4096 && w > ((int64_t)16 << 20));
 }
 static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {
     int64_t total = 0;

@@ -435,7 +435,7 @@ def extras(torch, ext, dev):
         out["prefill_linear_error"] = f"{type(e).__name__}: {e}"
     try:
         args, routes_for, per_slot_bytes = moe_setup(torch, dev)
-        for T in (1, 16, 128):                                # 8 / 128 slots per expert stream, 1024 grouped by expert
+        for T in (1, 16, 128, 256):                           # 8 / 128 slots per expert stream, 1024 / 2048 grouped by expert
             xb, routes = routes_for(T)
             us = _graph_time(torch, lambda: [ext.glq_fused_moe_trellis_3inst_cuda(xb, i, w, *args) for i, w in routes],
                              len(routes))
@@ -450,7 +450,7 @@ def extras(torch, ext, dev):
 
 
 CASES = ("trellis_gemv_16384", "e8_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
-         "e8_prefill_256", "e8_prefill_32", "trellis_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128")
+         "e8_prefill_256", "e8_prefill_32", "trellis_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128", "moe_experts_256")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 

@@ -493,12 +493,95 @@ struct tr_moe_group_args {
     int n_slots, x_div;
 };
 
-template <int R>
-__global__ void __launch_bounds__(TR_THREADS)
-tr_mma_moe_grouped_kernel(tr_moe_group_args g, const f16 *__restrict__ x, int m, int k, int S, int CH) {
-    extern __shared__ u32x4 xs_lds[];
-    __shared__ int slotmap[16];
+// One pass over the K slot for NT tiles of 16 of the expert's rows, positions [t0, t0 + 16 NT) of its run in perm.
+template <int R, int NT>
+__device__ __forceinline__ void moe_group_pass(const tr_moe_group_args &g, const f16 *__restrict__ x, int m, int k,
+                                               int kp0, int kp1, int CH, const uint8_t *lane_base, const mma_lane a,
+                                               int wave, int o0, int cnt, int t0, float pscale, int kslot,
+                                               u32x4 *xs_lds, int *slotmap) {
     constexpr int TPS = mma_tps<16>();
+    constexpr int REC = 4 * R;
+    constexpr int G = mma_red_groups<NT>();                      // row groups per round of the final sum
+    constexpr int PER_WAVE = G * NT * 256;
+    uint32_t *xs = (uint32_t *)xs_lds;
+    float *red = (float *)xs_lds;                                // [TR_WAVES][G][NT][4][64]
+    __syncthreads();                                             // the previous pass is done with slotmap and red
+    if (threadIdx.x < 16 * NT)
+        slotmap[threadIdx.x] = t0 + (int)threadIdx.x < cnt ? g.perm[o0 + t0 + threadIdx.x] : -1;
+    int kp = kp0 + wave;
+    tr_record<R> cur = {};
+    if (kp < kp1) cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
+    mma_acc<NT> acc;
+#pragma unroll
+    for (int sg = 0; sg < 4; ++sg)
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) acc.v[sg][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c0 = kp0; c0 < kp1; c0 += CH) {
+        const int c1 = min(c0 + CH, kp1), n = c1 - c0;
+        fht_barrier<true>();                                     // slotmap written / previous chunk consumed
+        // one item = 32 bytes of one row: columns 16 ks .. 16 ks + 15 of k-pair c0 + u
+        for (int idx = threadIdx.x; idx < 32 * NT * n; idx += TR_THREADS) {
+            const int ks = idx & 1, u = (idx >> 1) % n, tk = (idx >> 1) / n;
+            const int tt = tk >> 4, tl = tk & 15;
+            const int sl = slotmap[tk];
+            const f16 *p = x + (int64_t)(sl < 0 ? 0 : sl / g.x_div) * k + 32 * (c0 + u) + 16 * ks;
+            u32x4 l0 = *(const u32x4 *)p, l1 = *(const u32x4 *)(p + 8);
+            if (sl < 0) l0 = l1 = u32x4{0u, 0u, 0u, 0u};
+            uint32_t *dst = xs + (((((u * NT + tt) * 2 + ks) * 4) * TPS) + tl) * 4;
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq)
+                *(u32x4 *)(dst + qq * TPS * 4) =
+                    u32x4{splat_lo(l0[qq]), splat_hi(l0[qq]), splat_lo(l1[qq]), splat_hi(l1[qq])};
+        }
+        fht_barrier<true>();
+        for (; kp < c1; kp += TR_WAVES) {
+            tr_record<R> nxt = cur;
+            if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
+            acc = mma_record<R, 16, NT>(cur, a.next1, a.next2, xs_lds + ((kp - c0) * NT * 8 + a.q) * TPS + a.tokl, acc);
+            cur = nxt;
+        }
+    }
+    // the four waves' sums in wave order, G row groups per round, then one row of part per (K slot, slot)
+#pragma unroll
+    for (int s0 = 0; s0 < 4; s0 += G) {
+        __syncthreads();
+        {
+            const int cl = a.q * 16 + a.tokl;
+#pragma unroll
+            for (int sg = 0; sg < G; ++sg)
+#pragma unroll
+                for (int tt = 0; tt < NT; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        red[wave * PER_WAVE + ((sg * NT + tt) * 4 + r) * 64 + cl] = acc.v[s0 + sg][tt][r];
+        }
+        __syncthreads();
+        for (int i2 = threadIdx.x; i2 < PER_WAVE; i2 += TR_THREADS) {
+            const int cl = i2 & 63, r = (i2 >> 6) & 3, tt = (i2 >> 8) % NT, sg = (i2 >> 8) / NT;
+            const int i = 4 * (cl >> 4) + r;
+            const int row = 64 * blockIdx.x + 32 * (i >> 3) + (i & 7) + 8 * (s0 + sg);
+            const int sl = slotmap[16 * tt + (cl & 15)];
+            if (sl < 0 || row >= m) continue;
+            float v = red[i2];
+#pragma unroll
+            for (int w = 1; w < TR_WAVES; ++w) v += red[w * PER_WAVE + i2];
+            g.part[((int64_t)kslot * g.n_slots + sl) * m + row] = pscale * v;
+        }
+    }
+}
+
+// Chunk lengths (k-pairs staged per barrier pair) of the passes with one, two and four row tiles.
+struct moe_chunks {
+    int ch1, ch2, ch4;
+};
+
+// WIDE = false: passes of 16 rows only (few rows per expert: the registers of the wide passes would cost
+// occupancy for nothing).
+template <int R, bool WIDE>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_moe_grouped_kernel(tr_moe_group_args g, const f16 *__restrict__ x, int m, int k, int S, moe_chunks ch) {
+    extern __shared__ u32x4 xs_lds[];
+    __shared__ int slotmap[64];
     const int e = blockIdx.z;
     const int o0 = g.offs[e], cnt = g.offs[e + 1] - o0;
     if (cnt <= 0) return;                                        // uniform over the workgroup
@@ -515,62 +598,19 @@ tr_mma_moe_grouped_kernel(tr_moe_group_args g, const f16 *__restrict__ x, int m,
     const int mp = min(2 * (int)blockIdx.x + a.hm, mpairs - 1);
     constexpr int REC = 4 * R;
     const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
-    uint32_t *xs = (uint32_t *)xs_lds;
-    float *red = (float *)xs_lds;                                // [TR_WAVES][4 row groups][4][64]
 
-    for (int t0 = 0; t0 < cnt; t0 += 16) {
-        __syncthreads();                                         // the previous tile is done with slotmap and red
-        if (threadIdx.x < 16) slotmap[threadIdx.x] = t0 + (int)threadIdx.x < cnt ? g.perm[o0 + t0 + threadIdx.x] : -1;
-        int kp = kp0 + wave;
-        tr_record<R> cur = {};
-        if (kp < kp1) cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
-        mma_acc<1> acc;
-#pragma unroll
-        for (int sg = 0; sg < 4; ++sg) acc.v[sg][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int c0 = kp0; c0 < kp1; c0 += CH) {
-            const int c1 = min(c0 + CH, kp1), n = c1 - c0;
-            fht_barrier<true>();                                 // slotmap written / previous chunk consumed
-            // one item = 32 bytes of one row: columns 16 ks .. 16 ks + 15 of k-pair c0 + u
-            for (int idx = threadIdx.x; idx < 32 * n; idx += TR_THREADS) {
-                const int ks = idx & 1, u = (idx >> 1) % n, tl = (idx >> 1) / n;
-                const int sl = slotmap[tl];
-                const f16 *p = x + (int64_t)(sl < 0 ? 0 : sl / g.x_div) * k + 32 * (c0 + u) + 16 * ks;
-                u32x4 l0 = *(const u32x4 *)p, l1 = *(const u32x4 *)(p + 8);
-                if (sl < 0) l0 = l1 = u32x4{0u, 0u, 0u, 0u};
-                uint32_t *dst = xs + ((((u * 2 + ks) * 4) * TPS) + tl) * 4;
-#pragma unroll
-                for (int qq = 0; qq < 4; ++qq)
-                    *(u32x4 *)(dst + qq * TPS * 4) =
-                        u32x4{splat_lo(l0[qq]), splat_hi(l0[qq]), splat_lo(l1[qq]), splat_hi(l1[qq])};
-            }
-            fht_barrier<true>();
-            for (; kp < c1; kp += TR_WAVES) {
-                tr_record<R> nxt = cur;
-                if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
-                acc = mma_record<R, 16, 1>(cur, a.next1, a.next2, xs_lds + ((kp - c0) * 8 + a.q) * TPS + a.tokl, acc);
-                cur = nxt;
-            }
-        }
-        // the four waves' sums in wave order, then one row of part per (K slot, slot)
-        __syncthreads();
-        {
-            const int cl = a.q * 16 + a.tokl;
-#pragma unroll
-            for (int sg = 0; sg < 4; ++sg)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) red[wave * 1024 + (sg * 4 + r) * 64 + cl] = acc.v[sg][0][r];
-        }
-        __syncthreads();
-        for (int i2 = threadIdx.x; i2 < 1024; i2 += TR_THREADS) {
-            const int cl = i2 & 63, r = (i2 >> 6) & 3, sg = i2 >> 8;
-            const int i = 4 * (cl >> 4) + r;
-            const int row = 64 * blockIdx.x + 32 * (i >> 3) + (i & 7) + 8 * sg;
-            const int sl = slotmap[cl & 15];
-            if (sl < 0 || row >= m) continue;
-            float v = red[i2];
-#pragma unroll
-            for (int w = 1; w < TR_WAVES; ++w) v += red[w * 1024 + i2];
-            g.part[((int64_t)kslot * g.n_slots + sl) * m + row] = pscale * v;
+    // The stream is read once per pass: as many of the expert's rows per pass as there are, up to 64.
+    for (int t0 = 0; t0 < cnt;) {
+        const int rem = WIDE ? cnt - t0 : 0;
+        if (rem > 32) {
+            moe_group_pass<R, 4>(g, x, m, k, kp0, kp1, ch.ch4, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap);
+            t0 += 64;
+        } else if (rem > 16) {
+            moe_group_pass<R, 2>(g, x, m, k, kp0, kp1, ch.ch2, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap);
+            t0 += 32;
+        } else {
+            moe_group_pass<R, 1>(g, x, m, k, kp0, kp1, ch.ch1, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap);
+            t0 += 16;
         }
     }
 }
@@ -635,7 +675,8 @@ template <int R>
 int mma_init_R() {
     return mma_set_lds(tr_mma_kernel<R, 1, 1>) || mma_set_lds(tr_mma_kernel<R, 4, 1>) ||
            mma_set_lds(tr_mma_kernel<R, 16, 1>) || mma_set_lds(tr_mma_kernel<R, 16, 2>) ||
-           mma_set_lds(tr_mma_kernel<R, 16, 4>) || mma_set_lds(tr_mma_moe_grouped_kernel<R>);
+           mma_set_lds(tr_mma_kernel<R, 16, 4>) || mma_set_lds(tr_mma_moe_grouped_kernel<R, false>) ||
+           mma_set_lds(tr_mma_moe_grouped_kernel<R, true>);
 }
 
 }  // namespace
@@ -802,6 +843,15 @@ int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes,
     return glqh_fail("routed experts: R (bits/weight) 1-4, got %d", R);
 }
 
+static int moe_wide_min_rows() {                                // GLQ_MOE_WIDE_MIN_ROWS: average rows per expert
+    static const int v = [] {
+        const char *e = getenv("GLQ_MOE_WIDE_MIN_ROWS");
+        const int n = e ? atoi(e) : 12;
+        return n < 1 ? 1 : n;
+    }();
+    return v;
+}
+
 // One projection of all routed experts, rows grouped by expert: part[K slot][slot][row].
 int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes, int R, const int *perm,
                                         const int *offs, int n_slots, int n_experts, int x_div,
@@ -811,15 +861,30 @@ int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes
     GLQH_REQUIRE(n_experts >= 1 && n_experts <= 65535 && n_slots >= 1 && x_div >= 1,
                  "routed experts: %d experts (1..65535), %d slots", n_experts, n_slots);
     GLQH_REQUIRE(S >= 1 && ksplit >= 1 && (int64_t)S * ksplit >= k / 32, "routed experts: K plan does not cover the row");
-    int CH = mma_chunk_cap<16, 1>();
-    if (CH > S) CH = (S + 3) & ~3;
-    size_t lds = (size_t)CH * mma_slot_bytes(16, 1);
-    if (lds < (size_t)TR_WAVES * 1024 * sizeof(float)) lds = (size_t)TR_WAVES * 1024 * sizeof(float);
+    // Wide passes from an average of 12 rows per expert on (a third of the experts then has more than 16).
+    const bool wide = (int64_t)n_slots >= (int64_t)moe_wide_min_rows() * n_experts;
+    // chunk of the one-tile pass as in tr_mma_kernel; the wider passes take what the same LDS holds
+    moe_chunks ch;
+    ch.ch1 = mma_chunk_cap<16, 1>();
+    ch.ch2 = std::max(4, (ch.ch1 / 2) & ~3);
+    ch.ch4 = std::max(4, (ch.ch1 / 4) & ~3);
+    const int s4 = (S + 3) & ~3;
+    ch.ch1 = std::min(ch.ch1, s4);
+    ch.ch2 = std::min(ch.ch2, s4);
+    ch.ch4 = std::min(ch.ch4, s4);
+    size_t lds = std::max({(size_t)ch.ch1 * mma_slot_bytes(16, 1), (size_t)ch.ch2 * mma_slot_bytes(16, 2),
+                           (size_t)ch.ch4 * mma_slot_bytes(16, 4), (size_t)mma_red_bytes<16, 4>()});
     tr_moe_group_args g = {(const uint8_t *)packed, stride_bytes, perm, offs, pscale_dev, part, n_slots, x_div};
     const dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, (unsigned)n_experts);
 #define GLQH_MOEG(RR)                                                                                        \
-    hipLaunchKernelGGL((tr_mma_moe_grouped_kernel<RR>), grid, dim3(TR_THREADS), lds, stream, g, (const f16 *)x_f16, \
-                       (int)m, (int)k, S, CH)
+    do {                                                                                                     \
+        if (wide)                                                                                            \
+            hipLaunchKernelGGL((tr_mma_moe_grouped_kernel<RR, true>), grid, dim3(TR_THREADS), lds, stream, g, \
+                               (const f16 *)x_f16, (int)m, (int)k, S, ch);                                    \
+        else                                                                                                 \
+            hipLaunchKernelGGL((tr_mma_moe_grouped_kernel<RR, false>), grid, dim3(TR_THREADS), lds, stream, g, \
+                               (const f16 *)x_f16, (int)m, (int)k, S, ch);                                    \
+    } while (0)
     switch (R) {
     case 1: GLQH_MOEG(1); break;
     case 2: GLQH_MOEG(2); break;

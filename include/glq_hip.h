@@ -240,7 +240,8 @@ size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int64_t top_k,
  * torch.ops.glq.fused_moe_trellis_3inst (glq_vllm/custom_ops.py:22-36).  With few (token,
  * choice) slots every slot is one fused-input GEMV on its expert's stream; from
  * max(16, 3/4 num_experts) slots on a routing launch groups the slots by expert and every
- * expert's stream is read once per 16 of its rows (GLQ_MOE_GROUP_MIN sets that count).
+ * expert's stream is read once per 16 of its rows (GLQ_MOE_GROUP_MIN sets that count), once
+ * per up to 64 rows from an average of 12 rows per expert on (GLQ_MOE_WIDE_MIN_ROWS).
  * Intermediate results are rounded to
  * fp16 where the reference rounds them (after each output transform and after the
  * activation), the weighted sum runs over the choices in order in fp32.  activation_type:

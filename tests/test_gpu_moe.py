@@ -206,10 +206,13 @@ def test_refusals(ext):
         ext.glq_fused_moe_trellis_3inst_cuda(x, ids, w, *b)
 
 
-@pytest.mark.parametrize("hidden,inter,T,K,K2", [(256, 128, 16, 4, 0), (320, 192, 40, 2, 0), (320, 192, 33, 3, 2)])
+@pytest.mark.parametrize("hidden,inter,T,K,K2", [(256, 128, 16, 4, 0), (320, 192, 40, 2, 0), (320, 192, 33, 3, 2),
+                                                 (256, 128, 24, 4, 0), (256, 128, 90, 2, 0), (256, 128, 80, 3, 1)])
 def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     """From max(16, 3/4 of the experts) slots on the rows are grouped by expert.  Skewed routing: every token's first choice is
-    expert 2 (more than two tiles of 16 rows for it), expert 5 gets nothing, some ids are out of range."""
+    expert 2 (more than two tiles of 16 rows for it), expert 5 gets nothing, some ids are out of range.  From an
+    average of 12 rows per expert on, a pass over an expert's stream takes up to 64 of its rows: the cases give
+    expert 2 one pass of 16 (T = 16), of 32 (24), of 64 (33, 40), 64 + 32 (90) and 64 + 16 (80) rows."""
     say("moe grouped", hidden, inter, T, K, K2)
     ex = experts(6, hidden, inter, 4, K2, seed=2)
     rng = np.random.default_rng(T)
@@ -227,19 +230,20 @@ def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     assert torch.equal(y, ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a))
 
 
-@pytest.mark.parametrize("group_min", ["1", "1000000"])
-def test_both_forms_on_every_case_in_a_fresh_process(group_min):
+@pytest.mark.parametrize("group_min,wide_min", [("1", "1"), ("1", "1000000"), ("1000000", "12")])
+def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min):
     """GLQ_MOE_GROUP_MIN (read once by the library) moves the slot count from which rows are grouped by
     expert: with 1 every case of this file runs in the grouped form, with 1000000 in the per-slot form,
-    each against the oracle, in a process of its own."""
+    each against the oracle, in a process of its own.  GLQ_MOE_WIDE_MIN_ROWS moves the average number of rows
+    per expert from which the grouped form takes up to 64 rows per pass: 1 = always, 1000000 = never."""
     import os
     import subprocess
     import sys
-    say("moe forms, child process", group_min)
+    say("moe forms, child process", group_min, wide_min)
     r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu",
                         "-k", "not fresh_process", "--timeout", "300", "--timeout-method", "thread",
                         "-p", "no:cacheprovider"],
-                       env={**os.environ, "GLQ_MOE_GROUP_MIN": group_min}, capture_output=True, text=True, timeout=900,
+                       env={**os.environ, "GLQ_MOE_GROUP_MIN": group_min, "GLQ_MOE_WIDE_MIN_ROWS": wide_min}, capture_output=True, text=True, timeout=900,
                        cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
 

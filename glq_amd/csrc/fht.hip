@@ -3,6 +3,7 @@
 // One workgroup transforms one power-of-two sub-block of one token in fp32 and
 // multiplies once with 1/sqrt(bs) (glq/hadamard.py:10-28, glq/csrc/glq_fht.cuh:14-21,
 // glq/csrc/glq_cuda.cu:1756-1839, 2005-2079, 2092-2208).
+#include <algorithm>
 #include "common.h"
 #include "fht_device.h"
 
@@ -147,6 +148,34 @@ __device__ __forceinline__ void reg_gather_runs(float (&v)[E], int log_len, floa
     }
 }
 
+// What a thread of a whole-block workgroup does.  Blocks of 1024 points and more: one token (row) per
+// workgroup, thread te = tid.  Blocks of at most 512 points are transformed inside one wave (eight elements
+// per thread, no exchange through LDS), so a workgroup takes 4096 / bs tokens at once: thread tid works on
+// token tid / (bs / 8) of them as thread te = tid % (bs / 8), with staging space of its own.
+struct wide_role {
+    int te, tok, nthr, lds_off;                              // tok: the token's number inside the workgroup
+    bool active;                                             // false: past the workgroup's tokens
+};
+
+__device__ __forceinline__ wide_role wide_role_of(const rht_slice &blk, int ntok) {
+    wide_role r;
+    const int tid = threadIdx.x;
+    if (blk.log_bs > 9) {
+        r.te = tid; r.tok = 0; r.nthr = REG_THREADS; r.lds_off = 0; r.active = true;
+    } else {
+        const int lthr = blk.log_bs - 3;
+        r.te = tid & ((1 << lthr) - 1);
+        r.tok = tid >> lthr;
+        r.nthr = 1 << lthr;
+        r.lds_off = r.tok * (blk.bs + (blk.bs >> 3) + 8);
+        r.active = r.tok < ntok;
+    }
+    return r;
+}
+constexpr int WIDE_SMALL_LOG = 9;                            // blocks up to 512 points: 4096 / bs tokens per workgroup
+// LDS for the staging of a small block's tokens (layout 2: blocks of 32 points and more)
+constexpr size_t WIDE_SMALL_LDS = (size_t)(4096 + 512 + 8 * 128) * sizeof(float);
+
 // LAYOUT of the transformed row: 0 = row-major (out + token * n_pad); 1 and 2 = the tile kernels'
 // operand layouts out[col / 32][token][4][8]: 32 columns of one token are 64 contiguous bytes, as
 // four 8-column blocks in order (1, E8) or as the four slots q = 0..3 holding columns
@@ -155,10 +184,12 @@ template <int E, typename XT, typename OT, int LAYOUT>
 __device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, int64_t x_stride,
                                                    const f16 *__restrict__ sv, OT *__restrict__ out,
                                                    int in_features, int n_pad, int Mp, int token,
-                                                   const rht_slice &blk, float *s) {
-    const int tid = threadIdx.x;
-    const bool active = E * tid < blk.bs;
-    const int i = E * tid;
+                                                   const rht_slice &blk, float *s, const wide_role role) {
+    // te: the thread's number among those of its token; st: the token's staging space in LDS
+    const int tid = threadIdx.x, te = role.te;
+    const bool active = role.active && E * te < blk.bs;
+    float *st = s + role.lds_off;
+    const int i = E * te;
     float v[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = 0.0f;
@@ -187,15 +218,15 @@ __device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, in
         __syncthreads();                                      // the exchange buffer has been read
         if (active) {
 #pragma unroll
-            for (int q = 0; q < E; ++q) s[reg_pad(strided ? tid + q * nthr : E * tid + q)] = v[q] * blk.norm;
+            for (int q = 0; q < E; ++q) st[reg_pad(strided ? te + q * nthr : E * te + q)] = v[q] * blk.norm;
         }
         __syncthreads();
-        for (int p = tid; p < (blk.bs >> 3); p += REG_THREADS) {   // blocks are multiples of 32 columns
+        for (int p = te; role.active && p < (blk.bs >> 3); p += role.nthr) {   // blocks are multiples of 32 columns
             const int kp = p >> 2, q = p & 3;
             float w[8];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const f32x2 t = *(const f32x2 *)(s + reg_pad(32 * kp + 2 * q + 8 * j));
+                const f32x2 t = *(const f32x2 *)(st + reg_pad(32 * kp + 2 * q + 8 * j));
                 w[2 * j] = t[0];
                 w[2 * j + 1] = t[1];
             }
@@ -222,10 +253,13 @@ __device__ __forceinline__ void input_rht_wide_body(const XT *__restrict__ x, in
 }
 
 // blocks of 8192 points take 16 elements per thread, smaller ones 8 (all 512 threads busy on 4096).
-// One-dimensional grid of 8 * ceil(B / 8) * n_blocks workgroups: workgroup L runs on XCD L % 8, and
-// the tokens are dealt out so that XCD r owns tokens r * ceil(B / 8) ..., consecutive ones
-// back to back: in the token-fast layouts the 16-byte pieces of eight consecutive tokens share a
-// 128-byte line, which is then completed inside one L2 instead of written back in eight parts.
+// One-dimensional grid: workgroup L runs on XCD L % 8, XCD r owns tokens r * ceil(B / 8) ..., and the
+// workgroups of an XCD come in sets of eight that take the same block of eight consecutive tokens: in the
+// token-fast layouts the 16-byte pieces of eight consecutive tokens share a 128-byte line, which is then
+// completed inside one L2 instead of written back in eight parts; and the blocks of a row differ in size
+// (11008 = 8192 + 2048 + 512 + 256), so dealing a token's four blocks to neighbouring workgroups, which go
+// to the four shader engines of an XCD in turn, put every 8192-point block on the same engine
+// (4096 x 11008: 112 -> 70 us; rows of one or three blocks: no change).
 template <typename XT, typename OT, int LAYOUT>
 __global__ void __launch_bounds__(REG_THREADS)
 input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
@@ -234,13 +268,29 @@ input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__r
     extern __shared__ float s[];
     const int L = blockIdx.x, per_xcd = (B + 7) >> 3;
     const int j = L >> 3;
-    const int token = (L & 7) * per_xcd + j / n_blocks;
-    if (token >= B || j / n_blocks >= per_xcd) return;        // uniform over the workgroup
-    const rht_slice blk = rht_slice_of(margs, single_norm, j % n_blocks);
+    const int member = j & 7, rest = j >> 3, g = rest / n_blocks;
+    const rht_slice blk = rht_slice_of(margs, single_norm, rest % n_blocks);
+    if (blk.log_bs <= WIDE_SMALL_LOG) {
+        // one workgroup of 4096 / bs / 8 sets takes all their tokens (the eight members in turn, so that the
+        // work reaches every shader engine), the others retire
+        const int lsets = 12 - blk.log_bs - 3;
+        if ((g & ((1 << lsets) - 1)) != 0 || member != ((g >> lsets) & 7)) return;
+        const int t_in = g * 8, tok0 = (L & 7) * per_xcd + t_in;
+        if (t_in >= per_xcd || tok0 >= B) return;
+        const int ntok = min(8 << lsets, min(per_xcd - t_in, B - tok0));
+        const wide_role role = wide_role_of(blk, ntok);
+        input_rht_wide_body<8, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp,
+                                               tok0 + min(role.tok, ntok - 1), blk, s, role);
+        return;
+    }
+    const int t_in = g * 8 + member;                          // token, counted inside the XCD's share
+    const int token = (L & 7) * per_xcd + t_in;
+    if (token >= B || t_in >= per_xcd) return;                // uniform over the workgroup
+    const wide_role role = wide_role_of(blk, 1);
     if (blk.log_bs > 12)
-        input_rht_wide_body<16, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s);
+        input_rht_wide_body<16, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s, role);
     else
-        input_rht_wide_body<8, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s);
+        input_rht_wide_body<8, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s, role);
 }
 
 // v = the transformed sums of elements E * tid .. E * tid + E - 1 of block `blk`, row b (before the
@@ -248,8 +298,8 @@ input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__r
 // Every thread of the workgroup calls.
 template <int E>
 __device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysrc &src, int64_t b, int m_pad,
-                                                   const rht_slice &blk, float *s, int tid, bool active) {
-    const int i = E * tid;
+                                                   const rht_slice &blk, float *s, int tid, bool active, int te) {
+    const int i = E * te;
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = 0.0f;
     if (active) {
@@ -296,13 +346,13 @@ __device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysr
 template <int E, typename YT>
 __device__ __forceinline__ void output_rht_wide_body(const glqh_ysrc &src, const f16 *__restrict__ su,
                                                     YT *__restrict__ y, int64_t y_stride, int out_features,
-                                                    int m_pad, const rht_slice &blk, float *s) {
-    const int64_t b = blockIdx.y;
+                                                    int m_pad, const rht_slice &blk, float *s, int64_t b,
+                                                    const wide_role role) {
     const int tid = threadIdx.x;
-    const bool active = E * tid < blk.bs;
+    const bool active = role.active && E * role.te < blk.bs;
     float v[E];
-    output_wide_values<E>(v, src, b, m_pad, blk, s, tid, active);
-    const int row = blk.off + E * tid;
+    output_wide_values<E>(v, src, b, m_pad, blk, s, tid, active, role.te);
+    const int row = blk.off + E * role.te;
     if (active && row < out_features) {
         float f[E];
 #pragma unroll
@@ -324,11 +374,30 @@ __device__ __forceinline__ void output_rht_wide_body(const glqh_ysrc &src, const
 template <typename YT>
 __global__ void __launch_bounds__(REG_THREADS)
 output_rht_wide_kernel(glqh_ysrc src, const f16 *__restrict__ su, YT *__restrict__ y, int64_t y_stride,
-                      int out_features, int m_pad, glqh_meta_args margs, float single_norm) {
+                      int out_features, int m_pad, int B, int n_blocks, glqh_meta_args margs, float single_norm) {
     extern __shared__ float s[];
-    const rht_slice blk = rht_get_slice(nullptr, margs, single_norm, 1, WIDE_LOG_MAX);
-    if (blk.log_bs > 12) output_rht_wide_body<16, YT>(src, su, y, y_stride, out_features, m_pad, blk, s);
-    else output_rht_wide_body<8, YT>(src, su, y, y_stride, out_features, m_pad, blk, s);
+    // Workgroup L runs on XCD L % 8 and, inside it, on shader engine (L / 8) % 4: the 64 workgroups that
+    // follow each other take the same block of 64 consecutive rows, so that the large blocks of a row of
+    // several (11008 = 8192 + 2048 + 512 + 256) reach every engine.  Dealt out block by block, a row of four
+    // blocks put every 8192-point block on the same engine of each XCD: 4096 x 11008 127 -> 72 us.
+    const int L = blockIdx.x, xcd = L & 7, member = (L >> 3) & 7, rest = L >> 6, g = rest / n_blocks;
+    const rht_slice blk = rht_slice_of(margs, single_norm, rest % n_blocks);
+    const int r0 = g * 64 + member * 8;                       // first row of the eight workgroups (member, 0..7)
+    if (blk.log_bs <= WIDE_SMALL_LOG) {
+        // one workgroup of every 4096 / bs rows takes them all (the XCDs in turn), the others retire
+        const int lt = 12 - blk.log_bs, T = 1 << lt;
+        if ((r0 & (T - 1)) != 0 || xcd != ((r0 >> lt) & 7) || r0 >= B) return;
+        const int ntok = min(T, B - r0);
+        const wide_role role = wide_role_of(blk, ntok);
+        output_rht_wide_body<8, YT>(src, su, y, y_stride, out_features, m_pad, blk, s,
+                                    (int64_t)r0 + min(role.tok, ntok - 1), role);
+        return;
+    }
+    const int64_t b = (int64_t)r0 + xcd;
+    if (b >= B) return;                                       // uniform over the workgroup
+    const wide_role role = wide_role_of(blk, 1);
+    if (blk.log_bs > 12) output_rht_wide_body<16, YT>(src, su, y, y_stride, out_features, m_pad, blk, s, b, role);
+    else output_rht_wide_body<8, YT>(src, su, y, y_stride, out_features, m_pad, blk, s, b, role);
 }
 
 template <typename YT, bool PARTS>
@@ -579,10 +648,10 @@ int launch_input_rht_wide(const void *x, int x_dtype, int64_t x_stride, const vo
                           int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
                           const glqh_meta_args &margs, int n_blocks, int64_t max_bs, float rsqrt_n,
                           hipStream_t stream) {
-    const int64_t wgs = 8 * ((B + 7) / 8) * n_blocks;
+    const int64_t wgs = 64 * (((B + 7) / 8 + 7) / 8) * n_blocks;
     GLQH_REQUIRE(wgs <= 2147483647ll, "input_rht: too many blocks");
     const dim3 wgrid((unsigned)wgs);
-    const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
+    const size_t lds = std::max(rht_reg_lds_bytes(ilog2(max_bs)), layout == 2 ? WIDE_SMALL_LDS : (size_t)0);
 #define GLQH_INW_LAUNCH(XT, OT, LAYOUT)                                                             \
     hipLaunchKernelGGL((input_rht_wide_kernel<XT, OT, LAYOUT>), wgrid, dim3(REG_THREADS), lds, stream, \
                        (const XT *)x, x_stride, (const f16 *)sv, (OT *)out, (int)in_features,       \
@@ -729,11 +798,12 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
         const int64_t Bw = ((B >= 32 && m_pad >= 8192) || B > 32) ? 65 : B;
         if (rht_wide_ok(Bw, margs, m_pad, max_bs) && src_ok && aligned16(y) && aligned16(su) &&
             (y_stride * y_size) % 16 == 0) {
-            dim3 wgrid((unsigned)n_blocks, (unsigned)B);
+            dim3 wgrid((unsigned)(64 * ((B + 63) / 64) * n_blocks));
             const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
 #define GLQH_OUTW_LAUNCH(YT)                                                                        \
     hipLaunchKernelGGL((output_rht_wide_kernel<YT>), wgrid, dim3(REG_THREADS), lds, stream, src,    \
-                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, margs, rsqrt_m)
+                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, (int)B, (int)n_blocks, margs, \
+                       rsqrt_m)
             if (y_dtype == GLQH_F16) GLQH_OUTW_LAUNCH(f16);
             else if (y_dtype == GLQH_BF16) GLQH_OUTW_LAUNCH(uint16_t);
             else GLQH_OUTW_LAUNCH(float);
@@ -819,8 +889,9 @@ moe_output_rht_kernel(moe_out_args a, f16 *__restrict__ h, int64_t h_stride, glq
     }
     const glqh_ysrc src = moe_src(a, a.wscale_dev[e]);
     const f16 *su = a.su_base + e * a.m_pad;
-    if (blk.log_bs > 12) output_rht_wide_body<16, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s);
-    else output_rht_wide_body<8, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s);
+    const wide_role role = {(int)threadIdx.x, 0, REG_THREADS, 0, true};   // one row per workgroup
+    if (blk.log_bs > 12) output_rht_wide_body<16, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s, slot, role);
+    else output_rht_wide_body<8, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s, slot, role);
 }
 
 // out[slot][i] = act(h[slot][i]) * h[slot][intermediate + i]: 0 SiLU, 1 GELU (tanh form), 2 squared ReLU

@@ -113,6 +113,10 @@ SIGNATURES = {
     "glqh_trellis_qkv_rope_attn_bf16": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
                 c_i64, c_i64, c_int, c_vp, c_sz, c_vp]),
+    "glqh_trellis_qkv_rope_attn_shared_bf16": (
+        c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64,
+                c_i64, c_i64, c_int, c_vp, c_sz, c_vp, c_sz, c_vp]),
+    "glqh_attn_split_state_bytes": (c_sz, [c_i64, c_i64]),
     "glqh_trellis_gate_up_silu_bf16": (
         c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_vp, c_i64, c_vp, c_vp, c_sz, c_vp]),
 }

@@ -1028,13 +1028,14 @@ extern "C" int glqh_trellis_qkv_rope_store_bf16(const void *x, int64_t in_featur
                                       v_cache, head_dim, max_len, apply_rope, st);
 }
 
-extern "C" int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_features, const glqh_trellis_shard *qkv,
-                                               const int64_t *blocks_n, int64_t n_blocks_n,
-                                               const glqh_block_meta *bn_meta_dev, int64_t n_pad,
-                                               const int64_t *pos, const void *cos_t, const void *sin_t,
-                                               void *k_cache, void *v_cache, void *out, int64_t heads,
-                                               int64_t kv_heads, int64_t head_dim, int64_t max_len,
-                                               int apply_rope, void *ws, size_t ws_bytes, void *stream) {
+extern "C" int glqh_trellis_qkv_rope_attn_shared_bf16(const void *x, int64_t in_features,
+                                                      const glqh_trellis_shard *qkv, const int64_t *blocks_n,
+                                                      int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                                                      int64_t n_pad, const int64_t *pos, const void *cos_t,
+                                                      const void *sin_t, void *k_cache, void *v_cache, void *out,
+                                                      int64_t heads, int64_t kv_heads, int64_t head_dim,
+                                                      int64_t max_len, int apply_rope, void *ws, size_t ws_bytes,
+                                                      void *state, size_t state_bytes, void *stream) {
     GLQH_INIT();
     GLQH_REQUIRE(qkv, "qkv+rope+attention: null pointer");
     hipStream_t st = (hipStream_t)stream;
@@ -1049,7 +1050,19 @@ extern "C" int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_feature
                         ws, ws_bytes, st, &c))
         return 1;
     return glqh_launch_out_rope_attn(c.parts, c.su, c.scale, c.m_pads, c.ks, pos, cos_t, sin_t, k_cache, v_cache,
-                                     out, heads, kv_heads, head_dim, max_len, apply_rope, st);
+                                     out, heads, kv_heads, head_dim, max_len, apply_rope, state, state_bytes, st);
+}
+
+extern "C" int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_features, const glqh_trellis_shard *qkv,
+                                               const int64_t *blocks_n, int64_t n_blocks_n,
+                                               const glqh_block_meta *bn_meta_dev, int64_t n_pad,
+                                               const int64_t *pos, const void *cos_t, const void *sin_t,
+                                               void *k_cache, void *v_cache, void *out, int64_t heads,
+                                               int64_t kv_heads, int64_t head_dim, int64_t max_len,
+                                               int apply_rope, void *ws, size_t ws_bytes, void *stream) {
+    return glqh_trellis_qkv_rope_attn_shared_bf16(x, in_features, qkv, blocks_n, n_blocks_n, bn_meta_dev, n_pad, pos,
+                                                  cos_t, sin_t, k_cache, v_cache, out, heads, kv_heads, head_dim,
+                                                  max_len, apply_rope, ws, ws_bytes, nullptr, 0, stream);
 }
 
 // ---- E8 shell ------------------------------------------------------------------------

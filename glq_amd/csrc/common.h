@@ -218,5 +218,6 @@ int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3
                               const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
                               const void *sin_t, void *k_cache, void *v_cache, void *out, int64_t heads,
                               int64_t kv_heads, int64_t head_dim, int64_t max_len, int apply_rope,
-                              hipStream_t stream);
+                              void *split_state, size_t split_state_bytes, hipStream_t stream);
+int glqh_attn_split_shares(int64_t max_len);
 int glqh_trellis_init(void);

@@ -123,23 +123,31 @@ __device__ __forceinline__ attn_vregs attn_load_v(const uint16_t *__restrict__ V
     return r;
 }
 
-// `first_k`: the thread's first round of keys when the caller has requested it already
-// (attn_load_k(K, threadIdx.x >> 3, last) with last as computed here), else nullptr.
-template <bool NEWROW>
+// FIRST: `first_k` holds the thread's first round of keys, which the caller has requested already
+// (attn_load_k(K, j_lo + threadIdx.x >> 3, last) with last as computed here).
+// Keys j_lo .. j_hi - 1 of the n: the whole row (0, n) or one workgroup's share of it.  With `pbuf` the share's
+// running maximum, sum of exponentials and unnormalised weighted rows go there (2 + D floats, written past the
+// L2 of this XCD for the workgroup that merges the shares) instead of the finished row to `out`.
+constexpr int AT_PART = 2 + 128;
+
+template <bool NEWROW, bool FIRST = false>
 __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__restrict__ K,
                                           const uint16_t *__restrict__ V, int n, const uint16_t *knew,
                                           const uint16_t *vnew, float *sc, float *red,
                                           float (*part)[128], uint16_t *__restrict__ out,
-                                          const attn_kregs *first_k = nullptr) {
+                                          const attn_kregs first_k = {}, int j_lo = 0, int j_hi = -1,
+                                          float *pbuf = nullptr) {
     constexpr int D = 128;
+    if (j_hi < 0) j_hi = n;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int last = NEWROW ? max(n - 2, 0) : n - 1;          // last row that is read from the cache
+    // last row that is read from the cache (row n - 1 comes from knew / vnew when NEWROW)
+    const int last = NEWROW && j_hi == n ? max(n - 2, 0) : j_hi - 1;
     const int sub = threadIdx.x & 7;
     float mx = -3.0e38f;
     // four keys per thread in flight (512 keys per round of the workgroup)
-    for (int j0 = threadIdx.x >> 3; j0 < n; j0 += 4 * (AT_THREADS / 8)) {
+    for (int j0 = j_lo + (threadIdx.x >> 3); j0 < j_hi; j0 += 4 * (AT_THREADS / 8)) {
         attn_kregs kr;
-        if (first_k && j0 == (int)(threadIdx.x >> 3)) kr = *first_k;
+        if (FIRST && j0 == j_lo + (int)(threadIdx.x >> 3)) kr = first_k;
         else kr = attn_load_k(K, j0, last);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -161,8 +169,8 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
             s += __shfl_xor(s, 1, GLQH_WAVE);
             s += __shfl_xor(s, 2, GLQH_WAVE);
             s += __shfl_xor(s, 4, GLQH_WAVE);
-            if (j < n) {
-                if (sub == 0) sc[j] = s;
+            if (j < j_hi) {
+                if (sub == 0) sc[j - j_lo] = s;
                 mx = fmaxf(mx, s);
             }
         }
@@ -171,7 +179,7 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
     // per load and four loads in flight: 256 keys per round of the workgroup.  The first round
     // is requested here, ahead of the softmax, every later one a round ahead of its use.
     const int vr = lane >> 4, vcol = lane & 15;
-    const int vj0 = wave * 4 + vr;
+    const int vj0 = j_lo + wave * 4 + vr;
     attn_vregs vcur = attn_load_v(V, vj0, last);
     mx = wave_max(mx);
     if (lane == 0) red[wave] = mx;
@@ -181,7 +189,7 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
     for (int w = 1; w < AT_WAVES; ++w) mx = fmaxf(mx, red[w]);
     __syncthreads();
     float sum = 0.0f;
-    for (int j = threadIdx.x; j < n; j += AT_THREADS) {
+    for (int j = threadIdx.x; j < j_hi - j_lo; j += AT_THREADS) {
         const float e = __expf(sc[j] - mx);
         sc[j] = e;
         sum += e;
@@ -195,15 +203,15 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
     float a[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) a[e] = 0.0f;
-    for (int j0 = vj0; j0 < n; j0 += 4 * 4 * AT_WAVES) {
+    for (int j0 = vj0; j0 < j_hi; j0 += 4 * 4 * AT_WAVES) {
         attn_vregs vnext = vcur;
-        if (j0 + 4 * 4 * AT_WAVES < n) vnext = attn_load_v(V, j0 + 4 * 4 * AT_WAVES, last);
+        if (j0 + 4 * 4 * AT_WAVES < j_hi) vnext = attn_load_v(V, j0 + 4 * 4 * AT_WAVES, last);
         float pw[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int j = j0 + u * 4 * AT_WAVES;
             if (NEWROW && j == n - 1) vcur.v[u] = *(const u32x4 *)(vnew + 8 * vcol);
-            pw[u] = j < n ? sc[j] : 0.0f;
+            pw[u] = j < j_hi ? sc[j - j_lo] : 0.0f;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
@@ -229,8 +237,47 @@ __device__ __forceinline__ void attn_core(const float *qs, const uint16_t *__res
         float acc = 0.0f;
 #pragma unroll
         for (int w = 0; w < AT_WAVES; ++w) acc += part[w][threadIdx.x];
-        out[threadIdx.x] = f32_to_bf16_bits(acc / tot);
+        if (pbuf) {
+            __hip_atomic_store(pbuf + 2 + threadIdx.x, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (threadIdx.x == 0) {
+                __hip_atomic_store(pbuf, mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(pbuf + 1, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        } else {
+            out[threadIdx.x] = f32_to_bf16_bits(acc / tot);
+        }
     }
+}
+
+// The shares of one head, ns of them, merged by the workgroup that finishes last: every workgroup waits until
+// its own share has left, then adds one to the head's counter; the one that brings it to ns resets it (the
+// state is all zeros again when the launch ends), reads the shares past its L2 and writes the row:
+//   out = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s,  M = max_s m_s, shares in ascending order.
+// Nobody waits for anybody: a workgroup that is not the last simply ends.
+__device__ __forceinline__ void attn_merge_shares(float *hbuf, unsigned int *cnt, int ns, uint16_t *__restrict__ out,
+                                                  int *flag) {
+    constexpr int D = 128;
+    __builtin_amdgcn_s_waitcnt(0);                               // this wave's share has left
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned int before = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int lastone = before + 1u == (unsigned int)ns;
+        if (lastone) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = lastone;
+    }
+    __syncthreads();
+    if (!*flag || threadIdx.x >= D) return;
+    float M = -3.0e38f;
+    for (int s = 0; s < ns; ++s)
+        M = fmaxf(M, __hip_atomic_load(hbuf + s * AT_PART, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    float L = 0.0f, o = 0.0f;
+    for (int s = 0; s < ns; ++s) {
+        const float *pb = hbuf + s * AT_PART;
+        const float w = __expf(__hip_atomic_load(pb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - M);
+        L += w * __hip_atomic_load(pb + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        o += w * __hip_atomic_load(pb + 2 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    out[threadIdx.x] = f32_to_bf16_bits(o / L);
 }
 
 __global__ void __launch_bounds__(AT_THREADS)
@@ -553,12 +600,13 @@ __device__ __forceinline__ rht_slice slice_of_row(int m, int row, int log_slice)
     return blk;
 }
 
+template <bool SHARED>
 __global__ void __launch_bounds__(AT_THREADS)
 out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
                      const uint16_t *__restrict__ cos_t, const uint16_t *__restrict__ sin_t,
                      uint16_t *__restrict__ kc, uint16_t *__restrict__ vc, uint16_t *__restrict__ out, int heads,
                      int kv_heads, int max_len, int apply_rope, float scale, int log_slice, int sc_floats,
-                     int buf_floats) {
+                     int buf_floats, float *split_buf, unsigned int *split_cnt, int split_min) {
     constexpr int D = 128, half = D / 2;
     extern __shared__ float lds[];                 // scores, then the three transform buffers
     __shared__ float qs[D];
@@ -570,6 +618,18 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
     const int64_t p = pos_ptr[0];
     if (p < 0 || p >= max_len) return;             // position outside the cache and the score buffer
     const int n = (int)p + 1;
+    // gridDim.y workgroups per head share the keys once there are split_min of them for each: share s takes
+    // keys [s * chunk, (s + 1) * chunk), the last one the new row as well; a head with one share is finished by
+    // its workgroup alone, exactly as without shares
+    int ns = 1, share = 0, j_lo = 0, j_hi = n;
+    if constexpr (SHARED) {
+        ns = min((int)gridDim.y, max(n / split_min, 1));
+        share = blockIdx.y;
+        if (share >= ns) return;                                // uniform over the workgroup
+        const int chunk = (n + ns - 1) / ns;
+        j_lo = share * chunk;
+        j_hi = min(n, j_lo + chunk);
+    }
     const int tid = threadIdx.x;
     const int grp = tid < 512 ? 0 : tid < 768 ? 1 : 2;         // q | k | v, whole waves each
     const int gt = grp == 0 ? tid : grp == 1 ? tid - 512 : tid - 768;
@@ -603,7 +663,7 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
         for (int q = 0; q < 4; ++q) idx[q] = fht_wave_index<4>(blk.log_len, live ? gt : 0, q);
         stage_partials_quad_n(zq, src, blk, 0, m, gt);
         // the first round of cached keys travels while the transform and the rotation run
-        first_k = attn_load_k(Kh, tid >> 3, max(n - 2, 0));
+        first_k = attn_load_k(Kh, j_lo + (tid >> 3), j_hi == n ? max(n - 2, 0) : j_hi - 1);
         // barriers that wait for LDS only: the key loads stay in flight across them
         fht_wave<4, true, true>(zq, blk.log_len, buf, gt);
         fht_barrier<true>();                       // the exchanges have been read: buf takes the result
@@ -631,7 +691,7 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
             uint16_t *nw = grp == 1 ? knew : vnew;
             nw[d] = o0;
             nw[d + half] = o1;
-            if (h % per == 0) {                                  // one writer per key/value head
+            if (h % per == 0 && share == 0) {                    // one writer per key/value head
                 uint16_t *dst = (grp == 1 ? kc : vc) + ((int64_t)g * max_len + p) * D;
                 dst[d] = o0;
                 dst[d + half] = o1;
@@ -639,7 +699,14 @@ out_rope_attn_kernel(qkv_fin a, int ksplit, const int64_t *__restrict__ pos_ptr,
         }
     }
     fht_barrier<true>();                           // qs, knew, vnew are in LDS
-    attn_core<true>(qs, Kh, Vh, n, knew, vnew, sc, red, part, out + (int64_t)h * D, &first_k);
+    if constexpr (!SHARED) {
+        attn_core<true, true>(qs, Kh, Vh, n, knew, vnew, sc, red, part, out + (int64_t)h * D, first_k);
+    } else {
+        float *hbuf = split_buf + (int64_t)h * gridDim.y * AT_PART;
+        attn_core<true, true>(qs, Kh, Vh, n, knew, vnew, sc, red, part, out + (int64_t)h * D, first_k, j_lo, j_hi,
+                        ns > 1 ? hbuf + share * AT_PART : nullptr);
+        if (ns > 1) attn_merge_shares(hbuf, split_cnt + h, ns, out + (int64_t)h * D, (int *)red);
+    }
 }
 
 // Output head of the decode step: logits[r] = <h, E[r, :]> (bf16 x bf16, fp32 sums) over a
@@ -873,11 +940,27 @@ int glqh_launch_out_rope_store(const float *const part[3], const void *const su[
     return 0;
 }
 
+#ifndef ATTN_SPLIT_MIN
+#define ATTN_SPLIT_MIN 512                                      // keys per share at least
+#endif
+constexpr int ATTN_SPLIT_MAX_HEADS = 256;                       // counters at the head of the state buffer
+
+int glqh_attn_split_shares(int64_t max_len) {
+    const int64_t s = (max_len - 1) / ATTN_SPLIT_MIN;            // a cache of 1024 positions never holds two shares
+    return s < 1 ? 1 : s > 8 ? 8 : (int)s;
+}
+
+extern "C" size_t glqh_attn_split_state_bytes(int64_t heads, int64_t max_len) {
+    if (glqh_attn_split_shares(max_len) == 1) return 0;         // too short for shares: no state needed
+    return ATTN_SPLIT_MAX_HEADS * sizeof(unsigned int) +
+           (size_t)heads * glqh_attn_split_shares(max_len) * AT_PART * sizeof(float);
+}
+
 int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3], const float scale[3],
                               const int64_t m[3], int ksplit, const int64_t *pos, const void *cos_t,
                               const void *sin_t, void *k_cache, void *v_cache, void *out, int64_t heads,
                               int64_t kv_heads, int64_t head_dim, int64_t max_len, int apply_rope,
-                              hipStream_t stream) {
+                              void *split_state, size_t split_state_bytes, hipStream_t stream) {
     GLQH_REQUIRE(pos && k_cache && v_cache && out && ksplit >= 1, "out+rope+attention: bad arguments");
     GLQH_REQUIRE(!apply_rope || (cos_t && sin_t), "out+rope+attention: missing angle tables");
     GLQH_REQUIRE(head_dim == 128, "out+rope+attention: head_dim must be 128, got %lld", (long long)head_dim);
@@ -893,14 +976,32 @@ int glqh_launch_out_rope_attn(const float *const part[3], const void *const su[3
     }
     const int log_slice = 10;
     const int buf_floats = (1 << log_slice) + (1 << log_slice) / 32 + 32;
-    const int sc_floats = (int)((max_len + 31) / 32 * 32);
+    // With a state buffer the keys of a long context are shared by up to eight workgroups per head, each with at
+    // least ATTN_SPLIT_MIN keys: a share then holds fewer than 2 * ATTN_SPLIT_MIN keys or an eighth of the cache.
+    int shares = 1;
+    if (split_state && glqh_attn_split_shares(max_len) > 1) {
+        shares = glqh_attn_split_shares(max_len);
+        GLQH_REQUIRE(split_state_bytes >= glqh_attn_split_state_bytes(heads, max_len) && ((uintptr_t)split_state & 15) == 0,
+                     "out+rope+attention: state buffer of %zu bytes needed (16-byte aligned), got %zu",
+                     glqh_attn_split_state_bytes(heads, max_len), split_state_bytes);
+        GLQH_REQUIRE(heads <= ATTN_SPLIT_MAX_HEADS, "out+rope+attention: at most %d heads with a state buffer", ATTN_SPLIT_MAX_HEADS);
+    }
+    const int64_t longest = shares == 1 ? max_len : std::max<int64_t>(2 * ATTN_SPLIT_MIN, (max_len + shares - 1) / shares);
+    const int sc_floats = (int)((longest + 31) / 32 * 32);
     const size_t lds = (size_t)(sc_floats + 3 * buf_floats) * sizeof(float);
     GLQH_REQUIRE(lds <= 60 * 1024, "out+rope+attention: cache of %lld positions does not fit the score buffer",
                  (long long)max_len);
-    hipLaunchKernelGGL(out_rope_attn_kernel, dim3((unsigned)heads), dim3(AT_THREADS), lds, stream, a, ksplit, pos,
-                       (const uint16_t *)cos_t, (const uint16_t *)sin_t, (uint16_t *)k_cache, (uint16_t *)v_cache,
-                       (uint16_t *)out, (int)heads, (int)kv_heads, (int)max_len, apply_rope,
-                       1.0f / sqrtf((float)head_dim), log_slice, sc_floats, buf_floats);
+    unsigned int *cnt = (unsigned int *)split_state;
+    float *sbuf = split_state ? (float *)((char *)split_state + ATTN_SPLIT_MAX_HEADS * sizeof(unsigned int)) : nullptr;
+#define GLQH_ATTN_LAUNCH(SHARED)                                                                              \
+    hipLaunchKernelGGL(out_rope_attn_kernel<SHARED>, dim3((unsigned)heads, (unsigned)shares), dim3(AT_THREADS), lds, \
+                       stream, a, ksplit, pos, (const uint16_t *)cos_t, (const uint16_t *)sin_t,                  \
+                       (uint16_t *)k_cache, (uint16_t *)v_cache, (uint16_t *)out, (int)heads, (int)kv_heads,      \
+                       (int)max_len, apply_rope, 1.0f / sqrtf((float)head_dim), log_slice, sc_floats, buf_floats, \
+                       sbuf, cnt, ATTN_SPLIT_MIN)
+    if (shares > 1) GLQH_ATTN_LAUNCH(true);
+    else GLQH_ATTN_LAUNCH(false);
+#undef GLQH_ATTN_LAUNCH
     GLQH_LAUNCH_CHECK("out+rope+attention launch");
     return 0;
 }

@@ -14,6 +14,7 @@ captured once in a HIP graph and replayed per token; position and token live on 
 from __future__ import annotations
 
 import ctypes as C
+import os
 import time
 from dataclasses import dataclass
 
@@ -123,16 +124,28 @@ def _qkv_rope_store(q, k, v, h, pos, cos, sin, qr, kc, vc, head_dim, max_len, ap
         max_len, int(apply_rope), ws.data_ptr(), ws.numel(), _stream()))
 
 
-def _qkv_rope_attn(q, k, v, h, pos, cos, sin, kc, vc, out, heads, kv_heads, head_dim, max_len, apply_rope):
+def attn_state(heads, max_len, device):
+    """Zeroed state buffer of the attention launch that shares a long context's keys between workgroups
+    (one per decoder: calls that overlap on one GPU need one each); None when max_len is too short for shares."""
+    if os.environ.get("GLQ_ATTN_SHARED_KEYS", "1") == "0":
+        return None
+    nbytes = int(_lib.load().glqh_attn_split_state_bytes(heads, max_len))
+    return torch.zeros(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
+def _qkv_rope_attn(q, k, v, h, pos, cos, sin, kc, vc, out, heads, kv_heads, head_dim, max_len, apply_rope,
+                   state=None):
     """q/k/v projections of one token, rotated, appended to the cache and attended over:
-    decode launch + one finishing launch."""
+    decode launch + one finishing launch.  state (attn_state): from 1024 cached positions on the keys are
+    shared by several workgroups per head."""
     ws = _group_ws((q, k, v), h.device)
     bn, nbn = ext._host_i64(q.bn)
     arr = _shard_array((q, k, v))                                # kept alive across the call
-    check(_lib.load().glqh_trellis_qkv_rope_attn_bf16(
+    check(_lib.load().glqh_trellis_qkv_rope_attn_shared_bf16(
         h.data_ptr(), q.n, C.addressof(arr), bn, nbn, q.bn_meta.data_ptr() if nbn > 1 else None, q.n,
         pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(), heads,
-        kv_heads, head_dim, max_len, int(apply_rope), ws.data_ptr(), ws.numel(), _stream()))
+        kv_heads, head_dim, max_len, int(apply_rope), ws.data_ptr(), ws.numel(),
+        state.data_ptr() if state is not None else None, state.numel() if state is not None else 0, _stream()))
 
 
 def _rms_norm(x, w, eps):
@@ -195,6 +208,7 @@ class TrellisDecoder:
         self.tok = torch.zeros(1, dtype=torch.int64, device=dev)     # token to feed next
         self.arange = torch.arange(max_len, device=dev)
         self.graph = None
+        self.attn_state = attn_state(cfg.heads, max_len, dev)        # long contexts: keys shared between workgroups
         # one-token steps: output head and arg-max in the library (table streamed once)
         self.fast_head = H in (2048, 4096)
         if self.fast_head:
@@ -223,7 +237,7 @@ class TrellisDecoder:
         if T == 1 and self.fuse_epilogues and D == 128:
             a = torch.empty(1, cfg.heads * D, dtype=torch.bfloat16, device=x.device)
             _qkv_rope_attn(L["q"], L["k"], L["v"], h, pos, self.cos, self.sin, self.kc[li], self.vc[li], a,
-                           cfg.heads, cfg.kv_heads, D, self.max_len, apply_rope)
+                           cfg.heads, cfg.kv_heads, D, self.max_len, apply_rope, self.attn_state)
             x, h = _linear_add_rms_norm(L["o"], a, x, L["ln2"], cfg.rms_eps)
             return x, (L["down"], _gate_up_silu(L["gate"], L["up"], h))
         if T <= 4:

@@ -102,6 +102,24 @@ int glqh_trellis_qkv_rope_attn_bf16(const void *x, int64_t in_features, const gl
                                     int64_t kv_heads, int64_t head_dim, int64_t max_len,
                                     int apply_rope, void *ws, size_t ws_bytes, void *stream);
 
+/* The same with the keys of a long context shared by several workgroups per head.  state:
+ * glqh_attn_split_state_bytes(heads, max_len) bytes that the caller sets to zero once and then leaves to
+ * this entry (every call returns them to zero; calls that overlap on one GPU need a state buffer each).
+ * Up to min(8, (max_len - 1) / 512) workgroups per head take a share of the keys once the context holds 512 keys for
+ * each (from 1024 positions on), write (maximum, sum, weighted rows) of their share, and the one that finishes
+ * last merges the shares in ascending order: no workgroup waits for another.  Below 1024 positions, and with
+ * state == NULL, one workgroup per head finishes alone, bit-identical to the entry above; with shares the row
+ * differs from it by rounding (another order of summation).  max_len <= ~90000; at most 256 heads. */
+size_t glqh_attn_split_state_bytes(int64_t heads, int64_t max_len);
+int glqh_trellis_qkv_rope_attn_shared_bf16(const void *x, int64_t in_features, const glqh_trellis_shard *qkv,
+                                           const int64_t *blocks_n, int64_t n_blocks_n,
+                                           const glqh_block_meta *bn_meta_dev, int64_t n_pad,
+                                           const int64_t *pos, const void *cos_t, const void *sin_t,
+                                           void *k_cache, void *v_cache, void *out, int64_t heads,
+                                           int64_t kv_heads, int64_t head_dim, int64_t max_len,
+                                           int apply_rope, void *ws, size_t ws_bytes, void *state,
+                                           size_t state_bytes, void *stream);
+
 size_t glqh_lm_head_workspace_bytes(void);
 
 /* Output head of a decode step: logits[r] = <h, table[r, :]> for a (vocab, hidden) bf16 table and

@@ -186,6 +186,61 @@ def test_fused_qkv_rope_store_is_bit_identical(rope):
     assert torch.equal(a3.view(heads, hd), vc3[:, 0].repeat_interleave(heads // kvh, 0))
 
 
+@pytest.mark.parametrize("L,positions", [(4096, (0, 700, 1023, 1024, 1535, 1536, 2600, 4095)), (1536, (1023, 1400, 1535)),
+                                         (20000, (19999,))])
+def test_attention_with_shared_keys(L, positions):
+    """From 1024 cached positions on, up to eight workgroups per head take a share of the keys and the last one to
+    finish merges them: against the one-workgroup entry (same bits below 1024 positions, rounding above), against
+    softmax(q K^T) V in fp64 from the cache the launch left, the state buffer back to zero, two calls the same bits.
+    A cache of 20000 positions only fits the score buffer with shares."""
+    from glq_amd import decoder as D
+    say("shared-key attention", L, positions)
+    g = torch.Generator(device=DEV).manual_seed(11)
+    hidden, heads, kvh, hd = 2048, 16, 4, 128
+    q, k, v = (D._Linear(heads * hd, hidden, 4, g, DEV), D._Linear(kvh * hd, hidden, 4, g, DEV),
+               D._Linear(kvh * hd, hidden, 4, g, DEV))
+    h = torch.randn(1, hidden, generator=g, device=DEV).to(torch.bfloat16)
+    inv = 1.0 / (2e6 ** (torch.arange(0, hd, 2, device=DEV, dtype=torch.float32) / hd))
+    ang = torch.arange(L, device=DEV, dtype=torch.float32)[:, None] * inv[None]
+    ang = torch.cat((ang, ang), -1)
+    cos, sin = ang.cos().to(torch.bfloat16), ang.sin().to(torch.bfloat16)
+    kc0 = (torch.randn(kvh, L, hd, generator=g, device=DEV) * 2.0).to(torch.bfloat16)
+    vc0 = torch.randn(kvh, L, hd, generator=g, device=DEV).to(torch.bfloat16)
+    state = D.attn_state(heads, L, DEV)
+    assert state is not None and int(state.count_nonzero()) == 0
+    for p in positions:
+        pos = torch.tensor([p], device=DEV)
+        kc1, vc1, a1 = kc0.clone(), vc0.clone(), torch.zeros(1, heads * hd, dtype=torch.bfloat16, device=DEV)
+        D._qkv_rope_attn(q, k, v, h, pos, cos, sin, kc1, vc1, a1, heads, kvh, hd, L, 1, state)
+        torch.cuda.synchronize()
+        assert int(state[:1024].count_nonzero()) == 0, p          # the counters are back at zero
+        kc2, vc2, a2 = kc0.clone(), vc0.clone(), torch.zeros_like(a1)
+        D._qkv_rope_attn(q, k, v, h, pos, cos, sin, kc2, vc2, a2, heads, kvh, hd, L, 1, state)
+        assert torch.equal(a1, a2) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2), p
+        n = p + 1
+        if L <= 8192:                                             # the one-workgroup entry holds max_len scores in LDS
+            kc3, vc3, a3 = kc0.clone(), vc0.clone(), torch.zeros_like(a1)
+            D._qkv_rope_attn(q, k, v, h, pos, cos, sin, kc3, vc3, a3, heads, kvh, hd, L, 1, None)
+            assert torch.equal(kc1, kc3) and torch.equal(vc1, vc3), p
+            if n < 1024:
+                assert torch.equal(a1, a3), p
+            else:
+                assert rel(a1, a3.float().cpu().numpy()) < 6e-3, (p, rel(a1, a3.float().cpu().numpy()))
+        # reference from the cache rows the launch wrote and the query it used: q is not returned, so take it
+        # from the store-only entry
+        qr = torch.zeros(1, heads * hd, dtype=torch.bfloat16, device=DEV)
+        kc4, vc4 = kc0.clone(), vc0.clone()
+        D._qkv_rope_store(q, k, v, h, pos, cos, sin, qr, kc4, vc4, hd, L, 1)
+        assert torch.equal(kc4, kc1) and torch.equal(vc4, vc1), p
+        qd = qr.view(heads, hd).double()
+        Kd = kc1[:, :n].double().repeat_interleave(heads // kvh, 0)
+        Vd = vc1[:, :n].double().repeat_interleave(heads // kvh, 0)
+        sc = torch.einsum("hd,hnd->hn", qd, Kd) / (hd ** 0.5)
+        ref = torch.einsum("hn,hnd->hd", torch.softmax(sc, -1), Vd).reshape(1, -1)
+        e = rel(a1, ref.cpu().numpy())
+        assert e < 6e-3, (p, e)
+
+
 @pytest.mark.parametrize("hidden,vocab", [(2048, 128256), (4096, 1000), (2048, 7)])
 def test_output_head_and_argmax(hidden, vocab):
     """Logits of the library's output head against a float64 product, its arg-max against the

@@ -240,6 +240,14 @@ static bool tr_fuse_input_enabled() {
     return on;
 }
 
+static int tr_f16_sums_max_slots() {                           // GLQ_TRELLIS_F16_SUMS_SLOTS: K slots up to which the sums are fp16
+    static const int v = [] {
+        const char *e = getenv("GLQ_TRELLIS_F16_SUMS_SLOTS");
+        return e ? atoi(e) : 16;
+    }();
+    return v;
+}
+
 static bool tr_f16_sums_enabled() {
     static const bool on = [] {
         const char *e = getenv("GLQ_TRELLIS_F16_SUMS");
@@ -526,11 +534,13 @@ extern "C" int glqh_fused_linear_trellis_3inst(
             return 1;
         ks = plan.ks;
         if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
-        // Many tokens, one K slot: the tile kernel rounds its sums to fp16 on the way out, as the
-        // reference's many-token route does (its library GEMM of two fp16 matrices returns fp16,
+        // Many tokens: the tile kernel rounds its sums to fp16 on the way out, as the reference's
+        // many-token route does (its library GEMM of two fp16 matrices returns fp16,
         // glq/csrc/glq_trellis.cu:1322-1334) -- half the bytes between the product and the output
-        // transform.  GLQ_TRELLIS_F16_SUMS=0 keeps them fp32.
-        f16_sums = plan.tile && ks == 1 && B > 64 && !y_rht_out && y && tr_f16_sums_enabled() &&
+        // transform.  With several K slots (small layers at a few hundred tokens) every slot's sum is
+        // rounded and the transform adds them in fp32 (3B-shape layer at 512 tokens: 413 -> 394 us for
+        // its seven linears).  GLQ_TRELLIS_F16_SUMS=0 keeps them fp32.
+        f16_sums = plan.tile && ks <= tr_f16_sums_max_slots() && B > 64 && !y_rht_out && y && tr_f16_sums_enabled() &&
                    glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad);
         if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st, 1.0f, f16_sums)) return 1;
         if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2, f16_sums)) return 1;

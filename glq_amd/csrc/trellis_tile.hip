@@ -395,7 +395,11 @@ tr_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, i
     }
 }
 
-int tt_ntw(int64_t M) { return M <= 128 ? 1 : M <= 256 ? 2 : 4; }
+int tt_ntw(int64_t M) {
+    static const int forced = [] { const char *e = getenv("GLQ_TT_NTW"); return e ? atoi(e) : 0; }();
+    if (forced && M > 256) return forced;
+    return M <= 128 ? 1 : M <= 256 ? 2 : 4;
+}
 
 int64_t tt_padded_tokens(int64_t M) {
     const int64_t tile = TT_WAVES * 16 * tt_ntw(M);

@@ -60,6 +60,11 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
                              hipStream_t stream, int out_f16 = 0);
 int64_t glqh_trellis_tile_padded_tokens(int64_t M);
+int glqh_trellis_tile_group_ksplit(const int64_t *m, int n_layers, int64_t k, int64_t M);
+int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void *const packed[], int R,
+                                   const int64_t m[], int n_layers, int64_t k, float *const out[], int out_f16,
+                                   hipStream_t stream);
+int glqh_launch_trellis_pack(const void *x_f16, void *xb, int64_t M, int64_t k, hipStream_t stream);
 int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages);
 // input transform straight into a tile kernel's operand layout (fht.hip); -1 = not eligible, nothing launched
 int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, const void *sv, void *xb,
@@ -628,6 +633,12 @@ static bool tr_group_plain(int64_t total_m_pad, int64_t n_pad, int64_t B) {
     if (B == 1) return w > ((int64_t)96 << 20);
     return w > ((int64_t)48 << 20) || (B >= 3 && n_pad >= 4096 && w > ((int64_t)16 << 20));
 }
+// The grouped call at many tokens: more than 64 tokens, at most four layers.  The K split of a group is at most
+// that of a single 128-row layer of the same width (fewer row tiles, more slots).
+constexpr int64_t TR_GROUP_MANY_MIN = 64;
+constexpr int TR_GROUP_MANY_MAX = 4;
+constexpr int64_t TT_GROUP_ROWS_FLOOR = 128;
+
 static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int64_t B, int *steps, int *ks) {
     int64_t total = 0;
     for (int i = 0; i < n_shards; ++i) total += m_pads[i];
@@ -637,6 +648,15 @@ static int tr_group_plan(const int64_t *m_pads, int n_shards, int64_t n_pad, int
 
 extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad, int64_t total_m_pad,
                                                                   int n_shards) {
+    if (B > TR_GROUP_MANY_MIN && n_shards >= 1 && n_shards <= TR_GROUP_MANY_MAX && total_m_pad >= 32 && n_pad >= 64) {
+        // many tokens: every layer's blocked activations, a row-major copy for transforms that cannot write
+        // them, and the partial sums of the largest K split a group of these rows can get (fp32)
+        glqh_init();
+        const int64_t one[1] = {TT_GROUP_ROWS_FLOOR};
+        const int ks = glqh_trellis_tile_group_ksplit(one, 1, n_pad, B);
+        return (size_t)n_shards * (256 + align256(glqh_trellis_tile_xb_bytes(n_pad, B))) +
+               align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ks * B * total_m_pad * sizeof(float));
+    }
     if (B < 1 || B > 4 || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64) return 0;
     glqh_init();
     int steps = 0, ks = 0;
@@ -655,6 +675,107 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
 
 // Decode launch of a group: checks, K plan, partial-sum layout in ws.  On return parts[i] holds
 // layer i's [slot][token][row] fp32 partial sums and *ks_out the slot count.
+// Layers that read the same activations, many tokens (prefill of fused q/k/v, gate/up): per distinct sign vector
+// one input transform straight into the tile kernel's layout, ONE launch of the tile kernel over the row tiles of
+// all layers (small layers do not fill the chip one by one: 512 tokens x (2048 -> 2048 + 512 + 512): 16 + 4 + 4
+// row tiles), then every layer's output transform from fp16 sums.
+static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B, const glqh_trellis_shard *shards,
+                         int n_shards, const int64_t *blocks_n, int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                         int64_t in_features, int64_t n_pad, int y_dtype, int64_t y_stride, void *ws, size_t ws_bytes,
+                         hipStream_t st) {
+    GLQH_REQUIRE(x && shards && ws, "trellis group: null pointer");
+    GLQH_REQUIRE(n_shards >= 1 && n_shards <= TR_GROUP_MANY_MAX, "trellis group: %d layers at %lld tokens (1..%d)",
+                 n_shards, (long long)B, TR_GROUP_MANY_MAX);
+    GLQH_REQUIRE(B <= 65535, "trellis group: B=%lld out of range", (long long)B);
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis group: x must be f16 or bf16");
+    GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad && n_pad % 64 == 0, "trellis group: bad in_features / n_pad");
+    GLQH_REQUIRE(n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : (n_pad & (n_pad - 1)) == 0,
+                 "trellis group: input block sizes missing");
+    int R = 0;
+    int64_t total = 0, m_pads[TR_GROUP_MANY_MAX];
+    const void *packed[TR_GROUP_MANY_MAX];
+    for (int i = 0; i < n_shards; ++i) {
+        const glqh_trellis_shard &sh = shards[i];
+        GLQH_REQUIRE(sh.sv_f16 && sh.packed && sh.su_f16 && sh.y, "trellis group: null pointer in shard %d", i);
+        int Ri;
+        if (tr_bits_from_packed(sh.packed_cols, 0, &Ri) || tr_check_shape(sh.m_pad, n_pad, sh.packed_rows)) return 1;
+        GLQH_REQUIRE(i == 0 || Ri == R, "trellis group: shards of %d and %d bits/weight cannot share a launch", R, Ri);
+        R = Ri;
+        GLQH_REQUIRE(sh.out_features >= 1 && sh.out_features <= sh.m_pad, "trellis group: out_features exceeds m_pad");
+        m_pads[i] = sh.m_pad;
+        packed[i] = sh.packed;
+        total += sh.m_pad;
+    }
+    const int ks = glqh_trellis_tile_group_ksplit(m_pads, n_shards, n_pad, B);
+    const size_t xb_one = align256(glqh_trellis_tile_xb_bytes(n_pad, B));
+    const size_t rows = align256((size_t)B * n_pad * sizeof(f16));
+    const size_t need = (size_t)n_shards * xb_one + rows + align256((size_t)ks * B * total * sizeof(float));
+    GLQH_REQUIRE(ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    char *base = (char *)ws;
+    f16 *x_rows = (f16 *)(base + (size_t)n_shards * xb_one);
+    char *pbase = base + (size_t)n_shards * xb_one + rows;
+    const int64_t Mp = glqh_trellis_tile_padded_tokens(B);
+    const void *xb[TR_GROUP_MANY_MAX];
+    float *parts[TR_GROUP_MANY_MAX];
+    // fp16 sums need the whole-block output kernels for every layer (canonical blocks of at most 8192 rows)
+    bool f16_sums = tr_f16_sums_enabled() && ks <= tr_f16_sums_max_slots();
+    for (int i = 0; i < n_shards && f16_sums; ++i) {
+        int64_t top = 1;
+        while (top * 2 <= m_pads[i]) top *= 2;
+        if (top > 8192 || m_pads[i] % 8 != 0) f16_sums = false;
+    }
+    const size_t esz = f16_sums ? sizeof(f16) : sizeof(float);
+    size_t poff = 0;
+    for (int i = 0; i < n_shards; ++i) {
+        // layers quantized with the same sign vector share one transform of x
+        int same = -1;
+        for (int j = 0; j < i; ++j)
+            if (shards[j].sv_f16 == shards[i].sv_f16) { same = j; break; }
+        if (same >= 0) {
+            xb[i] = xb[same];
+        } else {
+            void *dst = base + (size_t)i * xb_one;
+            const int rc = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, shards[i].sv_f16, dst, 2, Mp, B, in_features,
+                                                         n_pad, blocks_n, n_blocks_n, st);
+            if (rc > 0) return 1;
+            if (rc < 0) {                                        // rows first, then repacked
+                if (glqh_launch_input_rht(x, x_dtype, x_stride, shards[i].sv_f16, x_rows, GLQH_F16, B, in_features, n_pad,
+                                          bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st) ||
+                    glqh_launch_trellis_pack(x_rows, dst, B, n_pad, st))
+                    return 1;
+            }
+            xb[i] = dst;
+        }
+        parts[i] = (float *)(pbase + poff);
+        poff += align256((size_t)ks * B * m_pads[i] * esz);
+    }
+    if (glqh_launch_trellis_tile_group(xb, B, packed, R, m_pads, n_shards, n_pad, parts, f16_sums ? 1 : 0, st)) return 1;
+    for (int i = 0; i < n_shards; ++i) {
+        const glqh_trellis_shard &sh = shards[i];
+        glqh_ysrc src = {};
+        src.nparts = 1;
+        src.part = parts[i];
+        src.part_kstride = B * sh.m_pad;
+        src.ksplit = ks;
+        src.part_f16 = f16_sums;
+        src.scale[0] = (float)sh.wscale;
+        const int64_t ys = y_stride > 0 ? y_stride : sh.out_features;   // y_stride 0: every layer's rows packed
+        int rc = glqh_launch_output_rht_canon_wide(src, sh.su_f16, sh.y, y_dtype, ys, B, sh.out_features, sh.m_pad, st);
+        if (rc > 0) return 1;
+        if (rc < 0) {
+            GLQH_REQUIRE(!f16_sums, "trellis group: layer %d: output blocks not served by the whole-block transform", i);
+            // canonical blocks above 8192 rows: the sliced kernels of the grouped launcher
+            const float *pt[1] = {parts[i]};
+            const void *sus[1] = {sh.su_f16};
+            const float sc[1] = {(float)sh.wscale};
+            void *yl[1] = {sh.y};
+            if (glqh_launch_output_rht_group(pt, sus, yl, sc, &sh.m_pad, &sh.out_features, 1, y_dtype, ys, B, ks, st))
+                return 1;
+        }
+    }
+    return 0;
+}
+
 struct tr_group_ctx {
     int R, ks, fi_mode;
     int64_t m_pads[GLQH_MAX_SHARDS], outs[GLQH_MAX_SHARDS];
@@ -758,6 +879,11 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
                                                      size_t ws_bytes, void *stream) {
     GLQH_INIT();
     hipStream_t st = (hipStream_t)stream;
+    GLQH_REQUIRE(y_stride > 0 || B > TR_GROUP_MANY_MIN, "trellis group: y_stride 0 (packed rows per layer) needs more than %lld tokens",
+                 (long long)TR_GROUP_MANY_MIN);
+    if (B > TR_GROUP_MANY_MIN)
+        return tr_group_many(x, x_dtype, x_stride, B, shards, n_shards, blocks_n, n_blocks_n, bn_meta_dev, in_features,
+                             n_pad, y_dtype, y_stride, ws, ws_bytes, st);
     tr_group_ctx c;
     if (tr_group_decode(x, x_dtype, x_stride, B, shards, n_shards, blocks_n, n_blocks_n, bn_meta_dev, in_features,
                         n_pad, ws, ws_bytes, st, &c))

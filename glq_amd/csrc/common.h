@@ -149,6 +149,9 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
                            int64_t n_blocks, int64_t max_bs_hint, float rsqrt_m,
                            hipStream_t stream);
 
+int glqh_launch_output_rht_canon_wide(const glqh_ysrc &src, const void *su, void *y, int y_dtype, int64_t y_stride,
+                                      int64_t B, int64_t out_features, int64_t m_pad, hipStream_t stream);
+
 // out[tok, row] = (accum ? out : 0) + scale * sum_s part[s * kstride + tok * m + row]
 int glqh_launch_reduce_splits(const float *part, int ksplit, int64_t kstride, int64_t B, int64_t m,
                               float scale, float *out, int64_t out_stride, int accum,

@@ -754,6 +754,51 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
     return 0;
 }
 
+namespace {
+// The whole-block kernels for canonical blocks and many rows; -1 (nothing launched) when they do not apply.
+int launch_output_rht_wide(const glqh_ysrc &src, const void *su, void *y, int y_dtype, int64_t y_stride, int64_t B,
+                           int64_t out_features, int64_t m_pad, const glqh_meta_args &margs, int64_t n_blocks,
+                           int64_t max_bs, float rsqrt_m, hipStream_t stream) {
+    const int y_size = y_dtype == GLQH_F32 ? 4 : 2;
+    const int pq = src.part_f16 ? 8 : 4;                     // elements per 16 bytes of partial sums
+    const bool src_ok = src.nparts == 0
+        ? (aligned16(src.direct) && src.stride % 4 == 0)
+        : (aligned16(src.part) && m_pad % pq == 0 && src.part_kstride % pq == 0 && src.part_sstride % pq == 0 &&
+           (!src.copy_out || (aligned16(src.copy_out) && src.copy_stride % 4 == 0)));
+    // whole blocks per workgroup also from 32 tokens on when the rows are many (whole linear,
+    // 64 tokens: 11008 x 2048 56.9 -> 45.3 us, 14336 x 4096 70.4 -> 61.6; 2048 x 11008 41.5 -> 43.7)
+    const int64_t Bw = ((B >= 32 && m_pad >= 8192) || B > 32) ? 65 : B;
+    if (!(rht_wide_ok(Bw, margs, m_pad, max_bs) && src_ok && aligned16(y) && aligned16(su) &&
+          (y_stride * y_size) % 16 == 0))
+        return -1;
+    dim3 wgrid((unsigned)(64 * ((B + 63) / 64) * n_blocks));
+    const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
+#define GLQH_OUTW_LAUNCH(YT)                                                                        \
+    hipLaunchKernelGGL((output_rht_wide_kernel<YT>), wgrid, dim3(REG_THREADS), lds, stream, src,    \
+                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, (int)B, (int)n_blocks, margs, \
+                       rsqrt_m)
+    if (y_dtype == GLQH_F16) GLQH_OUTW_LAUNCH(f16);
+    else if (y_dtype == GLQH_BF16) GLQH_OUTW_LAUNCH(uint16_t);
+    else GLQH_OUTW_LAUNCH(float);
+#undef GLQH_OUTW_LAUNCH
+    GLQH_LAUNCH_CHECK("output_rht launch");
+    return 0;
+}
+}  // namespace
+
+// Output transform of a layer whose blocks are the canonical ones of m_pad (descending powers of two), many rows:
+// the whole-block kernels.  -1 (nothing launched) when they do not apply (a block above 8192 rows, alignment).
+int glqh_launch_output_rht_canon_wide(const glqh_ysrc &src, const void *su, void *y, int y_dtype, int64_t y_stride,
+                                      int64_t B, int64_t out_features, int64_t m_pad, hipStream_t stream) {
+    int64_t blocks[64];
+    int n = 0;
+    for (int bit = 62; bit >= 0; --bit)
+        if (m_pad & ((int64_t)1 << bit)) blocks[n++] = (int64_t)1 << bit;
+    glqh_meta_args margs;
+    if (n == 0 || !glqh_fill_meta_args(&margs, n > 1 ? blocks : nullptr, n > 1 ? n : 1, m_pad)) return -1;
+    return launch_output_rht_wide(src, su, y, y_dtype, y_stride, B, out_features, m_pad, margs, n, blocks[0], 0.0f, stream);
+}
+
 int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_dtype,
                            int64_t y_stride, int64_t B, int64_t out_features, int64_t m_pad,
                            const glqh_block_meta *meta_dev, const int64_t *blocks_host,
@@ -787,30 +832,9 @@ int glqh_launch_output_rht(const glqh_ysrc &src, const void *su, void *y, int y_
     if (meta_dev && !blocks_host) margs.canon = 0;         // shard-batched call: device meta only
     else if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, m_pad)) margs.canon = 0;
     {
-        const int y_size = y_dtype == GLQH_F32 ? 4 : 2;
-        const int pq = src.part_f16 ? 8 : 4;                     // elements per 16 bytes of partial sums
-        const bool src_ok = src.nparts == 0
-            ? (aligned16(src.direct) && src.stride % 4 == 0)
-            : (aligned16(src.part) && m_pad % pq == 0 && src.part_kstride % pq == 0 && src.part_sstride % pq == 0 &&
-               (!src.copy_out || (aligned16(src.copy_out) && src.copy_stride % 4 == 0)));
-        // whole blocks per workgroup also from 32 tokens on when the rows are many (whole linear,
-        // 64 tokens: 11008 x 2048 56.9 -> 45.3 us, 14336 x 4096 70.4 -> 61.6; 2048 x 11008 41.5 -> 43.7)
-        const int64_t Bw = ((B >= 32 && m_pad >= 8192) || B > 32) ? 65 : B;
-        if (rht_wide_ok(Bw, margs, m_pad, max_bs) && src_ok && aligned16(y) && aligned16(su) &&
-            (y_stride * y_size) % 16 == 0) {
-            dim3 wgrid((unsigned)(64 * ((B + 63) / 64) * n_blocks));
-            const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
-#define GLQH_OUTW_LAUNCH(YT)                                                                        \
-    hipLaunchKernelGGL((output_rht_wide_kernel<YT>), wgrid, dim3(REG_THREADS), lds, stream, src,    \
-                       (const f16 *)su, (YT *)y, y_stride, (int)out_features, (int)m_pad, (int)B, (int)n_blocks, margs, \
-                       rsqrt_m)
-            if (y_dtype == GLQH_F16) GLQH_OUTW_LAUNCH(f16);
-            else if (y_dtype == GLQH_BF16) GLQH_OUTW_LAUNCH(uint16_t);
-            else GLQH_OUTW_LAUNCH(float);
-#undef GLQH_OUTW_LAUNCH
-            GLQH_LAUNCH_CHECK("output_rht launch");
-            return 0;
-        }
+        const int rc = launch_output_rht_wide(src, su, y, y_dtype, y_stride, B, out_features, m_pad, margs, n_blocks,
+                                              max_bs, rsqrt_m, stream);
+        if (rc >= 0) return rc;
     }
     GLQH_REQUIRE(!src.part_f16, "output_rht: fp16 partial sums need the whole-block kernels (more than 32 tokens, "
                                 "canonical blocks of at most 8192 rows)");

@@ -51,6 +51,19 @@ struct tt_args {
     int rt0;                                       // first row tile of this launch (RT counts from there)
 };
 
+// Several layers that share the activations' shape (fused q/k/v, gate/up: glq_vllm/linear_method.py:664-710) in
+// one launch of the tile kernel: their row tiles are numbered through, layer l owns tiles rt0[l] .. rt0[l + 1) - 1
+// and has its own stream, rows, repacked activations (layers quantized with different input signs see different
+// transformed activations) and output.  The K plan is common.
+constexpr int TT_MAX_GROUP = 4;
+struct tt_group {
+    const uint8_t *packed[TT_MAX_GROUP];
+    const f16 *xb[TT_MAX_GROUP];
+    float *out[TT_MAX_GROUP];
+    int m[TT_MAX_GROUP], rt0[TT_MAX_GROUP];
+    int n;
+};
+
 __device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global prefetches stay in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -94,13 +107,12 @@ __device__ __forceinline__ void tt_emit(const tr_record<R> &r, int unit, int kpi
     }
 }
 
-template <int R, int NTW>
-__global__ void __launch_bounds__(TT_THREADS)
-tr_tile_kernel(const tt_args a) {
+template <int R, int NTW, bool GROUP>
+__device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g) {
     extern __shared__ u32x4 abuf[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
-    const int nkp = a.k >> 5, nds = a.k >> 6, mpairs = a.m >> 5;
+    const int nkp = a.k >> 5, nds = a.k >> 6;
     constexpr int REC = 4 * R;
 
     // decode role
@@ -116,12 +128,26 @@ tr_tile_kernel(const tt_args a) {
     for (int w = bx; w < per_xcd; w += nbx) {
         const int item = xcd * per_xcd + w;
         if (item >= nitems) break;                              // uniform
-        const int rt = item % a.RT, slot = (item / a.RT) % a.KS, tt0 = item / (a.RT * a.KS);
-        const int r0 = (a.rt0 + rt) * TT_ROWS, tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW;
+        const int slot = (item / a.RT) % a.KS, tt0 = item / (a.RT * a.KS);
+        int rt = a.rt0 + item % a.RT;                           // row tile of its layer
+        int lm = a.m;
+        const uint8_t *lpacked = a.packed;
+        const f16 *lxb = a.xb;
+        float *lout = a.out;
+        if constexpr (GROUP) {
+            int first = 0;
+            lm = g.m[0]; lpacked = g.packed[0]; lxb = g.xb[0]; lout = g.out[0];
+#pragma unroll
+            for (int j = 1; j < TT_MAX_GROUP; ++j)
+                if (j < g.n && rt >= g.rt0[j]) { first = g.rt0[j]; lm = g.m[j]; lpacked = g.packed[j]; lxb = g.xb[j]; lout = g.out[j]; }
+            rt -= first;
+        }
+        const int mpairs = lm >> 5;
+        const int r0 = rt * TT_ROWS, tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW;
         const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
 
-        const int mp = min(2 * (2 * (a.rt0 + rt) + unit) + hm, mpairs - 1);
-        const uint8_t *rec_base = a.packed + ((int64_t)mp * nkp * 32 + l) * REC + (int64_t)kpi * 32 * REC;
+        const int mp = min(2 * (2 * rt + unit) + hm, mpairs - 1);
+        const uint8_t *rec_base = lpacked + ((int64_t)mp * nkp * 32 + l) * REC + (int64_t)kpi * 32 * REC;
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
@@ -131,7 +157,7 @@ tr_tile_kernel(const tt_args a) {
         // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(kp * Mp + token) * 4 + q]
         // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
         const int64_t bstep = (int64_t)a.Mp * 32;               // elements from one k-pair to the next
-        const f16 *xrow = a.xb + (int64_t)(tok0 + i) * 32 + q * 8;
+        const f16 *xrow = lxb + (int64_t)(tok0 + i) * 32 + q * 8;
 
         f32x4 acc[TT_FRAGS][NTW];
 #pragma unroll
@@ -199,18 +225,18 @@ tr_tile_kernel(const tt_args a) {
 #pragma unroll
             for (int f = 0; f < TT_FRAGS; ++f) {
                 const int row = r0 + 64 * (f >> 2) + 8 * (f & 3) + rlane;
-                if (row >= a.m) continue;                       // m is a multiple of 32: whole groups of four
+                if (row >= lm) continue;                        // m is a multiple of 32: whole groups of four
                 if (!a.direct) {
-                    const int64_t e = ((int64_t)slot * a.M + tok) * a.m + row;
+                    const int64_t e = ((int64_t)slot * a.M + tok) * lm + row;
                     if (a.out_f16) {
                         typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
                         const f32x4 v = acc[f][tt];
-                        *(f16x4 *)((f16 *)a.out + e) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+                        *(f16x4 *)((f16 *)lout + e) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
                     } else {
-                        *(f32x4 *)(a.out + e) = acc[f][tt];
+                        *(f32x4 *)(lout + e) = acc[f][tt];
                     }
                 } else {
-                    float *o = a.out + (int64_t)tok * a.out_stride + row;
+                    float *o = lout + (int64_t)tok * a.out_stride + row;
                     if ((a.out_stride & 3) == 0) {
                         f32x4 v = acc[f][tt] * a.scale;
                         if (a.accum) v += *(f32x4 *)o;
@@ -223,6 +249,18 @@ tr_tile_kernel(const tt_args a) {
             }
         }
     }
+}
+
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_kernel(const tt_args a) {
+    tr_tile_body<R, NTW, false>(a, tt_group{});
+}
+
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_group_kernel(const tt_args a, const tt_group g) {
+    tr_tile_body<R, NTW, true>(a, g);
 }
 
 // Up to 64 tokens: one barrier per group of four steps instead of one per step, and the eight waves split a
@@ -565,3 +603,84 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     default: return tt_launch<4, 2>(tail, a, stream);
     }
 }
+
+// ---- several layers in one launch (many tokens) ---------------------------------------------------
+namespace {
+void tt_make_group_plan(const int64_t *m, int n_layers, int64_t k, int64_t M, tt_plan *p) {
+    int64_t rt = 0, mtot = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        rt += (m[l] + TT_ROWS - 1) / TT_ROWS;
+        mtot += m[l];
+    }
+    tt_make_plan(TT_ROWS * rt, k, M, p);                        // same rule, on the row tiles of all layers
+    (void)mtot;
+}
+
+template <int R>
+int tt_launch_group_R(const tt_plan &p, const tt_args &a, const tt_group &g, hipStream_t stream) {
+#define GLQH_TTG(NTW)                                                                                      \
+    hipLaunchKernelGGL((tr_tile_group_kernel<R, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a, g)
+    if (p.NTW == 1) GLQH_TTG(1);
+    else if (p.NTW == 2) GLQH_TTG(2);
+    else GLQH_TTG(4);
+#undef GLQH_TTG
+    GLQH_LAUNCH_CHECK("trellis tile group launch");
+    return 0;
+}
+}  // namespace
+
+int glqh_trellis_tile_group_ksplit(const int64_t *m, int n_layers, int64_t k, int64_t M) {
+    tt_plan p;
+    tt_make_group_plan(m, n_layers, k, M, &p);
+    return p.KS;
+}
+
+// Layers l < n_layers (at most 4) of the same width k and bits/weight against the same M > 64 tokens: partial
+// sums out[l][(slot * M + token) * m[l] + row] (fp16 with out_f16), K slots from glqh_trellis_tile_group_ksplit.
+// xb[l]: the layer's activations in the blocked layout (glqh_trellis_tile_padded_tokens(M) tokens).
+int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void *const packed[], int R,
+                                   const int64_t m[], int n_layers, int64_t k, float *const out[], int out_f16,
+                                   hipStream_t stream) {
+    GLQH_REQUIRE(n_layers >= 1 && n_layers <= TT_MAX_GROUP, "trellis tile group: %d layers (1..%d)", n_layers, TT_MAX_GROUP);
+    GLQH_REQUIRE(M > 64, "trellis tile group: more than 64 tokens");
+    tt_plan p;
+    tt_make_group_plan(m, n_layers, k, M, &p);
+    tt_args a = {};
+    tt_group g = {};
+    g.n = n_layers;
+    int rt = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        g.packed[l] = (const uint8_t *)packed[l];
+        g.xb[l] = (const f16 *)xb[l];
+        g.out[l] = out[l];
+        g.m[l] = (int)m[l];
+        g.rt0[l] = rt;
+        rt += (int)((m[l] + TT_ROWS - 1) / TT_ROWS);
+    }
+    a.M = (int)M;
+    a.Mp = (int)tt_padded_tokens(M);
+    a.m = 0;
+    a.k = (int)k;
+    a.RT = p.RT;
+    a.TT = p.TT;
+    a.KS = p.KS;
+    a.slot_ds = p.slot_ds;
+    a.out_f16 = out_f16;
+    switch (R) {
+    case 1: return tt_launch_group_R<1>(p, a, g, stream);
+    case 2: return tt_launch_group_R<2>(p, a, g, stream);
+    case 3: return tt_launch_group_R<3>(p, a, g, stream);
+    case 4: return tt_launch_group_R<4>(p, a, g, stream);
+    }
+    return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}
+
+// x (M, k) fp16 row-major -> the blocked layout of the tile kernels (glqh_trellis_tile_xb_bytes)
+int glqh_launch_trellis_pack(const void *x_f16, void *xb, int64_t M, int64_t k, hipStream_t stream) {
+    const int Mp = (int)tt_padded_tokens(M);
+    hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)), dim3(256), 0,
+                       stream, (const f16 *)x_f16, (f16 *)xb, (int)M, Mp, (int)k);
+    GLQH_LAUNCH_CHECK("trellis pack launch");
+    return 0;
+}
+

@@ -65,12 +65,13 @@ class _Linear:
         return self.packed.numel() * 2
 
 
-def _group(x, lins):
-    """Layers that read the same activations, two launches for all of them."""
+def _group(x, lins, separate=False):
+    """Layers that read the same activations: one decode launch (1..4 tokens) or one launch of the many-token
+    kernel (more than 64 tokens, separate=True: one contiguous tensor per layer) for all of them."""
     a = lins[0]
     return ext.glq_fused_linear_trellis_3inst_group(
         x, [(l.sv, l.su, l.packed, l.wscale, l.m, l.m) for l in lins], a.bn, a.bn_meta, a.n, a.n,
-        out_dtype=torch.bfloat16)
+        out_dtype=torch.bfloat16, separate=separate)
 
 
 def _shard_array(lins):
@@ -246,6 +247,8 @@ class TrellisDecoder:
             q, k, v = qkv[:, :nq], qkv[:, nq:nq + nk], qkv[:, nq + nk:]
             if T > 1:
                 q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        elif T > 64:
+            q, k, v = _group(h, (L["q"], L["k"], L["v"]), separate=True)
         else:
             q, k, v = L["q"](h), L["k"](h), L["v"](h)
         qr = torch.empty_like(q)
@@ -270,6 +273,8 @@ class TrellisDecoder:
         if T == 1:
             gu = _group(h, (L["gate"], L["up"]))
             gate, up = gu[:, :cfg.ffn], gu[:, cfg.ffn:]               # one row: both halves contiguous
+        elif T > 64:
+            gate, up = _group(h, (L["gate"], L["up"]), separate=True)
         else:
             gate, up = L["gate"](h), L["up"](h)
         act = torch.empty(T, cfg.ffn, dtype=torch.bfloat16, device=x.device)

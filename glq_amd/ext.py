@@ -378,16 +378,18 @@ class _TrellisShard(C.Structure):
 
 
 def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_features, n_pad,
-                                         out_dtype=None, decode_only=False):
+                                         out_dtype=None, decode_only=False, separate=False):
     """Several separately quantized trellis layers on the same x (fused q/k/v, gate/up) with
     one decode launch and one output-transform launch: the per-shard loop of the reference's
     vLLM linear method (glq_vllm/linear_method.py:664-710) as a single call.
 
     shards: sequence of (sv, su, trellis_packed, wscale, out_features, m_pad).  Returns one
     (B, sum(out_features)) tensor, shard s in columns [off_s, off_s + out_features_s).
-    Needs 1..4 tokens, single-stage layers of one rate and block_decompose block sizes; raises
-    RuntimeError otherwise (callers then use the per-layer op).  decode_only=True stops
-    after the decode launch (no output transform, returns None): a measurement hook."""
+    Needs 1..4 tokens (any number of layers up to 8) or more than 64 (up to four layers: one launch of
+    the many-token kernel over the row tiles of all of them), single-stage layers of one rate and
+    block_decompose block sizes; raises RuntimeError otherwise (callers then use the per-layer op).
+    decode_only=True stops after the decode launch (no output transform, returns None): a measurement
+    hook.  separate=True (more than 64 tokens): a list of contiguous (B, out_features_s) tensors instead."""
     lib = _lib.load()
     _chk(x, "x", (torch.float16, torch.bfloat16))
     B = x.shape[0]
@@ -395,9 +397,13 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
     total_out = sum(int(s[4]) for s in shards)
     total_m = sum(int(s[5]) for s in shards)
     y = None if decode_only else torch.empty((B, total_out), dtype=dt, device=x.device)
+    if separate and y is not None:
+        if B <= 64:
+            raise RuntimeError("separate outputs need more than 64 tokens")
+        y = y.view(-1)                                           # layer s: rows packed at element B * off_s
     arr = (_TrellisShard * len(shards))()
     off = 0
-    esz = torch.empty((), dtype=dt).element_size()
+    esz = torch.empty((), dtype=dt).element_size() * (B if separate else 1)
     for i, (sv, su, packed, wscale, out_f, m_pad) in enumerate(shards):
         _chk(sv, "sv", torch.float16)
         _chk(su, "su", torch.float16)
@@ -414,7 +420,13 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
         check(lib.glqh_fused_linear_trellis_3inst_group(
             _p(x), _DT[x.dtype], x.shape[1], B, C.addressof(arr), len(shards), bn, nbn,
             _meta_ptr(blocks_n_meta) if nbn > 1 else None, int(in_features), int(n_pad), _DT[dt],
-            total_out, _p(ws), ws.numel(), _stream()))
+            0 if separate else total_out, _p(ws), ws.numel(), _stream()))
+    if separate and y is not None:
+        outs, off = [], 0
+        for s in shards:
+            outs.append(y[B * off:B * (off + int(s[4]))].view(B, int(s[4])))
+            off += int(s[4])
+        return outs
     return y
 
 

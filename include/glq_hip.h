@@ -200,7 +200,12 @@ size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad,
  * gives, per shard, the result of glqh_fused_linear_trellis_3inst on that shard up to the
  * rounding of a different K split.  Single-stage layers of one rate R, at most 4 tokens,
  * canonical (block_decompose) output block sizes; anything else is refused and the caller
- * falls back to per-layer calls. */
+ * falls back to per-layer calls.
+ * More than 64 tokens (up to four layers, every y given): one input transform per distinct sign
+ * vector, ONE launch of the many-token kernel over the row tiles of all layers (small layers do not
+ * fill the chip one by one) and one output transform per layer.  y_stride 0 there: every layer's rows
+ * are packed (row stride = its out_features), so that each layer's output is a contiguous matrix.
+ * 5..64 tokens are refused. */
 int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
                                           const glqh_trellis_shard *shards, int n_shards,
                                           const int64_t *blocks_n, int64_t n_blocks_n,

@@ -25,6 +25,11 @@ from .quantized_linear import E8RHTLinear
 # GLQ_TRELLIS_BATCH_OUT_RHT=0 gives every shard its own output transform and concatenates
 # (glq_vllm/linear_method.py:616).
 _GLQ_BATCH_OUT_RHT = os.environ.get("GLQ_TRELLIS_BATCH_OUT_RHT", "1") != "0"
+# GLQ_MERGED_GROUPED=1: merged single-stage shards go through the library's grouped call (one decode or
+# many-token launch for all shards) at 1-4 and at more than 64 tokens instead of the reference's per-shard
+# sequence; same result up to the rounding of another K split.  Off by default: the default is the
+# reference's own op sequence.
+_GLQ_MERGED_GROUPED = os.environ.get("GLQ_MERGED_GROUPED", "0") == "1"
 
 # Largest output block of the shard-batched transform.  The reference stops at 8192 (shared-memory
 # budget of its kernel, glq_vllm/linear_method.py:618-623); the kernel here cuts blocks into
@@ -195,9 +200,24 @@ class MergedTrellisLinear:
             y = y + bias.to(y.dtype)
         return y.reshape(*shape[:-1], y.shape[-1])
 
+    def _grouped_ok(self, B):
+        metas = self._glq_trellis_meta
+        if not (self.glq_is_fused and all(m["loaded"] and not m["has_s2"] for m in metas)):
+            return False
+        if len({self.trellis_packed.get_shard(i).shape[1] for i in range(len(metas))}) != 1:
+            return False
+        return B <= 4 or (B > 64 and len(metas) <= 4)
+
     def _apply_2d(self, x):
         _apply = E8RHTLinear._trellis_linear_apply
         metas = self._glq_trellis_meta
+        if _GLQ_MERGED_GROUPED and x.dtype in (torch.float16, torch.bfloat16) and self._grouped_ok(x.shape[0]):
+            from . import ext
+            m0 = metas[0]
+            return ext.glq_fused_linear_trellis_3inst_group(
+                x.contiguous(), [(self.SV.get_shard(i), self.SU.get_shard(i), self.trellis_packed.get_shard(i),
+                                  m["wscale"], m["out"], m["m_pad"]) for i, m in enumerate(metas)],
+                m0["_bn"], m0["_bnm"], m0["in"], m0["n_pad"], out_dtype=x.dtype)
         if self.glq_is_fused:
             s4b = self._glq_s4b
             if s4b is not None and _GLQ_BATCH_OUT_RHT:

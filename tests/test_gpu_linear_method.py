@@ -182,3 +182,24 @@ def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, s
         torch.cuda.synchronize()
         assert torch.equal(static_y, eager)
         assert rel(static_y, _oracle(x, arts, n)) < TOL
+
+
+@pytest.mark.parametrize("B", [2, 100])
+def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
+    """GLQ_MERGED_GROUPED: single-stage merged shards through the library's grouped call (one decode launch at
+    1-4 tokens, one launch of the many-token kernel above 64) against the oracle and against the default sequence
+    of registered ops; token counts in between and two-stage shards keep the default sequence."""
+    from glq_amd import linear_method as LM
+    say("merged linear, grouped call", B)
+    n = 512
+    layer, arts = _merged(n, [(256, 4, 0), (64, 4, 0), (64, 4, 0)], 4)
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * 0.5).to(torch.bfloat16).to(DEV)
+    y_ref = layer.apply(x)
+    monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
+    assert layer._grouped_ok(B) and not layer._grouped_ok(32)
+    y = layer.apply(x)
+    assert y.dtype == x.dtype and y.shape == y_ref.shape
+    assert rel(y, _oracle(x, arts, n)) < TOL
+    assert rel(y, y_ref.float().cpu().numpy()) < 6e-3
+    two, _ = _merged(n, [(352, 4, 2), (352, 4, 2)], 6)
+    assert not two._grouped_ok(B)

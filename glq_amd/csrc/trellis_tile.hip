@@ -36,7 +36,10 @@ constexpr int TT_THREADS = TT_WAVES * GLQH_WAVE;
 constexpr int TT_FRAGS = 8;                        // 16-row operands per 64-column half-step: 128 rows
 constexpr int TT_ROWS = 128;
 constexpr int TT_BUF = 2 * TT_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer
-constexpr size_t TT_LDS = (size_t)2 * TT_BUF * 16; // 32 KB
+constexpr int TT_EP_STRIDE = TT_ROWS + 4;          // floats per token of a wave's output staging space
+// two operand buffers (32 KB); after the last step every wave stages 16 tokens x 128 sums there (66 KB)
+constexpr size_t TT_LDS = (size_t)TT_WAVES * 16 * TT_EP_STRIDE * sizeof(float);
+static_assert(TT_LDS >= (size_t)2 * TT_BUF * 16, "the operand buffers fit the staging space");
 
 struct tt_args {
     const uint8_t *packed;
@@ -215,39 +218,58 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             r2 = r3;
           }
         }
-        // lane holds four consecutive rows of token i for every (operand, token tile): operand
-        // f = 4 unit' + s covers rows 64 unit' + 32 h + 8 s + (0..7), h = 0, 1
+        // Lane (i, q) holds four consecutive rows of token i for every (operand, token tile): operand
+        // f = 4 unit' + s covers rows 64 unit' + 32 h + 8 s + (0..7), h = 0, 1 -- sixteen bytes here, sixteen
+        // bytes 44 KB further on for the next token: stored like that, a wave's instruction touches 64 lines and
+        // the sums of a tile leave as 16384 separate requests (a tenth of a 4096-token linear, a fifth of a
+        // 512-token one).  So every wave passes its sums through LDS once (its own 16 tokens x 128 rows, no
+        // barrier: a wave's LDS operations complete in order) and stores whole runs of a token's rows: two
+        // tokens x 512 bytes per instruction in fp32, four tokens x 256 bytes in fp16.
         const int rlane = 32 * (q >> 1) + 4 * (q & 1);
+        float *ep = (float *)abuf + wave * (16 * TT_EP_STRIDE);
 #pragma unroll
         for (int tt = 0; tt < NTW; ++tt) {
-            const int tok = tok0 + 16 * tt + i;
-            if (tok >= a.M) continue;
 #pragma unroll
-            for (int f = 0; f < TT_FRAGS; ++f) {
-                const int row = r0 + 64 * (f >> 2) + 8 * (f & 3) + rlane;
-                if (row >= lm) continue;                        // m is a multiple of 32: whole groups of four
-                if (!a.direct) {
+            for (int f = 0; f < TT_FRAGS; ++f)
+                *(f32x4 *)(ep + i * TT_EP_STRIDE + 64 * (f >> 2) + 8 * (f & 3) + rlane) = acc[f][tt];
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (!a.direct && a.out_f16) {                       // uniform
+                const int rl = 8 * (lane & 15), row = r0 + rl;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int tl = 4 * j + (lane >> 4), tok = tok0 + 16 * tt + tl;
+                    const f32x4 v0 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
+                    const f32x4 v1 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl + 4);
+                    if (tok >= a.M || row >= lm) continue;      // m is a multiple of 32: whole runs of eight
+                    typedef _Float16 f16x8o __attribute__((ext_vector_type(8)));
                     const int64_t e = ((int64_t)slot * a.M + tok) * lm + row;
-                    if (a.out_f16) {
-                        typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-                        const f32x4 v = acc[f][tt];
-                        *(f16x4 *)((f16 *)lout + e) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
-                    } else {
-                        *(f32x4 *)(lout + e) = acc[f][tt];
-                    }
-                } else {
-                    float *o = lout + (int64_t)tok * a.out_stride + row;
-                    if ((a.out_stride & 3) == 0) {
-                        f32x4 v = acc[f][tt] * a.scale;
-                        if (a.accum) v += *(f32x4 *)o;
-                        *(f32x4 *)o = v;
-                    } else {
+                    *(f16x8o *)((f16 *)lout + e) = f16x8o{(f16)v0[0], (f16)v0[1], (f16)v0[2], (f16)v0[3],
+                                                           (f16)v1[0], (f16)v1[1], (f16)v1[2], (f16)v1[3]};
+                }
+            } else {
+                const int rl = 4 * (lane & 31), row = r0 + rl;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) o[e] = a.accum ? o[e] + acc[f][tt][e] * a.scale : acc[f][tt][e] * a.scale;
+                for (int j = 0; j < 8; ++j) {
+                    const int tl = 2 * j + (lane >> 5), tok = tok0 + 16 * tt + tl;
+                    const f32x4 v = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
+                    if (tok >= a.M || row >= lm) continue;
+                    if (!a.direct) {
+                        *(f32x4 *)(lout + ((int64_t)slot * a.M + tok) * lm + row) = v;
+                    } else {
+                        float *o = lout + (int64_t)tok * a.out_stride + row;
+                        if ((a.out_stride & 3) == 0) {
+                            f32x4 w = v * a.scale;
+                            if (a.accum) w += *(f32x4 *)o;
+                            *(f32x4 *)o = w;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) o[e] = a.accum ? o[e] + v[e] * a.scale : v[e] * a.scale;
+                        }
                     }
                 }
             }
         }
+        tt_barrier();                                           // the next item's first operands overwrite this space
     }
 }
 
@@ -505,7 +527,10 @@ int tt_set_lds(K kernel) {
 
 template <int R>
 int tt_init_R() {
-    return tt_set_lds(tr_tile_small_kernel<R, 2, 1>) || tt_set_lds(tr_tile_small_kernel<R, 4, 1>);
+    return tt_set_lds(tr_tile_small_kernel<R, 2, 1>) || tt_set_lds(tr_tile_small_kernel<R, 4, 1>) ||
+           tt_set_lds(tr_tile_kernel<R, 1>) || tt_set_lds(tr_tile_kernel<R, 2>) || tt_set_lds(tr_tile_kernel<R, 4>) ||
+           tt_set_lds(tr_tile_group_kernel<R, 1>) || tt_set_lds(tr_tile_group_kernel<R, 2>) ||
+           tt_set_lds(tr_tile_group_kernel<R, 4>);
 }
 
 }  // namespace

@@ -24,6 +24,7 @@
 // order that gives the CUs of one XCD the same tokens at the same time.  K is split into slots only
 // while the tiles alone would leave CUs idle; partial sums [slot][token][row] are combined in slot
 // order by the consumer, or, with one slot, the scaled result is written (or added) in place.
+#include <algorithm>
 #include "common.h"
 #include "trellis_device.h"
 
@@ -470,8 +471,9 @@ struct tt_plan {
     int NTW, RT, TT, KS, slot_ds, grid;
 };
 
-void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p) {
-    p->NTW = tt_ntw(M);
+// K slots and grid for token tiles of 128 NTW tokens
+void tt_plan_for(int NTW, int64_t m, int64_t k, int64_t M, tt_plan *p) {
+    p->NTW = NTW;
     const int tile_tok = TT_WAVES * 16 * p->NTW;
     p->RT = (int)((m + TT_ROWS - 1) / TT_ROWS);
     p->TT = (int)((M + tile_tok - 1) / tile_tok);
@@ -491,6 +493,48 @@ void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p) {
     p->KS = (nds + p->slot_ds - 1) / p->slot_ds;
     const int64_t items = base * p->KS;
     p->grid = (int)(items < cus ? items : cus);
+}
+
+// Microseconds a plan is expected to take: rounds of workgroups x steps x the time of a step (2.26 us with
+// 512-token tiles, 1.7 with 256), a last round that counts at least half, a step that is slower when a single
+// round leaves CUs idle (+ 0.6 x the idle share: 172 workgroups on 256 CUs take 2.75 / 2.0 us per step, measured),
+// and what K slots cost on top (their sums, esz bytes each, written and read again at about 4 TB/s).
+double tt_plan_cost(const tt_plan &p, int64_t m, int64_t M, int esz) {
+    const int cus = glqh_device_cus();
+    const int64_t items = (int64_t)p.RT * p.TT * p.KS;
+    const int64_t full = items / cus, rem = items % cus;
+    double rounds = (double)full, slow = 1.0;
+    if (full == 0) {
+        rounds = 1.0;
+        slow = 1.0 + 0.6 * (1.0 - (double)items / cus);
+    } else if (rem > 0) {
+        rounds += std::max(0.5, (double)rem / cus);
+    }
+    const double step = p.NTW == 4 ? 2.26 : p.NTW == 2 ? 1.7 : 1.3;
+    double t = rounds * p.slot_ds * step * slow;
+    if (p.KS > 1) t += 2.0 * p.KS * (double)M * (double)m * esz / 4.0e6;
+    return t;
+}
+
+// Up to 256 tokens the tile follows the token count; above, 512-token tiles unless 256-token tiles are expected
+// to be at least 5 % faster: few row tiles (small layers, a few hundred tokens) fill the chip with neither, and
+// the smaller tile then needs fewer K slots or leaves a shorter last round (2048 x 2048 at 2048 tokens: 4 x 4
+// tiles x 2 slots -> 8 x 4 tiles x 1 slot, 73 -> 58 us; 11008 x 11008 at 1024 tokens: 172 tiles in one round ->
+// 344 in two short ones, 474 -> 366 us).  The model is rough: on a sweep of 15 shapes (512..14336 rows x
+// 2048..11008 columns) x 512..4096 tokens through the matmul entry it ends within 3 % of the faster tile in 48 of
+// 60 cases, 25 % off at worst (14336 x 2048 at 512 tokens, a gain it misses), 3 % below 512-token tiles everywhere
+// in total; the seven linears of a 3B-shape layer: 505 -> 444 us at 1024 tokens.  GLQ_TT_NTW forces a tile
+// above 256 tokens.
+void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p) {
+    const int top = tt_ntw(M);
+    tt_plan_for(top, m, k, M, p);
+    static const bool forced = getenv("GLQ_TT_NTW") != nullptr;
+    if (top < 4 || forced) return;
+    tt_plan p2;
+    tt_plan_for(2, m, k, M, &p2);
+    // (3 bytes per sum, between fp16 and fp32: the K-slot query and the launch must arrive at the same plan,
+    // whatever the width the sums leave with)
+    if (tt_plan_cost(p2, m, M, 3) < 0.95 * tt_plan_cost(*p, m, M, 3)) *p = p2;
 }
 
 template <int R, int NTW>

@@ -404,10 +404,11 @@ def extras(torch, ext, dev):
         q2 = torch.randint(-32768, 32768, (m, n // 8), device=dev, dtype=torch.int16)
         ext.e8_prepare(q1, cbh, q2, cbh)
         e8_fold_default = ext.E8_FOLD_BATCH_MAX
-        for M, route in ((256, ""), (4096, ""), (4096, "_library"), (8192, ""), (8192, "_compressed")):
-            # "" = the route the library picks (compressed up to 4096 tokens: the tile kernels on the packed
-            # stream / the folded streams; dequantize + library GEMM above); "_library" / "_compressed" = the
-            # other route forced, for the comparison at the threshold and beyond it
+        for M, route in ((256, ""), (4096, ""), (4096, "_library"), (8192, ""), (8192, "_library"),
+                         (8192, "_compressed")):
+            # "" = the route the library picks (compressed up to 8192 tokens for the trellis, 4096 for E8: the
+            # tile kernels on the packed stream / the folded streams; dequantize + library GEMM above);
+            # "_library" / "_compressed" = a route forced, for the comparison at the threshold and beyond it
             lim = {"": None, "_library": 64, "_compressed": 1 << 30}[route]
             ext.TRELLIS_BATCH_MAX = tr_default if lim is None else lim
             ext.E8_BATCH_MAX = e8_default if lim is None else lim

@@ -37,8 +37,11 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 # the indices 201 / 211 and 196 / 209 at 1024, 400 / 335 and 312 / 327 at 2048, 639 / 552 and 553 / 511 at
 # 4096 (the 14336-row shape pays for 448 and 896 tiles on 256 CUs).  The thresholds are the reference's
 # tunable and its E8 counterpart: GLQ_TRELLIS_BATCH_MAX=<n> / GLQ_E8_BATCH_MAX=<n> send calls above n
-# tokens to the library route (a large n keeps every call compressed).
-TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "4096")))
+# tokens to the library route (a large n keeps every call compressed).  Trellis, after the tile kernel's
+# staged output and grouped launches: 562 / 611 and 472 / 480 at 4096 tokens, 1129 / 1089 and 994 / 981 at 8192,
+# 2147 / 2061 and 2004 / 1872 at 16384; 4096 x 4096 306 / 312 at 8192, 641 / 610 at 16384; 11008 x 2048 520 / 562
+# and 1058 / 1105: level at 8192 tokens, so trellis calls stay compressed up to there.
+TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "8192")))
 # GLQ_TRELLIS_DENSE (set to anything) sends every fused trellis call to that dense route, the
 # reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
 TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ

@@ -104,7 +104,7 @@ def test_ops_namespace_runs_the_hip_path():
 def test_trellis_many_tokens(B, route, monkeypatch):
     """More than 16 tokens: the tile kernels over the compressed stream, and the
     dequantize-then-GEMM route the reference takes (GLQ_TRELLIS_BATCH_MAX; by default above
-    2048 tokens)."""
+    8192 tokens)."""
     from glq_amd import ext, hadamard as H
     monkeypatch.setattr(ext, "TRELLIS_BATCH_MAX", 16 if route == "dense" else 1 << 30)
     m, n = 256, 512

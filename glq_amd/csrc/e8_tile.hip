@@ -623,7 +623,11 @@ e8_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, i
 
 // token tiles per wave: 512-token workgroup tiles from 257 tokens on; layers of three and four stages
 // stay at 256 (the registers of their longer lookup pipeline)
-static int et_ntw(int64_t M, int nstages) { return M <= 128 ? 1 : (M <= 256 || nstages > 2) ? 2 : 4; }
+static int et_ntw(int64_t M, int nstages) {
+    static const int forced = [] { const char *e = getenv("GLQ_ET_NTW"); return e ? atoi(e) : 0; }();
+    if (forced && M > 256 && nstages <= 2) return forced;
+    return M <= 128 ? 1 : (M <= 256 || nstages > 2) ? 2 : 4;
+}
 
 static int64_t et_padded_tokens(int64_t M, int nstages) {
     const int64_t tile = ET_WAVES * 16 * et_ntw(M, nstages);
@@ -639,10 +643,8 @@ struct et_plan {
 // activations to the same width with zeros (the kernel's n_pad is then the padded width).
 static int64_t et_width(int64_t n_pad) { return (n_pad + 255) / 256 * 256; }
 
-int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *p) {
-    if (M < 1 || m_pad < 1 || n_pad < 256 || (n_pad & 255) || M > ((int64_t)1 << 22) || m_pad > ((int64_t)1 << 24))
-        return 0;
-    p->NTW = et_ntw(M, nstages);
+static int et_plan_for(int NTW, int64_t m_pad, int64_t n_pad, int64_t M, et_plan *p) {
+    p->NTW = NTW;
     const int tile_tok = ET_WAVES * 16 * p->NTW;
     p->RT = (int)((m_pad + ET_ROWS - 1) / ET_ROWS);
     p->TT = (int)((M + tile_tok - 1) / tile_tok);
@@ -663,6 +665,42 @@ int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *
     p->KS = (nds + p->slot_ds - 1) / p->slot_ds;
     const int64_t items = base * p->KS;
     p->grid = (int)(items < cus ? items : cus);
+    return 1;
+}
+
+// Expected microseconds of a plan, as for the trellis tile kernel: rounds x steps x the time of a step (2.75 us
+// with 512-token tiles, 1.65 with 256: two-stage layers on folded streams, full chip), a last round of at least
+// half, +0.6 x the idle share when a single round leaves CUs idle, and the K slots' fp32 sums written and read
+// at about 4 TB/s.
+static double et_plan_cost(const et_plan &p, int64_t m_pad, int64_t M) {
+    const int cus = glqh_device_cus();
+    const int64_t items = (int64_t)p.RT * p.TT * p.KS;
+    const int64_t full = items / cus, rem = items % cus;
+    double rounds = (double)full, slow = 1.0;
+    if (full == 0) {
+        rounds = 1.0;
+        slow = 1.0 + 0.6 * (1.0 - (double)items / cus);
+    } else if (rem > 0) {
+        rounds += std::max(0.5, (double)rem / cus);
+    }
+    double t = rounds * p.slot_ds * (p.NTW == 4 ? 2.75 : 1.65) * slow;
+    if (p.KS > 1) t += 2.0 * p.KS * (double)M * (double)m_pad * 4.0 / 4.0e6;
+    return t;
+}
+
+// Above 256 tokens: 512-token tiles (one- and two-stage layers) unless 256-token tiles are expected to be at
+// least 5 % faster, which they are where row tiles are few (11008 x 11008 at 1024 tokens: 548 -> 384 us,
+// 11008 x 2048: 151 -> 115).  GLQ_ET_NTW forces a tile.
+int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *p) {
+    if (M < 1 || m_pad < 1 || n_pad < 256 || (n_pad & 255) || M > ((int64_t)1 << 22) || m_pad > ((int64_t)1 << 24))
+        return 0;
+    const int top = et_ntw(M, nstages);
+    et_plan_for(top, m_pad, n_pad, M, p);
+    static const bool forced = getenv("GLQ_ET_NTW") != nullptr;
+    if (top < 4 || forced) return 1;
+    et_plan p2;
+    et_plan_for(2, m_pad, n_pad, M, &p2);
+    if (et_plan_cost(p2, m_pad, M) < 0.95 * et_plan_cost(*p, m_pad, M)) *p = p2;
     return 1;
 }
 

@@ -35,6 +35,11 @@ static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages, bool
 }
 
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
+int glqh_launch_trellis_mma_fusein_rvq(const void *packed, const void *packed2, int R2, float rs2, const void *x,
+                                       int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
+                                       int64_t in_features, int S, int ksplit, float *part,
+                                       const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                                       hipStream_t stream);
 int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const sv[], float *const part[],
                                    const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
                                    int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
@@ -47,10 +52,11 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
 // shapes: 9.8 vs 10.7 us per launch on average); below that the launch is pure latency and the
 // smaller workgroups of the v_dot2 form spread it over more CUs.
 #define GLQH_FUSEIN_MMA_MIN_STRIPS 32
-static int tr_fusein_plan(const int64_t *m_pads, int n, int64_t n_pad, int64_t B, int *S, int *ks) {
+static int tr_fusein_plan(const int64_t *m_pads, int n, int64_t n_pad, int64_t B, int *S, int *ks,
+                          int mma_min_strips = GLQH_FUSEIN_MMA_MIN_STRIPS) {
     int64_t total = 0, wgs = 0;
     for (int i = 0; i < n; ++i) { total += m_pads[i]; wgs += (m_pads[i] + 63) / 64; }
-    if (wgs >= GLQH_FUSEIN_MMA_MIN_STRIPS) return glqh_trellis_mma_fusein_plan(wgs, n_pad, B, S, ks) ? 2 : 0;
+    if (wgs >= mma_min_strips) return glqh_trellis_mma_fusein_plan(wgs, n_pad, B, S, ks) ? 2 : 0;
     return glqh_trellis_fusein_plan(total, n_pad, B, S, ks) ? 1 : 0;
 }
 // many-token kernel (trellis_tile.hip): weights decoded once per 128-row x 512-token tile
@@ -235,6 +241,15 @@ extern "C" int glqh_init(void) {
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
+// GLQ_TRELLIS_FUSE_STAGES=0: one token of a two-stage layer decodes its stages in two launches again.
+static bool tr_fuse_stages_enabled() {
+    static const bool on = [] {
+        const char *e = getenv("GLQ_TRELLIS_FUSE_STAGES");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 // GLQ_TRELLIS_FUSE_INPUT=0 keeps the input transform a launch of its own at every token count,
 // the reference's switch of the same name (glq/csrc/glq_trellis.cu:1270-1274).  Read once.
 static bool tr_fuse_input_enabled() {
@@ -411,6 +426,8 @@ static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
     int ks = tr_plain_plan(m_pad, n_pad, B).ks;
     int steps = 0, ks2 = 0;
     if (tr_fusein_plan(&m_pad, 1, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
+    // one token of a two-stage layer plans the MFMA form at every height
+    if (B == 1 && tr_fusein_plan(&m_pad, 1, n_pad, B, &steps, &ks2, 1) && ks2 > ks) ks = ks2;
     return align256((size_t)ks * B * m_pad * sizeof(float));
 }
 
@@ -471,14 +488,15 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                            glqh_fill_meta_args(&canon_m, n_blocks_m > 1 ? blocks_m : nullptr,
                                                n_blocks_m > 1 ? n_blocks_m : 1, m_pad) &&
                            canon_m.canon == m_pad;
-    const bool merge2 = has_s2 && canon_out && !(y && y_rht_out) && !tr_plain_plan(m_pad, n_pad, B).tile;
+    bool merge2 = has_s2 && canon_out && !(y && y_rht_out) && !tr_plain_plan(m_pad, n_pad, B).tile;
     const float ps2 = merge2 ? (float)inv_resid_scale2 : 1.0f;
+    bool two_parts = has_s2;                                   // false once one launch has added both stages
 
     // Up to four tokens the input transform is folded into the GEMV launch.  A two-stage layer
-    // repeats it in both launches at one token, where that is cheaper than a launch of its own
-    // (2048 x 2048: 14.5 against 17.4 us; at four tokens 23.9 against 18.0, so two to four
-    // tokens transform x once); only the MFMA form takes a pre-scaled second stage.  Everything
-    // else transforms x once into scratch and reads it from every workgroup.
+    // at one token decodes both streams in that one launch (first stage of 4 bits/weight, as the
+    // reference's recipes have it; any other repeats the transform in two launches: 2048 x 2048 14.5
+    // against 17.4 us; at four tokens 23.9 against 18.0, so two to four tokens transform x once).
+    // Everything else transforms x once into scratch and reads it from every workgroup.
     int ks = 0, fi_steps = 0, fi_mode = 0, f16_sums = 0;
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
     const bool fi_blocks = n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n;
@@ -492,11 +510,18 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     // 12.1 / 15.5, 8192 x 3072 15.2 / 17.3, 2048 x 6144 10.9 / 12.9, 6144 x 2048 11.5 / 12.6, 1536 x 1536 8.1 / 9.3,
     // 5120 x 5120 17.0 / 15.8 -- the one loss; two tokens: 4096 x 4096 15.0 / 16.1, but 3072 x 8192 19.3 / 16.2 and
     // 6144 x 2048 14.7 / 13.2, hence the size bound on two tokens).
-    const bool fi_pays = tr_fuse_input_enabled() && m_pad * n_pad <= ((int64_t)32 << 20) &&
+    // One token of a two-stage layer (first stage 4 bits/weight) takes the MFMA form at every height and up to
+    // four times the size, both streams in one launch: the alternative is a transform, two decode launches
+    // and a finishing one (whole linear, us, one launch / two or three: 4096 x 4096 at 4+2 15.5 / 22.0, 2048 x 2048
+    // 9.5 / 14.4, 11008 x 2048 17.7 / 25.0, 512 x 2048 8.7 / 15.0, 128 x 4096 10.9 / 17.0, 14336 x 4096 at 4+4
+    // 28.7 / 35.2, 8192 x 8192 32.4 / 41.2, 16384 x 8192 52.3 / 59.2; 28672 x 8192: 94.4 / 95.4 at 4+4 but
+    // 108.8 / 98.6 at 4+2, hence the bound).
+    const bool fuse2 = has_s2 && B == 1 && R1 == 4 && tr_fuse_stages_enabled();
+    const bool fi_pays = tr_fuse_input_enabled() && m_pad * n_pad <= ((int64_t)(fuse2 ? 128 : 32) << 20) &&
                          (B == 1 || (B == 2 && pow2_n && n_pad <= 4096 && m_pad <= 4096));
     if (fi_pays && fi_blocks && (x_dtype == GLQH_F16 || x_dtype == GLQH_BF16) &&
-        (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks)) != 0 &&
-        (!has_s2 || (B == 1 && fi_mode == 2 && merge2))) {
+        (fi_mode = tr_fusein_plan(&m_pad, 1, n_pad, B, &fi_steps, &ks, fuse2 ? 1 : GLQH_FUSEIN_MMA_MIN_STRIPS)) != 0 &&
+        (!has_s2 || (B == 1 && fi_mode == 2 && (merge2 || fuse2)))) {
         if (n_blocks_n > 1) {
             int64_t sum = 0;
             for (int64_t i = 0; i < n_blocks_n; ++i) {
@@ -509,8 +534,18 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                          (long long)sum, (long long)n_pad);
         }
         GLQH_REQUIRE(in_features >= 1, "fused trellis linear: in_features must be positive");
+        // One token of a 4 + R2 layer: both streams in one launch against one transform of x, the second
+        // stage's sums added in registers (4096 x 4096 at 6 bpw: three launches become two).
+        if (fuse2) {
+            if (glqh_launch_trellis_mma_fusein_rvq(packed, packed2, R2, (float)inv_resid_scale2, x, x_dtype, x_stride,
+                                                   sv_f16, m_pad, n_pad, in_features, fi_steps, ks, part1, bn_meta_dev,
+                                                   blocks_n, (int)n_blocks_n, st))
+                return 1;
+            two_parts = merge2 = false;
+        }
         if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
-        for (int stage = 0; stage < (has_s2 ? 2 : 1); ++stage) {
+        const int n_launches = has_s2 ? (two_parts ? 2 : 0) : 1;
+        for (int stage = 0; stage < n_launches; ++stage) {
             const void *pk[1] = {stage ? packed2 : packed}, *svs[1] = {sv_f16};
             float *pt[1] = {stage ? part2 : part1};
             const int R = stage ? R2 : R1;
@@ -556,12 +591,12 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     if (!y) {
         // stop at the RHT-domain product: combine the split-K partials into the caller's rows
         if (glqh_launch_reduce_splits(part1, ks_all, B * m_pad, B, m_pad, s1, y_rht_out, y_rht_stride, 0, st)) return 1;
-        if (has_s2 && !merge2 &&
+        if (two_parts && !merge2 &&
             glqh_launch_reduce_splits(part2, ks, B * m_pad, B, m_pad, s2, y_rht_out, y_rht_stride, 1, st))
             return 1;
         return 0;
     }
-    if ((!has_s2 || merge2) && !y_rht_out && canon_out) {
+    if ((!two_parts || merge2) && !y_rht_out && canon_out) {
         // canonical blocks, small batch: the grouped launcher's kernels (a group of one)
         const float *pt[1] = {part1};
         const void *sus[1] = {su_f16};
@@ -570,7 +605,7 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         return glqh_launch_output_rht_group(pt, sus, ys, sc, &m_pad, &out_features, 1, y_dtype, y_stride, B, ks_all, st);
     }
     glqh_ysrc src = {};
-    src.nparts = has_s2 ? 2 : 1;
+    src.nparts = two_parts ? 2 : 1;
     src.part = part1;
     src.part_sstride = (int64_t)(pb / (f16_sums ? sizeof(f16) : sizeof(float)));
     src.part_kstride = B * m_pad;

@@ -271,12 +271,16 @@ __host__ __device__ constexpr int fi_xs_slots(int S) {
     return S * 8 * mma_tps<TP>() + (TP < 16 ? 8 * mma_tps<TP>() : 0);          // slots + zero block
 }
 
-template <int R, typename XT, int TP>
+// R2 > 0: a residual stage of R2 bits/weight (glq/trellis.py stacked RVQ) decoded in the same launch against the
+// same activations: its own stream, its own accumulators, added with its scale rs2 before the waves' sums are
+// combined -- one launch, one transform of x and one set of partial sums where two launches wrote two.
+template <int R, typename XT, int TP, int R2 = 0>
 __device__ __forceinline__ void
 tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x, int64_t x_stride,
                    const f16 *__restrict__ sv, int B, int m, int k, int in_features, int S,
                    const glqh_block_meta *__restrict__ bn_meta, int n_blocks, glqh_meta_args margs,
-                   float *__restrict__ part, float pscale, u32x4 *lds, int part_B = 0) {
+                   float *__restrict__ part, float pscale, u32x4 *lds, int part_B = 0,
+                   const uint8_t *__restrict__ packed2 = nullptr, float rs2 = 0.0f) {
     constexpr int TPS = mma_tps<TP>();
     const int Ls = S << 5;
     uint32_t *xs32 = (uint32_t *)lds;
@@ -295,8 +299,11 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
 
     constexpr int REC = 4 * R;
     const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
+    constexpr int RB = R2 > 0 ? R2 : 1, REC2 = 4 * RB;
+    const uint8_t *lane_base2 = R2 > 0 ? packed2 + ((int64_t)mp * nkp * 32 + a.l) * REC2 : nullptr;
     int kp = kp0 + wave;
     tr_record<R> cur, nx1;
+    tr_record<RB> curb = {}, nx1b = {};
     bool requested = false;
 
     if constexpr (TP < 16) {
@@ -326,6 +333,10 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
                     requested = true;
                     cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
                     nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
+                    if constexpr (R2 > 0) {
+                        curb = tr_load_record<RB>(lane_base2 + (int64_t)min(kp, kp1 - 1) * 32 * REC2);
+                        nx1b = tr_load_record<RB>(lane_base2 + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC2);
+                    }
                 }
             };
             const bool quad_rows = quads && (bm.offset & 3) == 0 && log_len >= 2 && bm.offset + bm.bs <= in_features;
@@ -380,6 +391,10 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
     if (!requested) {
         cur = tr_load_record<R>(lane_base + (int64_t)min(kp, kp1 - 1) * 32 * REC);
         nx1 = tr_load_record<R>(lane_base + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC);
+        if constexpr (R2 > 0) {
+            curb = tr_load_record<RB>(lane_base2 + (int64_t)min(kp, kp1 - 1) * 32 * REC2);
+            nx1b = tr_load_record<RB>(lane_base2 + (int64_t)min(kp + TR_WAVES, kp1 - 1) * 32 * REC2);
+        }
     }
     if constexpr (TP > 1) {
         // tokens past B read zeros: clear their slots once (every k-pair of the slot)
@@ -390,16 +405,27 @@ tr_mma_fusein_body(const uint8_t *__restrict__ packed, const XT *__restrict__ x,
     }
     __syncthreads();
 
-    mma_acc<1> acc;
+    mma_acc<1> acc, accb;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) acc.v[s][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < 4; ++s) acc.v[s][0] = accb.v[s][0] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (; kp < kp1; kp += TR_WAVES) {
         tr_record<R> nx2 = nx1;                                  // nothing is requested past the wave's last record
-        if (kp + 2 * TR_WAVES < kp1) nx2 = tr_load_record<R>(lane_base + (int64_t)(kp + 2 * TR_WAVES) * 32 * REC);
+        tr_record<RB> nx2b = nx1b;
+        if (kp + 2 * TR_WAVES < kp1) {
+            nx2 = tr_load_record<R>(lane_base + (int64_t)(kp + 2 * TR_WAVES) * 32 * REC);
+            if constexpr (R2 > 0) nx2b = tr_load_record<RB>(lane_base2 + (int64_t)(kp + 2 * TR_WAVES) * 32 * REC2);
+        }
         const u32x4 *xsl = a.live ? lds + ((kp - kp0) * 8 + a.q) * TPS + a.tokl : zero_blk;
         acc = mma_record<R, TP, 1>(cur, a.next1, a.next2, xsl, acc);
+        if constexpr (R2 > 0) accb = mma_record<RB, TP, 1>(curb, a.next1, a.next2, xsl, accb);
         cur = nx1;
         nx1 = nx2;
+        curb = nx1b;
+        nx1b = nx2b;
+    }
+    if constexpr (R2 > 0) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc.v[s][0] += rs2 * accb.v[s][0];
     }
     // part_B: rows per K slot of the partial-sum array when it holds more rows than this call's
     // tokens (the routed-expert launch: one row per (token, expert) slot, `part` offset to this one)
@@ -416,6 +442,19 @@ tr_mma_fusein_kernel(const uint8_t *__restrict__ packed, const XT *__restrict__ 
     extern __shared__ u32x4 xs_lds[];
     tr_mma_fusein_body<R, XT, TP>(packed, x, x_stride, sv, B, m, k, in_features, S, bn_meta, n_blocks, margs,
                                   part, pscale, xs_lds);
+}
+
+// Both stages of a stacked layer (first stage 4 bits/weight, as every recipe of the reference has it:
+// glq_vllm/linear_method.py trellis recipes 5..8 bpw = 4 + 1..4), one token.
+template <int R2, typename XT>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_fusein_rvq_kernel(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ packed2, float rs2,
+                         const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv, int m, int k,
+                         int in_features, int S, const glqh_block_meta *__restrict__ bn_meta, int n_blocks,
+                         glqh_meta_args margs, float *__restrict__ part) {
+    extern __shared__ u32x4 xs_lds[];
+    tr_mma_fusein_body<4, XT, 1, R2>(packed, x, x_stride, sv, 1, m, k, in_features, S, bn_meta, n_blocks, margs,
+                                     part, 1.0f, xs_lds, 0, packed2, rs2);
 }
 
 // Several layers that read the same activations (fused q/k/v, gate/up:
@@ -793,6 +832,42 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
     return glqh_fail("fused-input trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
+// One token through both stages of a stacked layer (4 + R2 bits/weight) in one launch: part[K slot][row].
+int glqh_launch_trellis_mma_fusein_rvq(const void *packed, const void *packed2, int R2, float rs2, const void *x,
+                                       int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
+                                       int64_t in_features, int S, int ksplit, float *part,
+                                       const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                                       hipStream_t stream) {
+    glqh_range range("dequant_matmul");
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "fused-input trellis kernel: x must be f16 or bf16");
+    glqh_meta_args margs;
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
+    const glqh_block_meta *meta = n_blocks > 1 ? bn_meta : nullptr;
+    const int nb = n_blocks > 1 ? n_blocks : 1;
+    const size_t lds = fi_lds_bytes<1>(S);
+    const dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, 1);
+#define GLQH_FI2(RR, XT)                                                                                        \
+    hipLaunchKernelGGL((tr_mma_fusein_rvq_kernel<RR, XT>), grid, dim3(TR_THREADS), lds, stream,                 \
+                       (const uint8_t *)packed, (const uint8_t *)packed2, rs2, (const XT *)x, x_stride,         \
+                       (const f16 *)sv, (int)m, (int)k, (int)in_features, S, meta, nb, margs, part)
+#define GLQH_FI2_R(RR)                                                \
+    do {                                                              \
+        if (x_dtype == GLQH_F16) GLQH_FI2(RR, f16);                   \
+        else GLQH_FI2(RR, uint16_t);                                  \
+    } while (0)
+    switch (R2) {
+    case 1: GLQH_FI2_R(1); break;
+    case 2: GLQH_FI2_R(2); break;
+    case 3: GLQH_FI2_R(3); break;
+    case 4: GLQH_FI2_R(4); break;
+    default: return glqh_fail("fused-input trellis kernel: second stage of 1-4 bits/weight, got %d", R2);
+    }
+#undef GLQH_FI2_R
+#undef GLQH_FI2
+    GLQH_LAUNCH_CHECK("trellis fused-input two-stage launch");
+    return 0;
+}
+
 template <int R, typename XT>
 static int launch_mma_fusein_moe(const tr_moe_args &g, const void *x, int64_t x_stride, const void *sv, int64_t m,
                                  int64_t k, int64_t in_features, int S, int ksplit, const glqh_block_meta *bn_meta,
@@ -908,6 +983,7 @@ template <int R>
 static int fi_init_R() {
     const size_t b1 = fi_lds_bytes<1>(FI_MAX_S), b4 = fi_lds_bytes<4>(FI_MAX_S_TP4);
     if (fi_set_lds(tr_mma_fusein_moe_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_moe_kernel<R, uint16_t>, b1)) return 1;
+    if (fi_set_lds(tr_mma_fusein_rvq_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_rvq_kernel<R, uint16_t>, b1)) return 1;
     return fi_set_lds(tr_mma_fusein_kernel<R, f16, 1>, b1) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 1>, b1) ||
            fi_set_lds(tr_mma_fusein_kernel<R, f16, 4>, b4) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 4>, b4) ||
            fi_set_lds(tr_mma_fusein_group_kernel<R, f16, 1>, b1) ||

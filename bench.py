@@ -184,7 +184,8 @@ def moe_setup(torch, dev):
     2048 -> 2 x 768 -> 2048, top-8, 4 bpw, random code bits: 302 MB of streams, more than the 256 MB
     Infinity Cache).  Returns the op's weight arguments, a maker of (x, eight routing tables) for a
     token count, and the packed bytes of one expert.  Up to 95 slots every slot reads its expert's
-    stream; from 96 on the rows are grouped by expert."""
+    stream; from 96 on the rows are grouped by expert, and from 24 rows per expert on average (384 tokens)
+    the sorted rows go through the tile kernel."""
     from glq_amd import hadamard as H
     E, hid, inter, K = 128, 2048, 768, 8
     gen = torch.Generator().manual_seed(0)
@@ -436,13 +437,16 @@ def extras(torch, ext, dev):
         out["prefill_linear_error"] = f"{type(e).__name__}: {e}"
     try:
         args, routes_for, per_slot_bytes = moe_setup(torch, dev)
-        for T in (1, 16, 128, 256):                           # 8 / 128 slots per expert stream, 1024 / 2048 grouped by expert
+        # 8 / 128 slots per expert stream, 1024 / 2048 grouped by expert, 8192 / 32768 through the tile kernel
+        for T in (1, 16, 128, 256, 1024, 4096):
             xb, routes = routes_for(T)
             us = _graph_time(torch, lambda: [ext.glq_fused_moe_trellis_3inst_cuda(xb, i, w, *args) for i, w in routes],
-                             len(routes))
+                             len(routes), reps=20 if T <= 256 else 5)
             out[f"moe_experts_qwen3_30b_shape_T{T}_us"] = round(us, 2)
             if T == 1:                                        # eight expert streams read once each
                 out["moe_experts_qwen3_30b_shape_T1_GBs"] = round(per_slot_bytes * 8 / us / 1e3, 1)
+            if T >= 1024:                                     # two flops per weight and slot (4 bits per weight)
+                out[f"moe_experts_qwen3_30b_shape_T{T}_TFLOPs"] = round(2 * per_slot_bytes * 2 * 8 * T / us / 1e6, 1)
         del args
         torch.cuda.empty_cache()
     except Exception as e:
@@ -451,7 +455,7 @@ def extras(torch, ext, dev):
 
 
 CASES = ("trellis_gemv_16384", "e8_gemv_16384", "trellis_prefill_4096", "trellis_prefill_256", "e8_gemv_2stage", "e8_prefill_4096",
-         "e8_prefill_256", "e8_prefill_32", "trellis_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128", "moe_experts_256")
+         "e8_prefill_256", "e8_prefill_32", "trellis_prefill_32", "decoder", "batch1_step", "moe_experts_1", "moe_experts_16", "moe_experts_128", "moe_experts_256", "moe_experts_1024", "moe_experts_4096")
 E8_SETS = 10            # rotated E8 index sets of 29.4 MB: 294 MB, more than the 256 MB Infinity Cache
 
 

@@ -935,7 +935,7 @@ int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes,
                                        int64_t k, int64_t in_features, int S, int ksplit, float *part,
                                        const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
                                        hipStream_t stream);
-int glqh_launch_moe_output_rht(const float *part, int ks, int n_slots, int n_experts, const int64_t *topk_ids,
+int glqh_launch_moe_output_rht(const float *part, int ks, int part_f16, int n_slots, int n_experts, const int64_t *topk_ids,
                                const void *su_base, const float *wscale_dev, int64_t out_features, int64_t m_pad,
                                const int64_t *blocks_m, int64_t n_blocks_m, void *h_f16, int64_t h_stride,
                                hipStream_t stream);
@@ -945,15 +945,41 @@ int glqh_launch_moe_weighted_sum(const void *y_f16, int64_t y_stride, int num_to
                                  const int64_t *topk_ids, const float *topk_w, int64_t out_features, void *out,
                                  int out_dtype, int64_t out_stride, hipStream_t stream);
 
-int glqh_launch_moe_route(const int64_t *topk_ids, int n_slots, int n_experts, int *perm, int *offs,
-                          hipStream_t stream);
+int glqh_moe_mid_eligible(int64_t m_pad13, const int64_t *blocks_m13, int64_t n_blocks_m13, int64_t n_pad2,
+                          const int64_t *blocks_n2, int64_t n_blocks_n2);
+int glqh_launch_moe_mid(const float *part, int ks, int part_f16, int n_slots, int n_experts, const int64_t *topk_ids,
+                        const void *su_base, const float *wscale_dev, int64_t out_features13, int64_t m_pad13,
+                        const int64_t *blocks_m13, int64_t n_blocks_m13, const int *perm, const int *pexp, const int *n_valid,
+                        int64_t intermediate, int act, const void *sv2, int64_t n_pad2, const int64_t *blocks_n2,
+                        int64_t n_blocks_n2, void *out_f16, int layout, int64_t Mp, hipStream_t stream);
+int glqh_launch_moe_final(const float *part, int ks, int part_f16, int num_tokens, int top_k, int n_experts,
+                          const int64_t *topk_ids, const float *topk_w, const void *su_base, const float *wscale_dev,
+                          int64_t out_features, int64_t m_pad, const int64_t *blocks_m, int64_t n_blocks_m, void *out,
+                          int out_dtype, int64_t out_stride, hipStream_t stream);
+int glqh_moe_route_segments(int n_slots, int n_experts);
+size_t glqh_moe_route_scratch_ints(int n_slots, int n_experts);
+int glqh_launch_moe_route(const int64_t *topk_ids, int n_slots, int n_experts, int *perm, int *pexp, int *offs,
+                          int *scratch, hipStream_t stream);
 int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes, int R, const int *perm,
                                         const int *offs, int n_slots, int n_experts, int x_div,
                                         const float *pscale_dev, const void *x_f16, int64_t m, int64_t k, int S,
                                         int ksplit, float *part, hipStream_t stream);
 
+// many rows per expert: the tile kernel on the expert-sorted slots (trellis_tile.hip)
+int glqh_trellis_tile_moe_tokens(int64_t n_slots, int64_t n_experts);
+int64_t glqh_trellis_tile_moe_padded(int64_t n_slots, int64_t n_experts);
+int64_t glqh_trellis_tile_moe_max_tiles(int64_t n_slots, int64_t n_experts);
+int glqh_launch_trellis_tile_moe_table(const int *offs, int n_slots, int n_experts, void *tiles, int *n_tiles,
+                                       hipStream_t stream);
+int glqh_launch_trellis_pack_moe(const void *x_f16, void *xb, const int *perm, const int *offs, int n_slots,
+                                 int n_experts, int x_div, int64_t k, hipStream_t stream);
+int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t stride_bytes, int R, const int *perm,
+                                 const void *tiles, const int *n_tiles, const float *pscale_dev, int n_slots,
+                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream);
+
 struct moe_plan {
     int R1, R2, S, ks, ks_all;
+    int tile;                                                  // the tile kernel's form: one K slot, fp16 sums
     size_t part_bytes;
 };
 
@@ -973,6 +999,36 @@ static int64_t moe_group_min(int64_t n_experts) {
     return d < 16 ? 16 : d;
 }
 
+// From this many rows per expert on average (slots / experts that can have rows) the grouped form hands over to
+// the tile kernel's: below, an expert's stream is read once per 64 of its rows by a GEMV-shaped workgroup; above,
+// its decoded weights meet up to 256 rows at a time on the matrix cores.  GLQ_MOE_TILE_MIN_ROWS overrides (read
+// once; 0 = never).
+static int64_t moe_tile_min_rows() {
+    static const int64_t v = [] {
+        const char *e = getenv("GLQ_MOE_TILE_MIN_ROWS");
+        return (int64_t)(e && *e ? atoll(e) : 24);
+    }();
+    return v;
+}
+
+static bool moe_tile_form(int64_t n_slots, int64_t n_experts) {
+    const int64_t live = n_experts < n_slots ? n_experts : n_slots, mn = moe_tile_min_rows();
+    return mn > 0 && n_slots >= moe_group_min(n_experts) && n_slots >= mn * live;
+}
+
+// GLQ_MOE_FUSE=0 (read once): the launches between and after the decode launches stay separate at every slot count
+// (output transform, activation, input transform, repack; output transform, weighted sum).
+static bool moe_fuse_enabled() {
+    static const bool on = [] {
+        const char *e = getenv("GLQ_MOE_FUSE");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+// from this many slots on (below, the separate launches are as fast or faster: 128 slots 108.8 us separate against
+// 112.6 fused, 512 slots 147.1 / 148.2, 1024 slots 161.2 / 161.5, 2048 slots 222 / 215, 8192 slots 531 / 493)
+constexpr int MOE_FUSE_MIN_SLOTS = 1024;
+
 static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, int64_t n_experts, const char *what, moe_plan *p) {
     GLQH_REQUIRE(w && w->packed && w->su_f16 && w->sv_f16 && w->wscale_dev, "routed experts %s: null pointer", what);
     if (tr_bits_from_packed(w->packed_cols, 0, &p->R1) || tr_check_shape(w->m_pad, w->n_pad, w->packed_rows)) return 1;
@@ -989,7 +1045,12 @@ static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, int64_t n_expe
     const bool pow2_n = (w->n_pad & (w->n_pad - 1)) == 0;
     GLQH_REQUIRE(w->n_blocks_n > 1 ? (w->bn_meta_dev != nullptr && w->blocks_n != nullptr) : pow2_n,
                  "routed experts %s: input block sizes missing", what);
-    if (n_slots >= moe_group_min(n_experts)) {
+    p->tile = 0;
+    if (moe_tile_form(n_slots, n_experts)) {
+        p->tile = 1;
+        p->S = 0;
+        p->ks = 1;
+    } else if (n_slots >= moe_group_min(n_experts)) {
         // about four workgroups per CU if every expert that can have rows has some
         const int64_t nkp = w->n_pad / 32, wgs = ((w->m_pad + 63) / 64) * (n_experts < n_slots ? n_experts : n_slots);
         int64_t ks = ((int64_t)glqh_device_cus() * 4 + wgs - 1) / wgs;
@@ -1007,10 +1068,11 @@ static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, int64_t n_expe
 }
 
 // workspace: part13 | h (slots x 2I f16) | a (slots x I f16) | part2 | y (slots x hidden f16), and for the
-// grouped form: perm (slots int) | offs (experts + 1 int) | transformed activations (fp16 rows of both
+// grouped form: perm | pexp (slots int each) | offs (experts + 1 int) | routing scratch | transformed activations (fp16 rows of both
 // projections in turn)
+// and for the tile form: the activations packed in sorted order | the token tiles (int4 each) | their number
 struct moe_ws {
-    size_t part13, h, a, part2, y, perm, offs, xhat, total;
+    size_t part13, h, a, part2, y, perm, pexp, offs, route, xhat, xb, tiles, n_tiles, total;
 };
 
 static moe_ws moe_ws_layout(const glqh_moe_proj *w13, const glqh_moe_proj *w2, const moe_plan &p13, const moe_plan &p2,
@@ -1022,12 +1084,21 @@ static moe_ws moe_ws_layout(const glqh_moe_proj *w13, const glqh_moe_proj *w2, c
     l.a = o; o += align256((size_t)n_slots * w2->in_features * sizeof(f16));
     l.part2 = o; o += p2.part_bytes;
     l.y = o; o += align256((size_t)n_slots * w2->out_features * sizeof(f16));
-    l.perm = l.offs = l.xhat = o;
+    l.perm = l.pexp = l.offs = l.route = l.xhat = o;
     if (n_slots >= moe_group_min(n_experts)) {
         l.perm = o; o += align256((size_t)n_slots * sizeof(int));
+        l.pexp = o; o += align256((size_t)n_slots * sizeof(int));
         l.offs = o; o += align256((size_t)(n_experts + 1) * sizeof(int));
+        l.route = o; o += align256(glqh_moe_route_scratch_ints((int)n_slots, (int)n_experts) * sizeof(int));
         const size_t x13 = (size_t)num_tokens * w13->n_pad, x2 = (size_t)n_slots * w2->n_pad;
         l.xhat = o; o += align256((x13 > x2 ? x13 : x2) * sizeof(f16));
+    }
+    l.xb = l.tiles = l.n_tiles = o;
+    if (p13.tile) {
+        const size_t Mp = (size_t)glqh_trellis_tile_moe_padded(n_slots, n_experts);
+        l.xb = o; o += align256(Mp * (size_t)(w13->n_pad > w2->n_pad ? w13->n_pad : w2->n_pad) * sizeof(f16));
+        l.tiles = o; o += align256((size_t)glqh_trellis_tile_moe_max_tiles(n_slots, n_experts) * 16);
+        l.n_tiles = o; o += 256;
     }
     l.total = o;
     return l;
@@ -1047,8 +1118,9 @@ extern "C" size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int
 static int moe_decode_grouped(const glqh_moe_proj *w, const moe_plan &p, const int *perm, const int *offs, int n_slots,
                               int n_experts, int x_div, const void *x, int x_dtype, int64_t x_stride, int64_t x_rows,
                               void *xhat, float *part, hipStream_t st) {
-    if (glqh_launch_input_rht(x, x_dtype, x_stride, w->sv_f16, xhat, GLQH_F16, x_rows, w->in_features, w->n_pad,
-                              w->bn_meta_dev, w->blocks_n, w->n_blocks_n, 0.0f, st))
+    // x == nullptr: xhat already holds the transformed rows
+    if (x && glqh_launch_input_rht(x, x_dtype, x_stride, w->sv_f16, xhat, GLQH_F16, x_rows, w->in_features, w->n_pad,
+                                   w->bn_meta_dev, w->blocks_n, w->n_blocks_n, 0.0f, st))
         return 1;
     if (glqh_launch_trellis_mma_moe_grouped(w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, offs, n_slots,
                                             n_experts, x_div, nullptr, xhat, w->m_pad, w->n_pad, p.S, p.ks, part, st))
@@ -1057,6 +1129,27 @@ static int moe_decode_grouped(const glqh_moe_proj *w, const moe_plan &p, const i
         glqh_launch_trellis_mma_moe_grouped(w->packed2, w->packed_rows * w->packed2_cols * 2, p.R2, perm, offs, n_slots,
                                             n_experts, x_div, w->inv_rs2_dev, xhat, w->m_pad, w->n_pad, p.S, p.ks,
                                             part + (int64_t)p.ks * n_slots * w->m_pad, st))
+        return 1;
+    return 0;
+}
+
+// one projection through the tile kernel: input transform of the rows, their packed copy in sorted order, one
+// launch per stage into fp16 sums [stage][slot][row] (the second stage's already times its scale)
+static int moe_decode_tile(const glqh_moe_proj *w, const moe_plan &p, const int *perm, const int *offs, const void *tiles,
+                           const int *n_tiles, int n_slots, int n_experts, int x_div, const void *x, int x_dtype,
+                           int64_t x_stride, int64_t x_rows, void *xhat, void *xb, float *part, hipStream_t st) {
+    if (x) {                                                   // nullptr: xb already holds the packed activations
+        if (glqh_launch_input_rht(x, x_dtype, x_stride, w->sv_f16, xhat, GLQH_F16, x_rows, w->in_features, w->n_pad,
+                                  w->bn_meta_dev, w->blocks_n, w->n_blocks_n, 0.0f, st))
+            return 1;
+        if (glqh_launch_trellis_pack_moe(xhat, xb, perm, offs, n_slots, n_experts, x_div, w->n_pad, st)) return 1;
+    }
+    if (glqh_launch_trellis_tile_moe(xb, w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, tiles, n_tiles,
+                                     nullptr, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st))
+        return 1;
+    if (p.R2 && glqh_launch_trellis_tile_moe(xb, w->packed2, w->packed_rows * w->packed2_cols * 2, p.R2, perm, tiles,
+                                             n_tiles, w->inv_rs2_dev, n_slots, n_experts, w->m_pad, w->n_pad,
+                                             (f16 *)part + (int64_t)n_slots * w->m_pad, 1, st))
         return 1;
     return 0;
 }
@@ -1109,23 +1202,52 @@ extern "C" int glqh_fused_moe_trellis_3inst(const void *x, int x_dtype, int64_t 
     void *xhat = base + l.xhat;
     const bool grouped = n_slots >= moe_group_min(num_experts);
     GLQH_REQUIRE(!grouped || num_experts <= 65535, "routed experts: at most 65535 experts, got %lld", (long long)num_experts);
-    if (grouped && glqh_launch_moe_route(topk_ids, n_slots, (int)num_experts, perm, offs, st)) return 1;
+    int *pexp = (int *)(base + l.pexp);
+    if (grouped && glqh_launch_moe_route(topk_ids, n_slots, (int)num_experts, perm, pexp, offs, (int *)(base + l.route), st))
+        return 1;
+    const bool tile = p13.tile != 0;
+    void *xb = base + l.xb, *tiles = base + l.tiles;
+    int *n_tiles = (int *)(base + l.n_tiles);
+    if (tile && glqh_launch_trellis_tile_moe_table(offs, n_slots, (int)num_experts, tiles, n_tiles, st)) return 1;
     // gate | up of every slot: decode on the token's row, output transform with the expert's signs
-    if (grouped ? moe_decode_grouped(w13, p13, perm, offs, n_slots, (int)num_experts, (int)top_k, x, x_dtype, x_stride,
-                                     num_tokens, xhat, part13, st)
-                : moe_decode(w13, p13, topk_ids, n_slots, (int)num_experts, (int)top_k, x, x_dtype, x_stride, part13, st))
+    if (tile ? moe_decode_tile(w13, p13, perm, offs, tiles, n_tiles, n_slots, (int)num_experts, (int)top_k, x, x_dtype,
+                               x_stride, num_tokens, xhat, xb, part13, st)
+        : grouped ? moe_decode_grouped(w13, p13, perm, offs, n_slots, (int)num_experts, (int)top_k, x, x_dtype, x_stride,
+                                       num_tokens, xhat, part13, st)
+                  : moe_decode(w13, p13, topk_ids, n_slots, (int)num_experts, (int)top_k, x, x_dtype, x_stride, part13, st))
         return 1;
-    if (glqh_launch_moe_output_rht(part13, p13.ks_all, n_slots, (int)num_experts, topk_ids, w13->su_f16,
-                                   w13->wscale_dev, w13->out_features, w13->m_pad, w13->blocks_m, w13->n_blocks_m, h,
-                                   w13->out_features, st))
-        return 1;
-    if (glqh_launch_moe_gated_act(h, w13->out_features, hact, n_slots, intermediate_size, activation_type, st)) return 1;
+    // between the decode launches: one launch per slot row for the grouped forms, three or four otherwise
+    const bool mid = grouped && n_slots >= MOE_FUSE_MIN_SLOTS && moe_fuse_enabled() &&
+                     glqh_moe_mid_eligible(w13->m_pad, w13->blocks_m, w13->n_blocks_m, w2->n_pad, w2->blocks_n,
+                                           w2->n_blocks_n);
+    const void *x2 = hact;
+    if (mid) {
+        if (glqh_launch_moe_mid(part13, p13.ks_all, tile, n_slots, (int)num_experts, topk_ids, w13->su_f16, w13->wscale_dev,
+                                w13->out_features, w13->m_pad, w13->blocks_m, w13->n_blocks_m, perm, pexp, offs + num_experts,
+                                intermediate_size, activation_type, w2->sv_f16, w2->n_pad, w2->blocks_n, w2->n_blocks_n,
+                                tile ? xb : xhat, tile ? 2 : 0,
+                                tile ? glqh_trellis_tile_moe_padded(n_slots, num_experts) : 0, st))
+            return 1;
+        x2 = nullptr;
+    } else {
+        if (glqh_launch_moe_output_rht(part13, p13.ks_all, tile, n_slots, (int)num_experts, topk_ids, w13->su_f16,
+                                       w13->wscale_dev, w13->out_features, w13->m_pad, w13->blocks_m, w13->n_blocks_m, h,
+                                       w13->out_features, st))
+            return 1;
+        if (glqh_launch_moe_gated_act(h, w13->out_features, hact, n_slots, intermediate_size, activation_type, st)) return 1;
+    }
     // down projection of every slot, then the weighted sum over each token's choices, in their order
-    if (grouped ? moe_decode_grouped(w2, p2, perm, offs, n_slots, (int)num_experts, 1, hact, GLQH_F16, intermediate_size,
-                                     n_slots, xhat, part2, st)
-                : moe_decode(w2, p2, topk_ids, n_slots, (int)num_experts, 1, hact, GLQH_F16, intermediate_size, part2, st))
+    if (tile ? moe_decode_tile(w2, p2, perm, offs, tiles, n_tiles, n_slots, (int)num_experts, 1, x2, GLQH_F16,
+                               intermediate_size, n_slots, xhat, xb, part2, st)
+        : grouped ? moe_decode_grouped(w2, p2, perm, offs, n_slots, (int)num_experts, 1, x2, GLQH_F16, intermediate_size,
+                                       n_slots, xhat, part2, st)
+                  : moe_decode(w2, p2, topk_ids, n_slots, (int)num_experts, 1, hact, GLQH_F16, intermediate_size, part2, st))
         return 1;
-    if (glqh_launch_moe_output_rht(part2, p2.ks_all, n_slots, (int)num_experts, topk_ids, w2->su_f16, w2->wscale_dev,
+    if (n_slots >= MOE_FUSE_MIN_SLOTS && moe_fuse_enabled())
+        return glqh_launch_moe_final(part2, p2.ks_all, tile, (int)num_tokens, (int)top_k, (int)num_experts, topk_ids,
+                                     topk_weights, w2->su_f16, w2->wscale_dev, w2->out_features, w2->m_pad, w2->blocks_m,
+                                     w2->n_blocks_m, out, out_dtype, out_stride, st);
+    if (glqh_launch_moe_output_rht(part2, p2.ks_all, tile, n_slots, (int)num_experts, topk_ids, w2->su_f16, w2->wscale_dev,
                                    w2->out_features, w2->m_pad, w2->blocks_m, w2->n_blocks_m, yslot, w2->out_features,
                                    st))
         return 1;

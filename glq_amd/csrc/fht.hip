@@ -296,9 +296,11 @@ input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__r
 // v = the transformed sums of elements E * tid .. E * tid + E - 1 of block `blk`, row b (before the
 // signs and the 1/sqrt(bs)): direct rows or split-K partial sums in, register transform, runs restored.
 // Every thread of the workgroup calls.
+// (the first half, what a thread reads: callers that transform several rows in turn request the next row's
+// sums before they transform this one's)
 template <int E>
-__device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysrc &src, int64_t b, int m_pad,
-                                                   const rht_slice &blk, float *s, int tid, bool active, int te) {
+__device__ __forceinline__ void output_wide_load(float (&v)[E], const glqh_ysrc &src, int64_t b, int m_pad,
+                                                 const rht_slice &blk, bool active, int te) {
     const int i = E * te;
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = 0.0f;
@@ -339,8 +341,19 @@ __device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysr
             }
         }
     }
+}
+
+template <int E>
+__device__ __forceinline__ void output_wide_transform(float (&v)[E], const rht_slice &blk, float *s, int tid, bool active) {
     fht_wave<E>(v, blk.log_len, s, tid);
     reg_gather_runs<E>(v, blk.log_len, s, tid, active);
+}
+
+template <int E>
+__device__ __forceinline__ void output_wide_values(float (&v)[E], const glqh_ysrc &src, int64_t b, int m_pad,
+                                                   const rht_slice &blk, float *s, int tid, bool active, int te) {
+    output_wide_load<E>(v, src, b, m_pad, blk, active, te);
+    output_wide_transform<E>(v, blk, s, tid, active);
 }
 
 template <int E, typename YT>
@@ -882,7 +895,7 @@ int glqh_rht_init(void) { return 0; }
 namespace {
 struct moe_out_args {
     const float *part;
-    int ks, n_slots, n_experts;
+    int ks, part_f16, n_slots, n_experts;
     const int64_t *topk_ids;
     const f16 *su_base;
     const float *wscale_dev;
@@ -894,6 +907,7 @@ __device__ __forceinline__ glqh_ysrc moe_src(const moe_out_args &a, float scale)
     src.part = a.part;
     src.part_kstride = (int64_t)a.n_slots * a.m_pad;
     src.ksplit = a.ks;
+    src.part_f16 = a.part_f16;
     src.scale[0] = scale;
     src.nparts = 1;
     return src;
@@ -918,20 +932,243 @@ moe_output_rht_kernel(moe_out_args a, f16 *__restrict__ h, int64_t h_stride, glq
     else output_rht_wide_body<8, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s, slot, role);
 }
 
+// The same for many slots, dealt out like output_rht_wide_kernel's rows: eight slots per workgroup group on the
+// eight XCDs, blocks of up to 512 rows with 4096 / bs slots per workgroup.  A thread's slot decides its signs and
+// scale; slots of an invalid expert read nothing (their sums were never written) and get zeros.
+template <int E>
+__device__ __forceinline__ void moe_output_wide_row(const moe_out_args &a, f16 *__restrict__ h, int64_t h_stride,
+                                                    const rht_slice &blk, float *s, int64_t slot, const wide_role role) {
+    const int64_t e = a.topk_ids[slot];
+    const bool valid = e >= 0 && e < a.n_experts;
+    const glqh_ysrc src = moe_src(a, valid ? a.wscale_dev[e] : 0.0f);
+    const f16 *su = a.su_base + (valid ? e : 0) * a.m_pad;
+    wide_role r = role;
+    r.active = role.active && valid;
+    output_rht_wide_body<E, f16>(src, su, h, h_stride, a.out_features, a.m_pad, blk, s, slot, r);
+    if (role.active && !valid && E * role.te < blk.bs) {
+        const int row = blk.off + E * role.te;
+#pragma unroll
+        for (int j = 0; j < E; ++j)
+            if (row + j < a.out_features) h[slot * h_stride + row + j] = (f16)0.0f;
+    }
+}
+
+__global__ void __launch_bounds__(REG_THREADS)
+moe_output_rht_wide_kernel(moe_out_args a, f16 *__restrict__ h, int64_t h_stride, int n_blocks, glqh_meta_args margs) {
+    extern __shared__ float s[];
+    const int L = blockIdx.x, xcd = L & 7, member = (L >> 3) & 7, rest = L >> 6, g = rest / n_blocks;
+    const rht_slice blk = rht_slice_of(margs, 0.0f, rest % n_blocks);
+    const int r0 = g * 64 + member * 8, B = a.n_slots;
+    if (blk.log_bs <= WIDE_SMALL_LOG) {
+        const int lt = 12 - blk.log_bs, T = 1 << lt;
+        if ((r0 & (T - 1)) != 0 || xcd != ((r0 >> lt) & 7) || r0 >= B) return;
+        const int ntok = min(T, B - r0);
+        const wide_role role = wide_role_of(blk, ntok);
+        moe_output_wide_row<8>(a, h, h_stride, blk, s, (int64_t)r0 + min(role.tok, ntok - 1), role);
+        return;
+    }
+    const int64_t b = (int64_t)r0 + xcd;
+    if (b >= B) return;                                       // uniform over the workgroup
+    const wide_role role = wide_role_of(blk, 1);
+    if (blk.log_bs > 12) moe_output_wide_row<16>(a, h, h_stride, blk, s, b, role);
+    else moe_output_wide_row<8>(a, h, h_stride, blk, s, b, role);
+}
+
+__device__ __forceinline__ float moe_gate(float g, int act) {
+    if (act == 0) return g / (1.0f + expf(-g));
+    if (act == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    const float q = fmaxf(g, 0.0f);
+    return q * q;
+}
+
+// Everything between the two decode launches for a slot whose rows are grouped by expert, in one workgroup per
+// slot: the first projection's output transform (sums -> h, rounded to fp16 as the separate launch stores
+// it), act(gate) * up (fp16), and the second projection's input transform, written where its decode launch reads:
+// LAYOUT 0 row `slot` of (n_slots, n_pad2), LAYOUT 2 position `pos` of the tile kernel's blocked operand.  h and
+// the activated row live in LDS only.  The workgroups walk the sorted order (eight neighbouring positions on
+// one XCD: in the blocked layout their 16-byte pieces share lines); slots of an invalid expert are not in it.
+struct moe_mid_args {
+    moe_out_args o;
+    const f16 *sv2;
+    const int *perm, *pexp, *n_valid;                            // slot and expert of every position of the sorted order
+    int intermediate, act, n_pad2, Mp, nb13, nb2, s_floats;
+};
+
+template <int LAYOUT>
+__global__ void __launch_bounds__(REG_THREADS)
+moe_mid_kernel(moe_mid_args a, f16 *__restrict__ out, glqh_meta_args m13, glqh_meta_args m2) {
+    extern __shared__ float s[];
+    const int L = blockIdx.x, pos = (L >> 6) * 64 + (L & 7) * 8 + ((L >> 3) & 7);
+    if (pos >= *a.n_valid) return;                               // uniform over the workgroup
+    const int slot = a.perm[pos];
+    const int64_t e = a.pexp[pos];
+    f16 *hrow = (f16 *)(s + a.s_floats), *arow = hrow + a.o.m_pad;
+    const int tid = threadIdx.x;
+    const wide_role role = {tid, 0, (int)blockDim.x, 0, true};
+    const glqh_ysrc src = moe_src(a.o, a.o.wscale_dev[e]);
+    const f16 *su = a.o.su_base + e * a.o.m_pad;
+    // the blocks of the first projection's row in turn, eight elements per thread; the next block's sums and
+    // signs are requested before this one's are transformed (a block of 8192 points: sixteen per thread, by itself)
+    struct req {
+        float v[8], f[8];
+    };
+    auto request = [&](req &r, const rht_slice &blk) {
+        const bool active = 8 * tid < blk.bs;
+        output_wide_load<8>(r.v, src, slot, a.o.m_pad, blk, active, tid);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r.f[j] = 0.0f;
+        if (active && blk.off + 8 * tid < a.o.out_features) load8<f16>(su + blk.off + 8 * tid, r.f);
+    };
+    const int big = rht_slice_of(m13, 0.0f, 0).bs > 8 * (int)blockDim.x ? 1 : 0;   // only the first block can be
+    if (big) output_rht_wide_body<16, f16>(src, su, hrow, 0, a.o.out_features, a.o.m_pad, rht_slice_of(m13, 0.0f, 0), s, slot, role);
+    req cur, nxt;
+    if (big < a.nb13) request(cur, rht_slice_of(m13, 0.0f, big));
+    for (int bi = big; bi < a.nb13; ++bi) {
+        const rht_slice blk = rht_slice_of(m13, 0.0f, bi);
+        if (bi + 1 < a.nb13) request(nxt, rht_slice_of(m13, 0.0f, bi + 1));
+        if (bi) __syncthreads();                                 // the previous block is done with the exchange space
+        const bool active = 8 * tid < blk.bs;
+        output_wide_transform<8>(cur.v, blk, s, tid, active);
+        const int row = blk.off + 8 * tid;
+        if (active && row < a.o.out_features) {
+            float w[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w[j] = cur.v[j] * (blk.norm * cur.f[j]);
+            if (row + 8 <= a.o.out_features) {
+                store8<f16>(hrow + row, w);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (row + j < a.o.out_features) hrow[row + j] = (f16)w[j];
+            }
+        }
+        cur = nxt;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < a.intermediate; i += blockDim.x)
+        arow[i] = (f16)(moe_gate((float)hrow[i], a.act) * (float)hrow[a.intermediate + i]);
+    for (int bi = 0; bi < a.nb2; ++bi) {
+        const rht_slice blk = rht_slice_of(m2, 0.0f, bi);
+        __syncthreads();                                         // arow written / the previous block done with s
+        const int token = LAYOUT == 2 ? pos : slot;
+        if (blk.bs > 8 * (int)blockDim.x)
+            input_rht_wide_body<16, f16, f16, LAYOUT>(arow, 0, a.sv2, out, a.intermediate, a.n_pad2, a.Mp, token, blk, s, role);
+        else
+            input_rht_wide_body<8, f16, f16, LAYOUT>(arow, 0, a.sv2, out, a.intermediate, a.n_pad2, a.Mp, token, blk, s, role);
+    }
+}
+
+// The second projection's output transform and the weighted sum over a token's choices in one launch, for many
+// tokens: rows = tokens, dealt out like output_rht_wide_kernel's; a thread transforms its part of every choice in
+// turn, rounds it to fp16 as the separate launch stores it, and adds it times the routing weight in fp32, choices
+// in order (glq_moe_weighted_scatter_reduce_kernel, glq/csrc/glq_cuda.cu:4520-4537).
+template <int E, typename YT>
+__device__ __forceinline__ void moe_final_row(const moe_out_args &a, const float *__restrict__ topk_w, int top_k,
+                                              YT *__restrict__ out, int64_t out_stride, const rht_slice &blk, float *s,
+                                              int64_t token, const wide_role role) {
+    const int tid = threadIdx.x;
+    const bool active = role.active && E * role.te < blk.bs;
+    const int row = blk.off + E * role.te;
+    float acc[E];
+#pragma unroll
+    for (int j = 0; j < E; ++j) acc[j] = 0.0f;
+    // the next choice's sums, signs and weight are requested before this one's are transformed
+    struct choice {
+        float v[E], f[E], w;
+        bool valid;
+    };
+    auto request = [&](choice &ch, int c) {
+        const int64_t slot = token * top_k + c;
+        const int64_t e = a.topk_ids[slot];
+        ch.valid = e >= 0 && e < a.n_experts;
+        const glqh_ysrc src = moe_src(a, ch.valid ? a.wscale_dev[e] : 0.0f);
+        output_wide_load<E>(ch.v, src, slot, a.m_pad, blk, active && ch.valid, role.te);
+        ch.w = 0.0f;
+#pragma unroll
+        for (int j = 0; j < E; ++j) ch.f[j] = 0.0f;
+        if (active && ch.valid && row < a.out_features) {
+#pragma unroll
+            for (int j = 0; j < E; j += 8) load8<f16>(a.su_base + e * a.m_pad + row + j, ch.f + j);
+            ch.w = topk_w[slot];
+        }
+    };
+    choice cur, nxt;
+    request(cur, 0);
+    for (int c = 0; c < top_k; ++c) {
+        if (c + 1 < top_k) request(nxt, c + 1);
+        if (c) __syncthreads();                                  // the previous choice is done with the exchange space
+        output_wide_transform<E>(cur.v, blk, s, tid, active && cur.valid);
+        if (active && cur.valid && row < a.out_features) {
+#pragma unroll
+            for (int j = 0; j < E; ++j) acc[j] += cur.w * (float)(f16)(cur.v[j] * (blk.norm * cur.f[j]));
+        }
+        cur = nxt;
+    }
+    if (active && row < a.out_features) {
+        YT *orow = out + token * out_stride;
+        if (row + E <= a.out_features) {
+#pragma unroll
+            for (int j = 0; j < E; j += 8) store8<YT>(orow + row + j, acc + j);
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+                if (row + j < a.out_features) orow[row + j] = f32_to_act<YT>(acc[j]);
+        }
+    }
+}
+
+// BIG: the row has a block of 8192 points (sixteen elements per thread there, and their registers: a kernel of
+// its own, so that the others keep their occupancy)
+template <typename YT, bool BIG>
+__global__ void __launch_bounds__(REG_THREADS)
+moe_final_kernel(moe_out_args a, const float *__restrict__ topk_w, int top_k, int num_tokens, YT *__restrict__ out,
+                 int64_t out_stride, int n_blocks, glqh_meta_args margs) {
+    extern __shared__ float s[];
+    const int L = blockIdx.x, xcd = L & 7, member = (L >> 3) & 7, rest = L >> 6, g = rest / n_blocks;
+    const rht_slice blk = rht_slice_of(margs, 0.0f, rest % n_blocks);
+    const int r0 = g * 64 + member * 8, B = num_tokens;
+    if (blk.log_bs <= WIDE_SMALL_LOG) {
+        const int lt = 12 - blk.log_bs, T = 1 << lt;
+        if ((r0 & (T - 1)) != 0 || xcd != ((r0 >> lt) & 7) || r0 >= B) return;
+        const int ntok = min(T, B - r0);
+        const wide_role role = wide_role_of(blk, ntok);
+        moe_final_row<8, YT>(a, topk_w, top_k, out, out_stride, blk, s, (int64_t)r0 + min(role.tok, ntok - 1), role);
+        return;
+    }
+    const int64_t b = (int64_t)r0 + xcd;
+    if (b >= B) return;                                       // uniform over the workgroup
+    const wide_role role = wide_role_of(blk, 1);
+    if constexpr (BIG) {
+        if (blk.log_bs > 12) {
+            moe_final_row<16, YT>(a, topk_w, top_k, out, out_stride, blk, s, b, role);
+            return;
+        }
+    }
+    moe_final_row<8, YT>(a, topk_w, top_k, out, out_stride, blk, s, b, role);
+}
+
 // out[slot][i] = act(h[slot][i]) * h[slot][intermediate + i]: 0 SiLU, 1 GELU (tanh form), 2 squared ReLU
-// (glq/csrc/glq_cuda.cu:4540-4559)
+// (glq/csrc/glq_cuda.cu:4540-4559).  V elements per thread (8 when the rows allow 16-byte accesses).
+template <int V>
 __global__ void __launch_bounds__(256)
 moe_gated_act_kernel(const f16 *__restrict__ h, int64_t h_stride, f16 *__restrict__ out, int n_slots,
                      int intermediate, int act) {
+    const int per_row = intermediate / V;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (int64_t)n_slots * intermediate) return;
-    const int slot = (int)(idx / intermediate), i = (int)(idx % intermediate);
-    const float g = (float)h[slot * h_stride + i], up = (float)h[slot * h_stride + intermediate + i];
-    float v;
-    if (act == 0) v = g / (1.0f + expf(-g));
-    else if (act == 1) v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-    else { const float r = fmaxf(g, 0.0f); v = r * r; }
-    out[idx] = (f16)(v * up);
+    if (idx >= (int64_t)n_slots * per_row) return;
+    const int slot = (int)(idx / per_row), i = V * (int)(idx % per_row);
+    float g[V], up[V], r[V];
+    if constexpr (V == 8) {
+        load8<f16>(h + slot * h_stride + i, g);
+        load8<f16>(h + slot * h_stride + intermediate + i, up);
+    } else {
+        g[0] = (float)h[slot * h_stride + i];
+        up[0] = (float)h[slot * h_stride + intermediate + i];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) r[j] = (float)(f16)(moe_gate(g[j], act) * up[j]);
+    if constexpr (V == 8) store8<f16>(out + (int64_t)slot * intermediate + i, r);
+    else out[(int64_t)slot * intermediate + i] = (f16)r[0];
 }
 
 // out[token][row] = sum_j w[token][j] * y[token * top_k + j][row], j in order, fp32 accumulation of the fp16
@@ -964,7 +1201,7 @@ moe_weighted_sum_kernel(const f16 *__restrict__ y, int64_t y_stride, const int64
 // slot order, from that position on.  Fixed by the routing alone: the same table on every call.
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const int64_t *__restrict__ topk_ids, int n_slots, int n_experts, int *__restrict__ perm,
-                 int *__restrict__ offs) {
+                 int *__restrict__ pexp, int *__restrict__ offs) {
     const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (e > n_experts) return;                                   // uniform over the wave
     constexpr int U = 8;                                         // 512 slots requested before the first is looked at
@@ -986,7 +1223,81 @@ moe_route_kernel(const int64_t *__restrict__ topk_ids, int n_slots, int n_expert
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const unsigned long long hit = __ballot(id[u] == e);
-            if (id[u] == e) perm[below + mine + __builtin_popcountll(hit & ((1ull << lane) - 1ull))] = base + 64 * u + lane;
+            if (id[u] == e) {
+                const int at = below + mine + __builtin_popcountll(hit & ((1ull << lane) - 1ull));
+                perm[at] = base + 64 * u + lane;
+                pexp[at] = e;
+            }
+            mine += __builtin_popcountll(hit);
+        }
+    }
+}
+
+// The same table for many slots, in two launches: the slots in SEG segments, wave (expert, segment) first counts
+// its expert's slots in its segment (cnt[segment][expert], expert n_experts = every valid slot), then finds its
+// first position from the counts of the experts below and of the segments before it.  The one launch above has
+// every expert's wave walk all the slots twice: 80 us at 32768 slots, 21 us at 8192.
+constexpr int MOE_ROUTE_SEG_SLOTS = 2048;
+constexpr int MOE_ROUTE_MAX_SEG = 32;
+constexpr int MOE_OUT_WIDE_MIN = 64;
+
+__device__ __forceinline__ int moe_route_count(const int64_t *__restrict__ topk_ids, int s0, int s1, int e, int n_experts,
+                                               int lane) {
+    int n = 0;
+    constexpr int U = 8;
+    for (int base = s0; base < s1; base += 64 * U) {
+        int64_t id[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) id[u] = base + 64 * u + lane < s1 ? topk_ids[base + 64 * u + lane] : -1;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            n += __builtin_popcountll(__ballot(e == n_experts ? (id[u] >= 0 && id[u] < n_experts) : id[u] == e));
+    }
+    return n;
+}
+
+__global__ void __launch_bounds__(256)
+moe_route_count_kernel(const int64_t *__restrict__ topk_ids, int n_slots, int n_experts, int seg_slots,
+                       int *__restrict__ cnt) {
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, seg = blockIdx.y;
+    if (e > n_experts) return;                                   // uniform over the wave
+    const int s0 = seg * seg_slots, s1 = min(s0 + seg_slots, n_slots);
+    const int n = moe_route_count(topk_ids, s0, s1, e, n_experts, lane);
+    if (lane == 0) cnt[seg * (n_experts + 1) + e] = n;
+}
+
+__global__ void __launch_bounds__(256)
+moe_route_place_kernel(const int64_t *__restrict__ topk_ids, int n_slots, int n_experts, int seg_slots, int n_seg,
+                       const int *__restrict__ cnt, int *__restrict__ perm, int *__restrict__ pexp,
+                       int *__restrict__ offs) {
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, seg = blockIdx.y;
+    if (e > n_experts) return;                                   // uniform over the wave
+    // slots of the experts below e in every segment, and of e itself in the segments before this one
+    int below = 0;
+    const int stride = n_experts + 1;
+    for (int idx = lane; idx < n_seg * stride; idx += 64) {
+        const int sg = idx / stride, ex = idx - sg * stride;
+        if (ex < n_experts && (ex < e || (ex == e && sg < seg))) below += cnt[idx];
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) below += __shfl_xor(below, d, 64);
+    if (seg == 0 && lane == 0) offs[e] = below;                  // e = n_experts: the total
+    if (e == n_experts) return;
+    const int s0 = seg * seg_slots, s1 = min(s0 + seg_slots, n_slots);
+    int mine = 0;
+    constexpr int U = 8;
+    for (int base = s0; base < s1; base += 64 * U) {
+        int64_t id[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) id[u] = base + 64 * u + lane < s1 ? topk_ids[base + 64 * u + lane] : -1;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned long long hit = __ballot(id[u] == e);
+            if (id[u] == e) {
+                const int at = below + mine + __builtin_popcountll(hit & ((1ull << lane) - 1ull));
+                perm[at] = base + 64 * u + lane;
+                pexp[at] = e;
+            }
             mine += __builtin_popcountll(hit);
         }
     }
@@ -1004,7 +1315,7 @@ int moe_check_blocks(const int64_t *blocks_m, int64_t n_blocks_m, int64_t m_pad,
 }
 }  // namespace
 
-int glqh_launch_moe_output_rht(const float *part, int ks, int n_slots, int n_experts, const int64_t *topk_ids,
+int glqh_launch_moe_output_rht(const float *part, int ks, int part_f16, int n_slots, int n_experts, const int64_t *topk_ids,
                                const void *su_base, const float *wscale_dev, int64_t out_features, int64_t m_pad,
                                const int64_t *blocks_m, int64_t n_blocks_m, void *h_f16, int64_t h_stride,
                                hipStream_t stream) {
@@ -1014,11 +1325,15 @@ int glqh_launch_moe_output_rht(const float *part, int ks, int n_slots, int n_exp
     if (moe_check_blocks(blocks_m, n_blocks_m, m_pad, &margs, &max_bs)) return 1;
     GLQH_REQUIRE(aligned16(part) && aligned16(su_base) && aligned16(h_f16) && (h_stride & 7) == 0,
                  "routed experts: unaligned rows");
-    const moe_out_args a = {part, ks, n_slots, n_experts, topk_ids, (const f16 *)su_base, wscale_dev,
+    const moe_out_args a = {part, ks, part_f16, n_slots, n_experts, topk_ids, (const f16 *)su_base, wscale_dev,
                             (int)out_features, (int)m_pad};
     const int nb = __builtin_popcountll((unsigned long long)m_pad);
-    hipLaunchKernelGGL(moe_output_rht_kernel, dim3((unsigned)nb, (unsigned)n_slots), dim3(REG_THREADS),
-                       rht_reg_lds_bytes(ilog2(max_bs)), stream, a, (f16 *)h_f16, h_stride, margs);
+    if (n_slots >= MOE_OUT_WIDE_MIN)
+        hipLaunchKernelGGL(moe_output_rht_wide_kernel, dim3((unsigned)(64 * ((n_slots + 63) / 64) * nb)), dim3(REG_THREADS),
+                           rht_reg_lds_bytes(ilog2(max_bs)), stream, a, (f16 *)h_f16, h_stride, nb, margs);
+    else
+        hipLaunchKernelGGL(moe_output_rht_kernel, dim3((unsigned)nb, (unsigned)n_slots), dim3(REG_THREADS),
+                           rht_reg_lds_bytes(ilog2(max_bs)), stream, a, (f16 *)h_f16, h_stride, margs);
     GLQH_LAUNCH_CHECK("routed-expert output_rht launch");
     return 0;
 }
@@ -1027,16 +1342,136 @@ int glqh_launch_moe_gated_act(const void *h_f16, int64_t h_stride, void *out_f16
                               int act, hipStream_t stream) {
     GLQH_REQUIRE(act >= 0 && act <= 2, "routed experts: gated activations 0 (silu), 1 (gelu-tanh), 2 (relu2), got %d", act);
     const int64_t total = (int64_t)n_slots * intermediate;
-    hipLaunchKernelGGL(moe_gated_act_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                       (const f16 *)h_f16, h_stride, (f16 *)out_f16, n_slots, (int)intermediate, act);
+    // (eight elements per thread only where there are many: a few slots finish sooner spread over more threads)
+    if (n_slots >= 1024 && intermediate % 8 == 0 && h_stride % 8 == 0 && aligned16(h_f16) && aligned16(out_f16))
+        hipLaunchKernelGGL(moe_gated_act_kernel<8>, dim3((unsigned)((total / 8 + 255) / 256)), dim3(256), 0, stream,
+                           (const f16 *)h_f16, h_stride, (f16 *)out_f16, n_slots, (int)intermediate, act);
+    else
+        hipLaunchKernelGGL(moe_gated_act_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                           (const f16 *)h_f16, h_stride, (f16 *)out_f16, n_slots, (int)intermediate, act);
     GLQH_LAUNCH_CHECK("routed-expert activation launch");
     return 0;
 }
 
-int glqh_launch_moe_route(const int64_t *topk_ids, int n_slots, int n_experts, int *perm, int *offs,
-                          hipStream_t stream) {
-    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((n_experts + 1 + 3) / 4)), dim3(256), 0, stream, topk_ids,
-                       n_slots, n_experts, perm, offs);
+// 1 when the launch below serves these shapes: canonical blocks of at most 8192 points on both sides, the
+// second projection's a multiple of 32 columns
+int glqh_moe_mid_eligible(int64_t m_pad13, const int64_t *blocks_m13, int64_t n_blocks_m13, int64_t n_pad2,
+                          const int64_t *blocks_n2, int64_t n_blocks_n2) {
+    glqh_meta_args m13, m2;
+    if (!glqh_fill_meta_args(&m13, n_blocks_m13 > 1 ? blocks_m13 : nullptr, n_blocks_m13 > 1 ? n_blocks_m13 : 1, m_pad13) ||
+        m13.canon != m_pad13)
+        return 0;
+    if (!glqh_fill_meta_args(&m2, n_blocks_n2 > 1 ? blocks_n2 : nullptr, n_blocks_n2 > 1 ? n_blocks_n2 : 1, n_pad2) ||
+        m2.canon != n_pad2)
+        return 0;
+    const int64_t b13 = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)m_pad13));
+    const int64_t b2 = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)n_pad2));
+    return b13 <= (1 << WIDE_LOG_MAX) && b2 <= (1 << WIDE_LOG_MAX) && (m_pad13 & 7) == 0 && (n_pad2 & 31) == 0;
+}
+
+// sums of the first projection -> transformed activations of the second (layout 0: rows by slot; 2: the tile
+// kernel's blocked operand by sorted position, Mp positions), for the slots listed in perm[0 .. *n_valid)
+int glqh_launch_moe_mid(const float *part, int ks, int part_f16, int n_slots, int n_experts, const int64_t *topk_ids,
+                        const void *su_base, const float *wscale_dev, int64_t out_features13, int64_t m_pad13,
+                        const int64_t *blocks_m13, int64_t n_blocks_m13, const int *perm, const int *pexp, const int *n_valid,
+                        int64_t intermediate, int act, const void *sv2, int64_t n_pad2, const int64_t *blocks_n2,
+                        int64_t n_blocks_n2, void *out_f16, int layout, int64_t Mp, hipStream_t stream) {
+    glqh_range range("output_rht");
+    GLQH_REQUIRE(glqh_moe_mid_eligible(m_pad13, blocks_m13, n_blocks_m13, n_pad2, blocks_n2, n_blocks_n2),
+                 "routed experts: block sizes not served by the fused middle launch");
+    GLQH_REQUIRE(act >= 0 && act <= 2, "routed experts: gated activations 0 (silu), 1 (gelu-tanh), 2 (relu2), got %d", act);
+    GLQH_REQUIRE(aligned16(part) && aligned16(su_base) && aligned16(sv2) && aligned16(out_f16), "routed experts: unaligned rows");
+    glqh_meta_args m13, m2;
+    glqh_fill_meta_args(&m13, n_blocks_m13 > 1 ? blocks_m13 : nullptr, n_blocks_m13 > 1 ? n_blocks_m13 : 1, m_pad13);
+    glqh_fill_meta_args(&m2, n_blocks_n2 > 1 ? blocks_n2 : nullptr, n_blocks_n2 > 1 ? n_blocks_n2 : 1, n_pad2);
+    const int64_t b13 = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)m_pad13));
+    const int64_t b2 = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)n_pad2));
+    const int64_t max_bs = b13 > b2 ? b13 : b2;
+    int threads = 64;
+    while (threads < REG_THREADS && 8 * threads < max_bs) threads <<= 1;
+    const size_t s_bytes = (rht_reg_lds_bytes(ilog2(max_bs)) + 15) & ~(size_t)15;
+    const size_t lds = s_bytes + (size_t)(m_pad13 + n_pad2) * sizeof(f16);
+    moe_mid_args a = {};
+    a.o = {part, ks, part_f16, n_slots, n_experts, topk_ids, (const f16 *)su_base, wscale_dev, (int)out_features13,
+           (int)m_pad13};
+    a.sv2 = (const f16 *)sv2;
+    a.perm = perm;
+    a.pexp = pexp;
+    a.n_valid = n_valid;
+    a.intermediate = (int)intermediate;
+    a.act = act;
+    a.n_pad2 = (int)n_pad2;
+    a.Mp = (int)Mp;
+    a.nb13 = __builtin_popcountll((unsigned long long)m_pad13);
+    a.nb2 = __builtin_popcountll((unsigned long long)n_pad2);
+    a.s_floats = (int)(s_bytes / sizeof(float));
+    const dim3 grid((unsigned)(64 * ((n_slots + 63) / 64)));
+    if (layout == 2)
+        hipLaunchKernelGGL(moe_mid_kernel<2>, grid, dim3((unsigned)threads), lds, stream, a, (f16 *)out_f16, m13, m2);
+    else
+        hipLaunchKernelGGL(moe_mid_kernel<0>, grid, dim3((unsigned)threads), lds, stream, a, (f16 *)out_f16, m13, m2);
+    GLQH_LAUNCH_CHECK("routed-expert middle launch");
+    return 0;
+}
+
+// out[token] = sum over the token's choices of w * (second projection's output row of the slot), many tokens
+int glqh_launch_moe_final(const float *part, int ks, int part_f16, int num_tokens, int top_k, int n_experts,
+                          const int64_t *topk_ids, const float *topk_w, const void *su_base, const float *wscale_dev,
+                          int64_t out_features, int64_t m_pad, const int64_t *blocks_m, int64_t n_blocks_m, void *out,
+                          int out_dtype, int64_t out_stride, hipStream_t stream) {
+    glqh_range range("output_rht");
+    glqh_meta_args margs;
+    int64_t max_bs;
+    if (moe_check_blocks(blocks_m, n_blocks_m, m_pad, &margs, &max_bs)) return 1;
+    GLQH_REQUIRE(out_dtype == GLQH_F16 || out_dtype == GLQH_BF16, "routed experts: output must be f16 or bf16");
+    GLQH_REQUIRE(aligned16(part) && aligned16(su_base) && aligned16(out) && (out_stride & 7) == 0,
+                 "routed experts: unaligned rows");
+    const moe_out_args a = {part, ks, part_f16, num_tokens * top_k, n_experts, topk_ids, (const f16 *)su_base, wscale_dev,
+                            (int)out_features, (int)m_pad};
+    const int nb = __builtin_popcountll((unsigned long long)m_pad);
+    const dim3 grid((unsigned)(64 * ((num_tokens + 63) / 64) * nb));
+    const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
+    // rows without small blocks (which take several tokens per workgroup of 512 threads): as many threads as the
+    // largest block has groups of eight elements
+    int threads = REG_THREADS;
+    if ((m_pad & 1023) == 0 && max_bs <= 2048) threads = (int)(max_bs / 8);
+#define GLQH_MOE_FINAL(YT, BIG)                                                                                  \
+    hipLaunchKernelGGL((moe_final_kernel<YT, BIG>), grid, dim3((unsigned)threads), lds, stream, a, topk_w, top_k, num_tokens, \
+                       (YT *)out, out_stride, nb, margs)
+    const bool big = max_bs > 4096;
+    if (out_dtype == GLQH_F16) { if (big) GLQH_MOE_FINAL(f16, true); else GLQH_MOE_FINAL(f16, false); }
+    else { if (big) GLQH_MOE_FINAL(uint16_t, true); else GLQH_MOE_FINAL(uint16_t, false); }
+#undef GLQH_MOE_FINAL
+    GLQH_LAUNCH_CHECK("routed-expert final launch");
+    return 0;
+}
+
+// segments of the two-launch form (1: the single launch), and the ints of scratch it needs
+int glqh_moe_route_segments(int n_slots, int n_experts) {
+    if (n_slots < 2 * MOE_ROUTE_SEG_SLOTS || n_experts > 4096) return 1;
+    const int n = (n_slots + MOE_ROUTE_SEG_SLOTS - 1) / MOE_ROUTE_SEG_SLOTS;
+    return n < MOE_ROUTE_MAX_SEG ? n : MOE_ROUTE_MAX_SEG;
+}
+
+size_t glqh_moe_route_scratch_ints(int n_slots, int n_experts) {
+    const int n = glqh_moe_route_segments(n_slots, n_experts);
+    return n > 1 ? (size_t)n * (n_experts + 1) : 0;
+}
+
+// perm / pexp: slot and expert of every position of the expert-sorted order, offs: first position per expert
+int glqh_launch_moe_route(const int64_t *topk_ids, int n_slots, int n_experts, int *perm, int *pexp, int *offs,
+                          int *scratch, hipStream_t stream) {
+    const int n_seg = glqh_moe_route_segments(n_slots, n_experts);
+    const unsigned wgs = (unsigned)((n_experts + 1 + 3) / 4);
+    if (n_seg == 1) {
+        hipLaunchKernelGGL(moe_route_kernel, dim3(wgs), dim3(256), 0, stream, topk_ids, n_slots, n_experts, perm, pexp, offs);
+    } else {
+        const int seg_slots = ((n_slots + n_seg - 1) / n_seg + 63) & ~63;
+        hipLaunchKernelGGL(moe_route_count_kernel, dim3(wgs, (unsigned)n_seg), dim3(256), 0, stream, topk_ids, n_slots,
+                           n_experts, seg_slots, scratch);
+        hipLaunchKernelGGL(moe_route_place_kernel, dim3(wgs, (unsigned)n_seg), dim3(256), 0, stream, topk_ids, n_slots,
+                           n_experts, seg_slots, n_seg, scratch, perm, pexp, offs);
+    }
     GLQH_LAUNCH_CHECK("routed-expert routing launch");
     return 0;
 }

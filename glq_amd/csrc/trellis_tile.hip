@@ -68,6 +68,24 @@ struct tt_group {
     int n;
 };
 
+// Routed experts of a mixture-of-experts layer with many rows per expert (glq/csrc/glq_trellis.cu:1475-1540 is the
+// reference's grouped kernel; its caller loops over whole per-expert linears beyond 256 tokens,
+// glq_vllm/fused_moe_method.py:702): the (token, choice) slots sorted by expert are the "tokens" of the tile
+// kernel, the activations are packed in that order, and a token tile is a run of up to 128 NTW positions of ONE
+// expert, listed by a small launch from the routing's offsets -- an expert with 300 rows gets two tiles of 160 and
+// 140 positions, not one full and one almost empty.  Waves whose 16 NTW positions lie past the end of the run
+// only decode.  Sums leave for row perm[position] of the output, times the expert's factor (a second stage's
+// scale) if there is one.
+struct tt_moe {
+    int64_t stride_bytes;                          // expert e's stream at packed + e * stride_bytes
+    const int *perm;                               // position in the expert-sorted order -> slot
+    const int4 *tiles;                             // (expert, first position, positions, -)
+    const int *n_tiles;
+    const float *pscale_dev;
+};
+
+enum { TT_PLAIN = 0, TT_GROUP = 1, TT_MOE = 2 };
+
 __device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global prefetches stay in flight
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -111,8 +129,9 @@ __device__ __forceinline__ void tt_emit(const tr_record<R> &r, int unit, int kpi
     }
 }
 
-template <int R, int NTW, bool GROUP>
-__device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g) {
+template <int R, int NTW, int MODE>
+__device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g, const tt_moe &mo) {
+    constexpr bool GROUP = MODE == TT_GROUP, MOE = MODE == TT_MOE;
     extern __shared__ u32x4 abuf[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
@@ -125,7 +144,8 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
     const int l1 = (l + 1) & 31, l2 = (l + 2) & 31;
     const int next1 = 16 * (l1 & 3) + 8 * hm + (l1 >> 2), next2 = 16 * (l2 & 3) + 8 * hm + (l2 >> 2);
 
-    const int nitems = a.TT * a.KS * a.RT;
+    int nitems = a.TT * a.KS * a.RT;
+    if constexpr (MOE) nitems = *mo.n_tiles * a.RT;             // one K slot
     const int per_xcd = (nitems + 7) >> 3;
     const int xcd = blockIdx.x & 7, bx = blockIdx.x >> 3;
     const int nbx = ((int)gridDim.x - xcd + 7) >> 3;
@@ -147,7 +167,19 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             rt -= first;
         }
         const int mpairs = lm >> 5;
-        const int r0 = rt * TT_ROWS, tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW;
+        int tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW, limit = a.M;
+        float osc = 1.0f;
+        bool active = true;                                     // uniform over the wave
+        if constexpr (MOE) {
+            const int4 tile = mo.tiles[item / a.RT];
+            if (tile.z <= 0) continue;                          // uniform over the workgroup
+            lpacked = a.packed + tile.x * mo.stride_bytes;
+            tok0 = tile.y + wave * 16 * NTW;
+            limit = tile.y + tile.z;
+            if (mo.pscale_dev) osc = mo.pscale_dev[tile.x];
+            active = __builtin_amdgcn_readfirstlane((int)(tok0 < limit)) != 0;
+        }
+        const int r0 = rt * TT_ROWS;
         const int ds0 = slot * a.slot_ds, ds1 = min(ds0 + a.slot_ds, nds);
 
         const int mp = min(2 * (2 * rt + unit) + hm, mpairs - 1);
@@ -194,6 +226,10 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             const u32x4 *rd = abuf + par * TT_BUF;
             u32x4 *wr = abuf + (par ^ 1) * TT_BUF;
             const tr_record<R> r3 = load_rec(d + 3);
+            if (MOE && !active) {                               // no positions of the run left for this wave
+                emit(r1, wr, 0);
+                emit(r1, wr, 1);
+            } else {
             f16x8 ring[2];
             ring[0] = __builtin_bit_cast(f16x8, rd[lane]);
             ring[1] = __builtin_bit_cast(f16x8, rd[GLQH_WAVE + lane]);
@@ -214,6 +250,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
                 if (kk == 1) emit(r1, wr, 0);
                 if (kk == TT_FRAGS + 1) emit(r1, wr, 1);
             }
+            }
             tt_barrier();                                       // rd has been read, wr is written
             r1 = r2;
             r2 = r3;
@@ -230,6 +267,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         float *ep = (float *)abuf + wave * (16 * TT_EP_STRIDE);
 #pragma unroll
         for (int tt = 0; tt < NTW; ++tt) {
+            if (MOE && !active) break;
 #pragma unroll
             for (int f = 0; f < TT_FRAGS; ++f)
                 *(f32x4 *)(ep + i * TT_EP_STRIDE + 64 * (f >> 2) + 8 * (f & 3) + rlane) = acc[f][tt];
@@ -238,10 +276,13 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
                 const int rl = 8 * (lane & 15), row = r0 + rl;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int tl = 4 * j + (lane >> 4), tok = tok0 + 16 * tt + tl;
-                    const f32x4 v0 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
-                    const f32x4 v1 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl + 4);
-                    if (tok >= a.M || row >= lm) continue;      // m is a multiple of 32: whole runs of eight
+                    const int tl = 4 * j + (lane >> 4);
+                    int tok = tok0 + 16 * tt + tl;
+                    f32x4 v0 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
+                    f32x4 v1 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl + 4);
+                    if constexpr (MOE) { v0 *= osc; v1 *= osc; }
+                    if (tok >= limit || row >= lm) continue;    // m is a multiple of 32: whole runs of eight
+                    if constexpr (MOE) tok = mo.perm[tok];
                     typedef _Float16 f16x8o __attribute__((ext_vector_type(8)));
                     const int64_t e = ((int64_t)slot * a.M + tok) * lm + row;
                     *(f16x8o *)((f16 *)lout + e) = f16x8o{(f16)v0[0], (f16)v0[1], (f16)v0[2], (f16)v0[3],
@@ -251,9 +292,12 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
                 const int rl = 4 * (lane & 31), row = r0 + rl;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const int tl = 2 * j + (lane >> 5), tok = tok0 + 16 * tt + tl;
-                    const f32x4 v = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
-                    if (tok >= a.M || row >= lm) continue;
+                    const int tl = 2 * j + (lane >> 5);
+                    int tok = tok0 + 16 * tt + tl;
+                    f32x4 v = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
+                    if constexpr (MOE) v *= osc;
+                    if (tok >= limit || row >= lm) continue;
+                    if constexpr (MOE) tok = mo.perm[tok];
                     if (!a.direct) {
                         *(f32x4 *)(lout + ((int64_t)slot * a.M + tok) * lm + row) = v;
                     } else {
@@ -277,13 +321,43 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
 template <int R, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_kernel(const tt_args a) {
-    tr_tile_body<R, NTW, false>(a, tt_group{});
+    tr_tile_body<R, NTW, TT_PLAIN>(a, tt_group{}, tt_moe{});
 }
 
 template <int R, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_group_kernel(const tt_args a, const tt_group g) {
-    tr_tile_body<R, NTW, true>(a, g);
+    tr_tile_body<R, NTW, TT_GROUP>(a, g, tt_moe{});
+}
+
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_moe_kernel(const tt_args a, const tt_moe mo) {
+    tr_tile_body<R, NTW, TT_MOE>(a, tt_group{}, mo);
+}
+
+// Token tiles of the routed experts: expert e's positions [offs[e], offs[e + 1]) of the sorted order in
+// ceil(count / tile_tok) runs of equal length (a multiple of 32, the last one shorter).  One workgroup; thread t
+// takes experts t * per .. (t + 1) * per - 1.
+__global__ void __launch_bounds__(256)
+tr_moe_tiles_kernel(const int *__restrict__ offs, int n_experts, int tile_tok, int4 *__restrict__ tiles,
+                    int *__restrict__ n_tiles) {
+    __shared__ int sums[256];
+    const int t = threadIdx.x, per = (n_experts + 255) / 256;
+    const int e0 = min(t * per, n_experts), e1 = min(e0 + per, n_experts);
+    int mine = 0;
+    for (int e = e0; e < e1; ++e) mine += (offs[e + 1] - offs[e] + tile_tok - 1) / tile_tok;
+    sums[t] = mine;
+    __syncthreads();
+    int at = 0;
+    for (int j = 0; j < t; ++j) at += sums[j];
+    if (t == 255) *n_tiles = at + mine;
+    for (int e = e0; e < e1; ++e) {
+        const int o0 = offs[e], cnt = offs[e + 1] - o0, nt = (cnt + tile_tok - 1) / tile_tok;
+        if (nt == 0) continue;
+        const int len = ((cnt + nt - 1) / nt + 31) & ~31;
+        for (int j = 0; j < nt; ++j) tiles[at++] = int4{e, o0 + j * len, max(0, min(len, cnt - j * len)), 0};
+    }
 }
 
 // Up to 64 tokens: one barrier per group of four steps instead of one per step, and the eight waves split a
@@ -433,14 +507,24 @@ tr_tile_small_kernel(const tt_args a) {
 // (M, k) row-major fp16 -> xb[k-pair][token][q][8]: slot q of a k-pair takes columns
 // 2q + {0,1,8,9,16,17,24,25}, i.e. dword q of each of its four 16-byte items.  64 tokens x 4
 // k-pairs per workgroup through LDS; reads in runs of 256 bytes, writes in runs of 4 KB.
+// GATHER: token t of xb is row perm[t] / x_div of x, for the *n_valid first t (the expert-sorted order of the
+// routed experts' slots).
+template <bool GATHER>
 __global__ void __launch_bounds__(256)
-tr_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, int Mp, int k) {
+tr_pack_blocked_kernel(const f16 *__restrict__ x, f16 *__restrict__ xb, int M, int Mp, int k,
+                       const int *__restrict__ perm, const int *__restrict__ n_valid, int x_div) {
     __shared__ u32x4 tile[16][65];                              // [k-pair * 4 + q][token]
     const int tok0 = blockIdx.x * 64, kp0 = blockIdx.y * 4, nkp = k >> 5;
     const int t = threadIdx.x;
+    if constexpr (GATHER) {
+        M = *n_valid;
+        if (tok0 >= M) return;                                  // uniform
+    }
     {
         const int kpi = t & 3, tl = t >> 2;
-        const int tok = min(tok0 + tl, M - 1), kp = min(kp0 + kpi, nkp - 1);
+        int tok = min(tok0 + tl, M - 1);
+        if constexpr (GATHER) tok = perm[tok] / x_div;
+        const int kp = min(kp0 + kpi, nkp - 1);
         const u32x4 *src = (const u32x4 *)(x + (int64_t)tok * k + 32 * kp);
         const u32x4 v0 = src[0], v1 = src[1], v2 = src[2], v3 = src[3];
 #pragma unroll
@@ -574,7 +658,8 @@ int tt_init_R() {
     return tt_set_lds(tr_tile_small_kernel<R, 2, 1>) || tt_set_lds(tr_tile_small_kernel<R, 4, 1>) ||
            tt_set_lds(tr_tile_kernel<R, 1>) || tt_set_lds(tr_tile_kernel<R, 2>) || tt_set_lds(tr_tile_kernel<R, 4>) ||
            tt_set_lds(tr_tile_group_kernel<R, 1>) || tt_set_lds(tr_tile_group_kernel<R, 2>) ||
-           tt_set_lds(tr_tile_group_kernel<R, 4>);
+           tt_set_lds(tr_tile_group_kernel<R, 4>) || tt_set_lds(tr_tile_moe_kernel<R, 1>) ||
+           tt_set_lds(tr_tile_moe_kernel<R, 2>) || tt_set_lds(tr_tile_moe_kernel<R, 4>);
 }
 
 }  // namespace
@@ -606,8 +691,9 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     if (out_f16 && (direct || M <= 64)) return glqh_fail("trellis tile kernel: fp16 sums are partial sums of the large tiles");
     const int Mp = (int)tt_padded_tokens(M);
     if (x_f16) {                                               // NULL: xb_scratch already holds the blocked layout
-        hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)),
-                           dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, Mp, (int)k);
+        hipLaunchKernelGGL(tr_pack_blocked_kernel<false>, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)),
+                           dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb_scratch, (int)M, Mp, (int)k,
+                           (const int *)nullptr, (const int *)nullptr, 1);
         GLQH_LAUNCH_CHECK("trellis pack launch");
     }
     tt_args a;
@@ -747,9 +833,97 @@ int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void
 // x (M, k) fp16 row-major -> the blocked layout of the tile kernels (glqh_trellis_tile_xb_bytes)
 int glqh_launch_trellis_pack(const void *x_f16, void *xb, int64_t M, int64_t k, hipStream_t stream) {
     const int Mp = (int)tt_padded_tokens(M);
-    hipLaunchKernelGGL(tr_pack_blocked_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)), dim3(256), 0,
-                       stream, (const f16 *)x_f16, (f16 *)xb, (int)M, Mp, (int)k);
+    hipLaunchKernelGGL(tr_pack_blocked_kernel<false>, dim3((unsigned)((M + 63) / 64), (unsigned)((k / 32 + 3) / 4)), dim3(256), 0,
+                       stream, (const f16 *)x_f16, (f16 *)xb, (int)M, Mp, (int)k, (const int *)nullptr,
+                       (const int *)nullptr, 1);
     GLQH_LAUNCH_CHECK("trellis pack launch");
     return 0;
 }
 
+
+// ---- routed experts with many rows per expert -----------------------------------------------------
+// Positions per token tile of the routed-expert form for n_slots slots over n_experts experts, by the average
+// number of rows per expert: 128 below 96, 256 below 224, 512 above (whole call, 128 experts of 2048 -> 2 x 768 ->
+// 2048 with 8 choices, us with 128 / 256 / 512: 64 rows 393 / 403 / 473, 128 rows 660 / 587 / 614, 256 rows 1187 /
+// 1034 / 997).  GLQ_MOE_TILE_NTW (1, 2, 4; read once) forces 128 / 256 / 512.
+int glqh_trellis_tile_moe_tokens(int64_t n_slots, int64_t n_experts) {
+    static const int forced = [] { const char *e = getenv("GLQ_MOE_TILE_NTW"); return e ? atoi(e) : 0; }();
+    if (forced == 1 || forced == 2 || forced == 4) return 128 * forced;
+    const int64_t live = n_experts < n_slots ? n_experts : n_slots;
+    const int64_t avg = n_slots / (live > 0 ? live : 1);
+    return avg >= 224 ? 512 : avg >= 96 ? 256 : 128;
+}
+
+// positions of the packed activations: the slots plus one tile that a run's last tile may read into
+int64_t glqh_trellis_tile_moe_padded(int64_t n_slots, int64_t n_experts) {
+    return (n_slots + glqh_trellis_tile_moe_tokens(n_slots, n_experts) + 63) / 64 * 64;
+}
+
+// upper bound on the token tiles: every expert with rows ends in at most one partial tile
+int64_t glqh_trellis_tile_moe_max_tiles(int64_t n_slots, int64_t n_experts) {
+    const int64_t live = n_experts < n_slots ? n_experts : n_slots;
+    return n_slots / glqh_trellis_tile_moe_tokens(n_slots, n_experts) + live + 1;
+}
+
+// tiles (glqh_trellis_tile_moe_max_tiles int4) and *n_tiles from the routing's offsets
+int glqh_launch_trellis_tile_moe_table(const int *offs, int n_slots, int n_experts, void *tiles, int *n_tiles,
+                                       hipStream_t stream) {
+    hipLaunchKernelGGL(tr_moe_tiles_kernel, dim3(1), dim3(256), 0, stream, offs, n_experts,
+                       glqh_trellis_tile_moe_tokens(n_slots, n_experts), (int4 *)tiles, n_tiles);
+    GLQH_LAUNCH_CHECK("routed-expert tile table launch");
+    return 0;
+}
+
+// xb[k-pair][position][q][8] from the transformed rows x (row of slot s = s / x_div), positions in the sorted order
+int glqh_launch_trellis_pack_moe(const void *x_f16, void *xb, const int *perm, const int *offs, int n_slots,
+                                 int n_experts, int x_div, int64_t k, hipStream_t stream) {
+    const int Mp = (int)glqh_trellis_tile_moe_padded(n_slots, n_experts);
+    hipLaunchKernelGGL(tr_pack_blocked_kernel<true>, dim3((unsigned)((n_slots + 63) / 64), (unsigned)((k / 32 + 3) / 4)),
+                       dim3(256), 0, stream, (const f16 *)x_f16, (f16 *)xb, n_slots, Mp, (int)k, perm, offs + n_experts,
+                       x_div);
+    GLQH_LAUNCH_CHECK("routed-expert pack launch");
+    return 0;
+}
+
+// out[slot][row] (fp16 with out_f16) = pscale[expert] * sum over k, for every slot with a valid expert
+int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t stride_bytes, int R, const int *perm,
+                                 const void *tiles, const int *n_tiles, const float *pscale_dev, int n_slots,
+                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream) {
+    const int tile_tok = glqh_trellis_tile_moe_tokens(n_slots, n_experts);
+    tt_args a = {};
+    a.packed = (const uint8_t *)packed;
+    a.xb = (const f16 *)xb;
+    a.M = n_slots;
+    a.Mp = (int)glqh_trellis_tile_moe_padded(n_slots, n_experts);
+    a.m = (int)m;
+    a.k = (int)k;
+    a.RT = (int)((m + TT_ROWS - 1) / TT_ROWS);
+    a.TT = 0;
+    a.KS = 1;
+    a.slot_ds = (int)(k / 64);
+    a.out = (float *)out;
+    a.out_f16 = out_f16;
+    const tt_moe mo = {stride_bytes, perm, (const int4 *)tiles, n_tiles, pscale_dev};
+    const int64_t max_items = glqh_trellis_tile_moe_max_tiles(n_slots, n_experts) * a.RT;
+    const int cus = glqh_device_cus();
+    const dim3 grid((unsigned)(max_items < cus ? max_items : cus));
+#define GLQH_TTM(RR)                                                                                          \
+    do {                                                                                                      \
+        if (tile_tok == 128)                                                                                  \
+            hipLaunchKernelGGL((tr_tile_moe_kernel<RR, 1>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);    \
+        else if (tile_tok == 256)                                                                             \
+            hipLaunchKernelGGL((tr_tile_moe_kernel<RR, 2>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);    \
+        else                                                                                                  \
+            hipLaunchKernelGGL((tr_tile_moe_kernel<RR, 4>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);    \
+    } while (0)
+    switch (R) {
+    case 1: GLQH_TTM(1); break;
+    case 2: GLQH_TTM(2); break;
+    case 3: GLQH_TTM(3); break;
+    case 4: GLQH_TTM(4); break;
+    default: return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+    }
+#undef GLQH_TTM
+    GLQH_LAUNCH_CHECK("routed-expert tile launch");
+    return 0;
+}

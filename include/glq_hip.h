@@ -246,8 +246,13 @@ size_t glqh_fused_moe_trellis_workspace_bytes(int64_t num_tokens, int64_t top_k,
  * choice) slots every slot is one fused-input GEMV on its expert's stream; from
  * max(16, 3/4 num_experts) slots on a routing launch groups the slots by expert and every
  * expert's stream is read once per 16 of its rows (GLQ_MOE_GROUP_MIN sets that count), once
- * per up to 64 rows from an average of 12 rows per expert on (GLQ_MOE_WIDE_MIN_ROWS).
- * Intermediate results are rounded to
+ * per up to 64 rows from an average of 12 rows per expert on (GLQ_MOE_WIDE_MIN_ROWS); from an
+ * average of 24 rows per expert on (GLQ_MOE_TILE_MIN_ROWS, 0 = never) the expert-sorted slots go
+ * through the many-token tile kernel in runs of up to 128-512 rows of one expert, the decoded
+ * weights of a 128-row tile meeting the whole run on the matrix cores.  From 1024 slots on the
+ * launches between the two projections (output transform, activation, input transform) and after
+ * them (output transform, weighted sum) are one launch each (GLQ_MOE_FUSE=0: separate), with the
+ * same roundings and the same bits.  Intermediate results are rounded to
  * fp16 where the reference rounds them (after each output transform and after the
  * activation), the weighted sum runs over the choices in order in fp32.  activation_type:
  * 0 SiLU, 1 GELU (tanh form), 2 squared ReLU, each times the up half.  Expert ids outside

@@ -207,12 +207,18 @@ def test_refusals(ext):
 
 
 @pytest.mark.parametrize("hidden,inter,T,K,K2", [(256, 128, 16, 4, 0), (320, 192, 40, 2, 0), (320, 192, 33, 3, 2),
-                                                 (256, 128, 24, 4, 0), (256, 128, 90, 2, 0), (256, 128, 80, 3, 1)])
+                                                 (256, 128, 24, 4, 0), (256, 128, 90, 2, 0), (256, 128, 80, 3, 1),
+                                                 (256, 128, 200, 3, 0), (320, 192, 300, 2, 2), (256, 128, 530, 2, 0),
+                                                 (256, 128, 1100, 4, 0)])
 def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     """From max(16, 3/4 of the experts) slots on the rows are grouped by expert.  Skewed routing: every token's first choice is
     expert 2 (more than two tiles of 16 rows for it), expert 5 gets nothing, some ids are out of range.  From an
     average of 12 rows per expert on, a pass over an expert's stream takes up to 64 of its rows: the cases give
-    expert 2 one pass of 16 (T = 16), of 32 (24), of 64 (33, 40), 64 + 32 (90) and 64 + 16 (80) rows."""
+    expert 2 one pass of 16 (T = 16), of 32 (24), of 64 (33, 40), 64 + 32 (90) and 64 + 16 (80) rows.  From 48 rows
+    per expert on average the sorted slots go through the tile kernel in runs of up to 256 positions of one
+    expert: expert 2 has one run of 199 (T = 200), two of 160 and 139 (300), three of 192, 192 and 145 (530), the
+    other experts one partial run each.  T = 1100: 4400 slots, whose routing table is made by two launches over
+    three segments of the slots, and runs of up to 512 positions."""
     say("moe grouped", hidden, inter, T, K, K2)
     ex = experts(6, hidden, inter, 4, K2, seed=2)
     rng = np.random.default_rng(T)
@@ -230,20 +236,28 @@ def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     assert torch.equal(y, ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a))
 
 
-@pytest.mark.parametrize("group_min,wide_min", [("1", "1"), ("1", "1000000"), ("1000000", "12")])
-def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min):
+@pytest.mark.parametrize("group_min,wide_min,tile_min,tile_ntw,fuse", [
+    ("1", "1", "0", "", "1"), ("1", "1000000", "0", "", "0"), ("1000000", "12", "0", "", "1"), ("1", "12", "1", "", "1"),
+    ("1", "12", "1", "1", "0"), ("1", "12", "1", "4", "1"), ("1000000", "12", "0", "", "0")])
+def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min, tile_min, tile_ntw, fuse):
     """GLQ_MOE_GROUP_MIN (read once by the library) moves the slot count from which rows are grouped by
     expert: with 1 every case of this file runs in the grouped form, with 1000000 in the per-slot form,
     each against the oracle, in a process of its own.  GLQ_MOE_WIDE_MIN_ROWS moves the average number of rows
-    per expert from which the grouped form takes up to 64 rows per pass: 1 = always, 1000000 = never."""
+    per expert from which the grouped form takes up to 64 rows per pass: 1 = always, 1000000 = never.
+    GLQ_MOE_TILE_MIN_ROWS the average from which the tile kernel takes the grouped rows: 0 = never, 1 = always,
+    then with runs of up to 256 positions, or 128 / 512 with GLQ_MOE_TILE_NTW = 1 / 4.  GLQ_MOE_FUSE=0 keeps the
+    launches between and after the two decode launches separate (output transform, activation, input
+    transform; output transform, weighted sum) where one launch each is the default."""
     import os
     import subprocess
     import sys
-    say("moe forms, child process", group_min, wide_min)
+    say("moe forms, child process", group_min, wide_min, tile_min, tile_ntw, fuse)
     r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu",
                         "-k", "not fresh_process", "--timeout", "300", "--timeout-method", "thread",
                         "-p", "no:cacheprovider"],
-                       env={**os.environ, "GLQ_MOE_GROUP_MIN": group_min, "GLQ_MOE_WIDE_MIN_ROWS": wide_min}, capture_output=True, text=True, timeout=900,
+                       env={**os.environ, "GLQ_MOE_GROUP_MIN": group_min, "GLQ_MOE_WIDE_MIN_ROWS": wide_min,
+                            "GLQ_MOE_TILE_MIN_ROWS": tile_min, "GLQ_MOE_FUSE": fuse, **({"GLQ_MOE_TILE_NTW": tile_ntw} if tile_ntw else {})},
+                       capture_output=True, text=True, timeout=900,
                        cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
 

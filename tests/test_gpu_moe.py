@@ -236,6 +236,26 @@ def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     assert torch.equal(y, ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a))
 
 
+@pytest.mark.parametrize("hidden,inter", [(256, 4096), (8192, 128)])
+def test_rows_with_a_block_of_8192_points(ext, hidden, inter):
+    """The first projection's row (2 x 4096 = one block of 8192 points) or the second's (hidden 8192) takes sixteen
+    elements per thread in the launches between and after the projections; 600 tokens x 2 choices over 3 experts
+    (tile kernel, fused launches)."""
+    say("moe large blocks", hidden, inter)
+    ex = experts(3, hidden, inter, seed=5)
+    T, K = 600, 2
+    rng = np.random.default_rng(1)
+    ids = np.stack([rng.permutation(3)[:K] for _ in range(T)]).astype(np.int64)
+    ids[7, 1] = -1
+    w = rng.random((T, K)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((T, hidden)).astype(np.float32)).bfloat16()
+    a = ex.device_args(0)
+    y = ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a)
+    ref = ex.oracle(x.float().numpy(), ids, w, 0)
+    assert rel(y, ref) < TOL, rel(y, ref)
+    assert torch.equal(y, ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a))
+
+
 @pytest.mark.parametrize("group_min,wide_min,tile_min,tile_ntw,fuse", [
     ("1", "1", "0", "", "1"), ("1", "1000000", "0", "", "0"), ("1000000", "12", "0", "", "1"), ("1", "12", "1", "", "1"),
     ("1", "12", "1", "1", "0"), ("1", "12", "1", "4", "1"), ("1000000", "12", "0", "", "0")])
@@ -262,10 +282,12 @@ def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min, tile_m
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
 
 
-@pytest.mark.parametrize("T", [1, 4])
+@pytest.mark.parametrize("T", [1, 4, 40, 140])
 def test_qwen3_moe_expert_shapes(ext, T):
     """Expert shapes of a Qwen3-MoE layer (hidden 2048, intermediate 768, top-8), 16 of the experts,
-    4 bpw, bf16 activations: every chosen expert decoded whole by the oracle."""
+    4 bpw, bf16 activations: every chosen expert decoded whole by the oracle.  One and four tokens run slot by
+    slot, 40 tokens grouped by expert (20 rows each on average), 140 tokens through the tile kernel (70 rows
+    each, runs of up to 128 positions, 1120 slots: with the fused launches around the second projection)."""
     say("moe qwen3 shapes", T)
     ex = experts(16, 2048, 768, seed=3)
     ids, w = routing(T, 8, 16, T)

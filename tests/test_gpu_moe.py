@@ -147,13 +147,16 @@ def test_single_choice_equals_the_fused_linears(ext):
     assert rel(y, y2) < 2e-3, rel(y, y2)
 
 
-def test_registered_op_and_graph_replay(ext):
-    say("moe op + graph")
+@pytest.mark.parametrize("T", [4, 700])
+def test_registered_op_and_graph_replay(ext, T):
+    """T = 700: 1400 slots on 6 experts, the tile kernel's form, whose token tiles are listed on the device
+    from the routing of each replay."""
+    say("moe op + graph", T)
     from glq_amd import custom_ops
     custom_ops.register()
     ex = experts(6, 256, 128)
-    ids, w = routing(4, 2, 6, 11)
-    x = torch.from_numpy(np.random.default_rng(9).standard_normal((4, 256)).astype(np.float32)).half().to(DEV)
+    ids, w = routing(T, 2, 6, 11)
+    x = torch.from_numpy(np.random.default_rng(9).standard_normal((T, 256)).astype(np.float32)).half().to(DEV)
     a = ex.device_args(0)
     ids_d, w_d = t(ids), t(w)
     eager = ext.glq_fused_moe_trellis_3inst_cuda(x, ids_d, w_d, *a)
@@ -169,7 +172,10 @@ def test_registered_op_and_graph_replay(ext):
     with torch.cuda.graph(g):
         out = ext.glq_fused_moe_trellis_3inst_cuda(x, ids_d, w_d, *a)
     for rep in range(3):
-        ids2, w2 = routing(4, 2, 6, 20 + rep)
+        ids2, w2 = routing(T, 2, 6, 20 + rep)
+        if rep == 1:                                           # skewed: expert 2 is every token's first choice
+            ids2[:, 1] = np.where(ids2[:, 1] == 2, ids2[:, 0], ids2[:, 1])
+            ids2[:, 0] = 2
         ids_d.copy_(t(ids2)); w_d.copy_(t(w2))
         want = ext.glq_fused_moe_trellis_3inst_cuda(x, ids_d, w_d, *a)
         torch.cuda.synchronize()

@@ -35,6 +35,8 @@ static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages, bool
 }
 
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
+int glqh_launch_trellis_mma_rvq(const void *x_f16, int64_t B, const void *packed, const void *packed2, int R2, float rs2,
+                                int64_t m, int64_t k, int S, int ksplit, float *part, hipStream_t stream);
 int glqh_launch_trellis_mma_fusein_rvq(const void *packed, const void *packed2, int R2, float rs2, const void *x,
                                        int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
                                        int64_t in_features, int S, int ksplit, float *part,
@@ -582,8 +584,17 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         // its seven linears).  GLQ_TRELLIS_F16_SUMS=0 keeps them fp32.
         f16_sums = plan.tile && ks <= tr_f16_sums_max_slots() && B > 64 && !y_rht_out && y && tr_f16_sums_enabled() &&
                    glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad);
-        if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st, 1.0f, f16_sums)) return 1;
-        if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2, f16_sums)) return 1;
+        if (has_s2 && !plan.tile && R1 == 4 && tr_fuse_stages_enabled()) {
+            // up to 16 tokens of a 4 + R2 layer: both streams in one pass over the staged activations
+            glqh_range range("dequant_matmul");
+            if (glqh_launch_trellis_mma_rvq(x_in, B, packed, packed2, R2, (float)inv_resid_scale2, m_pad, n_pad, plan.S,
+                                            plan.ks, part1, st))
+                return 1;
+            two_parts = merge2 = false;
+        } else {
+            if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st, 1.0f, f16_sums)) return 1;
+            if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2, f16_sums)) return 1;
+        }
     }
 
     const float s1 = (float)wscale, s2 = (float)(wscale * inv_resid_scale2);

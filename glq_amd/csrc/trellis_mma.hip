@@ -200,12 +200,14 @@ __device__ __forceinline__ void mma_stage(uint32_t *xs, const f16 *__restrict__ 
 // grid = (ceil(m/64), ksplit, ceil(B / (16*NT))); slot s owns k-pairs [s*S, (s+1)*S); the
 // slot's activations are staged through LDS in chunks of CH k-pairs (CH % 4 == 0).
 // ---------------------------------------------------------------------------------
-template <int R, int TP, int NT>
-__global__ void __launch_bounds__(TR_THREADS)
-tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int B, int m, int k,
-              int S, int CH, float *__restrict__ part, int direct, float scale, int accum,
-              int64_t out_stride) {
-    extern __shared__ u32x4 xs_lds[];
+// R2 > 0: a residual stage of R2 bits/weight decoded in the same pass against the same staged activations, its
+// sums added times rs2 before the waves' sums are combined (one launch and one set of partial sums for a stacked
+// layer at 1..16 tokens).
+template <int R, int TP, int NT, int R2 = 0>
+__device__ __forceinline__ void
+tr_mma_body(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int B, int m, int k, int S, int CH,
+            float *__restrict__ part, int direct, float scale, int accum, int64_t out_stride, u32x4 *xs_lds,
+            const uint8_t *__restrict__ packed2 = nullptr, float rs2 = 0.0f) {
     constexpr int TPS = mma_tps<TP>();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -220,15 +222,21 @@ tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int
 
     constexpr int REC = 4 * R;
     const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;   // + kp * 32 * REC
+    constexpr int RB = R2 > 0 ? R2 : 1, REC2 = 4 * RB;
+    const uint8_t *lane_base2 = R2 > 0 ? packed2 + ((int64_t)mp * nkp * 32 + a.l) * REC2 : nullptr;
     int kp = kp0 + wave;
     tr_record<R> cur = {};
-    if (kp < kp1) cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
+    tr_record<RB> curb = {};
+    if (kp < kp1) {
+        cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
+        if constexpr (R2 > 0) curb = tr_load_record<RB>(lane_base2 + (int64_t)kp * 32 * REC2);
+    }
 
-    mma_acc<NT> acc;
+    mma_acc<NT> acc, accb;
 #pragma unroll
     for (int s = 0; s < 4; ++s)
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) acc.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < NT; ++tt) acc.v[s][tt] = accb.v[s][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // lanes past the token count read a zeroed block (one k-pair's worth, after the chunk)
     u32x4 *zero_blk = xs_lds + CH * (NT * 8 * TPS);
@@ -243,14 +251,44 @@ tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int
         fht_barrier<true>();
         for (; kp < c1; kp += TR_WAVES) {
             tr_record<R> nxt = cur;
-            if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
+            tr_record<RB> nxtb = curb;
+            if (kp + TR_WAVES < kp1) {
+                nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
+                if constexpr (R2 > 0) nxtb = tr_load_record<RB>(lane_base2 + (int64_t)(kp + TR_WAVES) * 32 * REC2);
+            }
             const u32x4 *xs = a.live ? xs_lds + ((kp - c0) * NT * 8 + a.q) * TPS + a.tokl : zero_blk;
             acc = mma_record<R, TP, NT>(cur, a.next1, a.next2, xs, acc);
+            if constexpr (R2 > 0) accb = mma_record<RB, TP, NT>(curb, a.next1, a.next2, xs, accb);
             cur = nxt;
+            curb = nxtb;
         }
+    }
+    if constexpr (R2 > 0) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) acc.v[s][tt] += rs2 * accb.v[s][tt];
     }
     mma_reduce_store<TP, NT>(acc, (float *)xs_lds, a, wave, B, m, tok0, 64 * blockIdx.x, slot, part,
                              direct, scale, accum, out_stride);
+}
+
+template <int R, int TP, int NT>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_kernel(const uint8_t *__restrict__ packed, const f16 *__restrict__ x, int B, int m, int k,
+              int S, int CH, float *__restrict__ part, int direct, float scale, int accum,
+              int64_t out_stride) {
+    extern __shared__ u32x4 xs_lds[];
+    tr_mma_body<R, TP, NT>(packed, x, B, m, k, S, CH, part, direct, scale, accum, out_stride, xs_lds);
+}
+
+// both stages of a stacked layer (first stage 4 bits/weight), 1..16 tokens
+template <int R2, int TP>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_rvq_kernel(const uint8_t *__restrict__ packed, const uint8_t *__restrict__ packed2, float rs2,
+                  const f16 *__restrict__ x, int B, int m, int k, int S, int CH, float *__restrict__ part) {
+    extern __shared__ u32x4 xs_lds[];
+    tr_mma_body<4, TP, 1, R2>(packed, x, B, m, k, S, CH, part, 0, 1.0f, 0, 0, xs_lds, packed2, rs2);
 }
 
 // ---------------------------------------------------------------------------------
@@ -690,6 +728,29 @@ int launch_mma(const void *x, int64_t B, const void *packed, int64_t m, int64_t 
     return 0;
 }
 
+template <int R2, int TP>
+int launch_mma_rvq(const void *x, int64_t B, const void *packed, const void *packed2, float rs2, int64_t m, int64_t k,
+                   int S, int ksplit, float *part, hipStream_t stream) {
+    const int per_kp = mma_slot_bytes(TP, 1);
+    int CH = mma_chunk_cap<TP, 1>();
+    if (CH > S) CH = (S + 3) & ~3;
+    size_t lds = (size_t)(CH + (TP < 16 ? 1 : 0)) * per_kp;
+    if (lds < (size_t)mma_red_bytes<TP, 1>()) lds = mma_red_bytes<TP, 1>();
+    dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, 1);
+    hipLaunchKernelGGL((tr_mma_rvq_kernel<R2, TP>), grid, dim3(TR_THREADS), lds, stream, (const uint8_t *)packed,
+                       (const uint8_t *)packed2, rs2, (const f16 *)x, (int)B, (int)m, (int)k, S, CH, part);
+    GLQH_LAUNCH_CHECK("trellis mma two-stage launch");
+    return 0;
+}
+
+template <int R2>
+int launch_mma_rvq_R(const void *x, int64_t B, const void *packed, const void *packed2, float rs2, int64_t m, int64_t k,
+                     int S, int ksplit, float *part, hipStream_t stream) {
+    if (B == 1) return launch_mma_rvq<R2, 1>(x, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+    if (B <= 4) return launch_mma_rvq<R2, 4>(x, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+    return launch_mma_rvq<R2, 16>(x, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+}
+
 template <int R>
 int launch_mma_R(const void *x, int64_t B, const void *packed, int64_t m, int64_t k, int S, int ksplit,
                  float *part, int direct, float scale, int accum, int64_t out_stride, hipStream_t stream) {
@@ -715,7 +776,8 @@ int mma_init_R() {
     return mma_set_lds(tr_mma_kernel<R, 1, 1>) || mma_set_lds(tr_mma_kernel<R, 4, 1>) ||
            mma_set_lds(tr_mma_kernel<R, 16, 1>) || mma_set_lds(tr_mma_kernel<R, 16, 2>) ||
            mma_set_lds(tr_mma_kernel<R, 16, 4>) || mma_set_lds(tr_mma_moe_grouped_kernel<R, false>) ||
-           mma_set_lds(tr_mma_moe_grouped_kernel<R, true>);
+           mma_set_lds(tr_mma_moe_grouped_kernel<R, true>) || mma_set_lds(tr_mma_rvq_kernel<R, 1>) ||
+           mma_set_lds(tr_mma_rvq_kernel<R, 4>) || mma_set_lds(tr_mma_rvq_kernel<R, 16>);
 }
 
 }  // namespace
@@ -746,6 +808,20 @@ int glqh_launch_trellis_mma(const void *x_f16, int64_t B, const void *packed, in
     case 4: return launch_mma_R<4>(x_f16, B, packed, m, k, S, ksplit, part, direct, scale, accum, out_stride, stream);
     }
     return glqh_fail("trellis kernel supports R (bits/weight) 1-4, got %d", R);
+}
+
+// Both stages of a stacked layer (4 + R2 bits/weight) against 1..16 transformed tokens in one launch:
+// part[(slot * B + token) * m + row] = sum1 + rs2 * sum2, K plan as glqh_launch_trellis_mma's.
+int glqh_launch_trellis_mma_rvq(const void *x_f16, int64_t B, const void *packed, const void *packed2, int R2, float rs2,
+                                int64_t m, int64_t k, int S, int ksplit, float *part, hipStream_t stream) {
+    if (B < 1 || B > 16) return glqh_fail("trellis two-stage kernel: 1..16 tokens, got %lld", (long long)B);
+    switch (R2) {
+    case 1: return launch_mma_rvq_R<1>(x_f16, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+    case 2: return launch_mma_rvq_R<2>(x_f16, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+    case 3: return launch_mma_rvq_R<3>(x_f16, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+    case 4: return launch_mma_rvq_R<4>(x_f16, B, packed, packed2, rs2, m, k, S, ksplit, part, stream);
+    }
+    return glqh_fail("trellis two-stage kernel: second stage of 1-4 bits/weight, got %d", R2);
 }
 
 // ---- fused-input GEMV (MFMA form): plan and launch -----------------------------------

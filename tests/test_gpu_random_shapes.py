@@ -146,34 +146,36 @@ def test_many_token_trellis_paths_of_large_layers(m, n, M, K):
     (32, 64, 4, 1, 64), (64, 4096, 4, 2, 4096), (160, 2368, 4, 3, 2300), (512, 2048, 4, 4, 2048),
     (960, 2560, 4, 2, 2560), (2048, 2048, 4, 1, 2048), (4096, 4096, 4, 2, 4000), (2048, 11008, 4, 4, 11008),
     (1088, 1088, 3, 2, 1088), (2048, 2048, 2, 2, 2048)])
-def test_one_token_of_two_stage_layers(m, n, K, K2, in_f):
-    """One token through a stacked layer: with a first stage of 4 bits/weight both streams are decoded in one
-    launch at every height (the last two cases, other first stages, take two launches); against the oracle,
-    through the finished output and through the RHT-domain product written into a wider row, and equal
-    bit for bit on a second call."""
+def test_few_tokens_of_two_stage_layers(m, n, K, K2, in_f):
+    """1, 3 and 16 tokens through a stacked layer: with a first stage of 4 bits/weight both streams are decoded in
+    one launch (at one token with the input transform folded in, at every height; at 2..16 tokens against the
+    staged transformed activations); the last two cases, other first stages, take a launch per stage.  Against
+    the oracle, through the finished output and through the RHT-domain product written into a wider row, and
+    equal bit for bit on a second call."""
     from glq_amd import ext, hadamard as H
-    say("one token two stages", m, n, K, K2, in_f)
+    say("few tokens two stages", m, n, K, K2, in_f)
     su, sv = O.rht_signs(m, n, 41)
     bn, bm = O.block_decompose(n), O.block_decompose(m)
     art = {"trellis_packed": O.random_packed(m, n, K, 11), "trellis_packed2": O.random_packed(m, n, K2, 12),
-           "inv_resid_scale2": np.float32(0.3), "SU": su.astype(np.float16), "SV": sv.astype(np.float16),
-           "Wscale": np.float32(0.02), "blocks_m": bm, "blocks_n": bn}
-    x = (torch.randn(1, in_f, generator=torch.Generator().manual_seed(m + n)) * 0.7).to(torch.bfloat16)
-    xp = np.zeros((1, n), np.float32)                         # columns past in_features are zero padding
-    xp[:, :in_f] = x.float().numpy()
+           "SU": su.astype(np.float16), "SV": sv.astype(np.float16)}
     W = (O.decode_layer(art["trellis_packed"], m, n, fast=True) +
          O.decode_layer(art["trellis_packed2"], m, n, fast=True) * np.float32(0.3)).astype(np.float32)
-    ref = O.linear_forward_rht(xp, W * np.float32(0.02), su.astype(np.float32), sv.astype(np.float32), bn, bm, n, m)
     bnt, bmt, bnm, bmm = torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV)
     p1, p2, svd, sud = t(art["trellis_packed"]), t(art["trellis_packed2"]), t(art["SV"]), t(art["SU"])
-    y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(x.to(DEV), svd, sud, p1, p2, bnt, bmt, bnm, bmm, 0.02, 0.3,
-                                                     in_f, m, n, m, out_dtype=torch.bfloat16)
-    assert rel(y, ref) < TOL, rel(y, ref)
-    assert torch.equal(y, ext.glq_fused_linear_trellis_3inst_rvq2_cuda(x.to(DEV), svd, sud, p1, p2, bnt, bmt, bnm, bmm,
-                                                                       0.02, 0.3, in_f, m, n, m, out_dtype=torch.bfloat16))
-    # the product before the output transform, into columns [32, 32 + m) of a wider row
-    wide = torch.full((1, m + 64), 7.0, dtype=torch.float32, device=DEV)
-    ext.glq_fused_linear_trellis_3inst_yrht_rvq2_cuda(x.to(DEV), svd, p1, p2, bnt, bnm, 0.02, 0.3, in_f, n, m, wide, 32)
-    xr = O.block_diag_fht(xp * sv.astype(np.float16).astype(np.float32)[None, :], bn)
-    assert rel(wide[:, 32:32 + m], (xr @ W.T) * np.float32(0.02)) < TOL
-    assert float(wide[:, :32].min()) == 7.0 and float(wide[:, 32 + m:].max()) == 7.0
+    for B in (1, 3, 16):
+        x = (torch.randn(B, in_f, generator=torch.Generator().manual_seed(m + n + B)) * 0.7).to(torch.bfloat16)
+        xp = np.zeros((B, n), np.float32)                     # columns past in_features are zero padding
+        xp[:, :in_f] = x.float().numpy()
+        ref = O.linear_forward_rht(xp, W * np.float32(0.02), su.astype(np.float32), sv.astype(np.float32), bn, bm, n, m)
+        y = ext.glq_fused_linear_trellis_3inst_rvq2_cuda(x.to(DEV), svd, sud, p1, p2, bnt, bmt, bnm, bmm, 0.02, 0.3,
+                                                         in_f, m, n, m, out_dtype=torch.bfloat16)
+        assert y.shape == (B, m)
+        assert rel(y, ref) < TOL, (B, rel(y, ref))
+        assert torch.equal(y, ext.glq_fused_linear_trellis_3inst_rvq2_cuda(x.to(DEV), svd, sud, p1, p2, bnt, bmt, bnm, bmm,
+                                                                           0.02, 0.3, in_f, m, n, m, out_dtype=torch.bfloat16))
+        # the product before the output transform, into columns [32, 32 + m) of a wider row
+        wide = torch.full((B, m + 64), 7.0, dtype=torch.float32, device=DEV)
+        ext.glq_fused_linear_trellis_3inst_yrht_rvq2_cuda(x.to(DEV), svd, p1, p2, bnt, bnm, 0.02, 0.3, in_f, n, m, wide, 32)
+        xr = O.block_diag_fht(xp * sv.astype(np.float16).astype(np.float32)[None, :], bn)
+        assert rel(wide[:, 32:32 + m], (xr @ W.T) * np.float32(0.02)) < TOL, B
+        assert float(wide[:, :32].min()) == 7.0 and float(wide[:, 32 + m:].max()) == 7.0

@@ -87,6 +87,9 @@ SIGNATURES = {
     "glqh_fused_linear_trellis_3inst_group": (
         c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_int, c_vp, c_i64, c_vp, c_i64, c_i64, c_int, c_i64,
                 c_vp, c_sz, c_vp]),
+    "glqh_fused_linear_trellis_3inst_group_rvq2": (
+        c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_vp, c_int, c_vp, c_i64, c_vp, c_i64, c_i64, c_int, c_i64,
+                c_vp, c_sz, c_vp]),
     "glqh_fused_moe_trellis_workspace_bytes": (c_sz, [c_i64, c_i64, c_i64, c_vp, c_vp]),
     "glqh_fused_moe_trellis_3inst": (
         c_int, [c_vp, c_int, c_i64, c_i64, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_i64, c_int, c_vp, c_int,

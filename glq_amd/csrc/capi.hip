@@ -37,11 +37,11 @@ static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages, bool
 int glqh_trellis_mma_fusein_plan(int64_t wgs_rows, int64_t k, int64_t B, int *S_out, int *ksplit_out);
 int glqh_launch_trellis_mma_rvq(const void *x_f16, int64_t B, const void *packed, const void *packed2, int R2, float rs2,
                                 int64_t m, int64_t k, int S, int ksplit, float *part, hipStream_t stream);
-int glqh_launch_trellis_mma_fusein_rvq(const void *packed, const void *packed2, int R2, float rs2, const void *x,
-                                       int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
-                                       int64_t in_features, int S, int ksplit, float *part,
-                                       const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
-                                       hipStream_t stream);
+int glqh_launch_trellis_mma_fusein_rvq(const void *const packed[], const void *const packed2[], int R2, const float rs2[],
+                                       const void *const sv[], float *const part[], const int64_t m[], int n_layers,
+                                       const void *x, int x_dtype, int64_t x_stride, int64_t k, int64_t in_features,
+                                       int S, int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                                       int n_blocks, hipStream_t stream);
 int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const sv[], float *const part[],
                                    const int64_t m[], int n_layers, int R, const void *x, int x_dtype,
                                    int64_t x_stride, int64_t B, int64_t k, int64_t in_features, int S,
@@ -539,9 +539,11 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         // One token of a 4 + R2 layer: both streams in one launch against one transform of x, the second
         // stage's sums added in registers (4096 x 4096 at 6 bpw: three launches become two).
         if (fuse2) {
-            if (glqh_launch_trellis_mma_fusein_rvq(packed, packed2, R2, (float)inv_resid_scale2, x, x_dtype, x_stride,
-                                                   sv_f16, m_pad, n_pad, in_features, fi_steps, ks, part1, bn_meta_dev,
-                                                   blocks_n, (int)n_blocks_n, st))
+            const void *pk1[1] = {packed}, *pk2[1] = {packed2}, *svs[1] = {sv_f16};
+            const float rs[1] = {(float)inv_resid_scale2};
+            float *pt[1] = {part1};
+            if (glqh_launch_trellis_mma_fusein_rvq(pk1, pk2, R2, rs, svs, pt, &m_pad, 1, x, x_dtype, x_stride, n_pad,
+                                                   in_features, fi_steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
                 return 1;
             two_parts = merge2 = false;
         }
@@ -937,6 +939,78 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
     if (!shards[0].y) return 0;                                // decode launch only: partial sums stay in ws
     return glqh_launch_output_rht_group(c.parts, c.su, c.ys, c.scale, c.m_pads, c.outs, n_shards, y_dtype, y_stride,
                                         B, c.ks, st);
+}
+
+// The same for stacked (two-stage) layers at one token: every layer's two streams decoded by one launch
+// (first stage 4 bits/weight, the second stages of one rate), finished like single-stage layers.
+extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                                          const glqh_trellis_shard *shards,
+                                                          const glqh_trellis_stage2 *stage2, int n_shards,
+                                                          const int64_t *blocks_n, int64_t n_blocks_n,
+                                                          const glqh_block_meta *bn_meta_dev, int64_t in_features,
+                                                          int64_t n_pad, int y_dtype, int64_t y_stride, void *ws,
+                                                          size_t ws_bytes, void *stream) {
+    GLQH_INIT();
+    hipStream_t st = (hipStream_t)stream;
+    GLQH_REQUIRE(x && shards && stage2, "trellis two-stage group: null pointer");
+    GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis two-stage group: %d shards (1..%d)", n_shards,
+                 GLQH_MAX_SHARDS);
+    GLQH_REQUIRE(B == 1, "trellis two-stage group: B=%lld (the grouped two-stage launch serves one token)", (long long)B);
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis two-stage group: x must be f16 or bf16");
+    GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad, "trellis two-stage group: in_features exceeds n_pad");
+    GLQH_REQUIRE(y_stride > 0, "trellis two-stage group: y_stride must be positive");
+    const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
+    GLQH_REQUIRE(n_blocks_n > 1 ? (bn_meta_dev != nullptr && blocks_n != nullptr) : pow2_n,
+                 "trellis two-stage group: input block sizes missing");
+    if (n_blocks_n > 1) {
+        int64_t sum = 0;
+        for (int64_t i = 0; i < n_blocks_n; ++i) {
+            GLQH_REQUIRE(blocks_n[i] > 0 && (blocks_n[i] & (blocks_n[i] - 1)) == 0,
+                         "trellis two-stage group: block size %lld is not a power of two", (long long)blocks_n[i]);
+            sum += blocks_n[i];
+        }
+        GLQH_REQUIRE(sum == n_pad, "trellis two-stage group: block sizes sum to %lld, expected %lld", (long long)sum,
+                     (long long)n_pad);
+    }
+    tr_group_ctx c;
+    const void *packed[GLQH_MAX_SHARDS], *packed2[GLQH_MAX_SHARDS], *sv[GLQH_MAX_SHARDS];
+    float rs2[GLQH_MAX_SHARDS];
+    int R2 = 0;
+    int64_t total = 0;
+    for (int i = 0; i < n_shards; ++i) {
+        const glqh_trellis_shard &sh = shards[i];
+        const glqh_trellis_stage2 &s2 = stage2[i];
+        GLQH_REQUIRE(sh.sv_f16 && sh.packed && sh.su_f16 && sh.y && s2.packed2, "trellis two-stage group: null pointer in shard %d", i);
+        GLQH_REQUIRE(s2.inv_resid_scale2 != 0.0, "trellis two-stage group: shard %d has a second stream but inv_resid_scale2 = 0", i);
+        int R1, Ri;
+        if (tr_bits_from_packed(sh.packed_cols, 0, &R1) || tr_check_shape(sh.m_pad, n_pad, sh.packed_rows)) return 1;
+        if (tr_bits_from_packed(s2.packed2_cols, 1, &Ri) || tr_check_shape(sh.m_pad, n_pad, s2.packed2_rows)) return 1;
+        GLQH_REQUIRE(R1 == 4, "trellis two-stage group: first stages of 4 bits/weight, shard %d has %d", i, R1);
+        GLQH_REQUIRE(i == 0 || Ri == R2, "trellis two-stage group: second stages of %d and %d bits/weight cannot share a launch",
+                     R2, Ri);
+        R2 = Ri;
+        GLQH_REQUIRE(sh.out_features >= 1 && sh.out_features <= sh.m_pad, "trellis two-stage group: out_features exceeds m_pad");
+        c.m_pads[i] = sh.m_pad; c.outs[i] = sh.out_features;
+        packed[i] = sh.packed; packed2[i] = s2.packed2; rs2[i] = (float)s2.inv_resid_scale2;
+        sv[i] = sh.sv_f16; c.su[i] = sh.su_f16; c.ys[i] = sh.y;
+        c.scale[i] = (float)sh.wscale;
+        total += sh.m_pad;
+    }
+    int steps = 0, ks = 0;
+    GLQH_REQUIRE(tr_fuse_input_enabled() && tr_fusein_plan(c.m_pads, n_shards, n_pad, 1, &steps, &ks, 1) == 2,
+                 "trellis two-stage group: shape not eligible");
+    const size_t need = align256((size_t)ks * total * sizeof(float));
+    GLQH_REQUIRE(ws && ws_bytes >= need, "trellis two-stage group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+    float *p = (float *)ws;
+    for (int i = 0; i < n_shards; ++i) {
+        c.parts[i] = p;
+        p += (size_t)ks * c.m_pads[i];
+    }
+    if (glqh_launch_trellis_mma_fusein_rvq(packed, packed2, R2, rs2, sv, c.parts, c.m_pads, n_shards, x, x_dtype, x_stride,
+                                           n_pad, in_features, steps, ks, bn_meta_dev, blocks_n, (int)n_blocks_n, st))
+        return 1;
+    return glqh_launch_output_rht_group(c.parts, c.su, c.ys, c.scale, c.m_pads, c.outs, n_shards, y_dtype, y_stride, 1,
+                                        ks, st);
 }
 
 // ---- routed experts of a mixture-of-experts layer ------------------------------------------------

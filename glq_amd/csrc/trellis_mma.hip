@@ -525,6 +525,32 @@ tr_mma_fusein_group_kernel(tr_fusein_group g, const XT *__restrict__ x, int64_t 
                                   part, 1.0f, xs_lds);
 }
 
+// several stacked layers (4 + R2 bits/weight each) on the same token: blockIdx.z = layer
+struct tr_fusein_group_rvq {
+    const uint8_t *packed2[GLQH_MAX_GROUP];
+    float rs2[GLQH_MAX_GROUP];
+};
+
+template <int R2, typename XT>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_fusein_group_rvq_kernel(tr_fusein_group g, tr_fusein_group_rvq g2, const XT *__restrict__ x, int64_t x_stride,
+                               int k, int in_features, int S, const glqh_block_meta *__restrict__ bn_meta,
+                               int n_blocks, glqh_meta_args margs) {
+    extern __shared__ u32x4 xs_lds[];
+    const int z = blockIdx.z;
+    const uint8_t *packed = g.packed[0], *packed2 = g2.packed2[0];
+    const f16 *sv = g.sv[0];
+    float *part = g.part[0];
+    float rs2 = g2.rs2[0];
+    int m = g.m[0];
+#pragma unroll
+    for (int i = 1; i < GLQH_MAX_GROUP; ++i)
+        if (i == z) { packed = g.packed[i]; packed2 = g2.packed2[i]; rs2 = g2.rs2[i]; sv = g.sv[i]; part = g.part[i]; m = g.m[i]; }
+    if ((int)blockIdx.x * 64 >= m) return;
+    tr_mma_fusein_body<4, XT, 1, R2>(packed, x, x_stride, sv, 1, m, k, in_features, S, bn_meta, n_blocks, margs, part, 1.0f,
+                                     xs_lds, 0, packed2, rs2);
+}
+
 // Routed experts of a mixture-of-experts layer, one token each (glq/csrc/glq_cuda.cu:5030-5250,
 // glq/csrc/glq_trellis.cu:539-588): blockIdx.z = slot = (token, choice); the slot's expert comes
 // from topk_ids on the device, so nothing about the routing is known to the host and the launch
@@ -908,24 +934,45 @@ int glqh_launch_trellis_mma_fusein(const void *const packed[], const void *const
     return glqh_fail("fused-input trellis kernel supports R (bits/weight) 1-4, got %d", R);
 }
 
-// One token through both stages of a stacked layer (4 + R2 bits/weight) in one launch: part[K slot][row].
-int glqh_launch_trellis_mma_fusein_rvq(const void *packed, const void *packed2, int R2, float rs2, const void *x,
-                                       int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
-                                       int64_t in_features, int S, int ksplit, float *part,
-                                       const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
-                                       hipStream_t stream) {
+// One token through both stages of stacked layers (4 + R2 bits/weight each, 1..GLQH_MAX_GROUP layers on the same
+// token) in one launch: part[l][K slot][row].
+int glqh_launch_trellis_mma_fusein_rvq(const void *const packed[], const void *const packed2[], int R2, const float rs2[],
+                                       const void *const sv[], float *const part[], const int64_t m[], int n_layers,
+                                       const void *x, int x_dtype, int64_t x_stride, int64_t k, int64_t in_features,
+                                       int S, int ksplit, const glqh_block_meta *bn_meta, const int64_t *blocks_host,
+                                       int n_blocks, hipStream_t stream) {
     glqh_range range("dequant_matmul");
+    GLQH_REQUIRE(n_layers >= 1 && n_layers <= GLQH_MAX_GROUP, "trellis group: 1..%d layers", GLQH_MAX_GROUP);
     GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "fused-input trellis kernel: x must be f16 or bf16");
     glqh_meta_args margs;
     if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
     const glqh_block_meta *meta = n_blocks > 1 ? bn_meta : nullptr;
     const int nb = n_blocks > 1 ? n_blocks : 1;
     const size_t lds = fi_lds_bytes<1>(S);
-    const dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, 1);
+    tr_fusein_group g = {};
+    tr_fusein_group_rvq g2 = {};
+    int64_t max_m = 0;
+    for (int i = 0; i < GLQH_MAX_GROUP; ++i) {
+        const int j = i < n_layers ? i : 0;
+        g.packed[i] = (const uint8_t *)packed[j];
+        g.sv[i] = (const f16 *)sv[j];
+        g.part[i] = part[j];
+        g.m[i] = (int)m[j];
+        g2.packed2[i] = (const uint8_t *)packed2[j];
+        g2.rs2[i] = rs2[j];
+        if (m[j] > max_m) max_m = m[j];
+    }
+    const dim3 grid((unsigned)((max_m + 63) / 64), (unsigned)ksplit, (unsigned)n_layers);
 #define GLQH_FI2(RR, XT)                                                                                        \
-    hipLaunchKernelGGL((tr_mma_fusein_rvq_kernel<RR, XT>), grid, dim3(TR_THREADS), lds, stream,                 \
-                       (const uint8_t *)packed, (const uint8_t *)packed2, rs2, (const XT *)x, x_stride,         \
-                       (const f16 *)sv, (int)m, (int)k, (int)in_features, S, meta, nb, margs, part)
+    do {                                                                                                        \
+        if (n_layers == 1)                                                                                      \
+            hipLaunchKernelGGL((tr_mma_fusein_rvq_kernel<RR, XT>), grid, dim3(TR_THREADS), lds, stream,         \
+                               g.packed[0], g2.packed2[0], g2.rs2[0], (const XT *)x, x_stride, g.sv[0], g.m[0], \
+                               (int)k, (int)in_features, S, meta, nb, margs, g.part[0]);                        \
+        else                                                                                                    \
+            hipLaunchKernelGGL((tr_mma_fusein_group_rvq_kernel<RR, XT>), grid, dim3(TR_THREADS), lds, stream, g, g2, \
+                               (const XT *)x, x_stride, (int)k, (int)in_features, S, meta, nb, margs);          \
+    } while (0)
 #define GLQH_FI2_R(RR)                                                \
     do {                                                              \
         if (x_dtype == GLQH_F16) GLQH_FI2(RR, f16);                   \
@@ -1060,6 +1107,8 @@ static int fi_init_R() {
     const size_t b1 = fi_lds_bytes<1>(FI_MAX_S), b4 = fi_lds_bytes<4>(FI_MAX_S_TP4);
     if (fi_set_lds(tr_mma_fusein_moe_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_moe_kernel<R, uint16_t>, b1)) return 1;
     if (fi_set_lds(tr_mma_fusein_rvq_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_rvq_kernel<R, uint16_t>, b1)) return 1;
+    if (fi_set_lds(tr_mma_fusein_group_rvq_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_group_rvq_kernel<R, uint16_t>, b1))
+        return 1;
     return fi_set_lds(tr_mma_fusein_kernel<R, f16, 1>, b1) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 1>, b1) ||
            fi_set_lds(tr_mma_fusein_kernel<R, f16, 4>, b4) || fi_set_lds(tr_mma_fusein_kernel<R, uint16_t, 4>, b4) ||
            fi_set_lds(tr_mma_fusein_group_kernel<R, f16, 1>, b1) ||

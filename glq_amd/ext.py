@@ -433,6 +433,53 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
     return y
 
 
+class _TrellisStage2(C.Structure):
+    _fields_ = [("packed2", C.c_void_p), ("packed2_rows", C.c_int64), ("packed2_cols", C.c_int64),
+                ("inv_resid_scale2", C.c_double)]
+
+
+def glq_fused_linear_trellis_3inst_group_rvq2(x, shards, blocks_n, blocks_n_meta, in_features, n_pad,
+                                              out_dtype=None):
+    """The grouped call for stacked (two-stage) layers at one token: the decode step of fused q/k/v or
+    gate/up of a 5-8 bpw checkpoint, whose per-shard loop in the reference is
+    fused_linear_trellis_3inst_yrht_rvq2 per shard + output_rht_shards (glq_vllm/linear_method.py:664-710).
+
+    shards: sequence of (sv, su, trellis_packed, trellis_packed2, wscale, inv_resid_scale2, out_features,
+    m_pad); first stages of 4 bpw, second stages of one common rate.  Returns (1, sum(out_features)).
+    Raises RuntimeError for other token counts or rates (callers then use the per-layer op)."""
+    lib = _lib.load()
+    _chk(x, "x", (torch.float16, torch.bfloat16))
+    B = x.shape[0]
+    dt = out_dtype or torch.float16
+    total_out = sum(int(s[6]) for s in shards)
+    total_m = sum(int(s[7]) for s in shards)
+    y = torch.empty((B, total_out), dtype=dt, device=x.device)
+    arr = (_TrellisShard * len(shards))()
+    arr2 = (_TrellisStage2 * len(shards))()
+    off = 0
+    esz = torch.empty((), dtype=dt).element_size()
+    for i, (sv, su, packed, packed2, wscale, inv2, out_f, m_pad) in enumerate(shards):
+        _chk(sv, "sv", torch.float16)
+        _chk(su, "su", torch.float16)
+        _chk(packed, "trellis_packed", torch.int16)
+        _chk(packed2, "trellis_packed2", torch.int16)
+        if packed.dim() != 2 or packed2.dim() != 2:
+            raise RuntimeError("trellis_packed / trellis_packed2 must be 2-D [(m/16)*(k/16), 16*R]")
+        arr[i] = _TrellisShard(_p(sv), _p(su), _p(packed), packed.shape[0], packed.shape[1], float(wscale),
+                               int(out_f), int(m_pad), y.data_ptr() + off * esz)
+        arr2[i] = _TrellisStage2(_p(packed2), packed2.shape[0], packed2.shape[1], float(inv2))
+        off += int(out_f)
+    bn, nbn = _host_i64(blocks_n)
+    with torch.cuda.device(x.device):
+        nb = lib.glqh_fused_linear_trellis_group_workspace_bytes(1, int(n_pad), total_m, len(shards))
+        ws = _ws(max(nb, 256), x.device)
+        check(lib.glqh_fused_linear_trellis_3inst_group_rvq2(
+            _p(x), _DT[x.dtype], x.shape[1], B, C.addressof(arr), C.addressof(arr2), len(shards), bn, nbn,
+            _meta_ptr(blocks_n_meta) if nbn > 1 else None, int(in_features), int(n_pad), _DT[dt], total_out,
+            _p(ws), ws.numel(), _stream()))
+    return y
+
+
 class _MoeProj(C.Structure):
     _fields_ = [("packed", C.c_void_p), ("packed_rows", C.c_int64), ("packed_cols", C.c_int64),
                 ("packed2", C.c_void_p), ("packed2_cols", C.c_int64), ("su", C.c_void_p), ("sv", C.c_void_p),

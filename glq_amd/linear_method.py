@@ -26,8 +26,9 @@ from .quantized_linear import E8RHTLinear
 # (glq_vllm/linear_method.py:616).
 _GLQ_BATCH_OUT_RHT = os.environ.get("GLQ_TRELLIS_BATCH_OUT_RHT", "1") != "0"
 # GLQ_MERGED_GROUPED=1: merged single-stage shards go through the library's grouped call (one decode or
-# many-token launch for all shards) at 1-4 and at more than 64 tokens instead of the reference's per-shard
-# sequence; same result up to the rounding of another K split.  Off by default: the default is the
+# many-token launch for all shards) at 1-4 and at more than 64 tokens, merged two-stage shards at one token
+# through its two-stage form, instead of the reference's per-shard sequence; same result up to the rounding of
+# another K split.  Off by default: the default is the
 # reference's own op sequence.
 _GLQ_MERGED_GROUPED = os.environ.get("GLQ_MERGED_GROUPED", "0") == "1"
 
@@ -208,9 +209,27 @@ class MergedTrellisLinear:
             return False
         return B <= 4 or (B > 64 and len(metas) <= 4)
 
+    def _grouped_rvq2_ok(self, B):
+        """One token of merged stacked shards (first stages of 4 bpw, second stages of one rate): the library's
+        grouped two-stage call."""
+        metas = self._glq_trellis_meta
+        if B != 1 or not (self.glq_is_fused and all(m["loaded"] and m["has_s2"] for m in metas)):
+            return False
+        n = range(len(metas))
+        return ({self.trellis_packed.get_shard(i).shape[1] for i in n} == {64} and
+                len({self.trellis_packed2.get_shard(i).shape[1] for i in n}) == 1)
+
     def _apply_2d(self, x):
         _apply = E8RHTLinear._trellis_linear_apply
         metas = self._glq_trellis_meta
+        if _GLQ_MERGED_GROUPED and x.dtype in (torch.float16, torch.bfloat16) and self._grouped_rvq2_ok(x.shape[0]):
+            from . import ext
+            m0 = metas[0]
+            return ext.glq_fused_linear_trellis_3inst_group_rvq2(
+                x.contiguous(), [(self.SV.get_shard(i), self.SU.get_shard(i), self.trellis_packed.get_shard(i),
+                                  self.trellis_packed2.get_shard(i), m["wscale"], m["inv_rs2"], m["out"], m["m_pad"])
+                                 for i, m in enumerate(metas)],
+                m0["_bn"], m0["_bnm"], m0["in"], m0["n_pad"], out_dtype=x.dtype)
         if _GLQ_MERGED_GROUPED and x.dtype in (torch.float16, torch.bfloat16) and self._grouped_ok(x.shape[0]):
             from . import ext
             m0 = metas[0]

@@ -214,6 +214,29 @@ int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_
                                           int y_dtype, int64_t y_stride,
                                           void *ws, size_t ws_bytes, void *stream);
 
+/* Second stage of a stacked (two-stage, 5-8 bits/weight) shard: the residual stream and its
+ * scale, trellis_packed2 / inv_resid_scale2 of glq/quantized_linear.py:986-1010. */
+typedef struct {
+    const void *packed2;      /* ((m_pad/16) * (n_pad/16), 16 * R2) int16 */
+    int64_t packed2_rows, packed2_cols;
+    double inv_resid_scale2;
+} glqh_trellis_stage2;
+
+/* The grouped call for stacked layers at ONE token (the decode step of fused q/k/v and gate/up of a
+ * 5-8 bits/weight checkpoint; the reference runs fused_linear_trellis_3inst_yrht_rvq2 per shard,
+ * glq_vllm/linear_method.py:664-710): one decode launch reads both streams of every layer (first
+ * stages of 4 bits/weight, second stages of one common rate, stage2[i] belongs to shards[i]) and one
+ * launch finishes them.  Workspace: glqh_fused_linear_trellis_group_workspace_bytes(1, ...).  Every
+ * shard's y must be given; other token counts and rates are refused (per-layer calls serve them). */
+int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_dtype, int64_t x_stride, int64_t B,
+                                               const glqh_trellis_shard *shards,
+                                               const glqh_trellis_stage2 *stage2, int n_shards,
+                                               const int64_t *blocks_n, int64_t n_blocks_n,
+                                               const glqh_block_meta *bn_meta_dev,
+                                               int64_t in_features, int64_t n_pad,
+                                               int y_dtype, int64_t y_stride,
+                                               void *ws, size_t ws_bytes, void *stream);
+
 /* One projection (gate/up "w13" or down "w2") of the routed experts of a mixture-of-experts
  * layer, the experts stacked along the first dimension (glq/csrc/glq_cuda.cu:5043-5064). */
 typedef struct {

@@ -1020,6 +1020,13 @@ int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes,
                                        int64_t k, int64_t in_features, int S, int ksplit, float *part,
                                        const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
                                        hipStream_t stream);
+int glqh_launch_trellis_mma_fusein_moe_rvq(const void *packed, int64_t stride_bytes, const void *packed2,
+                                           int64_t stride2_bytes, int R2, const float *inv_rs2_dev,
+                                           const int64_t *topk_ids, int n_slots, int n_experts, int x_div, const void *x,
+                                           int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
+                                           int64_t in_features, int S, int ksplit, float *part,
+                                           const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                                           hipStream_t stream);
 int glqh_launch_moe_output_rht(const float *part, int ks, int part_f16, int n_slots, int n_experts, const int64_t *topk_ids,
                                const void *su_base, const float *wscale_dev, int64_t out_features, int64_t m_pad,
                                const int64_t *blocks_m, int64_t n_blocks_m, void *h_f16, int64_t h_stride,
@@ -1065,6 +1072,7 @@ int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t str
 struct moe_plan {
     int R1, R2, S, ks, ks_all;
     int tile;                                                  // the tile kernel's form: one K slot, fp16 sums
+    int fuse2;                                                 // per-slot form, two stages in one launch: ks slots
     size_t part_bytes;
 };
 
@@ -1147,7 +1155,8 @@ static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, int64_t n_expe
         GLQH_REQUIRE(glqh_trellis_mma_fusein_plan((w->m_pad / 64) * n_slots, w->n_pad, 1, &p->S, &p->ks),
                      "routed experts %s: no plan", what);
     }
-    p->ks_all = p->R2 ? 2 * p->ks : p->ks;
+    p->fuse2 = p->R2 && p->R1 == 4 && !p->tile && n_slots < moe_group_min(n_experts) && tr_fuse_stages_enabled();
+    p->ks_all = p->R2 && !p->fuse2 ? 2 * p->ks : p->ks;
     p->part_bytes = align256((size_t)p->ks_all * n_slots * w->m_pad * sizeof(float));
     return 0;
 }
@@ -1242,6 +1251,12 @@ static int moe_decode_tile(const glqh_moe_proj *w, const moe_plan &p, const int 
 // one projection: decode launch per stage into part[K slot][slot][row]
 static int moe_decode(const glqh_moe_proj *w, const moe_plan &p, const int64_t *topk_ids, int n_slots, int n_experts,
                       int x_div, const void *x, int x_dtype, int64_t x_stride, float *part, hipStream_t st) {
+    if (p.fuse2)
+        return glqh_launch_trellis_mma_fusein_moe_rvq(w->packed, w->packed_rows * w->packed_cols * 2, w->packed2,
+                                                      w->packed_rows * w->packed2_cols * 2, p.R2, w->inv_rs2_dev, topk_ids,
+                                                      n_slots, n_experts, x_div, x, x_dtype, x_stride, w->sv_f16, w->m_pad,
+                                                      w->n_pad, w->in_features, p.S, p.ks, part, w->bn_meta_dev, w->blocks_n,
+                                                      (int)w->n_blocks_n, st);
     if (glqh_launch_trellis_mma_fusein_moe(w->packed, w->packed_rows * w->packed_cols * 2, p.R1, topk_ids, n_slots,
                                            n_experts, x_div, nullptr, x, x_dtype, x_stride, w->sv_f16, w->m_pad,
                                            w->n_pad, w->in_features, p.S, p.ks, part, w->bn_meta_dev, w->blocks_n,

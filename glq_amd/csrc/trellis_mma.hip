@@ -582,6 +582,24 @@ tr_mma_fusein_moe_kernel(tr_moe_args g, const XT *__restrict__ x, int64_t x_stri
                                  g.n_slots);
 }
 
+// Two-stage experts (first stage 4 bits/weight): both streams of the slot's expert in the same launch, the second
+// one's sums times the expert's inv_resid_scale2 (read on the device) added in registers.
+template <int R2, typename XT>
+__global__ void __launch_bounds__(TR_THREADS)
+tr_mma_fusein_moe_rvq_kernel(tr_moe_args g, const uint8_t *__restrict__ packed2, int64_t stride2_bytes,
+                             const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv, int m, int k,
+                             int in_features, int S, const glqh_block_meta *__restrict__ bn_meta, int n_blocks,
+                             glqh_meta_args margs) {
+    extern __shared__ u32x4 xs_lds[];
+    const int slot = blockIdx.z;
+    const int64_t e = g.topk_ids[slot];
+    if (e < 0 || e >= g.n_experts) return;                      // uniform over the workgroup
+    tr_mma_fusein_body<4, XT, 1, R2>(g.packed + e * g.stride_bytes, x + (int64_t)(slot / g.x_div) * x_stride, x_stride,
+                                     sv, 1, m, k, in_features, S, bn_meta, n_blocks, margs,
+                                     g.part + (int64_t)slot * m, 1.0f, xs_lds, g.n_slots, packed2 + e * stride2_bytes,
+                                     g.pscale_dev[e]);
+}
+
 // The same step for many slots: the slots are grouped by expert (perm: slot numbers sorted by
 // expert, offs: first position of every expert, both made on the device by the routing launch), and
 // workgroup (row block, K slot, expert) reads its expert's stream once per 16 of the expert's rows
@@ -1041,6 +1059,55 @@ int glqh_launch_trellis_mma_fusein_moe(const void *packed, int64_t stride_bytes,
     return glqh_fail("routed experts: R (bits/weight) 1-4, got %d", R);
 }
 
+// Both stages of two-stage experts (4 + R2 bits/weight) per slot in one launch: part[K slot][slot][row] =
+// sum1 + inv_rs2_dev[expert] * sum2.
+int glqh_launch_trellis_mma_fusein_moe_rvq(const void *packed, int64_t stride_bytes, const void *packed2,
+                                           int64_t stride2_bytes, int R2, const float *inv_rs2_dev,
+                                           const int64_t *topk_ids, int n_slots, int n_experts, int x_div, const void *x,
+                                           int x_dtype, int64_t x_stride, const void *sv, int64_t m, int64_t k,
+                                           int64_t in_features, int S, int ksplit, float *part,
+                                           const glqh_block_meta *bn_meta, const int64_t *blocks_host, int n_blocks,
+                                           hipStream_t stream) {
+    glqh_range range("dequant_matmul");
+    GLQH_REQUIRE(n_slots >= 1 && n_slots <= 65535, "routed experts: %d slots (1..65535)", n_slots);
+    GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "routed experts: x must be f16 or bf16");
+    GLQH_REQUIRE(inv_rs2_dev && packed2, "routed experts: second stage missing");
+    tr_moe_args g;
+    g.packed = (const uint8_t *)packed;
+    g.stride_bytes = stride_bytes;
+    g.topk_ids = topk_ids;
+    g.pscale_dev = inv_rs2_dev;
+    g.part = part;
+    g.n_slots = n_slots;
+    g.n_experts = n_experts;
+    g.x_div = x_div;
+    glqh_meta_args margs;
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, k)) margs.canon = 0;
+    const glqh_block_meta *meta = n_blocks > 1 ? bn_meta : nullptr;
+    const int nb = n_blocks > 1 ? n_blocks : 1;
+    const dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, (unsigned)n_slots);
+#define GLQH_MOE2(RR, XT)                                                                                          \
+    hipLaunchKernelGGL((tr_mma_fusein_moe_rvq_kernel<RR, XT>), grid, dim3(TR_THREADS), fi_lds_bytes<1>(S), stream, g, \
+                       (const uint8_t *)packed2, stride2_bytes, (const XT *)x, x_stride, (const f16 *)sv, (int)m,  \
+                       (int)k, (int)in_features, S, meta, nb, margs)
+#define GLQH_MOE2_R(RR)                                               \
+    do {                                                              \
+        if (x_dtype == GLQH_F16) GLQH_MOE2(RR, f16);                  \
+        else GLQH_MOE2(RR, uint16_t);                                 \
+    } while (0)
+    switch (R2) {
+    case 1: GLQH_MOE2_R(1); break;
+    case 2: GLQH_MOE2_R(2); break;
+    case 3: GLQH_MOE2_R(3); break;
+    case 4: GLQH_MOE2_R(4); break;
+    default: return glqh_fail("routed experts: second stage of 1-4 bits/weight, got %d", R2);
+    }
+#undef GLQH_MOE2_R
+#undef GLQH_MOE2
+    GLQH_LAUNCH_CHECK("trellis routed-expert two-stage gemv launch");
+    return 0;
+}
+
 static int moe_wide_min_rows() {                                // GLQ_MOE_WIDE_MIN_ROWS: average rows per expert
     static const int v = [] {
         const char *e = getenv("GLQ_MOE_WIDE_MIN_ROWS");
@@ -1106,6 +1173,8 @@ template <int R>
 static int fi_init_R() {
     const size_t b1 = fi_lds_bytes<1>(FI_MAX_S), b4 = fi_lds_bytes<4>(FI_MAX_S_TP4);
     if (fi_set_lds(tr_mma_fusein_moe_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_moe_kernel<R, uint16_t>, b1)) return 1;
+    if (fi_set_lds(tr_mma_fusein_moe_rvq_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_moe_rvq_kernel<R, uint16_t>, b1))
+        return 1;
     if (fi_set_lds(tr_mma_fusein_rvq_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_rvq_kernel<R, uint16_t>, b1)) return 1;
     if (fi_set_lds(tr_mma_fusein_group_rvq_kernel<R, f16>, b1) || fi_set_lds(tr_mma_fusein_group_rvq_kernel<R, uint16_t>, b1))
         return 1;

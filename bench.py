@@ -288,7 +288,20 @@ def extras(torch, ext, dev):
             torch, lambda: [ext.glq_fused_linear_trellis_3inst_rvq2_cuda(xb, sv, sv, a, b, bnt, bnt, bnm, bnm, 0.02, 0.3,
                                                                          n, m, n, m, out_dtype=torch.bfloat16)
                             for a, b in zip(p4, p2)], len(p4)), 2)
-        del p4, p2
+        xb4 = torch.randn(4, n, device=dev).to(torch.bfloat16)
+        out["trellis_linear_4096x4096_6bpw_B4_us"] = round(_graph_time(
+            torch, lambda: [ext.glq_fused_linear_trellis_3inst_rvq2_cuda(xb4, sv, sv, a, b, bnt, bnt, bnm, bnm, 0.02, 0.3,
+                                                                         n, m, n, m, out_dtype=torch.bfloat16)
+                            for a, b in zip(p4, p2)], len(p4)), 2)
+        # fused q/k/v of a 6 bpw 4096-wide model (4096 + 1024 + 1024 rows), one token: both streams of the three
+        # layers in one decode launch, one finishing launch
+        rows = (4096, 1024, 1024)
+        groups = [[(sv, sv[:r], p4[3 * g + i][:(r // 16) * (n // 16)], p2[3 * g + i][:(r // 16) * (n // 16)], 0.02, 0.3, r, r)
+                   for i, r in enumerate(rows)] for g in range(12)]
+        out["trellis_group_qkv_4096_6bpw_B1_us"] = round(_graph_time(
+            torch, lambda: [ext.glq_fused_linear_trellis_3inst_group_rvq2(xb, sh, bnt, bnm, n, n, out_dtype=torch.bfloat16)
+                            for sh in groups], len(groups)), 2)
+        del p4, p2, groups
         m, n, M = 14336, 4096, 4096
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
         xh = torch.randn(M, n, device=dev).to(torch.float16)

@@ -215,7 +215,7 @@ def test_refusals(ext):
 @pytest.mark.parametrize("hidden,inter,T,K,K2", [(256, 128, 16, 4, 0), (320, 192, 40, 2, 0), (320, 192, 33, 3, 2),
                                                  (256, 128, 24, 4, 0), (256, 128, 90, 2, 0), (256, 128, 80, 3, 1),
                                                  (256, 128, 200, 3, 0), (320, 192, 300, 2, 2), (256, 128, 530, 2, 0),
-                                                 (256, 128, 1100, 4, 0)])
+                                                 (256, 128, 1100, 4, 0), (320, 192, 600, 2, 2)])
 def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     """From max(16, 3/4 of the experts) slots on the rows are grouped by expert.  Skewed routing: every token's first choice is
     expert 2 (more than two tiles of 16 rows for it), expert 5 gets nothing, some ids are out of range.  From an
@@ -224,7 +224,8 @@ def test_many_slots_grouped_by_expert(ext, hidden, inter, T, K, K2):
     per expert on average the sorted slots go through the tile kernel in runs of up to 256 positions of one
     expert: expert 2 has one run of 199 (T = 200), two of 160 and 139 (300), three of 192, 192 and 145 (530), the
     other experts one partial run each.  T = 1100: 4400 slots, whose routing table is made by two launches over
-    three segments of the slots, and runs of up to 512 positions."""
+    three segments of the slots, and runs of up to 512 positions.  T = 600 with two-stage experts: 1200 slots, from
+    1024 on one launch between the projections and one after them, here on the sums of both stages."""
     say("moe grouped", hidden, inter, T, K, K2)
     ex = experts(6, hidden, inter, 4, K2, seed=2)
     rng = np.random.default_rng(T)

@@ -1020,9 +1020,9 @@ moe_mid_kernel(moe_mid_args a, f16 *__restrict__ out, glqh_meta_args m13, glqh_m
         if (active && blk.off + 8 * tid < a.o.out_features) load8<f16>(su + blk.off + 8 * tid, r.f);
     };
     const int big = rht_slice_of(m13, 0.0f, 0).bs > 8 * (int)blockDim.x ? 1 : 0;   // only the first block can be
-    if (big) output_rht_wide_body<16, f16>(src, su, hrow, 0, a.o.out_features, a.o.m_pad, rht_slice_of(m13, 0.0f, 0), s, slot, role);
     req cur, nxt;
     if (big < a.nb13) request(cur, rht_slice_of(m13, 0.0f, big));
+    if (big) output_rht_wide_body<16, f16>(src, su, hrow, 0, a.o.out_features, a.o.m_pad, rht_slice_of(m13, 0.0f, 0), s, slot, role);
     for (int bi = big; bi < a.nb13; ++bi) {
         const rht_slice blk = rht_slice_of(m13, 0.0f, bi);
         if (bi + 1 < a.nb13) request(nxt, rht_slice_of(m13, 0.0f, bi + 1));
@@ -1139,7 +1139,7 @@ moe_final_kernel(moe_out_args a, const float *__restrict__ topk_w, int top_k, in
     if (b >= B) return;                                       // uniform over the workgroup
     const wide_role role = wide_role_of(blk, 1);
     if constexpr (BIG) {
-        if (blk.log_bs > 12) {
+        if (blk.bs > 8 * (int)blockDim.x) {
             moe_final_row<16, YT>(a, topk_w, top_k, out, out_stride, blk, s, b, role);
             return;
         }
@@ -1387,8 +1387,10 @@ int glqh_launch_moe_mid(const float *part, int ks, int part_f16, int n_slots, in
     const int64_t b13 = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)m_pad13));
     const int64_t b2 = (int64_t)1 << (63 - __builtin_clzll((unsigned long long)n_pad2));
     const int64_t max_bs = b13 > b2 ? b13 : b2;
+    // sixteen elements per thread on the largest block, eight on the others (each at most half of it): a row of
+    // 1024 + 512 points is one wave's work, with no exchange between waves
     int threads = 64;
-    while (threads < REG_THREADS && 8 * threads < max_bs) threads <<= 1;
+    while (threads < REG_THREADS && 16 * threads < max_bs) threads <<= 1;
     const size_t s_bytes = (rht_reg_lds_bytes(ilog2(max_bs)) + 15) & ~(size_t)15;
     const size_t lds = s_bytes + (size_t)(m_pad13 + n_pad2) * sizeof(f16);
     moe_mid_args a = {};
@@ -1433,12 +1435,14 @@ int glqh_launch_moe_final(const float *part, int ks, int part_f16, int num_token
     const size_t lds = rht_reg_lds_bytes(ilog2(max_bs));
     // rows without small blocks (which take several tokens per workgroup of 512 threads): as many threads as the
     // largest block has groups of eight elements
+    // (sixteen elements per thread on half as many threads: slower, the whole call of 32768 slots x 2048 rows 701 -> 714 us
+    // -- the registers of two choices in flight cost occupancy)
     int threads = REG_THREADS;
     if ((m_pad & 1023) == 0 && max_bs <= 2048) threads = (int)(max_bs / 8);
 #define GLQH_MOE_FINAL(YT, BIG)                                                                                  \
     hipLaunchKernelGGL((moe_final_kernel<YT, BIG>), grid, dim3((unsigned)threads), lds, stream, a, topk_w, top_k, num_tokens, \
                        (YT *)out, out_stride, nb, margs)
-    const bool big = max_bs > 4096;
+    const bool big = max_bs > 8 * threads;
     if (out_dtype == GLQH_F16) { if (big) GLQH_MOE_FINAL(f16, true); else GLQH_MOE_FINAL(f16, false); }
     else { if (big) GLQH_MOE_FINAL(uint16_t, true); else GLQH_MOE_FINAL(uint16_t, false); }
 #undef GLQH_MOE_FINAL

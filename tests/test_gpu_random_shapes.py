@@ -179,3 +179,21 @@ def test_few_tokens_of_two_stage_layers(m, n, K, K2, in_f):
         xr = O.block_diag_fht(xp * sv.astype(np.float16).astype(np.float32)[None, :], bn)
         assert rel(wide[:, 32:32 + m], (xr @ W.T) * np.float32(0.02)) < TOL, B
         assert float(wide[:, :32].min()) == 7.0 and float(wide[:, 32 + m:].max()) == 7.0
+
+
+def test_two_stage_layers_with_a_launch_per_stage_in_a_fresh_process():
+    """GLQ_TRELLIS_FUSE_STAGES=0 (read once by the library): two-stage layers decode their stages in two launches
+    at every token count; the two-stage cases of this file and of the module tests against the oracle that way, in
+    a process of their own."""
+    import os
+    import subprocess
+    import sys
+    say("two-stage layers, a launch per stage, child process")
+    here = os.path.dirname(os.path.abspath(__file__))
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.abspath(__file__), os.path.join(here, "test_gpu_module.py"),
+                        "-x", "-q", "-m", "gpu", "-k", "two_stage and not fresh_process", "--timeout", "300",
+                        "--timeout-method", "thread", "-p", "no:cacheprovider"],
+                       env={**os.environ, "GLQ_TRELLIS_FUSE_STAGES": "0"}, capture_output=True, text=True, timeout=900,
+                       cwd=os.path.dirname(here))
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
+    assert " passed" in r.stdout and "no tests ran" not in r.stdout, r.stdout[-500:]

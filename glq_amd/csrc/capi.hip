@@ -63,10 +63,11 @@ static int tr_fusein_plan(const int64_t *m_pads, int n, int64_t n_pad, int64_t B
 }
 // many-token kernel (trellis_tile.hip): weights decoded once per 128-row x 512-token tile
 size_t glqh_trellis_tile_xb_bytes(int64_t k, int64_t M);
-int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M);
+int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M, int two_stage = 0);
 int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
-                             hipStream_t stream, int out_f16 = 0);
+                             hipStream_t stream, int out_f16 = 0, const void *packed2 = nullptr, int R2 = 0,
+                             float rs2 = 0.0f);
 int64_t glqh_trellis_tile_padded_tokens(int64_t M);
 int glqh_trellis_tile_group_ksplit(const int64_t *m, int n_layers, int64_t k, int64_t M);
 int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void *const packed[], int R,
@@ -426,6 +427,7 @@ extern "C" int glqh_output_rht_shards(const float *y_rht, const void *su_f16, vo
 // workspace layout: [x_rht f16 (B, n_pad)] [partials stage 1] [partials stage 2]
 static size_t tr_fused_part_bytes(int64_t B, int64_t n_pad, int64_t m_pad) {
     int ks = tr_plain_plan(m_pad, n_pad, B).ks;
+    if (B > tr_small_batch()) ks = std::max(ks, glqh_trellis_tile_ksplit(m_pad, n_pad, B, 1));   // a stacked layer's plan
     int steps = 0, ks2 = 0;
     if (tr_fusein_plan(&m_pad, 1, n_pad, B, &steps, &ks2) && ks2 > ks) ks = ks2;
     // one token of a two-stage layer plans the MFMA form at every height
@@ -576,7 +578,11 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         else if (glqh_launch_input_rht(x, x_dtype, x_stride, sv_f16, x_rht, GLQH_F16, B, in_features, n_pad,
                                        bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
             return 1;
-        ks = plan.ks;
+        // 17 tokens and more of a 4 + R2 layer: the tile kernels decode both streams into one operand,
+        // W = fp16(W1 + inv_resid_scale2 * W2) -- the weight of the reference's many-token route -- in tiles of at
+        // most 256 tokens: one launch with the products of a single-stage layer instead of two
+        const bool tile2 = has_s2 && plan.tile && R1 == 4 && tr_fuse_stages_enabled();
+        ks = tile2 ? glqh_trellis_tile_ksplit(m_pad, n_pad, B, 1) : plan.ks;
         if (merge2) part2 = part1 + (int64_t)ks * B * m_pad;
         // Many tokens: the tile kernel rounds its sums to fp16 on the way out, as the reference's
         // many-token route does (its library GEMM of two fp16 matrices returns fp16,
@@ -586,7 +592,13 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         // its seven linears).  GLQ_TRELLIS_F16_SUMS=0 keeps them fp32.
         f16_sums = plan.tile && ks <= tr_f16_sums_max_slots() && B > 64 && !y_rht_out && y && tr_f16_sums_enabled() &&
                    glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad);
-        if (has_s2 && !plan.tile && R1 == 4 && tr_fuse_stages_enabled()) {
+        if (tile2) {
+            glqh_range range("dequant_matmul");
+            if (glqh_launch_trellis_tile(x_in, xb_tile, B, packed, R1, m_pad, n_pad, part1, 0, 1.0f, 0, 0, st, f16_sums,
+                                         packed2, R2, (float)inv_resid_scale2))
+                return 1;
+            two_parts = merge2 = false;
+        } else if (has_s2 && !plan.tile && R1 == 4 && tr_fuse_stages_enabled()) {
             // up to 16 tokens of a 4 + R2 layer: both streams in one pass over the staged activations
             glqh_range range("dequant_matmul");
             if (glqh_launch_trellis_mma_rvq(x_in, B, packed, packed2, R2, (float)inv_resid_scale2, m_pad, n_pad, plan.S,

@@ -53,6 +53,8 @@ struct tt_args {
     int64_t out_stride;
     int out_f16;                                   // partial sums as fp16 (not with direct)
     int rt0;                                       // first row tile of this launch (RT counts from there)
+    const uint8_t *packed2;                        // the residual stage's stream of a stacked layer (kernels with R2 > 0)
+    float rs2;                                     // and its scale
 };
 
 // Several layers that share the activations' shape (fused q/k/v, gate/up: glq_vllm/linear_method.py:664-710) in
@@ -95,8 +97,7 @@ __device__ __forceinline__ void tt_barrier() {     // waits for LDS only: global
 // first (the dequantizer's rounding), written in operand layout (lane L's 16 bytes at slot L of operand
 // kpi * 8 + unit * 4 + 2 ms + rh).  half = -1: both operands; 0 / 1: operand rh = half only.
 template <int R>
-__device__ __forceinline__ void tt_emit(const tr_record<R> &r, int unit, int kpi, int ms, int next1, int next2, int lane,
-                                        u32x4 *dst, int half = -1) {
+__device__ __forceinline__ void tt_decode(const tr_record<R> &r, int ms, int next1, int next2, u32x4 (&af)[2], int half) {
     uint32_t c0 = ms ? r.c[1] : r.c[0], c1 = ms ? r.c[3] : r.c[2];
     uint32_t n0, n1;
     if constexpr (R >= 2) {
@@ -123,15 +124,45 @@ __device__ __forceinline__ void tt_emit(const tr_record<R> &r, int unit, int kpi
     for (int rh = 0; rh < 2; ++rh) {
         if (half >= 0 && rh != half) continue;
         const int j0 = 2 * rh;
-        const u32x4 af = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1], h1[j0 + 4],
-                                   h1[j0 + 5]);
-        dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af;
+        af[rh] = pair_sum4(h0[j0], h0[j0 + 1], h0[j0 + 4], h0[j0 + 5], h1[j0], h1[j0 + 1], h1[j0 + 4], h1[j0 + 5]);
     }
 }
 
-template <int R, int NTW, int MODE>
+template <int R>
+__device__ __forceinline__ void tt_emit(const tr_record<R> &r, int unit, int kpi, int ms, int next1, int next2, int lane,
+                                        u32x4 *dst, int half = -1) {
+    u32x4 af[2];
+    tt_decode<R>(r, ms, next1, next2, af, half);
+#pragma unroll
+    for (int rh = 0; rh < 2; ++rh)
+        if (half < 0 || rh == half) dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = af[rh];
+}
+
+// A stacked layer (glq/trellis.py:923-933: W = W1 + inv_resid_scale2 * W2): both stages' weights of the operand,
+// combined in fp32 and rounded to fp16 once -- the weight of the reference's many-token route, which adds the
+// decompressed stages into one fp16 matrix before its GEMM (glq/csrc/glq_trellis.cu:1322-1334,
+// glq/quantized_linear.py:986-1010) -- so the products of a stacked layer are those of a single one.
+template <int R, int R2>
+__device__ __forceinline__ void tt_emit2(const tr_record<R> &r, const tr_record<R2> &rb, float rs2, int unit, int kpi,
+                                         int ms, int next1, int next2, int lane, u32x4 *dst, int half = -1) {
+    u32x4 af[2], bf[2];
+    tt_decode<R>(r, ms, next1, next2, af, half);
+    tt_decode<R2>(rb, ms, next1, next2, bf, half);
+#pragma unroll
+    for (int rh = 0; rh < 2; ++rh) {
+        if (half >= 0 && rh != half) continue;
+        const f16x8 x = __builtin_bit_cast(f16x8, af[rh]), y = __builtin_bit_cast(f16x8, bf[rh]);
+        f16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (f16)((float)x[e] + rs2 * (float)y[e]);
+        dst[(kpi * TT_FRAGS + unit * 4 + 2 * ms + rh) * GLQH_WAVE + lane] = __builtin_bit_cast(u32x4, o);
+    }
+}
+
+template <int R, int NTW, int MODE, int R2 = 0>
 __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g, const tt_moe &mo) {
     constexpr bool GROUP = MODE == TT_GROUP, MOE = MODE == TT_MOE;
+    constexpr int RB = R2 > 0 ? R2 : 1, REC2 = 4 * RB;
     extern __shared__ u32x4 abuf[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
@@ -187,8 +218,15 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
-        auto emit = [&](const tr_record<R> &r, u32x4 *dst, int half = -1) {
-            tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst, half);
+        const uint8_t *rec_base2 = R2 > 0 ? a.packed2 + ((int64_t)mp * nkp * 32 + l) * REC2 + (int64_t)kpi * 32 * REC2 : nullptr;
+        auto load_rec2 = [&](int d) {
+            tr_record<RB> r = {};
+            if constexpr (R2 > 0) r = tr_load_record<RB>(rec_base2 + (int64_t)min(d, ds1 - 1) * 64 * REC2);
+            return r;
+        };
+        auto emit = [&](const tr_record<R> &r, const tr_record<RB> &rb, u32x4 *dst, int half = -1) {
+            if constexpr (R2 > 0) tt_emit2<R, RB>(r, rb, a.rs2, unit, kpi, ms, next1, next2, lane, dst, half);
+            else tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst, half);
         };
         // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(kp * Mp + token) * 4 + q]
         // (the token dimension of xb is padded to whole tiles: no clamping, constant offsets)
@@ -212,10 +250,12 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             for (int tt = 0; tt < NTW; ++tt) dst[tt] = *(const u32x4 *)(xrow + (2 * d + (hidx & 1)) * bstep + tt * 512);
         };
         tr_record<R> rc = load_rec(ds0);
+        tr_record<RB> rcb = load_rec2(ds0);
         load_half(bs[0], 0);
         load_half(bs[1], 1);
         tr_record<R> r1 = load_rec(ds0 + 1), r2 = load_rec(ds0 + 2);
-        emit(rc, abuf);
+        tr_record<RB> r1b = load_rec2(ds0 + 1), r2b = load_rec2(ds0 + 2);
+        emit(rc, rcb, abuf);
         tt_barrier();
         for (int d0 = ds0; d0 < ds1; d0 += 3) {
 #pragma unroll
@@ -226,9 +266,10 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             const u32x4 *rd = abuf + par * TT_BUF;
             u32x4 *wr = abuf + (par ^ 1) * TT_BUF;
             const tr_record<R> r3 = load_rec(d + 3);
+            const tr_record<RB> r3b = load_rec2(d + 3);
             if (MOE && !active) {                               // no positions of the run left for this wave
-                emit(r1, wr, 0);
-                emit(r1, wr, 1);
+                emit(r1, r1b, wr, 0);
+                emit(r1, r1b, wr, 1);
             } else {
             f16x8 ring[2];
             ring[0] = __builtin_bit_cast(f16x8, rd[lane]);
@@ -247,13 +288,15 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
                 for (int tt = 0; tt < NTW; ++tt)
                     acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                         af, __builtin_bit_cast(f16x8, bs[(2 * j + u) % 3][tt]), acc[f][tt], 0, 0, 0);
-                if (kk == 1) emit(r1, wr, 0);
-                if (kk == TT_FRAGS + 1) emit(r1, wr, 1);
+                if (kk == 1) emit(r1, r1b, wr, 0);
+                if (kk == TT_FRAGS + 1) emit(r1, r1b, wr, 1);
             }
             }
             tt_barrier();                                       // rd has been read, wr is written
             r1 = r2;
             r2 = r3;
+            r1b = r2b;
+            r2b = r3b;
           }
         }
         // Lane (i, q) holds four consecutive rows of token i for every (operand, token tile): operand
@@ -324,6 +367,13 @@ tr_tile_kernel(const tt_args a) {
     tr_tile_body<R, NTW, TT_PLAIN>(a, tt_group{}, tt_moe{});
 }
 
+// a stacked layer (first stage 4 bits/weight): both streams decoded into one operand
+template <int R2, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_rvq_kernel(const tt_args a) {
+    tr_tile_body<4, NTW, TT_PLAIN, R2>(a, tt_group{}, tt_moe{});
+}
+
 template <int R, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_group_kernel(const tt_args a, const tt_group g) {
@@ -371,10 +421,11 @@ tr_moe_tiles_kernel(const int *__restrict__ offs, int n_experts, int tile_tok, i
 // block pair w >> 2, k-pair (w >> 1) & 1, m-tile w & 1).  Same K slots and order of summation as above.
 constexpr size_t TT_SMALL_LDS = (size_t)8 * TT_BUF * 16;       // 128 KB
 
-template <int R, int TG, int NTW>
+template <int R, int TG, int NTW, int R2 = 0>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_small_kernel(const tt_args a) {
     constexpr int RG = TT_FRAGS / TG;                          // operand groups
+    constexpr int RB = R2 > 0 ? R2 : 1, REC2 = 4 * RB;         // R2 > 0: a stacked layer, both streams into one operand
     extern __shared__ u32x4 abuf[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
@@ -400,7 +451,16 @@ tr_tile_small_kernel(const tt_args a) {
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
-        auto emit = [&](const tr_record<R> r, u32x4 *dst) { tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst); };
+        const uint8_t *rec_base2 = R2 > 0 ? a.packed2 + ((int64_t)mp * nkp * 32 + l) * REC2 + (int64_t)kpi * 32 * REC2 : nullptr;
+        auto load_rec2 = [&](int d) {
+            tr_record<RB> r = {};
+            if constexpr (R2 > 0) r = tr_load_record<RB>(rec_base2 + (int64_t)min(d, ds1 - 1) * 64 * REC2);
+            return r;
+        };
+        auto emit = [&](const tr_record<R> r, const tr_record<RB> rb, u32x4 *dst) {
+            if constexpr (R2 > 0) tt_emit2<R, RB>(r, rb, a.rs2, unit, kpi, ms, next1, next2, lane, dst);
+            else tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst);
+        };
         // multiply role: token 16 * tt + i of the wave's token group
         const int64_t bstep = (int64_t)a.Mp * 32;               // elements from one k-pair to the next
         const f16 *xrow = a.xb + (int64_t)(16 * NTW * tg + i) * 32 + q * 8;
@@ -422,16 +482,17 @@ tr_tile_small_kernel(const tt_args a) {
         // records of a group arrive a group ahead, activations three steps ahead (a step is a few hundred
         // cycles, less than an L2 round trip)
         tr_record<R> rc[4], rn[4];
+        tr_record<RB> rcb[4], rnb[4];
         u32x4 b[4][NTW][2];
 #pragma unroll
-        for (int dd = 0; dd < 4; ++dd) rc[dd] = load_rec(ds0 + dd);
+        for (int dd = 0; dd < 4; ++dd) { rc[dd] = load_rec(ds0 + dd); rcb[dd] = load_rec2(ds0 + dd); }
 #pragma unroll
         for (int j = 0; j < 3; ++j) load_b(b[j], ds0 + j);
 #pragma unroll
-        for (int dd = 0; dd < 4; ++dd) rn[dd] = load_rec(ds0 + 4 + dd);
+        for (int dd = 0; dd < 4; ++dd) { rn[dd] = load_rec(ds0 + 4 + dd); rnb[dd] = load_rec2(ds0 + 4 + dd); }
         if (item != (int)blockIdx.x) tt_barrier();              // the previous item's last buffer has been read
 #pragma unroll
-        for (int dd = 0; dd < 4; ++dd) emit(rc[dd], abuf + dd * TT_BUF);
+        for (int dd = 0; dd < 4; ++dd) emit(rc[dd], rcb[dd], abuf + dd * TT_BUF);
         tt_barrier();
         for (int qd = 0; qd < nquads; qd += 2) {
 #pragma unroll
@@ -444,6 +505,8 @@ tr_tile_small_kernel(const tt_args a) {
                     for (int dd = 0; dd < 4; ++dd) {
                         rc[dd] = rn[dd];
                         rn[dd] = load_rec(d0 + 8 + dd);
+                        rcb[dd] = rnb[dd];
+                        rnb[dd] = load_rec2(d0 + 8 + dd);
                     }
 #pragma unroll
                     for (int dd = 0; dd < 4; ++dd) {
@@ -456,7 +519,7 @@ tr_tile_small_kernel(const tt_args a) {
 #pragma unroll
                         for (int kk = 0; kk < PF; ++kk) ring[kk] = frag(kk);
                         load_b(b[(dd + 3) & 3], d0 + dd + 3);
-                        emit(rc[dd], wr + dd * TT_BUF);         // operands of the next group (unused after the last)
+                        emit(rc[dd], rcb[dd], wr + dd * TT_BUF);   // operands of the next group (unused after the last)
                         if (d0 + dd < ds1) {                    // uniform: a slot need not be whole groups
 #pragma unroll
                             for (int kk = 0; kk < NK; ++kk) {
@@ -609,8 +672,10 @@ double tt_plan_cost(const tt_plan &p, int64_t m, int64_t M, int esz) {
 // 60 cases, 25 % off at worst (14336 x 2048 at 512 tokens, a gain it misses), 3 % below 512-token tiles everywhere
 // in total; the seven linears of a 3B-shape layer: 505 -> 444 us at 1024 tokens.  GLQ_TT_NTW forces a tile
 // above 256 tokens.
-void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p) {
-    const int top = tt_ntw(M);
+// max_ntw = 2: a stacked layer decoded into one operand (two streams' records and temporaries do not fit beside the
+// accumulators of a 512-token tile).
+void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p, int max_ntw = 4) {
+    const int top = std::min(tt_ntw(M), max_ntw);
     tt_plan_for(top, m, k, M, p);
     static const bool forced = getenv("GLQ_TT_NTW") != nullptr;
     if (top < 4 || forced) return;
@@ -625,6 +690,17 @@ template <int R, int NTW>
 int tt_launch(const tt_plan &p, const tt_args &a, hipStream_t stream) {
     hipLaunchKernelGGL((tr_tile_kernel<R, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a);
     GLQH_LAUNCH_CHECK("trellis tile launch");
+    return 0;
+}
+
+template <int R2>
+int tt_launch_rvq(const tt_plan &p, const tt_args &a, hipStream_t stream) {
+    const dim3 grid((unsigned)p.grid), block(TT_THREADS);
+    if (a.M <= 32) hipLaunchKernelGGL((tr_tile_small_kernel<4, 2, 1, R2>), grid, block, TT_SMALL_LDS, stream, a);
+    else if (a.M <= 64) hipLaunchKernelGGL((tr_tile_small_kernel<4, 4, 1, R2>), grid, block, TT_SMALL_LDS, stream, a);
+    else if (p.NTW == 1) hipLaunchKernelGGL((tr_tile_rvq_kernel<R2, 1>), grid, block, TT_LDS, stream, a);
+    else hipLaunchKernelGGL((tr_tile_rvq_kernel<R2, 2>), grid, block, TT_LDS, stream, a);
+    GLQH_LAUNCH_CHECK("trellis two-stage tile launch");
     return 0;
 }
 
@@ -658,6 +734,8 @@ int tt_init_R() {
     return tt_set_lds(tr_tile_small_kernel<R, 2, 1>) || tt_set_lds(tr_tile_small_kernel<R, 4, 1>) ||
            tt_set_lds(tr_tile_kernel<R, 1>) || tt_set_lds(tr_tile_kernel<R, 2>) || tt_set_lds(tr_tile_kernel<R, 4>) ||
            tt_set_lds(tr_tile_group_kernel<R, 1>) || tt_set_lds(tr_tile_group_kernel<R, 2>) ||
+           tt_set_lds(tr_tile_small_kernel<4, 2, 1, R>) || tt_set_lds(tr_tile_small_kernel<4, 4, 1, R>) ||
+           tt_set_lds(tr_tile_rvq_kernel<R, 1>) || tt_set_lds(tr_tile_rvq_kernel<R, 2>) ||
            tt_set_lds(tr_tile_group_kernel<R, 4>) || tt_set_lds(tr_tile_moe_kernel<R, 1>) ||
            tt_set_lds(tr_tile_moe_kernel<R, 2>) || tt_set_lds(tr_tile_moe_kernel<R, 4>);
 }
@@ -670,9 +748,9 @@ int glqh_trellis_tile_init(void) { return tt_init_R<1>() || tt_init_R<2>() || tt
 size_t glqh_trellis_tile_xb_bytes(int64_t k, int64_t M) { return (size_t)tt_padded_tokens(M) * k * sizeof(f16); }
 
 // K slots the many-token kernel uses for this call (1: it can write the result in place)
-int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M) {
+int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M, int two_stage) {
     tt_plan p;
-    tt_make_plan(m, k, M, &p);
+    tt_make_plan(m, k, M, &p, two_stage ? 2 : 4);
     return p.KS;
 }
 
@@ -682,11 +760,15 @@ int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M) {
 // tokens of the blocked activation layout: M padded to whole workgroup tiles
 int64_t glqh_trellis_tile_padded_tokens(int64_t M) { return tt_padded_tokens(M); }
 
+// packed2 (with R2, rs2): the residual stage of a stacked layer whose first stage has 4 bits/weight; both streams are
+// decoded into one operand, W = fp16(W1 + rs2 * W2), in tiles of at most 256 tokens
+// (glqh_trellis_tile_ksplit(.., two_stage = 1) gives the K slots).
 int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *packed, int R, int64_t m,
                              int64_t k, float *out, int direct, float scale, int accum, int64_t out_stride,
-                             hipStream_t stream, int out_f16) {
+                             hipStream_t stream, int out_f16, const void *packed2, int R2, float rs2) {
+    if (packed2 && R != 4) return glqh_fail("trellis tile kernel: two streams in one operand need a first stage of 4 bits/weight");
     tt_plan p;
-    tt_make_plan(m, k, M, &p);
+    tt_make_plan(m, k, M, &p, packed2 ? 2 : 4);
     if (direct && p.KS != 1) return glqh_fail("trellis tile kernel: in-place output needs a single K slot");
     if (out_f16 && (direct || M <= 64)) return glqh_fail("trellis tile kernel: fp16 sums are partial sums of the large tiles");
     const int Mp = (int)tt_padded_tokens(M);
@@ -714,6 +796,17 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     a.out_stride = out_stride;
     a.out_f16 = out_f16;
     a.rt0 = 0;
+    a.packed2 = (const uint8_t *)packed2;
+    a.rs2 = rs2;
+    if (packed2) {
+        switch (R2) {
+        case 1: return tt_launch_rvq<1>(p, a, stream);
+        case 2: return tt_launch_rvq<2>(p, a, stream);
+        case 3: return tt_launch_rvq<3>(p, a, stream);
+        case 4: return tt_launch_rvq<4>(p, a, stream);
+        }
+        return glqh_fail("trellis tile kernel: second stage of 1-4 bits/weight, got %d", R2);
+    }
     // The last round of tiles: when the 512-token tiles fill at most half of the CUs in their last round,
     // the row tiles of that remainder go to a second launch as 256-token tiles, twice as many, each a good
     // half of the time (14336 rows at 4096 tokens: 896 tiles on 256 CUs = 3.5 rounds -> 3 rounds of 96 row

@@ -1079,12 +1079,13 @@ int glqh_launch_trellis_pack_moe(const void *x_f16, void *xb, const int *perm, c
                                  int n_experts, int x_div, int64_t k, hipStream_t stream);
 int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t stride_bytes, int R, const int *perm,
                                  const void *tiles, const int *n_tiles, const float *pscale_dev, int n_slots,
-                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream);
+                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream,
+                                 const void *packed2 = nullptr, int64_t stride2_bytes = 0, int R2 = 0);
 
 struct moe_plan {
     int R1, R2, S, ks, ks_all;
     int tile;                                                  // the tile kernel's form: one K slot, fp16 sums
-    int fuse2;                                                 // per-slot form, two stages in one launch: ks slots
+    int fuse2;                                                 // per-slot and tile forms, two stages in one launch: ks slots
     size_t part_bytes;
 };
 
@@ -1167,7 +1168,8 @@ static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, int64_t n_expe
         GLQH_REQUIRE(glqh_trellis_mma_fusein_plan((w->m_pad / 64) * n_slots, w->n_pad, 1, &p->S, &p->ks),
                      "routed experts %s: no plan", what);
     }
-    p->fuse2 = p->R2 && p->R1 == 4 && !p->tile && n_slots < moe_group_min(n_experts) && tr_fuse_stages_enabled();
+    // both stages in one launch: the per-slot form (sums added in fp32) and the tile form (one fp16 operand)
+    p->fuse2 = p->R2 && p->R1 == 4 && (p->tile || n_slots < moe_group_min(n_experts)) && tr_fuse_stages_enabled();
     p->ks_all = p->R2 && !p->fuse2 ? 2 * p->ks : p->ks;
     p->part_bytes = align256((size_t)p->ks_all * n_slots * w->m_pad * sizeof(float));
     return 0;
@@ -1250,6 +1252,10 @@ static int moe_decode_tile(const glqh_moe_proj *w, const moe_plan &p, const int 
             return 1;
         if (glqh_launch_trellis_pack_moe(xhat, xb, perm, offs, n_slots, n_experts, x_div, w->n_pad, st)) return 1;
     }
+    if (p.fuse2)                                               // both streams of a stacked expert into one operand
+        return glqh_launch_trellis_tile_moe(xb, w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, tiles, n_tiles,
+                                            w->inv_rs2_dev, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st, w->packed2,
+                                            w->packed_rows * w->packed2_cols * 2, p.R2);
     if (glqh_launch_trellis_tile_moe(xb, w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, tiles, n_tiles,
                                      nullptr, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st))
         return 1;

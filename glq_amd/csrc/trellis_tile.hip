@@ -80,6 +80,7 @@ struct tt_group {
 // scale) if there is one.
 struct tt_moe {
     int64_t stride_bytes;                          // expert e's stream at packed + e * stride_bytes
+    int64_t stride2_bytes;                         // and its residual stream at packed2 + e * stride2_bytes (R2 > 0)
     const int *perm;                               // position in the expert-sorted order -> slot
     const int4 *tiles;                             // (expert, first position, positions, -)
     const int *n_tiles;
@@ -176,7 +177,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
     const int next1 = 16 * (l1 & 3) + 8 * hm + (l1 >> 2), next2 = 16 * (l2 & 3) + 8 * hm + (l2 >> 2);
 
     int nitems = a.TT * a.KS * a.RT;
-    if constexpr (MOE) nitems = *mo.n_tiles * a.RT;             // one K slot
+    if constexpr (MOE) nitems = *mo.n_tiles * a.RT * a.TT;      // one K slot; TT = workgroup tiles per run
     const int per_xcd = (nitems + 7) >> 3;
     const int xcd = blockIdx.x & 7, bx = blockIdx.x >> 3;
     const int nbx = ((int)gridDim.x - xcd + 7) >> 3;
@@ -201,13 +202,25 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         int tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW, limit = a.M;
         float osc = 1.0f;
         bool active = true;                                     // uniform over the wave
+        const uint8_t *lpacked2 = a.packed2;
+        float lrs2 = a.rs2;
         if constexpr (MOE) {
-            const int4 tile = mo.tiles[item / a.RT];
-            if (tile.z <= 0) continue;                          // uniform over the workgroup
+            // a run of the table may be longer than this kernel's tile (a stacked expert's streams are decoded
+            // into one operand in tiles of at most 256 positions): TT workgroup tiles per run, in order
+            constexpr int WG_TOK = TT_WAVES * 16 * NTW;
+            const int4 tile = mo.tiles[item / (a.RT * a.TT)];
+            const int sub = (item / a.RT) % a.TT;
+            const int first = tile.y + sub * WG_TOK, cnt = min(WG_TOK, tile.z - sub * WG_TOK);
+            if (cnt <= 0) continue;                             // uniform over the workgroup
             lpacked = a.packed + tile.x * mo.stride_bytes;
-            tok0 = tile.y + wave * 16 * NTW;
-            limit = tile.y + tile.z;
-            if (mo.pscale_dev) osc = mo.pscale_dev[tile.x];
+            tok0 = first + wave * 16 * NTW;
+            limit = first + cnt;
+            if constexpr (R2 > 0) {
+                lpacked2 = a.packed2 + tile.x * mo.stride2_bytes;
+                lrs2 = mo.pscale_dev[tile.x];
+            } else if (mo.pscale_dev) {
+                osc = mo.pscale_dev[tile.x];
+            }
             active = __builtin_amdgcn_readfirstlane((int)(tok0 < limit)) != 0;
         }
         const int r0 = rt * TT_ROWS;
@@ -218,14 +231,14 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         auto load_rec = [&](int d) {                            // the record of k-pair 2d + kpi
             return tr_load_record<R>(rec_base + (int64_t)min(d, ds1 - 1) * 64 * REC);
         };
-        const uint8_t *rec_base2 = R2 > 0 ? a.packed2 + ((int64_t)mp * nkp * 32 + l) * REC2 + (int64_t)kpi * 32 * REC2 : nullptr;
+        const uint8_t *rec_base2 = R2 > 0 ? lpacked2 + ((int64_t)mp * nkp * 32 + l) * REC2 + (int64_t)kpi * 32 * REC2 : nullptr;
         auto load_rec2 = [&](int d) {
             tr_record<RB> r = {};
             if constexpr (R2 > 0) r = tr_load_record<RB>(rec_base2 + (int64_t)min(d, ds1 - 1) * 64 * REC2);
             return r;
         };
         auto emit = [&](const tr_record<R> &r, const tr_record<RB> &rb, u32x4 *dst, int half = -1) {
-            if constexpr (R2 > 0) tt_emit2<R, RB>(r, rb, a.rs2, unit, kpi, ms, next1, next2, lane, dst, half);
+            if constexpr (R2 > 0) tt_emit2<R, RB>(r, rb, lrs2, unit, kpi, ms, next1, next2, lane, dst, half);
             else tt_emit<R>(r, unit, kpi, ms, next1, next2, lane, dst, half);
         };
         // multiply role: token 16 * tt + i of the wave's tokens; k-pair kp, slot q at xb[(kp * Mp + token) * 4 + q]
@@ -384,6 +397,13 @@ template <int R, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_moe_kernel(const tt_args a, const tt_moe mo) {
     tr_tile_body<R, NTW, TT_MOE>(a, tt_group{}, mo);
+}
+
+// stacked experts (first stage 4 bits/weight): both streams of the run's expert into one operand
+template <int R2, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_moe_rvq_kernel(const tt_args a, const tt_moe mo) {
+    tr_tile_body<4, NTW, TT_MOE, R2>(a, tt_group{}, mo);
 }
 
 // Token tiles of the routed experts: expert e's positions [offs[e], offs[e + 1]) of the sorted order in
@@ -736,6 +756,7 @@ int tt_init_R() {
            tt_set_lds(tr_tile_group_kernel<R, 1>) || tt_set_lds(tr_tile_group_kernel<R, 2>) ||
            tt_set_lds(tr_tile_small_kernel<4, 2, 1, R>) || tt_set_lds(tr_tile_small_kernel<4, 4, 1, R>) ||
            tt_set_lds(tr_tile_rvq_kernel<R, 1>) || tt_set_lds(tr_tile_rvq_kernel<R, 2>) ||
+           tt_set_lds(tr_tile_moe_rvq_kernel<R, 1>) || tt_set_lds(tr_tile_moe_rvq_kernel<R, 2>) ||
            tt_set_lds(tr_tile_group_kernel<R, 4>) || tt_set_lds(tr_tile_moe_kernel<R, 1>) ||
            tt_set_lds(tr_tile_moe_kernel<R, 2>) || tt_set_lds(tr_tile_moe_kernel<R, 4>);
 }
@@ -979,10 +1000,14 @@ int glqh_launch_trellis_pack_moe(const void *x_f16, void *xb, const int *perm, c
 }
 
 // out[slot][row] (fp16 with out_f16) = pscale[expert] * sum over k, for every slot with a valid expert
+// packed2 (with stride2_bytes, R2; R = 4): stacked experts, both streams decoded into one operand with the expert's
+// pscale_dev as the residual scale, W = fp16(W1 + pscale[e] * W2), in workgroup tiles of at most 256 positions.
 int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t stride_bytes, int R, const int *perm,
                                  const void *tiles, const int *n_tiles, const float *pscale_dev, int n_slots,
-                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream) {
+                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream,
+                                 const void *packed2, int64_t stride2_bytes, int R2) {
     const int tile_tok = glqh_trellis_tile_moe_tokens(n_slots, n_experts);
+    if (packed2 && (R != 4 || !pscale_dev)) return glqh_fail("routed experts: two streams in one operand need a 4-bit first stage and the residual scales");
     tt_args a = {};
     a.packed = (const uint8_t *)packed;
     a.xb = (const f16 *)xb;
@@ -991,15 +1016,35 @@ int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t str
     a.m = (int)m;
     a.k = (int)k;
     a.RT = (int)((m + TT_ROWS - 1) / TT_ROWS);
-    a.TT = 0;
+    a.TT = packed2 && tile_tok == 512 ? 2 : 1;                  // workgroup tiles per run of the table
     a.KS = 1;
     a.slot_ds = (int)(k / 64);
     a.out = (float *)out;
     a.out_f16 = out_f16;
-    const tt_moe mo = {stride_bytes, perm, (const int4 *)tiles, n_tiles, pscale_dev};
-    const int64_t max_items = glqh_trellis_tile_moe_max_tiles(n_slots, n_experts) * a.RT;
+    a.packed2 = (const uint8_t *)packed2;
+    const tt_moe mo = {stride_bytes, stride2_bytes, perm, (const int4 *)tiles, n_tiles, pscale_dev};
+    const int64_t max_items = glqh_trellis_tile_moe_max_tiles(n_slots, n_experts) * a.RT * a.TT;
     const int cus = glqh_device_cus();
     const dim3 grid((unsigned)(max_items < cus ? max_items : cus));
+    if (packed2) {
+#define GLQH_TTM2(RR)                                                                                              \
+    do {                                                                                                           \
+        if (tile_tok == 128)                                                                                       \
+            hipLaunchKernelGGL((tr_tile_moe_rvq_kernel<RR, 1>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);     \
+        else                                                                                                       \
+            hipLaunchKernelGGL((tr_tile_moe_rvq_kernel<RR, 2>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);     \
+    } while (0)
+        switch (R2) {
+        case 1: GLQH_TTM2(1); break;
+        case 2: GLQH_TTM2(2); break;
+        case 3: GLQH_TTM2(3); break;
+        case 4: GLQH_TTM2(4); break;
+        default: return glqh_fail("routed experts: second stage of 1-4 bits/weight, got %d", R2);
+        }
+#undef GLQH_TTM2
+        GLQH_LAUNCH_CHECK("routed-expert two-stage tile launch");
+        return 0;
+    }
 #define GLQH_TTM(RR)                                                                                          \
     do {                                                                                                      \
         if (tile_tok == 128)                                                                                  \

@@ -72,7 +72,7 @@ int64_t glqh_trellis_tile_padded_tokens(int64_t M);
 int glqh_trellis_tile_group_ksplit(const int64_t *m, int n_layers, int64_t k, int64_t M);
 int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void *const packed[], int R,
                                    const int64_t m[], int n_layers, int64_t k, float *const out[], int out_f16,
-                                   hipStream_t stream);
+                                   hipStream_t stream, const float f16_scale[] = nullptr);
 int glqh_launch_trellis_pack(const void *x_f16, void *xb, int64_t M, int64_t k, hipStream_t stream);
 int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages);
 // input transform straight into a tile kernel's operand layout (fht.hip); -1 = not eligible, nothing launched
@@ -114,9 +114,12 @@ static tr_plan tr_plain_plan(int64_t m, int64_t k, int64_t B) {
 // stage stored pre-scaled is just more K slots to whoever sums them.  xb: scratch of
 // plan.xb_bytes for the tile kernel (unused otherwise).
 static int tr_plain_partial(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
-                            int64_t k, float *part, void *xb, hipStream_t st, float pscale = 1.0f, int f16_sums = 0) {
+                            int64_t k, float *part, void *xb, hipStream_t st, float pscale = 1.0f, int f16_sums = 0,
+                            float f16_scale = 1.0f) {
     glqh_range range("dequant_matmul");
-    if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, part, 0, 1.0f, 0, 0, st, f16_sums);
+    // fp16 sums leave the tile kernel times f16_scale (the layer's scale: a long row of large activations then stays
+    // inside the fp16 range wherever the layer's output does)
+    if (p.tile) return glqh_launch_trellis_tile(x_f16, xb, B, packed, R, m, k, part, 0, f16_sums ? f16_scale : 1.0f, 0, 0, st, f16_sums);
     return glqh_launch_trellis_mma(x_f16, B, packed, R, m, k, p.S, p.ks, part, 0, pscale, 0, 0, st);
 }
 static int tr_plain_direct(tr_plan p, const void *x_f16, int64_t B, const void *packed, int R, int64_t m,
@@ -594,8 +597,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                    glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad);
         if (tile2) {
             glqh_range range("dequant_matmul");
-            if (glqh_launch_trellis_tile(x_in, xb_tile, B, packed, R1, m_pad, n_pad, part1, 0, 1.0f, 0, 0, st, f16_sums,
-                                         packed2, R2, (float)inv_resid_scale2))
+            if (glqh_launch_trellis_tile(x_in, xb_tile, B, packed, R1, m_pad, n_pad, part1, 0, f16_sums ? (float)wscale : 1.0f,
+                                         0, 0, st, f16_sums, packed2, R2, (float)inv_resid_scale2))
                 return 1;
             two_parts = merge2 = false;
         } else if (has_s2 && !plan.tile && R1 == 4 && tr_fuse_stages_enabled()) {
@@ -606,8 +609,11 @@ extern "C" int glqh_fused_linear_trellis_3inst(
                 return 1;
             two_parts = merge2 = false;
         } else {
-            if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st, 1.0f, f16_sums)) return 1;
-            if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2, f16_sums)) return 1;
+            if (tr_plain_partial(plan, x_in, B, packed, R1, m_pad, n_pad, part1, xb_tile, st, 1.0f, f16_sums, (float)wscale))
+                return 1;
+            if (has_s2 && tr_plain_partial(plan, x_in, B, packed2, R2, m_pad, n_pad, part2, xb_tile, st, ps2, f16_sums,
+                                           (float)(wscale * inv_resid_scale2)))
+                return 1;
         }
     }
 
@@ -636,8 +642,8 @@ extern "C" int glqh_fused_linear_trellis_3inst(
     src.part_kstride = B * m_pad;
     src.ksplit = ks;
     src.part_f16 = f16_sums;
-    src.scale[0] = s1;
-    src.scale[1] = s2;
+    src.scale[0] = f16_sums ? 1.0f : s1;                       // fp16 sums carry their scales already
+    src.scale[1] = f16_sums ? 1.0f : s2;
     src.copy_out = y_rht_out;
     src.copy_stride = y_rht_stride;
     return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,
@@ -809,7 +815,9 @@ static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B
         parts[i] = (float *)(pbase + poff);
         poff += align256((size_t)ks * B * m_pads[i] * esz);
     }
-    if (glqh_launch_trellis_tile_group(xb, B, packed, R, m_pads, n_shards, n_pad, parts, f16_sums ? 1 : 0, st)) return 1;
+    float wscales[TR_GROUP_MANY_MAX];                          // fp16 sums carry the layer's scale already
+    for (int i = 0; i < n_shards; ++i) wscales[i] = (float)shards[i].wscale;
+    if (glqh_launch_trellis_tile_group(xb, B, packed, R, m_pads, n_shards, n_pad, parts, f16_sums ? 1 : 0, st, wscales)) return 1;
     for (int i = 0; i < n_shards; ++i) {
         const glqh_trellis_shard &sh = shards[i];
         glqh_ysrc src = {};
@@ -818,7 +826,7 @@ static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B
         src.part_kstride = B * sh.m_pad;
         src.ksplit = ks;
         src.part_f16 = f16_sums;
-        src.scale[0] = (float)sh.wscale;
+        src.scale[0] = f16_sums ? 1.0f : (float)sh.wscale;
         const int64_t ys = y_stride > 0 ? y_stride : sh.out_features;   // y_stride 0: every layer's rows packed
         int rc = glqh_launch_output_rht_canon_wide(src, sh.su_f16, sh.y, y_dtype, ys, B, sh.out_features, sh.m_pad, st);
         if (rc > 0) return 1;
@@ -1064,10 +1072,12 @@ int glqh_moe_route_segments(int n_slots, int n_experts);
 size_t glqh_moe_route_scratch_ints(int n_slots, int n_experts);
 int glqh_launch_moe_route(const int64_t *topk_ids, int n_slots, int n_experts, int *perm, int *pexp, int *offs,
                           int *scratch, hipStream_t stream);
+int glqh_moe_grouped_wide(int n_slots, int n_experts);
 int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes, int R, const int *perm,
                                         const int *offs, int n_slots, int n_experts, int x_div,
                                         const float *pscale_dev, const void *x_f16, int64_t m, int64_t k, int S,
-                                        int ksplit, float *part, hipStream_t stream);
+                                        int ksplit, float *part, hipStream_t stream, const void *packed2 = nullptr,
+                                        int64_t stride2_bytes = 0, int R2 = 0);
 
 // many rows per expert: the tile kernel on the expert-sorted slots (trellis_tile.hip)
 int glqh_trellis_tile_moe_tokens(int64_t n_slots, int64_t n_experts);
@@ -1078,14 +1088,14 @@ int glqh_launch_trellis_tile_moe_table(const int *offs, int n_slots, int n_exper
 int glqh_launch_trellis_pack_moe(const void *x_f16, void *xb, const int *perm, const int *offs, int n_slots,
                                  int n_experts, int x_div, int64_t k, hipStream_t stream);
 int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t stride_bytes, int R, const int *perm,
-                                 const void *tiles, const int *n_tiles, const float *pscale_dev, int n_slots,
-                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream,
-                                 const void *packed2 = nullptr, int64_t stride2_bytes = 0, int R2 = 0);
+                                 const void *tiles, const int *n_tiles, const float *pscale_dev, const float *wscale_dev,
+                                 int n_slots, int n_experts, int64_t m, int64_t k, void *out, int out_f16,
+                                 hipStream_t stream, const void *packed2 = nullptr, int64_t stride2_bytes = 0, int R2 = 0);
 
 struct moe_plan {
     int R1, R2, S, ks, ks_all;
     int tile;                                                  // the tile kernel's form: one K slot, fp16 sums
-    int fuse2;                                                 // per-slot and tile forms, two stages in one launch: ks slots
+    int fuse2;                                                 // two stages in one launch: ks slots (first stage 4 bits/weight)
     size_t part_bytes;
 };
 
@@ -1168,8 +1178,10 @@ static int moe_proj_plan(const glqh_moe_proj *w, int64_t n_slots, int64_t n_expe
         GLQH_REQUIRE(glqh_trellis_mma_fusein_plan((w->m_pad / 64) * n_slots, w->n_pad, 1, &p->S, &p->ks),
                      "routed experts %s: no plan", what);
     }
-    // both stages in one launch: the per-slot form (sums added in fp32) and the tile form (one fp16 operand)
-    p->fuse2 = p->R2 && p->R1 == 4 && (p->tile || n_slots < moe_group_min(n_experts)) && tr_fuse_stages_enabled();
+    // both stages in one launch: the per-slot form and the grouped form's passes of 16 rows add the sums in fp32, the
+    // tile form multiplies with one fp16 operand; the grouped form's passes of up to 64 rows keep a launch per stage
+    p->fuse2 = p->R2 && p->R1 == 4 && tr_fuse_stages_enabled() &&
+               (p->tile || n_slots < moe_group_min(n_experts) || !glqh_moe_grouped_wide((int)n_slots, (int)n_experts));
     p->ks_all = p->R2 && !p->fuse2 ? 2 * p->ks : p->ks;
     p->part_bytes = align256((size_t)p->ks_all * n_slots * w->m_pad * sizeof(float));
     return 0;
@@ -1230,6 +1242,10 @@ static int moe_decode_grouped(const glqh_moe_proj *w, const moe_plan &p, const i
     if (x && glqh_launch_input_rht(x, x_dtype, x_stride, w->sv_f16, xhat, GLQH_F16, x_rows, w->in_features, w->n_pad,
                                    w->bn_meta_dev, w->blocks_n, w->n_blocks_n, 0.0f, st))
         return 1;
+    if (p.fuse2)                                               // both streams of stacked experts in the same passes
+        return glqh_launch_trellis_mma_moe_grouped(w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, offs, n_slots,
+                                                   n_experts, x_div, w->inv_rs2_dev, xhat, w->m_pad, w->n_pad, p.S, p.ks,
+                                                   part, st, w->packed2, w->packed_rows * w->packed2_cols * 2, p.R2);
     if (glqh_launch_trellis_mma_moe_grouped(w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, offs, n_slots,
                                             n_experts, x_div, nullptr, xhat, w->m_pad, w->n_pad, p.S, p.ks, part, st))
         return 1;
@@ -1242,7 +1258,7 @@ static int moe_decode_grouped(const glqh_moe_proj *w, const moe_plan &p, const i
 }
 
 // one projection through the tile kernel: input transform of the rows, their packed copy in sorted order, one
-// launch per stage into fp16 sums [stage][slot][row] (the second stage's already times its scale)
+// launch per stage into fp16 sums [stage][slot][row], times the expert's scale (and the second stage's)
 static int moe_decode_tile(const glqh_moe_proj *w, const moe_plan &p, const int *perm, const int *offs, const void *tiles,
                            const int *n_tiles, int n_slots, int n_experts, int x_div, const void *x, int x_dtype,
                            int64_t x_stride, int64_t x_rows, void *xhat, void *xb, float *part, hipStream_t st) {
@@ -1254,13 +1270,13 @@ static int moe_decode_tile(const glqh_moe_proj *w, const moe_plan &p, const int 
     }
     if (p.fuse2)                                               // both streams of a stacked expert into one operand
         return glqh_launch_trellis_tile_moe(xb, w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, tiles, n_tiles,
-                                            w->inv_rs2_dev, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st, w->packed2,
+                                            w->inv_rs2_dev, w->wscale_dev, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st, w->packed2,
                                             w->packed_rows * w->packed2_cols * 2, p.R2);
     if (glqh_launch_trellis_tile_moe(xb, w->packed, w->packed_rows * w->packed_cols * 2, p.R1, perm, tiles, n_tiles,
-                                     nullptr, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st))
+                                     nullptr, w->wscale_dev, n_slots, n_experts, w->m_pad, w->n_pad, part, 1, st))
         return 1;
     if (p.R2 && glqh_launch_trellis_tile_moe(xb, w->packed2, w->packed_rows * w->packed2_cols * 2, p.R2, perm, tiles,
-                                             n_tiles, w->inv_rs2_dev, n_slots, n_experts, w->m_pad, w->n_pad,
+                                             n_tiles, w->inv_rs2_dev, w->wscale_dev, n_slots, n_experts, w->m_pad, w->n_pad,
                                              (f16 *)part + (int64_t)n_slots * w->m_pad, 1, st))
         return 1;
     return 0;

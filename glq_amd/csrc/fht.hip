@@ -902,7 +902,10 @@ struct moe_out_args {
     int out_features, m_pad;
 };
 
+// (fp16 sums -- the tile form's -- carry the expert's scale already: an unscaled sum over a long row of large
+// activations can pass the fp16 range where the scaled one, of the size of the layer's output, does not)
 __device__ __forceinline__ glqh_ysrc moe_src(const moe_out_args &a, float scale) {
+    if (a.part_f16 && scale != 0.0f) scale = 1.0f;
     glqh_ysrc src = {};
     src.part = a.part;
     src.part_kstride = (int64_t)a.n_slots * a.m_pad;

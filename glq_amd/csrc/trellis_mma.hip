@@ -608,6 +608,8 @@ tr_mma_fusein_moe_rvq_kernel(tr_moe_args g, const uint8_t *__restrict__ packed2,
 struct tr_moe_group_args {
     const uint8_t *packed;
     int64_t stride_bytes;
+    const uint8_t *packed2;                      // residual streams of stacked experts (kernels with R2 > 0): pscale_dev
+    int64_t stride2_bytes;                       // is then their scale, applied to the second stream's sums
     const int *perm, *offs;
     const float *pscale_dev;
     float *part;                                 // [K slot][slot][row]
@@ -615,13 +617,14 @@ struct tr_moe_group_args {
 };
 
 // One pass over the K slot for NT tiles of 16 of the expert's rows, positions [t0, t0 + 16 NT) of its run in perm.
-template <int R, int NT>
+template <int R, int NT, int R2 = 0>
 __device__ __forceinline__ void moe_group_pass(const tr_moe_group_args &g, const f16 *__restrict__ x, int m, int k,
                                                int kp0, int kp1, int CH, const uint8_t *lane_base, const mma_lane a,
                                                int wave, int o0, int cnt, int t0, float pscale, int kslot,
-                                               u32x4 *xs_lds, int *slotmap) {
+                                               u32x4 *xs_lds, int *slotmap, const uint8_t *lane_base2 = nullptr) {
     constexpr int TPS = mma_tps<16>();
     constexpr int REC = 4 * R;
+    constexpr int RB = R2 > 0 ? R2 : 1, REC2 = 4 * RB;
     constexpr int G = mma_red_groups<NT>();                      // row groups per round of the final sum
     constexpr int PER_WAVE = G * NT * 256;
     uint32_t *xs = (uint32_t *)xs_lds;
@@ -631,12 +634,16 @@ __device__ __forceinline__ void moe_group_pass(const tr_moe_group_args &g, const
         slotmap[threadIdx.x] = t0 + (int)threadIdx.x < cnt ? g.perm[o0 + t0 + threadIdx.x] : -1;
     int kp = kp0 + wave;
     tr_record<R> cur = {};
-    if (kp < kp1) cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
-    mma_acc<NT> acc;
+    tr_record<RB> curb = {};
+    if (kp < kp1) {
+        cur = tr_load_record<R>(lane_base + (int64_t)kp * 32 * REC);
+        if constexpr (R2 > 0) curb = tr_load_record<RB>(lane_base2 + (int64_t)kp * 32 * REC2);
+    }
+    mma_acc<NT> acc, accb;
 #pragma unroll
     for (int sg = 0; sg < 4; ++sg)
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) acc.v[sg][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < NT; ++tt) acc.v[sg][tt] = accb.v[sg][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int c0 = kp0; c0 < kp1; c0 += CH) {
         const int c1 = min(c0 + CH, kp1), n = c1 - c0;
         fht_barrier<true>();                                     // slotmap written / previous chunk consumed
@@ -657,10 +664,24 @@ __device__ __forceinline__ void moe_group_pass(const tr_moe_group_args &g, const
         fht_barrier<true>();
         for (; kp < c1; kp += TR_WAVES) {
             tr_record<R> nxt = cur;
-            if (kp + TR_WAVES < kp1) nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
-            acc = mma_record<R, 16, NT>(cur, a.next1, a.next2, xs_lds + ((kp - c0) * NT * 8 + a.q) * TPS + a.tokl, acc);
+            tr_record<RB> nxtb = curb;
+            if (kp + TR_WAVES < kp1) {
+                nxt = tr_load_record<R>(lane_base + (int64_t)(kp + TR_WAVES) * 32 * REC);
+                if constexpr (R2 > 0) nxtb = tr_load_record<RB>(lane_base2 + (int64_t)(kp + TR_WAVES) * 32 * REC2);
+            }
+            const u32x4 *xsl = xs_lds + ((kp - c0) * NT * 8 + a.q) * TPS + a.tokl;
+            acc = mma_record<R, 16, NT>(cur, a.next1, a.next2, xsl, acc);
+            if constexpr (R2 > 0) accb = mma_record<RB, 16, NT>(curb, a.next1, a.next2, xsl, accb);
             cur = nxt;
+            curb = nxtb;
         }
+    }
+    if constexpr (R2 > 0) {                                      // pscale is the residual scale here, not a factor of the sum
+#pragma unroll
+        for (int sg = 0; sg < 4; ++sg)
+#pragma unroll
+            for (int tt = 0; tt < NT; ++tt) acc.v[sg][tt] += pscale * accb.v[sg][tt];
+        pscale = 1.0f;
     }
     // the four waves' sums in wave order, G row groups per round, then one row of part per (K slot, slot)
 #pragma unroll
@@ -698,7 +719,7 @@ struct moe_chunks {
 
 // WIDE = false: passes of 16 rows only (few rows per expert: the registers of the wide passes would cost
 // occupancy for nothing).
-template <int R, bool WIDE>
+template <int R, bool WIDE, int R2 = 0>
 __global__ void __launch_bounds__(TR_THREADS)
 tr_mma_moe_grouped_kernel(tr_moe_group_args g, const f16 *__restrict__ x, int m, int k, int S, moe_chunks ch) {
     extern __shared__ u32x4 xs_lds[];
@@ -719,18 +740,21 @@ tr_mma_moe_grouped_kernel(tr_moe_group_args g, const f16 *__restrict__ x, int m,
     const int mp = min(2 * (int)blockIdx.x + a.hm, mpairs - 1);
     constexpr int REC = 4 * R;
     const uint8_t *lane_base = packed + ((int64_t)mp * nkp * 32 + a.l) * REC;
+    constexpr int REC2 = 4 * (R2 > 0 ? R2 : 1);
+    const uint8_t *lane_base2 =
+        R2 > 0 ? g.packed2 + (int64_t)e * g.stride2_bytes + ((int64_t)mp * nkp * 32 + a.l) * REC2 : nullptr;
 
     // The stream is read once per pass: as many of the expert's rows per pass as there are, up to 64.
     for (int t0 = 0; t0 < cnt;) {
         const int rem = WIDE ? cnt - t0 : 0;
         if (rem > 32) {
-            moe_group_pass<R, 4>(g, x, m, k, kp0, kp1, ch.ch4, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap);
+            moe_group_pass<R, 4, R2>(g, x, m, k, kp0, kp1, ch.ch4, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap, lane_base2);
             t0 += 64;
         } else if (rem > 16) {
-            moe_group_pass<R, 2>(g, x, m, k, kp0, kp1, ch.ch2, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap);
+            moe_group_pass<R, 2, R2>(g, x, m, k, kp0, kp1, ch.ch2, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap, lane_base2);
             t0 += 32;
         } else {
-            moe_group_pass<R, 1>(g, x, m, k, kp0, kp1, ch.ch1, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap);
+            moe_group_pass<R, 1, R2>(g, x, m, k, kp0, kp1, ch.ch1, lane_base, a, wave, o0, cnt, t0, pscale, kslot, xs_lds, slotmap, lane_base2);
             t0 += 16;
         }
     }
@@ -820,7 +844,8 @@ int mma_init_R() {
     return mma_set_lds(tr_mma_kernel<R, 1, 1>) || mma_set_lds(tr_mma_kernel<R, 4, 1>) ||
            mma_set_lds(tr_mma_kernel<R, 16, 1>) || mma_set_lds(tr_mma_kernel<R, 16, 2>) ||
            mma_set_lds(tr_mma_kernel<R, 16, 4>) || mma_set_lds(tr_mma_moe_grouped_kernel<R, false>) ||
-           mma_set_lds(tr_mma_moe_grouped_kernel<R, true>) || mma_set_lds(tr_mma_rvq_kernel<R, 1>) ||
+           mma_set_lds(tr_mma_moe_grouped_kernel<R, true>) || mma_set_lds(tr_mma_moe_grouped_kernel<4, false, R>) ||
+           mma_set_lds(tr_mma_rvq_kernel<R, 1>) ||
            mma_set_lds(tr_mma_rvq_kernel<R, 4>) || mma_set_lds(tr_mma_rvq_kernel<R, 16>);
 }
 
@@ -1118,16 +1143,29 @@ static int moe_wide_min_rows() {                                // GLQ_MOE_WIDE_
 }
 
 // One projection of all routed experts, rows grouped by expert: part[K slot][slot][row].
+// 1: the grouped launch of this many slots takes up to 64 rows per pass (an average of GLQ_MOE_WIDE_MIN_ROWS rows
+// per expert, 12 unless set)
+int glqh_moe_grouped_wide(int n_slots, int n_experts) {
+    return (int64_t)n_slots >= (int64_t)moe_wide_min_rows() * n_experts;
+}
+
+// packed2 (with stride2_bytes, R2; R = 4; passes of 16 rows only): stacked experts, both streams in the same passes,
+// the second one's sums times pscale_dev[expert] added in registers.  (With the passes of up to 64 rows the second
+// set of accumulators costs the occupancy: 166 registers, 256 tokens of 6 bpw experts 421 -> 578 us; those keep a
+// launch per stage.)
 int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes, int R, const int *perm,
                                         const int *offs, int n_slots, int n_experts, int x_div,
                                         const float *pscale_dev, const void *x_f16, int64_t m, int64_t k, int S,
-                                        int ksplit, float *part, hipStream_t stream) {
+                                        int ksplit, float *part, hipStream_t stream, const void *packed2,
+                                        int64_t stride2_bytes, int R2) {
     glqh_range range("dequant_matmul");
+    GLQH_REQUIRE(!packed2 || (R == 4 && pscale_dev), "routed experts: two streams per pass need a 4-bit first stage and the residual scales");
     GLQH_REQUIRE(n_experts >= 1 && n_experts <= 65535 && n_slots >= 1 && x_div >= 1,
                  "routed experts: %d experts (1..65535), %d slots", n_experts, n_slots);
     GLQH_REQUIRE(S >= 1 && ksplit >= 1 && (int64_t)S * ksplit >= k / 32, "routed experts: K plan does not cover the row");
     // Wide passes from an average of 12 rows per expert on (a third of the experts then has more than 16).
-    const bool wide = (int64_t)n_slots >= (int64_t)moe_wide_min_rows() * n_experts;
+    const bool wide = glqh_moe_grouped_wide(n_slots, n_experts) != 0;
+    GLQH_REQUIRE(!(packed2 && wide), "routed experts: two streams per pass are served with passes of 16 rows only");
     // chunk of the one-tile pass as in tr_mma_kernel; the wider passes take what the same LDS holds
     moe_chunks ch;
     ch.ch1 = mma_chunk_cap<16, 1>();
@@ -1139,8 +1177,24 @@ int glqh_launch_trellis_mma_moe_grouped(const void *packed, int64_t stride_bytes
     ch.ch4 = std::min(ch.ch4, s4);
     size_t lds = std::max({(size_t)ch.ch1 * mma_slot_bytes(16, 1), (size_t)ch.ch2 * mma_slot_bytes(16, 2),
                            (size_t)ch.ch4 * mma_slot_bytes(16, 4), (size_t)mma_red_bytes<16, 4>()});
-    tr_moe_group_args g = {(const uint8_t *)packed, stride_bytes, perm, offs, pscale_dev, part, n_slots, x_div};
+    tr_moe_group_args g = {(const uint8_t *)packed, stride_bytes, (const uint8_t *)packed2, stride2_bytes, perm, offs,
+                           pscale_dev, part, n_slots, x_div};
     const dim3 grid((unsigned)((m + 63) / 64), (unsigned)ksplit, (unsigned)n_experts);
+    if (packed2) {
+#define GLQH_MOEG2(RR)                                                                                          \
+    hipLaunchKernelGGL((tr_mma_moe_grouped_kernel<4, false, RR>), grid, dim3(TR_THREADS), lds, stream, g,        \
+                       (const f16 *)x_f16, (int)m, (int)k, S, ch)
+        switch (R2) {
+        case 1: GLQH_MOEG2(1); break;
+        case 2: GLQH_MOEG2(2); break;
+        case 3: GLQH_MOEG2(3); break;
+        case 4: GLQH_MOEG2(4); break;
+        default: return glqh_fail("routed experts: second stage of 1-4 bits/weight, got %d", R2);
+        }
+#undef GLQH_MOEG2
+        GLQH_LAUNCH_CHECK("trellis grouped routed-expert two-stage launch");
+        return 0;
+    }
 #define GLQH_MOEG(RR)                                                                                        \
     do {                                                                                                     \
         if (wide)                                                                                            \

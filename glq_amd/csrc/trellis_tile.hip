@@ -67,6 +67,7 @@ struct tt_group {
     const f16 *xb[TT_MAX_GROUP];
     float *out[TT_MAX_GROUP];
     int m[TT_MAX_GROUP], rt0[TT_MAX_GROUP];
+    float scale[TT_MAX_GROUP];                     // factor of the layer's fp16 sums (its Wscale)
     int n;
 };
 
@@ -85,6 +86,7 @@ struct tt_moe {
     const int4 *tiles;                             // (expert, first position, positions, -)
     const int *n_tiles;
     const float *pscale_dev;
+    const float *wscale_dev;                       // the expert's scale, applied before the sums are rounded to fp16
 };
 
 enum { TT_PLAIN = 0, TT_GROUP = 1, TT_MOE = 2 };
@@ -190,12 +192,15 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         const uint8_t *lpacked = a.packed;
         const f16 *lxb = a.xb;
         float *lout = a.out;
+        // fp16 sums leave times the layer's scale: an unscaled sum over a long row of large activations can pass
+        // the fp16 range where the scaled one, of the size of the layer's output, does not
+        float f16sc = a.scale;
         if constexpr (GROUP) {
             int first = 0;
-            lm = g.m[0]; lpacked = g.packed[0]; lxb = g.xb[0]; lout = g.out[0];
+            lm = g.m[0]; lpacked = g.packed[0]; lxb = g.xb[0]; lout = g.out[0]; f16sc = g.scale[0];
 #pragma unroll
             for (int j = 1; j < TT_MAX_GROUP; ++j)
-                if (j < g.n && rt >= g.rt0[j]) { first = g.rt0[j]; lm = g.m[j]; lpacked = g.packed[j]; lxb = g.xb[j]; lout = g.out[j]; }
+                if (j < g.n && rt >= g.rt0[j]) { first = g.rt0[j]; lm = g.m[j]; lpacked = g.packed[j]; lxb = g.xb[j]; lout = g.out[j]; f16sc = g.scale[j]; }
             rt -= first;
         }
         const int mpairs = lm >> 5;
@@ -215,11 +220,12 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             lpacked = a.packed + tile.x * mo.stride_bytes;
             tok0 = first + wave * 16 * NTW;
             limit = first + cnt;
+            osc = mo.wscale_dev[tile.x];
             if constexpr (R2 > 0) {
                 lpacked2 = a.packed2 + tile.x * mo.stride2_bytes;
                 lrs2 = mo.pscale_dev[tile.x];
             } else if (mo.pscale_dev) {
-                osc = mo.pscale_dev[tile.x];
+                osc *= mo.pscale_dev[tile.x];
             }
             active = __builtin_amdgcn_readfirstlane((int)(tok0 < limit)) != 0;
         }
@@ -337,6 +343,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
                     f32x4 v0 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl);
                     f32x4 v1 = *(const f32x4 *)(ep + tl * TT_EP_STRIDE + rl + 4);
                     if constexpr (MOE) { v0 *= osc; v1 *= osc; }
+                    else { v0 *= f16sc; v1 *= f16sc; }
                     if (tok >= limit || row >= lm) continue;    // m is a multiple of 32: whole runs of eight
                     if constexpr (MOE) tok = mo.perm[tok];
                     typedef _Float16 f16x8o __attribute__((ext_vector_type(8)));
@@ -775,7 +782,7 @@ int glqh_trellis_tile_ksplit(int64_t m, int64_t k, int64_t M, int two_stage) {
     return p.KS;
 }
 
-// direct == 0: out[(slot * M + token) * m + row] = the slot's partial sum, unscaled;
+// direct == 0: out[(slot * M + token) * m + row] = the slot's partial sum, unscaled (fp32) or times scale (out_f16);
 // direct == 1 (one slot only): out[token * out_stride + row] = (accum ? out : 0) + scale * sum.
 // x_f16 is (M, k) row-major; xb_scratch takes its repacked copy (glqh_trellis_tile_xb_bytes).
 // tokens of the blocked activation layout: M padded to whole workgroup tiles
@@ -905,11 +912,12 @@ int glqh_trellis_tile_group_ksplit(const int64_t *m, int n_layers, int64_t k, in
 }
 
 // Layers l < n_layers (at most 4) of the same width k and bits/weight against the same M > 64 tokens: partial
-// sums out[l][(slot * M + token) * m[l] + row] (fp16 with out_f16), K slots from glqh_trellis_tile_group_ksplit.
+// sums out[l][(slot * M + token) * m[l] + row] (fp16 with out_f16, then times f16_scale[l] if given), K slots from
+// glqh_trellis_tile_group_ksplit.
 // xb[l]: the layer's activations in the blocked layout (glqh_trellis_tile_padded_tokens(M) tokens).
 int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void *const packed[], int R,
                                    const int64_t m[], int n_layers, int64_t k, float *const out[], int out_f16,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, const float f16_scale[]) {
     GLQH_REQUIRE(n_layers >= 1 && n_layers <= TT_MAX_GROUP, "trellis tile group: %d layers (1..%d)", n_layers, TT_MAX_GROUP);
     GLQH_REQUIRE(M > 64, "trellis tile group: more than 64 tokens");
     tt_plan p;
@@ -922,6 +930,7 @@ int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void
         g.packed[l] = (const uint8_t *)packed[l];
         g.xb[l] = (const f16 *)xb[l];
         g.out[l] = out[l];
+        g.scale[l] = out_f16 && f16_scale ? f16_scale[l] : 1.0f;
         g.m[l] = (int)m[l];
         g.rt0[l] = rt;
         rt += (int)((m[l] + TT_ROWS - 1) / TT_ROWS);
@@ -999,13 +1008,14 @@ int glqh_launch_trellis_pack_moe(const void *x_f16, void *xb, const int *perm, c
     return 0;
 }
 
-// out[slot][row] (fp16 with out_f16) = pscale[expert] * sum over k, for every slot with a valid expert
+// out[slot][row] (fp16 with out_f16) = wscale[expert] * pscale[expert] * sum over k, for every slot with a valid expert
 // packed2 (with stride2_bytes, R2; R = 4): stacked experts, both streams decoded into one operand with the expert's
 // pscale_dev as the residual scale, W = fp16(W1 + pscale[e] * W2), in workgroup tiles of at most 256 positions.
 int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t stride_bytes, int R, const int *perm,
-                                 const void *tiles, const int *n_tiles, const float *pscale_dev, int n_slots,
-                                 int n_experts, int64_t m, int64_t k, void *out, int out_f16, hipStream_t stream,
-                                 const void *packed2, int64_t stride2_bytes, int R2) {
+                                 const void *tiles, const int *n_tiles, const float *pscale_dev, const float *wscale_dev,
+                                 int n_slots, int n_experts, int64_t m, int64_t k, void *out, int out_f16,
+                                 hipStream_t stream, const void *packed2, int64_t stride2_bytes, int R2) {
+    if (!wscale_dev) return glqh_fail("routed experts: the tile form needs the experts' scales");
     const int tile_tok = glqh_trellis_tile_moe_tokens(n_slots, n_experts);
     if (packed2 && (R != 4 || !pscale_dev)) return glqh_fail("routed experts: two streams in one operand need a 4-bit first stage and the residual scales");
     tt_args a = {};
@@ -1022,7 +1032,7 @@ int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t str
     a.out = (float *)out;
     a.out_f16 = out_f16;
     a.packed2 = (const uint8_t *)packed2;
-    const tt_moe mo = {stride_bytes, stride2_bytes, perm, (const int4 *)tiles, n_tiles, pscale_dev};
+    const tt_moe mo = {stride_bytes, stride2_bytes, perm, (const int4 *)tiles, n_tiles, pscale_dev, wscale_dev};
     const int64_t max_items = glqh_trellis_tile_moe_max_tiles(n_slots, n_experts) * a.RT * a.TT;
     const int cus = glqh_device_cus();
     const dim3 grid((unsigned)(max_items < cus ? max_items : cus));

@@ -263,6 +263,24 @@ def test_rows_with_a_block_of_8192_points(ext, hidden, inter):
     assert torch.equal(y, ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *a))
 
 
+def test_large_activations_stay_finite_in_the_tile_form(ext):
+    """Squared-ReLU experts on activations of a few units: the second projection's unscaled sums pass the fp16
+    range while the result does not; the tile form's fp16 sums carry the expert's scale, so it stays finite and
+    inside the bound (1500 tokens x 5 choices over 22 experts, two-stage experts, runs of up to 512 positions)."""
+    say("moe large activations")
+    ex = experts(22, 448, 320, 4, 1, seed=9)
+    rng = np.random.default_rng(3)
+    T, K = 1500, 5
+    ids = np.stack([rng.permutation(22)[:K] for _ in range(T)]).astype(np.int64)
+    w = rng.random((T, K)).astype(np.float32)
+    x = torch.from_numpy(rng.standard_normal((T, 448)).astype(np.float32)).bfloat16()
+    ref = ex.oracle(x.float().numpy(), ids, w, 2)
+    assert bool(np.isfinite(ref).all())
+    y = ext.glq_fused_moe_trellis_3inst_cuda(x.to(DEV), t(ids), t(w), *ex.device_args(2))
+    assert bool(torch.isfinite(y.float()).all())
+    assert rel(y, ref) < TOL, rel(y, ref)
+
+
 @pytest.mark.parametrize("group_min,wide_min,tile_min,tile_ntw,fuse", [
     ("1", "1", "0", "", "1"), ("1", "1000000", "0", "", "0"), ("1000000", "12", "0", "", "1"), ("1", "12", "1", "", "1"),
     ("1", "12", "1", "1", "0"), ("1", "12", "1", "4", "1"), ("1000000", "12", "0", "", "0")])

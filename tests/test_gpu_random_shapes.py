@@ -197,3 +197,31 @@ def test_two_stage_layers_with_a_launch_per_stage_in_a_fresh_process():
                        cwd=os.path.dirname(here))
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
     assert " passed" in r.stdout and "no tests ran" not in r.stdout, r.stdout[-500:]
+
+
+def test_large_activations_stay_finite_at_many_tokens():
+    """Activations of a few thousand: the unscaled sum over a row of 2048 columns passes the fp16 range, the
+    layer's output (the sum times Wscale) does not.  The fp16 sums between the tile kernel and the output transform
+    carry the scale, so the many-token path stays finite and inside the bound, one- and two-stage layers alike."""
+    from glq_amd import ext, hadamard as H
+    m, n, B = 1024, 2048, 100
+    say("large activations", m, n, B)
+    su, sv = O.rht_signs(m, n, 5)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    p1, p2 = O.random_packed(m, n, 4, 21), O.random_packed(m, n, 2, 22)
+    W1 = O.decode_layer(p1, m, n, fast=True)
+    W2 = O.decode_layer(p2, m, n, fast=True)
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(1)) * 3000.0).to(torch.bfloat16)
+    meta = (torch.tensor(bn), torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV))
+    svd, sud = t(sv.astype(np.float16)), t(su.astype(np.float16))
+    for W, call in ((W1, lambda: ext.glq_fused_linear_trellis_3inst_cuda(x.to(DEV), svd, sud, t(p1), *meta, 0.02, n, m, n, m,
+                                                                        out_dtype=torch.bfloat16)),
+                    (W1 + np.float32(0.3) * W2,
+                     lambda: ext.glq_fused_linear_trellis_3inst_rvq2_cuda(x.to(DEV), svd, sud, t(p1), t(p2), *meta, 0.02, 0.3,
+                                                                          n, m, n, m, out_dtype=torch.bfloat16))):
+        ref = O.linear_forward_rht(x.float().numpy(), W.astype(np.float32) * np.float32(0.02), su.astype(np.float32),
+                                   sv.astype(np.float32), bn, bm, n, m)
+        assert float(np.abs(ref).max()) < 6.0e4 and float(np.abs(ref).max()) / 0.02 > 7.0e4   # the case is what it claims
+        y = call()
+        assert bool(torch.isfinite(y.float()).all())
+        assert rel(y, ref) < TOL, rel(y, ref)

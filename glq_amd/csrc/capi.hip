@@ -593,8 +593,12 @@ extern "C" int glqh_fused_linear_trellis_3inst(
         // transform.  With several K slots (small layers at a few hundred tokens) every slot's sum is
         // rounded and the transform adds them in fp32 (3B-shape layer at 512 tokens: 413 -> 394 us for
         // its seven linears).  GLQ_TRELLIS_F16_SUMS=0 keeps them fp32.
+        // (the whole-block output transform, the one that reads fp16 sums, stores 16 bytes at a time: rows of y
+        // that do not start on 16 bytes -- out_features not a multiple of 8 -- keep fp32 sums)
+        const int64_t y_esz = y_dtype == GLQH_F32 ? 4 : 2;
         f16_sums = plan.tile && ks <= tr_f16_sums_max_slots() && B > 64 && !y_rht_out && y && tr_f16_sums_enabled() &&
-                   glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad);
+                   glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad) && ((uintptr_t)y & 15) == 0 &&
+                   ((uintptr_t)su_f16 & 15) == 0 && (y_stride * y_esz) % 16 == 0;
         if (tile2) {
             glqh_range range("dequant_matmul");
             if (glqh_launch_trellis_tile(x_in, xb_tile, B, packed, R1, m_pad, n_pad, part1, 0, f16_sums ? (float)wscale : 1.0f,
@@ -789,6 +793,10 @@ static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B
         int64_t top = 1;
         while (top * 2 <= m_pads[i]) top *= 2;
         if (top > 8192 || m_pads[i] % 8 != 0) f16_sums = false;
+        // and rows of y that start on 16 bytes (the whole-block transform stores 16 bytes at a time)
+        const int64_t ys = y_stride > 0 ? y_stride : shards[i].out_features, y_esz = y_dtype == GLQH_F32 ? 4 : 2;
+        if (((uintptr_t)shards[i].y & 15) != 0 || ((uintptr_t)shards[i].su_f16 & 15) != 0 || (ys * y_esz) % 16 != 0)
+            f16_sums = false;
     }
     const size_t esz = f16_sums ? sizeof(f16) : sizeof(float);
     size_t poff = 0;

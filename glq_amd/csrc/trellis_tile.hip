@@ -218,7 +218,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             const int first = tile.y + sub * WG_TOK, cnt = min(WG_TOK, tile.z - sub * WG_TOK);
             if (cnt <= 0) continue;                             // uniform over the workgroup
             lpacked = a.packed + tile.x * mo.stride_bytes;
-            tok0 = first + wave * 16 * NTW;
+            tok0 = first + __builtin_amdgcn_readfirstlane(wave) * 16 * NTW;   // uniform: scalar registers
             limit = first + cnt;
             osc = mo.wscale_dev[tile.x];
             if constexpr (R2 > 0) {

@@ -225,3 +225,27 @@ def test_large_activations_stay_finite_at_many_tokens():
         y = call()
         assert bool(torch.isfinite(y.float()).all())
         assert rel(y, ref) < TOL, rel(y, ref)
+
+
+def test_ragged_out_features_at_many_tokens():
+    """out_features that is not a multiple of 8 (rows of y that do not start on 16 bytes) at more than 64 tokens:
+    the whole-block output transform that reads fp16 sums does not apply, the sums stay fp32; one layer and two
+    layers through the grouped call (the second layer's columns start at an odd offset)."""
+    from glq_amd import ext, hadamard as H
+    m, n, B, out_f = 1856, 2496, 513, 1853
+    say("ragged out_features, many tokens", m, n, B, out_f)
+    su, sv = O.rht_signs(m, n, 8)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    p1 = O.random_packed(m, n, 4, 31)
+    W = O.decode_layer(p1, m, n, fast=True).astype(np.float32)
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(2)) * 0.7).to(torch.bfloat16)
+    ref = O.linear_forward_rht(x.float().numpy(), W * np.float32(0.02), su.astype(np.float32), sv.astype(np.float32), bn, bm, n, m)
+    bnt, bnm = torch.tensor(bn), H.pack_block_meta(bn).to(DEV)
+    svd, sud, pd = t(sv.astype(np.float16)), t(su.astype(np.float16)), t(p1)
+    y = ext.glq_fused_linear_trellis_3inst_cuda(x.to(DEV), svd, sud, pd, bnt, torch.tensor(bm), bnm, H.pack_block_meta(bm).to(DEV),
+                                                0.02, n, out_f, n, m, out_dtype=torch.bfloat16)
+    assert y.shape == (B, out_f) and rel(y, ref[:, :out_f]) < TOL
+    yg = ext.glq_fused_linear_trellis_3inst_group(x.to(DEV), [(svd, sud, pd, 0.02, out_f, m), (svd, sud, pd, 0.02, m, m)],
+                                                  bnt, bnm, n, n, out_dtype=torch.bfloat16)
+    assert yg.shape == (B, out_f + m)
+    assert rel(yg[:, :out_f], ref[:, :out_f]) < TOL and rel(yg[:, out_f:], ref) < TOL

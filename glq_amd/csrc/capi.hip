@@ -27,7 +27,9 @@ int glqh_e8_tile_ksplit(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, in
 size_t glqh_e8_tile_xb_bytes(int64_t n_pad, int64_t M);
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
-                        int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold);
+                        int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold, int out_f16 = 0,
+                        float f16_scale = 1.0f);
+int glqh_e8_tile_f16_sums_ok(int64_t M, int fold, int64_t m_pad);
 // Above 16 tokens the weights are decoded once per 128 x 512 tile instead of once per 16 tokens.
 #define GLQH_E8_SMALL_BATCH 16
 static int e8_tile_ks(int64_t m_pad, int64_t n_pad, int64_t B, int nstages, bool fold) {
@@ -1817,17 +1819,27 @@ extern "C" int glqh_fused_linear_e8_folded(const void *x, int x_dtype, int64_t x
         return 1;
     if (tks > 0) {
         // many tokens: one combined product on the compressed indices, summed over its K slots and
-        // scaled by the output transform
+        // scaled by the output transform.  From 257 tokens on folded streams the sums are rounded to fp16 on
+        // the way out, times Wscale (half the bytes between the product and the output transform, as on the
+        // trellis route; GLQ_E8_F16_SUMS=0 keeps them fp32).  The whole-block transform that reads them stores
+        // 16 bytes at a time: rows of y that do not start on 16 bytes keep fp32 sums.
+        static const bool f16_on = [] { const char *e = getenv("GLQ_E8_F16_SUMS"); return !(e && e[0] == '0'); }();
+        const int64_t y_esz = y_dtype == GLQH_F32 ? 4 : 2;
+        const int f16_sums = f16_on && tks <= tr_f16_sums_max_slots() && glqh_e8_tile_f16_sums_ok(B, folded != nullptr, m_pad) &&
+                             glqh_output_rht_wide_eligible(B, blocks_m, n_blocks_m, m_pad) && ((uintptr_t)y & 15) == 0 &&
+                             ((uintptr_t)su_f16 & 15) == 0 && (y_stride * y_esz) % 16 == 0;
         const float rel[3] = {(float)inv_rs, (float)inv_rs2, (float)inv_rs3};
         if (glqh_launch_e8_tile(blocked == 0 ? nullptr : x_rht, (char *)ws + xb + tile_part, B, sg.q, sg.n, table1,
-                                table2 ? table2 : table1, table2 ? n_entries2 : 65536, rel, m_pad, n_pad, part, st, folded))
+                                table2 ? table2 : table1, table2 ? n_entries2 : 65536, rel, m_pad, n_pad, part, st, folded,
+                                f16_sums, (float)wscale))
             return 1;
         glqh_ysrc src = {};
         src.nparts = 1;
-        src.scale[0] = (float)wscale;
+        src.scale[0] = f16_sums ? 1.0f : (float)wscale;        // fp16 sums carry the scale already
         src.part = part;
         src.part_kstride = B * m_pad;
         src.ksplit = tks;
+        src.part_f16 = f16_sums;
         return glqh_launch_output_rht(src, su_f16, y, y_dtype, y_stride, B, out_features, m_pad, bm_meta_dev,
                                       blocks_m, n_blocks_m, 0, 0.0f, st);
     }

@@ -48,6 +48,8 @@ constexpr int ET_SMALL_TOKENS = 256;               // up to here the folded form
 constexpr uint32_t ET_MISS = 0xFFFFFFFFu;          // no table word has a code above 12
 constexpr int ET_BUF = 2 * ET_FRAGS * GLQH_WAVE;   // 16-byte slots per A buffer: 2 sub-steps x 8 fragments
 constexpr size_t ET_LDS = (size_t)(ET_P + 1) * 4 + (size_t)2 * ET_BUF * 16;   // 128 KB + 32 KB
+constexpr int ET_EP_STRIDE = ET_ROWS + 4;          // floats per token of a wave's output staging space (FOLD)
+constexpr size_t ET_EP_BYTES = (size_t)ET_WAVES * 16 * ET_EP_STRIDE * sizeof(float);   // 66 KB
 
 struct et_args {
     const uint16_t *q[4];                          // FOLD: the 16-bit words of the folded streams
@@ -62,6 +64,9 @@ struct et_args {
     int M, m_pad, n_pad;
     int RT, TT, KS, slot_ds;                       // row tiles, token tiles, K slots, 64-column steps per slot
     float *part;                                   // [slot][token][row]
+    int staged;                                    // FOLD: sums leave through LDS (m_pad % 4 == 0; % 8 with out_f16)
+    int out_f16;                                   // FOLD, staged: sums as fp16, times scale
+    float scale;
 };
 
 __device__ __forceinline__ void et_barrier() {     // waits for LDS only: global prefetches stay in flight
@@ -390,7 +395,46 @@ e8_tile_kernel(const et_args a) {
             }
         }
 
-        // lane holds rows 4g .. 4g+3 of token i of every (fragment, token tile)
+        // lane holds rows 4g .. 4g+3 of token i of every (fragment, token tile): sixteen bytes here, sixteen
+        // bytes a whole row of sums further on for the next token -- stored like that a wave's instruction
+        // touches 64 lines.  On the folded streams (whose tables leave the room) every wave passes its sums
+        // through LDS once, its own 16 tokens x 128 rows in a space of its own (no barrier: a wave's LDS
+        // operations complete in order), and stores whole runs of a token's rows: two tokens x 512 bytes per
+        // instruction in fp32, four tokens x 256 bytes in fp16.
+        if constexpr (FOLD) {
+            if (a.staged) {                                     // uniform
+                float *ep = (float *)(abuf + 2 * ET_BUF) + wave * (16 * ET_EP_STRIDE);
+#pragma unroll
+                for (int tt = 0; tt < NTW; ++tt) {
+#pragma unroll
+                    for (int f = 0; f < ET_FRAGS; ++f) *(f32x4 *)(ep + i * ET_EP_STRIDE + 16 * f + 4 * g) = acc[f][tt];
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    if (a.out_f16) {
+                        const int rl = 8 * (lane & 15), row = r0 + rl;
+#pragma unroll 2
+                        for (int j = 0; j < 4; ++j) {
+                            const int tl = 4 * j + (lane >> 4), tok = tok0 + 16 * tt + tl;
+                            const f32x4 v0 = *(const f32x4 *)(ep + tl * ET_EP_STRIDE + rl) * a.scale;
+                            const f32x4 v1 = *(const f32x4 *)(ep + tl * ET_EP_STRIDE + rl + 4) * a.scale;
+                            if (tok >= a.M || row >= a.m_pad) continue;   // m_pad is a multiple of 8: whole runs of eight
+                            typedef _Float16 f16x8o __attribute__((ext_vector_type(8)));
+                            *(f16x8o *)((f16 *)a.part + ((int64_t)slot * a.M + tok) * a.m_pad + row) =
+                                f16x8o{(f16)v0[0], (f16)v0[1], (f16)v0[2], (f16)v0[3], (f16)v1[0], (f16)v1[1], (f16)v1[2], (f16)v1[3]};
+                        }
+                    } else {
+                        const int rl = 4 * (lane & 31), row = r0 + rl;
+#pragma unroll 2
+                        for (int j = 0; j < 8; ++j) {
+                            const int tl = 2 * j + (lane >> 5), tok = tok0 + 16 * tt + tl;
+                            const f32x4 v = *(const f32x4 *)(ep + tl * ET_EP_STRIDE + rl);
+                            if (tok >= a.M || row >= a.m_pad) continue;   // m_pad is a multiple of 4
+                            *(f32x4 *)(a.part + ((int64_t)slot * a.M + tok) * a.m_pad + row) = v;
+                        }
+                    }
+                }
+                continue;
+            }
+        }
         const bool vec = (a.m_pad & 3) == 0;
 #pragma unroll
         for (int tt = 0; tt < NTW; ++tt) {
@@ -705,12 +749,12 @@ int et_make_plan(int64_t m_pad, int64_t n_pad, int64_t M, int nstages, et_plan *
 }
 
 // FOLD: two tables of at most 2048 half codewords of 8 bytes, and the A buffers
-constexpr size_t ET_LDS_FOLD = (size_t)2 * 2048 * 8 + (size_t)2 * ET_BUF * 16;
+constexpr size_t ET_LDS_FOLD = (size_t)2 * 2048 * 8 + (size_t)2 * ET_BUF * 16 + ET_EP_BYTES;
 
 template <int NS, int NTW, bool FOLD>
 int et_launch(const et_plan &p, const et_args &a, hipStream_t stream) {
     size_t lds = ET_LDS;
-    if (FOLD) lds = (size_t)(((a.nh1 + 1u) & ~1u) + (a.t2_is_t1 ? 0u : (a.nh2 + 1u) & ~1u)) * 8 + (size_t)2 * ET_BUF * 16;
+    if (FOLD) lds = (size_t)(((a.nh1 + 1u) & ~1u) + (a.t2_is_t1 ? 0u : (a.nh2 + 1u) & ~1u)) * 8 + (size_t)2 * ET_BUF * 16 + ET_EP_BYTES;
     hipLaunchKernelGGL((e8_tile_kernel<NS, NTW, FOLD>), dim3((unsigned)p.grid), dim3(ET_THREADS), lds, stream, a);
     GLQH_LAUNCH_CHECK("e8 tile launch");
     return 0;
@@ -783,17 +827,24 @@ __global__ void __launch_bounds__(256) et_zero_kernel(u32x4 *__restrict__ p, int
 }
 }  // namespace
 
+// fp16 sums are written by the large tiles of the folded form only
+int glqh_e8_tile_f16_sums_ok(int64_t M, int fold, int64_t m_pad) { return fold && M > ET_SMALL_TOKENS && m_pad % 8 == 0; }
+
 // part[(slot * M + token) * m_pad + row] = sum over the slot's columns of x[token, k] * W[row, k],
-// W = cb[q0] + rel[0] * cb2[q1] + rel[1] * cb[q2] + rel[2] * cb[q3] (nstages terms), unscaled.
+// W = cb[q0] + rel[0] * cb2[q1] + rel[1] * cb[q2] + rel[2] * cb[q3] (nstages terms), unscaled (fp32), or
+// times f16_scale and rounded to fp16 with out_f16 (glqh_e8_tile_f16_sums_ok).
 // x_f16 is (M, n_pad) row-major; xb_scratch takes its repacked copy (glqh_e8_tile_xb_bytes).
 // tokens of the blocked activation layout: M padded to whole workgroup tiles
 int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages) { return et_padded_tokens(M, nstages); }
 
 int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const void *const q[4], int nstages,
                         const uint32_t *t1, const uint32_t *t2, int64_t n2, const float rel[3], int64_t m_pad,
-                        int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold) {
+                        int64_t n_pad, float *part, hipStream_t stream, const glqh_e8_folded *fold, int out_f16,
+                        float f16_scale) {
     glqh_range range("dequant_matmul");
     et_plan p;
+    if (out_f16 && !glqh_e8_tile_f16_sums_ok(M, fold != nullptr, m_pad))
+        return glqh_fail("e8 tile kernel: fp16 sums are partial sums of the large tiles on folded streams");
     const int64_t n_cols = n_pad;                              // columns the caller's rows and activations have
     if (fold && n_pad >= 32 && (n_pad & 31) == 0) n_pad = et_width(n_pad);
     if (!et_make_plan(m_pad, n_pad, M, nstages, &p))
@@ -846,6 +897,9 @@ int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const vo
     a.KS = p.KS;
     a.slot_ds = p.slot_ds;
     a.part = part;
+    a.staged = fold && m_pad % 4 == 0;
+    a.out_f16 = out_f16;
+    a.scale = out_f16 ? f16_scale : 1.0f;
     if (fold && M <= ET_SMALL_TOKENS) {                        // one token tile: TT = 1
         switch (nstages) {
         case 1: return et_launch_small_NS<1>(p, a, stream);
@@ -854,6 +908,9 @@ int glqh_launch_e8_tile(const void *x_f16, void *xb_scratch, int64_t M, const vo
         case 4: return et_launch_small_NS<4>(p, a, stream);
         }
     }
+    // (A second launch of 256-token tiles for a half-empty last round, as the trellis tile launcher has, was
+    // measured here and not kept: 14336 x 4096 at 4096 tokens 593 -> 617 us, at 2048 tokens 289 -> 297;
+    // 11008 x 2048 at 2048 tokens 170 -> 162.)
     switch (nstages * 2 + (fold ? 1 : 0)) {
     case 2: return et_launch_NS<1, false>(p, a, stream);
     case 3: return et_launch_NS<1, true>(p, a, stream);

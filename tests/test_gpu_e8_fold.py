@@ -223,6 +223,37 @@ def test_fused_linear_on_folded_streams_and_under_capture(ext):
     assert rel(y_fold, O.e8_linear_forward(x.float().cpu().numpy(), art, n, m)) < TOL
 
 
+@pytest.mark.parametrize("m,n,B", [(1536, 1024, 300), (1536, 1024, 700), (1000, 2048, 520), (1004, 1024, 300), (1002, 1024, 300),
+                                   (4096, 512, 1100)])
+@pytest.mark.parametrize("stages", [1, 2, 4])
+def test_fused_linear_at_many_tokens_on_folded_streams(ext, m, n, B, stages):
+    """From 257 tokens on the folded form hands its sums to the output transform as fp16, times Wscale, when
+    the rows of the sums and of y start on 16 bytes (m a multiple of 8), and as fp32 otherwise; both are the
+    oracle's linear, also with activations large enough to take unscaled sums past the fp16 range."""
+    say("e8 folded fused linear, many tokens", m, n, B, stages)
+    from glq_amd import hadamard as H
+    q = [t(a) for a in _indices(m, n, stages, 3 * m + stages + B)]
+    su, sv = O.rht_signs(m, n, 42)
+    bn, bm = O.block_decompose(n), O.block_decompose(m)
+    cb = e8_table_f16()
+    inv = [1 / 3.0, 1 / 9.0, 1 / 27.0]
+    extra = []
+    for s in range(1, 4):
+        extra += [q[s] if s < stages else None, cb if s < stages else None, inv[s - 1] if s < stages else 0.0]
+    qs = q + [None] * (4 - stages)
+    assert ext.e8_prepare(qs[0], cb, qs[1], cb, qs[2], qs[3]) > 0
+    args = (t(sv.astype(np.float16)), t(su.astype(np.float16)), q[0], cb, 0.02, n, m, n, m, torch.tensor(bn),
+            torch.tensor(bm), H.pack_block_meta(bn).to(DEV), H.pack_block_meta(bm).to(DEV), *extra)
+    W = sum(O.e8_table()[q[s].cpu().numpy().view(np.uint16).astype(np.int64)].reshape(m, n) * (3.0 ** -s)
+            for s in range(stages)).astype(np.float32) * np.float32(0.02)
+    for amp in (1.0, 600.0):
+        x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * amp).bfloat16().to(DEV)
+        y = ext.glq_fused_linear_block_diag_cuda(x, *args, out_dtype=torch.bfloat16)
+        assert torch.isfinite(y).all()
+        want = O.linear_forward_rht(x.float().cpu().numpy(), W, su.astype(np.float32), sv.astype(np.float32), bn, bm, n, m)
+        assert rel(y, want) < TOL
+
+
 def test_fresh_views_of_the_indices_hit_the_one_fold(ext):
     """A caller that passes a new view object of the same index memory on every call (a shard of a
     stacked tensor, `.view()`) finds the one folded copy: nothing is folded again, nothing dropped."""

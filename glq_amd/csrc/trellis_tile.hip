@@ -162,9 +162,16 @@ __device__ __forceinline__ void tt_emit2(const tr_record<R> &r, const tr_record<
     }
 }
 
-template <int R, int NTW, int MODE, int R2 = 0>
+// PC: the waves of a SIMD take one role each instead of both in turn.  Waves 0..3 (one per SIMD) only MULTIPLY,
+// 16 NTW tokens each against all 16 operands of a step; waves 4..7 only DECODE, a whole record per lane and step
+// (both m-tiles: block pair (w >> 1) & 1, k-pair w & 1).  The tile is 128 rows x 64 NTW tokens: half as many waves
+// read the operands back from LDS (64 KB per step and workgroup instead of 128, which at 16 or 32 tokens per
+// wave costs more cycles than their products), and a SIMD's decode runs beside its products instead of between
+// them.  Same tiles, K slots and order of summation as the plain form with NTW / 2: the same bits.
+template <int R, int NTW, int MODE, int R2 = 0, bool PC = false>
 __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g, const tt_moe &mo) {
     constexpr bool GROUP = MODE == TT_GROUP, MOE = MODE == TT_MOE;
+    constexpr int MW = PC ? 4 : TT_WAVES;                       // multiplying waves
     constexpr int RB = R2 > 0 ? R2 : 1, REC2 = 4 * RB;
     extern __shared__ u32x4 abuf[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -172,8 +179,10 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
     const int nkp = a.k >> 5, nds = a.k >> 6;
     constexpr int REC = 4 * R;
 
-    // decode role
-    const int unit = wave >> 2, kpi = (wave >> 1) & 1, ms = wave & 1;
+    // decode role (PC: of waves 4..7, both m-tiles)
+    const bool producer = PC && wave >= 4;                      // uniform over the wave
+    const int dw = PC ? 2 * (wave & 3) : wave;
+    const int unit = dw >> 2, kpi = (dw >> 1) & 1, ms = dw & 1;
     const int hm = i >> 3, l = 4 * (i & 7) + q;
     const int l1 = (l + 1) & 31, l2 = (l + 2) & 31;
     const int next1 = 16 * (l1 & 3) + 8 * hm + (l1 >> 2), next2 = 16 * (l2 & 3) + 8 * hm + (l2 >> 2);
@@ -204,7 +213,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             rt -= first;
         }
         const int mpairs = lm >> 5;
-        int tok0 = tt0 * (TT_WAVES * 16 * NTW) + wave * 16 * NTW, limit = a.M;
+        int tok0 = tt0 * (MW * 16 * NTW) + (PC ? wave & 3 : wave) * 16 * NTW, limit = a.M;
         float osc = 1.0f;
         bool active = true;                                     // uniform over the wave
         const uint8_t *lpacked2 = a.packed2;
@@ -212,13 +221,13 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         if constexpr (MOE) {
             // a run of the table may be longer than this kernel's tile (a stacked expert's streams are decoded
             // into one operand in tiles of at most 256 positions): TT workgroup tiles per run, in order
-            constexpr int WG_TOK = TT_WAVES * 16 * NTW;
+            constexpr int WG_TOK = MW * 16 * NTW;
             const int4 tile = mo.tiles[item / (a.RT * a.TT)];
             const int sub = (item / a.RT) % a.TT;
             const int first = tile.y + sub * WG_TOK, cnt = min(WG_TOK, tile.z - sub * WG_TOK);
             if (cnt <= 0) continue;                             // uniform over the workgroup
             lpacked = a.packed + tile.x * mo.stride_bytes;
-            tok0 = first + __builtin_amdgcn_readfirstlane(wave) * 16 * NTW;   // uniform: scalar registers
+            tok0 = first + __builtin_amdgcn_readfirstlane(PC ? wave & 3 : wave) * 16 * NTW;   // uniform: scalar registers
             limit = first + cnt;
             osc = mo.wscale_dev[tile.x];
             if constexpr (R2 > 0) {
@@ -268,13 +277,49 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
 #pragma unroll
             for (int tt = 0; tt < NTW; ++tt) dst[tt] = *(const u32x4 *)(xrow + (2 * d + (hidx & 1)) * bstep + tt * 512);
         };
-        tr_record<R> rc = load_rec(ds0);
-        tr_record<RB> rcb = load_rec2(ds0);
+        if constexpr (PC) {
+            if (producer) {                                     // as many barriers as the multiplying waves meet
+                auto emit_both = [&](const tr_record<R> &r, const tr_record<RB> &rb, u32x4 *dst) {
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt) {
+                        if constexpr (R2 > 0) tt_emit2<R, RB>(r, rb, lrs2, unit, kpi, mt, next1, next2, lane, dst);
+                        else tt_emit<R>(r, unit, kpi, mt, next1, next2, lane, dst);
+                    }
+                };
+                tr_record<R> p1 = load_rec(ds0 + 1), p2 = load_rec(ds0 + 2);
+                tr_record<RB> p1b = load_rec2(ds0 + 1), p2b = load_rec2(ds0 + 2);
+                emit_both(load_rec(ds0), load_rec2(ds0), abuf);
+                tt_barrier();
+                for (int d = ds0; d < ds1; ++d) {
+                    const tr_record<R> p3 = load_rec(d + 3);
+                    const tr_record<RB> p3b = load_rec2(d + 3);
+                    emit_both(p1, p1b, abuf + (((d - ds0) & 1) ^ 1) * TT_BUF);
+                    tt_barrier();
+                    p1 = p2;
+                    p2 = p3;
+                    p1b = p2b;
+                    p2b = p3b;
+                }
+            }
+        }
+        auto load_rec_m = [&](int d) {                          // PC: the multiplying waves hold no records
+            tr_record<R> r = {};
+            if constexpr (!PC) r = load_rec(d);
+            return r;
+        };
+        auto load_rec2_m = [&](int d) {
+            tr_record<RB> r = {};
+            if constexpr (!PC) r = load_rec2(d);
+            return r;
+        };
+        if (!producer) {
+        tr_record<R> rc = load_rec_m(ds0);
+        tr_record<RB> rcb = load_rec2_m(ds0);
         load_half(bs[0], 0);
         load_half(bs[1], 1);
-        tr_record<R> r1 = load_rec(ds0 + 1), r2 = load_rec(ds0 + 2);
-        tr_record<RB> r1b = load_rec2(ds0 + 1), r2b = load_rec2(ds0 + 2);
-        emit(rc, rcb, abuf);
+        tr_record<R> r1 = load_rec_m(ds0 + 1), r2 = load_rec_m(ds0 + 2);
+        tr_record<RB> r1b = load_rec2_m(ds0 + 1), r2b = load_rec2_m(ds0 + 2);
+        if constexpr (!PC) emit(rc, rcb, abuf);
         tt_barrier();
         for (int d0 = ds0; d0 < ds1; d0 += 3) {
 #pragma unroll
@@ -284,11 +329,13 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             const int par = (d - ds0) & 1;
             const u32x4 *rd = abuf + par * TT_BUF;
             u32x4 *wr = abuf + (par ^ 1) * TT_BUF;
-            const tr_record<R> r3 = load_rec(d + 3);
-            const tr_record<RB> r3b = load_rec2(d + 3);
+            const tr_record<R> r3 = load_rec_m(d + 3);
+            const tr_record<RB> r3b = load_rec2_m(d + 3);
             if (MOE && !active) {                               // no positions of the run left for this wave
-                emit(r1, r1b, wr, 0);
-                emit(r1, r1b, wr, 1);
+                if constexpr (!PC) {
+                    emit(r1, r1b, wr, 0);
+                    emit(r1, r1b, wr, 1);
+                }
             } else {
             f16x8 ring[2];
             ring[0] = __builtin_bit_cast(f16x8, rd[lane]);
@@ -307,8 +354,10 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
                 for (int tt = 0; tt < NTW; ++tt)
                     acc[f][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                         af, __builtin_bit_cast(f16x8, bs[(2 * j + u) % 3][tt]), acc[f][tt], 0, 0, 0);
-                if (kk == 1) emit(r1, r1b, wr, 0);
-                if (kk == TT_FRAGS + 1) emit(r1, r1b, wr, 1);
+                if constexpr (!PC) {
+                    if (kk == 1) emit(r1, r1b, wr, 0);
+                    if (kk == TT_FRAGS + 1) emit(r1, r1b, wr, 1);
+                }
             }
             }
             tt_barrier();                                       // rd has been read, wr is written
@@ -317,6 +366,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
             r1b = r2b;
             r2b = r3b;
           }
+        }
         }
         // Lane (i, q) holds four consecutive rows of token i for every (operand, token tile): operand
         // f = 4 unit' + s covers rows 64 unit' + 32 h + 8 s + (0..7), h = 0, 1 -- sixteen bytes here, sixteen
@@ -329,7 +379,7 @@ __device__ __forceinline__ void tr_tile_body(const tt_args &a, const tt_group &g
         float *ep = (float *)abuf + wave * (16 * TT_EP_STRIDE);
 #pragma unroll
         for (int tt = 0; tt < NTW; ++tt) {
-            if (MOE && !active) break;
+            if ((MOE && !active) || producer) break;
 #pragma unroll
             for (int f = 0; f < TT_FRAGS; ++f)
                 *(f32x4 *)(ep + i * TT_EP_STRIDE + 64 * (f >> 2) + 8 * (f & 3) + rlane) = acc[f][tt];
@@ -387,6 +437,25 @@ tr_tile_kernel(const tt_args a) {
     tr_tile_body<R, NTW, TT_PLAIN>(a, tt_group{}, tt_moe{});
 }
 
+// up to 256 tokens per tile: decoding and multiplying waves (NTW = 2, 4: tiles of 128, 256 tokens)
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_pc_kernel(const tt_args a) {
+    tr_tile_body<R, NTW, TT_PLAIN, 0, true>(a, tt_group{}, tt_moe{});
+}
+
+template <int R2, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_rvq_pc_kernel(const tt_args a) {
+    tr_tile_body<4, NTW, TT_PLAIN, R2, true>(a, tt_group{}, tt_moe{});
+}
+
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_group_pc_kernel(const tt_args a, const tt_group g) {
+    tr_tile_body<R, NTW, TT_GROUP, 0, true>(a, g, tt_moe{});
+}
+
 // a stacked layer (first stage 4 bits/weight): both streams decoded into one operand
 template <int R2, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
@@ -404,6 +473,18 @@ template <int R, int NTW>
 __global__ void __launch_bounds__(TT_THREADS)
 tr_tile_moe_kernel(const tt_args a, const tt_moe mo) {
     tr_tile_body<R, NTW, TT_MOE>(a, tt_group{}, mo);
+}
+
+template <int R, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_moe_pc_kernel(const tt_args a, const tt_moe mo) {
+    tr_tile_body<R, NTW, TT_MOE, 0, true>(a, tt_group{}, mo);
+}
+
+template <int R2, int NTW>
+__global__ void __launch_bounds__(TT_THREADS)
+tr_tile_moe_rvq_pc_kernel(const tt_args a, const tt_moe mo) {
+    tr_tile_body<4, NTW, TT_MOE, R2, true>(a, tt_group{}, mo);
 }
 
 // stacked experts (first stage 4 bits/weight): both streams of the run's expert into one operand
@@ -713,6 +794,21 @@ void tt_make_plan(int64_t m, int64_t k, int64_t M, tt_plan *p, int max_ntw = 4) 
     if (tt_plan_cost(p2, m, M, 3) < 0.95 * tt_plan_cost(*p, m, M, 3)) *p = p2;
 }
 
+// Tiles of up to 256 tokens run with decoding and multiplying waves (the tr_tile_*_pc_kernel forms) when a K
+// slot has min_steps steps or more; GLQ_TT_PC=0: never, GLQ_TT_PC_STEPS: another shortest slot.  Whole linears,
+// both forms in one run, us: 14336 x 4096 at 96 / 128 / 192 / 256 tokens 50.9 / 52.7 / 64.1 / 66.0 -> 47.1 / 48.4 /
+// 59.8 / 61.4, 4096 x 14336 48.5 / 50.3 / 61.5 / 63.5 -> 43.8 / 45.7 / 57.0 / 59.1; with slots of 8 steps a
+// single-stage layer loses (4096 x 4096 at 96 / 128 tokens 30.5 / 33.6 -> 35.2 / 35.1: the first operands of a
+// slot are decoded by half as many waves), so it asks for 16.  Stacked layers, whose decode is twice as long, and
+// grouped layers gain from 8 steps on: 4 + 2 bits 14336 x 4096 75.5 / 76.3 / 89.9 -> 60.0 / 62.3 / 72.4 at 96 /
+// 128 / 256 tokens and 154 -> 120 at 512, 4096 x 4096 35.4 / 45.1 / 61.3 -> 33.2 / 42.1 / 53.2 at 128 / 256 / 512;
+// grouped gate/up of a 4096-wide model 84.2 / 84.6 / 110.8 -> 72.1 / 74.3 / 98.5, q/k/v 43.3 / 51.7 -> 41.6 / 50.2.
+bool tt_split_roles(const tt_plan &p, int min_steps) {
+    static const int pc = [] { const char *e = getenv("GLQ_TT_PC"); return e ? atoi(e) : 1; }();
+    static const int pc_steps = [] { const char *e = getenv("GLQ_TT_PC_STEPS"); return e ? atoi(e) : 0; }();
+    return pc && p.NTW <= 2 && p.slot_ds >= (pc_steps > 0 ? pc_steps : min_steps);
+}
+
 template <int R, int NTW>
 int tt_launch(const tt_plan &p, const tt_args &a, hipStream_t stream) {
     hipLaunchKernelGGL((tr_tile_kernel<R, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a);
@@ -725,6 +821,8 @@ int tt_launch_rvq(const tt_plan &p, const tt_args &a, hipStream_t stream) {
     const dim3 grid((unsigned)p.grid), block(TT_THREADS);
     if (a.M <= 32) hipLaunchKernelGGL((tr_tile_small_kernel<4, 2, 1, R2>), grid, block, TT_SMALL_LDS, stream, a);
     else if (a.M <= 64) hipLaunchKernelGGL((tr_tile_small_kernel<4, 4, 1, R2>), grid, block, TT_SMALL_LDS, stream, a);
+    else if (tt_split_roles(p, 8) && p.NTW == 1) hipLaunchKernelGGL((tr_tile_rvq_pc_kernel<R2, 2>), grid, block, TT_LDS, stream, a);
+    else if (tt_split_roles(p, 8)) hipLaunchKernelGGL((tr_tile_rvq_pc_kernel<R2, 4>), grid, block, TT_LDS, stream, a);
     else if (p.NTW == 1) hipLaunchKernelGGL((tr_tile_rvq_kernel<R2, 1>), grid, block, TT_LDS, stream, a);
     else hipLaunchKernelGGL((tr_tile_rvq_kernel<R2, 2>), grid, block, TT_LDS, stream, a);
     GLQH_LAUNCH_CHECK("trellis two-stage tile launch");
@@ -744,6 +842,12 @@ int tt_launch_R(const tt_plan &p, const tt_args &a, hipStream_t stream) {
     // 31.4 against 33.3 us at 128 tokens, 4096 x 14336 59.7 against 64.4 at 256, both in one run)
     if (a.M <= 32) return tt_launch_small<R, 2, 1>(p, a, stream);
     if (a.M <= 64) return tt_launch_small<R, 4, 1>(p, a, stream);
+    if (tt_split_roles(p, 16)) {
+        if (p.NTW == 1) hipLaunchKernelGGL((tr_tile_pc_kernel<R, 2>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a);
+        else hipLaunchKernelGGL((tr_tile_pc_kernel<R, 4>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a);
+        GLQH_LAUNCH_CHECK("trellis tile launch");
+        return 0;
+    }
     if (p.NTW == 1) return tt_launch<R, 1>(p, a, stream);
     if (p.NTW == 2) return tt_launch<R, 2>(p, a, stream);
     return tt_launch<R, 4>(p, a, stream);
@@ -760,6 +864,11 @@ template <int R>
 int tt_init_R() {
     return tt_set_lds(tr_tile_small_kernel<R, 2, 1>) || tt_set_lds(tr_tile_small_kernel<R, 4, 1>) ||
            tt_set_lds(tr_tile_kernel<R, 1>) || tt_set_lds(tr_tile_kernel<R, 2>) || tt_set_lds(tr_tile_kernel<R, 4>) ||
+           tt_set_lds(tr_tile_pc_kernel<R, 2>) || tt_set_lds(tr_tile_pc_kernel<R, 4>) ||
+           tt_set_lds(tr_tile_rvq_pc_kernel<R, 2>) || tt_set_lds(tr_tile_rvq_pc_kernel<R, 4>) ||
+           tt_set_lds(tr_tile_group_pc_kernel<R, 2>) || tt_set_lds(tr_tile_group_pc_kernel<R, 4>) ||
+           tt_set_lds(tr_tile_moe_pc_kernel<R, 2>) || tt_set_lds(tr_tile_moe_pc_kernel<R, 4>) ||
+           tt_set_lds(tr_tile_moe_rvq_pc_kernel<R, 2>) || tt_set_lds(tr_tile_moe_rvq_pc_kernel<R, 4>) ||
            tt_set_lds(tr_tile_group_kernel<R, 1>) || tt_set_lds(tr_tile_group_kernel<R, 2>) ||
            tt_set_lds(tr_tile_small_kernel<4, 2, 1, R>) || tt_set_lds(tr_tile_small_kernel<4, 4, 1, R>) ||
            tt_set_lds(tr_tile_rvq_kernel<R, 1>) || tt_set_lds(tr_tile_rvq_kernel<R, 2>) ||
@@ -896,10 +1005,15 @@ template <int R>
 int tt_launch_group_R(const tt_plan &p, const tt_args &a, const tt_group &g, hipStream_t stream) {
 #define GLQH_TTG(NTW)                                                                                      \
     hipLaunchKernelGGL((tr_tile_group_kernel<R, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a, g)
-    if (p.NTW == 1) GLQH_TTG(1);
+#define GLQH_TTGP(NTW)                                                                                     \
+    hipLaunchKernelGGL((tr_tile_group_pc_kernel<R, NTW>), dim3((unsigned)p.grid), dim3(TT_THREADS), TT_LDS, stream, a, g)
+    if (tt_split_roles(p, 8) && p.NTW == 1) GLQH_TTGP(2);
+    else if (tt_split_roles(p, 8)) GLQH_TTGP(4);
+    else if (p.NTW == 1) GLQH_TTG(1);
     else if (p.NTW == 2) GLQH_TTG(2);
     else GLQH_TTG(4);
 #undef GLQH_TTG
+#undef GLQH_TTGP
     GLQH_LAUNCH_CHECK("trellis tile group launch");
     return 0;
 }
@@ -1036,10 +1150,18 @@ int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t str
     const int64_t max_items = glqh_trellis_tile_moe_max_tiles(n_slots, n_experts) * a.RT * a.TT;
     const int cus = glqh_device_cus();
     const dim3 grid((unsigned)(max_items < cus ? max_items : cus));
+    tt_plan pl = {};
+    pl.NTW = tile_tok == 128 ? 1 : 2;
+    pl.slot_ds = a.slot_ds;
+    const bool split = (packed2 || tile_tok <= 256) && tt_split_roles(pl, 8);
     if (packed2) {
 #define GLQH_TTM2(RR)                                                                                              \
     do {                                                                                                           \
-        if (tile_tok == 128)                                                                                       \
+        if (split && tile_tok == 128)                                                                              \
+            hipLaunchKernelGGL((tr_tile_moe_rvq_pc_kernel<RR, 2>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);  \
+        else if (split)                                                                                            \
+            hipLaunchKernelGGL((tr_tile_moe_rvq_pc_kernel<RR, 4>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);  \
+        else if (tile_tok == 128)                                                                                  \
             hipLaunchKernelGGL((tr_tile_moe_rvq_kernel<RR, 1>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);     \
         else                                                                                                       \
             hipLaunchKernelGGL((tr_tile_moe_rvq_kernel<RR, 2>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);     \
@@ -1057,7 +1179,11 @@ int glqh_launch_trellis_tile_moe(const void *xb, const void *packed, int64_t str
     }
 #define GLQH_TTM(RR)                                                                                          \
     do {                                                                                                      \
-        if (tile_tok == 128)                                                                                  \
+        if (split && tile_tok == 128)                                                                         \
+            hipLaunchKernelGGL((tr_tile_moe_pc_kernel<RR, 2>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo); \
+        else if (split)                                                                                       \
+            hipLaunchKernelGGL((tr_tile_moe_pc_kernel<RR, 4>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo); \
+        else if (tile_tok == 128)                                                                             \
             hipLaunchKernelGGL((tr_tile_moe_kernel<RR, 1>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);    \
         else if (tile_tok == 256)                                                                             \
             hipLaunchKernelGGL((tr_tile_moe_kernel<RR, 2>), grid, dim3(TT_THREADS), TT_LDS, stream, a, mo);    \

@@ -281,10 +281,12 @@ def test_large_activations_stay_finite_in_the_tile_form(ext):
     assert rel(y, ref) < TOL, rel(y, ref)
 
 
-@pytest.mark.parametrize("group_min,wide_min,tile_min,tile_ntw,fuse", [
-    ("1", "1", "0", "", "1"), ("1", "1000000", "0", "", "0"), ("1000000", "12", "0", "", "1"), ("1", "12", "1", "", "1"),
-    ("1", "12", "1", "1", "0"), ("1", "12", "1", "4", "1"), ("1000000", "12", "0", "", "0")])
-def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min, tile_min, tile_ntw, fuse):
+@pytest.mark.parametrize("group_min,wide_min,tile_min,tile_ntw,fuse,pc_steps", [
+    ("1", "1", "0", "", "1", ""), ("1", "1000000", "0", "", "0", ""), ("1000000", "12", "0", "", "1", ""),
+    ("1", "12", "1", "", "1", ""), ("1", "12", "1", "1", "0", ""), ("1", "12", "1", "4", "1", ""),
+    ("1000000", "12", "0", "", "0", ""), ("1", "12", "1", "", "1", "1"), ("1", "12", "1", "1", "0", "1"),
+    ("1", "12", "1", "4", "1", "1")])
+def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min, tile_min, tile_ntw, fuse, pc_steps):
     """GLQ_MOE_GROUP_MIN (read once by the library) moves the slot count from which rows are grouped by
     expert: with 1 every case of this file runs in the grouped form, with 1000000 in the per-slot form,
     each against the oracle, in a process of its own.  GLQ_MOE_WIDE_MIN_ROWS moves the average number of rows
@@ -292,16 +294,19 @@ def test_both_forms_on_every_case_in_a_fresh_process(group_min, wide_min, tile_m
     GLQ_MOE_TILE_MIN_ROWS the average from which the tile kernel takes the grouped rows: 0 = never, 1 = always,
     then with runs of up to 256 positions, or 128 / 512 with GLQ_MOE_TILE_NTW = 1 / 4.  GLQ_MOE_FUSE=0 keeps the
     launches between and after the two decode launches separate (output transform, activation, input
-    transform; output transform, weighted sum) where one launch each is the default."""
+    transform; output transform, weighted sum) where one launch each is the default.  GLQ_TT_PC_STEPS=1: runs of
+    up to 256 positions with four decoding and four multiplying waves whatever the length of the rows (by
+    default from 8 steps of 64 columns on)."""
     import os
     import subprocess
     import sys
-    say("moe forms, child process", group_min, wide_min, tile_min, tile_ntw, fuse)
+    say("moe forms, child process", group_min, wide_min, tile_min, tile_ntw, fuse, pc_steps)
     r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-m", "gpu",
                         "-k", "not fresh_process", "--timeout", "300", "--timeout-method", "thread",
                         "-p", "no:cacheprovider"],
                        env={**os.environ, "GLQ_MOE_GROUP_MIN": group_min, "GLQ_MOE_WIDE_MIN_ROWS": wide_min,
-                            "GLQ_MOE_TILE_MIN_ROWS": tile_min, "GLQ_MOE_FUSE": fuse, **({"GLQ_MOE_TILE_NTW": tile_ntw} if tile_ntw else {})},
+                            "GLQ_MOE_TILE_MIN_ROWS": tile_min, "GLQ_MOE_FUSE": fuse, **({"GLQ_MOE_TILE_NTW": tile_ntw} if tile_ntw else {}),
+                            **({"GLQ_TT_PC_STEPS": pc_steps} if pc_steps else {})},
                        capture_output=True, text=True, timeout=900,
                        cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])

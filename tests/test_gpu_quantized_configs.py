@@ -286,9 +286,11 @@ def test_e8_prefill_quantized_layer_up_to_4096_tokens(ext, m, n, monkeypatch):
     rows = _sample_rows(4096)
     r = x[rows].float().numpy() @ W_hat.T
     assert sqnr(r, ys[4096][torch.from_numpy(rows).to(DEV)].float().cpu().numpy()) > 35.0
-    # the tile kernel on the indices themselves (no folded streams): the same operands, the same bits
+    # the tile kernel on the indices themselves (no folded streams): the same operands and fp32 sums, where the
+    # folded form hands fp16 sums to the output transform from 257 tokens on (the matmul entry, fp32 on both,
+    # is bit-identical: test_gpu_e8_fold.py)
     monkeypatch.setattr(ext, "E8_FOLD", False)
-    assert torch.equal(e8_forward(ext, xd, art, m, n, torch.bfloat16), ys[4096])
+    assert rel(e8_forward(ext, xd, art, m, n, torch.bfloat16), ys[4096].float().cpu().numpy()) < 2e-3
     monkeypatch.setattr(ext, "E8_FOLD", True)
     # the library route, the default above 4096 tokens (above 1024 without folded streams)
     monkeypatch.setattr(ext, "E8_BATCH_MAX", 1024)

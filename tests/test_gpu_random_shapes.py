@@ -199,6 +199,26 @@ def test_two_stage_layers_with_a_launch_per_stage_in_a_fresh_process():
     assert " passed" in r.stdout and "no tests ran" not in r.stdout, r.stdout[-500:]
 
 
+@pytest.mark.parametrize("env", [{"GLQ_TT_PC_STEPS": "1"}, {"GLQ_TT_PC": "0"}])
+def test_tile_kernels_with_either_split_of_the_waves_in_a_fresh_process(env):
+    """Tiles of up to 256 tokens run with four decoding and four multiplying waves when their K slots are long
+    enough, with eight waves that do both otherwise (switches read once by the library).  GLQ_TT_PC_STEPS=1: the
+    split form wherever the tile allows it; GLQ_TT_PC=0: never.  The many-token cases of this file and the grouped
+    many-token calls against the oracle under both, each in a process of its own."""
+    import os
+    import subprocess
+    import sys
+    say("tile kernels, wave roles, child process", env)
+    here = os.path.dirname(os.path.abspath(__file__))
+    r = subprocess.run([sys.executable, "-u", "-m", "pytest", os.path.abspath(__file__), os.path.join(here, "test_gpu_group_many.py"),
+                        "-x", "-q", "-m", "gpu", "-k",
+                        "(trellis_fused_linear_random_shapes or large_activations or ragged_out or grouped_many_tokens) and not fresh_process",
+                        "--timeout", "300", "--timeout-method", "thread", "-p", "no:cacheprovider"],
+                       env={**os.environ, **env}, capture_output=True, text=True, timeout=900, cwd=os.path.dirname(here))
+    assert r.returncode == 0, (r.stdout[-3000:], r.stderr[-1000:])
+    assert " passed" in r.stdout and "no tests ran" not in r.stdout, r.stdout[-500:]
+
+
 def test_large_activations_stay_finite_at_many_tokens():
     """Activations of a few thousand: the unscaled sum over a row of 2048 columns passes the fp16 range, the
     layer's output (the sum times Wscale) does not.  The fp16 sums between the tile kernel and the output transform

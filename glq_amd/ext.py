@@ -42,6 +42,12 @@ _DT = {torch.float16: GLQH_F16, torch.bfloat16: GLQH_BF16, torch.float32: GLQH_F
 # 2147 / 2061 and 2004 / 1872 at 16384; 4096 x 4096 306 / 312 at 8192, 641 / 610 at 16384; 11008 x 2048 520 / 562
 # and 1058 / 1105: level at 8192 tokens, so trellis calls stay compressed up to there.
 TRELLIS_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "8192")))
+# Stacked (two-stage) layers decode two streams per tile of at most 256 tokens, and the library route adds
+# the second stage once: compressed / library, us, 4 + 2 bits, 14336 x 4096 and 4096 x 14336: 119 / 223 and
+# 109 / 243 at 512 tokens, 216 / 280 and 192 / 290 at 1024, 419 / 404 and 365 / 409 at 2048, 811 / 682 and
+# 766 / 597 at 4096, 1581 / 1191 and 1528 / 1051 at 8192 (4096 x 4096: 126 / 140 at 2048, 229 / 203 at 4096).
+# They take the library route above the smaller of the two limits.
+TRELLIS_STACKED_BATCH_MAX = max(1, int(os.environ.get("GLQ_TRELLIS_BATCH_MAX", "2048")))
 # GLQ_TRELLIS_DENSE (set to anything) sends every fused trellis call to that dense route, the
 # reference's A/B switch of the same name (glq/csrc/glq_trellis.cu:1023-1029, 1269).
 TRELLIS_DENSE = "GLQ_TRELLIS_DENSE" in os.environ
@@ -317,7 +323,8 @@ def _fused_trellis(x, sv, su, packed, packed2, blocks_n, blocks_m, bn_meta, bm_m
     yrp, yrs = C.c_void_p(0), 0
     if y_rht_out is not None:
         yrp, yrs = y_rht_out
-    if (TRELLIS_DENSE or B > TRELLIS_BATCH_MAX) and y_rht_out is None:
+    batch_max = min(TRELLIS_BATCH_MAX, TRELLIS_STACKED_BATCH_MAX) if has2 else TRELLIS_BATCH_MAX
+    if (TRELLIS_DENSE or B > batch_max) and y_rht_out is None:
         if (packed2 is not None and packed2.numel() > 0) != (float(inv_rs2) != 0.0):
             raise RuntimeError("trellis RVQ stage 2 is half-configured: trellis_packed2 is "
                                f"{'present' if has2 else 'absent'} but inv_resid_scale2 = {inv_rs2}")

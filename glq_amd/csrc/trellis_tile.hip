@@ -1080,15 +1080,16 @@ int glqh_launch_trellis_pack(const void *x_f16, void *xb, int64_t M, int64_t k, 
 
 // ---- routed experts with many rows per expert -----------------------------------------------------
 // Positions per token tile of the routed-expert form for n_slots slots over n_experts experts, by the average
-// number of rows per expert: 128 below 96, 256 below 224, 512 above (whole call, 128 experts of 2048 -> 2 x 768 ->
-// 2048 with 8 choices, us with 128 / 256 / 512: 64 rows 393 / 403 / 473, 128 rows 660 / 587 / 614, 256 rows 1187 /
-// 1034 / 997).  GLQ_MOE_TILE_NTW (1, 2, 4; read once) forces 128 / 256 / 512.
+// number of rows per expert: 128 below 112, 256 below 224, 512 above (whole call, 128 experts of 2048 -> 2 x 768 ->
+// 2048 with 8 choices, us with 128 / 256 / 512, the first two with decoding and multiplying waves: 48 rows 287 /
+// 338 / 383, 96 rows 340 / 386 / 431, 128 rows 471 / 416 / 462, 160 rows 597 / 450 / 493, 192 rows 630 / 496 / 533,
+// 256 rows 802 / 684 / 670).  GLQ_MOE_TILE_NTW (1, 2, 4; read once) forces 128 / 256 / 512.
 int glqh_trellis_tile_moe_tokens(int64_t n_slots, int64_t n_experts) {
     static const int forced = [] { const char *e = getenv("GLQ_MOE_TILE_NTW"); return e ? atoi(e) : 0; }();
     if (forced == 1 || forced == 2 || forced == 4) return 128 * forced;
     const int64_t live = n_experts < n_slots ? n_experts : n_slots;
     const int64_t avg = n_slots / (live > 0 ? live : 1);
-    return avg >= 224 ? 512 : avg >= 96 ? 256 : 128;
+    return avg >= 224 ? 512 : avg >= 112 ? 256 : 128;
 }
 
 // positions of the packed activations: the slots plus one tile that a run's last tile may read into

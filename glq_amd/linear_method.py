@@ -25,12 +25,17 @@ from .quantized_linear import E8RHTLinear
 # GLQ_TRELLIS_BATCH_OUT_RHT=0 gives every shard its own output transform and concatenates
 # (glq_vllm/linear_method.py:616).
 _GLQ_BATCH_OUT_RHT = os.environ.get("GLQ_TRELLIS_BATCH_OUT_RHT", "1") != "0"
-# GLQ_MERGED_GROUPED=1: merged single-stage shards go through the library's grouped call (one decode or
-# many-token launch for all shards) at 1-4 and at more than 64 tokens, merged two-stage shards at one token
-# through its two-stage form, instead of the reference's per-shard sequence; same result up to the rounding of
-# another K split.  Off by default: the default is the
-# reference's own op sequence.
-_GLQ_MERGED_GROUPED = os.environ.get("GLQ_MERGED_GROUPED", "0") == "1"
+# Merged single-stage shards go through the library's grouped call (one decode or many-token launch for all
+# shards) at 1-4 and at more than 64 tokens, merged two-stage shards at one token through its two-stage form:
+# same result up to the rounding of another K split.  Whole merged linear, reference op sequence / grouped call,
+# us: q/k/v of a 2048-wide model 39.5 / 31.3 at one token, 52.5 / 36.0 at 4, 68.5 / 45.4 at 128, 95.3 / 52.7 at
+# 512; gate/up 2048 -> 2 x 11008 39.9 / 33.7, 43.7 / 37.7, 122 / 74, 277 / 108 (756 / 279 at 2048 tokens); q/k/v
+# of a 4096-wide 6 bpw model at one token 55.1 / 36.7.  GLQ_MERGED_GROUPED=0 keeps the reference's per-shard
+# sequence (fused_linear_trellis_3inst_yrht per shard + output_rht_shards, glq_vllm/linear_method.py:664-710)
+# at every token count; otherwise 5-63 tokens and, up to 63 tokens, shards the grouped call does not take
+# (stacked beyond one token, mixed, more than four) take it, and from 64 tokens on those run as whole fused
+# linears, concatenated.
+_GLQ_MERGED_GROUPED = os.environ.get("GLQ_MERGED_GROUPED", "1") != "0"
 
 # Largest output block of the shard-batched transform.  The reference stops at 8192 (shared-memory
 # budget of its kernel, glq_vllm/linear_method.py:618-623); the kernel here cuts blocks into
@@ -239,7 +244,13 @@ class MergedTrellisLinear:
                 m0["_bn"], m0["_bnm"], m0["in"], m0["n_pad"], out_dtype=x.dtype)
         if self.glq_is_fused:
             s4b = self._glq_s4b
-            if s4b is not None and _GLQ_BATCH_OUT_RHT:
+            # from 64 tokens on, shards the grouped call does not take (stacked, mixed, more than four) run as
+            # whole fused linears, concatenated: their sums stay fp16 between the tile kernel and the output
+            # transform and stacked shards take the library route above 2048 tokens, which a shared fp32 y_rht
+            # rules out (gate/up 4096 -> 2 x 14336 at 6 bpw, 512 / 2048 / 4096 tokens: 334 / 1262 / 2407 -> 251 /
+            # 935 / 1509 us; q/k/v 160 / 339 / 634 -> 116 / 247 / 436)
+            whole = _GLQ_MERGED_GROUPED and x.shape[0] >= 64
+            if s4b is not None and _GLQ_BATCH_OUT_RHT and not whole:
                 yrht = _op("fused_linear_trellis_3inst_yrht")
                 yrht2 = _op("fused_linear_trellis_3inst_yrht_rvq2") if s4b["has_s2"] else None
                 shards_rht = _op("output_rht_shards")

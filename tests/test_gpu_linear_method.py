@@ -56,7 +56,7 @@ def _oracle(x16, arts, n):
                                         (6, [(352, 4, 2), (352, 4, 2)]),                  # gate/up, 4+2 bits
                                         (5, [(2048, 4, 1), (512, 4, 1), (512, 4, 1)])])   # SmolLM3 q/k/v rows, 4+1
 @pytest.mark.parametrize("B", [1, 3, 40])
-def test_s4b_sequence_through_registered_ops_matches_oracle(ops, bpw, shards, B):
+def test_s4b_sequence_through_registered_ops_matches_oracle(ops, bpw, shards, B, monkeypatch):
     """`fused_linear_trellis_3inst_yrht[_rvq2]` per shard into one (B, total_m) buffer + one
     `output_rht_shards`, each called as `torch.ops.glq.<op>`: every shard's columns within 1e-2 of
     the oracle's fp32 CPU forward of that shard; equal to the per-shard fused op's result up to the
@@ -89,7 +89,9 @@ def test_s4b_sequence_through_registered_ops_matches_oracle(ops, bpw, shards, B)
         e = rel(y[:, col:col + m], ref[:, col:col + m])
         assert e < TOL, (m, e)
         col += m
-    # the layer object's apply() is that sequence
+    # the layer object's apply() is that sequence (with GLQ_MERGED_GROUPED=0 at every token count)
+    from glq_amd import linear_method as LM
+    monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
     ya = layer.apply(x)
     assert ya.dtype == x.dtype and torch.equal(ya, y)
     assert torch.equal(layer.apply(x), ya)
@@ -112,6 +114,7 @@ def test_batched_output_transform_switch_and_unloaded_shard(ops, monkeypatch):
     layer, arts = _merged(n, shards, 4)
     x = torch.randn(4, n, generator=torch.Generator().manual_seed(3)).to(DEV, torch.bfloat16)
     ref = _oracle(x, arts, n)
+    monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)      # the reference's sequence, not the grouped call
     y_batched = layer.apply(x)
     monkeypatch.setattr(LM, "_GLQ_BATCH_OUT_RHT", False)
     y_per_shard = layer.apply(x)
@@ -153,13 +156,16 @@ def test_load_time_invariants(ops):
         fresh.apply(torch.zeros(1, n, device=DEV, dtype=torch.float16))
 
 
+@pytest.mark.parametrize("grouped", [False, True])
 @pytest.mark.parametrize("bpw,shards", [(4, [(2048, 4, 0), (512, 4, 0), (512, 4, 0)]), (6, [(352, 4, 2), (352, 4, 2)])])
-def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, shards):
-    """The whole apply() -- yrht ops, the shared buffer, output_rht_shards, the cast -- captured once;
-    replays with new contents in the static input equal the eager result bit for bit, replay after
-    replay, with eager work in between."""
+def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, shards, grouped, monkeypatch):
+    """The whole apply() -- yrht ops, the shared buffer, output_rht_shards, the cast; or the library's grouped
+    call, the default at this token count -- captured once; replays with new contents in the static input equal
+    the eager result bit for bit, replay after replay, with eager work in between."""
+    from glq_amd import linear_method as LM
+    monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", grouped)
     n = 2048 if shards[0][0] == 2048 else 512
-    say("s4b graph", bpw)
+    say("s4b graph", bpw, grouped)
     layer, arts = _merged(n, shards, bpw)
     gen = torch.Generator().manual_seed(11)
     xs = [torch.randn(2, n, generator=gen).to(DEV, torch.bfloat16) for _ in range(4)]
@@ -186,7 +192,7 @@ def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, s
 
 @pytest.mark.parametrize("B", [2, 100])
 def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
-    """GLQ_MERGED_GROUPED: single-stage merged shards through the library's grouped call (one decode launch at
+    """Single-stage merged shards through the library's grouped call, the default (one decode launch at
     1-4 tokens, one launch of the many-token kernel above 64) against the oracle and against the default sequence
     of registered ops; token counts in between and two-stage shards keep the default sequence."""
     from glq_amd import linear_method as LM
@@ -194,6 +200,7 @@ def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
     n = 512
     layer, arts = _merged(n, [(256, 4, 0), (64, 4, 0), (64, 4, 0)], 4)
     x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * 0.5).to(torch.bfloat16).to(DEV)
+    monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
     y_ref = layer.apply(x)
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
     assert layer._grouped_ok(B) and not layer._grouped_ok(32)
@@ -208,13 +215,14 @@ def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
 @pytest.mark.parametrize("n,shards,bpw", [(512, [(352, 4, 2), (352, 4, 2)], 6), (2048, [(2048, 4, 1), (512, 4, 1), (512, 4, 1)], 5),
                                           (576, [(1184, 4, 4), (1184, 4, 4)], 8)])
 def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, shards, bpw):
-    """GLQ_MERGED_GROUPED: one token of merged stacked shards (5, 6, 8 bpw = 4 + 1, 2, 4) through the library's grouped
+    """One token of merged stacked shards (5, 6, 8 bpw = 4 + 1, 2, 4) through the library's grouped
     two-stage call (one decode launch for both streams of every shard, one finishing launch) against the oracle
     and against the default sequence of registered ops; more tokens keep the default sequence."""
     from glq_amd import linear_method as LM
     say("merged two-stage linear, grouped call", n, bpw)
     layer, arts = _merged(n, shards, bpw)
     x = (torch.randn(1, n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16).to(DEV)
+    monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
     y_ref = layer.apply(x)
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
     assert layer._grouped_rvq2_ok(1) and not layer._grouped_rvq2_ok(2) and not layer._grouped_ok(1)
@@ -225,3 +233,23 @@ def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, s
     assert torch.equal(y, layer.apply(x))
     mixed, _ = _merged(512, [(352, 4, 2), (352, 4, 1)], 6)
     assert not mixed._grouped_rvq2_ok(1)
+
+
+@pytest.mark.parametrize("B", [64, 200])
+def test_merged_stacked_shards_at_many_tokens_run_as_whole_linears(ops, monkeypatch, B):
+    """From 64 tokens on, shards the grouped call does not take (here 4+2-bit gate/up and a mixed pair) run as
+    whole fused linears, concatenated: against the oracle and against the reference's shard-batched sequence."""
+    from glq_amd import linear_method as LM
+    say("merged stacked shards, many tokens", B)
+    for n, shards, bpw in ((512, [(352, 4, 2), (352, 4, 2)], 6), (512, [(256, 4, 2), (96, 4, 1)], 6)):
+        layer, arts = _merged(n, shards, bpw)
+        x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * 0.5).to(torch.bfloat16).to(DEV)
+        monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
+        y_ref = layer.apply(x)
+        monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
+        assert not layer._grouped_ok(B) and not layer._grouped_rvq2_ok(B)
+        y = layer.apply(x)
+        assert y.dtype == x.dtype and y.shape == y_ref.shape
+        assert rel(y, _oracle(x, arts, n)) < TOL
+        assert rel(y, y_ref.float().cpu().numpy()) < 6e-3
+        assert torch.equal(y, layer.apply(x))

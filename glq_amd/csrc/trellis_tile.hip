@@ -981,6 +981,18 @@ int glqh_launch_trellis_tile(const void *x_f16, void *xb_scratch, int64_t M, con
     a.rt0 = p.RT;
     a.RT = tail.RT;
     a.TT = tail.TT;
+    tail.slot_ds = p.slot_ds;
+    if (tt_split_roles(tail, 16)) {                            // 256-token tiles: decoding and multiplying waves
+        const dim3 tgrid((unsigned)tail.grid), tblock(TT_THREADS);
+        switch (R) {
+        case 1: hipLaunchKernelGGL((tr_tile_pc_kernel<1, 4>), tgrid, tblock, TT_LDS, stream, a); break;
+        case 2: hipLaunchKernelGGL((tr_tile_pc_kernel<2, 4>), tgrid, tblock, TT_LDS, stream, a); break;
+        case 3: hipLaunchKernelGGL((tr_tile_pc_kernel<3, 4>), tgrid, tblock, TT_LDS, stream, a); break;
+        default: hipLaunchKernelGGL((tr_tile_pc_kernel<4, 4>), tgrid, tblock, TT_LDS, stream, a); break;
+        }
+        GLQH_LAUNCH_CHECK("trellis tile launch");
+        return 0;
+    }
     switch (R) {
     case 1: return tt_launch<1, 2>(tail, a, stream);
     case 2: return tt_launch<2, 2>(tail, a, stream);

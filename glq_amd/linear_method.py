@@ -292,10 +292,154 @@ class MergedTrellisLinear:
                       trellis_packed2=self.trellis_packed2.get_shard(0), inv_resid_scale2=meta["inv_rs2"])
 
 
+class MergedShellLinear:
+    """Separately quantized E8-shell shards that read the same activations and whose outputs are
+    concatenated (fused q/k/v, gate/up), or a single layer (one shard): the shell side of
+    `GLQLinearMethod.apply` (glq_vllm/linear_method.py:1490-1522) with `_glq_apply_shard` per shard
+    (:394-522).
+
+    Attributes follow the reference's layer object: `Qidxs`, `Qidxs2`, `Qidxs3`, `Qidxs4`, `SU`, `SV`, `Wscale`,
+    `inv_resid_scale`, `inv_resid_scale2`, `inv_resid_scale3` (`GLQShards`), `glq_in_features`,
+    `glq_shard_sizes`, `glq_num_shards`, `glq_is_fused`; after `process_weights_after_loading()` also
+    `_glq_shard_meta` (per shard: `wscale`, `has_stage2`, `n_stages`, `inv_rs`, `inv_rs2`, `inv_rs3`, `out`,
+    `in`, `m_pad`, `n_pad`, `log_n`, `log_m`, `bd_meta`).  Block-diagonal shards (buffers of the layer's own
+    sizes) run as one `fused_linear_block_diag` each, legacy shards (buffers padded to powers of two) as one
+    `fused_linear` each (the reference issues `input_rht`, `dequant_matmul`, `output_rht` there); activations
+    keep their dtype (fp16 or bf16) where the reference casts to fp16 and back."""
+
+    glq_is_trellis = False
+
+    def __init__(self, in_features, shard_sizes, codebook, codebook2=None):
+        self.glq_in_features = int(in_features)
+        self.glq_shard_sizes = [int(s) for s in shard_sizes]
+        self.glq_num_shards = len(self.glq_shard_sizes)
+        self.glq_is_fused = self.glq_num_shards > 1
+        self.codebook, self.codebook2 = codebook, codebook2    # (65536, 8) table; stage 2's own table if it has one
+        n = self.glq_num_shards
+        i16 = lambda: torch.zeros(0, dtype=torch.int16)      # noqa: E731
+        f32 = lambda: torch.zeros((), dtype=torch.float32)   # noqa: E731
+        for name in ("Qidxs", "Qidxs2", "Qidxs3", "Qidxs4"):
+            setattr(self, name, GLQShards(i16() for _ in range(n)))
+        for name in ("Wscale", "inv_resid_scale", "inv_resid_scale2", "inv_resid_scale3"):
+            setattr(self, name, GLQShards(f32() for _ in range(n)))
+        self.SU = GLQShards(torch.ones(s, dtype=torch.float16) for s in self.glq_shard_sizes)
+        self.SV = GLQShards(torch.ones(self.glq_in_features, dtype=torch.float16) for _ in range(n))
+        self._glq_shard_meta = None
+
+    @classmethod
+    def from_linears(cls, linears):
+        """Merge shell `E8RHTLinear` modules that share `in_features` and tables."""
+        linears = list(linears)
+        if not linears or any(l._is_trellis for l in linears):
+            raise RuntimeError("MergedShellLinear.from_linears needs E8-shell layers")
+        if len({l.in_features for l in linears}) != 1:
+            raise RuntimeError("merged shards must share in_features")
+        if any(l.codebook is None for l in linears):
+            raise RuntimeError("set_codebook() must be called on every layer before merging")
+        self = cls(linears[0].in_features, [l.out_features for l in linears], linears[0].codebook,
+                   linears[0].codebook2)
+        for name in ("Qidxs", "Qidxs2", "Qidxs3", "Qidxs4", "SU", "SV", "Wscale", "inv_resid_scale",
+                     "inv_resid_scale2", "inv_resid_scale3"):
+            setattr(self, name, GLQShards(getattr(l, name) for l in linears))
+        return self
+
+    def process_weights_after_loading(self, device=None):
+        """Everything that reads the host or allocates, once, before any capture
+        (glq_vllm/linear_method.py:1031-1110): buffers and tables to the device, scalars to Python floats,
+        block lists and their device copies, and the library's load-time step per shard (packed tables,
+        folded index streams: `ext.e8_prepare`)."""
+        from . import ext
+        from .hadamard import next_pow2
+        dev = torch.device(device) if device is not None else self.Qidxs.get_shard(0).device
+        names = ("Qidxs", "Qidxs2", "Qidxs3", "Qidxs4", "SU", "SV", "Wscale", "inv_resid_scale",
+                 "inv_resid_scale2", "inv_resid_scale3")
+        for name in names:
+            sh = getattr(self, name)
+            sh._shard_data = [t.to(dev) for t in sh._shard_data]
+        half = lambda t: None if t is None else t.to(dev).half().contiguous()   # noqa: E731
+        self._cb, self._cb2 = half(self.codebook), half(self.codebook2)
+        self._empty_i16 = torch.zeros(0, dtype=torch.int16, device=dev)
+        self._empty_f16 = torch.zeros(0, dtype=torch.float16, device=dev)
+        metas = []
+        for i, out in enumerate(self.glq_shard_sizes):
+            q = self.Qidxs.get_shard(i)
+            if q.dim() != 2 or q.dtype != torch.int16:
+                raise RuntimeError(f"shard {i}: Qidxs must be a 2-D int16 tensor")
+            m_pad, n_pad = int(q.shape[0]), int(q.shape[1]) * 8
+            inv = [float(getattr(self, nm).get_shard(i).item())
+                   for nm in ("inv_resid_scale", "inv_resid_scale2", "inv_resid_scale3")]
+            n_stages = 1
+            for s, nm in enumerate(("Qidxs2", "Qidxs3", "Qidxs4")):
+                present = getattr(self, nm).get_shard(i).numel() > 0
+                if present != (inv[s] != 0.0):
+                    raise RuntimeError(f"shard {i}: stage {s + 2} is half-configured: {nm} is "
+                                       f"{'present' if present else 'absent'} but its scale is {inv[s]}")
+                if present:
+                    if n_stages != s + 1:
+                        raise RuntimeError(f"shard {i}: stage {s + 2} without stage {s + 1}")
+                    n_stages = s + 2
+            legacy = (m_pad, n_pad) == (next_pow2(out), next_pow2(self.glq_in_features)) and \
+                (m_pad, n_pad) != (out, self.glq_in_features)
+            if not legacy and (m_pad < out or n_pad < self.glq_in_features):
+                raise RuntimeError(f"shard {i}: buffers of {m_pad} x {n_pad} for a {out} x {self.glq_in_features} layer")
+            bd = None
+            if not legacy:
+                bn, bm = block_decompose(n_pad), block_decompose(m_pad)
+                bd = dict(blocks_n_tensor=torch.tensor(bn, dtype=torch.int64), blocks_m_tensor=torch.tensor(bm, dtype=torch.int64),
+                          blocks_n_meta_gpu=pack_block_meta(bn).to(dev), blocks_m_meta_gpu=pack_block_meta(bm).to(dev))
+            cb2 = self._cb2 if self._cb2 is not None else self._cb
+            ext.e8_prepare(q, self._cb, self.Qidxs2.get_shard(i) if n_stages >= 2 else None, cb2 if n_stages >= 2 else None,
+                           self.Qidxs3.get_shard(i) if n_stages >= 3 else None,
+                           self.Qidxs4.get_shard(i) if n_stages >= 4 else None)
+            metas.append(dict(wscale=float(self.Wscale.get_shard(i).item()), has_stage2=n_stages >= 2, n_stages=n_stages,
+                              inv_rs=inv[0], inv_rs2=inv[1], inv_rs3=inv[2], out=out, **{"in": self.glq_in_features},
+                              m_pad=m_pad, n_pad=n_pad, log_n=n_pad.bit_length() - 1, log_m=m_pad.bit_length() - 1,
+                              bd_meta=bd))
+        self._glq_shard_meta = metas
+        return self
+
+    def _apply_shard(self, x, i):
+        """`_glq_apply_shard` (glq_vllm/linear_method.py:394-522) for shard i."""
+        meta = self._glq_shard_meta[i]
+        n = meta["n_stages"]
+        cb2 = self._cb2 if self._cb2 is not None else self._cb
+        q2 = self.Qidxs2.get_shard(i) if n >= 2 else self._empty_i16
+        q3 = self.Qidxs3.get_shard(i) if n >= 3 else self._empty_i16
+        q4 = self.Qidxs4.get_shard(i) if n >= 4 else self._empty_i16
+        stages = (q2, cb2 if n >= 2 else self._empty_f16, meta["inv_rs"] if n >= 2 else 0.0,
+                  q3, self._cb if n >= 3 else self._empty_f16, meta["inv_rs2"] if n >= 3 else 0.0,
+                  q4, self._cb if n >= 4 else self._empty_f16, meta["inv_rs3"] if n >= 4 else 0.0)
+        bd = meta["bd_meta"]
+        if bd is not None:
+            return _op("fused_linear_block_diag")(
+                x, self.SV.get_shard(i), self.SU.get_shard(i), self.Qidxs.get_shard(i), self._cb, meta["wscale"],
+                meta["in"], meta["out"], meta["n_pad"], meta["m_pad"], bd["blocks_n_tensor"], bd["blocks_m_tensor"],
+                bd["blocks_n_meta_gpu"], bd["blocks_m_meta_gpu"], *stages)
+        return _op("fused_linear")(
+            x, self.SV.get_shard(i), self.SU.get_shard(i), self.Qidxs.get_shard(i), self._cb, meta["wscale"],
+            meta["in"], meta["out"], meta["n_pad"], meta["m_pad"], meta["log_n"], meta["log_m"], *stages)
+
+    def apply(self, x, bias=None):
+        """(.., in_features) -> (.., sum(shard_sizes)) in x's dtype: every shard on its own, concatenated,
+        plus the bias add of `GLQLinearMethod.apply`."""
+        if self._glq_shard_meta is None:
+            raise RuntimeError("process_weights_after_loading() must run before apply()")
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        xin = (x2 if x2.dtype in (torch.float16, torch.bfloat16) else x2.half()).contiguous()
+        outs = [self._apply_shard(xin, i) for i in range(self.glq_num_shards)]
+        y = outs[0] if len(outs) == 1 else torch.cat(outs, dim=-1)
+        if y.dtype != x.dtype:
+            y = y.to(x.dtype)
+        if bias is not None:
+            y = y + bias.unsqueeze(0).to(y.dtype)
+        return y.reshape(*shape[:-1], y.shape[-1])
+
+
 def process_weights_after_loading(layer, device=None):
-    """Load-time step for either kind of layer: `MergedTrellisLinear` (above) or an `E8RHTLinear`
+    """Load-time step for any kind of layer: `MergedTrellisLinear`, `MergedShellLinear` (above) or an `E8RHTLinear`
     module (`prepare()`: scalars, metas, packed tables and folded index streams)."""
-    if isinstance(layer, MergedTrellisLinear):
+    if isinstance(layer, (MergedTrellisLinear, MergedShellLinear)):
         return layer.process_weights_after_loading(device)
     if isinstance(layer, E8RHTLinear):
         if device is not None and layer.SV.device != torch.device(device):

@@ -253,3 +253,86 @@ def test_merged_stacked_shards_at_many_tokens_run_as_whole_linears(ops, monkeypa
         assert rel(y, _oracle(x, arts, n)) < TOL
         assert rel(y, y_ref.float().cpu().numpy()) < 6e-3
         assert torch.equal(y, layer.apply(x))
+
+
+def _shell_indices(m, n, stages, seed):
+    rng = np.random.default_rng(seed)
+    lo = rng.integers(0, 30000, size=(stages, m, n // 8))
+    hi = rng.integers(0, 65536, size=(stages, m, n // 8))
+    return np.where(rng.random((stages, m, n // 8)) < 0.6, lo, hi).astype(np.uint16).view(np.int16)
+
+
+@pytest.mark.parametrize("B", [1, 5, 70, 300])
+def test_merged_shell_linear(ops, B):
+    """E8-shell shards behind one activation (glq_vllm/linear_method.py:1490-1522 with `_glq_apply_shard` per
+    shard): block-diagonal shards of one, two and four stages and a legacy shard padded to powers of two, each
+    column range against the oracle's forward of that shard; the load-time step folds the index streams, so a
+    captured first call equals the eager one."""
+    from glq_amd import ext
+    from glq_amd.linear_method import GLQShards, MergedShellLinear, process_weights_after_loading
+    from tests.gpu_util import e8_table_f16
+    say("merged shell linear", B)
+    n, cb = 512, e8_table_f16()
+    table = O.e8_table()
+    inv = [1 / 3.0, 1 / 9.0, 1 / 27.0]
+
+    def build(shards, n_in, legacy=False):
+        layer = MergedShellLinear(n_in, [m for m, _ in shards], cb)
+        arts = []
+        for i, (m, stages) in enumerate(shards):
+            m_pad, n_pad = (1 << (m - 1).bit_length(), 1 << (n_in - 1).bit_length()) if legacy else (m, n_in)
+            q = _shell_indices(m_pad, n_pad, stages, 10 * i + stages)
+            su, sv = O.rht_signs(m_pad, n_pad, 300 + i)
+            W = sum(table[q[s].view(np.uint16).astype(np.int64)].reshape(m_pad, n_pad) * np.float32(inv[s - 1] if s else 1.0)
+                    for s in range(stages)).astype(np.float32) * np.float32(0.02 + 0.001 * i)
+            arts.append(dict(q=q, su=su, sv=sv, W=W, m=m, m_pad=m_pad, n_pad=n_pad, stages=stages, ws=0.02 + 0.001 * i))
+        empty = torch.zeros(0, dtype=torch.int16)
+        for s, name in enumerate(("Qidxs", "Qidxs2", "Qidxs3", "Qidxs4")):
+            setattr(layer, name, GLQShards(torch.from_numpy(a["q"][s].copy()) if s < a["stages"] else empty for a in arts))
+        layer.SU = GLQShards(torch.from_numpy(a["su"].astype(np.float16)) for a in arts)
+        layer.SV = GLQShards(torch.from_numpy(a["sv"].astype(np.float16)) for a in arts)
+        layer.Wscale = GLQShards(torch.tensor(a["ws"], dtype=torch.float32) for a in arts)
+        for s, name in enumerate(("inv_resid_scale", "inv_resid_scale2", "inv_resid_scale3")):
+            setattr(layer, name, GLQShards(torch.tensor(inv[s] if s + 2 <= a["stages"] else 0.0, dtype=torch.float32)
+                                           for a in arts))
+        process_weights_after_loading(layer, DEV)
+        return layer, arts
+
+    def check(layer, arts, n_in, x):
+        y = layer.apply(x)
+        assert y.dtype == x.dtype and y.shape == (x.shape[0], sum(a["m"] for a in arts))
+        col = 0
+        for a in arts:
+            legacy = a["m_pad"] != a["m"] or a["n_pad"] != n_in
+            bn = [a["n_pad"]] if legacy else O.block_decompose(a["n_pad"])
+            bm = [a["m_pad"]] if legacy else O.block_decompose(a["m_pad"])
+            want = O.linear_forward_rht(np.pad(x.float().cpu().numpy(), ((0, 0), (0, a["n_pad"] - n_in))), a["W"],
+                                        a["su"].astype(np.float32), a["sv"].astype(np.float32), bn, bm, a["n_pad"], a["m"])
+            e = rel(y[:, col:col + a["m"]], want)
+            assert e < TOL, (a["m"], a["stages"], e)
+            col += a["m"]
+        return y
+
+    layer, arts = build([(256, 2), (64, 1), (96, 4)], n)
+    assert all(m["bd_meta"] is not None for m in layer._glq_shard_meta)
+    assert [m["n_stages"] for m in layer._glq_shard_meta] == [2, 1, 4]
+    assert ext._FOLD_STREAMS.holds(layer.Qidxs.get_shard(0))     # folded at load time
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * 0.5).to(torch.bfloat16).to(DEV)
+    y = check(layer, arts, n, x)
+    assert torch.equal(y, layer.apply(x))
+    if B == 1:                                                   # a captured first call of a fresh layer
+        fresh, _ = build([(256, 2), (64, 1), (96, 4)], n)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            yc = fresh.apply(x)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yc, y)
+    legacy, larts = build([(200, 2)], 300, legacy=True)          # buffers of 256 x 512
+    assert legacy._glq_shard_meta[0]["bd_meta"] is None and legacy._glq_shard_meta[0]["m_pad"] == 256
+    xl = (torch.randn(B, 300, generator=torch.Generator().manual_seed(B + 1)) * 0.5).half().to(DEV)
+    check(legacy, larts, 300, xl)
+    bad, _ = build([(64, 1)], n)
+    bad.inv_resid_scale._shard_data[0] = torch.tensor(0.3)
+    with pytest.raises(RuntimeError, match="half-configured"):
+        bad.process_weights_after_loading(DEV)

@@ -145,3 +145,19 @@ def test_merged_trellis_linear_host_side():
         MergedTrellisLinear.from_linears([])
     sh = GLQShards([torch.zeros(1), torch.ones(2)])
     assert len(sh) == 2 and sh.get_shard(1).numel() == 2
+
+
+def test_merged_shell_linear_host_side():
+    """Shard bookkeeping and refusals of the E8-shell merged-linear holder that need no GPU."""
+    import pytest
+    from glq_amd.linear_method import MergedShellLinear
+    table = torch.zeros(65536, 8, dtype=torch.float16)
+    layer = MergedShellLinear(960, [960, 320, 320], table)
+    assert layer.glq_is_fused and layer.glq_num_shards == 3 and not layer.glq_is_trellis
+    assert len(layer.Qidxs) == 3 and layer.Qidxs2.get_shard(1).numel() == 0 and layer.SU.get_shard(2).shape == (320,)
+    assert float(layer.inv_resid_scale3.get_shard(0)) == 0.0
+    assert not MergedShellLinear(512, [256], table).glq_is_fused
+    with pytest.raises(RuntimeError, match="process_weights_after_loading"):
+        layer.apply(torch.zeros(1, 960))
+    with pytest.raises(RuntimeError, match="E8-shell layers"):
+        MergedShellLinear.from_linears([])

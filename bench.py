@@ -444,7 +444,16 @@ def extras(torch, ext, dev):
         out["e8_2stage_linear_14336x4096_M32_us"] = round(_graph_time(torch, lambda: ext.glq_fused_linear_block_diag_cuda(
             xb, sv, su, q1, cbh, 0.02, n, m, n, m, bnt, bmt, bnm, bmm, q2, cbh, 1 / 3.0,
             out_dtype=torch.bfloat16), 1, reps=10), 1)
-        del p, q1, q2
+        # a stacked 6 bpw (4 + 2) layer of the same shape at 256 and 1024 tokens: both streams decoded into one
+        # operand by the decoding waves of the 256-token tiles
+        p2 = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 32), device=dev, dtype=torch.int16)
+        for M in (256, 1024):
+            xb = torch.randn(M, n, device=dev).to(torch.bfloat16)
+            us = _graph_time(torch, lambda: ext.glq_fused_linear_trellis_3inst_rvq2_cuda(
+                xb, sv, su, p, p2, bnt, bmt, bnm, bmm, 0.02, 0.25, n, m, n, m, out_dtype=torch.bfloat16), 1, reps=5)
+            out[f"trellis_linear_14336x4096_6bpw_M{M}_us"] = round(us, 1)
+            out[f"trellis_linear_14336x4096_6bpw_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
+        del p, p2, q1, q2
         torch.cuda.empty_cache()
     except Exception as e:
         out["prefill_linear_error"] = f"{type(e).__name__}: {e}"

@@ -36,6 +36,7 @@ _GLQ_BATCH_OUT_RHT = os.environ.get("GLQ_TRELLIS_BATCH_OUT_RHT", "1") != "0"
 # (stacked beyond one token, mixed, more than four) take it, and from 64 tokens on those run as whole fused
 # linears, concatenated.
 _GLQ_MERGED_GROUPED = os.environ.get("GLQ_MERGED_GROUPED", "1") != "0"
+_GROUP_MAX_SHARDS = 4                                          # layers per grouped call (GLQH_MAX_SHARDS)
 
 # Largest output block of the shard-batched transform.  The reference stops at 8192 (shared-memory
 # budget of its kernel, glq_vllm/linear_method.py:618-623); the kernel here cuts blocks into
@@ -212,13 +213,14 @@ class MergedTrellisLinear:
             return False
         if len({self.trellis_packed.get_shard(i).shape[1] for i in range(len(metas))}) != 1:
             return False
-        return B <= 4 or (B > 64 and len(metas) <= 4)
+        return len(metas) <= _GROUP_MAX_SHARDS and (B <= 4 or B > 64)
 
     def _grouped_rvq2_ok(self, B):
         """One token of merged stacked shards (first stages of 4 bpw, second stages of one rate): the library's
         grouped two-stage call."""
         metas = self._glq_trellis_meta
-        if B != 1 or not (self.glq_is_fused and all(m["loaded"] and m["has_s2"] for m in metas)):
+        if B != 1 or len(metas) > _GROUP_MAX_SHARDS or \
+                not (self.glq_is_fused and all(m["loaded"] and m["has_s2"] for m in metas)):
             return False
         n = range(len(metas))
         return ({self.trellis_packed.get_shard(i).shape[1] for i in n} == {64} and

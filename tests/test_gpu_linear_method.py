@@ -336,3 +336,16 @@ def test_merged_shell_linear(ops, B):
     bad.inv_resid_scale._shard_data[0] = torch.tensor(0.3)
     with pytest.raises(RuntimeError, match="half-configured"):
         bad.process_weights_after_loading(DEV)
+
+
+@pytest.mark.parametrize("B", [1, 3, 100])
+def test_more_shards_than_a_grouped_call_takes(ops, B):
+    """Five merged shards: the grouped call takes at most four layers, so the default falls back to the
+    reference's sequence (whole fused linears from 64 tokens on); against the oracle."""
+    say("merged linear, five shards", B)
+    n = 512
+    layer, arts = _merged(n, [(64, 4, 0)] * 5, 4)
+    assert not layer._grouped_ok(B)
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * 0.5).to(torch.bfloat16).to(DEV)
+    y = layer.apply(x)
+    assert y.shape == (B, 320) and rel(y, _oracle(x, arts, n)) < TOL

@@ -20,7 +20,7 @@ import os
 import torch
 
 from .hadamard import block_decompose, pack_block_meta, pack_shard_meta
-from .quantized_linear import E8RHTLinear
+from .quantized_linear import E8RHTLinear, _MAX_TOKENS_PER_CALL
 
 # GLQ_TRELLIS_BATCH_OUT_RHT=0 gives every shard its own output transform and concatenates
 # (glq_vllm/linear_method.py:616).
@@ -202,7 +202,12 @@ class MergedTrellisLinear:
             raise RuntimeError("process_weights_after_loading() must run before apply()")
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
-        y = self._apply_2d(x2)
+        if x2.shape[0] == 0:                                   # no tokens: nothing to launch
+            return x.new_empty(*shape[:-1], sum(self.glq_shard_sizes))
+        if x2.shape[0] > _MAX_TOKENS_PER_CALL:                 # the kernels' grids carry the token index in 16 bits
+            y = torch.cat([self._apply_2d(c) for c in x2.split(_MAX_TOKENS_PER_CALL)])
+        else:
+            y = self._apply_2d(x2)
         if bias is not None:
             y = y + bias.to(y.dtype)
         return y.reshape(*shape[:-1], y.shape[-1])
@@ -428,9 +433,15 @@ class MergedShellLinear:
             raise RuntimeError("process_weights_after_loading() must run before apply()")
         shape = x.shape
         x2 = x.reshape(-1, shape[-1])
+        if x2.shape[0] == 0:                                   # no tokens: nothing to launch
+            return x.new_empty(*shape[:-1], sum(self.glq_shard_sizes))
         xin = (x2 if x2.dtype in (torch.float16, torch.bfloat16) else x2.half()).contiguous()
-        outs = [self._apply_shard(xin, i) for i in range(self.glq_num_shards)]
-        y = outs[0] if len(outs) == 1 else torch.cat(outs, dim=-1)
+        chunks = xin.split(_MAX_TOKENS_PER_CALL)               # the kernels' grids carry the token index in 16 bits
+        rows = []
+        for c in chunks:
+            outs = [self._apply_shard(c, i) for i in range(self.glq_num_shards)]
+            rows.append(outs[0] if len(outs) == 1 else torch.cat(outs, dim=-1))
+        y = rows[0] if len(rows) == 1 else torch.cat(rows)
         if y.dtype != x.dtype:
             y = y.to(x.dtype)
         if bias is not None:

@@ -349,3 +349,28 @@ def test_more_shards_than_a_grouped_call_takes(ops, B):
     x = (torch.randn(B, n, generator=torch.Generator().manual_seed(B)) * 0.5).to(torch.bfloat16).to(DEV)
     y = layer.apply(x)
     assert y.shape == (B, 320) and rel(y, _oracle(x, arts, n)) < TOL
+
+
+def test_merged_linears_without_tokens_and_with_more_than_a_launch_takes(ops):
+    """An empty batch gives an empty result without a launch; more tokens than one call takes (32768, as in
+    E8RHTLinear.forward) are served in pieces: rows of the long call equal the rows of a short one."""
+    from glq_amd.linear_method import MergedShellLinear
+    from tests.gpu_util import e8_table_f16
+    say("merged linears, 0 and 70000 tokens")
+    n = 512
+    layer, _ = _merged(n, [(256, 4, 0), (64, 4, 0), (64, 4, 0)], 4)
+    two, _ = _merged(n, [(352, 4, 2), (352, 4, 2)], 6)
+    shell = MergedShellLinear(n, [128, 64], e8_table_f16())
+    from glq_amd.linear_method import GLQShards
+    shell.Qidxs = GLQShards(torch.from_numpy(_shell_indices(m, n, 1, m)[0].copy()) for m in (128, 64))
+    shell.Wscale = GLQShards(torch.tensor(0.02) for _ in range(2))
+    shell.process_weights_after_loading(DEV)
+    for L, width in ((layer, 384), (two, 704), (shell, 192)):
+        y0 = L.apply(torch.zeros(0, n, dtype=torch.bfloat16, device=DEV))
+        assert y0.shape == (0, width) and y0.dtype == torch.bfloat16
+        assert L.apply(torch.zeros(2, 0, n, dtype=torch.float16, device=DEV)).shape == (2, 0, width)
+        x = (torch.randn(70000, n, generator=torch.Generator().manual_seed(1)) * 0.5).to(torch.bfloat16).to(DEV)
+        y = L.apply(x)
+        assert y.shape == (70000, width) and bool(torch.isfinite(y.float()).all())
+        for lo in (0, 32763, 65535, 69990):
+            assert rel(y[lo:lo + 10], L.apply(x[lo:lo + 10]).float().cpu().numpy()) < 6e-3

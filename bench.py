@@ -314,7 +314,7 @@ def extras(torch, ext, dev):
         o = torch.empty(256, m, dtype=torch.float32, device=dev)
         us = _graph_time(torch, lambda: ext.glq_decode_matmul_trellis_3inst_cuda(xh, p, m, n, 1.0, out=o), 1, reps=10)
         out["trellis_prefill_14336x4096_M256_TFLOPs"] = round(2.0 * 256 * m * n / us / 1e6, 1)
-        mfma("tr_tile_kernel<4,2> + activation repack + K-slot sum", "configs[3]: trellis 4 bpw 14336x4096, 256 tokens",
+        mfma("tr_tile_pc_kernel<4,4> + activation repack + K-slot sum", "configs[3]: trellis 4 bpw 14336x4096, 256 tokens",
              2.0 * 256 * m * n, us)
         del p, xh, o
         torch.cuda.empty_cache()
@@ -376,7 +376,8 @@ def extras(torch, ext, dev):
             us = _graph_time(torch, lambda: ext.glq_dequant_matmul_cuda(xh, qs[0][0], cb, 0.02, qs[0][1], cb, 1 / 3.0),
                              1, reps=5)
             out[f"e8_2stage_matmul_4096x14336_M{M}_TFLOPs"] = round(2.0 * M * m * n / us / 1e6, 1)
-            mfma("e8_tile_kernel<2,FOLD> + activation repack + K-slot sum (matmul entry on transformed rows)",
+            mfma(("e8_tile_small_kernel<2,8,2>" if M <= 256 else "e8_tile_kernel<2,4,FOLD>") +
+                 " + activation repack + K-slot sum (matmul entry on transformed rows)",
                  f"configs[3]: E8 two-stage 4 bpw 4096x14336, {M} tokens", 2.0 * M * m * n, us)
         ext.E8_BATCH_MAX = e8_default
         del qs, i1, i2

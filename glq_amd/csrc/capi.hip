@@ -702,12 +702,16 @@ static bool tr_group_plain(int64_t total_m_pad, int64_t n_pad, int64_t B) {
     // ties); three and four tokens on q/k/v of a 3072-wide model lose 1-4 us folded (21.7 / 20.5, 24.4 / 20.2),
     // which the rule below does not catch.
     if (!tr_fuse_input_enabled()) return true;
+    if (B > 4) return true;                                  // 5..16 tokens: the fused-input launches serve up to four
     if (B == 1) return w > ((int64_t)96 << 20);
     return w > ((int64_t)48 << 20) || (B >= 3 && n_pad >= 4096 && w > ((int64_t)16 << 20));
 }
 // The grouped call at many tokens: more than 64 tokens, at most four layers.  The K split of a group is at most
 // that of a single 128-row layer of the same width (fewer row tiles, more slots).
 constexpr int64_t TR_GROUP_MANY_MIN = 64;
+// 5..16 tokens: one transform launch per distinct sign vector, one small-batch decode launch per layer under the
+// K plan of the tallest, one finishing launch for all layers (no K-slot sum launches, no shared fp32 buffer)
+constexpr int64_t TR_GROUP_SMALL_MAX = 16;
 constexpr int TR_GROUP_MANY_MAX = 4;
 constexpr int64_t TT_GROUP_ROWS_FLOOR = 128;
 
@@ -729,8 +733,18 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
         return (size_t)n_shards * (256 + align256(glqh_trellis_tile_xb_bytes(n_pad, B))) +
                align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ks * B * total_m_pad * sizeof(float));
     }
-    if (B < 1 || B > 4 || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64) return 0;
+    if (B < 1 || B > TR_GROUP_SMALL_MAX || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64)
+        return 0;
     glqh_init();
+    if (B > 4) {
+        // x_rht and the partial sums under the K plan of the tallest layer, which has at least total / n_shards
+        // rows (the plan's slot count does not grow with the rows)
+        int S = 0, ksb = 0;
+        const int64_t mmin = total_m_pad / n_shards / 32 * 32;
+        glqh_trellis_mma_plan(mmin < 32 ? 32 : mmin, n_pad, &S, &ksb);
+        return (size_t)n_shards * 256 + align256((size_t)B * n_pad * sizeof(f16)) +
+               align256((size_t)ksb * B * total_m_pad * sizeof(float));
+    }
     int steps = 0, ks = 0;
     // upper bound over how the rows may be split among the layers: the most workgroups (and
     // so the fewest K slots) arise from many short layers, the most slots from one tall layer
@@ -870,7 +884,8 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
     GLQH_REQUIRE(x && shards, "trellis group: null pointer");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis group: %d shards (1..%d)", n_shards,
                  GLQH_MAX_SHARDS);
-    GLQH_REQUIRE(B >= 1 && B <= 4, "trellis group: B=%lld (the grouped launch serves 1..4 tokens)", (long long)B);
+    GLQH_REQUIRE(B >= 1 && B <= TR_GROUP_SMALL_MAX, "trellis group: B=%lld (the grouped call serves 1..16 and more than 64 tokens)",
+                 (long long)B);
     GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis group: x must be f16 or bf16");
     GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad, "trellis group: in_features exceeds n_pad");
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;

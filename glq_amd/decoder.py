@@ -66,7 +66,7 @@ class _Linear:
 
 
 def _group(x, lins, separate=False):
-    """Layers that read the same activations: one decode launch (1..4 tokens) or one launch of the many-token
+    """Layers that read the same activations: one decode launch (1..4 tokens; 5..16: one per layer) or one launch of the many-token
     kernel (more than 64 tokens, separate=True: one contiguous tensor per layer) for all of them."""
     a = lins[0]
     return ext.glq_fused_linear_trellis_3inst_group(

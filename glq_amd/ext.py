@@ -395,7 +395,8 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
 
     shards: sequence of (sv, su, trellis_packed, wscale, out_features, m_pad).  Returns one
     (B, sum(out_features)) tensor, shard s in columns [off_s, off_s + out_features_s).
-    Needs 1..4 tokens (any number of layers up to 8) or more than 64 (up to four layers: one launch of
+    Needs 1..16 tokens (up to four layers; 5..16: one decode launch per layer between one transform launch per
+    sign vector and one finishing launch) or more than 64 (up to four layers: one launch of
     the many-token kernel over the row tiles of all of them), single-stage layers of one rate and
     block_decompose block sizes; raises RuntimeError otherwise (callers then use the per-layer op).
     decode_only=True stops after the decode launch (no output transform, returns None): a measurement

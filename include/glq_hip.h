@@ -201,11 +201,14 @@ size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad,
  * rounding of a different K split.  Single-stage layers of one rate R, at most 4 tokens,
  * canonical (block_decompose) output block sizes; anything else is refused and the caller
  * falls back to per-layer calls.
+ * 5..16 tokens: one input transform per distinct sign vector, one small-batch decode launch per layer
+ * under the K plan of the tallest, and one output-transform launch for all layers (no K-slot sums, no
+ * shared fp32 buffer in between).
  * More than 64 tokens (up to four layers, every y given): one input transform per distinct sign
  * vector, ONE launch of the many-token kernel over the row tiles of all layers (small layers do not
  * fill the chip one by one) and one output transform per layer.  y_stride 0 there: every layer's rows
  * are packed (row stride = its out_features), so that each layer's output is a contiguous matrix.
- * 5..64 tokens are refused. */
+ * 17..64 tokens are refused. */
 int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
                                           const glqh_trellis_shard *shards, int n_shards,
                                           const int64_t *blocks_n, int64_t n_blocks_n,

@@ -190,11 +190,11 @@ def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, s
         assert rel(static_y, _oracle(x, arts, n)) < TOL
 
 
-@pytest.mark.parametrize("B", [2, 100])
+@pytest.mark.parametrize("B", [2, 7, 16, 100])
 def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
     """Single-stage merged shards through the library's grouped call, the default (one decode launch at
-    1-4 tokens, one launch of the many-token kernel above 64) against the oracle and against the default sequence
-    of registered ops; token counts in between and two-stage shards keep the default sequence."""
+    1-4 tokens, one per shard at 5-16, one launch of the many-token kernel above 64) against the oracle and against
+    the reference's sequence of registered ops; token counts in between and two-stage shards keep that sequence."""
     from glq_amd import linear_method as LM
     say("merged linear, grouped call", B)
     n = 512

@@ -756,7 +756,17 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
     if (tr_group_plain(total_m_pad, n_pad, B))
         plain = align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)64 * B * total_m_pad * sizeof(float));
     const size_t fused = align256((size_t)ks * B * total_m_pad * sizeof(float));
-    return (size_t)n_shards * 256 + (plain > fused ? plain : fused);
+    // (2..4 tokens of stacked layers, glqh_fused_linear_trellis_3inst_group_rvq2: x_rht and the sums under the K
+    // plan of the tallest layer, which has at least total / n_shards rows)
+    size_t stacked = 0;
+    if (B > 1) {
+        int S = 0, ksb = 0;
+        const int64_t mmin = total_m_pad / n_shards / 32 * 32;
+        glqh_trellis_mma_plan(mmin < 32 ? 32 : mmin, n_pad, &S, &ksb);
+        stacked = align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ksb * B * total_m_pad * sizeof(float));
+    }
+    const size_t most = plain > fused ? plain : fused;
+    return (size_t)n_shards * 256 + (stacked > most ? stacked : most);
 }
 
 // Decode launch of a group: checks, K plan, partial-sum layout in ws.  On return parts[i] holds
@@ -1000,7 +1010,8 @@ extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_d
     GLQH_REQUIRE(x && shards && stage2, "trellis two-stage group: null pointer");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis two-stage group: %d shards (1..%d)", n_shards,
                  GLQH_MAX_SHARDS);
-    GLQH_REQUIRE(B == 1, "trellis two-stage group: B=%lld (the grouped two-stage launch serves one token)", (long long)B);
+    GLQH_REQUIRE(B >= 1 && B <= TR_GROUP_SMALL_MAX, "trellis two-stage group: B=%lld (the grouped two-stage call serves 1..16 tokens)",
+                 (long long)B);
     GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis two-stage group: x must be f16 or bf16");
     GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad, "trellis two-stage group: in_features exceeds n_pad");
     GLQH_REQUIRE(y_stride > 0, "trellis two-stage group: y_stride must be positive");
@@ -1042,6 +1053,33 @@ extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_d
         total += sh.m_pad;
     }
     int steps = 0, ks = 0;
+    if (B > 1) {
+        // 2..16 tokens: one transform launch per distinct sign vector, one small-batch launch per layer that decodes
+        // both streams against the staged activations, under the K plan of the tallest layer, one finishing launch
+        int64_t mmax = 0;
+        for (int i = 0; i < n_shards; ++i) mmax = c.m_pads[i] > mmax ? c.m_pads[i] : mmax;
+        int S = 0;
+        glqh_trellis_mma_plan(mmax, n_pad, &S, &ks);
+        const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
+        const size_t need = xb + align256((size_t)ks * B * total * sizeof(float));
+        GLQH_REQUIRE(ws && ws_bytes >= need, "trellis two-stage group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+        f16 *x_rht = (f16 *)ws;
+        float *p = (float *)((char *)ws + xb);
+        for (int i = 0; i < n_shards; ++i) {
+            if ((i == 0 || sv[i] != sv[i - 1]) &&
+                glqh_launch_input_rht(x, x_dtype, x_stride, sv[i], x_rht, GLQH_F16, B, in_features, n_pad, bn_meta_dev,
+                                      blocks_n, n_blocks_n, 0.0f, st))
+                return 1;
+            c.parts[i] = p;
+            p += (size_t)ks * B * c.m_pads[i];
+            glqh_range range("dequant_matmul");
+            if (glqh_launch_trellis_mma_rvq(x_rht, B, packed[i], packed2[i], R2, rs2[i], c.m_pads[i], n_pad, S, ks,
+                                            c.parts[i], st))
+                return 1;
+        }
+        return glqh_launch_output_rht_group(c.parts, c.su, c.ys, c.scale, c.m_pads, c.outs, n_shards, y_dtype, y_stride,
+                                            B, ks, st);
+    }
     GLQH_REQUIRE(tr_fuse_input_enabled() && tr_fusein_plan(c.m_pads, n_shards, n_pad, 1, &steps, &ks, 1) == 2,
                  "trellis two-stage group: shape not eligible");
     const size_t need = align256((size_t)ks * total * sizeof(float));

@@ -448,12 +448,14 @@ class _TrellisStage2(C.Structure):
 
 def glq_fused_linear_trellis_3inst_group_rvq2(x, shards, blocks_n, blocks_n_meta, in_features, n_pad,
                                               out_dtype=None):
-    """The grouped call for stacked (two-stage) layers at one token: the decode step of fused q/k/v or
+    """The grouped call for stacked (two-stage) layers at 1..16 tokens: the decode step of fused q/k/v or
     gate/up of a 5-8 bpw checkpoint, whose per-shard loop in the reference is
     fused_linear_trellis_3inst_yrht_rvq2 per shard + output_rht_shards (glq_vllm/linear_method.py:664-710).
+    One token: one decode launch for both streams of every shard; 2..16: one transform launch per distinct
+    sign vector and one decode launch per shard; one finishing launch either way.
 
     shards: sequence of (sv, su, trellis_packed, trellis_packed2, wscale, inv_resid_scale2, out_features,
-    m_pad); first stages of 4 bpw, second stages of one common rate.  Returns (1, sum(out_features)).
+    m_pad); first stages of 4 bpw, second stages of one common rate.  Returns (B, sum(out_features)).
     Raises RuntimeError for other token counts or rates (callers then use the per-layer op)."""
     lib = _lib.load()
     _chk(x, "x", (torch.float16, torch.bfloat16))
@@ -479,7 +481,7 @@ def glq_fused_linear_trellis_3inst_group_rvq2(x, shards, blocks_n, blocks_n_meta
         off += int(out_f)
     bn, nbn = _host_i64(blocks_n)
     with torch.cuda.device(x.device):
-        nb = lib.glqh_fused_linear_trellis_group_workspace_bytes(1, int(n_pad), total_m, len(shards))
+        nb = lib.glqh_fused_linear_trellis_group_workspace_bytes(B, int(n_pad), total_m, len(shards))
         ws = _ws(max(nb, 256), x.device)
         check(lib.glqh_fused_linear_trellis_3inst_group_rvq2(
             _p(x), _DT[x.dtype], x.shape[1], B, C.addressof(arr), C.addressof(arr2), len(shards), bn, nbn,

@@ -225,12 +225,14 @@ typedef struct {
     double inv_resid_scale2;
 } glqh_trellis_stage2;
 
-/* The grouped call for stacked layers at ONE token (the decode step of fused q/k/v and gate/up of a
+/* The grouped call for stacked layers at 1..16 tokens (at one token the decode step of fused q/k/v and gate/up of a
  * 5-8 bits/weight checkpoint; the reference runs fused_linear_trellis_3inst_yrht_rvq2 per shard,
  * glq_vllm/linear_method.py:664-710): one decode launch reads both streams of every layer (first
  * stages of 4 bits/weight, second stages of one common rate, stage2[i] belongs to shards[i]) and one
- * launch finishes them.  Workspace: glqh_fused_linear_trellis_group_workspace_bytes(1, ...).  Every
- * shard's y must be given; other token counts and rates are refused (per-layer calls serve them). */
+ * launch finishes them.  2..16 tokens: one input transform per distinct sign vector, one small-batch
+ * launch per layer that decodes both streams, one finishing launch.  Workspace:
+ * glqh_fused_linear_trellis_group_workspace_bytes(B, ...).  Every shard's y must be given; other token
+ * counts and rates are refused (per-layer calls serve them). */
 int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_dtype, int64_t x_stride, int64_t B,
                                                const glqh_trellis_shard *shards,
                                                const glqh_trellis_stage2 *stage2, int n_shards,

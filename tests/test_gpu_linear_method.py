@@ -214,25 +214,27 @@ def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
 
 @pytest.mark.parametrize("n,shards,bpw", [(512, [(352, 4, 2), (352, 4, 2)], 6), (2048, [(2048, 4, 1), (512, 4, 1), (512, 4, 1)], 5),
                                           (576, [(1184, 4, 4), (1184, 4, 4)], 8)])
-def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, shards, bpw):
+@pytest.mark.parametrize("B", [1, 2, 9, 16])
+def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, shards, bpw, B):
     """One token of merged stacked shards (5, 6, 8 bpw = 4 + 1, 2, 4) through the library's grouped
-    two-stage call (one decode launch for both streams of every shard, one finishing launch) against the oracle
-    and against the default sequence of registered ops; more tokens keep the default sequence."""
+    two-stage call (one token: one decode launch for both streams of every shard; 2-16: one per shard; one
+    finishing launch) against the oracle and against the reference's sequence of registered ops; more tokens keep
+    that sequence."""
     from glq_amd import linear_method as LM
-    say("merged two-stage linear, grouped call", n, bpw)
+    say("merged two-stage linear, grouped call", n, bpw, B)
     layer, arts = _merged(n, shards, bpw)
-    x = (torch.randn(1, n, generator=torch.Generator().manual_seed(n)) * 0.5).to(torch.bfloat16).to(DEV)
+    x = (torch.randn(B, n, generator=torch.Generator().manual_seed(n + B)) * 0.5).to(torch.bfloat16).to(DEV)
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
     y_ref = layer.apply(x)
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
-    assert layer._grouped_rvq2_ok(1) and not layer._grouped_rvq2_ok(2) and not layer._grouped_ok(1)
+    assert layer._grouped_rvq2_ok(B) and not layer._grouped_rvq2_ok(17) and not layer._grouped_ok(B)
     y = layer.apply(x)
     assert y.dtype == x.dtype and y.shape == y_ref.shape
     assert rel(y, _oracle(x, arts, n)) < TOL
     assert rel(y, y_ref.float().cpu().numpy()) < 6e-3
     assert torch.equal(y, layer.apply(x))
     mixed, _ = _merged(512, [(352, 4, 2), (352, 4, 1)], 6)
-    assert not mixed._grouped_rvq2_ok(1)
+    assert not mixed._grouped_rvq2_ok(B)
 
 
 @pytest.mark.parametrize("B", [64, 200])

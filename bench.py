@@ -301,7 +301,32 @@ def extras(torch, ext, dev):
         out["trellis_group_qkv_4096_6bpw_B1_us"] = round(_graph_time(
             torch, lambda: [ext.glq_fused_linear_trellis_3inst_group_rvq2(xb, sh, bnt, bnm, n, n, out_dtype=torch.bfloat16)
                             for sh in groups], len(groups)), 2)
+        xb8 = torch.randn(8, n, device=dev).to(torch.bfloat16)
+        out["trellis_group_qkv_4096_6bpw_B8_us"] = round(_graph_time(
+            torch, lambda: [ext.glq_fused_linear_trellis_3inst_group_rvq2(xb8, sh, bnt, bnm, n, n, out_dtype=torch.bfloat16)
+                            for sh in groups], len(groups)), 2)
         del p4, p2, groups
+        # the merged linear of the serving layer (fused q/k/v of a 2048-wide 4 bpw model) at 8 and 512 tokens: the
+        # library's grouped calls, its default, against the reference's per-shard op sequence
+        try:
+            from glq_amd import custom_ops, linear_method as LM
+            custom_ops.register()
+            nq = 2048
+            ml = LM.MergedTrellisLinear(nq, [2048, 512, 512], bpw=4)
+            ml.trellis_packed = LM.GLQShards(torch.randint(-32768, 32768, ((r // 16) * (nq // 16), 64), dtype=torch.int16)
+                                             for r in (2048, 512, 512))
+            ml.Wscale = LM.GLQShards(torch.tensor(0.02) for _ in range(3))
+            ml.process_weights_after_loading(dev)
+            for Bm in (8, 512):
+                xm = torch.randn(Bm, nq, device=dev).to(torch.bfloat16)
+                for tag, grouped in (("", True), ("_reference_sequence", False)):
+                    LM._GLQ_MERGED_GROUPED = grouped
+                    out[f"merged_qkv_2048_4bpw_B{Bm}{tag}_us"] = round(_graph_time(
+                        torch, lambda: [ml.apply(xm) for _ in range(10)], 10, reps=5), 2)
+            LM._GLQ_MERGED_GROUPED = True
+            del ml
+        except Exception as e:
+            out["merged_linear_error"] = f"{type(e).__name__}: {e}"
         m, n, M = 14336, 4096, 4096
         p = torch.randint(-32768, 32768, ((m // 16) * (n // 16), 64), device=dev, dtype=torch.int16)
         xh = torch.randn(M, n, device=dev).to(torch.float16)

@@ -733,9 +733,17 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
         return (size_t)n_shards * (256 + align256(glqh_trellis_tile_xb_bytes(n_pad, B))) +
                align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ks * B * total_m_pad * sizeof(float));
     }
-    if (B < 1 || B > TR_GROUP_SMALL_MAX || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64)
+    if (B < 1 || B > TR_GROUP_MANY_MIN || n_shards < 1 || n_shards > GLQH_MAX_SHARDS || total_m_pad < 32 || n_pad < 64)
         return 0;
     glqh_init();
+    if (B > TR_GROUP_SMALL_MAX) {
+        // 17..64 tokens: blocked and row-major activations and every layer's sums under its own K plan, bounded by
+        // the plan of a 128-row layer (fewer row tiles, more slots)
+        const int ks1 = glqh_trellis_tile_ksplit(TT_GROUP_ROWS_FLOOR, n_pad, B), ks2 = glqh_trellis_tile_ksplit(TT_GROUP_ROWS_FLOOR, n_pad, B, 1);
+        const int ksb = ks1 > ks2 ? ks1 : ks2;                 // (single-stage and stacked layers)
+        return (size_t)n_shards * 256 + align256(glqh_trellis_tile_xb_bytes(n_pad, B)) +
+               align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ksb * B * total_m_pad * sizeof(float));
+    }
     if (B > 4) {
         // x_rht and the partial sums under the K plan of the tallest layer, which has at least total / n_shards
         // rows (the plan's slot count does not grow with the rows)
@@ -880,12 +888,37 @@ static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B
 
 struct tr_group_ctx {
     int R, ks, fi_mode;
+    int ks_layer[GLQH_MAX_SHARDS];                             // 17..64 tokens: every layer's own slot count (ks = 0 when they differ)
     int64_t m_pads[GLQH_MAX_SHARDS], outs[GLQH_MAX_SHARDS];
     const void *su[GLQH_MAX_SHARDS];
     void *ys[GLQH_MAX_SHARDS];
     float scale[GLQH_MAX_SHARDS];
     float *parts[GLQH_MAX_SHARDS];
 };
+
+// One finishing launch for all layers of a group; at 17..64 tokens, where every layer has its own K plan, one per
+// layer when their slot counts differ.
+static int tr_group_finish(const tr_group_ctx &c, int n_shards, int64_t B, int y_dtype, int64_t y_stride, hipStream_t st) {
+    if (B > TR_GROUP_SMALL_MAX && c.ks == 0) {
+        for (int i = 0; i < n_shards; ++i) {
+            glqh_ysrc src = {};
+            src.nparts = 1;
+            src.part = c.parts[i];
+            src.part_kstride = B * c.m_pads[i];
+            src.ksplit = c.ks_layer[i];
+            src.scale[0] = c.scale[i];
+            if (glqh_launch_output_rht_canon_wide(src, c.su[i], c.ys[i], y_dtype, y_stride, B, c.outs[i], c.m_pads[i], st) != 0) {
+                const float *pt[1] = {c.parts[i]};
+                if (glqh_launch_output_rht_group(pt, &c.su[i], &c.ys[i], &c.scale[i], &c.m_pads[i], &c.outs[i], 1, y_dtype,
+                                                 y_stride, B, c.ks_layer[i], st))
+                    return 1;
+            }
+        }
+        return 0;
+    }
+    return glqh_launch_output_rht_group(c.parts, c.su, c.ys, c.scale, c.m_pads, c.outs, n_shards, y_dtype, y_stride,
+                                        B, c.ks, st);
+}
 
 static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t B,
                            const glqh_trellis_shard *shards, int n_shards, const int64_t *blocks_n,
@@ -894,8 +927,7 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
     GLQH_REQUIRE(x && shards, "trellis group: null pointer");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis group: %d shards (1..%d)", n_shards,
                  GLQH_MAX_SHARDS);
-    GLQH_REQUIRE(B >= 1 && B <= TR_GROUP_SMALL_MAX, "trellis group: B=%lld (the grouped call serves 1..16 and more than 64 tokens)",
-                 (long long)B);
+    GLQH_REQUIRE(B >= 1 && B <= TR_GROUP_MANY_MIN, "trellis group: B=%lld", (long long)B);
     GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis group: x must be f16 or bf16");
     GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad, "trellis group: in_features exceeds n_pad");
     const bool pow2_n = (n_pad & (n_pad - 1)) == 0;
@@ -931,6 +963,42 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
         total += sh.m_pad;
     }
     int steps = 0, ks = 0;
+    if (B > TR_GROUP_SMALL_MAX) {
+        // 17..64 tokens: one transform launch per distinct sign vector, straight into the tile kernel's layout where
+        // it can, one launch of the small-tile kernel per layer (its own K plan), sums left for the finishing launch
+        const size_t xbb = align256(glqh_trellis_tile_xb_bytes(n_pad, B)), xrm = align256((size_t)B * n_pad * sizeof(f16));
+        size_t sums = 0;
+        bool same = true;
+        for (int i = 0; i < n_shards; ++i) {
+            c->ks_layer[i] = glqh_trellis_tile_ksplit(c->m_pads[i], n_pad, B);
+            same = same && c->ks_layer[i] == c->ks_layer[0];
+            sums += align256((size_t)c->ks_layer[i] * B * c->m_pads[i] * sizeof(float));
+        }
+        const size_t need = xbb + xrm + sums;
+        GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+        void *xb = ws;
+        f16 *x_rht = (f16 *)((char *)ws + xbb);
+        char *p = (char *)ws + xbb + xrm;
+        c->R = R; c->ks = same ? c->ks_layer[0] : 0; c->fi_mode = 0;
+        int blocked = -1;
+        for (int i = 0; i < n_shards; ++i) {
+            if (i == 0 || sv[i] != sv[i - 1]) {
+                blocked = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, sv[i], xb, 2, glqh_trellis_tile_padded_tokens(B),
+                                                        B, in_features, n_pad, blocks_n, n_blocks_n, st);
+                if (blocked > 0) return 1;
+                if (blocked != 0 && glqh_launch_input_rht(x, x_dtype, x_stride, sv[i], x_rht, GLQH_F16, B, in_features, n_pad,
+                                                          bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
+                    return 1;
+            }
+            c->parts[i] = (float *)p;
+            p += align256((size_t)c->ks_layer[i] * B * c->m_pads[i] * sizeof(float));
+            glqh_range range("dequant_matmul");
+            if (glqh_launch_trellis_tile(blocked == 0 ? nullptr : x_rht, xb, B, packed[i], R, c->m_pads[i], n_pad, c->parts[i],
+                                         0, 1.0f, 0, 0, st, 0))
+                return 1;
+        }
+        return 0;
+    }
     if (tr_group_plain(total, n_pad, B)) {
         // one K plan for all layers (that of the tallest), so that the finishing launch sees one slot count
         int64_t mmax = 0;
@@ -992,8 +1060,7 @@ extern "C" int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype,
                         n_pad, ws, ws_bytes, st, &c))
         return 1;
     if (!shards[0].y) return 0;                                // decode launch only: partial sums stay in ws
-    return glqh_launch_output_rht_group(c.parts, c.su, c.ys, c.scale, c.m_pads, c.outs, n_shards, y_dtype, y_stride,
-                                        B, c.ks, st);
+    return tr_group_finish(c, n_shards, B, y_dtype, y_stride, st);
 }
 
 // The same for stacked (two-stage) layers at one token: every layer's two streams decoded by one launch
@@ -1010,7 +1077,7 @@ extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_d
     GLQH_REQUIRE(x && shards && stage2, "trellis two-stage group: null pointer");
     GLQH_REQUIRE(n_shards >= 1 && n_shards <= GLQH_MAX_SHARDS, "trellis two-stage group: %d shards (1..%d)", n_shards,
                  GLQH_MAX_SHARDS);
-    GLQH_REQUIRE(B >= 1 && B <= TR_GROUP_SMALL_MAX, "trellis two-stage group: B=%lld (the grouped two-stage call serves 1..16 tokens)",
+    GLQH_REQUIRE(B >= 1 && B <= TR_GROUP_MANY_MIN, "trellis two-stage group: B=%lld (the grouped two-stage call serves 1..64 tokens)",
                  (long long)B);
     GLQH_REQUIRE(x_dtype == GLQH_F16 || x_dtype == GLQH_BF16, "trellis two-stage group: x must be f16 or bf16");
     GLQH_REQUIRE(in_features >= 1 && in_features <= n_pad, "trellis two-stage group: in_features exceeds n_pad");
@@ -1053,6 +1120,43 @@ extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_d
         total += sh.m_pad;
     }
     int steps = 0, ks = 0;
+    if (B > TR_GROUP_SMALL_MAX) {
+        // 17..64 tokens: one transform launch per distinct sign vector, one launch of the small-tile kernel per layer,
+        // which decodes both streams into one operand, finishing as for single-stage layers
+        GLQH_REQUIRE(tr_fuse_stages_enabled(), "trellis two-stage group: more than 16 tokens need both streams in one operand");
+        const size_t xbb = align256(glqh_trellis_tile_xb_bytes(n_pad, B)), xrm = align256((size_t)B * n_pad * sizeof(f16));
+        size_t sums = 0;
+        bool same = true;
+        for (int i = 0; i < n_shards; ++i) {
+            c.ks_layer[i] = glqh_trellis_tile_ksplit(c.m_pads[i], n_pad, B, 1);
+            same = same && c.ks_layer[i] == c.ks_layer[0];
+            sums += align256((size_t)c.ks_layer[i] * B * c.m_pads[i] * sizeof(float));
+        }
+        const size_t need = xbb + xrm + sums;
+        GLQH_REQUIRE(ws && ws_bytes >= need, "trellis two-stage group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
+        void *xb = ws;
+        f16 *x_rht = (f16 *)((char *)ws + xbb);
+        char *p = (char *)ws + xbb + xrm;
+        c.ks = same ? c.ks_layer[0] : 0;
+        int blocked = -1;
+        for (int i = 0; i < n_shards; ++i) {
+            if (i == 0 || sv[i] != sv[i - 1]) {
+                blocked = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, sv[i], xb, 2, glqh_trellis_tile_padded_tokens(B),
+                                                        B, in_features, n_pad, blocks_n, n_blocks_n, st);
+                if (blocked > 0) return 1;
+                if (blocked != 0 && glqh_launch_input_rht(x, x_dtype, x_stride, sv[i], x_rht, GLQH_F16, B, in_features, n_pad,
+                                                          bn_meta_dev, blocks_n, n_blocks_n, 0.0f, st))
+                    return 1;
+            }
+            c.parts[i] = (float *)p;
+            p += align256((size_t)c.ks_layer[i] * B * c.m_pads[i] * sizeof(float));
+            glqh_range range("dequant_matmul");
+            if (glqh_launch_trellis_tile(blocked == 0 ? nullptr : x_rht, xb, B, packed[i], 4, c.m_pads[i], n_pad, c.parts[i], 0,
+                                         1.0f, 0, 0, st, 0, packed2[i], R2, rs2[i]))
+                return 1;
+        }
+        return tr_group_finish(c, n_shards, B, y_dtype, y_stride, st);
+    }
     if (B > 1) {
         // 2..16 tokens: one transform launch per distinct sign vector, one small-batch launch per layer that decodes
         // both streams against the staged activations, under the K plan of the tallest layer, one finishing launch

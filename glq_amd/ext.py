@@ -395,10 +395,10 @@ def glq_fused_linear_trellis_3inst_group(x, shards, blocks_n, blocks_n_meta, in_
 
     shards: sequence of (sv, su, trellis_packed, wscale, out_features, m_pad).  Returns one
     (B, sum(out_features)) tensor, shard s in columns [off_s, off_s + out_features_s).
-    Needs 1..16 tokens (up to four layers; 5..16: one decode launch per layer between one transform launch per
-    sign vector and one finishing launch) or more than 64 (up to four layers: one launch of
-    the many-token kernel over the row tiles of all of them), single-stage layers of one rate and
-    block_decompose block sizes; raises RuntimeError otherwise (callers then use the per-layer op).
+    Up to four layers.  1..4 tokens: one decode launch; 5..64: one decode launch per layer (the small-batch
+    kernel to 16 tokens, the small-tile kernel above) between one transform launch per sign vector and one
+    finishing launch; more than 64: one launch of the many-token kernel over the row tiles of all of them.
+    Single-stage layers of one rate and block_decompose block sizes; raises RuntimeError otherwise (callers then use the per-layer op).
     decode_only=True stops after the decode launch (no output transform, returns None): a measurement
     hook.  separate=True (more than 64 tokens): a list of contiguous (B, out_features_s) tensors instead."""
     lib = _lib.load()
@@ -448,11 +448,12 @@ class _TrellisStage2(C.Structure):
 
 def glq_fused_linear_trellis_3inst_group_rvq2(x, shards, blocks_n, blocks_n_meta, in_features, n_pad,
                                               out_dtype=None):
-    """The grouped call for stacked (two-stage) layers at 1..16 tokens: the decode step of fused q/k/v or
+    """The grouped call for stacked (two-stage) layers at 1..64 tokens: the decode step of fused q/k/v or
     gate/up of a 5-8 bpw checkpoint, whose per-shard loop in the reference is
     fused_linear_trellis_3inst_yrht_rvq2 per shard + output_rht_shards (glq_vllm/linear_method.py:664-710).
-    One token: one decode launch for both streams of every shard; 2..16: one transform launch per distinct
-    sign vector and one decode launch per shard; one finishing launch either way.
+    One token: one decode launch for both streams of every shard; 2..64: one transform launch per distinct
+    sign vector and one decode launch per shard (the small-batch kernel to 16 tokens, the small-tile kernel
+    above); one finishing launch either way.
 
     shards: sequence of (sv, su, trellis_packed, trellis_packed2, wscale, inv_resid_scale2, out_features,
     m_pad); first stages of 4 bpw, second stages of one common rate.  Returns (B, sum(out_features)).

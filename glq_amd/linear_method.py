@@ -27,14 +27,14 @@ from .quantized_linear import E8RHTLinear, _MAX_TOKENS_PER_CALL
 _GLQ_BATCH_OUT_RHT = os.environ.get("GLQ_TRELLIS_BATCH_OUT_RHT", "1") != "0"
 # Merged single-stage shards go through the library's grouped call (one decode or many-token launch for all
 # shards at 1-4 and at more than 64 tokens, one decode launch per shard between one transform launch per sign
-# vector and one finishing launch at 5-16), merged two-stage shards at 1-16 tokens through its two-stage form:
+# vector and one finishing launch at 5-64), merged two-stage shards at 1-64 tokens through its two-stage form:
 # same result up to the rounding of another K split.  Whole merged linear, reference op sequence / grouped call,
 # us: q/k/v of a 2048-wide model 39.5 / 31.3 at one token, 52.5 / 36.0 at 4, 68.5 / 45.4 at 128, 95.3 / 52.7 at
 # 512; gate/up 2048 -> 2 x 11008 39.9 / 33.7, 43.7 / 37.7, 122 / 74, 277 / 108 (756 / 279 at 2048 tokens); q/k/v
 # of a 4096-wide 6 bpw model at one token 55.1 / 36.7.  GLQ_MERGED_GROUPED=0 keeps the reference's per-shard
 # sequence (fused_linear_trellis_3inst_yrht per shard + output_rht_shards, glq_vllm/linear_method.py:664-710)
-# at every token count; otherwise 17-63 tokens and, up to 63 tokens, shards the grouped call does not take
-# (stacked beyond 16 tokens, mixed, more than four) take it, and from 64 tokens on those run as whole fused
+# at every token count; otherwise, up to 63 tokens, shards the grouped call does not take
+# (mixed, more than four) take it, and from 64 tokens on those run as whole fused
 # linears, concatenated.
 _GLQ_MERGED_GROUPED = os.environ.get("GLQ_MERGED_GROUPED", "1") != "0"
 _GROUP_MAX_SHARDS = 4                                          # layers per grouped call (GLQH_MAX_SHARDS)
@@ -219,13 +219,13 @@ class MergedTrellisLinear:
             return False
         if len({self.trellis_packed.get_shard(i).shape[1] for i in range(len(metas))}) != 1:
             return False
-        return len(metas) <= _GROUP_MAX_SHARDS and (B <= 16 or B > 64)
+        return len(metas) <= _GROUP_MAX_SHARDS
 
     def _grouped_rvq2_ok(self, B):
-        """Up to 16 tokens of merged stacked shards (first stages of 4 bpw, second stages of one rate): the
+        """Up to 64 tokens of merged stacked shards (first stages of 4 bpw, second stages of one rate): the
         library's grouped two-stage call."""
         metas = self._glq_trellis_meta
-        if B < 1 or B > 16 or len(metas) > _GROUP_MAX_SHARDS or \
+        if B < 1 or B > 64 or len(metas) > _GROUP_MAX_SHARDS or \
                 not (self.glq_is_fused and all(m["loaded"] and m["has_s2"] for m in metas)):
             return False
         n = range(len(metas))

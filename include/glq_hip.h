@@ -201,14 +201,15 @@ size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int64_t n_pad,
  * rounding of a different K split.  Single-stage layers of one rate R, at most 4 tokens,
  * canonical (block_decompose) output block sizes; anything else is refused and the caller
  * falls back to per-layer calls.
- * 5..16 tokens: one input transform per distinct sign vector, one small-batch decode launch per layer
- * under the K plan of the tallest, and one output-transform launch for all layers (no K-slot sums, no
- * shared fp32 buffer in between).
+ * 5..64 tokens: one input transform per distinct sign vector, one decode launch per layer (the small-batch
+ * kernel under the K plan of the tallest up to 16 tokens, the small-tile kernel under its own plan above)
+ * and one output-transform launch for all layers, or one per layer where their K plans differ (no K-slot
+ * sum launches, no shared fp32 buffer in between).
  * More than 64 tokens (up to four layers, every y given): one input transform per distinct sign
  * vector, ONE launch of the many-token kernel over the row tiles of all layers (small layers do not
  * fill the chip one by one) and one output transform per layer.  y_stride 0 there: every layer's rows
  * are packed (row stride = its out_features), so that each layer's output is a contiguous matrix.
- * 17..64 tokens are refused. */
+ */
 int glqh_fused_linear_trellis_3inst_group(const void *x, int x_dtype, int64_t x_stride, int64_t B,
                                           const glqh_trellis_shard *shards, int n_shards,
                                           const int64_t *blocks_n, int64_t n_blocks_n,
@@ -225,12 +226,13 @@ typedef struct {
     double inv_resid_scale2;
 } glqh_trellis_stage2;
 
-/* The grouped call for stacked layers at 1..16 tokens (at one token the decode step of fused q/k/v and gate/up of a
+/* The grouped call for stacked layers at 1..64 tokens (at one token the decode step of fused q/k/v and gate/up of a
  * 5-8 bits/weight checkpoint; the reference runs fused_linear_trellis_3inst_yrht_rvq2 per shard,
  * glq_vllm/linear_method.py:664-710): one decode launch reads both streams of every layer (first
  * stages of 4 bits/weight, second stages of one common rate, stage2[i] belongs to shards[i]) and one
- * launch finishes them.  2..16 tokens: one input transform per distinct sign vector, one small-batch
- * launch per layer that decodes both streams, one finishing launch.  Workspace:
+ * launch finishes them.  2..64 tokens: one input transform per distinct sign vector, one launch per layer
+ * that decodes both streams (the small-batch kernel to 16 tokens, the small-tile kernel above), one
+ * finishing launch.  Workspace:
  * glqh_fused_linear_trellis_group_workspace_bytes(B, ...).  Every shard's y must be given; other token
  * counts and rates are refused (per-layer calls serve them). */
 int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_dtype, int64_t x_stride, int64_t B,

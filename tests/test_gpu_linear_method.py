@@ -190,11 +190,11 @@ def test_s4b_sequence_captured_in_a_graph_replays_on_new_activations(ops, bpw, s
         assert rel(static_y, _oracle(x, arts, n)) < TOL
 
 
-@pytest.mark.parametrize("B", [2, 7, 16, 100])
+@pytest.mark.parametrize("B", [2, 7, 16, 30, 64, 100])
 def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
     """Single-stage merged shards through the library's grouped call, the default (one decode launch at
-    1-4 tokens, one per shard at 5-16, one launch of the many-token kernel above 64) against the oracle and against
-    the reference's sequence of registered ops; token counts in between and two-stage shards keep that sequence."""
+    1-4 tokens, one per shard at 5-64, one launch of the many-token kernel above 64) against the oracle and against
+    the reference's sequence of registered ops; two-stage shards take their own grouped call or that sequence."""
     from glq_amd import linear_method as LM
     say("merged linear, grouped call", B)
     n = 512
@@ -203,7 +203,7 @@ def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
     y_ref = layer.apply(x)
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
-    assert layer._grouped_ok(B) and not layer._grouped_ok(32)
+    assert layer._grouped_ok(B)
     y = layer.apply(x)
     assert y.dtype == x.dtype and y.shape == y_ref.shape
     assert rel(y, _oracle(x, arts, n)) < TOL
@@ -214,10 +214,10 @@ def test_merged_linear_through_the_grouped_call(ops, monkeypatch, B):
 
 @pytest.mark.parametrize("n,shards,bpw", [(512, [(352, 4, 2), (352, 4, 2)], 6), (2048, [(2048, 4, 1), (512, 4, 1), (512, 4, 1)], 5),
                                           (576, [(1184, 4, 4), (1184, 4, 4)], 8)])
-@pytest.mark.parametrize("B", [1, 2, 9, 16])
+@pytest.mark.parametrize("B", [1, 2, 9, 16, 17, 40, 64])
 def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, shards, bpw, B):
     """One token of merged stacked shards (5, 6, 8 bpw = 4 + 1, 2, 4) through the library's grouped
-    two-stage call (one token: one decode launch for both streams of every shard; 2-16: one per shard; one
+    two-stage call (one token: one decode launch for both streams of every shard; 2-64: one per shard; one
     finishing launch) against the oracle and against the reference's sequence of registered ops; more tokens keep
     that sequence."""
     from glq_amd import linear_method as LM
@@ -227,7 +227,7 @@ def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, s
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", False)
     y_ref = layer.apply(x)
     monkeypatch.setattr(LM, "_GLQ_MERGED_GROUPED", True)
-    assert layer._grouped_rvq2_ok(B) and not layer._grouped_rvq2_ok(17) and not layer._grouped_ok(B)
+    assert layer._grouped_rvq2_ok(B) and not layer._grouped_rvq2_ok(65) and not layer._grouped_ok(B)
     y = layer.apply(x)
     assert y.dtype == x.dtype and y.shape == y_ref.shape
     assert rel(y, _oracle(x, arts, n)) < TOL
@@ -237,9 +237,9 @@ def test_merged_two_stage_linear_through_the_grouped_call(ops, monkeypatch, n, s
     assert not mixed._grouped_rvq2_ok(B)
 
 
-@pytest.mark.parametrize("B", [64, 200])
+@pytest.mark.parametrize("B", [65, 200])
 def test_merged_stacked_shards_at_many_tokens_run_as_whole_linears(ops, monkeypatch, B):
-    """From 64 tokens on, shards the grouped call does not take (here 4+2-bit gate/up and a mixed pair) run as
+    """Above 64 tokens, shards the grouped call does not take (here 4+2-bit gate/up and a mixed pair) run as
     whole fused linears, concatenated: against the oracle and against the reference's shard-batched sequence."""
     from glq_amd import linear_method as LM
     say("merged stacked shards, many tokens", B)

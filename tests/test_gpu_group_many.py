@@ -79,9 +79,12 @@ def test_grouped_many_tokens_refusals():
     x = torch.zeros(100, 256, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError, match="layers"):
         ext.glq_fused_linear_trellis_3inst_group(x, shards, torch.tensor(bn), bn_meta, 256, 256, out_dtype=torch.bfloat16)
-    with pytest.raises(RuntimeError):                            # 5..64 tokens: the per-layer op serves those
-        ext.glq_fused_linear_trellis_3inst_group(x[:32], shards[:2], torch.tensor(bn), bn_meta, 256, 256,
+    with pytest.raises(RuntimeError):                            # 32 tokens are served, five layers are not
+        ext.glq_fused_linear_trellis_3inst_group(x[:32], shards, torch.tensor(bn), bn_meta, 256, 256,
                                                  out_dtype=torch.bfloat16)
+    y32 = ext.glq_fused_linear_trellis_3inst_group(x[:32], shards[:2], torch.tensor(bn), bn_meta, 256, 256,
+                                                   out_dtype=torch.bfloat16)
+    assert y32.shape == (32, 512) and float(y32.abs().max()) == 0.0   # zero activations
     with pytest.raises(RuntimeError, match="separate"):
         ext.glq_fused_linear_trellis_3inst_group(x[:2], shards[:2], torch.tensor(bn), bn_meta, 256, 256,
                                                  out_dtype=torch.bfloat16, separate=True)

@@ -77,6 +77,10 @@ int glqh_launch_trellis_tile_group(const void *const xb[], int64_t M, const void
                                    hipStream_t stream, const float f16_scale[] = nullptr);
 int glqh_launch_trellis_pack(const void *x_f16, void *xb, int64_t M, int64_t k, hipStream_t stream);
 int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages);
+// several sign vectors on the same few rows in one launch (fht.hip); -1 = not eligible, nothing launched
+int glqh_launch_input_rht_multi(const void *x, int x_dtype, int64_t x_stride, const void *const sv[], void *const out[],
+                                int n, int64_t B, int64_t in_features, int64_t n_pad, const glqh_block_meta *meta_dev,
+                                const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
 // input transform straight into a tile kernel's operand layout (fht.hip); -1 = not eligible, nothing launched
 int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, const void *sv, void *xb,
                                   int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
@@ -750,7 +754,7 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
         int S = 0, ksb = 0;
         const int64_t mmin = total_m_pad / n_shards / 32 * 32;
         glqh_trellis_mma_plan(mmin < 32 ? 32 : mmin, n_pad, &S, &ksb);
-        return (size_t)n_shards * 256 + align256((size_t)B * n_pad * sizeof(f16)) +
+        return (size_t)n_shards * (256 + align256((size_t)B * n_pad * sizeof(f16))) +
                align256((size_t)ksb * B * total_m_pad * sizeof(float));
     }
     int steps = 0, ks = 0;
@@ -762,7 +766,7 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
     // the separate-transform route of large groups: slots of the plain plan (at most 64) and x_rht
     size_t plain = 0;
     if (tr_group_plain(total_m_pad, n_pad, B))
-        plain = align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)64 * B * total_m_pad * sizeof(float));
+        plain = (size_t)n_shards * align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)64 * B * total_m_pad * sizeof(float));
     const size_t fused = align256((size_t)ks * B * total_m_pad * sizeof(float));
     // (2..4 tokens of stacked layers, glqh_fused_linear_trellis_3inst_group_rvq2: x_rht and the sums under the K
     // plan of the tallest layer, which has at least total / n_shards rows)
@@ -771,7 +775,8 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
         int S = 0, ksb = 0;
         const int64_t mmin = total_m_pad / n_shards / 32 * 32;
         glqh_trellis_mma_plan(mmin < 32 ? 32 : mmin, n_pad, &S, &ksb);
-        stacked = align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ksb * B * total_m_pad * sizeof(float));
+        stacked = (size_t)n_shards * align256((size_t)B * n_pad * sizeof(f16)) +
+                  align256((size_t)ksb * B * total_m_pad * sizeof(float));
     }
     const size_t most = plain > fused ? plain : fused;
     return (size_t)n_shards * 256 + (stacked > most ? stacked : most);
@@ -896,6 +901,37 @@ struct tr_group_ctx {
     float *parts[GLQH_MAX_SHARDS];
 };
 
+// x under every distinct sign vector of a group of layers, fp16 rows at ws + j * xb_one (few tokens): one launch for
+// all of them where the small-batch kernel serves the call, one per sign vector otherwise.  x_of[i] = layer i's rows.
+static int tr_group_transform(const void *x, int x_dtype, int64_t x_stride, int64_t B, const void *const sv[], int n_shards,
+                              const int64_t *blocks_n, int64_t n_blocks_n, const glqh_block_meta *bn_meta_dev,
+                              int64_t in_features, int64_t n_pad, void *ws, size_t xb_one, const f16 *x_of[],
+                              hipStream_t st) {
+    const void *dsv[GLQH_MAX_SHARDS];
+    void *dout[GLQH_MAX_SHARDS];
+    int nd = 0;
+    for (int i = 0; i < n_shards; ++i) {
+        int j = 0;
+        while (j < nd && dsv[j] != sv[i]) ++j;
+        if (j == nd) {
+            dsv[nd] = sv[i];
+            dout[nd] = (char *)ws + (size_t)nd * xb_one;
+            ++nd;
+        }
+        x_of[i] = (const f16 *)dout[j];
+    }
+    int rc = nd > 1 ? glqh_launch_input_rht_multi(x, x_dtype, x_stride, dsv, dout, nd, B, in_features, n_pad, bn_meta_dev,
+                                                  blocks_n, n_blocks_n, st)
+                    : -1;
+    if (rc > 0) return 1;
+    if (rc == 0) return 0;
+    for (int j = 0; j < nd; ++j)
+        if (glqh_launch_input_rht(x, x_dtype, x_stride, dsv[j], dout[j], GLQH_F16, B, in_features, n_pad, bn_meta_dev,
+                                  blocks_n, n_blocks_n, 0.0f, st))
+            return 1;
+    return 0;
+}
+
 // One finishing launch for all layers of a group; at 17..64 tokens, where every layer has its own K plan, one per
 // layer when their slot counts differ.
 static int tr_group_finish(const tr_group_ctx &c, int n_shards, int64_t B, int y_dtype, int64_t y_stride, hipStream_t st) {
@@ -1006,21 +1042,19 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
         int S = 0;
         glqh_trellis_mma_plan(mmax, n_pad, &S, &ks);
         const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
-        const size_t need = xb + align256((size_t)ks * B * total * sizeof(float));
+        const size_t need = (size_t)n_shards * xb + align256((size_t)ks * B * total * sizeof(float));
         GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
-        f16 *x_rht = (f16 *)ws;
-        float *p = (float *)((char *)ws + xb);
+        float *p = (float *)((char *)ws + (size_t)n_shards * xb);
         c->R = R; c->ks = ks; c->fi_mode = 0;
+        // layers quantized with the same sign vector share one transform of x
+        const f16 *x_of[GLQH_MAX_SHARDS];
+        if (tr_group_transform(x, x_dtype, x_stride, B, sv, n_shards, blocks_n, n_blocks_n, bn_meta_dev, in_features, n_pad,
+                               ws, xb, x_of, st))
+            return 1;
         for (int i = 0; i < n_shards; ++i) {
-            // layers quantized with the same sign vector share one transform of x; launches on
-            // one stream run in order, so x_rht can be rewritten between layers
-            if ((i == 0 || sv[i] != sv[i - 1]) &&
-                glqh_launch_input_rht(x, x_dtype, x_stride, sv[i], x_rht, GLQH_F16, B, in_features, n_pad, bn_meta_dev,
-                                      blocks_n, n_blocks_n, 0.0f, st))
-                return 1;
             c->parts[i] = p;
             p += (size_t)ks * B * c->m_pads[i];
-            if (glqh_launch_trellis_mma(x_rht, B, packed[i], R, c->m_pads[i], n_pad, S, ks, c->parts[i], 0, 1.0f, 0, 0, st))
+            if (glqh_launch_trellis_mma(x_of[i], B, packed[i], R, c->m_pads[i], n_pad, S, ks, c->parts[i], 0, 1.0f, 0, 0, st))
                 return 1;
         }
         return 0;
@@ -1165,19 +1199,18 @@ extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_d
         int S = 0;
         glqh_trellis_mma_plan(mmax, n_pad, &S, &ks);
         const size_t xb = align256((size_t)B * n_pad * sizeof(f16));
-        const size_t need = xb + align256((size_t)ks * B * total * sizeof(float));
+        const size_t need = (size_t)n_shards * xb + align256((size_t)ks * B * total * sizeof(float));
         GLQH_REQUIRE(ws && ws_bytes >= need, "trellis two-stage group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
-        f16 *x_rht = (f16 *)ws;
-        float *p = (float *)((char *)ws + xb);
+        float *p = (float *)((char *)ws + (size_t)n_shards * xb);
+        const f16 *x_of[GLQH_MAX_SHARDS];
+        if (tr_group_transform(x, x_dtype, x_stride, B, sv, n_shards, blocks_n, n_blocks_n, bn_meta_dev, in_features, n_pad,
+                               ws, xb, x_of, st))
+            return 1;
         for (int i = 0; i < n_shards; ++i) {
-            if ((i == 0 || sv[i] != sv[i - 1]) &&
-                glqh_launch_input_rht(x, x_dtype, x_stride, sv[i], x_rht, GLQH_F16, B, in_features, n_pad, bn_meta_dev,
-                                      blocks_n, n_blocks_n, 0.0f, st))
-                return 1;
             c.parts[i] = p;
             p += (size_t)ks * B * c.m_pads[i];
             glqh_range range("dequant_matmul");
-            if (glqh_launch_trellis_mma_rvq(x_rht, B, packed[i], packed2[i], R2, rs2[i], c.m_pads[i], n_pad, S, ks,
+            if (glqh_launch_trellis_mma_rvq(x_of[i], B, packed[i], packed2[i], R2, rs2[i], c.m_pads[i], n_pad, S, ks,
                                             c.parts[i], st))
                 return 1;
         }

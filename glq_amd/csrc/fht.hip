@@ -16,12 +16,11 @@ constexpr int RHT_THREADS = GLQH_RHT_THREADS;
 
 // XT / OT: element types (bf16 travels as uint16_t)
 template <typename XT, typename OT>
-__global__ void __launch_bounds__(RHT_THREADS)
-input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
-                 OT *__restrict__ out, int in_features, int n_pad,
-                 const glqh_block_meta *__restrict__ meta, glqh_meta_args margs,
-                 float single_norm, int spb, int log_slice) {
-    extern __shared__ float s[];
+__device__ __forceinline__ void
+input_rht_body(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
+               OT *__restrict__ out, int in_features, int n_pad,
+               const glqh_block_meta *__restrict__ meta, const glqh_meta_args &margs,
+               float single_norm, int spb, int log_slice, float *s) {
     const rht_slice blk = rht_get_slice(meta, margs, single_norm, spb, log_slice);
     if (!blk.live) return;
     const XT *xr = x + (int64_t)blockIdx.y * x_stride;
@@ -55,6 +54,32 @@ input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restri
     if (blk.nsub == 1 && blk.log_len >= 11) stage_signed_slices<RHT_THREADS, 8, 1>(s, blk.log_len, 1, 0, val);
     else stage_signed_slices<RHT_THREADS>(s, blk.log_len, blk.nsub, blk.r, val);
     fht_staged(s, blk.log_len, store);
+}
+
+template <typename XT, typename OT>
+__global__ void __launch_bounds__(RHT_THREADS)
+input_rht_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__restrict__ sv,
+                 OT *__restrict__ out, int in_features, int n_pad,
+                 const glqh_block_meta *__restrict__ meta, glqh_meta_args margs,
+                 float single_norm, int spb, int log_slice) {
+    extern __shared__ float s[];
+    input_rht_body<XT, OT>(x, x_stride, sv, out, in_features, n_pad, meta, margs, single_norm, spb, log_slice, s);
+}
+
+// The same rows under several sign vectors in one launch (layers of a group that were quantized with their own
+// input signs): blockIdx.z picks the sign vector and its output.
+struct rht_in_multi {
+    const f16 *sv[GLQH_MAX_GROUP];
+    f16 *out[GLQH_MAX_GROUP];
+};
+template <typename XT>
+__global__ void __launch_bounds__(RHT_THREADS)
+input_rht_multi_kernel(const XT *__restrict__ x, int64_t x_stride, rht_in_multi g, int in_features, int n_pad,
+                       const glqh_block_meta *__restrict__ meta, glqh_meta_args margs, float single_norm, int spb,
+                       int log_slice) {
+    extern __shared__ float s[];
+    input_rht_body<XT, f16>(x, x_stride, g.sv[blockIdx.z], g.out[blockIdx.z], in_features, n_pad, meta, margs,
+                            single_norm, spb, log_slice, s);
 }
 
 // ---- many tokens: whole blocks, 16-byte accesses ------------------------------------
@@ -764,6 +789,45 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
     }
 #undef GLQH_IN_LAUNCH
     GLQH_LAUNCH_CHECK("input_rht launch");
+    return 0;
+}
+
+// n (up to GLQH_MAX_GROUP) sign vectors on the same rows, fp16 out, few rows (the small-batch kernel): one launch.
+// -1 (nothing launched) when the call is one for the whole-block kernels or the dtypes are others.
+int glqh_launch_input_rht_multi(const void *x, int x_dtype, int64_t x_stride, const void *const sv[], void *const out[],
+                                int n, int64_t B, int64_t in_features, int64_t n_pad, const glqh_block_meta *meta_dev,
+                                const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream) {
+    if (n < 1 || n > GLQH_MAX_GROUP || B < 1 || B > 65535 || in_features < 1 || in_features > n_pad) return -1;
+    if (x_dtype != GLQH_F16 && x_dtype != GLQH_BF16) return -1;
+    int64_t max_bs = n_pad;
+    glqh_meta_args margs;
+    if (n_blocks > 1) {
+        if (!meta_dev || !blocks_host || check_blocks(blocks_host, n_blocks, n_pad, &max_bs, "input_rht")) return -1;
+    } else {
+        if ((n_pad & (n_pad - 1)) != 0) return -1;
+        meta_dev = nullptr;
+        n_blocks = 1;
+    }
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, n_pad)) margs.canon = 0;
+    if (rht_wide_ok(B, margs, n_pad, max_bs)) return -1;       // many rows: the whole-block kernels, one launch each
+    glqh_range range("input_rht");
+    const int log_slice = rht_log_slice(B);
+    const int spb = rht_slices_per_block(max_bs, log_slice);
+    if (n_blocks * spb > 2147483647ll) return -1;
+    rht_in_multi g = {};
+    for (int i = 0; i < GLQH_MAX_GROUP; ++i) {
+        g.sv[i] = (const f16 *)sv[i < n ? i : 0];
+        g.out[i] = (f16 *)out[i < n ? i : 0];
+    }
+    dim3 grid((unsigned)(n_blocks * spb), (unsigned)B, (unsigned)n);
+    if (x_dtype == GLQH_F16)
+        hipLaunchKernelGGL((input_rht_multi_kernel<f16>), grid, dim3(RHT_THREADS), rht_lds_bytes(log_slice), stream,
+                           (const f16 *)x, x_stride, g, (int)in_features, (int)n_pad, meta_dev, margs, 0.0f, spb, log_slice);
+    else
+        hipLaunchKernelGGL((input_rht_multi_kernel<uint16_t>), grid, dim3(RHT_THREADS), rht_lds_bytes(log_slice), stream,
+                           (const uint16_t *)x, x_stride, g, (int)in_features, (int)n_pad, meta_dev, margs, 0.0f, spb,
+                           log_slice);
+    GLQH_LAUNCH_CHECK("input_rht group launch");
     return 0;
 }
 

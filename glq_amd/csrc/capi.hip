@@ -81,6 +81,9 @@ int64_t glqh_e8_tile_padded_tokens(int64_t M, int nstages);
 int glqh_launch_input_rht_multi(const void *x, int x_dtype, int64_t x_stride, const void *const sv[], void *const out[],
                                 int n, int64_t B, int64_t in_features, int64_t n_pad, const glqh_block_meta *meta_dev,
                                 const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
+int glqh_launch_input_rht_blocked_multi(const void *x, int x_dtype, int64_t x_stride, const void *const sv[],
+                                        void *const xb[], int n, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
+                                        const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream);
 // input transform straight into a tile kernel's operand layout (fht.hip); -1 = not eligible, nothing launched
 int glqh_launch_input_rht_blocked(const void *x, int x_dtype, int64_t x_stride, const void *sv, void *xb,
                                   int layout, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
@@ -745,7 +748,7 @@ extern "C" size_t glqh_fused_linear_trellis_group_workspace_bytes(int64_t B, int
         // the plan of a 128-row layer (fewer row tiles, more slots)
         const int ks1 = glqh_trellis_tile_ksplit(TT_GROUP_ROWS_FLOOR, n_pad, B), ks2 = glqh_trellis_tile_ksplit(TT_GROUP_ROWS_FLOOR, n_pad, B, 1);
         const int ksb = ks1 > ks2 ? ks1 : ks2;                 // (single-stage and stacked layers)
-        return (size_t)n_shards * 256 + align256(glqh_trellis_tile_xb_bytes(n_pad, B)) +
+        return (size_t)n_shards * (256 + align256(glqh_trellis_tile_xb_bytes(n_pad, B))) +
                align256((size_t)B * n_pad * sizeof(f16)) + align256((size_t)ksb * B * total_m_pad * sizeof(float));
     }
     if (B > 4) {
@@ -932,6 +935,29 @@ static int tr_group_transform(const void *x, int x_dtype, int64_t x_stride, int6
     return 0;
 }
 
+// 17..64 tokens: x under every distinct sign vector of a group straight into the tile kernels' layout, buffer j at
+// ws + j * xbb, in one launch.  0: done, xb_of[i] = layer i's buffer; -1: not applicable, nothing launched.
+static int tr_group_transform_blocked(const void *x, int x_dtype, int64_t x_stride, int64_t B, const void *const sv[],
+                                      int n_shards, const int64_t *blocks_n, int64_t n_blocks_n, int64_t in_features,
+                                      int64_t n_pad, void *ws, size_t xbb, void *xb_of[], hipStream_t st) {
+    const void *dsv[GLQH_MAX_SHARDS];
+    void *dout[GLQH_MAX_SHARDS];
+    int nd = 0;
+    for (int i = 0; i < n_shards; ++i) {
+        int j = 0;
+        while (j < nd && dsv[j] != sv[i]) ++j;
+        if (j == nd) {
+            dsv[nd] = sv[i];
+            dout[nd] = (char *)ws + (size_t)nd * xbb;
+            ++nd;
+        }
+        xb_of[i] = dout[j];
+    }
+    if (nd < 2) return -1;
+    return glqh_launch_input_rht_blocked_multi(x, x_dtype, x_stride, dsv, dout, nd, glqh_trellis_tile_padded_tokens(B), B,
+                                               in_features, n_pad, blocks_n, n_blocks_n, st);
+}
+
 // One finishing launch for all layers of a group; at 17..64 tokens, where every layer has its own K plan, one per
 // layer when their slot counts differ.
 static int tr_group_finish(const tr_group_ctx &c, int n_shards, int64_t B, int y_dtype, int64_t y_stride, hipStream_t st) {
@@ -1010,14 +1036,27 @@ static int tr_group_decode(const void *x, int x_dtype, int64_t x_stride, int64_t
             same = same && c->ks_layer[i] == c->ks_layer[0];
             sums += align256((size_t)c->ks_layer[i] * B * c->m_pads[i] * sizeof(float));
         }
-        const size_t need = xbb + xrm + sums;
+        const size_t need = (size_t)n_shards * xbb + xrm + sums;
         GLQH_REQUIRE(ws && ws_bytes >= need, "trellis group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
         void *xb = ws;
-        f16 *x_rht = (f16 *)((char *)ws + xbb);
-        char *p = (char *)ws + xbb + xrm;
+        f16 *x_rht = (f16 *)((char *)ws + (size_t)n_shards * xbb);
+        char *p = (char *)ws + (size_t)n_shards * xbb + xrm;
         c->R = R; c->ks = same ? c->ks_layer[0] : 0; c->fi_mode = 0;
+        void *xb_of[GLQH_MAX_SHARDS];
+        const int all = tr_group_transform_blocked(x, x_dtype, x_stride, B, sv, n_shards, blocks_n, n_blocks_n, in_features,
+                                                   n_pad, ws, xbb, xb_of, st);
+        if (all > 0) return 1;
         int blocked = -1;
         for (int i = 0; i < n_shards; ++i) {
+            if (all == 0) {                                    // every sign vector's activations are in place
+                c->parts[i] = (float *)p;
+                p += align256((size_t)c->ks_layer[i] * B * c->m_pads[i] * sizeof(float));
+                glqh_range range("dequant_matmul");
+                if (glqh_launch_trellis_tile(nullptr, xb_of[i], B, packed[i], R, c->m_pads[i], n_pad, c->parts[i], 0, 1.0f, 0,
+                                             0, st, 0))
+                    return 1;
+                continue;
+            }
             if (i == 0 || sv[i] != sv[i - 1]) {
                 blocked = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, sv[i], xb, 2, glqh_trellis_tile_padded_tokens(B),
                                                         B, in_features, n_pad, blocks_n, n_blocks_n, st);
@@ -1166,14 +1205,27 @@ extern "C" int glqh_fused_linear_trellis_3inst_group_rvq2(const void *x, int x_d
             same = same && c.ks_layer[i] == c.ks_layer[0];
             sums += align256((size_t)c.ks_layer[i] * B * c.m_pads[i] * sizeof(float));
         }
-        const size_t need = xbb + xrm + sums;
+        const size_t need = (size_t)n_shards * xbb + xrm + sums;
         GLQH_REQUIRE(ws && ws_bytes >= need, "trellis two-stage group: workspace of %zu bytes needed, got %zu", need, ws_bytes);
         void *xb = ws;
-        f16 *x_rht = (f16 *)((char *)ws + xbb);
-        char *p = (char *)ws + xbb + xrm;
+        f16 *x_rht = (f16 *)((char *)ws + (size_t)n_shards * xbb);
+        char *p = (char *)ws + (size_t)n_shards * xbb + xrm;
         c.ks = same ? c.ks_layer[0] : 0;
+        void *xb_of[GLQH_MAX_SHARDS];
+        const int all = tr_group_transform_blocked(x, x_dtype, x_stride, B, sv, n_shards, blocks_n, n_blocks_n, in_features,
+                                                   n_pad, ws, xbb, xb_of, st);
+        if (all > 0) return 1;
         int blocked = -1;
         for (int i = 0; i < n_shards; ++i) {
+            if (all == 0) {                                    // every sign vector's activations are in place
+                c.parts[i] = (float *)p;
+                p += align256((size_t)c.ks_layer[i] * B * c.m_pads[i] * sizeof(float));
+                glqh_range range("dequant_matmul");
+                if (glqh_launch_trellis_tile(nullptr, xb_of[i], B, packed[i], 4, c.m_pads[i], n_pad, c.parts[i], 0, 1.0f, 0, 0,
+                                             st, 0, packed2[i], R2, rs2[i]))
+                    return 1;
+                continue;
+            }
             if (i == 0 || sv[i] != sv[i - 1]) {
                 blocked = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, sv[i], xb, 2, glqh_trellis_tile_padded_tokens(B),
                                                         B, in_features, n_pad, blocks_n, n_blocks_n, st);

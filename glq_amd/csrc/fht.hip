@@ -318,6 +318,43 @@ input_rht_wide_kernel(const XT *__restrict__ x, int64_t x_stride, const f16 *__r
         input_rht_wide_body<8, XT, OT, LAYOUT>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s, role);
 }
 
+// The same rows under several sign vectors in one launch, trellis operand layout out (layers of a group that were
+// quantized with their own input signs, 17..64 tokens): blockIdx.y picks the sign vector and its output; the
+// dealing of rows and blocks is input_rht_wide_kernel's.
+struct rht_in_wide_multi {
+    const f16 *sv[GLQH_MAX_GROUP];
+    f16 *out[GLQH_MAX_GROUP];
+};
+template <typename XT>
+__global__ void __launch_bounds__(REG_THREADS)
+input_rht_wide_multi_kernel(const XT *__restrict__ x, int64_t x_stride, rht_in_wide_multi mg, int in_features, int n_pad,
+                            int Mp, int B, int n_blocks, glqh_meta_args margs, float single_norm) {
+    extern __shared__ float s[];
+    const f16 *sv = mg.sv[blockIdx.y];
+    f16 *out = mg.out[blockIdx.y];
+    const int L = blockIdx.x, per_xcd = (B + 7) >> 3;
+    const int j = L >> 3;
+    const int member = j & 7, rest = j >> 3, g = rest / n_blocks;
+    const rht_slice blk = rht_slice_of(margs, single_norm, rest % n_blocks);
+    if (blk.log_bs <= WIDE_SMALL_LOG) {
+        const int lsets = 12 - blk.log_bs - 3;
+        if ((g & ((1 << lsets) - 1)) != 0 || member != ((g >> lsets) & 7)) return;
+        const int t_in = g * 8, tok0 = (L & 7) * per_xcd + t_in;
+        if (t_in >= per_xcd || tok0 >= B) return;
+        const int ntok = min(8 << lsets, min(per_xcd - t_in, B - tok0));
+        const wide_role role = wide_role_of(blk, ntok);
+        input_rht_wide_body<8, XT, f16, 2>(x, x_stride, sv, out, in_features, n_pad, Mp, tok0 + min(role.tok, ntok - 1), blk, s,
+                                           role);
+        return;
+    }
+    const int t_in = g * 8 + member;
+    const int token = (L & 7) * per_xcd + t_in;
+    if (token >= B || t_in >= per_xcd) return;                // uniform over the workgroup
+    const wide_role role = wide_role_of(blk, 1);
+    if (blk.log_bs > 12) input_rht_wide_body<16, XT, f16, 2>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s, role);
+    else input_rht_wide_body<8, XT, f16, 2>(x, x_stride, sv, out, in_features, n_pad, Mp, token, blk, s, role);
+}
+
 // v = the transformed sums of elements E * tid .. E * tid + E - 1 of block `blk`, row b (before the
 // signs and the 1/sqrt(bs)): direct rows or split-K partial sums in, register transform, runs restored.
 // Every thread of the workgroup calls.
@@ -789,6 +826,48 @@ int glqh_launch_input_rht(const void *x, int x_dtype, int64_t x_stride, const vo
     }
 #undef GLQH_IN_LAUNCH
     GLQH_LAUNCH_CHECK("input_rht launch");
+    return 0;
+}
+
+// n (up to GLQH_MAX_GROUP) sign vectors on the same rows, each into its own buffer in the trellis tile kernels' operand
+// layout: one launch.  -1 (nothing launched) where glqh_launch_input_rht_blocked would not apply either.
+int glqh_launch_input_rht_blocked_multi(const void *x, int x_dtype, int64_t x_stride, const void *const sv[],
+                                        void *const xb[], int n, int64_t Mp, int64_t B, int64_t in_features, int64_t n_pad,
+                                        const int64_t *blocks_host, int64_t n_blocks, hipStream_t stream) {
+    if (!x || n < 1 || n > GLQH_MAX_GROUP || B < 1 || in_features < 1 || in_features > n_pad) return -1;
+    if (x_dtype != GLQH_F16 && x_dtype != GLQH_BF16) return -1;
+    glqh_meta_args margs;
+    int64_t max_bs = n_pad;
+    if (n_blocks > 1) {
+        if (!blocks_host) return -1;
+        max_bs = 0;
+        for (int64_t i = 0; i < n_blocks; ++i) max_bs = blocks_host[i] > max_bs ? blocks_host[i] : max_bs;
+    } else {
+        n_blocks = 1;
+    }
+    if (!glqh_fill_meta_args(&margs, blocks_host, n_blocks, n_pad) || margs.canon != n_pad) return -1;
+    if (max_bs > (1 << WIDE_LOG_MAX) || (n_pad & 31) != 0) return -1;
+    if (!aligned16(x) || (x_stride * 2) % 16 != 0) return -1;
+    rht_in_wide_multi mg = {};
+    for (int i = 0; i < GLQH_MAX_GROUP; ++i) {
+        const int j = i < n ? i : 0;
+        if (!sv[j] || !xb[j] || !aligned16(sv[j]) || !aligned16(xb[j])) return -1;
+        mg.sv[i] = (const f16 *)sv[j];
+        mg.out[i] = (f16 *)xb[j];
+    }
+    const int64_t wgs = 64 * (((B + 7) / 8 + 7) / 8) * n_blocks;
+    if (wgs > 2147483647ll) return -1;
+    glqh_range range("input_rht");
+    const dim3 wgrid((unsigned)wgs, (unsigned)n);
+    const size_t lds = std::max(rht_reg_lds_bytes(ilog2(max_bs)), WIDE_SMALL_LDS);
+    if (x_dtype == GLQH_F16)
+        hipLaunchKernelGGL((input_rht_wide_multi_kernel<f16>), wgrid, dim3(REG_THREADS), lds, stream, (const f16 *)x, x_stride,
+                           mg, (int)in_features, (int)n_pad, (int)Mp, (int)B, (int)n_blocks, margs, 0.0f);
+    else
+        hipLaunchKernelGGL((input_rht_wide_multi_kernel<uint16_t>), wgrid, dim3(REG_THREADS), lds, stream,
+                           (const uint16_t *)x, x_stride, mg, (int)in_features, (int)n_pad, (int)Mp, (int)B, (int)n_blocks,
+                           margs, 0.0f);
+    GLQH_LAUNCH_CHECK("input_rht group launch");
     return 0;
 }
 

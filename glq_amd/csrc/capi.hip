@@ -842,6 +842,26 @@ static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B
     }
     const size_t esz = f16_sums ? sizeof(f16) : sizeof(float);
     size_t poff = 0;
+    // all distinct sign vectors in one transform launch where it applies (layer i's activations in buffer i)
+    int all = -1;
+    {
+        const void *dsv[GLQH_MAX_SHARDS];
+        void *dout[GLQH_MAX_SHARDS];
+        int nd = 0;
+        for (int i = 0; i < n_shards; ++i) {
+            int j = 0;
+            while (j < nd && dsv[j] != shards[i].sv_f16) ++j;
+            if (j == nd) {
+                dsv[nd] = shards[i].sv_f16;
+                dout[nd] = base + (size_t)i * xb_one;
+                ++nd;
+            }
+        }
+        if (nd > 1)
+            all = glqh_launch_input_rht_blocked_multi(x, x_dtype, x_stride, dsv, dout, nd, Mp, B, in_features, n_pad, blocks_n,
+                                                      n_blocks_n, st);
+        if (all > 0) return 1;
+    }
     for (int i = 0; i < n_shards; ++i) {
         // layers quantized with the same sign vector share one transform of x
         int same = -1;
@@ -849,6 +869,8 @@ static int tr_group_many(const void *x, int x_dtype, int64_t x_stride, int64_t B
             if (shards[j].sv_f16 == shards[i].sv_f16) { same = j; break; }
         if (same >= 0) {
             xb[i] = xb[same];
+        } else if (all == 0) {
+            xb[i] = base + (size_t)i * xb_one;
         } else {
             void *dst = base + (size_t)i * xb_one;
             const int rc = glqh_launch_input_rht_blocked(x, x_dtype, x_stride, shards[i].sv_f16, dst, 2, Mp, B, in_features,
